@@ -1,0 +1,481 @@
+"""numpy oracle for dicee's KvsAll scoring and link-prediction path.
+
+TEST INFRASTRUCTURE ONLY (see ``oracle/__init__.py``): never imported by the
+shipped package.
+
+Every function restates, in plain numpy, what the cited reference lines compute.
+Arithmetic runs in float64 unless ``dtype`` says otherwise, so the oracle is a
+tighter reference than the fp32 torch code it mirrors.
+
+Pinning status (independent checks live in ``tests/test_oracle_pins.py``)
+------------------------------------------------------------------------
+* ``distmult_*``      brute-force triple loop; closed form ``(h*r).e``.
+* ``complex_*``       ``Re<h, r, conj(t)>`` in numpy complex128; per-triple
+                      formula of ``dicee/models/complex.py:229-238``.
+* ``quaternion_normalize`` unit norm of every group of 4 consecutive elements,
+                      zero-vector ``eps`` case, hand-computed d=8 fixture.
+* ``qmult_*``         Hamilton product against an independently built 4x4x4
+                      structure-constant table and against
+                      ``scipy.spatial.transform.Rotation`` composition; the
+                      block-split vs consecutive-group quirk has a d=8 fixture.
+* ``keci_*``          (p,q)=(0,0) == DistMult; (0,1), c=1 == ComplEx; (0,1),
+                      c=0 == DistMult on the first half; general (p,q) against a
+                      brute-force geometric-algebra product on bitmask blades;
+                      thresholds p>=2 / q>=2 / (p>=2 and q>=2) by fixtures.
+* ``layer_norm`` / ``batch_norm_eval``  torch.nn.functional library routines.
+* ``filtered_rank_counts``  explicit masking + stable argsort brute force;
+                      invariants (duplicates idempotent, -inf never outranks,
+                      target never masked, empty filter); torch.sort placement
+                      lies inside ``[lo, hi]``.
+* ``topk``            ``numpy.argsort`` brute force; sigmoid identity.
+* ``bce_multihot``    ``torch.nn.functional.binary_cross_entropy_with_logits``
+                      on a dense target, with and without label smoothing.
+* ``bf16_round`` / ``quantize_int8_rows``  torch's bf16 cast; closed forms.
+No function is "parity unpinned" with respect to the arithmetic.  What stays
+unpinned is the position an *unstable* ``torch.sort`` gives a tied target
+(``dicee/evaluation/evaluator.py:503``): that is torch's behaviour, not the
+reference's, and the oracle reports the admissible interval instead.
+"""
+from __future__ import annotations
+
+import numpy as np
+
+MODELS = ("DistMult", "ComplEx", "QMult", "Keci")
+
+# --------------------------------------------------------------------------
+# storage emulation (exists only in this build; the reference is fp32-only)
+# --------------------------------------------------------------------------
+
+
+def bf16_round(x: np.ndarray) -> np.ndarray:
+    """Round fp32 to the nearest bf16 (ties to even), returned as fp32."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    u = x.view(np.uint32).astype(np.uint64)
+    nan = np.isnan(x)
+    rounded = ((u + 0x7FFF + ((u >> 16) & 1)) >> 16) << 16
+    out = rounded.astype(np.uint32).view(np.float32).copy()
+    out[nan] = np.nan
+    return out.reshape(x.shape)
+
+
+def bf16_bits(x: np.ndarray) -> np.ndarray:
+    """uint16 bit patterns of ``bf16_round(x)``."""
+    return (bf16_round(x).view(np.uint32) >> 16).astype(np.uint16)
+
+
+def bf16_from_bits(b: np.ndarray) -> np.ndarray:
+    return (b.astype(np.uint32) << 16).view(np.float32)
+
+
+def quantize_int8_rows(x: np.ndarray):
+    """Per-row symmetric int8: ``scale = max|row|/127``, ``q = rint(row/scale)``."""
+    x = np.asarray(x, dtype=np.float32)
+    amax = np.abs(x).max(axis=1)
+    scale = (amax / 127.0).astype(np.float32)
+    safe = np.where(scale > 0, scale, 1.0).astype(np.float32)
+    q = np.rint(x / safe[:, None]).clip(-127, 127).astype(np.int8)
+    return q, scale
+
+
+def dequantize_int8_rows(q: np.ndarray, scale: np.ndarray) -> np.ndarray:
+    return q.astype(np.float32) * scale.astype(np.float32)[:, None]
+
+
+# --------------------------------------------------------------------------
+# G2: gather (+ optional normalisation)   dicee/models/base_model.py:377-384
+# --------------------------------------------------------------------------
+
+
+def layer_norm(x, weight, bias, eps=1e-5):
+    """torch.nn.LayerNorm over the last axis (base_model.py:283-288)."""
+    x = np.asarray(x, dtype=np.float64)
+    mu = x.mean(axis=-1, keepdims=True)
+    var = ((x - mu) ** 2).mean(axis=-1, keepdims=True)
+    return (x - mu) / np.sqrt(var + eps) * np.asarray(weight, np.float64) + np.asarray(bias, np.float64)
+
+
+def batch_norm_eval(x, running_mean, running_var, eps=1e-5):
+    """torch.nn.BatchNorm1d(affine=False) in eval mode (base_model.py:289-294)."""
+    x = np.asarray(x, dtype=np.float64)
+    return (x - np.asarray(running_mean, np.float64)) / np.sqrt(np.asarray(running_var, np.float64) + eps)
+
+
+def gather_hr(E, R, hr, norm=None, dtype=np.float64):
+    """Head / relation rows for a batch of (head_id, relation_id) pairs.
+
+    Dropout is the identity in eval mode (base_model.py:149-151).  ``norm`` is
+    None (IdentityClass) or a dict: ``{"kind": "LayerNorm", "h_weight", "h_bias",
+    "r_weight", "r_bias", "eps"}`` / ``{"kind": "BatchNorm1d", "h_mean", "h_var",
+    "r_mean", "r_var", "eps"}``.
+    """
+    hr = np.asarray(hr)
+    h = np.take(np.asarray(E), hr[:, 0], axis=0).astype(dtype)
+    r = np.take(np.asarray(R), hr[:, 1], axis=0).astype(dtype)
+    if norm is not None:
+        eps = norm.get("eps", 1e-5)
+        if norm["kind"] == "LayerNorm":
+            h = layer_norm(h, norm["h_weight"], norm["h_bias"], eps).astype(dtype)
+            r = layer_norm(r, norm["r_weight"], norm["r_bias"], eps).astype(dtype)
+        elif norm["kind"] == "BatchNorm1d":
+            h = batch_norm_eval(h, norm["h_mean"], norm["h_var"], eps).astype(dtype)
+            r = batch_norm_eval(r, norm["r_mean"], norm["r_var"], eps).astype(dtype)
+        else:
+            raise NotImplementedError(norm["kind"])
+    return h, r
+
+
+# --------------------------------------------------------------------------
+# M1 DistMult   dicee/models/real.py:19-36
+# --------------------------------------------------------------------------
+
+
+def distmult_query(h, r):
+    return h * r
+
+
+def distmult_scores_ref_form(h, r, E):
+    """``mm(h*r, E^T)`` (real.py:32)."""
+    return (h * r) @ np.asarray(E, dtype=h.dtype).T
+
+
+# --------------------------------------------------------------------------
+# M2 ComplEx   dicee/models/complex.py:240-269
+# --------------------------------------------------------------------------
+
+
+def complex_query(h, r):
+    """Single-GEMM form: Q = [hr*rr - hi*ri | hr*ri + hi*rr]."""
+    d2 = h.shape[1] // 2
+    hr_, hi_ = h[:, :d2], h[:, d2:]
+    rr_, ri_ = r[:, :d2], r[:, d2:]
+    return np.concatenate([hr_ * rr_ - hi_ * ri_, hr_ * ri_ + hi_ * rr_], axis=1)
+
+
+def complex_scores_ref_form(h, r, E):
+    """The four ``torch.mm`` of complex.py:260-264, in that order."""
+    E = np.asarray(E, dtype=h.dtype)
+    d2 = h.shape[1] // 2
+    hr_, hi_ = h[:, :d2], h[:, d2:]
+    rr_, ri_ = r[:, :d2], r[:, d2:]
+    tr, ti = E[:, :d2].T, E[:, d2:].T
+    return (hr_ * rr_) @ tr + (hr_ * ri_) @ ti + (hi_ * rr_) @ ti - (hi_ * ri_) @ tr
+
+
+# --------------------------------------------------------------------------
+# M3-M5 QMult   dicee/models/quaternion.py:74-100,124-171; static_funcs.py:4-18
+# --------------------------------------------------------------------------
+
+
+def quaternion_normalize(x, eps=1e-12):
+    """``F.normalize(x.view(B, d/4, 4), p=2, dim=-1)`` (quaternion.py:97-100).
+
+    Groups are 4 *consecutive* elements; each is divided by ``max(||g||, eps)``.
+    """
+    B, d = x.shape
+    g = x.reshape(B, d // 4, 4)
+    n = np.sqrt((g * g).sum(axis=-1, keepdims=True))
+    return (g / np.maximum(n, eps)).reshape(B, d)
+
+
+def hamilton_product_blocks(h, r):
+    """``quaternion_mul`` on block-split parts (static_funcs.py:13-17)."""
+    d4 = h.shape[1] // 4
+    a, b, c, d_ = (h[:, i * d4:(i + 1) * d4] for i in range(4))
+    p, q, u, v = (r[:, i * d4:(i + 1) * d4] for i in range(4))
+    r_val = a * p - b * q - c * u - d_ * v
+    i_val = a * q + b * p + c * v - d_ * u
+    j_val = a * u - b * v + c * p + d_ * q
+    k_val = a * v + b * u - c * q + d_ * p
+    return r_val, i_val, j_val, k_val
+
+
+def qmult_query(h, r, normalize_relation=True):
+    """Single-GEMM form: Q = [r_val | i_val | j_val | k_val].
+
+    ``normalize_relation`` is True when the model's
+    ``normalize_relation_embeddings`` is the IdentityClass (quaternion.py:138-139).
+    """
+    if normalize_relation:
+        r = quaternion_normalize(r)
+    return np.concatenate(hamilton_product_blocks(h, r), axis=1)
+
+
+def qmult_scores_ref_form(h, r, E, normalize_relation=True):
+    """The four ``torch.mm`` of quaternion.py:152-156."""
+    E = np.asarray(E, dtype=h.dtype)
+    if normalize_relation:
+        r = quaternion_normalize(r)
+    d4 = h.shape[1] // 4
+    parts = hamilton_product_blocks(h, r)
+    out = 0
+    for i, part in enumerate(parts):
+        out = out + part @ E[:, i * d4:(i + 1) * d4].T
+    return out
+
+
+# --------------------------------------------------------------------------
+# M6-M9 Keci   dicee/models/clifford.py:4-28,105-113,162-192,258-305
+# --------------------------------------------------------------------------
+
+
+def keci_split(x, r, p, q):
+    """``construct_cl_multivector`` (clifford.py:162-192): a0 [B,r], ap [B,r,p], aq [B,r,q]."""
+    B = x.shape[0]
+    a0 = x[:, :r]
+    ap = x[:, r:r + r * p].reshape(B, r, p)
+    aq = x[:, r + r * p:r + r * p + r * q].reshape(B, r, q)
+    return a0, ap, aq
+
+
+def keci_query(h, r_emb, p, q, coeff_p=None, coeff_q=None):
+    """Single-GEMM form of ``Keci.k_vs_all_score``: returns (Q [B,d], bias [B]).
+
+    Q[:, :r]               = h0 r0 + sum_i hp_i rp_i - sum_j hq_j rq_j
+    Q[:, r + rho*p + i]    = h0[rho] rp[rho,i] + hp[rho,i] r0[rho]
+    Q[:, r+r*p + rho*q+j]  = h0[rho] rq[rho,j] + hq[rho,j] r0[rho]
+    bias = sigma_pp (p>=2) + sigma_qq (q>=2) + sigma_pq (p>=2 and q>=2).
+    Both h and r parts are scaled by the coefficients (clifford.py:105-113).
+    """
+    B, d = h.shape
+    assert d % (p + q + 1) == 0
+    r = d // (p + q + 1)
+    h0, hp, hq = keci_split(h, r, p, q)
+    r0, rp, rq = keci_split(r_emb, r, p, q)
+    if p > 0:
+        cp = np.asarray(coeff_p, dtype=h.dtype).reshape(1, 1, p)
+        hp, rp = hp * cp, rp * cp
+    if q > 0:
+        cq = np.asarray(coeff_q, dtype=h.dtype).reshape(1, 1, q)
+        hq, rq = hq * cq, rq * cq
+    q0 = h0 * r0 + (hp * rp).sum(axis=2) - (hq * rq).sum(axis=2)
+    qp = h0[:, :, None] * rp + hp * r0[:, :, None]
+    qq = h0[:, :, None] * rq + hq * r0[:, :, None]
+    Q = np.concatenate([q0, qp.reshape(B, r * p), qq.reshape(B, r * q)], axis=1)
+    bias = np.zeros(B, dtype=h.dtype)
+    if p >= 2:
+        for i in range(p - 1):
+            for k in range(i + 1, p):
+                bias += (hp[:, :, i] * rp[:, :, k] - hp[:, :, k] * rp[:, :, i]).sum(axis=1)
+    if q >= 2:
+        for j in range(q - 1):
+            for k in range(j + 1, q):
+                bias += (hq[:, :, j] * rq[:, :, k] - hq[:, :, k] * rq[:, :, j]).sum(axis=1)
+    if p >= 2 and q >= 2:
+        for i in range(p):
+            for j in range(q):
+                bias += (hp[:, :, i] * rq[:, :, j] - hq[:, :, j] * rp[:, :, i]).sum(axis=1)
+    return Q, bias
+
+
+def keci_scores_ref_form(h, r_emb, E, p, q, coeff_p=None, coeff_q=None):
+    """The einsum sequence of clifford.py:258-305, term by term."""
+    E = np.asarray(E, dtype=h.dtype)
+    B, d = h.shape
+    N = E.shape[0]
+    r = d // (p + q + 1)
+    h0, hp, hq = keci_split(h, r, p, q)
+    r0, rp, rq = keci_split(r_emb, r, p, q)
+    if p > 0:
+        cp = np.asarray(coeff_p, dtype=h.dtype).reshape(1, 1, p)
+        hp, rp = hp * cp, rp * cp
+    if q > 0:
+        cq = np.asarray(coeff_q, dtype=h.dtype).reshape(1, 1, q)
+        hq, rq = hq * cq, rq * cq
+    t0 = E[:, :r]
+    out = np.einsum("br,er->be", h0 * r0, t0)
+    if p > 0:
+        tp = E[:, r:r + r * p].reshape(N, r, p)
+        out = out + np.einsum("brp,er->be", hp * rp, t0) \
+            + np.einsum("brp,erp->be", h0[:, :, None] * rp, tp) \
+            + np.einsum("brp,erp->be", hp * r0[:, :, None], tp)
+    if q > 0:
+        tq = E[:, d - r * q:].reshape(N, r, q)
+        out = out + np.einsum("brq,erq->be", h0[:, :, None] * rq, tq) \
+            + np.einsum("brq,erq->be", hq * r0[:, :, None], tq) \
+            - np.einsum("brq,er->be", hq * rq, t0)
+    if p >= 2:
+        iu = np.triu_indices(p, k=1)
+        spp = np.einsum("nrp,nrx->nrpx", hp, rp) - np.einsum("nrx,nrp->nrpx", hp, rp)
+        out = out + spp[:, :, iu[0], iu[1]].sum(axis=(1, 2))[:, None]
+    if q >= 2:
+        iu = np.triu_indices(q, k=1)
+        sqq = np.einsum("nrp,nrx->nrpx", hq, rq) - np.einsum("nrx,nrp->nrpx", hq, rq)
+        out = out + sqq[:, :, iu[0], iu[1]].sum(axis=(1, 2))[:, None]
+    if p >= 2 and q >= 2:
+        spq = np.einsum("nrp,nrq->nrpq", hp, rq) - np.einsum("nrq,nrp->nrpq", hq, rp)
+        out = out + spq.sum(axis=(1, 2, 3))[:, None]
+    return out
+
+
+# --------------------------------------------------------------------------
+# model dispatch
+# --------------------------------------------------------------------------
+
+
+def build_query(model, E, R, hr, p=0, q=0, coeff_p=None, coeff_q=None,
+                normalize_relation=True, norm=None, dtype=np.float64):
+    """(Q [B,d], bias [B]) such that ``scores = Q @ E.T + bias[:, None]``."""
+    h, r = gather_hr(E, R, hr, norm=norm, dtype=dtype)
+    if model == "DistMult":
+        return distmult_query(h, r), np.zeros(len(h), dtype)
+    if model == "ComplEx":
+        return complex_query(h, r), np.zeros(len(h), dtype)
+    if model == "QMult":
+        return qmult_query(h, r, normalize_relation), np.zeros(len(h), dtype)
+    if model in ("Keci", "CKeci"):
+        return keci_query(h, r, p, q, coeff_p, coeff_q)
+    raise ValueError(model)
+
+
+def k_vs_all_scores(model, E, R, hr, **kw):
+    """``forward_k_vs_all``: [B,N] scores via the single-GEMM form."""
+    dtype = kw.get("dtype", np.float64)
+    Q, bias = build_query(model, E, R, hr, **kw)
+    return Q @ np.asarray(E, dtype=dtype).T + bias[:, None]
+
+
+def k_vs_all_scores_ref_form(model, E, R, hr, p=0, q=0, coeff_p=None, coeff_q=None,
+                             normalize_relation=True, norm=None, dtype=np.float64):
+    """``forward_k_vs_all`` via the reference's own multi-mm / einsum decomposition."""
+    h, r = gather_hr(E, R, hr, norm=norm, dtype=dtype)
+    if model == "DistMult":
+        return distmult_scores_ref_form(h, r, E)
+    if model == "ComplEx":
+        return complex_scores_ref_form(h, r, E)
+    if model == "QMult":
+        return qmult_scores_ref_form(h, r, E, normalize_relation)
+    if model in ("Keci", "CKeci"):
+        return keci_scores_ref_form(h, r, E, p, q, coeff_p, coeff_q)
+    raise ValueError(model)
+
+
+# --------------------------------------------------------------------------
+# R1: filtered rank   dicee/evaluation/evaluator.py:473-510
+# --------------------------------------------------------------------------
+
+
+def filtered_rank_counts(scores_row, target, filt):
+    """Closed form of the reference's mask + sort + where for one row.
+
+    Returns (G, T, TL): over entities not removed by the filter (the target is
+    always kept, evaluator.py:494-501), ``G`` scores strictly greater than the
+    target's, ``T`` other entities tying with it, ``TL`` of those with a lower
+    index.  The reference's rank lies in ``[1+G, 1+G+T]``; a stable descending
+    sort gives ``1+G+TL``.
+    """
+    s = np.asarray(scores_row)
+    N = s.shape[0]
+    keep = np.ones(N, dtype=bool)
+    if filt is not None and len(filt):
+        keep[np.asarray(filt, dtype=np.int64)] = False
+    keep[target] = True
+    st = s[target]
+    G = int(np.count_nonzero(keep & (s > st)))
+    eq = keep & (s == st)
+    eq[target] = False
+    T = int(np.count_nonzero(eq))
+    TL = int(np.count_nonzero(eq[:target]))
+    return G, T, TL
+
+
+def filtered_rank_bruteforce(scores_row, target, filt):
+    """The reference's literal procedure with a *stable* descending sort."""
+    s = np.array(scores_row, dtype=np.float64, copy=True)
+    tv = s[target]
+    if filt is not None and len(filt):
+        s[np.asarray(filt, dtype=np.int64)] = -np.inf
+    s[target] = tv
+    order = np.argsort(-s, kind="stable")
+    return int(np.where(order == target)[0][0]) + 1
+
+
+def filtered_ranks(scores, targets, filters, tie="stable"):
+    """Ranks for a batch. ``filters[j]`` is a sequence of entity ids (or None)."""
+    out = np.empty(len(targets), dtype=np.int64)
+    for j, t in enumerate(targets):
+        G, T, TL = filtered_rank_counts(scores[j], int(t), filters[j])
+        out[j] = 1 + G + {"stable": TL, "optimistic": 0, "pessimistic": T}[tie]
+    return out
+
+
+def rank_interval_with_tolerance(scores_row, target, filt, tol):
+    """[lo, hi] of ranks admissible when scores are only known to ``+-tol``."""
+    s = np.asarray(scores_row, dtype=np.float64)
+    keep = np.ones(s.shape[0], dtype=bool)
+    if filt is not None and len(filt):
+        keep[np.asarray(filt, dtype=np.int64)] = False
+    keep[target] = False
+    st = s[target]
+    lo = 1 + int(np.count_nonzero(keep & (s > st + tol)))
+    hi = 1 + int(np.count_nonzero(keep & (s >= st - tol)))
+    return lo, hi
+
+
+# --------------------------------------------------------------------------
+# U1: metrics   dicee/evaluation/utils.py:73-118
+# --------------------------------------------------------------------------
+
+
+def metrics_from_ranks(ranks):
+    ranks = np.asarray(ranks)
+    n = len(ranks)
+    return {
+        "H@1": float(np.count_nonzero(ranks <= 1)) / n,
+        "H@3": float(np.count_nonzero(ranks <= 3)) / n,
+        "H@10": float(np.count_nonzero(ranks <= 10)) / n,
+        "MRR": np.mean(1.0 / np.array(ranks)),
+    }
+
+
+# --------------------------------------------------------------------------
+# K1/K2: top-k   dicee/knowledge_graph_embeddings.py:397-401,568
+# --------------------------------------------------------------------------
+
+
+def topk(scores, k):
+    """Descending top-k per row; ties broken towards the lower index."""
+    s = np.asarray(scores)
+    order = np.argsort(-s, axis=1, kind="stable")[:, :k]
+    return np.take_along_axis(s, order, axis=1), order
+
+
+def sigmoid(x):
+    x = np.asarray(x, dtype=np.float64)
+    return 1.0 / (1.0 + np.exp(-x))
+
+
+# --------------------------------------------------------------------------
+# L1: multi-hot BCE   base_model.py:138; dataset_classes.py:354-361
+# --------------------------------------------------------------------------
+
+
+def softplus(x):
+    x = np.asarray(x, dtype=np.float64)
+    return np.maximum(x, 0.0) + np.log1p(np.exp(-np.abs(x)))
+
+
+def bce_multihot(scores, positives, label_smoothing=0.0):
+    """``BCEWithLogitsLoss()(scores, y)`` (mean over B*N) with ``y`` the multi-hot
+    of ``positives[b]`` and the KvsAll smoothing ``y*(1-eps) + 1/N`` applied only
+    when ``eps`` is non-zero (dataset_classes.py:359-360)."""
+    s = np.asarray(scores, dtype=np.float64)
+    B, N = s.shape
+    total = softplus(s).sum()
+    pos_sum = 0.0
+    for b in range(B):
+        idx = np.unique(np.asarray(positives[b], dtype=np.int64))
+        pos_sum += s[b, idx].sum()
+    if label_smoothing:
+        total -= (1.0 - label_smoothing) * pos_sum + s.sum() / N
+    else:
+        total -= pos_sum
+    return total / (B * N)
+
+
+def dense_multihot(positives, N, label_smoothing=0.0, dtype=np.float32):
+    y = np.zeros((len(positives), N), dtype=dtype)
+    for b, idx in enumerate(positives):
+        y[b, np.asarray(idx, dtype=np.int64)] = 1.0
+    if label_smoothing:
+        y = y * (1 - label_smoothing) + 1.0 / N
+    return y

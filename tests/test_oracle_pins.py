@@ -1,0 +1,385 @@
+"""Independent checks that pin the CPU oracle (no GPU, no reference import).
+
+Each test compares an oracle function with something that does not share its
+formula: a brute-force loop, a textbook/library routine, a different algebraic
+representation (complex128, a structure-constant table, a bitmask geometric
+algebra), a hand-computed fixture under ``tests/golden``, or an invariant.
+"""
+import itertools
+import json
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import kge_oracle as ko
+from oracle import torch_cpu_path as tcp
+
+GOLD = os.path.join(os.path.dirname(__file__), "golden")
+
+
+def _tables(rng, N, R, d, sd=0.1):
+    return rng.normal(0, sd, (N, d)), rng.normal(0, sd, (R, d))
+
+
+def _hr(rng, N, R, B):
+    return np.stack([rng.integers(0, N, B), rng.integers(0, R, B)], axis=1)
+
+
+# ------------------------------------------------------------------ DistMult
+def test_distmult_bruteforce():
+    rng = np.random.default_rng(0)
+    E, R = _tables(rng, 7, 3, 6)
+    hr = _hr(rng, 7, 3, 5)
+    S = ko.k_vs_all_scores("DistMult", E, R, hr)
+    for b, (h, r) in enumerate(hr):
+        for e in range(7):
+            acc = 0.0
+            for k in range(6):
+                acc += E[h, k] * R[r, k] * E[e, k]
+            assert S[b, e] == pytest.approx(acc, rel=1e-12, abs=1e-15)
+
+
+# ------------------------------------------------------------------- ComplEx
+def test_complex_vs_complex128_hermitian_product():
+    rng = np.random.default_rng(1)
+    N, Rn, d = 11, 4, 10
+    E, R = _tables(rng, N, Rn, d)
+    hr = _hr(rng, N, Rn, 6)
+    S = ko.k_vs_all_scores("ComplEx", E, R, hr)
+    Ec = E[:, :d // 2] + 1j * E[:, d // 2:]
+    Rc = R[:, :d // 2] + 1j * R[:, d // 2:]
+    ref = np.real((Ec[hr[:, 0]] * Rc[hr[:, 1]]) @ np.conj(Ec).T)
+    np.testing.assert_allclose(S, ref, rtol=1e-12, atol=1e-15)
+    # the reference's 4-mm decomposition agrees with the single-GEMM form
+    np.testing.assert_allclose(ko.k_vs_all_scores_ref_form("ComplEx", E, R, hr), S, rtol=1e-12, atol=1e-15)
+
+
+def test_complex_sign_of_each_term():
+    # one-hot probes: a wrong sign or swapped half flips exactly one of these
+    d = 2
+    E = np.array([[1.0, 0.0], [0.0, 1.0]])      # e0 = 1, e1 = i
+    R = np.array([[1.0, 0.0], [0.0, 1.0]])      # r0 = 1, r1 = i
+    hr = np.array([[0, 0], [0, 1], [1, 0], [1, 1]])
+    S = ko.k_vs_all_scores("ComplEx", E, R, hr)
+    # Re(h r conj(t)):  (1*1)->[1,0]; (1*i)=i->[0,1]; (i*1)=i->[0,1]; (i*i)=-1->[-1,0]
+    np.testing.assert_array_equal(S, np.array([[1, 0], [0, 1], [0, 1], [-1, 0]], dtype=float))
+
+
+# --------------------------------------------------------------------- QMult
+def _structure_constants():
+    """T[i,j,k] with e_i e_j = sum_k T[i,j,k] e_k for (1,i,j,k), built from the
+    defining relations i^2=j^2=k^2=ijk=-1 by closure, not from the product formula."""
+    T = np.zeros((4, 4, 4))
+    for a in range(4):
+        T[0, a, a] = 1
+        T[a, 0, a] = 1
+    for a in (1, 2, 3):
+        T[a, a, 0] = -1
+    for a, b, c in ((1, 2, 3), (2, 3, 1), (3, 1, 2)):   # ij=k, jk=i, ki=j
+        T[a, b, c] = 1
+        T[b, a, c] = -1
+    return T
+
+
+def test_hamilton_product_vs_structure_constants_and_scipy():
+    from scipy.spatial.transform import Rotation
+    rng = np.random.default_rng(2)
+    B, d4 = 5, 3
+    h = rng.normal(size=(B, 4 * d4))
+    r = rng.normal(size=(B, 4 * d4))
+    parts = ko.hamilton_product_blocks(h, r)
+    T = _structure_constants()
+    hq = h.reshape(B, 4, d4)
+    rq = r.reshape(B, 4, d4)
+    ref = np.einsum("bin,bjn,ijk->bkn", hq, rq, T)
+    for k in range(4):
+        np.testing.assert_allclose(parts[k], ref[:, k, :], rtol=1e-12, atol=1e-14)
+    # library cross-check on unit quaternions (scipy stores scalar last)
+    a = rng.normal(size=4)
+    a /= np.linalg.norm(a)
+    b = rng.normal(size=4)
+    b /= np.linalg.norm(b)
+    prod = (Rotation.from_quat(np.r_[a[1:], a[0]]) * Rotation.from_quat(np.r_[b[1:], b[0]])).as_quat()
+    mine = np.array([p[0, 0] for p in ko.hamilton_product_blocks(a[None, :], b[None, :])])
+    mine_sl = np.r_[mine[1:], mine[0]]
+    assert np.allclose(mine_sl, prod, atol=1e-12) or np.allclose(mine_sl, -prod, atol=1e-12)
+
+
+def test_quaternion_normalizer_groups_and_eps():
+    rng = np.random.default_rng(3)
+    x = rng.normal(size=(4, 16))
+    x[0, 4:8] = 0.0
+    y = ko.quaternion_normalize(x)
+    norms = np.linalg.norm(y.reshape(4, 4, 4), axis=-1)
+    np.testing.assert_allclose(norms[1:], 1.0, rtol=1e-12)
+    assert norms[0, 1] == 0.0 and np.all(y[0, 4:8] == 0.0)
+    # library routine
+    ref = torch.nn.functional.normalize(torch.tensor(x).view(4, 4, 4), p=2, dim=-1).view(4, 16).numpy()
+    np.testing.assert_allclose(y, ref, rtol=1e-12, atol=0)
+
+
+def test_qmult_block_vs_consecutive_quirk_fixture():
+    """d=8: normalisation groups are (0..3),(4..7) but the Hamilton product pairs
+    elements (g, g+2, g+4, g+6).  Expected values were computed by hand."""
+    with open(os.path.join(GOLD, "qmult_d8_quirk.json")) as f:
+        fx = json.load(f)
+    E = np.array(fx["E"])
+    R = np.array(fx["R"])
+    hr = np.array(fx["hr"])
+    S = ko.k_vs_all_scores("QMult", E, R, hr)
+    np.testing.assert_allclose(S, np.array(fx["scores"]), rtol=1e-12, atol=1e-12)
+    np.testing.assert_allclose(ko.k_vs_all_scores_ref_form("QMult", E, R, hr), S, rtol=1e-12, atol=1e-14)
+
+
+def test_qmult_single_gemm_identity():
+    rng = np.random.default_rng(4)
+    E, R = _tables(rng, 9, 3, 16)
+    hr = _hr(rng, 9, 3, 7)
+    a = ko.k_vs_all_scores("QMult", E, R, hr)
+    b = ko.k_vs_all_scores_ref_form("QMult", E, R, hr)
+    np.testing.assert_allclose(a, b, rtol=1e-11, atol=1e-14)
+    c = ko.k_vs_all_scores("QMult", E, R, hr, normalize_relation=False)
+    assert not np.allclose(a, c)
+
+
+# ---------------------------------------------------------------------- Keci
+class _GA:
+    """Geometric algebra Cl(p,q) on bitmask blades; e_i^2=+1 for i<p, -1 for p<=i<p+q."""
+
+    def __init__(self, p, q):
+        self.p, self.q, self.n = p, q, p + q
+
+    def blade_mul(self, a, b):
+        sign = 1
+        t = a >> 1
+        while t:                      # count swaps to reorder
+            if bin(t & b).count("1") & 1:
+                sign = -sign
+            t >>= 1
+        common = a & b
+        for i in range(self.n):
+            if common >> i & 1 and i >= self.p:
+                sign = -sign
+        return a ^ b, sign
+
+    def mul(self, x, y):
+        out = {}
+        for a, va in x.items():
+            for b, vb in y.items():
+                c, s = self.blade_mul(a, b)
+                out[c] = out.get(c, 0.0) + s * va * vb
+        return out
+
+
+def _keci_bruteforce(E, R, hr, p, q, cp, cq):
+    """score = <grade0,1 of (h r), t> + sum of grade-2 coefficients (with the
+    reference's thresholds: pp needs p>=2, qq needs q>=2, pq needs both)."""
+    N, d = E.shape
+    r = d // (p + q + 1)
+    ga = _GA(p, q)
+
+    def mv(x, rho):
+        m = {0: x[rho]}
+        for i in range(p):
+            m[1 << i] = x[r + rho * p + i] * cp[i]
+        for j in range(q):
+            m[1 << (p + j)] = x[r + r * p + rho * q + j] * cq[j]
+        return m
+
+    S = np.zeros((len(hr), N))
+    for b, (hi, ri) in enumerate(hr):
+        for rho in range(r):
+            prod = ga.mul(mv(E[hi], rho), mv(R[ri], rho))
+            g2 = 0.0
+            for blade, v in prod.items():
+                bits = [i for i in range(p + q) if blade >> i & 1]
+                if len(bits) != 2:
+                    continue
+                in_p = [i < p for i in bits]
+                if all(in_p):
+                    g2 += v if p >= 2 else 0.0
+                elif not any(in_p):
+                    g2 += v if q >= 2 else 0.0
+                else:
+                    g2 += v if (p >= 2 and q >= 2) else 0.0
+            for e in range(N):
+                t = E[e]
+                s = prod.get(0, 0.0) * t[rho]
+                for i in range(p):
+                    s += prod.get(1 << i, 0.0) * t[r + rho * p + i]
+                for j in range(q):
+                    s += prod.get(1 << (p + j), 0.0) * t[r + r * p + rho * q + j]
+                S[b, e] += s + g2
+    return S
+
+
+@pytest.mark.parametrize("p,q", [(0, 0), (0, 1), (1, 0), (1, 1), (2, 0), (0, 2), (2, 2), (3, 2), (1, 3)])
+def test_keci_vs_geometric_algebra(p, q):
+    rng = np.random.default_rng(10 * p + q)
+    r = 3
+    d = r * (p + q + 1)
+    E, R = _tables(rng, 6, 3, d, sd=1.0)
+    hr = _hr(rng, 6, 3, 4)
+    cp = rng.normal(size=p)
+    cq = rng.normal(size=q)
+    S = ko.k_vs_all_scores("Keci", E, R, hr, p=p, q=q, coeff_p=cp, coeff_q=cq)
+    ref = _keci_bruteforce(E, R, hr, p, q, cp, cq)
+    np.testing.assert_allclose(S, ref, rtol=1e-10, atol=1e-12)
+    np.testing.assert_allclose(
+        ko.k_vs_all_scores_ref_form("Keci", E, R, hr, p=p, q=q, coeff_p=cp, coeff_q=cq), S, rtol=1e-10, atol=1e-12)
+
+
+def test_keci_reductions():
+    rng = np.random.default_rng(5)
+    E, R = _tables(rng, 8, 3, 12)
+    hr = _hr(rng, 8, 3, 5)
+    # (0,0) is DistMult
+    np.testing.assert_allclose(ko.k_vs_all_scores("Keci", E, R, hr, p=0, q=0),
+                               ko.k_vs_all_scores("DistMult", E, R, hr), rtol=1e-13)
+    # (0,1) with c_q=1 is ComplEx
+    np.testing.assert_allclose(ko.k_vs_all_scores("Keci", E, R, hr, p=0, q=1, coeff_q=[1.0]),
+                               ko.k_vs_all_scores("ComplEx", E, R, hr), rtol=1e-12, atol=1e-15)
+    # (0,1) with c_q=0 (the reference's initial value) is DistMult on the first half
+    half = ko.k_vs_all_scores("DistMult", E[:, :6], R[:, :6], hr)
+    np.testing.assert_allclose(ko.k_vs_all_scores("Keci", E, R, hr, p=0, q=1, coeff_q=[0.0]), half,
+                               rtol=1e-13, atol=1e-16)
+
+
+def test_keci_sigma_thresholds_fixture():
+    """p=q=1: the e_p e_q bivector term is dropped; p=q=2: it is added."""
+    with open(os.path.join(GOLD, "keci_thresholds.json")) as f:
+        fx = json.load(f)
+    for case in fx["cases"]:
+        E = np.array(case["E"])
+        R = np.array(case["R"])
+        Q, bias = ko.build_query("Keci", E, R, np.array(case["hr"]), p=case["p"], q=case["q"],
+                                 coeff_p=case["cp"], coeff_q=case["cq"])
+        np.testing.assert_allclose(bias, case["bias"], rtol=1e-12, atol=1e-12)
+        np.testing.assert_allclose(Q, case["Q"], rtol=1e-12, atol=1e-12)
+
+
+# --------------------------------------------------------- torch-CPU op port
+@pytest.mark.parametrize("model,d,kw", [
+    ("DistMult", 8, {}), ("ComplEx", 8, {}), ("QMult", 8, {}),
+    ("Keci", 12, dict(p=1, q=2, coeff_p=[0.7], coeff_q=[1.3, -0.4])),
+    ("Keci", 15, dict(p=2, q=2, coeff_p=[0.7, 0.2], coeff_q=[1.3, -0.4])),
+])
+def test_torch_port_matches_numpy_oracle(model, d, kw):
+    rng = np.random.default_rng(6)
+    E, R = _tables(rng, 13, 4, d, sd=1.0)
+    hr = _hr(rng, 13, 4, 6)
+    want = ko.k_vs_all_scores(model, E, R, hr, **kw)
+    tkw = dict(kw)
+    for key in ("coeff_p", "coeff_q"):
+        if key in tkw:
+            tkw[key] = torch.tensor(tkw[key], dtype=torch.float64)
+    got = tcp.forward_k_vs_all(model, torch.tensor(E), torch.tensor(R), torch.tensor(hr), **tkw).numpy()
+    np.testing.assert_allclose(got, want, rtol=1e-10, atol=1e-12)
+
+
+# -------------------------------------------------------------- norm layers
+def test_layernorm_batchnorm_vs_torch():
+    rng = np.random.default_rng(7)
+    x = rng.normal(size=(5, 12))
+    w, b = rng.normal(size=12), rng.normal(size=12)
+    ref = torch.nn.functional.layer_norm(torch.tensor(x), (12,), torch.tensor(w), torch.tensor(b), 1e-5).numpy()
+    np.testing.assert_allclose(ko.layer_norm(x, w, b), ref, rtol=1e-12, atol=1e-13)
+    m, v = rng.normal(size=12), rng.uniform(0.5, 2, size=12)
+    ref = torch.nn.functional.batch_norm(torch.tensor(x), torch.tensor(m), torch.tensor(v), training=False,
+                                         eps=1e-5).numpy()
+    np.testing.assert_allclose(ko.batch_norm_eval(x, m, v), ref, rtol=1e-12, atol=1e-13)
+
+
+# ----------------------------------------------------------------- ranking
+def test_rank_counts_vs_bruteforce_and_invariants():
+    rng = np.random.default_rng(8)
+    N = 40
+    for trial in range(200):
+        s = rng.integers(-3, 4, N).astype(np.float64)        # many exact ties
+        t = int(rng.integers(0, N))
+        filt = list(rng.integers(0, N, rng.integers(0, 12)))
+        if trial % 2:
+            filt.append(t)                                   # target listed in its own filter
+        G, T, TL = ko.filtered_rank_counts(s, t, filt)
+        assert 1 + G + TL == ko.filtered_rank_bruteforce(s, t, filt)
+        # duplicates in the filter are idempotent
+        assert (G, T, TL) == ko.filtered_rank_counts(s, t, filt + filt)
+        # torch's unstable sort lands inside [lo, hi]
+        sm = torch.tensor(s).clone()
+        if filt:
+            sm[torch.tensor(filt)] = -np.inf
+        sm[t] = s[t]
+        _, order = torch.sort(sm[None, :], dim=1, descending=True)
+        pos = int(torch.where(order[0] == t)[0].item()) + 1
+        assert 1 + G <= pos <= 1 + G + T
+    # empty filter: plain rank
+    s = np.array([0.1, 0.5, 0.3, 0.5])
+    assert ko.filtered_rank_counts(s, 2, []) == (2, 0, 0)
+    assert ko.filtered_rank_counts(s, 3, None) == (0, 1, 1)
+    # -inf never outranks a finite target
+    assert ko.filtered_rank_counts(np.array([-np.inf, 0.0, -np.inf]), 1, []) == (0, 0, 0)
+
+
+def test_evaluator_port_matches_closed_form_without_ties():
+    rng = np.random.default_rng(9)
+    N, Rn, d = 50, 5, 8
+    E, R = _tables(rng, N, Rn, d, sd=1.0)
+    triples = np.stack([rng.integers(0, N, 64), rng.integers(0, Rn, 64), rng.integers(0, N, 64)], axis=1)
+    er = {}
+    for h, r, t in triples:
+        er.setdefault((int(h), int(r)), []).append(int(t))
+    ranks = tcp.evaluate_entity_prediction("ComplEx", torch.tensor(E), torch.tensor(R), triples, er, 16)
+    S = ko.k_vs_all_scores("ComplEx", E, R, triples[:, :2])
+    want = ko.filtered_ranks(S, triples[:, 2], [er[(int(h), int(r))] for h, r, _ in triples])
+    assert ranks == list(want)
+    m = ko.metrics_from_ranks(ranks)
+    assert m["MRR"] == pytest.approx(sum(1.0 / r for r in ranks) / len(ranks))
+    assert m["H@3"] == sum(r <= 3 for r in ranks) / len(ranks)
+
+
+# -------------------------------------------------------------- top-k, BCE
+def test_topk_vs_bruteforce_and_torch():
+    rng = np.random.default_rng(11)
+    s = rng.normal(size=(6, 30))
+    v, idx = ko.topk(s, 5)
+    tv, tidx = torch.topk(torch.tensor(s), 5, dim=1)
+    np.testing.assert_array_equal(idx, tidx.numpy())
+    np.testing.assert_array_equal(v, tv.numpy())
+    for b in range(6):
+        assert list(idx[b]) == sorted(range(30), key=lambda e: (-s[b, e], e))[:5]
+    np.testing.assert_allclose(ko.sigmoid(v), torch.sigmoid(tv).numpy(), rtol=1e-14)
+
+
+@pytest.mark.parametrize("eps", [0.0, 0.1])
+def test_bce_multihot_vs_torch_dense(eps):
+    rng = np.random.default_rng(12)
+    B, N = 7, 23
+    s = rng.normal(0, 3, (B, N))
+    pos = [list(rng.integers(0, N, rng.integers(0, 6))) for _ in range(B)]
+    y = ko.dense_multihot(pos, N, eps, dtype=np.float64)
+    ref = torch.nn.functional.binary_cross_entropy_with_logits(torch.tensor(s), torch.tensor(y)).item()
+    assert ko.bce_multihot(s, pos, eps) == pytest.approx(ref, rel=1e-12)
+
+
+# ------------------------------------------------------------ bf16 / int8
+def test_bf16_round_vs_torch():
+    rng = np.random.default_rng(13)
+    x = np.concatenate([rng.normal(0, 1, 5000), rng.normal(0, 1e-20, 100), [0.0, -0.0, 1.0, 3.3895314e38]])
+    x = x.astype(np.float32)
+    ref = torch.tensor(x).to(torch.bfloat16).to(torch.float32).numpy()
+    np.testing.assert_array_equal(ko.bf16_round(x), ref)
+    np.testing.assert_array_equal(ko.bf16_from_bits(ko.bf16_bits(x)), ref)
+
+
+def test_int8_rows_closed_form():
+    rng = np.random.default_rng(14)
+    x = rng.normal(0, 0.1, (20, 16)).astype(np.float32)
+    x[3] = 0.0
+    q, s = ko.quantize_int8_rows(x)
+    assert q.dtype == np.int8 and np.abs(q).max() <= 127
+    assert np.all(np.abs(q[np.arange(20) != 3]).max(axis=1) == 127)
+    assert np.all(q[3] == 0) and s[3] == 0.0
+    err = np.abs(ko.dequantize_int8_rows(q, s) - x)
+    assert np.all(err <= 0.5 * s[:, None] * (1 + 1e-6))
