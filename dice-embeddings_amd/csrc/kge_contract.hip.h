@@ -1,0 +1,555 @@
+// Query x all-entity contraction on MFMA with fused epilogues (gfx950).
+//
+// Two main loops share one epilogue interface:
+//   qreg_kernel   bf16 MFMA (32x32x16), entity table bf16 or per-row int8, d <= 128.  Each wave keeps
+//                 the bf16 fragments of 128 queries in registers for the whole kernel and streams
+//                 64-row entity stages through a double-buffered, padded LDS panel.
+//   kloop_kernel  fp32 MFMA (32x32x2), any d.  Classic 128x128 workgroup tile, K staged through LDS
+//                 in chunks of 32.
+// Reduction order of one score is fixed (k ascending in steps of the MFMA depth, nothing else), so
+// every kernel that forms dot(Q[b], E[e]) with these helpers produces the same fp32 bit pattern.
+//
+// Orientation: by default the entity tile is the MFMA "A" operand (rows) and the query tile the "B"
+// operand (columns), so each lane owns ONE query per tile (column = lane % 32) and 16 entities:
+// per-query epilogue state (threshold, counters) lives in one register per lane.  Epilogues that
+// write scores set SWAP so that consecutive lanes hold consecutive entities (coalesced stores).
+#pragma once
+#include "kge_internal.h"
+
+namespace kge {
+
+struct ContractArgs {
+  const float* Q;
+  const void* E;
+  const float* scale;
+  int64_t B, N;
+  int64_t e_begin, e_end;  // entity rows scanned by this launch
+  int64_t n_chunks;
+  int d;
+  int chunk_rows;
+  int n_qgroups;
+};
+
+__device__ __forceinline__ f32x16 mfma_bf16(bf16x8 a, bf16x8 b, f32x16 c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+}
+__device__ __forceinline__ f32x16 mfma_f32(float a, float b, f32x16 c) {
+  return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0);
+}
+
+__device__ __forceinline__ bf16x8 cvt_bf16x8(f32x4 lo, f32x4 hi) {
+  bf16x8 r;
+  r[0] = (__bf16)lo[0]; r[1] = (__bf16)lo[1]; r[2] = (__bf16)lo[2]; r[3] = (__bf16)lo[3];
+  r[4] = (__bf16)hi[0]; r[5] = (__bf16)hi[1]; r[6] = (__bf16)hi[2]; r[7] = (__bf16)hi[3];
+  return r;
+}
+
+// two int8 (bytes `lo`,`hi` of w selected by shift) -> packed pair of bf16; exact for |v| <= 127
+__device__ __forceinline__ uint32_t i8x2_to_bf16x2(uint32_t w, int shift) {
+  float f0 = (float)(int)(int8_t)(w >> shift);
+  float f1 = (float)(int)(int8_t)(w >> (shift + 8));
+  return (__float_as_uint(f0) >> 16) | (__float_as_uint(f1) & 0xffff0000u);
+}
+__device__ __forceinline__ u32x4 i8x8_to_bf16x8(uint32_t w0, uint32_t w1) {
+  u32x4 r;
+  r[0] = i8x2_to_bf16x2(w0, 0);
+  r[1] = i8x2_to_bf16x2(w0, 16);
+  r[2] = i8x2_to_bf16x2(w1, 0);
+  r[3] = i8x2_to_bf16x2(w1, 16);
+  return r;
+}
+
+// XCD-aware decomposition of a flat workgroup id: hardware deals consecutive ids round-robin over
+// the 8 XCDs, so ids with the same (id % 8) share an L2.  Consecutive slots on one XCD walk the
+// query groups of ONE entity chunk, which keeps that chunk's rows hot in that XCD's L2.
+__device__ __forceinline__ bool decompose_wg(const ContractArgs& a, int& qg, int64_t& chunk) {
+  const int64_t wg = blockIdx.x;
+  const int xcd = (int)(wg & 7);
+  const int64_t slot = wg >> 3;
+  qg = (int)(slot % a.n_qgroups);
+  chunk = (slot / a.n_qgroups) * 8 + xcd;
+  return chunk < a.n_chunks;
+}
+
+// ============================================================================================
+// Epilogues.  tile<HAS_SCALE>(qt, acc, sc16, sc_col, e_base, limit): `acc` is one finished 32x32
+// tile; without SWAP acc[i] = score(entity e_base + row_of(i,hf), query of this lane in tile qt);
+// with SWAP acc[i] = score(query row_of(i,hf) of tile qt, entity e_base + c).  Entities >= limit
+// are padding.  sc16[i] / sc_col are the int8 row scales of the entities this lane holds.
+// ============================================================================================
+
+struct StoreArgs {
+  float* S;
+  const float* bias;
+  int64_t ldS;
+};
+template <int NQT>
+struct StoreEpi {
+  static constexpr bool SWAP = true;
+  using Args = StoreArgs;
+  Args a;
+  int64_t q0, B;
+  int c, hf;
+  __device__ void init(const Args& args, int64_t q0_, int c_, int hf_, int64_t B_) {
+    a = args; q0 = q0_; c = c_; hf = hf_; B = B_;
+  }
+  template <bool HAS_SCALE>
+  __device__ __forceinline__ void tile(int qt, const f32x16& acc, const float* sc16, float sc_col, int64_t e_base,
+                                       int64_t limit) {
+    const int64_t e = e_base + c;
+    if (e >= limit) return;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int64_t q = q0 + 32 * qt + row_of(i, hf);
+      if (q < B) {
+        float s = acc[i];
+        if (HAS_SCALE) s *= sc_col;
+        if (a.bias) s += a.bias[q];
+        a.S[q * a.ldS + e] = s;
+      }
+    }
+  }
+  __device__ void finish() {}
+};
+
+struct RankArgs {
+  const float* thr;  // raw target score per query
+  const int64_t* target;
+  int32_t* n_gt;
+  int32_t* n_eq;
+  int32_t* n_eql;
+};
+template <int NQT>
+struct RankEpi {
+  static constexpr bool SWAP = false;
+  using Args = RankArgs;
+  Args a;
+  float thr[NQT];
+  int32_t tgt[NQT];
+  int32_t gt[NQT], eq[NQT], eql[NQT];
+  int64_t q0, B;
+  int c, hf;
+  __device__ void init(const Args& args, int64_t q0_, int c_, int hf_, int64_t B_) {
+    a = args; q0 = q0_; c = c_; hf = hf_; B = B_;
+#pragma unroll
+    for (int t = 0; t < NQT; ++t) {
+      const int64_t q = q0 + 32 * t + c;
+      thr[t] = (q < B) ? a.thr[q] : __uint_as_float(0x7fc00000u);  // NaN never compares
+      tgt[t] = (q < B) ? (int32_t)a.target[q] : -1;
+      gt[t] = eq[t] = eql[t] = 0;
+    }
+  }
+  template <bool HAS_SCALE>
+  __device__ __forceinline__ void tile(int qt, const f32x16& acc, const float* sc16, float sc_col, int64_t e_base,
+                                       int64_t limit) {
+    const float th = thr[qt];
+    unsigned long long tie = 0;
+    int32_t g = 0;
+    if (e_base + 32 <= limit) {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        float s = acc[i];
+        if (HAS_SCALE) s *= sc16[i];
+        g += (s > th) ? 1 : 0;
+        tie |= __builtin_amdgcn_ballot_w64(s == th);
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        float s = acc[i];
+        if (HAS_SCALE) s *= sc16[i];
+        const bool ok = e_base + row_of(i, hf) < limit;
+        g += (ok && s > th) ? 1 : 0;
+        tie |= __builtin_amdgcn_ballot_w64(ok && s == th);
+      }
+    }
+    gt[qt] += g;
+    if (tie) {  // rare: some lane of this wave saw an exact tie
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        float s = acc[i];
+        if (HAS_SCALE) s *= sc16[i];
+        const int64_t e = e_base + row_of(i, hf);
+        if (e < limit && s == th) {
+          eq[qt] += 1;
+          eql[qt] += (e < (int64_t)tgt[qt]) ? 1 : 0;
+        }
+      }
+    }
+  }
+  __device__ void finish() {
+#pragma unroll
+    for (int t = 0; t < NQT; ++t) {
+      const int64_t q = q0 + 32 * t + c;
+      // both halves of the wave hold the same query: fold them, lanes < 32 publish
+      int32_t g = gt[t] + __shfl_xor(gt[t], 32, 64);
+      int32_t e = eq[t] + __shfl_xor(eq[t], 32, 64);
+      int32_t l = eql[t] + __shfl_xor(eql[t], 32, 64);
+      if (hf == 0 && q < B) {
+        if (g) atomicAdd(&a.n_gt[q], g);
+        if (e) atomicAdd(&a.n_eq[q], e);
+        if (l) atomicAdd(&a.n_eql[q], l);
+      }
+    }
+  }
+};
+
+struct TopkArgs {
+  const float* tau;          // per query: k-th best score so far (-inf while fewer than k known)
+  const int32_t* active;     // NULL = all queries; else only queries with active[b] != 0 collect
+  int32_t* cnt;              // per query: candidates appended this round
+  unsigned long long* cand;  // [B, cap] packed (ordered score << 32 | 0xffffffff - entity)
+  int32_t cap;
+};
+template <int NQT>
+struct TopkEpi {
+  static constexpr bool SWAP = false;
+  using Args = TopkArgs;
+  Args a;
+  float tau[NQT];
+  int64_t q0, B;
+  int c, hf;
+  __device__ void init(const Args& args, int64_t q0_, int c_, int hf_, int64_t B_) {
+    a = args; q0 = q0_; c = c_; hf = hf_; B = B_;
+#pragma unroll
+    for (int t = 0; t < NQT; ++t) {
+      const int64_t q = q0 + 32 * t + c;
+      const bool on = q < B && (a.active == nullptr || a.active[q] != 0);
+      tau[t] = on ? a.tau[q] : __uint_as_float(0x7f800000u);  // +inf: nothing qualifies
+    }
+  }
+  template <bool HAS_SCALE>
+  __device__ __forceinline__ void tile(int qt, const f32x16& acc, const float* sc16, float sc_col, int64_t e_base,
+                                       int64_t limit) {
+    const float th = tau[qt];
+    unsigned long long hit = 0;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      float s = acc[i];
+      if (HAS_SCALE) s *= sc16[i];
+      hit |= __builtin_amdgcn_ballot_w64(s > th);
+    }
+    if (hit) {
+      const int64_t q = q0 + 32 * qt + c;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        float s = acc[i];
+        if (HAS_SCALE) s *= sc16[i];
+        const int64_t e = e_base + row_of(i, hf);
+        if (s > th && e < limit) {
+          int32_t slot = atomicAdd(&a.cnt[q], 1);
+          if (slot >= a.cap) {
+            // Buffer full: the query is repaired by a later rescan.  Keep a uniform sample of what
+            // arrives (reservoir sampling) so that the threshold derived from the kept entries
+            // tightens geometrically whatever order the entities come in.
+            uint32_t h = ((uint32_t)e * 2654435761u) ^ ((uint32_t)slot * 0x9e3779b9u);
+            h ^= h >> 15; h *= 0x2c1b3c6du; h ^= h >> 12;
+            const uint32_t r = h % (uint32_t)(slot + 1);
+            slot = (r < (uint32_t)a.cap) ? (int32_t)r : -1;
+          }
+          if (slot >= 0)
+            a.cand[q * a.cap + slot] =
+                ((unsigned long long)f32_to_ordered(s) << 32) | (unsigned long long)(0xffffffffu - (uint32_t)e);
+        }
+      }
+    }
+  }
+  __device__ void finish() {}
+};
+
+struct BceArgs {
+  const float* bias;
+  double* sums;  // [0] sum softplus(s), [1] sum s
+  int32_t want_s;
+};
+template <int NQT>
+struct BceEpi {
+  static constexpr bool SWAP = false;
+  using Args = BceArgs;
+  Args a;
+  float bias[NQT];
+  bool valid[NQT];
+  double sp, ss;
+  int hf;
+  __device__ void init(const Args& args, int64_t q0, int c, int hf_, int64_t B) {
+    a = args; hf = hf_;
+    sp = 0.0; ss = 0.0;
+#pragma unroll
+    for (int t = 0; t < NQT; ++t) {
+      const int64_t q = q0 + 32 * t + c;
+      valid[t] = q < B;
+      bias[t] = (valid[t] && a.bias) ? a.bias[q] : 0.f;
+    }
+  }
+  template <bool HAS_SCALE>
+  __device__ __forceinline__ void tile(int qt, const f32x16& acc, const float* sc16, float sc_col, int64_t e_base,
+                                       int64_t limit) {
+    if (!valid[qt]) return;
+    float tsp = 0.f, tss = 0.f;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      float s = acc[i];
+      if (HAS_SCALE) s *= sc16[i];
+      s += bias[qt];
+      const bool ok = e_base + row_of(i, hf) < limit;
+      // softplus(s) = max(s,0) + log(1 + exp(-|s|))
+      const float t = fmaxf(s, 0.f) + __logf(1.0f + __expf(-fabsf(s)));
+      tsp += ok ? t : 0.f;
+      tss += ok ? s : 0.f;
+    }
+    sp += (double)tsp;
+    ss += (double)tss;
+  }
+  __device__ void finish() {
+    double x = sp, y = ss;
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) {
+      x += __shfl_xor(x, o, 64);
+      y += __shfl_xor(y, o, 64);
+    }
+    if ((threadIdx.x & 63) == 0) {
+      atomicAdd(&a.sums[0], x);
+      if (a.want_s) atomicAdd(&a.sums[1], y);
+    }
+  }
+};
+
+// ============================================================================================
+// qreg_kernel: bf16 MFMA, register-stationary queries, LDS-streamed entity rows.
+// ============================================================================================
+constexpr int QREG_NQT = 4;            // 32-query tiles per wave
+constexpr int QREG_WG_QUERIES = 512;   // 4 waves x 128 queries
+constexpr int QREG_STAGE_ROWS = 64;
+constexpr int QREG_ROW_BYTES = 272;    // 256 B of bf16 + 16 B pad: conflict-free ds_read_b128 across rows
+
+template <int EDT, template <int> class EpiT>
+__global__ void __launch_bounds__(256, 1) qreg_kernel(ContractArgs a, typename EpiT<QREG_NQT>::Args ea) {
+  using Epi = EpiT<QREG_NQT>;
+  constexpr bool HAS_SCALE = (EDT == KGE_I8);
+  __shared__ __attribute__((aligned(16))) unsigned char lds_e[2][QREG_STAGE_ROWS * QREG_ROW_BYTES];
+  __shared__ float lds_sc[2][QREG_STAGE_ROWS];
+
+  int qg;
+  int64_t chunk;
+  if (!decompose_wg(a, qg, chunk)) return;
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, c = lane & 31, hf = lane >> 5;
+  const int d = a.d;
+  const int64_t q0 = (int64_t)qg * QREG_WG_QUERIES + wave * (32 * QREG_NQT);
+
+  // ---- query fragments: lane (c, hf) holds k = 16 s + 8 hf .. +8 of query q0 + 32 t + c ----
+  bf16x8 qf[QREG_NQT][8];
+#pragma unroll
+  for (int t = 0; t < QREG_NQT; ++t) {
+    const int64_t q = q0 + 32 * t + c;
+#pragma unroll
+    for (int s = 0; s < 8; ++s) {
+      const int k = 16 * s + 8 * hf;
+      f32x4 lo = {0.f, 0.f, 0.f, 0.f}, hi = {0.f, 0.f, 0.f, 0.f};
+      if (q < a.B && k < d) {
+        const f32x4* src = (const f32x4*)(a.Q + q * d + k);
+        lo = src[0];
+        hi = src[1];
+      }
+      qf[t][s] = cvt_bf16x8(lo, hi);
+    }
+  }
+  Epi epi;
+  epi.init(ea, q0, c, hf, a.B);
+
+  const int64_t r0 = a.e_begin + chunk * a.chunk_rows;
+  const int64_t r1 = (r0 + a.chunk_rows < a.e_end) ? r0 + a.chunk_rows : a.e_end;
+  const int nst = (int)((r1 - r0 + QREG_STAGE_ROWS - 1) / QREG_STAGE_ROWS);
+
+  constexpr int NLD = (EDT == KGE_BF16) ? 4 : 2;
+  u32x4 stage[NLD];
+  float stage_sc = 0.f;
+
+  auto stage_load = [&](int64_t row0) {
+    if (EDT == KGE_BF16) {
+#pragma unroll
+      for (int j = 0; j < NLD; ++j) {
+        const int idx = tid + 256 * j, row = idx >> 4, piece = idx & 15;
+        const int64_t g = row0 + row;
+        u32x4 v = {0u, 0u, 0u, 0u};
+        if (g < r1 && piece * 8 < d) v = *(const u32x4*)((const uint16_t*)a.E + g * d + piece * 8);
+        stage[j] = v;
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < NLD; ++j) {
+        const int idx = tid + 256 * j, row = idx >> 3, piece = idx & 7;
+        const int64_t g = row0 + row;
+        u32x4 v = {0u, 0u, 0u, 0u};
+        if (g < r1 && piece * 16 < d) v = *(const u32x4*)((const int8_t*)a.E + g * d + piece * 16);
+        stage[j] = v;
+      }
+      if (tid < QREG_STAGE_ROWS) stage_sc = (row0 + tid < r1) ? a.scale[row0 + tid] : 0.f;
+    }
+  };
+  auto stage_store = [&](int buf) {
+    if (EDT == KGE_BF16) {
+#pragma unroll
+      for (int j = 0; j < NLD; ++j) {
+        const int idx = tid + 256 * j, row = idx >> 4, piece = idx & 15;
+        *(u32x4*)(&lds_e[buf][row * QREG_ROW_BYTES + piece * 16]) = stage[j];
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < NLD; ++j) {
+        const int idx = tid + 256 * j, row = idx >> 3, piece = idx & 7;
+        unsigned char* dst = &lds_e[buf][row * QREG_ROW_BYTES + piece * 32];
+        *(u32x4*)(dst) = i8x8_to_bf16x8(stage[j][0], stage[j][1]);
+        *(u32x4*)(dst + 16) = i8x8_to_bf16x8(stage[j][2], stage[j][3]);
+      }
+      if (tid < QREG_STAGE_ROWS) lds_sc[buf][tid] = stage_sc;
+    }
+  };
+
+  stage_load(r0);
+  stage_store(0);
+  __syncthreads();
+  for (int st = 0; st < nst; ++st) {
+    const int buf = st & 1;
+    const int64_t row0 = r0 + (int64_t)st * QREG_STAGE_ROWS;
+    if (st + 1 < nst) stage_load(row0 + QREG_STAGE_ROWS);
+#pragma unroll
+    for (int et = 0; et < QREG_STAGE_ROWS / 32; ++et) {
+      const int64_t e_base = row0 + et * 32;
+      if (e_base < r1) {
+        bf16x8 ef[8];
+        const unsigned char* src = &lds_e[buf][(et * 32 + c) * QREG_ROW_BYTES + hf * 16];
+#pragma unroll
+        for (int s = 0; s < 8; ++s) ef[s] = *(const bf16x8*)(src + s * 32);
+        float sc16[16];
+        float sc_col = 1.f;
+        if (HAS_SCALE) {
+          if (Epi::SWAP) {
+            sc_col = lds_sc[buf][et * 32 + c];
+          } else {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) sc16[i] = lds_sc[buf][et * 32 + row_of(i, hf)];
+          }
+        }
+#pragma unroll
+        for (int t = 0; t < QREG_NQT; ++t) {
+          f32x16 acc = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int s = 0; s < 8; ++s)
+            acc = Epi::SWAP ? mfma_bf16(qf[t][s], ef[s], acc) : mfma_bf16(ef[s], qf[t][s], acc);
+          epi.template tile<HAS_SCALE>(t, acc, sc16, sc_col, e_base, r1);
+        }
+      }
+    }
+    if (st + 1 < nst) stage_store(buf ^ 1);
+    __syncthreads();
+  }
+  epi.finish();
+}
+
+// ============================================================================================
+// kloop_kernel: fp32 MFMA, 128 entities x 128 queries per workgroup, K chunks of 32 through LDS.
+// Chain order per score: k-blocks of 8 ascending; inside a block MFMA step j (0..3) consumes
+// k0 + j (lanes 0-31) and k0 + 4 + j (lanes 32-63).
+// ============================================================================================
+constexpr int KLOOP_NQT = 2;
+constexpr int KLOOP_WG_QUERIES = 128;
+constexpr int KLOOP_TILE_ROWS = 128;
+constexpr int KLOOP_KC = 32;
+constexpr int KLOOP_LDK = 36;  // floats per LDS row: 32 + 4 pad
+
+template <template <int> class EpiT>
+__global__ void __launch_bounds__(256, 2) kloop_kernel(ContractArgs a, typename EpiT<KLOOP_NQT>::Args ea) {
+  using Epi = EpiT<KLOOP_NQT>;
+  __shared__ __attribute__((aligned(16))) float lds_e[KLOOP_TILE_ROWS * KLOOP_LDK];
+  __shared__ __attribute__((aligned(16))) float lds_q[KLOOP_WG_QUERIES * KLOOP_LDK];
+
+  int qg;
+  int64_t chunk;
+  if (!decompose_wg(a, qg, chunk)) return;
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, c = lane & 31, hf = lane >> 5;
+  const int we = wave >> 1, wq = wave & 1;
+  const int d = a.d;
+  const bool vec_ok = (d & 3) == 0;
+  const int64_t q_base = (int64_t)qg * KLOOP_WG_QUERIES;
+  const int64_t q0 = q_base + 64 * wq;
+  Epi epi;
+  epi.init(ea, q0, c, hf, a.B);
+
+  const int64_t r0 = a.e_begin + chunk * a.chunk_rows;
+  const int64_t r1 = (r0 + a.chunk_rows < a.e_end) ? r0 + a.chunk_rows : a.e_end;
+  const int nkc = (d + KLOOP_KC - 1) / KLOOP_KC;
+  const float* Ef = (const float*)a.E;
+
+  auto load4 = [&](const float* base, int64_t row, bool row_ok, int k) -> f32x4 {
+    f32x4 v = {0.f, 0.f, 0.f, 0.f};
+    if (row_ok) {
+      const float* p = base + row * d + k;
+      if (vec_ok) {
+        if (k < d) v = *(const f32x4*)p;
+      } else {
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          if (k + j < d) v[j] = p[j];
+      }
+    }
+    return v;
+  };
+
+  for (int64_t et0 = r0; et0 < r1; et0 += KLOOP_TILE_ROWS) {
+    f32x16 acc[2][2];
+#pragma unroll
+    for (int te = 0; te < 2; ++te)
+#pragma unroll
+      for (int tq = 0; tq < 2; ++tq)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[te][tq][i] = 0.f;
+
+    for (int kc = 0; kc < nkc; ++kc) {
+      f32x4 ve[4], vq[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int idx = tid + 256 * j, row = idx >> 3, piece = idx & 7;
+        const int k = kc * KLOOP_KC + piece * 4;
+        ve[j] = load4(Ef, et0 + row, et0 + row < r1, k);
+        vq[j] = load4(a.Q, q_base + row, q_base + row < a.B, k);
+      }
+      __syncthreads();  // previous chunk's fragment reads are done
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int idx = tid + 256 * j, row = idx >> 3, piece = idx & 7;
+        *(f32x4*)&lds_e[row * KLOOP_LDK + piece * 4] = ve[j];
+        *(f32x4*)&lds_q[row * KLOOP_LDK + piece * 4] = vq[j];
+      }
+      __syncthreads();
+#pragma unroll
+      for (int kb = 0; kb < KLOOP_KC / 8; ++kb) {
+        f32x4 fe[2], fq[2];
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+          fe[t] = *(const f32x4*)&lds_e[(64 * we + 32 * t + c) * KLOOP_LDK + kb * 8 + 4 * hf];
+          fq[t] = *(const f32x4*)&lds_q[(64 * wq + 32 * t + c) * KLOOP_LDK + kb * 8 + 4 * hf];
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+          for (int te = 0; te < 2; ++te)
+#pragma unroll
+            for (int tq = 0; tq < 2; ++tq)
+              acc[te][tq] = Epi::SWAP ? mfma_f32(fq[tq][j], fe[te][j], acc[te][tq])
+                                      : mfma_f32(fe[te][j], fq[tq][j], acc[te][tq]);
+      }
+    }
+    float sc16[16];
+#pragma unroll
+    for (int te = 0; te < 2; ++te) {
+      const int64_t e_base = et0 + 64 * we + 32 * te;
+      if (e_base < r1) {
+#pragma unroll
+        for (int tq = 0; tq < 2; ++tq) epi.template tile<false>(tq, acc[te][tq], sc16, 1.f, e_base, r1);
+      }
+    }
+  }
+  epi.finish();
+}
+
+}  // namespace kge

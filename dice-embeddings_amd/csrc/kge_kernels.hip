@@ -1,0 +1,687 @@
+// Entry points of the contraction path: materialised scores, fused filtered rank, fused top-k and
+// fused multi-hot BCE, plus the small helper kernels around the two MFMA main loops.
+#include "kge_contract.hip.h"
+
+#include <string.h>
+
+namespace kge {
+
+// ---- thread-local error text --------------------------------------------------------------
+static thread_local char g_err[512] = "";
+int set_error(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+void clear_error() { g_err[0] = 0; }
+
+namespace {
+
+// ============================================================================================
+// One 32x32 tile straight from global memory: entity rows as A, query rows as B, in the same
+// reduction order as the two main loops.  Lane (c, hf) supplies entity row `e_row` and query row
+// `q_row` (either may be -1: a zero row).  Used where rows are gathered (targets, filter lists).
+// ============================================================================================
+template <int EDT>
+__device__ __forceinline__ f32x16 chain_direct(const void* E, int d, int64_t e_row, const float* Q, int64_t q_row,
+                                               int hf) {
+  f32x16 acc;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) acc[i] = 0.f;
+  if (EDT == KGE_F32) {
+    const float* Ef = (const float*)E;
+    const bool vec_ok = (d & 3) == 0;
+    const int nkb = (d + 7) >> 3;
+    for (int kb = 0; kb < nkb; ++kb) {
+      const int k = kb * 8 + 4 * hf;
+      f32x4 fe = {0.f, 0.f, 0.f, 0.f}, fq = {0.f, 0.f, 0.f, 0.f};
+      if (vec_ok) {
+        if (k < d) {
+          if (e_row >= 0) fe = *(const f32x4*)(Ef + e_row * d + k);
+          if (q_row >= 0) fq = *(const f32x4*)(Q + q_row * d + k);
+        }
+      } else {
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          if (k + j < d) {
+            if (e_row >= 0) fe[j] = Ef[e_row * d + k + j];
+            if (q_row >= 0) fq[j] = Q[q_row * d + k + j];
+          }
+      }
+#pragma unroll
+      for (int j = 0; j < 4; ++j) acc = mfma_f32(fe[j], fq[j], acc);
+    }
+  } else {
+#pragma unroll
+    for (int s = 0; s < 8; ++s) {
+      const int k = 16 * s + 8 * hf;
+      u32x4 ev = {0u, 0u, 0u, 0u};
+      f32x4 lo = {0.f, 0.f, 0.f, 0.f}, hi = {0.f, 0.f, 0.f, 0.f};
+      if (k < d) {
+        if (e_row >= 0) {
+          if (EDT == KGE_BF16) {
+            ev = *(const u32x4*)((const uint16_t*)E + e_row * d + k);
+          } else {
+            const u32x2 w = *(const u32x2*)((const int8_t*)E + e_row * d + k);
+            ev = i8x8_to_bf16x8(w[0], w[1]);
+          }
+        }
+        if (q_row >= 0) {
+          const f32x4* src = (const f32x4*)(Q + q_row * d + k);
+          lo = src[0];
+          hi = src[1];
+        }
+      }
+      bf16x8 ef = __builtin_bit_cast(bf16x8, ev);
+      acc = mfma_bf16(ef, cvt_bf16x8(lo, hi), acc);
+    }
+  }
+  return acc;
+}
+
+// ---- raw score of each query's target (the rank threshold) + counter initialisation ---------
+template <int EDT>
+__global__ void __launch_bounds__(256) target_score_kernel(ContractArgs a, const int64_t* target, const float* bias,
+                                                          float* thr, float* target_score, int32_t* n_gt,
+                                                          int32_t* n_eq, int32_t* n_eql) {
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, c = lane & 31, hf = lane >> 5;
+  const int64_t q = ((int64_t)blockIdx.x * 4 + wave) * 32 + c;
+  const int64_t t = (q < a.B) ? target[q] : -1;
+  const bool ok = t >= 0 && t < a.N;
+  f32x16 acc = chain_direct<EDT>(a.E, a.d, ok ? t : -1, a.Q, (q < a.B) ? q : -1, hf);
+  // diagonal element (entity row c, query column c)
+  const int isel = ((c >> 3) << 2) | (c & 3);
+  float v = 0.f;
+#pragma unroll
+  for (int i = 0; i < 16; ++i)
+    if (i == isel) v = acc[i];
+  if (hf == ((c >> 2) & 1) && q < a.B) {
+    float raw = __uint_as_float(0x7fc00000u);
+    if (ok) raw = (EDT == KGE_I8) ? v * a.scale[t] : v;
+    thr[q] = raw;
+    target_score[q] = raw + (bias ? bias[q] : 0.f);
+    n_gt[q] = 0;
+    n_eq[q] = ok ? -1 : 0;  // the main pass counts the target as tying with itself
+    n_eql[q] = 0;
+  }
+}
+
+// ---- sort (csr_row, query) pairs of one sub-batch so queries sharing a filter row are adjacent
+constexpr int SORT_MAX = 8192;
+__global__ void __launch_bounds__(1024) sort_rows_kernel(const int64_t* csr_row, int64_t b0, int nb, int64_t n_rows,
+                                                        unsigned long long* out, int npad) {
+  extern __shared__ unsigned long long keys[];
+  const int tid = threadIdx.x;
+  for (int i = tid; i < npad; i += 1024) {
+    unsigned long long key = ~0ull;
+    if (i < nb) {
+      const int64_t r = csr_row[b0 + i];
+      if (r >= 0 && r < n_rows) key = ((unsigned long long)r << 24) | (unsigned long long)i;
+    }
+    keys[i] = key;
+  }
+  __syncthreads();
+  for (int k = 2; k <= npad; k <<= 1) {
+    for (int j = k >> 1; j > 0; j >>= 1) {
+      for (int i = tid; i < npad; i += 1024) {
+        const int ixj = i ^ j;
+        if (ixj > i) {
+          const bool up = (i & k) == 0;
+          const unsigned long long x = keys[i], y = keys[ixj];
+          if ((x > y) == up) {
+            keys[i] = y;
+            keys[ixj] = x;
+          }
+        }
+      }
+      __syncthreads();
+    }
+  }
+  for (int i = tid; i < npad; i += 1024) out[i] = keys[i];
+}
+
+// ---- take the filtered entities back out of the counters ------------------------------------
+// One workgroup per (first query of a group sharing a filter row, slice of that row).  Scores of
+// the slice's entities are formed once per group, then every query of the group compares them
+// with its own threshold.
+constexpr int FIX_CAP = 2048;
+template <int EDT>
+__global__ void __launch_bounds__(256) filter_fix_kernel(ContractArgs a, const unsigned long long* skey, int nb,
+                                                        int64_t b0, const int64_t* row_ptr, const int32_t* col,
+                                                        const int64_t* target, const float* thr, int32_t* n_gt,
+                                                        int32_t* n_eq, int32_t* n_eql) {
+  __shared__ float s_s[FIX_CAP];
+  __shared__ float s_sc[FIX_CAP];
+  __shared__ int32_t s_e[FIX_CAP];
+  __shared__ int s_m;
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, c = lane & 31, hf = lane >> 5;
+  const int i0 = blockIdx.x;
+  const unsigned long long key = skey[i0];
+  if (key == ~0ull) return;
+  const int64_t row = (int64_t)(key >> 24);
+  if (i0 > 0 && (int64_t)(skey[i0 - 1] >> 24) == row) return;  // not the first of its group
+
+  if (tid == 0) s_m = nb - i0;
+  __syncthreads();
+  for (int base = 1;; base += 256) {
+    const int pos = i0 + base + tid;
+    if (pos < nb && (int64_t)(skey[pos] >> 24) != row) atomicMin(&s_m, pos - i0);
+    __syncthreads();
+    const int m_now = s_m;
+    __syncthreads();
+    if (m_now < base + 256 || i0 + base + 256 >= nb) break;
+  }
+  const int m = s_m;
+
+  const int64_t L0 = row_ptr[row], L1 = row_ptr[row + 1];
+  const int64_t L = L1 - L0;
+  const int64_t split = gridDim.y;
+  const int64_t per = (((L + split - 1) / split) + 31) & ~(int64_t)31;
+  const int64_t z0 = L0 + (int64_t)blockIdx.y * per;
+  const int64_t z1 = (z0 + per < L1) ? z0 + per : L1;
+  if (z0 >= z1) return;
+  const int64_t bq = b0 + (int64_t)(key & 0xffffffull);
+
+  for (int64_t pass = z0; pass < z1; pass += FIX_CAP) {
+    const int n_here = (int)((z1 - pass < FIX_CAP) ? z1 - pass : FIX_CAP);
+    const int ntile = (n_here + 31) >> 5;
+    for (int tile = wave; tile < ntile; tile += 4) {
+      const int j = tile * 32 + c;
+      const int32_t e = (j < n_here) ? col[pass + j] : -1;
+      const bool ok = e >= 0 && (int64_t)e < a.N;
+      f32x16 acc = chain_direct<EDT>(a.E, a.d, ok ? (int64_t)e : -1, a.Q, bq, hf);
+      if (c == 0) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) s_s[tile * 32 + row_of(i, hf)] = acc[i];
+      }
+      if (hf == 0) {
+        s_e[j] = ok ? e : -1;
+        s_sc[j] = (EDT == KGE_I8 && ok) ? a.scale[e] : 1.f;
+      }
+    }
+    __syncthreads();
+    for (int mi = tid; mi < m; mi += 256) {
+      const int64_t b = b0 + (int64_t)(skey[i0 + mi] & 0xffffffull);
+      const float th = thr[b];
+      const int64_t t = target[b];
+      int32_t g = 0, eq = 0, eql = 0;
+      for (int j = 0; j < n_here; ++j) {
+        const int32_t e = s_e[j];
+        float s = s_s[j];
+        if (EDT == KGE_I8) s *= s_sc[j];
+        if (e >= 0 && (int64_t)e != t) {
+          g += (s > th) ? 1 : 0;
+          if (s == th) {
+            eq += 1;
+            eql += ((int64_t)e < t) ? 1 : 0;
+          }
+        }
+      }
+      if (g) atomicSub(&n_gt[b], g);
+      if (eq) atomicSub(&n_eq[b], eq);
+      if (eql) atomicSub(&n_eql[b], eql);
+    }
+    __syncthreads();
+  }
+}
+
+// ---- top-k bookkeeping ------------------------------------------------------------------------
+constexpr int TOPK_CAP = 4096;      // candidates a query can collect in one round
+constexpr int TOPK_MAX_K = 1024;
+constexpr int TOPK_FIRST_ROWS = 4096;  // first round takes everything: must not exceed TOPK_CAP
+
+struct TopkWs {
+  float* tau;
+  int32_t* cnt;
+  int32_t* list_len;
+  int32_t* dirty;
+  int32_t* n_dirty;
+  unsigned long long* list;  // [B, kpad]
+  unsigned long long* cand;  // [B, TOPK_CAP]
+  int64_t kpad;
+};
+
+static size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
+
+size_t topk_ws_layout(int64_t B, int64_t k, void* base, TopkWs* ws) {
+  size_t off = 0;
+  char* p = (char*)base;
+  const int64_t kpad = (k + 7) / 8 * 8;
+  auto take = [&](size_t bytes) {
+    size_t o = off;
+    off = align_up(off + bytes, 256);
+    return o;
+  };
+  size_t o_tau = take(B * 4), o_cnt = take(B * 4), o_len = take(B * 4), o_dirty = take(B * 4), o_nd = take(4);
+  size_t o_list = take((size_t)B * kpad * 8), o_cand = take((size_t)B * TOPK_CAP * 8);
+  if (ws) {
+    ws->tau = (float*)(p + o_tau);
+    ws->cnt = (int32_t*)(p + o_cnt);
+    ws->list_len = (int32_t*)(p + o_len);
+    ws->dirty = (int32_t*)(p + o_dirty);
+    ws->n_dirty = (int32_t*)(p + o_nd);
+    ws->list = (unsigned long long*)(p + o_list);
+    ws->cand = (unsigned long long*)(p + o_cand);
+    ws->kpad = kpad;
+  }
+  return off;
+}
+
+__global__ void topk_init_kernel(TopkWs w, int64_t B) {
+  const int64_t b = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (b < B) {
+    w.tau[b] = __uint_as_float(0xff800000u);  // -inf
+    w.cnt[b] = 0;
+    w.list_len[b] = 0;
+    w.dirty[b] = 0;
+  }
+  if (b == 0) *w.n_dirty = 0;
+}
+
+// Merge a query's kept list with this round's candidates, keep the best k, publish the new
+// threshold.  In `rescan` mode (only queries flagged dirty) list entries above the old threshold
+// are dropped first: the rescan finds all of them again.
+__global__ void __launch_bounds__(256) topk_select_kernel(TopkWs w, int k, int rescan) {
+  extern __shared__ unsigned long long keys[];
+  __shared__ int s_valid;
+  const int tid = threadIdx.x;
+  const int64_t b = blockIdx.x;
+  if (rescan && !w.dirty[b]) return;
+  const int len = w.list_len[b];
+  const int raw = w.cnt[b];
+  const int nc = raw < TOPK_CAP ? raw : TOPK_CAP;
+  const bool over = raw > TOPK_CAP;
+  const float tau_old = w.tau[b];
+  const int n = len + nc;
+  int npad = 2;
+  while (npad < n) npad <<= 1;
+  if (tid == 0) s_valid = 0;
+  for (int i = tid; i < npad; i += 256) {
+    unsigned long long key = 0;
+    if (i < len) {
+      key = w.list[b * w.kpad + i];
+      if (rescan && ordered_to_f32((uint32_t)(key >> 32)) > tau_old) key = 0;
+    } else if (i < n) {
+      key = w.cand[b * TOPK_CAP + (i - len)];
+    }
+    keys[i] = key;
+  }
+  __syncthreads();
+  for (int kk = 2; kk <= npad; kk <<= 1) {
+    for (int j = kk >> 1; j > 0; j >>= 1) {
+      for (int i = tid; i < npad; i += 256) {
+        const int ixj = i ^ j;
+        if (ixj > i) {
+          const bool down = (i & kk) == 0;
+          const unsigned long long x = keys[i], y = keys[ixj];
+          if ((x < y) == down) {
+            keys[i] = y;
+            keys[ixj] = x;
+          }
+        }
+      }
+      __syncthreads();
+    }
+  }
+  for (int i = tid; i < npad; i += 256)
+    if (keys[i] != 0 && (i + 1 == npad || keys[i + 1] == 0)) s_valid = i + 1;
+  __syncthreads();
+  const int n_valid = s_valid;
+  const int new_len = n_valid < k ? n_valid : k;
+  for (int i = tid; i < new_len; i += 256) w.list[b * w.kpad + i] = keys[i];
+  if (tid == 0) {
+    w.list_len[b] = new_len;
+    w.tau[b] = (new_len == k) ? ordered_to_f32((uint32_t)(keys[k - 1] >> 32)) : __uint_as_float(0xff800000u);
+    w.cnt[b] = 0;
+    if (!rescan) {
+      if (over && !w.dirty[b]) {
+        w.dirty[b] = 1;
+        atomicAdd(w.n_dirty, 1);
+      }
+    } else if (!over) {
+      w.dirty[b] = 0;
+      atomicSub(w.n_dirty, 1);
+    }
+  }
+}
+
+__global__ void topk_output_kernel(TopkWs w, int64_t B, int k, const float* bias, int apply_sigmoid,
+                                   float* out_scores, int64_t* out_idx) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= B * k) return;
+  const int64_t b = i / k;
+  const int j = (int)(i % k);
+  float s = __uint_as_float(0x7fc00000u);
+  int64_t e = -1;
+  if (j < w.list_len[b]) {
+    const unsigned long long key = w.list[b * w.kpad + j];
+    s = ordered_to_f32((uint32_t)(key >> 32));
+    e = (int64_t)(0xffffffffu - (uint32_t)(key & 0xffffffffull));
+    if (bias) s += bias[b];
+    if (apply_sigmoid) s = 1.0f / (1.0f + expf(-s));
+  }
+  out_scores[i] = s;
+  out_idx[i] = e;
+}
+
+// ---- BCE helpers --------------------------------------------------------------------------------
+__global__ void bce_init_kernel(double* sums) {
+  if (threadIdx.x < 3) sums[threadIdx.x] = 0.0;
+}
+
+// sum of the logits of the positive (query, tail) pairs: one wave per query
+template <int EDT>
+__global__ void __launch_bounds__(256) bce_pos_kernel(ContractArgs a, const float* bias, const int64_t* csr_row,
+                                                     const int64_t* row_ptr, const int32_t* col, int64_t n_rows,
+                                                     double* sums) {
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int64_t q = (int64_t)blockIdx.x * 4 + wave;
+  if (q >= a.B) return;
+  const int64_t row = csr_row[q];
+  double local = 0.0;
+  if (row >= 0 && row < n_rows) {
+    const float bq = bias ? bias[q] : 0.f;
+    const float* qv = a.Q + q * a.d;
+    for (int64_t j = row_ptr[row] + lane; j < row_ptr[row + 1]; j += 64) {
+      const int64_t e = col[j];
+      if (e < 0 || e >= a.N) continue;
+      float dot = 0.f;
+      for (int k = 0; k < a.d; ++k) {
+        float x;
+        float qk = qv[k];
+        if (EDT == KGE_F32) {
+          x = ((const float*)a.E)[e * a.d + k];
+        } else {
+          qk = (float)(__bf16)qk;
+          if (EDT == KGE_BF16)
+            x = __uint_as_float((uint32_t)((const uint16_t*)a.E)[e * a.d + k] << 16);
+          else
+            x = (float)((const int8_t*)a.E)[e * a.d + k];
+        }
+        dot = fmaf(qk, x, dot);
+      }
+      if (EDT == KGE_I8) dot *= a.scale[e];
+      local += (double)(dot + bq);
+    }
+  }
+#pragma unroll
+  for (int o = 32; o >= 1; o >>= 1) local += __shfl_xor(local, o, 64);
+  if (lane == 0 && local != 0.0) atomicAdd(&sums[2], local);
+}
+
+__global__ void bce_final_kernel(const double* sums, double B, double N, float eps, float* loss) {
+  if (threadIdx.x == 0 && blockIdx.x == 0) {
+    double t = sums[0];
+    if (eps != 0.f)
+      t -= (1.0 - (double)eps) * sums[2] + sums[1] / N;
+    else
+      t -= sums[2];
+    loss[0] = (float)(t / (B * N));
+  }
+}
+
+// ============================================================================================
+// host side
+// ============================================================================================
+int check_contract(const char* who, const float* Q, const void* E, int dtype, const float* scale, int64_t B,
+                   int64_t d, int64_t N) {
+  KGE_REQUIRE(B >= 0 && N >= 1, KGE_ERR_INVALID, "%s: B=%lld N=%lld", who, (long long)B, (long long)N);
+  KGE_REQUIRE(N <= 0x7fffffffLL, KGE_ERR_INVALID, "%s: N=%lld exceeds int32 entity ids", who, (long long)N);
+  KGE_REQUIRE(B <= (1 << 24), KGE_ERR_INVALID, "%s: B=%lld exceeds 2^24", who, (long long)B);
+  KGE_REQUIRE(Q && E, KGE_ERR_INVALID, "%s: null Q or E", who);
+  KGE_REQUIRE(((uintptr_t)Q & 15) == 0 && ((uintptr_t)E & 15) == 0, KGE_ERR_INVALID,
+              "%s: Q and E must be 16-byte aligned", who);
+  switch (dtype) {
+    case KGE_F32:
+      KGE_REQUIRE(d >= 1 && d <= 65536, KGE_ERR_INVALID, "%s: d=%lld", who, (long long)d);
+      break;
+    case KGE_BF16:
+      KGE_REQUIRE(d >= 8 && d % 8 == 0, KGE_ERR_INVALID, "%s: bf16 tables need d %% 8 == 0, got %lld", who,
+                  (long long)d);
+      KGE_REQUIRE(d <= 128, KGE_ERR_UNSUPPORTED, "%s: bf16 tables support d <= 128, got %lld", who, (long long)d);
+      break;
+    case KGE_I8:
+      KGE_REQUIRE(d >= 16 && d % 16 == 0, KGE_ERR_INVALID, "%s: int8 tables need d %% 16 == 0, got %lld", who,
+                  (long long)d);
+      KGE_REQUIRE(d <= 128, KGE_ERR_UNSUPPORTED, "%s: int8 tables support d <= 128, got %lld", who, (long long)d);
+      KGE_REQUIRE(scale, KGE_ERR_INVALID, "%s: int8 tables need per-row scales", who);
+      break;
+    default: return set_error(KGE_ERR_INVALID, "%s: unknown dtype %d", who, dtype);
+  }
+  return KGE_OK;
+}
+
+ContractArgs make_args(const float* Q, const void* E, int dtype, const float* scale, int64_t B, int64_t d,
+                       int64_t N, int64_t e_begin, int64_t e_end) {
+  ContractArgs a;
+  a.Q = Q;
+  a.E = E;
+  a.scale = scale;
+  a.B = B;
+  a.N = N;
+  a.e_begin = e_begin;
+  a.e_end = e_end;
+  a.d = (int)d;
+  const int wgq = (dtype == KGE_F32) ? KLOOP_WG_QUERIES : QREG_WG_QUERIES;
+  const int tile = (dtype == KGE_F32) ? KLOOP_TILE_ROWS : QREG_STAGE_ROWS;
+  const int max_chunk = (dtype == KGE_F32) ? 1024 : 2048;
+  a.n_qgroups = (int)((B + wgq - 1) / wgq);
+  const int64_t rows = e_end - e_begin;
+  int64_t chunk = rows * a.n_qgroups / 2048;  // aim for >= 2048 workgroups (8 per CU)
+  chunk = (chunk + tile - 1) / tile * tile;
+  if (chunk < tile) chunk = tile;
+  if (chunk > max_chunk) chunk = max_chunk;
+  a.chunk_rows = (int)chunk;
+  a.n_chunks = (rows + chunk - 1) / chunk;
+  return a;
+}
+
+template <template <int> class EpiT, class EArgs>
+int launch_contract(int dtype, const ContractArgs& a, const EArgs& ea, hipStream_t st, const char* name) {
+  if (a.B == 0 || a.e_end <= a.e_begin) return KGE_OK;
+  const int64_t nwg = (a.n_chunks + 7) / 8 * 8 * a.n_qgroups;
+  KGE_REQUIRE(nwg <= 0x7fffffffLL, KGE_ERR_INVALID, "%s: grid of %lld workgroups too large", name, (long long)nwg);
+  dim3 grid((unsigned)nwg), block(256);
+  if (dtype == KGE_F32)
+    hipLaunchKernelGGL((kloop_kernel<EpiT>), grid, block, 0, st, a, ea);
+  else if (dtype == KGE_BF16)
+    hipLaunchKernelGGL((qreg_kernel<KGE_BF16, EpiT>), grid, block, 0, st, a, ea);
+  else
+    hipLaunchKernelGGL((qreg_kernel<KGE_I8, EpiT>), grid, block, 0, st, a, ea);
+  KGE_LAUNCH_CHECK(name);
+  return KGE_OK;
+}
+
+#define KGE_DISPATCH_DTYPE(dtype, KERNEL, grid, block, shmem, st, ...)                       \
+  do {                                                                                       \
+    if ((dtype) == KGE_F32)                                                                  \
+      hipLaunchKernelGGL((KERNEL<KGE_F32>), grid, block, shmem, st, __VA_ARGS__);            \
+    else if ((dtype) == KGE_BF16)                                                            \
+      hipLaunchKernelGGL((KERNEL<KGE_BF16>), grid, block, shmem, st, __VA_ARGS__);           \
+    else                                                                                     \
+      hipLaunchKernelGGL((KERNEL<KGE_I8>), grid, block, shmem, st, __VA_ARGS__);             \
+  } while (0)
+
+struct RankWs {
+  float* thr;
+  unsigned long long* skey;
+};
+size_t rank_ws_layout(int64_t B, void* base, RankWs* ws) {
+  size_t o_thr = 0;
+  size_t o_key = align_up((size_t)B * 4, 256);
+  size_t total = o_key + align_up((size_t)SORT_MAX * 8, 256);
+  if (ws) {
+    ws->thr = (float*)((char*)base + o_thr);
+    ws->skey = (unsigned long long*)((char*)base + o_key);
+  }
+  return total;
+}
+
+}  // namespace
+}  // namespace kge
+
+using namespace kge;
+
+extern "C" const char* kge_last_error(void) { return g_err; }
+extern "C" int kge_abi_version(void) { return KGE_ABI_VERSION; }
+
+extern "C" int kge_scores(const float* Q, const float* bias, const void* E, int dtype, const float* scale, int64_t B,
+                          int64_t d, int64_t N, float* S, int64_t ldS, void* stream) {
+  clear_error();
+  int rc = check_contract("kge_scores", Q, E, dtype, scale, B, d, N);
+  if (rc) return rc;
+  KGE_REQUIRE(S && ldS >= N, KGE_ERR_INVALID, "kge_scores: S is null or ldS=%lld < N=%lld", (long long)ldS,
+              (long long)N);
+  ContractArgs a = make_args(Q, E, dtype, scale, B, d, N, 0, N);
+  StoreArgs ea{S, bias, ldS};
+  return launch_contract<StoreEpi>(dtype, a, ea, (hipStream_t)stream, "kge_scores");
+}
+
+extern "C" size_t kge_rank_workspace_bytes(int64_t B) { return rank_ws_layout(B < 1 ? 1 : B, nullptr, nullptr); }
+
+extern "C" int kge_rank_filtered(const float* Q, const float* bias, const void* E, int dtype, const float* scale,
+                                 int64_t B, int64_t d, int64_t N, const int64_t* target, const int64_t* csr_row,
+                                 const int64_t* row_ptr, const int32_t* col, int64_t n_rows, int32_t* n_greater,
+                                 int32_t* n_equal, int32_t* n_equal_lower, float* target_score, void* workspace,
+                                 size_t workspace_bytes, void* stream) {
+  clear_error();
+  int rc = check_contract("kge_rank_filtered", Q, E, dtype, scale, B, d, N);
+  if (rc) return rc;
+  if (B == 0) return KGE_OK;
+  KGE_REQUIRE(target && n_greater && n_equal && n_equal_lower && target_score, KGE_ERR_INVALID,
+              "kge_rank_filtered: null target or output pointer");
+  const bool filtered = csr_row != nullptr;
+  KGE_REQUIRE(!filtered || (row_ptr && col && n_rows >= 0), KGE_ERR_INVALID,
+              "kge_rank_filtered: csr_row given without row_ptr / col");
+  KGE_REQUIRE(n_rows < (1LL << 39), KGE_ERR_INVALID, "kge_rank_filtered: n_rows=%lld too large", (long long)n_rows);
+  KGE_REQUIRE(workspace && workspace_bytes >= kge_rank_workspace_bytes(B), KGE_ERR_WORKSPACE,
+              "kge_rank_filtered: workspace of %zu bytes, need %zu", workspace_bytes, kge_rank_workspace_bytes(B));
+  hipStream_t st = (hipStream_t)stream;
+  RankWs ws;
+  rank_ws_layout(B, workspace, &ws);
+
+  ContractArgs a = make_args(Q, E, dtype, scale, B, d, N, 0, N);
+  {
+    dim3 grid((unsigned)((B + 127) / 128)), block(256);
+    KGE_DISPATCH_DTYPE(dtype, target_score_kernel, grid, block, 0, st, a, target, bias, ws.thr, target_score,
+                       n_greater, n_equal, n_equal_lower);
+    KGE_LAUNCH_CHECK("target_score_kernel");
+  }
+  RankArgs ea{ws.thr, target, n_greater, n_equal, n_equal_lower};
+  rc = launch_contract<RankEpi>(dtype, a, ea, st, "kge_rank_filtered");
+  if (rc) return rc;
+  if (filtered && n_rows > 0) {
+    for (int64_t b0 = 0; b0 < B; b0 += SORT_MAX) {
+      const int nb = (int)((B - b0 < SORT_MAX) ? B - b0 : SORT_MAX);
+      int npad = 2;
+      while (npad < nb) npad <<= 1;
+      hipLaunchKernelGGL(sort_rows_kernel, dim3(1), dim3(1024), (size_t)npad * 8, st, csr_row, b0, nb, n_rows,
+                         ws.skey, npad);
+      KGE_LAUNCH_CHECK("sort_rows_kernel");
+      dim3 grid((unsigned)nb, 32), block(256);
+      KGE_DISPATCH_DTYPE(dtype, filter_fix_kernel, grid, block, 0, st, a, ws.skey, nb, b0, row_ptr, col, target,
+                         ws.thr, n_greater, n_equal, n_equal_lower);
+      KGE_LAUNCH_CHECK("filter_fix_kernel");
+    }
+  }
+  return KGE_OK;
+}
+
+extern "C" size_t kge_topk_workspace_bytes(int64_t B, int64_t N, int64_t k) {
+  (void)N;
+  if (B < 1) B = 1;
+  if (k < 1) k = 1;
+  if (k > TOPK_MAX_K) k = TOPK_MAX_K;
+  return topk_ws_layout(B, k, nullptr, nullptr);
+}
+
+extern "C" int kge_topk(const float* Q, const float* bias, const void* E, int dtype, const float* scale, int64_t B,
+                        int64_t d, int64_t N, int64_t k, float* out_scores, int64_t* out_idx, int apply_sigmoid,
+                        void* workspace, size_t workspace_bytes, void* stream) {
+  clear_error();
+  int rc = check_contract("kge_topk", Q, E, dtype, scale, B, d, N);
+  if (rc) return rc;
+  KGE_REQUIRE(k >= 1 && k <= N, KGE_ERR_INVALID, "kge_topk: k=%lld outside [1, N=%lld]", (long long)k, (long long)N);
+  KGE_REQUIRE(k <= TOPK_MAX_K, KGE_ERR_UNSUPPORTED, "kge_topk: k=%lld above the supported maximum %d", (long long)k,
+              TOPK_MAX_K);
+  if (B == 0) return KGE_OK;
+  KGE_REQUIRE(out_scores && out_idx, KGE_ERR_INVALID, "kge_topk: null output pointer");
+  KGE_REQUIRE(workspace && workspace_bytes >= kge_topk_workspace_bytes(B, N, k), KGE_ERR_WORKSPACE,
+              "kge_topk: workspace of %zu bytes, need %zu", workspace_bytes, kge_topk_workspace_bytes(B, N, k));
+  hipStream_t st = (hipStream_t)stream;
+  TopkWs ws;
+  topk_ws_layout(B, k, workspace, &ws);
+  hipLaunchKernelGGL(topk_init_kernel, dim3((unsigned)((B + 255) / 256)), dim3(256), 0, st, ws, B);
+  KGE_LAUNCH_CHECK("topk_init_kernel");
+
+  const size_t sel_lds = 8192 * sizeof(unsigned long long);  // kpad (<= 1024) + TOPK_CAP, padded to a power of two
+  const int64_t growth = (k <= 256) ? 4 : 2;  // round r scans (growth - 1) x what is already ranked
+  int64_t e0 = 0, e1 = (N < TOPK_FIRST_ROWS) ? N : TOPK_FIRST_ROWS;
+  while (e0 < N) {
+    ContractArgs a = make_args(Q, E, dtype, scale, B, d, N, e0, e1);
+    TopkArgs ea{ws.tau, nullptr, ws.cnt, ws.cand, TOPK_CAP};
+    rc = launch_contract<TopkEpi>(dtype, a, ea, st, "kge_topk scan");
+    if (rc) return rc;
+    hipLaunchKernelGGL(topk_select_kernel, dim3((unsigned)B), dim3(256), sel_lds, st, ws, (int)k, 0);
+    KGE_LAUNCH_CHECK("topk_select_kernel");
+    e0 = e1;
+    int64_t next = e1 * growth;
+    e1 = (next < N) ? next : N;
+  }
+  // queries whose candidate buffer overflowed in some round lost entries: rescan with their final
+  // (tight) threshold until nothing overflows.
+  int32_t n_dirty = 0;
+  KGE_HIP_CHECK(hipMemcpyAsync(&n_dirty, ws.n_dirty, sizeof(int32_t), hipMemcpyDeviceToHost, st));
+  KGE_HIP_CHECK(hipStreamSynchronize(st));
+  for (int iter = 0; n_dirty > 0 && iter < 16; ++iter) {
+    ContractArgs a = make_args(Q, E, dtype, scale, B, d, N, 0, N);
+    TopkArgs ea{ws.tau, ws.dirty, ws.cnt, ws.cand, TOPK_CAP};
+    rc = launch_contract<TopkEpi>(dtype, a, ea, st, "kge_topk rescan");
+    if (rc) return rc;
+    hipLaunchKernelGGL(topk_select_kernel, dim3((unsigned)B), dim3(256), sel_lds, st, ws, (int)k, 1);
+    KGE_LAUNCH_CHECK("topk_select_kernel");
+    KGE_HIP_CHECK(hipMemcpyAsync(&n_dirty, ws.n_dirty, sizeof(int32_t), hipMemcpyDeviceToHost, st));
+    KGE_HIP_CHECK(hipStreamSynchronize(st));
+  }
+  KGE_REQUIRE(n_dirty == 0, KGE_ERR_OVERFLOW, "kge_topk: %d queries still overflow their candidate buffers", n_dirty);
+  const int64_t total = B * k;
+  hipLaunchKernelGGL(topk_output_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, ws, B, (int)k, bias,
+                     apply_sigmoid, out_scores, out_idx);
+  KGE_LAUNCH_CHECK("topk_output_kernel");
+  return KGE_OK;
+}
+
+extern "C" size_t kge_bce_workspace_bytes(void) { return 256; }
+
+extern "C" int kge_bce_multihot(const float* Q, const float* bias, const void* E, int dtype, const float* scale,
+                                int64_t B, int64_t d, int64_t N, const int64_t* csr_row, const int64_t* row_ptr,
+                                const int32_t* col, int64_t n_rows, float label_smoothing, float* loss,
+                                void* workspace, size_t workspace_bytes, void* stream) {
+  clear_error();
+  int rc = check_contract("kge_bce_multihot", Q, E, dtype, scale, B, d, N);
+  if (rc) return rc;
+  KGE_REQUIRE(B >= 1, KGE_ERR_INVALID, "kge_bce_multihot: empty batch");
+  KGE_REQUIRE(loss, KGE_ERR_INVALID, "kge_bce_multihot: null loss pointer");
+  KGE_REQUIRE(!csr_row || (row_ptr && col), KGE_ERR_INVALID, "kge_bce_multihot: csr_row given without row_ptr / col");
+  KGE_REQUIRE(workspace && workspace_bytes >= kge_bce_workspace_bytes(), KGE_ERR_WORKSPACE,
+              "kge_bce_multihot: workspace of %zu bytes, need %zu", workspace_bytes, kge_bce_workspace_bytes());
+  KGE_REQUIRE(((uintptr_t)workspace & 7) == 0, KGE_ERR_WORKSPACE, "kge_bce_multihot: workspace must be 8-byte aligned");
+  hipStream_t st = (hipStream_t)stream;
+  double* sums = (double*)workspace;
+  hipLaunchKernelGGL(bce_init_kernel, dim3(1), dim3(64), 0, st, sums);
+  KGE_LAUNCH_CHECK("bce_init_kernel");
+  ContractArgs a = make_args(Q, E, dtype, scale, B, d, N, 0, N);
+  BceArgs ea{bias, sums, label_smoothing != 0.f ? 1 : 0};
+  rc = launch_contract<BceEpi>(dtype, a, ea, st, "kge_bce_multihot");
+  if (rc) return rc;
+  if (csr_row && n_rows > 0) {
+    dim3 grid((unsigned)((B + 3) / 4)), block(256);
+    KGE_DISPATCH_DTYPE(dtype, bce_pos_kernel, grid, block, 0, st, a, bias, csr_row, row_ptr, col, n_rows, sums);
+    KGE_LAUNCH_CHECK("bce_pos_kernel");
+  }
+  hipLaunchKernelGGL(bce_final_kernel, dim3(1), dim3(64), 0, st, sums, (double)B, (double)N, label_smoothing, loss);
+  KGE_LAUNCH_CHECK("bce_final_kernel");
+  return KGE_OK;
+}

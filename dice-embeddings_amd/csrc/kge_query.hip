@@ -1,0 +1,241 @@
+// Gather of head / relation rows fused with the model interaction -> one query vector per pair.
+// One wavefront per (head, relation) pair; both rows are staged in LDS as fp32, normalised
+// there if requested, and combined into Q[b, :] (and the per-row scalar bias of Keci).
+#include "kge_internal.h"
+
+namespace kge {
+namespace {
+
+struct QueryArgs {
+  const void* ent;
+  const float* ent_scale;
+  const void* rel;
+  const float* coeff_p;
+  const float* coeff_q;
+  const int64_t* hr;
+  float* Q;
+  float* bias;
+  kge_norm_params norm;
+  int64_t B, N, R;
+  int d, p, q, normalize_relation;
+};
+
+template <int DT>
+__device__ __forceinline__ float load_elem(const void* base, int64_t row, int d, int k, const float* scale) {
+  if (DT == KGE_F32) return ((const float*)base)[row * d + k];
+  if (DT == KGE_BF16) {
+    uint32_t u = ((const uint16_t*)base)[row * d + k];
+    return __uint_as_float(u << 16);
+  }
+  return (float)((const int8_t*)base)[row * d + k] * scale[row];
+}
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = 32; o >= 1; o >>= 1) v += __shfl_xor(v, o, 64);
+  return v;
+}
+
+__device__ void normalise_row(float* x, int d, int lane, int kind, float eps, const float* a, const float* b) {
+  if (kind == KGE_NORM_LAYERNORM) {
+    float s = 0.f;
+    for (int k = lane; k < d; k += 64) s += x[k];
+    float mu = wave_sum(s) / (float)d;
+    float v = 0.f;
+    for (int k = lane; k < d; k += 64) {
+      float t = x[k] - mu;
+      v += t * t;
+    }
+    float var = wave_sum(v) / (float)d;
+    float inv = 1.0f / sqrtf(var + eps);
+    for (int k = lane; k < d; k += 64) x[k] = (x[k] - mu) * inv * a[k] + b[k];
+  } else if (kind == KGE_NORM_BATCHNORM1D) {
+    for (int k = lane; k < d; k += 64) x[k] = (x[k] - a[k]) / sqrtf(b[k] + eps);
+  }
+}
+
+template <int EDT, int RDT>
+__global__ void __launch_bounds__(64) build_query_kernel(QueryArgs a, int model) {
+  extern __shared__ float lds[];
+  const int d = a.d;
+  float* sh = lds;
+  float* sr = lds + d;
+  const int lane = threadIdx.x;
+  const int64_t b = blockIdx.x;
+  const int64_t h_id = a.hr[2 * b], r_id = a.hr[2 * b + 1];
+  float* q = a.Q + b * d;
+  if (h_id < 0 || h_id >= a.N || r_id < 0 || r_id >= a.R) {
+    const float nan = __uint_as_float(0x7fc00000u);
+    for (int k = lane; k < d; k += 64) q[k] = nan;
+    if (lane == 0) a.bias[b] = nan;
+    return;
+  }
+  for (int k = lane; k < d; k += 64) {
+    sh[k] = load_elem<EDT>(a.ent, h_id, d, k, a.ent_scale);
+    sr[k] = load_elem<RDT>(a.rel, r_id, d, k, nullptr);
+  }
+  __syncthreads();
+  if (a.norm.kind != KGE_NORM_NONE) {
+    normalise_row(sh, d, lane, a.norm.kind, a.norm.eps, a.norm.h_a, a.norm.h_b);
+    normalise_row(sr, d, lane, a.norm.kind, a.norm.eps, a.norm.r_a, a.norm.r_b);
+    __syncthreads();
+  }
+  float bias = 0.f;
+  if (model == KGE_DISTMULT) {
+    for (int k = lane; k < d; k += 64) q[k] = sh[k] * sr[k];
+  } else if (model == KGE_COMPLEX) {
+    const int d2 = d >> 1;
+    for (int k = lane; k < d2; k += 64) {
+      float hr_ = sh[k], hi_ = sh[k + d2], rr_ = sr[k], ri_ = sr[k + d2];
+      q[k] = hr_ * rr_ - hi_ * ri_;
+      q[k + d2] = hr_ * ri_ + hi_ * rr_;
+    }
+  } else if (model == KGE_QMULT) {
+    if (a.normalize_relation) {
+      // groups of 4 consecutive elements, x / max(||x||, 1e-12)
+      for (int g = lane; g < (d >> 2); g += 64) {
+        float x0 = sr[4 * g], x1 = sr[4 * g + 1], x2 = sr[4 * g + 2], x3 = sr[4 * g + 3];
+        float n = sqrtf(x0 * x0 + x1 * x1 + x2 * x2 + x3 * x3);
+        float den = fmaxf(n, 1e-12f);
+        sr[4 * g] = x0 / den;
+        sr[4 * g + 1] = x1 / den;
+        sr[4 * g + 2] = x2 / den;
+        sr[4 * g + 3] = x3 / den;
+      }
+      __syncthreads();
+    }
+    const int d4 = d >> 2;
+    for (int g = lane; g < d4; g += 64) {
+      float ah = sh[g], bh = sh[g + d4], ch = sh[g + 2 * d4], dh = sh[g + 3 * d4];
+      float ar = sr[g], br = sr[g + d4], cr = sr[g + 2 * d4], dr = sr[g + 3 * d4];
+      q[g] = ah * ar - bh * br - ch * cr - dh * dr;
+      q[g + d4] = ah * br + bh * ar + ch * dr - dh * cr;
+      q[g + 2 * d4] = ah * cr - bh * dr + ch * ar + dh * br;
+      q[g + 3 * d4] = ah * dr + bh * cr - ch * br + dh * ar;
+    }
+  } else {  // KGE_KECI
+    const int p = a.p, qn = a.q;
+    const int r = d / (p + qn + 1);
+    // scale the p / q parts of both rows by their coefficients first, as the reference does
+    for (int k = lane; k < r * p; k += 64) {
+      float c = a.coeff_p[k % p];
+      sh[r + k] *= c;
+      sr[r + k] *= c;
+    }
+    const int qoff = r + r * p;
+    for (int k = lane; k < r * qn; k += 64) {
+      float c = a.coeff_q[k % qn];
+      sh[qoff + k] *= c;
+      sr[qoff + k] *= c;
+    }
+    __syncthreads();
+    for (int rho = lane; rho < r; rho += 64) {
+      const float h0 = sh[rho], r0 = sr[rho];
+      const float* hp = sh + r + rho * p;
+      const float* rp = sr + r + rho * p;
+      const float* hq = sh + qoff + rho * qn;
+      const float* rq = sr + qoff + rho * qn;
+      float q0 = h0 * r0;
+      for (int i = 0; i < p; ++i) {
+        q0 += hp[i] * rp[i];
+        q[r + rho * p + i] = h0 * rp[i] + hp[i] * r0;
+      }
+      for (int j = 0; j < qn; ++j) {
+        q0 -= hq[j] * rq[j];
+        q[qoff + rho * qn + j] = h0 * rq[j] + hq[j] * r0;
+      }
+      q[rho] = q0;
+      if (p >= 2)
+        for (int i = 0; i < p - 1; ++i)
+          for (int k = i + 1; k < p; ++k) bias += hp[i] * rp[k] - hp[k] * rp[i];
+      if (qn >= 2)
+        for (int j = 0; j < qn - 1; ++j)
+          for (int k = j + 1; k < qn; ++k) bias += hq[j] * rq[k] - hq[k] * rq[j];
+      if (p >= 2 && qn >= 2)
+        for (int i = 0; i < p; ++i)
+          for (int j = 0; j < qn; ++j) bias += hp[i] * rq[j] - hq[j] * rp[i];
+    }
+    bias = wave_sum(bias);
+  }
+  if (lane == 0) a.bias[b] = bias;
+}
+
+template <int EDT>
+int launch_build_query(const QueryArgs& a, int model, int rel_dtype, hipStream_t st) {
+  dim3 grid((unsigned)a.B), block(64);
+  size_t shmem = 2 * (size_t)a.d * sizeof(float);
+  if (rel_dtype == KGE_F32)
+    hipLaunchKernelGGL((build_query_kernel<EDT, KGE_F32>), grid, block, shmem, st, a, model);
+  else
+    hipLaunchKernelGGL((build_query_kernel<EDT, KGE_BF16>), grid, block, shmem, st, a, model);
+  KGE_LAUNCH_CHECK("build_query_kernel");
+  return KGE_OK;
+}
+
+}  // namespace
+}  // namespace kge
+
+extern "C" int kge_build_query(int model, int p, int q, const void* ent, int ent_dtype, const float* ent_scale,
+                               const void* rel, int rel_dtype, const float* coeff_p, const float* coeff_q,
+                               int normalize_relation, const kge_norm_params* norm, const int64_t* hr,
+                               int64_t B, int64_t d, int64_t N, int64_t R, float* Q, float* bias, void* stream) {
+  using namespace kge;
+  clear_error();
+  KGE_REQUIRE(B >= 0 && N > 0 && R > 0, KGE_ERR_INVALID, "kge_build_query: B=%lld N=%lld R=%lld", (long long)B,
+              (long long)N, (long long)R);
+  if (B == 0) return KGE_OK;
+  KGE_REQUIRE(ent && rel && hr && Q && bias, KGE_ERR_INVALID, "kge_build_query: null pointer argument");
+  KGE_REQUIRE(d >= 1 && d <= 8192, KGE_ERR_INVALID, "kge_build_query: d=%lld outside [1, 8192]", (long long)d);
+  KGE_REQUIRE(B <= 0x7fffffff, KGE_ERR_INVALID, "kge_build_query: B=%lld too large", (long long)B);
+  KGE_REQUIRE(ent_dtype == KGE_F32 || ent_dtype == KGE_BF16 || ent_dtype == KGE_I8, KGE_ERR_INVALID,
+              "kge_build_query: unknown entity dtype %d", ent_dtype);
+  KGE_REQUIRE(rel_dtype == KGE_F32 || rel_dtype == KGE_BF16, KGE_ERR_INVALID,
+              "kge_build_query: relation dtype must be f32 or bf16, got %d", rel_dtype);
+  KGE_REQUIRE(ent_dtype != KGE_I8 || ent_scale, KGE_ERR_INVALID, "kge_build_query: int8 entities need ent_scale");
+  switch (model) {
+    case KGE_DISTMULT: break;
+    case KGE_COMPLEX:
+      KGE_REQUIRE(d % 2 == 0, KGE_ERR_INVALID, "kge_build_query: ComplEx needs even d, got %lld", (long long)d);
+      break;
+    case KGE_QMULT:
+      KGE_REQUIRE(d % 4 == 0, KGE_ERR_INVALID, "kge_build_query: QMult needs d %% 4 == 0, got %lld", (long long)d);
+      break;
+    case KGE_KECI:
+      KGE_REQUIRE(p >= 0 && q >= 0 && d % (p + q + 1) == 0, KGE_ERR_INVALID,
+                  "kge_build_query: Keci needs d / (p + q + 1) whole, got d=%lld p=%d q=%d", (long long)d, p, q);
+      KGE_REQUIRE((p == 0 || coeff_p) && (q == 0 || coeff_q), KGE_ERR_INVALID,
+                  "kge_build_query: Keci with p=%d q=%d needs coefficient vectors", p, q);
+      break;
+    default: return set_error(KGE_ERR_INVALID, "kge_build_query: unknown model %d", model);
+  }
+  QueryArgs a;
+  a.ent = ent;
+  a.ent_scale = ent_scale;
+  a.rel = rel;
+  a.coeff_p = coeff_p;
+  a.coeff_q = coeff_q;
+  a.hr = hr;
+  a.Q = Q;
+  a.bias = bias;
+  a.norm.kind = KGE_NORM_NONE;
+  a.norm.eps = 0.f;
+  a.norm.h_a = a.norm.h_b = a.norm.r_a = a.norm.r_b = nullptr;
+  if (norm && norm->kind != KGE_NORM_NONE) {
+    KGE_REQUIRE(norm->kind == KGE_NORM_LAYERNORM || norm->kind == KGE_NORM_BATCHNORM1D, KGE_ERR_INVALID,
+                "kge_build_query: unknown normalisation %d", norm->kind);
+    KGE_REQUIRE(norm->h_a && norm->h_b && norm->r_a && norm->r_b, KGE_ERR_INVALID,
+                "kge_build_query: normalisation parameters missing");
+    a.norm = *norm;
+  }
+  a.B = B;
+  a.N = N;
+  a.R = R;
+  a.d = (int)d;
+  a.p = p;
+  a.q = q;
+  a.normalize_relation = normalize_relation;
+  hipStream_t st = (hipStream_t)stream;
+  if (ent_dtype == KGE_F32) return launch_build_query<KGE_F32>(a, model, rel_dtype, st);
+  if (ent_dtype == KGE_BF16) return launch_build_query<KGE_BF16>(a, model, rel_dtype, st);
+  return launch_build_query<KGE_I8>(a, model, rel_dtype, st);
+}

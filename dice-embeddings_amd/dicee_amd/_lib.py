@@ -1,0 +1,71 @@
+"""ctypes binding of ``libkge_hip.so`` (C ABI declared in ``include/kge_hip.h``)."""
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libkge_hip.so")
+
+KGE_OK = 0
+MODEL_IDS = {"DistMult": 0, "ComplEx": 1, "QMult": 2, "Keci": 3, "CKeci": 3}
+DTYPE_F32, DTYPE_BF16, DTYPE_I8 = 0, 1, 2
+NORM_NONE, NORM_LAYERNORM, NORM_BATCHNORM1D = 0, 1, 2
+
+_c_i64 = ctypes.c_int64
+_c_int = ctypes.c_int
+_c_f = ctypes.c_float
+_vp = ctypes.c_void_p
+_sz = ctypes.c_size_t
+
+
+class NormParams(ctypes.Structure):
+    _fields_ = [("kind", ctypes.c_int32), ("eps", ctypes.c_float),
+                ("h_a", _vp), ("h_b", _vp), ("r_a", _vp), ("r_b", _vp)]
+
+
+SIGNATURES = {
+    "kge_last_error": (ctypes.c_char_p, []),
+    "kge_abi_version": (_c_int, []),
+    "kge_build_query": (_c_int, [_c_int, _c_int, _c_int, _vp, _c_int, _vp, _vp, _c_int, _vp, _vp, _c_int,
+                                 ctypes.POINTER(NormParams), _vp, _c_i64, _c_i64, _c_i64, _c_i64, _vp, _vp, _vp]),
+    "kge_scores": (_c_int, [_vp, _vp, _vp, _c_int, _vp, _c_i64, _c_i64, _c_i64, _vp, _c_i64, _vp]),
+    "kge_rank_workspace_bytes": (_sz, [_c_i64]),
+    "kge_rank_filtered": (_c_int, [_vp, _vp, _vp, _c_int, _vp, _c_i64, _c_i64, _c_i64, _vp, _vp, _vp, _vp, _c_i64,
+                                   _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
+    "kge_topk_workspace_bytes": (_sz, [_c_i64, _c_i64, _c_i64]),
+    "kge_topk": (_c_int, [_vp, _vp, _vp, _c_int, _vp, _c_i64, _c_i64, _c_i64, _c_i64, _vp, _vp, _c_int, _vp, _sz,
+                          _vp]),
+    "kge_bce_workspace_bytes": (_sz, []),
+    "kge_bce_multihot": (_c_int, [_vp, _vp, _vp, _c_int, _vp, _c_i64, _c_i64, _c_i64, _vp, _vp, _vp, _c_i64, _c_f,
+                                  _vp, _vp, _sz, _vp]),
+}
+
+_lib = None
+
+
+class KgeError(RuntimeError):
+    def __init__(self, code, text):
+        super().__init__(f"libkge_hip error {code}: {text}")
+        self.code = code
+
+
+def load():
+    """Load the HIP library; raises if it has not been built (there is no fallback path)."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError(
+            f"{LIB_PATH} is missing: build it with `python -m dicee_amd.build` "
+            "(hipcc --offload-arch=gfx950). There is no CPU fallback for the scoring path.")
+    lib = ctypes.CDLL(LIB_PATH)
+    for name, (res, args) in SIGNATURES.items():
+        fn = getattr(lib, name)
+        fn.restype = res
+        fn.argtypes = args
+    _lib = lib
+    return lib
+
+
+def check(rc):
+    if rc != KGE_OK:
+        raise KgeError(rc, load().kge_last_error().decode("utf-8", "replace"))

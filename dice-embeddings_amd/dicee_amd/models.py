@@ -1,0 +1,235 @@
+"""Model containers with the reference's KvsAll call surface, backed by the HIP kernels.
+
+Parameter names follow dicee so that a dicee ``model.pt`` state_dict loads unchanged
+(``entity_embeddings.weight``, ``relation_embeddings.weight``, Keci's ``p_coefficients.weight`` /
+``q_coefficients.weight``, ``normalize_*_embeddings.*``): dicee/models/base_model.py:121-176,
+dicee/models/clifford.py:4-28.
+
+Only the inference-time semantics of the path are implemented: dropout is the identity
+(base_model.py:149-151 in eval mode) and BatchNorm1d uses its running statistics.
+"""
+import torch
+
+from . import ops
+
+
+class IdentityClass(torch.nn.Module):
+    """dicee/models/base_model.py:441-450; QMult also uses it as a type test (quaternion.py:138)."""
+
+    def __init__(self, args=None):
+        super().__init__()
+        self.args = args
+
+    @staticmethod
+    def forward(x):
+        return x
+
+
+class BaseKGE(torch.nn.Module):
+    name = "BaseKGE"
+
+    def __init__(self, args: dict):
+        super().__init__()
+        self.args = dict(args)
+        self.embedding_dim = int(args["embedding_dim"])
+        self.num_entities = int(args["num_entities"])
+        self.num_relations = int(args["num_relations"])
+        self.input_dropout_rate = float(args.get("input_dropout_rate", 0.0) or 0.0)
+        self.loss = torch.nn.BCEWithLogitsLoss()
+        self.normalize_head_entity_embeddings = IdentityClass()
+        self.normalize_relation_embeddings = IdentityClass()
+        self.hidden_normalizer = IdentityClass()
+        norm = args.get("normalization")
+        if norm == "LayerNorm":
+            self.normalize_head_entity_embeddings = torch.nn.LayerNorm(self.embedding_dim)
+            self.normalize_relation_embeddings = torch.nn.LayerNorm(self.embedding_dim)
+        elif norm == "BatchNorm1d":
+            self.normalize_head_entity_embeddings = torch.nn.BatchNorm1d(self.embedding_dim, affine=False)
+            self.normalize_relation_embeddings = torch.nn.BatchNorm1d(self.embedding_dim, affine=False)
+        elif norm is not None:
+            raise NotImplementedError(norm)
+        self.entity_embeddings = torch.nn.Embedding(self.num_entities, self.embedding_dim)
+        self.relation_embeddings = torch.nn.Embedding(self.num_relations, self.embedding_dim)
+        self._storage = "fp32"
+        self._table = None       # quantised / bf16 copy of the entity table
+        self._scale = None
+        self._rel_table = None
+
+    # ------------------------------------------------------------------ storage
+    def set_entity_storage(self, kind="fp32"):
+        """Keep the tables the kernels read as ``fp32`` (the parameters themselves), ``bf16``
+        (entities and relations rounded to bf16) or ``int8`` (entities per-row symmetric int8 with
+        an fp32 scale per row, relations fp32).  Scores then follow fp32 math on the dequantised
+        table."""
+        w = self.entity_embeddings.weight.detach()
+        if kind == "fp32":
+            self._table = self._scale = self._rel_table = None
+        elif kind == "bf16":
+            self._table = w.to(torch.bfloat16).contiguous()
+            self._scale = None
+            self._rel_table = self.relation_embeddings.weight.detach().to(torch.bfloat16).contiguous()
+        elif kind == "int8":
+            amax = w.abs().amax(dim=1)
+            scale = (amax / 127.0).to(torch.float32)
+            safe = torch.where(scale > 0, scale, torch.ones_like(scale))
+            self._table = torch.round(w / safe[:, None]).clamp(-127, 127).to(torch.int8).contiguous()
+            self._scale = scale.contiguous()
+            self._rel_table = None
+        else:
+            raise ValueError(kind)
+        self._storage = kind
+        return self
+
+    def table(self):
+        """(entity table the kernels read, per-row scale or None)."""
+        if self._table is not None:
+            return self._table, self._scale
+        return self.entity_embeddings.weight.detach(), None
+
+    def _rel(self):
+        return self._rel_table if self._rel_table is not None else self.relation_embeddings.weight.detach()
+
+    # ------------------------------------------------------------------ query construction
+    def _norm_params(self):
+        nh, nr = self.normalize_head_entity_embeddings, self.normalize_relation_embeddings
+        if isinstance(nh, torch.nn.LayerNorm):
+            return {"kind": "LayerNorm", "eps": nh.eps, "h_a": nh.weight.detach(), "h_b": nh.bias.detach(),
+                    "r_a": nr.weight.detach(), "r_b": nr.bias.detach()}
+        if isinstance(nh, torch.nn.BatchNorm1d):
+            return {"kind": "BatchNorm1d", "eps": nh.eps, "h_a": nh.running_mean, "h_b": nh.running_var,
+                    "r_a": nr.running_mean, "r_b": nr.running_var}
+        return None
+
+    def _query_kwargs(self):
+        return {}
+
+    def query(self, x):
+        """(Q [B,d], bias [B]) for ``x`` [B,2]: gather + interaction
+        (get_head_relation_representation, base_model.py:377-384, then the model's elementwise part)."""
+        E, scale = self.table()
+        x = x.to(device=E.device, dtype=torch.int64).contiguous()
+        return ops.build_query(self.name if self.name != "CKeci" else "Keci", E, self._rel(), x, ent_scale=scale,
+                               norm=self._norm_params(), **self._query_kwargs())
+
+    # ------------------------------------------------------------------ reference call surface
+    def forward(self, x, y_idx=None):
+        """Shape dispatch of BaseKGE.forward (base_model.py:310-344); only the KvsAll case is built."""
+        if isinstance(x, tuple):
+            raise NotImplementedError("forward_k_vs_sample is outside the accelerated path")
+        if x.dim() == 2 and x.shape[1] == 2:
+            return self.forward_k_vs_all(x=x)
+        if x.dim() == 2 and x.shape[1] == 3:
+            raise NotImplementedError("forward_triples is outside the accelerated path")
+        raise NotImplementedError("byte-pair-encoded inputs are outside the accelerated path")
+
+    def forward_k_vs_all(self, x):
+        """[B,N] fp32 scores of every entity as tail; the caller owns (and may mutate) the result."""
+        Q, bias = self.query(x)
+        E, scale = self.table()
+        return ops.scores(Q, bias, E, scale)
+
+    def k_vs_all_score(self, emb_h, emb_r, emb_E):
+        """Scores from already gathered rows: [B,d],[B,d],[N,d] -> [B,N]."""
+        B = emb_h.shape[0]
+        idx = torch.arange(B, device=emb_h.device, dtype=torch.int64)
+        hr = torch.stack([idx, idx], dim=1).contiguous()
+        Q, bias = ops.build_query(self.name if self.name != "CKeci" else "Keci", emb_h.contiguous().float(),
+                                  emb_r.contiguous().float(), hr, **self._query_kwargs())
+        return ops.scores(Q, bias, emb_E.contiguous().float())
+
+    # ------------------------------------------------------------------ fused consumers
+    def rank_filtered(self, x, target, csr=None):
+        """Fused filtered-rank counters for queries ``x`` [B,2] and true tails ``target`` [B]."""
+        Q, bias = self.query(x)
+        E, scale = self.table()
+        target = target.to(device=E.device, dtype=torch.int64).contiguous()
+        if csr is None:
+            return ops.rank_filtered(Q, bias, E, scale, target)
+        rows = csr.rows_for(x.to(device=E.device, dtype=torch.int64))
+        return ops.rank_filtered(Q, bias, E, scale, target, rows, csr.row_ptr, csr.col)
+
+    def topk(self, x, k, sigmoid=False):
+        Q, bias = self.query(x)
+        E, scale = self.table()
+        return ops.topk(Q, bias, E, scale, k, sigmoid=sigmoid)
+
+    def kvsall_bce_loss(self, x, csr, label_smoothing=0.0):
+        """Forward + loss of training_step (base_model.py:25-46) for a KvsAll batch whose multi-hot
+        target is given by the CSR rows of ``x`` (dataset_classes.py:354-361)."""
+        Q, bias = self.query(x)
+        E, scale = self.table()
+        rows = csr.rows_for(x.to(device=E.device, dtype=torch.int64))
+        return ops.bce_multihot(Q, bias, E, scale, rows, csr.row_ptr, csr.col, label_smoothing)[0]
+
+
+class DistMult(BaseKGE):
+    """dicee/models/real.py:10-36."""
+    name = "DistMult"
+
+
+class ComplEx(BaseKGE):
+    """dicee/models/complex.py:223-269."""
+    name = "ComplEx"
+
+
+class QMult(BaseKGE):
+    """dicee/models/quaternion.py:24-171."""
+    name = "QMult"
+
+    def _query_kwargs(self):
+        # the quaternion normaliser runs only when no other relation normaliser is set (quaternion.py:138)
+        return {"normalize_relation": isinstance(self.normalize_relation_embeddings, IdentityClass)}
+
+
+class Keci(BaseKGE):
+    """dicee/models/clifford.py:3-329."""
+    name = "Keci"
+
+    def __init__(self, args):
+        super().__init__(args)
+        self.p = int(args.get("p", 0) or 0)
+        self.q = int(args.get("q", 0) or 0)
+        r = self.embedding_dim / (self.p + self.q + 1)
+        if not float(r).is_integer():
+            raise AssertionError(f"r = embedding_dim / (p + q+ 1) must be a whole number\n"
+                                 f"Currently {r}={self.embedding_dim} / ({self.p}+ {self.q} +1)")
+        self.r = int(r)
+        if self.p > 0:
+            self.p_coefficients = torch.nn.Embedding(num_embeddings=1, embedding_dim=self.p)
+            torch.nn.init.zeros_(self.p_coefficients.weight)
+        if self.q > 0:
+            self.q_coefficients = torch.nn.Embedding(num_embeddings=1, embedding_dim=self.q)
+            torch.nn.init.zeros_(self.q_coefficients.weight)
+
+    def _query_kwargs(self):
+        kw = {"p": self.p, "q": self.q}
+        if self.p > 0:
+            kw["coeff_p"] = self.p_coefficients.weight.detach().reshape(-1).float().contiguous()
+        if self.q > 0:
+            kw["coeff_q"] = self.q_coefficients.weight.detach().reshape(-1).float().contiguous()
+        return kw
+
+
+class CKeci(Keci):
+    """Keci without learned dimension scaling (clifford.py:563-576)."""
+    name = "CKeci"
+
+    def __init__(self, args):
+        super().__init__(args)
+        if self.p > 0:
+            torch.nn.init.ones_(self.p_coefficients.weight)
+            self.p_coefficients.weight.requires_grad_(False)
+        if self.q > 0:
+            torch.nn.init.ones_(self.q_coefficients.weight)
+            self.q_coefficients.weight.requires_grad_(False)
+
+
+MODEL_REGISTRY = {"DistMult": DistMult, "ComplEx": ComplEx, "QMult": QMult, "Keci": Keci, "CKeci": CKeci}
+
+
+def initialize_model(args: dict):
+    """(model, 'EntityPrediction') as dicee.static_funcs.intialize_model (static_funcs.py:483-509)."""
+    name = args["model"]
+    if name not in MODEL_REGISTRY:
+        raise ValueError(f"--model_name: {name} is not found.")
+    return MODEL_REGISTRY[name](args), "EntityPrediction"

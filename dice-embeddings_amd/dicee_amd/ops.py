@@ -1,0 +1,142 @@
+"""Tensor-level wrappers of the C ABI.  torch is used for device memory and streams only."""
+import ctypes
+
+import torch
+
+from . import _lib
+from ._lib import MODEL_IDS, DTYPE_F32, DTYPE_BF16, DTYPE_I8, NormParams
+
+_TORCH_TO_KGE = {torch.float32: DTYPE_F32, torch.bfloat16: DTYPE_BF16, torch.int8: DTYPE_I8}
+
+
+def _require_gpu(*tensors):
+    for t in tensors:
+        if t is None:
+            continue
+        if not t.is_cuda:
+            raise RuntimeError("dicee_amd ops need tensors on the GPU (there is no CPU path)")
+        if not t.is_contiguous():
+            raise ValueError("dicee_amd ops need contiguous tensors")
+
+
+def _ptr(t):
+    return None if t is None else ctypes.c_void_p(t.data_ptr())
+
+
+def _stream():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _table_dtype(E):
+    try:
+        return _TORCH_TO_KGE[E.dtype]
+    except KeyError:
+        raise TypeError(f"unsupported table dtype {E.dtype}; use float32, bfloat16 or int8") from None
+
+
+def _norm_struct(norm):
+    """norm: None or dict(kind='LayerNorm'|'BatchNorm1d', h_a, h_b, r_a, r_b, eps) of fp32 GPU tensors."""
+    if norm is None:
+        return None, ()
+    kind = {"LayerNorm": _lib.NORM_LAYERNORM, "BatchNorm1d": _lib.NORM_BATCHNORM1D}[norm["kind"]]
+    keep = tuple(norm[k].contiguous().float() for k in ("h_a", "h_b", "r_a", "r_b"))
+    _require_gpu(*keep)
+    s = NormParams(kind, float(norm.get("eps", 1e-5)), *[t.data_ptr() for t in keep])
+    return s, keep
+
+
+def build_query(model, ent, rel, hr, *, ent_scale=None, p=0, q=0, coeff_p=None, coeff_q=None,
+                normalize_relation=True, norm=None):
+    """(Q [B,d] fp32, bias [B] fp32) with ``forward_k_vs_all(x) == Q @ E^T + bias[:, None]``."""
+    lib = _lib.load()
+    _require_gpu(ent, rel, hr, ent_scale, coeff_p, coeff_q)
+    if hr.dtype != torch.int64 or hr.dim() != 2 or hr.shape[1] != 2:
+        raise ValueError("hr must be an int64 tensor of shape [B, 2]")
+    B, (N, d), R = hr.shape[0], ent.shape, rel.shape[0]
+    if rel.shape[1] != d:
+        raise ValueError("entity and relation tables must have the same embedding dim")
+    Q = torch.empty((B, d), dtype=torch.float32, device=ent.device)
+    bias = torch.empty((B,), dtype=torch.float32, device=ent.device)
+    ns, keep = _norm_struct(norm)
+    rc = lib.kge_build_query(MODEL_IDS[model], int(p), int(q), _ptr(ent), _table_dtype(ent), _ptr(ent_scale),
+                             _ptr(rel), _table_dtype(rel), _ptr(coeff_p), _ptr(coeff_q), int(bool(normalize_relation)),
+                             ctypes.byref(ns) if ns is not None else None, _ptr(hr), B, d, N, R, _ptr(Q), _ptr(bias),
+                             _stream())
+    _lib.check(rc)
+    del keep
+    return Q, bias
+
+
+def scores(Q, bias, E, scale=None, out=None):
+    """Materialised [B,N] fp32 scores."""
+    lib = _lib.load()
+    _require_gpu(Q, bias, E, scale)
+    B, d = Q.shape
+    N = E.shape[0]
+    if out is None:
+        out = torch.empty((B, N), dtype=torch.float32, device=Q.device)
+    _require_gpu(out)
+    rc = lib.kge_scores(_ptr(Q), _ptr(bias), _ptr(E), _table_dtype(E), _ptr(scale), B, d, N, _ptr(out),
+                        out.stride(0) if B > 0 else N, _stream())
+    _lib.check(rc)
+    return out
+
+
+def rank_filtered(Q, bias, E, scale, target, csr_row=None, row_ptr=None, col=None):
+    """Fused filtered rank. Returns dict of int32 ``n_greater, n_equal, n_equal_lower`` and fp32
+    ``target_score`` (all [B])."""
+    lib = _lib.load()
+    _require_gpu(Q, bias, E, scale, target, csr_row, row_ptr, col)
+    B, d = Q.shape
+    N = E.shape[0]
+    dev = Q.device
+    out = {k: torch.empty((B,), dtype=torch.int32, device=dev) for k in ("n_greater", "n_equal", "n_equal_lower")}
+    out["target_score"] = torch.empty((B,), dtype=torch.float32, device=dev)
+    ws_bytes = lib.kge_rank_workspace_bytes(B)
+    ws = torch.empty((ws_bytes,), dtype=torch.uint8, device=dev)
+    n_rows = 0 if row_ptr is None else row_ptr.numel() - 1
+    if csr_row is not None:
+        if csr_row.dtype != torch.int64 or row_ptr.dtype != torch.int64 or col.dtype != torch.int32:
+            raise TypeError("csr_row/row_ptr must be int64 and col int32")
+    if target.dtype != torch.int64:
+        raise TypeError("target must be int64")
+    rc = lib.kge_rank_filtered(_ptr(Q), _ptr(bias), _ptr(E), _table_dtype(E), _ptr(scale), B, d, N, _ptr(target),
+                               _ptr(csr_row), _ptr(row_ptr), _ptr(col), n_rows, _ptr(out["n_greater"]),
+                               _ptr(out["n_equal"]), _ptr(out["n_equal_lower"]), _ptr(out["target_score"]), _ptr(ws),
+                               ws_bytes, _stream())
+    _lib.check(rc)
+    return out
+
+
+def topk(Q, bias, E, scale, k, sigmoid=False):
+    """Fused top-k over all entities: ([B,k] fp32 descending, [B,k] int64)."""
+    lib = _lib.load()
+    _require_gpu(Q, bias, E, scale)
+    B, d = Q.shape
+    N = E.shape[0]
+    dev = Q.device
+    out_s = torch.empty((B, k), dtype=torch.float32, device=dev)
+    out_i = torch.empty((B, k), dtype=torch.int64, device=dev)
+    ws_bytes = lib.kge_topk_workspace_bytes(B, N, k)
+    ws = torch.empty((ws_bytes,), dtype=torch.uint8, device=dev)
+    rc = lib.kge_topk(_ptr(Q), _ptr(bias), _ptr(E), _table_dtype(E), _ptr(scale), B, d, N, int(k), _ptr(out_s),
+                      _ptr(out_i), int(bool(sigmoid)), _ptr(ws), ws_bytes, _stream())
+    _lib.check(rc)
+    return out_s, out_i
+
+
+def bce_multihot(Q, bias, E, scale, csr_row, row_ptr, col, label_smoothing=0.0):
+    """Mean BCE-with-logits of the [B,N] scores against the multi-hot of the CSR rows: [1] fp32 tensor."""
+    lib = _lib.load()
+    _require_gpu(Q, bias, E, scale, csr_row, row_ptr, col)
+    B, d = Q.shape
+    N = E.shape[0]
+    loss = torch.empty((1,), dtype=torch.float32, device=Q.device)
+    ws_bytes = lib.kge_bce_workspace_bytes()
+    ws = torch.empty((ws_bytes // 8,), dtype=torch.float64, device=Q.device)
+    n_rows = 0 if row_ptr is None else row_ptr.numel() - 1
+    rc = lib.kge_bce_multihot(_ptr(Q), _ptr(bias), _ptr(E), _table_dtype(E), _ptr(scale), B, d, N, _ptr(csr_row),
+                              _ptr(row_ptr), _ptr(col), n_rows, float(label_smoothing), _ptr(loss), _ptr(ws),
+                              ws_bytes, _stream())
+    _lib.check(rc)
+    return loss

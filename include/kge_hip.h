@@ -1,0 +1,148 @@
+/*
+ * kge_hip.h - C ABI of the MI355X (gfx950) KvsAll scoring / link-prediction kernels.
+ *
+ * The reference (dicee 0.3.2) is pure Python on torch and has no FFI of its own; the seam this
+ * library sits behind is the tensor-level protocol of its models and evaluator.  Every entry
+ * point below names the reference code whose arithmetic it replaces.
+ *
+ * Conventions
+ *   - Every pointer is a DEVICE pointer owned by the caller unless stated otherwise.
+ *   - `stream` is a hipStream_t passed as void*; work is enqueued on it and, unless noted, the
+ *     call returns without waiting for it.
+ *   - Return value: KGE_OK (0) or an error code; kge_last_error() gives the thread-local text.
+ *     Arguments are validated on the host before anything is launched.
+ *   - Entity/relation ids are int64 (what torch.LongTensor holds).  Kernels never dereference an
+ *     id outside [0,N) / [0,R): such a row yields NaN scores instead of a memory fault.
+ *   - Tables are row-major [rows, d].  dtype KGE_F32 computes with fp32 MFMA; KGE_BF16 and
+ *     KGE_I8 (per-row symmetric int8 with a float scale per row) compute with bf16 MFMA and
+ *     fp32 accumulation and currently require d <= 128, d % 8 == 0 (bf16) / d % 16 == 0 (int8).
+ *   - A score is `dot(Q[b], E[e]) (* scale[e]) (+ bias[b])`.  The fp32 value of the dot product
+ *     is the same bit pattern in every entry point (fixed reduction order), so a rank computed
+ *     by kge_rank_filtered equals the rank counted on kge_scores output exactly.
+ */
+#ifndef KGE_HIP_H
+#define KGE_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define KGE_ABI_VERSION 1
+
+enum kge_status {
+  KGE_OK = 0,
+  KGE_ERR_INVALID = 1,      /* bad argument (null pointer, size, model/d mismatch, k > N ...) */
+  KGE_ERR_UNSUPPORTED = 2,  /* valid request this build has no kernel for */
+  KGE_ERR_WORKSPACE = 3,    /* workspace missing or too small */
+  KGE_ERR_HIP = 4,          /* a HIP runtime call failed */
+  KGE_ERR_OVERFLOW = 5      /* top-k candidate buffers overflowed beyond recovery */
+};
+
+enum kge_model { KGE_DISTMULT = 0, KGE_COMPLEX = 1, KGE_QMULT = 2, KGE_KECI = 3 };
+enum kge_dtype { KGE_F32 = 0, KGE_BF16 = 1, KGE_I8 = 2 };
+enum kge_norm_kind { KGE_NORM_NONE = 0, KGE_NORM_LAYERNORM = 1, KGE_NORM_BATCHNORM1D = 2 };
+
+/* Optional input normalisation of the gathered head / relation rows
+ * (dicee/models/base_model.py:283-294, applied at :381-383).
+ * LayerNorm: a = weight[d], b = bias[d].  BatchNorm1d(affine=False), eval: a = running_mean[d],
+ * b = running_var[d]. */
+typedef struct kge_norm_params {
+  int32_t kind; /* enum kge_norm_kind */
+  float eps;
+  const float* h_a;
+  const float* h_b;
+  const float* r_a;
+  const float* r_b;
+} kge_norm_params;
+
+/* Text of the last error raised on the calling thread ("" if none). */
+const char* kge_last_error(void);
+
+/* KGE_ABI_VERSION the library was built with. */
+int kge_abi_version(void);
+
+/*
+ * Gather + model interaction: one query vector per (head, relation) pair so that
+ * forward_k_vs_all(x) == Q @ E^T + bias[:, None].
+ * Replaces BaseKGE.get_head_relation_representation (dicee/models/base_model.py:377-384) and the
+ * elementwise part of k_vs_all_score of DistMult (dicee/models/real.py:32), ComplEx
+ * (dicee/models/complex.py:254-263), QMult (dicee/models/quaternion.py:138-144 with
+ * quaternion_normalizer :74-100 and quaternion_mul dicee/models/static_funcs.py:4-18) and Keci
+ * (dicee/models/clifford.py:260-304 with apply_coefficients :105-113).
+ *   ent [N,d] (ent_dtype; ent_scale [N] for KGE_I8 else NULL), rel [R,d] (KGE_F32 or KGE_BF16)
+ *   p,q,coeff_p[p],coeff_q[q]: Keci only.  normalize_relation: QMult only (1 when the model's
+ *   relation normaliser is the identity, quaternion.py:138).  norm: NULL or see above.
+ *   hr [B,2] int64.  Q [B,d] fp32 out.  bias [B] fp32 out (all zero except Keci with p>=2 or q>=2).
+ */
+int kge_build_query(int model, int p, int q, const void* ent, int ent_dtype, const float* ent_scale,
+                    const void* rel, int rel_dtype, const float* coeff_p, const float* coeff_q,
+                    int normalize_relation, const kge_norm_params* norm, const int64_t* hr,
+                    int64_t B, int64_t d, int64_t N, int64_t R, float* Q, float* bias, void* stream);
+
+/*
+ * Materialised scores S[b, e] = dot(Q[b], E[e]) (* scale[e]) (+ bias[b]); S has row stride ldS.
+ * Replaces the torch.mm / einsum calls and B x N adds of real.py:32, complex.py:260-264,
+ * quaternion.py:152-156, clifford.py:269-305.  For callers that need the whole matrix
+ * (KGE.predict, dicee/knowledge_graph_embeddings.py:404-408; model(x) itself).
+ */
+int kge_scores(const float* Q, const float* bias, const void* E, int dtype, const float* scale,
+               int64_t B, int64_t d, int64_t N, float* S, int64_t ldS, void* stream);
+
+/*
+ * Fused filtered rank: the per-row mask loop, full torch.sort and torch.where of
+ * Evaluator._evaluate_entity_prediction (dicee/evaluation/evaluator.py:484-508; same loop in
+ * dicee/evaluation/link_prediction.py:144-171) without writing the B x N scores.
+ *   target [B]: id of the true tail.  csr_row [B]: row of the filter CSR for (h,r), or -1.
+ *   row_ptr [n_rows+1] int64, col [nnz] int32: known tails per (h,r), each row sorted and
+ *   without duplicates (the target may be listed; it is never filtered, evaluator.py:494-501).
+ *   csr_row/row_ptr/col may be NULL together (no filter).
+ * Outputs, over entities not removed by the filter:
+ *   n_greater[b]     = #{e : s_e >  s_target}
+ *   n_equal[b]       = #{e != target : s_e == s_target}
+ *   n_equal_lower[b] = #{e <  target : s_e == s_target}
+ *   target_score[b]  = s_target (+ bias[b] if bias != NULL; bias does not change ranks)
+ * so the reference's rank lies in [1+n_greater, 1+n_greater+n_equal] and a stable descending
+ * sort gives 1+n_greater+n_equal_lower.
+ * workspace: kge_rank_workspace_bytes(B) bytes of device memory.
+ */
+size_t kge_rank_workspace_bytes(int64_t B);
+int kge_rank_filtered(const float* Q, const float* bias, const void* E, int dtype, const float* scale,
+                      int64_t B, int64_t d, int64_t N, const int64_t* target, const int64_t* csr_row,
+                      const int64_t* row_ptr, const int32_t* col, int64_t n_rows,
+                      int32_t* n_greater, int32_t* n_equal, int32_t* n_equal_lower,
+                      float* target_score, void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * Fused top-k over all entities: torch.topk(model(batch_hr), k, dim=1) of
+ * KGE.predict_missing_tail_entity (dicee/knowledge_graph_embeddings.py:397-401) and, with
+ * apply_sigmoid, the torch.sigmoid of KGE.predict_topk (:568), without writing B x N scores.
+ *   out_scores [B,k] fp32 descending, out_idx [B,k] int64; equal scores are ordered by
+ *   ascending entity id.  Requires 1 <= k <= min(N, 1024).
+ * This call synchronises `stream` once before returning (it reads back one overflow counter).
+ */
+size_t kge_topk_workspace_bytes(int64_t B, int64_t N, int64_t k);
+int kge_topk(const float* Q, const float* bias, const void* E, int dtype, const float* scale,
+             int64_t B, int64_t d, int64_t N, int64_t k, float* out_scores, int64_t* out_idx,
+             int apply_sigmoid, void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * Fused KvsAll BCE: mean over B*N of BCEWithLogits(s, y) with y the multi-hot of the CSR row
+ * (KvsAll.__getitem__, dicee/dataset_classes.py:354-361, incl. its label smoothing
+ * y*(1-eps) + 1/N when eps != 0) and the default loss of dicee/models/base_model.py:138, as
+ * used by training_step (:25-46).  Neither the dense target nor the logits are materialised.
+ *   csr_row [B] (-1 = no positives), row_ptr, col as in kge_rank_filtered.  loss [1] fp32 out.
+ * workspace: kge_bce_workspace_bytes() bytes.
+ */
+size_t kge_bce_workspace_bytes(void);
+int kge_bce_multihot(const float* Q, const float* bias, const void* E, int dtype, const float* scale,
+                     int64_t B, int64_t d, int64_t N, const int64_t* csr_row, const int64_t* row_ptr,
+                     const int32_t* col, int64_t n_rows, float label_smoothing, float* loss,
+                     void* workspace, size_t workspace_bytes, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* KGE_HIP_H */

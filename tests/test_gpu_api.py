@@ -1,0 +1,187 @@
+"""The Python call surface (models, Evaluator, KGE) on the GPU against the oracle, including the
+consistency checks the reference's own tests make: two rank loops agree exactly
+(tests/test_link_prediction_evaluation.py:98-107), ``predict`` is deterministic
+(tests/test_predict_kge.py:68-73), ``predict_topk`` equals ``sigmoid(predict)`` at the same entity
+within 1e-6 (:85-95) and is identical for batch sizes 1, 2, 4, 8 (:107-119)."""
+from types import SimpleNamespace
+
+import numpy as np
+import pytest
+import torch
+
+from helpers import score_close
+from oracle import kge_oracle as ko
+from oracle import torch_cpu_path as tcp
+
+pytestmark = pytest.mark.gpu
+
+
+def _toy(model_name, d, N=135, R=46, n=2000, seed=0, **extra):
+    from dicee_amd import models
+    rng = np.random.default_rng(seed)
+    args = {"model": model_name, "embedding_dim": d, "num_entities": N, "num_relations": R, **extra}
+    torch.manual_seed(seed)
+    m = models.MODEL_REGISTRY[model_name](args)
+    with torch.no_grad():
+        m.entity_embeddings.weight.normal_(0, 0.1)
+        m.relation_embeddings.weight.normal_(0, 0.1)
+        if hasattr(m, "p_coefficients"):
+            m.p_coefficients.weight.normal_(1.0, 0.3)
+        if hasattr(m, "q_coefficients"):
+            m.q_coefficients.weight.normal_(1.0, 0.3)
+    triples = np.stack([rng.integers(0, N, n), rng.integers(0, R, n), rng.integers(0, N, n)], axis=1)
+    return m, triples
+
+
+def _oracle_kw(m):
+    kw = {}
+    if m.name in ("Keci", "CKeci"):
+        kw = {"p": m.p, "q": m.q}
+        if m.p:
+            kw["coeff_p"] = m.p_coefficients.weight.detach().cpu().numpy().reshape(-1)
+        if m.q:
+            kw["coeff_q"] = m.q_coefficients.weight.detach().cpu().numpy().reshape(-1)
+    return kw
+
+
+@pytest.mark.parametrize("name,d,extra", [("DistMult", 32, {}), ("ComplEx", 32, {}), ("QMult", 32, {}),
+                                          ("Keci", 30, {"p": 2, "q": 2}), ("CKeci", 32, {"p": 0, "q": 1})])
+def test_forward_k_vs_all_is_a_drop_in(name, d, extra):
+    m, triples = _toy(name, d, **extra)
+    E = m.entity_embeddings.weight.detach().numpy().copy()
+    Rel = m.relation_embeddings.weight.detach().numpy().copy()
+    kw = _oracle_kw(m)
+    m = m.to("cuda").eval()
+    x = torch.from_numpy(triples[:200, :2].copy()).cuda()
+    with torch.no_grad():
+        S = m(x)                                                  # BaseKGE.forward shape dispatch
+    assert S.shape == (200, 135) and S.dtype == torch.float32 and S.is_cuda
+    ref = ko.k_vs_all_scores("Keci" if name == "CKeci" else name, E, Rel, triples[:200, :2], **kw)
+    ok, worst = score_close(S.cpu().numpy(), ref, 1e-5)
+    assert ok, worst
+    S[0, :5] = -np.inf                                            # callers mutate the result in place
+    # k_vs_all_score on gathered rows
+    S2 = m.k_vs_all_score(m.entity_embeddings(x[:, 0]), m.relation_embeddings(x[:, 1]), m.entity_embeddings.weight)
+    ok, worst = score_close(S2.cpu().numpy(), ref, 1e-5)
+    assert ok, worst
+
+
+@pytest.mark.parametrize("name,d,extra", [("DistMult", 32, {}), ("ComplEx", 64, {}), ("QMult", 64, {}),
+                                          ("Keci", 48, {"p": 1, "q": 1})])
+@pytest.mark.parametrize("batch_size", [64, 1000])
+def test_evaluator_matches_the_reference_loop(name, d, extra, batch_size):
+    from dicee_amd import Evaluator
+    m, triples = _toy(name, d, n=1500, seed=3, **extra)
+    E = m.entity_embeddings.weight.detach().clone()
+    Rel = m.relation_embeddings.weight.detach().clone()
+    kw = _oracle_kw(m)
+    er = {}
+    for h, r, t in triples:
+        er.setdefault((int(h), int(r)), []).append(int(t))
+    ds = SimpleNamespace(num_entities=135, num_relations=46, er_vocab=er, train_set=triples,
+                         valid_set=triples[:300], test_set=triples[300:700])
+    ev = Evaluator(SimpleNamespace(batch_size=batch_size, eval_model="train_val_test", scoring_technique="KvsAll",
+                                   full_storage_path=None))
+    m = m.to("cuda")
+    report = ev.eval(ds, m, "EntityPrediction", during_training=True)
+    assert set(report) == {"Train", "Val", "Test"}
+    assert set(report["Test"]) == {"H@1", "H@3", "H@10", "MRR"}
+    # the reference's op sequence on torch CPU (mask loop + unstable sort)
+    tkw = {k: (torch.tensor(v) if k.startswith("coeff") else v) for k, v in kw.items()}
+    ref_ranks = tcp.evaluate_entity_prediction("Keci" if name == "CKeci" else name, E, Rel, triples[300:700], er,
+                                               batch_size, **tkw)
+    got = ev.last_ranks
+    # every rank inside the fp64 oracle's tolerance interval; identical to the CPU loop except at near-ties
+    S = ko.k_vs_all_scores(name, E.numpy(), Rel.numpy(), triples[300:700, :2], **kw)
+    for j, (h, r, t) in enumerate(triples[300:700]):
+        tol = 1e-5 * np.sqrt((S[j] ** 2).mean())
+        lo, hi = ko.rank_interval_with_tolerance(S[j], int(t), er[(int(h), int(r))], tol)
+        assert lo <= got[j] <= hi
+        if lo == hi:
+            assert got[j] == ref_ranks[j]
+    agree = np.mean(np.asarray(ref_ranks) == got)
+    assert agree >= 0.99
+    want = ko.metrics_from_ranks(got)
+    assert report["Test"]["MRR"] == pytest.approx(want["MRR"]) and report["Test"]["H@10"] == want["H@10"]
+    # the counters-based evaluator and an evaluation on materialised scores agree exactly
+    x = torch.from_numpy(triples[300:700, :2].copy()).cuda()
+    with torch.no_grad():
+        Sg = m(x).cpu().numpy() - m.query(x)[1].cpu().numpy()[:, None]
+    if name != "Keci":
+        own = ko.filtered_ranks(Sg, triples[300:700, 2], [er[(int(h), int(r))] for h, r, _ in triples[300:700]])
+        np.testing.assert_array_equal(own, got)
+
+
+def test_predict_topk_and_predict_invariants():
+    from dicee_amd import KGE
+    m, _ = _toy("Keci", 32, p=0, q=1, seed=5)
+    m = m.to("cuda")
+    ents = [f"e{i}" for i in range(135)]
+    rels = [f"r{i}" for i in range(46)]
+    kge = KGE(m, {e: i for i, e in enumerate(ents)}, {r: i for i, r in enumerate(rels)})
+    # deterministic
+    a = kge.predict(h=["e3"], r=["r7"])
+    b = kge.predict(h=["e3"], r=["r7"])
+    assert torch.equal(a, b) and a.shape == (135,)
+    # top-k equals sigmoid(predict) at the same entity
+    top = kge.predict_topk(h=["e3"], r=["r7"], topk=10)
+    assert len(top) == 1 and len(top[0]) == 10
+    probs = kge.predict(h=["e3"], r=["r7"], logits=False)
+    for ent, score in top[0]:
+        assert abs(probs[kge.entity_to_idx[ent]].item() - score) <= 1e-6
+    scores = [s for _, s in top[0]]
+    assert scores == sorted(scores, reverse=True)
+    assert top[0][0][0] == ents[int(torch.argmax(probs))]
+    # batch-size invariance, bitwise, heads-major cartesian order
+    heads, rs = ["e1", "e9", "e30", "e77"], ["r0", "r5"]
+    base = kge.predict_topk(h=heads, r=rs, topk=5, batch_size=1)
+    assert len(base) == 8
+    for bs in (2, 4, 8):
+        assert kge.predict_topk(h=heads, r=rs, topk=5, batch_size=bs) == base
+    single = kge.predict_topk(h="e9", r="r0", topk=5)
+    assert single[0] == base[2]
+    with pytest.raises(KeyError):
+        kge.predict_topk(h=["nope"], r=["r0"])
+    with pytest.raises(AttributeError):
+        kge.predict_topk(h=["e1"], r=["r0"], t=["e2"])
+    with pytest.raises(AssertionError):
+        kge.predict_topk(h=3, r=["r0"])
+
+
+@pytest.mark.parametrize("storage", ["bf16", "int8"])
+def test_quantised_storage_follows_dequantised_fp32_math(storage):
+    m, triples = _toy("QMult" if storage == "bf16" else "DistMult", 128, N=3000, R=11, n=600, seed=7)
+    m = m.to("cuda").set_entity_storage(storage)
+    E, scale = m.table()
+    if storage == "bf16":
+        Ev = E.float().cpu().numpy()
+        Rv = m._rel().float().cpu().numpy()
+    else:
+        Ev = (E.float() * scale[:, None]).cpu().numpy()
+        Rv = m.relation_embeddings.weight.detach().cpu().numpy()
+    x = torch.from_numpy(triples[:, :2].copy()).cuda()
+    S = m(x).cpu().numpy()
+    ref = ko.k_vs_all_scores(m.name, Ev, Rv, triples[:, :2])
+    ok, worst = score_close(S, ref, 2e-2)
+    assert ok, worst
+    vals, idx = m.topk(x, 10)
+    wv, wi = ko.topk(S, 10)
+    np.testing.assert_array_equal(idx.cpu().numpy(), wi)
+
+
+def test_kvsall_bce_loss_matches_training_step_forward():
+    from dicee_amd.csr import FilterCSR
+    m, triples = _toy("CKeci", 64, N=2000, R=18, n=3000, seed=9, p=0, q=1)
+    E = m.entity_embeddings.weight.detach().clone()
+    Rel = m.relation_embeddings.weight.detach().clone()
+    csr = FilterCSR.from_triples(triples, 18)
+    keys = csr.keys_np[:256]
+    x_np = np.stack([keys // 18, keys % 18], axis=1)
+    pos = [csr.tails(int(h), int(r)) for h, r in x_np]
+    m = m.to("cuda")
+    csr.to("cuda")
+    for eps in (0.0, 0.1):
+        loss = m.kvsall_bce_loss(torch.from_numpy(x_np).cuda(), csr, eps).item()
+        want = tcp.kvsall_bce_step("Keci", E, Rel, torch.from_numpy(x_np), pos, eps, p=0, q=1,
+                                   coeff_q=torch.ones(1)).item()
+        assert loss == pytest.approx(want, rel=2e-5)

@@ -1,0 +1,340 @@
+"""Parity of the HIP kernels (through the C ABI) against the CPU oracle on seeded inputs.
+
+Bars: fp32 scores within 1e-5 relative, bf16 / int8 within 2e-2 relative (relative to
+max(|s|, row RMS)); ranks, tie counters and top-k indices bit-exact with respect to the scores the
+library itself materialises, and inside the oracle's tolerance interval.
+"""
+import numpy as np
+import pytest
+import torch
+
+from helpers import RTOL, score_close, random_tables, random_hr, stored_tables, dev, random_csr
+from oracle import kge_oracle as ko
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from dicee_amd import ops as _ops
+    return _ops
+
+
+@pytest.fixture(scope="module")
+def FilterCSR():
+    from dicee_amd.csr import FilterCSR as F
+    return F
+
+
+MODEL_CASES = [
+    # model, d, kwargs
+    ("DistMult", 32, {}),
+    ("ComplEx", 200, {}),
+    ("QMult", 128, {}),
+    ("QMult", 64, {"normalize_relation": False}),
+    ("Keci", 256, {"p": 0, "q": 1, "coeff_q": [1.0]}),
+    ("Keci", 28, {"p": 1, "q": 2, "coeff_p": [0.7], "coeff_q": [1.3, -0.4]}),
+    ("Keci", 35, {"p": 3, "q": 3, "coeff_p": [0.7, 1.1, -0.3], "coeff_q": [1.3, -0.4, 0.9]}),
+    ("Keci", 24, {"p": 2, "q": 0, "coeff_p": [0.5, 2.0]}),
+    ("Keci", 16, {"p": 0, "q": 0}),
+]
+
+
+def _gpu_kwargs(kw):
+    out = dict(kw)
+    for k in ("coeff_p", "coeff_q"):
+        if k in out:
+            out[k] = torch.tensor(out[k], dtype=torch.float32, device="cuda")
+    return out
+
+
+@pytest.mark.parametrize("model,d,kw", MODEL_CASES)
+def test_build_query_fp32(ops, model, d, kw):
+    rng = np.random.default_rng(100 + d)
+    N, R, B = 300, 17, 77
+    E, Rel = random_tables(rng, N, R, d, std=0.5)
+    hr = random_hr(rng, N, R, B)
+    Q, bias = ops.build_query(model, dev(torch.from_numpy(E)), dev(torch.from_numpy(Rel)),
+                              dev(torch.from_numpy(hr)), **_gpu_kwargs(kw))
+    Qr, br = ko.build_query(model, E, Rel, hr, **kw)
+    ok, worst = score_close(Q.cpu().numpy(), Qr, 1e-5)
+    assert ok, worst
+    ok, worst = score_close(bias.cpu().numpy(), br, 1e-5)
+    assert ok or np.abs(br).max() == 0, worst
+    if np.abs(br).max() == 0:
+        assert float(bias.abs().max()) == 0.0
+
+
+@pytest.mark.parametrize("storage", ["bf16", "int8"])
+@pytest.mark.parametrize("model", ["DistMult", "ComplEx", "QMult"])
+def test_build_query_quantised_tables(ops, model, storage):
+    rng = np.random.default_rng(7)
+    N, R, d, B = 200, 9, 128, 50
+    E, Rel = random_tables(rng, N, R, d)
+    hr = random_hr(rng, N, R, B)
+    Et, sc, Rt, Ev, Rv = stored_tables(E, Rel, storage)
+    Q, _ = ops.build_query(model, dev(Et), dev(Rt), dev(torch.from_numpy(hr)), ent_scale=dev(sc))
+    Qr, _ = ko.build_query(model, Ev, Rv, hr)
+    ok, worst = score_close(Q.cpu().numpy(), Qr, 1e-5)      # the gather itself is exact fp32 math
+    assert ok, worst
+
+
+@pytest.mark.parametrize("kind", ["LayerNorm", "BatchNorm1d"])
+def test_build_query_with_normalisation(ops, kind):
+    rng = np.random.default_rng(8)
+    N, R, d, B = 100, 5, 48, 40
+    E, Rel = random_tables(rng, N, R, d, std=1.0)
+    hr = random_hr(rng, N, R, B)
+    a_h, a_r = rng.normal(size=d).astype(np.float32), rng.normal(size=d).astype(np.float32)
+    b_h, b_r = rng.uniform(0.5, 2, d).astype(np.float32), rng.uniform(0.5, 2, d).astype(np.float32)
+    if kind == "LayerNorm":
+        onorm = {"kind": kind, "h_weight": a_h, "h_bias": b_h, "r_weight": a_r, "r_bias": b_r}
+    else:
+        onorm = {"kind": kind, "h_mean": a_h, "h_var": b_h, "r_mean": a_r, "r_var": b_r}
+    gnorm = {"kind": kind, "eps": 1e-5, "h_a": dev(torch.from_numpy(a_h)), "h_b": dev(torch.from_numpy(b_h)),
+             "r_a": dev(torch.from_numpy(a_r)), "r_b": dev(torch.from_numpy(b_r))}
+    for model in ("ComplEx", "QMult"):
+        kw = {"normalize_relation": False} if model == "QMult" else {}
+        Q, _ = ops.build_query(model, dev(torch.from_numpy(E)), dev(torch.from_numpy(Rel)),
+                               dev(torch.from_numpy(hr)), norm=gnorm, **kw)
+        Qr, _ = ko.build_query(model, E, Rel, hr, norm=onorm, **kw)
+        ok, worst = score_close(Q.cpu().numpy(), Qr, 2e-5)
+        assert ok, worst
+
+
+def test_build_query_bad_ids_give_nan_not_fault(ops):
+    rng = np.random.default_rng(9)
+    E, Rel = random_tables(rng, 50, 4, 16)
+    hr = np.array([[0, 0], [50, 1], [3, 4], [-1, 0], [49, 3]], dtype=np.int64)
+    Q, bias = ops.build_query("DistMult", dev(torch.from_numpy(E)), dev(torch.from_numpy(Rel)),
+                              dev(torch.from_numpy(hr)))
+    Q = Q.cpu().numpy()
+    assert np.isnan(Q[1]).all() and np.isnan(Q[2]).all() and np.isnan(Q[3]).all()
+    assert np.isfinite(Q[0]).all() and np.isfinite(Q[4]).all()
+
+
+SCORE_CASES = [
+    # model, N, R, d, B, storage, kw
+    ("DistMult", 135, 46, 32, 512, "fp32", {}),
+    ("ComplEx", 1003, 11, 200, 301, "fp32", {}),
+    ("Keci", 257, 6, 28, 33, "fp32", {"p": 1, "q": 2, "coeff_p": [0.7], "coeff_q": [1.3, -0.4]}),
+    ("Keci", 300, 6, 35, 70, "fp32", {"p": 3, "q": 3, "coeff_p": [0.7, 1.1, -0.3], "coeff_q": [1.3, -0.4, 0.9]}),
+    ("DistMult", 64, 3, 7, 5, "fp32", {}),
+    ("QMult", 999, 5, 128, 130, "bf16", {}),
+    ("DistMult", 5000, 7, 128, 600, "bf16", {}),
+    ("ComplEx", 321, 7, 64, 40, "bf16", {}),
+    ("DistMult", 777, 9, 128, 70, "int8", {}),
+    ("ComplEx", 2100, 9, 96, 520, "int8", {}),
+]
+
+
+def _setup(ops, model, N, R, d, B, storage, kw, seed=0, std=0.1):
+    rng = np.random.default_rng(seed)
+    E, Rel = random_tables(rng, N, R, d, std=std)
+    hr = random_hr(rng, N, R, B)
+    Et, sc, Rt, Ev, Rv = stored_tables(E, Rel, storage)
+    Eg, scg = dev(Et), dev(sc)
+    Q, bias = ops.build_query(model, Eg, dev(Rt), dev(torch.from_numpy(hr)), ent_scale=scg, **_gpu_kwargs(kw))
+    return rng, hr, Eg, scg, Q, bias, Ev, Rv
+
+
+@pytest.mark.parametrize("model,N,R,d,B,storage,kw", SCORE_CASES)
+def test_scores_vs_oracle(ops, model, N, R, d, B, storage, kw):
+    rng, hr, Eg, scg, Q, bias, Ev, Rv = _setup(ops, model, N, R, d, B, storage, kw)
+    S = ops.scores(Q, bias, Eg, scg).cpu().numpy()
+    ref = ko.k_vs_all_scores(model, Ev, Rv, hr, **kw)
+    ok, worst = score_close(S, ref, RTOL[storage])
+    assert ok, f"worst error / bound = {worst}"
+    # the reference's own multi-mm / einsum decomposition gives the same matrix
+    ref2 = ko.k_vs_all_scores_ref_form(model, Ev, Rv, hr, **kw)
+    ok, worst = score_close(S, ref2, RTOL[storage])
+    assert ok, worst
+
+
+def _expected_counts(S_raw, targets, filters):
+    out = np.array([ko.filtered_rank_counts(S_raw[j], int(targets[j]), filters[j]) for j in range(len(targets))])
+    return out[:, 0], out[:, 1], out[:, 2]
+
+
+@pytest.mark.parametrize("model,N,R,d,B,storage,kw", SCORE_CASES)
+def test_rank_filtered_exact_against_own_scores(ops, FilterCSR, model, N, R, d, B, storage, kw):
+    rng, hr, Eg, scg, Q, bias, Ev, Rv = _setup(ops, model, N, R, d, B, storage, kw, seed=1)
+    targets = rng.integers(0, N, B).astype(np.int64)
+    er = random_csr(rng, hr, targets, N, R)
+    csr = FilterCSR.from_er_vocab(er, R, device="cuda")
+    hr_g = dev(torch.from_numpy(hr))
+    rows = csr.rows_for(hr_g)
+    out = ops.rank_filtered(Q, bias, Eg, scg, dev(torch.from_numpy(targets)), rows, csr.row_ptr, csr.col)
+    S_raw = ops.scores(Q, None, Eg, scg).cpu().numpy()
+    filters = [er[(int(h), int(r))] for h, r in hr]
+    g, t, tl = _expected_counts(S_raw, targets, filters)
+    np.testing.assert_array_equal(out["n_greater"].cpu().numpy(), g)
+    np.testing.assert_array_equal(out["n_equal"].cpu().numpy(), t)
+    np.testing.assert_array_equal(out["n_equal_lower"].cpu().numpy(), tl)
+    ts = out["target_score"].cpu().numpy()
+    want_ts = S_raw[np.arange(B), targets] + bias.cpu().numpy()
+    np.testing.assert_array_equal(ts, want_ts.astype(np.float32))
+    # and inside the fp64 oracle's tolerance interval
+    ref = ko.k_vs_all_scores(model, Ev, Rv, hr, **kw) - ko.build_query(model, Ev, Rv, hr, **kw)[1][:, None]
+    ranks = 1 + g + tl
+    for j in range(B):
+        tol = RTOL[storage] * max(abs(ref[j, targets[j]]), np.sqrt((ref[j] ** 2).mean()))
+        lo, hi = ko.rank_interval_with_tolerance(ref[j], int(targets[j]), filters[j], tol)
+        assert lo <= ranks[j] <= hi
+
+
+@pytest.mark.parametrize("storage,d", [("fp32", 40), ("bf16", 128), ("int8", 64)])
+def test_rank_hub_rows_shared_filters_and_ties(ops, FilterCSR, storage, d):
+    """Long filter rows (several slices and passes of the correction kernel), many queries sharing one
+    (h, r) row, duplicated / zero entity rows (exact ties), unknown (h, r) pairs and no filter at all."""
+    rng = np.random.default_rng(5)
+    N, R, B = 9000, 3, 700
+    E, Rel = random_tables(rng, N, R, d)
+    E[100] = E[7000] = E[42]            # exact duplicates -> exact ties
+    E[200:210] = 0.0                    # zero rows tie with each other
+    hr = random_hr(rng, 40, R, B)       # few distinct pairs: big groups
+    hr[:300] = hr[0]                    # one group of 300 queries
+    targets = rng.integers(0, N, B).astype(np.int64)
+    targets[:50] = 42
+    targets[50:80] = 7000
+    targets[80:100] = 205
+    er = random_csr(rng, hr, targets, N, R, max_len=3, hub_rows=[(0, 5000), (400, 2500)])
+    some = (int(hr[650, 0]), int(hr[650, 1]))
+    Et, sc, Rt, Ev, Rv = stored_tables(E, Rel, storage)
+    Eg, scg = dev(Et), dev(sc)
+    hr_g = dev(torch.from_numpy(hr))
+    Q, bias = ops.build_query("DistMult", Eg, dev(Rt), hr_g, ent_scale=scg)
+    csr = FilterCSR.from_er_vocab({k: v for k, v in er.items() if k != some}, R, device="cuda")
+    rows = csr.rows_for(hr_g)
+    assert int((rows < 0).sum()) > 0
+    tg = dev(torch.from_numpy(targets))
+    out = ops.rank_filtered(Q, bias, Eg, scg, tg, rows, csr.row_ptr, csr.col)
+    S_raw = ops.scores(Q, None, Eg, scg).cpu().numpy()
+    filters = [er[(int(h), int(r))] if (int(h), int(r)) != some else [] for h, r in hr]
+    g, t, tl = _expected_counts(S_raw, targets, filters)
+    np.testing.assert_array_equal(out["n_greater"].cpu().numpy(), g)
+    np.testing.assert_array_equal(out["n_equal"].cpu().numpy(), t)
+    np.testing.assert_array_equal(out["n_equal_lower"].cpu().numpy(), tl)
+    assert t[:50].min() >= 1                                   # the duplicates really tie
+    # no filter at all
+    out2 = ops.rank_filtered(Q, bias, Eg, scg, tg)
+    g2, t2, tl2 = _expected_counts(S_raw, targets, [None] * B)
+    np.testing.assert_array_equal(out2["n_greater"].cpu().numpy(), g2)
+    np.testing.assert_array_equal(out2["n_equal"].cpu().numpy(), t2)
+    np.testing.assert_array_equal(out2["n_equal_lower"].cpu().numpy(), tl2)
+
+
+def test_rank_all_scores_equal(ops):
+    """Zero embeddings: every score ties, the rank interval is [1, N]."""
+    N, R, d, B = 500, 2, 32, 9
+    E = torch.zeros((N, d), device="cuda")
+    Rel = torch.zeros((R, d), device="cuda")
+    hr = torch.zeros((B, 2), dtype=torch.int64, device="cuda")
+    t = torch.arange(B, dtype=torch.int64, device="cuda") * 50
+    Q, bias = ops.build_query("DistMult", E, Rel, hr)
+    out = ops.rank_filtered(Q, bias, E, None, t)
+    assert out["n_greater"].abs().max().item() == 0
+    assert (out["n_equal"] == N - 1).all()
+    np.testing.assert_array_equal(out["n_equal_lower"].cpu().numpy(), np.arange(B) * 50)
+
+
+TOPK_CASES = [
+    ("DistMult", 135, 46, 32, 64, "fp32", 10),
+    ("ComplEx", 20011, 11, 200, 130, "fp32", 100),
+    ("QMult", 20011, 5, 128, 600, "bf16", 10),
+    ("DistMult", 30000, 9, 128, 70, "int8", 100),
+    ("DistMult", 5000, 9, 64, 33, "bf16", 1),
+    ("DistMult", 6000, 9, 64, 20, "fp32", 1024),
+]
+
+
+@pytest.mark.parametrize("model,N,R,d,B,storage,k", TOPK_CASES)
+def test_topk_exact_against_own_scores(ops, model, N, R, d, B, storage, k):
+    rng, hr, Eg, scg, Q, bias, Ev, Rv = _setup(ops, model, N, R, d, B, storage, {}, seed=2)
+    vals, idx = ops.topk(Q, bias, Eg, scg, k)
+    S = ops.scores(Q, bias, Eg, scg).cpu().numpy()
+    wv, wi = ko.topk(S, k)
+    np.testing.assert_array_equal(idx.cpu().numpy(), wi)
+    np.testing.assert_array_equal(vals.cpu().numpy(), wv)
+    # sigmoid variant equals sigmoid of the logits at the same entities
+    sv, si = ops.topk(Q, bias, Eg, scg, k, sigmoid=True)
+    np.testing.assert_array_equal(si.cpu().numpy(), wi)
+    np.testing.assert_allclose(sv.cpu().numpy(), ko.sigmoid(wv), rtol=1e-6, atol=1e-7)
+    # against the fp64 oracle: same index set wherever the k-th / (k+1)-th gap exceeds tolerance
+    ref = ko.k_vs_all_scores(model, Ev, Rv, hr)
+    for b in range(B):
+        order = np.argsort(-ref[b], kind="stable")
+        tol = RTOL[storage] * np.sqrt((ref[b] ** 2).mean())
+        if k < N and ref[b, order[k - 1]] - ref[b, order[k]] > 2 * tol:
+            assert set(order[:k]) == set(wi[b])
+
+
+def test_topk_adversarial_order_overflows_and_recovers(ops):
+    """Scores that increase with the entity id defeat the running threshold: every new row beats it,
+    the candidate buffers overflow and the rescan path has to repair the result."""
+    N, d, B, k = 60000, 16, 40, 10
+    rng = np.random.default_rng(3)
+    v = rng.standard_normal(d).astype(np.float32)
+    E = (np.arange(N, dtype=np.float32)[:, None] / N) * v[None, :]
+    Q = (np.abs(rng.standard_normal((B, 1))).astype(np.float32) + 0.5) * v[None, :]
+    Eg, Qg = dev(torch.from_numpy(E)), dev(torch.from_numpy(Q))
+    vals, idx = ops.topk(Qg, None, Eg, None, k)
+    S = ops.scores(Qg, None, Eg, None).cpu().numpy()
+    wv, wi = ko.topk(S, k)
+    np.testing.assert_array_equal(idx.cpu().numpy(), wi)
+    np.testing.assert_array_equal(vals.cpu().numpy(), wv)
+
+
+def test_topk_ties_prefer_lower_ids_and_k_equals_n(ops):
+    N, d, B = 300, 16, 5
+    E = torch.zeros((N, d), device="cuda")
+    Q = torch.ones((B, d), device="cuda")
+    vals, idx = ops.topk(Q, None, E, None, 7)
+    np.testing.assert_array_equal(idx.cpu().numpy(), np.tile(np.arange(7), (B, 1)))
+    vals, idx = ops.topk(Q, None, E, None, N)
+    np.testing.assert_array_equal(idx.cpu().numpy(), np.tile(np.arange(N), (B, 1)))
+
+
+@pytest.mark.parametrize("model,N,R,d,B,storage,kw", [
+    ("Keci", 4099, 18, 256, 300, "fp32", {"p": 0, "q": 1, "coeff_q": [1.0]}),
+    ("Keci", 1000, 6, 35, 70, "fp32", {"p": 3, "q": 3, "coeff_p": [0.7, 1.1, -0.3], "coeff_q": [1.3, -0.4, 0.9]}),
+    ("QMult", 3000, 5, 128, 530, "bf16", {}),
+    ("DistMult", 2000, 5, 64, 100, "int8", {}),
+])
+@pytest.mark.parametrize("eps", [0.0, 0.1])
+def test_bce_multihot_vs_oracle(ops, FilterCSR, model, N, R, d, B, storage, kw, eps):
+    rng, hr, Eg, scg, Q, bias, Ev, Rv = _setup(ops, model, N, R, d, B, storage, kw, seed=4, std=0.5)
+    er = random_csr(rng, hr, rng.integers(0, N, B), N, R, max_len=5, hub_rows=[(0, 400)])
+    er[(int(hr[1, 0]), int(hr[1, 1]))] = er.get((int(hr[1, 0]), int(hr[1, 1])), [])
+    csr = FilterCSR.from_er_vocab(er, R, device="cuda")
+    rows = csr.rows_for(dev(torch.from_numpy(hr)))
+    loss = ops.bce_multihot(Q, bias, Eg, scg, rows, csr.row_ptr, csr.col, eps).item()
+    ref = ko.k_vs_all_scores(model, Ev, Rv, hr, **kw)
+    want = ko.bce_multihot(ref, [er[(int(h), int(r))] for h, r in hr], eps)
+    tol = 1e-5 if storage == "fp32" else 2e-2
+    assert loss == pytest.approx(want, rel=tol)
+
+
+def test_argument_validation(ops):
+    from dicee_amd._lib import KgeError
+    E = torch.zeros((100, 24), device="cuda")
+    Q = torch.zeros((4, 24), device="cuda")
+    with pytest.raises(KgeError):
+        ops.topk(Q, None, E, None, 101)                      # k > N
+    with pytest.raises(KgeError):
+        ops.topk(Q, None, E, None, 0)
+    with pytest.raises(KgeError):
+        ops.build_query("QMult", torch.zeros((10, 6), device="cuda"), torch.zeros((2, 6), device="cuda"),
+                        torch.zeros((1, 2), dtype=torch.int64, device="cuda"))   # d % 4 != 0
+    with pytest.raises(KgeError):
+        ops.build_query("Keci", torch.zeros((10, 7), device="cuda"), torch.zeros((2, 7), device="cuda"),
+                        torch.zeros((1, 2), dtype=torch.int64, device="cuda"), p=1, q=1,
+                        coeff_p=torch.ones(1, device="cuda"), coeff_q=torch.ones(1, device="cuda"))
+    with pytest.raises(KgeError):
+        ops.scores(torch.zeros((4, 256), device="cuda"), None,
+                   torch.zeros((10, 256), device="cuda", dtype=torch.bfloat16))  # bf16 d > 128
+    with pytest.raises(RuntimeError):
+        ops.scores(torch.zeros((4, 24)), None, torch.zeros((10, 24)))            # CPU tensors
+    # empty batch is a no-op
+    out = ops.scores(torch.zeros((0, 24), device="cuda"), None, E)
+    assert out.shape == (0, 100)

@@ -1,0 +1,144 @@
+"""CPU-only checks: host-side logic of the package, and that the C-ABI library loads and exports
+every symbol ``include/kge_hip.h`` declares (no kernel is launched here)."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import kge_oracle as ko
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.fixture(scope="module")
+def lib_path():
+    from dicee_amd import _lib, build
+    if not os.path.exists(_lib.LIB_PATH):
+        build.build()
+    return _lib.LIB_PATH
+
+
+def test_library_exports_every_declared_symbol(lib_path):
+    header = open(os.path.join(ROOT, "include", "kge_hip.h")).read()
+    header = re.sub(r"/\*.*?\*/", "", header, flags=re.S)
+    declared = sorted(set(re.findall(r"\b(kge_[a-z_0-9]+)\s*\(", header)))
+    assert {"kge_build_query", "kge_scores", "kge_rank_filtered", "kge_topk", "kge_bce_multihot",
+            "kge_last_error", "kge_abi_version", "kge_rank_workspace_bytes", "kge_topk_workspace_bytes",
+            "kge_bce_workspace_bytes"} <= set(declared)
+    lib = ctypes.CDLL(lib_path)
+    for name in declared:
+        assert hasattr(lib, name), f"{name} declared in kge_hip.h but not exported"
+    from dicee_amd import _lib
+    assert set(_lib.SIGNATURES) == set(declared)
+    loaded = _lib.load()
+    assert loaded.kge_abi_version() == 1
+    assert loaded.kge_last_error() == b""
+    assert loaded.kge_rank_workspace_bytes(4096) >= 4096 * 4 + 8192 * 8
+    assert loaded.kge_topk_workspace_bytes(8, 1000, 10) >= 8 * 4096 * 8
+
+
+def test_host_side_argument_validation_without_gpu(lib_path):
+    """Validation happens before anything touches the device, so it can be exercised here."""
+    from dicee_amd import _lib
+    lib = _lib.load()
+    rc = lib.kge_scores(None, None, None, 0, None, 4, 16, 100, None, 100, None)
+    assert rc == 1 and b"null" in lib.kge_last_error()
+    rc = lib.kge_topk(ctypes.c_void_p(256), None, ctypes.c_void_p(256), 0, None, 4, 16, 100, 200, None, None, 0,
+                      None, 0, None)
+    assert rc == 1 and b"k=200" in lib.kge_last_error()
+    rc = lib.kge_scores(ctypes.c_void_p(256), None, ctypes.c_void_p(256), 1, None, 4, 256, 100,
+                        ctypes.c_void_p(256), 100, None)
+    assert rc == 2                                              # bf16 with d > 128: unsupported
+    rc = lib.kge_build_query(3, 1, 1, ctypes.c_void_p(256), 0, None, ctypes.c_void_p(256), 0, None, None, 1, None,
+                             ctypes.c_void_p(256), 1, 7, 10, 2, ctypes.c_void_p(256), ctypes.c_void_p(256), None)
+    assert rc == 1 and b"Keci" in lib.kge_last_error()
+
+
+def test_filter_csr_builders():
+    from dicee_amd.csr import FilterCSR
+    rng = np.random.default_rng(0)
+    N, R, n = 50, 4, 400
+    triples = np.stack([rng.integers(0, N, n), rng.integers(0, R, n), rng.integers(0, N, n)], axis=1)
+    triples = np.concatenate([triples, triples[:50]])              # duplicates
+    brute = {}
+    for h, r, t in triples:
+        brute.setdefault((int(h), int(r)), set()).add(int(t))
+    csr = FilterCSR.from_triples(triples, R)
+    assert csr.num_rows == len(brute) and csr.nnz == sum(len(v) for v in brute.values())
+    for (h, r), tails in brute.items():
+        np.testing.assert_array_equal(csr.tails(h, r), sorted(tails))
+    er = {}
+    for h, r, t in triples:
+        er.setdefault((int(h), int(r)), []).append(int(t))         # the reference's list-with-duplicates form
+    csr2 = FilterCSR.from_er_vocab(er, R)
+    np.testing.assert_array_equal(csr2.row_ptr_np, csr.row_ptr_np)
+    np.testing.assert_array_equal(csr2.col_np, csr.col_np)
+    rows = csr.rows_for_numpy(np.array([[0, 0], [N + 5, 1], [triples[0, 0], triples[0, 1]]]))
+    assert rows[1] == -1 and rows[2] >= 0
+    t_rows = csr.to("cpu").rows_for(torch.tensor([[0, 0], [N + 5, 1], [int(triples[0, 0]), int(triples[0, 1])]]))
+    np.testing.assert_array_equal(t_rows.numpy(), rows)
+    capped = FilterCSR.from_triples(triples, R, max_per_row=2)
+    assert np.diff(capped.row_ptr_np).max() <= 2
+    assert len(FilterCSR.from_triples(np.empty((0, 3), dtype=np.int64), R).tails(1, 1)) == 0
+
+
+def test_metrics_and_tie_rules():
+    from dicee_amd.evaluator import compute_metrics_from_ranks_simple, create_hits_dict, update_hits, \
+        ranks_from_counts
+    ranks = [1, 2, 3, 4, 11, 1, 10]
+    hits = create_hits_dict()
+    for r in ranks:
+        update_hits(hits, r)
+    m = compute_metrics_from_ranks_simple(ranks, len(ranks), hits)
+    want = ko.metrics_from_ranks(ranks)
+    assert m == want
+    assert m["MRR"] == pytest.approx(sum(1.0 / r for r in ranks) / len(ranks))
+    g, e, l = torch.tensor([0, 5]), torch.tensor([4, 0]), torch.tensor([1, 0])
+    assert ranks_from_counts(g, e, l, "stable").tolist() == [2, 6]
+    assert ranks_from_counts(g, e, l, "optimistic").tolist() == [1, 6]
+    assert ranks_from_counts(g, e, l, "pessimistic").tolist() == [5, 6]
+    assert ranks_from_counts(g, e, l, "mean").tolist() == [3, 6]
+
+
+def test_models_mirror_reference_parameters_and_have_no_cpu_fallback():
+    from dicee_amd import models
+    args = {"model": "Keci", "embedding_dim": 12, "num_entities": 9, "num_relations": 3, "p": 1, "q": 2}
+    m, form = models.initialize_model(args)
+    assert form == "EntityPrediction"
+    assert set(m.state_dict()) == {"entity_embeddings.weight", "relation_embeddings.weight",
+                                   "p_coefficients.weight", "q_coefficients.weight"}
+    assert m.r == 3 and float(m.q_coefficients.weight.abs().sum()) == 0.0       # reference init: zeros
+    c = models.CKeci(args)
+    assert float(c.p_coefficients.weight.sum()) == 1.0 and not c.q_coefficients.weight.requires_grad
+    with pytest.raises(AssertionError):
+        models.Keci({**args, "embedding_dim": 13})
+    with pytest.raises(ValueError):
+        models.initialize_model({**args, "model": "TransE"})
+    ln = models.ComplEx({"model": "ComplEx", "embedding_dim": 8, "num_entities": 5, "num_relations": 2,
+                         "normalization": "LayerNorm"})
+    assert "normalize_head_entity_embeddings.weight" in ln.state_dict()
+    d = models.DistMult({"model": "DistMult", "embedding_dim": 8, "num_entities": 5, "num_relations": 2})
+    with pytest.raises(RuntimeError):
+        d(torch.zeros((2, 2), dtype=torch.int64))                  # CPU tensors: refuses, never falls back
+    with pytest.raises(NotImplementedError):
+        d(torch.zeros((2, 3), dtype=torch.int64))
+
+
+def test_synthetic_configs_small_scale():
+    from dicee_amd import synthetic
+    c1 = synthetic.make_config("c1")
+    assert c1.E.shape == (135, 32) and c1.Rel.shape == (46, 32) and c1.triples.shape == (5216, 3)
+    assert c1.queries.shape == (512, 3) and c1.csr.nnz <= 5216
+    c4 = synthetic.make_config("c4", scale=0.002)
+    assert c4.E.shape[1] == 128 and c4.queries[:, 2].max() < c4.N
+    assert np.diff(c4.csr.row_ptr_np).max() <= 50000
+    c3 = synthetic.make_config("c3", scale=0.05)
+    assert np.diff(c3.csr.row_ptr_np).max() <= 400
+    assert len(np.unique(c3.queries[:, 0] * c3.R + c3.queries[:, 1])) == len(c3.queries)
+    c5 = synthetic.make_config("c5", scale=0.0001)
+    assert c5.csr is None and c5.queries.shape[1] == 3
+    p = synthetic.zipf_probs(10, 1.1)
+    assert p[0] > p[1] > p[-1] and p.sum() == pytest.approx(1.0)
