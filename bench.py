@@ -1,0 +1,170 @@
+#!/usr/bin/env python3
+"""Benchmark of the KvsAll filtered-rank / top-k / BCE path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c4] [--no-cpu-baseline]
+
+A step is one pass of the hot path over one batch of synthetic queries: gather + interaction
+(kge_build_query), then the fused epilogue the configuration names (filtered rank for c1/c2/c4, BCE for
+c3, top-k for c5).  Default workload: c4 = QMult filtered-rank evaluation, 2.5M entities x d=128, bf16
+tables with fp32 accumulation, batches of 4096 out of 50k queries whose (h, r) filter rows hold up to
+50k known tails.  Tables and index arrays are resident in HBM before the timed region.
+
+Prints ONE JSON line.  `value` = entity scores per second (B*N per step) over the timed region;
+`roofline` prices the MFMA main loop (2*d flop per score) against the published dense peak with the
+kernel time measured by HIP events on its own stream; `cpu_baseline` times the reference's op sequence
+(torch CPU mm + per-row mask loop + full sort) on a small sample of the same queries.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for _p in (ROOT, os.path.join(ROOT, "dice-embeddings_amd")):
+    if _p not in sys.path:
+        sys.path.insert(0, _p)
+
+PEAK_TFLOPS = {"bf16": 2500.0, "fp32": 157.3}       # MI355X dense MFMA peaks
+MODE = {"c1": "rank", "c2": "rank", "c3": "bce", "c4": "rank", "c5": "topk"}
+
+
+def cpu_baseline(cfg, model, mode, seconds_budget=25.0):
+    """The reference's CPU op sequence (oracle/torch_cpu_path.py) on a bounded sample of the workload."""
+    import numpy as np
+    import torch
+    from oracle import torch_cpu_path as tcp
+    threads = torch.get_num_threads()
+    E, scale = model.table()
+    E = E.float().cpu()
+    if scale is not None:
+        E = E * scale.float().cpu()[:, None]                    # the dequantised fp32 table
+    Rel = model._rel().float().cpu()
+    N = E.shape[0]
+    name = "Keci" if cfg.model == "Keci" else cfg.model
+    kw = {}
+    if name == "Keci":
+        kw = {"p": cfg.p, "q": cfg.q, "coeff_p": torch.ones(cfg.p), "coeff_q": torch.ones(cfg.q)}
+    # sample size: keep B*N*4 bytes of scores around 0.5 GB per batch
+    bs = int(max(1, min(cfg.B, (1 << 27) // max(N, 1))))
+    q = cfg.queries
+    done, t_total, nb = 0, 0.0, 0
+    while t_total < seconds_budget and done + bs <= len(q) and nb < 8:
+        batch = q[done:done + bs]
+        t0 = time.perf_counter()
+        if mode == "rank":
+            er = {}
+            if cfg.csr is not None:
+                for h, r, _ in batch:
+                    er[(int(h), int(r))] = cfg.csr.tails(int(h), int(r)).astype(np.int64)
+            tcp.evaluate_entity_prediction(name, E, Rel, batch, er, bs, **kw)
+        elif mode == "topk":
+            tcp.predict_topk_indices(name, E, Rel, torch.from_numpy(batch[:, :2].copy()), cfg.k, bs, **kw)
+        else:
+            pos = [cfg.csr.tails(int(h), int(r)).astype(np.int64) for h, r, _ in batch]
+            tcp.kvsall_bce_step(name, E, Rel, torch.from_numpy(batch[:, :2].copy()), pos, 0.0, **kw)
+        dt = time.perf_counter() - t0
+        if nb > 0 or dt > 2.0:                                  # first small batch is a warm-up
+            t_total += dt
+            done += bs
+        nb += 1
+    n_q = max(done, 1)
+    t_total = max(t_total, 1e-9)
+    return {"value": n_q * N / t_total, "unit": "scores/s", "cores": threads, "kind": "port",
+            "queries_per_sec": n_q / t_total,
+            "sample": f"{n_q} queries of {cfg.name} in batches of {bs} against all {N} entities, "
+                      f"torch {torch.__version__} CPU, {threads} threads"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=None)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--config", default="c4", choices=sorted(MODE))
+    ap.add_argument("--scale", type=float, default=1.0, help="shrink the workload (testing only)")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on ONE GPU (no sharding, no collectives); rerun with --gpus 1",
+              file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+    from dicee_amd import synthetic, ops
+
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    dev = torch.device("cuda:0")
+    mode = MODE[args.config]
+    t_setup = time.perf_counter()
+    big = args.config in ("c4", "c5") and args.scale == 1.0
+    cfg = synthetic.make_config(args.config, scale=args.scale, with_tables=not big)
+    model = synthetic.make_model(cfg, dev, tables_on_device=big)
+    if cfg.csr is not None:
+        cfg.csr.to(dev)
+    q_all = torch.from_numpy(np.ascontiguousarray(cfg.queries)).to(dev)
+    batches = [(q_all[i:i + cfg.B, :2].contiguous(), q_all[i:i + cfg.B, 2].contiguous())
+               for i in range(0, len(q_all), cfg.B)]
+    steps = args.steps if args.steps is not None else max(2 * len(batches), 20)
+    torch.cuda.synchronize()
+    t_setup = time.perf_counter() - t_setup
+
+    def step(i):
+        x, t = batches[i % len(batches)]
+        if mode == "rank":
+            return model.rank_filtered(x, t, cfg.csr)
+        if mode == "topk":
+            return model.topk(x, cfg.k)
+        return model.kvsall_bce_loss(x, cfg.csr)
+
+    for i in range(args.warmup):
+        step(i)
+    torch.cuda.synchronize()
+    ops.profile_begin()
+    t0 = time.perf_counter()
+    n_queries = 0
+    for i in range(steps):
+        step(i)
+        n_queries += batches[i % len(batches)][0].shape[0]
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    kernel_ms, launches = ops.profile_end()
+
+    N, d = cfg.N, cfg.d
+    scores = float(n_queries) * N
+    compute = "fp32" if cfg.storage == "fp32" else "bf16"
+    flops = 2.0 * d * scores                                    # algorithmic: 2*d flop per entity score
+    achieved = flops / (kernel_ms * 1e-3) / 1e12 if kernel_ms > 0 else 0.0
+    out = {
+        "metric": {"rank": "filtered_rank_entity_scores_per_sec", "topk": "topk_entity_scores_per_sec",
+                   "bce": "kvsall_bce_entity_scores_per_sec"}[mode],
+        "value": scores / elapsed,
+        "unit": "scores/s",
+        "queries_per_sec": n_queries / elapsed,
+        "n_gpus": 1, "steps": steps, "warmup": args.warmup,
+        "ms_per_step": elapsed * 1e3 / steps,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": {"fp32": "f32", "bf16": "bf16 x bf16 -> f32", "int8": "int8 table as bf16 x bf16 -> f32"}[cfg.storage],
+        "data": "synthetic",
+        "config": {"workload": f"{args.config}: {cfg.model} {mode}, N={N} entities, d={d}, {cfg.storage} tables, "
+                               f"batch {cfg.B}, {len(q_all)} queries"
+                               + (f", filter CSR nnz={cfg.csr.nnz} max row {int(np.diff(cfg.csr.row_ptr_np).max())}"
+                                  if cfg.csr is not None and mode == "rank" else "")
+                               + (f", k={cfg.k}" if mode == "topk" else ""),
+                   "scale": args.scale},
+        "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_TFLOPS[compute], "unit": "TFLOP/s",
+                     "frac": achieved / PEAK_TFLOPS[compute], "traffic": None,
+                     "kernel": "qreg_kernel" if compute == "bf16" else "kloop_kernel",
+                     "kernel_ms_avg": kernel_ms / max(launches, 1), "launches": launches,
+                     "kernel_time_share": kernel_ms * 1e-3 / elapsed},
+        "setup_s": t_setup,
+        "device": torch.cuda.get_device_name(0),
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(cfg, model, mode)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -4,6 +4,10 @@
 
 #include <string.h>
 
+#include <mutex>
+#include <utility>
+#include <vector>
+
 namespace kge {
 
 // ---- thread-local error text --------------------------------------------------------------
@@ -16,6 +20,11 @@ int set_error(int code, const char* fmt, ...) {
   return code;
 }
 void clear_error() { g_err[0] = 0; }
+
+// ---- optional timing of the contraction launches (measurement aid) ------------------------
+static std::mutex g_prof_mu;
+static bool g_prof_on = false;
+static std::vector<std::pair<hipEvent_t, hipEvent_t>> g_prof_events;
 
 namespace {
 
@@ -484,6 +493,17 @@ int launch_contract(int dtype, const ContractArgs& a, const EArgs& ea, hipStream
   const int64_t nwg = (a.n_chunks + 7) / 8 * 8 * a.n_qgroups;
   KGE_REQUIRE(nwg <= 0x7fffffffLL, KGE_ERR_INVALID, "%s: grid of %lld workgroups too large", name, (long long)nwg);
   dim3 grid((unsigned)nwg), block(256);
+  hipEvent_t ev0 = nullptr, ev1 = nullptr;
+  bool timed = false;
+  {
+    std::lock_guard<std::mutex> lk(g_prof_mu);
+    timed = g_prof_on;
+  }
+  if (timed) {
+    KGE_HIP_CHECK(hipEventCreate(&ev0));
+    KGE_HIP_CHECK(hipEventCreate(&ev1));
+    KGE_HIP_CHECK(hipEventRecord(ev0, st));
+  }
   if (dtype == KGE_F32)
     hipLaunchKernelGGL((kloop_kernel<EpiT>), grid, block, 0, st, a, ea);
   else if (dtype == KGE_BF16)
@@ -491,6 +511,11 @@ int launch_contract(int dtype, const ContractArgs& a, const EArgs& ea, hipStream
   else
     hipLaunchKernelGGL((qreg_kernel<KGE_I8, EpiT>), grid, block, 0, st, a, ea);
   KGE_LAUNCH_CHECK(name);
+  if (timed) {
+    KGE_HIP_CHECK(hipEventRecord(ev1, st));
+    std::lock_guard<std::mutex> lk(g_prof_mu);
+    g_prof_events.emplace_back(ev0, ev1);
+  }
   return KGE_OK;
 }
 
@@ -526,6 +551,42 @@ using namespace kge;
 
 extern "C" const char* kge_last_error(void) { return g_err; }
 extern "C" int kge_abi_version(void) { return KGE_ABI_VERSION; }
+
+extern "C" int kge_profile_begin(void) {
+  clear_error();
+  std::lock_guard<std::mutex> lk(g_prof_mu);
+  for (auto& p : g_prof_events) {
+    hipEventDestroy(p.first);
+    hipEventDestroy(p.second);
+  }
+  g_prof_events.clear();
+  g_prof_on = true;
+  return KGE_OK;
+}
+
+extern "C" int kge_profile_end(double* total_ms, int64_t* launches) {
+  clear_error();
+  std::vector<std::pair<hipEvent_t, hipEvent_t>> evs;
+  {
+    std::lock_guard<std::mutex> lk(g_prof_mu);
+    g_prof_on = false;
+    evs.swap(g_prof_events);
+  }
+  double total = 0.0;
+  int rc = KGE_OK;
+  for (auto& p : evs) {
+    float ms = 0.f;
+    hipError_t e = hipEventSynchronize(p.second);
+    if (e == hipSuccess) e = hipEventElapsedTime(&ms, p.first, p.second);
+    if (e != hipSuccess) rc = set_error(KGE_ERR_HIP, "kge_profile_end: %s", hipGetErrorString(e));
+    total += ms;
+    hipEventDestroy(p.first);
+    hipEventDestroy(p.second);
+  }
+  if (total_ms) *total_ms = total;
+  if (launches) *launches = (int64_t)evs.size();
+  return rc;
+}
 
 extern "C" int kge_scores(const float* Q, const float* bias, const void* E, int dtype, const float* scale, int64_t B,
                           int64_t d, int64_t N, float* S, int64_t ldS, void* stream) {

@@ -34,6 +34,8 @@ SIGNATURES = {
     "kge_topk_workspace_bytes": (_sz, [_c_i64, _c_i64, _c_i64]),
     "kge_topk": (_c_int, [_vp, _vp, _vp, _c_int, _vp, _c_i64, _c_i64, _c_i64, _c_i64, _vp, _vp, _c_int, _vp, _sz,
                           _vp]),
+    "kge_profile_begin": (_c_int, []),
+    "kge_profile_end": (_c_int, [ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_int64)]),
     "kge_bce_workspace_bytes": (_sz, []),
     "kge_bce_multihot": (_c_int, [_vp, _vp, _vp, _c_int, _vp, _c_i64, _c_i64, _c_i64, _vp, _vp, _vp, _c_i64, _c_f,
                                   _vp, _vp, _sz, _vp]),

@@ -140,3 +140,16 @@ def bce_multihot(Q, bias, E, scale, csr_row, row_ptr, col, label_smoothing=0.0):
                               ws_bytes, _stream())
     _lib.check(rc)
     return loss
+
+
+def profile_begin():
+    """Start bracketing every contraction launch with HIP events on its stream."""
+    _lib.check(_lib.load().kge_profile_begin())
+
+
+def profile_end():
+    """(total kernel milliseconds, number of launches) since ``profile_begin``; waits for the events."""
+    ms = ctypes.c_double(0.0)
+    n = ctypes.c_int64(0)
+    _lib.check(_lib.load().kge_profile_end(ctypes.byref(ms), ctypes.byref(n)))
+    return ms.value, n.value

@@ -142,6 +142,16 @@ int kge_bce_multihot(const float* Q, const float* bias, const void* E, int dtype
                      const int32_t* col, int64_t n_rows, float label_smoothing, float* loss,
                      void* workspace, size_t workspace_bytes, void* stream);
 
+/*
+ * Measurement aid; no counterpart in the reference.  Between kge_profile_begin() and
+ * kge_profile_end(), every launch of a contraction main loop (the MFMA kernel inside kge_scores,
+ * kge_rank_filtered, kge_topk and kge_bce_multihot) is bracketed by two HIP events recorded on the
+ * stream it is launched on.  kge_profile_end waits for those events and returns the summed
+ * kernel time in milliseconds and the number of launches.  Process-wide; not for concurrent use.
+ */
+int kge_profile_begin(void);
+int kge_profile_end(double* total_ms, int64_t* launches);
+
 #ifdef __cplusplus
 }
 #endif

@@ -215,13 +215,13 @@ def test_rank_hub_rows_shared_filters_and_ties(ops, FilterCSR, storage, d):
     np.testing.assert_array_equal(out["n_greater"].cpu().numpy(), g)
     np.testing.assert_array_equal(out["n_equal"].cpu().numpy(), t)
     np.testing.assert_array_equal(out["n_equal_lower"].cpu().numpy(), tl)
-    assert t[:50].min() >= 1                                   # the duplicates really tie
     # no filter at all
     out2 = ops.rank_filtered(Q, bias, Eg, scg, tg)
     g2, t2, tl2 = _expected_counts(S_raw, targets, [None] * B)
     np.testing.assert_array_equal(out2["n_greater"].cpu().numpy(), g2)
     np.testing.assert_array_equal(out2["n_equal"].cpu().numpy(), t2)
     np.testing.assert_array_equal(out2["n_equal_lower"].cpu().numpy(), tl2)
+    assert t2[:50].min() >= 2 and t2[80:100].min() >= 9        # duplicated / zero rows really tie
 
 
 def test_rank_all_scores_equal(ops):
