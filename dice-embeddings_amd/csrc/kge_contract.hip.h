@@ -139,42 +139,48 @@ struct RankEpi {
       gt[t] = eq[t] = eql[t] = 0;
     }
   }
+  // Rare path (padding rows in the tile, or some lane saw an exact tie).  Out of line and free of
+  // `this` so that the epilogue state stays in registers and the hot loop stays one basic block.
+  // Returns the corrections (d_gt, eq, eq_lower) for one lane.
+  struct Fix {
+    int32_t dg, eq, eql;
+  };
+  static __device__ __attribute__((noinline)) Fix tile_fix(f32x16 s, float th, int32_t tg, int64_t e_base,
+                                                           int64_t limit, int hf) {
+    Fix f{0, 0, 0};
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int64_t e = e_base + row_of(i, hf);
+      if (e < limit) {
+        if (s[i] == th) {
+          f.eq += 1;
+          f.eql += (e < (int64_t)tg) ? 1 : 0;
+        }
+      } else {
+        f.dg -= (s[i] > th) ? 1 : 0;  // the fast path counted this padding row
+      }
+    }
+    return f;
+  }
   template <bool HAS_SCALE>
   __device__ __forceinline__ void tile(int qt, const f32x16& acc, const float* sc16, float sc_col, int64_t e_base,
                                        int64_t limit) {
     const float th = thr[qt];
     unsigned long long tie = 0;
     int32_t g = 0;
-    if (e_base + 32 <= limit) {
+    f32x16 s;
 #pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        float s = acc[i];
-        if (HAS_SCALE) s *= sc16[i];
-        g += (s > th) ? 1 : 0;
-        tie |= __builtin_amdgcn_ballot_w64(s == th);
-      }
-    } else {
-#pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        float s = acc[i];
-        if (HAS_SCALE) s *= sc16[i];
-        const bool ok = e_base + row_of(i, hf) < limit;
-        g += (ok && s > th) ? 1 : 0;
-        tie |= __builtin_amdgcn_ballot_w64(ok && s == th);
-      }
+    for (int i = 0; i < 16; ++i) {
+      s[i] = HAS_SCALE ? acc[i] * sc16[i] : acc[i];
+      g += (s[i] > th) ? 1 : 0;
+      tie |= __builtin_amdgcn_ballot_w64(s[i] == th);
     }
     gt[qt] += g;
-    if (tie) {  // rare: some lane of this wave saw an exact tie
-#pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        float s = acc[i];
-        if (HAS_SCALE) s *= sc16[i];
-        const int64_t e = e_base + row_of(i, hf);
-        if (e < limit && s == th) {
-          eq[qt] += 1;
-          eql[qt] += (e < (int64_t)tgt[qt]) ? 1 : 0;
-        }
-      }
+    if (__builtin_expect(tie != 0 || e_base + 32 > limit, 0)) {
+      const Fix f = tile_fix(s, th, tgt[qt], e_base, limit, hf);
+      gt[qt] += f.dg;
+      eq[qt] += f.eq;
+      eql[qt] += f.eql;
     }
   }
   __device__ void finish() {
@@ -317,13 +323,13 @@ struct BceEpi {
 // ============================================================================================
 // qreg_kernel: bf16 MFMA, register-stationary queries, LDS-streamed entity rows.
 // ============================================================================================
-constexpr int QREG_NQT = 4;            // 32-query tiles per wave
-constexpr int QREG_WG_QUERIES = 512;   // 4 waves x 128 queries
+constexpr int QREG_NQT = 2;            // 32-query tiles per wave
+constexpr int QREG_WG_QUERIES = 256;   // 4 waves x 64 queries
 constexpr int QREG_STAGE_ROWS = 64;
 constexpr int QREG_ROW_BYTES = 272;    // 256 B of bf16 + 16 B pad: conflict-free ds_read_b128 across rows
 
 template <int EDT, template <int> class EpiT>
-__global__ void __launch_bounds__(256, 1) qreg_kernel(ContractArgs a, typename EpiT<QREG_NQT>::Args ea) {
+__global__ void __launch_bounds__(256, 2) qreg_kernel(ContractArgs a, typename EpiT<QREG_NQT>::Args ea) {
   using Epi = EpiT<QREG_NQT>;
   constexpr bool HAS_SCALE = (EDT == KGE_I8);
   __shared__ __attribute__((aligned(16))) unsigned char lds_e[2][QREG_STAGE_ROWS * QREG_ROW_BYTES];
@@ -405,6 +411,20 @@ __global__ void __launch_bounds__(256, 1) qreg_kernel(ContractArgs a, typename E
     }
   };
 
+  // Software pipeline over the 32x32 tiles: the MFMA chain of tile j is issued together with the
+  // epilogue of tile j-1 (they are independent), and the scheduler is told to interleave them, so
+  // the VALU compare/count work of one tile hides under the matrix pipe time of the next.
+  constexpr int ET = QREG_STAGE_ROWS / 32;
+  constexpr int TILES = ET * QREG_NQT;
+  f32x16 acc_prev;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) acc_prev[i] = 0.f;
+  float sc_prev[16];
+#pragma unroll
+  for (int i = 0; i < 16; ++i) sc_prev[i] = 0.f;
+  float sc_col_prev = 0.f;
+  int64_t e_prev = r1;  // "nothing to do" for the first epilogue: a tile entirely past the limit
+
   stage_load(r0);
   stage_store(0);
   __syncthreads();
@@ -412,37 +432,182 @@ __global__ void __launch_bounds__(256, 1) qreg_kernel(ContractArgs a, typename E
     const int buf = st & 1;
     const int64_t row0 = r0 + (int64_t)st * QREG_STAGE_ROWS;
     if (st + 1 < nst) stage_load(row0 + QREG_STAGE_ROWS);
+    bf16x8 ef[ET][8];
 #pragma unroll
-    for (int et = 0; et < QREG_STAGE_ROWS / 32; ++et) {
-      const int64_t e_base = row0 + et * 32;
-      if (e_base < r1) {
-        bf16x8 ef[8];
-        const unsigned char* src = &lds_e[buf][(et * 32 + c) * QREG_ROW_BYTES + hf * 16];
+    for (int et = 0; et < ET; ++et) {
+      const unsigned char* src = &lds_e[buf][(et * 32 + c) * QREG_ROW_BYTES + hf * 16];
 #pragma unroll
-        for (int s = 0; s < 8; ++s) ef[s] = *(const bf16x8*)(src + s * 32);
-        float sc16[16];
-        float sc_col = 1.f;
-        if (HAS_SCALE) {
-          if (Epi::SWAP) {
-            sc_col = lds_sc[buf][et * 32 + c];
-          } else {
+      for (int s = 0; s < 8; ++s) ef[et][s] = *(const bf16x8*)(src + s * 32);
+    }
 #pragma unroll
-            for (int i = 0; i < 16; ++i) sc16[i] = lds_sc[buf][et * 32 + row_of(i, hf)];
-          }
-        }
+    for (int j = 0; j < TILES; ++j) {
+      constexpr int dummy = 0;
+      (void)dummy;
+      const int et = j / QREG_NQT, t = j % QREG_NQT;
+      const int t_prev = (j + QREG_NQT - 1) % QREG_NQT;
+      f32x16 acc;
 #pragma unroll
-        for (int t = 0; t < QREG_NQT; ++t) {
-          f32x16 acc = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+      for (int i = 0; i < 16; ++i) acc[i] = 0.f;
 #pragma unroll
-          for (int s = 0; s < 8; ++s)
-            acc = Epi::SWAP ? mfma_bf16(qf[t][s], ef[s], acc) : mfma_bf16(ef[s], qf[t][s], acc);
-          epi.template tile<HAS_SCALE>(t, acc, sc16, sc_col, e_base, r1);
+      for (int s = 0; s < 8; ++s)
+        acc = Epi::SWAP ? mfma_bf16(qf[t][s], ef[et][s], acc) : mfma_bf16(ef[et][s], qf[t][s], acc);
+      epi.template tile<HAS_SCALE>(t_prev, acc_prev, sc_prev, sc_col_prev, e_prev, r1);
+#pragma unroll
+      for (int g = 0; g < 8; ++g) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // one MFMA
+        __builtin_amdgcn_sched_group_barrier(0x002, 6, 0);  // six VALU ops of the previous tile's epilogue
+        __builtin_amdgcn_sched_group_barrier(0x004, 2, 0);  // and their scalar mask merges
+      }
+      acc_prev = acc;
+      e_prev = row0 + et * 32;
+      if (HAS_SCALE) {
+        if (Epi::SWAP) {
+          sc_col_prev = lds_sc[buf][et * 32 + c];
+        } else if (t == 0) {
+#pragma unroll
+          for (int i = 0; i < 16; ++i) sc_prev[i] = lds_sc[buf][et * 32 + row_of(i, hf)];
         }
       }
     }
     if (st + 1 < nst) stage_store(buf ^ 1);
     __syncthreads();
   }
+  epi.template tile<HAS_SCALE>(QREG_NQT - 1, acc_prev, sc_prev, sc_col_prev, e_prev, r1);
+  epi.finish();
+}
+
+// ============================================================================================
+// qreg_async_kernel: the bf16, d == 128 fast path.  Same tiles, same reduction order and same
+// epilogues as qreg_kernel, but entity rows go from global memory straight into LDS
+// (global_load_lds_dwordx4: no staging registers, no ds_write), in 128-row stages, and each wave
+// prefetches the next stage while it computes the current one.
+//
+// LDS layout of a stage: row r is 256 B = 16 pieces of 16 B; piece p of row r sits in slot
+// r*16 + (p ^ (r & 15)).  A direct-to-LDS load writes 64 consecutive slots per wave, so the swizzle
+// is applied on the global side (which piece a lane fetches); fragment reads (ds_read_b128 of piece
+// 2s+hf for rows c..c+15 at a time) then hit 16 distinct 16-byte bank groups.
+// ============================================================================================
+constexpr int QA_STAGE_ROWS = 128;
+constexpr int QA_BUF_BYTES = QA_STAGE_ROWS * 256;
+
+template <template <int> class EpiT>
+__global__ void __launch_bounds__(256, 2) qreg_async_kernel(ContractArgs a, typename EpiT<QREG_NQT>::Args ea) {
+  using Epi = EpiT<QREG_NQT>;
+  __shared__ __attribute__((aligned(1024))) unsigned char lds_e[2 * QA_BUF_BYTES];
+
+  int qg;
+  int64_t chunk;
+  if (!decompose_wg(a, qg, chunk)) return;
+  const int tid = threadIdx.x, lane = tid & 63, c = lane & 31, hf = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  constexpr int d = 128;
+  const int64_t q0 = (int64_t)qg * QREG_WG_QUERIES + wave * (32 * QREG_NQT);
+
+  bf16x8 qf[QREG_NQT][8];
+#pragma unroll
+  for (int t = 0; t < QREG_NQT; ++t) {
+    const int64_t q = q0 + 32 * t + c;
+#pragma unroll
+    for (int s = 0; s < 8; ++s) {
+      const int k = 16 * s + 8 * hf;
+      f32x4 lo = {0.f, 0.f, 0.f, 0.f}, hi = {0.f, 0.f, 0.f, 0.f};
+      if (q < a.B) {
+        const f32x4* src = (const f32x4*)(a.Q + q * d + k);
+        lo = src[0];
+        hi = src[1];
+      }
+      qf[t][s] = cvt_bf16x8(lo, hi);
+    }
+  }
+  Epi epi;
+  epi.init(ea, q0, c, hf, a.B);
+
+  const int64_t r0 = a.e_begin + chunk * a.chunk_rows;
+  const int64_t r1 = (r0 + a.chunk_rows < a.e_end) ? r0 + a.chunk_rows : a.e_end;
+  const int nst = (int)((r1 - r0 + QA_STAGE_ROWS - 1) / QA_STAGE_ROWS);
+
+  // this lane's share of a stage: rows lrow + 16 j (j = 0..7), always the same swizzled piece
+  const int lrow = wave * 4 + (lane >> 4);
+  const int lpiece = (lane & 15) ^ (lrow & 15);
+  const unsigned char* Eb = (const unsigned char*)a.E;
+  auto stage_issue = [&](int64_t row0, int buf) {
+    unsigned char* dst = lds_e + buf * QA_BUF_BYTES + wave * 1024;
+    if (row0 + QA_STAGE_ROWS <= r1) {
+      const unsigned char* src = Eb + (row0 + lrow) * 256 + lpiece * 16;
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src + j * 4096),
+                                         (__attribute__((address_space(3))) void*)(dst + j * 4096), 16, 0, 0);
+    } else {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        int64_t g = row0 + lrow + 16 * j;
+        g = (g < r1) ? g : r1 - 1;  // padding rows repeat the last valid row; the epilogue ignores them
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(Eb + g * 256 + lpiece * 16),
+                                         (__attribute__((address_space(3))) void*)(dst + j * 4096), 16, 0, 0);
+      }
+    }
+  };
+
+  // fragment addresses of this lane inside a stage buffer (row c of e-tile 0)
+  int foff[8];
+#pragma unroll
+  for (int s = 0; s < 8; ++s) foff[s] = c * 256 + (((2 * s + hf) ^ (c & 15)) << 4);
+
+  constexpr int ET = QA_STAGE_ROWS / 32;
+  f32x16 acc_prev;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) acc_prev[i] = 0.f;
+  float sc_dummy[16];
+#pragma unroll
+  for (int i = 0; i < 16; ++i) sc_dummy[i] = 1.f;
+  int64_t e_prev = r1;
+
+  stage_issue(r0, 0);
+  for (int st = 0; st < nst; ++st) {
+    const int buf = st & 1;
+    const int64_t row0 = r0 + (int64_t)st * QA_STAGE_ROWS;
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();  // stage st has landed for every wave; everyone is done reading the other buffer
+    if (st + 1 < nst) stage_issue(row0 + QA_STAGE_ROWS, buf ^ 1);
+    const unsigned char* base = lds_e + buf * QA_BUF_BYTES;
+    bf16x8 ef[8];
+#pragma unroll
+    for (int s = 0; s < 8; ++s) ef[s] = *(const bf16x8*)(base + foff[s]);
+#pragma unroll
+    for (int et = 0; et < ET; ++et) {
+#pragma unroll
+      for (int t = 0; t < QREG_NQT; ++t) {
+        const int t_prev = (t + QREG_NQT - 1) % QREG_NQT;
+        const bool refill = (t == QREG_NQT - 1) && (et + 1 < ET);
+        bf16x8 efn[8];
+        f32x16 acc;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[i] = 0.f;
+#pragma unroll
+        for (int s = 0; s < 8; ++s) {
+          acc = Epi::SWAP ? mfma_bf16(qf[t][s], ef[s], acc) : mfma_bf16(ef[s], qf[t][s], acc);
+          // last use of fragment s for this e-tile: fetch the next e-tile's fragment into its place
+          if (refill) efn[s] = *(const bf16x8*)(base + (et + 1) * 8192 + foff[s]);
+        }
+        epi.template tile<false>(t_prev, acc_prev, sc_dummy, 1.f, e_prev, r1);
+#pragma unroll
+        for (int g = 0; g < 8; ++g) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // one MFMA
+          if (refill) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // one fragment read
+          __builtin_amdgcn_sched_group_barrier(0x002, 6, 0);  // VALU of the previous tile's epilogue
+          __builtin_amdgcn_sched_group_barrier(0x004, 2, 0);  // its scalar mask merges
+        }
+        if (refill) {
+#pragma unroll
+          for (int s = 0; s < 8; ++s) ef[s] = efn[s];
+        }
+        acc_prev = acc;
+        e_prev = row0 + et * 32;
+      }
+    }
+  }
+  epi.template tile<false>(QREG_NQT - 1, acc_prev, sc_dummy, 1.f, e_prev, r1);
   epi.finish();
 }
 

@@ -439,7 +439,7 @@ int check_contract(const char* who, const float* Q, const void* E, int dtype, co
   KGE_REQUIRE(B >= 0 && N >= 1, KGE_ERR_INVALID, "%s: B=%lld N=%lld", who, (long long)B, (long long)N);
   KGE_REQUIRE(N <= 0x7fffffffLL, KGE_ERR_INVALID, "%s: N=%lld exceeds int32 entity ids", who, (long long)N);
   KGE_REQUIRE(B <= (1 << 24), KGE_ERR_INVALID, "%s: B=%lld exceeds 2^24", who, (long long)B);
-  KGE_REQUIRE(Q && E, KGE_ERR_INVALID, "%s: null Q or E", who);
+  KGE_REQUIRE(B == 0 || (Q && E), KGE_ERR_INVALID, "%s: null Q or E", who);
   KGE_REQUIRE(((uintptr_t)Q & 15) == 0 && ((uintptr_t)E & 15) == 0, KGE_ERR_INVALID,
               "%s: Q and E must be 16-byte aligned", who);
   switch (dtype) {
@@ -474,7 +474,7 @@ ContractArgs make_args(const float* Q, const void* E, int dtype, const float* sc
   a.e_end = e_end;
   a.d = (int)d;
   const int wgq = (dtype == KGE_F32) ? KLOOP_WG_QUERIES : QREG_WG_QUERIES;
-  const int tile = (dtype == KGE_F32) ? KLOOP_TILE_ROWS : QREG_STAGE_ROWS;
+  const int tile = (dtype == KGE_F32) ? KLOOP_TILE_ROWS : (dtype == KGE_BF16 && d == 128) ? QA_STAGE_ROWS : QREG_STAGE_ROWS;
   const int max_chunk = (dtype == KGE_F32) ? 1024 : 2048;
   a.n_qgroups = (int)((B + wgq - 1) / wgq);
   const int64_t rows = e_end - e_begin;
@@ -506,6 +506,8 @@ int launch_contract(int dtype, const ContractArgs& a, const EArgs& ea, hipStream
   }
   if (dtype == KGE_F32)
     hipLaunchKernelGGL((kloop_kernel<EpiT>), grid, block, 0, st, a, ea);
+  else if (dtype == KGE_BF16 && a.d == 128)
+    hipLaunchKernelGGL((qreg_async_kernel<EpiT>), grid, block, 0, st, a, ea);
   else if (dtype == KGE_BF16)
     hipLaunchKernelGGL((qreg_kernel<KGE_BF16, EpiT>), grid, block, 0, st, a, ea);
   else
@@ -593,6 +595,7 @@ extern "C" int kge_scores(const float* Q, const float* bias, const void* E, int 
   clear_error();
   int rc = check_contract("kge_scores", Q, E, dtype, scale, B, d, N);
   if (rc) return rc;
+  if (B == 0) return KGE_OK;
   KGE_REQUIRE(S && ldS >= N, KGE_ERR_INVALID, "kge_scores: S is null or ldS=%lld < N=%lld", (long long)ldS,
               (long long)N);
   ContractArgs a = make_args(Q, E, dtype, scale, B, d, N, 0, N);
