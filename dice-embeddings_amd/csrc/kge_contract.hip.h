@@ -162,20 +162,28 @@ struct RankEpi {
     }
     return f;
   }
+  // Hot path, VALU only (no compare-to-mask / scalar round trips, which stall on this hardware):
+  // d = thr - s is exact in sign and is zero only for an exact tie; the sign bits are shifted into
+  // one register (v_alignbit) and counted once per tile, min |d| detects ties.
   template <bool HAS_SCALE>
   __device__ __forceinline__ void tile(int qt, const f32x16& acc, const float* sc16, float sc_col, int64_t e_base,
                                        int64_t limit) {
     const float th = thr[qt];
-    unsigned long long tie = 0;
-    int32_t g = 0;
     f32x16 s;
+    uint32_t bits = 0;
+    float mn = 0.f;
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
+    for (int i = 0; i < 16; i += 2) {
       s[i] = HAS_SCALE ? acc[i] * sc16[i] : acc[i];
-      g += (s[i] > th) ? 1 : 0;
-      tie |= __builtin_amdgcn_ballot_w64(s[i] == th);
+      s[i + 1] = HAS_SCALE ? acc[i + 1] * sc16[i + 1] : acc[i + 1];
+      const float d0 = th - s[i], d1 = th - s[i + 1];
+      bits = __builtin_amdgcn_alignbit(bits, __float_as_uint(d0), 31);
+      bits = __builtin_amdgcn_alignbit(bits, __float_as_uint(d1), 31);
+      mn = (i == 0) ? __builtin_fminf(__builtin_fabsf(d0), __builtin_fabsf(d1))
+                    : __builtin_fminf(__builtin_fminf(mn, __builtin_fabsf(d0)), __builtin_fabsf(d1));
     }
-    gt[qt] += g;
+    gt[qt] += __builtin_popcount(bits);
+    const unsigned long long tie = __builtin_amdgcn_ballot_w64(mn == 0.f);
     if (__builtin_expect(tie != 0 || e_base + 32 > limit, 0)) {
       const Fix f = tile_fix(s, th, tgt[qt], e_base, limit, hf);
       gt[qt] += f.dg;
@@ -191,7 +199,7 @@ struct RankEpi {
       int32_t g = gt[t] + __shfl_xor(gt[t], 32, 64);
       int32_t e = eq[t] + __shfl_xor(eq[t], 32, 64);
       int32_t l = eql[t] + __shfl_xor(eql[t], 32, 64);
-      if (hf == 0 && q < B) {
+      if (hf == 0 && q < B && thr[t] == thr[t]) {  // a NaN threshold (invalid target) publishes nothing
         if (g) atomicAdd(&a.n_gt[q], g);
         if (e) atomicAdd(&a.n_eq[q], e);
         if (l) atomicAdd(&a.n_eql[q], l);
@@ -228,14 +236,15 @@ struct TopkEpi {
   __device__ __forceinline__ void tile(int qt, const f32x16& acc, const float* sc16, float sc_col, int64_t e_base,
                                        int64_t limit) {
     const float th = tau[qt];
-    unsigned long long hit = 0;
+    float mx = 0.f;
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      float s = acc[i];
-      if (HAS_SCALE) s *= sc16[i];
-      hit |= __builtin_amdgcn_ballot_w64(s > th);
+    for (int i = 0; i < 16; i += 2) {
+      const float s0 = HAS_SCALE ? acc[i] * sc16[i] : acc[i];
+      const float s1 = HAS_SCALE ? acc[i + 1] * sc16[i + 1] : acc[i + 1];
+      mx = (i == 0) ? __builtin_fmaxf(s0, s1) : __builtin_fmaxf(__builtin_fmaxf(mx, s0), s1);
     }
-    if (hit) {
+    const unsigned long long hit = __builtin_amdgcn_ballot_w64(mx > th);
+    if (__builtin_expect(hit != 0, 0)) {
       const int64_t q = q0 + 32 * qt + c;
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
