@@ -16,6 +16,10 @@
 #pragma once
 #include "kge_internal.h"
 
+#ifndef KGE_SCHED_HINTS
+#define KGE_SCHED_HINTS 0
+#endif
+
 namespace kge {
 
 struct ContractArgs {
@@ -461,12 +465,14 @@ __global__ void __launch_bounds__(256, 2) qreg_kernel(ContractArgs a, typename E
       for (int s = 0; s < 8; ++s)
         acc = Epi::SWAP ? mfma_bf16(qf[t][s], ef[et][s], acc) : mfma_bf16(ef[et][s], qf[t][s], acc);
       epi.template tile<HAS_SCALE>(t_prev, acc_prev, sc_prev, sc_col_prev, e_prev, r1);
+#if KGE_SCHED_HINTS
 #pragma unroll
       for (int g = 0; g < 8; ++g) {
         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // one MFMA
         __builtin_amdgcn_sched_group_barrier(0x002, 6, 0);  // six VALU ops of the previous tile's epilogue
         __builtin_amdgcn_sched_group_barrier(0x004, 2, 0);  // and their scalar mask merges
       }
+#endif
       acc_prev = acc;
       e_prev = row0 + et * 32;
       if (HAS_SCALE) {
@@ -600,6 +606,7 @@ __global__ void __launch_bounds__(256, 2) qreg_async_kernel(ContractArgs a, type
           if (refill) efn[s] = *(const bf16x8*)(base + (et + 1) * 8192 + foff[s]);
         }
         epi.template tile<false>(t_prev, acc_prev, sc_dummy, 1.f, e_prev, r1);
+#if KGE_SCHED_HINTS
 #pragma unroll
         for (int g = 0; g < 8; ++g) {
           __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // one MFMA
@@ -607,6 +614,7 @@ __global__ void __launch_bounds__(256, 2) qreg_async_kernel(ContractArgs a, type
           __builtin_amdgcn_sched_group_barrier(0x002, 6, 0);  // VALU of the previous tile's epilogue
           __builtin_amdgcn_sched_group_barrier(0x004, 2, 0);  // its scalar mask merges
         }
+#endif
         if (refill) {
 #pragma unroll
           for (int s = 0; s < 8; ++s) ef[s] = efn[s];

@@ -117,11 +117,28 @@ __global__ void __launch_bounds__(256) target_score_kernel(ContractArgs a, const
   }
 }
 
-// ---- sort (csr_row, query) pairs of one sub-batch so queries sharing a filter row are adjacent
+// ---- group the queries of one sub-batch by filter row and plan the correction work -----------
+// One workgroup.  (1) sort (csr_row, query) keys so queries sharing a filter row are adjacent;
+// (2) for the first query of each group, find the group's end; (3) cut every group's filter row
+// into slices of `slice` entries (chosen so the work list stays within WORK_MAX items) and emit
+// one work item (first position, slice index) per slice.
 constexpr int SORT_MAX = 8192;
-__global__ void __launch_bounds__(1024) sort_rows_kernel(const int64_t* csr_row, int64_t b0, int nb, int64_t n_rows,
-                                                        unsigned long long* out, int npad) {
-  extern __shared__ unsigned long long keys[];
+constexpr int WORK_MAX = 4 * SORT_MAX;
+constexpr int SLICE_MIN = 1024;
+
+struct FixPlan {
+  unsigned long long* skey;  // [SORT_MAX] sorted keys: csr_row << 24 | position in sub-batch (~0 = no filter)
+  int32_t* gend;             // [SORT_MAX] for a group's first position: one past its last position
+  int32_t* work;             // [WORK_MAX][2] (first position, slice index)
+  int32_t* meta;             // [0] number of work items, [1] slice length
+};
+
+__global__ void __launch_bounds__(1024) plan_fix_kernel(const int64_t* csr_row, int64_t b0, int nb, int64_t n_rows,
+                                                       const int64_t* row_ptr, FixPlan plan, int npad) {
+  extern __shared__ unsigned long long keys[];  // npad keys, then npad ints of scan space
+  int32_t* scan = (int32_t*)(keys + npad);
+  __shared__ unsigned long long s_total;
+  __shared__ int s_slice;
   const int tid = threadIdx.x;
   for (int i = tid; i < npad; i += 1024) {
     unsigned long long key = ~0ull;
@@ -131,6 +148,7 @@ __global__ void __launch_bounds__(1024) sort_rows_kernel(const int64_t* csr_row,
     }
     keys[i] = key;
   }
+  if (tid == 0) s_total = 0;
   __syncthreads();
   for (int k = 2; k <= npad; k <<= 1) {
     for (int j = k >> 1; j > 0; j >>= 1) {
@@ -148,91 +166,150 @@ __global__ void __launch_bounds__(1024) sort_rows_kernel(const int64_t* csr_row,
       __syncthreads();
     }
   }
-  for (int i = tid; i < npad; i += 1024) out[i] = keys[i];
+  // group heads, group ends (binary search for the first key of a later row), total filter length
+  unsigned long long my_total = 0;
+  for (int i = tid; i < npad; i += 1024) {
+    const unsigned long long key = keys[i];
+    plan.skey[i] = key;
+    int32_t ge = 0;
+    if (key != ~0ull && (i == 0 || (keys[i - 1] >> 24) != (key >> 24))) {
+      const unsigned long long next_row_key = ((key >> 24) + 1) << 24;
+      int lo = i + 1, hi = npad;
+      while (lo < hi) {
+        const int mid = (lo + hi) >> 1;
+        if (keys[mid] < next_row_key) lo = mid + 1; else hi = mid;
+      }
+      ge = lo;
+      const int64_t row = (int64_t)(key >> 24);
+      my_total += (unsigned long long)(row_ptr[row + 1] - row_ptr[row]);
+    }
+    plan.gend[i] = ge;   // 0 for positions that do not start a group
+    scan[i] = ge;
+  }
+  if (my_total) atomicAdd(&s_total, my_total);
+  __syncthreads();
+  if (tid == 0) {
+    // slice length: at least SLICE_MIN, large enough that extra slices fit the work list
+    const unsigned long long room = (unsigned long long)(WORK_MAX - npad);
+    unsigned long long sl = (s_total + room - 1) / room;
+    sl = (sl + 31) & ~31ull;
+    if (sl < SLICE_MIN) sl = SLICE_MIN;
+    s_slice = (int)(sl > 0x7fffffe0ull ? 0x7fffffe0ull : sl);
+  }
+  __syncthreads();
+  const int slice = s_slice;
+  // number of slices per position (0 unless it starts a group), then an exclusive scan
+  constexpr int PER = SORT_MAX / 1024;  // positions per thread when npad == SORT_MAX
+  int cnt[PER];
+  int local = 0;
+  const int per = (npad + 1023) / 1024;
+  for (int j = 0; j < per; ++j) {
+    const int i = tid * per + j;
+    int n = 0;
+    if (i < npad && scan[i] != 0) {
+      const int64_t row = (int64_t)(keys[i] >> 24);
+      const int64_t L = row_ptr[row + 1] - row_ptr[row];
+      n = (int)((L + slice - 1) / slice);   // a group with an empty row needs no work
+    }
+    cnt[j] = n;
+    local += n;
+  }
+  __syncthreads();
+  int32_t* part = scan;  // reuse: 1024 partial sums
+  part[tid] = local;
+  __syncthreads();
+  for (int off = 1; off < 1024; off <<= 1) {
+    const int v = (tid >= off) ? part[tid - off] : 0;
+    __syncthreads();
+    part[tid] += v;
+    __syncthreads();
+  }
+  int base = part[tid] - local;
+  for (int j = 0; j < per; ++j) {
+    const int i = tid * per + j;
+    for (int z = 0; z < cnt[j]; ++z) {
+      plan.work[2 * (base + z)] = i;
+      plan.work[2 * (base + z) + 1] = z;
+    }
+    base += cnt[j];
+  }
+  if (tid == 1023) {
+    plan.meta[0] = part[1023];
+    plan.meta[1] = slice;
+  }
 }
 
 // ---- take the filtered entities back out of the counters ------------------------------------
-// One workgroup per (first query of a group sharing a filter row, slice of that row).  Scores of
-// the slice's entities are formed once per group, then every query of the group compares them
-// with its own threshold.
+// Work item = (group of queries sharing a filter row, slice of that row).  The slice's entity scores
+// are formed once (gathered rows, same MFMA chain as the main loop), then every query of the
+// group compares them with its own threshold.
 constexpr int FIX_CAP = 2048;
 template <int EDT>
-__global__ void __launch_bounds__(256) filter_fix_kernel(ContractArgs a, const unsigned long long* skey, int nb,
-                                                        int64_t b0, const int64_t* row_ptr, const int32_t* col,
+__global__ void __launch_bounds__(256) filter_fix_kernel(ContractArgs a, FixPlan plan, int64_t b0,
+                                                        const int64_t* row_ptr, const int32_t* col,
                                                         const int64_t* target, const float* thr, int32_t* n_gt,
                                                         int32_t* n_eq, int32_t* n_eql) {
   __shared__ float s_s[FIX_CAP];
   __shared__ float s_sc[FIX_CAP];
   __shared__ int32_t s_e[FIX_CAP];
-  __shared__ int s_m;
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, c = lane & 31, hf = lane >> 5;
-  const int i0 = blockIdx.x;
-  const unsigned long long key = skey[i0];
-  if (key == ~0ull) return;
-  const int64_t row = (int64_t)(key >> 24);
-  if (i0 > 0 && (int64_t)(skey[i0 - 1] >> 24) == row) return;  // not the first of its group
-
-  if (tid == 0) s_m = nb - i0;
-  __syncthreads();
-  for (int base = 1;; base += 256) {
-    const int pos = i0 + base + tid;
-    if (pos < nb && (int64_t)(skey[pos] >> 24) != row) atomicMin(&s_m, pos - i0);
-    __syncthreads();
-    const int m_now = s_m;
-    __syncthreads();
-    if (m_now < base + 256 || i0 + base + 256 >= nb) break;
-  }
-  const int m = s_m;
-
-  const int64_t L0 = row_ptr[row], L1 = row_ptr[row + 1];
-  const int64_t L = L1 - L0;
-  const int64_t split = gridDim.y;
-  const int64_t per = (((L + split - 1) / split) + 31) & ~(int64_t)31;
-  const int64_t z0 = L0 + (int64_t)blockIdx.y * per;
-  const int64_t z1 = (z0 + per < L1) ? z0 + per : L1;
-  if (z0 >= z1) return;
-  const int64_t bq = b0 + (int64_t)(key & 0xffffffull);
-
-  for (int64_t pass = z0; pass < z1; pass += FIX_CAP) {
-    const int n_here = (int)((z1 - pass < FIX_CAP) ? z1 - pass : FIX_CAP);
-    const int ntile = (n_here + 31) >> 5;
-    for (int tile = wave; tile < ntile; tile += 4) {
-      const int j = tile * 32 + c;
-      const int32_t e = (j < n_here) ? col[pass + j] : -1;
-      const bool ok = e >= 0 && (int64_t)e < a.N;
-      f32x16 acc = chain_direct<EDT>(a.E, a.d, ok ? (int64_t)e : -1, a.Q, bq, hf);
-      if (c == 0) {
+  const int n_work = plan.meta[0];
+  const int64_t slice = plan.meta[1];
+  for (int w = blockIdx.x; w < n_work; w += gridDim.x) {
+    const int i0 = plan.work[2 * w];
+    const int64_t z = plan.work[2 * w + 1];
+    const unsigned long long key = plan.skey[i0];
+    const int64_t row = (int64_t)(key >> 24);
+    const int m = plan.gend[i0] - i0;
+    const int64_t L0 = row_ptr[row], L1 = row_ptr[row + 1];
+    const int64_t z0 = L0 + z * slice;
+    const int64_t z1 = (z0 + slice < L1) ? z0 + slice : L1;
+    const int64_t bq = b0 + (int64_t)(key & 0xffffffull);
+    // threads per member in the compare phase: spread a small group over the whole workgroup
+    int tpm = 1;
+    while (tpm * 2 * m <= 256) tpm *= 2;
+    for (int64_t pass = z0; pass < z1; pass += FIX_CAP) {
+      const int n_here = (int)((z1 - pass < FIX_CAP) ? z1 - pass : FIX_CAP);
+      const int ntile = (n_here + 31) >> 5;
+      for (int tile = wave; tile < ntile; tile += 4) {
+        const int j = tile * 32 + c;
+        const int32_t e = (j < n_here) ? col[pass + j] : -1;
+        const bool ok = e >= 0 && (int64_t)e < a.N;
+        f32x16 acc = chain_direct<EDT>(a.E, a.d, ok ? (int64_t)e : -1, a.Q, bq, hf);
+        if (c == 0) {
 #pragma unroll
-        for (int i = 0; i < 16; ++i) s_s[tile * 32 + row_of(i, hf)] = acc[i];
-      }
-      if (hf == 0) {
-        s_e[j] = ok ? e : -1;
-        s_sc[j] = (EDT == KGE_I8 && ok) ? a.scale[e] : 1.f;
-      }
-    }
-    __syncthreads();
-    for (int mi = tid; mi < m; mi += 256) {
-      const int64_t b = b0 + (int64_t)(skey[i0 + mi] & 0xffffffull);
-      const float th = thr[b];
-      const int64_t t = target[b];
-      int32_t g = 0, eq = 0, eql = 0;
-      for (int j = 0; j < n_here; ++j) {
-        const int32_t e = s_e[j];
-        float s = s_s[j];
-        if (EDT == KGE_I8) s *= s_sc[j];
-        if (e >= 0 && (int64_t)e != t) {
-          g += (s > th) ? 1 : 0;
-          if (s == th) {
-            eq += 1;
-            eql += ((int64_t)e < t) ? 1 : 0;
-          }
+          for (int i = 0; i < 16; ++i) s_s[tile * 32 + row_of(i, hf)] = acc[i];
+        }
+        if (hf == 0) {
+          s_e[j] = ok ? e : -1;
+          s_sc[j] = (EDT == KGE_I8 && ok) ? a.scale[e] : 1.f;
         }
       }
-      if (g) atomicSub(&n_gt[b], g);
-      if (eq) atomicSub(&n_eq[b], eq);
-      if (eql) atomicSub(&n_eql[b], eql);
+      __syncthreads();
+      const int sub = tid % tpm;
+      for (int mi = tid / tpm; mi < m; mi += 256 / tpm) {
+        const int64_t b = b0 + (int64_t)(plan.skey[i0 + mi] & 0xffffffull);
+        const float th = thr[b];
+        const int64_t t = target[b];
+        int32_t g = 0, eq = 0, eql = 0;
+        for (int j = sub; j < n_here; j += tpm) {
+          const int32_t e = s_e[j];
+          float s = s_s[j];
+          if (EDT == KGE_I8) s *= s_sc[j];
+          if (e >= 0 && (int64_t)e != t) {
+            g += (s > th) ? 1 : 0;
+            if (s == th) {
+              eq += 1;
+              eql += ((int64_t)e < t) ? 1 : 0;
+            }
+          }
+        }
+        if (g) atomicSub(&n_gt[b], g);
+        if (eq) atomicSub(&n_eq[b], eq);
+        if (eql) atomicSub(&n_eql[b], eql);
+      }
+      __syncthreads();
     }
-    __syncthreads();
   }
 }
 
@@ -533,17 +610,26 @@ int launch_contract(int dtype, const ContractArgs& a, const EArgs& ea, hipStream
 
 struct RankWs {
   float* thr;
-  unsigned long long* skey;
+  FixPlan plan;
 };
 size_t rank_ws_layout(int64_t B, void* base, RankWs* ws) {
-  size_t o_thr = 0;
-  size_t o_key = align_up((size_t)B * 4, 256);
-  size_t total = o_key + align_up((size_t)SORT_MAX * 8, 256);
+  size_t off = 0;
+  auto take = [&](size_t bytes) {
+    size_t o = off;
+    off = align_up(off + bytes, 256);
+    return o;
+  };
+  const size_t o_thr = take((size_t)B * 4), o_key = take((size_t)SORT_MAX * 8), o_gend = take((size_t)SORT_MAX * 4);
+  const size_t o_work = take((size_t)WORK_MAX * 8), o_meta = take(16);
   if (ws) {
-    ws->thr = (float*)((char*)base + o_thr);
-    ws->skey = (unsigned long long*)((char*)base + o_key);
+    char* p = (char*)base;
+    ws->thr = (float*)(p + o_thr);
+    ws->plan.skey = (unsigned long long*)(p + o_key);
+    ws->plan.gend = (int32_t*)(p + o_gend);
+    ws->plan.work = (int32_t*)(p + o_work);
+    ws->plan.meta = (int32_t*)(p + o_meta);
   }
-  return total;
+  return off;
 }
 
 }  // namespace
@@ -639,14 +725,17 @@ extern "C" int kge_rank_filtered(const float* Q, const float* bias, const void* 
   if (filtered && n_rows > 0) {
     for (int64_t b0 = 0; b0 < B; b0 += SORT_MAX) {
       const int nb = (int)((B - b0 < SORT_MAX) ? B - b0 : SORT_MAX);
-      int npad = 2;
+      int npad = 1024;
       while (npad < nb) npad <<= 1;
-      hipLaunchKernelGGL(sort_rows_kernel, dim3(1), dim3(1024), (size_t)npad * 8, st, csr_row, b0, nb, n_rows,
-                         ws.skey, npad);
-      KGE_LAUNCH_CHECK("sort_rows_kernel");
-      dim3 grid((unsigned)nb, 32), block(256);
-      KGE_DISPATCH_DTYPE(dtype, filter_fix_kernel, grid, block, 0, st, a, ws.skey, nb, b0, row_ptr, col, target,
-                         ws.thr, n_greater, n_equal, n_equal_lower);
+      if ((size_t)npad * 12 > 65536)  // more dynamic LDS than the default limit: opt in (idempotent)
+        KGE_HIP_CHECK(hipFuncSetAttribute((const void*)plan_fix_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                          SORT_MAX * 12));
+      hipLaunchKernelGGL(plan_fix_kernel, dim3(1), dim3(1024), (size_t)npad * 12, st, csr_row, b0, nb, n_rows,
+                         row_ptr, ws.plan, npad);
+      KGE_LAUNCH_CHECK("plan_fix_kernel");
+      dim3 grid(2048), block(256);
+      KGE_DISPATCH_DTYPE(dtype, filter_fix_kernel, grid, block, 0, st, a, ws.plan, b0, row_ptr, col, target, ws.thr,
+                         n_greater, n_equal, n_equal_lower);
       KGE_LAUNCH_CHECK("filter_fix_kernel");
     }
   }

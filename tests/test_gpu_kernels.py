@@ -338,3 +338,27 @@ def test_argument_validation(ops):
     # empty batch is a no-op
     out = ops.scores(torch.zeros((0, 24), device="cuda"), None, E)
     assert out.shape == (0, 100)
+
+
+def test_rank_large_batch_spans_several_filter_plans(ops, FilterCSR):
+    """B > 8192: the filter correction is planned per sub-batch of 8192 queries (the largest plan,
+    which also needs the opt-in LDS size); one shared hub row, thousands of distinct rows."""
+    rng = np.random.default_rng(11)
+    N, R, d, B = 3000, 50, 64, 8192 + 700
+    E, Rel = random_tables(rng, N, R, d)
+    hr = random_hr(rng, N, R, B)
+    hr[::7] = hr[0]
+    targets = rng.integers(0, N, B).astype(np.int64)
+    er = random_csr(rng, hr, targets, N, R, max_len=4, hub_rows=[(0, 2500)])
+    Et, sc, Rt, Ev, Rv = stored_tables(E, Rel, "bf16")
+    Eg = dev(Et)
+    hr_g = dev(torch.from_numpy(hr))
+    Q, bias = ops.build_query("ComplEx", Eg, dev(Rt), hr_g)
+    csr = FilterCSR.from_er_vocab(er, R, device="cuda")
+    out = ops.rank_filtered(Q, bias, Eg, None, dev(torch.from_numpy(targets)), csr.rows_for(hr_g), csr.row_ptr,
+                            csr.col)
+    S_raw = ops.scores(Q, None, Eg, None).cpu().numpy()
+    g, t, tl = _expected_counts(S_raw, targets, [er[(int(h), int(r))] for h, r in hr])
+    np.testing.assert_array_equal(out["n_greater"].cpu().numpy(), g)
+    np.testing.assert_array_equal(out["n_equal"].cpu().numpy(), t)
+    np.testing.assert_array_equal(out["n_equal_lower"].cpu().numpy(), tl)
