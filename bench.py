@@ -84,6 +84,9 @@ def main():
     ap.add_argument("--config", default="c4", choices=sorted(MODE))
     ap.add_argument("--scale", type=float, default=1.0, help="shrink the workload (testing only)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run one plain 1 GiB-in / 1 GiB-out elementwise kernel (reference point for "
+                         "FETCH_SIZE / WRITE_SIZE counters under rocprofv3 --pmc)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU (no sharding, no collectives); rerun with --gpus 1",
@@ -118,6 +121,12 @@ def main():
             return model.topk(x, cfg.k)
         return model.kvsall_bce_loss(x, cfg.csr)
 
+    if args.copy_calibration:
+        src = torch.zeros(1 << 28, dtype=torch.float32, device=dev)
+        dst = torch.empty_like(src)
+        torch.add(src, 1.0, out=dst)          # reads 2^30 bytes, writes 2^30 bytes
+        torch.cuda.synchronize()
+        del src, dst
     for i in range(args.warmup):
         step(i)
     torch.cuda.synchronize()
