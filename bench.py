@@ -26,6 +26,9 @@ for _p in (ROOT, os.path.join(ROOT, "dice-embeddings_amd")):
         sys.path.insert(0, _p)
 
 PEAK_TFLOPS = {"bf16": 2500.0, "fp32": 157.3}       # MI355X dense MFMA peaks
+# HBM bytes per launch of the main loop measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on the full-size
+# workload (each scaled by what the same counter reads for a plain 1 GiB copy kernel: x2.00 and x1.00).
+MEASURED_TRAFFIC_BYTES = {"c4": 684.0e6}
 MODE = {"c1": "rank", "c2": "rank", "c3": "bce", "c4": "rank", "c5": "topk"}
 
 
@@ -163,7 +166,8 @@ def main():
                                + (f", k={cfg.k}" if mode == "topk" else ""),
                    "scale": args.scale},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_TFLOPS[compute], "unit": "TFLOP/s",
-                     "frac": achieved / PEAK_TFLOPS[compute], "traffic": None,
+                     "frac": achieved / PEAK_TFLOPS[compute],
+                     "traffic": MEASURED_TRAFFIC_BYTES.get(args.config) if args.scale == 1.0 else None,
                      "kernel": "qreg_kernel" if compute == "bf16" else "kloop_kernel",
                      "kernel_ms_avg": kernel_ms / max(launches, 1), "launches": launches,
                      "kernel_time_share": kernel_ms * 1e-3 / elapsed},
