@@ -32,6 +32,7 @@ struct ContractArgs {
   int d;
   int chunk_rows;
   int n_qgroups;
+  int n_lanes;  // persistent kernels: entity-chunk lanes per (XCD, query group)
 };
 
 __device__ __forceinline__ f32x16 mfma_bf16(bf16x8 a, bf16x8 b, f32x16 c) {
@@ -333,6 +334,28 @@ struct BceEpi {
   }
 };
 
+#ifdef KGE_DEBUG
+// Measurement-only epilogue: keeps the accumulators alive with two VALU ops per tile.
+struct NullArgs {
+  float* out;
+};
+template <int NQT>
+struct NullEpi {
+  static constexpr bool SWAP = false;
+  using Args = NullArgs;
+  Args a;
+  float sink;
+  __device__ void init(const Args& args, int64_t, int, int, int64_t) { a = args; sink = 0.f; }
+  template <bool HAS_SCALE>
+  __device__ __forceinline__ void tile(int, const f32x16& acc, const float*, float, int64_t, int64_t) {
+    sink += acc[0] + acc[15];
+  }
+  __device__ void finish() {
+    if (sink == 12345.678f) a.out[0] = sink;
+  }
+};
+#endif
+
 // ============================================================================================
 // qreg_kernel: bf16 MFMA, register-stationary queries, LDS-streamed entity rows.
 // ============================================================================================
@@ -502,25 +525,59 @@ __global__ void __launch_bounds__(256, 2) qreg_kernel(ContractArgs a, typename E
 // is applied on the global side (which piece a lane fetches); fragment reads (ds_read_b128 of piece
 // 2s+hf for rows c..c+15 at a time) then hit 16 distinct 16-byte bank groups.
 // ============================================================================================
+#ifndef KGE_QA_NQT
+#define KGE_QA_NQT 2
+#endif
+#ifndef KGE_QA_WAVES
+#define KGE_QA_WAVES 2
+#endif
+constexpr int QA_NQT = KGE_QA_NQT;                // 32-query tiles per wave
+constexpr int QA_WAVES_PER_SIMD = KGE_QA_WAVES;   // occupancy the register budget is sized for
+#ifndef KGE_QA_WG_WAVES
+#define KGE_QA_WG_WAVES 4
+#endif
+constexpr int QA_WG_WAVES = KGE_QA_WG_WAVES;      // waves per workgroup (4 or 8)
+constexpr int QA_WG_QUERIES = QA_WG_WAVES * 32 * QA_NQT;
+constexpr int QA_WGS_PER_CU = 4 * QA_WAVES_PER_SIMD / QA_WG_WAVES;
 constexpr int QA_STAGE_ROWS = 128;
 constexpr int QA_BUF_BYTES = QA_STAGE_ROWS * 256;
 
+// Work decomposition: persistent workgroups.  Flat id -> (xcd = id % 8, query group, lane); the
+// workgroup keeps its query group for its whole life and walks the entity chunks
+// xcd + 8 * (lane + n_lanes * i), i = 0, 1, ...  All query groups of a (xcd, lane) pair walk the same
+// chunks in the same order, so a chunk is pulled from HBM once and shared through that XCD's L2.
+// Stages run back to back across chunk boundaries (the prefetch never drains).
 template <template <int> class EpiT>
-__global__ void __launch_bounds__(256, 2) qreg_async_kernel(ContractArgs a, typename EpiT<QREG_NQT>::Args ea) {
-  using Epi = EpiT<QREG_NQT>;
+__global__ void __launch_bounds__(64 * QA_WG_WAVES, QA_WAVES_PER_SIMD) qreg_async_kernel(ContractArgs a, typename EpiT<QA_NQT>::Args ea) {
+  using Epi = EpiT<QA_NQT>;
   __shared__ __attribute__((aligned(1024))) unsigned char lds_e[2 * QA_BUF_BYTES];
 
-  int qg;
-  int64_t chunk;
-  if (!decompose_wg(a, qg, chunk)) return;
+  const int64_t wg = blockIdx.x;
+  const int xcd = (int)(wg & 7);
+  const int64_t slot = wg >> 3;
+  const int qg = (int)(slot % a.n_qgroups);
+  const int wlane = (int)(slot / a.n_qgroups);
   const int tid = threadIdx.x, lane = tid & 63, c = lane & 31, hf = lane >> 5;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   constexpr int d = 128;
-  const int64_t q0 = (int64_t)qg * QREG_WG_QUERIES + wave * (32 * QREG_NQT);
+  const int64_t q0 = (int64_t)qg * QA_WG_QUERIES + wave * (32 * QA_NQT);
 
-  bf16x8 qf[QREG_NQT][8];
+  // chunks of this workgroup: first, stride, count
+  const int64_t c_first = xcd + 8 * (int64_t)wlane;
+  const int64_t c_stride = 8 * (int64_t)a.n_lanes;
+  if (c_first >= a.n_chunks) return;
+  const int my_chunks = (int)((a.n_chunks - 1 - c_first) / c_stride) + 1;
+  const int spc = a.chunk_rows / QA_STAGE_ROWS;  // stages per chunk
+  const int total_stages = my_chunks * spc;
+  const int64_t r_end = a.e_end;
+  auto stage_row = [&](int k) -> int64_t {
+    const int ci = k / spc, so = k - ci * spc;
+    return a.e_begin + (c_first + c_stride * ci) * a.chunk_rows + (int64_t)so * QA_STAGE_ROWS;
+  };
+
+  bf16x8 qf[QA_NQT][8];
 #pragma unroll
-  for (int t = 0; t < QREG_NQT; ++t) {
+  for (int t = 0; t < QA_NQT; ++t) {
     const int64_t q = q0 + 32 * t + c;
 #pragma unroll
     for (int s = 0; s < 8; ++s) {
@@ -537,29 +594,27 @@ __global__ void __launch_bounds__(256, 2) qreg_async_kernel(ContractArgs a, type
   Epi epi;
   epi.init(ea, q0, c, hf, a.B);
 
-  const int64_t r0 = a.e_begin + chunk * a.chunk_rows;
-  const int64_t r1 = (r0 + a.chunk_rows < a.e_end) ? r0 + a.chunk_rows : a.e_end;
-  const int nst = (int)((r1 - r0 + QA_STAGE_ROWS - 1) / QA_STAGE_ROWS);
-
-  // this lane's share of a stage: rows lrow + 16 j (j = 0..7), always the same swizzled piece
+  // this lane's share of a stage: rows lrow + RPI * j, always the same swizzled piece (RPI is a multiple of 16)
+  constexpr int RPI = 4 * QA_WG_WAVES;            // rows one workgroup-wide load instruction covers
+  constexpr int NLD = QA_STAGE_ROWS / RPI;        // load instructions per lane per stage
   const int lrow = wave * 4 + (lane >> 4);
   const int lpiece = (lane & 15) ^ (lrow & 15);
   const unsigned char* Eb = (const unsigned char*)a.E;
   auto stage_issue = [&](int64_t row0, int buf) {
     unsigned char* dst = lds_e + buf * QA_BUF_BYTES + wave * 1024;
-    if (row0 + QA_STAGE_ROWS <= r1) {
+    if (row0 + QA_STAGE_ROWS <= r_end) {
       const unsigned char* src = Eb + (row0 + lrow) * 256 + lpiece * 16;
 #pragma unroll
-      for (int j = 0; j < 8; ++j)
-        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src + j * 4096),
-                                         (__attribute__((address_space(3))) void*)(dst + j * 4096), 16, 0, 0);
+      for (int j = 0; j < NLD; ++j)
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src + j * (RPI * 256)),
+                                         (__attribute__((address_space(3))) void*)(dst + j * (RPI * 256)), 16, 0, 0);
     } else {
 #pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        int64_t g = row0 + lrow + 16 * j;
-        g = (g < r1) ? g : r1 - 1;  // padding rows repeat the last valid row; the epilogue ignores them
+      for (int j = 0; j < NLD; ++j) {
+        int64_t g = row0 + lrow + RPI * j;
+        g = (g < r_end) ? g : r_end - 1;  // padding rows repeat the last valid row; the epilogue ignores them
         __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(Eb + g * 256 + lpiece * 16),
-                                         (__attribute__((address_space(3))) void*)(dst + j * 4096), 16, 0, 0);
+                                         (__attribute__((address_space(3))) void*)(dst + j * (RPI * 256)), 16, 0, 0);
       }
     }
   };
@@ -576,15 +631,26 @@ __global__ void __launch_bounds__(256, 2) qreg_async_kernel(ContractArgs a, type
   float sc_dummy[16];
 #pragma unroll
   for (int i = 0; i < 16; ++i) sc_dummy[i] = 1.f;
-  int64_t e_prev = r1;
+  int64_t e_prev = r_end;  // "nothing to do" for the first epilogue: a tile entirely past the limit
 
-  stage_issue(r0, 0);
-  for (int st = 0; st < nst; ++st) {
+  int64_t row_next = stage_row(0);
+  stage_issue(row_next, 0);
+  for (int st = 0; st < total_stages; ++st) {
     const int buf = st & 1;
-    const int64_t row0 = r0 + (int64_t)st * QA_STAGE_ROWS;
+    const int64_t row0 = row_next;
+    if (row0 >= r_end) break;  // only the trailing stages of the table's last chunk can be empty
+#ifndef KGE_DBG_NO_BARRIER
+#ifndef KGE_DBG_NO_VMWAIT
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#endif
     __syncthreads();  // stage st has landed for every wave; everyone is done reading the other buffer
-    if (st + 1 < nst) stage_issue(row0 + QA_STAGE_ROWS, buf ^ 1);
+#endif
+    if (st + 1 < total_stages) {
+      row_next = stage_row(st + 1);
+#ifndef KGE_DBG_NO_GLOBAL
+      if (row_next < r_end) stage_issue(row_next, buf ^ 1);
+#endif
+    }
     const unsigned char* base = lds_e + buf * QA_BUF_BYTES;
     bf16x8 ef[8];
 #pragma unroll
@@ -592,9 +658,9 @@ __global__ void __launch_bounds__(256, 2) qreg_async_kernel(ContractArgs a, type
 #pragma unroll
     for (int et = 0; et < ET; ++et) {
 #pragma unroll
-      for (int t = 0; t < QREG_NQT; ++t) {
-        const int t_prev = (t + QREG_NQT - 1) % QREG_NQT;
-        const bool refill = (t == QREG_NQT - 1) && (et + 1 < ET);
+      for (int t = 0; t < QA_NQT; ++t) {
+        const int t_prev = (t + QA_NQT - 1) % QA_NQT;
+        const bool refill = (t == QA_NQT - 1) && (et + 1 < ET);
         bf16x8 efn[8];
         f32x16 acc;
 #pragma unroll
@@ -603,9 +669,13 @@ __global__ void __launch_bounds__(256, 2) qreg_async_kernel(ContractArgs a, type
         for (int s = 0; s < 8; ++s) {
           acc = Epi::SWAP ? mfma_bf16(qf[t][s], ef[s], acc) : mfma_bf16(ef[s], qf[t][s], acc);
           // last use of fragment s for this e-tile: fetch the next e-tile's fragment into its place
+#ifndef KGE_DBG_NO_LDSREAD
           if (refill) efn[s] = *(const bf16x8*)(base + (et + 1) * 8192 + foff[s]);
+#else
+          if (refill) efn[s] = ef[s];
+#endif
         }
-        epi.template tile<false>(t_prev, acc_prev, sc_dummy, 1.f, e_prev, r1);
+        epi.template tile<false>(t_prev, acc_prev, sc_dummy, 1.f, e_prev, r_end);
 #if KGE_SCHED_HINTS
 #pragma unroll
         for (int g = 0; g < 8; ++g) {
@@ -624,7 +694,7 @@ __global__ void __launch_bounds__(256, 2) qreg_async_kernel(ContractArgs a, type
       }
     }
   }
-  epi.template tile<false>(QREG_NQT - 1, acc_prev, sc_dummy, 1.f, e_prev, r1);
+  epi.template tile<false>(QA_NQT - 1, acc_prev, sc_dummy, 1.f, e_prev, r_end);
   epi.finish();
 }
 

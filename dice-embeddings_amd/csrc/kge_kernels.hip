@@ -550,11 +550,25 @@ ContractArgs make_args(const float* Q, const void* E, int dtype, const float* sc
   a.e_begin = e_begin;
   a.e_end = e_end;
   a.d = (int)d;
-  const int wgq = (dtype == KGE_F32) ? KLOOP_WG_QUERIES : QREG_WG_QUERIES;
-  const int tile = (dtype == KGE_F32) ? KLOOP_TILE_ROWS : (dtype == KGE_BF16 && d == 128) ? QA_STAGE_ROWS : QREG_STAGE_ROWS;
-  const int max_chunk = (dtype == KGE_F32) ? 1024 : 2048;
+  const int wgq = (dtype == KGE_F32) ? KLOOP_WG_QUERIES : (dtype == KGE_BF16 && d == 128) ? QA_WG_QUERIES : QREG_WG_QUERIES;
   a.n_qgroups = (int)((B + wgq - 1) / wgq);
+  if (a.n_qgroups < 1) a.n_qgroups = 1;
   const int64_t rows = e_end - e_begin;
+  a.n_lanes = 1;
+  if (dtype == KGE_BF16 && d == 128) {
+    // persistent path: resident workgroups per XCD (32 CUs x QA_WAVES_PER_SIMD) shared by the query groups
+    a.n_lanes = 32 * QA_WGS_PER_CU / a.n_qgroups;
+    if (a.n_lanes < 1) a.n_lanes = 1;
+    int64_t chunk = rows / (8 * (int64_t)a.n_lanes * 4);  // aim for >= 4 chunks per workgroup
+    chunk = (chunk + QA_STAGE_ROWS - 1) / QA_STAGE_ROWS * QA_STAGE_ROWS;
+    if (chunk < QA_STAGE_ROWS) chunk = QA_STAGE_ROWS;
+    if (chunk > 1024) chunk = 1024;
+    a.chunk_rows = (int)chunk;
+    a.n_chunks = (rows + chunk - 1) / chunk;
+    return a;
+  }
+  const int tile = (dtype == KGE_F32) ? KLOOP_TILE_ROWS : QREG_STAGE_ROWS;
+  const int max_chunk = (dtype == KGE_F32) ? 1024 : 2048;
   int64_t chunk = rows * a.n_qgroups / 2048;  // aim for >= 2048 workgroups (8 per CU)
   chunk = (chunk + tile - 1) / tile * tile;
   if (chunk < tile) chunk = tile;
@@ -567,9 +581,10 @@ ContractArgs make_args(const float* Q, const void* E, int dtype, const float* sc
 template <template <int> class EpiT, class EArgs>
 int launch_contract(int dtype, const ContractArgs& a, const EArgs& ea, hipStream_t st, const char* name) {
   if (a.B == 0 || a.e_end <= a.e_begin) return KGE_OK;
-  const int64_t nwg = (a.n_chunks + 7) / 8 * 8 * a.n_qgroups;
+  const bool persistent = (dtype == KGE_BF16 && a.d == 128);
+  const int64_t nwg = persistent ? 8 * (int64_t)a.n_qgroups * a.n_lanes : (a.n_chunks + 7) / 8 * 8 * a.n_qgroups;
   KGE_REQUIRE(nwg <= 0x7fffffffLL, KGE_ERR_INVALID, "%s: grid of %lld workgroups too large", name, (long long)nwg);
-  dim3 grid((unsigned)nwg), block(256);
+  dim3 grid((unsigned)nwg), block(persistent ? 64 * QA_WG_WAVES : 256);
   hipEvent_t ev0 = nullptr, ev1 = nullptr;
   bool timed = false;
   {
@@ -838,3 +853,14 @@ extern "C" int kge_bce_multihot(const float* Q, const float* bias, const void* E
   KGE_LAUNCH_CHECK("bce_final_kernel");
   return KGE_OK;
 }
+
+#ifdef KGE_DEBUG
+// Measurement-only: the contraction main loop with an (almost) empty epilogue.
+extern "C" int kge_debug_contract_null(const float* Q, const void* E, int dtype, const float* scale, int64_t B,
+                                       int64_t d, int64_t N, float* out, void* stream) {
+  clear_error();
+  ContractArgs a = make_args(Q, E, dtype, scale, B, d, N, 0, N);
+  NullArgs ea{out};
+  return launch_contract<NullEpi>(dtype, a, ea, (hipStream_t)stream, "kge_debug_contract_null");
+}
+#endif
