@@ -43,24 +43,35 @@ __device__ __forceinline__ f32x16 chain_direct(const void* E, int d, int64_t e_r
     const float* Ef = (const float*)E;
     const bool vec_ok = (d & 3) == 0;
     const int nkb = (d + 7) >> 3;
-    for (int kb = 0; kb < nkb; ++kb) {
-      const int k = kb * 8 + 4 * hf;
-      f32x4 fe = {0.f, 0.f, 0.f, 0.f}, fq = {0.f, 0.f, 0.f, 0.f};
-      if (vec_ok) {
-        if (k < d) {
-          if (e_row >= 0) fe = *(const f32x4*)(Ef + e_row * d + k);
-          if (q_row >= 0) fq = *(const f32x4*)(Q + q_row * d + k);
-        }
-      } else {
+    // eight k-blocks per trip: all sixteen loads are issued before the first MFMA needs one
+    for (int kb0 = 0; kb0 < nkb; kb0 += 8) {
+      f32x4 fe[8], fq[8];
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
-          if (k + j < d) {
-            if (e_row >= 0) fe[j] = Ef[e_row * d + k + j];
-            if (q_row >= 0) fq[j] = Q[q_row * d + k + j];
+      for (int u = 0; u < 8; ++u) {
+        const int k = (kb0 + u) * 8 + 4 * hf;
+        fe[u] = f32x4{0.f, 0.f, 0.f, 0.f};
+        fq[u] = f32x4{0.f, 0.f, 0.f, 0.f};
+        if (vec_ok) {
+          if (k < d) {
+            if (e_row >= 0) fe[u] = *(const f32x4*)(Ef + e_row * d + k);
+            if (q_row >= 0) fq[u] = *(const f32x4*)(Q + q_row * d + k);
           }
+        } else {
+#pragma unroll
+          for (int j = 0; j < 4; ++j)
+            if (k + j < d) {
+              if (e_row >= 0) fe[u][j] = Ef[e_row * d + k + j];
+              if (q_row >= 0) fq[u][j] = Q[q_row * d + k + j];
+            }
+        }
       }
 #pragma unroll
-      for (int j = 0; j < 4; ++j) acc = mfma_f32(fe[j], fq[j], acc);
+      for (int u = 0; u < 8; ++u) {
+        if (kb0 + u < nkb) {  // uniform: whole k-blocks past d are skipped (they would only add zeros)
+#pragma unroll
+          for (int j = 0; j < 4; ++j) acc = mfma_f32(fe[u][j], fq[u][j], acc);
+        }
+      }
     }
   } else {
 #pragma unroll
@@ -115,6 +126,20 @@ __global__ void __launch_bounds__(256) target_score_kernel(ContractArgs a, const
     n_eq[q] = ok ? -1 : 0;  // the main pass counts the target as tying with itself
     n_eql[q] = 0;
   }
+}
+
+// ---- (head, relation) -> filter row: binary search in the sorted key array -----------------------
+__global__ void csr_lookup_kernel(const int64_t* hr, int64_t B, const int64_t* keys, int64_t n_rows,
+                                  int64_t num_relations, int64_t* csr_row) {
+  const int64_t b = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (b >= B) return;
+  const int64_t key = hr[2 * b] * num_relations + hr[2 * b + 1];
+  int64_t lo = 0, hi = n_rows;
+  while (lo < hi) {
+    const int64_t mid = (lo + hi) >> 1;
+    if (keys[mid] < key) lo = mid + 1; else hi = mid;
+  }
+  csr_row[b] = (lo < n_rows && keys[lo] == key) ? lo : -1;
 }
 
 // ---- group the queries of one sub-batch by filter row and plan the correction work -----------
@@ -271,18 +296,31 @@ __global__ void __launch_bounds__(256) filter_fix_kernel(ContractArgs a, FixPlan
     for (int64_t pass = z0; pass < z1; pass += FIX_CAP) {
       const int n_here = (int)((z1 - pass < FIX_CAP) ? z1 - pass : FIX_CAP);
       const int ntile = (n_here + 31) >> 5;
-      for (int tile = wave; tile < ntile; tile += 4) {
-        const int j = tile * 32 + c;
-        const int32_t e = (j < n_here) ? col[pass + j] : -1;
-        const bool ok = e >= 0 && (int64_t)e < a.N;
-        f32x16 acc = chain_direct<EDT>(a.E, a.d, ok ? (int64_t)e : -1, a.Q, bq, hf);
+      // two tiles per trip so that both row gathers are in flight before the first MFMA chain
+      for (int tile = wave; tile < ntile; tile += 8) {
+        const int j0 = tile * 32 + c, j1 = (tile + 4) * 32 + c;
+        const int32_t e0 = (j0 < n_here) ? col[pass + j0] : -1;
+        const int32_t e1 = (j1 < n_here) ? col[pass + j1] : -1;
+        const bool ok0 = e0 >= 0 && (int64_t)e0 < a.N, ok1 = e1 >= 0 && (int64_t)e1 < a.N;
+        const bool two = tile + 4 < ntile;  // uniform per wave
+        f32x16 acc0 = chain_direct<EDT>(a.E, a.d, ok0 ? (int64_t)e0 : -1, a.Q, bq, hf);
+        f32x16 acc1;
+        if (two) acc1 = chain_direct<EDT>(a.E, a.d, ok1 ? (int64_t)e1 : -1, a.Q, bq, hf);
         if (c == 0) {
 #pragma unroll
-          for (int i = 0; i < 16; ++i) s_s[tile * 32 + row_of(i, hf)] = acc[i];
+          for (int i = 0; i < 16; ++i) s_s[tile * 32 + row_of(i, hf)] = acc0[i];
+          if (two) {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) s_s[(tile + 4) * 32 + row_of(i, hf)] = acc1[i];
+          }
         }
         if (hf == 0) {
-          s_e[j] = ok ? e : -1;
-          s_sc[j] = (EDT == KGE_I8 && ok) ? a.scale[e] : 1.f;
+          s_e[j0] = ok0 ? e0 : -1;
+          s_sc[j0] = (EDT == KGE_I8 && ok0) ? a.scale[e0] : 1.f;
+          if (two) {
+            s_e[j1] = ok1 ? e1 : -1;
+            s_sc[j1] = (EDT == KGE_I8 && ok1) ? a.scale[e1] : 1.f;
+          }
         }
       }
       __syncthreads();
@@ -702,6 +740,19 @@ extern "C" int kge_scores(const float* Q, const float* bias, const void* E, int 
   ContractArgs a = make_args(Q, E, dtype, scale, B, d, N, 0, N);
   StoreArgs ea{S, bias, ldS};
   return launch_contract<StoreEpi>(dtype, a, ea, (hipStream_t)stream, "kge_scores");
+}
+
+extern "C" int kge_csr_lookup(const int64_t* hr, int64_t B, const int64_t* keys, int64_t n_rows,
+                              int64_t num_relations, int64_t* csr_row, void* stream) {
+  clear_error();
+  KGE_REQUIRE(B >= 0 && n_rows >= 0 && num_relations >= 1, KGE_ERR_INVALID, "kge_csr_lookup: B=%lld n_rows=%lld R=%lld",
+              (long long)B, (long long)n_rows, (long long)num_relations);
+  if (B == 0) return KGE_OK;
+  KGE_REQUIRE(hr && csr_row && (keys || n_rows == 0), KGE_ERR_INVALID, "kge_csr_lookup: null pointer argument");
+  hipLaunchKernelGGL(csr_lookup_kernel, dim3((unsigned)((B + 255) / 256)), dim3(256), 0, (hipStream_t)stream, hr, B, keys,
+                     n_rows, num_relations, csr_row);
+  KGE_LAUNCH_CHECK("csr_lookup_kernel");
+  return KGE_OK;
 }
 
 extern "C" size_t kge_rank_workspace_bytes(int64_t B) { return rank_ws_layout(B < 1 ? 1 : B, nullptr, nullptr); }

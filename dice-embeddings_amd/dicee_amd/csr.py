@@ -76,14 +76,9 @@ class FilterCSR:
         return len(self.col_np)
 
     def rows_for(self, hr):
-        """CSR row of every (h, r) pair of ``hr`` ([B,2] int64 tensor on the CSR's device); -1 if unknown."""
-        key = hr[:, 0] * self.num_relations + hr[:, 1]
-        if self.keys.numel() == 0:
-            return torch.full_like(key, -1)
-        pos = torch.searchsorted(self.keys, key)
-        pos_c = pos.clamp(max=self.keys.numel() - 1)
-        hit = self.keys[pos_c] == key
-        return torch.where(hit, pos_c, torch.full_like(pos_c, -1)).contiguous()
+        """CSR row of every (h, r) pair of ``hr`` ([B,2] int64 GPU tensor); -1 if unknown (kge_csr_lookup)."""
+        from . import ops
+        return ops.csr_lookup(hr.contiguous(), self.keys, self.num_relations)
 
     def rows_for_numpy(self, hr):
         hr = np.asarray(hr, dtype=np.int64)

@@ -82,6 +82,20 @@ def scores(Q, bias, E, scale=None, out=None):
     return out
 
 
+def csr_lookup(hr, keys, num_relations):
+    """CSR row of every (h, r) pair of ``hr`` [B,2] in the sorted key array ``keys``; -1 if unknown."""
+    lib = _lib.load()
+    _require_gpu(hr, keys)
+    if hr.dtype != torch.int64 or keys.dtype != torch.int64:
+        raise TypeError("hr and keys must be int64")
+    B = hr.shape[0]
+    out = torch.empty((B,), dtype=torch.int64, device=hr.device)
+    rc = lib.kge_csr_lookup(_ptr(hr), B, _ptr(keys) if keys.numel() else None, keys.numel(), int(num_relations),
+                            _ptr(out), _stream())
+    _lib.check(rc)
+    return out
+
+
 def rank_filtered(Q, bias, E, scale, target, csr_row=None, row_ptr=None, col=None):
     """Fused filtered rank. Returns dict of int32 ``n_greater, n_equal, n_equal_lower`` and fp32
     ``target_score`` (all [B])."""

@@ -92,6 +92,16 @@ int kge_scores(const float* Q, const float* bias, const void* E, int dtype, cons
                int64_t B, int64_t d, int64_t N, float* S, int64_t ldS, void* stream);
 
 /*
+ * Filter row of every (head, relation) pair: csr_row[b] = index of key hr[b,0]*num_relations + hr[b,1]
+ * in `keys` (sorted, unique, int64 [n_rows]: the CSR's row order), or -1 if the pair has no known
+ * tails.  Replaces the dict lookup `self.er_vocab[(id_e, id_r)]` of
+ * dicee/evaluation/evaluator.py:493 (vocabulary built at
+ * dicee/read_preprocess_save_load_kg/util.py:355-363).
+ */
+int kge_csr_lookup(const int64_t* hr, int64_t B, const int64_t* keys, int64_t n_rows,
+                   int64_t num_relations, int64_t* csr_row, void* stream);
+
+/*
  * Fused filtered rank: the per-row mask loop, full torch.sort and torch.where of
  * Evaluator._evaluate_entity_prediction (dicee/evaluation/evaluator.py:484-508; same loop in
  * dicee/evaluation/link_prediction.py:144-171) without writing the B x N scores.

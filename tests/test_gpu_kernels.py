@@ -362,3 +362,16 @@ def test_rank_large_batch_spans_several_filter_plans(ops, FilterCSR):
     np.testing.assert_array_equal(out["n_greater"].cpu().numpy(), g)
     np.testing.assert_array_equal(out["n_equal"].cpu().numpy(), t)
     np.testing.assert_array_equal(out["n_equal_lower"].cpu().numpy(), tl)
+
+
+def test_csr_lookup_matches_host_search(ops, FilterCSR):
+    rng = np.random.default_rng(12)
+    N, R = 500, 7
+    triples = np.stack([rng.integers(0, N, 3000), rng.integers(0, R, 3000), rng.integers(0, N, 3000)], axis=1)
+    csr = FilterCSR.from_triples(triples, R, device="cuda")
+    hr = np.stack([rng.integers(0, N + 20, 4000), rng.integers(0, R, 4000)], axis=1).astype(np.int64)
+    got = csr.rows_for(dev(torch.from_numpy(hr))).cpu().numpy()
+    np.testing.assert_array_equal(got, csr.rows_for_numpy(hr))
+    assert (got < 0).any() and (got >= 0).any()
+    empty = FilterCSR.from_triples(np.empty((0, 3), dtype=np.int64), R, device="cuda")
+    assert (empty.rows_for(dev(torch.from_numpy(hr[:5]))).cpu().numpy() == -1).all()
