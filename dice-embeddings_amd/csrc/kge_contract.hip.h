@@ -91,6 +91,12 @@ struct StoreArgs {
 template <int NQT>
 struct StoreEpi {
   static constexpr bool SWAP = true;
+  static constexpr bool STAGE_HOOK = false;
+  struct Shared {
+    int unused;
+  };
+  __device__ void bind(Shared*) {}
+  __device__ void stage_end() {}
   using Args = StoreArgs;
   Args a;
   int64_t q0, B;
@@ -127,6 +133,12 @@ struct RankArgs {
 template <int NQT>
 struct RankEpi {
   static constexpr bool SWAP = false;
+  static constexpr bool STAGE_HOOK = false;
+  struct Shared {
+    int unused;
+  };
+  __device__ void bind(Shared*) {}
+  __device__ void stage_end() {}
   using Args = RankArgs;
   Args a;
   float thr[NQT];
@@ -220,11 +232,21 @@ struct TopkArgs {
   unsigned long long* cand;  // [B, cap] packed (ordered score << 32 | 0xffffffff - entity)
   int32_t cap;
 };
+constexpr int TOPK_LQ = 1024;  // candidates a workgroup parks in LDS between flushes
 template <int NQT>
 struct TopkEpi {
   static constexpr bool SWAP = false;
+  static constexpr bool STAGE_HOOK = true;
   using Args = TopkArgs;
+  // Candidates are parked in LDS (cheap atomics) and moved to the per-query global buffers in bulk
+  // at stage boundaries, so the hot loop never waits for a global atomic's round trip.
+  struct Shared {
+    int n;
+    int q[TOPK_LQ];
+    unsigned long long key[TOPK_LQ];
+  };
   Args a;
+  Shared* sh;
   float tau[NQT];
   int64_t q0, B;
   int c, hf;
@@ -237,44 +259,79 @@ struct TopkEpi {
       tau[t] = on ? a.tau[q] : __uint_as_float(0x7f800000u);  // +inf: nothing qualifies
     }
   }
-  template <bool HAS_SCALE>
-  __device__ __forceinline__ void tile(int qt, const f32x16& acc, const float* sc16, float sc_col, int64_t e_base,
-                                       int64_t limit) {
-    const float th = tau[qt];
-    float mx = 0.f;
-#pragma unroll
-    for (int i = 0; i < 16; i += 2) {
-      const float s0 = HAS_SCALE ? acc[i] * sc16[i] : acc[i];
-      const float s1 = HAS_SCALE ? acc[i + 1] * sc16[i + 1] : acc[i + 1];
-      mx = (i == 0) ? __builtin_fmaxf(s0, s1) : __builtin_fmaxf(__builtin_fmaxf(mx, s0), s1);
+  __device__ void bind(Shared* s) {
+    sh = s;
+    if (threadIdx.x == 0) s->n = 0;
+    __syncthreads();
+  }
+  // One candidate into its query's global buffer.  A full buffer keeps a uniform sample of what
+  // arrives (reservoir sampling): the query is repaired by a later rescan, and the threshold derived
+  // from the kept entries tightens geometrically whatever order the entities come in.
+  static __device__ __forceinline__ void publish(int64_t q, unsigned long long key, int32_t* cnt,
+                                                 unsigned long long* cand, int32_t cap) {
+    int32_t slot = atomicAdd(&cnt[q], 1);
+    if (slot >= cap) {
+      const uint32_t e = 0xffffffffu - (uint32_t)(key & 0xffffffffull);
+      uint32_t h = (e * 2654435761u) ^ ((uint32_t)slot * 0x9e3779b9u);
+      h ^= h >> 15; h *= 0x2c1b3c6du; h ^= h >> 12;
+      const uint32_t r = h % (uint32_t)(slot + 1);
+      slot = (r < (uint32_t)cap) ? (int32_t)r : -1;
     }
-    const unsigned long long hit = __builtin_amdgcn_ballot_w64(mx > th);
-    if (__builtin_expect(hit != 0, 0)) {
-      const int64_t q = q0 + 32 * qt + c;
+    if (slot >= 0) cand[q * cap + slot] = key;
+  }
+  // Rare path: some element of the tile beats its query's threshold.  Out of line, so it stays out of
+  // the hot loop's register budget.
+  static __device__ __attribute__((noinline)) void collect(f32x16 s, float th, int64_t q, int64_t e_base, int64_t limit,
+                                                           int hf, Shared* sh, int32_t* cnt, unsigned long long* cand,
+                                                           int32_t cap) {
 #pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        float s = acc[i];
-        if (HAS_SCALE) s *= sc16[i];
-        const int64_t e = e_base + row_of(i, hf);
-        if (s > th && e < limit) {
-          int32_t slot = atomicAdd(&a.cnt[q], 1);
-          if (slot >= a.cap) {
-            // Buffer full: the query is repaired by a later rescan.  Keep a uniform sample of what
-            // arrives (reservoir sampling) so that the threshold derived from the kept entries
-            // tightens geometrically whatever order the entities come in.
-            uint32_t h = ((uint32_t)e * 2654435761u) ^ ((uint32_t)slot * 0x9e3779b9u);
-            h ^= h >> 15; h *= 0x2c1b3c6du; h ^= h >> 12;
-            const uint32_t r = h % (uint32_t)(slot + 1);
-            slot = (r < (uint32_t)a.cap) ? (int32_t)r : -1;
-          }
-          if (slot >= 0)
-            a.cand[q * a.cap + slot] =
-                ((unsigned long long)f32_to_ordered(s) << 32) | (unsigned long long)(0xffffffffu - (uint32_t)e);
+    for (int i = 0; i < 16; ++i) {
+      const int64_t e = e_base + row_of(i, hf);
+      if (s[i] > th && e < limit) {
+        const unsigned long long key =
+            ((unsigned long long)f32_to_ordered(s[i]) << 32) | (unsigned long long)(0xffffffffu - (uint32_t)e);
+        const int idx = atomicAdd(&sh->n, 1);
+        if (idx < TOPK_LQ) {
+          sh->q[idx] = (int)q;
+          sh->key[idx] = key;
+        } else {
+          publish(q, key, cnt, cand, cap);  // LDS queue full: go to global memory directly
         }
       }
     }
   }
-  __device__ void finish() {}
+  template <bool HAS_SCALE>
+  __device__ __forceinline__ void tile(int qt, const f32x16& acc, const float* sc16, float sc_col, int64_t e_base,
+                                       int64_t limit) {
+    const float th = tau[qt];
+    f32x16 s;
+    float mx = 0.f;
+#pragma unroll
+    for (int i = 0; i < 16; i += 2) {
+      s[i] = HAS_SCALE ? acc[i] * sc16[i] : acc[i];
+      s[i + 1] = HAS_SCALE ? acc[i + 1] * sc16[i + 1] : acc[i + 1];
+      mx = (i == 0) ? __builtin_fmaxf(s[i], s[i + 1]) : __builtin_fmaxf(__builtin_fmaxf(mx, s[i]), s[i + 1]);
+    }
+    const unsigned long long hit = __builtin_amdgcn_ballot_w64(mx > th);
+    if (__builtin_expect(hit != 0, 0))
+      collect(s, th, q0 + 32 * qt + c, e_base, limit, hf, sh, a.cnt, a.cand, a.cap);
+  }
+  // Workgroup-uniform; call right after a barrier.  Empties the LDS queue once it is half full.
+  __device__ void flush(bool force) {
+    const int n = sh->n;
+    if (n >= TOPK_LQ / 2 || (force && n > 0)) {
+      const int m = n < TOPK_LQ ? n : TOPK_LQ;
+      for (int i = threadIdx.x; i < m; i += blockDim.x) publish(sh->q[i], sh->key[i], a.cnt, a.cand, a.cap);
+      __syncthreads();
+      if (threadIdx.x == 0) sh->n = 0;
+      __syncthreads();
+    }
+  }
+  __device__ void stage_end() { flush(false); }
+  __device__ void finish() {
+    __syncthreads();
+    flush(true);
+  }
 };
 
 struct BceArgs {
@@ -285,6 +342,12 @@ struct BceArgs {
 template <int NQT>
 struct BceEpi {
   static constexpr bool SWAP = false;
+  static constexpr bool STAGE_HOOK = false;
+  struct Shared {
+    int unused;
+  };
+  __device__ void bind(Shared*) {}
+  __device__ void stage_end() {}
   using Args = BceArgs;
   Args a;
   float bias[NQT];
@@ -342,6 +405,12 @@ struct NullArgs {
 template <int NQT>
 struct NullEpi {
   static constexpr bool SWAP = false;
+  static constexpr bool STAGE_HOOK = false;
+  struct Shared {
+    int unused;
+  };
+  __device__ void bind(Shared*) {}
+  __device__ void stage_end() {}
   using Args = NullArgs;
   Args a;
   float sink;
@@ -397,6 +466,8 @@ __global__ void __launch_bounds__(256, 2) qreg_kernel(ContractArgs a, typename E
   }
   Epi epi;
   epi.init(ea, q0, c, hf, a.B);
+  __shared__ typename Epi::Shared epi_sh;
+  epi.bind(&epi_sh);
 
   const int64_t r0 = a.e_begin + chunk * a.chunk_rows;
   const int64_t r1 = (r0 + a.chunk_rows < a.e_end) ? r0 + a.chunk_rows : a.e_end;
@@ -509,6 +580,7 @@ __global__ void __launch_bounds__(256, 2) qreg_kernel(ContractArgs a, typename E
     }
     if (st + 1 < nst) stage_store(buf ^ 1);
     __syncthreads();
+    if (Epi::STAGE_HOOK) epi.stage_end();
   }
   epi.template tile<HAS_SCALE>(QREG_NQT - 1, acc_prev, sc_prev, sc_col_prev, e_prev, r1);
   epi.finish();
@@ -593,6 +665,8 @@ __global__ void __launch_bounds__(64 * QA_WG_WAVES, QA_WAVES_PER_SIMD) qreg_asyn
   }
   Epi epi;
   epi.init(ea, q0, c, hf, a.B);
+  __shared__ typename Epi::Shared epi_sh;
+  epi.bind(&epi_sh);
 
   // this lane's share of a stage: rows lrow + RPI * j, always the same swizzled piece (RPI is a multiple of 16)
   constexpr int RPI = 4 * QA_WG_WAVES;            // rows one workgroup-wide load instruction covers
@@ -645,6 +719,7 @@ __global__ void __launch_bounds__(64 * QA_WG_WAVES, QA_WAVES_PER_SIMD) qreg_asyn
 #endif
     __syncthreads();  // stage st has landed for every wave; everyone is done reading the other buffer
 #endif
+    if (Epi::STAGE_HOOK) epi.stage_end();
     if (st + 1 < total_stages) {
       row_next = stage_row(st + 1);
 #ifndef KGE_DBG_NO_GLOBAL
@@ -699,6 +774,151 @@ __global__ void __launch_bounds__(64 * QA_WG_WAVES, QA_WAVES_PER_SIMD) qreg_asyn
 }
 
 // ============================================================================================
+// qreg_i8_kernel: per-row int8 table, d == 128.  Same persistent work decomposition, 128-row
+// stages, swizzled LDS layout, tiles and reduction order as qreg_async_kernel.  Rows cannot go
+// straight into LDS because they are widened to bf16 (exactly) on the way: each thread keeps its
+// share of the next stage in registers while the current stage is consumed, then converts and
+// stores it.  The fp32 row scales of a stage ride along in LDS.
+// ============================================================================================
+template <template <int> class EpiT>
+__global__ void __launch_bounds__(256, 2) qreg_i8_kernel(ContractArgs a, typename EpiT<QREG_NQT>::Args ea) {
+  using Epi = EpiT<QREG_NQT>;
+  __shared__ __attribute__((aligned(1024))) unsigned char lds_e[2 * QA_BUF_BYTES];
+  __shared__ __attribute__((aligned(16))) float lds_sc[2][QA_STAGE_ROWS];
+
+  const int64_t wg = blockIdx.x;
+  const int xcd = (int)(wg & 7);
+  const int64_t slot = wg >> 3;
+  const int qg = (int)(slot % a.n_qgroups);
+  const int wlane = (int)(slot / a.n_qgroups);
+  const int tid = threadIdx.x, lane = tid & 63, c = lane & 31, hf = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  constexpr int d = 128;
+  const int64_t q0 = (int64_t)qg * QREG_WG_QUERIES + wave * (32 * QREG_NQT);
+
+  const int64_t c_first = xcd + 8 * (int64_t)wlane;
+  const int64_t c_stride = 8 * (int64_t)a.n_lanes;
+  if (c_first >= a.n_chunks) return;
+  const int my_chunks = (int)((a.n_chunks - 1 - c_first) / c_stride) + 1;
+  const int spc = a.chunk_rows / QA_STAGE_ROWS;
+  const int total_stages = my_chunks * spc;
+  const int64_t r_end = a.e_end;
+  auto stage_row = [&](int k) -> int64_t {
+    const int ci = k / spc, so = k - ci * spc;
+    return a.e_begin + (c_first + c_stride * ci) * a.chunk_rows + (int64_t)so * QA_STAGE_ROWS;
+  };
+
+  bf16x8 qf[QREG_NQT][8];
+#pragma unroll
+  for (int t = 0; t < QREG_NQT; ++t) {
+    const int64_t q = q0 + 32 * t + c;
+#pragma unroll
+    for (int s = 0; s < 8; ++s) {
+      const int k = 16 * s + 8 * hf;
+      f32x4 lo = {0.f, 0.f, 0.f, 0.f}, hi = {0.f, 0.f, 0.f, 0.f};
+      if (q < a.B) {
+        const f32x4* src = (const f32x4*)(a.Q + q * d + k);
+        lo = src[0];
+        hi = src[1];
+      }
+      qf[t][s] = cvt_bf16x8(lo, hi);
+    }
+  }
+  Epi epi;
+  epi.init(ea, q0, c, hf, a.B);
+  __shared__ typename Epi::Shared epi_sh;
+  epi.bind(&epi_sh);
+
+  // staging: 128 rows x 128 B = 1024 pieces of 16 int8; thread handles pieces tid + 256 j
+  u32x4 stage[4];
+  float stage_sc = 0.f;
+  const int8_t* Eb = (const int8_t*)a.E;
+  auto stage_load = [&](int64_t row0) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int idx = tid + 256 * j, row = idx >> 3, piece = idx & 7;
+      int64_t g = row0 + row;
+      g = (g < r_end) ? g : r_end - 1;  // padding rows repeat the last valid row; epilogues ignore them
+      stage[j] = *(const u32x4*)(Eb + g * d + piece * 16);
+    }
+    if (tid < QA_STAGE_ROWS) {
+      int64_t g = row0 + tid;
+      g = (g < r_end) ? g : r_end - 1;
+      stage_sc = a.scale[g];
+    }
+  };
+  auto stage_store = [&](int buf) {
+    unsigned char* base = lds_e + buf * QA_BUF_BYTES;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int idx = tid + 256 * j, row = idx >> 3, piece = idx & 7;
+      const int p0 = 2 * piece, sw = row & 15;
+      *(u32x4*)(base + row * 256 + ((p0 ^ sw) << 4)) = i8x8_to_bf16x8(stage[j][0], stage[j][1]);
+      *(u32x4*)(base + row * 256 + (((p0 + 1) ^ sw) << 4)) = i8x8_to_bf16x8(stage[j][2], stage[j][3]);
+    }
+    if (tid < QA_STAGE_ROWS) lds_sc[buf][tid] = stage_sc;
+  };
+
+  int foff[8];
+#pragma unroll
+  for (int s = 0; s < 8; ++s) foff[s] = c * 256 + (((2 * s + hf) ^ (c & 15)) << 4);
+
+  constexpr int ET = QA_STAGE_ROWS / 32;
+  int64_t row_next = stage_row(0);
+  stage_load(row_next);
+  stage_store(0);
+  __syncthreads();
+  for (int st = 0; st < total_stages; ++st) {
+    const int buf = st & 1;
+    const int64_t row0 = row_next;
+    if (row0 >= r_end) break;
+    bool have_next = false;
+    if (st + 1 < total_stages) {
+      row_next = stage_row(st + 1);
+      have_next = row_next < r_end;
+      if (have_next) stage_load(row_next);
+    } else {
+      row_next = r_end;
+    }
+    const unsigned char* base = lds_e + buf * QA_BUF_BYTES;
+#pragma unroll
+    for (int et = 0; et < ET; ++et) {
+      bf16x8 ef[8];
+#pragma unroll
+      for (int s = 0; s < 8; ++s) ef[s] = *(const bf16x8*)(base + et * 8192 + foff[s]);
+      float sc16[16];
+      float sc_col = 1.f;
+      if (Epi::SWAP) {
+        sc_col = lds_sc[buf][et * 32 + c];
+      } else {
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const f32x4 v = *(const f32x4*)&lds_sc[buf][et * 32 + 8 * g + 4 * hf];
+          sc16[4 * g] = v[0];
+          sc16[4 * g + 1] = v[1];
+          sc16[4 * g + 2] = v[2];
+          sc16[4 * g + 3] = v[3];
+        }
+      }
+#pragma unroll
+      for (int t = 0; t < QREG_NQT; ++t) {
+        f32x16 acc;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[i] = 0.f;
+#pragma unroll
+        for (int s = 0; s < 8; ++s)
+          acc = Epi::SWAP ? mfma_bf16(qf[t][s], ef[s], acc) : mfma_bf16(ef[s], qf[t][s], acc);
+        epi.template tile<true>(t, acc, sc16, sc_col, row0 + et * 32, r_end);
+      }
+    }
+    if (have_next) stage_store(buf ^ 1);
+    __syncthreads();
+    if (Epi::STAGE_HOOK) epi.stage_end();
+  }
+  epi.finish();
+}
+
+// ============================================================================================
 // kloop_kernel: fp32 MFMA, 128 entities x 128 queries per workgroup, K chunks of 32 through LDS.
 // Chain order per score: k-blocks of 8 ascending; inside a block MFMA step j (0..3) consumes
 // k0 + j (lanes 0-31) and k0 + 4 + j (lanes 32-63).
@@ -726,6 +946,8 @@ __global__ void __launch_bounds__(256, 2) kloop_kernel(ContractArgs a, typename 
   const int64_t q0 = q_base + 64 * wq;
   Epi epi;
   epi.init(ea, q0, c, hf, a.B);
+  __shared__ typename Epi::Shared epi_sh;
+  epi.bind(&epi_sh);
 
   const int64_t r0 = a.e_begin + chunk * a.chunk_rows;
   const int64_t r1 = (r0 + a.chunk_rows < a.e_end) ? r0 + a.chunk_rows : a.e_end;
@@ -799,6 +1021,10 @@ __global__ void __launch_bounds__(256, 2) kloop_kernel(ContractArgs a, typename 
 #pragma unroll
         for (int tq = 0; tq < 2; ++tq) epi.template tile<false>(tq, acc[te][tq], sc16, 1.f, e_base, r1);
       }
+    }
+    if (Epi::STAGE_HOOK) {
+      __syncthreads();
+      epi.stage_end();
     }
   }
   epi.finish();

@@ -149,7 +149,7 @@ __global__ void csr_lookup_kernel(const int64_t* hr, int64_t B, const int64_t* k
 // one work item (first position, slice index) per slice.
 constexpr int SORT_MAX = 8192;
 constexpr int WORK_MAX = 4 * SORT_MAX;
-constexpr int SLICE_MIN = 1024;
+constexpr int SLICE_MIN = 128;
 
 struct FixPlan {
   unsigned long long* skey;  // [SORT_MAX] sorted keys: csr_row << 24 | position in sub-batch (~0 = no filter)
@@ -277,6 +277,7 @@ __global__ void __launch_bounds__(256) filter_fix_kernel(ContractArgs a, FixPlan
   __shared__ float s_s[FIX_CAP];
   __shared__ float s_sc[FIX_CAP];
   __shared__ int32_t s_e[FIX_CAP];
+  __shared__ int32_t s_cnt[3 * 256];
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, c = lane & 31, hf = lane >> 5;
   const int n_work = plan.meta[0];
   const int64_t slice = plan.meta[1];
@@ -324,29 +325,52 @@ __global__ void __launch_bounds__(256) filter_fix_kernel(ContractArgs a, FixPlan
         }
       }
       __syncthreads();
-      const int sub = tid % tpm;
-      for (int mi = tid / tpm; mi < m; mi += 256 / tpm) {
-        const int64_t b = b0 + (int64_t)(plan.skey[i0 + mi] & 0xffffffull);
-        const float th = thr[b];
-        const int64_t t = target[b];
-        int32_t g = 0, eq = 0, eql = 0;
-        for (int j = sub; j < n_here; j += tpm) {
-          const int32_t e = s_e[j];
-          float s = s_s[j];
-          if (EDT == KGE_I8) s *= s_sc[j];
-          if (e >= 0 && (int64_t)e != t) {
-            g += (s > th) ? 1 : 0;
-            if (s == th) {
-              eq += 1;
-              eql += ((int64_t)e < t) ? 1 : 0;
+      // compare phase: `tpm` threads share one query; their partial counts meet in LDS so that each
+      // query receives ONE global atomic per counter (hundreds of same-address atomics serialise)
+      const int sub = tid % tpm, mslot = tid / tpm, mstep = 256 / tpm;
+      for (int mbase = 0; mbase < m; mbase += mstep) {
+        const int mi = mbase + mslot;
+        s_cnt[tid] = 0;
+        s_cnt[256 + tid] = 0;
+        s_cnt[512 + tid] = 0;
+        __syncthreads();
+        int64_t b = 0;
+        if (mi < m) {
+          b = b0 + (int64_t)(plan.skey[i0 + mi] & 0xffffffull);
+          const float th = thr[b];
+          const int64_t t = target[b];
+          int32_t g = 0, eq = 0, eql = 0;
+          for (int j = sub; j < n_here; j += tpm) {
+            const int32_t e = s_e[j];
+            float s = s_s[j];
+            if (EDT == KGE_I8) s *= s_sc[j];
+            if (e >= 0 && (int64_t)e != t) {
+              g += (s > th) ? 1 : 0;
+              if (s == th) {
+                eq += 1;
+                eql += ((int64_t)e < t) ? 1 : 0;
+              }
             }
           }
+          if (tpm == 1) {
+            s_cnt[mslot] = g;
+            s_cnt[256 + mslot] = eq;
+            s_cnt[512 + mslot] = eql;
+          } else {
+            if (g) atomicAdd(&s_cnt[mslot], g);
+            if (eq) atomicAdd(&s_cnt[256 + mslot], eq);
+            if (eql) atomicAdd(&s_cnt[512 + mslot], eql);
+          }
         }
-        if (g) atomicSub(&n_gt[b], g);
-        if (eq) atomicSub(&n_eq[b], eq);
-        if (eql) atomicSub(&n_eql[b], eql);
+        __syncthreads();
+        if (mi < m && sub == 0) {
+          const int32_t g = s_cnt[mslot], eq = s_cnt[256 + mslot], eql = s_cnt[512 + mslot];
+          if (g) atomicSub(&n_gt[b], g);
+          if (eq) atomicSub(&n_eq[b], eq);
+          if (eql) atomicSub(&n_eql[b], eql);
+        }
+        __syncthreads();
       }
-      __syncthreads();
     }
   }
 }
@@ -354,7 +378,7 @@ __global__ void __launch_bounds__(256) filter_fix_kernel(ContractArgs a, FixPlan
 // ---- top-k bookkeeping ------------------------------------------------------------------------
 constexpr int TOPK_CAP = 4096;      // candidates a query can collect in one round
 constexpr int TOPK_MAX_K = 1024;
-constexpr int TOPK_FIRST_ROWS = 4096;  // first round takes everything: must not exceed TOPK_CAP
+constexpr int TOPK_FIRST_ROWS = 1024;  // first round takes everything: must not exceed TOPK_CAP
 
 struct TopkWs {
   float* tau;
@@ -588,14 +612,16 @@ ContractArgs make_args(const float* Q, const void* E, int dtype, const float* sc
   a.e_begin = e_begin;
   a.e_end = e_end;
   a.d = (int)d;
-  const int wgq = (dtype == KGE_F32) ? KLOOP_WG_QUERIES : (dtype == KGE_BF16 && d == 128) ? QA_WG_QUERIES : QREG_WG_QUERIES;
+  const bool fast_bf16 = (dtype == KGE_BF16 && d == 128), fast_i8 = (dtype == KGE_I8 && d == 128);
+  const int wgq = (dtype == KGE_F32) ? KLOOP_WG_QUERIES : fast_bf16 ? QA_WG_QUERIES : QREG_WG_QUERIES;
   a.n_qgroups = (int)((B + wgq - 1) / wgq);
   if (a.n_qgroups < 1) a.n_qgroups = 1;
   const int64_t rows = e_end - e_begin;
   a.n_lanes = 1;
-  if (dtype == KGE_BF16 && d == 128) {
-    // persistent path: resident workgroups per XCD (32 CUs x QA_WAVES_PER_SIMD) shared by the query groups
-    a.n_lanes = 32 * QA_WGS_PER_CU / a.n_qgroups;
+  if (fast_bf16 || fast_i8) {
+    // persistent paths: the workgroups resident on one XCD (32 CUs x workgroups per CU) are shared out
+    // among the query groups
+    a.n_lanes = 32 * (fast_bf16 ? QA_WGS_PER_CU : 2) / a.n_qgroups;
     if (a.n_lanes < 1) a.n_lanes = 1;
     int64_t chunk = rows / (8 * (int64_t)a.n_lanes * 4);  // aim for >= 4 chunks per workgroup
     chunk = (chunk + QA_STAGE_ROWS - 1) / QA_STAGE_ROWS * QA_STAGE_ROWS;
@@ -619,10 +645,11 @@ ContractArgs make_args(const float* Q, const void* E, int dtype, const float* sc
 template <template <int> class EpiT, class EArgs>
 int launch_contract(int dtype, const ContractArgs& a, const EArgs& ea, hipStream_t st, const char* name) {
   if (a.B == 0 || a.e_end <= a.e_begin) return KGE_OK;
-  const bool persistent = (dtype == KGE_BF16 && a.d == 128);
+  const bool fast_i8 = (dtype == KGE_I8 && a.d == 128);
+  const bool persistent = (dtype == KGE_BF16 && a.d == 128) || fast_i8;
   const int64_t nwg = persistent ? 8 * (int64_t)a.n_qgroups * a.n_lanes : (a.n_chunks + 7) / 8 * 8 * a.n_qgroups;
   KGE_REQUIRE(nwg <= 0x7fffffffLL, KGE_ERR_INVALID, "%s: grid of %lld workgroups too large", name, (long long)nwg);
-  dim3 grid((unsigned)nwg), block(persistent ? 64 * QA_WG_WAVES : 256);
+  dim3 grid((unsigned)nwg), block((persistent && !fast_i8) ? 64 * QA_WG_WAVES : 256);
   hipEvent_t ev0 = nullptr, ev1 = nullptr;
   bool timed = false;
   {
@@ -640,6 +667,8 @@ int launch_contract(int dtype, const ContractArgs& a, const EArgs& ea, hipStream
     hipLaunchKernelGGL((qreg_async_kernel<EpiT>), grid, block, 0, st, a, ea);
   else if (dtype == KGE_BF16)
     hipLaunchKernelGGL((qreg_kernel<KGE_BF16, EpiT>), grid, block, 0, st, a, ea);
+  else if (fast_i8)
+    hipLaunchKernelGGL((qreg_i8_kernel<EpiT>), grid, block, 0, st, a, ea);
   else
     hipLaunchKernelGGL((qreg_kernel<KGE_I8, EpiT>), grid, block, 0, st, a, ea);
   KGE_LAUNCH_CHECK(name);
