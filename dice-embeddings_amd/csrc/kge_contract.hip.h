@@ -232,7 +232,7 @@ struct TopkArgs {
   unsigned long long* cand;  // [B, cap] packed (ordered score << 32 | 0xffffffff - entity)
   int32_t cap;
 };
-constexpr int TOPK_LQ = 1024;  // candidates a workgroup parks in LDS between flushes
+constexpr int TOPK_LQ = 512;   // candidates a workgroup parks in LDS between flushes
 template <int NQT>
 struct TopkEpi {
   static constexpr bool SWAP = false;
@@ -932,8 +932,8 @@ constexpr int KLOOP_LDK = 36;  // floats per LDS row: 32 + 4 pad
 template <template <int> class EpiT>
 __global__ void __launch_bounds__(256, 2) kloop_kernel(ContractArgs a, typename EpiT<KLOOP_NQT>::Args ea) {
   using Epi = EpiT<KLOOP_NQT>;
-  __shared__ __attribute__((aligned(16))) float lds_e[KLOOP_TILE_ROWS * KLOOP_LDK];
-  __shared__ __attribute__((aligned(16))) float lds_q[KLOOP_WG_QUERIES * KLOOP_LDK];
+  __shared__ __attribute__((aligned(16))) float lds_e[2][KLOOP_TILE_ROWS * KLOOP_LDK];
+  __shared__ __attribute__((aligned(16))) float lds_q[2][KLOOP_WG_QUERIES * KLOOP_LDK];
 
   int qg;
   int64_t chunk;
@@ -969,62 +969,87 @@ __global__ void __launch_bounds__(256, 2) kloop_kernel(ContractArgs a, typename 
     return v;
   };
 
-  for (int64_t et0 = r0; et0 < r1; et0 += KLOOP_TILE_ROWS) {
-    f32x16 acc[2][2];
+  // Flat pipeline over (entity tile, K chunk): the next chunk's global loads are in flight while the
+  // current chunk is multiplied; LDS is double-buffered, one barrier per chunk.
+  const int n_et = (int)((r1 - r0 + KLOOP_TILE_ROWS - 1) / KLOOP_TILE_ROWS);
+  const int n_it = n_et * nkc;
+  f32x4 ve[4], vq[4];
+  auto chunk_load = [&](int it) {
+    const int et = it / nkc, kc = it - et * nkc;
+    const int64_t et0 = r0 + (int64_t)et * KLOOP_TILE_ROWS;
 #pragma unroll
-    for (int te = 0; te < 2; ++te)
+    for (int j = 0; j < 4; ++j) {
+      const int idx = tid + 256 * j, row = idx >> 3, piece = idx & 7;
+      const int k = kc * KLOOP_KC + piece * 4;
+      ve[j] = load4(Ef, et0 + row, et0 + row < r1, k);
+      vq[j] = load4(a.Q, q_base + row, q_base + row < a.B, k);
+    }
+  };
+  auto chunk_store = [&](int buf) {
 #pragma unroll
-      for (int tq = 0; tq < 2; ++tq)
+    for (int j = 0; j < 4; ++j) {
+      const int idx = tid + 256 * j, row = idx >> 3, piece = idx & 7;
+      *(f32x4*)&lds_e[buf][row * KLOOP_LDK + piece * 4] = ve[j];
+      *(f32x4*)&lds_q[buf][row * KLOOP_LDK + piece * 4] = vq[j];
+    }
+  };
+  f32x16 acc[2][2];
 #pragma unroll
-        for (int i = 0; i < 16; ++i) acc[te][tq][i] = 0.f;
+  for (int te = 0; te < 2; ++te)
+#pragma unroll
+    for (int tq = 0; tq < 2; ++tq)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc[te][tq][i] = 0.f;
 
-    for (int kc = 0; kc < nkc; ++kc) {
-      f32x4 ve[4], vq[4];
+  if (n_it > 0) {
+    chunk_load(0);
+    chunk_store(0);
+  }
+  __syncthreads();
+  int kc = 0;
+  int64_t et0 = r0;
+  for (int it = 0; it < n_it; ++it) {
+    const int buf = it & 1;
+    if (it + 1 < n_it) chunk_load(it + 1);
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const int idx = tid + 256 * j, row = idx >> 3, piece = idx & 7;
-        const int k = kc * KLOOP_KC + piece * 4;
-        ve[j] = load4(Ef, et0 + row, et0 + row < r1, k);
-        vq[j] = load4(a.Q, q_base + row, q_base + row < a.B, k);
+    for (int kb = 0; kb < KLOOP_KC / 8; ++kb) {
+      f32x4 fe[2], fq[2];
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+        fe[t] = *(const f32x4*)&lds_e[buf][(64 * we + 32 * t + c) * KLOOP_LDK + kb * 8 + 4 * hf];
+        fq[t] = *(const f32x4*)&lds_q[buf][(64 * wq + 32 * t + c) * KLOOP_LDK + kb * 8 + 4 * hf];
       }
-      __syncthreads();  // previous chunk's fragment reads are done
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const int idx = tid + 256 * j, row = idx >> 3, piece = idx & 7;
-        *(f32x4*)&lds_e[row * KLOOP_LDK + piece * 4] = ve[j];
-        *(f32x4*)&lds_q[row * KLOOP_LDK + piece * 4] = vq[j];
-      }
-      __syncthreads();
+      for (int j = 0; j < 4; ++j)
 #pragma unroll
-      for (int kb = 0; kb < KLOOP_KC / 8; ++kb) {
-        f32x4 fe[2], fq[2];
+        for (int te = 0; te < 2; ++te)
 #pragma unroll
-        for (int t = 0; t < 2; ++t) {
-          fe[t] = *(const f32x4*)&lds_e[(64 * we + 32 * t + c) * KLOOP_LDK + kb * 8 + 4 * hf];
-          fq[t] = *(const f32x4*)&lds_q[(64 * wq + 32 * t + c) * KLOOP_LDK + kb * 8 + 4 * hf];
+          for (int tq = 0; tq < 2; ++tq)
+            acc[te][tq] = Epi::SWAP ? mfma_f32(fq[tq][j], fe[te][j], acc[te][tq])
+                                    : mfma_f32(fe[te][j], fq[tq][j], acc[te][tq]);
+    }
+    if (it + 1 < n_it) chunk_store(buf ^ 1);
+    if (kc == nkc - 1) {  // this entity tile is complete
+      float sc16[16];
+#pragma unroll
+      for (int te = 0; te < 2; ++te) {
+        const int64_t e_base = et0 + 64 * we + 32 * te;
+        if (e_base < r1) {
+#pragma unroll
+          for (int tq = 0; tq < 2; ++tq) epi.template tile<false>(tq, acc[te][tq], sc16, 1.f, e_base, r1);
         }
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
+        for (int tq = 0; tq < 2; ++tq)
 #pragma unroll
-          for (int te = 0; te < 2; ++te)
-#pragma unroll
-            for (int tq = 0; tq < 2; ++tq)
-              acc[te][tq] = Epi::SWAP ? mfma_f32(fq[tq][j], fe[te][j], acc[te][tq])
-                                      : mfma_f32(fe[te][j], fq[tq][j], acc[te][tq]);
+          for (int i = 0; i < 16; ++i) acc[te][tq][i] = 0.f;
       }
-    }
-    float sc16[16];
-#pragma unroll
-    for (int te = 0; te < 2; ++te) {
-      const int64_t e_base = et0 + 64 * we + 32 * te;
-      if (e_base < r1) {
-#pragma unroll
-        for (int tq = 0; tq < 2; ++tq) epi.template tile<false>(tq, acc[te][tq], sc16, 1.f, e_base, r1);
-      }
-    }
-    if (Epi::STAGE_HOOK) {
+      kc = 0;
+      et0 += KLOOP_TILE_ROWS;
       __syncthreads();
-      epi.stage_end();
+      if (Epi::STAGE_HOOK) epi.stage_end();
+    } else {
+      ++kc;
+      __syncthreads();
     }
   }
   epi.finish();

@@ -631,14 +631,28 @@ ContractArgs make_args(const float* Q, const void* E, int dtype, const float* sc
     a.n_chunks = (rows + chunk - 1) / chunk;
     return a;
   }
+  // non-persistent paths: one workgroup per (query group, chunk).  512 workgroups are resident at a
+  // time (2 per CU); choose the chunk length whose last round of workgroups is fullest, preferring
+  // longer chunks (less per-workgroup set-up) among near-equal candidates.
   const int tile = (dtype == KGE_F32) ? KLOOP_TILE_ROWS : QREG_STAGE_ROWS;
   const int max_chunk = (dtype == KGE_F32) ? 1024 : 2048;
-  int64_t chunk = rows * a.n_qgroups / 2048;  // aim for >= 2048 workgroups (8 per CU)
-  chunk = (chunk + tile - 1) / tile * tile;
-  if (chunk < tile) chunk = tile;
-  if (chunk > max_chunk) chunk = max_chunk;
-  a.chunk_rows = (int)chunk;
-  a.n_chunks = (rows + chunk - 1) / chunk;
+  int64_t best_chunk = tile;
+  double best_eff = -1.0;
+  for (int64_t chunk = tile; chunk <= max_chunk; chunk += tile) {
+    const int64_t n_chunks = (rows + chunk - 1) / chunk;
+    const int64_t wgs = (n_chunks + 7) / 8 * 8 * a.n_qgroups;
+    const int64_t rounds = (wgs + 511) / 512;
+    const double eff = (double)rows * a.n_qgroups / ((double)rounds * 512.0 * (double)chunk);
+    if (eff > best_eff + 0.02) {
+      best_eff = eff;
+      best_chunk = chunk;
+    } else if (eff > best_eff - 0.02 && rounds >= 2) {
+      best_chunk = chunk;  // about as full, fewer and longer workgroups
+      if (eff > best_eff) best_eff = eff;
+    }
+  }
+  a.chunk_rows = (int)best_chunk;
+  a.n_chunks = (rows + best_chunk - 1) / best_chunk;
   return a;
 }
 
