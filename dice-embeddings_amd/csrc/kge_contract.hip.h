@@ -92,31 +92,44 @@ template <int NQT>
 struct StoreEpi {
   static constexpr bool SWAP = true;
   static constexpr bool STAGE_HOOK = false;
-  struct Shared {
-    int unused;
-  };
-  __device__ void bind(Shared*) {}
-  __device__ void stage_end() {}
   using Args = StoreArgs;
+  struct Shared {
+    float bias[8 * 32 * NQT];  // per wave: the biases of its 32 * NQT queries (up to 8 waves per workgroup)
+  };
   Args a;
+  const float* lb;  // this wave's slice of Shared::bias
   int64_t q0, B;
   int c, hf;
   __device__ void init(const Args& args, int64_t q0_, int c_, int hf_, int64_t B_) {
     a = args; q0 = q0_; c = c_; hf = hf_; B = B_;
   }
+  __device__ void bind(Shared* sh) {
+    float* mine = sh->bias + (threadIdx.x >> 6) * (32 * NQT);
+    for (int j = (threadIdx.x & 63); j < 32 * NQT; j += 64) {
+      const int64_t q = q0 + j;
+      mine[j] = (a.bias && q < B) ? a.bias[q] : 0.f;
+    }
+    lb = mine;
+    __syncthreads();
+  }
+  __device__ void stage_end() {}
   template <bool HAS_SCALE>
   __device__ __forceinline__ void tile(int qt, const f32x16& acc, const float* sc16, float sc_col, int64_t e_base,
                                        int64_t limit) {
     const int64_t e = e_base + c;
     if (e >= limit) return;
+    const int64_t qrow = q0 + 32 * qt + 4 * hf;  // query row of acc[0]; acc[4g + r] is row qrow + 8g + r
+    float* p = a.S + qrow * a.ldS + e;
+    const bool full = q0 + 32 * qt + 32 <= B;
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      const int64_t q = q0 + 32 * qt + row_of(i, hf);
-      if (q < B) {
-        float s = acc[i];
-        if (HAS_SCALE) s *= sc_col;
-        if (a.bias) s += a.bias[q];
-        a.S[q * a.ldS + e] = s;
+    for (int g = 0; g < 4; ++g) {
+      const f32x4 b4 = *(const f32x4*)(lb + 32 * qt + 8 * g + 4 * hf);
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        float v = acc[4 * g + r];
+        if (HAS_SCALE) v *= sc_col;
+        v += b4[r];
+        if (full || qrow + 8 * g + r < B) p[(int64_t)(8 * g + r) * a.ldS] = v;
       }
     }
   }
