@@ -11,10 +11,24 @@ import torch
 
 
 class KGE:
-    def __init__(self, model, entity_to_idx, relation_to_idx):
-        """``model``: one of ``dicee_amd.models``; ``*_to_idx``: dict str -> int (what
-        ``entity_to_idx.csv`` / ``relation_to_idx.csv`` hold in a dicee experiment folder)."""
-        self.model = model
+    def __init__(self, path=None, model=None, entity_to_idx=None, relation_to_idx=None, model_name=None,
+                 device="cuda"):
+        """Either ``path``: a dicee experiment folder (``model.pt``, ``configuration.json``, ``report.json``,
+        ``entity_to_idx.csv``, ``relation_to_idx.csv``; BaseInteractiveKGE.__init__, dicee/abstracts.py:170-213),
+        or an in-memory ``model`` of ``dicee_amd.models`` with its two ``str -> id`` vocabularies."""
+        if path is not None:
+            from .loader import load_model, load_json
+            self.path = path
+            self.model, (entity_to_idx, relation_to_idx) = load_model(
+                path, model_name=model_name or "model.pt", device=device)
+            self.configs = load_json(path + "/configuration.json")
+            self.configs.update(load_json(path + "/report.json"))
+        else:
+            if model is None or entity_to_idx is None or relation_to_idx is None:
+                raise ValueError("KGE needs either `path` or `model` with both vocabularies")
+            self.path = None
+            self.model = model
+            self.configs = dict(getattr(model, "args", {}))
         self.model.eval()
         self.entity_to_idx = dict(entity_to_idx)
         self.relation_to_idx = dict(relation_to_idx)

@@ -118,7 +118,8 @@ def test_predict_topk_and_predict_invariants():
     m = m.to("cuda")
     ents = [f"e{i}" for i in range(135)]
     rels = [f"r{i}" for i in range(46)]
-    kge = KGE(m, {e: i for i, e in enumerate(ents)}, {r: i for i, r in enumerate(rels)})
+    kge = KGE(model=m, entity_to_idx={e: i for i, e in enumerate(ents)},
+              relation_to_idx={r: i for i, r in enumerate(rels)})
     # deterministic
     a = kge.predict(h=["e3"], r=["r7"])
     b = kge.predict(h=["e3"], r=["r7"])
@@ -185,3 +186,19 @@ def test_kvsall_bce_loss_matches_training_step_forward():
         want = tcp.kvsall_bce_step("Keci", E, Rel, torch.from_numpy(x_np), pos, eps, p=0, q=1,
                                    coeff_q=torch.ones(1)).item()
         assert loss == pytest.approx(want, rel=2e-5)
+
+
+def test_kge_from_a_dicee_experiment_folder(tmp_path):
+    """model.pt / configuration.json / report.json / *_to_idx.csv round trip, then predict_topk."""
+    from dicee_amd import KGE, save_experiment
+    m, _ = _toy("Keci", 32, p=1, q=2, seed=11)
+    ents = {f"e{i}": i for i in range(135)}
+    rels = {f"r{i}": i for i in range(46)}
+    save_experiment(str(tmp_path), m, ents, rels)
+    kge = KGE(path=str(tmp_path))
+    assert kge.model.name == "Keci" and kge.model.p == 1 and kge.model.q == 2
+    assert kge.num_entities == 135 and kge.configs["num_relations"] == 46
+    for k, v in m.state_dict().items():
+        assert torch.equal(kge.model.state_dict()[k].cpu(), v)
+    ref = KGE(model=m.to("cuda"), entity_to_idx=ents, relation_to_idx=rels)
+    assert kge.predict_topk(h=["e5", "e6"], r=["r1"], topk=7) == ref.predict_topk(h=["e5", "e6"], r=["r1"], topk=7)

@@ -142,3 +142,19 @@ def test_synthetic_configs_small_scale():
     assert c5.csr is None and c5.queries.shape[1] == 3
     p = synthetic.zipf_probs(10, 1.1)
     assert p[0] > p[1] > p[-1] and p.sum() == pytest.approx(1.0)
+
+
+def test_experiment_folder_round_trip_on_cpu(tmp_path):
+    from dicee_amd import models
+    from dicee_amd.loader import load_model, save_experiment
+    m = models.QMult({"model": "QMult", "embedding_dim": 8, "num_entities": 6, "num_relations": 3})
+    ents = {"a,b": 0, "c": 1, "d e": 2, "f": 3, "g": 4, "h": 5}          # names with comma / space survive the csv
+    rels = {"r0": 0, "r1": 1, "r2": 2}
+    save_experiment(str(tmp_path), m, ents, rels)
+    loaded, (e2i, r2i) = load_model(str(tmp_path))
+    assert e2i == ents and r2i == rels and loaded.name == "QMult"
+    assert all(not p.requires_grad for p in loaded.parameters()) and not loaded.training
+    for k, v in m.state_dict().items():
+        assert torch.equal(loaded.state_dict()[k], v)
+    with pytest.raises(AssertionError):
+        load_model(str(tmp_path / "missing"))
