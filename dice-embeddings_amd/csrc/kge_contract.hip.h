@@ -619,7 +619,7 @@ __global__ void __launch_bounds__(256, 2) qreg_kernel(ContractArgs a, typename E
 constexpr int QA_NQT = KGE_QA_NQT;                // 32-query tiles per wave
 constexpr int QA_WAVES_PER_SIMD = KGE_QA_WAVES;   // occupancy the register budget is sized for
 #ifndef KGE_QA_WG_WAVES
-#define KGE_QA_WG_WAVES 4
+#define KGE_QA_WG_WAVES 8
 #endif
 constexpr int QA_WG_WAVES = KGE_QA_WG_WAVES;      // waves per workgroup (4 or 8)
 constexpr int QA_WG_QUERIES = QA_WG_WAVES * 32 * QA_NQT;

@@ -145,17 +145,18 @@ __global__ void csr_lookup_kernel(const int64_t* hr, int64_t B, const int64_t* k
 // ---- group the queries of one sub-batch by filter row and plan the correction work -----------
 // One workgroup.  (1) sort (csr_row, query) keys so queries sharing a filter row are adjacent;
 // (2) for the first query of each group, find the group's end; (3) cut every group's filter row
-// into slices of `slice` entries (chosen so the work list stays within WORK_MAX items) and emit
-// one work item (first position, slice index) per slice.
+// into slices of `slice` entries (chosen so that there are at most WORK_MAX work items) and emit
+// one record per group (first position, index of its first work item); work item w is slice
+// w - first of the group found by binary search.
 constexpr int SORT_MAX = 8192;
-constexpr int WORK_MAX = 4 * SORT_MAX;
+constexpr int WORK_MAX = 16 * SORT_MAX;  // upper bound on work items per sub-batch (bounds the slice count only)
 constexpr int SLICE_MIN = 128;
 
 struct FixPlan {
   unsigned long long* skey;  // [SORT_MAX] sorted keys: csr_row << 24 | position in sub-batch (~0 = no filter)
   int32_t* gend;             // [SORT_MAX] for a group's first position: one past its last position
-  int32_t* work;             // [WORK_MAX][2] (first position, slice index)
-  int32_t* meta;             // [0] number of work items, [1] slice length
+  int32_t* work;             // [SORT_MAX][2] per group, in order: (first position, index of its first work item)
+  int32_t* meta;             // [0] work items, [1] slice length, [2] groups
 };
 
 __global__ void __launch_bounds__(1024) plan_fix_kernel(const int64_t* csr_row, int64_t b0, int nb, int64_t n_rows,
@@ -223,44 +224,47 @@ __global__ void __launch_bounds__(1024) plan_fix_kernel(const int64_t* csr_row, 
   }
   __syncthreads();
   const int slice = s_slice;
-  // number of slices per position (0 unless it starts a group), then an exclusive scan
+  // per position: (is a group head, number of slices); one exclusive scan of the packed pair gives
+  // every group its index and the index of its first work item
   constexpr int PER = SORT_MAX / 1024;  // positions per thread when npad == SORT_MAX
-  int cnt[PER];
-  int local = 0;
+  unsigned long long val[PER];
+  unsigned long long local = 0;
   const int per = (npad + 1023) / 1024;
   for (int j = 0; j < per; ++j) {
     const int i = tid * per + j;
-    int n = 0;
+    unsigned long long v = 0;
     if (i < npad && scan[i] != 0) {
       const int64_t row = (int64_t)(keys[i] >> 24);
       const int64_t L = row_ptr[row + 1] - row_ptr[row];
-      n = (int)((L + slice - 1) / slice);   // a group with an empty row needs no work
+      const unsigned long long n = (unsigned long long)((L + slice - 1) / slice);  // an empty row needs no work
+      if (n > 0) v = (1ull << 32) | n;
     }
-    cnt[j] = n;
-    local += n;
+    val[j] = v;
+    local += v;
   }
   __syncthreads();
-  int32_t* part = scan;  // reuse: 1024 partial sums
+  __shared__ unsigned long long part[1024];
   part[tid] = local;
   __syncthreads();
   for (int off = 1; off < 1024; off <<= 1) {
-    const int v = (tid >= off) ? part[tid - off] : 0;
+    const unsigned long long v = (tid >= off) ? part[tid - off] : 0;
     __syncthreads();
     part[tid] += v;
     __syncthreads();
   }
-  int base = part[tid] - local;
+  unsigned long long base = part[tid] - local;
   for (int j = 0; j < per; ++j) {
-    const int i = tid * per + j;
-    for (int z = 0; z < cnt[j]; ++z) {
-      plan.work[2 * (base + z)] = i;
-      plan.work[2 * (base + z) + 1] = z;
+    if (val[j]) {
+      const int g = (int)(base >> 32);
+      plan.work[2 * g] = tid * per + j;
+      plan.work[2 * g + 1] = (int)(base & 0xffffffffull);
     }
-    base += cnt[j];
+    base += val[j];
   }
   if (tid == 1023) {
-    plan.meta[0] = part[1023];
+    plan.meta[0] = (int)(part[1023] & 0xffffffffull);
     plan.meta[1] = slice;
+    plan.meta[2] = (int)(part[1023] >> 32);
   }
 }
 
@@ -281,9 +285,15 @@ __global__ void __launch_bounds__(256) filter_fix_kernel(ContractArgs a, FixPlan
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, c = lane & 31, hf = lane >> 5;
   const int n_work = plan.meta[0];
   const int64_t slice = plan.meta[1];
+  const int n_groups = plan.meta[2];
   for (int w = blockIdx.x; w < n_work; w += gridDim.x) {
-    const int i0 = plan.work[2 * w];
-    const int64_t z = plan.work[2 * w + 1];
+    int lo = 0, hi = n_groups;  // last group whose first work item is <= w
+    while (hi - lo > 1) {
+      const int mid = (lo + hi) >> 1;
+      if (plan.work[2 * mid + 1] <= w) lo = mid; else hi = mid;
+    }
+    const int i0 = plan.work[2 * lo];
+    const int64_t z = w - plan.work[2 * lo + 1];
     const unsigned long long key = plan.skey[i0];
     const int64_t row = (int64_t)(key >> 24);
     const int m = plan.gend[i0] - i0;
@@ -716,7 +726,7 @@ size_t rank_ws_layout(int64_t B, void* base, RankWs* ws) {
     return o;
   };
   const size_t o_thr = take((size_t)B * 4), o_key = take((size_t)SORT_MAX * 8), o_gend = take((size_t)SORT_MAX * 4);
-  const size_t o_work = take((size_t)WORK_MAX * 8), o_meta = take(16);
+  const size_t o_work = take((size_t)SORT_MAX * 8), o_meta = take(16);
   if (ws) {
     char* p = (char*)base;
     ws->thr = (float*)(p + o_thr);
