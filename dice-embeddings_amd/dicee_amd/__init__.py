@@ -10,7 +10,8 @@ this package is the thin Python side that mirrors the reference's call surface:
 * ``kge``        ``KGE.predict_topk`` / ``predict`` / ``predict_missing_tail_entity``
                  (dicee/knowledge_graph_embeddings.py:314-579)
 * ``csr``        the known-answer filter as a CSR (dicee's ``er_vocab``)
-* ``loader``     ``load_model`` for a dicee experiment folder (dicee/static_funcs.py:246-299)
+* ``loader``     ``load_model`` / ``load_splits`` / ``evaluate_experiment`` for a dicee experiment folder
+                 (dicee/static_funcs.py:246-299, read_preprocess_save_load_kg/save_load_disk.py:40-44)
 * ``ops``        tensor-level wrappers of the C ABI
 
 There is no CPU fallback: every scoring call raises if the HIP library is not built or no GPU is
@@ -21,6 +22,6 @@ from .csr import FilterCSR  # noqa: F401
 from .models import DistMult, ComplEx, QMult, Keci, CKeci, MODEL_REGISTRY, initialize_model  # noqa: F401
 from .evaluator import Evaluator, compute_metrics_from_ranks_simple  # noqa: F401
 from .kge import KGE  # noqa: F401
-from .loader import load_model, save_experiment  # noqa: F401
+from .loader import load_model, load_splits, evaluate_experiment, save_experiment  # noqa: F401
 
 __version__ = "0.1.0"

@@ -12,10 +12,11 @@ import torch
 
 class FilterCSR:
     def __init__(self, keys, row_ptr, col, num_relations, device=None):
-        self.keys_np = np.ascontiguousarray(keys, dtype=np.int64)       # sorted unique h*R + r
-        self.row_ptr_np = np.ascontiguousarray(row_ptr, dtype=np.int64)
-        self.col_np = np.ascontiguousarray(col, dtype=np.int32)
+        self._host = (np.ascontiguousarray(keys, dtype=np.int64),       # sorted unique h*R + r
+                      np.ascontiguousarray(row_ptr, dtype=np.int64),
+                      np.ascontiguousarray(col, dtype=np.int32))
         self.num_relations = int(num_relations)
+        self.kind = "er"
         self.device = None
         self.keys = self.row_ptr = self.col = None
         if device is not None:
@@ -46,6 +47,26 @@ class FilterCSR:
         return cls(ukeys, row_ptr, t.astype(np.int32), num_relations, device)
 
     @classmethod
+    def from_triples_gpu(cls, triples, num_entities, num_relations, kind="er"):
+        """Build on the GPU (kge_csr_build).  ``triples``: int64 [n,3] GPU tensor of (h, r, t) ids, all splits
+        concatenated.  ``kind``: ``"er"`` (h, r) -> tails, the evaluator's filter; ``"re"`` (r, t) -> heads;
+        ``"ee"`` (h, t) -> relations.  Out-of-range ids raise ``ValueError``."""
+        from . import ops
+        N, R = int(num_entities), int(num_relations)
+        columns, ranges = {"er": ((0, 1, 2), (N, R, N)), "re": ((1, 2, 0), (R, N, N)),
+                           "ee": ((0, 2, 1), (N, N, R))}[kind]
+        keys, row_ptr, col, dropped = ops.csr_build(triples.contiguous(), columns, ranges)
+        if dropped:
+            raise ValueError(f"{dropped} triples hold an id outside [0, {N}) x [0, {R})")
+        self = cls.__new__(cls)
+        self.num_relations = ranges[1]                                   # multiplier of the key: a * range_b + b
+        self.kind = kind
+        self.device = triples.device
+        self.keys, self.row_ptr, self.col = keys.clone(), row_ptr.clone(), col.clone()
+        self._host = None
+        return self
+
+    @classmethod
     def from_er_vocab(cls, er_vocab, num_relations, device=None):
         """``er_vocab``: dict (h, r) -> iterable of tails (the reference's structure)."""
         n = sum(len(v) for v in er_vocab.values())
@@ -60,8 +81,28 @@ class FilterCSR:
         return cls.from_triples(triples, num_relations, device)
 
     # ---------------------------------------------------------------- access
+    def _host_arrays(self):
+        if self._host is None:                                           # built on the GPU: mirror on first use
+            self._host = (self.keys.cpu().numpy(), self.row_ptr.cpu().numpy(), self.col.cpu().numpy())
+        return self._host
+
+    @property
+    def keys_np(self):
+        return self._host_arrays()[0]
+
+    @property
+    def row_ptr_np(self):
+        return self._host_arrays()[1]
+
+    @property
+    def col_np(self):
+        return self._host_arrays()[2]
+
     def to(self, device):
-        self.device = torch.device(device)
+        device = torch.device(device)
+        if self.keys is not None and self.keys.device == device:
+            return self
+        self.device = device
         self.keys = torch.from_numpy(self.keys_np).to(self.device)
         self.row_ptr = torch.from_numpy(self.row_ptr_np).to(self.device)
         self.col = torch.from_numpy(self.col_np).to(self.device)
@@ -69,11 +110,11 @@ class FilterCSR:
 
     @property
     def num_rows(self):
-        return len(self.keys_np)
+        return len(self._host[0]) if self._host is not None else self.keys.numel()
 
     @property
     def nnz(self):
-        return len(self.col_np)
+        return len(self._host[2]) if self._host is not None else self.col.numel()
 
     def rows_for(self, hr):
         """CSR row of every (h, r) pair of ``hr`` ([B,2] int64 GPU tensor); -1 if unknown (kge_csr_lookup)."""

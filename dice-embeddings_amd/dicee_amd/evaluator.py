@@ -75,9 +75,10 @@ class Evaluator:
         self.last_ranks = None
 
     # ------------------------------------------------------------------ filter preparation
-    def vocab_preparation(self, dataset):
+    def vocab_preparation(self, dataset, device=None):
         """Build the filter CSR from ``dataset.er_vocab`` (dict or Future of one, evaluator.py:83-96) or,
-        if the dataset has none, from its train/valid/test triples (preprocess.py:51-60)."""
+        if the dataset has none, from its train/valid/test triples (preprocess.py:51-60): on the GPU when
+        ``device`` is one (kge_csr_build), else with numpy."""
         self.num_entities = dataset.num_entities
         self.num_relations = dataset.num_relations
         er = getattr(dataset, "er_vocab", None)
@@ -89,7 +90,12 @@ class Evaluator:
         else:
             parts = [np.asarray(s) for s in (dataset.train_set, getattr(dataset, "valid_set", None),
                                              getattr(dataset, "test_set", None)) if s is not None]
-            self.csr = FilterCSR.from_triples(np.concatenate(parts, axis=0), self.num_relations)
+            triples = np.concatenate(parts, axis=0)
+            if device is not None and torch.device(device).type == "cuda":
+                on_dev = torch.from_numpy(np.ascontiguousarray(triples.astype(np.int64))).to(device)
+                self.csr = FilterCSR.from_triples_gpu(on_dev, self.num_entities, self.num_relations)
+            else:
+                self.csr = FilterCSR.from_triples(triples, self.num_relations)
 
     def set_filter(self, csr_or_er_vocab, num_relations=None):
         if isinstance(csr_or_er_vocab, FilterCSR):
@@ -103,7 +109,7 @@ class Evaluator:
     def eval(self, dataset, trained_model, form_of_labelling, during_training=False):
         self.during_training = during_training
         if self.csr is None:
-            self.vocab_preparation(dataset)
+            self.vocab_preparation(dataset, device=trained_model.entity_embeddings.weight.device)
         if self.args.scoring_technique not in ["AllvsAll", "KvsAll", "1vsSample", "KvsSample", "1vsAll"]:
             raise ValueError(f"Invalid scoring technique: {self.args.scoring_technique}")
         self.eval_with_vs_all(train_set=dataset.train_set, valid_set=getattr(dataset, "valid_set", None),

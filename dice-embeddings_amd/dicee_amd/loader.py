@@ -11,6 +11,7 @@ import csv
 import json
 import os
 
+import numpy as np
 import torch
 
 from .models import MODEL_REGISTRY, initialize_model
@@ -60,9 +61,44 @@ def load_model(path_of_experiment_folder, model_name="model.pt", device=None):
     return model, (entity_to_idx, relation_to_idx)
 
 
-def save_experiment(path, model, entity_to_idx, relation_to_idx, extra_config=None):
+def load_splits(path_of_experiment_folder):
+    """``{'train_set': ndarray[n,3], 'valid_set': ..., 'test_set': ...}`` from the ``*_set.npy`` files a dicee run
+    leaves next to its model (dicee/read_preprocess_save_load_kg/save_load_disk.py:40-44; integer ids in the
+    narrowest type that holds them, dicee/static_funcs.py:373-392).  Missing splits are ``None``."""
+    out = {}
+    for name in ("train_set", "valid_set", "test_set"):
+        f = os.path.join(path_of_experiment_folder, name + ".npy")
+        out[name] = np.load(f, allow_pickle=False) if os.path.isfile(f) else None
+    if out["train_set"] is None:
+        raise FileNotFoundError(os.path.join(path_of_experiment_folder, "train_set.npy"))
+    return out
+
+
+def evaluate_experiment(path_of_experiment_folder, eval_model="train_val_test", batch_size=None, device="cuda",
+                        tie="stable"):
+    """Filtered link-prediction report of a stored dicee run: model and id triples from the folder, the filter
+    vocabulary built on the GPU over all stored splits, one fused rank call per batch.  Returns the dict the
+    reference writes to ``eval_report.json`` (``{'Train': {'H@1', 'H@3', 'H@10', 'MRR'}, 'Val': ..., 'Test': ...}``)."""
+    from types import SimpleNamespace
+    from .evaluator import Evaluator
+    model, _ = load_model(path_of_experiment_folder, device=device)
+    splits = load_splits(path_of_experiment_folder)
+    configs = load_json(os.path.join(path_of_experiment_folder, "configuration.json"))
+    args = SimpleNamespace(batch_size=int(batch_size or configs.get("batch_size") or 1024), eval_model=eval_model,
+                           scoring_technique="KvsAll", full_storage_path=None)
+    dataset = SimpleNamespace(num_entities=model.num_entities, num_relations=model.num_relations, er_vocab=None,
+                              **splits)
+    evaluator = Evaluator(args, tie=tie)
+    report = evaluator.eval(dataset, model, "EntityPrediction", during_training=True)
+    return report, evaluator
+
+
+def save_experiment(path, model, entity_to_idx, relation_to_idx, extra_config=None, splits=None):
     """Write ``model`` and its vocabularies in dicee's on-disk layout (used by tests and examples)."""
     os.makedirs(path, exist_ok=True)
+    for name, triples in (splits or {}).items():
+        if triples is not None:
+            np.save(os.path.join(path, name + ".npy"), np.asarray(triples))
     torch.save({k: v.detach().cpu() for k, v in model.state_dict().items()}, os.path.join(path, "model.pt"))
     cfg = {k: v for k, v in model.args.items() if isinstance(v, (int, float, str, bool, type(None)))}
     cfg["model"] = model.name

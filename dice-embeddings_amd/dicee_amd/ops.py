@@ -96,6 +96,35 @@ def csr_lookup(hr, keys, num_relations):
     return out
 
 
+def csr_build(triples, columns, ranges):
+    """Sorted, de-duplicated CSR of ``(triples[:, a], triples[:, b]) -> triples[:, v]`` built on the GPU.
+
+    ``triples`` int64 [n,3] on the GPU, ``columns`` = (a, b, v), ``ranges`` = (range_a, range_b, range_v).
+    Returns ``keys`` int64 [n_rows] (= a * range_b + b), ``row_ptr`` int64 [n_rows+1], ``col`` int32 [nnz] and
+    the number of triples dropped for an out-of-range id.  Reads three integers back (one stream sync)."""
+    lib = _lib.load()
+    _require_gpu(triples)
+    if triples.dtype != torch.int64 or triples.dim() != 2 or triples.shape[1] != 3:
+        raise TypeError("triples must be an int64 [n,3] tensor")
+    n = triples.shape[0]
+    dev = triples.device
+    keys = torch.empty((max(n, 1),), dtype=torch.int64, device=dev)
+    row_ptr = torch.empty((n + 1,), dtype=torch.int64, device=dev)
+    col = torch.empty((max(n, 1),), dtype=torch.int32, device=dev)
+    counts = torch.empty((3,), dtype=torch.int64, device=dev)
+    ws_bytes = lib.kge_csr_build_workspace_bytes(n)
+    if ws_bytes == 0:
+        raise _lib.KgeError(-1, lib.kge_last_error().decode("utf-8", "replace"))
+    ws = torch.empty((ws_bytes,), dtype=torch.uint8, device=dev)
+    a, b, v = (int(c) for c in columns)
+    ra, rb, rv = (int(r) for r in ranges)
+    rc = lib.kge_csr_build(_ptr(triples) if n else None, n, a, b, v, ra, rb, rv, _ptr(keys), _ptr(row_ptr), _ptr(col),
+                           _ptr(counts), _ptr(ws), ws_bytes, _stream())
+    _lib.check(rc)
+    n_rows, nnz, dropped = (int(c) for c in counts.cpu())
+    return keys[:n_rows], row_ptr[:n_rows + 1], col[:nnz], dropped
+
+
 def rank_filtered(Q, bias, E, scale, target, csr_row=None, row_ptr=None, col=None):
     """Fused filtered rank. Returns dict of int32 ``n_greater, n_equal, n_equal_lower`` and fp32
     ``target_score`` (all [B])."""

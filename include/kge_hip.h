@@ -102,6 +102,26 @@ int kge_csr_lookup(const int64_t* hr, int64_t B, const int64_t* keys, int64_t n_
                    int64_t num_relations, int64_t* csr_row, void* stream);
 
 /*
+ * Known-answer vocabulary as a CSR, built on the GPU from id triples.  For every distinct pair
+ * (a, b) = (triple[col_a], triple[col_b]) the sorted, de-duplicated values triple[col_v]:
+ *   keys    int64 [n_rows]     a * range_b + b, ascending (the row order kge_csr_lookup searches)
+ *   row_ptr int64 [n_rows + 1]
+ *   col     int32 [nnz]
+ *   counts  int64 [3]          n_rows, nnz, number of triples dropped for an id outside its range
+ * all device memory; keys and col need room for n entries, row_ptr for n + 1.  Columns (0, 1, 2)
+ * give the (head, relation) -> tails vocabulary of get_er_vocab
+ * (dicee/read_preprocess_save_load_kg/util.py:355-363; the evaluator's filter, built over
+ * train + valid + test at dicee/read_preprocess_save_load_kg/preprocess.py:51-60); (1, 2, 0) gives
+ * get_re_vocab (:366-374) and (0, 2, 1) get_ee_vocab (:377-385).  The reference keeps insertion
+ * order and duplicates; both are irrelevant to masking, which is all these lists are used for.
+ * n < 2^31; the three id ranges must fit a 62-bit packed key (KGE_ERR_UNSUPPORTED otherwise).
+ */
+size_t kge_csr_build_workspace_bytes(int64_t n);
+int kge_csr_build(const int64_t* triples, int64_t n, int col_a, int col_b, int col_v, int64_t range_a,
+                  int64_t range_b, int64_t range_v, int64_t* keys, int64_t* row_ptr, int32_t* col,
+                  int64_t* counts, void* workspace, size_t workspace_bytes, void* stream);
+
+/*
  * Fused filtered rank: the per-row mask loop, full torch.sort and torch.where of
  * Evaluator._evaluate_entity_prediction (dicee/evaluation/evaluator.py:484-508; same loop in
  * dicee/evaluation/link_prediction.py:144-171) without writing the B x N scores.

@@ -31,6 +31,9 @@ Pinning status (independent checks live in ``tests/test_oracle_pins.py``)
 * ``bce_multihot``    ``torch.nn.functional.binary_cross_entropy_with_logits``
                       on a dense target, with and without label smoothing.
 * ``bf16_round`` / ``quantize_int8_rows``  torch's bf16 cast; closed forms.
+* ``vocab`` / ``vocab_csr``  hand-written 7-triple fixture; set identities
+                      (every triple recoverable from exactly one row, rows
+                      partition the distinct triples).
 No function is "parity unpinned" with respect to the arithmetic.  What stays
 unpinned is the position an *unstable* ``torch.sort`` gives a tied target
 (``dicee/evaluation/evaluator.py:503``): that is torch's behaviour, not the
@@ -41,6 +44,38 @@ from __future__ import annotations
 import numpy as np
 
 MODELS = ("DistMult", "ComplEx", "QMult", "Keci")
+
+# --------------------------------------------------------------------------
+# known-answer vocabularies
+# --------------------------------------------------------------------------
+
+_VOCAB_COLUMNS = {"er": (0, 1, 2), "re": (1, 2, 0), "ee": (0, 2, 1)}
+
+
+def vocab(triples, kind="er"):
+    """dict pair -> list of values, insertion order, duplicates kept: ``get_er_vocab`` /
+    ``get_re_vocab`` / ``get_ee_vocab`` (dicee/read_preprocess_save_load_kg/util.py:355-385)."""
+    a, b, v = _VOCAB_COLUMNS[kind]
+    out = {}
+    for triple in triples:
+        out.setdefault((int(triple[a]), int(triple[b])), []).append(int(triple[v]))
+    return out
+
+
+def vocab_csr(triples, kind, range_b):
+    """The same vocabulary in the layout the kernels take: rows ordered by ``a * range_b + b``, values
+    sorted and de-duplicated.  Returns (keys int64, row_ptr int64, col int32)."""
+    voc = vocab(triples, kind)
+    pairs = sorted(voc, key=lambda ab: ab[0] * range_b + ab[1])
+    keys = np.array([a * range_b + b for a, b in pairs], dtype=np.int64)
+    row_ptr = np.zeros(len(pairs) + 1, dtype=np.int64)
+    col = []
+    for i, ab in enumerate(pairs):
+        vals = sorted(set(voc[ab]))
+        col.extend(vals)
+        row_ptr[i + 1] = len(col)
+    return keys, row_ptr, np.array(col, dtype=np.int32)
+
 
 # --------------------------------------------------------------------------
 # storage emulation (exists only in this build; the reference is fp32-only)

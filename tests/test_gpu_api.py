@@ -202,3 +202,28 @@ def test_kge_from_a_dicee_experiment_folder(tmp_path):
         assert torch.equal(kge.model.state_dict()[k].cpu(), v)
     ref = KGE(model=m.to("cuda"), entity_to_idx=ents, relation_to_idx=rels)
     assert kge.predict_topk(h=["e5", "e6"], r=["r1"], topk=7) == ref.predict_topk(h=["e5", "e6"], r=["r1"], topk=7)
+
+
+def test_stored_experiment_evaluates_end_to_end(tmp_path):
+    """Folder with model.pt + *_set.npy (int16 ids, as dicee stores small graphs) -> report; the filter is built on
+    the GPU from the stored splits and the ranks equal the oracle's on materialised fp64 scores."""
+    from dicee_amd import evaluate_experiment, save_experiment
+    m, triples = _toy("ComplEx", 32, n=1200, seed=13)
+    E = m.entity_embeddings.weight.detach().numpy().copy()
+    Rel = m.relation_embeddings.weight.detach().numpy().copy()
+    splits = {"train_set": triples[:800].astype(np.int16), "valid_set": triples[800:1000].astype(np.int16),
+              "test_set": triples[1000:].astype(np.int16)}
+    save_experiment(str(tmp_path), m, {f"e{i}": i for i in range(135)}, {f"r{i}": i for i in range(46)},
+                    extra_config={"batch_size": 128}, splits=splits)
+    report, ev = evaluate_experiment(str(tmp_path), eval_model="val_test")
+    assert set(report) == {"Val", "Test"} and ev.args.batch_size == 128
+    keys, row_ptr, col = ko.vocab_csr(triples, "er", 46)
+    np.testing.assert_array_equal(ev.csr.col.cpu().numpy(), col)
+    er = ko.vocab(triples, "er")
+    S = ko.k_vs_all_scores("ComplEx", E, Rel, triples[1000:, :2])
+    got = ev.last_ranks                                              # of the last split evaluated: Test
+    for j, (h, r, t) in enumerate(triples[1000:]):
+        lo, hi = ko.rank_interval_with_tolerance(S[j], int(t), er[(int(h), int(r))], 1e-5 * np.sqrt((S[j] ** 2).mean()))
+        assert lo <= got[j] <= hi
+    want = ko.metrics_from_ranks(got)
+    assert report["Test"]["MRR"] == pytest.approx(want["MRR"]) and report["Test"]["H@3"] == want["H@3"]

@@ -375,3 +375,64 @@ def test_csr_lookup_matches_host_search(ops, FilterCSR):
     assert (got < 0).any() and (got >= 0).any()
     empty = FilterCSR.from_triples(np.empty((0, 3), dtype=np.int64), R, device="cuda")
     assert (empty.rows_for(dev(torch.from_numpy(hr[:5]))).cpu().numpy() == -1).all()
+
+
+# ---------------------------------------------------------------------------------------------
+# vocabulary -> CSR on the GPU
+# ---------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("kind", ["er", "re", "ee"])
+@pytest.mark.parametrize("n,N,R", [(1, 5, 3), (700, 40, 7), (60000, 3000, 11), (300000, 200000, 1300)])
+def test_csr_build_matches_the_vocabulary_oracle(kind, n, N, R):
+    from dicee_amd.csr import FilterCSR
+    rng = np.random.default_rng(n + len(kind))
+    t = np.stack([rng.integers(0, N, n), rng.integers(0, R, n), rng.integers(0, N, n)], axis=1)
+    t[n // 2:] = t[:n - n // 2]                                          # half of the triples are duplicates
+    hub = rng.random(n) < 0.2
+    t[hub, 0], t[hub, 1] = 1 % N, 2 % R                                  # one long (h, r) row
+    csr = FilterCSR.from_triples_gpu(torch.from_numpy(t).cuda(), N, R, kind=kind)
+    rb = {"er": R, "re": N, "ee": N}[kind]
+    keys, row_ptr, col = ko.vocab_csr(t, kind, rb)
+    assert csr.keys.dtype == torch.int64 and csr.row_ptr.dtype == torch.int64 and csr.col.dtype == torch.int32
+    np.testing.assert_array_equal(csr.keys.cpu().numpy(), keys)
+    np.testing.assert_array_equal(csr.row_ptr.cpu().numpy(), row_ptr)
+    np.testing.assert_array_equal(csr.col.cpu().numpy(), col)
+    assert csr.num_rows == len(keys) and csr.nnz == len(col)
+    a, b, _ = {"er": (0, 1, 2), "re": (1, 2, 0), "ee": (0, 2, 1)}[kind]
+    rows = csr.rows_for(torch.from_numpy(np.ascontiguousarray(t[:50][:, [a, b]])).cuda()).cpu().numpy()
+    np.testing.assert_array_equal(keys[rows], t[:50, a] * rb + t[:50, b])
+
+
+def test_csr_build_edge_cases():
+    from dicee_amd import ops
+    from dicee_amd.csr import FilterCSR
+    empty = FilterCSR.from_triples_gpu(torch.empty((0, 3), dtype=torch.int64, device="cuda"), 10, 3)
+    assert empty.num_rows == 0 and empty.nnz == 0 and empty.row_ptr.tolist() == [0]
+    t = torch.tensor([[1, 0, 2], [9, 0, 2], [1, 3, 2], [1, 0, -1], [1, 0, 2], [0, 2, 9]], device="cuda")
+    keys, row_ptr, col, dropped = ops.csr_build(t, (0, 1, 2), (9, 3, 10))      # h = 9, r = 3 and t = -1 are out of range
+    assert dropped == 3 and keys.tolist() == [2, 3] and row_ptr.tolist() == [0, 1, 2] and col.tolist() == [9, 2]
+    with pytest.raises(ValueError):
+        FilterCSR.from_triples_gpu(t, 9, 3)
+    only_bad = torch.tensor([[50, 0, 0]], device="cuda")
+    keys, row_ptr, col, dropped = ops.csr_build(only_bad, (0, 1, 2), (9, 3, 10))
+    assert dropped == 1 and keys.numel() == 0 and row_ptr.tolist() == [0] and col.numel() == 0
+    with pytest.raises(TypeError):
+        ops.csr_build(t.int(), (0, 1, 2), (9, 3, 10))
+
+
+def test_csr_built_on_the_gpu_filters_like_the_host_built_one():
+    from dicee_amd import ops
+    from dicee_amd.csr import FilterCSR
+    rng = np.random.default_rng(77)
+    N, R, d, B, n = 5000, 9, 64, 300, 40000
+    E, Rel = random_tables(rng, N, R, d)
+    t = np.stack([rng.integers(0, 60, n), rng.integers(0, R, n), rng.integers(0, N, n)], axis=1)
+    host = FilterCSR.from_triples(t, R).to("cuda")
+    gpu = FilterCSR.from_triples_gpu(torch.from_numpy(t).cuda(), N, R)
+    hr = torch.from_numpy(np.ascontiguousarray(t[:B, :2])).cuda()
+    tgt = torch.from_numpy(np.ascontiguousarray(t[:B, 2])).cuda()
+    Eg, Rg = dev(E), dev(Rel)
+    Q, bias = ops.build_query("DistMult", Eg, Rg, hr)
+    a = ops.rank_filtered(Q, bias, Eg, None, tgt, host.rows_for(hr), host.row_ptr, host.col)
+    b = ops.rank_filtered(Q, bias, Eg, None, tgt, gpu.rows_for(hr), gpu.row_ptr, gpu.col)
+    for key in a:
+        assert torch.equal(a[key], b[key])

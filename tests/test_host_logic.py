@@ -55,6 +55,13 @@ def test_host_side_argument_validation_without_gpu(lib_path):
     rc = lib.kge_build_query(3, 1, 1, ctypes.c_void_p(256), 0, None, ctypes.c_void_p(256), 0, None, None, 1, None,
                              ctypes.c_void_p(256), 1, 7, 10, 2, ctypes.c_void_p(256), ctypes.c_void_p(256), None)
     assert rc == 1 and b"Keci" in lib.kge_last_error()
+    p256 = ctypes.c_void_p(256)
+    rc = lib.kge_csr_build(p256, 10, 0, 1, 1, 5, 5, 5, p256, p256, p256, p256, p256, 1 << 20, None)
+    assert rc == 1 and b"permutation" in lib.kge_last_error()
+    rc = lib.kge_csr_build(p256, 10, 0, 1, 2, 1 << 30, 1 << 20, 1 << 30, p256, p256, p256, p256, p256, 1 << 20, None)
+    assert rc == 2 and b"62-bit" in lib.kge_last_error()
+    rc = lib.kge_csr_build(p256, -1, 0, 1, 2, 5, 5, 5, p256, p256, p256, p256, p256, 1 << 20, None)
+    assert rc == 1
 
 
 def test_filter_csr_builders():
@@ -67,6 +74,10 @@ def test_filter_csr_builders():
     for h, r, t in triples:
         brute.setdefault((int(h), int(r)), set()).add(int(t))
     csr = FilterCSR.from_triples(triples, R)
+    keys, row_ptr, col = ko.vocab_csr(triples, "er", R)
+    np.testing.assert_array_equal(csr.keys_np, keys)
+    np.testing.assert_array_equal(csr.row_ptr_np, row_ptr)
+    np.testing.assert_array_equal(csr.col_np, col)
     assert csr.num_rows == len(brute) and csr.nnz == sum(len(v) for v in brute.values())
     for (h, r), tails in brute.items():
         np.testing.assert_array_equal(csr.tails(h, r), sorted(tails))

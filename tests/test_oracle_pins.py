@@ -383,3 +383,27 @@ def test_int8_rows_closed_form():
     assert np.all(q[3] == 0) and s[3] == 0.0
     err = np.abs(ko.dequantize_int8_rows(q, s) - x)
     assert np.all(err <= 0.5 * s[:, None] * (1 + 1e-6))
+
+
+def test_vocab_csr_against_a_hand_written_fixture_and_set_identities():
+    # 7 triples (h, r, t), one duplicate, one pair with three tails given out of order
+    triples = [(2, 1, 5), (0, 0, 3), (2, 1, 4), (2, 1, 5), (1, 0, 3), (2, 1, 0), (0, 1, 3)]
+    assert ko.vocab(triples, "er") == {(2, 1): [5, 4, 5, 0], (0, 0): [3], (1, 0): [3], (0, 1): [3]}
+    assert ko.vocab(triples, "re") == {(1, 5): [2, 2], (0, 3): [0, 1], (1, 4): [2], (1, 0): [2], (1, 3): [0]}
+    assert ko.vocab(triples, "ee") == {(2, 5): [1, 1], (0, 3): [0, 1], (2, 4): [1], (1, 3): [0], (2, 0): [1]}
+    keys, row_ptr, col = ko.vocab_csr(triples, "er", range_b=2)          # R = 2: key = 2h + r
+    assert keys.tolist() == [0, 1, 2, 5] and row_ptr.tolist() == [0, 1, 2, 3, 6] and col.tolist() == [3, 3, 3, 0, 4, 5]
+    keys, row_ptr, col = ko.vocab_csr(triples, "re", range_b=6)          # N = 6: key = 6r + t
+    assert keys.tolist() == [3, 6, 9, 10, 11] and row_ptr.tolist() == [0, 2, 3, 4, 5, 6]
+    assert col.tolist() == [0, 1, 2, 0, 2, 2]
+    # identities on random data: the rows partition the distinct triples
+    rng = np.random.default_rng(3)
+    t = np.stack([rng.integers(0, 9, 300), rng.integers(0, 4, 300), rng.integers(0, 9, 300)], axis=1)
+    for kind, rb, (a, b, v) in (("er", 4, (0, 1, 2)), ("re", 9, (1, 2, 0)), ("ee", 9, (0, 2, 1))):
+        keys, row_ptr, col = ko.vocab_csr(t, kind, rb)
+        assert np.all(np.diff(keys) > 0) and row_ptr[0] == 0 and row_ptr[-1] == len(col)
+        rebuilt = {(int(k) // rb, int(k) % rb, int(c)) for i, k in enumerate(keys) for c in col[row_ptr[i]:row_ptr[i + 1]]}
+        assert rebuilt == {(int(x[a]), int(x[b]), int(x[v])) for x in t}
+        assert len(col) == len(rebuilt)
+        for i in range(len(keys)):
+            assert np.all(np.diff(col[row_ptr[i]:row_ptr[i + 1]]) > 0)
