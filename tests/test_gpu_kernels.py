@@ -430,7 +430,7 @@ def test_csr_built_on_the_gpu_filters_like_the_host_built_one():
     gpu = FilterCSR.from_triples_gpu(torch.from_numpy(t).cuda(), N, R)
     hr = torch.from_numpy(np.ascontiguousarray(t[:B, :2])).cuda()
     tgt = torch.from_numpy(np.ascontiguousarray(t[:B, 2])).cuda()
-    Eg, Rg = dev(E), dev(Rel)
+    Eg, Rg = dev(torch.from_numpy(E)), dev(torch.from_numpy(Rel))
     Q, bias = ops.build_query("DistMult", Eg, Rg, hr)
     a = ops.rank_filtered(Q, bias, Eg, None, tgt, host.rows_for(hr), host.row_ptr, host.col)
     b = ops.rank_filtered(Q, bias, Eg, None, tgt, gpu.rows_for(hr), gpu.row_ptr, gpu.col)
