@@ -83,7 +83,7 @@ def main_loop_kernel(storage, d, mode):
     """Name of the contraction kernel the library picks for this table type and width."""
     epi = {"rank": "RankEpi", "topk": "TopkEpi", "bce": "BceEpi"}[mode]
     if storage == "fp32":
-        return f"kloop_kernel<{epi}>"
+        return f"kloop_async_kernel<{epi}>" if d % 4 == 0 else f"kloop_kernel<{epi}>"
     if d == 128:
         return f"qreg_async_kernel<{epi}>" if storage == "bf16" else f"qreg_i8_kernel<{epi}>"
     return f"qreg_kernel<{storage}, {epi}>"

@@ -1023,7 +1023,9 @@ __global__ void __launch_bounds__(256, 2) kloop_kernel(ContractArgs a, typename 
   int64_t et0 = r0;
   for (int it = 0; it < n_it; ++it) {
     const int buf = it & 1;
+#ifndef KGE_DBG_NO_GLOBAL
     if (it + 1 < n_it) chunk_load(it + 1);
+#endif
 #pragma unroll
     for (int kb = 0; kb < KLOOP_KC / 8; ++kb) {
       f32x4 fe[2], fq[2];
@@ -1041,7 +1043,9 @@ __global__ void __launch_bounds__(256, 2) kloop_kernel(ContractArgs a, typename 
             acc[te][tq] = Epi::SWAP ? mfma_f32(fq[tq][j], fe[te][j], acc[te][tq])
                                     : mfma_f32(fe[te][j], fq[tq][j], acc[te][tq]);
     }
+#ifndef KGE_DBG_NO_LDSWRITE
     if (it + 1 < n_it) chunk_store(buf ^ 1);
+#endif
     if (kc == nkc - 1) {  // this entity tile is complete
       float sc16[16];
 #pragma unroll
@@ -1063,6 +1067,155 @@ __global__ void __launch_bounds__(256, 2) kloop_kernel(ContractArgs a, typename 
     } else {
       ++kc;
       __syncthreads();
+    }
+  }
+  epi.finish();
+}
+
+// ============================================================================================
+// kloop_async_kernel: the fp32 path for rows that are 16-byte aligned (d % 4 == 0).  Same tiles, same
+// reduction order and same epilogues as kloop_kernel, but both operands of a K chunk go from global
+// memory straight into LDS (global_load_lds_dwordx4: no staging registers, no ds_write) while the
+// previous chunk is multiplied.
+//
+// LDS layout of a stage: 128 entity rows then 128 query rows, each 128 B = 8 pieces of 16 B; piece p
+// of row r sits in slot r*8 + (p ^ (r & 7)).  A direct-to-LDS load writes 64 consecutive slots per
+// wave, so the swizzle is applied on the global side (which piece a lane fetches); a fragment read
+// (ds_read_b128 of piece 2*kb + hf of rows c..c+7 at a time) then covers all 32 banks once.
+// ============================================================================================
+constexpr int KA_PART_BYTES = KLOOP_TILE_ROWS * KLOOP_KC * 4;  // 16 KB: one operand of one stage
+constexpr int KA_STAGE_BYTES = 2 * KA_PART_BYTES;
+
+template <template <int> class EpiT>
+__global__ void __launch_bounds__(256, 2) kloop_async_kernel(ContractArgs a, typename EpiT<KLOOP_NQT>::Args ea) {
+  using Epi = EpiT<KLOOP_NQT>;
+  static_assert(KLOOP_TILE_ROWS == 128 && KLOOP_WG_QUERIES == 128 && KLOOP_KC == 32, "stage layout");
+  __shared__ __attribute__((aligned(1024))) unsigned char lds[2 * KA_STAGE_BYTES];
+
+  int qg;
+  int64_t chunk;
+  if (!decompose_wg(a, qg, chunk)) return;
+  const int tid = threadIdx.x, lane = tid & 63, c = lane & 31, hf = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int we = wave >> 1, wq = wave & 1;
+  const int d = a.d;
+  const int64_t q_base = (int64_t)qg * KLOOP_WG_QUERIES;
+  const int64_t q0 = q_base + 64 * wq;
+  Epi epi;
+  epi.init(ea, q0, c, hf, a.B);
+  __shared__ typename Epi::Shared epi_sh;
+  epi.bind(&epi_sh);
+
+  const int64_t r0 = a.e_begin + chunk * a.chunk_rows;
+  const int64_t r1 = (r0 + a.chunk_rows < a.e_end) ? r0 + a.chunk_rows : a.e_end;
+  const int nkc = (d + KLOOP_KC - 1) / KLOOP_KC;
+  const int n_et = (int)((r1 - r0 + KLOOP_TILE_ROWS - 1) / KLOOP_TILE_ROWS);
+  const int n_it = n_et * nkc;
+  const float* Ef = (const float*)a.E;
+
+  // this lane's share of a stage: load instruction j covers rows lrow + 32 j of each operand, always the
+  // same swizzled piece (32 is a multiple of 8)
+  const int lrow = wave * 8 + (lane >> 3);
+  const int lk = ((lane & 7) ^ (lane >> 3)) * 4;  // float offset of the piece inside the K chunk
+  // query rows of this lane (fixed for the whole kernel); rows past B repeat the last query
+  const float* qsrc[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    int64_t q = q_base + lrow + 32 * j;
+    q = (q < a.B) ? q : a.B - 1;
+    qsrc[j] = a.Q + q * d + lk;
+  }
+  auto stage_issue = [&](int it, int buf) {
+    const int et = it / nkc, kc = it - et * nkc;
+    const int64_t et0 = r0 + (int64_t)et * KLOOP_TILE_ROWS;
+    const int k0 = kc * KLOOP_KC;
+    unsigned char* dst = lds + buf * KA_STAGE_BYTES + wave * 1024;
+    if (k0 + lk < d) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        int64_t g = et0 + lrow + 32 * j;
+        g = (g < r1) ? g : r1 - 1;  // padding rows repeat the last valid row; the epilogue ignores them
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(Ef + g * d + k0 + lk),
+                                         (__attribute__((address_space(3))) void*)(dst + j * 4096), 16, 0, 0);
+      }
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(qsrc[j] + k0),
+                                         (__attribute__((address_space(3))) void*)(dst + KA_PART_BYTES + j * 4096), 16,
+                                         0, 0);
+    } else {  // past the end of the rows (last chunk when d % 32 != 0): the piece is zero
+      const f32x4 z = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        *(f32x4*)(dst + j * 4096 + lane * 16) = z;
+        *(f32x4*)(dst + KA_PART_BYTES + j * 4096 + lane * 16) = z;
+      }
+    }
+  };
+
+  // fragment offsets of this lane inside an operand part (row c of tile 0)
+  int foff[KLOOP_KC / 8];
+#pragma unroll
+  for (int kb = 0; kb < KLOOP_KC / 8; ++kb) foff[kb] = c * 128 + (((2 * kb + hf) ^ (c & 7)) << 4);
+
+  f32x16 acc[2][2];
+#pragma unroll
+  for (int te = 0; te < 2; ++te)
+#pragma unroll
+    for (int tq = 0; tq < 2; ++tq)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc[te][tq][i] = 0.f;
+
+  if (n_it > 0) stage_issue(0, 0);
+  int kc = 0;
+  int64_t et0 = r0;
+  for (int it = 0; it < n_it; ++it) {
+    const int buf = it & 1;
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();  // stage `it` has landed for every wave; everyone is done reading the other buffer
+    if (Epi::STAGE_HOOK) epi.stage_end();
+#ifndef KGE_DBG_NO_GLOBAL
+    if (it + 1 < n_it) stage_issue(it + 1, buf ^ 1);
+#endif
+    const unsigned char* be = lds + buf * KA_STAGE_BYTES + (64 * we) * 128;
+    const unsigned char* bq = lds + buf * KA_STAGE_BYTES + KA_PART_BYTES + (64 * wq) * 128;
+    const int k_left = d - kc * KLOOP_KC;  // the last chunk of a row may hold fewer than 4 blocks of 8
+#pragma unroll
+    for (int kb = 0; kb < KLOOP_KC / 8; ++kb) {
+      if (kb * 8 >= k_left) break;  // blocks of zeros add nothing to any score
+      f32x4 fe[2], fq[2];
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+        fe[t] = *(const f32x4*)(be + t * 4096 + foff[kb]);
+        fq[t] = *(const f32x4*)(bq + t * 4096 + foff[kb]);
+      }
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int te = 0; te < 2; ++te)
+#pragma unroll
+          for (int tq = 0; tq < 2; ++tq)
+            acc[te][tq] = Epi::SWAP ? mfma_f32(fq[tq][j], fe[te][j], acc[te][tq])
+                                    : mfma_f32(fe[te][j], fq[tq][j], acc[te][tq]);
+    }
+    if (kc == nkc - 1) {  // this entity tile is complete
+      float sc16[16];
+#pragma unroll
+      for (int te = 0; te < 2; ++te) {
+        const int64_t e_base = et0 + 64 * we + 32 * te;
+        if (e_base < r1) {
+#pragma unroll
+          for (int tq = 0; tq < 2; ++tq) epi.template tile<false>(tq, acc[te][tq], sc16, 1.f, e_base, r1);
+        }
+#pragma unroll
+        for (int tq = 0; tq < 2; ++tq)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) acc[te][tq][i] = 0.f;
+      }
+      kc = 0;
+      et0 += KLOOP_TILE_ROWS;
+    } else {
+      ++kc;
     }
   }
   epi.finish();

@@ -685,7 +685,10 @@ int launch_contract(int dtype, const ContractArgs& a, const EArgs& ea, hipStream
     KGE_HIP_CHECK(hipEventCreate(&ev1));
     KGE_HIP_CHECK(hipEventRecord(ev0, st));
   }
-  if (dtype == KGE_F32)
+  const bool rows_aligned = (a.d % 4 == 0) && (((uintptr_t)a.E | (uintptr_t)a.Q) % 16 == 0);
+  if (dtype == KGE_F32 && rows_aligned)
+    hipLaunchKernelGGL((kloop_async_kernel<EpiT>), grid, block, 0, st, a, ea);
+  else if (dtype == KGE_F32)
     hipLaunchKernelGGL((kloop_kernel<EpiT>), grid, block, 0, st, a, ea);
   else if (dtype == KGE_BF16 && a.d == 128)
     hipLaunchKernelGGL((qreg_async_kernel<EpiT>), grid, block, 0, st, a, ea);
