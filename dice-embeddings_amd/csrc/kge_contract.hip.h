@@ -793,11 +793,20 @@ __global__ void __launch_bounds__(64 * QA_WG_WAVES, QA_WAVES_PER_SIMD) qreg_asyn
 // share of the next stage in registers while the current stage is consumed, then converts and
 // stores it.  The fp32 row scales of a stage ride along in LDS.
 // ============================================================================================
+#ifndef KGE_I8_WG_WAVES
+#define KGE_I8_WG_WAVES 8
+#endif
+constexpr int I8_WG_WAVES = KGE_I8_WG_WAVES;
+constexpr int I8_WG_QUERIES = I8_WG_WAVES * 32 * QREG_NQT;
+constexpr int I8_WGS_PER_CU = 8 / I8_WG_WAVES;  // 2 waves per SIMD
+
 template <template <int> class EpiT>
-__global__ void __launch_bounds__(256, 2) qreg_i8_kernel(ContractArgs a, typename EpiT<QREG_NQT>::Args ea) {
+__global__ void __launch_bounds__(64 * I8_WG_WAVES, 2) qreg_i8_kernel(ContractArgs a, typename EpiT<QREG_NQT>::Args ea) {
   using Epi = EpiT<QREG_NQT>;
   __shared__ __attribute__((aligned(1024))) unsigned char lds_e[2 * QA_BUF_BYTES];
   __shared__ __attribute__((aligned(16))) float lds_sc[2][QA_STAGE_ROWS];
+  constexpr int NT = 64 * I8_WG_WAVES;
+  constexpr int NPIECE = QA_STAGE_ROWS * 8 / NT;  // 16-byte pieces of int8 a thread stages per stage
 
   const int64_t wg = blockIdx.x;
   const int xcd = (int)(wg & 7);
@@ -807,7 +816,7 @@ __global__ void __launch_bounds__(256, 2) qreg_i8_kernel(ContractArgs a, typenam
   const int tid = threadIdx.x, lane = tid & 63, c = lane & 31, hf = lane >> 5;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   constexpr int d = 128;
-  const int64_t q0 = (int64_t)qg * QREG_WG_QUERIES + wave * (32 * QREG_NQT);
+  const int64_t q0 = (int64_t)qg * I8_WG_QUERIES + wave * (32 * QREG_NQT);
 
   const int64_t c_first = xcd + 8 * (int64_t)wlane;
   const int64_t c_stride = 8 * (int64_t)a.n_lanes;
@@ -842,14 +851,14 @@ __global__ void __launch_bounds__(256, 2) qreg_i8_kernel(ContractArgs a, typenam
   __shared__ typename Epi::Shared epi_sh;
   epi.bind(&epi_sh);
 
-  // staging: 128 rows x 128 B = 1024 pieces of 16 int8; thread handles pieces tid + 256 j
-  u32x4 stage[4];
+  // staging: 128 rows x 128 B = 1024 pieces of 16 int8; thread handles pieces tid + NT j
+  u32x4 stage[NPIECE];
   float stage_sc = 0.f;
   const int8_t* Eb = (const int8_t*)a.E;
   auto stage_load = [&](int64_t row0) {
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int idx = tid + 256 * j, row = idx >> 3, piece = idx & 7;
+    for (int j = 0; j < NPIECE; ++j) {
+      const int idx = tid + NT * j, row = idx >> 3, piece = idx & 7;
       int64_t g = row0 + row;
       g = (g < r_end) ? g : r_end - 1;  // padding rows repeat the last valid row; epilogues ignore them
       stage[j] = *(const u32x4*)(Eb + g * d + piece * 16);
@@ -863,8 +872,8 @@ __global__ void __launch_bounds__(256, 2) qreg_i8_kernel(ContractArgs a, typenam
   auto stage_store = [&](int buf) {
     unsigned char* base = lds_e + buf * QA_BUF_BYTES;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int idx = tid + 256 * j, row = idx >> 3, piece = idx & 7;
+    for (int j = 0; j < NPIECE; ++j) {
+      const int idx = tid + NT * j, row = idx >> 3, piece = idx & 7;
       const int p0 = 2 * piece, sw = row & 15;
       *(u32x4*)(base + row * 256 + ((p0 ^ sw) << 4)) = i8x8_to_bf16x8(stage[j][0], stage[j][1]);
       *(u32x4*)(base + row * 256 + (((p0 + 1) ^ sw) << 4)) = i8x8_to_bf16x8(stage[j][2], stage[j][3]);
@@ -877,6 +886,11 @@ __global__ void __launch_bounds__(256, 2) qreg_i8_kernel(ContractArgs a, typenam
   for (int s = 0; s < 8; ++s) foff[s] = c * 256 + (((2 * s + hf) ^ (c & 15)) << 4);
 
   constexpr int ET = QA_STAGE_ROWS / 32;
+  // A tile's epilogue runs right after its MFMA chain (deferring it under the next chain, as the bf16
+  // path does, does not fit the register budget next to the row scales).
+  float sc16[16] = {};
+  float sc_col = 1.f;
+
   int64_t row_next = stage_row(0);
   stage_load(row_next);
   stage_store(0);
@@ -899,20 +913,6 @@ __global__ void __launch_bounds__(256, 2) qreg_i8_kernel(ContractArgs a, typenam
       bf16x8 ef[8];
 #pragma unroll
       for (int s = 0; s < 8; ++s) ef[s] = *(const bf16x8*)(base + et * 8192 + foff[s]);
-      float sc16[16];
-      float sc_col = 1.f;
-      if (Epi::SWAP) {
-        sc_col = lds_sc[buf][et * 32 + c];
-      } else {
-#pragma unroll
-        for (int g = 0; g < 4; ++g) {
-          const f32x4 v = *(const f32x4*)&lds_sc[buf][et * 32 + 8 * g + 4 * hf];
-          sc16[4 * g] = v[0];
-          sc16[4 * g + 1] = v[1];
-          sc16[4 * g + 2] = v[2];
-          sc16[4 * g + 3] = v[3];
-        }
-      }
 #pragma unroll
       for (int t = 0; t < QREG_NQT; ++t) {
         f32x16 acc;
@@ -921,6 +921,20 @@ __global__ void __launch_bounds__(256, 2) qreg_i8_kernel(ContractArgs a, typenam
 #pragma unroll
         for (int s = 0; s < 8; ++s)
           acc = Epi::SWAP ? mfma_bf16(qf[t][s], ef[s], acc) : mfma_bf16(ef[s], qf[t][s], acc);
+        if (t == 0) {  // row scales of this entity tile: fetched under the first chain
+          if (Epi::SWAP) {
+            sc_col = lds_sc[buf][et * 32 + c];
+          } else {
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+              const f32x4 v = *(const f32x4*)&lds_sc[buf][et * 32 + 8 * g + 4 * hf];
+              sc16[4 * g] = v[0];
+              sc16[4 * g + 1] = v[1];
+              sc16[4 * g + 2] = v[2];
+              sc16[4 * g + 3] = v[3];
+            }
+          }
+        }
         epi.template tile<true>(t, acc, sc16, sc_col, row0 + et * 32, r_end);
       }
     }

@@ -623,7 +623,7 @@ ContractArgs make_args(const float* Q, const void* E, int dtype, const float* sc
   a.e_end = e_end;
   a.d = (int)d;
   const bool fast_bf16 = (dtype == KGE_BF16 && d == 128), fast_i8 = (dtype == KGE_I8 && d == 128);
-  const int wgq = (dtype == KGE_F32) ? KLOOP_WG_QUERIES : fast_bf16 ? QA_WG_QUERIES : QREG_WG_QUERIES;
+  const int wgq = (dtype == KGE_F32) ? KLOOP_WG_QUERIES : fast_bf16 ? QA_WG_QUERIES : fast_i8 ? I8_WG_QUERIES : QREG_WG_QUERIES;
   a.n_qgroups = (int)((B + wgq - 1) / wgq);
   if (a.n_qgroups < 1) a.n_qgroups = 1;
   const int64_t rows = e_end - e_begin;
@@ -631,7 +631,7 @@ ContractArgs make_args(const float* Q, const void* E, int dtype, const float* sc
   if (fast_bf16 || fast_i8) {
     // persistent paths: the workgroups resident on one XCD (32 CUs x workgroups per CU) are shared out
     // among the query groups
-    a.n_lanes = 32 * (fast_bf16 ? QA_WGS_PER_CU : 2) / a.n_qgroups;
+    a.n_lanes = 32 * (fast_bf16 ? QA_WGS_PER_CU : I8_WGS_PER_CU) / a.n_qgroups;
     if (a.n_lanes < 1) a.n_lanes = 1;
     int64_t chunk = rows / (8 * (int64_t)a.n_lanes * 4);  // aim for >= 4 chunks per workgroup
     chunk = (chunk + QA_STAGE_ROWS - 1) / QA_STAGE_ROWS * QA_STAGE_ROWS;
@@ -673,7 +673,7 @@ int launch_contract(int dtype, const ContractArgs& a, const EArgs& ea, hipStream
   const bool persistent = (dtype == KGE_BF16 && a.d == 128) || fast_i8;
   const int64_t nwg = persistent ? 8 * (int64_t)a.n_qgroups * a.n_lanes : (a.n_chunks + 7) / 8 * 8 * a.n_qgroups;
   KGE_REQUIRE(nwg <= 0x7fffffffLL, KGE_ERR_INVALID, "%s: grid of %lld workgroups too large", name, (long long)nwg);
-  dim3 grid((unsigned)nwg), block((persistent && !fast_i8) ? 64 * QA_WG_WAVES : 256);
+  dim3 grid((unsigned)nwg), block(fast_i8 ? 64 * I8_WG_WAVES : persistent ? 64 * QA_WG_WAVES : 256);
   hipEvent_t ev0 = nullptr, ev1 = nullptr;
   bool timed = false;
   {
