@@ -441,7 +441,13 @@ __global__ void topk_init_kernel(TopkWs w, int64_t B) {
 // Merge a query's kept list with this round's candidates, keep the best k, publish the new
 // threshold.  In `rescan` mode (only queries flagged dirty) list entries above the old threshold
 // are dropped first: the rescan finds all of them again.
-__global__ void __launch_bounds__(256) topk_select_kernel(TopkWs w, int k, int rescan) {
+// Two launches cover a round: one wave per query (NT = 64, SELECT_SMALL keys of LDS, many queries
+// resident per CU) for the queries with at most SELECT_SMALL entries to rank, which is nearly all
+// of them, then four waves per query with room for a full candidate buffer for the rest.  A query
+// ranked by the first launch has its candidate count reset, so the second one skips it.
+constexpr int SELECT_SMALL = 1024;
+template <int NT>
+__global__ void __launch_bounds__(NT) topk_select_kernel(TopkWs w, int k, int rescan) {
   extern __shared__ unsigned long long keys[];
   __shared__ int s_valid;
   const int tid = threadIdx.x;
@@ -453,10 +459,11 @@ __global__ void __launch_bounds__(256) topk_select_kernel(TopkWs w, int k, int r
   const bool over = raw > TOPK_CAP;
   const float tau_old = w.tau[b];
   const int n = len + nc;
+  if ((NT == 64) != (n <= SELECT_SMALL)) return;
   int npad = 2;
   while (npad < n) npad <<= 1;
   if (tid == 0) s_valid = 0;
-  for (int i = tid; i < npad; i += 256) {
+  for (int i = tid; i < npad; i += NT) {
     unsigned long long key = 0;
     if (i < len) {
       key = w.list[b * w.kpad + i];
@@ -469,7 +476,7 @@ __global__ void __launch_bounds__(256) topk_select_kernel(TopkWs w, int k, int r
   __syncthreads();
   for (int kk = 2; kk <= npad; kk <<= 1) {
     for (int j = kk >> 1; j > 0; j >>= 1) {
-      for (int i = tid; i < npad; i += 256) {
+      for (int i = tid; i < npad; i += NT) {
         const int ixj = i ^ j;
         if (ixj > i) {
           const bool down = (i & kk) == 0;
@@ -483,12 +490,12 @@ __global__ void __launch_bounds__(256) topk_select_kernel(TopkWs w, int k, int r
       __syncthreads();
     }
   }
-  for (int i = tid; i < npad; i += 256)
+  for (int i = tid; i < npad; i += NT)
     if (keys[i] != 0 && (i + 1 == npad || keys[i + 1] == 0)) s_valid = i + 1;
   __syncthreads();
   const int n_valid = s_valid;
   const int new_len = n_valid < k ? n_valid : k;
-  for (int i = tid; i < new_len; i += 256) w.list[b * w.kpad + i] = keys[i];
+  for (int i = tid; i < new_len; i += NT) w.list[b * w.kpad + i] = keys[i];
   if (tid == 0) {
     w.list_len[b] = new_len;
     w.tau[b] = (new_len == k) ? ordered_to_f32((uint32_t)(keys[k - 1] >> 32)) : __uint_as_float(0xff800000u);
@@ -891,7 +898,14 @@ extern "C" int kge_topk(const float* Q, const float* bias, const void* E, int dt
   hipLaunchKernelGGL(topk_init_kernel, dim3((unsigned)((B + 255) / 256)), dim3(256), 0, st, ws, B);
   KGE_LAUNCH_CHECK("topk_init_kernel");
 
-  const size_t sel_lds = 8192 * sizeof(unsigned long long);  // kpad (<= 1024) + TOPK_CAP, padded to a power of two
+  // ranks the list (<= k entries) and this round's candidates (<= min(TOPK_CAP, rows scanned) entries) of every query
+  auto launch_select = [&](int64_t rows, int rescan) {
+    hipLaunchKernelGGL(topk_select_kernel<64>, dim3((unsigned)B), dim3(64), SELECT_SMALL * sizeof(unsigned long long), st,
+                       ws, (int)k, rescan);
+    if (k + (rows < TOPK_CAP ? rows : TOPK_CAP) > SELECT_SMALL)  // kpad (<= 1024) + TOPK_CAP, padded to a power of two
+      hipLaunchKernelGGL(topk_select_kernel<256>, dim3((unsigned)B), dim3(256), 8192 * sizeof(unsigned long long), st,
+                         ws, (int)k, rescan);
+  };
   const int64_t growth = (k <= 256) ? 4 : 2;  // round r scans (growth - 1) x what is already ranked
   int64_t e0 = 0, e1 = (N < TOPK_FIRST_ROWS) ? N : TOPK_FIRST_ROWS;
   while (e0 < N) {
@@ -899,7 +913,7 @@ extern "C" int kge_topk(const float* Q, const float* bias, const void* E, int dt
     TopkArgs ea{ws.tau, nullptr, ws.cnt, ws.cand, TOPK_CAP};
     rc = launch_contract<TopkEpi>(dtype, a, ea, st, "kge_topk scan");
     if (rc) return rc;
-    hipLaunchKernelGGL(topk_select_kernel, dim3((unsigned)B), dim3(256), sel_lds, st, ws, (int)k, 0);
+    launch_select(e1 - e0, 0);
     KGE_LAUNCH_CHECK("topk_select_kernel");
     e0 = e1;
     int64_t next = e1 * growth;
@@ -915,7 +929,7 @@ extern "C" int kge_topk(const float* Q, const float* bias, const void* E, int dt
     TopkArgs ea{ws.tau, ws.dirty, ws.cnt, ws.cand, TOPK_CAP};
     rc = launch_contract<TopkEpi>(dtype, a, ea, st, "kge_topk rescan");
     if (rc) return rc;
-    hipLaunchKernelGGL(topk_select_kernel, dim3((unsigned)B), dim3(256), sel_lds, st, ws, (int)k, 1);
+    launch_select(N, 1);
     KGE_LAUNCH_CHECK("topk_select_kernel");
     KGE_HIP_CHECK(hipMemcpyAsync(&n_dirty, ws.n_dirty, sizeof(int32_t), hipMemcpyDeviceToHost, st));
     KGE_HIP_CHECK(hipStreamSynchronize(st));
