@@ -1,6 +1,11 @@
 // Gather of head / relation rows fused with the model interaction -> one query vector per pair.
 // One wavefront per (head, relation) pair; both rows are staged in LDS as fp32, normalised
 // there if requested, and combined into Q[b, :] (and the per-row scalar bias of Keci).
+//
+// Head direction (pairs are (relation, tail), the unknown is the head): every model's triple score
+// is linear in the head row, score(x, r, t) = Q'(r, t) . E[x].  DistMult: r * t.  ComplEx:
+// conj(r) * t as complex numbers.  QMult: t (x) conj(r^) as quaternions.  Keci: the coefficient of
+// each head component, including those of the sigma sums (which hold h and r but not t).
 #include "kge_internal.h"
 
 namespace kge {
@@ -18,6 +23,7 @@ struct QueryArgs {
   kge_norm_params norm;
   int64_t B, N, R;
   int d, p, q, normalize_relation;
+  int head_mode;  // pairs are (relation, tail) and Q is the head-direction query
 };
 
 template <int DT>
@@ -62,7 +68,8 @@ __global__ void __launch_bounds__(64) build_query_kernel(QueryArgs a, int model)
   float* sr = lds + d;
   const int lane = threadIdx.x;
   const int64_t b = blockIdx.x;
-  const int64_t h_id = a.hr[2 * b], r_id = a.hr[2 * b + 1];
+  // the entity row of the pair (head, or tail in head mode) goes to sh, the relation row to sr
+  const int64_t h_id = a.hr[2 * b + (a.head_mode ? 1 : 0)], r_id = a.hr[2 * b + (a.head_mode ? 0 : 1)];
   float* q = a.Q + b * d;
   if (h_id < 0 || h_id >= a.N || r_id < 0 || r_id >= a.R) {
     const float nan = __uint_as_float(0x7fc00000u);
@@ -85,8 +92,9 @@ __global__ void __launch_bounds__(64) build_query_kernel(QueryArgs a, int model)
     for (int k = lane; k < d; k += 64) q[k] = sh[k] * sr[k];
   } else if (model == KGE_COMPLEX) {
     const int d2 = d >> 1;
+    const float conj = a.head_mode ? -1.f : 1.f;
     for (int k = lane; k < d2; k += 64) {
-      float hr_ = sh[k], hi_ = sh[k + d2], rr_ = sr[k], ri_ = sr[k + d2];
+      float hr_ = sh[k], hi_ = sh[k + d2], rr_ = sr[k], ri_ = conj * sr[k + d2];
       q[k] = hr_ * rr_ - hi_ * ri_;
       q[k + d2] = hr_ * ri_ + hi_ * rr_;
     }
@@ -105,13 +113,55 @@ __global__ void __launch_bounds__(64) build_query_kernel(QueryArgs a, int model)
       __syncthreads();
     }
     const int d4 = d >> 2;
+    const float conj = a.head_mode ? -1.f : 1.f;
     for (int g = lane; g < d4; g += 64) {
       float ah = sh[g], bh = sh[g + d4], ch = sh[g + 2 * d4], dh = sh[g + 3 * d4];
-      float ar = sr[g], br = sr[g + d4], cr = sr[g + 2 * d4], dr = sr[g + 3 * d4];
+      float ar = sr[g], br = conj * sr[g + d4], cr = conj * sr[g + 2 * d4], dr = conj * sr[g + 3 * d4];
       q[g] = ah * ar - bh * br - ch * cr - dh * dr;
       q[g + d4] = ah * br + bh * ar + ch * dr - dh * cr;
       q[g + 2 * d4] = ah * cr - bh * dr + ch * ar + dh * br;
       q[g + 3 * d4] = ah * dr + bh * cr - ch * br + dh * ar;
+    }
+  } else if (a.head_mode) {  // KGE_KECI, head direction: sh holds the tail row (its parts are not scaled)
+    const int p = a.p, qn = a.q;
+    const int r = d / (p + qn + 1);
+    const int qoff = r + r * p;
+    for (int k = lane; k < r * p; k += 64) sr[r + k] *= a.coeff_p[k % p];
+    for (int k = lane; k < r * qn; k += 64) sr[qoff + k] *= a.coeff_q[k % qn];
+    __syncthreads();
+    for (int rho = lane; rho < r; rho += 64) {
+      const float t0 = sh[rho], r0 = sr[rho];
+      const float* tp = sh + r + rho * p;
+      const float* rp = sr + r + rho * p;
+      const float* tq = sh + qoff + rho * qn;
+      const float* rq = sr + qoff + rho * qn;
+      float q0 = r0 * t0, sum_rp = 0.f, sum_rq = 0.f;
+      for (int i = 0; i < p; ++i) {
+        q0 += rp[i] * tp[i];
+        sum_rp += rp[i];
+      }
+      for (int j = 0; j < qn; ++j) {
+        q0 += rq[j] * tq[j];
+        sum_rq += rq[j];
+      }
+      q[rho] = q0;
+      const bool pq = p >= 2 && qn >= 2;
+      float before = 0.f;  // sum of rp[k], k < i
+      for (int i = 0; i < p; ++i) {
+        float v = rp[i] * t0 + r0 * tp[i];
+        if (p >= 2) v += (sum_rp - before - rp[i]) - before;  // d sigma_pp / d hp_i
+        if (pq) v += sum_rq;                                   // d sigma_pq / d hp_i
+        q[r + rho * p + i] = v * a.coeff_p[i];                 // the head's own part is scaled too
+        before += rp[i];
+      }
+      before = 0.f;
+      for (int j = 0; j < qn; ++j) {
+        float v = -rq[j] * t0 + r0 * tq[j];
+        if (qn >= 2) v += (sum_rq - before - rq[j]) - before;  // d sigma_qq / d hq_j
+        if (pq) v -= sum_rp;                                   // d sigma_pq / d hq_j
+        q[qoff + rho * qn + j] = v * a.coeff_q[j];
+        before += rq[j];
+      }
     }
   } else {  // KGE_KECI
     const int p = a.p, qn = a.q;
@@ -175,12 +225,15 @@ int launch_build_query(const QueryArgs& a, int model, int rel_dtype, hipStream_t
 }  // namespace
 }  // namespace kge
 
-extern "C" int kge_build_query(int model, int p, int q, const void* ent, int ent_dtype, const float* ent_scale,
-                               const void* rel, int rel_dtype, const float* coeff_p, const float* coeff_q,
-                               int normalize_relation, const kge_norm_params* norm, const int64_t* hr,
-                               int64_t B, int64_t d, int64_t N, int64_t R, float* Q, float* bias, void* stream) {
+static int build_query_impl(int head_mode, int model, int p, int q, const void* ent, int ent_dtype,
+                            const float* ent_scale, const void* rel, int rel_dtype, const float* coeff_p,
+                            const float* coeff_q, int normalize_relation, const kge_norm_params* norm,
+                            const int64_t* hr, int64_t B, int64_t d, int64_t N, int64_t R, float* Q, float* bias,
+                            void* stream) {
   using namespace kge;
   clear_error();
+  KGE_REQUIRE(!head_mode || !norm || norm->kind == KGE_NORM_NONE, KGE_ERR_UNSUPPORTED,
+              "kge_build_query_head: a normalised head row is not a row of the table; only normalisation 'none'");
   KGE_REQUIRE(B >= 0 && N > 0 && R > 0, KGE_ERR_INVALID, "kge_build_query: B=%lld N=%lld R=%lld", (long long)B,
               (long long)N, (long long)R);
   if (B == 0) return KGE_OK;
@@ -234,8 +287,25 @@ extern "C" int kge_build_query(int model, int p, int q, const void* ent, int ent
   a.p = p;
   a.q = q;
   a.normalize_relation = normalize_relation;
+  a.head_mode = head_mode;
   hipStream_t st = (hipStream_t)stream;
   if (ent_dtype == KGE_F32) return launch_build_query<KGE_F32>(a, model, rel_dtype, st);
   if (ent_dtype == KGE_BF16) return launch_build_query<KGE_BF16>(a, model, rel_dtype, st);
   return launch_build_query<KGE_I8>(a, model, rel_dtype, st);
+}
+
+extern "C" int kge_build_query(int model, int p, int q, const void* ent, int ent_dtype, const float* ent_scale,
+                               const void* rel, int rel_dtype, const float* coeff_p, const float* coeff_q,
+                               int normalize_relation, const kge_norm_params* norm, const int64_t* hr,
+                               int64_t B, int64_t d, int64_t N, int64_t R, float* Q, float* bias, void* stream) {
+  return build_query_impl(0, model, p, q, ent, ent_dtype, ent_scale, rel, rel_dtype, coeff_p, coeff_q,
+                          normalize_relation, norm, hr, B, d, N, R, Q, bias, stream);
+}
+
+extern "C" int kge_build_query_head(int model, int p, int q, const void* ent, int ent_dtype, const float* ent_scale,
+                                    const void* rel, int rel_dtype, const float* coeff_p, const float* coeff_q,
+                                    int normalize_relation, const kge_norm_params* norm, const int64_t* rt,
+                                    int64_t B, int64_t d, int64_t N, int64_t R, float* Q, float* bias, void* stream) {
+  return build_query_impl(1, model, p, q, ent, ent_dtype, ent_scale, rel, rel_dtype, coeff_p, coeff_q,
+                          normalize_relation, norm, rt, B, d, N, R, Q, bias, stream);
 }

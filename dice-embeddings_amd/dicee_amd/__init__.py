@@ -7,6 +7,7 @@ this package is the thin Python side that mirrors the reference's call surface:
 * ``models``     ``DistMult/ComplEx/QMult/Keci/CKeci`` with ``forward``, ``forward_k_vs_all``,
                  ``k_vs_all_score`` (dicee/models/*.py)
 * ``evaluator``  ``Evaluator.evaluate_lp_k_vs_all`` (dicee/evaluation/evaluator.py:394-510)
+* ``link_prediction``  ``evaluate_lp``: head and tail direction (dicee/evaluation/link_prediction.py:351-473)
 * ``kge``        ``KGE.predict_topk`` / ``predict`` / ``predict_missing_tail_entity``
                  (dicee/knowledge_graph_embeddings.py:314-579)
 * ``csr``        the known-answer filter as a CSR (dicee's ``er_vocab``)
@@ -22,6 +23,7 @@ from .csr import FilterCSR  # noqa: F401
 from .models import DistMult, ComplEx, QMult, Keci, CKeci, MODEL_REGISTRY, initialize_model  # noqa: F401
 from .evaluator import Evaluator, compute_metrics_from_ranks_simple  # noqa: F401
 from .kge import KGE  # noqa: F401
+from .link_prediction import evaluate_lp  # noqa: F401
 from .loader import load_model, load_splits, evaluate_experiment, save_experiment  # noqa: F401
 
 __version__ = "0.1.0"

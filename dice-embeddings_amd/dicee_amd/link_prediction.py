@@ -1,0 +1,73 @@
+"""Filtered link prediction in both directions through the fused rank kernel.
+
+Mirrors ``evaluate_lp`` (dicee/evaluation/link_prediction.py:351-473), the evaluation dicee runs for
+models trained with negative sampling: for every test triple the true tail is ranked among
+``score(h, r, x)`` and the true head among ``score(x, r, t)`` over all entities x, known answers
+filtered out (``er_vocab`` for tails, ``re_vocab`` for heads), and the hit rates and the MRR are
+averaged over both directions.  The reference scores ``chunk_size`` entities at a time with
+``batch * chunk`` per-triple forward passes and sorts every row; here each direction of a batch is
+one query build plus one fused rank call (the head direction is the same table contraction as the
+tail direction, with the query vector ``Q'(r, t)``).
+"""
+import numpy as np
+import torch
+
+from .csr import FilterCSR
+from .evaluator import ranks_from_counts
+
+
+def _as_csr(vocab, key_mult, device):
+    if vocab is None or isinstance(vocab, FilterCSR):
+        csr = vocab
+    else:
+        csr = FilterCSR.from_er_vocab(vocab, key_mult)           # dict (a, b) -> list of values
+    if csr is not None:
+        csr.to(device)
+    return csr
+
+
+@torch.no_grad()
+def evaluate_lp(model, triple_idx, num_entities=None, er_vocab=None, re_vocab=None, info="Eval Starts",
+                batch_size=128, chunk_size=1000, tie="stable", return_ranks=False):
+    """``{'H@1', 'H@3', 'H@10', 'MRR'}`` over head and tail prediction.
+
+    ``er_vocab`` / ``re_vocab``: the reference's dicts ``(h, r) -> [t]`` / ``(r, t) -> [h]``, or ``FilterCSR``
+    objects (``FilterCSR.from_triples_gpu(..., kind="er" | "re")``).  ``chunk_size`` is accepted for
+    signature compatibility; nothing is chunked.  ``return_ranks``: also return (head_ranks, tail_ranks)."""
+    assert model is not None, "Model must be provided"
+    assert triple_idx is not None, "triple_idx must be provided"
+    assert er_vocab is not None, "er_vocab must be provided"
+    assert re_vocab is not None, "re_vocab must be provided"
+    model.eval()
+    N, R = model.num_entities, model.num_relations
+    assert num_entities is None or num_entities == N, "num_entities does not match the model"
+    triple_idx = np.asarray(triple_idx)
+    if triple_idx.ndim != 2 or triple_idx.shape[1] != 3:
+        raise ValueError("triple_idx must have shape [n, 3]")
+    n = len(triple_idx)
+    if n and (triple_idx[:, [0, 2]].min() < 0 or triple_idx[:, [0, 2]].max() >= N or triple_idx[:, 1].min() < 0
+              or triple_idx[:, 1].max() >= R):
+        raise IndexError("triple_idx holds an entity or relation id outside the model's tables")
+    if info:
+        print(info)
+        print(f"Num of triples {n}")
+    dev = model.entity_embeddings.weight.device
+    er = _as_csr(er_vocab, R, dev)
+    re = _as_csr(re_vocab, N, dev)
+    trip = torch.from_numpy(np.ascontiguousarray(triple_idx.astype(np.int64))).to(dev)
+    tail_ranks = torch.empty((n,), dtype=torch.int64, device=dev)
+    head_ranks = torch.empty((n,), dtype=torch.int64, device=dev)
+    bs = int(batch_size)
+    for i in range(0, n, bs):
+        b = trip[i:i + bs]
+        c = model.rank_filtered(b[:, :2].contiguous(), b[:, 2].contiguous(), er)
+        tail_ranks[i:i + bs] = ranks_from_counts(c["n_greater"], c["n_equal"], c["n_equal_lower"], tie)
+        c = model.rank_filtered(b[:, 1:].contiguous(), b[:, 0].contiguous(), re, heads=True)
+        head_ranks[i:i + bs] = ranks_from_counts(c["n_greater"], c["n_equal"], c["n_equal_lower"], tie)
+    hr_, tr_ = head_ranks.cpu().numpy(), tail_ranks.cpu().numpy()
+    divisor = float(2 * n) if n else 1.0
+    results = {f"H@{k}": float((np.count_nonzero(hr_ <= k) + np.count_nonzero(tr_ <= k)) / divisor) for k in (1, 3, 10)}
+    results["MRR"] = float((1.0 / hr_ + 1.0 / tr_).sum() / divisor)
+    if info:
+        print(results)
+    return (results, (hr_, tr_)) if return_ranks else results

@@ -103,13 +103,15 @@ class BaseKGE(torch.nn.Module):
     def _query_kwargs(self):
         return {}
 
-    def query(self, x):
+    def query(self, x, heads=False):
         """(Q [B,d], bias [B]) for ``x`` [B,2]: gather + interaction
-        (get_head_relation_representation, base_model.py:377-384, then the model's elementwise part)."""
+        (get_head_relation_representation, base_model.py:377-384, then the model's elementwise part).
+        ``heads=True``: ``x`` holds (relation, tail) pairs and ``Q @ E^T`` scores every entity as the head of
+        (x, r, t): what ``forward_triples`` gives triple by triple (base_model.py:346-362)."""
         E, scale = self.table()
         x = x.to(device=E.device, dtype=torch.int64).contiguous()
         return ops.build_query(self.name if self.name != "CKeci" else "Keci", E, self._rel(), x, ent_scale=scale,
-                               norm=self._norm_params(), **self._query_kwargs())
+                               norm=self._norm_params(), head=heads, **self._query_kwargs())
 
     # ------------------------------------------------------------------ reference call surface
     def forward(self, x, y_idx=None):
@@ -128,6 +130,12 @@ class BaseKGE(torch.nn.Module):
         E, scale = self.table()
         return ops.scores(Q, bias, E, scale)
 
+    def forward_all_heads(self, rt):
+        """[B,N] fp32: score(x, r, t) of every entity x as head, for ``rt`` [B,2] = (relation, tail) pairs."""
+        Q, bias = self.query(rt, heads=True)
+        E, scale = self.table()
+        return ops.scores(Q, bias, E, scale)
+
     def k_vs_all_score(self, emb_h, emb_r, emb_E):
         """Scores from already gathered rows: [B,d],[B,d],[N,d] -> [B,N]."""
         B = emb_h.shape[0]
@@ -138,9 +146,11 @@ class BaseKGE(torch.nn.Module):
         return ops.scores(Q, bias, emb_E.contiguous().float())
 
     # ------------------------------------------------------------------ fused consumers
-    def rank_filtered(self, x, target, csr=None):
-        """Fused filtered-rank counters for queries ``x`` [B,2] and true tails ``target`` [B]."""
-        Q, bias = self.query(x)
+    def rank_filtered(self, x, target, csr=None, heads=False):
+        """Fused filtered-rank counters for queries ``x`` [B,2] and true tails ``target`` [B].
+        ``heads=True``: ``x`` = (relation, tail) pairs, ``target`` the true heads, ``csr`` the (r, t) -> heads
+        vocabulary."""
+        Q, bias = self.query(x, heads=heads)
         E, scale = self.table()
         target = target.to(device=E.device, dtype=torch.int64).contiguous()
         if csr is None:
@@ -148,8 +158,8 @@ class BaseKGE(torch.nn.Module):
         rows = csr.rows_for(x.to(device=E.device, dtype=torch.int64))
         return ops.rank_filtered(Q, bias, E, scale, target, rows, csr.row_ptr, csr.col)
 
-    def topk(self, x, k, sigmoid=False):
-        Q, bias = self.query(x)
+    def topk(self, x, k, sigmoid=False, heads=False):
+        Q, bias = self.query(x, heads=heads)
         E, scale = self.table()
         return ops.topk(Q, bias, E, scale, k, sigmoid=sigmoid)
 

@@ -46,8 +46,9 @@ def _norm_struct(norm):
 
 
 def build_query(model, ent, rel, hr, *, ent_scale=None, p=0, q=0, coeff_p=None, coeff_q=None,
-                normalize_relation=True, norm=None):
-    """(Q [B,d] fp32, bias [B] fp32) with ``forward_k_vs_all(x) == Q @ E^T + bias[:, None]``."""
+                normalize_relation=True, norm=None, head=False):
+    """(Q [B,d] fp32, bias [B] fp32) with ``forward_k_vs_all(x) == Q @ E^T + bias[:, None]``.
+    ``head=True``: ``hr`` holds (relation, tail) pairs and ``Q @ E^T`` scores every entity as the head."""
     lib = _lib.load()
     _require_gpu(ent, rel, hr, ent_scale, coeff_p, coeff_q)
     if hr.dtype != torch.int64 or hr.dim() != 2 or hr.shape[1] != 2:
@@ -58,10 +59,10 @@ def build_query(model, ent, rel, hr, *, ent_scale=None, p=0, q=0, coeff_p=None, 
     Q = torch.empty((B, d), dtype=torch.float32, device=ent.device)
     bias = torch.empty((B,), dtype=torch.float32, device=ent.device)
     ns, keep = _norm_struct(norm)
-    rc = lib.kge_build_query(MODEL_IDS[model], int(p), int(q), _ptr(ent), _table_dtype(ent), _ptr(ent_scale),
-                             _ptr(rel), _table_dtype(rel), _ptr(coeff_p), _ptr(coeff_q), int(bool(normalize_relation)),
-                             ctypes.byref(ns) if ns is not None else None, _ptr(hr), B, d, N, R, _ptr(Q), _ptr(bias),
-                             _stream())
+    fn = lib.kge_build_query_head if head else lib.kge_build_query
+    rc = fn(MODEL_IDS[model], int(p), int(q), _ptr(ent), _table_dtype(ent), _ptr(ent_scale),
+            _ptr(rel), _table_dtype(rel), _ptr(coeff_p), _ptr(coeff_q), int(bool(normalize_relation)),
+            ctypes.byref(ns) if ns is not None else None, _ptr(hr), B, d, N, R, _ptr(Q), _ptr(bias), _stream())
     _lib.check(rc)
     del keep
     return Q, bias

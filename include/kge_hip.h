@@ -83,6 +83,24 @@ int kge_build_query(int model, int p, int q, const void* ent, int ent_dtype, con
                     int64_t B, int64_t d, int64_t N, int64_t R, float* Q, float* bias, void* stream);
 
 /*
+ * The same for the head direction: one query vector per (relation, tail) pair so that
+ * score(x, r, t) == dot(Q[b], E[x]) for every entity x (bias is written as zero: every term of every
+ * model's triple score holds the head).  With kge_rank_filtered / kge_topk / kge_scores this replaces
+ * the head half of evaluate_lp (dicee/evaluation/link_prediction.py:421-429 scores every
+ * (x, r, t) triple through forward_triples: DistMult.score dicee/models/real.py:48-49, ComplEx.score
+ * dicee/models/complex.py:229-238, QMult.score dicee/models/quaternion.py:102-122, Keci.score
+ * dicee/models/clifford.py:448-499).  For Keci with p > 0 the per-triple value is the one the
+ * model's own KvsAll path gives, forward_k_vs_all((x, r))[t]; the reference's forward_triples sums
+ * two of its einsums over the batch as well (clifford.py:528-529).
+ *   rt [B,2] int64 = (relation id, tail id).  norm must be NULL or KGE_NORM_NONE (a normalised head
+ *   row is not a row of the table): KGE_ERR_UNSUPPORTED otherwise.  Other arguments as above.
+ */
+int kge_build_query_head(int model, int p, int q, const void* ent, int ent_dtype, const float* ent_scale,
+                         const void* rel, int rel_dtype, const float* coeff_p, const float* coeff_q,
+                         int normalize_relation, const kge_norm_params* norm, const int64_t* rt,
+                         int64_t B, int64_t d, int64_t N, int64_t R, float* Q, float* bias, void* stream);
+
+/*
  * Materialised scores S[b, e] = dot(Q[b], E[e]) (* scale[e]) (+ bias[b]); S has row stride ldS.
  * Replaces the torch.mm / einsum calls and B x N adds of real.py:32, complex.py:260-264,
  * quaternion.py:152-156, clifford.py:269-305.  For callers that need the whole matrix

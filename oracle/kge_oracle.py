@@ -31,6 +31,11 @@ Pinning status (independent checks live in ``tests/test_oracle_pins.py``)
 * ``bce_multihot``    ``torch.nn.functional.binary_cross_entropy_with_logits``
                       on a dense target, with and without label smoothing.
 * ``bf16_round`` / ``quantize_int8_rows``  torch's bf16 cast; closed forms.
+* ``triple_scores``  equal to column t of the (pinned) KvsAll scores of (h, r) for all four models
+                      and every (p, q); ComplEx against complex128 ``Re<h, r, conj t>``.
+* ``head_query`` / ``all_head_scores``  column h of the head-direction scores of (r, t) equals
+                      ``triple_scores`` and the tail-direction score of the same triple;
+                      linearity in the head row.
 * ``vocab`` / ``vocab_csr``  hand-written 7-triple fixture; set identities
                       (every triple recoverable from exactly one row, rows
                       partition the distinct triples).
@@ -382,6 +387,130 @@ def k_vs_all_scores_ref_form(model, E, R, hr, p=0, q=0, coeff_p=None, coeff_q=No
     if model in ("Keci", "CKeci"):
         return keci_scores_ref_form(h, r, E, p, q, coeff_p, coeff_q)
     raise ValueError(model)
+
+
+# --------------------------------------------------------------------------
+# per-triple scores and the head direction   dicee/evaluation/link_prediction.py:351-473
+# --------------------------------------------------------------------------
+# ``evaluate_lp`` ranks the true tail among ``score(h, r, x)`` and the true head among
+# ``score(x, r, t)`` over all entities x, scored triple by triple with the model's ``score`` /
+# ``forward_triples``.  ``triple_scores`` restates those per-triple formulas; ``head_query`` is the
+# vector Q'(r, t) with ``score(x, r, t) = Q' . E[x]`` for every x, so the head direction is the same
+# table contraction as the tail direction.  Keci with p > 0: the reference's ``forward_triples``
+# (clifford.py:525-531) contracts its ``'brp, erp -> b'`` einsums over the batch index of the tails
+# as well, which couples unrelated triples of a batch; the per-triple value restated here is the one
+# its own KvsAll path gives, ``forward_k_vs_all((h, r))[t]``.
+
+
+def triple_scores(model, E, R, triples, p=0, q=0, coeff_p=None, coeff_q=None, normalize_relation=True,
+                  dtype=np.float64):
+    """score(h, r, t) for every row of ``triples`` [n,3]: DistMult.score (real.py:48-49),
+    ComplEx.score (complex.py:229-238), QMult.score (quaternion.py:102-122), Keci.score
+    (clifford.py:448-499), each written as explicit sums over the embedding parts."""
+    E = np.asarray(E, dtype=dtype)
+    R = np.asarray(R, dtype=dtype)
+    triples = np.asarray(triples)
+    h, r, t = E[triples[:, 0]], R[triples[:, 1]], E[triples[:, 2]]
+    n, d = h.shape
+    if model == "DistMult":
+        return (h * r * t).sum(axis=1)
+    if model == "ComplEx":
+        m = d // 2
+        hr_, hi_, rr_, ri_, tr_, ti_ = h[:, :m], h[:, m:], r[:, :m], r[:, m:], t[:, :m], t[:, m:]
+        return (hr_ * rr_ * tr_).sum(1) + (hr_ * ri_ * ti_).sum(1) + (hi_ * rr_ * ti_).sum(1) - (hi_ * ri_ * tr_).sum(1)
+    if model == "QMult":
+        if normalize_relation:
+            r = quaternion_normalize(r)
+        m = d // 4
+        ha, hb, hc, hd = (h[:, i * m:(i + 1) * m] for i in range(4))
+        ra, rb, rc, rd = (r[:, i * m:(i + 1) * m] for i in range(4))
+        ta, tb, tc, td = (t[:, i * m:(i + 1) * m] for i in range(4))
+        real = ha * ra - hb * rb - hc * rc - hd * rd
+        imi = ha * rb + hb * ra + hc * rd - hd * rc
+        imj = ha * rc - hb * rd + hc * ra + hd * rb
+        imk = ha * rd + hb * rc - hc * rb + hd * ra
+        return (real * ta).sum(1) + (imi * tb).sum(1) + (imj * tc).sum(1) + (imk * td).sum(1)
+    if model in ("Keci", "CKeci"):
+        rr = d // (p + q + 1)
+        out = np.zeros(n, dtype=dtype)
+        cp = np.asarray(coeff_p if p else [], dtype=dtype)
+        cq = np.asarray(coeff_q if q else [], dtype=dtype)
+        for b in range(n):
+            h0, hp, hq = (x[0] for x in keci_split(h[b:b + 1], rr, p, q))
+            r0, rp, rq = (x[0] for x in keci_split(r[b:b + 1], rr, p, q))
+            t0, tp, tq = (x[0] for x in keci_split(t[b:b + 1], rr, p, q))
+            hp, rp, hq, rq = hp * cp, rp * cp, hq * cq, rq * cq          # h and r parts scaled, t parts not
+            s = (h0 * r0 * t0).sum()
+            s += ((hp * rp).sum(1) * t0).sum() + (h0[:, None] * rp * tp).sum() + (hp * r0[:, None] * tp).sum()
+            s += -((hq * rq).sum(1) * t0).sum() + (h0[:, None] * rq * tq).sum() + (hq * r0[:, None] * tq).sum()
+            if p >= 2:
+                s += sum((hp[:, i] * rp[:, k] - hp[:, k] * rp[:, i]).sum() for i in range(p) for k in range(i + 1, p))
+            if q >= 2:
+                s += sum((hq[:, j] * rq[:, k] - hq[:, k] * rq[:, j]).sum() for j in range(q) for k in range(j + 1, q))
+            if p >= 2 and q >= 2:
+                s += sum((hp[:, i] * rq[:, j] - hq[:, j] * rp[:, i]).sum() for i in range(p) for j in range(q))
+            out[b] = s
+        return out
+    raise ValueError(model)
+
+
+def head_query(model, E, R, rt, p=0, q=0, coeff_p=None, coeff_q=None, normalize_relation=True, dtype=np.float64):
+    """Q' [B,d] with ``score(x, rt[b,0], rt[b,1]) = Q'[b] . E[x]`` (no bias: every term holds the head)."""
+    E = np.asarray(E, dtype=dtype)
+    R = np.asarray(R, dtype=dtype)
+    rt = np.asarray(rt)
+    r, t = R[rt[:, 0]], E[rt[:, 1]]
+    B, d = r.shape
+    if model == "DistMult":
+        return r * t
+    if model == "ComplEx":                                   # Re<h, r, conj t> = <h, conj(r) t>
+        m = d // 2
+        rr_, ri_, tr_, ti_ = r[:, :m], r[:, m:], t[:, :m], t[:, m:]
+        return np.concatenate([rr_ * tr_ + ri_ * ti_, rr_ * ti_ - ri_ * tr_], axis=1)
+    if model == "QMult":                                     # <h (x) r, t> = <h, t (x) conj r>
+        if normalize_relation:
+            r = quaternion_normalize(r)
+        m = d // 4
+        conj = np.concatenate([r[:, :m], -r[:, m:]], axis=1)
+        return np.concatenate(hamilton_product_blocks(t, conj), axis=1)
+    if model in ("Keci", "CKeci"):
+        rr = d // (p + q + 1)
+        r0, rp, rq = keci_split(r, rr, p, q)
+        t0, tp, tq = keci_split(t, rr, p, q)
+        cp = np.asarray(coeff_p if p else [], dtype=dtype).reshape(1, 1, p)
+        cq = np.asarray(coeff_q if q else [], dtype=dtype).reshape(1, 1, q)
+        rp, rq = rp * cp, rq * cq
+        q0 = r0 * t0 + (rp * tp).sum(2) + (rq * tq).sum(2)
+        qp = rp * t0[:, :, None] + r0[:, :, None] * tp
+        qq = -rq * t0[:, :, None] + r0[:, :, None] * tq
+        if p >= 2:                                           # d sigma_pp / d hp_i = sum_{k>i} rp_k - sum_{k<i} rp_k
+            for i in range(p):
+                qp[:, :, i] += rp[:, :, i + 1:].sum(2) - rp[:, :, :i].sum(2)
+        if q >= 2:
+            for j in range(q):
+                qq[:, :, j] += rq[:, :, j + 1:].sum(2) - rq[:, :, :j].sum(2)
+        if p >= 2 and q >= 2:                                # sigma_pq = sum_ij hp_i rq_j - hq_j rp_i
+            qp += rq.sum(2)[:, :, None]
+            qq -= rp.sum(2)[:, :, None]
+        qp, qq = qp * cp, qq * cq                            # the head's own parts are scaled too
+        return np.concatenate([q0, qp.reshape(B, rr * p), qq.reshape(B, rr * q)], axis=1)
+    raise ValueError(model)
+
+
+def all_head_scores(model, E, R, rt, **kw):
+    """[B,N]: score(x, r, t) for every entity x."""
+    dtype = kw.get("dtype", np.float64)
+    return head_query(model, E, R, rt, **kw) @ np.asarray(E, dtype=dtype).T
+
+
+def lp_metrics(head_ranks, tail_ranks):
+    """``evaluate_lp``'s reduction (link_prediction.py:452-468): hits count both directions over 2n,
+    MRR = sum(1/head_rank + 1/tail_rank) / 2n."""
+    hr_, tr_ = np.asarray(head_ranks, dtype=np.int64), np.asarray(tail_ranks, dtype=np.int64)
+    n2 = float(2 * len(hr_))
+    out = {f"H@{k}": float(((hr_ <= k).sum() + (tr_ <= k).sum()) / n2) for k in (1, 3, 10)}
+    out["MRR"] = float((1.0 / hr_ + 1.0 / tr_).sum() / n2)
+    return out
 
 
 # --------------------------------------------------------------------------

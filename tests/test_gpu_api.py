@@ -227,3 +227,46 @@ def test_stored_experiment_evaluates_end_to_end(tmp_path):
         assert lo <= got[j] <= hi
     want = ko.metrics_from_ranks(got)
     assert report["Test"]["MRR"] == pytest.approx(want["MRR"]) and report["Test"]["H@3"] == want["H@3"]
+
+
+@pytest.mark.parametrize("name,d,extra", [("DistMult", 32, {}), ("ComplEx", 64, {}), ("QMult", 64, {}),
+                                          ("Keci", 48, {"p": 0, "q": 1}), ("Keci", 40, {"p": 2, "q": 2})])
+def test_evaluate_lp_both_directions(name, d, extra):
+    """Head and tail ranks inside the fp64 oracle's tolerance interval, exact where there is no near-tie; metrics
+    reduced as evaluate_lp does; dict and GPU-built vocabularies give the same ranks."""
+    from dicee_amd import evaluate_lp, FilterCSR
+    m, triples = _toy(name, d, n=1500, seed=21, **extra)
+    E = m.entity_embeddings.weight.detach().numpy().copy()
+    Rel = m.relation_embeddings.weight.detach().numpy().copy()
+    kw = _oracle_kw(m)
+    er, re = ko.vocab(triples, "er"), ko.vocab(triples, "re")
+    m = m.to("cuda")
+    test = triples[300:640]
+    res, (hr_, tr_) = evaluate_lp(m, test, 135, er, re, info=None, batch_size=100, return_ranks=True)
+    St = ko.k_vs_all_scores(name, E, Rel, test[:, :2], **kw)
+    Sh = ko.all_head_scores(name, E, Rel, test[:, 1:], **kw)
+    exact = 0
+    for j, (h, r, t) in enumerate(test):
+        h, r, t = int(h), int(r), int(t)
+        lo, hi = ko.rank_interval_with_tolerance(St[j], t, er[(h, r)], 1e-5 * np.sqrt((St[j] ** 2).mean()))
+        assert lo <= tr_[j] <= hi
+        lo2, hi2 = ko.rank_interval_with_tolerance(Sh[j], h, re[(r, t)], 1e-5 * np.sqrt((Sh[j] ** 2).mean()))
+        assert lo2 <= hr_[j] <= hi2
+        exact += (lo == hi) + (lo2 == hi2)
+    assert exact >= 2 * len(test) * 0.95
+    want = ko.lp_metrics(hr_, tr_)
+    for key in ("H@1", "H@3", "H@10", "MRR"):
+        assert res[key] == pytest.approx(want[key])
+    dev_trip = torch.from_numpy(triples).cuda()
+    res2, (hr2, tr2) = evaluate_lp(m, test, 135, FilterCSR.from_triples_gpu(dev_trip, 135, 46, kind="er"),
+                                   FilterCSR.from_triples_gpu(dev_trip, 135, 46, kind="re"), info=None,
+                                   batch_size=512, return_ranks=True)
+    np.testing.assert_array_equal(hr2, hr_)
+    np.testing.assert_array_equal(tr2, tr_)
+    assert res2 == res
+    # the head-direction score matrix itself, materialised
+    Sg = m.forward_all_heads(torch.from_numpy(test[:50, 1:].copy()).cuda()).cpu().numpy()
+    ok, worst = score_close(Sg, Sh[:50], 1e-5)
+    assert ok, worst
+    with pytest.raises(AssertionError):
+        evaluate_lp(m, test, 135, er, None, info=None)

@@ -436,3 +436,60 @@ def test_csr_built_on_the_gpu_filters_like_the_host_built_one():
     b = ops.rank_filtered(Q, bias, Eg, None, tgt, gpu.rows_for(hr), gpu.row_ptr, gpu.col)
     for key in a:
         assert torch.equal(a[key], b[key])
+
+
+# ---------------------------------------------------------------------------------------------
+# head direction: Q'(r, t) with score(x, r, t) = Q' . E[x]
+# ---------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("model,d,kw", MODEL_CASES)
+def test_build_query_head_fp32(ops, model, d, kw):
+    rng = np.random.default_rng(200 + d)
+    N, R, B = 300, 17, 77
+    E, Rel = random_tables(rng, N, R, d, std=0.5)
+    rt = np.stack([rng.integers(0, R, B), rng.integers(0, N, B)], axis=1).astype(np.int64)
+    Q, bias = ops.build_query(model, dev(torch.from_numpy(E)), dev(torch.from_numpy(Rel)),
+                              dev(torch.from_numpy(rt)), head=True, **_gpu_kwargs(kw))
+    Qr = ko.head_query(model, E, Rel, rt, **kw)
+    ok, worst = score_close(Q.cpu().numpy(), Qr, 1e-5)
+    assert ok, worst
+    assert float(bias.abs().max()) == 0.0
+    # one triple, both directions, through the library: S_tail[b, t] == S_head[b, h]
+    h = rng.integers(0, N, B).astype(np.int64)
+    hr = np.stack([h, rt[:, 0]], axis=1)
+    Eg = dev(torch.from_numpy(E))
+    Qt, bt = ops.build_query(model, Eg, dev(torch.from_numpy(Rel)), dev(torch.from_numpy(hr)), **_gpu_kwargs(kw))
+    St = ops.scores(Qt, bt, Eg).cpu().numpy()[np.arange(B), rt[:, 1]]
+    Sh = ops.scores(Q, bias, Eg).cpu().numpy()[np.arange(B), h]
+    ref = ko.triple_scores(model, E, Rel, np.stack([h, rt[:, 0], rt[:, 1]], axis=1), **kw)
+    scale = np.sqrt((ref ** 2).mean())
+    assert np.abs(St - ref).max() <= 2e-5 * scale and np.abs(Sh - ref).max() <= 2e-5 * scale
+
+
+@pytest.mark.parametrize("storage", ["bf16", "int8"])
+@pytest.mark.parametrize("model", ["DistMult", "ComplEx", "QMult"])
+def test_build_query_head_quantised_tables(ops, model, storage):
+    rng = np.random.default_rng(17)
+    N, R, d, B = 200, 9, 128, 50
+    E, Rel = random_tables(rng, N, R, d)
+    rt = np.stack([rng.integers(0, R, B), rng.integers(0, N, B)], axis=1).astype(np.int64)
+    Et, sc, Rt, Ev, Rv = stored_tables(E, Rel, storage)
+    Q, _ = ops.build_query(model, dev(Et), dev(Rt), dev(torch.from_numpy(rt)), ent_scale=dev(sc), head=True)
+    ok, worst = score_close(Q.cpu().numpy(), ko.head_query(model, Ev, Rv, rt), 1e-5)
+    assert ok, worst
+
+
+def test_build_query_head_argument_checks(ops):
+    from dicee_amd._lib import KgeError
+    rng = np.random.default_rng(19)
+    E, Rel = random_tables(rng, 50, 4, 16)
+    Eg, Rg = dev(torch.from_numpy(E)), dev(torch.from_numpy(Rel))
+    rt = np.array([[0, 0], [4, 1], [3, 50], [0, -1], [3, 49]], dtype=np.int64)       # (relation, tail)
+    Q, bias = ops.build_query("ComplEx", Eg, Rg, dev(torch.from_numpy(rt)), head=True)
+    Q = Q.cpu().numpy()
+    assert np.isnan(Q[1]).all() and np.isnan(Q[2]).all() and np.isnan(Q[3]).all()
+    assert np.isfinite(Q[0]).all() and np.isfinite(Q[4]).all()
+    ones = torch.ones(16, device="cuda")
+    norm = {"kind": "LayerNorm", "eps": 1e-5, "h_a": ones, "h_b": ones, "r_a": ones, "r_b": ones}
+    with pytest.raises(KgeError) as err:
+        ops.build_query("ComplEx", Eg, Rg, dev(torch.from_numpy(rt)), head=True, norm=norm)
+    assert err.value.code == 2

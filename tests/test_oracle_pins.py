@@ -407,3 +407,49 @@ def test_vocab_csr_against_a_hand_written_fixture_and_set_identities():
         assert len(col) == len(rebuilt)
         for i in range(len(keys)):
             assert np.all(np.diff(col[row_ptr[i]:row_ptr[i + 1]]) > 0)
+
+
+_LP_CASES = [("DistMult", 12, {}), ("ComplEx", 12, {}), ("QMult", 16, {}), ("QMult", 16, {"normalize_relation": False}),
+             ("Keci", 12, {"p": 0, "q": 0}), ("Keci", 12, {"p": 0, "q": 1}), ("Keci", 12, {"p": 1, "q": 1}),
+             ("Keci", 12, {"p": 2, "q": 0}), ("Keci", 12, {"p": 0, "q": 2}), ("Keci", 15, {"p": 2, "q": 2}),
+             ("Keci", 18, {"p": 3, "q": 2}), ("Keci", 18, {"p": 1, "q": 4})]
+
+
+@pytest.mark.parametrize("model,d,kw", _LP_CASES)
+def test_triple_scores_and_head_direction_agree_with_the_kvsall_oracle(model, d, kw):
+    """One triple, three routes: the per-triple formula, column t of the tail-direction scores of (h, r),
+    column h of the head-direction scores of (r, t).  The tail direction is pinned above."""
+    rng = np.random.default_rng(d + len(kw))
+    N, R, n = 23, 5, 40
+    E, Rel = rng.standard_normal((N, d)), rng.standard_normal((R, d))
+    kw = dict(kw)
+    if model == "Keci":
+        kw["coeff_p"] = rng.standard_normal(kw["p"]) + 1.0
+        kw["coeff_q"] = rng.standard_normal(kw["q"]) + 1.0
+    triples = np.stack([rng.integers(0, N, n), rng.integers(0, R, n), rng.integers(0, N, n)], axis=1)
+    per_triple = ko.triple_scores(model, E, Rel, triples, **kw)
+    tails = ko.k_vs_all_scores(model, E, Rel, triples[:, :2], **kw)
+    np.testing.assert_allclose(per_triple, tails[np.arange(n), triples[:, 2]], rtol=1e-11, atol=1e-12)
+    heads = ko.all_head_scores(model, E, Rel, triples[:, 1:], **kw)
+    assert heads.shape == (n, N)
+    np.testing.assert_allclose(heads[np.arange(n), triples[:, 0]], per_triple, rtol=1e-11, atol=1e-12)
+    # every other column too: score(x, r, t) for a replaced head
+    for x in (0, N - 1):
+        swapped = triples.copy()
+        swapped[:, 0] = x
+        np.testing.assert_allclose(heads[:, x], ko.triple_scores(model, E, Rel, swapped, **kw), rtol=1e-11, atol=1e-12)
+
+
+def test_complex_triple_score_is_the_hermitian_product():
+    rng = np.random.default_rng(5)
+    E, Rel = rng.standard_normal((9, 10)), rng.standard_normal((3, 10))
+    triples = np.stack([rng.integers(0, 9, 20), rng.integers(0, 3, 20), rng.integers(0, 9, 20)], axis=1)
+    z = lambda x: x[:, :5] + 1j * x[:, 5:]
+    want = (z(E[triples[:, 0]]) * z(Rel[triples[:, 1]]) * np.conj(z(E[triples[:, 2]]))).sum(axis=1).real
+    np.testing.assert_allclose(ko.triple_scores("ComplEx", E, Rel, triples), want, rtol=1e-12)
+
+
+def test_lp_metrics_closed_form():
+    m = ko.lp_metrics([1, 4, 11], [2, 1, 3])
+    assert m["H@1"] == pytest.approx(2 / 6) and m["H@3"] == pytest.approx(4 / 6) and m["H@10"] == pytest.approx(5 / 6)
+    assert m["MRR"] == pytest.approx((1 + 1 / 4 + 1 / 11 + 1 / 2 + 1 + 1 / 3) / 6)
