@@ -1,9 +1,10 @@
-"""Interactive tail prediction on top of the fused top-k kernel.
+"""Interactive tail and head prediction on top of the fused top-k kernel.
 
-Mirrors the tail branch of dicee's ``KGE`` (dicee/knowledge_graph_embeddings.py):
-``predict_missing_tail_entity`` (:314-413), ``predict`` (:415-466) and ``predict_topk`` (:468-579).
-Head and relation prediction go through ``forward_triples`` in the reference and are outside this
-build: they raise ``NotImplementedError``.
+Mirrors dicee's ``KGE`` (dicee/knowledge_graph_embeddings.py): ``predict_missing_tail_entity``
+(:314-413), ``predict_missing_head_entity`` (:134-228), ``predict`` (:415-466) and ``predict_topk``
+(:468-579).  The reference scores every (x, r, t) triple through ``forward_triples`` for a missing
+head; here that is one head-direction query and the same table contraction as for tails.  Relation
+prediction is outside this build: it raises ``NotImplementedError``.
 """
 from typing import List, Union
 
@@ -36,6 +37,8 @@ class KGE:
         self.idx_to_relations = {v: k for k, v in self.relation_to_idx.items()}
         self.num_entities = len(self.entity_to_idx)
         self.num_relations = len(self.relation_to_idx)
+        base = [rel for rel in self.relation_to_idx if not str(rel).endswith("_inverse")]
+        self.all_have_inverse = all(f"{rel}_inverse" in self.relation_to_idx for rel in base)
 
     # ------------------------------------------------------------------ helpers
     def _hr_pairs(self, head_entity, relation):
@@ -76,6 +79,41 @@ class KGE:
             return scores.flatten(), indices.flatten()
         return scores
 
+    def predict_missing_head_entity(self, relation: Union[List[str], str], tail_entity: Union[List[str], str],
+                                    within: List[str] = None, batch_size=2, topk=1, return_indices=False):
+        """Scores (or the top-k) of every entity as head of (?, r, t); pairs are ordered tails-major
+        (``cartesian_prod(tail, relation)``).  With reciprocal relations in the vocabulary the question is asked
+        as the tail of (t, r_inverse, ?), as the reference does (:166-171)."""
+        if self.all_have_inverse:
+            relation = [f"{relation}_inverse"] if isinstance(relation, str) else [f"{rel}_inverse" for rel in relation]
+            return self.predict_missing_tail_entity(tail_entity, relation, within, batch_size, topk, return_indices)
+        if within is not None:
+            raise NotImplementedError("`within` needs the byte-pair-encoded path, which is outside this build")
+        rel = torch.LongTensor([self.relation_to_idx[i] for i in (relation if isinstance(relation, list) else [relation])])
+        tail = torch.LongTensor([self.entity_to_idx[i] for i in
+                                 (tail_entity if isinstance(tail_entity, list) else [tail_entity])])
+        tr_pairs = torch.cartesian_prod(tail, rel).view(-1, 2)
+        P, H = tr_pairs.size(0), self.num_entities
+        dev = self.model.entity_embeddings.weight.device
+        if return_indices:
+            scores = torch.zeros(P, topk)
+            indices = torch.zeros(P, topk, dtype=torch.long)
+        else:
+            scores = torch.zeros(P * H)
+        for i in range(0, P, batch_size):
+            batch = tr_pairs[i:i + batch_size]
+            rt = torch.stack([batch[:, 1], batch[:, 0]], dim=1).to(dev)      # the kernels take (relation, tail)
+            B = rt.size(0)
+            if return_indices:
+                s, idx = self.model.topk(rt, topk, heads=True)
+                scores[i:i + batch_size, :] = s.cpu()
+                indices[i:i + batch_size, :] = idx.cpu()
+            else:
+                scores[i * H:i * H + B * H] = self.model.forward_all_heads(rt).flatten().cpu()
+        if return_indices:
+            return scores.flatten(), indices.flatten()
+        return scores
+
     def predict(self, *, h: Union[List[str], str] = None, r: Union[List[str], str] = None,
                 t: Union[List[str], str] = None, within=None, logits=True) -> torch.FloatTensor:
         if h is not None:
@@ -84,11 +122,13 @@ class KGE:
             assert isinstance(r, (list, str))
         if t is not None:
             assert isinstance(t, (list, str))
-        if t is None:
-            assert h is not None and r is not None
+        if h is None:
+            assert r is not None and t is not None
+            scores = self.predict_missing_head_entity(r, t, within)
+        elif r is None:
+            raise NotImplementedError("relation prediction is outside the accelerated path")
+        elif t is None:
             scores = self.predict_missing_tail_entity(h, r, within)
-        elif h is None or r is None:
-            raise NotImplementedError("head / relation prediction is outside the accelerated path")
         else:
             raise NotImplementedError("triple_score is outside the accelerated path")
         return scores if logits else torch.sigmoid(scores)
@@ -103,17 +143,23 @@ class KGE:
             assert isinstance(r, (list, str))
         if t is not None:
             assert isinstance(t, (list, str))
-        if h is None or r is None:
-            raise NotImplementedError("head / relation prediction is outside the accelerated path")
-        if t is not None:
+        if h is None:
+            assert r is not None and t is not None
+            r = [r] if isinstance(r, str) else r
+            t = [t] if isinstance(t, str) else t
+            flat_scores, flat_indices = self.predict_missing_head_entity(r, t, within, batch_size, topk,
+                                                                         return_indices=True)
+            num_hr_pairs = len(r) * len(t)
+        elif r is None:
+            raise NotImplementedError("relation prediction is outside the accelerated path")
+        elif t is not None:
             raise AttributeError("Use triple_score method")
-        flat_scores, flat_indices = self.predict_missing_tail_entity(h, r, within, batch_size, topk,
-                                                                     return_indices=True)
-        if isinstance(h, str):
-            h = [h]
-        if isinstance(r, str):
-            r = [r]
-        num_hr_pairs = len(h) * len(r)
+        else:
+            flat_scores, flat_indices = self.predict_missing_tail_entity(h, r, within, batch_size, topk,
+                                                                         return_indices=True)
+            h = [h] if isinstance(h, str) else h
+            r = [r] if isinstance(r, str) else r
+            num_hr_pairs = len(h) * len(r)
         scores_2d = flat_scores.view(num_hr_pairs, topk)
         indices_2d = flat_indices.view(num_hr_pairs, topk)
         topk_scores = torch.sigmoid(scores_2d).tolist()

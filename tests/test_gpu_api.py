@@ -270,3 +270,37 @@ def test_evaluate_lp_both_directions(name, d, extra):
     assert ok, worst
     with pytest.raises(AssertionError):
         evaluate_lp(m, test, 135, er, None, info=None)
+
+
+def test_predict_missing_head():
+    from dicee_amd import KGE
+    m, _ = _toy("ComplEx", 32, seed=23)
+    E = m.entity_embeddings.weight.detach().numpy().copy()
+    Rel = m.relation_embeddings.weight.detach().numpy().copy()
+    m = m.to("cuda")
+    ents = {f"e{i}": i for i in range(135)}
+    rels = {f"r{i}": i for i in range(46)}
+    kge = KGE(model=m, entity_to_idx=ents, relation_to_idx=rels)
+    assert not kge.all_have_inverse
+    top = kge.predict_topk(r=["r3", "r4"], t=["e10", "e20", "e30"], topk=5, batch_size=4)
+    assert len(top) == 6 and all(len(row) == 5 for row in top)
+    # pairs are tails-major: (e10,r3), (e10,r4), (e20,r3), ...
+    rt = np.array([[3, 10], [4, 10], [3, 20], [4, 20], [3, 30], [4, 30]])
+    S = ko.all_head_scores("ComplEx", E, Rel, rt)
+    _, wi = ko.topk(S, 5)
+    for row, want_idx, srow in zip(top, wi, S):
+        assert [ents[e] for e, _ in row] == want_idx.tolist()
+        np.testing.assert_allclose([p for _, p in row], ko.sigmoid(srow[want_idx]), rtol=1e-5)
+    full = kge.predict(r=["r3"], t=["e10"])
+    assert full.shape == (135,)
+    ok, worst = score_close(full.numpy()[None, :], S[:1], 1e-5)
+    assert ok, worst
+    assert kge.predict_topk(r="r3", t="e10", topk=5)[0] == top[0]
+    with pytest.raises(NotImplementedError):
+        kge.predict_topk(h=["e1"], t=["e2"])
+    # reciprocal vocabulary: the head question is asked as a tail question with r_inverse
+    rels2 = {f"r{i}": i for i in range(23)}
+    rels2.update({f"r{i}_inverse": 23 + i for i in range(23)})
+    kge2 = KGE(model=m, entity_to_idx=ents, relation_to_idx=rels2)
+    assert kge2.all_have_inverse
+    assert kge2.predict_topk(r=["r3"], t=["e10"], topk=4) == kge2.predict_topk(h=["e10"], r=["r3_inverse"], topk=4)
