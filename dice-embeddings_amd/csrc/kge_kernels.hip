@@ -143,80 +143,86 @@ __global__ void csr_lookup_kernel(const int64_t* hr, int64_t B, const int64_t* k
 }
 
 // ---- group the queries of one sub-batch by filter row and plan the correction work -----------
-// One workgroup.  (1) sort (csr_row, query) keys so queries sharing a filter row are adjacent;
-// (2) for the first query of each group, find the group's end; (3) cut every group's filter row
-// into slices of `slice` entries (chosen so that there are at most WORK_MAX work items) and emit
-// one record per group (first position, index of its first work item); work item w is slice
-// w - first of the group found by binary search.
-constexpr int SORT_MAX = 8192;
+// One workgroup, no sort: (1) every query claims the slot of its filter row in an LDS hash table
+// (compare-and-swap on the row number) and takes a ticket from the slot's counter; the query with
+// ticket 0 leads the group and fetches the row's length; (2) total filter length -> slice length
+// (chosen so that there are at most WORK_MAX work items); (3) one exclusive scan over the leaders
+// of three packed counters gives every group its index, the position of its first member and the
+// index of its first work item; (4) members are written to their positions.  A group is the set of
+// queries of the sub-batch that share a filter row (= the same (head, relation) pair, hence the
+// same query vector); work item w is slice w - first of the group found by binary search in the
+// group records.
+constexpr int SORT_MAX = 8192;           // queries per sub-batch
 constexpr int WORK_MAX = 16 * SORT_MAX;  // upper bound on work items per sub-batch (bounds the slice count only)
 constexpr int SLICE_MIN = 128;
+constexpr int PLAN_SLOTS = 2 * SORT_MAX;  // hash table size: load factor <= 0.5
 
 struct FixPlan {
-  unsigned long long* skey;  // [SORT_MAX] sorted keys: csr_row << 24 | position in sub-batch (~0 = no filter)
+  unsigned long long* skey;  // [SORT_MAX] csr_row << 24 | position in sub-batch, the members of a group adjacent
   int32_t* gend;             // [SORT_MAX] for a group's first position: one past its last position
-  int32_t* work;             // [SORT_MAX][2] per group, in order: (first position, index of its first work item)
+  int32_t* work;             // [SORT_MAX][2] per group: (first position, index of its first work item)
   int32_t* meta;             // [0] work items, [1] slice length, [2] groups
 };
 
 __global__ void __launch_bounds__(1024) plan_fix_kernel(const int64_t* csr_row, int64_t b0, int nb, int64_t n_rows,
-                                                       const int64_t* row_ptr, FixPlan plan, int npad) {
-  extern __shared__ unsigned long long keys[];  // npad keys, then npad ints of scan space
-  int32_t* scan = (int32_t*)(keys + npad);
+                                                       const int64_t* row_ptr, FixPlan plan) {
+  __shared__ int32_t tab_row[PLAN_SLOTS];  // filter row + 1 that owns the slot, 0 = free
+  __shared__ int32_t tab_cnt[PLAN_SLOTS];  // members of the slot's group; later: position of its first member
+  __shared__ unsigned long long part[1024];
   __shared__ unsigned long long s_total;
   __shared__ int s_slice;
+  constexpr int QPT = SORT_MAX / 1024;     // queries per thread
   const int tid = threadIdx.x;
-  for (int i = tid; i < npad; i += 1024) {
-    unsigned long long key = ~0ull;
-    if (i < nb) {
-      const int64_t r = csr_row[b0 + i];
-      if (r >= 0 && r < n_rows) key = ((unsigned long long)r << 24) | (unsigned long long)i;
-    }
-    keys[i] = key;
+  for (int i = tid; i < PLAN_SLOTS; i += 1024) {
+    tab_row[i] = 0;
+    tab_cnt[i] = 0;
   }
   if (tid == 0) s_total = 0;
+  // the filter rows of this thread's queries (independent loads, all in flight together)
+  int64_t my_row[QPT];
+#pragma unroll
+  for (int j = 0; j < QPT; ++j) {
+    const int i = tid + 1024 * j;
+    int64_t r = -1;
+    if (i < nb) r = csr_row[b0 + i];
+    my_row[j] = (r >= 0 && r < n_rows) ? r : -1;
+  }
   __syncthreads();
-  for (int k = 2; k <= npad; k <<= 1) {
-    for (int j = k >> 1; j > 0; j >>= 1) {
-      for (int i = tid; i < npad; i += 1024) {
-        const int ixj = i ^ j;
-        if (ixj > i) {
-          const bool up = (i & k) == 0;
-          const unsigned long long x = keys[i], y = keys[ixj];
-          if ((x > y) == up) {
-            keys[i] = y;
-            keys[ixj] = x;
-          }
-        }
+  // (1) claim slots, take tickets
+  int my_slot[QPT], my_pos[QPT];
+#pragma unroll
+  for (int j = 0; j < QPT; ++j) {
+    my_slot[j] = -1;
+    my_pos[j] = -1;
+    if (my_row[j] >= 0) {
+      const int32_t key = (int32_t)my_row[j] + 1;
+      uint32_t h = ((uint32_t)my_row[j] * 2654435761u) >> 18;  // top 14 bits: PLAN_SLOTS = 2^14
+      static_assert(PLAN_SLOTS == (1 << 14), "hash width");
+      for (;;) {
+        const int32_t old = atomicCAS(&tab_row[h], 0, key);
+        if (old == 0 || old == key) break;
+        h = (h + 1) & (PLAN_SLOTS - 1);
       }
-      __syncthreads();
+      my_slot[j] = (int)h;
+      my_pos[j] = atomicAdd(&tab_cnt[h], 1);
     }
   }
-  // group heads, group ends (binary search for the first key of a later row), total filter length
+  // leaders fetch their row's length (unconditional loads of a valid row keep them in flight together)
+  int64_t len[QPT];
   unsigned long long my_total = 0;
-  for (int i = tid; i < npad; i += 1024) {
-    const unsigned long long key = keys[i];
-    plan.skey[i] = key;
-    int32_t ge = 0;
-    if (key != ~0ull && (i == 0 || (keys[i - 1] >> 24) != (key >> 24))) {
-      const unsigned long long next_row_key = ((key >> 24) + 1) << 24;
-      int lo = i + 1, hi = npad;
-      while (lo < hi) {
-        const int mid = (lo + hi) >> 1;
-        if (keys[mid] < next_row_key) lo = mid + 1; else hi = mid;
-      }
-      ge = lo;
-      const int64_t row = (int64_t)(key >> 24);
-      my_total += (unsigned long long)(row_ptr[row + 1] - row_ptr[row]);
-    }
-    plan.gend[i] = ge;   // 0 for positions that do not start a group
-    scan[i] = ge;
+#pragma unroll
+  for (int j = 0; j < QPT; ++j) {
+    const bool lead = my_pos[j] == 0;
+    const int64_t rr = lead ? my_row[j] : 0;
+    const int64_t l = row_ptr[rr + 1] - row_ptr[rr];
+    len[j] = lead ? l : 0;
+    my_total += (unsigned long long)len[j];
   }
   if (my_total) atomicAdd(&s_total, my_total);
   __syncthreads();
+  // (2) slice length: at least SLICE_MIN, large enough that extra slices fit the work list
   if (tid == 0) {
-    // slice length: at least SLICE_MIN, large enough that extra slices fit the work list
-    const unsigned long long room = (unsigned long long)(WORK_MAX - npad);
+    const unsigned long long room = (unsigned long long)(WORK_MAX - SORT_MAX);
     unsigned long long sl = (s_total + room - 1) / room;
     sl = (sl + 31) & ~31ull;
     if (sl < SLICE_MIN) sl = SLICE_MIN;
@@ -224,26 +230,15 @@ __global__ void __launch_bounds__(1024) plan_fix_kernel(const int64_t* csr_row, 
   }
   __syncthreads();
   const int slice = s_slice;
-  // per position: (is a group head, number of slices); one exclusive scan of the packed pair gives
-  // every group its index and the index of its first work item
-  constexpr int PER = SORT_MAX / 1024;  // positions per thread when npad == SORT_MAX
-  unsigned long long val[PER];
+  // (3) per leader with work: groups (bits 48..), members (bits 32..47), slices (bits 0..31)
+  unsigned long long val[QPT];
   unsigned long long local = 0;
-  const int per = (npad + 1023) / 1024;
-  for (int j = 0; j < per; ++j) {
-    const int i = tid * per + j;
-    unsigned long long v = 0;
-    if (i < npad && scan[i] != 0) {
-      const int64_t row = (int64_t)(keys[i] >> 24);
-      const int64_t L = row_ptr[row + 1] - row_ptr[row];
-      const unsigned long long n = (unsigned long long)((L + slice - 1) / slice);  // an empty row needs no work
-      if (n > 0) v = (1ull << 32) | n;
-    }
-    val[j] = v;
-    local += v;
+#pragma unroll
+  for (int j = 0; j < QPT; ++j) {
+    const unsigned long long n = (unsigned long long)((len[j] + slice - 1) / slice);  // an empty row needs no work
+    val[j] = (n > 0) ? ((1ull << 48) | ((unsigned long long)tab_cnt[my_slot[j]] << 32) | n) : 0;
+    local += val[j];
   }
-  __syncthreads();
-  __shared__ unsigned long long part[1024];
   part[tid] = local;
   __syncthreads();
   for (int off = 1; off < 1024; off <<= 1) {
@@ -253,18 +248,33 @@ __global__ void __launch_bounds__(1024) plan_fix_kernel(const int64_t* csr_row, 
     __syncthreads();
   }
   unsigned long long base = part[tid] - local;
-  for (int j = 0; j < per; ++j) {
+#pragma unroll
+  for (int j = 0; j < QPT; ++j) {
     if (val[j]) {
-      const int g = (int)(base >> 32);
-      plan.work[2 * g] = tid * per + j;
+      const int g = (int)(base >> 48), first = (int)((base >> 32) & 0xffffull);
+      plan.work[2 * g] = first;
       plan.work[2 * g + 1] = (int)(base & 0xffffffffull);
+      plan.gend[first] = first + tab_cnt[my_slot[j]];
+      tab_cnt[my_slot[j]] = first;  // only this leader reads or writes its group's slot in this phase
+    } else if (my_pos[j] == 0) {
+      tab_cnt[my_slot[j]] = -1;     // empty filter row: nothing to take out for this group
     }
     base += val[j];
   }
   if (tid == 1023) {
     plan.meta[0] = (int)(part[1023] & 0xffffffffull);
     plan.meta[1] = slice;
-    plan.meta[2] = (int)(part[1023] >> 32);
+    plan.meta[2] = (int)(part[1023] >> 48);
+  }
+  __syncthreads();
+  // (4) members to their positions
+#pragma unroll
+  for (int j = 0; j < QPT; ++j) {
+    if (my_slot[j] >= 0) {
+      const int first = tab_cnt[my_slot[j]];
+      if (first >= 0)
+        plan.skey[first + my_pos[j]] = ((unsigned long long)my_row[j] << 24) | (unsigned long long)(tid + 1024 * j);
+    }
   }
 }
 
@@ -834,7 +844,7 @@ extern "C" int kge_rank_filtered(const float* Q, const float* bias, const void* 
   const bool filtered = csr_row != nullptr;
   KGE_REQUIRE(!filtered || (row_ptr && col && n_rows >= 0), KGE_ERR_INVALID,
               "kge_rank_filtered: csr_row given without row_ptr / col");
-  KGE_REQUIRE(n_rows < (1LL << 39), KGE_ERR_INVALID, "kge_rank_filtered: n_rows=%lld too large", (long long)n_rows);
+  KGE_REQUIRE(n_rows < 0x7fffffffLL, KGE_ERR_INVALID, "kge_rank_filtered: n_rows=%lld too large", (long long)n_rows);
   KGE_REQUIRE(workspace && workspace_bytes >= kge_rank_workspace_bytes(B), KGE_ERR_WORKSPACE,
               "kge_rank_filtered: workspace of %zu bytes, need %zu", workspace_bytes, kge_rank_workspace_bytes(B));
   hipStream_t st = (hipStream_t)stream;
@@ -854,13 +864,7 @@ extern "C" int kge_rank_filtered(const float* Q, const float* bias, const void* 
   if (filtered && n_rows > 0) {
     for (int64_t b0 = 0; b0 < B; b0 += SORT_MAX) {
       const int nb = (int)((B - b0 < SORT_MAX) ? B - b0 : SORT_MAX);
-      int npad = 1024;
-      while (npad < nb) npad <<= 1;
-      if ((size_t)npad * 12 > 65536)  // more dynamic LDS than the default limit: opt in (idempotent)
-        KGE_HIP_CHECK(hipFuncSetAttribute((const void*)plan_fix_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                          SORT_MAX * 12));
-      hipLaunchKernelGGL(plan_fix_kernel, dim3(1), dim3(1024), (size_t)npad * 12, st, csr_row, b0, nb, n_rows,
-                         row_ptr, ws.plan, npad);
+      hipLaunchKernelGGL(plan_fix_kernel, dim3(1), dim3(1024), 0, st, csr_row, b0, nb, n_rows, row_ptr, ws.plan);
       KGE_LAUNCH_CHECK("plan_fix_kernel");
       dim3 grid(2048), block(256);
       KGE_DISPATCH_DTYPE(dtype, filter_fix_kernel, grid, block, 0, st, a, ws.plan, b0, row_ptr, col, target, ws.thr,
