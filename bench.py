@@ -81,7 +81,7 @@ def cpu_baseline(cfg, model, mode, seconds_budget=25.0):
 
 def main_loop_kernel(storage, d, mode):
     """Name of the contraction kernel the library picks for this table type and width."""
-    epi = {"rank": "RankEpi", "topk": "TopkEpi", "bce": "BceEpi"}[mode]
+    epi = {"rank": "RankEpi", "headrank": "RankEpi", "topk": "TopkEpi", "bce": "BceEpi"}[mode]
     if storage == "fp32":
         return f"kloop_async_kernel<{epi}>" if d % 4 == 0 else f"kloop_kernel<{epi}>"
     if d == 128:
@@ -95,6 +95,9 @@ def main():
     ap.add_argument("--steps", type=int, default=None)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--config", default="c4", choices=sorted(MODE))
+    ap.add_argument("--mode", default=None, choices=["rank", "topk", "bce", "headrank"],
+                    help="epilogue to run instead of the configuration's own (headrank: rank the true head of "
+                         "(?, r, t) with the (r, t) -> heads filter)")
     ap.add_argument("--scale", type=float, default=1.0, help="shrink the workload (testing only)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -112,16 +115,27 @@ def main():
 
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     dev = torch.device("cuda:0")
-    mode = MODE[args.config]
+    mode = args.mode or MODE[args.config]
     t_setup = time.perf_counter()
     big = args.config in ("c4", "c5") and args.scale == 1.0
     cfg = synthetic.make_config(args.config, scale=args.scale, with_tables=not big)
     model = synthetic.make_model(cfg, dev, tables_on_device=big)
+    if mode in ("rank", "bce", "headrank") and cfg.csr is None:
+        print(f"bench.py: --mode {mode} needs a configuration with triples", file=sys.stderr)
+        sys.exit(2)
     if cfg.csr is not None:
         cfg.csr.to(dev)
     q_all = torch.from_numpy(np.ascontiguousarray(cfg.queries)).to(dev)
-    batches = [(q_all[i:i + cfg.B, :2].contiguous(), q_all[i:i + cfg.B, 2].contiguous())
-               for i in range(0, len(q_all), cfg.B)]
+    re_csr = None
+    if mode == "headrank":
+        from dicee_amd.csr import FilterCSR
+        re_csr = FilterCSR.from_triples_gpu(torch.from_numpy(np.ascontiguousarray(cfg.triples)).to(dev), cfg.N, cfg.R,
+                                            kind="re")
+        batches = [(q_all[i:i + cfg.B, 1:].contiguous(), q_all[i:i + cfg.B, 0].contiguous())
+                   for i in range(0, len(q_all), cfg.B)]
+    else:
+        batches = [(q_all[i:i + cfg.B, :2].contiguous(), q_all[i:i + cfg.B, 2].contiguous())
+                   for i in range(0, len(q_all), cfg.B)]
     steps = args.steps if args.steps is not None else max(2 * len(batches), 20)
     torch.cuda.synchronize()
     t_setup = time.perf_counter() - t_setup
@@ -130,6 +144,8 @@ def main():
         x, t = batches[i % len(batches)]
         if mode == "rank":
             return model.rank_filtered(x, t, cfg.csr)
+        if mode == "headrank":
+            return model.rank_filtered(x, t, re_csr, heads=True)
         if mode == "topk":
             return model.topk(x, cfg.k)
         return model.kvsall_bce_loss(x, cfg.csr)
@@ -160,7 +176,7 @@ def main():
     achieved = flops / (kernel_ms * 1e-3) / 1e12 if kernel_ms > 0 else 0.0
     out = {
         "metric": {"rank": "filtered_rank_entity_scores_per_sec", "topk": "topk_entity_scores_per_sec",
-                   "bce": "kvsall_bce_entity_scores_per_sec"}[mode],
+                   "bce": "kvsall_bce_entity_scores_per_sec", "headrank": "filtered_head_rank_entity_scores_per_sec"}[mode],
         "value": scores / elapsed,
         "unit": "scores/s",
         "queries_per_sec": n_queries / elapsed,
@@ -173,11 +189,14 @@ def main():
                                f"batch {cfg.B}, {len(q_all)} queries"
                                + (f", filter CSR nnz={cfg.csr.nnz} max row {int(np.diff(cfg.csr.row_ptr_np).max())}"
                                   if cfg.csr is not None and mode == "rank" else "")
+                               + (f", (r,t)->heads CSR nnz={re_csr.nnz} max row {int(np.diff(re_csr.row_ptr_np).max())}"
+                                  if mode == "headrank" else "")
                                + (f", k={cfg.k}" if mode == "topk" else ""),
                    "scale": args.scale},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_TFLOPS[compute], "unit": "TFLOP/s",
                      "frac": achieved / PEAK_TFLOPS[compute],
-                     "traffic": MEASURED_TRAFFIC_BYTES.get(args.config) if args.scale == 1.0 else None,
+                     "traffic": MEASURED_TRAFFIC_BYTES.get(args.config)
+                     if args.scale == 1.0 and args.mode is None else None,
                      "kernel": main_loop_kernel(cfg.storage, d, mode),
                      "kernel_ms_avg": kernel_ms / max(launches, 1), "launches": launches,
                      "kernel_time_share": kernel_ms * 1e-3 / elapsed},
@@ -198,7 +217,7 @@ def main():
         out["csr_build"] = {"ms": tb * 1e3, "triples": int(trip.shape[0]), "rows": built.num_rows, "nnz": built.nnz,
                             "triples_per_sec": trip.shape[0] / tb}
         del trip, built
-    if not args.no_cpu_baseline:
+    if not args.no_cpu_baseline and mode != "headrank":
         out["cpu_baseline"] = cpu_baseline(cfg, model, mode)
     print(json.dumps(out))
 
