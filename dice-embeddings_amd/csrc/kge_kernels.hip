@@ -451,13 +451,121 @@ __global__ void topk_init_kernel(TopkWs w, int64_t B) {
 // Merge a query's kept list with this round's candidates, keep the best k, publish the new
 // threshold.  In `rescan` mode (only queries flagged dirty) list entries above the old threshold
 // are dropped first: the rescan finds all of them again.
-// Two launches cover a round: one wave per query (NT = 64, SELECT_SMALL keys of LDS, many queries
-// resident per CU) for the queries with at most SELECT_SMALL entries to rank, which is nearly all
-// of them, then four waves per query with room for a full candidate buffer for the rest.  A query
-// ranked by the first launch has its candidate count reset, so the second one skips it.
+// Bitonic sort, descending, of 64 * KPL keys held by one wave: element i = lane * KPL + s sits in
+// v[s] of `lane`.  Exchanges at distance < KPL stay inside a lane's registers; larger distances are
+// a lane shuffle.  No LDS, no barriers.
+template <int KPL>
+__device__ __forceinline__ void wave_sort_desc(unsigned long long (&v)[KPL], int lane) {
+  constexpr int N = 64 * KPL;
+#pragma unroll
+  for (int kk = 2; kk <= N; kk <<= 1) {
+#pragma unroll
+    for (int j = kk >> 1; j > 0; j >>= 1) {
+      if (j < KPL) {
+#pragma unroll
+        for (int s = 0; s < KPL; ++s) {
+          if ((s & j) == 0) {
+            // element index i = lane * KPL + s; the pair is ordered "larger first" iff (i & kk) == 0
+            const bool down = (kk < KPL) ? ((s & kk) == 0) : (((lane * KPL) & kk) == 0);
+            const unsigned long long x = v[s], y = v[s | j];
+            const unsigned long long hi = x > y ? x : y, lo = x > y ? y : x;
+            v[s] = down ? hi : lo;
+            v[s | j] = down ? lo : hi;
+          }
+        }
+      } else {
+        const int jl = j / KPL;
+        const bool lower = (lane & jl) == 0;
+        const bool down = ((lane * KPL) & kk) == 0;  // kk > j >= KPL: a function of the lane only
+        const bool keep_max = lower == down;
+#pragma unroll
+        for (int s = 0; s < KPL; ++s) {
+          const unsigned long long x = v[s];
+          const unsigned long long y = __shfl_xor(x, jl, 64);
+          const unsigned long long hi = x > y ? x : y, lo = x > y ? y : x;
+          v[s] = keep_max ? hi : lo;
+        }
+      }
+    }
+  }
+}
+
+// Two launches cover a round.  First one wave per query, keys in registers (wave_sort_desc), for the
+// queries with at most SELECT_SMALL entries to rank, which is nearly all of them; then four waves
+// per query with the keys in LDS and room for a full candidate buffer for the rest.  A query ranked
+// by the first launch has its candidate count reset, so the second one skips it.
 constexpr int SELECT_SMALL = 1024;
-template <int NT>
-__global__ void __launch_bounds__(NT) topk_select_kernel(TopkWs w, int k, int rescan) {
+
+__device__ __forceinline__ void select_finish(const TopkWs& w, int64_t b, int k, int rescan, bool over, int new_len,
+                                              bool have_tau, float tau) {
+  w.list_len[b] = new_len;
+  w.tau[b] = have_tau ? tau : __uint_as_float(0xff800000u);
+  w.cnt[b] = 0;
+  if (!rescan) {
+    if (over && !w.dirty[b]) {
+      w.dirty[b] = 1;
+      atomicAdd(w.n_dirty, 1);
+    }
+  } else if (!over) {
+    w.dirty[b] = 0;
+    atomicSub(w.n_dirty, 1);
+  }
+}
+
+template <int KPL>
+__device__ __forceinline__ void select_in_registers(const TopkWs& w, int64_t b, int k, int rescan, int len, int nc,
+                                                    float tau_old, int lane) {
+  unsigned long long v[KPL];
+#pragma unroll
+  for (int s = 0; s < KPL; ++s) {
+    const int i = lane * KPL + s;
+    unsigned long long key = 0;
+    if (i < len) {
+      key = w.list[b * w.kpad + i];
+      if (rescan && ordered_to_f32((uint32_t)(key >> 32)) > tau_old) key = 0;
+    } else if (i < len + nc) {
+      key = w.cand[b * TOPK_CAP + (i - len)];
+    }
+    v[s] = key;
+  }
+  wave_sort_desc<KPL>(v, lane);
+  int valid = 0;
+#pragma unroll
+  for (int s = 0; s < KPL; ++s) valid += v[s] != 0 ? 1 : 0;
+#pragma unroll
+  for (int o = 32; o >= 1; o >>= 1) valid += __shfl_xor(valid, o, 64);
+  const int new_len = valid < k ? valid : k;
+  unsigned long long kth = 0;  // the key at position k - 1, if this wave holds that position
+#pragma unroll
+  for (int s = 0; s < KPL; ++s) {
+    const int i = lane * KPL + s;
+    if (i < new_len) w.list[b * w.kpad + i] = v[s];
+    if (i == k - 1) kth = v[s];
+  }
+#pragma unroll
+  for (int o = 32; o >= 1; o >>= 1) kth |= __shfl_xor(kth, o, 64);  // one lane at most holds it
+  if (lane == 0)
+    select_finish(w, b, k, rescan, false, new_len, new_len == k, ordered_to_f32((uint32_t)(kth >> 32)));
+}
+
+// Merge a query's kept list with this round's candidates, keep the best k, publish the new
+// threshold.  In `rescan` mode (only queries flagged dirty) list entries above the old threshold
+// are dropped first: the rescan finds all of them again.
+__global__ void __launch_bounds__(64) topk_select_wave_kernel(TopkWs w, int k, int rescan) {
+  const int lane = threadIdx.x;
+  const int64_t b = blockIdx.x;
+  if (rescan && !w.dirty[b]) return;
+  const int len = w.list_len[b];
+  const int raw = w.cnt[b];
+  if (raw > TOPK_CAP || len + raw > SELECT_SMALL) return;  // left to topk_select_kernel
+  const float tau_old = w.tau[b];
+  if (len + raw <= 512)
+    select_in_registers<8>(w, b, k, rescan, len, raw, tau_old, lane);
+  else
+    select_in_registers<16>(w, b, k, rescan, len, raw, tau_old, lane);
+}
+
+__global__ void __launch_bounds__(256) topk_select_kernel(TopkWs w, int k, int rescan) {
   extern __shared__ unsigned long long keys[];
   __shared__ int s_valid;
   const int tid = threadIdx.x;
@@ -469,11 +577,11 @@ __global__ void __launch_bounds__(NT) topk_select_kernel(TopkWs w, int k, int re
   const bool over = raw > TOPK_CAP;
   const float tau_old = w.tau[b];
   const int n = len + nc;
-  if ((NT == 64) != (n <= SELECT_SMALL)) return;
+  if (n <= SELECT_SMALL) return;  // ranked by topk_select_wave_kernel (which reset the candidate count)
   int npad = 2;
   while (npad < n) npad <<= 1;
   if (tid == 0) s_valid = 0;
-  for (int i = tid; i < npad; i += NT) {
+  for (int i = tid; i < npad; i += 256) {
     unsigned long long key = 0;
     if (i < len) {
       key = w.list[b * w.kpad + i];
@@ -486,7 +594,7 @@ __global__ void __launch_bounds__(NT) topk_select_kernel(TopkWs w, int k, int re
   __syncthreads();
   for (int kk = 2; kk <= npad; kk <<= 1) {
     for (int j = kk >> 1; j > 0; j >>= 1) {
-      for (int i = tid; i < npad; i += NT) {
+      for (int i = tid; i < npad; i += 256) {
         const int ixj = i ^ j;
         if (ixj > i) {
           const bool down = (i & kk) == 0;
@@ -500,26 +608,14 @@ __global__ void __launch_bounds__(NT) topk_select_kernel(TopkWs w, int k, int re
       __syncthreads();
     }
   }
-  for (int i = tid; i < npad; i += NT)
+  for (int i = tid; i < npad; i += 256)
     if (keys[i] != 0 && (i + 1 == npad || keys[i + 1] == 0)) s_valid = i + 1;
   __syncthreads();
   const int n_valid = s_valid;
   const int new_len = n_valid < k ? n_valid : k;
-  for (int i = tid; i < new_len; i += NT) w.list[b * w.kpad + i] = keys[i];
-  if (tid == 0) {
-    w.list_len[b] = new_len;
-    w.tau[b] = (new_len == k) ? ordered_to_f32((uint32_t)(keys[k - 1] >> 32)) : __uint_as_float(0xff800000u);
-    w.cnt[b] = 0;
-    if (!rescan) {
-      if (over && !w.dirty[b]) {
-        w.dirty[b] = 1;
-        atomicAdd(w.n_dirty, 1);
-      }
-    } else if (!over) {
-      w.dirty[b] = 0;
-      atomicSub(w.n_dirty, 1);
-    }
-  }
+  for (int i = tid; i < new_len; i += 256) w.list[b * w.kpad + i] = keys[i];
+  if (tid == 0)
+    select_finish(w, b, k, rescan, over, new_len, new_len == k, ordered_to_f32((uint32_t)(keys[k - 1] >> 32)));
 }
 
 __global__ void topk_output_kernel(TopkWs w, int64_t B, int k, const float* bias, int apply_sigmoid,
@@ -904,11 +1000,10 @@ extern "C" int kge_topk(const float* Q, const float* bias, const void* E, int dt
 
   // ranks the list (<= k entries) and this round's candidates (<= min(TOPK_CAP, rows scanned) entries) of every query
   auto launch_select = [&](int64_t rows, int rescan) {
-    hipLaunchKernelGGL(topk_select_kernel<64>, dim3((unsigned)B), dim3(64), SELECT_SMALL * sizeof(unsigned long long), st,
-                       ws, (int)k, rescan);
+    hipLaunchKernelGGL(topk_select_wave_kernel, dim3((unsigned)B), dim3(64), 0, st, ws, (int)k, rescan);
     if (k + (rows < TOPK_CAP ? rows : TOPK_CAP) > SELECT_SMALL)  // kpad (<= 1024) + TOPK_CAP, padded to a power of two
-      hipLaunchKernelGGL(topk_select_kernel<256>, dim3((unsigned)B), dim3(256), 8192 * sizeof(unsigned long long), st,
-                         ws, (int)k, rescan);
+      hipLaunchKernelGGL(topk_select_kernel, dim3((unsigned)B), dim3(256), 8192 * sizeof(unsigned long long), st, ws,
+                         (int)k, rescan);
   };
   const int64_t growth = (k <= 256) ? 4 : 2;  // round r scans (growth - 1) x what is already ranked
   int64_t e0 = 0, e1 = (N < TOPK_FIRST_ROWS) ? N : TOPK_FIRST_ROWS;

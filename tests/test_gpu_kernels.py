@@ -245,6 +245,10 @@ TOPK_CASES = [
     ("DistMult", 30000, 9, 128, 70, "int8", 100),
     ("DistMult", 5000, 9, 64, 33, "bf16", 1),
     ("DistMult", 6000, 9, 64, 20, "fp32", 1024),
+    ("DistMult", 700, 9, 64, 20, "fp32", 600),       # k above half of the one-wave select's capacity
+    ("DistMult", 1000, 9, 32, 10, "fp32", 1000),     # k == N
+    ("DistMult", 3000, 5, 64, 40, "bf16", 300),
+    ("ComplEx", 9000, 5, 64, 24, "fp32", 511),
 ]
 
 
