@@ -283,6 +283,7 @@ __global__ void __launch_bounds__(1024) plan_fix_kernel(const int64_t* csr_row, 
 // are formed once (gathered rows, same MFMA chain as the main loop), then every query of the
 // group compares them with its own threshold.
 constexpr int FIX_CAP = 2048;
+constexpr int FIX_ITEMS = 16;  // work items a workgroup resolves side by side
 template <int EDT>
 __global__ void __launch_bounds__(256) filter_fix_kernel(ContractArgs a, FixPlan plan, int64_t b0,
                                                         const int64_t* row_ptr, const int32_t* col,
@@ -296,21 +297,40 @@ __global__ void __launch_bounds__(256) filter_fix_kernel(ContractArgs a, FixPlan
   const int n_work = plan.meta[0];
   const int64_t slice = plan.meta[1];
   const int n_groups = plan.meta[2];
-  for (int w = blockIdx.x; w < n_work; w += gridDim.x) {
-    int lo = 0, hi = n_groups;  // last group whose first work item is <= w
-    while (hi - lo > 1) {
-      const int mid = (lo + hi) >> 1;
-      if (plan.work[2 * mid + 1] <= w) lo = mid; else hi = mid;
+  // This workgroup's work items are w = blockIdx.x + k * gridDim.x.  Up to FIX_ITEMS of them at a time are
+  // resolved by one thread each, side by side (group by binary search, then the group's row and extent),
+  // so that their chains of dependent loads overlap instead of running once per item.
+  __shared__ int32_t it_i0[FIX_ITEMS], it_m[FIX_ITEMS], it_bq[FIX_ITEMS];
+  __shared__ int64_t it_z0[FIX_ITEMS], it_z1[FIX_ITEMS];
+  for (int k0 = 0; blockIdx.x + (int64_t)k0 * gridDim.x < n_work; k0 += FIX_ITEMS) {
+    __syncthreads();
+    if (tid < FIX_ITEMS) {
+      const int64_t w = blockIdx.x + (int64_t)(k0 + tid) * gridDim.x;
+      if (w < n_work) {
+        int lo = 0, hi = n_groups;  // last group whose first work item is <= w
+        while (hi - lo > 1) {
+          const int mid = (lo + hi) >> 1;
+          if (plan.work[2 * mid + 1] <= w) lo = mid; else hi = mid;
+        }
+        const int i0 = plan.work[2 * lo];
+        const int64_t z = w - plan.work[2 * lo + 1];
+        const unsigned long long key = plan.skey[i0];
+        const int64_t row = (int64_t)(key >> 24);
+        const int64_t L0 = row_ptr[row], L1 = row_ptr[row + 1];
+        const int64_t z0 = L0 + z * slice;
+        it_i0[tid] = i0;
+        it_m[tid] = plan.gend[i0] - i0;
+        it_bq[tid] = (int32_t)(key & 0xffffffull);
+        it_z0[tid] = z0;
+        it_z1[tid] = (z0 + slice < L1) ? z0 + slice : L1;
+      }
     }
-    const int i0 = plan.work[2 * lo];
-    const int64_t z = w - plan.work[2 * lo + 1];
-    const unsigned long long key = plan.skey[i0];
-    const int64_t row = (int64_t)(key >> 24);
-    const int m = plan.gend[i0] - i0;
-    const int64_t L0 = row_ptr[row], L1 = row_ptr[row + 1];
-    const int64_t z0 = L0 + z * slice;
-    const int64_t z1 = (z0 + slice < L1) ? z0 + slice : L1;
-    const int64_t bq = b0 + (int64_t)(key & 0xffffffull);
+    __syncthreads();
+  for (int kk = 0; kk < FIX_ITEMS && blockIdx.x + (int64_t)(k0 + kk) * gridDim.x < n_work; ++kk) {
+    const int i0 = it_i0[kk];
+    const int m = it_m[kk];
+    const int64_t z0 = it_z0[kk], z1 = it_z1[kk];
+    const int64_t bq = b0 + (int64_t)it_bq[kk];
     // threads per member in the compare phase: spread a small group over the whole workgroup
     int tpm = 1;
     while (tpm * 2 * m <= 256) tpm *= 2;
@@ -392,6 +412,7 @@ __global__ void __launch_bounds__(256) filter_fix_kernel(ContractArgs a, FixPlan
         __syncthreads();
       }
     }
+  }
   }
 }
 
