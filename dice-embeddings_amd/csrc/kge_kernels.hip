@@ -663,24 +663,26 @@ __global__ void bce_init_kernel(double* sums) {
   if (threadIdx.x < 3) sums[threadIdx.x] = 0.0;
 }
 
-// sum of the logits of the positive (query, tail) pairs: one wave per query
+// sum of the logits of the positive (query, tail) pairs.  A workgroup strides over the queries; its four
+// waves take a row's positives in turn, the lanes of a wave split the embedding dimension.  One atomic per
+// workgroup at the end: thousands of double-precision atomics on one address would serialise.
 template <int EDT>
 __global__ void __launch_bounds__(256) bce_pos_kernel(ContractArgs a, const float* bias, const int64_t* csr_row,
                                                      const int64_t* row_ptr, const int32_t* col, int64_t n_rows,
                                                      double* sums) {
+  __shared__ double s_part[4];
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
-  const int64_t q = (int64_t)blockIdx.x * 4 + wave;
-  if (q >= a.B) return;
-  const int64_t row = csr_row[q];
-  double local = 0.0;
-  if (row >= 0 && row < n_rows) {
+  double local = 0.0;  // every lane of a wave holds the same sum
+  for (int64_t q = blockIdx.x; q < a.B; q += gridDim.x) {
+    const int64_t row = csr_row[q];
+    if (row < 0 || row >= n_rows) continue;
     const float bq = bias ? bias[q] : 0.f;
     const float* qv = a.Q + q * a.d;
-    for (int64_t j = row_ptr[row] + lane; j < row_ptr[row + 1]; j += 64) {
+    for (int64_t j = row_ptr[row] + wave; j < row_ptr[row + 1]; j += 4) {
       const int64_t e = col[j];
-      if (e < 0 || e >= a.N) continue;
+      if (e < 0 || e >= a.N) continue;  // uniform across the wave
       float dot = 0.f;
-      for (int k = 0; k < a.d; ++k) {
+      for (int k = lane; k < a.d; k += 64) {
         float x;
         float qk = qv[k];
         if (EDT == KGE_F32) {
@@ -694,13 +696,18 @@ __global__ void __launch_bounds__(256) bce_pos_kernel(ContractArgs a, const floa
         }
         dot = fmaf(qk, x, dot);
       }
+#pragma unroll
+      for (int o = 32; o >= 1; o >>= 1) dot += __shfl_xor(dot, o, 64);
       if (EDT == KGE_I8) dot *= a.scale[e];
       local += (double)(dot + bq);
     }
   }
-#pragma unroll
-  for (int o = 32; o >= 1; o >>= 1) local += __shfl_xor(local, o, 64);
-  if (lane == 0 && local != 0.0) atomicAdd(&sums[2], local);
+  if (lane == 0) s_part[wave] = local;
+  __syncthreads();
+  if (tid == 0) {
+    const double t = s_part[0] + s_part[1] + s_part[2] + s_part[3];
+    if (t != 0.0) atomicAdd(&sums[2], t);
+  }
 }
 
 __global__ void bce_final_kernel(const double* sums, double B, double N, float eps, float* loss) {
@@ -1086,7 +1093,7 @@ extern "C" int kge_bce_multihot(const float* Q, const float* bias, const void* E
   rc = launch_contract<BceEpi>(dtype, a, ea, st, "kge_bce_multihot");
   if (rc) return rc;
   if (csr_row && n_rows > 0) {
-    dim3 grid((unsigned)((B + 3) / 4)), block(256);
+    dim3 grid((unsigned)(B < 512 ? B : 512)), block(256);
     KGE_DISPATCH_DTYPE(dtype, bce_pos_kernel, grid, block, 0, st, a, bias, csr_row, row_ptr, col, n_rows, sums);
     KGE_LAUNCH_CHECK("bce_pos_kernel");
   }
