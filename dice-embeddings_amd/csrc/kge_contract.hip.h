@@ -347,9 +347,10 @@ struct TopkEpi {
   }
 };
 
+constexpr int BCE_SLOTS = 128;  // the accumulator is spread: same-address double atomics serialise
 struct BceArgs {
   const float* bias;
-  double* sums;  // [0] sum softplus(s), [1] sum s
+  double* sums;  // [0, BCE_SLOTS) partial sums of softplus(s), [BCE_SLOTS, 2 BCE_SLOTS) partial sums of s
   int32_t want_s;
 };
 template <int NQT>
@@ -404,8 +405,9 @@ struct BceEpi {
       y += __shfl_xor(y, o, 64);
     }
     if ((threadIdx.x & 63) == 0) {
-      atomicAdd(&a.sums[0], x);
-      if (a.want_s) atomicAdd(&a.sums[1], y);
+      const int slot = (int)((blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6)) & (BCE_SLOTS - 1));
+      atomicAdd(&a.sums[slot], x);
+      if (a.want_s) atomicAdd(&a.sums[BCE_SLOTS + slot], y);
     }
   }
 };

@@ -659,8 +659,9 @@ __global__ void topk_output_kernel(TopkWs w, int64_t B, int k, const float* bias
 }
 
 // ---- BCE helpers --------------------------------------------------------------------------------
+// accumulators: BCE_SLOTS partial sums of softplus(s), BCE_SLOTS of s, then the sum over the positives
 __global__ void bce_init_kernel(double* sums) {
-  if (threadIdx.x < 3) sums[threadIdx.x] = 0.0;
+  for (int i = threadIdx.x; i < 2 * BCE_SLOTS + 1; i += blockDim.x) sums[i] = 0.0;
 }
 
 // sum of the logits of the positive (query, tail) pairs.  A workgroup strides over the queries; its four
@@ -706,17 +707,22 @@ __global__ void __launch_bounds__(256) bce_pos_kernel(ContractArgs a, const floa
   __syncthreads();
   if (tid == 0) {
     const double t = s_part[0] + s_part[1] + s_part[2] + s_part[3];
-    if (t != 0.0) atomicAdd(&sums[2], t);
+    if (t != 0.0) atomicAdd(&sums[2 * BCE_SLOTS], t);
   }
 }
 
 __global__ void bce_final_kernel(const double* sums, double B, double N, float eps, float* loss) {
   if (threadIdx.x == 0 && blockIdx.x == 0) {
-    double t = sums[0];
+    double t = 0.0, s = 0.0;
+    for (int i = 0; i < BCE_SLOTS; ++i) {
+      t += sums[i];
+      s += sums[BCE_SLOTS + i];
+    }
+    const double pos = sums[2 * BCE_SLOTS];
     if (eps != 0.f)
-      t -= (1.0 - (double)eps) * sums[2] + sums[1] / N;
+      t -= (1.0 - (double)eps) * pos + s / N;
     else
-      t -= sums[2];
+      t -= pos;
     loss[0] = (float)(t / (B * N));
   }
 }
@@ -1069,7 +1075,7 @@ extern "C" int kge_topk(const float* Q, const float* bias, const void* E, int dt
   return KGE_OK;
 }
 
-extern "C" size_t kge_bce_workspace_bytes(void) { return 256; }
+extern "C" size_t kge_bce_workspace_bytes(void) { return (2 * BCE_SLOTS + 1) * sizeof(double) + 248; }
 
 extern "C" int kge_bce_multihot(const float* Q, const float* bias, const void* E, int dtype, const float* scale,
                                 int64_t B, int64_t d, int64_t N, const int64_t* csr_row, const int64_t* row_ptr,
@@ -1086,7 +1092,7 @@ extern "C" int kge_bce_multihot(const float* Q, const float* bias, const void* E
   KGE_REQUIRE(((uintptr_t)workspace & 7) == 0, KGE_ERR_WORKSPACE, "kge_bce_multihot: workspace must be 8-byte aligned");
   hipStream_t st = (hipStream_t)stream;
   double* sums = (double*)workspace;
-  hipLaunchKernelGGL(bce_init_kernel, dim3(1), dim3(64), 0, st, sums);
+  hipLaunchKernelGGL(bce_init_kernel, dim3(1), dim3(256), 0, st, sums);
   KGE_LAUNCH_CHECK("bce_init_kernel");
   ContractArgs a = make_args(Q, E, dtype, scale, B, d, N, 0, N);
   BceArgs ea{bias, sums, label_smoothing != 0.f ? 1 : 0};
