@@ -128,6 +128,27 @@ __global__ void __launch_bounds__(256) target_score_kernel(ContractArgs a, const
   }
 }
 
+// ---- score of one given entity per query (forward_triples): the same chain, nothing else ----------
+template <int EDT>
+__global__ void __launch_bounds__(256) triple_score_kernel(ContractArgs a, const int64_t* target, const float* bias,
+                                                          float* out) {
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, c = lane & 31, hf = lane >> 5;
+  const int64_t q = ((int64_t)blockIdx.x * 4 + wave) * 32 + c;
+  const int64_t t = (q < a.B) ? target[q] : -1;
+  const bool ok = t >= 0 && t < a.N;
+  f32x16 acc = chain_direct<EDT>(a.E, a.d, ok ? t : -1, a.Q, (q < a.B) ? q : -1, hf);
+  const int isel = ((c >> 3) << 2) | (c & 3);  // diagonal element (entity row c, query column c)
+  float v = 0.f;
+#pragma unroll
+  for (int i = 0; i < 16; ++i)
+    if (i == isel) v = acc[i];
+  if (hf == ((c >> 2) & 1) && q < a.B) {
+    float raw = __uint_as_float(0x7fc00000u);  // NaN for an id outside the table
+    if (ok) raw = (EDT == KGE_I8) ? v * a.scale[t] : v;
+    out[q] = raw + (bias ? bias[q] : 0.f);
+  }
+}
+
 // ---- (head, relation) -> filter row: binary search in the sorted key array -----------------------
 __global__ void csr_lookup_kernel(const int64_t* hr, int64_t B, const int64_t* keys, int64_t n_rows,
                                   int64_t num_relations, int64_t* csr_row) {
@@ -943,6 +964,21 @@ extern "C" int kge_scores(const float* Q, const float* bias, const void* E, int 
   ContractArgs a = make_args(Q, E, dtype, scale, B, d, N, 0, N);
   StoreArgs ea{S, bias, ldS};
   return launch_contract<StoreEpi>(dtype, a, ea, (hipStream_t)stream, "kge_scores");
+}
+
+extern "C" int kge_triple_scores(const float* Q, const float* bias, const void* E, int dtype, const float* scale,
+                                 int64_t B, int64_t d, int64_t N, const int64_t* entity, float* out, void* stream) {
+  clear_error();
+  int rc = check_contract("kge_triple_scores", Q, E, dtype, scale, B, d, N);
+  if (rc) return rc;
+  if (B == 0) return KGE_OK;
+  KGE_REQUIRE(entity && out, KGE_ERR_INVALID, "kge_triple_scores: null entity or output pointer");
+  ContractArgs a = make_args(Q, E, dtype, scale, B, d, N, 0, N);
+  dim3 grid((unsigned)((B + 127) / 128)), block(256);
+  hipStream_t st = (hipStream_t)stream;
+  KGE_DISPATCH_DTYPE(dtype, triple_score_kernel, grid, block, 0, st, a, entity, bias, out);
+  KGE_LAUNCH_CHECK("triple_score_kernel");
+  return KGE_OK;
 }
 
 extern "C" int kge_csr_lookup(const int64_t* hr, int64_t B, const int64_t* keys, int64_t n_rows,

@@ -23,7 +23,8 @@ from .csr import FilterCSR  # noqa: F401
 from .models import DistMult, ComplEx, QMult, Keci, CKeci, MODEL_REGISTRY, initialize_model  # noqa: F401
 from .evaluator import Evaluator, compute_metrics_from_ranks_simple  # noqa: F401
 from .kge import KGE  # noqa: F401
-from .link_prediction import evaluate_lp  # noqa: F401
+from .link_prediction import (evaluate_lp, evaluate_link_prediction_performance,  # noqa: F401
+                              evaluate_link_prediction_performance_with_reciprocals)
 from .loader import load_model, load_splits, evaluate_experiment, save_experiment  # noqa: F401
 
 __version__ = "0.1.0"

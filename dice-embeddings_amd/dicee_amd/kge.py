@@ -130,8 +130,22 @@ class KGE:
         elif t is None:
             scores = self.predict_missing_tail_entity(h, r, within)
         else:
-            raise NotImplementedError("triple_score is outside the accelerated path")
+            scores = self.triple_score(h, r, t, logits=True).cpu()
         return scores if logits else torch.sigmoid(scores)
+
+    def triple_score(self, h: Union[List[str], str] = None, r: Union[List[str], str] = None,
+                     t: Union[List[str], str] = None, logits=False) -> torch.FloatTensor:
+        """Score (sigmoid unless ``logits``) of the given triples; lists are taken element-wise (:581-650)."""
+        if isinstance(h, list) and isinstance(r, list) and isinstance(t, list):
+            hh = [self.entity_to_idx[i] for i in h]
+            rr = [self.relation_to_idx[i] for i in r]
+            tt = [self.entity_to_idx[i] for i in t]
+        else:
+            hh, rr, tt = [self.entity_to_idx[h]], [self.relation_to_idx[r]], [self.entity_to_idx[t]]
+        x = torch.stack([torch.LongTensor(hh), torch.LongTensor(rr), torch.LongTensor(tt)], dim=1)
+        with torch.no_grad():
+            s = self.model(x.to(self.model.entity_embeddings.weight.device))
+        return s if logits else torch.sigmoid(s)
 
     def predict_topk(self, *, h: Union[str, List[str]] = None, r: Union[str, List[str]] = None,
                      t: Union[str, List[str]] = None, topk: int = 10, within: List[str] = None,

@@ -71,3 +71,59 @@ def evaluate_lp(model, triple_idx, num_entities=None, er_vocab=None, re_vocab=No
     if info:
         print(results)
     return (results, (hr_, tr_)) if return_ranks else results
+
+
+def _ids_of_string_triples(model, triples):
+    e2i, r2i = model.entity_to_idx, model.relation_to_idx
+    return np.array([[e2i[s_], r2i[p_], e2i[o_]] for s_, p_, o_ in triples], dtype=np.int64).reshape(-1, 3)
+
+
+def _csr_of_string_vocab(vocab, first, second, values, key_mult, device):
+    """``vocab``: dict (str, str) -> list of str, as dicee stores vocabularies of string triples; ``first`` /
+    ``second`` / ``values`` are the str -> id maps of the key's two parts and of the list entries."""
+    ids = {(first[a], second[b]): [values[v] for v in vs] for (a, b), vs in vocab.items()}
+    return FilterCSR.from_er_vocab(ids, key_mult).to(device)
+
+
+@torch.no_grad()
+def evaluate_link_prediction_performance_with_reciprocals(model, triples, er_vocab, tie="stable"):
+    """Tail-only filtered evaluation of string triples for models trained with reciprocal relations
+    (dicee/evaluation/link_prediction.py:116-174).  ``model``: a ``KGE`` (``.model``, ``.entity_to_idx``,
+    ``.relation_to_idx``); ``er_vocab``: (head str, relation str) -> list of tail strs.  Batches of
+    ``model.model.args["batch_size"]`` triples, one fused rank call each."""
+    from .evaluator import compute_metrics_from_ranks_simple, create_hits_dict, ALL_HITS_RANGE
+    net = model.model
+    net.eval()
+    dev = net.entity_embeddings.weight.device
+    ids = _ids_of_string_triples(model, triples)
+    csr = _csr_of_string_vocab(er_vocab, model.entity_to_idx, model.relation_to_idx, model.entity_to_idx,
+                               net.num_relations, dev)
+    trip = torch.from_numpy(ids).to(dev)
+    n = len(ids)
+    bs = int(net.args.get("batch_size", 1024) or 1024)
+    out = torch.empty((n,), dtype=torch.int64, device=dev)
+    for i in range(0, n, bs):
+        b = trip[i:i + bs]
+        c = net.rank_filtered(b[:, :2].contiguous(), b[:, 2].contiguous(), csr)
+        out[i:i + bs] = ranks_from_counts(c["n_greater"], c["n_equal"], c["n_equal_lower"], tie)
+    ranks = out.cpu().numpy()
+    assert len(triples) == len(ranks) == n
+    hits = create_hits_dict()
+    for level in ALL_HITS_RANGE:
+        hits[level] = [1.0] * int(np.count_nonzero(ranks <= level))
+    return compute_metrics_from_ranks_simple(ranks, n, hits)
+
+
+@torch.no_grad()
+def evaluate_link_prediction_performance(model, triples, er_vocab, re_vocab, tie="stable"):
+    """Head and tail filtered evaluation of string triples (dicee/evaluation/link_prediction.py:22-113):
+    ``er_vocab`` (head str, relation str) -> tails, ``re_vocab`` (relation str, tail str) -> heads."""
+    net = model.model
+    dev = net.entity_embeddings.weight.device
+    ids = _ids_of_string_triples(model, triples)
+    er = _csr_of_string_vocab(er_vocab, model.entity_to_idx, model.relation_to_idx, model.entity_to_idx,
+                              net.num_relations, dev)
+    re = _csr_of_string_vocab(re_vocab, model.relation_to_idx, model.entity_to_idx, model.entity_to_idx,
+                              net.num_entities, dev)
+    return evaluate_lp(net, ids, net.num_entities, er, re, info=None, batch_size=int(net.args.get("batch_size", 1024) or 1024),
+                       tie=tie)

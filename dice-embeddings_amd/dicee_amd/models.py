@@ -115,13 +115,13 @@ class BaseKGE(torch.nn.Module):
 
     # ------------------------------------------------------------------ reference call surface
     def forward(self, x, y_idx=None):
-        """Shape dispatch of BaseKGE.forward (base_model.py:310-344); only the KvsAll case is built."""
+        """Shape dispatch of BaseKGE.forward (base_model.py:310-344): [B,2] -> KvsAll scores, [n,3] -> triple scores."""
         if isinstance(x, tuple):
             raise NotImplementedError("forward_k_vs_sample is outside the accelerated path")
         if x.dim() == 2 and x.shape[1] == 2:
             return self.forward_k_vs_all(x=x)
         if x.dim() == 2 and x.shape[1] == 3:
-            raise NotImplementedError("forward_triples is outside the accelerated path")
+            return self.forward_triples(x)
         raise NotImplementedError("byte-pair-encoded inputs are outside the accelerated path")
 
     def forward_k_vs_all(self, x):
@@ -129,6 +129,14 @@ class BaseKGE(torch.nn.Module):
         Q, bias = self.query(x)
         E, scale = self.table()
         return ops.scores(Q, bias, E, scale)
+
+    def forward_triples(self, x):
+        """[n] fp32 scores of the triples ``x`` [n,3] = (h, r, t) (base_model.py:346-362): the query of (h, r)
+        against the one row E[t], with the reduction order of the KvsAll kernels."""
+        E, scale = self.table()
+        x = x.to(device=E.device, dtype=torch.int64)
+        Q, bias = self.query(x[:, :2].contiguous())
+        return ops.triple_scores(Q, bias, E, scale, x[:, 2].contiguous())
 
     def forward_all_heads(self, rt):
         """[B,N] fp32: score(x, r, t) of every entity x as head, for ``rt`` [B,2] = (relation, tail) pairs."""

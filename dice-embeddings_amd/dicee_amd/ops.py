@@ -83,6 +83,20 @@ def scores(Q, bias, E, scale=None, out=None):
     return out
 
 
+def triple_scores(Q, bias, E, scale, entity):
+    """out[b] = Q[b] . E[entity[b]] (* scale) + bias[b]: the score of one given entity per query."""
+    lib = _lib.load()
+    _require_gpu(Q, bias, E, scale, entity)
+    if entity.dtype != torch.int64:
+        raise TypeError("entity must be int64")
+    B, d = Q.shape
+    out = torch.empty((B,), dtype=torch.float32, device=Q.device)
+    rc = lib.kge_triple_scores(_ptr(Q), _ptr(bias), _ptr(E), _table_dtype(E), _ptr(scale), B, d, E.shape[0],
+                               _ptr(entity), _ptr(out), _stream())
+    _lib.check(rc)
+    return out
+
+
 def csr_lookup(hr, keys, num_relations):
     """CSR row of every (h, r) pair of ``hr`` [B,2] in the sorted key array ``keys``; -1 if unknown."""
     lib = _lib.load()

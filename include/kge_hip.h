@@ -110,6 +110,18 @@ int kge_scores(const float* Q, const float* bias, const void* E, int dtype, cons
                int64_t B, int64_t d, int64_t N, float* S, int64_t ldS, void* stream);
 
 /*
+ * Score of ONE given entity per query: out[b] = dot(Q[b], E[entity[b]]) (* scale) (+ bias[b]), formed
+ * with the reduction order of the contraction kernels (the same bits as S[b, entity[b]] of kge_scores).
+ * With kge_build_query on the (head, relation) columns and the tails as `entity` this is
+ * forward_triples for the four models (BaseKGE.forward_triples dicee/models/base_model.py:346-362
+ * with DistMult.score dicee/models/real.py:48-49, ComplEx.score dicee/models/complex.py:229-238,
+ * QMult.score dicee/models/quaternion.py:102-122, Keci.forward_triples dicee/models/clifford.py:501-561;
+ * for Keci with p > 0 see kge_build_query_head).  entity ids outside [0, N) give NaN.
+ */
+int kge_triple_scores(const float* Q, const float* bias, const void* E, int dtype, const float* scale,
+                      int64_t B, int64_t d, int64_t N, const int64_t* entity, float* out, void* stream);
+
+/*
  * Filter row of every (head, relation) pair: csr_row[b] = index of key hr[b,0]*num_relations + hr[b,1]
  * in `keys` (sorted, unique, int64 [n_rows]: the CSR's row order), or -1 if the pair has no known
  * tails.  Replaces the dict lookup `self.er_vocab[(id_e, id_r)]` of

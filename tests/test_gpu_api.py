@@ -304,3 +304,64 @@ def test_predict_missing_head():
     kge2 = KGE(model=m, entity_to_idx=ents, relation_to_idx=rels2)
     assert kge2.all_have_inverse
     assert kge2.predict_topk(r=["r3"], t=["e10"], topk=4) == kge2.predict_topk(h=["e10"], r=["r3_inverse"], topk=4)
+
+
+@pytest.mark.parametrize("name,d,extra", [("DistMult", 32, {}), ("ComplEx", 32, {}), ("QMult", 32, {}),
+                                          ("Keci", 30, {"p": 2, "q": 2})])
+def test_forward_triples_and_triple_score(name, d, extra):
+    from dicee_amd import KGE
+    m, triples = _toy(name, d, n=400, seed=31, **extra)
+    E = m.entity_embeddings.weight.detach().numpy().copy()
+    Rel = m.relation_embeddings.weight.detach().numpy().copy()
+    kw = _oracle_kw(m)
+    m = m.to("cuda").eval()
+    x = torch.from_numpy(triples).cuda()
+    with torch.no_grad():
+        s = m(x)                                                   # three columns -> forward_triples
+    assert s.shape == (400,) and s.dtype == torch.float32
+    ref = ko.triple_scores(name, E, Rel, triples, **kw)
+    assert np.abs(s.cpu().numpy() - ref).max() <= 1e-5 * np.sqrt((ref ** 2).mean()) + 1e-7
+    # the same bits as the matching column of the KvsAll scores
+    S = m(x[:, :2].contiguous())
+    assert torch.equal(S[torch.arange(400), x[:, 2]], s)
+    ents = {f"e{i}": i for i in range(135)}
+    rels = {f"r{i}": i for i in range(46)}
+    kge = KGE(model=m, entity_to_idx=ents, relation_to_idx=rels)
+    h, r, t = (int(v) for v in triples[7])
+    one = kge.triple_score(f"e{h}", f"r{r}", f"e{t}")
+    assert one.shape == (1,) and abs(float(one) - float(ko.sigmoid(ref[7:8])[0])) <= 1e-6
+    many = kge.triple_score([f"e{a}" for a in triples[:5, 0]], [f"r{a}" for a in triples[:5, 1]],
+                            [f"e{a}" for a in triples[:5, 2]], logits=True)
+    assert torch.equal(many, s[:5])
+    assert torch.allclose(kge.predict(h=[f"e{h}"], r=[f"r{r}"], t=[f"e{t}"]), s[7:8].cpu())
+    with pytest.raises(KeyError):
+        kge.triple_score("nobody", "r0", "e1")
+
+
+def test_string_triple_evaluators():
+    from dicee_amd import (KGE, evaluate_lp, evaluate_link_prediction_performance,
+                           evaluate_link_prediction_performance_with_reciprocals)
+    m, triples = _toy("ComplEx", 32, n=900, seed=33, batch_size=64)
+    ents = {f"e{i}": i for i in range(135)}
+    rels = {f"r{i}": i for i in range(46)}
+    m = m.to("cuda")
+    kge = KGE(model=m, entity_to_idx=ents, relation_to_idx=rels)
+    strs = [(f"e{h}", f"r{r}", f"e{t}") for h, r, t in triples]
+    er_s, re_s = {}, {}
+    for h, r, t in strs:
+        er_s.setdefault((h, r), []).append(t)
+        re_s.setdefault((r, t), []).append(h)
+    test = strs[600:]
+    both = evaluate_link_prediction_performance(kge, test, er_s, re_s)
+    want = evaluate_lp(m, triples[600:], 135, ko.vocab(triples, "er"), ko.vocab(triples, "re"), info=None, batch_size=64)
+    assert both == want
+    tails = evaluate_link_prediction_performance_with_reciprocals(kge, test, er_s)
+    from dicee_amd import Evaluator
+    ev = Evaluator(SimpleNamespace(batch_size=64, eval_model="test", scoring_technique="KvsAll", full_storage_path=None))
+    ev.set_filter(ko.vocab(triples, "er"), 46)
+    want_t = ev.evaluate_lp_k_vs_all(m, triples[600:])
+    assert set(tails) == {"H@1", "H@3", "H@10", "MRR"}
+    for key in tails:
+        assert tails[key] == pytest.approx(want_t[key])
+    with pytest.raises(KeyError):
+        evaluate_link_prediction_performance_with_reciprocals(kge, [("e1", "r1", "stranger")], er_s)

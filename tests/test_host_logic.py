@@ -134,8 +134,10 @@ def test_models_mirror_reference_parameters_and_have_no_cpu_fallback():
     d = models.DistMult({"model": "DistMult", "embedding_dim": 8, "num_entities": 5, "num_relations": 2})
     with pytest.raises(RuntimeError):
         d(torch.zeros((2, 2), dtype=torch.int64))                  # CPU tensors: refuses, never falls back
+    with pytest.raises(RuntimeError):
+        d(torch.zeros((2, 3), dtype=torch.int64))                  # forward_triples: the same rule
     with pytest.raises(NotImplementedError):
-        d(torch.zeros((2, 3), dtype=torch.int64))
+        d(torch.zeros((2, 3, 4), dtype=torch.int64))               # byte-pair-encoded input
 
 
 def test_synthetic_configs_small_scale():
