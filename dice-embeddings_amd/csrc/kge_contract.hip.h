@@ -412,6 +412,65 @@ struct BceEpi {
   }
 };
 
+// Smallest and largest raw score of every query over all entities (the per-row min-max
+// normalisation of ensemble evaluation needs them before any score can be combined).
+struct MinMaxArgs {
+  uint32_t* kmin;  // [B] order-preserving keys (f32_to_ordered), combined with atomicMin
+  uint32_t* kmax;  // [B] combined with atomicMax
+};
+template <int NQT>
+struct MinMaxEpi {
+  static constexpr bool SWAP = false;
+  static constexpr bool STAGE_HOOK = false;
+  struct Shared {
+    int unused;
+  };
+  __device__ void bind(Shared*) {}
+  __device__ void stage_end() {}
+  using Args = MinMaxArgs;
+  Args a;
+  float lo[NQT], hi[NQT];
+  int64_t q0, B;
+  int c, hf;
+  __device__ void init(const Args& args, int64_t q0_, int c_, int hf_, int64_t B_) {
+    a = args; q0 = q0_; c = c_; hf = hf_; B = B_;
+#pragma unroll
+    for (int t = 0; t < NQT; ++t) {
+      lo[t] = __uint_as_float(0x7f800000u);
+      hi[t] = __uint_as_float(0xff800000u);
+    }
+  }
+  template <bool HAS_SCALE>
+  __device__ __forceinline__ void tile(int qt, const f32x16& acc, const float* sc16, float sc_col, int64_t e_base,
+                                       int64_t limit) {
+    const bool full = e_base + 32 <= limit;  // uniform
+    float l = lo[qt], h = hi[qt];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const float s = HAS_SCALE ? acc[i] * sc16[i] : acc[i];
+      if (full || e_base + row_of(i, hf) < limit) {
+        l = __builtin_fminf(l, s);
+        h = __builtin_fmaxf(h, s);
+      }
+    }
+    lo[qt] = l;
+    hi[qt] = h;
+  }
+  __device__ void finish() {
+#pragma unroll
+    for (int t = 0; t < NQT; ++t) {
+      // the two halves of the wave hold different entity rows of the same query
+      const float l = __builtin_fminf(lo[t], __shfl_xor(lo[t], 32, 64));
+      const float h = __builtin_fmaxf(hi[t], __shfl_xor(hi[t], 32, 64));
+      const int64_t q = q0 + 32 * t + c;
+      if (hf == 0 && q < B && l <= h) {
+        atomicMin(&a.kmin[q], f32_to_ordered(l));
+        atomicMax(&a.kmax[q], f32_to_ordered(h));
+      }
+    }
+  }
+};
+
 #ifdef KGE_DEBUG
 // Measurement-only epilogue: keeps the accumulators alive with two VALU ops per tile.
 struct NullArgs {

@@ -679,6 +679,23 @@ __global__ void topk_output_kernel(TopkWs w, int64_t B, int k, const float* bias
   out_idx[i] = e;
 }
 
+// ---- row minimum / maximum ----------------------------------------------------------------------
+__global__ void minmax_init_kernel(uint32_t* kmin, uint32_t* kmax, int64_t B) {
+  const int64_t b = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (b < B) {
+    kmin[b] = 0xffffffffu;
+    kmax[b] = 0u;
+  }
+}
+__global__ void minmax_final_kernel(uint32_t* kmin, uint32_t* kmax, const float* bias, int64_t B) {
+  const int64_t b = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (b < B) {
+    const float add = bias ? bias[b] : 0.f;
+    ((float*)kmin)[b] = ordered_to_f32(kmin[b]) + add;
+    ((float*)kmax)[b] = ordered_to_f32(kmax[b]) + add;
+  }
+}
+
 // ---- BCE helpers --------------------------------------------------------------------------------
 // accumulators: BCE_SLOTS partial sums of softplus(s), BCE_SLOTS of s, then the sum over the positives
 __global__ void bce_init_kernel(double* sums) {
@@ -1108,6 +1125,28 @@ extern "C" int kge_topk(const float* Q, const float* bias, const void* E, int dt
   hipLaunchKernelGGL(topk_output_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, ws, B, (int)k, bias,
                      apply_sigmoid, out_scores, out_idx);
   KGE_LAUNCH_CHECK("topk_output_kernel");
+  return KGE_OK;
+}
+
+extern "C" int kge_row_minmax(const float* Q, const float* bias, const void* E, int dtype, const float* scale,
+                              int64_t B, int64_t d, int64_t N, float* out_min, float* out_max, void* stream) {
+  clear_error();
+  int rc = check_contract("kge_row_minmax", Q, E, dtype, scale, B, d, N);
+  if (rc) return rc;
+  if (B == 0) return KGE_OK;
+  KGE_REQUIRE(out_min && out_max && out_min != out_max, KGE_ERR_INVALID, "kge_row_minmax: null or aliased output pointers");
+  hipStream_t st = (hipStream_t)stream;
+  uint32_t* kmin = (uint32_t*)out_min;  // the outputs hold order-preserving keys until the last kernel
+  uint32_t* kmax = (uint32_t*)out_max;
+  const dim3 g1((unsigned)((B + 255) / 256)), b1(256);
+  hipLaunchKernelGGL(minmax_init_kernel, g1, b1, 0, st, kmin, kmax, B);
+  KGE_LAUNCH_CHECK("minmax_init_kernel");
+  ContractArgs a = make_args(Q, E, dtype, scale, B, d, N, 0, N);
+  MinMaxArgs ea{kmin, kmax};
+  rc = launch_contract<MinMaxEpi>(dtype, a, ea, st, "kge_row_minmax");
+  if (rc) return rc;
+  hipLaunchKernelGGL(minmax_final_kernel, g1, b1, 0, st, kmin, kmax, bias, B);
+  KGE_LAUNCH_CHECK("minmax_final_kernel");
   return KGE_OK;
 }
 

@@ -8,6 +8,7 @@ this package is the thin Python side that mirrors the reference's call surface:
                  ``k_vs_all_score`` (dicee/models/*.py)
 * ``evaluator``  ``Evaluator.evaluate_lp_k_vs_all`` (dicee/evaluation/evaluator.py:394-510)
 * ``link_prediction``  ``evaluate_lp``: head and tail direction (dicee/evaluation/link_prediction.py:351-473)
+* ``ensemble``   ``evaluate_ensemble_link_prediction_performance`` (dicee/evaluation/ensemble.py:20-135)
 * ``kge``        ``KGE.predict_topk`` / ``predict`` / ``predict_missing_tail_entity``
                  (dicee/knowledge_graph_embeddings.py:314-579)
 * ``csr``        the known-answer filter as a CSR (dicee's ``er_vocab``)
@@ -23,6 +24,7 @@ from .csr import FilterCSR  # noqa: F401
 from .models import DistMult, ComplEx, QMult, Keci, CKeci, MODEL_REGISTRY, initialize_model  # noqa: F401
 from .evaluator import Evaluator, compute_metrics_from_ranks_simple  # noqa: F401
 from .kge import KGE  # noqa: F401
+from .ensemble import evaluate_ensemble_link_prediction_performance  # noqa: F401
 from .link_prediction import (evaluate_lp, evaluate_link_prediction_performance,  # noqa: F401
                               evaluate_link_prediction_performance_with_reciprocals)
 from .loader import load_model, load_splits, evaluate_experiment, save_experiment  # noqa: F401

@@ -43,6 +43,7 @@ SIGNATURES = {
                           _vp]),
     "kge_profile_begin": (_c_int, []),
     "kge_profile_end": (_c_int, [ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_int64)]),
+    "kge_row_minmax": (_c_int, [_vp, _vp, _vp, _c_int, _vp, _c_i64, _c_i64, _c_i64, _vp, _vp, _vp]),
     "kge_bce_workspace_bytes": (_sz, []),
     "kge_bce_multihot": (_c_int, [_vp, _vp, _vp, _c_int, _vp, _c_i64, _c_i64, _c_i64, _vp, _vp, _vp, _c_i64, _c_f,
                                   _vp, _vp, _sz, _vp]),

@@ -97,6 +97,19 @@ def triple_scores(Q, bias, E, scale, entity):
     return out
 
 
+def row_minmax(Q, bias, E, scale=None):
+    """(min [B], max [B]) of every query's scores over all entities, without the [B,N] matrix."""
+    lib = _lib.load()
+    _require_gpu(Q, bias, E, scale)
+    B, d = Q.shape
+    lo = torch.empty((B,), dtype=torch.float32, device=Q.device)
+    hi = torch.empty((B,), dtype=torch.float32, device=Q.device)
+    rc = lib.kge_row_minmax(_ptr(Q), _ptr(bias), _ptr(E), _table_dtype(E), _ptr(scale), B, d, E.shape[0], _ptr(lo),
+                            _ptr(hi), _stream())
+    _lib.check(rc)
+    return lo, hi
+
+
 def csr_lookup(hr, keys, num_relations):
     """CSR row of every (h, r) pair of ``hr`` [B,2] in the sorted key array ``keys``; -1 if unknown."""
     lib = _lib.load()

@@ -189,6 +189,18 @@ int kge_topk(const float* Q, const float* bias, const void* E, int dtype, const 
              int apply_sigmoid, void* workspace, size_t workspace_bytes, void* stream);
 
 /*
+ * Smallest and largest score of every query over all N entities: out_min[b] = min_e S[b, e],
+ * out_max[b] = max_e S[b, e] (bias included), without writing S.  Replaces the `preds_raw.min(dim=1)` /
+ * `.max(dim=1)` pair of the per-sample min-max normalisation in
+ * evaluate_ensemble_link_prediction_performance (dicee/evaluation/ensemble.py:93-96); with the
+ * per-model factors w_m / (max_m - min_m + 1e-8) folded into the query vectors the weighted average of
+ * the normalised scores of M models is ONE contraction against the column-wise concatenation of their
+ * entity tables, ranked by kge_rank_filtered.
+ */
+int kge_row_minmax(const float* Q, const float* bias, const void* E, int dtype, const float* scale,
+                   int64_t B, int64_t d, int64_t N, float* out_min, float* out_max, void* stream);
+
+/*
  * Fused KvsAll BCE: mean over B*N of BCEWithLogits(s, y) with y the multi-hot of the CSR row
  * (KvsAll.__getitem__, dicee/dataset_classes.py:354-361, incl. its label smoothing
  * y*(1-eps) + 1/N when eps != 0) and the default loss of dicee/models/base_model.py:138, as

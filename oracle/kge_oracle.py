@@ -36,6 +36,8 @@ Pinning status (independent checks live in ``tests/test_oracle_pins.py``)
 * ``head_query`` / ``all_head_scores``  column h of the head-direction scores of (r, t) equals
                       ``triple_scores`` and the tail-direction score of the same triple;
                       linearity in the head row.
+* ``ensemble_scores``  rows lie in [0, sum of weights]; invariance under a positive affine map of one
+                      model's scores; hand-computed 2-model fixture.
 * ``vocab`` / ``vocab_csr``  hand-written 7-triple fixture; set identities
                       (every triple recoverable from exactly one row, rows
                       partition the distinct triples).
@@ -501,6 +503,23 @@ def all_head_scores(model, E, R, rt, **kw):
     """[B,N]: score(x, r, t) for every entity x."""
     dtype = kw.get("dtype", np.float64)
     return head_query(model, E, R, rt, **kw) @ np.asarray(E, dtype=dtype).T
+
+
+def ensemble_scores(score_list, weights=None, weighted_averaging=True, normalize_scores=True):
+    """Combined [B,N] scores of an ensemble (dicee/evaluation/ensemble.py:88-110): per model and row min-max
+    normalisation ``(s - min) / (max - min + 1e-8)``, then the weighted sum (or the plain mean)."""
+    preds = []
+    for S in score_list:
+        S = np.asarray(S, dtype=np.float64)
+        if normalize_scores:
+            lo, hi = S.min(axis=1, keepdims=True), S.max(axis=1, keepdims=True)
+            S = (S - lo) / (hi - lo + 1e-8)
+        preds.append(S)
+    stack = np.stack(preds, axis=0)
+    if weighted_averaging:
+        w = np.asarray(weights, dtype=np.float64).reshape(-1, 1, 1)
+        return (stack * w).sum(axis=0)
+    return stack.mean(axis=0)
 
 
 def lp_metrics(head_ranks, tail_ranks):

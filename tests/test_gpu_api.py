@@ -365,3 +365,41 @@ def test_string_triple_evaluators():
         assert tails[key] == pytest.approx(want_t[key])
     with pytest.raises(KeyError):
         evaluate_link_prediction_performance_with_reciprocals(kge, [("e1", "r1", "stranger")], er_s)
+
+
+@pytest.mark.parametrize("normalize,weighted", [(True, True), (True, False), (False, True)])
+def test_ensemble_evaluation(normalize, weighted):
+    from dicee_amd import evaluate_ensemble_link_prediction_performance as ens_eval
+    from dicee_amd import ops
+    members = [_toy("DistMult", 32, n=1200, seed=41), _toy("ComplEx", 64, n=1200, seed=42),
+               _toy("Keci", 30, n=1200, seed=43, p=2, q=2)]
+    triples = members[0][1]
+    er = ko.vocab(triples, "er")
+    test = triples[700:1000]
+    weights = [0.5, 0.3, 0.2]
+    S = []
+    for (m, _), name in zip(members, ("DistMult", "ComplEx", "Keci")):
+        S.append(ko.k_vs_all_scores(name, m.entity_embeddings.weight.detach().numpy(),
+                                    m.relation_embeddings.weight.detach().numpy(), test[:, :2], **_oracle_kw(m)))
+    want = ko.ensemble_scores(S, weights, weighted, normalize)
+    gpu_models = [m.to("cuda") for m, _ in members]
+    # the fused row extrema against the oracle's
+    x = torch.from_numpy(test[:, :2].copy()).cuda()
+    Q, bias = gpu_models[1].query(x)
+    lo, hi = ops.row_minmax(Q, bias, *gpu_models[1].table())
+    assert np.abs(lo.cpu().numpy() - S[1].min(1)).max() <= 1e-5 * np.abs(S[1]).max()
+    assert np.abs(hi.cpu().numpy() - S[1].max(1)).max() <= 1e-5 * np.abs(S[1]).max()
+    res, ranks = ens_eval(gpu_models, test, er, weights=weights if weighted else None, batch_size=128,
+                          weighted_averaging=weighted, normalize_scores=normalize, return_ranks=True)
+    exact = 0
+    for j, (h, r, t) in enumerate(test):
+        tol = 2e-5 * (1.0 if normalize else np.sqrt((want[j] ** 2).mean()))
+        lo_r, hi_r = ko.rank_interval_with_tolerance(want[j], int(t), er[(int(h), int(r))], tol)
+        assert lo_r <= ranks[j] <= hi_r
+        exact += lo_r == hi_r
+    assert exact >= 0.9 * len(test)
+    wm = ko.metrics_from_ranks(ranks)
+    assert res["MRR"] == pytest.approx(wm["MRR"]) and res["H@10"] == wm["H@10"]
+    if weighted:
+        with pytest.raises(AssertionError):
+            ens_eval(gpu_models, test, er, weights=[1.0], weighted_averaging=True)

@@ -453,3 +453,18 @@ def test_lp_metrics_closed_form():
     m = ko.lp_metrics([1, 4, 11], [2, 1, 3])
     assert m["H@1"] == pytest.approx(2 / 6) and m["H@3"] == pytest.approx(4 / 6) and m["H@10"] == pytest.approx(5 / 6)
     assert m["MRR"] == pytest.approx((1 + 1 / 4 + 1 / 11 + 1 / 2 + 1 + 1 / 3) / 6)
+
+
+def test_ensemble_scores_fixture_and_invariances():
+    A = np.array([[0.0, 2.0, 4.0]])
+    B = np.array([[10.0, 0.0, 5.0]])
+    got = ko.ensemble_scores([A, B], weights=[0.25, 0.75])
+    np.testing.assert_allclose(got, [[0.75, 0.125, 0.625]], rtol=1e-7)      # 0.25*[0,.5,1] + 0.75*[1,0,.5]
+    np.testing.assert_allclose(ko.ensemble_scores([A, B], weighted_averaging=False), [[0.5, 0.25, 0.75]], rtol=1e-7)
+    np.testing.assert_allclose(ko.ensemble_scores([A, B], weights=[1, 1], normalize_scores=False), A + B)
+    rng = np.random.default_rng(0)
+    S1, S2 = rng.standard_normal((6, 40)), rng.standard_normal((6, 40))
+    base = ko.ensemble_scores([S1, S2], weights=[0.4, 0.6])
+    moved = ko.ensemble_scores([3.0 * S1 - 7.0, S2], weights=[0.4, 0.6])      # min-max removes a positive affine map
+    np.testing.assert_allclose(moved, base, atol=1e-7)
+    assert base.min() >= 0.0 and base.max() <= 1.0 + 1e-12
