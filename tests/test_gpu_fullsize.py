@@ -68,6 +68,37 @@ def test_c4_topk_matches_materialised_scores(c4):
     assert bool((vals[:, :-1] >= vals[:, 1:]).all())                   # sorted descending
 
 
+def test_c4_vocabularies_built_on_the_gpu_and_head_direction(c4):
+    """10M triples -> (h, r) and (r, t) vocabularies on the GPU; the first against the numpy builder, the second
+    used to rank true heads, checked against materialised head-direction scores of sampled queries."""
+    from dicee_amd.csr import FilterCSR
+    cfg, model = c4
+    trip = torch.from_numpy(cfg.triples).cuda()
+    er = FilterCSR.from_triples_gpu(trip, cfg.N, cfg.R, kind="er")
+    host = FilterCSR.from_triples(cfg.triples, cfg.R)                  # no per-row cap, unlike cfg.csr
+    assert torch.equal(er.keys.cpu(), torch.from_numpy(host.keys_np))
+    assert torch.equal(er.row_ptr.cpu(), torch.from_numpy(host.row_ptr_np))
+    assert torch.equal(er.col.cpu(), torch.from_numpy(host.col_np))
+    re = FilterCSR.from_triples_gpu(trip, cfg.N, cfg.R, kind="re")
+    assert re.nnz == er.nnz                                            # both hold every distinct triple once
+    q = torch.from_numpy(cfg.queries[:2048].copy()).cuda()
+    rt, h = q[:, 1:].contiguous(), q[:, 0].contiguous()
+    full = model.rank_filtered(rt, h, re, heads=True)
+    lens = np.diff(re.row_ptr_np)[re.rows_for_numpy(cfg.queries[:2048, 1:])]
+    pick = np.unique(np.concatenate([np.argsort(-lens)[:2], [0, 777, 2047]]))
+    S = model.forward_all_heads(rt[pick].contiguous()).cpu().numpy()
+    for j, b in enumerate(pick):
+        hh, r, t = (int(v) for v in cfg.queries[b])
+        heads = re.col_np[re.row_ptr_np[re.rows_for_numpy(np.array([[r, t]]))[0]]:][:lens[b]]
+        g, e, el = ko.filtered_rank_counts(S[j], hh, heads)
+        assert (g, e, el) == (int(full["n_greater"][b]), int(full["n_equal"][b]), int(full["n_equal_lower"][b]))
+        assert float(full["target_score"][b]) == S[j, hh]
+    # one triple, both directions: the head-direction score of (r, t) at h equals the tail-direction score of (h, r) at t
+    both = model.forward_triples(q[:2048])
+    err = (full["target_score"] - both).abs()                          # different bf16 roundings of the two query vectors
+    assert float(err.max()) <= 2e-2 * float(both.pow(2).mean().sqrt())
+
+
 def test_c5_int8_topk_matches_materialised_scores():
     from dicee_amd import synthetic
     cfg = synthetic.make_config("c5", with_tables=False)
