@@ -5,7 +5,8 @@
 // Head direction (pairs are (relation, tail), the unknown is the head): every model's triple score
 // is linear in the head row, score(x, r, t) = Q'(r, t) . E[x].  DistMult: r * t.  ComplEx:
 // conj(r) * t as complex numbers.  QMult: t (x) conj(r^) as quaternions.  Keci: the coefficient of
-// each head component, including those of the sigma sums (which hold h and r but not t).
+// each head component, including those of the sigma sums (which hold h and r but not t).  OMult:
+// the coefficient of head part i is sum_j sign[j][i] * r^_(i xor j) * t_j.
 #include "kge_internal.h"
 
 namespace kge {
@@ -121,6 +122,51 @@ __global__ void __launch_bounds__(64) build_query_kernel(QueryArgs a, int model)
       q[g + d4] = ah * br + bh * ar + ch * dr - dh * cr;
       q[g + 2 * d4] = ah * cr - bh * dr + ch * ar + dh * br;
       q[g + 3 * d4] = ah * dr + bh * cr - ch * br + dh * ar;
+    }
+  } else if (model == KGE_OMULT) {
+    // octonion product e_j = sum_i sign[j][i] * x_i * y_(i xor j); bit i of OCT_MINUS[j] set = minus
+    constexpr unsigned char OCT_MINUS[8] = {0xfe, 0x68, 0xc2, 0xa4, 0x0e, 0x54, 0x98, 0x32};
+    const int d8 = d >> 3;
+    for (int g = lane; g < d8; g += 64) {
+      float x[8], y[8], o[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        x[i] = sh[g + i * d8];
+        y[i] = sr[g + i * d8];
+      }
+      if (a.normalize_relation) {  // no epsilon, as the reference: a zero octonion gives NaN
+        float n2 = 0.f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) n2 += y[i] * y[i];
+        const float den = sqrtf(n2);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) y[i] = y[i] / den;
+      }
+      if (!a.head_mode) {  // x = head: o_j = sum_i sign[j][i] x_i y_(i^j)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          float acc = 0.f;
+#pragma unroll
+          for (int i = 0; i < 8; ++i) {
+            const float t = x[i] * y[i ^ j];
+            acc += ((OCT_MINUS[j] >> i) & 1) ? -t : t;
+          }
+          o[j] = acc;
+        }
+      } else {  // x = tail: coefficient of head part i: sum_j sign[j][i] y_(i^j) x_j
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          float acc = 0.f;
+#pragma unroll
+          for (int j = 0; j < 8; ++j) {
+            const float t = y[i ^ j] * x[j];
+            acc += ((OCT_MINUS[j] >> i) & 1) ? -t : t;
+          }
+          o[i] = acc;
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < 8; ++i) q[g + i * d8] = o[i];
     }
   } else if (a.head_mode) {  // KGE_KECI, head direction: sh holds the tail row (its parts are not scaled)
     const int p = a.p, qn = a.q;
@@ -252,6 +298,9 @@ static int build_query_impl(int head_mode, int model, int p, int q, const void* 
       break;
     case KGE_QMULT:
       KGE_REQUIRE(d % 4 == 0, KGE_ERR_INVALID, "kge_build_query: QMult needs d %% 4 == 0, got %lld", (long long)d);
+      break;
+    case KGE_OMULT:
+      KGE_REQUIRE(d % 8 == 0, KGE_ERR_INVALID, "kge_build_query: OMult needs d %% 8 == 0, got %lld", (long long)d);
       break;
     case KGE_KECI:
       KGE_REQUIRE(p >= 0 && q >= 0 && d % (p + q + 1) == 0, KGE_ERR_INVALID,

@@ -1,10 +1,10 @@
 """MI355X-native KvsAll scoring, filtered-rank evaluation and top-k prediction for dicee-style
-knowledge-graph-embedding models (DistMult, ComplEx, QMult, Keci).
+knowledge-graph-embedding models (DistMult, ComplEx, QMult, OMult, Keci).
 
 The compute path is a hand-written HIP library (``libkge_hip.so``, C ABI in ``include/kge_hip.h``);
 this package is the thin Python side that mirrors the reference's call surface:
 
-* ``models``     ``DistMult/ComplEx/QMult/Keci/CKeci`` with ``forward``, ``forward_k_vs_all``,
+* ``models``     ``DistMult/ComplEx/QMult/OMult/Keci/CKeci`` with ``forward``, ``forward_k_vs_all``,
                  ``k_vs_all_score`` (dicee/models/*.py)
 * ``evaluator``  ``Evaluator.evaluate_lp_k_vs_all`` (dicee/evaluation/evaluator.py:394-510)
 * ``link_prediction``  ``evaluate_lp``: head and tail direction (dicee/evaluation/link_prediction.py:351-473)
@@ -21,7 +21,7 @@ present.
 """
 from . import _lib  # noqa: F401
 from .csr import FilterCSR  # noqa: F401
-from .models import DistMult, ComplEx, QMult, Keci, CKeci, MODEL_REGISTRY, initialize_model  # noqa: F401
+from .models import DistMult, ComplEx, QMult, OMult, Keci, CKeci, MODEL_REGISTRY, initialize_model  # noqa: F401
 from .evaluator import Evaluator, compute_metrics_from_ranks_simple  # noqa: F401
 from .kge import KGE  # noqa: F401
 from .ensemble import evaluate_ensemble_link_prediction_performance  # noqa: F401

@@ -6,7 +6,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libkge_hip.so")
 
 KGE_OK = 0
-MODEL_IDS = {"DistMult": 0, "ComplEx": 1, "QMult": 2, "Keci": 3, "CKeci": 3}
+MODEL_IDS = {"DistMult": 0, "ComplEx": 1, "QMult": 2, "Keci": 3, "CKeci": 3, "OMult": 4}
 DTYPE_F32, DTYPE_BF16, DTYPE_I8 = 0, 1, 2
 NORM_NONE, NORM_LAYERNORM, NORM_BATCHNORM1D = 0, 1, 2
 

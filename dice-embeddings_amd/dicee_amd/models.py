@@ -199,6 +199,19 @@ class QMult(BaseKGE):
         return {"normalize_relation": isinstance(self.normalize_relation_embeddings, IdentityClass)}
 
 
+class OMult(BaseKGE):
+    """dicee/models/octonion.py:51-163."""
+    name = "OMult"
+
+    def __init__(self, args):
+        super().__init__(args)
+        assert self.embedding_dim % 8 == 0, "OMult needs an embedding dimension divisible by 8"
+
+    def _query_kwargs(self):
+        # the octonion normaliser runs only when no other relation normaliser is set (octonion.py:121)
+        return {"normalize_relation": isinstance(self.normalize_relation_embeddings, IdentityClass)}
+
+
 class Keci(BaseKGE):
     """dicee/models/clifford.py:3-329."""
     name = "Keci"
@@ -242,7 +255,8 @@ class CKeci(Keci):
             self.q_coefficients.weight.requires_grad_(False)
 
 
-MODEL_REGISTRY = {"DistMult": DistMult, "ComplEx": ComplEx, "QMult": QMult, "Keci": Keci, "CKeci": CKeci}
+MODEL_REGISTRY = {"DistMult": DistMult, "ComplEx": ComplEx, "QMult": QMult, "OMult": OMult, "Keci": Keci,
+                  "CKeci": CKeci}
 
 
 def initialize_model(args: dict):

@@ -41,7 +41,7 @@ enum kge_status {
   KGE_ERR_OVERFLOW = 5      /* top-k candidate buffers overflowed beyond recovery */
 };
 
-enum kge_model { KGE_DISTMULT = 0, KGE_COMPLEX = 1, KGE_QMULT = 2, KGE_KECI = 3 };
+enum kge_model { KGE_DISTMULT = 0, KGE_COMPLEX = 1, KGE_QMULT = 2, KGE_KECI = 3, KGE_OMULT = 4 };
 enum kge_dtype { KGE_F32 = 0, KGE_BF16 = 1, KGE_I8 = 2 };
 enum kge_norm_kind { KGE_NORM_NONE = 0, KGE_NORM_LAYERNORM = 1, KGE_NORM_BATCHNORM1D = 2 };
 
@@ -71,10 +71,13 @@ int kge_abi_version(void);
  * elementwise part of k_vs_all_score of DistMult (dicee/models/real.py:32), ComplEx
  * (dicee/models/complex.py:254-263), QMult (dicee/models/quaternion.py:138-144 with
  * quaternion_normalizer :74-100 and quaternion_mul dicee/models/static_funcs.py:4-18) and Keci
- * (dicee/models/clifford.py:260-304 with apply_coefficients :105-113).
+ * (dicee/models/clifford.py:260-304 with apply_coefficients :105-113), and of OMult
+ * (dicee/models/octonion.py:112-152 with octonion_normalizer :57-70 and octonion_mul :5-19).
  *   ent [N,d] (ent_dtype; ent_scale [N] for KGE_I8 else NULL), rel [R,d] (KGE_F32 or KGE_BF16)
  *   p,q,coeff_p[p],coeff_q[q]: Keci only.  normalize_relation: QMult only (1 when the model's
- *   relation normaliser is the identity, quaternion.py:138).  norm: NULL or see above.
+ *   relation normaliser is the identity, quaternion.py:138; the same switch for OMult's octonion
+ *   normaliser, octonion.py:121, which has no epsilon: a zero relation octonion gives NaN).  norm:
+ *   NULL or see above.
  *   hr [B,2] int64.  Q [B,d] fp32 out.  bias [B] fp32 out (all zero except Keci with p>=2 or q>=2).
  */
 int kge_build_query(int model, int p, int q, const void* ent, int ent_dtype, const float* ent_scale,

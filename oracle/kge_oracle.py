@@ -18,6 +18,10 @@ Pinning status (independent checks live in ``tests/test_oracle_pins.py``)
                       structure-constant table and against
                       ``scipy.spatial.transform.Rotation`` composition; the
                       block-split vs consecutive-group quirk has a d=8 fixture.
+* ``octonion_*`` / ``omult_query``  composition-algebra identities the sign table must satisfy:
+                      |xy| = |x||y|, x conj(x) = |x|^2, e_i^2 = -1, alternativity x(xy) = (xx)y and
+                      (xy)y = x(yy), the quaternion subalgebra on parts 0-3 equals the (pinned)
+                      Hamilton product; per-triple score against the KvsAll column.
 * ``keci_*``          (p,q)=(0,0) == DistMult; (0,1), c=1 == ComplEx; (0,1),
                       c=0 == DistMult on the first half; general (p,q) against a
                       brute-force geometric-algebra product on bitmask blades;
@@ -50,7 +54,7 @@ from __future__ import annotations
 
 import numpy as np
 
-MODELS = ("DistMult", "ComplEx", "QMult", "Keci")
+MODELS = ("DistMult", "ComplEx", "QMult", "Keci", "OMult")
 
 # --------------------------------------------------------------------------
 # known-answer vocabularies
@@ -256,6 +260,45 @@ def qmult_scores_ref_form(h, r, E, normalize_relation=True):
 
 
 # --------------------------------------------------------------------------
+# OMult   dicee/models/octonion.py:5-19 (octonion_mul), :57-70 (normaliser), :112-152 (k_vs_all_score)
+# --------------------------------------------------------------------------
+# e_j = sum_i SIGN[j][i] * x_i * y_(i xor j): the eight lines of octonion_mul, read off term by term.
+OCTONION_SIGN = np.array([
+    [+1, -1, -1, -1, -1, -1, -1, -1],
+    [+1, +1, +1, -1, +1, -1, -1, +1],
+    [+1, -1, +1, +1, +1, +1, -1, -1],
+    [+1, +1, -1, +1, +1, -1, +1, -1],
+    [+1, -1, -1, -1, +1, +1, +1, +1],
+    [+1, +1, -1, +1, -1, +1, -1, +1],
+    [+1, +1, +1, -1, -1, +1, +1, -1],
+    [+1, -1, +1, +1, -1, -1, +1, +1]], dtype=np.float64)
+
+
+def octonion_parts(x):
+    m = x.shape[1] // 8
+    return [x[:, i * m:(i + 1) * m] for i in range(8)]
+
+
+def octonion_normalize(r):
+    """Each octonion (element g of the 8 blocks) divided by its norm; no epsilon (octonion.py:57-70)."""
+    parts = octonion_parts(r)
+    den = np.sqrt(sum(p * p for p in parts))
+    with np.errstate(divide="ignore", invalid="ignore"):
+        return np.concatenate([p / den for p in parts], axis=1)
+
+
+def octonion_product_blocks(x, y):
+    xp, yp = octonion_parts(x), octonion_parts(y)
+    return [sum(OCTONION_SIGN[j][i] * xp[i] * yp[i ^ j] for i in range(8)) for j in range(8)]
+
+
+def omult_query(h, r, normalize_relation=True):
+    if normalize_relation:
+        r = octonion_normalize(r)
+    return np.concatenate(octonion_product_blocks(h, r), axis=1)
+
+
+# --------------------------------------------------------------------------
 # M6-M9 Keci   dicee/models/clifford.py:4-28,105-113,162-192,258-305
 # --------------------------------------------------------------------------
 
@@ -364,6 +407,8 @@ def build_query(model, E, R, hr, p=0, q=0, coeff_p=None, coeff_q=None,
         return complex_query(h, r), np.zeros(len(h), dtype)
     if model == "QMult":
         return qmult_query(h, r, normalize_relation), np.zeros(len(h), dtype)
+    if model == "OMult":
+        return omult_query(h, r, normalize_relation), np.zeros(len(h), dtype)
     if model in ("Keci", "CKeci"):
         return keci_query(h, r, p, q, coeff_p, coeff_q)
     raise ValueError(model)
@@ -432,6 +477,10 @@ def triple_scores(model, E, R, triples, p=0, q=0, coeff_p=None, coeff_q=None, no
         imj = ha * rc - hb * rd + hc * ra + hd * rb
         imk = ha * rd + hb * rc - hc * rb + hd * ra
         return (real * ta).sum(1) + (imi * tb).sum(1) + (imj * tc).sum(1) + (imk * td).sum(1)
+    if model == "OMult":                                     # OMult.score (octonion.py:72-110)
+        if normalize_relation:
+            r = octonion_normalize(r)
+        return sum((e * tp).sum(1) for e, tp in zip(octonion_product_blocks(h, r), octonion_parts(t)))
     if model in ("Keci", "CKeci"):
         rr = d // (p + q + 1)
         out = np.zeros(n, dtype=dtype)
@@ -475,6 +524,11 @@ def head_query(model, E, R, rt, p=0, q=0, coeff_p=None, coeff_q=None, normalize_
         m = d // 4
         conj = np.concatenate([r[:, :m], -r[:, m:]], axis=1)
         return np.concatenate(hamilton_product_blocks(t, conj), axis=1)
+    if model == "OMult":                                     # coefficient of head part i: sum_j SIGN[j][i] y_(i^j) t_j
+        if normalize_relation:
+            r = octonion_normalize(r)
+        yp, tp = octonion_parts(r), octonion_parts(t)
+        return np.concatenate([sum(OCTONION_SIGN[j][i] * yp[i ^ j] * tp[j] for j in range(8)) for i in range(8)], axis=1)
     if model in ("Keci", "CKeci"):
         rr = d // (p + q + 1)
         r0, rp, rq = keci_split(r, rr, p, q)

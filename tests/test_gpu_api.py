@@ -45,6 +45,7 @@ def _oracle_kw(m):
 
 
 @pytest.mark.parametrize("name,d,extra", [("DistMult", 32, {}), ("ComplEx", 32, {}), ("QMult", 32, {}),
+                                          ("OMult", 32, {}),
                                           ("Keci", 30, {"p": 2, "q": 2}), ("CKeci", 32, {"p": 0, "q": 1})])
 def test_forward_k_vs_all_is_a_drop_in(name, d, extra):
     m, triples = _toy(name, d, **extra)
@@ -230,6 +231,7 @@ def test_stored_experiment_evaluates_end_to_end(tmp_path):
 
 
 @pytest.mark.parametrize("name,d,extra", [("DistMult", 32, {}), ("ComplEx", 64, {}), ("QMult", 64, {}),
+                                          ("OMult", 64, {}),
                                           ("Keci", 48, {"p": 0, "q": 1}), ("Keci", 40, {"p": 2, "q": 2})])
 def test_evaluate_lp_both_directions(name, d, extra):
     """Head and tail ranks inside the fp64 oracle's tolerance interval, exact where there is no near-tie; metrics

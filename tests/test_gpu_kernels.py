@@ -37,6 +37,8 @@ MODEL_CASES = [
     ("Keci", 35, {"p": 3, "q": 3, "coeff_p": [0.7, 1.1, -0.3], "coeff_q": [1.3, -0.4, 0.9]}),
     ("Keci", 24, {"p": 2, "q": 0, "coeff_p": [0.5, 2.0]}),
     ("Keci", 16, {"p": 0, "q": 0}),
+    ("OMult", 128, {}),
+    ("OMult", 24, {"normalize_relation": False}),
 ]
 
 
@@ -66,7 +68,7 @@ def test_build_query_fp32(ops, model, d, kw):
 
 
 @pytest.mark.parametrize("storage", ["bf16", "int8"])
-@pytest.mark.parametrize("model", ["DistMult", "ComplEx", "QMult"])
+@pytest.mark.parametrize("model", ["DistMult", "ComplEx", "QMult", "OMult"])
 def test_build_query_quantised_tables(ops, model, storage):
     rng = np.random.default_rng(7)
     N, R, d, B = 200, 9, 128, 50

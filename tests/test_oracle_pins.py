@@ -409,7 +409,7 @@ def test_vocab_csr_against_a_hand_written_fixture_and_set_identities():
             assert np.all(np.diff(col[row_ptr[i]:row_ptr[i + 1]]) > 0)
 
 
-_LP_CASES = [("DistMult", 12, {}), ("ComplEx", 12, {}), ("QMult", 16, {}), ("QMult", 16, {"normalize_relation": False}),
+_LP_CASES = [("OMult", 16, {}), ("OMult", 24, {"normalize_relation": False}), ("DistMult", 12, {}), ("ComplEx", 12, {}), ("QMult", 16, {}), ("QMult", 16, {"normalize_relation": False}),
              ("Keci", 12, {"p": 0, "q": 0}), ("Keci", 12, {"p": 0, "q": 1}), ("Keci", 12, {"p": 1, "q": 1}),
              ("Keci", 12, {"p": 2, "q": 0}), ("Keci", 12, {"p": 0, "q": 2}), ("Keci", 15, {"p": 2, "q": 2}),
              ("Keci", 18, {"p": 3, "q": 2}), ("Keci", 18, {"p": 1, "q": 4})]
@@ -468,3 +468,36 @@ def test_ensemble_scores_fixture_and_invariances():
     moved = ko.ensemble_scores([3.0 * S1 - 7.0, S2], weights=[0.4, 0.6])      # min-max removes a positive affine map
     np.testing.assert_allclose(moved, base, atol=1e-7)
     assert base.min() >= 0.0 and base.max() <= 1.0 + 1e-12
+
+
+def test_octonion_table_is_a_composition_algebra():
+    """A wrong sign or index in the 8x8 table breaks at least one of these identities."""
+    rng = np.random.default_rng(11)
+    x, y = rng.standard_normal((50, 8)), rng.standard_normal((50, 8))
+    mul = lambda a, b: np.concatenate(ko.octonion_product_blocks(a, b), axis=1)
+    norm = lambda a: np.sqrt((a * a).sum(1))
+    np.testing.assert_allclose(norm(mul(x, y)), norm(x) * norm(y), rtol=1e-12)           # |xy| = |x||y|
+    conj = x * np.array([1, -1, -1, -1, -1, -1, -1, -1.0])
+    xc = mul(x, conj)
+    np.testing.assert_allclose(xc[:, 0], (x * x).sum(1), rtol=1e-12)                      # x conj(x) = |x|^2
+    np.testing.assert_allclose(xc[:, 1:], 0.0, atol=1e-12)
+    eye = np.eye(8)
+    for i in range(1, 8):
+        np.testing.assert_allclose(mul(eye[i:i + 1], eye[i:i + 1]), -eye[0:1], atol=0)    # e_i^2 = -1
+        np.testing.assert_allclose(mul(eye[0:1], eye[i:i + 1]), eye[i:i + 1], atol=0)     # 1 is the unit
+        np.testing.assert_allclose(mul(eye[i:i + 1], eye[0:1]), eye[i:i + 1], atol=0)
+        for j in range(1, 8):
+            if i != j:                                                                    # imaginary units anticommute
+                np.testing.assert_allclose(mul(eye[i:i + 1], eye[j:j + 1]), -mul(eye[j:j + 1], eye[i:i + 1]), atol=0)
+    np.testing.assert_allclose(mul(x, mul(x, y)), mul(mul(x, x), y), rtol=1e-10, atol=1e-10)   # alternativity
+    np.testing.assert_allclose(mul(mul(x, y), y), mul(x, mul(y, y)), rtol=1e-10, atol=1e-10)
+    # parts 0-3 form the quaternions with the Hamilton product pinned above
+    q1, q2 = rng.standard_normal((20, 4)), rng.standard_normal((20, 4))
+    pad = lambda q: np.concatenate([q, np.zeros_like(q)], axis=1)
+    got = mul(pad(q1), pad(q2))
+    np.testing.assert_allclose(got[:, :4], np.concatenate(ko.hamilton_product_blocks(q1, q2), axis=1), rtol=1e-12)
+    np.testing.assert_allclose(got[:, 4:], 0.0, atol=0)
+    # normaliser: unit octonions, block layout (element g of each of the 8 blocks)
+    r = rng.standard_normal((5, 24))
+    rn = ko.octonion_normalize(r)
+    np.testing.assert_allclose(sum(p * p for p in ko.octonion_parts(rn)), 1.0, rtol=1e-12)
