@@ -2,9 +2,10 @@
 
 Mirrors dicee's ``KGE`` (dicee/knowledge_graph_embeddings.py): ``predict_missing_tail_entity``
 (:314-413), ``predict_missing_head_entity`` (:134-228), ``predict`` (:415-466) and ``predict_topk``
-(:468-579).  The reference scores every (x, r, t) triple through ``forward_triples`` for a missing
-head; here that is one head-direction query and the same table contraction as for tails.  Relation
-prediction is outside this build: it raises ``NotImplementedError``.
+(:468-579), ``triple_score`` (:581-650) and ``answer_multi_hop_query`` (:670-1170).  The reference
+scores every (x, r, t) triple through ``forward_triples`` for a missing head; here that is one
+head-direction query and the same table contraction as for tails.  Relation prediction is outside
+this build: it raises ``NotImplementedError``.
 """
 from typing import List, Union
 
@@ -181,3 +182,101 @@ class KGE:
         lookup = self.idx_to_entity
         return [[(lookup[idx], score) for idx, score in zip(row_idxs, row_scores)]
                 for row_idxs, row_scores in zip(topk_idxs, topk_scores)]
+
+    # ------------------------------------------------------------------ multi-hop queries
+    @staticmethod
+    def t_norm(tens_1, tens_2, tnorm="min"):
+        """dicee/abstracts.py:443-447."""
+        if "min" in tnorm:
+            return torch.min(tens_1, tens_2)
+        if "prod" in tnorm:
+            return tens_1 * tens_2
+
+    @staticmethod
+    def t_conorm(tens_1, tens_2, tconorm="min"):
+        """dicee/abstracts.py:460-464."""
+        if "min" in tconorm:
+            return torch.max(tens_1, tens_2)
+        if "prod" in tconorm:
+            return (tens_1 + tens_2) - (tens_1 * tens_2)
+
+    @staticmethod
+    def negnorm(tens_1, lambda_, neg_norm="standard"):
+        """dicee/abstracts.py:466-472."""
+        if "standard" in neg_norm:
+            return 1 - tens_1
+        if "sugeno" in neg_norm:
+            return (1 - tens_1) / (1 + lambda_ * tens_1)
+        if "yager" in neg_norm:
+            return (1 - torch.pow(tens_1, lambda_)) ** (1 / lambda_)
+
+    def _atom(self, head_ids, relation: str):
+        """[len(head_ids), N] logits of (head, relation, ?) on the GPU: ONE batched KvsAll call where the
+        reference calls ``predict`` once per substitution."""
+        dev = self.model.entity_embeddings.weight.device
+        head_ids = torch.as_tensor(head_ids, dtype=torch.int64, device=dev).reshape(-1)
+        rel = torch.full_like(head_ids, self.relation_to_idx[relation])
+        with torch.no_grad():
+            return self.model.forward_k_vs_all(torch.stack([head_ids, rel], dim=1).contiguous())
+
+    def _multi_hop_scores(self, query_type, query, tnorm, neg_norm, lambda_, k):
+        """[N] GPU tensor: score of every entity as the answer (the norms act on logits, as in the reference,
+        whose ``predict`` defaults to ``logits=True``)."""
+        one = lambda e, r: self._atom([self.entity_to_idx[e]], r)[0]
+
+        def hop(prev, r):          # keep the k best substitutions of the variable, then the best t-norm per answer
+            s, idx = torch.sort(prev, descending=True, stable=True)
+            return torch.max(self.t_norm(s[:k, None], self._atom(idx[:k], r), tnorm), dim=0)[0]
+        if query_type == "1p":
+            e, (r1,) = query
+            return one(e, r1)
+        if query_type == "2p":
+            e, (r1, r2) = query
+            return hop(one(e, r1), r2)
+        if query_type == "3p":
+            e, (r1, r2, r3) = query
+            return hop(hop(one(e, r1), r2), r3)
+        if query_type in ("2i", "3i", "2in", "3in", "2u"):
+            vals = []
+            for e, rel in (part for part in query if part != ("u",)):
+                v = one(e, rel[0])
+                vals.append(self.negnorm(v, lambda_, neg_norm) if rel[-1] == "n" else v)
+            out = vals[0]
+            for v in vals[1:]:
+                out = self.t_conorm(out, v, tnorm) if query_type == "2u" else self.t_norm(out, v, tnorm)
+            return out
+        if query_type in ("ip", "inp", "up"):
+            inner, (r,) = query
+            inner_type = {"ip": "2i", "inp": "2in", "up": "2u"}[query_type]
+            return hop(self._multi_hop_scores(inner_type, inner, tnorm, neg_norm, lambda_, k), r)
+        if query_type in ("pi", "pin", "pni"):
+            (e1, rels), (e3, rel3) = query
+            s, idx = torch.sort(one(e1, rels[0]), descending=True, stable=True)
+            a2 = self._atom(idx[:k], rels[1])
+            if query_type == "pni":
+                a2 = self.negnorm(a2, lambda_, neg_norm)
+            two_p = torch.max(self.t_norm(s[:k, None], a2, tnorm), dim=0)[0]
+            last = one(e3, rel3[0])
+            if query_type == "pin":
+                last = self.negnorm(last, lambda_, neg_norm)
+            return self.t_norm(two_p, last, tnorm)
+        raise ValueError(f"Invalid query type: {query_type}")
+
+    def answer_multi_hop_query(self, query_type: str = None, query=None, queries=None, tnorm: str = "prod",
+                               neg_norm: str = "standard", lambda_: float = 0.0, k: int = 10, only_scores=False):
+        """Answers of an EPFO query with negation and disjunction (types 1p 2p 3p 2i 3i ip pi 2in 3in inp pin pni
+        2u up; query encodings as in the reference, e.g. 2p = ``(e, (r1, r2))``, 2i = ``((e1, (r1,)), (e2, (r2,)))``).
+        ``only_scores``: the [N] score tensor; else ``[(entity, score), ...]`` sorted by score, the best k for the
+        path types 1p / 2p / 3p and all entities for the others."""
+        if queries is not None:
+            assert query is None
+            return [self.answer_multi_hop_query(query_type=query_type, query=q, tnorm=tnorm, neg_norm=neg_norm,
+                                                lambda_=lambda_, k=k, only_scores=only_scores) for q in queries]
+        assert len(self.entity_to_idx) >= k >= 0
+        scores = self._multi_hop_scores(query_type, query, tnorm, neg_norm, lambda_, k).cpu()
+        if only_scores:
+            return scores
+        order = torch.sort(scores, descending=True, stable=True)[1].tolist()
+        if query_type in ("1p", "2p", "3p"):
+            order = order[:k]
+        return [(self.idx_to_entity[i], scores[i]) for i in order]

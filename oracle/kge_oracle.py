@@ -42,6 +42,9 @@ Pinning status (independent checks live in ``tests/test_oracle_pins.py``)
                       linearity in the head row.
 * ``ensemble_scores``  rows lie in [0, sum of weights]; invariance under a positive affine map of one
                       model's scores; hand-computed 2-model fixture.
+* ``multi_hop_scores`` / ``t_norm`` / ``t_conorm`` / ``neg_norm``  hand-computed answers on a 3-entity score
+                      table for 2p, 2i, 2in, 2u, ip, pi (min and prod norms); fuzzy-logic identities
+                      (De Morgan for the standard negation, 1p of a 2p with k = N and one-hot scores).
 * ``vocab`` / ``vocab_csr``  hand-written 7-triple fixture; set identities
                       (every triple recoverable from exactly one row, rows
                       partition the distinct triples).
@@ -574,6 +577,81 @@ def ensemble_scores(score_list, weights=None, weighted_averaging=True, normalize
         w = np.asarray(weights, dtype=np.float64).reshape(-1, 1, 1)
         return (stack * w).sum(axis=0)
     return stack.mean(axis=0)
+
+
+# --------------------------------------------------------------------------
+# multi-hop query answering   dicee/knowledge_graph_embeddings.py:670-1170, dicee/abstracts.py:443-472
+# --------------------------------------------------------------------------
+
+
+def t_norm(a, b, tnorm="min"):
+    return np.minimum(a, b) if "min" in tnorm else a * b
+
+
+def t_conorm(a, b, tconorm="min"):
+    return np.maximum(a, b) if "min" in tconorm else (a + b) - (a * b)
+
+
+def neg_norm(a, lambda_, kind="standard"):
+    if "standard" in kind:
+        return 1 - a
+    if "sugeno" in kind:
+        return (1 - a) / (1 + lambda_ * a)
+    return (1 - np.power(a, lambda_)) ** (1 / lambda_)
+
+
+def _top(scores, k):
+    idx = np.argsort(-scores, kind="stable")[:k]
+    return scores[idx], idx
+
+
+def multi_hop_scores(atom, query_type, query, tnorm="prod", neg="standard", lambda_=0.0, k=10):
+    """[N] scores of every entity as answer of an EPFO query.  ``atom(heads, r)`` -> [len(heads), N] scores of
+    (head, r, ?) for entity ids ``heads`` and relation ``r`` (the reference calls ``predict`` with its default
+    ``logits=True``, so the norms act on logits).  A projection after a sub-query keeps the k best
+    substitutions of the intermediate variable and takes, per answer, the best t-norm of
+    (substitution score, next atom)."""
+    def hop(prev_scores, r):                       # project: top-k substitutions, then max over them
+        s, idx = _top(prev_scores, k)
+        return t_norm(s[:, None], atom(list(idx), r), tnorm).max(axis=0)
+    one = lambda e, r: atom([e], r)[0]
+    if query_type == "1p":
+        e, (r1,) = query
+        return one(e, r1)
+    if query_type == "2p":
+        e, (r1, r2) = query
+        return hop(one(e, r1), r2)
+    if query_type == "3p":
+        e, (r1, r2, r3) = query
+        return hop(hop(one(e, r1), r2), r3)
+    if query_type in ("2i", "3i", "2in", "3in", "2u"):
+        parts = [q for q in query if q != ("u",)]
+        vals = []
+        for e, rel in parts:
+            v = one(e, rel[0])
+            vals.append(neg_norm(v, lambda_, neg) if rel[-1] == "n" else v)
+        comb = t_conorm if query_type == "2u" else t_norm
+        out = vals[0]
+        for v in vals[1:]:
+            out = comb(out, v, tnorm)
+        return out
+    if query_type in ("ip", "inp", "up"):
+        inner, (r,) = query
+        inner_type = {"ip": "2i", "inp": "2in", "up": "2u"}[query_type]
+        return hop(multi_hop_scores(atom, inner_type, inner, tnorm, neg, lambda_, k), r)
+    if query_type in ("pi", "pin", "pni"):
+        (e1, rels), (e3, rel3) = query
+        a1 = one(e1, rels[0])
+        s, idx = _top(a1, k)
+        a2 = atom(list(idx), rels[1])
+        if query_type == "pni":
+            a2 = neg_norm(a2, lambda_, neg)
+        two_p = t_norm(s[:, None], a2, tnorm).max(axis=0)
+        last = one(e3, rel3[0])
+        if query_type == "pin":
+            last = neg_norm(last, lambda_, neg)
+        return t_norm(two_p, last, tnorm)
+    raise ValueError(f"Invalid query type: {query_type}")
 
 
 def lp_metrics(head_ranks, tail_ranks):

@@ -405,3 +405,48 @@ def test_ensemble_evaluation(normalize, weighted):
     if weighted:
         with pytest.raises(AssertionError):
             ens_eval(gpu_models, test, er, weights=[1.0], weighted_averaging=True)
+
+
+def test_multi_hop_queries_against_the_oracle():
+    from dicee_amd import KGE
+    m, triples = _toy("ComplEx", 32, seed=51)
+    E = m.entity_embeddings.weight.detach().numpy().copy()
+    Rel = m.relation_embeddings.weight.detach().numpy().copy()
+    m = m.to("cuda")
+    ents = {f"e{i}": i for i in range(135)}
+    rels = {f"r{i}": i for i in range(46)}
+    kge = KGE(model=m, entity_to_idx=ents, relation_to_idx=rels)
+    atom = lambda heads, r: ko.k_vs_all_scores("ComplEx", E, Rel, np.array([[h, r] for h in heads]))
+    n = lambda q: q                                        # readability: queries are given with names
+    cases = [
+        ("1p", ("e3", ("r1",)), (3, (1,))),
+        ("2p", ("e3", ("r1", "r4")), (3, (1, 4))),
+        ("3p", ("e3", ("r1", "r4", "r9")), (3, (1, 4, 9))),
+        ("2i", (("e3", ("r1",)), ("e8", ("r2",))), ((3, (1,)), (8, (2,)))),
+        ("3i", (("e3", ("r1",)), ("e8", ("r2",)), ("e11", ("r5",))), ((3, (1,)), (8, (2,)), (11, (5,)))),
+        ("ip", ((("e3", ("r1",)), ("e8", ("r2",))), ("r7",)), (((3, (1,)), (8, (2,))), (7,))),
+        ("pi", (("e3", ("r1", "r4")), ("e8", ("r2",))), ((3, (1, 4)), (8, (2,)))),
+        ("2in", (("e3", ("r1",)), ("e8", ("r2", "n"))), ((3, (1,)), (8, (2, "n")))),
+        ("3in", (("e3", ("r1",)), ("e8", ("r2",)), ("e11", ("r5", "n"))), ((3, (1,)), (8, (2,)), (11, (5, "n")))),
+        ("inp", ((("e3", ("r1",)), ("e8", ("r2", "n"))), ("r7",)), (((3, (1,)), (8, (2, "n"))), (7,))),
+        ("pin", (("e3", ("r1", "r4")), ("e8", ("r2", "n"))), ((3, (1, 4)), (8, (2, "n")))),
+        ("pni", (("e3", ("r1", "r4", "n")), ("e8", ("r2",))), ((3, (1, 4, "n")), (8, (2,)))),
+        ("2u", (("e3", ("r1",)), ("e8", ("r2",)), ("u",)), ((3, (1,)), (8, (2,)), ("u",))),
+        ("up", ((("e3", ("r1",)), ("e8", ("r2",)), ("u",)), ("r7",)), (((3, (1,)), (8, (2,)), ("u",)), (7,))),
+    ]
+    for tnorm in ("min", "prod"):
+        for qtype, q_named, q_ids in cases:
+            got = kge.answer_multi_hop_query(query_type=qtype, query=n(q_named), tnorm=tnorm, k=5, only_scores=True)
+            want = ko.multi_hop_scores(atom, qtype, q_ids, tnorm=tnorm, k=5)
+            assert got.shape == (135,)
+            np.testing.assert_allclose(got.numpy(), want, rtol=2e-4, atol=2e-5, err_msg=f"{qtype} {tnorm}")
+    top = kge.answer_multi_hop_query(query_type="2p", query=("e3", ("r1", "r4")), tnorm="min", k=5)
+    assert len(top) == 5 and [s for _, s in top] == sorted((s for _, s in top), reverse=True)
+    want = ko.multi_hop_scores(atom, "2p", (3, (1, 4)), tnorm="min", k=5)
+    assert top[0][0] == f"e{int(np.argmax(want))}"
+    full = kge.answer_multi_hop_query(query_type="2i", query=(("e3", ("r1",)), ("e8", ("r2",))), tnorm="min")
+    assert len(full) == 135
+    both = kge.answer_multi_hop_query(query_type="1p", queries=[("e3", ("r1",)), ("e4", ("r2",))], only_scores=True)
+    assert len(both) == 2 and torch.equal(both[0], kge.predict(h=["e3"], r=["r1"]))
+    with pytest.raises(ValueError):
+        kge.answer_multi_hop_query(query_type="4p", query=("e3", ("r1",)))

@@ -501,3 +501,32 @@ def test_octonion_table_is_a_composition_algebra():
     r = rng.standard_normal((5, 24))
     rn = ko.octonion_normalize(r)
     np.testing.assert_allclose(sum(p * p for p in ko.octonion_parts(rn)), 1.0, rtol=1e-12)
+
+
+def test_multi_hop_scores_on_a_hand_made_score_table():
+    # 3 entities, 2 relations; T[r][h] = scores of (h, r, ?) over the 3 entities
+    T = {0: np.array([[0.9, 0.1, 0.5], [0.2, 0.8, 0.3], [0.4, 0.6, 0.7]]),
+         1: np.array([[0.3, 0.7, 0.2], [0.6, 0.1, 0.9], [0.5, 0.5, 0.4]])}
+    atom = lambda heads, r: T[r][np.asarray(heads)]
+    mh = lambda *a, **kw: ko.multi_hop_scores(atom, *a, **kw)
+    np.testing.assert_allclose(mh("1p", (0, (0,))), [0.9, 0.1, 0.5])
+    # 2p, k=2, min: substitutions of (0, r0, ?) = entity 0 (0.9), entity 2 (0.5);
+    # answers = max(min(0.9, T1[0]), min(0.5, T1[2])) = max([.3,.7,.2], [.5,.5,.4]) = [.5,.7,.4]
+    np.testing.assert_allclose(mh("2p", (0, (0, 1)), tnorm="min", k=2), [0.5, 0.7, 0.4])
+    # prod: max([.27,.63,.18], [.25,.25,.2]) = [.27,.63,.2]
+    np.testing.assert_allclose(mh("2p", (0, (0, 1)), tnorm="prod", k=2), [0.27, 0.63, 0.2])
+    np.testing.assert_allclose(mh("2i", ((0, (0,)), (1, (1,))), tnorm="min"), [0.6, 0.1, 0.5])
+    np.testing.assert_allclose(mh("2in", ((0, (0,)), (1, (1, "n"))), tnorm="min"), [0.4, 0.1, 0.1])
+    np.testing.assert_allclose(mh("2u", ((0, (0,)), (1, (1,)), ("u",)), tnorm="min"), [0.9, 0.1, 0.9])
+    np.testing.assert_allclose(mh("2u", ((0, (0,)), (1, (1,)), ("u",)), tnorm="prod"), [0.96, 0.19, 0.95])
+    # ip, k=1, min: 2i = [.6,.1,.5] -> entity 0 (0.6); min(0.6, T0[0]) = [.6,.1,.5]
+    np.testing.assert_allclose(mh("ip", (((0, (0,)), (1, (1,))), (0,)), tnorm="min", k=1), [0.6, 0.1, 0.5])
+    # pi, k=1, min: (0,r0) top = entity 0 (.9); 2p = min(.9, T1[0]) = [.3,.7,.2]; with (2, r0) = [.4,.6,.7] -> [.3,.6,.2]
+    np.testing.assert_allclose(mh("pi", ((0, (0, 1)), (2, (0,))), tnorm="min", k=1), [0.3, 0.6, 0.2])
+    # De Morgan with the standard negation: not(a or b) = not a and not b
+    a, b = T[0][0], T[1][1]
+    for norm in ("min", "prod"):
+        np.testing.assert_allclose(ko.neg_norm(ko.t_conorm(a, b, norm), 0.0),
+                                   ko.t_norm(ko.neg_norm(a, 0.0), ko.neg_norm(b, 0.0), norm), rtol=1e-12)
+    np.testing.assert_allclose(ko.neg_norm(a, 0.0, "sugeno"), 1 - a)          # lambda = 0 is the standard negation
+    np.testing.assert_allclose(ko.neg_norm(a, 1.0, "yager"), 1 - a)
