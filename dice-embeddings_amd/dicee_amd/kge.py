@@ -4,8 +4,8 @@ Mirrors dicee's ``KGE`` (dicee/knowledge_graph_embeddings.py): ``predict_missing
 (:314-413), ``predict_missing_head_entity`` (:134-228), ``predict`` (:415-466) and ``predict_topk``
 (:468-579), ``triple_score`` (:581-650) and ``answer_multi_hop_query`` (:670-1170).  The reference
 scores every (x, r, t) triple through ``forward_triples`` for a missing head; here that is one
-head-direction query and the same table contraction as for tails.  Relation prediction is outside
-this build: it raises ``NotImplementedError``.
+head-direction query and the same table contraction as for tails; a missing relation is scored as
+the reference does it, all ``(h, x, t)`` triples through ``forward_triples`` (``kge_triple_scores``).
 """
 from typing import List, Union
 
@@ -115,6 +115,42 @@ class KGE:
             return scores.flatten(), indices.flatten()
         return scores
 
+    def predict_missing_relations(self, head_entity: Union[List[str], str], tail_entity: Union[List[str], str],
+                                  within=None, batch_size=2, topk=1, return_indices=False):
+        """Scores (or the top-k) of every relation x for (h, x, t); pairs ordered heads-major
+        (``cartesian_prod(head, tail)``), every (h, x, t) triple scored by ``forward_triples`` (:229-312)."""
+        if within is not None:
+            raise NotImplementedError("`within` needs the byte-pair-encoded path, which is outside this build")
+        head = torch.LongTensor([self.entity_to_idx[i] for i in
+                                 (head_entity if isinstance(head_entity, list) else [head_entity])])
+        tail = torch.LongTensor([self.entity_to_idx[i] for i in
+                                 (tail_entity if isinstance(tail_entity, list) else [tail_entity])])
+        ht_pairs = torch.cartesian_prod(head, tail).view(-1, 2)
+        P, R = ht_pairs.size(0), self.num_relations
+        dev = self.model.entity_embeddings.weight.device
+        relation = torch.arange(0, R)
+        if return_indices:
+            scores = torch.zeros(P, topk)
+            indices = torch.zeros(P, topk, dtype=torch.long)
+        else:
+            scores = torch.zeros(P * R)
+        for i in range(0, P, batch_size):
+            batch = ht_pairs[i:i + batch_size]
+            B = batch.size(0)
+            triples = torch.stack([batch[:, 0].repeat_interleave(R), relation.repeat(B),
+                                   batch[:, 1].repeat_interleave(R)], dim=1).to(dev)
+            with torch.no_grad():
+                batch_scores = self.model.forward_triples(triples).view(B, R)
+            if return_indices:
+                s, idx = torch.topk(batch_scores, topk, dim=1)
+                scores[i:i + batch_size, :] = s.cpu()
+                indices[i:i + batch_size, :] = idx.cpu()
+            else:
+                scores[i * R:i * R + B * R] = batch_scores.flatten().cpu()
+        if return_indices:
+            return scores.flatten(), indices.flatten()
+        return scores
+
     def predict(self, *, h: Union[List[str], str] = None, r: Union[List[str], str] = None,
                 t: Union[List[str], str] = None, within=None, logits=True) -> torch.FloatTensor:
         if h is not None:
@@ -127,7 +163,8 @@ class KGE:
             assert r is not None and t is not None
             scores = self.predict_missing_head_entity(r, t, within)
         elif r is None:
-            raise NotImplementedError("relation prediction is outside the accelerated path")
+            assert h is not None and t is not None
+            scores = self.predict_missing_relations(h, t, within)
         elif t is None:
             scores = self.predict_missing_tail_entity(h, r, within)
         else:
@@ -166,7 +203,16 @@ class KGE:
                                                                          return_indices=True)
             num_hr_pairs = len(r) * len(t)
         elif r is None:
-            raise NotImplementedError("relation prediction is outside the accelerated path")
+            assert h is not None and t is not None
+            flat_scores, flat_indices = self.predict_missing_relations(h, t, within, batch_size, topk,
+                                                                       return_indices=True)
+            h = [h] if isinstance(h, str) else h
+            t = [t] if isinstance(t, str) else t
+            num_hr_pairs = len(h) * len(t)
+            scores_2d = flat_scores.view(num_hr_pairs, topk)
+            indices_2d = flat_indices.view(num_hr_pairs, topk)
+            return [[(self.idx_to_relations[idx], score) for idx, score in zip(row_idxs, row_scores)]
+                    for row_idxs, row_scores in zip(indices_2d.tolist(), torch.sigmoid(scores_2d).tolist())]
         elif t is not None:
             raise AttributeError("Use triple_score method")
         else:

@@ -298,8 +298,15 @@ def test_predict_missing_head():
     ok, worst = score_close(full.numpy()[None, :], S[:1], 1e-5)
     assert ok, worst
     assert kge.predict_topk(r="r3", t="e10", topk=5)[0] == top[0]
-    with pytest.raises(NotImplementedError):
-        kge.predict_topk(h=["e1"], t=["e2"])
+    # missing relation: every (h, x, t) scored as a triple
+    rel_top = kge.predict_topk(h=["e1", "e5"], t=["e2"], topk=3)
+    trip = np.array([[hh, x, 2] for hh in (1, 5) for x in range(46)])
+    ref_r = ko.triple_scores("ComplEx", E, Rel, trip).reshape(2, 46)
+    for row, want_row in zip(rel_top, ref_r):
+        order = np.argsort(-want_row, kind="stable")[:3]
+        assert [rels[name] for name, _ in row] == order.tolist()
+        np.testing.assert_allclose([p for _, p in row], ko.sigmoid(want_row[order]), rtol=1e-5)
+    assert kge.predict(h=["e1"], t=["e2"]).shape == (46,)
     # reciprocal vocabulary: the head question is asked as a tail question with r_inverse
     rels2 = {f"r{i}": i for i in range(23)}
     rels2.update({f"r{i}_inverse": 23 + i for i in range(23)})
