@@ -499,3 +499,71 @@ def test_build_query_head_argument_checks(ops):
     with pytest.raises(KgeError) as err:
         ops.build_query("ComplEx", Eg, Rg, dev(torch.from_numpy(rt)), head=True, norm=norm)
     assert err.value.code == 2
+
+
+# ---------------------------------------------------------------------------------------------
+# seeded sweep over awkward shapes: every fused epilogue against the library's own materialised scores
+# ---------------------------------------------------------------------------------------------
+def _sweep_cases():
+    rng = np.random.default_rng(2024)
+    cases = []
+    for i in range(36):
+        storage = ("fp32", "bf16", "int8")[i % 3]
+        if storage == "fp32":
+            d = int(rng.choice([1, 3, 4, 8, 20, 33, 64, 100, 200]))
+        elif storage == "bf16":
+            d = int(rng.choice([8, 16, 40, 64, 128]))
+        else:
+            d = int(rng.choice([16, 32, 64, 128]))
+        N = int(rng.choice([1, 2, 31, 32, 33, 127, 128, 129, 257, 1000, 1025, 4097]))
+        B = int(rng.choice([1, 2, 63, 64, 65, 255, 257, 513]))
+        cases.append((i, storage, d, N, B))
+    return cases
+
+
+@pytest.mark.parametrize("seed,storage,d,N,B", _sweep_cases())
+def test_shape_sweep_all_epilogues_agree_with_materialised_scores(ops, FilterCSR, seed, storage, d, N, B):
+    rng = np.random.default_rng(seed)
+    R = 3
+    E, Rel = random_tables(rng, N, R, d)
+    if N >= 3:
+        E[N - 1] = E[0]                                               # an exact tie at the table's last row
+    hr = random_hr(rng, N, R, B)
+    Et, sc, Rt, Ev, Rv = stored_tables(E, Rel, storage)
+    Eg, scg = dev(Et), dev(sc)
+    hr_g = dev(torch.from_numpy(hr))
+    Q, bias = ops.build_query("DistMult", Eg, dev(Rt), hr_g, ent_scale=scg)
+    S = ops.scores(Q, bias, Eg, scg)
+    assert S.shape == (B, N)
+    S_raw = ops.scores(Q, None, Eg, scg).cpu().numpy()
+    ref = ko.k_vs_all_scores("DistMult", Ev, Rv, hr)
+    # with a handful of entities a row has no typical score size to measure against: bound the error by the
+    # sizes of the two vectors instead (rounding both to bf16 perturbs a dot product by < 2^-8 |q| |e|)
+    qn = np.linalg.norm(Ev[hr[:, 0]] * Rv[hr[:, 1]], axis=1)[:, None] * np.linalg.norm(Ev, axis=1)[None, :]
+    assert np.all(np.abs(S.cpu().numpy() - ref) <= RTOL[storage] * np.maximum(qn, np.abs(ref)) + 1e-30)
+    # filtered rank
+    targets = rng.integers(0, N, B).astype(np.int64)
+    er = random_csr(rng, hr, targets, N, R, max_len=min(6, N))
+    csr = FilterCSR.from_er_vocab(er, R, device="cuda")
+    out = ops.rank_filtered(Q, bias, Eg, scg, dev(torch.from_numpy(targets)), csr.rows_for(hr_g), csr.row_ptr, csr.col)
+    g, t, tl = _expected_counts(S_raw, targets, [er[(int(h), int(r))] for h, r in hr])
+    np.testing.assert_array_equal(out["n_greater"].cpu().numpy(), g)
+    np.testing.assert_array_equal(out["n_equal"].cpu().numpy(), t)
+    np.testing.assert_array_equal(out["n_equal_lower"].cpu().numpy(), tl)
+    # top-k, k up to N
+    k = int(min(N, rng.choice([1, 2, 10, 100])))
+    vals, idx = ops.topk(Q, bias, Eg, scg, k)
+    wv, wi = ko.topk(S.cpu().numpy(), k)
+    np.testing.assert_array_equal(idx.cpu().numpy(), wi)
+    np.testing.assert_array_equal(vals.cpu().numpy(), wv)
+    # row extrema and one given entity per query
+    lo, hi = ops.row_minmax(Q, bias, Eg, scg)
+    np.testing.assert_array_equal(lo.cpu().numpy(), S.cpu().numpy().min(1))
+    np.testing.assert_array_equal(hi.cpu().numpy(), S.cpu().numpy().max(1))
+    one = ops.triple_scores(Q, bias, Eg, scg, dev(torch.from_numpy(targets)))
+    np.testing.assert_array_equal(one.cpu().numpy(), S.cpu().numpy()[np.arange(B), targets])
+    # BCE against the dense closed form on the library's scores (fp64 sum)
+    pos = [sorted(set(er[(int(h), int(r))])) for h, r in hr]
+    loss = ops.bce_multihot(Q, bias, Eg, scg, csr.rows_for(hr_g), csr.row_ptr, csr.col, 0.0)[0].item()
+    want = ko.bce_multihot(S.cpu().numpy().astype(np.float64), pos)
+    assert loss == pytest.approx(want, rel=1e-4, abs=1e-6)
