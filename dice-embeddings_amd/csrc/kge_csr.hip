@@ -184,6 +184,7 @@ extern "C" int kge_csr_build(const int64_t* triples, int64_t n, int col_a, int c
   KGE_REQUIRE(need != 0, KGE_ERR_HIP, "kge_csr_build: no HIP device to size the sort for");
   KGE_REQUIRE(workspace && workspace_bytes >= need, KGE_ERR_WORKSPACE, "kge_csr_build: workspace of %zu bytes, need %zu",
               workspace_bytes, need);
+  KGE_REQUIRE(((uintptr_t)workspace & 7) == 0, KGE_ERR_WORKSPACE, "kge_csr_build: workspace must be 8-byte aligned");
   const unsigned grid = (unsigned)((n + 255) / 256 < 4096 ? (n + 255) / 256 : 4096);
   const unsigned long long invalid = 1ull << key_bits;
   hipLaunchKernelGGL(csr_pack_kernel, dim3(grid), dim3(256), 0, st, triples, n, col_a, col_b, col_v, range_a, range_b,

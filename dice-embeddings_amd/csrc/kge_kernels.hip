@@ -1030,6 +1030,7 @@ extern "C" int kge_rank_filtered(const float* Q, const float* bias, const void* 
   KGE_REQUIRE(n_rows < 0x7fffffffLL, KGE_ERR_INVALID, "kge_rank_filtered: n_rows=%lld too large", (long long)n_rows);
   KGE_REQUIRE(workspace && workspace_bytes >= kge_rank_workspace_bytes(B), KGE_ERR_WORKSPACE,
               "kge_rank_filtered: workspace of %zu bytes, need %zu", workspace_bytes, kge_rank_workspace_bytes(B));
+  KGE_REQUIRE(((uintptr_t)workspace & 7) == 0, KGE_ERR_WORKSPACE, "kge_rank_filtered: workspace must be 8-byte aligned");
   hipStream_t st = (hipStream_t)stream;
   RankWs ws;
   rank_ws_layout(B, workspace, &ws);
@@ -1079,6 +1080,7 @@ extern "C" int kge_topk(const float* Q, const float* bias, const void* E, int dt
   KGE_REQUIRE(out_scores && out_idx, KGE_ERR_INVALID, "kge_topk: null output pointer");
   KGE_REQUIRE(workspace && workspace_bytes >= kge_topk_workspace_bytes(B, N, k), KGE_ERR_WORKSPACE,
               "kge_topk: workspace of %zu bytes, need %zu", workspace_bytes, kge_topk_workspace_bytes(B, N, k));
+  KGE_REQUIRE(((uintptr_t)workspace & 7) == 0, KGE_ERR_WORKSPACE, "kge_topk: workspace must be 8-byte aligned");
   hipStream_t st = (hipStream_t)stream;
   TopkWs ws;
   topk_ws_layout(B, k, workspace, &ws);
