@@ -19,6 +19,14 @@
 #ifndef KGE_SCHED_HINTS
 #define KGE_SCHED_HINTS 0
 #endif
+#ifndef KGE_KS_SCHED
+#define KGE_KS_SCHED 1
+#endif
+// 1: fp32 tables are multiplied on the bf16 MFMA as three bf16 parts per operand (ksplit_kernel);
+// 0: on the fp32 MFMA (kloop_async_kernel / kloop_kernel).  One switch for every kernel that forms a score.
+#ifndef KGE_F32_SPLIT
+#define KGE_F32_SPLIT 1
+#endif
 
 namespace kge {
 
@@ -47,6 +55,46 @@ __device__ __forceinline__ bf16x8 cvt_bf16x8(f32x4 lo, f32x4 hi) {
   r[0] = (__bf16)lo[0]; r[1] = (__bf16)lo[1]; r[2] = (__bf16)lo[2]; r[3] = (__bf16)lo[3];
   r[4] = (__bf16)hi[0]; r[5] = (__bf16)hi[1]; r[6] = (__bf16)hi[2]; r[7] = (__bf16)hi[3];
   return r;
+}
+
+// fp32 through the bf16 MFMA: x = x1 + x2 + x3 with three bf16 parts (8 + 8 + 8 mantissa bits: exact
+// unless the residual underflows), and a product x * y is taken as the six leading part products
+//   x1 y1, x1 y2, x2 y1, x1 y3, x2 y2, x3 y1      (the dropped ones are below 2^-24 of x y)
+// each exact in fp32 and summed by the MFMA's fp32 accumulator.  SPLIT_A / SPLIT_B give the parts of
+// the two operands for product p; every kernel that forms a score uses this order.
+constexpr int SPLIT_PRODUCTS = 6;
+__device__ constexpr int SPLIT_A[SPLIT_PRODUCTS] = {0, 0, 1, 0, 1, 2};
+__device__ constexpr int SPLIT_B[SPLIT_PRODUCTS] = {0, 1, 0, 2, 1, 0};
+// One pair: round both to bf16 (nearest even, one packed instruction), return the packed pair and leave the
+// residuals in r0, r1 (exact: a residual fits fp32).
+__device__ __forceinline__ uint32_t split_step(float& r0, float& r1) {
+  typedef __attribute__((ext_vector_type(2))) float f32x2;
+  typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+  const uint32_t pk = __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2{r0, r1}, bf16x2));
+  r0 = r0 - __uint_as_float(pk << 16);
+  r1 = r1 - __uint_as_float(pk & 0xffff0000u);
+  return pk;
+}
+__device__ __forceinline__ void split3_bf16x8(f32x4 lo, f32x4 hi, bf16x8 (&s)[3]) {
+  float r[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+#pragma unroll
+  for (int part = 0; part < 3; ++part) {
+    u32x4 w;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) w[j] = split_step(r[2 * j], r[2 * j + 1]);
+    s[part] = __builtin_bit_cast(bf16x8, w);
+  }
+}
+// the same split for four values
+__device__ __forceinline__ void split3_bf16x4(f32x4 v, bf16x4 (&s)[3]) {
+  float r[4] = {v[0], v[1], v[2], v[3]};
+#pragma unroll
+  for (int part = 0; part < 3; ++part) {
+    uint32_t w[2];
+#pragma unroll
+    for (int j = 0; j < 2; ++j) w[j] = split_step(r[2 * j], r[2 * j + 1]);
+    s[part] = __builtin_bit_cast(bf16x4, w);
+  }
 }
 
 // two int8 (bytes `lo`,`hi` of w selected by shift) -> packed pair of bf16; exact for |v| <= 127
@@ -1118,6 +1166,9 @@ __global__ void __launch_bounds__(256, 2) kloop_kernel(ContractArgs a, typename 
             acc[te][tq] = Epi::SWAP ? mfma_f32(fq[tq][j], fe[te][j], acc[te][tq])
                                     : mfma_f32(fe[te][j], fq[tq][j], acc[te][tq]);
     }
+#ifndef KGE_DBG_NO_SCHEDBAR
+    __builtin_amdgcn_sched_barrier(0);  // ... and waited for after them
+#endif
 #ifndef KGE_DBG_NO_LDSWRITE
     if (it + 1 < n_it) chunk_store(buf ^ 1);
 #endif
@@ -1291,6 +1342,206 @@ __global__ void __launch_bounds__(256, 2) kloop_async_kernel(ContractArgs a, typ
       et0 += KLOOP_TILE_ROWS;
     } else {
       ++kc;
+    }
+  }
+  epi.finish();
+}
+
+// ============================================================================================
+// ksplit_kernel: fp32 tables on the bf16 MFMA (split3_bf16x8).  256 entities x 128 queries per
+// workgroup of 8 waves (each wave 64 x 64), K in chunks of 32.  Both operands are loaded as fp32 into
+// registers while the previous chunk is multiplied, split into their three bf16 parts and stored as
+// three planes per operand in LDS; per 16-wide K step a wave reads 12 fragments and issues 24 MFMAs.
+// Chain order per score: K steps of 16 ascending, inside a step the six products in SPLIT order.
+//
+// LDS plane layout: row r is 64 B = 4 pieces of 16 B (8 bf16); piece p sits in slot
+// r*4 + (p ^ ((r >> 2) & 3)), so the 16 rows a fragment read touches at a time spread over all banks.
+// ============================================================================================
+constexpr int KS_NQT = 2;
+constexpr int KS_WG_QUERIES = 128;
+constexpr int KS_TILE_ROWS = 256;
+constexpr int KS_KC = 32;
+constexpr int KS_E_PLANE = KS_TILE_ROWS * 64;
+constexpr int KS_Q_PLANE = KS_WG_QUERIES * 64;
+constexpr int KS_STAGE_BYTES = 3 * KS_E_PLANE + 3 * KS_Q_PLANE;
+
+template <template <int> class EpiT, bool VEC>
+__global__ void __launch_bounds__(512, 2) ksplit_kernel(ContractArgs a, typename EpiT<KS_NQT>::Args ea) {
+  using Epi = EpiT<KS_NQT>;
+  __shared__ __attribute__((aligned(1024))) unsigned char lds[2 * KS_STAGE_BYTES];
+
+  int qg;
+  int64_t chunk;
+  if (!decompose_wg(a, qg, chunk)) return;
+  const int tid = threadIdx.x, lane = tid & 63, c = lane & 31, hf = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int we = wave >> 1, wq = wave & 1;
+  const int d = a.d;
+  const int64_t q_base = (int64_t)qg * KS_WG_QUERIES;
+  const int64_t q0 = q_base + 64 * wq;
+  Epi epi;
+  epi.init(ea, q0, c, hf, a.B);
+  __shared__ typename Epi::Shared epi_sh;
+  epi.bind(&epi_sh);
+
+  const int64_t r0 = a.e_begin + chunk * a.chunk_rows;
+  const int64_t r1 = (r0 + a.chunk_rows < a.e_end) ? r0 + a.chunk_rows : a.e_end;
+  const int nkc = (d + KS_KC - 1) / KS_KC;
+  const int n_et = (int)((r1 - r0 + KS_TILE_ROWS - 1) / KS_TILE_ROWS);
+  const int n_it = n_et * nkc;
+  const float* Ef = (const float*)a.E;
+
+  // Staging: a chunk is 384 rows (256 entity rows, then 128 query rows) of 128 B, taken in six passes of
+  // 64 rows; in pass g thread tid takes 16 B piece (tid & 7) of row 64 g + tid / 8, so eight neighbouring
+  // lanes read one whole 128 B line.  Loads are branch-free so that all six stay in flight: rows past the
+  // end repeat the last valid row (epilogues ignore them), columns past d are read from a clamped address
+  // and zeroed when stored.  Pass g of chunk i+2 is loaded right after pass g of chunk i+1 has been split
+  // and stored, both while chunk i is multiplied: one register set, and a whole iteration for a load to land.
+  const int s_row = tid >> 3, s_piece = tid & 7;
+  const int64_t q_last = a.B - 1, e_last = r1 - 1;
+  const float* q_ptr[2];
+#pragma unroll
+  for (int g = 0; g < 2; ++g) {
+    int64_t qr = q_base + 64 * g + s_row;
+    qr = qr < q_last ? qr : q_last;
+    q_ptr[g] = a.Q + qr * d;
+  }
+  f32x4 staged[6];             // passes 0..3: entity rows, 4..5: query rows
+  int st_valid = 0;            // how many of this thread's four columns of the staged chunk are inside d
+  int ld_valid = 0, ld_k = 0;  // the same, and the first column, for the chunk being loaded
+  int ld_kc = 0;               // K chunk and first row of the tile the next loads fetch
+  int64_t ld_row = r0 + s_row;
+  auto load_begin = [&]() {
+    ld_k = ld_kc * KS_KC + 4 * s_piece;
+    ld_valid = d - ld_k;
+  };
+  auto load_pass = [&](int g) {
+    const float* row_ptr;
+    if (g < 4) {
+      int64_t er = ld_row + 64 * g;
+      er = er < e_last ? er : e_last;
+      row_ptr = Ef + er * d;
+    } else {
+      row_ptr = q_ptr[g - 4];
+    }
+    if constexpr (VEC) {
+      staged[g] = *(const f32x4*)(row_ptr + (ld_k < d ? ld_k : 0));
+    } else {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) staged[g][j] = row_ptr[ld_k + j < d ? ld_k + j : 0];
+    }
+  };
+  auto load_end = [&]() {
+    const bool wrap = (ld_kc == nkc - 1);
+    ld_kc = wrap ? 0 : ld_kc + 1;
+    ld_row += wrap ? KS_TILE_ROWS : 0;
+    st_valid = ld_valid;
+  };
+  // 8-byte half (s_piece & 1) of 16-byte piece (s_piece >> 1); rows 64 g + s_row share the swizzle of s_row
+  const int st_off = s_row * 64 + ((((s_piece >> 1) ^ ((s_row >> 2) & 3)) << 4) | ((s_piece & 1) << 3));
+  auto store_pass = [&](int buf, int g) {
+    unsigned char* base = lds + buf * KS_STAGE_BYTES + st_off +
+                          (g < 4 ? g * 4096 : 3 * KS_E_PLANE + (g - 4) * 4096);
+    const int plane = g < 4 ? KS_E_PLANE : KS_Q_PLANE;
+    f32x4 v = staged[g];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) v[j] = (j < st_valid) ? v[j] : 0.f;
+    bf16x4 s[3];
+    split3_bf16x4(v, s);
+#pragma unroll
+    for (int part = 0; part < 3; ++part) *(bf16x4*)(base + part * plane) = s[part];
+  };
+
+  // fragment offsets of this lane inside a plane (row c of a 32-row tile), per K step of the chunk
+  int foff[KS_KC / 16];
+#pragma unroll
+  for (int ks = 0; ks < KS_KC / 16; ++ks) foff[ks] = c * 64 + (((2 * ks + hf) ^ ((c >> 2) & 3)) << 4);
+
+  f32x16 acc[2][2];
+#pragma unroll
+  for (int te = 0; te < 2; ++te)
+#pragma unroll
+    for (int tq = 0; tq < 2; ++tq)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc[te][tq][i] = 0.f;
+
+  if (n_it > 0) {
+    load_begin();
+#pragma unroll
+    for (int g = 0; g < 6; ++g) load_pass(g);
+    load_end();
+    load_begin();
+#pragma unroll
+    for (int g = 0; g < 6; ++g) {
+      store_pass(0, g);
+      load_pass(g);  // past the last chunk the clamped addresses still point into the tables
+    }
+    load_end();
+  }
+  __syncthreads();
+  int kc = 0;
+  int64_t et0 = r0;
+  for (int it = 0; it < n_it; ++it) {
+    const int buf = it & 1;
+    const unsigned char* be = lds + buf * KS_STAGE_BYTES + (64 * we) * 64;
+    const unsigned char* bq = lds + buf * KS_STAGE_BYTES + 3 * KS_E_PLANE + (64 * wq) * 64;
+    bf16x8 fe[2][3][2], fq[2][3][2];
+    auto read_step = [&](int ks) {
+#pragma unroll
+      for (int part = 0; part < 3; ++part)
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+          fe[ks][part][t] = *(const bf16x8*)(be + part * KS_E_PLANE + t * 2048 + foff[ks]);
+          fq[ks][part][t] = *(const bf16x8*)(bq + part * KS_Q_PLANE + t * 2048 + foff[ks]);
+        }
+    };
+    // The iteration in six slices, fenced so that each keeps its share of the work: eight of the chunk's
+    // 48 MFMAs, and the split + store of one staged pass of chunk it+1 followed by the load of that pass of
+    // chunk it+2.  Unconditional on purpose (no branches inside the iteration): after the last chunk this
+    // stores and loads a chunk nobody reads.
+    read_step(0);
+    load_begin();
+#pragma unroll
+    for (int sl = 0; sl < 6; ++sl) {
+      if (sl == 2) read_step(1);
+#ifndef KGE_DBG_NO_LDSWRITE
+      store_pass(buf ^ 1, sl);
+#endif
+#ifndef KGE_DBG_NO_GLOBAL
+      load_pass(sl);
+#endif
+#pragma unroll
+      for (int m = 8 * sl; m < 8 * sl + 8; ++m) {
+        const int ks = m / 24, p = (m % 24) / 4, te = (m >> 1) & 1, tq = m & 1;
+        acc[te][tq] = Epi::SWAP ? mfma_bf16(fq[ks][SPLIT_B[p]][tq], fe[ks][SPLIT_A[p]][te], acc[te][tq])
+                                : mfma_bf16(fe[ks][SPLIT_A[p]][te], fq[ks][SPLIT_B[p]][tq], acc[te][tq]);
+      }
+#if KGE_KS_SCHED
+      __builtin_amdgcn_sched_barrier(0);
+#endif
+    }
+    load_end();
+    if (kc == nkc - 1) {  // this entity tile is complete
+      float sc16[16];
+#pragma unroll
+      for (int te = 0; te < 2; ++te) {
+        const int64_t e_base = et0 + 64 * we + 32 * te;
+        if (e_base < r1) {
+#pragma unroll
+          for (int tq = 0; tq < 2; ++tq) epi.template tile<false>(tq, acc[te][tq], sc16, 1.f, e_base, r1);
+        }
+#pragma unroll
+        for (int tq = 0; tq < 2; ++tq)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) acc[te][tq][i] = 0.f;
+      }
+      kc = 0;
+      et0 += KS_TILE_ROWS;
+      __syncthreads();
+      if (Epi::STAGE_HOOK) epi.stage_end();
+    } else {
+      ++kc;
+      __syncthreads();
     }
   }
   epi.finish();

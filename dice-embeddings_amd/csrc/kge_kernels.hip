@@ -39,6 +39,49 @@ __device__ __forceinline__ f32x16 chain_direct(const void* E, int d, int64_t e_r
   f32x16 acc;
 #pragma unroll
   for (int i = 0; i < 16; ++i) acc[i] = 0.f;
+#if KGE_F32_SPLIT
+  if (EDT == KGE_F32) {
+    // fp32 rows on the bf16 MFMA: both rows split into three bf16 parts, six products per K step of 16
+    // (the order of ksplit_kernel).  Four K steps per trip: all sixteen loads are issued first.
+    const float* Ef = (const float*)E;
+    const bool vec_ok = (d & 3) == 0;
+    const int nks = (d + 15) >> 4;
+    for (int ks0 = 0; ks0 < nks; ks0 += 4) {
+      f32x4 fe[4][2], fq[4][2];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+          const int k = (ks0 + u) * 16 + 8 * hf + 4 * h;
+          fe[u][h] = f32x4{0.f, 0.f, 0.f, 0.f};
+          fq[u][h] = f32x4{0.f, 0.f, 0.f, 0.f};
+          if (vec_ok) {
+            if (k < d) {
+              if (e_row >= 0) fe[u][h] = *(const f32x4*)(Ef + e_row * d + k);
+              if (q_row >= 0) fq[u][h] = *(const f32x4*)(Q + q_row * d + k);
+            }
+          } else {
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+              if (k + j < d) {
+                if (e_row >= 0) fe[u][h][j] = Ef[e_row * d + k + j];
+                if (q_row >= 0) fq[u][h][j] = Q[q_row * d + k + j];
+              }
+          }
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        if (ks0 + u < nks) {  // uniform: whole K steps past d are skipped (they would only add zeros)
+          bf16x8 se[3], sq[3];
+          split3_bf16x8(fe[u][0], fe[u][1], se);
+          split3_bf16x8(fq[u][0], fq[u][1], sq);
+#pragma unroll
+          for (int p = 0; p < SPLIT_PRODUCTS; ++p) acc = mfma_bf16(se[SPLIT_A[p]], sq[SPLIT_B[p]], acc);
+        }
+      }
+    }
+#else
   if (EDT == KGE_F32) {
     const float* Ef = (const float*)E;
     const bool vec_ok = (d & 3) == 0;
@@ -73,6 +116,7 @@ __device__ __forceinline__ f32x16 chain_direct(const void* E, int d, int64_t e_r
         }
       }
     }
+#endif
   } else {
 #pragma unroll
     for (int s = 0; s < 8; ++s) {
@@ -808,7 +852,8 @@ ContractArgs make_args(const float* Q, const void* E, int dtype, const float* sc
   a.e_end = e_end;
   a.d = (int)d;
   const bool fast_bf16 = (dtype == KGE_BF16 && d == 128), fast_i8 = (dtype == KGE_I8 && d == 128);
-  const int wgq = (dtype == KGE_F32) ? KLOOP_WG_QUERIES : fast_bf16 ? QA_WG_QUERIES : fast_i8 ? I8_WG_QUERIES : QREG_WG_QUERIES;
+  const int f32_wgq = KGE_F32_SPLIT ? KS_WG_QUERIES : KLOOP_WG_QUERIES;
+  const int wgq = (dtype == KGE_F32) ? f32_wgq : fast_bf16 ? QA_WG_QUERIES : fast_i8 ? I8_WG_QUERIES : QREG_WG_QUERIES;
   a.n_qgroups = (int)((B + wgq - 1) / wgq);
   if (a.n_qgroups < 1) a.n_qgroups = 1;
   const int64_t rows = e_end - e_begin;
@@ -826,18 +871,20 @@ ContractArgs make_args(const float* Q, const void* E, int dtype, const float* sc
     a.n_chunks = (rows + chunk - 1) / chunk;
     return a;
   }
-  // non-persistent paths: one workgroup per (query group, chunk).  512 workgroups are resident at a
-  // time (2 per CU); choose the chunk length whose last round of workgroups is fullest, preferring
-  // longer chunks (less per-workgroup set-up) among near-equal candidates.
-  const int tile = (dtype == KGE_F32) ? KLOOP_TILE_ROWS : QREG_STAGE_ROWS;
+  // non-persistent paths: one workgroup per (query group, chunk).  `resident` workgroups run at a time
+  // (2 per CU, or 1 per CU for the 8-wave split kernel); choose the chunk length whose last round of
+  // workgroups is fullest, preferring longer chunks (less per-workgroup set-up) among near-equal candidates.
+  const bool f32_split = (dtype == KGE_F32) && KGE_F32_SPLIT;
+  const int tile = f32_split ? KS_TILE_ROWS : (dtype == KGE_F32) ? KLOOP_TILE_ROWS : QREG_STAGE_ROWS;
   const int max_chunk = (dtype == KGE_F32) ? 1024 : 2048;
+  const int64_t resident = f32_split ? 256 : 512;
   int64_t best_chunk = tile;
   double best_eff = -1.0;
   for (int64_t chunk = tile; chunk <= max_chunk; chunk += tile) {
     const int64_t n_chunks = (rows + chunk - 1) / chunk;
     const int64_t wgs = (n_chunks + 7) / 8 * 8 * a.n_qgroups;
-    const int64_t rounds = (wgs + 511) / 512;
-    const double eff = (double)rows * a.n_qgroups / ((double)rounds * 512.0 * (double)chunk);
+    const int64_t rounds = (wgs + resident - 1) / resident;
+    const double eff = (double)rows * a.n_qgroups / ((double)rounds * (double)resident * (double)chunk);
     if (eff > best_eff + 0.02) {
       best_eff = eff;
       best_chunk = chunk;
@@ -858,7 +905,8 @@ int launch_contract(int dtype, const ContractArgs& a, const EArgs& ea, hipStream
   const bool persistent = (dtype == KGE_BF16 && a.d == 128) || fast_i8;
   const int64_t nwg = persistent ? 8 * (int64_t)a.n_qgroups * a.n_lanes : (a.n_chunks + 7) / 8 * 8 * a.n_qgroups;
   KGE_REQUIRE(nwg <= 0x7fffffffLL, KGE_ERR_INVALID, "%s: grid of %lld workgroups too large", name, (long long)nwg);
-  dim3 grid((unsigned)nwg), block(fast_i8 ? 64 * I8_WG_WAVES : persistent ? 64 * QA_WG_WAVES : 256);
+  const bool f32_split = (dtype == KGE_F32) && KGE_F32_SPLIT;
+  dim3 grid((unsigned)nwg), block(fast_i8 ? 64 * I8_WG_WAVES : persistent ? 64 * QA_WG_WAVES : f32_split ? 512 : 256);
   hipEvent_t ev0 = nullptr, ev1 = nullptr;
   bool timed = false;
   {
@@ -871,7 +919,11 @@ int launch_contract(int dtype, const ContractArgs& a, const EArgs& ea, hipStream
     KGE_HIP_CHECK(hipEventRecord(ev0, st));
   }
   const bool rows_aligned = (a.d % 4 == 0) && (((uintptr_t)a.E | (uintptr_t)a.Q) % 16 == 0);
-  if (dtype == KGE_F32 && rows_aligned)
+  if (f32_split && rows_aligned)
+    hipLaunchKernelGGL((ksplit_kernel<EpiT, true>), grid, block, 0, st, a, ea);
+  else if (f32_split)
+    hipLaunchKernelGGL((ksplit_kernel<EpiT, false>), grid, block, 0, st, a, ea);
+  else if (dtype == KGE_F32 && rows_aligned)
     hipLaunchKernelGGL((kloop_async_kernel<EpiT>), grid, block, 0, st, a, ea);
   else if (dtype == KGE_F32)
     hipLaunchKernelGGL((kloop_kernel<EpiT>), grid, block, 0, st, a, ea);
