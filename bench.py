@@ -34,7 +34,7 @@ FP32_MFMA_PEAK_TFLOPS = 157.3
 # workload (each scaled by what the same counter reads for a plain 1 GiB copy kernel: x2.00 and x1.00).
 MEASURED_TRAFFIC_BYTES = {"c4": 658.0e6,     # per rank launch
                           "c5": 323.0e6,     # average over the 8 launches of a top-k call (2.59 GB per call)
-                          "c3": 59.2e6, "c2": 19.4e6}
+                          "c3": 59.4e6, "c2": 19.4e6}
 MODE = {"c1": "rank", "c2": "rank", "c3": "bce", "c4": "rank", "c5": "topk"}
 
 

@@ -43,36 +43,48 @@ __device__ __forceinline__ f32x16 chain_direct(const void* E, int d, int64_t e_r
   if (EDT == KGE_F32) {
     // fp32 rows on the bf16 MFMA: both rows split into three bf16 parts, six products per K step of 16
     // (the order of ksplit_kernel).  Four K steps per trip: all sixteen loads are issued first.
-    const float* Ef = (const float*)E;
+    const bool e_ok = e_row >= 0, q_ok = q_row >= 0;
+    const float* e_ptr = (const float*)E + (e_ok ? e_row : 0) * d;
+    const float* q_ptr = Q + (q_ok ? q_row : 0) * d;
     const bool vec_ok = (d & 3) == 0;
     const int nks = (d + 15) >> 4;
-    for (int ks0 = 0; ks0 < nks; ks0 += 4) {
-      f32x4 fe[4][2], fq[4][2];
+    // Branch-free loads (a missing row or a column past d reads a clamped address and is zeroed after), so
+    // that the sixteen loads of a trip of four K steps are in flight together.
+    auto load_trip = [&](int ks0, f32x4 (&fe)[4][2], f32x4 (&fq)[4][2]) {
 #pragma unroll
       for (int u = 0; u < 4; ++u) {
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
           const int k = (ks0 + u) * 16 + 8 * hf + 4 * h;
-          fe[u][h] = f32x4{0.f, 0.f, 0.f, 0.f};
-          fq[u][h] = f32x4{0.f, 0.f, 0.f, 0.f};
           if (vec_ok) {
-            if (k < d) {
-              if (e_row >= 0) fe[u][h] = *(const f32x4*)(Ef + e_row * d + k);
-              if (q_row >= 0) fq[u][h] = *(const f32x4*)(Q + q_row * d + k);
-            }
+            const int kk = (k < d) ? k : 0;
+            fe[u][h] = *(const f32x4*)(e_ptr + kk);
+            fq[u][h] = *(const f32x4*)(q_ptr + kk);
           } else {
 #pragma unroll
-            for (int j = 0; j < 4; ++j)
-              if (k + j < d) {
-                if (e_row >= 0) fe[u][h][j] = Ef[e_row * d + k + j];
-                if (q_row >= 0) fq[u][h][j] = Q[q_row * d + k + j];
-              }
+            for (int j = 0; j < 4; ++j) {
+              const int kk = (k + j < d) ? k + j : 0;
+              fe[u][h][j] = e_ptr[kk];
+              fq[u][h][j] = q_ptr[kk];
+            }
           }
         }
       }
+    };
+    auto mul_trip = [&](int ks0, f32x4 (&fe)[4][2], f32x4 (&fq)[4][2]) {
 #pragma unroll
       for (int u = 0; u < 4; ++u) {
         if (ks0 + u < nks) {  // uniform: whole K steps past d are skipped (they would only add zeros)
+#pragma unroll
+          for (int h = 0; h < 2; ++h) {
+            const int k = (ks0 + u) * 16 + 8 * hf + 4 * h;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+              const bool in = k + j < d;
+              fe[u][h][j] = (in && e_ok) ? fe[u][h][j] : 0.f;
+              fq[u][h][j] = (in && q_ok) ? fq[u][h][j] : 0.f;
+            }
+          }
           bf16x8 se[3], sq[3];
           split3_bf16x8(fe[u][0], fe[u][1], se);
           split3_bf16x8(fq[u][0], fq[u][1], sq);
@@ -80,6 +92,13 @@ __device__ __forceinline__ f32x16 chain_direct(const void* E, int d, int64_t e_r
           for (int p = 0; p < SPLIT_PRODUCTS; ++p) acc = mfma_bf16(se[SPLIT_A[p]], sq[SPLIT_B[p]], acc);
         }
       }
+    };
+    // (Issuing the next trip's loads before this trip is multiplied was measured slower: the second register
+    // set costs the gather kernels more in occupancy than the overlap returns.)
+    for (int ks0 = 0; ks0 < nks; ks0 += 4) {
+      f32x4 fe[4][2], fq[4][2];
+      load_trip(ks0, fe, fq);
+      mul_trip(ks0, fe, fq);
     }
 #else
   if (EDT == KGE_F32) {

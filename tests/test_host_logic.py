@@ -171,3 +171,44 @@ def test_experiment_folder_round_trip_on_cpu(tmp_path):
         assert torch.equal(loaded.state_dict()[k], v)
     with pytest.raises(AssertionError):
         load_model(str(tmp_path / "missing"))
+
+
+def test_three_part_bf16_split_arithmetic():
+    """The arithmetic ksplit_kernel relies on, emulated in numpy: an fp32 value is the exact sum of three bf16
+    parts (round to nearest even, each part taken from what the previous ones left), and the six leading part
+    products summed in fp32 reproduce an fp32 dot product to a few units of 2^-24 of sum(|x||y|)."""
+    def bf16_rne(x):
+        u = x.astype(np.float32).view(np.uint32).astype(np.uint64)
+        u = (u + 0x7FFF + ((u >> 16) & 1)) & 0xFFFF0000
+        return u.astype(np.uint32).view(np.float32)
+
+    def split3(x):
+        parts, r = [], x.astype(np.float32)
+        for _ in range(3):
+            b = bf16_rne(r)
+            parts.append(b)
+            r = (r - b).astype(np.float32)
+        return parts, r
+
+    rng = np.random.default_rng(7)
+    x = (rng.standard_normal(4096) * np.exp(rng.uniform(-8, 8, 4096))).astype(np.float32)
+    parts, rest = split3(x)
+    assert np.all(rest == 0)                                                 # 3 x 8 significant bits cover fp32's 24
+    assert np.array_equal((parts[0].astype(np.float64) + parts[1] + parts[2]).astype(np.float32), x)
+    d, n = 256, 64
+    X = rng.standard_normal((n, d)).astype(np.float32)
+    Y = rng.standard_normal((n, d)).astype(np.float32)
+    px, _ = split3(X)
+    py, _ = split3(Y)
+    order = [(0, 0), (0, 1), (1, 0), (0, 2), (1, 1), (2, 0)]                 # SPLIT_A / SPLIT_B of the kernels
+    acc = np.zeros(n, np.float32)
+    for k0 in range(0, d, 16):                                               # K steps of 16, fp32 accumulation
+        for a, b in order:
+            acc = (acc + np.einsum("nk,nk->n", px[a][:, k0:k0 + 16].astype(np.float64),
+                                   py[b][:, k0:k0 + 16].astype(np.float64)).astype(np.float32)).astype(np.float32)
+    exact = np.einsum("nk,nk->n", X.astype(np.float64), Y.astype(np.float64))
+    scale = np.einsum("nk,nk->n", np.abs(X).astype(np.float64), np.abs(Y).astype(np.float64))
+    assert np.max(np.abs(acc - exact) / scale) < 2.0 ** -21
+    dropped = sum(np.einsum("nk,nk->n", px[a].astype(np.float64), py[b].astype(np.float64))
+                  for a, b in [(1, 2), (2, 1), (2, 2)])
+    assert np.max(np.abs(dropped) / scale) < 2.0 ** -24
