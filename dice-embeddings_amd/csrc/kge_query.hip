@@ -18,12 +18,13 @@ struct QueryArgs {
   const void* rel;
   const float* coeff_p;
   const float* coeff_q;
+  const float* coeff_r;
   const int64_t* hr;
   float* Q;
   float* bias;
   kge_norm_params norm;
   int64_t B, N, R;
-  int d, p, q, normalize_relation;
+  int d, p, q, r, normalize_relation;
   int head_mode;  // pairs are (relation, tail) and Q is the head-direction query
 };
 
@@ -168,12 +169,13 @@ __global__ void __launch_bounds__(64) build_query_kernel(QueryArgs a, int model)
 #pragma unroll
       for (int i = 0; i < 8; ++i) q[g + i * d8] = o[i];
     }
-  } else if (a.head_mode) {  // KGE_KECI, head direction: sh holds the tail row (its parts are not scaled)
-    const int p = a.p, qn = a.q;
-    const int r = d / (p + qn + 1);
-    const int qoff = r + r * p;
+  } else if (a.head_mode) {  // KGE_KECI / KGE_DECAL, head direction: sh holds the tail row (its parts are not scaled)
+    const int p = a.p, qn = a.q, kn = a.r;
+    const int r = d / (p + qn + kn + 1);
+    const int qoff = r + r * p, koff = qoff + r * qn;
     for (int k = lane; k < r * p; k += 64) sr[r + k] *= a.coeff_p[k % p];
     for (int k = lane; k < r * qn; k += 64) sr[qoff + k] *= a.coeff_q[k % qn];
+    for (int k = lane; k < r * kn; k += 64) sr[koff + k] *= a.coeff_r[k % kn];
     __syncthreads();
     for (int rho = lane; rho < r; rho += 64) {
       const float t0 = sh[rho], r0 = sr[rho];
@@ -181,7 +183,9 @@ __global__ void __launch_bounds__(64) build_query_kernel(QueryArgs a, int model)
       const float* rp = sr + r + rho * p;
       const float* tq = sh + qoff + rho * qn;
       const float* rq = sr + qoff + rho * qn;
-      float q0 = r0 * t0, sum_rp = 0.f, sum_rq = 0.f;
+      const float* tk = sh + koff + rho * kn;
+      const float* rk = sr + koff + rho * kn;
+      float q0 = r0 * t0, sum_rp = 0.f, sum_rq = 0.f, sum_rk = 0.f;
       for (int i = 0; i < p; ++i) {
         q0 += rp[i] * tp[i];
         sum_rp += rp[i];
@@ -190,13 +194,18 @@ __global__ void __launch_bounds__(64) build_query_kernel(QueryArgs a, int model)
         q0 += rq[j] * tq[j];
         sum_rq += rq[j];
       }
+      for (int l = 0; l < kn; ++l) {
+        q0 += rk[l] * tk[l];
+        sum_rk += rk[l];
+      }
       q[rho] = q0;
-      const bool pq = p >= 2 && qn >= 2;
+      const bool pq = p >= 2 && qn >= 2, pr = p >= 2 && kn >= 2, qr = qn >= 2 && kn >= 2;
       float before = 0.f;  // sum of rp[k], k < i
       for (int i = 0; i < p; ++i) {
         float v = rp[i] * t0 + r0 * tp[i];
         if (p >= 2) v += (sum_rp - before - rp[i]) - before;  // d sigma_pp / d hp_i
         if (pq) v += sum_rq;                                   // d sigma_pq / d hp_i
+        if (pr) v += sum_rk;                                   // d sigma_pr / d hp_i
         q[r + rho * p + i] = v * a.coeff_p[i];                 // the head's own part is scaled too
         before += rp[i];
       }
@@ -205,24 +214,39 @@ __global__ void __launch_bounds__(64) build_query_kernel(QueryArgs a, int model)
         float v = -rq[j] * t0 + r0 * tq[j];
         if (qn >= 2) v += (sum_rq - before - rq[j]) - before;  // d sigma_qq / d hq_j
         if (pq) v -= sum_rp;                                   // d sigma_pq / d hq_j
+        if (qr) v += sum_rk;                                   // d sigma_qr / d hq_j
         q[qoff + rho * qn + j] = v * a.coeff_q[j];
         before += rq[j];
       }
+      before = 0.f;
+      for (int l = 0; l < kn; ++l) {
+        float v = r0 * tk[l];                                  // a degenerate base squares to zero: no t0 term
+        if (kn >= 2) v += (sum_rk - before - rk[l]) - before;  // d sigma_rr / d hk_l
+        if (pr) v -= sum_rp;                                   // d sigma_pr / d hk_l
+        if (qr) v -= sum_rq;                                   // d sigma_qr / d hk_l
+        q[koff + rho * kn + l] = v * a.coeff_r[l];
+        before += rk[l];
+      }
     }
-  } else {  // KGE_KECI
-    const int p = a.p, qn = a.q;
-    const int r = d / (p + qn + 1);
-    // scale the p / q parts of both rows by their coefficients first, as the reference does
+  } else {  // KGE_KECI (r = 0) / KGE_DECAL
+    const int p = a.p, qn = a.q, kn = a.r;
+    const int r = d / (p + qn + kn + 1);
+    // scale the p / q / r parts of both rows by their coefficients first, as the reference does
     for (int k = lane; k < r * p; k += 64) {
       float c = a.coeff_p[k % p];
       sh[r + k] *= c;
       sr[r + k] *= c;
     }
-    const int qoff = r + r * p;
+    const int qoff = r + r * p, koff = qoff + r * qn;
     for (int k = lane; k < r * qn; k += 64) {
       float c = a.coeff_q[k % qn];
       sh[qoff + k] *= c;
       sr[qoff + k] *= c;
+    }
+    for (int k = lane; k < r * kn; k += 64) {
+      float c = a.coeff_r[k % kn];
+      sh[koff + k] *= c;
+      sr[koff + k] *= c;
     }
     __syncthreads();
     for (int rho = lane; rho < r; rho += 64) {
@@ -231,6 +255,8 @@ __global__ void __launch_bounds__(64) build_query_kernel(QueryArgs a, int model)
       const float* rp = sr + r + rho * p;
       const float* hq = sh + qoff + rho * qn;
       const float* rq = sr + qoff + rho * qn;
+      const float* hk = sh + koff + rho * kn;
+      const float* rk = sr + koff + rho * kn;
       float q0 = h0 * r0;
       for (int i = 0; i < p; ++i) {
         q0 += hp[i] * rp[i];
@@ -240,6 +266,7 @@ __global__ void __launch_bounds__(64) build_query_kernel(QueryArgs a, int model)
         q0 -= hq[j] * rq[j];
         q[qoff + rho * qn + j] = h0 * rq[j] + hq[j] * r0;
       }
+      for (int l = 0; l < kn; ++l) q[koff + rho * kn + l] = h0 * rk[l] + hk[l] * r0;
       q[rho] = q0;
       if (p >= 2)
         for (int i = 0; i < p - 1; ++i)
@@ -247,9 +274,18 @@ __global__ void __launch_bounds__(64) build_query_kernel(QueryArgs a, int model)
       if (qn >= 2)
         for (int j = 0; j < qn - 1; ++j)
           for (int k = j + 1; k < qn; ++k) bias += hq[j] * rq[k] - hq[k] * rq[j];
+      if (kn >= 2)
+        for (int l = 0; l < kn - 1; ++l)
+          for (int k = l + 1; k < kn; ++k) bias += hk[l] * rk[k] - hk[k] * rk[l];
       if (p >= 2 && qn >= 2)
         for (int i = 0; i < p; ++i)
           for (int j = 0; j < qn; ++j) bias += hp[i] * rq[j] - hq[j] * rp[i];
+      if (p >= 2 && kn >= 2)
+        for (int i = 0; i < p; ++i)
+          for (int l = 0; l < kn; ++l) bias += hp[i] * rk[l] - hk[l] * rp[i];
+      if (qn >= 2 && kn >= 2)
+        for (int j = 0; j < qn; ++j)
+          for (int l = 0; l < kn; ++l) bias += hq[j] * rk[l] - hk[l] * rq[j];
     }
     bias = wave_sum(bias);
   }
@@ -271,9 +307,9 @@ int launch_build_query(const QueryArgs& a, int model, int rel_dtype, hipStream_t
 }  // namespace
 }  // namespace kge
 
-static int build_query_impl(int head_mode, int model, int p, int q, const void* ent, int ent_dtype,
+static int build_query_impl(int head_mode, int model, int p, int q, int r, const void* ent, int ent_dtype,
                             const float* ent_scale, const void* rel, int rel_dtype, const float* coeff_p,
-                            const float* coeff_q, int normalize_relation, const kge_norm_params* norm,
+                            const float* coeff_q, const float* coeff_r, int normalize_relation, const kge_norm_params* norm,
                             const int64_t* hr, int64_t B, int64_t d, int64_t N, int64_t R, float* Q, float* bias,
                             void* stream) {
   using namespace kge;
@@ -307,6 +343,14 @@ static int build_query_impl(int head_mode, int model, int p, int q, const void* 
                   "kge_build_query: Keci needs d / (p + q + 1) whole, got d=%lld p=%d q=%d", (long long)d, p, q);
       KGE_REQUIRE((p == 0 || coeff_p) && (q == 0 || coeff_q), KGE_ERR_INVALID,
                   "kge_build_query: Keci with p=%d q=%d needs coefficient vectors", p, q);
+      KGE_REQUIRE(r == 0, KGE_ERR_INVALID, "kge_build_query: Keci has no degenerate bases (r=%d)", r);
+      break;
+    case KGE_DECAL:
+      KGE_REQUIRE(p >= 0 && q >= 0 && r >= 0 && d % (p + q + r + 1) == 0, KGE_ERR_INVALID,
+                  "kge_build_query_decal: needs d / (p + q + r + 1) whole, got d=%lld p=%d q=%d r=%d", (long long)d, p,
+                  q, r);
+      KGE_REQUIRE((p == 0 || coeff_p) && (q == 0 || coeff_q) && (r == 0 || coeff_r), KGE_ERR_INVALID,
+                  "kge_build_query_decal: p=%d q=%d r=%d need their coefficient vectors", p, q, r);
       break;
     default: return set_error(KGE_ERR_INVALID, "kge_build_query: unknown model %d", model);
   }
@@ -316,6 +360,7 @@ static int build_query_impl(int head_mode, int model, int p, int q, const void* 
   a.rel = rel;
   a.coeff_p = coeff_p;
   a.coeff_q = coeff_q;
+  a.coeff_r = coeff_r;
   a.hr = hr;
   a.Q = Q;
   a.bias = bias;
@@ -335,6 +380,7 @@ static int build_query_impl(int head_mode, int model, int p, int q, const void* 
   a.d = (int)d;
   a.p = p;
   a.q = q;
+  a.r = (model == KGE_DECAL) ? r : 0;
   a.normalize_relation = normalize_relation;
   a.head_mode = head_mode;
   hipStream_t st = (hipStream_t)stream;
@@ -347,7 +393,9 @@ extern "C" int kge_build_query(int model, int p, int q, const void* ent, int ent
                                const void* rel, int rel_dtype, const float* coeff_p, const float* coeff_q,
                                int normalize_relation, const kge_norm_params* norm, const int64_t* hr,
                                int64_t B, int64_t d, int64_t N, int64_t R, float* Q, float* bias, void* stream) {
-  return build_query_impl(0, model, p, q, ent, ent_dtype, ent_scale, rel, rel_dtype, coeff_p, coeff_q,
+  if (model == KGE_DECAL)
+    return kge::set_error(KGE_ERR_INVALID, "kge_build_query: DeCaL takes three base counts, use kge_build_query_decal");
+  return build_query_impl(0, model, p, q, 0, ent, ent_dtype, ent_scale, rel, rel_dtype, coeff_p, coeff_q, nullptr,
                           normalize_relation, norm, hr, B, d, N, R, Q, bias, stream);
 }
 
@@ -355,6 +403,17 @@ extern "C" int kge_build_query_head(int model, int p, int q, const void* ent, in
                                     const void* rel, int rel_dtype, const float* coeff_p, const float* coeff_q,
                                     int normalize_relation, const kge_norm_params* norm, const int64_t* rt,
                                     int64_t B, int64_t d, int64_t N, int64_t R, float* Q, float* bias, void* stream) {
-  return build_query_impl(1, model, p, q, ent, ent_dtype, ent_scale, rel, rel_dtype, coeff_p, coeff_q,
+  if (model == KGE_DECAL)
+    return kge::set_error(KGE_ERR_INVALID, "kge_build_query_head: DeCaL takes three base counts, use kge_build_query_decal");
+  return build_query_impl(1, model, p, q, 0, ent, ent_dtype, ent_scale, rel, rel_dtype, coeff_p, coeff_q, nullptr,
                           normalize_relation, norm, rt, B, d, N, R, Q, bias, stream);
+}
+
+extern "C" int kge_build_query_decal(int head, int p, int q, int r, const void* ent, int ent_dtype,
+                                     const float* ent_scale, const void* rel, int rel_dtype, const float* coeff_p,
+                                     const float* coeff_q, const float* coeff_r, const kge_norm_params* norm,
+                                     const int64_t* pairs, int64_t B, int64_t d, int64_t N, int64_t R, float* Q,
+                                     float* bias, void* stream) {
+  return build_query_impl(head ? 1 : 0, KGE_DECAL, p, q, r, ent, ent_dtype, ent_scale, rel, rel_dtype, coeff_p, coeff_q,
+                          coeff_r, 0, norm, pairs, B, d, N, R, Q, bias, stream);
 }

@@ -6,7 +6,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libkge_hip.so")
 
 KGE_OK = 0
-MODEL_IDS = {"DistMult": 0, "ComplEx": 1, "QMult": 2, "Keci": 3, "CKeci": 3, "OMult": 4}
+MODEL_IDS = {"DistMult": 0, "ComplEx": 1, "QMult": 2, "Keci": 3, "CKeci": 3, "OMult": 4, "DeCaL": 5}
 DTYPE_F32, DTYPE_BF16, DTYPE_I8 = 0, 1, 2
 NORM_NONE, NORM_LAYERNORM, NORM_BATCHNORM1D = 0, 1, 2
 
@@ -29,6 +29,8 @@ SIGNATURES = {
                                  ctypes.POINTER(NormParams), _vp, _c_i64, _c_i64, _c_i64, _c_i64, _vp, _vp, _vp]),
     "kge_build_query_head": (_c_int, [_c_int, _c_int, _c_int, _vp, _c_int, _vp, _vp, _c_int, _vp, _vp, _c_int,
                                       ctypes.POINTER(NormParams), _vp, _c_i64, _c_i64, _c_i64, _c_i64, _vp, _vp, _vp]),
+    "kge_build_query_decal": (_c_int, [_c_int, _c_int, _c_int, _c_int, _vp, _c_int, _vp, _vp, _c_int, _vp, _vp, _vp,
+                                       ctypes.POINTER(NormParams), _vp, _c_i64, _c_i64, _c_i64, _c_i64, _vp, _vp, _vp]),
     "kge_scores": (_c_int, [_vp, _vp, _vp, _c_int, _vp, _c_i64, _c_i64, _c_i64, _vp, _c_i64, _vp]),
     "kge_triple_scores": (_c_int, [_vp, _vp, _vp, _c_int, _vp, _c_i64, _c_i64, _c_i64, _vp, _vp, _vp]),
     "kge_csr_lookup": (_c_int, [_vp, _c_i64, _vp, _c_i64, _c_i64, _vp, _vp]),

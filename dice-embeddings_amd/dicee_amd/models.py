@@ -255,8 +255,40 @@ class CKeci(Keci):
             self.q_coefficients.weight.requires_grad_(False)
 
 
+class DeCaL(BaseKGE):
+    """dicee/models/clifford.py:579-912: Cl(p, q, r) with r degenerate bases.  Parameter names and shapes as there
+    (``p_coefficients`` / ``q_coefficients`` / ``r_coefficients``: Embedding(1, count), zero-initialised); ``re`` is
+    the length of one part.  The reference truncates ``embedding_dim / (1 + p + q + r)``; a remainder would leave
+    columns that no term reads, so it is refused here."""
+    name = "DeCaL"
+
+    def __init__(self, args):
+        super().__init__(args)
+        self.p = int(args.get("p", 0) or 0)
+        self.q = int(args.get("q", 0) or 0)
+        self.r = int(args.get("r", 0) or 0)
+        parts = self.p + self.q + self.r + 1
+        if self.embedding_dim % parts:
+            raise AssertionError(f"embedding_dim / (p + q + r + 1) must be a whole number\n"
+                                 f"Currently {self.embedding_dim} / ({self.p} + {self.q} + {self.r} + 1)")
+        self.re = self.embedding_dim // parts
+        for count, attr in ((self.p, "p_coefficients"), (self.q, "q_coefficients"), (self.r, "r_coefficients")):
+            if count > 0:
+                emb = torch.nn.Embedding(num_embeddings=1, embedding_dim=count)
+                torch.nn.init.zeros_(emb.weight)
+                setattr(self, attr, emb)
+
+    def _query_kwargs(self):
+        kw = {"p": self.p, "q": self.q, "r": self.r}
+        for count, attr, key in ((self.p, "p_coefficients", "coeff_p"), (self.q, "q_coefficients", "coeff_q"),
+                                 (self.r, "r_coefficients", "coeff_r")):
+            if count > 0:
+                kw[key] = getattr(self, attr).weight.detach().reshape(-1).float().contiguous()
+        return kw
+
+
 MODEL_REGISTRY = {"DistMult": DistMult, "ComplEx": ComplEx, "QMult": QMult, "OMult": OMult, "Keci": Keci,
-                  "CKeci": CKeci}
+                  "CKeci": CKeci, "DeCaL": DeCaL}
 
 
 def initialize_model(args: dict):

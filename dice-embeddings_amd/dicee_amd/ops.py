@@ -45,12 +45,12 @@ def _norm_struct(norm):
     return s, keep
 
 
-def build_query(model, ent, rel, hr, *, ent_scale=None, p=0, q=0, coeff_p=None, coeff_q=None,
+def build_query(model, ent, rel, hr, *, ent_scale=None, p=0, q=0, r=0, coeff_p=None, coeff_q=None, coeff_r=None,
                 normalize_relation=True, norm=None, head=False):
     """(Q [B,d] fp32, bias [B] fp32) with ``forward_k_vs_all(x) == Q @ E^T + bias[:, None]``.
     ``head=True``: ``hr`` holds (relation, tail) pairs and ``Q @ E^T`` scores every entity as the head."""
     lib = _lib.load()
-    _require_gpu(ent, rel, hr, ent_scale, coeff_p, coeff_q)
+    _require_gpu(ent, rel, hr, ent_scale, coeff_p, coeff_q, coeff_r)
     if hr.dtype != torch.int64 or hr.dim() != 2 or hr.shape[1] != 2:
         raise ValueError("hr must be an int64 tensor of shape [B, 2]")
     B, (N, d), R = hr.shape[0], ent.shape, rel.shape[0]
@@ -59,6 +59,14 @@ def build_query(model, ent, rel, hr, *, ent_scale=None, p=0, q=0, coeff_p=None, 
     Q = torch.empty((B, d), dtype=torch.float32, device=ent.device)
     bias = torch.empty((B,), dtype=torch.float32, device=ent.device)
     ns, keep = _norm_struct(norm)
+    if model == "DeCaL":
+        rc = lib.kge_build_query_decal(int(bool(head)), int(p), int(q), int(r), _ptr(ent), _table_dtype(ent),
+                                       _ptr(ent_scale), _ptr(rel), _table_dtype(rel), _ptr(coeff_p), _ptr(coeff_q),
+                                       _ptr(coeff_r), ctypes.byref(ns) if ns is not None else None, _ptr(hr), B, d, N,
+                                       R, _ptr(Q), _ptr(bias), _stream())
+        _lib.check(rc)
+        del keep
+        return Q, bias
     fn = lib.kge_build_query_head if head else lib.kge_build_query
     rc = fn(MODEL_IDS[model], int(p), int(q), _ptr(ent), _table_dtype(ent), _ptr(ent_scale),
             _ptr(rel), _table_dtype(rel), _ptr(coeff_p), _ptr(coeff_q), int(bool(normalize_relation)),

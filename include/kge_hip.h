@@ -41,7 +41,7 @@ enum kge_status {
   KGE_ERR_OVERFLOW = 5      /* top-k candidate buffers overflowed beyond recovery */
 };
 
-enum kge_model { KGE_DISTMULT = 0, KGE_COMPLEX = 1, KGE_QMULT = 2, KGE_KECI = 3, KGE_OMULT = 4 };
+enum kge_model { KGE_DISTMULT = 0, KGE_COMPLEX = 1, KGE_QMULT = 2, KGE_KECI = 3, KGE_OMULT = 4, KGE_DECAL = 5 };
 enum kge_dtype { KGE_F32 = 0, KGE_BF16 = 1, KGE_I8 = 2 };
 enum kge_norm_kind { KGE_NORM_NONE = 0, KGE_NORM_LAYERNORM = 1, KGE_NORM_BATCHNORM1D = 2 };
 
@@ -102,6 +102,22 @@ int kge_build_query_head(int model, int p, int q, const void* ent, int ent_dtype
                          const void* rel, int rel_dtype, const float* coeff_p, const float* coeff_q,
                          int normalize_relation, const kge_norm_params* norm, const int64_t* rt,
                          int64_t B, int64_t d, int64_t N, int64_t R, float* Q, float* bias, void* stream);
+
+/*
+ * The same two builders for DeCaL, the Clifford model with degenerate bases Cl(p, q, r): a row is
+ * 1 + p + q + r parts of d / (1 + p + q + r) values, laid out [scalar | p-block | q-block | r-block] with
+ * element (rho, i) of a block at rho * count + i.  Follows DeCaL.forward_k_vs_all
+ * (dicee/models/clifford.py:808-899): head and relation parts are scaled by coeff_p[p] / coeff_q[q] /
+ * coeff_r[r] (apply_coefficients :901-912), Q holds h0*r0 + sum hp*rp - sum hq*rq against the tails'
+ * scalar part and h0*r_x + h_x*r0 against every base part, bias the six sigma sums (:859-886, each
+ * only when both of its base counts are >= 2, as there).  head != 0: pairs are (relation, tail) and Q
+ * is the coefficient vector of the head row, as kge_build_query_head (norm must then be none).
+ * With r = 0 this is Keci.
+ */
+int kge_build_query_decal(int head, int p, int q, int r, const void* ent, int ent_dtype, const float* ent_scale,
+                          const void* rel, int rel_dtype, const float* coeff_p, const float* coeff_q,
+                          const float* coeff_r, const kge_norm_params* norm, const int64_t* pairs, int64_t B,
+                          int64_t d, int64_t N, int64_t R, float* Q, float* bias, void* stream);
 
 /*
  * Materialised scores S[b, e] = dot(Q[b], E[e]) (* scale[e]) (+ bias[b]); S has row stride ldS.

@@ -26,6 +26,12 @@ Pinning status (independent checks live in ``tests/test_oracle_pins.py``)
                       c=0 == DistMult on the first half; general (p,q) against a
                       brute-force geometric-algebra product on bitmask blades;
                       thresholds p>=2 / q>=2 / (p>=2 and q>=2) by fixtures.
+* ``decal_*``         general (p,q,r) against the same brute-force geometric-algebra product with r
+                      bases that square to zero (bivector families counted under the reference's
+                      ">= 2 of each" conditions); r = 0 == Keci; single-GEMM form == einsum form;
+                      the head-direction vector against per-triple scores with replaced heads.
+                      ``triple_scores`` for DeCaL is defined as the KvsAll column (the reference's
+                      ``forward_triples`` skips the coefficients and contracts over the batch).
 * ``layer_norm`` / ``batch_norm_eval``  torch.nn.functional library routines.
 * ``filtered_rank_counts``  explicit masking + stable argsort brute force;
                       invariants (duplicates idempotent, -inf never outranks,
@@ -57,7 +63,7 @@ from __future__ import annotations
 
 import numpy as np
 
-MODELS = ("DistMult", "ComplEx", "QMult", "Keci", "OMult")
+MODELS = ("DistMult", "ComplEx", "QMult", "Keci", "OMult", "DeCaL")
 
 # --------------------------------------------------------------------------
 # known-answer vocabularies
@@ -396,24 +402,146 @@ def keci_scores_ref_form(h, r_emb, E, p, q, coeff_p=None, coeff_q=None):
 
 
 # --------------------------------------------------------------------------
+# DeCaL: Cl(p, q, r) with r degenerate bases   dicee/models/clifford.py:579-912
+# --------------------------------------------------------------------------
+
+
+def decal_split(x, re, p, q, r):
+    """construct_cl_multivector (clifford.py:914-953): [B,d] -> x0 [B,re], xp [B,re,p], xq [B,re,q], xk [B,re,r]."""
+    B = x.shape[0]
+    o1, o2, o3 = re, re + re * p, re + re * p + re * q
+    return (x[:, :re], x[:, o1:o2].reshape(B, re, p), x[:, o2:o3].reshape(B, re, q),
+            x[:, o3:o3 + re * r].reshape(B, re, r))
+
+
+def _decal_parts(h, r_emb, p, q, r, coeff_p, coeff_q, coeff_r):
+    d = h.shape[1]
+    assert d % (1 + p + q + r) == 0
+    re = d // (1 + p + q + r)
+    h0, hp, hq, hk = decal_split(h, re, p, q, r)
+    r0, rp, rq, rk = decal_split(r_emb, re, p, q, r)
+    # apply_coefficients (clifford.py:901-912): base parts of head and relation scaled, scalar parts not
+    if p > 0:
+        c = np.asarray(coeff_p, dtype=h.dtype).reshape(1, 1, p)
+        hp, rp = hp * c, rp * c
+    if q > 0:
+        c = np.asarray(coeff_q, dtype=h.dtype).reshape(1, 1, q)
+        hq, rq = hq * c, rq * c
+    if r > 0:
+        c = np.asarray(coeff_r, dtype=h.dtype).reshape(1, 1, r)
+        hk, rk = hk * c, rk * c
+    return re, (h0, hp, hq, hk), (r0, rp, rq, rk)
+
+
+def _decal_sigmas(hs, rs, p, q, r):
+    """The six sigma sums of clifford.py:859-886, each present only when both of its base counts are >= 2."""
+    _, hp, hq, hk = hs
+    _, rp, rq, rk = rs
+
+    def same(x, y, n):        # compute_sigma_pp / qq / rr: upper triangle of x_i y_k - x_k y_i
+        return sum((x[:, :, i] * y[:, :, k] - x[:, :, k] * y[:, :, i]).sum(axis=1)
+                   for i in range(n - 1) for k in range(i + 1, n))
+
+    def cross(xa, xb, ya, yb):  # compute_sigma_pq / pr / qr: xa_i yb_j - xb_j ya_i over all pairs
+        return (np.einsum("nri,nrj->n", xa, yb) - np.einsum("nrj,nri->n", xb, ya))
+
+    out = np.zeros(hp.shape[0], dtype=hp.dtype)
+    if p >= 2:
+        out = out + same(hp, rp, p)
+    if q >= 2:
+        out = out + same(hq, rq, q)
+    if r >= 2:
+        out = out + same(hk, rk, r)
+    if p >= 2 and q >= 2:
+        out = out + cross(hp, hq, rp, rq)
+    if p >= 2 and r >= 2:
+        out = out + cross(hp, hk, rp, rk)
+    if q >= 2 and r >= 2:
+        out = out + cross(hq, hk, rq, rk)
+    return out
+
+
+def decal_scores_ref_form(h, r_emb, E, p, q, r, coeff_p=None, coeff_q=None, coeff_r=None):
+    """DeCaL.forward_k_vs_all (clifford.py:808-899), einsum by einsum."""
+    E = np.asarray(E, dtype=h.dtype)
+    N = E.shape[0]
+    re, (h0, hp, hq, hk), (r0, rp, rq, rk) = _decal_parts(h, r_emb, p, q, r, coeff_p, coeff_q, coeff_r)
+    t0 = E[:, :re]
+    out = np.einsum("br,er->be", h0 * r0, t0)
+    if p > 0:
+        tp = E[:, re:re + re * p].reshape(N, re, p)
+        out = out + np.einsum("brp,er->be", hp * rp, t0) + np.einsum("brp,erp->be", h0[:, :, None] * rp, tp) \
+            + np.einsum("brp,erp->be", hp * r0[:, :, None], tp)
+    if q > 0:
+        o = re + re * p
+        tq = E[:, o:o + re * q].reshape(N, re, q)
+        out = out + np.einsum("brq,erq->be", h0[:, :, None] * rq, tq) + np.einsum("brq,erq->be", hq * r0[:, :, None], tq) \
+            - np.einsum("brq,er->be", hq * rq, t0)
+    if r > 0:
+        tk = E[:, E.shape[1] - re * r:].reshape(N, re, r)
+        out = out + np.einsum("brk,erk->be", h0[:, :, None] * rk, tk) + np.einsum("brk,erk->be", hk * r0[:, :, None], tk)
+    return out + _decal_sigmas((h0, hp, hq, hk), (r0, rp, rq, rk), p, q, r)[:, None]
+
+
+def decal_query(h, r_emb, p, q, r, coeff_p=None, coeff_q=None, coeff_r=None):
+    """Single-GEMM form: (Q [B,d], bias [B]) with ``forward_k_vs_all == Q @ E^T + bias``."""
+    B = h.shape[0]
+    re, (h0, hp, hq, hk), (r0, rp, rq, rk) = _decal_parts(h, r_emb, p, q, r, coeff_p, coeff_q, coeff_r)
+    q0 = h0 * r0 + (hp * rp).sum(axis=2) - (hq * rq).sum(axis=2)
+    blocks = [q0]
+    for hx, rx, n in ((hp, rp, p), (hq, rq, q), (hk, rk, r)):
+        blocks.append((h0[:, :, None] * rx + hx * r0[:, :, None]).reshape(B, re * n))
+    return np.concatenate(blocks, axis=1), _decal_sigmas((h0, hp, hq, hk), (r0, rp, rq, rk), p, q, r)
+
+
+def decal_head_query(r_emb, t, p, q, r, coeff_p=None, coeff_q=None, coeff_r=None):
+    """Q' with ``forward_k_vs_all((x, rel))[tail] = Q' . E[x]``: the coefficient of every head component."""
+    B = t.shape[0]
+    re, (t0, tp, tq, tk), (r0, rp, rq, rk) = _decal_parts(t, r_emb, p, q, r, None if not p else np.ones(p),
+                                                           None if not q else np.ones(q), None if not r else np.ones(r))
+    cs = [np.asarray(c if n else [], dtype=t.dtype).reshape(1, 1, n)
+          for c, n in ((coeff_p, p), (coeff_q, q), (coeff_r, r))]
+    rp, rq, rk = rp * cs[0], rq * cs[1], rk * cs[2]
+    q0 = r0 * t0 + (rp * tp).sum(2) + (rq * tq).sum(2) + (rk * tk).sum(2)
+    qp = rp * t0[:, :, None] + r0[:, :, None] * tp
+    qq = -rq * t0[:, :, None] + r0[:, :, None] * tq
+    qk = r0[:, :, None] * tk
+    for blk, rx, n in ((qp, rp, p), (qq, rq, q), (qk, rk, r)):
+        if n >= 2:                                           # d sigma_xx / d hx_i = sum_{k>i} rx_k - sum_{k<i} rx_k
+            for i in range(n):
+                blk[:, :, i] += rx[:, :, i + 1:].sum(2) - rx[:, :, :i].sum(2)
+    sp, sq, sk = rp.sum(2)[:, :, None], rq.sum(2)[:, :, None], rk.sum(2)[:, :, None]
+    if p >= 2 and q >= 2:
+        qp, qq = qp + sq, qq - sp
+    if p >= 2 and r >= 2:
+        qp, qk = qp + sk, qk - sp
+    if q >= 2 and r >= 2:
+        qq, qk = qq + sk, qk - sq
+    return np.concatenate([q0, (qp * cs[0]).reshape(B, re * p), (qq * cs[1]).reshape(B, re * q),
+                           (qk * cs[2]).reshape(B, re * r)], axis=1)
+
+
+# --------------------------------------------------------------------------
 # model dispatch
 # --------------------------------------------------------------------------
 
 
 def build_query(model, E, R, hr, p=0, q=0, coeff_p=None, coeff_q=None,
-                normalize_relation=True, norm=None, dtype=np.float64):
+                normalize_relation=True, norm=None, dtype=np.float64, r=0, coeff_r=None):
     """(Q [B,d], bias [B]) such that ``scores = Q @ E.T + bias[:, None]``."""
-    h, r = gather_hr(E, R, hr, norm=norm, dtype=dtype)
+    h, r_ = gather_hr(E, R, hr, norm=norm, dtype=dtype)
     if model == "DistMult":
-        return distmult_query(h, r), np.zeros(len(h), dtype)
+        return distmult_query(h, r_), np.zeros(len(h), dtype)
     if model == "ComplEx":
-        return complex_query(h, r), np.zeros(len(h), dtype)
+        return complex_query(h, r_), np.zeros(len(h), dtype)
     if model == "QMult":
-        return qmult_query(h, r, normalize_relation), np.zeros(len(h), dtype)
+        return qmult_query(h, r_, normalize_relation), np.zeros(len(h), dtype)
     if model == "OMult":
-        return omult_query(h, r, normalize_relation), np.zeros(len(h), dtype)
+        return omult_query(h, r_, normalize_relation), np.zeros(len(h), dtype)
     if model in ("Keci", "CKeci"):
-        return keci_query(h, r, p, q, coeff_p, coeff_q)
+        return keci_query(h, r_, p, q, coeff_p, coeff_q)
+    if model == "DeCaL":
+        return decal_query(h, r_, p, q, r, coeff_p, coeff_q, coeff_r)
     raise ValueError(model)
 
 
@@ -425,17 +553,19 @@ def k_vs_all_scores(model, E, R, hr, **kw):
 
 
 def k_vs_all_scores_ref_form(model, E, R, hr, p=0, q=0, coeff_p=None, coeff_q=None,
-                             normalize_relation=True, norm=None, dtype=np.float64):
+                             normalize_relation=True, norm=None, dtype=np.float64, r=0, coeff_r=None):
     """``forward_k_vs_all`` via the reference's own multi-mm / einsum decomposition."""
-    h, r = gather_hr(E, R, hr, norm=norm, dtype=dtype)
+    h, r_ = gather_hr(E, R, hr, norm=norm, dtype=dtype)
     if model == "DistMult":
-        return distmult_scores_ref_form(h, r, E)
+        return distmult_scores_ref_form(h, r_, E)
     if model == "ComplEx":
-        return complex_scores_ref_form(h, r, E)
+        return complex_scores_ref_form(h, r_, E)
     if model == "QMult":
-        return qmult_scores_ref_form(h, r, E, normalize_relation)
+        return qmult_scores_ref_form(h, r_, E, normalize_relation)
     if model in ("Keci", "CKeci"):
-        return keci_scores_ref_form(h, r, E, p, q, coeff_p, coeff_q)
+        return keci_scores_ref_form(h, r_, E, p, q, coeff_p, coeff_q)
+    if model == "DeCaL":
+        return decal_scores_ref_form(h, r_, E, p, q, r, coeff_p, coeff_q, coeff_r)
     raise ValueError(model)
 
 
@@ -453,13 +583,18 @@ def k_vs_all_scores_ref_form(model, E, R, hr, p=0, q=0, coeff_p=None, coeff_q=No
 
 
 def triple_scores(model, E, R, triples, p=0, q=0, coeff_p=None, coeff_q=None, normalize_relation=True,
-                  dtype=np.float64):
+                  dtype=np.float64, r=0, coeff_r=None):
     """score(h, r, t) for every row of ``triples`` [n,3]: DistMult.score (real.py:48-49),
     ComplEx.score (complex.py:229-238), QMult.score (quaternion.py:102-122), Keci.score
     (clifford.py:448-499), each written as explicit sums over the embedding parts."""
     E = np.asarray(E, dtype=dtype)
     R = np.asarray(R, dtype=dtype)
     triples = np.asarray(triples)
+    if model == "DeCaL":
+        # DeCaL.forward_triples (clifford.py:595-680) skips apply_coefficients and, like Keci's, contracts some
+        # einsums over the batch; the per-triple value here is the one its KvsAll path gives, one triple at a time.
+        return np.array([decal_scores_ref_form(E[t[0]:t[0] + 1], R[t[1]:t[1] + 1], E[t[2]:t[2] + 1], p, q, r,
+                                               coeff_p, coeff_q, coeff_r)[0, 0] for t in triples], dtype=dtype)
     h, r, t = E[triples[:, 0]], R[triples[:, 1]], E[triples[:, 2]]
     n, d = h.shape
     if model == "DistMult":
@@ -508,11 +643,14 @@ def triple_scores(model, E, R, triples, p=0, q=0, coeff_p=None, coeff_q=None, no
     raise ValueError(model)
 
 
-def head_query(model, E, R, rt, p=0, q=0, coeff_p=None, coeff_q=None, normalize_relation=True, dtype=np.float64):
+def head_query(model, E, R, rt, p=0, q=0, coeff_p=None, coeff_q=None, normalize_relation=True, dtype=np.float64,
+               r=0, coeff_r=None):
     """Q' [B,d] with ``score(x, rt[b,0], rt[b,1]) = Q'[b] . E[x]`` (no bias: every term holds the head)."""
     E = np.asarray(E, dtype=dtype)
     R = np.asarray(R, dtype=dtype)
     rt = np.asarray(rt)
+    if model == "DeCaL":
+        return decal_head_query(R[rt[:, 0]], E[rt[:, 1]], p, q, r, coeff_p, coeff_q, coeff_r)
     r, t = R[rt[:, 0]], E[rt[:, 1]]
     B, d = r.shape
     if model == "DistMult":

@@ -29,6 +29,8 @@ def _toy(model_name, d, N=135, R=46, n=2000, seed=0, **extra):
             m.p_coefficients.weight.normal_(1.0, 0.3)
         if hasattr(m, "q_coefficients"):
             m.q_coefficients.weight.normal_(1.0, 0.3)
+        if hasattr(m, "r_coefficients"):
+            m.r_coefficients.weight.normal_(1.0, 0.3)
     triples = np.stack([rng.integers(0, N, n), rng.integers(0, R, n), rng.integers(0, N, n)], axis=1)
     return m, triples
 
@@ -41,12 +43,19 @@ def _oracle_kw(m):
             kw["coeff_p"] = m.p_coefficients.weight.detach().cpu().numpy().reshape(-1)
         if m.q:
             kw["coeff_q"] = m.q_coefficients.weight.detach().cpu().numpy().reshape(-1)
+    if m.name == "DeCaL":
+        kw = {"p": m.p, "q": m.q, "r": m.r}
+        for n, key, attr in ((m.p, "coeff_p", "p_coefficients"), (m.q, "coeff_q", "q_coefficients"),
+                             (m.r, "coeff_r", "r_coefficients")):
+            if n:
+                kw[key] = getattr(m, attr).weight.detach().cpu().numpy().reshape(-1)
     return kw
 
 
 @pytest.mark.parametrize("name,d,extra", [("DistMult", 32, {}), ("ComplEx", 32, {}), ("QMult", 32, {}),
                                           ("OMult", 32, {}),
-                                          ("Keci", 30, {"p": 2, "q": 2}), ("CKeci", 32, {"p": 0, "q": 1})])
+                                          ("Keci", 30, {"p": 2, "q": 2}), ("CKeci", 32, {"p": 0, "q": 1}),
+                                          ("DeCaL", 32, {"p": 2, "q": 2, "r": 3}), ("DeCaL", 30, {"p": 1, "q": 1, "r": 3})])
 def test_forward_k_vs_all_is_a_drop_in(name, d, extra):
     m, triples = _toy(name, d, **extra)
     E = m.entity_embeddings.weight.detach().numpy().copy()
@@ -232,7 +241,8 @@ def test_stored_experiment_evaluates_end_to_end(tmp_path):
 
 @pytest.mark.parametrize("name,d,extra", [("DistMult", 32, {}), ("ComplEx", 64, {}), ("QMult", 64, {}),
                                           ("OMult", 64, {}),
-                                          ("Keci", 48, {"p": 0, "q": 1}), ("Keci", 40, {"p": 2, "q": 2})])
+                                          ("Keci", 48, {"p": 0, "q": 1}), ("Keci", 40, {"p": 2, "q": 2}),
+                                          ("DeCaL", 48, {"p": 2, "q": 2, "r": 3})])
 def test_evaluate_lp_both_directions(name, d, extra):
     """Head and tail ranks inside the fp64 oracle's tolerance interval, exact where there is no near-tie; metrics
     reduced as evaluate_lp does; dict and GPU-built vocabularies give the same ranks."""
@@ -316,7 +326,7 @@ def test_predict_missing_head():
 
 
 @pytest.mark.parametrize("name,d,extra", [("DistMult", 32, {}), ("ComplEx", 32, {}), ("QMult", 32, {}),
-                                          ("Keci", 30, {"p": 2, "q": 2})])
+                                          ("Keci", 30, {"p": 2, "q": 2}), ("DeCaL", 32, {"p": 2, "q": 2, "r": 3})])
 def test_forward_triples_and_triple_score(name, d, extra):
     from dicee_amd import KGE
     m, triples = _toy(name, d, n=400, seed=31, **extra)

@@ -39,12 +39,17 @@ MODEL_CASES = [
     ("Keci", 16, {"p": 0, "q": 0}),
     ("OMult", 128, {}),
     ("OMult", 24, {"normalize_relation": False}),
+    ("DeCaL", 28, {"p": 2, "q": 2, "r": 2, "coeff_p": [0.7, 1.1], "coeff_q": [1.3, -0.4], "coeff_r": [0.6, 1.2]}),
+    ("DeCaL", 256, {"p": 3, "q": 1, "r": 3, "coeff_p": [0.7, 1.1, -0.3], "coeff_q": [1.3], "coeff_r": [0.6, 1.2, -0.9]}),
+    ("DeCaL", 24, {"p": 0, "q": 0, "r": 2, "coeff_r": [0.5, 2.0]}),
+    ("DeCaL", 20, {"p": 1, "q": 1, "r": 2, "coeff_p": [0.7], "coeff_q": [1.3], "coeff_r": [0.6, 1.2]}),
+    ("DeCaL", 18, {"p": 1, "q": 1, "r": 0, "coeff_p": [0.7], "coeff_q": [1.3]}),
 ]
 
 
 def _gpu_kwargs(kw):
     out = dict(kw)
-    for k in ("coeff_p", "coeff_q"):
+    for k in ("coeff_p", "coeff_q", "coeff_r"):
         if k in out:
             out[k] = torch.tensor(out[k], dtype=torch.float32, device="cuda")
     return out

@@ -126,6 +126,12 @@ def test_models_mirror_reference_parameters_and_have_no_cpu_fallback():
     assert float(c.p_coefficients.weight.sum()) == 1.0 and not c.q_coefficients.weight.requires_grad
     with pytest.raises(AssertionError):
         models.Keci({**args, "embedding_dim": 13})
+    dc = models.DeCaL({**args, "model": "DeCaL", "embedding_dim": 14, "p": 2, "q": 2, "r": 2})
+    assert dc.re == 2 and dc.r_coefficients.weight.shape == (1, 2) and float(dc.r_coefficients.weight.abs().sum()) == 0
+    assert set(dc.state_dict()) == {"entity_embeddings.weight", "relation_embeddings.weight", "p_coefficients.weight",
+                                    "q_coefficients.weight", "r_coefficients.weight"}
+    with pytest.raises(AssertionError):
+        models.DeCaL({**args, "model": "DeCaL", "embedding_dim": 15, "p": 2, "q": 2, "r": 2})
     with pytest.raises(ValueError):
         models.initialize_model({**args, "model": "TransE"})
     ln = models.ComplEx({"model": "ComplEx", "embedding_dim": 8, "num_entities": 5, "num_relations": 2,

@@ -231,6 +231,77 @@ def test_keci_vs_geometric_algebra(p, q):
         ko.k_vs_all_scores_ref_form("Keci", E, R, hr, p=p, q=q, coeff_p=cp, coeff_q=cq), S, rtol=1e-10, atol=1e-12)
 
 
+class _GAr(_GA):
+    """Cl(p,q,r): r further bases that square to zero."""
+
+    def __init__(self, p, q, r):
+        super().__init__(p, q)
+        self.r = r
+
+    def blade_mul(self, a, b):
+        if (a & b) >> (self.p + self.q):
+            return a ^ b, 0
+        return super().blade_mul(a, b)
+
+
+def _decal_bruteforce(E, R, hr, p, q, r, cp, cq, cr):
+    """score = <grade 0 and 1 of (h r), t> + the sum of the grade-2 coefficients, a bivector e_x e_y counted
+    only when the family counts of x and of y are both >= 2 (the conditions of clifford.py:859-886)."""
+    N, d = E.shape
+    n = p + q + r
+    re = d // (n + 1)
+    ga = _GAr(p, q, r)
+    count = [p] * p + [q] * q + [r] * r
+    coeff = list(cp) + list(cq) + list(cr)
+
+    def col(rho, i):                  # column of base i (0-based over p, then q, then r) of slot rho
+        if i < p:
+            return re + rho * p + i
+        if i < p + q:
+            return re + re * p + rho * q + (i - p)
+        return re + re * p + re * q + rho * r + (i - p - q)
+
+    def mv(x, rho):
+        m = {0: x[rho]}
+        for i in range(n):
+            m[1 << i] = x[col(rho, i)] * coeff[i]
+        return m
+
+    S = np.zeros((len(hr), N))
+    for b, (hi, ri) in enumerate(hr):
+        for rho in range(re):
+            prod = ga.mul(mv(E[hi], rho), mv(R[ri], rho))
+            g2 = 0.0
+            for blade, v in prod.items():
+                bits = [i for i in range(n) if blade >> i & 1]
+                if len(bits) == 2 and count[bits[0]] >= 2 and count[bits[1]] >= 2:
+                    g2 += v
+            for e in range(N):
+                s = prod.get(0, 0.0) * E[e, rho]
+                for i in range(n):
+                    s += prod.get(1 << i, 0.0) * E[e, col(rho, i)]
+                S[b, e] += s + g2
+    return S
+
+
+@pytest.mark.parametrize("p,q,r", [(0, 0, 1), (0, 0, 3), (1, 1, 1), (2, 2, 2), (3, 2, 2), (2, 0, 3), (0, 3, 2), (1, 3, 2),
+                                   (2, 1, 0)])
+def test_decal_vs_geometric_algebra_with_degenerate_bases(p, q, r):
+    rng = np.random.default_rng(100 * p + 10 * q + r)
+    re = 3
+    d = re * (p + q + r + 1)
+    E, R = _tables(rng, 6, 3, d, sd=1.0)
+    hr = _hr(rng, 6, 3, 4)
+    cp, cq, cr = rng.normal(size=p), rng.normal(size=q), rng.normal(size=r)
+    kw = dict(p=p, q=q, r=r, coeff_p=cp, coeff_q=cq, coeff_r=cr)
+    S = ko.k_vs_all_scores("DeCaL", E, R, hr, **kw)
+    np.testing.assert_allclose(S, _decal_bruteforce(E, R, hr, p, q, r, cp, cq, cr), rtol=1e-10, atol=1e-12)
+    np.testing.assert_allclose(ko.k_vs_all_scores_ref_form("DeCaL", E, R, hr, **kw), S, rtol=1e-10, atol=1e-12)
+    if r == 0:                        # no degenerate base: Keci
+        np.testing.assert_allclose(ko.k_vs_all_scores("Keci", E, R, hr, p=p, q=q, coeff_p=cp, coeff_q=cq), S,
+                                   rtol=1e-12, atol=1e-12)
+
+
 def test_keci_reductions():
     rng = np.random.default_rng(5)
     E, R = _tables(rng, 8, 3, 12)
@@ -412,7 +483,9 @@ def test_vocab_csr_against_a_hand_written_fixture_and_set_identities():
 _LP_CASES = [("OMult", 16, {}), ("OMult", 24, {"normalize_relation": False}), ("DistMult", 12, {}), ("ComplEx", 12, {}), ("QMult", 16, {}), ("QMult", 16, {"normalize_relation": False}),
              ("Keci", 12, {"p": 0, "q": 0}), ("Keci", 12, {"p": 0, "q": 1}), ("Keci", 12, {"p": 1, "q": 1}),
              ("Keci", 12, {"p": 2, "q": 0}), ("Keci", 12, {"p": 0, "q": 2}), ("Keci", 15, {"p": 2, "q": 2}),
-             ("Keci", 18, {"p": 3, "q": 2}), ("Keci", 18, {"p": 1, "q": 4})]
+             ("Keci", 18, {"p": 3, "q": 2}), ("Keci", 18, {"p": 1, "q": 4}),
+             ("DeCaL", 14, {"p": 2, "q": 2, "r": 2}), ("DeCaL", 16, {"p": 3, "q": 1, "r": 3}),
+             ("DeCaL", 12, {"p": 0, "q": 0, "r": 2}), ("DeCaL", 12, {"p": 1, "q": 1, "r": 1})]
 
 
 @pytest.mark.parametrize("model,d,kw", _LP_CASES)
@@ -423,9 +496,11 @@ def test_triple_scores_and_head_direction_agree_with_the_kvsall_oracle(model, d,
     N, R, n = 23, 5, 40
     E, Rel = rng.standard_normal((N, d)), rng.standard_normal((R, d))
     kw = dict(kw)
-    if model == "Keci":
+    if model in ("Keci", "DeCaL"):
         kw["coeff_p"] = rng.standard_normal(kw["p"]) + 1.0
         kw["coeff_q"] = rng.standard_normal(kw["q"]) + 1.0
+    if model == "DeCaL":
+        kw["coeff_r"] = rng.standard_normal(kw["r"]) + 1.0
     triples = np.stack([rng.integers(0, N, n), rng.integers(0, R, n), rng.integers(0, N, n)], axis=1)
     per_triple = ko.triple_scores(model, E, Rel, triples, **kw)
     tails = ko.k_vs_all_scores(model, E, Rel, triples[:, :2], **kw)
