@@ -87,7 +87,8 @@ def cpu_baseline(cfg, model, mode, seconds_budget=25.0):
 
 def main_loop_kernel(storage, d, mode):
     """Name of the contraction kernel the library picks for this table type and width."""
-    epi = {"rank": "RankEpi", "headrank": "RankEpi", "topk": "TopkEpi", "bce": "BceEpi"}[mode]
+    epi = {"rank": "RankEpi", "headrank": "RankEpi", "topk": "TopkEpi", "bce": "BceEpi",
+           "bcegrad": "GradEpi | StoreEpi"}[mode]
     if storage == "fp32":
         return f"ksplit_kernel<{epi}, {'true' if d % 4 == 0 else 'false'}>"
     if d == 128:
@@ -101,9 +102,9 @@ def main():
     ap.add_argument("--steps", type=int, default=None)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--config", default="c4", choices=sorted(MODE))
-    ap.add_argument("--mode", default=None, choices=["rank", "topk", "bce", "headrank"],
+    ap.add_argument("--mode", default=None, choices=["rank", "topk", "bce", "bcegrad", "headrank"],
                     help="epilogue to run instead of the configuration's own (headrank: rank the true head of "
-                         "(?, r, t) with the (r, t) -> heads filter)")
+                         "(?, r, t) with the (r, t) -> heads filter; bcegrad: BCE loss and its gradients dQ, dbias, dE)")
     ap.add_argument("--scale", type=float, default=1.0, help="shrink the workload (testing only)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -126,7 +127,7 @@ def main():
     big = args.config in ("c4", "c5") and args.scale == 1.0
     cfg = synthetic.make_config(args.config, scale=args.scale, with_tables=not big)
     model = synthetic.make_model(cfg, dev, tables_on_device=big)
-    if mode in ("rank", "bce", "headrank") and cfg.csr is None:
+    if mode in ("rank", "bce", "bcegrad", "headrank") and cfg.csr is None:
         print(f"bench.py: --mode {mode} needs a configuration with triples", file=sys.stderr)
         sys.exit(2)
     if cfg.csr is not None:
@@ -154,6 +155,8 @@ def main():
             return model.rank_filtered(x, t, re_csr, heads=True)
         if mode == "topk":
             return model.topk(x, cfg.k)
+        if mode == "bcegrad":
+            return model.kvsall_bce_backward(x, cfg.csr)
         return model.kvsall_bce_loss(x, cfg.csr)
 
     if args.copy_calibration:
@@ -179,10 +182,13 @@ def main():
     scores = float(n_queries) * N
     compute = "fp32" if cfg.storage == "fp32" else "bf16"
     flops = 2.0 * d * scores                                    # algorithmic: 2*d flop per entity score
+    if mode == "bcegrad":
+        flops *= 3.0                                            # scores, dQ = g E, dE = g^T Q
     achieved = flops / (kernel_ms * 1e-3) / 1e12 if kernel_ms > 0 else 0.0
     out = {
         "metric": {"rank": "filtered_rank_entity_scores_per_sec", "topk": "topk_entity_scores_per_sec",
-                   "bce": "kvsall_bce_entity_scores_per_sec", "headrank": "filtered_head_rank_entity_scores_per_sec"}[mode],
+                   "bce": "kvsall_bce_entity_scores_per_sec",
+                   "bcegrad": "kvsall_bce_forward_backward_entity_scores_per_sec", "headrank": "filtered_head_rank_entity_scores_per_sec"}[mode],
         "value": scores / elapsed,
         "unit": "scores/s",
         "queries_per_sec": n_queries / elapsed,
@@ -203,7 +209,7 @@ def main():
                      "frac": achieved / PEAK_TFLOPS[compute],
                      **({"peak_basis": "bf16 dense MFMA 2500 / 6 products per fp32 product",
                          "vs_fp32_mfma_peak": achieved / FP32_MFMA_PEAK_TFLOPS} if compute == "fp32" else {}),
-                     "traffic": MEASURED_TRAFFIC_BYTES.get(args.config)
+                     "traffic": MEASURED_TRAFFIC_BYTES.get(args.config) if mode == MODE[args.config] else None
                      if args.scale == 1.0 and args.mode is None else None,
                      "kernel": main_loop_kernel(cfg.storage, d, mode),
                      "kernel_ms_avg": kernel_ms / max(launches, 1), "launches": launches,
@@ -225,7 +231,7 @@ def main():
         out["csr_build"] = {"ms": tb * 1e3, "triples": int(trip.shape[0]), "rows": built.num_rows, "nnz": built.nnz,
                             "triples_per_sec": trip.shape[0] / tb}
         del trip, built
-    if not args.no_cpu_baseline and mode != "headrank":
+    if not args.no_cpu_baseline and mode not in ("headrank", "bcegrad"):
         out["cpu_baseline"] = cpu_baseline(cfg, model, mode)
     print(json.dumps(out))
 

@@ -41,6 +41,10 @@ struct ContractArgs {
   int chunk_rows;
   int n_qgroups;
   int n_lanes;  // persistent kernels: entity-chunk lanes per (XCD, query group)
+  // ksplit_kernel only: row strides of Q and E in elements (0: d), and the length of the K range one
+  // workgroup sums (0: all of d; otherwise a multiple of 32, and blockIdx.y selects the range)
+  int ldq, lde;
+  int k_split_len;
 };
 
 __device__ __forceinline__ f32x16 mfma_bf16(bf16x8 a, bf16x8 b, f32x16 c) {
@@ -115,8 +119,14 @@ __device__ __forceinline__ u32x4 i8x8_to_bf16x8(uint32_t w0, uint32_t w1) {
 // XCD-aware decomposition of a flat workgroup id: hardware deals consecutive ids round-robin over
 // the 8 XCDs, so ids with the same (id % 8) share an L2.  Consecutive slots on one XCD walk the
 // query groups of ONE entity chunk, which keeps that chunk's rows hot in that XCD's L2.
+// contract_grid_wgs() (host) gives the matching grid size.
 __device__ __forceinline__ bool decompose_wg(const ContractArgs& a, int& qg, int64_t& chunk) {
   const int64_t wg = blockIdx.x;
+  if (a.n_chunks < 8) {  // too few chunks to give every XCD one: plain order, so that all XCDs get work
+    qg = (int)(wg % a.n_qgroups);
+    chunk = wg / a.n_qgroups;
+    return chunk < a.n_chunks;
+  }
   const int xcd = (int)(wg & 7);
   const int64_t slot = wg >> 3;
   qg = (int)(slot % a.n_qgroups);
@@ -135,6 +145,7 @@ struct StoreArgs {
   float* S;
   const float* bias;
   int64_t ldS;
+  int64_t split_stride;  // K-split launches: partial result of range y goes to S + y * split_stride
 };
 template <int NQT>
 struct StoreEpi {
@@ -150,6 +161,7 @@ struct StoreEpi {
   int c, hf;
   __device__ void init(const Args& args, int64_t q0_, int c_, int hf_, int64_t B_) {
     a = args; q0 = q0_; c = c_; hf = hf_; B = B_;
+    a.S += (int64_t)blockIdx.y * a.split_stride;
   }
   __device__ void bind(Shared* sh) {
     float* mine = sh->bias + (threadIdx.x >> 6) * (32 * NQT);
@@ -456,6 +468,120 @@ struct BceEpi {
       const int slot = (int)((blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6)) & (BCE_SLOTS - 1));
       atomicAdd(&a.sums[slot], x);
       if (a.want_s) atomicAdd(&a.sums[BCE_SLOTS + slot], y);
+    }
+  }
+};
+
+// Backward of the multi-hot BCE step: g = (sigmoid(s) - y') * inv_bn for the dense part of y' (the
+// known tails are subtracted afterwards from the CSR), written both as G [B, ldG] and as its
+// transpose GT [N, ldT] (the operands of the two gradient contractions), plus the loss sums of
+// BceEpi and the row sums of g (the gradient of the per-query bias).
+struct GradArgs {
+  const float* bias;
+  double* sums;      // as BceArgs::sums
+  float* G;
+  float* GT;
+  float* dbias;      // [B], zero-initialised; may be null
+  int64_t ldG, ldT;
+  float inv_bn;      // upstream gradient / (B * N)
+  float uniform;     // label smoothing: the 1/N every label carries, times inv_bn (0 without smoothing)
+  int32_t want_s;
+};
+template <int NQT>
+struct GradEpi {
+  static constexpr bool SWAP = true;
+  static constexpr bool STAGE_HOOK = false;
+  using Args = GradArgs;
+  struct Shared {
+    float bias[8 * 32 * NQT];
+  };
+  Args a;
+  const float* lb;
+  float rowsum[NQT][16];
+  double sp, ss;
+  int64_t q0, B;
+  int c, hf;
+  __device__ void init(const Args& args, int64_t q0_, int c_, int hf_, int64_t B_) {
+    a = args; q0 = q0_; c = c_; hf = hf_; B = B_;
+    sp = 0.0; ss = 0.0;
+#pragma unroll
+    for (int t = 0; t < NQT; ++t)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) rowsum[t][i] = 0.f;
+  }
+  __device__ void bind(Shared* sh) {
+    float* mine = sh->bias + (threadIdx.x >> 6) * (32 * NQT);
+    for (int j = (threadIdx.x & 63); j < 32 * NQT; j += 64) {
+      const int64_t q = q0 + j;
+      mine[j] = (a.bias && q < B) ? a.bias[q] : 0.f;
+    }
+    lb = mine;
+    __syncthreads();
+  }
+  __device__ void stage_end() {}
+  template <bool HAS_SCALE>
+  __device__ __forceinline__ void tile(int qt, const f32x16& acc, const float* sc16, float sc_col, int64_t e_base,
+                                       int64_t limit) {
+    const int64_t e = e_base + c;
+    if (e >= limit) return;
+    const int64_t qrow = q0 + 32 * qt + 4 * hf;  // query row of acc[0]; acc[4g + r] is row qrow + 8g + r
+    float* pg = a.G + qrow * a.ldG + e;
+    float* pt = a.GT + e * a.ldT + qrow;
+    const bool full = q0 + 32 * qt + 32 <= B;
+    float tsp = 0.f, tss = 0.f;
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const f32x4 b4 = *(const f32x4*)(lb + 32 * qt + 8 * g + 4 * hf);
+      f32x4 out;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        float v = acc[4 * g + r];
+        if (HAS_SCALE) v *= sc_col;
+        v += b4[r];
+        const bool ok = full || qrow + 8 * g + r < B;
+        const float ex = __expf(-fabsf(v));                       // in (0, 1]
+        const float sig = (v >= 0.f ? 1.0f : ex) / (1.0f + ex);    // sigmoid without overflow
+        const float gr = ok ? sig * a.inv_bn - a.uniform : 0.f;
+        tsp += ok ? fmaxf(v, 0.f) + __logf(1.0f + ex) : 0.f;
+        tss += ok ? v : 0.f;
+        out[r] = gr;
+        rowsum[qt][4 * g + r] += gr;
+        if (ok) pg[(int64_t)(8 * g + r) * a.ldG] = gr;
+      }
+      if (full) {
+        *(f32x4*)(pt + 8 * g) = out;
+      } else {
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+          if (qrow + 8 * g + r < B) pt[8 * g + r] = out[r];
+      }
+    }
+    sp += (double)tsp;
+    ss += (double)tss;
+  }
+  __device__ void finish() {
+    double x = sp, y = ss;
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) {
+      x += __shfl_xor(x, o, 64);
+      y += __shfl_xor(y, o, 64);
+    }
+    if ((threadIdx.x & 63) == 0) {
+      const int slot = (int)((blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6)) & (BCE_SLOTS - 1));
+      atomicAdd(&a.sums[slot], x);
+      if (a.want_s) atomicAdd(&a.sums[BCE_SLOTS + slot], y);
+    }
+    if (a.dbias) {
+#pragma unroll
+      for (int t = 0; t < NQT; ++t)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          float v = rowsum[t][i];
+#pragma unroll
+          for (int o = 16; o >= 1; o >>= 1) v += __shfl_xor(v, o, 64);  // over the 32 entity columns of this half
+          const int64_t q = q0 + 32 * t + 8 * (i >> 2) + 4 * hf + (i & 3);
+          if (c == 0 && q < B) atomicAdd(&a.dbias[q], v);
+        }
     }
   }
 };
@@ -1376,7 +1502,9 @@ __global__ void __launch_bounds__(512, 2) ksplit_kernel(ContractArgs a, typename
   const int tid = threadIdx.x, lane = tid & 63, c = lane & 31, hf = lane >> 5;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int we = wave >> 1, wq = wave & 1;
-  const int d = a.d;
+  const int ldq = a.ldq ? a.ldq : a.d, lde = a.lde ? a.lde : a.d;
+  const int k_off = a.k_split_len ? (int)blockIdx.y * a.k_split_len : 0;
+  const int d = (a.k_split_len && a.d - k_off > a.k_split_len) ? a.k_split_len : a.d - k_off;  // K range of this workgroup
   const int64_t q_base = (int64_t)qg * KS_WG_QUERIES;
   const int64_t q0 = q_base + 64 * wq;
   Epi epi;
@@ -1389,7 +1517,7 @@ __global__ void __launch_bounds__(512, 2) ksplit_kernel(ContractArgs a, typename
   const int nkc = (d + KS_KC - 1) / KS_KC;
   const int n_et = (int)((r1 - r0 + KS_TILE_ROWS - 1) / KS_TILE_ROWS);
   const int n_it = n_et * nkc;
-  const float* Ef = (const float*)a.E;
+  const float* Ef = (const float*)a.E + k_off;
 
   // Staging: a chunk is 384 rows (256 entity rows, then 128 query rows) of 128 B, taken in six passes of
   // 64 rows; in pass g thread tid takes 16 B piece (tid & 7) of row 64 g + tid / 8, so eight neighbouring
@@ -1404,7 +1532,7 @@ __global__ void __launch_bounds__(512, 2) ksplit_kernel(ContractArgs a, typename
   for (int g = 0; g < 2; ++g) {
     int64_t qr = q_base + 64 * g + s_row;
     qr = qr < q_last ? qr : q_last;
-    q_ptr[g] = a.Q + qr * d;
+    q_ptr[g] = a.Q + k_off + qr * ldq;
   }
   f32x4 staged[6];             // passes 0..3: entity rows, 4..5: query rows
   int st_valid = 0;            // how many of this thread's four columns of the staged chunk are inside d
@@ -1420,7 +1548,7 @@ __global__ void __launch_bounds__(512, 2) ksplit_kernel(ContractArgs a, typename
     if (g < 4) {
       int64_t er = ld_row + 64 * g;
       er = er < e_last ? er : e_last;
-      row_ptr = Ef + er * d;
+      row_ptr = Ef + er * lde;
     } else {
       row_ptr = q_ptr[g - 4];
     }

@@ -828,6 +828,59 @@ __global__ void bce_final_kernel(const double* sums, double B, double N, float e
   }
 }
 
+// ---- backward of the BCE step: helpers -------------------------------------------------------------
+__global__ void fill_zero_kernel(float* p, int64_t n) {
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) p[i] = 0.f;
+}
+
+// out[c, r] = in[r, c] for a rows x cols matrix (row strides ld_in, ld_out), 32 x 32 tiles through LDS
+__global__ void __launch_bounds__(256) transpose_kernel(const float* in, int64_t rows, int64_t cols, int64_t ld_in,
+                                                       float* out, int64_t ld_out) {
+  __shared__ float tile[32][33];
+  const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;  // 32 x 8
+  const int64_t c0 = (int64_t)blockIdx.x * 32, r0 = (int64_t)blockIdx.y * 32;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int64_t r = r0 + ty + 8 * j, c = c0 + tx;
+    tile[ty + 8 * j][tx] = (r < rows && c < cols) ? in[r * ld_in + c] : 0.f;
+  }
+  __syncthreads();
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int64_t c = c0 + ty + 8 * j, r = r0 + tx;
+    if (c < cols && r < rows) out[c * ld_out + r] = tile[tx][ty + 8 * j];
+  }
+}
+
+// the known tails: y = 1 there, so `pos` is subtracted from both copies of the gradient and from the row sums
+__global__ void __launch_bounds__(256) grad_pos_kernel(const int64_t* csr_row, const int64_t* row_ptr,
+                                                      const int32_t* col, int64_t n_rows, int64_t B, int64_t N, float* G,
+                                                      int64_t ldG, float* GT, int64_t ldT, float* dbias, float pos) {
+  for (int64_t q = blockIdx.x; q < B; q += gridDim.x) {
+    const int64_t row = csr_row[q];
+    if (row < 0 || row >= n_rows) continue;
+    const int64_t j0 = row_ptr[row], j1 = row_ptr[row + 1];
+    int n_valid = 0;
+    for (int64_t j = j0 + threadIdx.x; j < j1; j += blockDim.x) {
+      const int64_t e = col[j];
+      if (e < 0 || e >= N) continue;
+      G[q * ldG + e] -= pos;  // a row's tails are distinct: no two threads touch one element
+      GT[e * ldT + q] -= pos;
+      ++n_valid;
+    }
+    if (dbias && n_valid) atomicAdd(&dbias[q], -pos * (float)n_valid);
+  }
+}
+
+// out[i] = sum over y of partial[y][i], y ascending
+__global__ void reduce_splits_kernel(const float* partial, int n_splits, int64_t n, float* out) {
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) {
+    float v = 0.f;
+    for (int y = 0; y < n_splits; ++y) v += partial[(int64_t)y * n + i];
+    out[i] = v;
+  }
+}
+
 // ============================================================================================
 // host side
 // ============================================================================================
@@ -870,6 +923,8 @@ ContractArgs make_args(const float* Q, const void* E, int dtype, const float* sc
   a.e_begin = e_begin;
   a.e_end = e_end;
   a.d = (int)d;
+  a.ldq = a.lde = 0;
+  a.k_split_len = 0;
   const bool fast_bf16 = (dtype == KGE_BF16 && d == 128), fast_i8 = (dtype == KGE_I8 && d == 128);
   const int f32_wgq = KGE_F32_SPLIT ? KS_WG_QUERIES : KLOOP_WG_QUERIES;
   const int wgq = (dtype == KGE_F32) ? f32_wgq : fast_bf16 ? QA_WG_QUERIES : fast_i8 ? I8_WG_QUERIES : QREG_WG_QUERIES;
@@ -901,7 +956,7 @@ ContractArgs make_args(const float* Q, const void* E, int dtype, const float* sc
   double best_eff = -1.0;
   for (int64_t chunk = tile; chunk <= max_chunk; chunk += tile) {
     const int64_t n_chunks = (rows + chunk - 1) / chunk;
-    const int64_t wgs = (n_chunks + 7) / 8 * 8 * a.n_qgroups;
+    const int64_t wgs = (n_chunks < 8) ? n_chunks * a.n_qgroups : (n_chunks + 7) / 8 * 8 * a.n_qgroups;
     const int64_t rounds = (wgs + resident - 1) / resident;
     const double eff = (double)rows * a.n_qgroups / ((double)rounds * (double)resident * (double)chunk);
     if (eff > best_eff + 0.02) {
@@ -917,12 +972,17 @@ ContractArgs make_args(const float* Q, const void* E, int dtype, const float* sc
   return a;
 }
 
+// workgroups of a non-persistent contraction launch: what decompose_wg() expects
+static int64_t contract_grid_wgs(const ContractArgs& a) {
+  return (a.n_chunks < 8) ? a.n_chunks * a.n_qgroups : (a.n_chunks + 7) / 8 * 8 * a.n_qgroups;
+}
+
 template <template <int> class EpiT, class EArgs>
 int launch_contract(int dtype, const ContractArgs& a, const EArgs& ea, hipStream_t st, const char* name) {
   if (a.B == 0 || a.e_end <= a.e_begin) return KGE_OK;
   const bool fast_i8 = (dtype == KGE_I8 && a.d == 128);
   const bool persistent = (dtype == KGE_BF16 && a.d == 128) || fast_i8;
-  const int64_t nwg = persistent ? 8 * (int64_t)a.n_qgroups * a.n_lanes : (a.n_chunks + 7) / 8 * 8 * a.n_qgroups;
+  const int64_t nwg = persistent ? 8 * (int64_t)a.n_qgroups * a.n_lanes : contract_grid_wgs(a);
   KGE_REQUIRE(nwg <= 0x7fffffffLL, KGE_ERR_INVALID, "%s: grid of %lld workgroups too large", name, (long long)nwg);
   const bool f32_split = (dtype == KGE_F32) && KGE_F32_SPLIT;
   dim3 grid((unsigned)nwg), block(fast_i8 ? 64 * I8_WG_WAVES : persistent ? 64 * QA_WG_WAVES : f32_split ? 512 : 256);
@@ -954,6 +1014,41 @@ int launch_contract(int dtype, const ContractArgs& a, const EArgs& ea, hipStream
     hipLaunchKernelGGL((qreg_i8_kernel<EpiT>), grid, block, 0, st, a, ea);
   else
     hipLaunchKernelGGL((qreg_kernel<KGE_I8, EpiT>), grid, block, 0, st, a, ea);
+  KGE_LAUNCH_CHECK(name);
+  if (timed) {
+    KGE_HIP_CHECK(hipEventRecord(ev1, st));
+    std::lock_guard<std::mutex> lk(g_prof_mu);
+    g_prof_events.emplace_back(ev0, ev1);
+  }
+  return KGE_OK;
+}
+
+// ksplit_kernel alone (fp32 operands), with row strides and an optional split of K over grid.y.
+template <template <int> class EpiT, class EArgs>
+int launch_ksplit(const ContractArgs& a, const EArgs& ea, unsigned k_splits, hipStream_t st, const char* name) {
+  if (a.B == 0 || a.e_end <= a.e_begin) return KGE_OK;
+  const int64_t nwg = contract_grid_wgs(a);
+  KGE_REQUIRE(nwg <= 0x7fffffffLL && k_splits >= 1 && k_splits <= 65535, KGE_ERR_INVALID,
+              "%s: grid of %lld x %u workgroups too large", name, (long long)nwg, k_splits);
+  const int ldq = a.ldq ? a.ldq : a.d, lde = a.lde ? a.lde : a.d;
+  const bool rows_aligned = (ldq % 4 == 0) && (lde % 4 == 0) && (((uintptr_t)a.E | (uintptr_t)a.Q) % 16 == 0) &&
+                            (a.k_split_len % 4 == 0);
+  dim3 grid((unsigned)nwg, k_splits), block(512);
+  hipEvent_t ev0 = nullptr, ev1 = nullptr;
+  bool timed = false;
+  {
+    std::lock_guard<std::mutex> lk(g_prof_mu);
+    timed = g_prof_on;
+  }
+  if (timed) {
+    KGE_HIP_CHECK(hipEventCreate(&ev0));
+    KGE_HIP_CHECK(hipEventCreate(&ev1));
+    KGE_HIP_CHECK(hipEventRecord(ev0, st));
+  }
+  if (rows_aligned)
+    hipLaunchKernelGGL((ksplit_kernel<EpiT, true>), grid, block, 0, st, a, ea);
+  else
+    hipLaunchKernelGGL((ksplit_kernel<EpiT, false>), grid, block, 0, st, a, ea);
   KGE_LAUNCH_CHECK(name);
   if (timed) {
     KGE_HIP_CHECK(hipEventRecord(ev1, st));
@@ -1050,7 +1145,7 @@ extern "C" int kge_scores(const float* Q, const float* bias, const void* E, int 
   KGE_REQUIRE(S && ldS >= N, KGE_ERR_INVALID, "kge_scores: S is null or ldS=%lld < N=%lld", (long long)ldS,
               (long long)N);
   ContractArgs a = make_args(Q, E, dtype, scale, B, d, N, 0, N);
-  StoreArgs ea{S, bias, ldS};
+  StoreArgs ea{S, bias, ldS, 0};
   return launch_contract<StoreEpi>(dtype, a, ea, (hipStream_t)stream, "kge_scores");
 }
 
@@ -1253,6 +1348,135 @@ extern "C" int kge_bce_multihot(const float* Q, const float* bias, const void* E
   }
   hipLaunchKernelGGL(bce_final_kernel, dim3(1), dim3(64), 0, st, sums, (double)B, (double)N, label_smoothing, loss);
   KGE_LAUNCH_CHECK("bce_final_kernel");
+  return KGE_OK;
+}
+
+// ---- backward of the BCE step ------------------------------------------------------------------------
+namespace {
+struct BwdPlan {
+  int64_t ldG, ldT;      // row strides of G [B, ldG] and GT [N, ldT] (multiples of 4)
+  int k_splits, k_split_len;
+  size_t off_G, off_GT, off_ET, off_QT, off_part, total;
+};
+BwdPlan bwd_plan(int64_t B, int64_t d, int64_t N) {
+  BwdPlan p;
+  p.ldG = (N + 3) / 4 * 4;
+  p.ldT = (B + 3) / 4 * 4;
+  // dQ = G . E sums over N: split so that about 256 workgroups run
+  const int64_t tiles = ((B + KS_WG_QUERIES - 1) / KS_WG_QUERIES) * ((d + KS_TILE_ROWS - 1) / KS_TILE_ROWS);
+  int64_t splits = (256 + tiles - 1) / tiles;
+  if (splits > 64) splits = 64;
+  if (splits < 1) splits = 1;
+  int64_t len = ((N + splits - 1) / splits + 31) / 32 * 32;
+  p.k_split_len = (int)len;
+  p.k_splits = (int)((N + len - 1) / len);
+  auto up = [](size_t x) { return (x + 255) / 256 * 256; };
+  size_t off = up(kge_bce_workspace_bytes());
+  p.off_G = off;     off += up((size_t)B * p.ldG * sizeof(float));
+  p.off_GT = off;    off += up((size_t)N * p.ldT * sizeof(float));
+  p.off_ET = off;    off += up((size_t)d * p.ldG * sizeof(float));
+  p.off_QT = off;    off += up((size_t)d * p.ldT * sizeof(float));
+  p.off_part = off;  off += up((size_t)p.k_splits * B * d * sizeof(float));
+  p.total = off;
+  return p;
+}
+}  // namespace
+
+extern "C" size_t kge_bce_backward_workspace_bytes(int64_t B, int64_t d, int64_t N) {
+  if (B < 1 || d < 1 || N < 1) return 0;
+  return bwd_plan(B, d, N).total;
+}
+
+extern "C" int kge_bce_multihot_backward(const float* Q, const float* bias, const void* E, int dtype, int64_t B,
+                                         int64_t d, int64_t N, const int64_t* csr_row, const int64_t* row_ptr,
+                                         const int32_t* col, int64_t n_rows, float label_smoothing, float grad_out,
+                                         float* loss, float* dQ, float* dbias, float* dE, void* workspace,
+                                         size_t workspace_bytes, void* stream) {
+  clear_error();
+  KGE_REQUIRE(dtype == KGE_F32, KGE_ERR_UNSUPPORTED, "kge_bce_multihot_backward: fp32 tables only (got dtype %d)", dtype);
+  int rc = check_contract("kge_bce_multihot_backward", Q, E, dtype, nullptr, B, d, N);
+  if (rc) return rc;
+  KGE_REQUIRE(B >= 1, KGE_ERR_INVALID, "kge_bce_multihot_backward: empty batch");
+  KGE_REQUIRE(N <= (1 << 24), KGE_ERR_UNSUPPORTED, "kge_bce_multihot_backward: N=%lld exceeds 2^24", (long long)N);
+  KGE_REQUIRE(dQ && dE, KGE_ERR_INVALID, "kge_bce_multihot_backward: null dQ or dE");
+  KGE_REQUIRE((((uintptr_t)dQ | (uintptr_t)dE) & 15) == 0, KGE_ERR_INVALID,
+              "kge_bce_multihot_backward: dQ and dE must be 16-byte aligned");
+  KGE_REQUIRE(!csr_row || (row_ptr && col), KGE_ERR_INVALID,
+              "kge_bce_multihot_backward: csr_row given without row_ptr / col");
+  const BwdPlan p = bwd_plan(B, d, N);
+  KGE_REQUIRE(workspace && workspace_bytes >= p.total, KGE_ERR_WORKSPACE,
+              "kge_bce_multihot_backward: workspace of %zu bytes, need %zu", workspace_bytes, p.total);
+  KGE_REQUIRE(((uintptr_t)workspace & 255) == 0, KGE_ERR_WORKSPACE,
+              "kge_bce_multihot_backward: workspace must be 256-byte aligned");
+  hipStream_t st = (hipStream_t)stream;
+  char* ws = (char*)workspace;
+  double* sums = (double*)ws;
+  float* G = (float*)(ws + p.off_G);
+  float* GT = (float*)(ws + p.off_GT);
+  float* ET = (float*)(ws + p.off_ET);
+  float* QT = (float*)(ws + p.off_QT);
+  float* part = (float*)(ws + p.off_part);
+  const float inv_bn = grad_out / ((float)B * (float)N);
+
+  hipLaunchKernelGGL(bce_init_kernel, dim3(1), dim3(256), 0, st, sums);
+  KGE_LAUNCH_CHECK("bce_init_kernel");
+  if (dbias) {
+    hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)((B + 255) / 256)), dim3(256), 0, st, dbias, B);
+    KGE_LAUNCH_CHECK("fill_zero_kernel");
+  }
+  // (1) scores -> g = (sigmoid(s) - dense part of y') * inv_bn, both layouts, and the loss sums
+  ContractArgs a = make_args(Q, E, KGE_F32, nullptr, B, d, N, 0, N);
+  GradArgs ga{bias, sums, G, GT, dbias, p.ldG, p.ldT, inv_bn, label_smoothing != 0.f ? inv_bn / (float)N : 0.f,
+              label_smoothing != 0.f ? 1 : 0};
+  rc = launch_ksplit<GradEpi>(a, ga, 1, st, "kge_bce_multihot_backward: scores");
+  if (rc) return rc;
+  if (csr_row && n_rows > 0) {
+    dim3 grid((unsigned)(B < 512 ? B : 512)), block(256);
+    if (loss) {
+      hipLaunchKernelGGL((bce_pos_kernel<KGE_F32>), grid, block, 0, st, a, bias, csr_row, row_ptr, col, n_rows, sums);
+      KGE_LAUNCH_CHECK("bce_pos_kernel");
+    }
+    const float pos = (label_smoothing != 0.f ? 1.0f - label_smoothing : 1.0f) * inv_bn;
+    hipLaunchKernelGGL(grad_pos_kernel, grid, block, 0, st, csr_row, row_ptr, col, n_rows, B, N, G, p.ldG, GT, p.ldT,
+                       dbias, pos);
+    KGE_LAUNCH_CHECK("grad_pos_kernel");
+  }
+  if (loss) {
+    hipLaunchKernelGGL(bce_final_kernel, dim3(1), dim3(64), 0, st, sums, (double)B, (double)N, label_smoothing, loss);
+    KGE_LAUNCH_CHECK("bce_final_kernel");
+  }
+  // (2) the other operands with the summed index contiguous: ET [d, ldG], QT [d, ldT]
+  hipLaunchKernelGGL(transpose_kernel, dim3((unsigned)((d + 31) / 32), (unsigned)((N + 31) / 32)), dim3(256), 0, st,
+                     (const float*)E, N, d, d, ET, p.ldG);
+  KGE_LAUNCH_CHECK("transpose_kernel");
+  hipLaunchKernelGGL(transpose_kernel, dim3((unsigned)((d + 31) / 32), (unsigned)((B + 31) / 32)), dim3(256), 0, st, Q, B,
+                     d, d, QT, p.ldT);
+  KGE_LAUNCH_CHECK("transpose_kernel");
+  // (3) dQ [B, d] = G . E: rows of G against rows of ET, K = N split over grid.y, partial sums reduced in order
+  {
+    ContractArgs b = make_args(G, ET, KGE_F32, nullptr, B, N, d, 0, d);
+    b.ldq = (int)p.ldG;
+    b.lde = (int)p.ldG;
+    b.k_split_len = p.k_split_len;
+    StoreArgs sa{p.k_splits > 1 ? part : dQ, nullptr, d, (int64_t)B * d};
+    rc = launch_ksplit<StoreEpi>(b, sa, (unsigned)p.k_splits, st, "kge_bce_multihot_backward: dQ");
+    if (rc) return rc;
+    if (p.k_splits > 1) {
+      const int64_t n = B * d;
+      hipLaunchKernelGGL(reduce_splits_kernel, dim3((unsigned)((n + 255) / 256 < 2048 ? (n + 255) / 256 : 2048)),
+                         dim3(256), 0, st, part, p.k_splits, n, dQ);
+      KGE_LAUNCH_CHECK("reduce_splits_kernel");
+    }
+  }
+  // (4) dE [N, d] = G^T . Q: rows of GT against rows of QT, K = B
+  {
+    ContractArgs b = make_args(GT, QT, KGE_F32, nullptr, N, B, d, 0, d);
+    b.ldq = (int)p.ldT;
+    b.lde = (int)p.ldT;
+    StoreArgs sa{dE, nullptr, d, 0};
+    rc = launch_ksplit<StoreEpi>(b, sa, 1, st, "kge_bce_multihot_backward: dE");
+    if (rc) return rc;
+  }
   return KGE_OK;
 }
 

@@ -49,6 +49,9 @@ SIGNATURES = {
     "kge_bce_workspace_bytes": (_sz, []),
     "kge_bce_multihot": (_c_int, [_vp, _vp, _vp, _c_int, _vp, _c_i64, _c_i64, _c_i64, _vp, _vp, _vp, _c_i64, _c_f,
                                   _vp, _vp, _sz, _vp]),
+    "kge_bce_backward_workspace_bytes": (_sz, [_c_i64, _c_i64, _c_i64]),
+    "kge_bce_multihot_backward": (_c_int, [_vp, _vp, _vp, _c_int, _c_i64, _c_i64, _c_i64, _vp, _vp, _vp, _c_i64,
+                                           ctypes.c_float, ctypes.c_float, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
 }
 
 _lib = None

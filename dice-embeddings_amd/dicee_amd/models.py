@@ -179,6 +179,19 @@ class BaseKGE(torch.nn.Module):
         rows = csr.rows_for(x.to(device=E.device, dtype=torch.int64))
         return ops.bce_multihot(Q, bias, E, scale, rows, csr.row_ptr, csr.col, label_smoothing)[0]
 
+    def kvsall_bce_backward(self, x, csr, label_smoothing=0.0, grad_out=1.0):
+        """The same step with its backward through the scores: ``(loss, dQ [B,d], dbias [B], dE [N,d])`` where
+        ``dQ`` / ``dbias`` are the gradients at the query vectors and per-query biases of ``self.query(x)`` and ``dE``
+        the gradient the contraction sends to the entity table (fp32 tables only).  What
+        ``loss_batch.backward()`` computes for the ``torch.mm`` / ``einsum`` and the loss of the reference's step."""
+        Q, bias = self.query(x)
+        E, scale = self.table()
+        if scale is not None:
+            raise TypeError("the backward needs an fp32 entity table")
+        rows = csr.rows_for(x.to(device=E.device, dtype=torch.int64))
+        loss, dQ, dbias, dE = ops.bce_multihot_backward(Q, bias, E, rows, csr.row_ptr, csr.col, label_smoothing, grad_out)
+        return loss[0], dQ, dbias, dE
+
 
 class DistMult(BaseKGE):
     """dicee/models/real.py:10-36."""

@@ -221,6 +221,29 @@ def bce_multihot(Q, bias, E, scale, csr_row, row_ptr, col, label_smoothing=0.0):
     return loss
 
 
+def bce_multihot_backward(Q, bias, E, csr_row, row_ptr, col, label_smoothing=0.0, grad_out=1.0, want_loss=True):
+    """Gradients of ``bce_multihot`` with respect to ``Q`` [B,d], ``bias`` [B] and the fp32 table ``E`` [N,d]:
+    ``(loss or None, dQ, dbias, dE)``.  The [B,N] gradient of the scores lives only in the call's workspace."""
+    lib = _lib.load()
+    _require_gpu(Q, bias, E, csr_row, row_ptr, col)
+    if E.dtype != torch.float32:
+        raise TypeError("bce_multihot_backward needs an fp32 entity table")
+    B, d = Q.shape
+    N = E.shape[0]
+    loss = torch.empty((1,), dtype=torch.float32, device=Q.device) if want_loss else None
+    dQ = torch.empty((B, d), dtype=torch.float32, device=Q.device)
+    dbias = torch.empty((B,), dtype=torch.float32, device=Q.device)
+    dE = torch.empty((N, d), dtype=torch.float32, device=Q.device)
+    ws_bytes = lib.kge_bce_backward_workspace_bytes(B, d, N)
+    ws = torch.empty(((ws_bytes + 7) // 8,), dtype=torch.float64, device=Q.device)
+    n_rows = 0 if row_ptr is None else row_ptr.numel() - 1
+    rc = lib.kge_bce_multihot_backward(_ptr(Q), _ptr(bias), _ptr(E), _table_dtype(E), B, d, N, _ptr(csr_row),
+                                       _ptr(row_ptr), _ptr(col), n_rows, float(label_smoothing), float(grad_out),
+                                       _ptr(loss), _ptr(dQ), _ptr(dbias), _ptr(dE), _ptr(ws), ws_bytes, _stream())
+    _lib.check(rc)
+    return loss, dQ, dbias, dE
+
+
 def profile_begin():
     """Start bracketing every contraction launch with HIP events on its stream."""
     _lib.check(_lib.load().kge_profile_begin())

@@ -234,6 +234,24 @@ int kge_bce_multihot(const float* Q, const float* bias, const void* E, int dtype
                      void* workspace, size_t workspace_bytes, void* stream);
 
 /*
+ * Backward of the same step: with S = Q E^T + bias and the mean BCE loss L of kge_bce_multihot,
+ *   g    = grad_out * (sigmoid(S) - y') / (B * N)          (y' the smoothed multi-hot target)
+ *   dQ   [B,d] = g E          dE [N,d] = g^T Q          dbias [B] = row sums of g (may be NULL)
+ * which is what autograd computes behind `loss_batch.backward()` for the KvsAll training step
+ * (dicee/models/base_model.py:25-46 with the torch.nn.BCEWithLogitsLoss of :138; the two products are
+ * the backward of the torch.mm / einsum of the model's k_vs_all_score).  `loss` may be NULL; otherwise
+ * it receives L as kge_bce_multihot gives it.  dQ, dbias and dE are overwritten.  fp32 tables only
+ * (KGE_ERR_UNSUPPORTED otherwise), N <= 2^24.  g is formed once by the fused contraction and kept in
+ * the workspace in both layouts ([B,N] and [N,B]) for the two gradient contractions, which run on the
+ * same three-part bf16 MFMA kernel as the scores; the workspace is about 8 * B * N bytes.
+ */
+size_t kge_bce_backward_workspace_bytes(int64_t B, int64_t d, int64_t N);
+int kge_bce_multihot_backward(const float* Q, const float* bias, const void* E, int dtype, int64_t B, int64_t d,
+                              int64_t N, const int64_t* csr_row, const int64_t* row_ptr, const int32_t* col,
+                              int64_t n_rows, float label_smoothing, float grad_out, float* loss, float* dQ,
+                              float* dbias, float* dE, void* workspace, size_t workspace_bytes, void* stream);
+
+/*
  * Measurement aid; no counterpart in the reference.  Between kge_profile_begin() and
  * kge_profile_end(), every launch of a contraction main loop (the MFMA kernel inside kge_scores,
  * kge_rank_filtered, kge_topk and kge_bce_multihot) is bracketed by two HIP events recorded on the

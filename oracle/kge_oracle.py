@@ -40,6 +40,8 @@ Pinning status (independent checks live in ``tests/test_oracle_pins.py``)
 * ``topk``            ``numpy.argsort`` brute force; sigmoid identity.
 * ``bce_multihot``    ``torch.nn.functional.binary_cross_entropy_with_logits``
                       on a dense target, with and without label smoothing.
+* ``bce_multihot_backward``  torch autograd (float64) through ``binary_cross_entropy_with_logits`` of
+                      ``Q @ E.T + bias`` on the dense target, with and without label smoothing.
 * ``bf16_round`` / ``quantize_int8_rows``  torch's bf16 cast; closed forms.
 * ``triple_scores``  equal to column t of the (pinned) KvsAll scores of (h, r) for all four models
                       and every (p, q); ComplEx against complex128 ``Re<h, r, conj t>``.
@@ -923,6 +925,19 @@ def bce_multihot(scores, positives, label_smoothing=0.0):
     else:
         total -= pos_sum
     return total / (B * N)
+
+
+def bce_multihot_backward(Q, bias, E, positives, label_smoothing=0.0, grad_out=1.0):
+    """Gradients of ``bce_multihot(Q @ E.T + bias[:, None], positives)``: what autograd computes behind
+    ``loss_batch.backward()`` in the KvsAll training step (dicee/models/base_model.py:25-46).
+    d loss / d score = (sigmoid(s) - y') / (B N); returns (dQ [B,d], dbias [B], dE [N,d])."""
+    Q = np.asarray(Q, dtype=np.float64)
+    E = np.asarray(E, dtype=np.float64)
+    B, N = Q.shape[0], E.shape[0]
+    s = Q @ E.T + (0.0 if bias is None else np.asarray(bias, dtype=np.float64)[:, None])
+    y = dense_multihot(positives, N, label_smoothing, dtype=np.float64)
+    g = grad_out * (sigmoid(s) - y) / (B * N)
+    return g @ E, g.sum(axis=1), g.T @ Q
 
 
 def dense_multihot(positives, N, label_smoothing=0.0, dtype=np.float32):

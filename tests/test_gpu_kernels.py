@@ -326,6 +326,53 @@ def test_bce_multihot_vs_oracle(ops, FilterCSR, model, N, R, d, B, storage, kw, 
     assert loss == pytest.approx(want, rel=tol)
 
 
+@pytest.mark.parametrize("model,N,R,d,B,kw", [
+    ("Keci", 4099, 18, 256, 300, {"p": 0, "q": 1, "coeff_q": [1.0]}),
+    ("Keci", 1000, 6, 35, 70, {"p": 3, "q": 3, "coeff_p": [0.7, 1.1, -0.3], "coeff_q": [1.3, -0.4, 0.9]}),
+    ("DistMult", 777, 5, 64, 1, {}),
+    ("ComplEx", 130, 5, 200, 513, {}),
+    ("DistMult", 40, 3, 7, 33, {}),
+])
+@pytest.mark.parametrize("eps", [0.0, 0.1])
+def test_bce_backward_vs_oracle(ops, FilterCSR, model, N, R, d, B, kw, eps):
+    """dQ, dbias and dE of the fused BCE step against the fp64 closed form (sigmoid(S) - y') / (B N) pushed
+    through the two products.  Tolerance 1e-5 of each gradient's RMS (sums of up to N resp. B fp32 terms)."""
+    rng, hr, Eg, scg, Q, bias, Ev, Rv = _setup(ops, model, N, R, d, B, "fp32", kw, seed=6, std=0.5)
+    er = random_csr(rng, hr, rng.integers(0, N, B), N, R, max_len=5, hub_rows=[(0, min(400, N // 2))])
+    csr = FilterCSR.from_er_vocab(er, R, device="cuda")
+    rows = csr.rows_for(dev(torch.from_numpy(hr)))
+    loss, dQ, dbias, dE = ops.bce_multihot_backward(Q, bias, Eg, rows, csr.row_ptr, csr.col, eps, grad_out=1.5)
+    fwd = ops.bce_multihot(Q, bias, Eg, None, rows, csr.row_ptr, csr.col, eps)
+    assert loss.item() == pytest.approx(fwd.item(), rel=1e-6)
+    Qr, br = ko.build_query(model, Ev, Rv, hr, **kw)
+    positives = [er.get((int(h), int(r)), []) for h, r in hr]
+    wQ, wb, wE = ko.bce_multihot_backward(Qr, br, Ev, positives, eps, grad_out=1.5)
+    for got, want, name in ((dQ, wQ, "dQ"), (dE, wE, "dE")):
+        got = got.cpu().numpy()
+        assert got.shape == want.shape and np.isfinite(got).all(), name
+        rms = np.sqrt((want ** 2).mean())
+        assert np.abs(got - want).max() <= 1e-5 * rms + 1e-12, (name, np.abs(got - want).max() / rms)
+    # a row sum of the score gradient cancels (sigmoid part against the known tails): bound by the sum of magnitudes
+    S = Qr @ Ev.T + br[:, None]
+    g_abs = 1.5 * (ko.sigmoid(S) + ko.dense_multihot(positives, N, eps, dtype=np.float64)) / (B * N)
+    got = dbias.cpu().numpy()
+    assert got.shape == wb.shape
+    assert np.all(np.abs(got - wb) <= 2e-6 * g_abs.sum(axis=1)), np.max(np.abs(got - wb) / g_abs.sum(axis=1))
+
+
+def test_bce_backward_argument_checks(ops):
+    from dicee_amd._lib import KgeError
+    E = torch.zeros((64, 128), device="cuda", dtype=torch.bfloat16)
+    Q = torch.zeros((4, 128), device="cuda")
+    with pytest.raises(TypeError):
+        ops.bce_multihot_backward(Q, None, E, None, None, None)
+    lib = __import__("dicee_amd._lib", fromlist=["load"]).load()
+    assert lib.kge_bce_backward_workspace_bytes(0, 8, 8) == 0
+    rc = lib.kge_bce_multihot_backward(Q.data_ptr(), None, E.data_ptr(), 1, 4, 128, 64, None, None, None, 0, 0.0, 1.0,
+                                       None, Q.data_ptr(), None, Q.data_ptr(), Q.data_ptr(), 1 << 20, None)
+    assert rc == 2                                               # KGE_ERR_UNSUPPORTED: bf16 table
+
+
 def test_argument_validation(ops):
     from dicee_amd._lib import KgeError
     E = torch.zeros((100, 24), device="cuda")

@@ -435,6 +435,24 @@ def test_bce_multihot_vs_torch_dense(eps):
 
 
 # ------------------------------------------------------------ bf16 / int8
+@pytest.mark.parametrize("eps", [0.0, 0.1])
+def test_bce_backward_vs_torch_autograd(eps):
+    rng = np.random.default_rng(13)
+    B, N, d = 9, 31, 12
+    Q = torch.tensor(rng.standard_normal((B, d)), requires_grad=True)
+    E = torch.tensor(rng.standard_normal((N, d)), requires_grad=True)
+    bias = torch.tensor(rng.standard_normal(B), requires_grad=True)
+    positives = [sorted(set(rng.integers(0, N, rng.integers(0, 6)).tolist())) for _ in range(B)]
+    y = torch.from_numpy(ko.dense_multihot(positives, N, eps, dtype=np.float64))
+    loss = torch.nn.functional.binary_cross_entropy_with_logits(Q @ E.T + bias[:, None], y)
+    (2.5 * loss).backward()
+    dQ, dbias, dE = ko.bce_multihot_backward(Q.detach().numpy(), bias.detach().numpy(), E.detach().numpy(), positives,
+                                             eps, grad_out=2.5)
+    np.testing.assert_allclose(dQ, Q.grad.numpy(), rtol=1e-10, atol=1e-14)
+    np.testing.assert_allclose(dbias, bias.grad.numpy(), rtol=1e-10, atol=1e-14)
+    np.testing.assert_allclose(dE, E.grad.numpy(), rtol=1e-10, atol=1e-14)
+
+
 def test_bf16_round_vs_torch():
     rng = np.random.default_rng(13)
     x = np.concatenate([rng.normal(0, 1, 5000), rng.normal(0, 1e-20, 100), [0.0, -0.0, 1.0, 3.3895314e38]])
