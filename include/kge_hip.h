@@ -243,7 +243,8 @@ int kge_bce_multihot(const float* Q, const float* bias, const void* E, int dtype
  * it receives L as kge_bce_multihot gives it.  dQ, dbias and dE are overwritten.  fp32 tables only
  * (KGE_ERR_UNSUPPORTED otherwise), N <= 2^24.  g is formed once by the fused contraction and kept in
  * the workspace in both layouts ([B,N] and [N,B]) for the two gradient contractions, which run on the
- * same three-part bf16 MFMA kernel as the scores; the workspace is about 8 * B * N bytes.
+ * same three-part bf16 MFMA kernel as the scores; the workspace is about 8 * B * N bytes.  dQ and dE are
+ * reproducible bit for bit from call to call; dbias is summed with floating-point atomics (order varies).
  */
 size_t kge_bce_backward_workspace_bytes(int64_t B, int64_t d, int64_t N);
 int kge_bce_multihot_backward(const float* Q, const float* bias, const void* E, int dtype, int64_t B, int64_t d,

@@ -467,3 +467,32 @@ def test_multi_hop_queries_against_the_oracle():
     assert len(both) == 2 and torch.equal(both[0], kge.predict(h=["e3"], r=["r1"]))
     with pytest.raises(ValueError):
         kge.answer_multi_hop_query(query_type="4p", query=("e3", ("r1",)))
+
+
+@pytest.mark.parametrize("name,d,extra", [("DistMult", 32, {}), ("Keci", 30, {"p": 2, "q": 2}),
+                                          ("DeCaL", 32, {"p": 2, "q": 2, "r": 3})])
+def test_kvsall_bce_backward_through_the_model(name, d, extra):
+    """Loss and gradients of the KvsAll BCE step at the query vectors, the per-query biases and the entity table,
+    against the fp64 closed form on the oracle's query vectors."""
+    from dicee_amd import FilterCSR
+    m, triples = _toy(name, d, n=900, seed=51, **extra)
+    E = m.entity_embeddings.weight.detach().numpy().copy()
+    Rel = m.relation_embeddings.weight.detach().numpy().copy()
+    kw = _oracle_kw(m)
+    er = ko.vocab(triples, "er")
+    m = m.to("cuda").eval()
+    csr = FilterCSR.from_er_vocab(er, 46, device="cuda")
+    x_np = triples[:300, :2]
+    loss, dQ, dbias, dE = m.kvsall_bce_backward(torch.from_numpy(x_np.copy()).cuda(), csr, label_smoothing=0.1)
+    Qr, br = ko.build_query(name, E, Rel, x_np, **kw)
+    positives = [er[(int(h), int(r))] for h, r in x_np]
+    want_loss = ko.bce_multihot(Qr @ E.T + br[:, None], positives, 0.1)
+    assert loss.item() == pytest.approx(want_loss, rel=1e-5)
+    wQ, wb, wE = ko.bce_multihot_backward(Qr, br, E, positives, 0.1)
+    for got, want in ((dQ, wQ), (dE, wE)):
+        assert np.abs(got.cpu().numpy() - want).max() <= 1e-5 * np.sqrt((want ** 2).mean())
+    g_abs = (ko.sigmoid(Qr @ E.T + br[:, None]) + ko.dense_multihot(positives, 135, 0.1, dtype=np.float64)) / (300 * 135)
+    assert np.all(np.abs(dbias.cpu().numpy() - wb) <= 2e-6 * g_abs.sum(axis=1))
+    m.set_entity_storage("bf16")
+    with pytest.raises(TypeError):
+        m.kvsall_bce_backward(torch.from_numpy(x_np.copy()).cuda(), csr)

@@ -120,3 +120,49 @@ def test_c5_int8_topk_matches_materialised_scores():
     np.testing.assert_allclose(wv[0], ref, rtol=2e-2)
     del model
     torch.cuda.empty_cache()
+
+
+def test_c3_bce_step_and_its_backward_at_full_size():
+    """C3 (N=40,943, d=256, fp32, batch 2048): the fused loss against the library's own materialised scores, and
+    the gradients through identities that hold for any size: dE^T 1 = Q^T dbias, <dQ, Q> = <dE, E> = <g, S - bias>,
+    linearity in the upstream gradient, and a sampled block of dQ / dE against fp64 products of the dense gradient."""
+    from dicee_amd import synthetic, ops
+    cfg = synthetic.make_config("c3")
+    model = synthetic.make_model(cfg, torch.device("cuda:0"))
+    cfg.csr.to("cuda")
+    x = torch.from_numpy(cfg.queries[:cfg.B, :2].copy()).cuda()
+    eps = 0.1
+    loss, dQ, dbias, dE = model.kvsall_bce_backward(x, cfg.csr, label_smoothing=eps)
+    assert loss.item() == pytest.approx(model.kvsall_bce_loss(x, cfg.csr, label_smoothing=eps).item(), rel=1e-6)
+    Q, bias = model.query(x)
+    E, _ = model.table()
+    S = ops.scores(Q, bias, E).double()                                 # [2048, 40943]
+    rows = cfg.csr.rows_for(x)
+    y = torch.full_like(S, 1.0 / cfg.N)
+    rp, col = cfg.csr.row_ptr.cpu().numpy(), cfg.csr.col.cpu().numpy()
+    for b, r in enumerate(rows.cpu().numpy()):
+        if r >= 0:
+            y[b, col[rp[r]:rp[r + 1]].astype(np.int64)] += 1.0 - eps
+    want_loss = torch.nn.functional.binary_cross_entropy_with_logits(S, y).item()
+    assert loss.item() == pytest.approx(want_loss, rel=1e-5)
+    g = (torch.sigmoid(S) - y) / (cfg.B * cfg.N)
+    del y
+    Qd, Ed = Q.double(), E.double()
+    # fp32 sums of 40,943 (dQ, dbias) or 2048 (dE) products that largely cancel: bound each element by the sum of
+    # the magnitudes of its terms (2e-6 of it: a few units of fp32 rounding per term at most)
+    ga = g.abs()
+    for got, want, mag, name in ((dQ, g @ Ed, ga @ Ed.abs(), "dQ"), (dE, g.T @ Qd, ga.T @ Qd.abs(), "dE"),
+                                 (dbias, g.sum(1), ga.sum(1), "dbias")):
+        worst = ((got.double() - want).abs() / mag).max().item()
+        assert worst <= 2e-6, (name, worst)
+    del ga
+    # identities on the fp32 results themselves
+    lhs, rhs = dE.double().sum(0), dbias.double() @ Qd
+    assert (lhs - rhs).abs().max().item() <= 1e-5 * rhs.abs().max().item() + 1e-12
+    a, b = (dQ.double() * Qd).sum().item(), (dE.double() * Ed).sum().item()
+    assert a == pytest.approx(b, rel=1e-5)
+    _, dQ2, dbias2, dE2 = model.kvsall_bce_backward(x, cfg.csr, label_smoothing=eps, grad_out=2.0)
+    for one, two in ((dQ, dQ2), (dE, dE2)):
+        assert torch.equal(one * 2.0, two)                             # a power of two scales every product exactly
+    # the row sums are gathered with floating-point atomics: same value up to the order of the additions
+    assert (dbias2 - 2.0 * dbias).abs().max().item() <= 2e-6 * 2.0 * g.abs().sum(1).max().item()
