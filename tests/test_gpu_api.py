@@ -496,3 +496,44 @@ def test_kvsall_bce_backward_through_the_model(name, d, extra):
     m.set_entity_storage("bf16")
     with pytest.raises(TypeError):
         m.kvsall_bce_backward(torch.from_numpy(x_np.copy()).cuda(), csr)
+
+
+def test_rank_bce_and_backward_steps_replay_from_a_hip_graph():
+    """The entry points that neither allocate nor synchronise can be captured into a HIP graph by the caller: the
+    filtered-rank step, the BCE loss and its backward, replayed several times with eager work of the same library
+    between the replays, give the eager results every time (dbias: summed with atomics, so only to rounding)."""
+    from dicee_amd import FilterCSR
+    m, triples = _toy("Keci", 30, n=1200, seed=61, p=2, q=2)
+    er = ko.vocab(triples, "er")
+    m = m.to("cuda").eval()
+    csr = FilterCSR.from_er_vocab(er, 46, device="cuda")
+    x = torch.from_numpy(triples[:400, :2].copy()).cuda()
+    t = torch.from_numpy(triples[:400, 2].copy()).cuda()
+
+    def step():
+        r = m.rank_filtered(x, t, csr)
+        loss, dQ, dbias, dE = m.kvsall_bce_backward(x, csr, label_smoothing=0.1)
+        return r, m.kvsall_bce_loss(x, csr), loss, dQ, dbias, dE
+
+    eager = step()
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(2):
+            step()                                                # warm-up on a side stream, as capture requires
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        captured = step()
+    for _ in range(3):
+        graph.replay()
+        torch.cuda.synchronize()
+        for key in eager[0]:
+            assert torch.equal(captured[0][key], eager[0][key]), key
+        assert torch.equal(captured[1], eager[1]) or captured[1].item() == pytest.approx(eager[1].item(), rel=1e-6)
+        assert captured[2].item() == pytest.approx(eager[2].item(), rel=1e-6)
+        assert torch.equal(captured[3], eager[3]) and torch.equal(captured[5], eager[5])
+        assert (captured[4] - eager[4]).abs().max().item() <= 1e-6 * eager[4].abs().max().item() + 1e-12
+        step()                                                    # eager work between replays
+        torch.cuda.synchronize()
