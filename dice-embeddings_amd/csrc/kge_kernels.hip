@@ -1002,10 +1002,12 @@ int launch_contract(int dtype, const ContractArgs& a, const EArgs& ea, hipStream
     hipLaunchKernelGGL((ksplit_kernel<EpiT, true>), grid, block, 0, st, a, ea);
   else if (f32_split)
     hipLaunchKernelGGL((ksplit_kernel<EpiT, false>), grid, block, 0, st, a, ea);
+#if !KGE_F32_SPLIT  // the fp32-MFMA main loops are only built when the split path is switched off
   else if (dtype == KGE_F32 && rows_aligned)
     hipLaunchKernelGGL((kloop_async_kernel<EpiT>), grid, block, 0, st, a, ea);
   else if (dtype == KGE_F32)
     hipLaunchKernelGGL((kloop_kernel<EpiT>), grid, block, 0, st, a, ea);
+#endif
   else if (dtype == KGE_BF16 && a.d == 128)
     hipLaunchKernelGGL((qreg_async_kernel<EpiT>), grid, block, 0, st, a, ea);
   else if (dtype == KGE_BF16)
