@@ -1106,8 +1106,8 @@ extern "C" int kge_profile_begin(void) {
   clear_error();
   std::lock_guard<std::mutex> lk(g_prof_mu);
   for (auto& p : g_prof_events) {
-    hipEventDestroy(p.first);
-    hipEventDestroy(p.second);
+    (void)hipEventDestroy(p.first);
+    (void)hipEventDestroy(p.second);
   }
   g_prof_events.clear();
   g_prof_on = true;
@@ -1130,8 +1130,8 @@ extern "C" int kge_profile_end(double* total_ms, int64_t* launches) {
     if (e == hipSuccess) e = hipEventElapsedTime(&ms, p.first, p.second);
     if (e != hipSuccess) rc = set_error(KGE_ERR_HIP, "kge_profile_end: %s", hipGetErrorString(e));
     total += ms;
-    hipEventDestroy(p.first);
-    hipEventDestroy(p.second);
+    (void)hipEventDestroy(p.first);
+    (void)hipEventDestroy(p.second);
   }
   if (total_ms) *total_ms = total;
   if (launches) *launches = (int64_t)evs.size();
