@@ -88,7 +88,7 @@ def cpu_baseline(cfg, model, mode, seconds_budget=25.0):
 def main_loop_kernel(storage, d, mode):
     """Name of the contraction kernel the library picks for this table type and width."""
     epi = {"rank": "RankEpi", "headrank": "RankEpi", "topk": "TopkEpi", "bce": "BceEpi",
-           "bcegrad": "GradEpi | StoreEpi"}[mode]
+           "bcegrad": "GradEpi | StoreEpi", "train": "GradEpi | StoreEpi"}[mode]
     if storage == "fp32":
         return f"ksplit_kernel<{epi}, {'true' if d % 4 == 0 else 'false'}>"
     if d == 128:
@@ -102,9 +102,10 @@ def main():
     ap.add_argument("--steps", type=int, default=None)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--config", default="c4", choices=sorted(MODE))
-    ap.add_argument("--mode", default=None, choices=["rank", "topk", "bce", "bcegrad", "headrank"],
+    ap.add_argument("--mode", default=None, choices=["rank", "topk", "bce", "bcegrad", "train", "headrank"],
                     help="epilogue to run instead of the configuration's own (headrank: rank the true head of "
-                         "(?, r, t) with the (r, t) -> heads filter; bcegrad: BCE loss and its gradients dQ, dbias, dE)")
+                         "(?, r, t) with the (r, t) -> heads filter; bcegrad: BCE loss and its gradients dQ, dbias, dE; "
+                         "train: loss and the gradient of every parameter, i.e. bcegrad plus the query builder's backward)")
     ap.add_argument("--scale", type=float, default=1.0, help="shrink the workload (testing only)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--graph", action="store_true",
@@ -130,7 +131,7 @@ def main():
     big = args.config in ("c4", "c5") and args.scale == 1.0
     cfg = synthetic.make_config(args.config, scale=args.scale, with_tables=not big)
     model = synthetic.make_model(cfg, dev, tables_on_device=big)
-    if mode in ("rank", "bce", "bcegrad", "headrank") and cfg.csr is None:
+    if mode in ("rank", "bce", "bcegrad", "train", "headrank") and cfg.csr is None:
         print(f"bench.py: --mode {mode} needs a configuration with triples", file=sys.stderr)
         sys.exit(2)
     if cfg.csr is not None:
@@ -160,6 +161,8 @@ def main():
             return model.topk(x, cfg.k)
         if mode == "bcegrad":
             return model.kvsall_bce_backward(x, cfg.csr)
+        if mode == "train":
+            return model.kvsall_bce_gradients(x, cfg.csr)
         return model.kvsall_bce_loss(x, cfg.csr)
 
     if args.copy_calibration:
@@ -205,14 +208,15 @@ def main():
     scores = float(n_queries) * N
     compute = "fp32" if cfg.storage == "fp32" else "bf16"
     flops = 2.0 * d * scores                                    # algorithmic: 2*d flop per entity score
-    if mode == "bcegrad":
+    if mode in ("bcegrad", "train"):
         flops *= 3.0                                            # scores, dQ = g E, dE = g^T Q
     # (inside a replayed graph the launches cannot be bracketed by host-recorded events: no kernel figure then)
     achieved = flops / (kernel_ms * 1e-3) / 1e12 if kernel_ms > 0 else None
     out = {
         "metric": {"rank": "filtered_rank_entity_scores_per_sec", "topk": "topk_entity_scores_per_sec",
                    "bce": "kvsall_bce_entity_scores_per_sec",
-                   "bcegrad": "kvsall_bce_forward_backward_entity_scores_per_sec", "headrank": "filtered_head_rank_entity_scores_per_sec"}[mode],
+                   "bcegrad": "kvsall_bce_forward_backward_entity_scores_per_sec",
+                   "train": "kvsall_bce_all_parameter_gradients_entity_scores_per_sec", "headrank": "filtered_head_rank_entity_scores_per_sec"}[mode],
         "value": scores / elapsed,
         "unit": "scores/s",
         "queries_per_sec": n_queries / elapsed,
@@ -257,7 +261,7 @@ def main():
         out["csr_build"] = {"ms": tb * 1e3, "triples": int(trip.shape[0]), "rows": built.num_rows, "nnz": built.nnz,
                             "triples_per_sec": trip.shape[0] / tb}
         del trip, built
-    if not args.no_cpu_baseline and mode not in ("headrank", "bcegrad"):
+    if not args.no_cpu_baseline and mode not in ("headrank", "bcegrad", "train"):
         out["cpu_baseline"] = cpu_baseline(cfg, model, mode)
     print(json.dumps(out))
 

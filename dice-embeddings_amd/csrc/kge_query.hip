@@ -292,6 +292,240 @@ __global__ void __launch_bounds__(64) build_query_kernel(QueryArgs a, int model)
   if (lane == 0) a.bias[b] = bias;
 }
 
+// ---- backward of the query builder ---------------------------------------------------------------
+// Given dL/dQ[b, :] and dL/dbias[b], add dL/d(head row) to d_ent[h], dL/d(relation row) to d_rel[r] and, for
+// the Clifford models, dL/d(coefficients) to d_coeff_*.  One wavefront per pair; rows that several pairs share
+// are combined with floating-point atomics.  fp32 tables, no normalisation layer.
+struct QueryBwdArgs {
+  const float* ent;
+  const float* rel;
+  const float* coeff_p;
+  const float* coeff_q;
+  const float* coeff_r;
+  const int64_t* hr;
+  const float* dQ;
+  const float* dbias;
+  float* d_ent;
+  float* d_rel;
+  float* d_coeff_p;
+  float* d_coeff_q;
+  float* d_coeff_r;
+  int64_t B, N, R;
+  int d, p, q, r, normalize_relation;
+};
+
+__global__ void __launch_bounds__(64) build_query_backward_kernel(QueryBwdArgs a, int model) {
+  extern __shared__ float lds[];
+  const int d = a.d;
+  float* sh = lds;          // head row
+  float* sr = lds + d;      // relation row
+  float* sg = lds + 2 * d;  // dL/dQ row
+  const int lane = threadIdx.x;
+  const int64_t b = blockIdx.x;
+  const int64_t h_id = a.hr[2 * b], r_id = a.hr[2 * b + 1];
+  if (h_id < 0 || h_id >= a.N || r_id < 0 || r_id >= a.R) return;  // the forward gave NaN for this pair
+  for (int k = lane; k < d; k += 64) {
+    sh[k] = a.ent[h_id * d + k];
+    sr[k] = a.rel[r_id * d + k];
+    sg[k] = a.dQ[b * d + k];
+  }
+  __syncthreads();
+  float* gh = a.d_ent + h_id * d;
+  float* gr = a.d_rel + r_id * d;
+  if (model == KGE_DISTMULT) {
+    for (int k = lane; k < d; k += 64) {
+      atomicAdd(&gh[k], sg[k] * sr[k]);
+      atomicAdd(&gr[k], sg[k] * sh[k]);
+    }
+  } else if (model == KGE_COMPLEX) {
+    const int d2 = d >> 1;
+    for (int k = lane; k < d2; k += 64) {
+      const float hr_ = sh[k], hi_ = sh[k + d2], rr_ = sr[k], ri_ = sr[k + d2], g0 = sg[k], g1 = sg[k + d2];
+      atomicAdd(&gh[k], g0 * rr_ + g1 * ri_);
+      atomicAdd(&gh[k + d2], -g0 * ri_ + g1 * rr_);
+      atomicAdd(&gr[k], g0 * hr_ + g1 * hi_);
+      atomicAdd(&gr[k + d2], -g0 * hi_ + g1 * hr_);
+    }
+  } else if (model == KGE_QMULT) {
+    const int d4 = d >> 2;
+    // sr <- normalised relation (groups of 4 consecutive elements)
+    if (a.normalize_relation) {
+      for (int g = lane; g < d4; g += 64) {
+        const float x0 = sr[4 * g], x1 = sr[4 * g + 1], x2 = sr[4 * g + 2], x3 = sr[4 * g + 3];
+        const float den = fmaxf(sqrtf(x0 * x0 + x1 * x1 + x2 * x2 + x3 * x3), 1e-12f);
+        sr[4 * g] = x0 / den;
+        sr[4 * g + 1] = x1 / den;
+        sr[4 * g + 2] = x2 / den;
+        sr[4 * g + 3] = x3 / den;
+      }
+      __syncthreads();
+    }
+    // gradient at the head parts and at the NORMALISED relation parts (block layout); the latter overwrite sh
+    for (int g = lane; g < d4; g += 64) {
+      const float ah = sh[g], bh = sh[g + d4], ch = sh[g + 2 * d4], dh = sh[g + 3 * d4];
+      const float pr = sr[g], qr = sr[g + d4], ur = sr[g + 2 * d4], vr = sr[g + 3 * d4];
+      const float G0 = sg[g], G1 = sg[g + d4], G2 = sg[g + 2 * d4], G3 = sg[g + 3 * d4];
+      atomicAdd(&gh[g], G0 * pr + G1 * qr + G2 * ur + G3 * vr);
+      atomicAdd(&gh[g + d4], -G0 * qr + G1 * pr - G2 * vr + G3 * ur);
+      atomicAdd(&gh[g + 2 * d4], -G0 * ur + G1 * vr + G2 * pr - G3 * qr);
+      atomicAdd(&gh[g + 3 * d4], -G0 * vr - G1 * ur + G2 * qr + G3 * pr);
+      sh[g] = G0 * ah + G1 * bh + G2 * ch + G3 * dh;
+      sh[g + d4] = -G0 * bh + G1 * ah + G2 * dh - G3 * ch;
+      sh[g + 2 * d4] = -G0 * ch - G1 * dh + G2 * ah + G3 * bh;
+      sh[g + 3 * d4] = -G0 * dh + G1 * ch - G2 * bh + G3 * ah;
+    }
+    __syncthreads();
+    if (!a.normalize_relation) {
+      for (int k = lane; k < d; k += 64) atomicAdd(&gr[k], sh[k]);
+    } else {
+      // y = x / max(|x|, eps) per group of 4 consecutive elements: dx = (dy - y (y . dy)) / |x|, or dy / eps
+      // where the norm was clamped
+      for (int g = lane; g < d4; g += 64) {
+        const float* raw = a.rel + r_id * d + 4 * g;
+        const float x0 = raw[0], x1 = raw[1], x2 = raw[2], x3 = raw[3];
+        const float n = sqrtf(x0 * x0 + x1 * x1 + x2 * x2 + x3 * x3);
+        const float y0 = sr[4 * g], y1 = sr[4 * g + 1], y2 = sr[4 * g + 2], y3 = sr[4 * g + 3];
+        const float e0 = sh[4 * g], e1 = sh[4 * g + 1], e2 = sh[4 * g + 2], e3 = sh[4 * g + 3];
+        if (n < 1e-12f) {
+          atomicAdd(&gr[4 * g], e0 / 1e-12f);
+          atomicAdd(&gr[4 * g + 1], e1 / 1e-12f);
+          atomicAdd(&gr[4 * g + 2], e2 / 1e-12f);
+          atomicAdd(&gr[4 * g + 3], e3 / 1e-12f);
+        } else {
+          const float dot = y0 * e0 + y1 * e1 + y2 * e2 + y3 * e3;
+          atomicAdd(&gr[4 * g], (e0 - y0 * dot) / n);
+          atomicAdd(&gr[4 * g + 1], (e1 - y1 * dot) / n);
+          atomicAdd(&gr[4 * g + 2], (e2 - y2 * dot) / n);
+          atomicAdd(&gr[4 * g + 3], (e3 - y3 * dot) / n);
+        }
+      }
+    }
+  } else if (model == KGE_OMULT) {
+    constexpr unsigned char OCT_MINUS[8] = {0xfe, 0x68, 0xc2, 0xa4, 0x0e, 0x54, 0x98, 0x32};
+    const int d8 = d >> 3;
+    for (int g = lane; g < d8; g += 64) {
+      float x[8], y[8], G[8], dx[8], dy[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        x[i] = sh[g + i * d8];
+        y[i] = sr[g + i * d8];
+        G[i] = sg[g + i * d8];
+      }
+      float den = 1.f;
+      if (a.normalize_relation) {
+        float n2 = 0.f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) n2 += y[i] * y[i];
+        den = sqrtf(n2);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) y[i] = y[i] / den;
+      }
+      // o_j = sum_i sign[j][i] x_i y_(i^j):  d x_i = sum_j sign[j][i] y_(i^j) G_j,  d y_m = sum_j sign[j][m^j] x_(m^j) G_j
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        float ax = 0.f, ay = 0.f;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const float tx = y[i ^ j] * G[j];
+          ax += ((OCT_MINUS[j] >> i) & 1) ? -tx : tx;
+          const float ty = x[i ^ j] * G[j];
+          ay += ((OCT_MINUS[j] >> (i ^ j)) & 1) ? -ty : ty;
+        }
+        dx[i] = ax;
+        dy[i] = ay;
+      }
+      if (a.normalize_relation) {
+        float dot = 0.f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) dot += y[i] * dy[i];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) dy[i] = (dy[i] - y[i] * dot) / den;
+      }
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        atomicAdd(&gh[g + i * d8], dx[i]);
+        atomicAdd(&gr[g + i * d8], dy[i]);
+      }
+    }
+  } else {  // KGE_KECI (r = 0) / KGE_DECAL
+    const int p = a.p, qn = a.q, kn = a.r;
+    const int re = d / (p + qn + kn + 1);
+    const int poff = re, qoff = re + re * p, koff = qoff + re * qn;
+    const float gb = a.dbias ? a.dbias[b] : 0.f;
+    const bool pp = p >= 2, qq = qn >= 2, kk = kn >= 2;
+    // coefficient of base i (p, then q, then r bases), the sign of its square, and its family
+    auto coeff = [&](int i) { return i < p ? a.coeff_p[i] : i < p + qn ? a.coeff_q[i - p] : a.coeff_r[i - p - qn]; };
+    auto col = [&](int rho, int i) {
+      return i < p ? poff + rho * p + i : i < p + qn ? qoff + rho * qn + (i - p) : koff + rho * kn + (i - p - qn);
+    };
+    auto family = [&](int i) { return i < p ? 0 : i < p + qn ? 1 : 2; };
+    const int nb = p + qn + kn;
+    float dc[16];  // per-lane partial gradient of up to 16 coefficients (more are handled in further rounds)
+    for (int i0 = 0; i0 < nb || i0 == 0; i0 += 16) {
+#pragma unroll
+      for (int u = 0; u < 16; ++u) dc[u] = 0.f;
+      for (int rho = lane; rho < re; rho += 64) {
+        const float h0 = sh[rho], r0 = sr[rho], G0 = sg[rho];
+        // sums of the scaled parts of each family (for the sigma terms)
+        float sum_h[3] = {0.f, 0.f, 0.f}, sum_r[3] = {0.f, 0.f, 0.f};
+        float dh0 = G0 * r0, dr0 = G0 * h0;
+        for (int i = 0; i < nb; ++i) {
+          const float c = coeff(i), hs = c * sh[col(rho, i)], rs = c * sr[col(rho, i)], Gi = sg[col(rho, i)];
+          sum_h[family(i)] += hs;
+          sum_r[family(i)] += rs;
+          dh0 += Gi * rs;
+          dr0 += Gi * hs;
+        }
+        if (i0 == 0) {
+          atomicAdd(&gh[rho], dh0);
+          atomicAdd(&gr[rho], dr0);
+        }
+        const bool fam_on[3] = {pp, qq, kk};
+        float before_h[3] = {0.f, 0.f, 0.f}, before_r[3] = {0.f, 0.f, 0.f};
+        for (int i = 0; i < nb; ++i) {
+          const int f = family(i);
+          const float c = coeff(i), hraw = sh[col(rho, i)], rraw = sr[col(rho, i)], hs = c * hraw, rs = c * rraw;
+          const float Gi = sg[col(rho, i)];
+          const float sq = (f == 0) ? 1.f : (f == 1) ? -1.f : 0.f;  // e_i^2
+          float dhs = sq * G0 * rs + Gi * r0;                       // gradient at the scaled head part
+          float drs = sq * G0 * hs + Gi * h0;
+          if (fam_on[f]) {  // same-family sigma: sum_{i<k} (h_i r_k - h_k r_i)
+            dhs += gb * ((sum_r[f] - before_r[f] - rs) - before_r[f]);
+            drs += gb * (before_h[f] - (sum_h[f] - before_h[f] - hs));
+          }
+          // cross-family sigmas (x, y) with x before y: sum (h_x r_y - h_y r_x), present when both counts >= 2
+          for (int g2 = 0; g2 < 3; ++g2) {
+            if (g2 == f || !fam_on[f] || !fam_on[g2]) continue;
+            if (f < g2) {
+              dhs += gb * sum_r[g2];
+              drs -= gb * sum_h[g2];
+            } else {
+              dhs -= gb * sum_r[g2];
+              drs += gb * sum_h[g2];
+            }
+          }
+          before_h[f] += hs;
+          before_r[f] += rs;
+          if (i0 == 0) {
+            atomicAdd(&gh[col(rho, i)], c * dhs);
+            atomicAdd(&gr[col(rho, i)], c * drs);
+          }
+          if (i >= i0 && i < i0 + 16) dc[i - i0] += hraw * dhs + rraw * drs;
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < 16; ++u) {
+        const int i = i0 + u;
+        if (i >= nb) break;  // uniform
+        const float v = wave_sum(dc[u]);
+        float* dst = i < p ? a.d_coeff_p : i < p + qn ? a.d_coeff_q : a.d_coeff_r;
+        const int idx = i < p ? i : i < p + qn ? i - p : i - p - qn;
+        if (lane == 0 && dst) atomicAdd(&dst[idx], v);
+      }
+    }
+  }
+}
+
 template <int EDT>
 int launch_build_query(const QueryArgs& a, int model, int rel_dtype, hipStream_t st) {
   dim3 grid((unsigned)a.B), block(64);
@@ -416,4 +650,67 @@ extern "C" int kge_build_query_decal(int head, int p, int q, int r, const void* 
                                      float* bias, void* stream) {
   return build_query_impl(head ? 1 : 0, KGE_DECAL, p, q, r, ent, ent_dtype, ent_scale, rel, rel_dtype, coeff_p, coeff_q,
                           coeff_r, 0, norm, pairs, B, d, N, R, Q, bias, stream);
+}
+
+extern "C" int kge_build_query_backward(int model, int p, int q, int r, const float* ent, const float* rel,
+                                        const float* coeff_p, const float* coeff_q, const float* coeff_r,
+                                        int normalize_relation, const int64_t* hr, int64_t B, int64_t d, int64_t N,
+                                        int64_t R, const float* dQ, const float* dbias, float* d_ent, float* d_rel,
+                                        float* d_coeff_p, float* d_coeff_q, float* d_coeff_r, void* stream) {
+  using namespace kge;
+  clear_error();
+  KGE_REQUIRE(B >= 0 && N > 0 && R > 0, KGE_ERR_INVALID, "kge_build_query_backward: B=%lld N=%lld R=%lld", (long long)B,
+              (long long)N, (long long)R);
+  if (B == 0) return KGE_OK;
+  KGE_REQUIRE(ent && rel && hr && dQ && d_ent && d_rel, KGE_ERR_INVALID, "kge_build_query_backward: null pointer argument");
+  KGE_REQUIRE(d >= 1 && d <= 8192, KGE_ERR_INVALID, "kge_build_query_backward: d=%lld outside [1, 8192]", (long long)d);
+  KGE_REQUIRE(B <= 0x7fffffff, KGE_ERR_INVALID, "kge_build_query_backward: B=%lld too large", (long long)B);
+  if (model != KGE_DECAL) r = 0;
+  switch (model) {
+    case KGE_DISTMULT: break;
+    case KGE_COMPLEX:
+      KGE_REQUIRE(d % 2 == 0, KGE_ERR_INVALID, "kge_build_query_backward: ComplEx needs even d, got %lld", (long long)d);
+      break;
+    case KGE_QMULT:
+      KGE_REQUIRE(d % 4 == 0, KGE_ERR_INVALID, "kge_build_query_backward: QMult needs d %% 4 == 0, got %lld", (long long)d);
+      break;
+    case KGE_OMULT:
+      KGE_REQUIRE(d % 8 == 0, KGE_ERR_INVALID, "kge_build_query_backward: OMult needs d %% 8 == 0, got %lld", (long long)d);
+      break;
+    case KGE_KECI:
+    case KGE_DECAL:
+      KGE_REQUIRE(p >= 0 && q >= 0 && r >= 0 && d % (p + q + r + 1) == 0, KGE_ERR_INVALID,
+                  "kge_build_query_backward: needs d / (p + q + r + 1) whole, got d=%lld p=%d q=%d r=%d", (long long)d, p,
+                  q, r);
+      KGE_REQUIRE((p == 0 || coeff_p) && (q == 0 || coeff_q) && (r == 0 || coeff_r), KGE_ERR_INVALID,
+                  "kge_build_query_backward: p=%d q=%d r=%d need their coefficient vectors", p, q, r);
+      break;
+    default: return set_error(KGE_ERR_INVALID, "kge_build_query_backward: unknown model %d", model);
+  }
+  QueryBwdArgs a;
+  a.ent = ent;
+  a.rel = rel;
+  a.coeff_p = coeff_p;
+  a.coeff_q = coeff_q;
+  a.coeff_r = coeff_r;
+  a.hr = hr;
+  a.dQ = dQ;
+  a.dbias = dbias;
+  a.d_ent = d_ent;
+  a.d_rel = d_rel;
+  a.d_coeff_p = d_coeff_p;
+  a.d_coeff_q = d_coeff_q;
+  a.d_coeff_r = d_coeff_r;
+  a.B = B;
+  a.N = N;
+  a.R = R;
+  a.d = (int)d;
+  a.p = p;
+  a.q = q;
+  a.r = r;
+  a.normalize_relation = normalize_relation;
+  hipStream_t st = (hipStream_t)stream;
+  hipLaunchKernelGGL(build_query_backward_kernel, dim3((unsigned)B), dim3(64), 3 * (size_t)d * sizeof(float), st, a, model);
+  KGE_LAUNCH_CHECK("build_query_backward_kernel");
+  return KGE_OK;
 }

@@ -31,6 +31,8 @@ SIGNATURES = {
                                       ctypes.POINTER(NormParams), _vp, _c_i64, _c_i64, _c_i64, _c_i64, _vp, _vp, _vp]),
     "kge_build_query_decal": (_c_int, [_c_int, _c_int, _c_int, _c_int, _vp, _c_int, _vp, _vp, _c_int, _vp, _vp, _vp,
                                        ctypes.POINTER(NormParams), _vp, _c_i64, _c_i64, _c_i64, _c_i64, _vp, _vp, _vp]),
+    "kge_build_query_backward": (_c_int, [_c_int, _c_int, _c_int, _c_int, _vp, _vp, _vp, _vp, _vp, _c_int, _vp, _c_i64,
+                                          _c_i64, _c_i64, _c_i64, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     "kge_scores": (_c_int, [_vp, _vp, _vp, _c_int, _vp, _c_i64, _c_i64, _c_i64, _vp, _c_i64, _vp]),
     "kge_triple_scores": (_c_int, [_vp, _vp, _vp, _c_int, _vp, _c_i64, _c_i64, _c_i64, _vp, _vp, _vp]),
     "kge_csr_lookup": (_c_int, [_vp, _c_i64, _vp, _c_i64, _c_i64, _vp, _vp]),

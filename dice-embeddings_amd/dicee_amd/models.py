@@ -192,6 +192,29 @@ class BaseKGE(torch.nn.Module):
         loss, dQ, dbias, dE = ops.bce_multihot_backward(Q, bias, E, rows, csr.row_ptr, csr.col, label_smoothing, grad_out)
         return loss[0], dQ, dbias, dE
 
+    def kvsall_bce_gradients(self, x, csr, label_smoothing=0.0):
+        """Loss of the KvsAll BCE step and its gradient at every parameter the step reads:
+        ``(loss, {parameter name: gradient})`` with ``entity_embeddings.weight`` [N,d] (the contraction's gradient
+        plus the rows of the heads), ``relation_embeddings.weight`` [R,d] and, for Keci / DeCaL, the coefficient
+        embeddings.  What ``loss_batch.backward()`` leaves in ``.grad`` after ``training_step`` (base_model.py:25-46)
+        for fp32 tables without a normalisation layer."""
+        if self._norm_params() is not None:
+            raise NotImplementedError("the backward does not pass through LayerNorm / BatchNorm1d")
+        E, scale = self.table()
+        if scale is not None or E.dtype != torch.float32:
+            raise TypeError("the backward needs an fp32 entity table")
+        x = x.to(device=E.device, dtype=torch.int64).contiguous()
+        loss, dQ, dbias, dE = self.kvsall_bce_backward(x, csr, label_smoothing)
+        rel = self._rel()
+        dR = torch.zeros_like(rel)
+        name = self.name if self.name != "CKeci" else "Keci"
+        dcoeff = ops.build_query_backward(name, E, rel, x, dQ, dbias, dE, dR, **self._query_kwargs())
+        grads = {"entity_embeddings.weight": dE, "relation_embeddings.weight": dR}
+        for key, g in zip(("p_coefficients.weight", "q_coefficients.weight", "r_coefficients.weight"), dcoeff):
+            if g is not None:
+                grads[key] = g.reshape(1, -1)
+        return loss, grads
+
 
 class DistMult(BaseKGE):
     """dicee/models/real.py:10-36."""

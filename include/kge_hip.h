@@ -120,6 +120,24 @@ int kge_build_query_decal(int head, int p, int q, int r, const void* ent, int en
                           int64_t d, int64_t N, int64_t R, float* Q, float* bias, void* stream);
 
 /*
+ * Backward of kge_build_query (tail direction, fp32 tables, no normalisation layer): given dL/dQ [B,d] and
+ * dL/dbias [B] (may be NULL), ADDS dL/d(head row) into d_ent[hr[b,0], :], dL/d(relation row) into
+ * d_rel[hr[b,1], :] and, for Keci / DeCaL, dL/d(coefficients) into d_coeff_p/q/r (each may be NULL).  The
+ * caller zeroes the outputs or passes gradients to accumulate onto (d_ent may be the dE of
+ * kge_bce_multihot_backward: the entity table receives both).  Rows shared by several pairs are combined
+ * with floating-point atomics.  This is the part of `loss_batch.backward()` that autograd runs through
+ * get_head_relation_representation (dicee/models/base_model.py:377-384; the embedding lookups' scatter)
+ * and the models' elementwise interaction (real.py:32, complex.py:252-264, quaternion.py:136-156 incl.
+ * quaternion_normalizer :74-100, octonion.py:119-144 incl. octonion_normalizer, clifford.py:105-113 and
+ * :269-305, DeCaL clifford.py:808-912).  r is ignored unless model == KGE_DECAL.
+ */
+int kge_build_query_backward(int model, int p, int q, int r, const float* ent, const float* rel,
+                             const float* coeff_p, const float* coeff_q, const float* coeff_r,
+                             int normalize_relation, const int64_t* hr, int64_t B, int64_t d, int64_t N, int64_t R,
+                             const float* dQ, const float* dbias, float* d_ent, float* d_rel, float* d_coeff_p,
+                             float* d_coeff_q, float* d_coeff_r, void* stream);
+
+/*
  * Materialised scores S[b, e] = dot(Q[b], E[e]) (* scale[e]) (+ bias[b]); S has row stride ldS.
  * Replaces the torch.mm / einsum calls and B x N adds of real.py:32, complex.py:260-264,
  * quaternion.py:152-156, clifford.py:269-305.  For callers that need the whole matrix

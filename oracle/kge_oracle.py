@@ -42,6 +42,9 @@ Pinning status (independent checks live in ``tests/test_oracle_pins.py``)
                       on a dense target, with and without label smoothing.
 * ``bce_multihot_backward``  torch autograd (float64) through ``binary_cross_entropy_with_logits`` of
                       ``Q @ E.T + bias`` on the dense target, with and without label smoothing.
+* ``build_query_backward``  central differences of the (pinned) ``build_query`` itself, so no Jacobian is
+                      derived by hand; checked against torch autograd through a torch transcription of the
+                      DistMult / ComplEx / QMult (normalised) forward.
 * ``bf16_round`` / ``quantize_int8_rows``  torch's bf16 cast; closed forms.
 * ``triple_scores``  equal to column t of the (pinned) KvsAll scores of (h, r) for all four models
                       and every (p, q); ComplEx against complex128 ``Re<h, r, conj t>``.
@@ -545,6 +548,54 @@ def build_query(model, E, R, hr, p=0, q=0, coeff_p=None, coeff_q=None,
     if model == "DeCaL":
         return decal_query(h, r_, p, q, r, coeff_p, coeff_q, coeff_r)
     raise ValueError(model)
+
+
+def build_query_backward(model, E, R, hr, dQ, dbias=None, step=1e-6, **kw):
+    """Gradients of ``sum_b dQ[b] . Q[b] + dbias[b] * bias[b]`` (``Q, bias = build_query``) with respect to the
+    entity table, the relation table and the Clifford coefficients: what autograd sends back through the
+    embedding lookups and the model's interaction (dicee/models/base_model.py:377-384 and the elementwise part of
+    each ``forward_k_vs_all``).  Formed by central differences in float64, one coordinate of the gathered rows at
+    a time: independent of any hand-derived Jacobian (exact up to rounding for the bilinear models, ~1e-9
+    relative through the normalisers).  Returns (dE [N,d], dR [R,d], {"coeff_p": ..., ...})."""
+    E = np.asarray(E, dtype=np.float64)
+    R = np.asarray(R, dtype=np.float64)
+    hr = np.asarray(hr)
+    dQ = np.asarray(dQ, dtype=np.float64)
+    B, d = dQ.shape
+    db = np.zeros(B) if dbias is None else np.asarray(dbias, dtype=np.float64)
+    rows_h, rows_r = E[hr[:, 0]].copy(), R[hr[:, 1]].copy()
+    pairs = np.stack([np.arange(B), np.arange(B)], axis=1)
+    kw = {k: (np.asarray(v, dtype=np.float64) if k.startswith("coeff") and v is not None else v) for k, v in kw.items()}
+
+    def per_pair(h_rows, r_rows, kwargs):
+        Q, bias = build_query(model, h_rows, r_rows, pairs, dtype=np.float64, **kwargs)
+        return (dQ * Q).sum(axis=1) + db * bias
+
+    dE, dR = np.zeros_like(E), np.zeros_like(R)
+    for k in range(d):
+        for rows, out, ids, which in ((rows_h, dE, hr[:, 0], 0), (rows_r, dR, hr[:, 1], 1)):
+            plus, minus = rows.copy(), rows.copy()
+            plus[:, k] += step
+            minus[:, k] -= step
+            if which == 0:
+                g = (per_pair(plus, rows_r, kw) - per_pair(minus, rows_r, kw)) / (2 * step)
+            else:
+                g = (per_pair(rows_h, plus, kw) - per_pair(rows_h, minus, kw)) / (2 * step)
+            np.add.at(out[:, k], ids, g)
+    dcoeff = {}
+    for key in ("coeff_p", "coeff_q", "coeff_r"):
+        c = kw.get(key)
+        if c is None or len(c) == 0:
+            continue
+        grad = np.zeros(len(c))
+        for i in range(len(c)):
+            kp, km = dict(kw), dict(kw)
+            kp[key], km[key] = c.copy(), c.copy()
+            kp[key][i] += step
+            km[key][i] -= step
+            grad[i] = ((per_pair(rows_h, rows_r, kp) - per_pair(rows_h, rows_r, km)) / (2 * step)).sum()
+        dcoeff[key] = grad
+    return dE, dR, dcoeff
 
 
 def k_vs_all_scores(model, E, R, hr, **kw):

@@ -144,7 +144,7 @@ def kvsall_bce_step(model, E, R, x, positives, label_smoothing=0.0, **kw):
     N = E.shape[0]
     ys = []
     for idx in positives:
-        y = torch.zeros(N)
+        y = torch.zeros(N, dtype=E.dtype)
         y[torch.as_tensor(np.asarray(idx, dtype=np.int64))] = 1.0
         if label_smoothing:
             y = y * (1 - label_smoothing) + (1 / N)

@@ -537,3 +537,67 @@ def test_rank_bce_and_backward_steps_replay_from_a_hip_graph():
         assert (captured[4] - eager[4]).abs().max().item() <= 1e-6 * eager[4].abs().max().item() + 1e-12
         step()                                                    # eager work between replays
         torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize("name,d,extra", [("DistMult", 32, {}), ("ComplEx", 32, {}), ("QMult", 32, {}),
+                                          ("Keci", 30, {"p": 2, "q": 2})])
+def test_full_step_gradients_match_autograd_through_the_reference_op_sequence(name, d, extra):
+    """loss and every parameter gradient of one KvsAll BCE training step against torch autograd (float64, CPU)
+    through the reference's own op sequence: embedding lookups, the model's k_vs_all_score, BCEWithLogitsLoss on
+    the dense smoothed multi-hot target."""
+    from dicee_amd import FilterCSR
+    m, triples = _toy(name, d, n=900, seed=71, **extra)
+    er = ko.vocab(triples, "er")
+    kw = _oracle_kw(m)
+    E = m.entity_embeddings.weight.detach().double().clone().requires_grad_()
+    Rel = m.relation_embeddings.weight.detach().double().clone().requires_grad_()
+    tkw = {k: (torch.tensor(v, dtype=torch.float64, requires_grad=True) if k.startswith("coeff") else v)
+           for k, v in kw.items()}
+    x_np = triples[:256, :2]
+    positives = [er[(int(h), int(r))] for h, r in x_np]
+    ref = tcp.kvsall_bce_step(name, E, Rel, torch.from_numpy(x_np.copy()), positives, 0.1, **tkw)
+    ref.backward()
+    m = m.to("cuda").eval()
+    csr = FilterCSR.from_er_vocab(er, 46, device="cuda")
+    loss, grads = m.kvsall_bce_gradients(torch.from_numpy(x_np.copy()).cuda(), csr, label_smoothing=0.1)
+    assert loss.item() == pytest.approx(ref.item(), rel=1e-5)
+    want = {"entity_embeddings.weight": E.grad, "relation_embeddings.weight": Rel.grad}
+    if "coeff_p" in tkw:
+        want["p_coefficients.weight"] = tkw["coeff_p"].grad.reshape(1, -1)
+    if "coeff_q" in tkw:
+        want["q_coefficients.weight"] = tkw["coeff_q"].grad.reshape(1, -1)
+    assert set(grads) == set(want)
+    for key, w in want.items():
+        w = w.numpy()
+        g = grads[key].cpu().numpy()
+        assert g.shape == w.shape, key
+        rms = np.sqrt((w ** 2).mean())
+        assert np.abs(g - w).max() <= 3e-5 * rms + 1e-9, (key, np.abs(g - w).max() / rms)
+
+
+def test_full_step_gradients_of_omult_and_decal_against_the_composed_oracle():
+    from dicee_amd import FilterCSR
+    for name, d, extra in (("OMult", 32, {}), ("DeCaL", 32, {"p": 2, "q": 2, "r": 3})):
+        m, triples = _toy(name, d, n=900, seed=73, **extra)
+        E = m.entity_embeddings.weight.detach().numpy().astype(np.float64)
+        Rel = m.relation_embeddings.weight.detach().numpy().astype(np.float64)
+        kw = _oracle_kw(m)
+        er = ko.vocab(triples, "er")
+        x_np = triples[:200, :2]
+        positives = [er[(int(h), int(r))] for h, r in x_np]
+        Qr, br = ko.build_query(name, E, Rel, x_np, **kw)
+        dQ, dbias, dE = ko.bce_multihot_backward(Qr, br, E, positives, 0.1)
+        dE2, dR, dc = ko.build_query_backward(name, E, Rel, x_np, dQ, dbias, **kw)
+        m = m.to("cuda").eval()
+        csr = FilterCSR.from_er_vocab(er, 46, device="cuda")
+        loss, grads = m.kvsall_bce_gradients(torch.from_numpy(x_np.copy()).cuda(), csr, label_smoothing=0.1)
+        want = {"entity_embeddings.weight": dE + dE2, "relation_embeddings.weight": dR}
+        for key, attr in (("coeff_p", "p_coefficients.weight"), ("coeff_q", "q_coefficients.weight"),
+                          ("coeff_r", "r_coefficients.weight")):
+            if key in dc:
+                want[attr] = dc[key].reshape(1, -1)
+        assert set(grads) == set(want)
+        for key, w in want.items():
+            g = grads[key].cpu().numpy()
+            rms = np.sqrt((w ** 2).mean())
+            assert np.abs(g - w).max() <= 3e-5 * rms + 1e-9, (name, key, np.abs(g - w).max() / rms)

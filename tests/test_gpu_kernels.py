@@ -554,6 +554,38 @@ def test_build_query_head_argument_checks(ops):
 
 
 # ---------------------------------------------------------------------------------------------
+# backward of the query builder
+# ---------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("model,d,kw", MODEL_CASES)
+def test_build_query_backward_fp32(ops, model, d, kw):
+    """d_ent / d_rel / d_coeff against central differences of the oracle's query builder (fp64).  Pairs share
+    heads and relations (17 relations, 77 pairs), so the scatter with atomics is exercised too."""
+    rng = np.random.default_rng(300 + d)
+    N, R, B = 60, 17, 77
+    E, Rel = random_tables(rng, N, R, d, std=0.5)
+    hr = random_hr(rng, N, R, B)
+    dQ = rng.standard_normal((B, d)).astype(np.float32)
+    dbias = rng.standard_normal(B).astype(np.float32)
+    Eg, Rg = dev(torch.from_numpy(E)), dev(torch.from_numpy(Rel))
+    d_ent = torch.zeros_like(Eg)
+    d_rel = torch.zeros_like(Rg)
+    gkw = _gpu_kwargs(kw)
+    dcoeff = ops.build_query_backward(model, Eg, Rg, dev(torch.from_numpy(hr)), dev(torch.from_numpy(dQ)),
+                                      dev(torch.from_numpy(dbias)), d_ent, d_rel, **gkw)
+    wE, wR, wc = ko.build_query_backward(model, E, Rel, hr, dQ, dbias, **kw)
+    for got, want, name in ((d_ent, wE, "d_ent"), (d_rel, wR, "d_rel")):
+        got = got.cpu().numpy()
+        rms = np.sqrt((want ** 2).mean())
+        assert np.abs(got - want).max() <= 2e-5 * rms + 1e-6, (name, np.abs(got - want).max() / rms)
+    for got, key in zip(dcoeff, ("coeff_p", "coeff_q", "coeff_r")):
+        if key in wc:
+            want = wc[key]
+            assert np.abs(got.cpu().numpy() - want).max() <= 2e-5 * np.abs(want).max() + 1e-4, key
+        else:
+            assert got is None or kw.get(key) is not None
+
+
+# ---------------------------------------------------------------------------------------------
 # seeded sweep over awkward shapes: every fused epilogue against the library's own materialised scores
 # ---------------------------------------------------------------------------------------------
 def _sweep_cases():
