@@ -215,6 +215,19 @@ class BaseKGE(torch.nn.Module):
                 grads[key] = g.reshape(1, -1)
         return loss, grads
 
+    def kvsall_training_step(self, x, csr, label_smoothing=0.0):
+        """``training_step`` followed by ``loss.backward()`` (base_model.py:25-46) for one KvsAll batch: returns the
+        loss (detached) and ACCUMULATES the gradients into ``.grad`` of the parameters the step reads, as
+        autograd would, so that any ``torch.optim`` optimizer can take the step."""
+        loss, grads = self.kvsall_bce_gradients(x, csr, label_smoothing)
+        params = dict(self.named_parameters())
+        for name, g in grads.items():
+            prm = params[name]
+            if not prm.requires_grad:
+                continue
+            prm.grad = g if prm.grad is None else prm.grad + g
+        return loss
+
 
 class DistMult(BaseKGE):
     """dicee/models/real.py:10-36."""

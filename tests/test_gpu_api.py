@@ -601,3 +601,38 @@ def test_full_step_gradients_of_omult_and_decal_against_the_composed_oracle():
             g = grads[key].cpu().numpy()
             rms = np.sqrt((w ** 2).mean())
             assert np.abs(g - w).max() <= 3e-5 * rms + 1e-9, (name, key, np.abs(g - w).max() / rms)
+
+
+def test_a_few_optimizer_steps_track_the_reference_training_loop():
+    """Ten Adam steps on a small Keci model: losses from the fused step + torch.optim on the GPU against the
+    reference's op sequence with autograd on the CPU (float64), same initial weights and batches."""
+    from dicee_amd import FilterCSR
+    m, triples = _toy("Keci", 30, n=1500, seed=81, p=2, q=2)
+    er = ko.vocab(triples, "er")
+    E = m.entity_embeddings.weight.detach().double().clone().requires_grad_()
+    Rel = m.relation_embeddings.weight.detach().double().clone().requires_grad_()
+    cp = m.p_coefficients.weight.detach().double().reshape(-1).clone().requires_grad_()
+    cq = m.q_coefficients.weight.detach().double().reshape(-1).clone().requires_grad_()
+    ref_opt = torch.optim.Adam([E, Rel, cp, cq], lr=0.05)
+    m = m.to("cuda").train()
+    for prm in m.parameters():
+        prm.requires_grad_(True)
+    opt = torch.optim.Adam(m.parameters(), lr=0.05)
+    csr = FilterCSR.from_er_vocab(er, 46, device="cuda")
+    ours, theirs = [], []
+    for step in range(10):
+        x_np = triples[step * 128:(step + 1) * 128, :2]
+        positives = [er[(int(h), int(r))] for h, r in x_np]
+        ref_opt.zero_grad()
+        ref = tcp.kvsall_bce_step("Keci", E, Rel, torch.from_numpy(x_np.copy()), positives, 0.0, p=2, q=2,
+                                  coeff_p=cp, coeff_q=cq)
+        ref.backward()
+        ref_opt.step()
+        theirs.append(ref.item())
+        opt.zero_grad(set_to_none=True)
+        loss = m.kvsall_training_step(torch.from_numpy(x_np.copy()).cuda(), csr)
+        opt.step()
+        ours.append(loss.item())
+    assert theirs[-1] < theirs[0]
+    np.testing.assert_allclose(ours, theirs, rtol=2e-4)
+    np.testing.assert_allclose(m.entity_embeddings.weight.detach().cpu().numpy(), E.detach().numpy(), atol=2e-3)
