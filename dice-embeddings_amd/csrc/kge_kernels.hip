@@ -191,24 +191,28 @@ __global__ void __launch_bounds__(256) target_score_kernel(ContractArgs a, const
   }
 }
 
-// ---- score of one given entity per query (forward_triples): the same chain, nothing else ----------
+// ---- scores of given entities per query: the same chain, nothing else ------------------------------
+// entity [B * group]: query b is scored against entity[b * group .. b * group + group - 1]
+// (group = 1: forward_triples; group = k: forward_k_vs_sample)
 template <int EDT>
 __global__ void __launch_bounds__(256) triple_score_kernel(ContractArgs a, const int64_t* target, const float* bias,
-                                                          float* out) {
+                                                          float* out, int64_t group) {
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, c = lane & 31, hf = lane >> 5;
-  const int64_t q = ((int64_t)blockIdx.x * 4 + wave) * 32 + c;
-  const int64_t t = (q < a.B) ? target[q] : -1;
+  const int64_t i = ((int64_t)blockIdx.x * 4 + wave) * 32 + c;
+  const int64_t total = a.B * group;
+  const int64_t q = (i < total) ? i / group : -1;
+  const int64_t t = (i < total) ? target[i] : -1;
   const bool ok = t >= 0 && t < a.N;
-  f32x16 acc = chain_direct<EDT>(a.E, a.d, ok ? t : -1, a.Q, (q < a.B) ? q : -1, hf);
+  f32x16 acc = chain_direct<EDT>(a.E, a.d, ok ? t : -1, a.Q, q, hf);
   const int isel = ((c >> 3) << 2) | (c & 3);  // diagonal element (entity row c, query column c)
   float v = 0.f;
 #pragma unroll
-  for (int i = 0; i < 16; ++i)
-    if (i == isel) v = acc[i];
-  if (hf == ((c >> 2) & 1) && q < a.B) {
+  for (int k = 0; k < 16; ++k)
+    if (k == isel) v = acc[k];
+  if (hf == ((c >> 2) & 1) && i < total) {
     float raw = __uint_as_float(0x7fc00000u);  // NaN for an id outside the table
     if (ok) raw = (EDT == KGE_I8) ? v * a.scale[t] : v;
-    out[q] = raw + (bias ? bias[q] : 0.f);
+    out[i] = raw + (bias ? bias[q] : 0.f);
   }
 }
 
@@ -1161,7 +1165,27 @@ extern "C" int kge_triple_scores(const float* Q, const float* bias, const void* 
   ContractArgs a = make_args(Q, E, dtype, scale, B, d, N, 0, N);
   dim3 grid((unsigned)((B + 127) / 128)), block(256);
   hipStream_t st = (hipStream_t)stream;
-  KGE_DISPATCH_DTYPE(dtype, triple_score_kernel, grid, block, 0, st, a, entity, bias, out);
+  KGE_DISPATCH_DTYPE(dtype, triple_score_kernel, grid, block, 0, st, a, entity, bias, out, (int64_t)1);
+  KGE_LAUNCH_CHECK("triple_score_kernel");
+  return KGE_OK;
+}
+
+extern "C" int kge_sample_scores(const float* Q, const float* bias, const void* E, int dtype, const float* scale,
+                                 int64_t B, int64_t d, int64_t N, const int64_t* entity, int64_t k, float* out,
+                                 void* stream) {
+  clear_error();
+  int rc = check_contract("kge_sample_scores", Q, E, dtype, scale, B, d, N);
+  if (rc) return rc;
+  KGE_REQUIRE(k >= 0, KGE_ERR_INVALID, "kge_sample_scores: k=%lld", (long long)k);
+  if (B == 0 || k == 0) return KGE_OK;
+  KGE_REQUIRE(entity && out, KGE_ERR_INVALID, "kge_sample_scores: null entity or output pointer");
+  const int64_t total = B * k;
+  KGE_REQUIRE((total + 127) / 128 <= 0x7fffffffLL, KGE_ERR_INVALID, "kge_sample_scores: B * k = %lld too large",
+              (long long)total);
+  ContractArgs a = make_args(Q, E, dtype, scale, B, d, N, 0, N);
+  dim3 grid((unsigned)((total + 127) / 128)), block(256);
+  hipStream_t st = (hipStream_t)stream;
+  KGE_DISPATCH_DTYPE(dtype, triple_score_kernel, grid, block, 0, st, a, entity, bias, out, k);
   KGE_LAUNCH_CHECK("triple_score_kernel");
   return KGE_OK;
 }

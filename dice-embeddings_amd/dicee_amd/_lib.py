@@ -35,6 +35,7 @@ SIGNATURES = {
                                           _c_i64, _c_i64, _c_i64, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     "kge_scores": (_c_int, [_vp, _vp, _vp, _c_int, _vp, _c_i64, _c_i64, _c_i64, _vp, _c_i64, _vp]),
     "kge_triple_scores": (_c_int, [_vp, _vp, _vp, _c_int, _vp, _c_i64, _c_i64, _c_i64, _vp, _vp, _vp]),
+    "kge_sample_scores": (_c_int, [_vp, _vp, _vp, _c_int, _vp, _c_i64, _c_i64, _c_i64, _vp, _c_i64, _vp, _vp]),
     "kge_csr_lookup": (_c_int, [_vp, _c_i64, _vp, _c_i64, _c_i64, _vp, _vp]),
     "kge_csr_build_workspace_bytes": (_sz, [_c_i64]),
     "kge_csr_build": (_c_int, [_vp, _c_i64, _c_int, _c_int, _c_int, _c_i64, _c_i64, _c_i64, _vp, _vp, _vp, _vp, _vp,

@@ -117,7 +117,8 @@ class BaseKGE(torch.nn.Module):
     def forward(self, x, y_idx=None):
         """Shape dispatch of BaseKGE.forward (base_model.py:310-344): [B,2] -> KvsAll scores, [n,3] -> triple scores."""
         if isinstance(x, tuple):
-            raise NotImplementedError("forward_k_vs_sample is outside the accelerated path")
+            x, y_idx = x
+            return self.forward_k_vs_sample(x=x, target_entity_idx=y_idx)
         if x.dim() == 2 and x.shape[1] == 2:
             return self.forward_k_vs_all(x=x)
         if x.dim() == 2 and x.shape[1] == 3:
@@ -129,6 +130,15 @@ class BaseKGE(torch.nn.Module):
         Q, bias = self.query(x)
         E, scale = self.table()
         return ops.scores(Q, bias, E, scale)
+
+    def forward_k_vs_sample(self, x, target_entity_idx):
+        """[B,k] fp32 scores of the k entities ``target_entity_idx[b]`` as tails of ``x[b]`` (real.py:38-45 and its
+        siblings): the query of (h, r) against the sampled rows only, the same bits as those columns of the KvsAll
+        scores."""
+        E, scale = self.table()
+        Q, bias = self.query(x)
+        idx = target_entity_idx.to(device=E.device, dtype=torch.int64)
+        return ops.sample_scores(Q, bias, E, scale, idx)
 
     def forward_triples(self, x):
         """[n] fp32 scores of the triples ``x`` [n,3] = (h, r, t) (base_model.py:346-362): the query of (h, r)

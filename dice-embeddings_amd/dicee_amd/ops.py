@@ -125,6 +125,22 @@ def triple_scores(Q, bias, E, scale, entity):
     return out
 
 
+def sample_scores(Q, bias, E, scale, entity):
+    """out[b, j] = Q[b] . E[entity[b, j]] (* scale) + bias[b] for ``entity`` int64 [B,k]."""
+    lib = _lib.load()
+    _require_gpu(Q, bias, E, scale, entity)
+    if entity.dtype != torch.int64 or entity.dim() != 2 or entity.shape[0] != Q.shape[0]:
+        raise ValueError("entity must be an int64 tensor of shape [B, k]")
+    entity = entity.contiguous()
+    B, d = Q.shape
+    k = entity.shape[1]
+    out = torch.empty((B, k), dtype=torch.float32, device=Q.device)
+    rc = lib.kge_sample_scores(_ptr(Q), _ptr(bias), _ptr(E), _table_dtype(E), _ptr(scale), B, d, E.shape[0],
+                               _ptr(entity), k, _ptr(out), _stream())
+    _lib.check(rc)
+    return out
+
+
 def row_minmax(Q, bias, E, scale=None):
     """(min [B], max [B]) of every query's scores over all entities, without the [B,N] matrix."""
     lib = _lib.load()

@@ -159,6 +159,17 @@ int kge_triple_scores(const float* Q, const float* bias, const void* E, int dtyp
                       int64_t B, int64_t d, int64_t N, const int64_t* entity, float* out, void* stream);
 
 /*
+ * Scores of k given entities per query: out[b, j] = dot(Q[b], E[entity[b, j]]) (* scale) (+ bias[b]), entity
+ * int64 [B,k], out fp32 [B,k]; the same bits as S[b, entity[b,j]] of kge_scores.  With kge_build_query this
+ * is forward_k_vs_sample (DistMult dicee/models/real.py:38-45, ComplEx complex.py:271-289, QMult
+ * quaternion.py:173-215, Keci clifford.py:363-430), the branch BaseKGE.forward takes for a tuple input
+ * (base_model.py:324-326).  The reference's Keci raises NotImplementedError for p > 0 there; here every
+ * model gives the column of its own KvsAll scores.  ids outside [0, N) give NaN.
+ */
+int kge_sample_scores(const float* Q, const float* bias, const void* E, int dtype, const float* scale,
+                      int64_t B, int64_t d, int64_t N, const int64_t* entity, int64_t k, float* out, void* stream);
+
+/*
  * Filter row of every (head, relation) pair: csr_row[b] = index of key hr[b,0]*num_relations + hr[b,1]
  * in `keys` (sorted, unique, int64 [n_rows]: the CSR's row order), or -1 if the pair has no known
  * tails.  Replaces the dict lookup `self.er_vocab[(id_e, id_r)]` of

@@ -636,3 +636,32 @@ def test_a_few_optimizer_steps_track_the_reference_training_loop():
     assert theirs[-1] < theirs[0]
     np.testing.assert_allclose(ours, theirs, rtol=2e-4)
     np.testing.assert_allclose(m.entity_embeddings.weight.detach().cpu().numpy(), E.detach().numpy(), atol=2e-3)
+
+
+@pytest.mark.parametrize("name,d,extra,storage", [("DistMult", 32, {}, "fp32"), ("ComplEx", 32, {}, "fp32"),
+                                                  ("QMult", 32, {}, "fp32"), ("Keci", 30, {"p": 2, "q": 2}, "fp32"),
+                                                  ("QMult", 128, {}, "bf16"), ("DistMult", 128, {}, "int8")])
+def test_forward_k_vs_sample_is_the_sampled_columns_of_kvsall(name, d, extra, storage):
+    """BaseKGE.forward on a tuple (x, target_entity_idx): [B,k] scores equal, bit for bit, to the sampled columns
+    of the model's own KvsAll scores, and within tolerance of the oracle."""
+    m, triples = _toy(name, d, n=400, seed=91, **extra)
+    E = m.entity_embeddings.weight.detach().numpy().copy()
+    Rel = m.relation_embeddings.weight.detach().numpy().copy()
+    kw = _oracle_kw(m)
+    m = m.to("cuda").eval()
+    m.set_entity_storage(storage)
+    rng = np.random.default_rng(5)
+    x = torch.from_numpy(triples[:150, :2].copy()).cuda()
+    idx = torch.from_numpy(rng.integers(0, 135, (150, 7))).cuda()
+    with torch.no_grad():
+        out = m((x, idx))
+        full = m(x)
+    assert out.shape == (150, 7) and out.dtype == torch.float32
+    assert torch.equal(out, torch.gather(full, 1, idx))
+    if storage == "fp32":
+        ref = ko.k_vs_all_scores(name, E, Rel, triples[:150, :2], **kw)
+        want = np.take_along_axis(ref, idx.cpu().numpy(), axis=1)
+        assert np.abs(out.cpu().numpy() - want).max() <= 1e-5 * np.sqrt((ref ** 2).mean()) + 1e-7
+    bad = idx.clone()
+    bad[0, 0] = 135
+    assert torch.isnan(m((x, bad))[0, 0])

@@ -142,6 +142,8 @@ def test_models_mirror_reference_parameters_and_have_no_cpu_fallback():
         d(torch.zeros((2, 2), dtype=torch.int64))                  # CPU tensors: refuses, never falls back
     with pytest.raises(RuntimeError):
         d(torch.zeros((2, 3), dtype=torch.int64))                  # forward_triples: the same rule
+    with pytest.raises(RuntimeError):
+        d((torch.zeros((2, 2), dtype=torch.int64), torch.zeros((2, 3), dtype=torch.int64)))   # forward_k_vs_sample too
     with pytest.raises(NotImplementedError):
         d(torch.zeros((2, 3, 4), dtype=torch.int64))               # byte-pair-encoded input
 
