@@ -62,6 +62,25 @@ def test_host_side_argument_validation_without_gpu(lib_path):
     assert rc == 2 and b"62-bit" in lib.kge_last_error()
     rc = lib.kge_csr_build(p256, -1, 0, 1, 2, 5, 5, 5, p256, p256, p256, p256, p256, 1 << 20, None)
     assert rc == 1
+    # DeCaL goes through its own entry point; the gradient entry points validate before touching the device too
+    rc = lib.kge_build_query(5, 1, 1, p256, 0, None, p256, 0, None, None, 1, None, p256, 1, 8, 10, 2, p256, p256, None)
+    assert rc == 1 and b"kge_build_query_decal" in lib.kge_last_error()
+    rc = lib.kge_build_query_decal(0, 1, 1, 1, p256, 0, None, p256, 0, p256, p256, p256, None, p256, 1, 7, 10, 2, p256,
+                                   p256, None)
+    assert rc == 1 and b"p + q + r + 1" in lib.kge_last_error()
+    rc = lib.kge_build_query_backward(1, 0, 0, 0, p256, p256, None, None, None, 1, p256, 4, 7, 10, 2, p256, None, p256,
+                                      p256, None, None, None, None)
+    assert rc == 1 and b"ComplEx" in lib.kge_last_error()
+    rc = lib.kge_bce_multihot_backward(p256, None, p256, 2, 4, 16, 100, None, None, None, 0, 0.0, 1.0, None, p256, None,
+                                       p256, p256, 1 << 30, None)
+    assert rc == 2 and b"fp32" in lib.kge_last_error()
+    need = lib.kge_bce_backward_workspace_bytes(64, 32, 1000)
+    assert need >= 2 * 64 * 1000 * 4 and need % 256 == 0
+    rc = lib.kge_bce_multihot_backward(p256, None, p256, 0, 64, 32, 1000, None, None, None, 0, 0.0, 1.0, None, p256, None,
+                                       p256, p256, need - 1, None)
+    assert rc != 0 and b"workspace" in lib.kge_last_error()
+    rc = lib.kge_sample_scores(p256, None, p256, 0, None, 4, 16, 100, None, 3, None, None)
+    assert rc == 1 and b"null" in lib.kge_last_error()
 
 
 def test_filter_csr_builders():
