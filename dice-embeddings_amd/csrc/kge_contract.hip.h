@@ -1675,4 +1675,170 @@ __global__ void __launch_bounds__(512, 2) ksplit_kernel(ContractArgs a, typename
   epi.finish();
 }
 
+// ============================================================================================
+// kchunk_bf16_kernel: bf16 table of any width (d % 8 == 0); used for d > 128, where the queries no longer
+// fit the register file of the persistent kernel.  The shape of ksplit_kernel with one part per operand:
+// 256 entities x 128 queries per workgroup of 8 waves (64 x 64 per wave), K in chunks of 64, both operands
+// staged through registers into double-buffered LDS (the fp32 queries are rounded to bf16 on the way, as in
+// the other bf16 kernels), one MFMA per 32 x 32 x 16 block.  Reduction order per score: K ascending in steps of
+// 16, as everywhere else.
+//
+// LDS row: 128 B = 8 pieces of 16 B (8 bf16); piece p of row r sits in slot r*8 + (p ^ (r & 7)).
+// ============================================================================================
+constexpr int KB_KC = 64;
+constexpr int KB_E_PLANE = KS_TILE_ROWS * 128;
+constexpr int KB_Q_PLANE = KS_WG_QUERIES * 128;
+constexpr int KB_STAGE_BYTES = KB_E_PLANE + KB_Q_PLANE;
+
+template <template <int> class EpiT>
+__global__ void __launch_bounds__(512, 2) kchunk_bf16_kernel(ContractArgs a, typename EpiT<KS_NQT>::Args ea) {
+  using Epi = EpiT<KS_NQT>;
+  __shared__ __attribute__((aligned(1024))) unsigned char lds[2 * KB_STAGE_BYTES];
+
+  int qg;
+  int64_t chunk;
+  if (!decompose_wg(a, qg, chunk)) return;
+  const int tid = threadIdx.x, lane = tid & 63, c = lane & 31, hf = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int we = wave >> 1, wq = wave & 1;
+  const int d = a.d;
+  const int64_t q_base = (int64_t)qg * KS_WG_QUERIES;
+  const int64_t q0 = q_base + 64 * wq;
+  Epi epi;
+  epi.init(ea, q0, c, hf, a.B);
+  __shared__ typename Epi::Shared epi_sh;
+  epi.bind(&epi_sh);
+
+  const int64_t r0 = a.e_begin + chunk * a.chunk_rows;
+  const int64_t r1 = (r0 + a.chunk_rows < a.e_end) ? r0 + a.chunk_rows : a.e_end;
+  const int nkc = (d + KB_KC - 1) / KB_KC;
+  const int n_et = (int)((r1 - r0 + KS_TILE_ROWS - 1) / KS_TILE_ROWS);
+  const int n_it = n_et * nkc;
+  const uint16_t* Eb = (const uint16_t*)a.E;
+
+  // Staging (branch-free, clamped addresses, zeroing at store time): entity rows as 16-byte pieces of 8 bf16,
+  // 4 passes of 64 rows (8 lanes read one 128 B line); query rows as fp32, 4 passes of 32 rows (16 lanes read
+  // 256 B of one row), rounded to bf16 when stored.
+  const int e_row = tid >> 3, e_piece = tid & 7;
+  const int q_row = tid >> 4, q_piece = tid & 15;  // q_piece: which 4 of the chunk's 64 columns
+  const int64_t q_last = a.B - 1, e_last = r1 - 1;
+  const float* q_ptr[4];
+#pragma unroll
+  for (int g = 0; g < 4; ++g) {
+    int64_t qr = q_base + 32 * g + q_row;
+    qr = qr < q_last ? qr : q_last;
+    q_ptr[g] = a.Q + qr * d;
+  }
+  u32x4 se[4];
+  f32x4 sq[4];
+  bool st_e_ok = false, st_q_ok = false, ld_e_ok = false, ld_q_ok = false;
+  int ld_kc = 0;
+  int64_t ld_row = r0 + e_row;
+  auto chunk_load = [&]() {
+    const int ke = ld_kc * KB_KC + 8 * e_piece, kq = ld_kc * KB_KC + 4 * q_piece;
+    ld_e_ok = ke < d;  // d % 8 == 0: a piece is inside d or outside as a whole
+    ld_q_ok = kq < d;
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      int64_t er = ld_row + 64 * g;
+      er = er < e_last ? er : e_last;
+      se[g] = *(const u32x4*)(Eb + er * d + (ld_e_ok ? ke : 0));
+      sq[g] = *(const f32x4*)(q_ptr[g] + (ld_q_ok ? kq : 0));
+    }
+    const bool wrap = (ld_kc == nkc - 1);
+    ld_kc = wrap ? 0 : ld_kc + 1;
+    ld_row += wrap ? KS_TILE_ROWS : 0;
+  };
+  const int e_off = e_row * 128 + ((e_piece ^ (e_row & 7)) << 4);
+  const int q_off = q_row * 128 + ((((q_piece >> 1) ^ (q_row & 7)) << 4) | ((q_piece & 1) << 3));
+  auto chunk_store = [&](int buf) {
+    unsigned char* base = lds + buf * KB_STAGE_BYTES;
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      u32x4 v = se[g];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) v[j] = st_e_ok ? v[j] : 0u;
+      *(u32x4*)(base + g * 8192 + e_off) = v;
+      f32x4 w = sq[g];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) w[j] = st_q_ok ? w[j] : 0.f;
+      bf16x4 b;
+      b[0] = (__bf16)w[0]; b[1] = (__bf16)w[1]; b[2] = (__bf16)w[2]; b[3] = (__bf16)w[3];
+      *(bf16x4*)(base + KB_E_PLANE + g * 4096 + q_off) = b;
+    }
+  };
+
+  int foff[KB_KC / 16];
+#pragma unroll
+  for (int ks = 0; ks < KB_KC / 16; ++ks) foff[ks] = c * 128 + (((2 * ks + hf) ^ (c & 7)) << 4);
+
+  f32x16 acc[2][2];
+#pragma unroll
+  for (int te = 0; te < 2; ++te)
+#pragma unroll
+    for (int tq = 0; tq < 2; ++tq)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc[te][tq][i] = 0.f;
+
+  if (n_it > 0) {
+    chunk_load();
+    st_e_ok = ld_e_ok;
+    st_q_ok = ld_q_ok;
+    chunk_store(0);
+    chunk_load();  // past the last chunk the clamped addresses still point into the tables
+  }
+  __syncthreads();
+  int kc = 0;
+  int64_t et0 = r0;
+  for (int it = 0; it < n_it; ++it) {
+    const int buf = it & 1;
+    // chunk it+1 (loaded during the previous iteration) goes to the other buffer, then chunk it+2 is requested
+    st_e_ok = ld_e_ok;
+    st_q_ok = ld_q_ok;
+    chunk_store(buf ^ 1);
+    chunk_load();
+    const unsigned char* be = lds + buf * KB_STAGE_BYTES + (64 * we) * 128;
+    const unsigned char* bq = lds + buf * KB_STAGE_BYTES + KB_E_PLANE + (64 * wq) * 128;
+    const int k_left = d - kc * KB_KC;
+#pragma unroll
+    for (int ks = 0; ks < KB_KC / 16; ++ks) {
+      if (ks * 16 >= k_left) break;  // uniform: whole K steps past d are skipped, as in the other kernels
+      bf16x8 fe[2], fq[2];
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+        fe[t] = *(const bf16x8*)(be + t * 4096 + foff[ks]);
+        fq[t] = *(const bf16x8*)(bq + t * 4096 + foff[ks]);
+      }
+#pragma unroll
+      for (int te = 0; te < 2; ++te)
+#pragma unroll
+        for (int tq = 0; tq < 2; ++tq)
+          acc[te][tq] = Epi::SWAP ? mfma_bf16(fq[tq], fe[te], acc[te][tq]) : mfma_bf16(fe[te], fq[tq], acc[te][tq]);
+    }
+    if (kc == nkc - 1) {  // this entity tile is complete
+      float sc16[16];
+#pragma unroll
+      for (int te = 0; te < 2; ++te) {
+        const int64_t e_base = et0 + 64 * we + 32 * te;
+        if (e_base < r1) {
+#pragma unroll
+          for (int tq = 0; tq < 2; ++tq) epi.template tile<false>(tq, acc[te][tq], sc16, 1.f, e_base, r1);
+        }
+#pragma unroll
+        for (int tq = 0; tq < 2; ++tq)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) acc[te][tq][i] = 0.f;
+      }
+      kc = 0;
+      et0 += KS_TILE_ROWS;
+      __syncthreads();
+      if (Epi::STAGE_HOOK) epi.stage_end();
+    } else {
+      ++kc;
+      __syncthreads();
+    }
+  }
+  epi.finish();
+}
+
 }  // namespace kge

@@ -137,9 +137,10 @@ __device__ __forceinline__ f32x16 chain_direct(const void* E, int d, int64_t e_r
     }
 #endif
   } else {
+    for (int s0 = 0; s0 < d; s0 += 128)  // eight K steps per trip (one trip for d <= 128)
 #pragma unroll
     for (int s = 0; s < 8; ++s) {
-      const int k = 16 * s + 8 * hf;
+      const int k = s0 + 16 * s + 8 * hf;
       u32x4 ev = {0u, 0u, 0u, 0u};
       f32x4 lo = {0.f, 0.f, 0.f, 0.f}, hi = {0.f, 0.f, 0.f, 0.f};
       if (k < d) {
@@ -903,7 +904,7 @@ int check_contract(const char* who, const float* Q, const void* E, int dtype, co
     case KGE_BF16:
       KGE_REQUIRE(d >= 8 && d % 8 == 0, KGE_ERR_INVALID, "%s: bf16 tables need d %% 8 == 0, got %lld", who,
                   (long long)d);
-      KGE_REQUIRE(d <= 128, KGE_ERR_UNSUPPORTED, "%s: bf16 tables support d <= 128, got %lld", who, (long long)d);
+      KGE_REQUIRE(d <= 65536, KGE_ERR_INVALID, "%s: d=%lld", who, (long long)d);
       break;
     case KGE_I8:
       KGE_REQUIRE(d >= 16 && d % 16 == 0, KGE_ERR_INVALID, "%s: int8 tables need d %% 16 == 0, got %lld", who,
@@ -931,7 +932,9 @@ ContractArgs make_args(const float* Q, const void* E, int dtype, const float* sc
   a.k_split_len = 0;
   const bool fast_bf16 = (dtype == KGE_BF16 && d == 128), fast_i8 = (dtype == KGE_I8 && d == 128);
   const int f32_wgq = KGE_F32_SPLIT ? KS_WG_QUERIES : KLOOP_WG_QUERIES;
-  const int wgq = (dtype == KGE_F32) ? f32_wgq : fast_bf16 ? QA_WG_QUERIES : fast_i8 ? I8_WG_QUERIES : QREG_WG_QUERIES;
+  const bool wide_bf16 = (dtype == KGE_BF16 && d > 128);  // kchunk_bf16_kernel: the workgroup shape of the split kernel
+  const int wgq = (dtype == KGE_F32) ? f32_wgq : fast_bf16 ? QA_WG_QUERIES : fast_i8 ? I8_WG_QUERIES
+                  : wide_bf16 ? KS_WG_QUERIES : QREG_WG_QUERIES;
   a.n_qgroups = (int)((B + wgq - 1) / wgq);
   if (a.n_qgroups < 1) a.n_qgroups = 1;
   const int64_t rows = e_end - e_begin;
@@ -953,9 +956,10 @@ ContractArgs make_args(const float* Q, const void* E, int dtype, const float* sc
   // (2 per CU, or 1 per CU for the 8-wave split kernel); choose the chunk length whose last round of
   // workgroups is fullest, preferring longer chunks (less per-workgroup set-up) among near-equal candidates.
   const bool f32_split = (dtype == KGE_F32) && KGE_F32_SPLIT;
-  const int tile = f32_split ? KS_TILE_ROWS : (dtype == KGE_F32) ? KLOOP_TILE_ROWS : QREG_STAGE_ROWS;
-  const int max_chunk = (dtype == KGE_F32) ? 1024 : 2048;
-  const int64_t resident = f32_split ? 256 : 512;
+  const bool big_tile = f32_split || wide_bf16;  // 8-wave workgroups of 256 entity rows, one per CU
+  const int tile = big_tile ? KS_TILE_ROWS : (dtype == KGE_F32) ? KLOOP_TILE_ROWS : QREG_STAGE_ROWS;
+  const int max_chunk = (dtype == KGE_F32 || wide_bf16) ? 1024 : 2048;
+  const int64_t resident = big_tile ? 256 : 512;
   int64_t best_chunk = tile;
   double best_eff = -1.0;
   for (int64_t chunk = tile; chunk <= max_chunk; chunk += tile) {
@@ -989,7 +993,8 @@ int launch_contract(int dtype, const ContractArgs& a, const EArgs& ea, hipStream
   const int64_t nwg = persistent ? 8 * (int64_t)a.n_qgroups * a.n_lanes : contract_grid_wgs(a);
   KGE_REQUIRE(nwg <= 0x7fffffffLL, KGE_ERR_INVALID, "%s: grid of %lld workgroups too large", name, (long long)nwg);
   const bool f32_split = (dtype == KGE_F32) && KGE_F32_SPLIT;
-  dim3 grid((unsigned)nwg), block(fast_i8 ? 64 * I8_WG_WAVES : persistent ? 64 * QA_WG_WAVES : f32_split ? 512 : 256);
+  const bool wide_bf16 = (dtype == KGE_BF16 && a.d > 128);
+  dim3 grid((unsigned)nwg), block(fast_i8 ? 64 * I8_WG_WAVES : persistent ? 64 * QA_WG_WAVES : (f32_split || wide_bf16) ? 512 : 256);
   hipEvent_t ev0 = nullptr, ev1 = nullptr;
   bool timed = false;
   {
@@ -1014,6 +1019,8 @@ int launch_contract(int dtype, const ContractArgs& a, const EArgs& ea, hipStream
 #endif
   else if (dtype == KGE_BF16 && a.d == 128)
     hipLaunchKernelGGL((qreg_async_kernel<EpiT>), grid, block, 0, st, a, ea);
+  else if (wide_bf16)
+    hipLaunchKernelGGL((kchunk_bf16_kernel<EpiT>), grid, block, 0, st, a, ea);
   else if (dtype == KGE_BF16)
     hipLaunchKernelGGL((qreg_kernel<KGE_BF16, EpiT>), grid, block, 0, st, a, ea);
   else if (fast_i8)

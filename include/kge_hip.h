@@ -13,9 +13,10 @@
  *     Arguments are validated on the host before anything is launched.
  *   - Entity/relation ids are int64 (what torch.LongTensor holds).  Kernels never dereference an
  *     id outside [0,N) / [0,R): such a row yields NaN scores instead of a memory fault.
- *   - Tables are row-major [rows, d].  dtype KGE_F32 computes with fp32 MFMA; KGE_BF16 and
- *     KGE_I8 (per-row symmetric int8 with a float scale per row) compute with bf16 MFMA and
- *     fp32 accumulation and currently require d <= 128, d % 8 == 0 (bf16) / d % 16 == 0 (int8).
+ *   - Tables are row-major [rows, d].  All three storages compute on the bf16 MFMA with fp32 accumulation:
+ *     KGE_F32 splits every operand into three bf16 parts and sums the six leading part products (fp32-level
+ *     accuracy, any d); KGE_BF16 needs d % 8 == 0; KGE_I8 (per-row symmetric int8 with a float scale per
+ *     row) needs d % 16 == 0 and d <= 128.
  *   - A score is `dot(Q[b], E[e]) (* scale[e]) (+ bias[b])`.  The fp32 value of the dot product
  *     is the same bit pattern in every entry point (fixed reduction order), so a rank computed
  *     by kge_rank_filtered equals the rank counted on kge_scores output exactly.

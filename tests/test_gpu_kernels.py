@@ -130,6 +130,9 @@ SCORE_CASES = [
     ("QMult", 999, 5, 128, 130, "bf16", {}),
     ("DistMult", 5000, 7, 128, 600, "bf16", {}),
     ("ComplEx", 321, 7, 64, 40, "bf16", {}),
+    ("Keci", 1500, 6, 256, 300, "bf16", {"p": 0, "q": 1, "coeff_q": [1.0]}),      # d > 128: kchunk_bf16_kernel
+    ("ComplEx", 700, 7, 200, 150, "bf16", {}),
+    ("DistMult", 300, 5, 136, 70, "bf16", {}),
     ("DistMult", 777, 9, 128, 70, "int8", {}),
     ("ComplEx", 2100, 9, 96, 520, "int8", {}),
 ]
@@ -389,8 +392,8 @@ def test_argument_validation(ops):
                         torch.zeros((1, 2), dtype=torch.int64, device="cuda"), p=1, q=1,
                         coeff_p=torch.ones(1, device="cuda"), coeff_q=torch.ones(1, device="cuda"))
     with pytest.raises(KgeError):
-        ops.scores(torch.zeros((4, 256), device="cuda"), None,
-                   torch.zeros((10, 256), device="cuda", dtype=torch.bfloat16))  # bf16 d > 128
+        ops.scores(torch.zeros((4, 256), device="cuda"), None, torch.zeros((10, 256), device="cuda", dtype=torch.int8),
+                   torch.ones(10, device="cuda"))                               # int8 d > 128
     with pytest.raises(RuntimeError):
         ops.scores(torch.zeros((4, 24)), None, torch.zeros((10, 24)))            # CPU tensors
     # empty batch is a no-op
