@@ -69,6 +69,10 @@ def cpu_baseline(cfg, model, mode, seconds_budget=25.0):
             tcp.evaluate_entity_prediction(name, E, Rel, batch, er, bs, **kw)
         elif mode == "topk":
             tcp.predict_topk_indices(name, E, Rel, torch.from_numpy(batch[:, :2].copy()), cfg.k, bs, **kw)
+        elif mode in ("bcegrad", "train"):                     # the step with autograd, as loss_batch.backward()
+            pos = [cfg.csr.tails(int(h), int(r)).astype(np.int64) for h, r, _ in batch]
+            Eg, Rg = E.clone().requires_grad_(), Rel.clone().requires_grad_()
+            tcp.kvsall_bce_step(name, Eg, Rg, torch.from_numpy(batch[:, :2].copy()), pos, 0.0, **kw).backward()
         else:
             pos = [cfg.csr.tails(int(h), int(r)).astype(np.int64) for h, r, _ in batch]
             tcp.kvsall_bce_step(name, E, Rel, torch.from_numpy(batch[:, :2].copy()), pos, 0.0, **kw)
@@ -93,6 +97,8 @@ def main_loop_kernel(storage, d, mode):
         return f"ksplit_kernel<{epi}, {'true' if d % 4 == 0 else 'false'}>"
     if d == 128:
         return f"qreg_async_kernel<{epi}>" if storage == "bf16" else f"qreg_i8_kernel<{epi}>"
+    if storage == "bf16" and d > 128:
+        return f"kchunk_bf16_kernel<{epi}>"
     return f"qreg_kernel<{storage}, {epi}>"
 
 
@@ -261,7 +267,7 @@ def main():
         out["csr_build"] = {"ms": tb * 1e3, "triples": int(trip.shape[0]), "rows": built.num_rows, "nnz": built.nnz,
                             "triples_per_sec": trip.shape[0] / tb}
         del trip, built
-    if not args.no_cpu_baseline and mode not in ("headrank", "bcegrad", "train"):
+    if not args.no_cpu_baseline and mode != "headrank":
         out["cpu_baseline"] = cpu_baseline(cfg, model, mode)
     print(json.dumps(out))
 
