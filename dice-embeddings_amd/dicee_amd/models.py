@@ -163,6 +163,11 @@ class BaseKGE(torch.nn.Module):
                                   emb_r.contiguous().float(), hr, **self._query_kwargs())
         return ops.scores(Q, bias, emb_E.contiguous().float())
 
+    def get_embeddings(self):
+        """(entity embeddings, relation embeddings) as numpy arrays (base_model.py:431-438)."""
+        return (self.entity_embeddings.weight.detach().cpu().numpy(),
+                self.relation_embeddings.weight.detach().cpu().numpy())
+
     # ------------------------------------------------------------------ fused consumers
     def rank_filtered(self, x, target, csr=None, heads=False):
         """Fused filtered-rank counters for queries ``x`` [B,2] and true tails ``target`` [B].
