@@ -164,9 +164,9 @@ class BaseKGE(torch.nn.Module):
         return ops.scores(Q, bias, emb_E.contiguous().float())
 
     def get_embeddings(self):
-        """(entity embeddings, relation embeddings) as numpy arrays (base_model.py:431-438)."""
-        return (self.entity_embeddings.weight.detach().cpu().numpy(),
-                self.relation_embeddings.weight.detach().cpu().numpy())
+        """(entity embeddings, relation embeddings), detached tensors as the reference returns them
+        (base_model.py:431-438; its annotation says ndarray, its code returns tensors)."""
+        return self.entity_embeddings.weight.detach(), self.relation_embeddings.weight.detach()
 
     # ------------------------------------------------------------------ fused consumers
     def rank_filtered(self, x, target, csr=None, heads=False):
