@@ -253,6 +253,22 @@ def main():
         "setup_s": t_setup,
         "device": torch.cuda.get_device_name(0),
     }
+    # side figure, outside the timed region: the gather + interaction kernel alone (HBM-bound, launch-latency sized)
+    xg = batches[0][0]
+    for _ in range(3):
+        model.query(xg, heads=(mode == "headrank"))
+    torch.cuda.synchronize()
+    tg = time.perf_counter()
+    for _ in range(50):
+        model.query(xg, heads=(mode == "headrank"))
+    torch.cuda.synchronize()
+    tg = (time.perf_counter() - tg) / 50
+    esz = {"fp32": 4, "bf16": 2, "int8": 1}[cfg.storage]
+    gbytes = xg.shape[0] * d * (esz + (2 if cfg.storage == "bf16" else 4)) + 4 * xg.shape[0] * d + 16 * xg.shape[0]
+    out["gather"] = {"kernel": "build_query_kernel", "us_per_call": tg * 1e6, "bytes": gbytes,
+                     "GB/s": gbytes / tg / 1e9, "frac_of_hbm_peak": gbytes / tg / 8e12,
+                     "note": "head and relation rows read, query rows written; wall time of back-to-back calls from Python, "
+                             "so launch and binding overhead are inside (the kernel alone: see profiles/)"}
     if len(cfg.triples):
         # side figure, outside the timed region: the known-answer vocabulary of all triples as a CSR, built on
         # the GPU (kge_csr_build) from ids already resident in HBM
