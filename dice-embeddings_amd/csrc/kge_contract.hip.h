@@ -1,11 +1,11 @@
 // Query x all-entity contraction on MFMA with fused epilogues (gfx950).
 //
-// Two main loops share one epilogue interface:
-//   qreg_kernel   bf16 MFMA (32x32x16), entity table bf16 or per-row int8, d <= 128.  Each wave keeps
-//                 the bf16 fragments of 128 queries in registers for the whole kernel and streams
-//                 64-row entity stages through a double-buffered, padded LDS panel.
-//   kloop_kernel  fp32 MFMA (32x32x2), any d.  Classic 128x128 workgroup tile, K staged through LDS
-//                 in chunks of 32.
+// All main loops run on the bf16 MFMA (32x32x16) and share one epilogue interface:
+//   qreg_async_kernel   bf16 table, d == 128: persistent, queries register-resident, entity rows global -> LDS
+//   qreg_i8_kernel      per-row int8 table, d == 128: the same walk, rows widened to bf16 on the way into LDS
+//   qreg_kernel         bf16 / int8 with d < 128
+//   kchunk_bf16_kernel  bf16 with d > 128: K in chunks of 64 through LDS
+//   ksplit_kernel       fp32 tables, any d: every operand as three bf16 parts, six part products per product
 // Reduction order of one score is fixed (k ascending in steps of the MFMA depth, nothing else), so
 // every kernel that forms dot(Q[b], E[e]) with these helpers produces the same fp32 bit pattern.
 //
@@ -15,18 +15,6 @@
 // write scores set SWAP so that consecutive lanes hold consecutive entities (coalesced stores).
 #pragma once
 #include "kge_internal.h"
-
-#ifndef KGE_SCHED_HINTS
-#define KGE_SCHED_HINTS 0
-#endif
-#ifndef KGE_KS_SCHED
-#define KGE_KS_SCHED 1
-#endif
-// 1: fp32 tables are multiplied on the bf16 MFMA as three bf16 parts per operand (ksplit_kernel);
-// 0: on the fp32 MFMA (kloop_async_kernel / kloop_kernel).  One switch for every kernel that forms a score.
-#ifndef KGE_F32_SPLIT
-#define KGE_F32_SPLIT 1
-#endif
 
 namespace kge {
 
@@ -49,9 +37,6 @@ struct ContractArgs {
 
 __device__ __forceinline__ f32x16 mfma_bf16(bf16x8 a, bf16x8 b, f32x16 c) {
   return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
-}
-__device__ __forceinline__ f32x16 mfma_f32(float a, float b, f32x16 c) {
-  return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0);
 }
 
 __device__ __forceinline__ bf16x8 cvt_bf16x8(f32x4 lo, f32x4 hi) {
@@ -645,34 +630,6 @@ struct MinMaxEpi {
   }
 };
 
-#ifdef KGE_DEBUG
-// Measurement-only epilogue: keeps the accumulators alive with two VALU ops per tile.
-struct NullArgs {
-  float* out;
-};
-template <int NQT>
-struct NullEpi {
-  static constexpr bool SWAP = false;
-  static constexpr bool STAGE_HOOK = false;
-  struct Shared {
-    int unused;
-  };
-  __device__ void bind(Shared*) {}
-  __device__ void stage_end() {}
-  using Args = NullArgs;
-  Args a;
-  float sink;
-  __device__ void init(const Args& args, int64_t, int, int, int64_t) { a = args; sink = 0.f; }
-  template <bool HAS_SCALE>
-  __device__ __forceinline__ void tile(int, const f32x16& acc, const float*, float, int64_t, int64_t) {
-    sink += acc[0] + acc[15];
-  }
-  __device__ void finish() {
-    if (sink == 12345.678f) a.out[0] = sink;
-  }
-};
-#endif
-
 // ============================================================================================
 // qreg_kernel: bf16 MFMA, register-stationary queries, LDS-streamed entity rows.
 // ============================================================================================
@@ -796,8 +753,6 @@ __global__ void __launch_bounds__(256, 2) qreg_kernel(ContractArgs a, typename E
     }
 #pragma unroll
     for (int j = 0; j < TILES; ++j) {
-      constexpr int dummy = 0;
-      (void)dummy;
       const int et = j / QREG_NQT, t = j % QREG_NQT;
       const int t_prev = (j + QREG_NQT - 1) % QREG_NQT;
       f32x16 acc;
@@ -807,14 +762,6 @@ __global__ void __launch_bounds__(256, 2) qreg_kernel(ContractArgs a, typename E
       for (int s = 0; s < 8; ++s)
         acc = Epi::SWAP ? mfma_bf16(qf[t][s], ef[et][s], acc) : mfma_bf16(ef[et][s], qf[t][s], acc);
       epi.template tile<HAS_SCALE>(t_prev, acc_prev, sc_prev, sc_col_prev, e_prev, r1);
-#if KGE_SCHED_HINTS
-#pragma unroll
-      for (int g = 0; g < 8; ++g) {
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // one MFMA
-        __builtin_amdgcn_sched_group_barrier(0x002, 6, 0);  // six VALU ops of the previous tile's epilogue
-        __builtin_amdgcn_sched_group_barrier(0x004, 2, 0);  // and their scalar mask merges
-      }
-#endif
       acc_prev = acc;
       e_prev = row0 + et * 32;
       if (HAS_SCALE) {
@@ -961,18 +908,12 @@ __global__ void __launch_bounds__(64 * QA_WG_WAVES, QA_WAVES_PER_SIMD) qreg_asyn
     const int buf = st & 1;
     const int64_t row0 = row_next;
     if (row0 >= r_end) break;  // only the trailing stages of the table's last chunk can be empty
-#ifndef KGE_DBG_NO_BARRIER
-#ifndef KGE_DBG_NO_VMWAIT
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-#endif
     __syncthreads();  // stage st has landed for every wave; everyone is done reading the other buffer
-#endif
     if (Epi::STAGE_HOOK) epi.stage_end();
     if (st + 1 < total_stages) {
       row_next = stage_row(st + 1);
-#ifndef KGE_DBG_NO_GLOBAL
       if (row_next < r_end) stage_issue(row_next, buf ^ 1);
-#endif
     }
     const unsigned char* base = lds_e + buf * QA_BUF_BYTES;
     bf16x8 ef[8];
@@ -992,22 +933,9 @@ __global__ void __launch_bounds__(64 * QA_WG_WAVES, QA_WAVES_PER_SIMD) qreg_asyn
         for (int s = 0; s < 8; ++s) {
           acc = Epi::SWAP ? mfma_bf16(qf[t][s], ef[s], acc) : mfma_bf16(ef[s], qf[t][s], acc);
           // last use of fragment s for this e-tile: fetch the next e-tile's fragment into its place
-#ifndef KGE_DBG_NO_LDSREAD
           if (refill) efn[s] = *(const bf16x8*)(base + (et + 1) * 8192 + foff[s]);
-#else
-          if (refill) efn[s] = ef[s];
-#endif
         }
         epi.template tile<false>(t_prev, acc_prev, sc_dummy, 1.f, e_prev, r_end);
-#if KGE_SCHED_HINTS
-#pragma unroll
-        for (int g = 0; g < 8; ++g) {
-          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // one MFMA
-          if (refill) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // one fragment read
-          __builtin_amdgcn_sched_group_barrier(0x002, 6, 0);  // VALU of the previous tile's epilogue
-          __builtin_amdgcn_sched_group_barrier(0x004, 2, 0);  // its scalar mask merges
-        }
-#endif
         if (refill) {
 #pragma unroll
           for (int s = 0; s < 8; ++s) ef[s] = efn[s];
@@ -1181,299 +1109,6 @@ __global__ void __launch_bounds__(64 * I8_WG_WAVES, 2) qreg_i8_kernel(ContractAr
 }
 
 // ============================================================================================
-// kloop_kernel: fp32 MFMA, 128 entities x 128 queries per workgroup, K chunks of 32 through LDS.
-// Chain order per score: k-blocks of 8 ascending; inside a block MFMA step j (0..3) consumes
-// k0 + j (lanes 0-31) and k0 + 4 + j (lanes 32-63).
-// ============================================================================================
-constexpr int KLOOP_NQT = 2;
-constexpr int KLOOP_WG_QUERIES = 128;
-constexpr int KLOOP_TILE_ROWS = 128;
-constexpr int KLOOP_KC = 32;
-constexpr int KLOOP_LDK = 36;  // floats per LDS row: 32 + 4 pad
-
-template <template <int> class EpiT>
-__global__ void __launch_bounds__(256, 2) kloop_kernel(ContractArgs a, typename EpiT<KLOOP_NQT>::Args ea) {
-  using Epi = EpiT<KLOOP_NQT>;
-  __shared__ __attribute__((aligned(16))) float lds_e[2][KLOOP_TILE_ROWS * KLOOP_LDK];
-  __shared__ __attribute__((aligned(16))) float lds_q[2][KLOOP_WG_QUERIES * KLOOP_LDK];
-
-  int qg;
-  int64_t chunk;
-  if (!decompose_wg(a, qg, chunk)) return;
-  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, c = lane & 31, hf = lane >> 5;
-  const int we = wave >> 1, wq = wave & 1;
-  const int d = a.d;
-  const bool vec_ok = (d & 3) == 0;
-  const int64_t q_base = (int64_t)qg * KLOOP_WG_QUERIES;
-  const int64_t q0 = q_base + 64 * wq;
-  Epi epi;
-  epi.init(ea, q0, c, hf, a.B);
-  __shared__ typename Epi::Shared epi_sh;
-  epi.bind(&epi_sh);
-
-  const int64_t r0 = a.e_begin + chunk * a.chunk_rows;
-  const int64_t r1 = (r0 + a.chunk_rows < a.e_end) ? r0 + a.chunk_rows : a.e_end;
-  const int nkc = (d + KLOOP_KC - 1) / KLOOP_KC;
-  const float* Ef = (const float*)a.E;
-
-  auto load4 = [&](const float* base, int64_t row, bool row_ok, int k) -> f32x4 {
-    f32x4 v = {0.f, 0.f, 0.f, 0.f};
-    if (row_ok) {
-      const float* p = base + row * d + k;
-      if (vec_ok) {
-        if (k < d) v = *(const f32x4*)p;
-      } else {
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-          if (k + j < d) v[j] = p[j];
-      }
-    }
-    return v;
-  };
-
-  // Flat pipeline over (entity tile, K chunk): the next chunk's global loads are in flight while the
-  // current chunk is multiplied; LDS is double-buffered, one barrier per chunk.
-  const int n_et = (int)((r1 - r0 + KLOOP_TILE_ROWS - 1) / KLOOP_TILE_ROWS);
-  const int n_it = n_et * nkc;
-  f32x4 ve[4], vq[4];
-  auto chunk_load = [&](int it) {
-    const int et = it / nkc, kc = it - et * nkc;
-    const int64_t et0 = r0 + (int64_t)et * KLOOP_TILE_ROWS;
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int idx = tid + 256 * j, row = idx >> 3, piece = idx & 7;
-      const int k = kc * KLOOP_KC + piece * 4;
-      ve[j] = load4(Ef, et0 + row, et0 + row < r1, k);
-      vq[j] = load4(a.Q, q_base + row, q_base + row < a.B, k);
-    }
-  };
-  auto chunk_store = [&](int buf) {
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int idx = tid + 256 * j, row = idx >> 3, piece = idx & 7;
-      *(f32x4*)&lds_e[buf][row * KLOOP_LDK + piece * 4] = ve[j];
-      *(f32x4*)&lds_q[buf][row * KLOOP_LDK + piece * 4] = vq[j];
-    }
-  };
-  f32x16 acc[2][2];
-#pragma unroll
-  for (int te = 0; te < 2; ++te)
-#pragma unroll
-    for (int tq = 0; tq < 2; ++tq)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) acc[te][tq][i] = 0.f;
-
-  if (n_it > 0) {
-    chunk_load(0);
-    chunk_store(0);
-  }
-  __syncthreads();
-  int kc = 0;
-  int64_t et0 = r0;
-  for (int it = 0; it < n_it; ++it) {
-    const int buf = it & 1;
-#ifndef KGE_DBG_NO_GLOBAL
-    if (it + 1 < n_it) chunk_load(it + 1);
-#endif
-#pragma unroll
-    for (int kb = 0; kb < KLOOP_KC / 8; ++kb) {
-      f32x4 fe[2], fq[2];
-#pragma unroll
-      for (int t = 0; t < 2; ++t) {
-        fe[t] = *(const f32x4*)&lds_e[buf][(64 * we + 32 * t + c) * KLOOP_LDK + kb * 8 + 4 * hf];
-        fq[t] = *(const f32x4*)&lds_q[buf][(64 * wq + 32 * t + c) * KLOOP_LDK + kb * 8 + 4 * hf];
-      }
-#pragma unroll
-      for (int j = 0; j < 4; ++j)
-#pragma unroll
-        for (int te = 0; te < 2; ++te)
-#pragma unroll
-          for (int tq = 0; tq < 2; ++tq)
-            acc[te][tq] = Epi::SWAP ? mfma_f32(fq[tq][j], fe[te][j], acc[te][tq])
-                                    : mfma_f32(fe[te][j], fq[tq][j], acc[te][tq]);
-    }
-#ifndef KGE_DBG_NO_SCHEDBAR
-    __builtin_amdgcn_sched_barrier(0);  // ... and waited for after them
-#endif
-#ifndef KGE_DBG_NO_LDSWRITE
-    if (it + 1 < n_it) chunk_store(buf ^ 1);
-#endif
-    if (kc == nkc - 1) {  // this entity tile is complete
-      float sc16[16];
-#pragma unroll
-      for (int te = 0; te < 2; ++te) {
-        const int64_t e_base = et0 + 64 * we + 32 * te;
-        if (e_base < r1) {
-#pragma unroll
-          for (int tq = 0; tq < 2; ++tq) epi.template tile<false>(tq, acc[te][tq], sc16, 1.f, e_base, r1);
-        }
-#pragma unroll
-        for (int tq = 0; tq < 2; ++tq)
-#pragma unroll
-          for (int i = 0; i < 16; ++i) acc[te][tq][i] = 0.f;
-      }
-      kc = 0;
-      et0 += KLOOP_TILE_ROWS;
-      __syncthreads();
-      if (Epi::STAGE_HOOK) epi.stage_end();
-    } else {
-      ++kc;
-      __syncthreads();
-    }
-  }
-  epi.finish();
-}
-
-// ============================================================================================
-// kloop_async_kernel: the fp32 path for rows that are 16-byte aligned (d % 4 == 0).  Same tiles, same
-// reduction order and same epilogues as kloop_kernel, but both operands of a K chunk go from global
-// memory straight into LDS (global_load_lds_dwordx4: no staging registers, no ds_write) while the
-// previous chunk is multiplied.
-//
-// LDS layout of a stage: 128 entity rows then 128 query rows, each 128 B = 8 pieces of 16 B; piece p
-// of row r sits in slot r*8 + (p ^ (r & 7)).  A direct-to-LDS load writes 64 consecutive slots per
-// wave, so the swizzle is applied on the global side (which piece a lane fetches); a fragment read
-// (ds_read_b128 of piece 2*kb + hf of rows c..c+7 at a time) then covers all 32 banks once.
-// ============================================================================================
-constexpr int KA_PART_BYTES = KLOOP_TILE_ROWS * KLOOP_KC * 4;  // 16 KB: one operand of one stage
-constexpr int KA_STAGE_BYTES = 2 * KA_PART_BYTES;
-
-template <template <int> class EpiT>
-__global__ void __launch_bounds__(256, 2) kloop_async_kernel(ContractArgs a, typename EpiT<KLOOP_NQT>::Args ea) {
-  using Epi = EpiT<KLOOP_NQT>;
-  static_assert(KLOOP_TILE_ROWS == 128 && KLOOP_WG_QUERIES == 128 && KLOOP_KC == 32, "stage layout");
-  __shared__ __attribute__((aligned(1024))) unsigned char lds[2 * KA_STAGE_BYTES];
-
-  int qg;
-  int64_t chunk;
-  if (!decompose_wg(a, qg, chunk)) return;
-  const int tid = threadIdx.x, lane = tid & 63, c = lane & 31, hf = lane >> 5;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int we = wave >> 1, wq = wave & 1;
-  const int d = a.d;
-  const int64_t q_base = (int64_t)qg * KLOOP_WG_QUERIES;
-  const int64_t q0 = q_base + 64 * wq;
-  Epi epi;
-  epi.init(ea, q0, c, hf, a.B);
-  __shared__ typename Epi::Shared epi_sh;
-  epi.bind(&epi_sh);
-
-  const int64_t r0 = a.e_begin + chunk * a.chunk_rows;
-  const int64_t r1 = (r0 + a.chunk_rows < a.e_end) ? r0 + a.chunk_rows : a.e_end;
-  const int nkc = (d + KLOOP_KC - 1) / KLOOP_KC;
-  const int n_et = (int)((r1 - r0 + KLOOP_TILE_ROWS - 1) / KLOOP_TILE_ROWS);
-  const int n_it = n_et * nkc;
-  const float* Ef = (const float*)a.E;
-
-  // this lane's share of a stage: load instruction j covers rows lrow + 32 j of each operand, always the
-  // same swizzled piece (32 is a multiple of 8)
-  const int lrow = wave * 8 + (lane >> 3);
-  const int lk = ((lane & 7) ^ (lane >> 3)) * 4;  // float offset of the piece inside the K chunk
-  // query rows of this lane (fixed for the whole kernel); rows past B repeat the last query
-  const float* qsrc[4];
-#pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    int64_t q = q_base + lrow + 32 * j;
-    q = (q < a.B) ? q : a.B - 1;
-    qsrc[j] = a.Q + q * d + lk;
-  }
-  auto stage_issue = [&](int it, int buf) {
-    const int et = it / nkc, kc = it - et * nkc;
-    const int64_t et0 = r0 + (int64_t)et * KLOOP_TILE_ROWS;
-    const int k0 = kc * KLOOP_KC;
-    unsigned char* dst = lds + buf * KA_STAGE_BYTES + wave * 1024;
-    if (k0 + lk < d) {
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        int64_t g = et0 + lrow + 32 * j;
-        g = (g < r1) ? g : r1 - 1;  // padding rows repeat the last valid row; the epilogue ignores them
-        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(Ef + g * d + k0 + lk),
-                                         (__attribute__((address_space(3))) void*)(dst + j * 4096), 16, 0, 0);
-      }
-#pragma unroll
-      for (int j = 0; j < 4; ++j)
-        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(qsrc[j] + k0),
-                                         (__attribute__((address_space(3))) void*)(dst + KA_PART_BYTES + j * 4096), 16,
-                                         0, 0);
-    } else {  // past the end of the rows (last chunk when d % 32 != 0): the piece is zero
-      const f32x4 z = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        *(f32x4*)(dst + j * 4096 + lane * 16) = z;
-        *(f32x4*)(dst + KA_PART_BYTES + j * 4096 + lane * 16) = z;
-      }
-    }
-  };
-
-  // fragment offsets of this lane inside an operand part (row c of tile 0)
-  int foff[KLOOP_KC / 8];
-#pragma unroll
-  for (int kb = 0; kb < KLOOP_KC / 8; ++kb) foff[kb] = c * 128 + (((2 * kb + hf) ^ (c & 7)) << 4);
-
-  f32x16 acc[2][2];
-#pragma unroll
-  for (int te = 0; te < 2; ++te)
-#pragma unroll
-    for (int tq = 0; tq < 2; ++tq)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) acc[te][tq][i] = 0.f;
-
-  if (n_it > 0) stage_issue(0, 0);
-  int kc = 0;
-  int64_t et0 = r0;
-  for (int it = 0; it < n_it; ++it) {
-    const int buf = it & 1;
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();  // stage `it` has landed for every wave; everyone is done reading the other buffer
-    if (Epi::STAGE_HOOK) epi.stage_end();
-#ifndef KGE_DBG_NO_GLOBAL
-    if (it + 1 < n_it) stage_issue(it + 1, buf ^ 1);
-#endif
-    const unsigned char* be = lds + buf * KA_STAGE_BYTES + (64 * we) * 128;
-    const unsigned char* bq = lds + buf * KA_STAGE_BYTES + KA_PART_BYTES + (64 * wq) * 128;
-    const int k_left = d - kc * KLOOP_KC;  // the last chunk of a row may hold fewer than 4 blocks of 8
-#pragma unroll
-    for (int kb = 0; kb < KLOOP_KC / 8; ++kb) {
-      if (kb * 8 >= k_left) break;  // blocks of zeros add nothing to any score
-      f32x4 fe[2], fq[2];
-#pragma unroll
-      for (int t = 0; t < 2; ++t) {
-        fe[t] = *(const f32x4*)(be + t * 4096 + foff[kb]);
-        fq[t] = *(const f32x4*)(bq + t * 4096 + foff[kb]);
-      }
-#pragma unroll
-      for (int j = 0; j < 4; ++j)
-#pragma unroll
-        for (int te = 0; te < 2; ++te)
-#pragma unroll
-          for (int tq = 0; tq < 2; ++tq)
-            acc[te][tq] = Epi::SWAP ? mfma_f32(fq[tq][j], fe[te][j], acc[te][tq])
-                                    : mfma_f32(fe[te][j], fq[tq][j], acc[te][tq]);
-    }
-    if (kc == nkc - 1) {  // this entity tile is complete
-      float sc16[16];
-#pragma unroll
-      for (int te = 0; te < 2; ++te) {
-        const int64_t e_base = et0 + 64 * we + 32 * te;
-        if (e_base < r1) {
-#pragma unroll
-          for (int tq = 0; tq < 2; ++tq) epi.template tile<false>(tq, acc[te][tq], sc16, 1.f, e_base, r1);
-        }
-#pragma unroll
-        for (int tq = 0; tq < 2; ++tq)
-#pragma unroll
-          for (int i = 0; i < 16; ++i) acc[te][tq][i] = 0.f;
-      }
-      kc = 0;
-      et0 += KLOOP_TILE_ROWS;
-    } else {
-      ++kc;
-    }
-  }
-  epi.finish();
-}
-
-// ============================================================================================
 // ksplit_kernel: fp32 tables on the bf16 MFMA (split3_bf16x8).  256 entities x 128 queries per
 // workgroup of 8 waves (each wave 64 x 64), K in chunks of 32.  Both operands are loaded as fp32 into
 // registers while the previous chunk is multiplied, split into their three bf16 parts and stored as
@@ -1632,21 +1267,15 @@ __global__ void __launch_bounds__(512, 2) ksplit_kernel(ContractArgs a, typename
 #pragma unroll
     for (int sl = 0; sl < 6; ++sl) {
       if (sl == 2) read_step(1);
-#ifndef KGE_DBG_NO_LDSWRITE
       store_pass(buf ^ 1, sl);
-#endif
-#ifndef KGE_DBG_NO_GLOBAL
       load_pass(sl);
-#endif
 #pragma unroll
       for (int m = 8 * sl; m < 8 * sl + 8; ++m) {
         const int ks = m / 24, p = (m % 24) / 4, te = (m >> 1) & 1, tq = m & 1;
         acc[te][tq] = Epi::SWAP ? mfma_bf16(fq[ks][SPLIT_B[p]][tq], fe[ks][SPLIT_A[p]][te], acc[te][tq])
                                 : mfma_bf16(fe[ks][SPLIT_A[p]][te], fq[ks][SPLIT_B[p]][tq], acc[te][tq]);
       }
-#if KGE_KS_SCHED
       __builtin_amdgcn_sched_barrier(0);
-#endif
     }
     load_end();
     if (kc == nkc - 1) {  // this entity tile is complete

@@ -39,7 +39,6 @@ __device__ __forceinline__ f32x16 chain_direct(const void* E, int d, int64_t e_r
   f32x16 acc;
 #pragma unroll
   for (int i = 0; i < 16; ++i) acc[i] = 0.f;
-#if KGE_F32_SPLIT
   if (EDT == KGE_F32) {
     // fp32 rows on the bf16 MFMA: both rows split into three bf16 parts, six products per K step of 16
     // (the order of ksplit_kernel).  Four K steps per trip: all sixteen loads are issued first.
@@ -100,42 +99,6 @@ __device__ __forceinline__ f32x16 chain_direct(const void* E, int d, int64_t e_r
       load_trip(ks0, fe, fq);
       mul_trip(ks0, fe, fq);
     }
-#else
-  if (EDT == KGE_F32) {
-    const float* Ef = (const float*)E;
-    const bool vec_ok = (d & 3) == 0;
-    const int nkb = (d + 7) >> 3;
-    // eight k-blocks per trip: all sixteen loads are issued before the first MFMA needs one
-    for (int kb0 = 0; kb0 < nkb; kb0 += 8) {
-      f32x4 fe[8], fq[8];
-#pragma unroll
-      for (int u = 0; u < 8; ++u) {
-        const int k = (kb0 + u) * 8 + 4 * hf;
-        fe[u] = f32x4{0.f, 0.f, 0.f, 0.f};
-        fq[u] = f32x4{0.f, 0.f, 0.f, 0.f};
-        if (vec_ok) {
-          if (k < d) {
-            if (e_row >= 0) fe[u] = *(const f32x4*)(Ef + e_row * d + k);
-            if (q_row >= 0) fq[u] = *(const f32x4*)(Q + q_row * d + k);
-          }
-        } else {
-#pragma unroll
-          for (int j = 0; j < 4; ++j)
-            if (k + j < d) {
-              if (e_row >= 0) fe[u][j] = Ef[e_row * d + k + j];
-              if (q_row >= 0) fq[u][j] = Q[q_row * d + k + j];
-            }
-        }
-      }
-#pragma unroll
-      for (int u = 0; u < 8; ++u) {
-        if (kb0 + u < nkb) {  // uniform: whole k-blocks past d are skipped (they would only add zeros)
-#pragma unroll
-          for (int j = 0; j < 4; ++j) acc = mfma_f32(fe[u][j], fq[u][j], acc);
-        }
-      }
-    }
-#endif
   } else {
     for (int s0 = 0; s0 < d; s0 += 128)  // eight K steps per trip (one trip for d <= 128)
 #pragma unroll
@@ -369,8 +332,11 @@ __global__ void __launch_bounds__(1024) plan_fix_kernel(const int64_t* csr_row, 
 
 // ---- take the filtered entities back out of the counters ------------------------------------
 // Work item = (group of queries sharing a filter row, slice of that row).  The slice's entity scores
-// are formed once (gathered rows, same MFMA chain as the main loop), then every query of the
-// group compares them with its own threshold.
+// are formed once per distinct query vector of the group (gathered rows, same MFMA chain as the main
+// loop), then every query holding that vector compares them with its own threshold.  Queries built from
+// the same (head, relation) pair share both the row and the vector, so a group normally takes one round;
+// a caller that hands one filter row to different query vectors gets one round per distinct vector
+// (vectors are compared bit for bit against the round's leader).
 constexpr int FIX_CAP = 2048;
 constexpr int FIX_ITEMS = 16;  // work items a workgroup resolves side by side
 template <int EDT>
@@ -382,6 +348,8 @@ __global__ void __launch_bounds__(256) filter_fix_kernel(ContractArgs a, FixPlan
   __shared__ float s_sc[FIX_CAP];
   __shared__ int32_t s_e[FIX_CAP];
   __shared__ int32_t s_cnt[3 * 256];
+  __shared__ unsigned char s_state[SORT_MAX];  // per member of a group: 0 = waiting, 1 = in this round, 2 = done
+  __shared__ int s_next;                       // first member still waiting after this round
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, c = lane & 31, hf = lane >> 5;
   const int n_work = plan.meta[0];
   const int64_t slice = plan.meta[1];
@@ -389,7 +357,7 @@ __global__ void __launch_bounds__(256) filter_fix_kernel(ContractArgs a, FixPlan
   // This workgroup's work items are w = blockIdx.x + k * gridDim.x.  Up to FIX_ITEMS of them at a time are
   // resolved by one thread each, side by side (group by binary search, then the group's row and extent),
   // so that their chains of dependent loads overlap instead of running once per item.
-  __shared__ int32_t it_i0[FIX_ITEMS], it_m[FIX_ITEMS], it_bq[FIX_ITEMS];
+  __shared__ int32_t it_i0[FIX_ITEMS], it_m[FIX_ITEMS];
   __shared__ int64_t it_z0[FIX_ITEMS], it_z1[FIX_ITEMS];
   for (int k0 = 0; blockIdx.x + (int64_t)k0 * gridDim.x < n_work; k0 += FIX_ITEMS) {
     __syncthreads();
@@ -409,7 +377,6 @@ __global__ void __launch_bounds__(256) filter_fix_kernel(ContractArgs a, FixPlan
         const int64_t z0 = L0 + z * slice;
         it_i0[tid] = i0;
         it_m[tid] = plan.gend[i0] - i0;
-        it_bq[tid] = (int32_t)(key & 0xffffffull);
         it_z0[tid] = z0;
         it_z1[tid] = (z0 + slice < L1) ? z0 + slice : L1;
       }
@@ -419,87 +386,134 @@ __global__ void __launch_bounds__(256) filter_fix_kernel(ContractArgs a, FixPlan
     const int i0 = it_i0[kk];
     const int m = it_m[kk];
     const int64_t z0 = it_z0[kk], z1 = it_z1[kk];
-    const int64_t bq = b0 + (int64_t)it_bq[kk];
     // threads per member in the compare phase: spread a small group over the whole workgroup
     int tpm = 1;
     while (tpm * 2 * m <= 256) tpm *= 2;
-    for (int64_t pass = z0; pass < z1; pass += FIX_CAP) {
-      const int n_here = (int)((z1 - pass < FIX_CAP) ? z1 - pass : FIX_CAP);
-      const int ntile = (n_here + 31) >> 5;
-      // two tiles per trip so that both row gathers are in flight before the first MFMA chain
-      for (int tile = wave; tile < ntile; tile += 8) {
-        const int j0 = tile * 32 + c, j1 = (tile + 4) * 32 + c;
-        const int32_t e0 = (j0 < n_here) ? col[pass + j0] : -1;
-        const int32_t e1 = (j1 < n_here) ? col[pass + j1] : -1;
-        const bool ok0 = e0 >= 0 && (int64_t)e0 < a.N, ok1 = e1 >= 0 && (int64_t)e1 < a.N;
-        const bool two = tile + 4 < ntile;  // uniform per wave
-        f32x16 acc0 = chain_direct<EDT>(a.E, a.d, ok0 ? (int64_t)e0 : -1, a.Q, bq, hf);
-        f32x16 acc1;
-        if (two) acc1 = chain_direct<EDT>(a.E, a.d, ok1 ? (int64_t)e1 : -1, a.Q, bq, hf);
-        if (c == 0) {
-#pragma unroll
-          for (int i = 0; i < 16; ++i) s_s[tile * 32 + row_of(i, hf)] = acc0[i];
-          if (two) {
-#pragma unroll
-            for (int i = 0; i < 16; ++i) s_s[(tile + 4) * 32 + row_of(i, hf)] = acc1[i];
-          }
-        }
-        if (hf == 0) {
-          s_e[j0] = ok0 ? e0 : -1;
-          s_sc[j0] = (EDT == KGE_I8 && ok0) ? a.scale[e0] : 1.f;
-          if (two) {
-            s_e[j1] = ok1 ? e1 : -1;
-            s_sc[j1] = (EDT == KGE_I8 && ok1) ? a.scale[e1] : 1.f;
-          }
-        }
-      }
-      __syncthreads();
-      // compare phase: `tpm` threads share one query; their partial counts meet in LDS so that each
-      // query receives ONE global atomic per counter (hundreds of same-address atomics serialise)
-      const int sub = tid % tpm, mslot = tid / tpm, mstep = 256 / tpm;
-      for (int mbase = 0; mbase < m; mbase += mstep) {
-        const int mi = mbase + mslot;
-        s_cnt[tid] = 0;
-        s_cnt[256 + tid] = 0;
-        s_cnt[512 + tid] = 0;
+    const int sub = tid % tpm, mslot = tid / tpm, mstep = 256 / tpm;
+    if (m > 1) {
+      for (int i = tid; i < m; i += 256) s_state[i] = 0;
+    }
+    // one round per distinct query vector of the group; `lead` is the first member not yet served
+    for (int lead = 0; lead < m;) {
+      const int64_t bq = b0 + (int64_t)(plan.skey[i0 + lead] & 0xffffffull);
+      if (m > 1) {
+        // members whose query vector equals the leader's, bit for bit, join this round
         __syncthreads();
-        int64_t b = 0;
-        if (mi < m) {
-          b = b0 + (int64_t)(plan.skey[i0 + mi] & 0xffffffull);
-          const float th = thr[b];
-          const int64_t t = target[b];
-          int32_t g = 0, eq = 0, eql = 0;
-          for (int j = sub; j < n_here; j += tpm) {
-            const int32_t e = s_e[j];
-            float s = s_s[j];
-            if (EDT == KGE_I8) s *= s_sc[j];
-            if (e >= 0 && (int64_t)e != t) {
-              g += (s > th) ? 1 : 0;
-              if (s == th) {
-                eq += 1;
-                eql += ((int64_t)e < t) ? 1 : 0;
-              }
+        if (tid == 0) s_next = m;
+        __syncthreads();
+        const uint32_t* ql = (const uint32_t*)(a.Q + bq * a.d);
+        for (int mbase = lead; mbase < m; mbase += mstep) {
+          const int mi = mbase + mslot;
+          bool same = true;
+          if (mi < m && s_state[mi] == 0 && mi != lead) {
+            const uint32_t* qm = (const uint32_t*)(a.Q + (b0 + (int64_t)(plan.skey[i0 + mi] & 0xffffffull)) * a.d);
+            for (int k = sub; k < a.d; k += tpm) same = same && (qm[k] == ql[k]);
+          }
+          // all threads of a member agree before anyone writes its state
+          if (tpm > 1) {
+#pragma unroll
+            for (int o = 1; o < 64; o <<= 1)
+              if (o < tpm) same = __shfl_xor((int)same, o, 64) != 0 && same;
+          }
+          if (tpm > 64) {  // a member spread over several waves (m == 1 never comes here): meet in LDS
+            s_cnt[tid] = same ? 1 : 0;
+            __syncthreads();
+            bool all = true;
+            for (int t = (tid / tpm) * tpm; t < (tid / tpm) * tpm + tpm; t += 64) all = all && s_cnt[t] != 0;
+            same = all;
+            __syncthreads();
+          }
+          if (mi < m && sub == 0 && s_state[mi] == 0) {
+            if (same) s_state[mi] = 1;
+            else atomicMin(&s_next, mi);
+          }
+        }
+        __syncthreads();
+      }
+      for (int64_t pass = z0; pass < z1; pass += FIX_CAP) {
+        const int n_here = (int)((z1 - pass < FIX_CAP) ? z1 - pass : FIX_CAP);
+        const int ntile = (n_here + 31) >> 5;
+        // two tiles per trip so that both row gathers are in flight before the first MFMA chain
+        for (int tile = wave; tile < ntile; tile += 8) {
+          const int j0 = tile * 32 + c, j1 = (tile + 4) * 32 + c;
+          const int32_t e0 = (j0 < n_here) ? col[pass + j0] : -1;
+          const int32_t e1 = (j1 < n_here) ? col[pass + j1] : -1;
+          const bool ok0 = e0 >= 0 && (int64_t)e0 < a.N, ok1 = e1 >= 0 && (int64_t)e1 < a.N;
+          const bool two = tile + 4 < ntile;  // uniform per wave
+          f32x16 acc0 = chain_direct<EDT>(a.E, a.d, ok0 ? (int64_t)e0 : -1, a.Q, bq, hf);
+          f32x16 acc1;
+          if (two) acc1 = chain_direct<EDT>(a.E, a.d, ok1 ? (int64_t)e1 : -1, a.Q, bq, hf);
+          if (c == 0) {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) s_s[tile * 32 + row_of(i, hf)] = acc0[i];
+            if (two) {
+#pragma unroll
+              for (int i = 0; i < 16; ++i) s_s[(tile + 4) * 32 + row_of(i, hf)] = acc1[i];
             }
           }
-          if (tpm == 1) {
-            s_cnt[mslot] = g;
-            s_cnt[256 + mslot] = eq;
-            s_cnt[512 + mslot] = eql;
-          } else {
-            if (g) atomicAdd(&s_cnt[mslot], g);
-            if (eq) atomicAdd(&s_cnt[256 + mslot], eq);
-            if (eql) atomicAdd(&s_cnt[512 + mslot], eql);
+          if (hf == 0) {
+            s_e[j0] = ok0 ? e0 : -1;
+            s_sc[j0] = (EDT == KGE_I8 && ok0) ? a.scale[e0] : 1.f;
+            if (two) {
+              s_e[j1] = ok1 ? e1 : -1;
+              s_sc[j1] = (EDT == KGE_I8 && ok1) ? a.scale[e1] : 1.f;
+            }
           }
         }
         __syncthreads();
-        if (mi < m && sub == 0) {
-          const int32_t g = s_cnt[mslot], eq = s_cnt[256 + mslot], eql = s_cnt[512 + mslot];
-          if (g) atomicSub(&n_gt[b], g);
-          if (eq) atomicSub(&n_eq[b], eq);
-          if (eql) atomicSub(&n_eql[b], eql);
+        // compare phase: `tpm` threads share one query; their partial counts meet in LDS so that each
+        // query receives ONE global atomic per counter (hundreds of same-address atomics serialise)
+        for (int mbase = lead; mbase < m; mbase += mstep) {
+          const int mi = mbase + mslot;
+          const bool mine = mi < m && (m == 1 || s_state[mi] == 1);
+          s_cnt[tid] = 0;
+          s_cnt[256 + tid] = 0;
+          s_cnt[512 + tid] = 0;
+          __syncthreads();
+          int64_t b = 0;
+          if (mine) {
+            b = b0 + (int64_t)(plan.skey[i0 + mi] & 0xffffffull);
+            const float th = thr[b];
+            const int64_t t = target[b];
+            int32_t g = 0, eq = 0, eql = 0;
+            for (int j = sub; j < n_here; j += tpm) {
+              const int32_t e = s_e[j];
+              float s = s_s[j];
+              if (EDT == KGE_I8) s *= s_sc[j];
+              if (e >= 0 && (int64_t)e != t) {
+                g += (s > th) ? 1 : 0;
+                if (s == th) {
+                  eq += 1;
+                  eql += ((int64_t)e < t) ? 1 : 0;
+                }
+              }
+            }
+            if (tpm == 1) {
+              s_cnt[mslot] = g;
+              s_cnt[256 + mslot] = eq;
+              s_cnt[512 + mslot] = eql;
+            } else {
+              if (g) atomicAdd(&s_cnt[mslot], g);
+              if (eq) atomicAdd(&s_cnt[256 + mslot], eq);
+              if (eql) atomicAdd(&s_cnt[512 + mslot], eql);
+            }
+          }
+          __syncthreads();
+          if (mine && sub == 0) {
+            const int32_t g = s_cnt[mslot], eq = s_cnt[256 + mslot], eql = s_cnt[512 + mslot];
+            if (g) atomicSub(&n_gt[b], g);
+            if (eq) atomicSub(&n_eq[b], eq);
+            if (eql) atomicSub(&n_eql[b], eql);
+          }
+          __syncthreads();
         }
-        __syncthreads();
       }
+      if (m == 1) break;
+      // this round's members are done; the next round is led by the first member still waiting
+      __syncthreads();
+      for (int i = lead + tid; i < m; i += 256)
+        if (s_state[i] == 1) s_state[i] = 2;
+      lead = s_next;
     }
   }
   }
@@ -931,9 +945,8 @@ ContractArgs make_args(const float* Q, const void* E, int dtype, const float* sc
   a.ldq = a.lde = 0;
   a.k_split_len = 0;
   const bool fast_bf16 = (dtype == KGE_BF16 && d == 128), fast_i8 = (dtype == KGE_I8 && d == 128);
-  const int f32_wgq = KGE_F32_SPLIT ? KS_WG_QUERIES : KLOOP_WG_QUERIES;
   const bool wide_bf16 = (dtype == KGE_BF16 && d > 128);  // kchunk_bf16_kernel: the workgroup shape of the split kernel
-  const int wgq = (dtype == KGE_F32) ? f32_wgq : fast_bf16 ? QA_WG_QUERIES : fast_i8 ? I8_WG_QUERIES
+  const int wgq = (dtype == KGE_F32) ? KS_WG_QUERIES : fast_bf16 ? QA_WG_QUERIES : fast_i8 ? I8_WG_QUERIES
                   : wide_bf16 ? KS_WG_QUERIES : QREG_WG_QUERIES;
   a.n_qgroups = (int)((B + wgq - 1) / wgq);
   if (a.n_qgroups < 1) a.n_qgroups = 1;
@@ -955,9 +968,9 @@ ContractArgs make_args(const float* Q, const void* E, int dtype, const float* sc
   // non-persistent paths: one workgroup per (query group, chunk).  `resident` workgroups run at a time
   // (2 per CU, or 1 per CU for the 8-wave split kernel); choose the chunk length whose last round of
   // workgroups is fullest, preferring longer chunks (less per-workgroup set-up) among near-equal candidates.
-  const bool f32_split = (dtype == KGE_F32) && KGE_F32_SPLIT;
+  const bool f32_split = (dtype == KGE_F32);
   const bool big_tile = f32_split || wide_bf16;  // 8-wave workgroups of 256 entity rows, one per CU
-  const int tile = big_tile ? KS_TILE_ROWS : (dtype == KGE_F32) ? KLOOP_TILE_ROWS : QREG_STAGE_ROWS;
+  const int tile = big_tile ? KS_TILE_ROWS : QREG_STAGE_ROWS;
   const int max_chunk = (dtype == KGE_F32 || wide_bf16) ? 1024 : 2048;
   const int64_t resident = big_tile ? 256 : 512;
   int64_t best_chunk = tile;
@@ -992,7 +1005,7 @@ int launch_contract(int dtype, const ContractArgs& a, const EArgs& ea, hipStream
   const bool persistent = (dtype == KGE_BF16 && a.d == 128) || fast_i8;
   const int64_t nwg = persistent ? 8 * (int64_t)a.n_qgroups * a.n_lanes : contract_grid_wgs(a);
   KGE_REQUIRE(nwg <= 0x7fffffffLL, KGE_ERR_INVALID, "%s: grid of %lld workgroups too large", name, (long long)nwg);
-  const bool f32_split = (dtype == KGE_F32) && KGE_F32_SPLIT;
+  const bool f32_split = (dtype == KGE_F32);
   const bool wide_bf16 = (dtype == KGE_BF16 && a.d > 128);
   dim3 grid((unsigned)nwg), block(fast_i8 ? 64 * I8_WG_WAVES : persistent ? 64 * QA_WG_WAVES : (f32_split || wide_bf16) ? 512 : 256);
   hipEvent_t ev0 = nullptr, ev1 = nullptr;
@@ -1011,12 +1024,6 @@ int launch_contract(int dtype, const ContractArgs& a, const EArgs& ea, hipStream
     hipLaunchKernelGGL((ksplit_kernel<EpiT, true>), grid, block, 0, st, a, ea);
   else if (f32_split)
     hipLaunchKernelGGL((ksplit_kernel<EpiT, false>), grid, block, 0, st, a, ea);
-#if !KGE_F32_SPLIT  // the fp32-MFMA main loops are only built when the split path is switched off
-  else if (dtype == KGE_F32 && rows_aligned)
-    hipLaunchKernelGGL((kloop_async_kernel<EpiT>), grid, block, 0, st, a, ea);
-  else if (dtype == KGE_F32)
-    hipLaunchKernelGGL((kloop_kernel<EpiT>), grid, block, 0, st, a, ea);
-#endif
   else if (dtype == KGE_BF16 && a.d == 128)
     hipLaunchKernelGGL((qreg_async_kernel<EpiT>), grid, block, 0, st, a, ea);
   else if (wide_bf16)
@@ -1512,14 +1519,3 @@ extern "C" int kge_bce_multihot_backward(const float* Q, const float* bias, cons
   }
   return KGE_OK;
 }
-
-#ifdef KGE_DEBUG
-// Measurement-only: the contraction main loop with an (almost) empty epilogue.
-extern "C" int kge_debug_contract_null(const float* Q, const void* E, int dtype, const float* scale, int64_t B,
-                                       int64_t d, int64_t N, float* out, void* stream) {
-  clear_error();
-  ContractArgs a = make_args(Q, E, dtype, scale, B, d, N, 0, N);
-  NullArgs ea{out};
-  return launch_contract<NullEpi>(dtype, a, ea, (hipStream_t)stream, "kge_debug_contract_null");
-}
-#endif

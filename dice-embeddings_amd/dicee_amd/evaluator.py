@@ -1,8 +1,9 @@
 """Filtered link-prediction evaluation through the fused rank kernel.
 
-Mirrors dicee's ``Evaluator`` for the KvsAll entity-prediction route
-(dicee/evaluation/evaluator.py:114-198 routing, :363-392 ``eval_with_vs_all``, :394-438
-``evaluate_lp_k_vs_all``, :473-510 the rank loop) and its metric reduction
+Mirrors dicee's ``Evaluator`` for index-encoded (non byte-pair) models
+(dicee/evaluation/evaluator.py:114-198 routing, :246-272 ``eval_rank_of_head_and_tail_entity``, :363-392
+``eval_with_vs_all``, :394-438 ``evaluate_lp_k_vs_all``, :440-471 the relation-prediction loop, :473-510 the
+entity-prediction loop, :622-643 ``evaluate_lp``) and its metric reduction
 (dicee/evaluation/utils.py:73-132).  Where the reference scores a batch, masks it row by row in
 Python and sorts every row, this evaluator makes one fused kernel call per batch and receives three
 counters per query.
@@ -66,7 +67,12 @@ class Evaluator:
         self.args = args
         self.is_continual_training = is_continual_training
         self.er_vocab = None
-        self.csr = None
+        self.re_vocab = None
+        self.ee_vocab = None
+        self.csr = None          # (head, relation) -> tails: the entity-prediction filter
+        self.re_csr = None       # (relation, tail) -> heads: head direction of evaluate_lp
+        self.ee_csr = None       # (head, tail) -> relations: relation prediction
+        self._triples = None     # all splits, kept to build the other two vocabularies on demand
         self.num_entities = None
         self.num_relations = None
         self.report = {}
@@ -91,30 +97,80 @@ class Evaluator:
             parts = [np.asarray(s) for s in (dataset.train_set, getattr(dataset, "valid_set", None),
                                              getattr(dataset, "test_set", None)) if s is not None]
             triples = np.concatenate(parts, axis=0)
+            self._triples = triples
             if device is not None and torch.device(device).type == "cuda":
                 on_dev = torch.from_numpy(np.ascontiguousarray(triples.astype(np.int64))).to(device)
                 self.csr = FilterCSR.from_triples_gpu(on_dev, self.num_entities, self.num_relations)
             else:
                 self.csr = FilterCSR.from_triples(triples, self.num_relations)
 
-    def set_filter(self, csr_or_er_vocab, num_relations=None):
-        if isinstance(csr_or_er_vocab, FilterCSR):
-            self.csr = csr_or_er_vocab
+        # the other two vocabularies, when the dataset carries them (evaluator.py:83-96)
+        for attr, mine, mult in (("re_vocab", "re_csr", self.num_entities), ("ee_vocab", "ee_csr", self.num_entities)):
+            v = getattr(dataset, attr, None)
+            if v is not None and hasattr(v, "result"):
+                v = v.result()
+            if v is not None:
+                setattr(self, attr, v)
+                setattr(self, mine, FilterCSR.from_er_vocab(v, mult))
+
+    def set_filter(self, csr_or_vocab, num_relations=None, kind="er"):
+        """Install a filter: a ``FilterCSR`` or the reference's dict.  ``kind``: ``"er"`` (h, r) -> tails,
+        ``"re"`` (r, t) -> heads, ``"ee"`` (h, t) -> relations; ``num_relations`` is the multiplier of the
+        row key ``first * multiplier + second`` (the number of relations for ``"er"``, of entities otherwise)."""
+        attr = {"er": "csr", "re": "re_csr", "ee": "ee_csr"}[kind]
+        if isinstance(csr_or_vocab, FilterCSR):
+            setattr(self, attr, csr_or_vocab)
         else:
-            self.er_vocab = csr_or_er_vocab
-            self.csr = FilterCSR.from_er_vocab(csr_or_er_vocab, num_relations)
+            setattr(self, {"er": "er_vocab", "re": "re_vocab", "ee": "ee_vocab"}[kind], csr_or_vocab)
+            setattr(self, attr, FilterCSR.from_er_vocab(csr_or_vocab, num_relations))
         return self
+
+    def _other_vocab(self, kind, model):
+        """``re_csr`` / ``ee_csr``, built from the dataset's triples on first use when no vocabulary was given."""
+        attr = {"re": "re_csr", "ee": "ee_csr"}[kind]
+        csr = getattr(self, attr)
+        if csr is None:
+            if self._triples is None:
+                raise AssertionError(f"self.{kind}_vocab cannot be None")
+            dev = model.entity_embeddings.weight.device
+            N, R = model.num_entities, model.num_relations
+            if dev.type == "cuda":
+                on_dev = torch.from_numpy(np.ascontiguousarray(self._triples.astype(np.int64))).to(dev)
+                csr = FilterCSR.from_triples_gpu(on_dev, N, R, kind=kind)
+            else:
+                cols = {"re": [1, 2, 0], "ee": [0, 2, 1]}[kind]
+                csr = FilterCSR.from_triples(np.asarray(self._triples)[:, cols], N)
+            setattr(self, attr, csr)
+        return csr
 
     # ------------------------------------------------------------------ evaluation
     def eval(self, dataset, trained_model, form_of_labelling, during_training=False):
+        """Routing of Evaluator.eval (evaluator.py:114-198) for index-encoded models: ``NegSample`` ranks heads and
+        tails (``evaluate_lp``), the ``*vsAll`` / ``*vsSample`` techniques rank tails (or relations) with KvsAll
+        scoring.  Byte-pair-encoded models are outside the accelerated path."""
         self.during_training = during_training
+        if self.args.eval_model is None:
+            return None
+        if getattr(self.args, "byte_pair_encoding", False):
+            raise NotImplementedError("byte-pair-encoded models are outside the accelerated path")
+        if isinstance(self.args.eval_model, bool):
+            print("Wrong input:RESET")
+            self.args.eval_model = "train_val_test"
+        if "constraint" in self.args.eval_model:
+            # the reference's branch (evaluator.py:498-499) indexes range_constraints_per_rel, which is never set
+            raise NotImplementedError("'constraint' in eval_model: range constraints are not part of this path")
         if self.csr is None:
             self.vocab_preparation(dataset, device=trained_model.entity_embeddings.weight.device)
-        if self.args.scoring_technique not in ["AllvsAll", "KvsAll", "1vsSample", "KvsSample", "1vsAll"]:
+        if getattr(self.args, "num_folds_for_cv", 0) and self.args.num_folds_for_cv > 1:
+            return None
+        splits = dict(train_set=dataset.train_set, valid_set=getattr(dataset, "valid_set", None),
+                      test_set=getattr(dataset, "test_set", None), trained_model=trained_model)
+        if self.args.scoring_technique == "NegSample":
+            self.eval_rank_of_head_and_tail_entity(**splits)
+        elif self.args.scoring_technique in ["AllvsAll", "KvsAll", "1vsSample", "KvsSample", "1vsAll"]:
+            self.eval_with_vs_all(form_of_labelling=form_of_labelling, **splits)
+        else:
             raise ValueError(f"Invalid scoring technique: {self.args.scoring_technique}")
-        self.eval_with_vs_all(train_set=dataset.train_set, valid_set=getattr(dataset, "valid_set", None),
-                              test_set=getattr(dataset, "test_set", None), trained_model=trained_model,
-                              form_of_labelling=form_of_labelling)
         path = getattr(self.args, "full_storage_path", None)
         if not self.during_training and path:
             with open(os.path.join(path, "eval_report.json"), "w") as f:
@@ -136,15 +192,37 @@ class Evaluator:
                 trained_model, test_set, f"Evaluate {trained_model.name} on Test set",
                 form_of_labelling=form_of_labelling)
 
+    def eval_rank_of_head_and_tail_entity(self, *, train_set, valid_set=None, test_set=None, trained_model):
+        """Evaluation of models trained with negative sampling (evaluator.py:246-272): heads and tails."""
+        em = self.args.eval_model or ""
+        if "train" in em:
+            self.report["Train"] = self.evaluate_lp(trained_model, train_set,
+                                                    f"Evaluate {trained_model.name} on Train set")
+        if "val" in em and valid_set is not None:
+            self.report["Val"] = self.evaluate_lp(trained_model, valid_set,
+                                                  f"Evaluate {trained_model.name} of Validation set")
+        if test_set is not None and "test" in em:
+            self.report["Test"] = self.evaluate_lp(trained_model, test_set,
+                                                   f"Evaluate {trained_model.name} of Test set")
+
+    def evaluate_lp(self, model, triple_idx, info):
+        """evaluator.py:622-643: both directions through ``link_prediction.evaluate_lp``."""
+        from .link_prediction import evaluate_lp
+        assert self.csr is not None, "self.er_vocab cannot be None"
+        return evaluate_lp(model, triple_idx, num_entities=self.num_entities, er_vocab=self.csr,
+                           re_vocab=self._other_vocab("re", model), info=None if self.during_training else info,
+                           tie=self.tie)
+
     def evaluate_lp_k_vs_all(self, model, triple_idx, info=None, form_of_labelling=None):
         """Filtered link prediction with KvsAll scoring -> ``{'H@1','H@3','H@10','MRR'}``."""
-        if form_of_labelling == "RelationPrediction":
-            raise NotImplementedError("relation prediction is outside the accelerated path")
         model.eval()
         num_triples = len(triple_idx)
         if info and not self.during_training:
             print(info + ":", end=" ")
-        ranks = self._evaluate_entity_prediction(model, triple_idx, num_triples)
+        if form_of_labelling == "RelationPrediction":
+            ranks = self._evaluate_relation_prediction(model, triple_idx, num_triples)
+        else:
+            ranks = self._evaluate_entity_prediction(model, triple_idx, num_triples)
         assert len(triple_idx) == len(ranks) == num_triples
         hits = create_hits_dict()
         for level in ALL_HITS_RANGE:
@@ -155,6 +233,40 @@ class Evaluator:
             print(info)
             print(results)
         return results
+
+    def _evaluate_relation_prediction(self, model, triple_idx, num_triples):
+        """Ranks (numpy int64 [n]) as the reference's relation-prediction loop produces them
+        (evaluator.py:440-471), literally: ``forward_k_vs_all`` receives the (head, TAIL) pairs, so the tail id
+        is looked up in the relation table (an ``IndexError`` when it is not below the number of relations, as
+        the embedding lookup raises there), the resulting scores of all ENTITIES are masked at the columns
+        listed in ``ee_vocab[(head, tail)]`` (relation ids used as column numbers) and the rank is that of
+        column ``relation`` among all entity columns."""
+        triple_idx = np.asarray(triple_idx)
+        if triple_idx.ndim != 2 or triple_idx.shape[1] != 3:
+            raise ValueError("triple_idx must have shape [n, 3]")
+        N, R = model.num_entities, model.num_relations
+        if num_triples:
+            if triple_idx[:, 0].min() < 0 or triple_idx[:, 0].max() >= N:
+                raise IndexError("index out of range in self")          # entity_embeddings(head)
+            if triple_idx[:, 2].min() < 0 or triple_idx[:, 2].max() >= R:
+                raise IndexError("index out of range in self")          # relation_embeddings(tail)
+            if triple_idx[:, 1].min() < 0 or triple_idx[:, 1].max() >= N:
+                raise IndexError(f"index {int(triple_idx[:, 1].max())} is out of bounds for dimension 1 with size {N}")
+        dev = model.entity_embeddings.weight.device
+        csr = self._other_vocab("ee", model)
+        if csr.device is None or csr.device != dev:
+            csr.to(dev)
+        all_trip = torch.from_numpy(np.ascontiguousarray(triple_idx.astype(np.int64))).to(dev)
+        out = torch.empty((num_triples,), dtype=torch.int64, device=dev)
+        bs = int(self.args.batch_size)
+        with torch.no_grad():
+            for i in range(0, num_triples, bs):
+                batch = all_trip[i:i + bs]
+                x = batch[:, [0, 2]].contiguous()
+                r = batch[:, 1].contiguous()
+                c = model.rank_filtered(x, r, csr)
+                out[i:i + bs] = ranks_from_counts(c["n_greater"], c["n_equal"], c["n_equal_lower"], self.tie)
+        return out.cpu().numpy()
 
     def _evaluate_entity_prediction(self, model, triple_idx, num_triples):
         """Ranks (numpy int64 [n]) of the true tails; one fused kernel call per batch of

@@ -13,6 +13,53 @@ from oracle import kge_oracle as ko
 pytestmark = pytest.mark.gpu
 
 
+def test_c2_complex_filtered_mrr_eval_at_full_size():
+    """C2 as BASELINE.json states it: ComplEx, 14,541 entities, d = 200 fp32, 272k Zipf triples, 20k eval queries in
+    batches of 1024 (the last holds 544) through the Evaluator (dicee/evaluation/evaluator.py:473-510).  Every rank
+    lies inside the fp64 oracle's tolerance interval and equals the oracle's rank wherever that interval is one
+    point; the counters of sampled batches are bit-exact against the library's own materialised scores."""
+    from types import SimpleNamespace
+    from dicee_amd import synthetic
+    from dicee_amd.evaluator import Evaluator
+    cfg = synthetic.make_config("c2")
+    assert (cfg.N, cfg.R, cfg.d, cfg.B, len(cfg.queries), len(cfg.triples)) == (14541, 237, 200, 1024, 20000, 272000)
+    model = synthetic.make_model(cfg, torch.device("cuda:0"))
+    ev = Evaluator(SimpleNamespace(batch_size=cfg.B, eval_model="test", scoring_technique="KvsAll",
+                                   full_storage_path=None))
+    ev.set_filter(cfg.csr)
+    res = ev.evaluate_lp_k_vs_all(model, cfg.queries)
+    ranks = ev.last_ranks
+    assert ranks.shape == (20000,)
+    exact = inside = 0
+    for i in range(0, len(cfg.queries), cfg.B):
+        q = cfg.queries[i:i + cfg.B]
+        S = ko.k_vs_all_scores("ComplEx", cfg.E, cfg.Rel, q[:, :2])          # fp64 [<=1024, 14541]
+        rms = np.sqrt((S ** 2).mean(axis=1))
+        for j, (h, r, t) in enumerate(q):
+            filt = cfg.csr.tails(int(h), int(r))
+            tol = 1e-5 * max(abs(S[j, t]), rms[j])
+            lo, hi = ko.rank_interval_with_tolerance(S[j], int(t), filt, tol)
+            inside += lo <= ranks[i + j] <= hi
+            exact += lo == hi
+    assert inside == len(cfg.queries)
+    assert exact > 0.8 * len(cfg.queries)            # the interval is one point (the rank is pinned exactly) for most
+    want = ko.metrics_from_ranks(ranks)
+    for key in ("H@1", "H@3", "H@10", "MRR"):
+        assert res[key] == pytest.approx(want[key], rel=1e-12)
+    # counters bit-exact against the library's own scores: first batch, last (544-query) batch
+    cfg.csr.to("cuda")
+    for i in (0, 19 * cfg.B):
+        q = torch.from_numpy(cfg.queries[i:i + cfg.B].copy()).cuda()
+        x, t = q[:, :2].contiguous(), q[:, 2].contiguous()
+        c = model.rank_filtered(x, t, cfg.csr)
+        S = model(x).cpu().numpy()
+        tt = t.cpu().numpy()
+        for j in range(len(tt)):
+            filt = cfg.csr.tails(int(x[j, 0]), int(x[j, 1]))
+            g, e, el = ko.filtered_rank_counts(S[j], int(tt[j]), filt)
+            assert (g, e, el) == (int(c["n_greater"][j]), int(c["n_equal"][j]), int(c["n_equal_lower"][j]))
+
+
 @pytest.fixture(scope="module")
 def c4():
     from dicee_amd import synthetic

@@ -248,6 +248,101 @@ def test_rank_all_scores_equal(ops):
     np.testing.assert_array_equal(out["n_equal_lower"].cpu().numpy(), np.arange(B) * 50)
 
 
+def test_rank_one_filter_row_shared_by_different_query_vectors(ops, FilterCSR):
+    """The ABI takes Q and csr_row separately: queries may share a filter row without sharing a query vector
+    (a range constraint per relation, a custom mask).  Each query must be corrected with ITS OWN scores of the
+    filtered entities.  Rows: one long row shared by many distinct vectors, rows shared by a few, groups that mix
+    repeated and distinct vectors, -1 (no filter)."""
+    rng = np.random.default_rng(77)
+    N, d, B = 6000, 48, 900
+    E = (rng.standard_normal((N, d)) * 0.1).astype(np.float32)
+    Qh = (rng.standard_normal((B, d)) * 0.1).astype(np.float32)
+    Qh[100:160] = Qh[100]                      # 60 queries with one vector ...
+    Qh[160:170] = Qh[160]                      # ... and 10 with another, all on one row below
+    Qh[170, 3] = 0.0
+    Qh[171] = Qh[170]
+    Qh[171, 3] = -0.0                          # equal values, different bits: its own round, same counts
+    lens = [3000, 40, 7, 1, 0, 300, 2100]
+    row_ptr = np.concatenate([[0], np.cumsum(lens)]).astype(np.int64)
+    col = np.concatenate([np.sort(rng.choice(N, size=n, replace=False)) for n in lens]).astype(np.int32)
+    csr_row = rng.integers(-1, len(lens), B).astype(np.int64)
+    csr_row[:60] = 0                           # 60 distinct vectors on the long row
+    csr_row[100:172] = 6                       # the mixed group
+    targets = rng.integers(0, N, B).astype(np.int64)
+    targets[:20] = col[:20]                    # targets inside their own filter row stay unfiltered
+    Eg, Qg = dev(torch.from_numpy(E)), dev(torch.from_numpy(Qh))
+    out = ops.rank_filtered(Qg, None, Eg, None, dev(torch.from_numpy(targets)), dev(torch.from_numpy(csr_row)),
+                            dev(torch.from_numpy(row_ptr)), dev(torch.from_numpy(col)))
+    S_raw = ops.scores(Qg, None, Eg, None).cpu().numpy()
+    filters = [col[row_ptr[r]:row_ptr[r + 1]] if r >= 0 else None for r in csr_row]
+    g, t, tl = _expected_counts(S_raw, targets, filters)
+    np.testing.assert_array_equal(out["n_greater"].cpu().numpy(), g)
+    np.testing.assert_array_equal(out["n_equal"].cpu().numpy(), t)
+    np.testing.assert_array_equal(out["n_equal_lower"].cpu().numpy(), tl)
+
+
+@pytest.mark.parametrize("storage,d,N", [("bf16", 64, 4097), ("fp32", 1, 1000), ("fp32", 32, 3001), ("bf16", 128, 5000),
+                                         ("int8", 128, 2500), ("bf16", 256, 1300)])
+def test_rank_partial_last_query_group_with_a_bias(ops, FilterCSR, storage, d, N):
+    """B = 2500 leaves the last query group of every main loop partly filled (256-, 512- and 128-query groups), and
+    the per-query bias is non-zero: ranks compare un-biased scores, target_score carries the bias."""
+    rng = np.random.default_rng(1234 + d)
+    R, B = 7, 2500
+    E, Rel = random_tables(rng, N, R, d)
+    hr = random_hr(rng, N, R, B)
+    Et, sc, Rt, Ev, Rv = stored_tables(E, Rel, storage)
+    Eg, scg = dev(Et), dev(sc)
+    hr_g = dev(torch.from_numpy(hr))
+    Q, _ = ops.build_query("DistMult", Eg, dev(Rt), hr_g, ent_scale=scg)
+    bias = dev(torch.from_numpy((rng.standard_normal(B) * 3.0).astype(np.float32)))
+    targets = rng.integers(0, N, B).astype(np.int64)
+    er = random_csr(rng, hr, targets, N, R, max_len=4)
+    csr = FilterCSR.from_er_vocab(er, R, device="cuda")
+    out = ops.rank_filtered(Q, bias, Eg, scg, dev(torch.from_numpy(targets)), csr.rows_for(hr_g), csr.row_ptr, csr.col)
+    S_raw = ops.scores(Q, None, Eg, scg).cpu().numpy()
+    filters = [er[(int(h), int(r))] for h, r in hr]
+    g, t, tl = _expected_counts(S_raw, targets, filters)
+    np.testing.assert_array_equal(out["n_greater"].cpu().numpy(), g)
+    np.testing.assert_array_equal(out["n_equal"].cpu().numpy(), t)
+    np.testing.assert_array_equal(out["n_equal_lower"].cpu().numpy(), tl)
+    want_ts = (S_raw[np.arange(B), targets] + bias.cpu().numpy()).astype(np.float32)
+    np.testing.assert_array_equal(out["target_score"].cpu().numpy(), want_ts)
+    # the biased matrix: same bits as raw + bias, rounded once
+    S_b = ops.scores(Q, bias, Eg, scg).cpu().numpy()
+    np.testing.assert_array_equal(S_b, (S_raw + bias.cpu().numpy()[:, None]).astype(np.float32))
+
+
+@pytest.mark.parametrize("sq,se", [(1e-6, 1e-6), (1e6, 1e6), (1e-12, 1e-3), (1e-15, 1e-15), (3e17, 3e17), (1e-30, 1.0)])
+def test_fp32_scores_hold_their_accuracy_across_magnitudes(ops, sq, se):
+    """fp32 tables run as three bf16 parts per operand.  Inside the documented range (every product q*e of a score
+    at least 2^-100 in magnitude and every value's bf16 rounding finite) the scores stay within 1e-5 of fp64."""
+    rng = np.random.default_rng(5)
+    N, d, B = 700, 200, 130
+    E = (rng.standard_normal((N, d)) * se).astype(np.float32)
+    Qh = (rng.standard_normal((B, d)) * sq).astype(np.float32)
+    S = ops.scores(dev(torch.from_numpy(Qh)), None, dev(torch.from_numpy(E)), None).cpu().numpy()
+    ref = Qh.astype(np.float64) @ E.astype(np.float64).T
+    ok, worst = score_close(S, ref, 1e-5)
+    assert ok, worst
+
+
+def test_fp32_scores_below_the_documented_range_degrade_gracefully(ops):
+    """Products near the bottom of fp32's range (|q*e| ~ 1e-36): the low-order parts underflow, the leading bf16
+    products remain, so the result is still a bf16-grade score (2e-2), never garbage; products that underflow fp32
+    altogether give exact zeros, as fp32 arithmetic itself would."""
+    rng = np.random.default_rng(6)
+    N, d, B = 300, 64, 40
+    E = (rng.standard_normal((N, d)) * 1e-18).astype(np.float32)
+    Qh = (rng.standard_normal((B, d)) * 1e-18).astype(np.float32)
+    S = ops.scores(dev(torch.from_numpy(Qh)), None, dev(torch.from_numpy(E)), None).cpu().numpy()
+    ref = Qh.astype(np.float64) @ E.astype(np.float64).T
+    ok, worst = score_close(S, ref, 2e-2)
+    assert ok, worst
+    tiny = (rng.standard_normal((N, d)) * 1e-30).astype(np.float32)
+    S0 = ops.scores(dev(torch.from_numpy(tiny[:B].copy())), None, dev(torch.from_numpy(tiny)), None).cpu().numpy()
+    assert np.all(S0 == 0.0)
+
+
 TOPK_CASES = [
     ("DistMult", 135, 46, 32, 64, "fp32", 10),
     ("ComplEx", 20011, 11, 200, 130, "fp32", 100),
