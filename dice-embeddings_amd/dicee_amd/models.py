@@ -6,7 +6,9 @@ Parameter names follow dicee so that a dicee ``model.pt`` state_dict loads uncha
 dicee/models/clifford.py:4-28.
 
 Only the inference-time semantics of the path are implemented: dropout is the identity
-(base_model.py:149-151 in eval mode) and BatchNorm1d uses its running statistics.
+(base_model.py:149-151 in eval mode) and BatchNorm1d uses its running statistics.  A model in training mode
+whose dropout rates are not zero refuses to score (the reference would drop elements there) instead of
+silently scoring without dropout.
 """
 import torch
 
@@ -35,6 +37,7 @@ class BaseKGE(torch.nn.Module):
         self.num_entities = int(args["num_entities"])
         self.num_relations = int(args["num_relations"])
         self.input_dropout_rate = float(args.get("input_dropout_rate", 0.0) or 0.0)
+        self.hidden_dropout_rate = float(args.get("hidden_dropout_rate", 0.0) or 0.0)
         self.loss = torch.nn.BCEWithLogitsLoss()
         self.normalize_head_entity_embeddings = IdentityClass()
         self.normalize_relation_embeddings = IdentityClass()
@@ -54,6 +57,7 @@ class BaseKGE(torch.nn.Module):
         self._table = None       # quantised / bf16 copy of the entity table
         self._scale = None
         self._rel_table = None
+        self._snap_key = None    # identity and version of the parameters the bf16 / int8 copies were taken from
 
     # ------------------------------------------------------------------ storage
     def set_entity_storage(self, kind="fp32"):
@@ -78,16 +82,38 @@ class BaseKGE(torch.nn.Module):
         else:
             raise ValueError(kind)
         self._storage = kind
+        self._snap_key = self._parameter_key()
         return self
+
+    def _parameter_key(self):
+        we, wr = self.entity_embeddings.weight, self.relation_embeddings.weight
+        return (we.data_ptr(), we._version, wr.data_ptr(), wr._version)
+
+    def _refresh_storage(self):
+        """The bf16 / int8 tables are copies: take them again when the parameters have changed since (an
+        optimizer step, ``load_state_dict``, a move to another device), so that scoring never reads stale weights."""
+        if self._storage != "fp32" and self._snap_key != self._parameter_key():
+            self.set_entity_storage(self._storage)
 
     def table(self):
         """(entity table the kernels read, per-row scale or None)."""
+        self._refresh_storage()
         if self._table is not None:
             return self._table, self._scale
         return self.entity_embeddings.weight.detach(), None
 
     def _rel(self):
+        self._refresh_storage()
         return self._rel_table if self._rel_table is not None else self.relation_embeddings.weight.detach()
+
+    def _refuse_dropout_in_training(self):
+        """The reference applies Dropout to the gathered rows (base_model.py:381-383) and to the interaction
+        (e.g. real.py:32) whenever the module is in training mode; this path has no dropout."""
+        if self.training and (self.input_dropout_rate > 0.0 or self.hidden_dropout_rate > 0.0):
+            raise NotImplementedError(
+                f"{self.name} is in training mode with input_dropout_rate={self.input_dropout_rate}, "
+                f"hidden_dropout_rate={self.hidden_dropout_rate}: the accelerated path has no dropout; "
+                "call model.eval() or set the rates to zero")
 
     # ------------------------------------------------------------------ query construction
     def _norm_params(self):
@@ -108,6 +134,7 @@ class BaseKGE(torch.nn.Module):
         (get_head_relation_representation, base_model.py:377-384, then the model's elementwise part).
         ``heads=True``: ``x`` holds (relation, tail) pairs and ``Q @ E^T`` scores every entity as the head of
         (x, r, t): what ``forward_triples`` gives triple by triple (base_model.py:346-362)."""
+        self._refuse_dropout_in_training()
         E, scale = self.table()
         x = x.to(device=E.device, dtype=torch.int64).contiguous()
         return ops.build_query(self.name if self.name != "CKeci" else "Keci", E, self._rel(), x, ent_scale=scale,
@@ -156,6 +183,7 @@ class BaseKGE(torch.nn.Module):
 
     def k_vs_all_score(self, emb_h, emb_r, emb_E):
         """Scores from already gathered rows: [B,d],[B,d],[N,d] -> [B,N]."""
+        self._refuse_dropout_in_training()
         B = emb_h.shape[0]
         idx = torch.arange(B, device=emb_h.device, dtype=torch.int64)
         hr = torch.stack([idx, idx], dim=1).contiguous()

@@ -19,6 +19,20 @@ def _require_gpu(*tensors):
             raise ValueError("dicee_amd ops need contiguous tensors")
 
 
+def _check_qe(Q, E, scale=None, bias=None):
+    """Shapes the kernels rely on: Q [B,d] fp32 and E [N,d] share d; bias [B]; scale [N]."""
+    if Q.dim() != 2 or E.dim() != 2 or Q.shape[1] != E.shape[1]:
+        raise ValueError(f"Q {tuple(Q.shape)} and E {tuple(E.shape)} must be [B,d] and [N,d] with the same d")
+    if Q.dtype != torch.float32:
+        raise TypeError("Q must be float32")
+    if bias is not None and (bias.dtype != torch.float32 or bias.numel() != Q.shape[0]):
+        raise ValueError("bias must be float32 [B]")
+    if scale is not None and (scale.dtype != torch.float32 or scale.numel() != E.shape[0]):
+        raise ValueError("scale must be float32 [N]")
+    if E.dtype == torch.int8 and scale is None:
+        raise ValueError("int8 tables need per-row scales")
+
+
 def _ptr(t):
     return None if t is None else ctypes.c_void_p(t.data_ptr())
 
@@ -100,6 +114,7 @@ def scores(Q, bias, E, scale=None, out=None):
     """Materialised [B,N] fp32 scores."""
     lib = _lib.load()
     _require_gpu(Q, bias, E, scale)
+    _check_qe(Q, E, scale, bias)
     B, d = Q.shape
     N = E.shape[0]
     if out is None:
@@ -115,6 +130,7 @@ def triple_scores(Q, bias, E, scale, entity):
     """out[b] = Q[b] . E[entity[b]] (* scale) + bias[b]: the score of one given entity per query."""
     lib = _lib.load()
     _require_gpu(Q, bias, E, scale, entity)
+    _check_qe(Q, E, scale, bias)
     if entity.dtype != torch.int64:
         raise TypeError("entity must be int64")
     B, d = Q.shape
@@ -129,6 +145,7 @@ def sample_scores(Q, bias, E, scale, entity):
     """out[b, j] = Q[b] . E[entity[b, j]] (* scale) + bias[b] for ``entity`` int64 [B,k]."""
     lib = _lib.load()
     _require_gpu(Q, bias, E, scale, entity)
+    _check_qe(Q, E, scale, bias)
     if entity.dtype != torch.int64 or entity.dim() != 2 or entity.shape[0] != Q.shape[0]:
         raise ValueError("entity must be an int64 tensor of shape [B, k]")
     entity = entity.contiguous()
@@ -145,6 +162,7 @@ def row_minmax(Q, bias, E, scale=None):
     """(min [B], max [B]) of every query's scores over all entities, without the [B,N] matrix."""
     lib = _lib.load()
     _require_gpu(Q, bias, E, scale)
+    _check_qe(Q, E, scale, bias)
     B, d = Q.shape
     lo = torch.empty((B,), dtype=torch.float32, device=Q.device)
     hi = torch.empty((B,), dtype=torch.float32, device=Q.device)
@@ -202,6 +220,7 @@ def rank_filtered(Q, bias, E, scale, target, csr_row=None, row_ptr=None, col=Non
     ``target_score`` (all [B])."""
     lib = _lib.load()
     _require_gpu(Q, bias, E, scale, target, csr_row, row_ptr, col)
+    _check_qe(Q, E, scale, bias)
     B, d = Q.shape
     N = E.shape[0]
     dev = Q.device
@@ -227,6 +246,7 @@ def topk(Q, bias, E, scale, k, sigmoid=False):
     """Fused top-k over all entities: ([B,k] fp32 descending, [B,k] int64)."""
     lib = _lib.load()
     _require_gpu(Q, bias, E, scale)
+    _check_qe(Q, E, scale, bias)
     B, d = Q.shape
     N = E.shape[0]
     dev = Q.device
@@ -244,6 +264,7 @@ def bce_multihot(Q, bias, E, scale, csr_row, row_ptr, col, label_smoothing=0.0):
     """Mean BCE-with-logits of the [B,N] scores against the multi-hot of the CSR rows: [1] fp32 tensor."""
     lib = _lib.load()
     _require_gpu(Q, bias, E, scale, csr_row, row_ptr, col)
+    _check_qe(Q, E, scale, bias)
     B, d = Q.shape
     N = E.shape[0]
     loss = torch.empty((1,), dtype=torch.float32, device=Q.device)
@@ -262,6 +283,7 @@ def bce_multihot_backward(Q, bias, E, csr_row, row_ptr, col, label_smoothing=0.0
     ``(loss or None, dQ, dbias, dE)``.  The [B,N] gradient of the scores lives only in the call's workspace."""
     lib = _lib.load()
     _require_gpu(Q, bias, E, csr_row, row_ptr, col)
+    _check_qe(Q, E, None, bias)
     if E.dtype != torch.float32:
         raise TypeError("bce_multihot_backward needs an fp32 entity table")
     B, d = Q.shape

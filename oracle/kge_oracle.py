@@ -26,6 +26,9 @@ Pinning status (independent checks live in ``tests/test_oracle_pins.py``)
                       c=0 == DistMult on the first half; general (p,q) against a
                       brute-force geometric-algebra product on bitmask blades;
                       thresholds p>=2 / q>=2 / (p>=2 and q>=2) by fixtures.
+* ``relation_prediction_ranks``  hand-computed fixture ``tests/golden/relation_prediction_literal.json``
+                      (scores, masked columns, ranks and the IndexError case worked out on paper), and the
+                      torch op sequence of ``oracle/torch_cpu_path.py`` on random inputs.
 * ``decal_*``         general (p,q,r) against the same brute-force geometric-algebra product with r
                       bases that square to zero (bivector families counted under the reference's
                       ">= 2 of each" conditions); r = 0 == Keci; single-GEMM form == einsum form;
@@ -902,6 +905,27 @@ def filtered_ranks(scores, targets, filters, tie="stable"):
         G, T, TL = filtered_rank_counts(scores[j], int(t), filters[j])
         out[j] = 1 + G + {"stable": TL, "optimistic": 0, "pessimistic": T}[tie]
     return out
+
+
+def relation_prediction_ranks(model, E, R, triples, ee_vocab, tie="stable", **kw):
+    """Ranks of the reference's relation-prediction loop (dicee/evaluation/evaluator.py:440-471), literally.
+
+    The loop hands ``(head, tail)`` pairs to ``forward_k_vs_all`` (:450-454), which looks the second column up
+    in the RELATION table (base_model.py:377-384): a tail id that is not below the number of relations raises
+    ``IndexError`` there.  The result holds one score per ENTITY; the loop masks the columns listed in
+    ``ee_vocab[(head, tail)]`` (relation ids used as column numbers, :457-460, the target column restored) and
+    takes the position of column ``relation`` in a descending sort over all entity columns (:462-467).
+    ``ee_vocab``: dict ``(head, tail) -> [relation ids]`` (missing key: empty list, it is a defaultdict there).
+    """
+    triples = np.asarray(triples, dtype=np.int64)
+    N, nR = E.shape[0], R.shape[0]
+    if len(triples) and (triples[:, 2].max() >= nR or triples[:, 2].min() < 0):
+        raise IndexError("index out of range in self")
+    if len(triples) and (triples[:, 1].max() >= N or triples[:, 1].min() < 0):
+        raise IndexError("relation id used as a column of the entity scores is out of bounds")
+    S = k_vs_all_scores(model, E, R, triples[:, [0, 2]], **kw)
+    filters = [list(ee_vocab.get((int(h), int(t)), [])) for h, _, t in triples]
+    return filtered_ranks(S, triples[:, 1], filters, tie=tie)
 
 
 def rank_interval_with_tolerance(scores_row, target, filt, tol):

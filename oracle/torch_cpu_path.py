@@ -123,6 +123,30 @@ def evaluate_entity_prediction(model, E, R, triples, er_vocab, batch_size, **kw)
     return ranks
 
 
+def evaluate_relation_prediction(model, E, R, triples, ee_vocab, batch_size, **kw):
+    """``Evaluator._evaluate_relation_prediction`` (evaluator.py:440-471): list of ranks.  The (head, tail) pair
+    goes through ``forward_k_vs_all`` as the reference passes it; torch raises IndexError when a tail id is not a
+    valid row of the relation table."""
+    ranks = []
+    n = len(triples)
+    for i in range(0, n, batch_size):
+        data_batch = triples[i:i + batch_size]
+        e1_idx_e2_idx = torch.LongTensor(np.ascontiguousarray(data_batch[:, [0, 2]]))
+        r_idx = torch.LongTensor(np.ascontiguousarray(data_batch[:, 1]))
+        with torch.no_grad():
+            predictions = forward_k_vs_all(model, E, R, e1_idx_e2_idx, **kw)
+        for j in range(data_batch.shape[0]):
+            filt = ee_vocab.get((int(data_batch[j][0]), int(data_batch[j][2])), [])
+            target_value = predictions[j, r_idx[j]].item()
+            predictions[j, filt] = -np.inf
+            predictions[j, r_idx[j]] = target_value
+        _, sort_idxs = torch.sort(predictions, dim=1, descending=True)
+        for j in range(data_batch.shape[0]):
+            rank = torch.where(sort_idxs[j] == r_idx[j])[0].item() + 1
+            ranks.append(rank)
+    return ranks
+
+
 def predict_topk_indices(model, E, R, hr_pairs, topk, batch_size, **kw):
     """``KGE.predict_missing_tail_entity(..., return_indices=True)``
     (knowledge_graph_embeddings.py:374-411): ([P,k] scores, [P,k] int64 ids)."""

@@ -122,6 +122,84 @@ def test_evaluator_matches_the_reference_loop(name, d, extra, batch_size):
         np.testing.assert_array_equal(own, got)
 
 
+@pytest.mark.parametrize("name,d,extra", [("DistMult", 32, {}), ("QMult", 64, {})])
+def test_relation_prediction_follows_the_reference_loop_literally(name, d, extra):
+    """form_of_labelling='RelationPrediction' (evaluator.py:440-471): (head, tail) pairs through forward_k_vs_all,
+    the (head, tail) -> relations vocabulary as the mask, the rank of column `relation` among all entity columns;
+    IndexError when a tail id is not a row of the relation table."""
+    from dicee_amd import Evaluator
+    m, triples = _toy(name, d, n=900, seed=11, **extra)
+    triples[:, 2] = triples[:, 2] % 46                     # tails that are valid relation rows
+    triples[:40, [0, 2]] = triples[0, [0, 2]]              # one (head, tail) pair with many relations
+    E = m.entity_embeddings.weight.detach().clone().numpy()
+    Rel = m.relation_embeddings.weight.detach().clone().numpy()
+    ee = {}
+    for h, r, t in triples:
+        ee.setdefault((int(h), int(t)), []).append(int(r))
+    m = m.to("cuda")
+    args = SimpleNamespace(batch_size=256, eval_model="test", scoring_technique="KvsAll", full_storage_path=None)
+    # (a) the vocabulary given as the reference's dict
+    ds = SimpleNamespace(num_entities=135, num_relations=46, er_vocab={}, ee_vocab=ee, train_set=triples,
+                         valid_set=None, test_set=triples[200:700])
+    ev = Evaluator(args)
+    report = ev.eval(ds, m, "RelationPrediction", during_training=True)
+    got = ev.last_ranks
+    S = ko.k_vs_all_scores(name, E, Rel, triples[200:700][:, [0, 2]])
+    for j, (h, r, t) in enumerate(triples[200:700]):
+        tol = 1e-5 * np.sqrt((S[j] ** 2).mean())
+        lo, hi = ko.rank_interval_with_tolerance(S[j], int(r), ee[(int(h), int(t))], tol)
+        assert lo <= got[j] <= hi
+    want = ko.relation_prediction_ranks(name, E, Rel, triples[200:700], ee)
+    assert np.mean(want == got) >= 0.99
+    ref = tcp.evaluate_relation_prediction(name, torch.from_numpy(E), torch.from_numpy(Rel), triples[200:700], ee, 256)
+    assert np.mean(np.asarray(ref) == got) >= 0.99
+    assert report["Test"]["MRR"] == pytest.approx(ko.metrics_from_ranks(got)["MRR"])
+    # (b) the vocabulary built on the GPU from the dataset's splits
+    ds2 = SimpleNamespace(num_entities=135, num_relations=46, train_set=triples, valid_set=None,
+                          test_set=triples[200:700])
+    ev2 = Evaluator(args)
+    ev2.eval(ds2, m, "RelationPrediction", during_training=True)
+    np.testing.assert_array_equal(ev2.last_ranks, got)
+    # (c) a tail id that is not a relation row: the reference's embedding lookup raises
+    bad = triples[200:210].copy()
+    bad[3, 2] = 46
+    with pytest.raises(IndexError):
+        ev.evaluate_lp_k_vs_all(m, bad, form_of_labelling="RelationPrediction")
+
+
+def test_evaluator_routes_negative_sampling_models_to_both_directions():
+    """scoring_technique='NegSample' (evaluator.py:174-180, :246-272, :622-643): heads and tails through
+    evaluate_lp; the report equals a direct evaluate_lp call.  'constraint' in eval_model is refused."""
+    from dicee_amd import Evaluator
+    from dicee_amd.link_prediction import evaluate_lp
+    m, triples = _toy("ComplEx", 32, n=1200, seed=5)
+    er, re = {}, {}
+    for h, r, t in triples:
+        er.setdefault((int(h), int(r)), []).append(int(t))
+        re.setdefault((int(r), int(t)), []).append(int(h))
+    m = m.to("cuda")
+    ds = SimpleNamespace(num_entities=135, num_relations=46, er_vocab=er, re_vocab=re, train_set=triples,
+                         valid_set=triples[:100], test_set=triples[100:500])
+    ev = Evaluator(SimpleNamespace(batch_size=128, eval_model="val_test", scoring_technique="NegSample",
+                                   full_storage_path=None))
+    report = ev.eval(ds, m, "EntityPrediction", during_training=True)
+    assert set(report) == {"Val", "Test"}
+    want = evaluate_lp(m, triples[100:500], num_entities=135, er_vocab=er, re_vocab=re, info=None)
+    assert report["Test"] == want
+    ds2 = SimpleNamespace(num_entities=135, num_relations=46, train_set=triples, valid_set=None,
+                          test_set=triples[100:500])                       # vocabularies from the splits
+    ev2 = Evaluator(SimpleNamespace(batch_size=128, eval_model="test", scoring_technique="NegSample",
+                                    full_storage_path=None))
+    assert ev2.eval(ds2, m, "EntityPrediction", during_training=True)["Test"] == want
+    ev3 = Evaluator(SimpleNamespace(batch_size=128, eval_model="test_constraint", scoring_technique="KvsAll",
+                                    full_storage_path=None))
+    with pytest.raises(NotImplementedError):
+        ev3.eval(ds, m, "EntityPrediction", during_training=True)
+    ev4 = Evaluator(SimpleNamespace(batch_size=128, eval_model=None, scoring_technique="KvsAll",
+                                    full_storage_path=None))
+    assert ev4.eval(ds, m, "EntityPrediction") is None
+
+
 def test_predict_topk_and_predict_invariants():
     from dicee_amd import KGE
     m, _ = _toy("Keci", 32, p=0, q=1, seed=5)
@@ -178,6 +256,28 @@ def test_quantised_storage_follows_dequantised_fp32_math(storage):
     vals, idx = m.topk(x, 10)
     wv, wi = ko.topk(S, 10)
     np.testing.assert_array_equal(idx.cpu().numpy(), wi)
+
+
+@pytest.mark.parametrize("storage", ["bf16", "int8"])
+def test_quantised_tables_follow_the_parameters(storage):
+    """The bf16 / int8 tables are copies of the parameters: after an in-place update (an optimizer step,
+    load_state_dict) or a move to another device the next call scores the NEW weights."""
+    from dicee_amd import ops
+    m, triples = _toy("DistMult", 128, N=500, R=7, n=50, seed=9)
+    m = m.set_entity_storage(storage).to("cuda").eval()             # stored on the CPU, then moved
+    x = torch.from_numpy(triples[:20, :2].copy() % np.array([500, 7])).cuda()
+    before = m(x).clone()
+    with torch.no_grad():
+        m.entity_embeddings.weight.mul_(-2.0)                        # an exact change in every storage
+    after = m(x)
+    # DistMult: scores are cubic in a common scale of the entity table (head row and every tail row)
+    assert torch.equal(after, before * 4.0)
+    sd = {k: v.clone() for k, v in m.state_dict().items()}
+    sd["entity_embeddings.weight"] = sd["entity_embeddings.weight"] * -0.5
+    m.load_state_dict(sd)
+    assert torch.equal(m(x), before)
+    with pytest.raises(ValueError):
+        ops.scores(torch.zeros((4, 64), device="cuda"), None, m.table()[0], m.table()[1])   # d mismatch: refused
 
 
 def test_kvsall_bce_loss_matches_training_step_forward():

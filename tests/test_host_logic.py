@@ -167,6 +167,23 @@ def test_models_mirror_reference_parameters_and_have_no_cpu_fallback():
         d((torch.zeros((2, 2), dtype=torch.int64), torch.zeros((2, 3), dtype=torch.int64)))   # forward_k_vs_sample too
     with pytest.raises(NotImplementedError):
         d(torch.zeros((2, 3, 4), dtype=torch.int64))               # byte-pair-encoded input
+    # dropout: the reference drops elements in training mode (base_model.py:381-383); this path refuses instead
+    dp = models.DistMult({"model": "DistMult", "embedding_dim": 8, "num_entities": 5, "num_relations": 2,
+                          "input_dropout_rate": 0.3})
+    assert dp.training
+    for call in (lambda: dp(torch.zeros((2, 2), dtype=torch.int64)),
+                 lambda: dp.kvsall_training_step(torch.zeros((2, 2), dtype=torch.int64), None),
+                 lambda: dp.kvsall_bce_gradients(torch.zeros((2, 2), dtype=torch.int64), None),
+                 lambda: dp.rank_filtered(torch.zeros((2, 2), dtype=torch.int64), torch.zeros(2, dtype=torch.int64))):
+        with pytest.raises(NotImplementedError, match="dropout"):
+            call()
+    dp.eval()
+    with pytest.raises(RuntimeError):                              # eval mode: past the dropout check, then no CPU path
+        dp(torch.zeros((2, 2), dtype=torch.int64))
+    hd = models.ComplEx({"model": "ComplEx", "embedding_dim": 8, "num_entities": 5, "num_relations": 2,
+                         "hidden_dropout_rate": 0.1})
+    with pytest.raises(NotImplementedError, match="dropout"):
+        hd(torch.zeros((2, 2), dtype=torch.int64))
 
 
 def test_synthetic_configs_small_scale():

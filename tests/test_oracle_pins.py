@@ -410,6 +410,37 @@ def test_evaluator_port_matches_closed_form_without_ties():
     assert m["H@3"] == sum(r <= 3 for r in ranks) / len(ranks)
 
 
+def test_relation_prediction_literal_fixture_and_torch_sequence():
+    """The relation-prediction loop as the reference literally behaves (evaluator.py:440-471): the hand-computed
+    fixture pins scores, masked columns, ranks and the IndexError; random inputs pin the numpy closed form against
+    the reference's torch op sequence (mask with -inf, full sort, where)."""
+    with open(os.path.join(GOLD, "relation_prediction_literal.json")) as f:
+        fx = json.load(f)
+    E, Rel = np.array(fx["E"], dtype=np.float64), np.array(fx["Rel"], dtype=np.float64)
+    ee = {(int(k[0]), int(k[1])): v for k, v in fx["ee_vocab"]}
+    trip = np.array(fx["triples"])
+    S = ko.k_vs_all_scores("DistMult", E, Rel, trip[:, [0, 2]])
+    np.testing.assert_array_equal(S, np.array(fx["scores"], dtype=np.float64))
+    assert list(ko.relation_prediction_ranks("DistMult", E, Rel, trip, ee)) == fx["ranks"]
+    assert list(ko.relation_prediction_ranks("DistMult", E, Rel, trip, {})) == fx["unfiltered_ranks"]
+    assert tcp.evaluate_relation_prediction("DistMult", torch.tensor(E), torch.tensor(Rel), trip, ee, 3) == fx["ranks"]
+    bad = np.array([fx["index_error_triple"]])
+    with pytest.raises(IndexError):
+        ko.relation_prediction_ranks("DistMult", E, Rel, bad, ee)
+    with pytest.raises(IndexError):
+        tcp.evaluate_relation_prediction("DistMult", torch.tensor(E), torch.tensor(Rel), bad, ee, 3)
+    # random: tails below the number of relations, as the literal loop needs
+    rng = np.random.default_rng(12)
+    N, Rn, d = 60, 9, 8
+    E, R = _tables(rng, N, Rn, d, sd=1.0)
+    triples = np.stack([rng.integers(0, N, 80), rng.integers(0, Rn, 80), rng.integers(0, Rn, 80)], axis=1)
+    ee = {}
+    for h, r, t in triples:
+        ee.setdefault((int(h), int(t)), []).append(int(r))
+    got = tcp.evaluate_relation_prediction("ComplEx", torch.tensor(E), torch.tensor(R), triples, ee, 32)
+    assert got == list(ko.relation_prediction_ranks("ComplEx", E, R, triples, ee))
+
+
 # -------------------------------------------------------------- top-k, BCE
 def test_topk_vs_bruteforce_and_torch():
     rng = np.random.default_rng(11)
