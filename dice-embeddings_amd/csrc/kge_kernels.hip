@@ -1219,28 +1219,27 @@ extern "C" int kge_csr_lookup(const int64_t* hr, int64_t B, const int64_t* keys,
 
 extern "C" size_t kge_rank_workspace_bytes(int64_t B) { return rank_ws_layout(B < 1 ? 1 : B, nullptr, nullptr); }
 
-extern "C" int kge_rank_filtered(const float* Q, const float* bias, const void* E, int dtype, const float* scale,
-                                 int64_t B, int64_t d, int64_t N, const int64_t* target, const int64_t* csr_row,
-                                 const int64_t* row_ptr, const int32_t* col, int64_t n_rows, int32_t* n_greater,
-                                 int32_t* n_equal, int32_t* n_equal_lower, float* target_score, void* workspace,
-                                 size_t workspace_bytes, void* stream) {
-  clear_error();
-  int rc = check_contract("kge_rank_filtered", Q, E, dtype, scale, B, d, N);
+namespace {
+// argument checks shared by the two filtered-rank entry points
+int check_rank_args(const char* who, const float* Q, const void* E, int dtype, const float* scale, int64_t B, int64_t d,
+                    int64_t N, const int64_t* target, const int64_t* csr_row, const int64_t* row_ptr, const int32_t* col,
+                    int64_t n_rows, const int32_t* n_greater, const int32_t* n_equal, const int32_t* n_equal_lower,
+                    const float* target_score) {
+  int rc = check_contract(who, Q, E, dtype, scale, B, d, N);
   if (rc) return rc;
   if (B == 0) return KGE_OK;
   KGE_REQUIRE(target && n_greater && n_equal && n_equal_lower && target_score, KGE_ERR_INVALID,
-              "kge_rank_filtered: null target or output pointer");
-  const bool filtered = csr_row != nullptr;
-  KGE_REQUIRE(!filtered || (row_ptr && col && n_rows >= 0), KGE_ERR_INVALID,
-              "kge_rank_filtered: csr_row given without row_ptr / col");
-  KGE_REQUIRE(n_rows < 0x7fffffffLL, KGE_ERR_INVALID, "kge_rank_filtered: n_rows=%lld too large", (long long)n_rows);
-  KGE_REQUIRE(workspace && workspace_bytes >= kge_rank_workspace_bytes(B), KGE_ERR_WORKSPACE,
-              "kge_rank_filtered: workspace of %zu bytes, need %zu", workspace_bytes, kge_rank_workspace_bytes(B));
-  KGE_REQUIRE(((uintptr_t)workspace & 7) == 0, KGE_ERR_WORKSPACE, "kge_rank_filtered: workspace must be 8-byte aligned");
-  hipStream_t st = (hipStream_t)stream;
-  RankWs ws;
-  rank_ws_layout(B, workspace, &ws);
+              "%s: null target or output pointer", who);
+  KGE_REQUIRE(!csr_row || (row_ptr && col && n_rows >= 0), KGE_ERR_INVALID, "%s: csr_row given without row_ptr / col", who);
+  KGE_REQUIRE(n_rows < 0x7fffffffLL, KGE_ERR_INVALID, "%s: n_rows=%lld too large", who, (long long)n_rows);
+  return KGE_OK;
+}
 
+// the launches of a filtered-rank call; `ws` points into a caller's workspace or into the library's static scratch
+int rank_filtered_launch(const char* who, const float* Q, const float* bias, const void* E, int dtype, const float* scale,
+                         int64_t B, int64_t d, int64_t N, const int64_t* target, const int64_t* csr_row,
+                         const int64_t* row_ptr, const int32_t* col, int64_t n_rows, int32_t* n_greater, int32_t* n_equal,
+                         int32_t* n_equal_lower, float* target_score, const RankWs& ws, hipStream_t st) {
   ContractArgs a = make_args(Q, E, dtype, scale, B, d, N, 0, N);
   {
     dim3 grid((unsigned)((B + 127) / 128)), block(256);
@@ -1249,9 +1248,9 @@ extern "C" int kge_rank_filtered(const float* Q, const float* bias, const void* 
     KGE_LAUNCH_CHECK("target_score_kernel");
   }
   RankArgs ea{ws.thr, target, n_greater, n_equal, n_equal_lower};
-  rc = launch_contract<RankEpi>(dtype, a, ea, st, "kge_rank_filtered");
+  int rc = launch_contract<RankEpi>(dtype, a, ea, st, who);
   if (rc) return rc;
-  if (filtered && n_rows > 0) {
+  if (csr_row != nullptr && n_rows > 0) {
     for (int64_t b0 = 0; b0 < B; b0 += SORT_MAX) {
       const int nb = (int)((B - b0 < SORT_MAX) ? B - b0 : SORT_MAX);
       hipLaunchKernelGGL(plan_fix_kernel, dim3(1), dim3(1024), 0, st, csr_row, b0, nb, n_rows, row_ptr, ws.plan);
@@ -1263,6 +1262,82 @@ extern "C" int kge_rank_filtered(const float* Q, const float* bias, const void* 
     }
   }
   return KGE_OK;
+}
+}  // namespace
+
+extern "C" int kge_rank_filtered(const float* Q, const float* bias, const void* E, int dtype, const float* scale,
+                                 int64_t B, int64_t d, int64_t N, const int64_t* target, const int64_t* csr_row,
+                                 const int64_t* row_ptr, const int32_t* col, int64_t n_rows, int32_t* n_greater,
+                                 int32_t* n_equal, int32_t* n_equal_lower, float* target_score, void* workspace,
+                                 size_t workspace_bytes, void* stream) {
+  clear_error();
+  int rc = check_rank_args("kge_rank_filtered", Q, E, dtype, scale, B, d, N, target, csr_row, row_ptr, col, n_rows,
+                           n_greater, n_equal, n_equal_lower, target_score);
+  if (rc) return rc;
+  if (B == 0) return KGE_OK;
+  KGE_REQUIRE(workspace && workspace_bytes >= kge_rank_workspace_bytes(B), KGE_ERR_WORKSPACE,
+              "kge_rank_filtered: workspace of %zu bytes, need %zu", workspace_bytes, kge_rank_workspace_bytes(B));
+  KGE_REQUIRE(((uintptr_t)workspace & 7) == 0, KGE_ERR_WORKSPACE, "kge_rank_filtered: workspace must be 8-byte aligned");
+  RankWs ws;
+  rank_ws_layout(B, workspace, &ws);
+  return rank_filtered_launch("kge_rank_filtered", Q, bias, E, dtype, scale, B, d, N, target, csr_row, row_ptr, col,
+                              n_rows, n_greater, n_equal, n_equal_lower, target_score, ws, (hipStream_t)stream);
+}
+
+// ---- the same call for callers that cannot allocate ---------------------------------------------------
+// The workspace of kge_rank_filtered (thresholds, the plan of the filter correction) lives in a file-scope
+// device array instead of caller memory.  Every GPU the library runs on holds its own copy of the array at its
+// own address until the process ends; the address is looked up once per device and only that pointer is ever
+// handed to a kernel.  All calls on one GPU share the array: calls that overlap on one GPU race.
+static __device__ __align__(256) unsigned char scratch[4 * KGE_RANK_STATIC_MAX_B + 20 * SORT_MAX + 1024];
+
+namespace {
+constexpr int SCRATCH_MAX_DEVICES = 64;
+std::mutex g_scratch_mu;
+unsigned char* g_scratch_ptr[SCRATCH_MAX_DEVICES] = {};
+
+// device address of `scratch` on the current device (looked up on the first call on that device)
+int scratch_on_current_device(unsigned char** out) {
+  int dev = -1;
+  KGE_HIP_CHECK(hipGetDevice(&dev));
+  KGE_REQUIRE(dev >= 0 && dev < SCRATCH_MAX_DEVICES, KGE_ERR_UNSUPPORTED, "device ordinal %d outside [0, %d)", dev,
+              SCRATCH_MAX_DEVICES);
+  std::lock_guard<std::mutex> lk(g_scratch_mu);
+  if (g_scratch_ptr[dev] == nullptr) {
+    void* p = nullptr;
+    KGE_HIP_CHECK(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+    KGE_REQUIRE(p != nullptr, KGE_ERR_HIP, "hipGetSymbolAddress returned a null address for the scratch array");
+    g_scratch_ptr[dev] = (unsigned char*)p;
+  }
+  *out = g_scratch_ptr[dev];
+  return KGE_OK;
+}
+}  // namespace
+
+extern "C" int kge_rank_filtered_static(const float* Q, const float* bias, const void* E, int dtype, const float* scale,
+                                        int64_t B, int64_t d, int64_t N, const int64_t* target, const int64_t* csr_row,
+                                        const int64_t* row_ptr, const int32_t* col, int64_t n_rows, int32_t* n_greater,
+                                        int32_t* n_equal, int32_t* n_equal_lower, float* target_score, void* stream) {
+  clear_error();
+  int rc = check_rank_args("kge_rank_filtered_static", Q, E, dtype, scale, B, d, N, target, csr_row, row_ptr, col, n_rows,
+                           n_greater, n_equal, n_equal_lower, target_score);
+  if (rc) return rc;
+  KGE_REQUIRE(B <= KGE_RANK_STATIC_MAX_B, KGE_ERR_WORKSPACE,
+              "kge_rank_filtered_static: B=%lld exceeds the %d queries the static scratch array holds; split the batch "
+              "or call kge_rank_filtered with a workspace", (long long)B, KGE_RANK_STATIC_MAX_B);
+  if (B == 0) return KGE_OK;
+  KGE_REQUIRE(rank_ws_layout(B, nullptr, nullptr) <= sizeof(scratch), KGE_ERR_WORKSPACE,
+              "kge_rank_filtered_static: internal layout of %zu bytes exceeds the scratch array",
+              rank_ws_layout(B, nullptr, nullptr));
+  unsigned char* base = nullptr;
+  rc = scratch_on_current_device(&base);
+  if (rc) return rc;
+  // nothing in the scratch needs clearing: thresholds are written for every query and the plan is rebuilt per
+  // sub-batch before anything reads it, so what an earlier (larger) call left behind is never read
+  RankWs ws;
+  rank_ws_layout(B, base, &ws);
+  return rank_filtered_launch("kge_rank_filtered_static", Q, bias, E, dtype, scale, B, d, N, target, csr_row, row_ptr,
+                              col, n_rows, n_greater, n_equal, n_equal_lower, target_score, ws, (hipStream_t)stream);
 }
 
 extern "C" size_t kge_topk_workspace_bytes(int64_t B, int64_t N, int64_t k) {

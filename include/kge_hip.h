@@ -225,6 +225,23 @@ int kge_rank_filtered(const float* Q, const float* bias, const void* E, int dtyp
                       float* target_score, void* workspace, size_t workspace_bytes, void* stream);
 
 /*
+ * kge_rank_filtered without a workspace argument and without any allocation.  No counterpart in the reference:
+ * it exists for callers that cannot allocate device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc).  The thresholds and the plan of the filter correction live in a
+ * static device array inside the library (about 420 KB per GPU, held until the process ends), so
+ *   - B <= KGE_RANK_STATIC_MAX_B, KGE_ERR_WORKSPACE otherwise (split the batch, or use kge_rank_filtered);
+ *   - all calls on one GPU share that array: calls that overlap on one GPU (two streams, two threads) race;
+ *   - the current device must be the one the pointers and the stream belong to.
+ * Arguments, outputs and results are those of kge_rank_filtered, bit for bit.
+ */
+#define KGE_RANK_STATIC_MAX_B 65536
+int kge_rank_filtered_static(const float* Q, const float* bias, const void* E, int dtype, const float* scale,
+                             int64_t B, int64_t d, int64_t N, const int64_t* target, const int64_t* csr_row,
+                             const int64_t* row_ptr, const int32_t* col, int64_t n_rows,
+                             int32_t* n_greater, int32_t* n_equal, int32_t* n_equal_lower,
+                             float* target_score, void* stream);
+
+/*
  * Fused top-k over all entities: torch.topk(model(batch_hr), k, dim=1) of
  * KGE.predict_missing_tail_entity (dicee/knowledge_graph_embeddings.py:397-401) and, with
  * apply_sigmoid, the torch.sigmoid of KGE.predict_topk (:568), without writing B x N scores.
