@@ -136,6 +136,7 @@ template <int NQT>
 struct StoreEpi {
   static constexpr bool SWAP = true;
   static constexpr bool STAGE_HOOK = false;
+  static constexpr bool DEFER = false;
   using Args = StoreArgs;
   struct Shared {
     float bias[8 * 32 * NQT];  // per wave: the biases of its 32 * NQT queries (up to 8 waves per workgroup)
@@ -157,6 +158,7 @@ struct StoreEpi {
     lb = mine;
     __syncthreads();
   }
+  __device__ void stage_mark() {}
   __device__ void stage_end() {}
   template <bool HAS_SCALE>
   __device__ __forceinline__ void tile(int qt, const f32x16& acc, const float* sc16, float sc_col, int64_t e_base,
@@ -192,10 +194,12 @@ template <int NQT>
 struct RankEpi {
   static constexpr bool SWAP = false;
   static constexpr bool STAGE_HOOK = false;
+  static constexpr bool DEFER = false;
   struct Shared {
     int unused;
   };
   __device__ void bind(Shared*) {}
+  __device__ void stage_mark() {}
   __device__ void stage_end() {}
   using Args = RankArgs;
   Args a;
@@ -283,6 +287,97 @@ struct RankEpi {
   }
 };
 
+// The rank epilogue of qstream_kernel.  The hot path has no branch at all: the exact-tie test of a tile only
+// feeds a running minimum of |threshold - score| per stage buffer, padding rows are counted like any other,
+// and the kernel asks once per stage whether anything in it needs the exact treatment (a tie, or rows past
+// the end of the table); if so it forms that stage's tiles again and hands them to tile_slow().  Ties other
+// than a target with itself are rare and padding only exists in the last stage of the table, so the second
+// pass costs a fraction of a percent, and the main loop stays straight-line code.
+template <int NQT>
+struct RankFastEpi {
+  static constexpr bool SWAP = false;
+  static constexpr bool STAGE_HOOK = false;
+  static constexpr bool DEFER = true;
+  static constexpr int SLOTS = 3;  // stage buffers in flight: one running minimum each
+  struct Shared {
+    int unused;
+  };
+  __device__ void bind(Shared*) {}
+  __device__ void stage_mark() {}
+  __device__ void stage_end() {}
+  using Args = RankArgs;
+  Args a;
+  float thr[NQT];
+  int32_t gt[NQT];
+  float mn[SLOTS];
+  int64_t q0, B;
+  int c, hf;
+  __device__ void init(const Args& args, int64_t q0_, int c_, int hf_, int64_t B_) {
+    a = args; q0 = q0_; c = c_; hf = hf_; B = B_;
+#pragma unroll
+    for (int t = 0; t < NQT; ++t) {
+      const int64_t q = q0 + 32 * t + c;
+      thr[t] = (q < B) ? a.thr[q] : __uint_as_float(0x7fc00000u);  // NaN never compares
+      gt[t] = 0;
+    }
+#pragma unroll
+    for (int j = 0; j < SLOTS; ++j) mn[j] = __uint_as_float(0x7f800000u);
+  }
+  // d = thr - s is exact in sign and is zero only for an exact tie; the sign bits are shifted into one register
+  // (v_alignbit) and counted once per tile.  `slot`: the buffer of the stage the tile belongs to.
+  __device__ __forceinline__ void tile_fast(int slot, int qt, const f32x16& acc) {
+    const float th = thr[qt];
+    uint32_t bits = 0;
+    float m = mn[slot];
+#pragma unroll
+    for (int i = 0; i < 16; i += 2) {
+      const float d0 = th - acc[i], d1 = th - acc[i + 1];
+      bits = __builtin_amdgcn_alignbit(bits, __float_as_uint(d0), 31);
+      bits = __builtin_amdgcn_alignbit(bits, __float_as_uint(d1), 31);
+      m = __builtin_fminf(__builtin_fminf(m, __builtin_fabsf(d0)), __builtin_fabsf(d1));
+    }
+    mn[slot] = m;
+    gt[qt] += __builtin_popcount(bits);
+  }
+  // wave-uniform: does the stage whose tiles went to `slot` need the exact pass?  Resets the slot.
+  __device__ __forceinline__ bool stage_dirty(int slot, bool padded) {
+    const unsigned long long tie = __builtin_amdgcn_ballot_w64(mn[slot] == 0.f);
+    mn[slot] = __uint_as_float(0x7f800000u);
+    return tie != 0 || padded;
+  }
+  // one tile of a stage formed again: ties and padding rows, exactly (the hot path has already counted every
+  // element whose score is strictly greater, padding rows included).  Out of line and fed with scalars only, so
+  // that nothing of it (addresses of the target / tie counters) is kept in registers across the main loop.
+  static __device__ __attribute__((noinline)) int32_t slow_impl(f32x16 s, float th, int64_t q, int64_t B,
+                                                               const int64_t* target, int32_t* n_eq, int32_t* n_eql,
+                                                               int64_t e_base, int64_t limit, int hf) {
+    const int32_t tg = (q < B) ? (int32_t)target[q] : -1;
+    const typename RankEpi<NQT>::Fix f = RankEpi<NQT>::tile_fix(s, th, tg, e_base, limit, hf);
+    if (q < B && th == th) {
+      if (f.eq) atomicAdd(&n_eq[q], f.eq);
+      if (f.eql) atomicAdd(&n_eql[q], f.eql);
+    }
+    return f.dg;
+  }
+  __device__ __forceinline__ void tile_slow(int qt, const f32x16& s, int64_t e_base, int64_t limit) {
+    gt[qt] += slow_impl(s, thr[qt], q0 + 32 * qt + c, B, a.target, a.n_eq, a.n_eql, e_base, limit, hf);
+  }
+  // after a barrier: the thresholds pass through an opaque no-op, so that no epilogue arithmetic of a tile
+  // scheduled after the barrier is moved (and its results kept in registers) to before it
+  __device__ __forceinline__ void touch() {
+#pragma unroll
+    for (int t = 0; t < NQT; ++t) asm volatile("" : "+v"(thr[t]));
+  }
+  __device__ void finish() {
+#pragma unroll
+    for (int t = 0; t < NQT; ++t) {
+      const int64_t q = q0 + 32 * t + c;
+      const int32_t g = gt[t] + __shfl_xor(gt[t], 32, 64);  // both halves of the wave hold the same query
+      if (hf == 0 && q < B && thr[t] == thr[t] && g) atomicAdd(&a.n_gt[q], g);
+    }
+  }
+};
+
 struct TopkArgs {
   const float* tau;          // per query: k-th best score so far (-inf while fewer than k known)
   const int32_t* active;     // NULL = all queries; else only queries with active[b] != 0 collect
@@ -295,16 +390,19 @@ template <int NQT>
 struct TopkEpi {
   static constexpr bool SWAP = false;
   static constexpr bool STAGE_HOOK = true;
+  static constexpr bool DEFER = false;
   using Args = TopkArgs;
   // Candidates are parked in LDS (cheap atomics) and moved to the per-query global buffers in bulk
   // at stage boundaries, so the hot loop never waits for a global atomic's round trip.
   struct Shared {
     int n;
+    int snap[2];  // n as thread 0 saw it just before a stage barrier (by stage parity): the same value for every wave
     int q[TOPK_LQ];
     unsigned long long key[TOPK_LQ];
   };
   Args a;
   Shared* sh;
+  int par;  // parity of the stage barriers passed so far
   float tau[NQT];
   int64_t q0, B;
   int c, hf;
@@ -319,7 +417,11 @@ struct TopkEpi {
   }
   __device__ void bind(Shared* s) {
     sh = s;
-    if (threadIdx.x == 0) s->n = 0;
+    par = 0;
+    if (threadIdx.x == 0) {
+      s->n = 0;
+      s->snap[0] = s->snap[1] = 0;
+    }
     __syncthreads();
   }
   // One candidate into its query's global buffer.  A full buffer keeps a uniform sample of what
@@ -374,21 +476,30 @@ struct TopkEpi {
     if (__builtin_expect(hit != 0, 0))
       collect(s, th, q0 + 32 * qt + c, e_base, limit, hf, sh, a.cnt, a.cand, a.cap);
   }
-  // Workgroup-uniform; call right after a barrier.  Empties the LDS queue once it is half full.
-  __device__ void flush(bool force) {
+  // Empties the LDS queue.  Every wave of the workgroup is inside (nobody appends meanwhile).
+  __device__ void flush() {
     const int n = sh->n;
-    if (n >= TOPK_LQ / 2 || (force && n > 0)) {
-      const int m = n < TOPK_LQ ? n : TOPK_LQ;
-      for (int i = threadIdx.x; i < m; i += blockDim.x) publish(sh->q[i], sh->key[i], a.cnt, a.cand, a.cap);
-      __syncthreads();
-      if (threadIdx.x == 0) sh->n = 0;
-      __syncthreads();
-    }
+    const int m = n < TOPK_LQ ? n : TOPK_LQ;
+    for (int i = threadIdx.x; i < m; i += blockDim.x) publish(sh->q[i], sh->key[i], a.cnt, a.cand, a.cap);
+    __syncthreads();
+    if (threadIdx.x == 0) sh->n = 0;
+    __syncthreads();
   }
-  __device__ void stage_end() { flush(false); }
+  // Stage boundaries: stage_mark() before the workgroup's barrier, stage_end() after it.  The decision to
+  // flush (queue at least half full) is taken on the count thread 0 recorded before the barrier, so every
+  // wave takes the same branch even if a fast wave is already appending again.  Two slots, used in turn: a
+  // slot is rewritten two barriers later, which no wave can reach before every wave has read it.
+  __device__ void stage_mark() {
+    if (threadIdx.x == 0) sh->snap[par] = sh->n;
+  }
+  __device__ void stage_end() {
+    const int n = sh->snap[par];
+    par ^= 1;
+    if (n >= TOPK_LQ / 2) flush();
+  }
   __device__ void finish() {
     __syncthreads();
-    flush(true);
+    flush();
   }
 };
 
@@ -402,10 +513,12 @@ template <int NQT>
 struct BceEpi {
   static constexpr bool SWAP = false;
   static constexpr bool STAGE_HOOK = false;
+  static constexpr bool DEFER = false;
   struct Shared {
     int unused;
   };
   __device__ void bind(Shared*) {}
+  __device__ void stage_mark() {}
   __device__ void stage_end() {}
   using Args = BceArgs;
   Args a;
@@ -476,6 +589,7 @@ template <int NQT>
 struct GradEpi {
   static constexpr bool SWAP = true;
   static constexpr bool STAGE_HOOK = false;
+  static constexpr bool DEFER = false;
   using Args = GradArgs;
   struct Shared {
     float bias[8 * 32 * NQT];
@@ -503,6 +617,7 @@ struct GradEpi {
     lb = mine;
     __syncthreads();
   }
+  __device__ void stage_mark() {}
   __device__ void stage_end() {}
   template <bool HAS_SCALE>
   __device__ __forceinline__ void tile(int qt, const f32x16& acc, const float* sc16, float sc_col, int64_t e_base,
@@ -581,10 +696,12 @@ template <int NQT>
 struct MinMaxEpi {
   static constexpr bool SWAP = false;
   static constexpr bool STAGE_HOOK = false;
+  static constexpr bool DEFER = false;
   struct Shared {
     int unused;
   };
   __device__ void bind(Shared*) {}
+  __device__ void stage_mark() {}
   __device__ void stage_end() {}
   using Args = MinMaxArgs;
   Args a;
@@ -774,6 +891,7 @@ __global__ void __launch_bounds__(256, 2) qreg_kernel(ContractArgs a, typename E
       }
     }
     if (st + 1 < nst) stage_store(buf ^ 1);
+    if (Epi::STAGE_HOOK) epi.stage_mark();
     __syncthreads();
     if (Epi::STAGE_HOOK) epi.stage_end();
   }
@@ -909,6 +1027,7 @@ __global__ void __launch_bounds__(64 * QA_WG_WAVES, QA_WAVES_PER_SIMD) qreg_asyn
     const int64_t row0 = row_next;
     if (row0 >= r_end) break;  // only the trailing stages of the table's last chunk can be empty
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    if (Epi::STAGE_HOOK) epi.stage_mark();
     __syncthreads();  // stage st has landed for every wave; everyone is done reading the other buffer
     if (Epi::STAGE_HOOK) epi.stage_end();
     if (st + 1 < total_stages) {
@@ -946,6 +1065,258 @@ __global__ void __launch_bounds__(64 * QA_WG_WAVES, QA_WAVES_PER_SIMD) qreg_asyn
     }
   }
   epi.template tile<false>(QA_NQT - 1, acc_prev, sc_dummy, 1.f, e_prev, r_end);
+  epi.finish();
+}
+
+// ============================================================================================
+// qstream_kernel: bf16 table, d == 128, the persistent walk, tiles, swizzled LDS rows and reduction
+// order of qreg_async_kernel with a deeper pipeline:
+//   * entity rows go global -> LDS in 64-row stages through a ring of three buffers: the loads of stage
+//     k + 2 are issued while stage k is multiplied, so a load has two stages to land;
+//   * one barrier per stage, between the stage's two entity tiles, and it waits for nothing but the
+//     global -> LDS loads it guards; the fragments of the next entity tile (of this stage or the next)
+//     are fetched under the last MFMA chain of the current one, so no wave waits for LDS after a barrier;
+//   * NQT query tiles per wave reuse every fragment read;
+//   * everything between two barriers is straight-line code (loads are issued unconditionally with clamped
+//     rows, the epilogue defers its rare cases to a per-stage check), scheduled as one MFMA, a few VALU
+//     instructions of the previous tile's epilogue, one fragment read, and so on.
+// W waves per workgroup, OCC waves per SIMD: a workgroup covers W * 32 * NQT queries.
+// ============================================================================================
+constexpr int QS_STAGE_ROWS = 64;
+constexpr int QS_STAGE_BYTES = QS_STAGE_ROWS * 256;
+constexpr int QS_NBUF = 3;
+// VALU instructions of the previous tile's epilogue asked for behind each MFMA (an MFMA takes two of the eight
+// issue slots of its 32 cycles; about 42 epilogue instructions per 8 MFMAs: five per MFMA measured best of 4..8)
+constexpr int QS_VALU_PER_MFMA = 5;
+
+template <template <int> class EpiT, int NQT, int W, int OCC>
+__global__ void __launch_bounds__(64 * W, OCC) qstream_kernel(ContractArgs a, typename EpiT<NQT>::Args ea) {
+  using Epi = EpiT<NQT>;
+  __shared__ __attribute__((aligned(1024))) unsigned char lds_e[QS_NBUF * QS_STAGE_BYTES];
+
+  const int64_t wg = blockIdx.x;
+  const int xcd = (int)(wg & 7);
+  const int64_t slot = wg >> 3;
+  const int qg = (int)(slot % a.n_qgroups);
+  const int wlane = (int)(slot / a.n_qgroups);
+  const int tid = threadIdx.x, lane = tid & 63, c = lane & 31, hf = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  constexpr int d = 128;
+  const int64_t q0 = (int64_t)qg * (W * 32 * NQT) + wave * (32 * NQT);
+
+  // chunks of this workgroup: first, stride, count; stages that hold at least one valid row
+  const int64_t c_first = xcd + 8 * (int64_t)wlane;
+  const int64_t c_stride = 8 * (int64_t)a.n_lanes;
+  if (c_first >= a.n_chunks) return;
+  const int my_chunks = (int)((a.n_chunks - 1 - c_first) / c_stride) + 1;
+  const int spc = a.chunk_rows / QS_STAGE_ROWS;  // stages per chunk
+  const int64_t r_end = a.e_end;
+  const int64_t row_first = a.e_begin + c_first * a.chunk_rows;
+  const int64_t row_last_chunk = row_first + c_stride * (int64_t)(my_chunks - 1) * a.chunk_rows;
+  int valid_last = (int)((r_end - row_last_chunk + QS_STAGE_ROWS - 1) / QS_STAGE_ROWS);
+  valid_last = valid_last < spc ? valid_last : spc;
+  const int n_st = (my_chunks - 1) * spc + valid_last;
+  const int64_t chunk_skip = (c_stride - 1) * (int64_t)a.chunk_rows;
+
+  bf16x8 qf[NQT][8];
+#pragma unroll
+  for (int t = 0; t < NQT; ++t) {
+    const int64_t q = q0 + 32 * t + c;
+#pragma unroll
+    for (int s = 0; s < 8; ++s) {
+      const int k = 16 * s + 8 * hf;
+      f32x4 lo = {0.f, 0.f, 0.f, 0.f}, hi = {0.f, 0.f, 0.f, 0.f};
+      if (q < a.B) {
+        const f32x4* src = (const f32x4*)(a.Q + q * d + k);
+        lo = src[0];
+        hi = src[1];
+      }
+      qf[t][s] = cvt_bf16x8(lo, hi);
+    }
+  }
+  Epi epi;
+  epi.init(ea, q0, c, hf, a.B);
+  __shared__ typename Epi::Shared epi_sh;
+  epi.bind(&epi_sh);
+
+  // this lane's share of a stage: rows lrow + RPI * j, always the same swizzled piece (RPI is a multiple of 16).
+  // A full stage is a scalar base plus per-lane offsets that never change; in the table's last, partial stage the
+  // rows past the end repeat its last row (the epilogues ignore them).
+  constexpr int RPI = 4 * W;
+  constexpr int NLD = QS_STAGE_ROWS / RPI;
+  static_assert(RPI % 16 == 0 && QS_STAGE_ROWS % RPI == 0, "stage / workgroup shape");
+  const int lrow = wave * 4 + (lane >> 4);
+  const int lpiece = (lane & 15) ^ (lrow & 15);
+  const unsigned char* Eb = (const unsigned char*)a.E;
+  uint32_t voff[NLD];
+#pragma unroll
+  for (int j = 0; j < NLD; ++j) voff[j] = (uint32_t)((lrow + RPI * j) * 256 + lpiece * 16);
+  auto stage_issue = [&](int64_t row0, int buf) {
+    unsigned char* dst = lds_e + buf * QS_STAGE_BYTES + wave * 1024;
+    if (__builtin_expect(row0 + QS_STAGE_ROWS <= r_end, 1)) {
+      const unsigned char* src = Eb + row0 * 256;  // wave-uniform
+#pragma unroll
+      for (int j = 0; j < NLD; ++j)
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src + voff[j]),
+                                         (__attribute__((address_space(3))) void*)(dst + j * (RPI * 256)), 16, 0, 0);
+    } else {
+#pragma unroll
+      for (int j = 0; j < NLD; ++j) {
+        int64_t g = row0 + lrow + RPI * j;
+        g = (g < r_end) ? g : r_end - 1;
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(Eb + g * 256 + lpiece * 16),
+                                         (__attribute__((address_space(3))) void*)(dst + j * (RPI * 256)), 16, 0, 0);
+      }
+    }
+  };
+  // the stage the next issue fetches (two ahead of the one being multiplied) and its position in its chunk
+  int64_t issue_row = row_first;
+  int issue_so = 0;
+  auto issue_advance = [&]() {
+    issue_row += QS_STAGE_ROWS;
+    if (++issue_so == spc) {
+      issue_so = 0;
+      issue_row += chunk_skip;
+    }
+  };
+
+  // fragment addresses of this lane inside buffer 0 (row c of entity tile 0)
+  int foff[8];
+#pragma unroll
+  for (int s = 0; s < 8; ++s) foff[s] = c * 256 + (((2 * s + hf) ^ (c & 15)) << 4);
+
+  // the first epilogue has no tile to work on: e_prev past the limit says so to the branching epilogues, scores of
+  // -inf (never greater than, never equal to a threshold) to the deferring one
+  f32x16 acc_prev;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) acc_prev[i] = Epi::DEFER ? __uint_as_float(0xff800000u) : 0.f;
+  float sc_dummy[16];
+#pragma unroll
+  for (int i = 0; i < 16; ++i) sc_dummy[i] = 1.f;
+  int64_t e_prev = r_end;
+
+  // A barrier that orders nothing but the waves: the loads it guards are waited for explicitly, and the
+  // compiler is kept from moving LDS accesses across it.
+  auto wg_barrier = [&]() {
+    __builtin_amdgcn_sched_barrier(0);  // nothing is scheduled across: no epilogue value is kept alive over the wait
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
+  };
+
+  stage_issue(issue_row, 0);
+  issue_advance();
+  stage_issue(issue_row, 1);
+  issue_advance();
+  wg_barrier();
+  bf16x8 ef[8];
+#pragma unroll
+  for (int s = 0; s < 8; ++s) ef[s] = *(const bf16x8*)(lds_e + foff[s]);
+
+  int64_t row0 = row_first, prev_row0 = row_first;
+  int so = 0;
+  // a stage's tiles formed again from its buffer, for the exact pass of a deferring epilogue
+  auto fix_stage = [&](auto bufc, int64_t rows0) {
+    if constexpr (Epi::DEFER) {
+      constexpr int BUF = decltype(bufc)::value;
+      for (int et = 0; et < 2; ++et) {
+#pragma unroll
+        for (int t = 0; t < NQT; ++t) {
+          f32x16 acc;
+#pragma unroll
+          for (int i = 0; i < 16; ++i) acc[i] = 0.f;
+#pragma unroll
+          for (int s = 0; s < 8; ++s) {
+            const bf16x8 f = *(const bf16x8*)(lds_e + BUF * QS_STAGE_BYTES + et * 8192 + foff[s]);
+            acc = mfma_bf16(f, qf[t][s], acc);
+          }
+          epi.tile_slow(t, acc, rows0 + et * 32, r_end);
+        }
+      }
+    }
+  };
+  auto bufc_prev = [](auto bufc) { return std::integral_constant<int, (decltype(bufc)::value + QS_NBUF - 1) % QS_NBUF>{}; };
+  auto run_stage = [&](auto bufc, int k) {
+    constexpr int BUF = decltype(bufc)::value;
+    constexpr int NEXT = (BUF + 1) % QS_NBUF, NEXT2 = (BUF + 2) % QS_NBUF, PREV = NEXT2;
+#pragma unroll
+    for (int et = 0; et < 2; ++et) {
+      if (et == 1) {
+        if constexpr (Epi::DEFER) {
+          // every tile of the previous stage has been through the epilogue by now, and its buffer is intact
+          // until this wave passes the barrier below: the place for that stage's exact pass, if it needs one
+          if (k > 0 && epi.stage_dirty(PREV, prev_row0 + QS_STAGE_ROWS > r_end)) fix_stage(bufc_prev(bufc), prev_row0);
+        }
+        if (Epi::STAGE_HOOK) {
+          epi.stage_mark();
+          asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        }
+        // stage k + 1 has landed for every wave, and everyone is done with the buffer of stage k - 1
+        wg_barrier();
+        if constexpr (Epi::DEFER) epi.touch();
+        if (Epi::STAGE_HOOK) epi.stage_end();
+        // stage k + 2 (past the last stage: the last stage's rows once more, into a buffer nobody reads)
+        stage_issue(issue_row, NEXT2);
+        if (k + 3 < n_st) issue_advance();
+      }
+      // where the next entity tile's fragments come from: the second tile of this stage, or the first of the next
+      const int roff = (et == 0) ? BUF * QS_STAGE_BYTES + 8192 : NEXT * QS_STAGE_BYTES;
+#pragma unroll
+      for (int t = 0; t < NQT; ++t) {
+        const int t_prev = (t + NQT - 1) % NQT;
+        const bool refill = (t == NQT - 1);
+        f32x16 acc;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[i] = 0.f;
+#pragma unroll
+        for (int s = 0; s < 8; ++s) {
+          acc = Epi::SWAP ? mfma_bf16(qf[t][s], ef[s], acc) : mfma_bf16(ef[s], qf[t][s], acc);
+          if (refill) ef[s] = *(const bf16x8*)(lds_e + roff + foff[s]);  // last use of fragment s: fetch its successor
+        }
+        if constexpr (Epi::DEFER) {
+          epi.tile_fast((et == 0 && t == 0) ? PREV : BUF, t_prev, acc_prev);  // the stage the finished tile belongs to
+        } else {
+          epi.template tile<false>(t_prev, acc_prev, sc_dummy, 1.f, e_prev, r_end);
+        }
+        // the order the scheduler is asked for: each MFMA of this chain, then a share of the previous tile's
+        // epilogue, then (in a refilling chain) the read that replaces the fragment the MFMA consumed
+#pragma unroll
+        for (int s = 0; s < 8; ++s) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x002, QS_VALU_PER_MFMA, 0);
+          if (refill) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        }
+        acc_prev = acc;
+        e_prev = row0 + et * 32;
+      }
+    }
+    prev_row0 = row0;
+    row0 += QS_STAGE_ROWS;
+    if (++so == spc) {
+      so = 0;
+      row0 += chunk_skip;
+    }
+  };
+  // after the last stage: the epilogue of its last tile, then (deferring epilogues) its exact pass
+  auto tail = [&](auto bufc) {
+    if constexpr (Epi::DEFER) {
+      constexpr int BUF = decltype(bufc)::value;
+      epi.tile_fast(BUF, NQT - 1, acc_prev);
+      if (epi.stage_dirty(BUF, prev_row0 + QS_STAGE_ROWS > r_end)) fix_stage(bufc, prev_row0);
+    } else {
+      epi.template tile<false>(NQT - 1, acc_prev, sc_dummy, 1.f, e_prev, r_end);
+    }
+  };
+  for (int k = 0;;) {
+    run_stage(std::integral_constant<int, 0>{}, k);
+    if (++k >= n_st) { tail(std::integral_constant<int, 0>{}); break; }
+    run_stage(std::integral_constant<int, 1>{}, k);
+    if (++k >= n_st) { tail(std::integral_constant<int, 1>{}); break; }
+    run_stage(std::integral_constant<int, 2>{}, k);
+    if (++k >= n_st) { tail(std::integral_constant<int, 2>{}); break; }
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // no load may land in LDS after the workgroup has gone
   epi.finish();
 }
 
@@ -1102,6 +1473,7 @@ __global__ void __launch_bounds__(64 * I8_WG_WAVES, 2) qreg_i8_kernel(ContractAr
       }
     }
     if (have_next) stage_store(buf ^ 1);
+    if (Epi::STAGE_HOOK) epi.stage_mark();
     __syncthreads();
     if (Epi::STAGE_HOOK) epi.stage_end();
   }
@@ -1294,6 +1666,7 @@ __global__ void __launch_bounds__(512, 2) ksplit_kernel(ContractArgs a, typename
       }
       kc = 0;
       et0 += KS_TILE_ROWS;
+      if (Epi::STAGE_HOOK) epi.stage_mark();
       __syncthreads();
       if (Epi::STAGE_HOOK) epi.stage_end();
     } else {
@@ -1460,6 +1833,7 @@ __global__ void __launch_bounds__(512, 2) kchunk_bf16_kernel(ContractArgs a, typ
       }
       kc = 0;
       et0 += KS_TILE_ROWS;
+      if (Epi::STAGE_HOOK) epi.stage_mark();
       __syncthreads();
       if (Epi::STAGE_HOOK) epi.stage_end();
     } else {

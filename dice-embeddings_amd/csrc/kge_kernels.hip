@@ -1024,8 +1024,13 @@ int launch_contract(int dtype, const ContractArgs& a, const EArgs& ea, hipStream
     hipLaunchKernelGGL((ksplit_kernel<EpiT, true>), grid, block, 0, st, a, ea);
   else if (f32_split)
     hipLaunchKernelGGL((ksplit_kernel<EpiT, false>), grid, block, 0, st, a, ea);
-  else if (dtype == KGE_BF16 && a.d == 128)
-    hipLaunchKernelGGL((qreg_async_kernel<EpiT>), grid, block, 0, st, a, ea);
+  else if (dtype == KGE_BF16 && a.d == 128) {
+    // the rank epilogue has a branch-free form for the deeper-pipelined kernel (same workgroup shape, same counts)
+    if constexpr (std::is_same<EpiT<2>, RankEpi<2>>::value)
+      hipLaunchKernelGGL((qstream_kernel<RankFastEpi, QA_NQT, QA_WG_WAVES, QA_WAVES_PER_SIMD>), grid, block, 0, st, a, ea);
+    else
+      hipLaunchKernelGGL((qreg_async_kernel<EpiT>), grid, block, 0, st, a, ea);
+  }
   else if (wide_bf16)
     hipLaunchKernelGGL((kchunk_bf16_kernel<EpiT>), grid, block, 0, st, a, ea);
   else if (dtype == KGE_BF16)
