@@ -95,8 +95,10 @@ def main_loop_kernel(storage, d, mode):
            "bcegrad": "GradEpi | StoreEpi", "train": "GradEpi | StoreEpi"}[mode]
     if storage == "fp32":
         return f"ksplit_kernel<{epi}, {'true' if d % 4 == 0 else 'false'}>"
+    if d == 128 and storage == "bf16":
+        return "qstream_kernel<RankFastEpi, 2, 8, 2>" if epi == "RankEpi" else f"qreg_async_kernel<{epi}>"
     if d == 128:
-        return f"qreg_async_kernel<{epi}>" if storage == "bf16" else f"qreg_i8_kernel<{epi}>"
+        return f"qreg_i8_kernel<{epi}>"
     if storage == "bf16" and d > 128:
         return f"kchunk_bf16_kernel<{epi}>"
     return f"qreg_kernel<{storage}, {epi}>"
@@ -117,6 +119,11 @@ def main():
     ap.add_argument("--graph", action="store_true",
                     help="capture one HIP graph per batch before the timed region and replay the graphs (rank, bce and "
                          "bcegrad steps only: the top-k call reads a counter back on the host and cannot be captured)")
+    ap.add_argument("--sustain-seconds", type=float, default=2.0,
+                    help="length of the `sustained` side run (the same step repeated for this long, after the timed "
+                         "region; 0 switches it off)")
+    ap.add_argument("--no-ceiling", action="store_true",
+                    help="skip the `ceiling` side figures (vendor bf16 GEMM on random and on zero operands)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one plain 1 GiB-in / 1 GiB-out elementwise kernel (reference point for "
                          "FETCH_SIZE / WRITE_SIZE counters under rocprofv3 --pmc)")
@@ -153,7 +160,7 @@ def main():
     else:
         batches = [(q_all[i:i + cfg.B, :2].contiguous(), q_all[i:i + cfg.B, 2].contiguous())
                    for i in range(0, len(q_all), cfg.B)]
-    steps = args.steps if args.steps is not None else max(2 * len(batches), 20)
+    steps = args.steps if args.steps is not None else max(10 * len(batches), 100)
     torch.cuda.synchronize()
     t_setup = time.perf_counter() - t_setup
 
@@ -247,12 +254,84 @@ def main():
                         if compute == "fp32" else {}),
                      "traffic": MEASURED_TRAFFIC_BYTES.get(args.config) if mode == MODE[args.config] else None
                      if args.scale == 1.0 and args.mode is None else None,
+                     "traffic_source": "measured offline, not in this run: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on "
+                                       "this workload, scaled by a 1 GiB copy kernel (profiles/*_hbm_traffic.md)",
                      "kernel": main_loop_kernel(cfg.storage, d, mode),
                      "kernel_ms_avg": kernel_ms / max(launches, 1), "launches": launches,
                      "kernel_time_share": kernel_ms * 1e-3 / elapsed},
         "setup_s": t_setup,
         "device": torch.cuda.get_device_name(0),
     }
+    # side figure, outside the timed region: the same step repeated for --sustain-seconds, so that the clock the
+    # chip settles at under its power limit is inside the figure (the timed region above can be as short as 50 ms)
+    if args.sustain_seconds > 0 and not args.graph:
+        per_step = elapsed / steps
+        n_sus = max(steps, int(args.sustain_seconds / max(per_step, 1e-6)))
+        torch.cuda.synchronize()
+        ops.profile_begin()
+        ts = time.perf_counter()
+        nq = 0
+        for i in range(n_sus):
+            step(i)
+            nq += batches[i % len(batches)][0].shape[0]
+        torch.cuda.synchronize()
+        ts = time.perf_counter() - ts
+        k_ms, k_n = ops.profile_end()
+        f_sus = 2.0 * d * float(nq) * N * (3.0 if mode in ("bcegrad", "train") else 1.0)
+        a_sus = f_sus / (k_ms * 1e-3) / 1e12 if k_ms > 0 else None
+        out["sustained"] = {"seconds": ts, "steps": n_sus, "ms_per_step": ts * 1e3 / n_sus,
+                            "value": float(nq) * N / ts, "unit": "scores/s",
+                            "roofline_achieved": a_sus, "roofline_frac": a_sus / PEAK_TFLOPS[compute] if a_sus else None,
+                            "kernel_ms_avg": k_ms / max(k_n, 1), "launches": k_n}
+    # side figures, outside the timed region: what the vendor's bf16 GEMM (torch.matmul -> hipBLASLt) sustains on this
+    # box, on random and on all-zero operands (the gap is the power limit: random data toggles more), and at the
+    # workload's own shape, where it has to write the B x N score matrix that the fused kernels never form
+    if not args.no_ceiling and compute == "bf16" and args.scale == 1.0:
+        def gemm_rate(a_, b_, out_, seconds=0.7):
+            for _ in range(3):
+                torch.matmul(a_, b_, out=out_)
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            t0_, n_ = time.perf_counter(), 0
+            e0.record()
+            while True:
+                for _ in range(5):
+                    torch.matmul(a_, b_, out=out_)
+                n_ += 5
+                torch.cuda.synchronize()
+                if time.perf_counter() - t0_ > seconds:
+                    break
+            e1.record()
+            torch.cuda.synchronize()
+            ms = e0.elapsed_time(e1) / n_
+            return 2.0 * a_.shape[0] * a_.shape[1] * b_.shape[1] / (ms * 1e-3) / 1e12, ms
+        ceil = {"unit": "TFLOP/s", "peak": PEAK_TFLOPS["bf16"]}
+        g = torch.Generator(device=dev)
+        g.manual_seed(1234)
+        n_sq = 8192
+        A = torch.randn((n_sq, n_sq), device=dev, generator=g).to(torch.bfloat16)
+        Bm = torch.randn((n_sq, n_sq), device=dev, generator=g).to(torch.bfloat16)
+        C = torch.empty((n_sq, n_sq), device=dev, dtype=torch.bfloat16)
+        r, ms = gemm_rate(A, Bm, C)
+        ceil["torch_matmul_bf16_8192_cubed_randn"] = {"achieved": r, "frac": r / PEAK_TFLOPS["bf16"], "ms": ms}
+        A.zero_()
+        Bm.zero_()
+        r, ms = gemm_rate(A, Bm, C)
+        ceil["torch_matmul_bf16_8192_cubed_zeros"] = {"achieved": r, "frac": r / PEAK_TFLOPS["bf16"], "ms": ms}
+        del A, Bm, C
+        if d == 128:
+            E_t, _ = model.table()
+            if E_t.dtype == torch.bfloat16:
+                Bq = batches[0][0].shape[0]
+                Qb = torch.randn((Bq, d), device=dev, generator=g).to(torch.bfloat16)
+                S_out = torch.empty((Bq, N), device=dev, dtype=torch.bfloat16)
+                r, ms = gemm_rate(Qb, E_t.t(), S_out)
+                ceil["torch_matmul_bf16_workload_shape"] = {
+                    "achieved": r, "frac": r / PEAK_TFLOPS["bf16"], "ms": ms, "shape": [Bq, d, N],
+                    "note": "writes the B x N score matrix (bf16) that the fused kernel never forms"}
+                del Qb, S_out
+        out["ceiling"] = ceil
+        torch.cuda.empty_cache()
     # side figure, outside the timed region: the gather + interaction kernel alone (HBM-bound, launch-latency sized)
     xg = batches[0][0]
     for _ in range(3):
