@@ -503,7 +503,7 @@ struct TopkEpi {
   }
 };
 
-constexpr int BCE_SLOTS = 128;  // the accumulator is spread: same-address double atomics serialise
+using host::BCE_SLOTS;  // the accumulator is spread: same-address double atomics serialise
 struct BceArgs {
   const float* bias;
   double* sums;  // [0, BCE_SLOTS) partial sums of softplus(s), [BCE_SLOTS, 2 BCE_SLOTS) partial sums of s
@@ -1491,8 +1491,8 @@ __global__ void __launch_bounds__(64 * I8_WG_WAVES, 2) qreg_i8_kernel(ContractAr
 // r*4 + (p ^ ((r >> 2) & 3)), so the 16 rows a fragment read touches at a time spread over all banks.
 // ============================================================================================
 constexpr int KS_NQT = 2;
-constexpr int KS_WG_QUERIES = 128;
-constexpr int KS_TILE_ROWS = 256;
+using host::KS_WG_QUERIES;
+using host::KS_TILE_ROWS;
 constexpr int KS_KC = 32;
 constexpr int KS_E_PLANE = KS_TILE_ROWS * 64;
 constexpr int KS_Q_PLANE = KS_WG_QUERIES * 64;

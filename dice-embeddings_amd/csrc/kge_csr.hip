@@ -19,12 +19,6 @@
 namespace kge {
 namespace {
 
-inline int bits_for(int64_t range) {  // bits needed for values in [0, range)
-  int b = 1;
-  while (b < 63 && (1LL << b) < range) ++b;
-  return b;
-}
-
 struct CsrWs {
   unsigned long long* key_in;
   unsigned long long* key_sorted;
@@ -35,7 +29,7 @@ struct CsrWs {
   size_t scan_tmp_bytes;
 };
 
-inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+using host::align_up;
 
 // Returns the total size, or 0 when rocPRIM cannot size its temporaries (no device).
 size_t csr_ws_layout(int64_t n, void* base, CsrWs* ws, hipStream_t st) {
@@ -75,7 +69,7 @@ __global__ void __launch_bounds__(256) csr_pack_kernel(const int64_t* __restrict
   for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
     const int64_t a = triples[3 * i + col_a], b = triples[3 * i + col_b], v = triples[3 * i + col_v];
     const bool ok = a >= 0 && a < range_a && b >= 0 && b < range_b && v >= 0 && v < range_v;
-    key[i] = ok ? ((unsigned long long)(a * range_b + b) << vbits) | (unsigned long long)v : invalid;
+    key[i] = ok ? host::csr_pack_key(a, b, v, range_b, vbits) : invalid;
   }
 }
 
@@ -159,18 +153,10 @@ extern "C" int kge_csr_build(const int64_t* triples, int64_t n, int col_a, int c
                              int64_t range_b, int64_t range_v, int64_t* keys, int64_t* row_ptr, int32_t* col,
                              int64_t* counts, void* workspace, size_t workspace_bytes, void* stream) {
   clear_error();
-  KGE_REQUIRE(n >= 0 && n < (1LL << 31), KGE_ERR_INVALID, "kge_csr_build: n=%lld outside [0, 2^31)", (long long)n);
-  KGE_REQUIRE(col_a >= 0 && col_a < 3 && col_b >= 0 && col_b < 3 && col_v >= 0 && col_v < 3 && col_a != col_b &&
-                  col_a != col_v && col_b != col_v,
-              KGE_ERR_INVALID, "kge_csr_build: columns (%d, %d, %d) are not a permutation of 0..2", col_a, col_b, col_v);
-  KGE_REQUIRE(range_a >= 1 && range_b >= 1 && range_v >= 1 && range_v <= (1LL << 31), KGE_ERR_INVALID,
-              "kge_csr_build: ranges (%lld, %lld, %lld) must be positive and values fit int32", (long long)range_a,
-              (long long)range_b, (long long)range_v);
-  const int vbits = bits_for(range_v);
-  const int key_bits = bits_for(range_a) + bits_for(range_b) + vbits;  // a * range_b + b < 2^(bits_a + bits_b)
-  KGE_REQUIRE(key_bits <= 62, KGE_ERR_UNSUPPORTED,
-              "kge_csr_build: (%lld x %lld) pairs x %lld values do not fit a 62-bit key", (long long)range_a,
-              (long long)range_b, (long long)range_v);
+  const host::Status rules = host::csr_build_rules(n, col_a, col_b, col_v, range_a, range_b, range_v);
+  if (!rules.ok()) return set_error(rules.code, "%s", rules.msg);
+  const host::CsrKeyLayout layout = host::csr_key_layout(range_a, range_b, range_v);
+  const int vbits = layout.vbits, key_bits = layout.key_bits;
   KGE_REQUIRE(row_ptr && counts, KGE_ERR_INVALID, "kge_csr_build: null row_ptr or counts");
   hipStream_t st = (hipStream_t)stream;
   if (n == 0) {
@@ -186,7 +172,7 @@ extern "C" int kge_csr_build(const int64_t* triples, int64_t n, int col_a, int c
               workspace_bytes, need);
   KGE_REQUIRE(((uintptr_t)workspace & 7) == 0, KGE_ERR_WORKSPACE, "kge_csr_build: workspace must be 8-byte aligned");
   const unsigned grid = (unsigned)((n + 255) / 256 < 4096 ? (n + 255) / 256 : 4096);
-  const unsigned long long invalid = 1ull << key_bits;
+  const unsigned long long invalid = layout.invalid;
   hipLaunchKernelGGL(csr_pack_kernel, dim3(grid), dim3(256), 0, st, triples, n, col_a, col_b, col_v, range_a, range_b,
                      range_v, vbits, invalid, ws.key_in);
   KGE_LAUNCH_CHECK("csr_pack_kernel");

@@ -1,0 +1,335 @@
+// Host-side logic of the library that needs no GPU: argument rules, workspace layouts, the packed keys and
+// counters the kernels exchange, and a sequential model of the kernel that plans the filter correction.
+//
+// Plain C++17 with no HIP dependency: hipcc includes it into the device library, and g++ builds it (with
+// -fsanitize=address,undefined) into the CPU test driver tests/host_model_test.cpp, so that every layout and
+// every packed field is exercised with bounds checks where there is no GPU.
+#pragma once
+#include <stddef.h>
+#include <stdint.h>
+#include <stdio.h>
+
+#include <vector>
+
+#include "../../include/kge_hip.h"
+
+#if defined(__HIPCC__)
+#define KGE_HD __host__ __device__
+#else
+#define KGE_HD
+#endif
+
+namespace kge {
+namespace host {
+
+// ---- sizes shared by host and kernels -------------------------------------------------------------------
+constexpr int SORT_MAX = 8192;           // queries per sub-batch of the filter correction
+constexpr int WORK_MAX = 16 * SORT_MAX;  // upper bound on work items per sub-batch (bounds the slice count only)
+constexpr int SLICE_MIN = 128;           // shortest slice of a filter row
+constexpr int PLAN_SLOTS = 2 * SORT_MAX; // hash table of the plan kernel: load factor <= 0.5
+constexpr int PLAN_HASH_SHIFT = 18;      // 32 - log2(PLAN_SLOTS)
+static_assert(PLAN_SLOTS == (1 << (32 - PLAN_HASH_SHIFT)), "hash width");
+constexpr int TOPK_CAP = 4096;           // candidates a query can collect in one round
+constexpr int TOPK_MAX_K = 1024;
+constexpr int TOPK_FIRST_ROWS = 1024;    // first round takes everything: must not exceed TOPK_CAP
+constexpr int BCE_SLOTS = 128;
+constexpr int KS_WG_QUERIES = 128;       // workgroup shape of the fp32 contraction (also sizes the backward's K split)
+constexpr int KS_TILE_ROWS = 256;
+
+struct Status {
+  int code = KGE_OK;
+  char msg[256] = "";
+  bool ok() const { return code == KGE_OK; }
+};
+#define KGE_HOST_FAIL(st, c, ...)                      \
+  do {                                                 \
+    (st).code = (c);                                   \
+    snprintf((st).msg, sizeof((st).msg), __VA_ARGS__); \
+    return (st);                                       \
+  } while (0)
+
+inline size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
+
+// ---- argument rules of every contraction entry point ---------------------------------------------------
+inline Status contract_rules(const char* who, const void* Q, const void* E, int dtype, const void* scale, int64_t B,
+                             int64_t d, int64_t N) {
+  Status st;
+  if (!(B >= 0 && N >= 1)) KGE_HOST_FAIL(st, KGE_ERR_INVALID, "%s: B=%lld N=%lld", who, (long long)B, (long long)N);
+  if (N > 0x7fffffffLL) KGE_HOST_FAIL(st, KGE_ERR_INVALID, "%s: N=%lld exceeds int32 entity ids", who, (long long)N);
+  if (B > (1 << 24)) KGE_HOST_FAIL(st, KGE_ERR_INVALID, "%s: B=%lld exceeds 2^24", who, (long long)B);
+  if (!(B == 0 || (Q && E))) KGE_HOST_FAIL(st, KGE_ERR_INVALID, "%s: null Q or E", who);
+  if ((((uintptr_t)Q | (uintptr_t)E) & 15) != 0)
+    KGE_HOST_FAIL(st, KGE_ERR_INVALID, "%s: Q and E must be 16-byte aligned", who);
+  switch (dtype) {
+    case KGE_F32:
+      if (!(d >= 1 && d <= 65536)) KGE_HOST_FAIL(st, KGE_ERR_INVALID, "%s: d=%lld", who, (long long)d);
+      break;
+    case KGE_BF16:
+      if (!(d >= 8 && d % 8 == 0))
+        KGE_HOST_FAIL(st, KGE_ERR_INVALID, "%s: bf16 tables need d %% 8 == 0, got %lld", who, (long long)d);
+      if (d > 65536) KGE_HOST_FAIL(st, KGE_ERR_INVALID, "%s: d=%lld", who, (long long)d);
+      break;
+    case KGE_I8:
+      if (!(d >= 16 && d % 16 == 0))
+        KGE_HOST_FAIL(st, KGE_ERR_INVALID, "%s: int8 tables need d %% 16 == 0, got %lld", who, (long long)d);
+      if (d > 128) KGE_HOST_FAIL(st, KGE_ERR_UNSUPPORTED, "%s: int8 tables support d <= 128, got %lld", who, (long long)d);
+      if (!scale) KGE_HOST_FAIL(st, KGE_ERR_INVALID, "%s: int8 tables need per-row scales", who);
+      break;
+    default: KGE_HOST_FAIL(st, KGE_ERR_INVALID, "%s: unknown dtype %d", who, dtype);
+  }
+  return st;
+}
+
+// ---- workspace layouts ------------------------------------------------------------------------------------
+struct RankWsOffsets {
+  size_t thr, skey, gend, work, meta, total;
+};
+inline RankWsOffsets rank_ws_offsets(int64_t B) {
+  RankWsOffsets o{};
+  size_t off = 0;
+  auto take = [&](size_t bytes) {
+    const size_t at = off;
+    off = align_up(off + bytes, 256);
+    return at;
+  };
+  o.thr = take((size_t)B * 4);
+  o.skey = take((size_t)SORT_MAX * 8);
+  o.gend = take((size_t)SORT_MAX * 4);
+  o.work = take((size_t)SORT_MAX * 8);
+  o.meta = take(16);
+  o.total = off;
+  return o;
+}
+
+struct TopkWsOffsets {
+  size_t tau, cnt, list_len, dirty, n_dirty, list, cand, total;
+  int64_t kpad;
+};
+inline TopkWsOffsets topk_ws_offsets(int64_t B, int64_t k) {
+  TopkWsOffsets o{};
+  size_t off = 0;
+  auto take = [&](size_t bytes) {
+    const size_t at = off;
+    off = align_up(off + bytes, 256);
+    return at;
+  };
+  o.kpad = (k + 7) / 8 * 8;
+  o.tau = take((size_t)B * 4);
+  o.cnt = take((size_t)B * 4);
+  o.list_len = take((size_t)B * 4);
+  o.dirty = take((size_t)B * 4);
+  o.n_dirty = take(4);
+  o.list = take((size_t)B * (size_t)o.kpad * 8);
+  o.cand = take((size_t)B * TOPK_CAP * 8);
+  o.total = off;
+  return o;
+}
+
+inline size_t bce_ws_bytes() { return (2 * BCE_SLOTS + 1) * sizeof(double) + 248; }
+
+struct BwdPlan {
+  int64_t ldG, ldT;  // row strides of G [B, ldG] and GT [N, ldT] (multiples of 4)
+  int k_splits, k_split_len;
+  size_t off_G, off_GT, off_ET, off_QT, off_part, total;
+};
+inline BwdPlan bwd_plan(int64_t B, int64_t d, int64_t N) {
+  BwdPlan p{};
+  p.ldG = (N + 3) / 4 * 4;
+  p.ldT = (B + 3) / 4 * 4;
+  // dQ = G . E sums over N: split so that about 256 workgroups run
+  const int64_t tiles = ((B + KS_WG_QUERIES - 1) / KS_WG_QUERIES) * ((d + KS_TILE_ROWS - 1) / KS_TILE_ROWS);
+  int64_t splits = (256 + tiles - 1) / tiles;
+  if (splits > 64) splits = 64;
+  if (splits < 1) splits = 1;
+  const int64_t len = ((N + splits - 1) / splits + 31) / 32 * 32;
+  p.k_split_len = (int)len;
+  p.k_splits = (int)((N + len - 1) / len);
+  auto up = [](size_t x) { return (x + 255) / 256 * 256; };
+  size_t off = up(bce_ws_bytes());
+  p.off_G = off;     off += up((size_t)B * p.ldG * sizeof(float));
+  p.off_GT = off;    off += up((size_t)N * p.ldT * sizeof(float));
+  p.off_ET = off;    off += up((size_t)d * p.ldG * sizeof(float));
+  p.off_QT = off;    off += up((size_t)d * p.ldT * sizeof(float));
+  p.off_part = off;  off += up((size_t)p.k_splits * B * d * sizeof(float));
+  p.total = off;
+  return p;
+}
+
+// ---- vocabulary keys: ((a * range_b + b) << vbits) | v ----------------------------------------------------
+KGE_HD inline int bits_for(int64_t range) {  // bits needed for values in [0, range)
+  int b = 1;
+  while (b < 63 && (1LL << b) < range) ++b;
+  return b;
+}
+struct CsrKeyLayout {
+  int vbits, key_bits;
+  bool fits;                   // key_bits <= 62: room for the `invalid` marker one bit above every valid key
+  unsigned long long invalid;  // key of a triple with an id outside its range (sorts last)
+};
+KGE_HD inline CsrKeyLayout csr_key_layout(int64_t range_a, int64_t range_b, int64_t range_v) {
+  CsrKeyLayout l;
+  l.vbits = bits_for(range_v);
+  l.key_bits = bits_for(range_a) + bits_for(range_b) + l.vbits;  // a * range_b + b < 2^(bits_a + bits_b)
+  l.fits = l.key_bits <= 62;
+  l.invalid = l.fits ? 1ull << l.key_bits : 0ull;
+  return l;
+}
+KGE_HD inline unsigned long long csr_pack_key(int64_t a, int64_t b, int64_t v, int64_t range_b, int vbits) {
+  return ((unsigned long long)(a * range_b + b) << vbits) | (unsigned long long)v;
+}
+inline Status csr_build_rules(int64_t n, int col_a, int col_b, int col_v, int64_t range_a, int64_t range_b,
+                              int64_t range_v) {
+  Status st;
+  if (!(n >= 0 && n < (1LL << 31))) KGE_HOST_FAIL(st, KGE_ERR_INVALID, "kge_csr_build: n=%lld outside [0, 2^31)", (long long)n);
+  if (!(col_a >= 0 && col_a < 3 && col_b >= 0 && col_b < 3 && col_v >= 0 && col_v < 3 && col_a != col_b &&
+        col_a != col_v && col_b != col_v))
+    KGE_HOST_FAIL(st, KGE_ERR_INVALID, "kge_csr_build: columns (%d, %d, %d) are not a permutation of 0..2", col_a, col_b,
+                  col_v);
+  if (!(range_a >= 1 && range_b >= 1 && range_v >= 1 && range_v <= (1LL << 31)))
+    KGE_HOST_FAIL(st, KGE_ERR_INVALID, "kge_csr_build: ranges (%lld, %lld, %lld) must be positive and values fit int32",
+                  (long long)range_a, (long long)range_b, (long long)range_v);
+  if (!csr_key_layout(range_a, range_b, range_v).fits)
+    KGE_HOST_FAIL(st, KGE_ERR_UNSUPPORTED, "kge_csr_build: (%lld x %lld) pairs x %lld values do not fit a 62-bit key",
+                  (long long)range_a, (long long)range_b, (long long)range_v);
+  return st;
+}
+
+// ---- the plan of the filter correction --------------------------------------------------------------------
+// A sub-batch of at most SORT_MAX queries is grouped by filter row; every group's row is cut into slices of
+// `slice` entries, one work item each.  One exclusive scan over the group leaders carries three counters in
+// one 64-bit word: groups (bits 48..63), members (bits 32..47), slices (bits 0..31).  All three stay inside
+// their fields: at most SORT_MAX groups and members, and at most WORK_MAX slices (plan_slice_length).
+KGE_HD inline uint32_t plan_hash(int64_t row) { return ((uint32_t)row * 2654435761u) >> PLAN_HASH_SHIFT; }
+KGE_HD inline unsigned long long plan_pack(unsigned long long members, unsigned long long slices) {
+  return (1ull << 48) | (members << 32) | slices;
+}
+KGE_HD inline int plan_groups(unsigned long long v) { return (int)(v >> 48); }
+KGE_HD inline int plan_members(unsigned long long v) { return (int)((v >> 32) & 0xffffull); }
+KGE_HD inline unsigned int plan_slices(unsigned long long v) { return (unsigned int)(v & 0xffffffffull); }
+// slice length for a sub-batch whose groups' rows hold `total` entries together: at least SLICE_MIN, a multiple
+// of 32, and long enough that sum over groups of ceil(len / slice) <= total / slice + SORT_MAX <= WORK_MAX
+KGE_HD inline int plan_slice_length(unsigned long long total) {
+  const unsigned long long room = (unsigned long long)(WORK_MAX - SORT_MAX);
+  unsigned long long sl = (total + room - 1) / room;
+  sl = (sl + 31) & ~31ull;
+  if (sl < (unsigned long long)SLICE_MIN) sl = SLICE_MIN;
+  return (int)(sl > 0x7fffffe0ull ? 0x7fffffe0ull : sl);
+}
+// member key of the plan: filter row << 24 | position of the query in its sub-batch
+KGE_HD inline unsigned long long plan_member_key(int64_t row, int pos_in_batch) {
+  return ((unsigned long long)row << 24) | (unsigned long long)pos_in_batch;
+}
+KGE_HD inline int64_t plan_key_row(unsigned long long key) { return (int64_t)(key >> 24); }
+KGE_HD inline int plan_key_pos(unsigned long long key) { return (int)(key & 0xffffffull); }
+
+// What plan_fix_kernel writes, computed sequentially in the kernel's own order (thread t owns the queries
+// t, t + 1024, ...; the scan runs over threads, then over a thread's queries).  Every index and every packed
+// field is checked; `error` names the first violation.
+struct PlanModel {
+  std::vector<unsigned long long> skey;
+  std::vector<int32_t> gend, work;
+  int32_t meta[3] = {0, 0, 0};
+  const char* error = nullptr;
+};
+inline PlanModel plan_fix_model(const int64_t* csr_row, int nb, int64_t n_rows, const int64_t* row_ptr) {
+  PlanModel m;
+  m.skey.assign(SORT_MAX, ~0ull);
+  m.gend.assign(SORT_MAX, -1);
+  m.work.assign(2 * SORT_MAX, -1);
+  auto fail = [&](const char* what) {
+    if (!m.error) m.error = what;
+  };
+  if (nb < 0 || nb > SORT_MAX) {
+    fail("sub-batch larger than SORT_MAX");
+    return m;
+  }
+  constexpr int THREADS = 1024, QPT = SORT_MAX / THREADS;
+  std::vector<int32_t> tab_row(PLAN_SLOTS, 0), tab_cnt(PLAN_SLOTS, 0);
+  std::vector<int64_t> my_row(SORT_MAX, -1), len(SORT_MAX, 0);
+  std::vector<int> my_slot(SORT_MAX, -1), my_pos(SORT_MAX, -1);
+  for (int i = 0; i < nb; ++i) {
+    const int64_t r = csr_row[i];
+    my_row[i] = (r >= 0 && r < n_rows) ? r : -1;
+  }
+  // (1) claim slots, take tickets (any interleaving of the threads gives the same groups; tickets differ)
+  for (int i = 0; i < nb; ++i) {
+    if (my_row[i] < 0) continue;
+    if (my_row[i] + 1 > 0x7fffffffLL) fail("filter row + 1 does not fit the 32-bit slot key");
+    const int32_t key = (int32_t)my_row[i] + 1;
+    uint32_t h = plan_hash(my_row[i]);
+    int probes = 0;
+    for (;;) {
+      if (h >= (uint32_t)PLAN_SLOTS) fail("hash outside the table");
+      if (tab_row[h] == 0) tab_row[h] = key;
+      if (tab_row[h] == key) break;
+      h = (h + 1) & (PLAN_SLOTS - 1);
+      if (++probes > PLAN_SLOTS) {
+        fail("hash table full");
+        return m;
+      }
+    }
+    my_slot[i] = (int)h;
+    my_pos[i] = tab_cnt[h]++;
+  }
+  unsigned long long total = 0;
+  for (int i = 0; i < nb; ++i)
+    if (my_pos[i] == 0) {
+      const int64_t l = row_ptr[my_row[i] + 1] - row_ptr[my_row[i]];
+      if (l < 0) fail("row_ptr not ascending");
+      len[i] = l;
+      total += (unsigned long long)l;
+    }
+  // (2) slice length
+  const int slice = plan_slice_length(total);
+  if (slice < SLICE_MIN || slice % 32 != 0) fail("slice length");
+  // (3) exclusive scan of the packed counters in the kernel's order
+  unsigned long long base = 0;
+  for (int t = 0; t < THREADS; ++t)
+    for (int j = 0; j < QPT; ++j) {
+      const int i = t + THREADS * j;
+      if (i >= nb || my_pos[i] != 0) continue;
+      const unsigned long long n = (unsigned long long)((len[i] + slice - 1) / slice);
+      if (n == 0) {
+        tab_cnt[my_slot[i]] = -1;  // empty filter row: nothing to take out for this group
+        continue;
+      }
+      if (n > 0xffffffffull) fail("slices of one group overflow 32 bits");
+      const unsigned long long members = (unsigned long long)tab_cnt[my_slot[i]];
+      if (members > 0xffffull) fail("members of one group overflow their 16-bit field");
+      const unsigned long long val = plan_pack(members, n);
+      const int g = plan_groups(base), first = plan_members(base);
+      if (g < 0 || g >= SORT_MAX) fail("group index outside the plan");
+      if (first < 0 || first + (int)members > SORT_MAX) fail("member positions outside the plan");
+      if (m.error) return m;
+      m.work[2 * g] = first;
+      m.work[2 * g + 1] = (int32_t)plan_slices(base);
+      m.gend[first] = first + (int)members;
+      tab_cnt[my_slot[i]] = first;
+      const unsigned long long next = base + val;
+      if (plan_groups(next) != g + 1 || plan_members(next) != first + (int)members ||
+          (unsigned long long)plan_slices(next) != (unsigned long long)plan_slices(base) + n)
+        fail("a packed counter carried into its neighbour");
+      base = next;
+    }
+  m.meta[0] = (int32_t)plan_slices(base);
+  m.meta[1] = slice;
+  m.meta[2] = plan_groups(base);
+  if ((unsigned long long)plan_slices(base) > (unsigned long long)WORK_MAX) fail("more work items than WORK_MAX");
+  // (4) members to their positions
+  for (int i = 0; i < nb; ++i) {
+    if (my_slot[i] < 0) continue;
+    const int first = tab_cnt[my_slot[i]];
+    if (first < 0) continue;
+    const int at = first + my_pos[i];
+    if (at < 0 || at >= SORT_MAX) {
+      fail("member written outside the plan");
+      return m;
+    }
+    m.skey[at] = plan_member_key(my_row[i], i);
+    if (plan_key_row(m.skey[at]) != my_row[i] || plan_key_pos(m.skey[at]) != i) fail("member key does not round-trip");
+  }
+  return m;
+}
+
+}  // namespace host
+}  // namespace kge

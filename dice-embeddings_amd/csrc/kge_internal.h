@@ -7,6 +7,7 @@
 #include <type_traits>
 
 #include "../../include/kge_hip.h"
+#include "kge_host.h"
 
 namespace kge {
 

@@ -204,10 +204,8 @@ __global__ void csr_lookup_kernel(const int64_t* hr, int64_t B, const int64_t* k
 // queries of the sub-batch that share a filter row (= the same (head, relation) pair, hence the
 // same query vector); work item w is slice w - first of the group found by binary search in the
 // group records.
-constexpr int SORT_MAX = 8192;           // queries per sub-batch
-constexpr int WORK_MAX = 16 * SORT_MAX;  // upper bound on work items per sub-batch (bounds the slice count only)
-constexpr int SLICE_MIN = 128;
-constexpr int PLAN_SLOTS = 2 * SORT_MAX;  // hash table size: load factor <= 0.5
+using host::SORT_MAX;    // queries per sub-batch
+using host::PLAN_SLOTS;  // hash table size: load factor <= 0.5
 
 struct FixPlan {
   unsigned long long* skey;  // [SORT_MAX] csr_row << 24 | position in sub-batch, the members of a group adjacent
@@ -248,8 +246,7 @@ __global__ void __launch_bounds__(1024) plan_fix_kernel(const int64_t* csr_row, 
     my_pos[j] = -1;
     if (my_row[j] >= 0) {
       const int32_t key = (int32_t)my_row[j] + 1;
-      uint32_t h = ((uint32_t)my_row[j] * 2654435761u) >> 18;  // top 14 bits: PLAN_SLOTS = 2^14
-      static_assert(PLAN_SLOTS == (1 << 14), "hash width");
+      uint32_t h = host::plan_hash(my_row[j]);
       for (;;) {
         const int32_t old = atomicCAS(&tab_row[h], 0, key);
         if (old == 0 || old == key) break;
@@ -273,13 +270,7 @@ __global__ void __launch_bounds__(1024) plan_fix_kernel(const int64_t* csr_row, 
   if (my_total) atomicAdd(&s_total, my_total);
   __syncthreads();
   // (2) slice length: at least SLICE_MIN, large enough that extra slices fit the work list
-  if (tid == 0) {
-    const unsigned long long room = (unsigned long long)(WORK_MAX - SORT_MAX);
-    unsigned long long sl = (s_total + room - 1) / room;
-    sl = (sl + 31) & ~31ull;
-    if (sl < SLICE_MIN) sl = SLICE_MIN;
-    s_slice = (int)(sl > 0x7fffffe0ull ? 0x7fffffe0ull : sl);
-  }
+  if (tid == 0) s_slice = host::plan_slice_length(s_total);
   __syncthreads();
   const int slice = s_slice;
   // (3) per leader with work: groups (bits 48..), members (bits 32..47), slices (bits 0..31)
@@ -288,7 +279,7 @@ __global__ void __launch_bounds__(1024) plan_fix_kernel(const int64_t* csr_row, 
 #pragma unroll
   for (int j = 0; j < QPT; ++j) {
     const unsigned long long n = (unsigned long long)((len[j] + slice - 1) / slice);  // an empty row needs no work
-    val[j] = (n > 0) ? ((1ull << 48) | ((unsigned long long)tab_cnt[my_slot[j]] << 32) | n) : 0;
+    val[j] = (n > 0) ? host::plan_pack((unsigned long long)tab_cnt[my_slot[j]], n) : 0;
     local += val[j];
   }
   part[tid] = local;
@@ -303,9 +294,9 @@ __global__ void __launch_bounds__(1024) plan_fix_kernel(const int64_t* csr_row, 
 #pragma unroll
   for (int j = 0; j < QPT; ++j) {
     if (val[j]) {
-      const int g = (int)(base >> 48), first = (int)((base >> 32) & 0xffffull);
+      const int g = host::plan_groups(base), first = host::plan_members(base);
       plan.work[2 * g] = first;
-      plan.work[2 * g + 1] = (int)(base & 0xffffffffull);
+      plan.work[2 * g + 1] = (int)host::plan_slices(base);
       plan.gend[first] = first + tab_cnt[my_slot[j]];
       tab_cnt[my_slot[j]] = first;  // only this leader reads or writes its group's slot in this phase
     } else if (my_pos[j] == 0) {
@@ -314,9 +305,9 @@ __global__ void __launch_bounds__(1024) plan_fix_kernel(const int64_t* csr_row, 
     base += val[j];
   }
   if (tid == 1023) {
-    plan.meta[0] = (int)(part[1023] & 0xffffffffull);
+    plan.meta[0] = (int)host::plan_slices(part[1023]);
     plan.meta[1] = slice;
-    plan.meta[2] = (int)(part[1023] >> 48);
+    plan.meta[2] = host::plan_groups(part[1023]);
   }
   __syncthreads();
   // (4) members to their positions
@@ -325,7 +316,7 @@ __global__ void __launch_bounds__(1024) plan_fix_kernel(const int64_t* csr_row, 
     if (my_slot[j] >= 0) {
       const int first = tab_cnt[my_slot[j]];
       if (first >= 0)
-        plan.skey[first + my_pos[j]] = ((unsigned long long)my_row[j] << 24) | (unsigned long long)(tid + 1024 * j);
+        plan.skey[first + my_pos[j]] = host::plan_member_key(my_row[j], tid + 1024 * j);
     }
   }
 }
@@ -372,7 +363,7 @@ __global__ void __launch_bounds__(256) filter_fix_kernel(ContractArgs a, FixPlan
         const int i0 = plan.work[2 * lo];
         const int64_t z = w - plan.work[2 * lo + 1];
         const unsigned long long key = plan.skey[i0];
-        const int64_t row = (int64_t)(key >> 24);
+        const int64_t row = host::plan_key_row(key);
         const int64_t L0 = row_ptr[row], L1 = row_ptr[row + 1];
         const int64_t z0 = L0 + z * slice;
         it_i0[tid] = i0;
@@ -395,7 +386,7 @@ __global__ void __launch_bounds__(256) filter_fix_kernel(ContractArgs a, FixPlan
     }
     // one round per distinct query vector of the group; `lead` is the first member not yet served
     for (int lead = 0; lead < m;) {
-      const int64_t bq = b0 + (int64_t)(plan.skey[i0 + lead] & 0xffffffull);
+      const int64_t bq = b0 + (int64_t)host::plan_key_pos(plan.skey[i0 + lead]);
       if (m > 1) {
         // members whose query vector equals the leader's, bit for bit, join this round
         __syncthreads();
@@ -406,7 +397,7 @@ __global__ void __launch_bounds__(256) filter_fix_kernel(ContractArgs a, FixPlan
           const int mi = mbase + mslot;
           bool same = true;
           if (mi < m && s_state[mi] == 0 && mi != lead) {
-            const uint32_t* qm = (const uint32_t*)(a.Q + (b0 + (int64_t)(plan.skey[i0 + mi] & 0xffffffull)) * a.d);
+            const uint32_t* qm = (const uint32_t*)(a.Q + (b0 + (int64_t)host::plan_key_pos(plan.skey[i0 + mi])) * a.d);
             for (int k = sub; k < a.d; k += tpm) same = same && (qm[k] == ql[k]);
           }
           // all threads of a member agree before anyone writes its state
@@ -472,7 +463,7 @@ __global__ void __launch_bounds__(256) filter_fix_kernel(ContractArgs a, FixPlan
           __syncthreads();
           int64_t b = 0;
           if (mine) {
-            b = b0 + (int64_t)(plan.skey[i0 + mi] & 0xffffffull);
+            b = b0 + (int64_t)host::plan_key_pos(plan.skey[i0 + mi]);
             const float th = thr[b];
             const int64_t t = target[b];
             int32_t g = 0, eq = 0, eql = 0;
@@ -520,9 +511,9 @@ __global__ void __launch_bounds__(256) filter_fix_kernel(ContractArgs a, FixPlan
 }
 
 // ---- top-k bookkeeping ------------------------------------------------------------------------
-constexpr int TOPK_CAP = 4096;      // candidates a query can collect in one round
-constexpr int TOPK_MAX_K = 1024;
-constexpr int TOPK_FIRST_ROWS = 1024;  // first round takes everything: must not exceed TOPK_CAP
+using host::TOPK_CAP;         // candidates a query can collect in one round
+using host::TOPK_MAX_K;
+using host::TOPK_FIRST_ROWS;  // first round takes everything: must not exceed TOPK_CAP
 
 struct TopkWs {
   float* tau;
@@ -535,30 +526,20 @@ struct TopkWs {
   int64_t kpad;
 };
 
-static size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
-
 size_t topk_ws_layout(int64_t B, int64_t k, void* base, TopkWs* ws) {
-  size_t off = 0;
-  char* p = (char*)base;
-  const int64_t kpad = (k + 7) / 8 * 8;
-  auto take = [&](size_t bytes) {
-    size_t o = off;
-    off = align_up(off + bytes, 256);
-    return o;
-  };
-  size_t o_tau = take(B * 4), o_cnt = take(B * 4), o_len = take(B * 4), o_dirty = take(B * 4), o_nd = take(4);
-  size_t o_list = take((size_t)B * kpad * 8), o_cand = take((size_t)B * TOPK_CAP * 8);
+  const host::TopkWsOffsets o = host::topk_ws_offsets(B, k);
   if (ws) {
-    ws->tau = (float*)(p + o_tau);
-    ws->cnt = (int32_t*)(p + o_cnt);
-    ws->list_len = (int32_t*)(p + o_len);
-    ws->dirty = (int32_t*)(p + o_dirty);
-    ws->n_dirty = (int32_t*)(p + o_nd);
-    ws->list = (unsigned long long*)(p + o_list);
-    ws->cand = (unsigned long long*)(p + o_cand);
-    ws->kpad = kpad;
+    char* p = (char*)base;
+    ws->tau = (float*)(p + o.tau);
+    ws->cnt = (int32_t*)(p + o.cnt);
+    ws->list_len = (int32_t*)(p + o.list_len);
+    ws->dirty = (int32_t*)(p + o.dirty);
+    ws->n_dirty = (int32_t*)(p + o.n_dirty);
+    ws->list = (unsigned long long*)(p + o.list);
+    ws->cand = (unsigned long long*)(p + o.cand);
+    ws->kpad = o.kpad;
   }
-  return off;
+  return o.total;
 }
 
 __global__ void topk_init_kernel(TopkWs w, int64_t B) {
@@ -905,30 +886,8 @@ __global__ void reduce_splits_kernel(const float* partial, int n_splits, int64_t
 // ============================================================================================
 int check_contract(const char* who, const float* Q, const void* E, int dtype, const float* scale, int64_t B,
                    int64_t d, int64_t N) {
-  KGE_REQUIRE(B >= 0 && N >= 1, KGE_ERR_INVALID, "%s: B=%lld N=%lld", who, (long long)B, (long long)N);
-  KGE_REQUIRE(N <= 0x7fffffffLL, KGE_ERR_INVALID, "%s: N=%lld exceeds int32 entity ids", who, (long long)N);
-  KGE_REQUIRE(B <= (1 << 24), KGE_ERR_INVALID, "%s: B=%lld exceeds 2^24", who, (long long)B);
-  KGE_REQUIRE(B == 0 || (Q && E), KGE_ERR_INVALID, "%s: null Q or E", who);
-  KGE_REQUIRE(((uintptr_t)Q & 15) == 0 && ((uintptr_t)E & 15) == 0, KGE_ERR_INVALID,
-              "%s: Q and E must be 16-byte aligned", who);
-  switch (dtype) {
-    case KGE_F32:
-      KGE_REQUIRE(d >= 1 && d <= 65536, KGE_ERR_INVALID, "%s: d=%lld", who, (long long)d);
-      break;
-    case KGE_BF16:
-      KGE_REQUIRE(d >= 8 && d % 8 == 0, KGE_ERR_INVALID, "%s: bf16 tables need d %% 8 == 0, got %lld", who,
-                  (long long)d);
-      KGE_REQUIRE(d <= 65536, KGE_ERR_INVALID, "%s: d=%lld", who, (long long)d);
-      break;
-    case KGE_I8:
-      KGE_REQUIRE(d >= 16 && d % 16 == 0, KGE_ERR_INVALID, "%s: int8 tables need d %% 16 == 0, got %lld", who,
-                  (long long)d);
-      KGE_REQUIRE(d <= 128, KGE_ERR_UNSUPPORTED, "%s: int8 tables support d <= 128, got %lld", who, (long long)d);
-      KGE_REQUIRE(scale, KGE_ERR_INVALID, "%s: int8 tables need per-row scales", who);
-      break;
-    default: return set_error(KGE_ERR_INVALID, "%s: unknown dtype %d", who, dtype);
-  }
-  return KGE_OK;
+  const host::Status st = host::contract_rules(who, Q, E, dtype, scale, B, d, N);
+  return st.ok() ? KGE_OK : set_error(st.code, "%s", st.msg);
 }
 
 ContractArgs make_args(const float* Q, const void* E, int dtype, const float* scale, int64_t B, int64_t d,
@@ -1098,23 +1057,16 @@ struct RankWs {
   FixPlan plan;
 };
 size_t rank_ws_layout(int64_t B, void* base, RankWs* ws) {
-  size_t off = 0;
-  auto take = [&](size_t bytes) {
-    size_t o = off;
-    off = align_up(off + bytes, 256);
-    return o;
-  };
-  const size_t o_thr = take((size_t)B * 4), o_key = take((size_t)SORT_MAX * 8), o_gend = take((size_t)SORT_MAX * 4);
-  const size_t o_work = take((size_t)SORT_MAX * 8), o_meta = take(16);
+  const host::RankWsOffsets o = host::rank_ws_offsets(B);
   if (ws) {
     char* p = (char*)base;
-    ws->thr = (float*)(p + o_thr);
-    ws->plan.skey = (unsigned long long*)(p + o_key);
-    ws->plan.gend = (int32_t*)(p + o_gend);
-    ws->plan.work = (int32_t*)(p + o_work);
-    ws->plan.meta = (int32_t*)(p + o_meta);
+    ws->thr = (float*)(p + o.thr);
+    ws->plan.skey = (unsigned long long*)(p + o.skey);
+    ws->plan.gend = (int32_t*)(p + o.gend);
+    ws->plan.work = (int32_t*)(p + o.work);
+    ws->plan.meta = (int32_t*)(p + o.meta);
   }
-  return off;
+  return o.total;
 }
 
 }  // namespace
@@ -1438,7 +1390,7 @@ extern "C" int kge_row_minmax(const float* Q, const float* bias, const void* E, 
   return KGE_OK;
 }
 
-extern "C" size_t kge_bce_workspace_bytes(void) { return (2 * BCE_SLOTS + 1) * sizeof(double) + 248; }
+extern "C" size_t kge_bce_workspace_bytes(void) { return host::bce_ws_bytes(); }
 
 extern "C" int kge_bce_multihot(const float* Q, const float* bias, const void* E, int dtype, const float* scale,
                                 int64_t B, int64_t d, int64_t N, const int64_t* csr_row, const int64_t* row_ptr,
@@ -1472,35 +1424,8 @@ extern "C" int kge_bce_multihot(const float* Q, const float* bias, const void* E
 }
 
 // ---- backward of the BCE step ------------------------------------------------------------------------
-namespace {
-struct BwdPlan {
-  int64_t ldG, ldT;      // row strides of G [B, ldG] and GT [N, ldT] (multiples of 4)
-  int k_splits, k_split_len;
-  size_t off_G, off_GT, off_ET, off_QT, off_part, total;
-};
-BwdPlan bwd_plan(int64_t B, int64_t d, int64_t N) {
-  BwdPlan p;
-  p.ldG = (N + 3) / 4 * 4;
-  p.ldT = (B + 3) / 4 * 4;
-  // dQ = G . E sums over N: split so that about 256 workgroups run
-  const int64_t tiles = ((B + KS_WG_QUERIES - 1) / KS_WG_QUERIES) * ((d + KS_TILE_ROWS - 1) / KS_TILE_ROWS);
-  int64_t splits = (256 + tiles - 1) / tiles;
-  if (splits > 64) splits = 64;
-  if (splits < 1) splits = 1;
-  int64_t len = ((N + splits - 1) / splits + 31) / 32 * 32;
-  p.k_split_len = (int)len;
-  p.k_splits = (int)((N + len - 1) / len);
-  auto up = [](size_t x) { return (x + 255) / 256 * 256; };
-  size_t off = up(kge_bce_workspace_bytes());
-  p.off_G = off;     off += up((size_t)B * p.ldG * sizeof(float));
-  p.off_GT = off;    off += up((size_t)N * p.ldT * sizeof(float));
-  p.off_ET = off;    off += up((size_t)d * p.ldG * sizeof(float));
-  p.off_QT = off;    off += up((size_t)d * p.ldT * sizeof(float));
-  p.off_part = off;  off += up((size_t)p.k_splits * B * d * sizeof(float));
-  p.total = off;
-  return p;
-}
-}  // namespace
+using host::BwdPlan;
+using host::bwd_plan;
 
 extern "C" size_t kge_bce_backward_workspace_bytes(int64_t B, int64_t d, int64_t N) {
   if (B < 1 || d < 1 || N < 1) return 0;

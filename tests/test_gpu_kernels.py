@@ -520,6 +520,67 @@ def test_rank_large_batch_spans_several_filter_plans(ops, FilterCSR):
     np.testing.assert_array_equal(out["n_equal_lower"].cpu().numpy(), tl)
 
 
+def test_plan_written_by_the_gpu_satisfies_the_host_model_invariants(ops, FilterCSR):
+    """The plan of the filter correction as plan_fix_kernel leaves it in the workspace (layout and packed fields of
+    csrc/kge_host.h, whose sequential model the CPU suite runs under sanitizers): groups partition the queries that
+    have a non-empty filter row, member positions are contiguous, the work list covers every slice exactly once."""
+    import ctypes
+    from dicee_amd import _lib
+    lib = _lib.load()
+    rng = np.random.default_rng(21)
+    N, R, d, B = 3000, 5, 32, 3000
+    E, Rel = random_tables(rng, N, R, d)
+    hr = random_hr(rng, 300, R, B)
+    hr[:500] = hr[0]
+    targets = rng.integers(0, N, B).astype(np.int64)
+    er = random_csr(rng, hr, targets, N, R, max_len=3, hub_rows=[(0, 2900), (700, 1500)])
+    csr = FilterCSR.from_er_vocab(er, R, device="cuda")
+    Eg, hr_g = dev(torch.from_numpy(E)), dev(torch.from_numpy(hr))
+    Q, bias = ops.build_query("DistMult", Eg, dev(torch.from_numpy(Rel)), hr_g)
+    rows = csr.rows_for(hr_g)
+    out = [torch.empty((B,), dtype=torch.int32, device="cuda") for _ in range(3)] + [torch.empty((B,), device="cuda")]
+    ws_bytes = lib.kge_rank_workspace_bytes(B)
+    ws = torch.zeros((ws_bytes,), dtype=torch.uint8, device="cuda")
+    p = lambda t: ctypes.c_void_p(t.data_ptr())
+    rc = lib.kge_rank_filtered(p(Q), p(bias), p(Eg), _lib.DTYPE_F32, None, B, d, N, p(dev(torch.from_numpy(targets))),
+                               p(rows), p(csr.row_ptr), p(csr.col), csr.row_ptr.numel() - 1, p(out[0]), p(out[1]),
+                               p(out[2]), p(out[3]), p(ws), ws_bytes, ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+    assert rc == 0, lib.kge_last_error()
+    torch.cuda.synchronize()
+    up = lambda x: (x + 255) // 256 * 256
+    SORT_MAX = 8192
+    o_skey = up(4 * B)
+    o_gend = o_skey + up(8 * SORT_MAX)
+    o_work = o_gend + up(4 * SORT_MAX)
+    o_meta = o_work + up(8 * SORT_MAX)
+    assert o_meta + 256 == ws_bytes
+    raw = ws.cpu().numpy()
+    skey = raw[o_skey:o_skey + 8 * SORT_MAX].view(np.uint64)
+    gend = raw[o_gend:o_gend + 4 * SORT_MAX].view(np.int32)
+    work = raw[o_work:o_work + 8 * SORT_MAX].view(np.int32).reshape(-1, 2)
+    n_work, slice_len, n_groups = (int(v) for v in raw[o_meta:o_meta + 12].view(np.int32))
+    rp = csr.row_ptr.cpu().numpy()
+    rows_h = rows.cpu().numpy()
+    want = {}
+    for i, r in enumerate(rows_h):
+        if r >= 0 and rp[r + 1] > rp[r]:
+            want.setdefault(int(r), set()).add(i)
+    assert n_groups == len(want) and slice_len >= 128 and slice_len % 32 == 0
+    seen_work, seen_rows = 0, set()
+    for g in range(n_groups):
+        first, w0 = int(work[g, 0]), int(work[g, 1])
+        assert w0 == seen_work
+        end = int(gend[first])
+        row = int(skey[first] >> np.uint64(24))
+        assert row in want and row not in seen_rows
+        seen_rows.add(row)
+        members = {int(skey[i] & np.uint64(0xffffff)) for i in range(first, end)}
+        assert all(int(skey[i] >> np.uint64(24)) == row for i in range(first, end))
+        assert members == want[row]
+        seen_work += -(-(int(rp[row + 1] - rp[row])) // slice_len)
+    assert seen_work == n_work
+
+
 def test_csr_lookup_matches_host_search(ops, FilterCSR):
     rng = np.random.default_rng(12)
     N, R = 500, 7

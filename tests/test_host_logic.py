@@ -258,3 +258,23 @@ def test_three_part_bf16_split_arithmetic():
     dropped = sum(np.einsum("nk,nk->n", px[a].astype(np.float64), py[b].astype(np.float64))
                   for a, b in [(1, 2), (2, 1), (2, 2)])
     assert np.max(np.abs(dropped) / scale) < 2.0 ** -24
+
+
+def test_host_logic_builds_and_runs_under_address_and_ub_sanitizers(tmp_path):
+    """The library's host logic (csrc/kge_host.h: argument rules, workspace layouts, vocabulary keys, the packed
+    counters and the sequential model of the filter-correction plan) compiled by g++ with
+    -fsanitize=address,undefined and run on the cases that stress the packed fields: a full sub-batch in one group,
+    8192 singleton groups, a 50,000-entry row, a total length at the bound of the work list, int32-long rows."""
+    import shutil
+    import subprocess
+    if shutil.which("g++") is None:
+        pytest.skip("no g++")
+    exe = tmp_path / "host_model_test"
+    src = os.path.join(ROOT, "tests", "host_model_test.cpp")
+    build = subprocess.run(["g++", "-std=c++17", "-O1", "-g", "-fsanitize=address,undefined",
+                            "-fno-sanitize-recover=all", "-Wall", "-Wextra", "-Werror", "-o", str(exe), src],
+                           capture_output=True, text=True)
+    assert build.returncode == 0, build.stderr[-3000:]
+    run = subprocess.run([str(exe)], capture_output=True, text=True, timeout=300)
+    assert run.returncode == 0, (run.stdout + run.stderr)[-3000:]
+    assert "host logic ok" in run.stdout
