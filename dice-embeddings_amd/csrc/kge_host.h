@@ -81,8 +81,13 @@ inline Status contract_rules(const char* who, const void* Q, const void* E, int 
 }
 
 // ---- workspace layouts ------------------------------------------------------------------------------------
+// thresholds [B]; per query the leader of its filter group (`lead`, -1: none) and per leader whether its group holds
+// different query vectors (`mixed`); then one plan (member keys, group ends, group records, 4 counters) per
+// sub-batch of SORT_MAX queries
 struct RankWsOffsets {
-  size_t thr, skey, gend, work, meta, total;
+  size_t thr, lead, mixed, plans, total;
+  size_t plan_stride, skey, gend, work, meta;  // of one plan: stride between plans, offsets inside a plan
+  int64_t n_plans;
 };
 inline RankWsOffsets rank_ws_offsets(int64_t B) {
   RankWsOffsets o{};
@@ -92,12 +97,18 @@ inline RankWsOffsets rank_ws_offsets(int64_t B) {
     off = align_up(off + bytes, 256);
     return at;
   };
+  o.n_plans = (B + SORT_MAX - 1) / SORT_MAX;
+  if (o.n_plans < 1) o.n_plans = 1;
   o.thr = take((size_t)B * 4);
-  o.skey = take((size_t)SORT_MAX * 8);
-  o.gend = take((size_t)SORT_MAX * 4);
-  o.work = take((size_t)SORT_MAX * 8);
-  o.meta = take(16);
-  o.total = off;
+  o.lead = take((size_t)B * 4);
+  o.mixed = take((size_t)B * 4);
+  o.plans = off;
+  o.skey = 0;
+  o.gend = align_up((size_t)SORT_MAX * 8, 256);
+  o.work = o.gend + align_up((size_t)SORT_MAX * 4, 256);
+  o.meta = o.work + align_up((size_t)SORT_MAX * 8, 256);
+  o.plan_stride = o.meta + 256;
+  o.total = o.plans + (size_t)o.n_plans * o.plan_stride;
   return o;
 }
 

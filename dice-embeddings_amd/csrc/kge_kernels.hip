@@ -129,10 +129,15 @@ __device__ __forceinline__ f32x16 chain_direct(const void* E, int d, int64_t e_r
 }
 
 // ---- raw score of each query's target (the rank threshold) + counter initialisation ---------
+// and, when the batch is filtered, the check the filter correction relies on: the correction scores a slice of a
+// filter row once per group of queries that share the row, with the query vector of the group's leader.  A member
+// whose vector differs from the leader's, in any bit, marks the group `mixed`; such a group is corrected one
+// distinct vector at a time.  (Queries built from the same (head, relation) pair share row and vector.)
 template <int EDT>
 __global__ void __launch_bounds__(256) target_score_kernel(ContractArgs a, const int64_t* target, const float* bias,
                                                           float* thr, float* target_score, int32_t* n_gt,
-                                                          int32_t* n_eq, int32_t* n_eql) {
+                                                          int32_t* n_eq, int32_t* n_eql, const int32_t* lead,
+                                                          int32_t* mixed) {
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, c = lane & 31, hf = lane >> 5;
   const int64_t q = ((int64_t)blockIdx.x * 4 + wave) * 32 + c;
   const int64_t t = (q < a.B) ? target[q] : -1;
@@ -152,6 +157,26 @@ __global__ void __launch_bounds__(256) target_score_kernel(ContractArgs a, const
     n_gt[q] = 0;
     n_eq[q] = ok ? -1 : 0;  // the main pass counts the target as tying with itself
     n_eql[q] = 0;
+  }
+  if (lead != nullptr && q < a.B) {
+    // a member that is not its group's leader compares its vector with the leader's: the two halves of the wave
+    // take alternate 16-byte pieces of the row (alternate words when the rows are not 16-byte aligned)
+    const int32_t l = lead[q];
+    if (l >= 0 && (int64_t)l != q) {
+      const uint32_t* x = (const uint32_t*)a.Q + q * a.d;
+      const uint32_t* y = (const uint32_t*)a.Q + (int64_t)l * a.d;
+      bool differs = false;
+      if ((a.d & 3) == 0 && ((uintptr_t)a.Q & 15) == 0) {
+#pragma unroll 4
+        for (int64_t k = hf * 4; k < a.d; k += 8) {
+          const uint4 u = *(const uint4*)(x + k), w = *(const uint4*)(y + k);
+          differs = differs || u.x != w.x || u.y != w.y || u.z != w.z || u.w != w.w;
+        }
+      } else {
+        for (int64_t k = hf; k < a.d; k += 2) differs = differs || x[k] != y[k];
+      }
+      if (differs) mixed[l] = 1;
+    }
   }
 }
 
@@ -212,6 +237,8 @@ struct FixPlan {
   int32_t* gend;             // [SORT_MAX] for a group's first position: one past its last position
   int32_t* work;             // [SORT_MAX][2] per group: (first position, index of its first work item)
   int32_t* meta;             // [0] work items, [1] slice length, [2] groups
+  int32_t* lead;             // [B] per query: index of the first member of its group (itself for a leader), -1: no group
+  int32_t* mixed;            // [B] per leader: set when some member of its group holds another query vector
 };
 
 __global__ void __launch_bounds__(1024) plan_fix_kernel(const int64_t* csr_row, int64_t b0, int nb, int64_t n_rows,
@@ -299,6 +326,7 @@ __global__ void __launch_bounds__(1024) plan_fix_kernel(const int64_t* csr_row, 
       plan.work[2 * g + 1] = (int)host::plan_slices(base);
       plan.gend[first] = first + tab_cnt[my_slot[j]];
       tab_cnt[my_slot[j]] = first;  // only this leader reads or writes its group's slot in this phase
+      tab_row[my_slot[j]] = tid + 1024 * j;  // the slot's row number has done its work: now the leader's index
     } else if (my_pos[j] == 0) {
       tab_cnt[my_slot[j]] = -1;     // empty filter row: nothing to take out for this group
     }
@@ -310,13 +338,22 @@ __global__ void __launch_bounds__(1024) plan_fix_kernel(const int64_t* csr_row, 
     plan.meta[2] = host::plan_groups(part[1023]);
   }
   __syncthreads();
-  // (4) members to their positions
+  // (4) members to their positions; every query learns its group's leader (for the check that a group's members
+  // hold one and the same query vector, which the kernel that forms the thresholds makes)
 #pragma unroll
   for (int j = 0; j < QPT; ++j) {
+    const int i = tid + 1024 * j;
+    int32_t leader = -1;
     if (my_slot[j] >= 0) {
       const int first = tab_cnt[my_slot[j]];
-      if (first >= 0)
-        plan.skey[first + my_pos[j]] = host::plan_member_key(my_row[j], tid + 1024 * j);
+      if (first >= 0) {
+        plan.skey[first + my_pos[j]] = host::plan_member_key(my_row[j], i);
+        leader = (int32_t)b0 + tab_row[my_slot[j]];
+      }
+    }
+    if (i < nb) {
+      plan.lead[b0 + i] = leader;
+      plan.mixed[b0 + i] = 0;
     }
   }
 }
@@ -330,16 +367,22 @@ __global__ void __launch_bounds__(1024) plan_fix_kernel(const int64_t* csr_row, 
 // (vectors are compared bit for bit against the round's leader).
 constexpr int FIX_CAP = 2048;
 constexpr int FIX_ITEMS = 16;  // work items a workgroup resolves side by side
-template <int EDT>
+// ROWS256 (bf16 tables with d == 128: rows of 256 bytes): the slice's rows are gathered the way the main loop
+// streams them, 16 lanes per row straight into LDS (whole 128-byte lines per request) in the swizzled stage
+// layout, and the MFMA fragments are read from there; the generic path reads every row 16 bytes per lane at
+// a stride, which costs four requests per line.
+template <int EDT, bool ROWS256>
 __global__ void __launch_bounds__(256) filter_fix_kernel(ContractArgs a, FixPlan plan, int64_t b0,
                                                         const int64_t* row_ptr, const int32_t* col,
                                                         const int64_t* target, const float* thr, int32_t* n_gt,
                                                         int32_t* n_eq, int32_t* n_eql) {
-  __shared__ float s_s[FIX_CAP];
-  __shared__ float s_sc[FIX_CAP];
-  __shared__ int32_t s_e[FIX_CAP];
+  constexpr int CAP = ROWS256 ? 512 : FIX_CAP;  // entities per pass (the staged rows leave less LDS for the scores)
+  __shared__ float s_s[CAP];
+  __shared__ float s_sc[EDT == KGE_I8 ? CAP : 1];
+  __shared__ int32_t s_e[CAP];
   __shared__ int32_t s_cnt[3 * 256];
   __shared__ unsigned char s_state[SORT_MAX];  // per member of a group: 0 = waiting, 1 = in this round, 2 = done
+  __shared__ __attribute__((aligned(1024))) unsigned char s_rows[ROWS256 ? 4 * 8192 : 16];  // per wave: one 32-row tile
   __shared__ int s_next;                       // first member still waiting after this round
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, c = lane & 31, hf = lane >> 5;
   const int n_work = plan.meta[0];
@@ -348,7 +391,7 @@ __global__ void __launch_bounds__(256) filter_fix_kernel(ContractArgs a, FixPlan
   // This workgroup's work items are w = blockIdx.x + k * gridDim.x.  Up to FIX_ITEMS of them at a time are
   // resolved by one thread each, side by side (group by binary search, then the group's row and extent),
   // so that their chains of dependent loads overlap instead of running once per item.
-  __shared__ int32_t it_i0[FIX_ITEMS], it_m[FIX_ITEMS];
+  __shared__ int32_t it_i0[FIX_ITEMS], it_m[FIX_ITEMS], it_mixed[FIX_ITEMS];
   __shared__ int64_t it_z0[FIX_ITEMS], it_z1[FIX_ITEMS];
   for (int k0 = 0; blockIdx.x + (int64_t)k0 * gridDim.x < n_work; k0 += FIX_ITEMS) {
     __syncthreads();
@@ -368,6 +411,7 @@ __global__ void __launch_bounds__(256) filter_fix_kernel(ContractArgs a, FixPlan
         const int64_t z0 = L0 + z * slice;
         it_i0[tid] = i0;
         it_m[tid] = plan.gend[i0] - i0;
+        it_mixed[tid] = plan.mixed[b0 + host::plan_key_pos(key)];
         it_z0[tid] = z0;
         it_z1[tid] = (z0 + slice < L1) ? z0 + slice : L1;
       }
@@ -381,13 +425,16 @@ __global__ void __launch_bounds__(256) filter_fix_kernel(ContractArgs a, FixPlan
     int tpm = 1;
     while (tpm * 2 * m <= 256) tpm *= 2;
     const int sub = tid % tpm, mslot = tid / tpm, mstep = 256 / tpm;
-    if (m > 1) {
+    // a group whose members all hold the leader's query vector (the check is made once per group, by the kernel
+    // that forms the thresholds) takes one round; a mixed group one round per distinct vector
+    const bool rounds = m > 1 && it_mixed[kk] != 0;
+    if (rounds) {
       for (int i = tid; i < m; i += 256) s_state[i] = 0;
     }
-    // one round per distinct query vector of the group; `lead` is the first member not yet served
+    // `lead` is the first member not yet served
     for (int lead = 0; lead < m;) {
       const int64_t bq = b0 + (int64_t)host::plan_key_pos(plan.skey[i0 + lead]);
-      if (m > 1) {
+      if (rounds) {
         // members whose query vector equals the leader's, bit for bit, join this round
         __syncthreads();
         if (tid == 0) s_next = m;
@@ -421,9 +468,52 @@ __global__ void __launch_bounds__(256) filter_fix_kernel(ContractArgs a, FixPlan
         }
         __syncthreads();
       }
-      for (int64_t pass = z0; pass < z1; pass += FIX_CAP) {
-        const int n_here = (int)((z1 - pass < FIX_CAP) ? z1 - pass : FIX_CAP);
+      for (int64_t pass = z0; pass < z1; pass += CAP) {
+        const int n_here = (int)((z1 - pass < CAP) ? z1 - pass : CAP);
         const int ntile = (n_here + 31) >> 5;
+        if constexpr (ROWS256) {
+          // the round's query vector as MFMA fragments (the same one in every column)
+          bf16x8 qfrag[8];
+#pragma unroll
+          for (int sft = 0; sft < 8; ++sft) {
+            const f32x4* src = (const f32x4*)(a.Q + bq * 128 + 16 * sft + 8 * hf);
+            qfrag[sft] = cvt_bf16x8(src[0], src[1]);
+          }
+          const int wv = __builtin_amdgcn_readfirstlane(wave);
+          unsigned char* stage = s_rows + wv * 8192;
+          const unsigned char* Eb = (const unsigned char*)a.E;
+          for (int tile = wv; tile < ntile; tile += 4) {
+            const int j0 = tile * 32 + c;
+            const int32_t e0 = (j0 < n_here) ? col[pass + j0] : -1;
+            const bool ok0 = e0 >= 0 && (int64_t)e0 < a.N;
+            if (hf == 0) s_e[j0] = ok0 ? e0 : -1;
+            // lane l fetches piece (l & 15) ^ (row & 15) of row 4 j + l / 16 of the tile; an entry that is not a
+            // valid entity id fetches row 0 instead (its score is ignored: s_e says -1)
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+              const int row = 4 * j + (lane >> 4);
+              const int32_t e = s_e[tile * 32 + row];
+              const int64_t er = e >= 0 ? (int64_t)e : 0;
+              __builtin_amdgcn_global_load_lds(
+                  (const __attribute__((address_space(1))) void*)(Eb + er * 256 + (((lane & 15) ^ (row & 15)) << 4)),
+                  (__attribute__((address_space(3))) void*)(stage + j * 1024), 16, 0, 0);
+            }
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            f32x16 acc;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) acc[i] = 0.f;
+#pragma unroll
+            for (int sft = 0; sft < 8; ++sft) {
+              const bf16x8 ef = *(const bf16x8*)(stage + c * 256 + (((2 * sft + hf) ^ (c & 15)) << 4));
+              acc = mfma_bf16(ef, qfrag[sft], acc);
+            }
+            if (c == 0) {
+#pragma unroll
+              for (int i = 0; i < 16; ++i) s_s[tile * 32 + row_of(i, hf)] = acc[i];
+            }
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the fragments are read before the next tile's rows land
+          }
+        } else {
         // two tiles per trip so that both row gathers are in flight before the first MFMA chain
         for (int tile = wave; tile < ntile; tile += 8) {
           const int j0 = tile * 32 + c, j1 = (tile + 4) * 32 + c;
@@ -444,19 +534,20 @@ __global__ void __launch_bounds__(256) filter_fix_kernel(ContractArgs a, FixPlan
           }
           if (hf == 0) {
             s_e[j0] = ok0 ? e0 : -1;
-            s_sc[j0] = (EDT == KGE_I8 && ok0) ? a.scale[e0] : 1.f;
+            if (EDT == KGE_I8) s_sc[j0] = ok0 ? a.scale[e0] : 1.f;
             if (two) {
               s_e[j1] = ok1 ? e1 : -1;
-              s_sc[j1] = (EDT == KGE_I8 && ok1) ? a.scale[e1] : 1.f;
+              if (EDT == KGE_I8) s_sc[j1] = ok1 ? a.scale[e1] : 1.f;
             }
           }
+        }
         }
         __syncthreads();
         // compare phase: `tpm` threads share one query; their partial counts meet in LDS so that each
         // query receives ONE global atomic per counter (hundreds of same-address atomics serialise)
         for (int mbase = lead; mbase < m; mbase += mstep) {
           const int mi = mbase + mslot;
-          const bool mine = mi < m && (m == 1 || s_state[mi] == 1);
+          const bool mine = mi < m && (!rounds || s_state[mi] == 1);
           s_cnt[tid] = 0;
           s_cnt[256 + tid] = 0;
           s_cnt[512 + tid] = 0;
@@ -499,7 +590,7 @@ __global__ void __launch_bounds__(256) filter_fix_kernel(ContractArgs a, FixPlan
           __syncthreads();
         }
       }
-      if (m == 1) break;
+      if (!rounds) break;
       // this round's members are done; the next round is led by the first member still waiting
       __syncthreads();
       for (int i = lead + tid; i < m; i += 256)
@@ -1056,15 +1147,19 @@ struct RankWs {
   float* thr;
   FixPlan plan;
 };
-size_t rank_ws_layout(int64_t B, void* base, RankWs* ws) {
+// plan `sub` of the workspace laid out at `base` (one plan per sub-batch of SORT_MAX queries)
+size_t rank_ws_layout(int64_t B, void* base, RankWs* ws, int64_t sub = 0) {
   const host::RankWsOffsets o = host::rank_ws_offsets(B);
   if (ws) {
     char* p = (char*)base;
+    char* pl = p + o.plans + (size_t)sub * o.plan_stride;
     ws->thr = (float*)(p + o.thr);
-    ws->plan.skey = (unsigned long long*)(p + o.skey);
-    ws->plan.gend = (int32_t*)(p + o.gend);
-    ws->plan.work = (int32_t*)(p + o.work);
-    ws->plan.meta = (int32_t*)(p + o.meta);
+    ws->plan.skey = (unsigned long long*)(pl + o.skey);
+    ws->plan.gend = (int32_t*)(pl + o.gend);
+    ws->plan.work = (int32_t*)(pl + o.work);
+    ws->plan.meta = (int32_t*)(pl + o.meta);
+    ws->plan.lead = (int32_t*)(p + o.lead);
+    ws->plan.mixed = (int32_t*)(p + o.mixed);
   }
   return o.total;
 }
@@ -1192,29 +1287,53 @@ int check_rank_args(const char* who, const float* Q, const void* E, int dtype, c
   return KGE_OK;
 }
 
-// the launches of a filtered-rank call; `ws` points into a caller's workspace or into the library's static scratch
+// the launches of a filtered-rank call; `ws_base` is a caller's workspace or the library's static scratch.
+// Order: the plan of every sub-batch (it only needs the filter rows, and tells every query its group's leader),
+// thresholds + counters + the one-vector-per-group check, the main loop, the filter correction of every sub-batch.
 int rank_filtered_launch(const char* who, const float* Q, const float* bias, const void* E, int dtype, const float* scale,
                          int64_t B, int64_t d, int64_t N, const int64_t* target, const int64_t* csr_row,
                          const int64_t* row_ptr, const int32_t* col, int64_t n_rows, int32_t* n_greater, int32_t* n_equal,
-                         int32_t* n_equal_lower, float* target_score, const RankWs& ws, hipStream_t st) {
+                         int32_t* n_equal_lower, float* target_score, void* ws_base, hipStream_t st) {
   ContractArgs a = make_args(Q, E, dtype, scale, B, d, N, 0, N);
+  const bool filtered = csr_row != nullptr && n_rows > 0;
+  RankWs ws;
+  rank_ws_layout(B, ws_base, &ws);
+  if (filtered) {
+    for (int64_t b0 = 0, sub = 0; b0 < B; b0 += SORT_MAX, ++sub) {
+      const int nb = (int)((B - b0 < SORT_MAX) ? B - b0 : SORT_MAX);
+      RankWs wsub;
+      rank_ws_layout(B, ws_base, &wsub, sub);
+      hipLaunchKernelGGL(plan_fix_kernel, dim3(1), dim3(1024), 0, st, csr_row, b0, nb, n_rows, row_ptr, wsub.plan);
+      KGE_LAUNCH_CHECK("plan_fix_kernel");
+    }
+  }
   {
     dim3 grid((unsigned)((B + 127) / 128)), block(256);
     KGE_DISPATCH_DTYPE(dtype, target_score_kernel, grid, block, 0, st, a, target, bias, ws.thr, target_score,
-                       n_greater, n_equal, n_equal_lower);
+                       n_greater, n_equal, n_equal_lower, filtered ? (const int32_t*)ws.plan.lead : (const int32_t*)nullptr,
+                       ws.plan.mixed);
     KGE_LAUNCH_CHECK("target_score_kernel");
   }
   RankArgs ea{ws.thr, target, n_greater, n_equal, n_equal_lower};
   int rc = launch_contract<RankEpi>(dtype, a, ea, st, who);
   if (rc) return rc;
-  if (csr_row != nullptr && n_rows > 0) {
-    for (int64_t b0 = 0; b0 < B; b0 += SORT_MAX) {
-      const int nb = (int)((B - b0 < SORT_MAX) ? B - b0 : SORT_MAX);
-      hipLaunchKernelGGL(plan_fix_kernel, dim3(1), dim3(1024), 0, st, csr_row, b0, nb, n_rows, row_ptr, ws.plan);
-      KGE_LAUNCH_CHECK("plan_fix_kernel");
+  if (filtered) {
+    for (int64_t b0 = 0, sub = 0; b0 < B; b0 += SORT_MAX, ++sub) {
+      RankWs wsub;
+      rank_ws_layout(B, ws_base, &wsub, sub);
       dim3 grid(2048), block(256);
-      KGE_DISPATCH_DTYPE(dtype, filter_fix_kernel, grid, block, 0, st, a, ws.plan, b0, row_ptr, col, target, ws.thr,
-                         n_greater, n_equal, n_equal_lower);
+      if (dtype == KGE_F32)
+        hipLaunchKernelGGL((filter_fix_kernel<KGE_F32, false>), grid, block, 0, st, a, wsub.plan, b0, row_ptr, col, target,
+                           ws.thr, n_greater, n_equal, n_equal_lower);
+      else if (dtype == KGE_BF16 && d == 128)
+        hipLaunchKernelGGL((filter_fix_kernel<KGE_BF16, true>), grid, block, 0, st, a, wsub.plan, b0, row_ptr, col, target,
+                           ws.thr, n_greater, n_equal, n_equal_lower);
+      else if (dtype == KGE_BF16)
+        hipLaunchKernelGGL((filter_fix_kernel<KGE_BF16, false>), grid, block, 0, st, a, wsub.plan, b0, row_ptr, col, target,
+                           ws.thr, n_greater, n_equal, n_equal_lower);
+      else
+        hipLaunchKernelGGL((filter_fix_kernel<KGE_I8, false>), grid, block, 0, st, a, wsub.plan, b0, row_ptr, col, target,
+                           ws.thr, n_greater, n_equal, n_equal_lower);
       KGE_LAUNCH_CHECK("filter_fix_kernel");
     }
   }
@@ -1235,10 +1354,8 @@ extern "C" int kge_rank_filtered(const float* Q, const float* bias, const void* 
   KGE_REQUIRE(workspace && workspace_bytes >= kge_rank_workspace_bytes(B), KGE_ERR_WORKSPACE,
               "kge_rank_filtered: workspace of %zu bytes, need %zu", workspace_bytes, kge_rank_workspace_bytes(B));
   KGE_REQUIRE(((uintptr_t)workspace & 7) == 0, KGE_ERR_WORKSPACE, "kge_rank_filtered: workspace must be 8-byte aligned");
-  RankWs ws;
-  rank_ws_layout(B, workspace, &ws);
   return rank_filtered_launch("kge_rank_filtered", Q, bias, E, dtype, scale, B, d, N, target, csr_row, row_ptr, col,
-                              n_rows, n_greater, n_equal, n_equal_lower, target_score, ws, (hipStream_t)stream);
+                              n_rows, n_greater, n_equal, n_equal_lower, target_score, workspace, (hipStream_t)stream);
 }
 
 // ---- the same call for callers that cannot allocate ---------------------------------------------------
@@ -1246,7 +1363,7 @@ extern "C" int kge_rank_filtered(const float* Q, const float* bias, const void* 
 // device array instead of caller memory.  Every GPU the library runs on holds its own copy of the array at its
 // own address until the process ends; the address is looked up once per device and only that pointer is ever
 // handed to a kernel.  All calls on one GPU share the array: calls that overlap on one GPU race.
-static __device__ __align__(256) unsigned char scratch[4 * KGE_RANK_STATIC_MAX_B + 20 * SORT_MAX + 1024];
+static __device__ __align__(256) unsigned char scratch[KGE_RANK_STATIC_SCRATCH_BYTES];
 
 namespace {
 constexpr int SCRATCH_MAX_DEVICES = 64;
@@ -1289,12 +1406,11 @@ extern "C" int kge_rank_filtered_static(const float* Q, const float* bias, const
   unsigned char* base = nullptr;
   rc = scratch_on_current_device(&base);
   if (rc) return rc;
-  // nothing in the scratch needs clearing: thresholds are written for every query and the plan is rebuilt per
-  // sub-batch before anything reads it, so what an earlier (larger) call left behind is never read
-  RankWs ws;
-  rank_ws_layout(B, base, &ws);
+  // nothing in the scratch needs clearing: thresholds, leaders and the mixed-group flags are written for every
+  // query and every sub-batch's plan is rebuilt before anything reads it, so what an earlier call left behind is
+  // never read
   return rank_filtered_launch("kge_rank_filtered_static", Q, bias, E, dtype, scale, B, d, N, target, csr_row, row_ptr,
-                              col, n_rows, n_greater, n_equal, n_equal_lower, target_score, ws, (hipStream_t)stream);
+                              col, n_rows, n_greater, n_equal, n_equal_lower, target_score, base, (hipStream_t)stream);
 }
 
 extern "C" size_t kge_topk_workspace_bytes(int64_t B, int64_t N, int64_t k) {

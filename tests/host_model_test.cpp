@@ -64,8 +64,16 @@ static void check_disjoint(std::vector<std::pair<size_t, size_t>> parts, size_t 
 static void test_layouts() {
   for (int64_t B : {1LL, 2LL, 63LL, 4096LL, 8192LL, 8193LL, 65536LL, (1LL << 24)}) {
     const RankWsOffsets r = rank_ws_offsets(B);
-    check_disjoint({{r.thr, (size_t)B * 4}, {r.skey, (size_t)SORT_MAX * 8}, {r.gend, (size_t)SORT_MAX * 4},
-                    {r.work, (size_t)SORT_MAX * 8}, {r.meta, 16}}, r.total);
+    std::vector<std::pair<size_t, size_t>> parts = {{r.thr, (size_t)B * 4}, {r.lead, (size_t)B * 4}, {r.mixed, (size_t)B * 4}};
+    CHECK(r.n_plans * (int64_t)SORT_MAX >= B && (r.n_plans - 1) * (int64_t)SORT_MAX < std::max<int64_t>(B, 1));
+    for (int64_t s = 0; s < r.n_plans; ++s) {
+      const size_t base = r.plans + (size_t)s * r.plan_stride;
+      parts.push_back({base + r.skey, (size_t)SORT_MAX * 8});
+      parts.push_back({base + r.gend, (size_t)SORT_MAX * 4});
+      parts.push_back({base + r.work, (size_t)SORT_MAX * 8});
+      parts.push_back({base + r.meta, 16});
+    }
+    check_disjoint(parts, r.total);
     for (int64_t k : {1LL, 7LL, 8LL, 100LL, 1024LL}) {
       const TopkWsOffsets t = topk_ws_offsets(B, k);
       CHECK(t.kpad >= k && t.kpad % 8 == 0 && t.kpad < k + 8);
@@ -74,7 +82,7 @@ static void test_layouts() {
     }
   }
   // the static scratch array of kge_rank_filtered_static holds the layout of its largest batch
-  CHECK(rank_ws_offsets(KGE_RANK_STATIC_MAX_B).total <= 4 * (size_t)KGE_RANK_STATIC_MAX_B + 20 * SORT_MAX + 1024);
+  CHECK(rank_ws_offsets(KGE_RANK_STATIC_MAX_B).total <= KGE_RANK_STATIC_SCRATCH_BYTES);
   CHECK(TOPK_FIRST_ROWS <= TOPK_CAP);
   for (auto bdn : {std::array<int64_t, 3>{1, 1, 1}, {2048, 256, 40943}, {5, 7, 3}, {4096, 128, 1 << 24}}) {
     const BwdPlan p = bwd_plan(bdn[0], bdn[1], bdn[2]);

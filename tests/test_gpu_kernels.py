@@ -248,13 +248,14 @@ def test_rank_all_scores_equal(ops):
     np.testing.assert_array_equal(out["n_equal_lower"].cpu().numpy(), np.arange(B) * 50)
 
 
-def test_rank_one_filter_row_shared_by_different_query_vectors(ops, FilterCSR):
+@pytest.mark.parametrize("storage,d", [("fp32", 48), ("bf16", 128), ("bf16", 64), ("int8", 128)])
+def test_rank_one_filter_row_shared_by_different_query_vectors(ops, FilterCSR, storage, d):
     """The ABI takes Q and csr_row separately: queries may share a filter row without sharing a query vector
     (a range constraint per relation, a custom mask).  Each query must be corrected with ITS OWN scores of the
     filtered entities.  Rows: one long row shared by many distinct vectors, rows shared by a few, groups that mix
     repeated and distinct vectors, -1 (no filter)."""
     rng = np.random.default_rng(77)
-    N, d, B = 6000, 48, 900
+    N, B = 6000, 900
     E = (rng.standard_normal((N, d)) * 0.1).astype(np.float32)
     Qh = (rng.standard_normal((B, d)) * 0.1).astype(np.float32)
     Qh[100:160] = Qh[100]                      # 60 queries with one vector ...
@@ -270,10 +271,11 @@ def test_rank_one_filter_row_shared_by_different_query_vectors(ops, FilterCSR):
     csr_row[100:172] = 6                       # the mixed group
     targets = rng.integers(0, N, B).astype(np.int64)
     targets[:20] = col[:20]                    # targets inside their own filter row stay unfiltered
-    Eg, Qg = dev(torch.from_numpy(E)), dev(torch.from_numpy(Qh))
-    out = ops.rank_filtered(Qg, None, Eg, None, dev(torch.from_numpy(targets)), dev(torch.from_numpy(csr_row)),
+    Et, sc, _, _, _ = stored_tables(E, E[:1], storage)
+    Eg, scg, Qg = dev(Et), dev(sc), dev(torch.from_numpy(Qh))
+    out = ops.rank_filtered(Qg, None, Eg, scg, dev(torch.from_numpy(targets)), dev(torch.from_numpy(csr_row)),
                             dev(torch.from_numpy(row_ptr)), dev(torch.from_numpy(col)))
-    S_raw = ops.scores(Qg, None, Eg, None).cpu().numpy()
+    S_raw = ops.scores(Qg, None, Eg, scg).cpu().numpy()
     filters = [col[row_ptr[r]:row_ptr[r + 1]] if r >= 0 else None for r in csr_row]
     g, t, tl = _expected_counts(S_raw, targets, filters)
     np.testing.assert_array_equal(out["n_greater"].cpu().numpy(), g)
@@ -549,7 +551,10 @@ def test_plan_written_by_the_gpu_satisfies_the_host_model_invariants(ops, Filter
     torch.cuda.synchronize()
     up = lambda x: (x + 255) // 256 * 256
     SORT_MAX = 8192
-    o_skey = up(4 * B)
+    # thresholds, leaders, mixed-group flags (one int32 per query each), then one plan per 8192 queries
+    o_lead = up(4 * B)
+    o_mixed = o_lead + up(4 * B)
+    o_skey = o_mixed + up(4 * B)
     o_gend = o_skey + up(8 * SORT_MAX)
     o_work = o_gend + up(4 * SORT_MAX)
     o_meta = o_work + up(8 * SORT_MAX)
@@ -559,6 +564,8 @@ def test_plan_written_by_the_gpu_satisfies_the_host_model_invariants(ops, Filter
     gend = raw[o_gend:o_gend + 4 * SORT_MAX].view(np.int32)
     work = raw[o_work:o_work + 8 * SORT_MAX].view(np.int32).reshape(-1, 2)
     n_work, slice_len, n_groups = (int(v) for v in raw[o_meta:o_meta + 12].view(np.int32))
+    lead = raw[o_lead:o_lead + 4 * B].view(np.int32)
+    assert not raw[o_mixed:o_mixed + 4 * B].view(np.int32).any()
     rp = csr.row_ptr.cpu().numpy()
     rows_h = rows.cpu().numpy()
     want = {}
@@ -577,8 +584,12 @@ def test_plan_written_by_the_gpu_satisfies_the_host_model_invariants(ops, Filter
         members = {int(skey[i] & np.uint64(0xffffff)) for i in range(first, end)}
         assert all(int(skey[i] >> np.uint64(24)) == row for i in range(first, end))
         assert members == want[row]
+        # every member knows the group's leader (the query at the group's first sorted position); no group mixes vectors
+        assert all(int(lead[i]) == int(skey[first] & np.uint64(0xffffff)) for i in members)
         seen_work += -(-(int(rp[row + 1] - rp[row])) // slice_len)
     assert seen_work == n_work
+    no_row = [i for i, r in enumerate(rows_h) if not (r >= 0 and rp[r + 1] > rp[r])]
+    assert all(int(lead[i]) == -1 for i in no_row)
 
 
 def test_csr_lookup_matches_host_search(ops, FilterCSR):
