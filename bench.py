@@ -98,7 +98,7 @@ def main_loop_kernel(storage, d, mode):
     if d == 128 and storage == "bf16":
         return "qstream_kernel<RankFastEpi, 2, 8, 2>" if epi == "RankEpi" else f"qreg_async_kernel<{epi}>"
     if d == 128:
-        return f"qreg_i8_kernel<{epi}>"
+        return "topk_i8_filter_kernel" if epi == "TopkEpi" else f"qreg_i8_kernel<{epi}>"
     if storage == "bf16" and d > 128:
         return f"kchunk_bf16_kernel<{epi}>"
     return f"qreg_kernel<{storage}, {epi}>"

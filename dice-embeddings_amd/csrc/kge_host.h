@@ -112,11 +112,17 @@ inline RankWsOffsets rank_ws_offsets(int64_t B) {
   return o;
 }
 
+// tau: k-th best score per query; tau_scan: the threshold the next scan admits candidates with (tau, or a tighter
+// guess that the selection verifies); list: the best k so far as packed keys; cand: this round's candidates as packed
+// keys; cand_id: this round's candidates as entity ids (int8 filter scan, scored exactly before they are ranked);
+// rowmeta: one TOPK_ROWMETA_BYTES record per TOPK_ROWMETA_ROWS table rows (int8 filter scan)
+constexpr int TOPK_ROWMETA_ROWS = 64;
+constexpr int TOPK_ROWMETA_BYTES = 128;
 struct TopkWsOffsets {
-  size_t tau, cnt, list_len, dirty, n_dirty, list, cand, total;
+  size_t tau, tau_scan, cnt, list_len, dirty, n_dirty, list, cand, cand_id, rowmeta, total;
   int64_t kpad;
 };
-inline TopkWsOffsets topk_ws_offsets(int64_t B, int64_t k) {
+inline TopkWsOffsets topk_ws_offsets(int64_t B, int64_t N, int64_t k) {
   TopkWsOffsets o{};
   size_t off = 0;
   auto take = [&](size_t bytes) {
@@ -126,14 +132,37 @@ inline TopkWsOffsets topk_ws_offsets(int64_t B, int64_t k) {
   };
   o.kpad = (k + 7) / 8 * 8;
   o.tau = take((size_t)B * 4);
+  o.tau_scan = take((size_t)B * 4);
   o.cnt = take((size_t)B * 4);
   o.list_len = take((size_t)B * 4);
   o.dirty = take((size_t)B * 4);
   o.n_dirty = take(4);
   o.list = take((size_t)B * (size_t)o.kpad * 8);
   o.cand = take((size_t)B * TOPK_CAP * 8);
+  o.cand_id = take((size_t)B * TOPK_CAP * 4);
+  o.rowmeta = take((size_t)((N + TOPK_ROWMETA_ROWS - 1) / TOPK_ROWMETA_ROWS) * TOPK_ROWMETA_BYTES);
   o.total = off;
   return o;
+}
+
+// The threshold a scan of `n_next` more rows may use once `ranked` rows are ranked: the j-th best score so far, j as
+// small as the order statistics allow.  Of the best k of all ranked + n_next rows, the number X that are among
+// the rows already ranked is hypergeometric (rows in exchangeable order), mean k rho, variance below
+// k rho (1 - rho), rho = ranked / (ranked + n_next); the j-th best so far is below the final k-th best whenever
+// j > X.  Five standard deviations: a query in a few million falls short (the selection notices, and the query is
+// scanned again with its k-th best).
+inline int64_t topk_speculative_rank(int64_t k, int64_t ranked, int64_t n_next) {
+  if (n_next <= 0 || ranked <= 0) return k;
+  const double rho = (double)ranked / ((double)ranked + (double)n_next);
+  const double mean = (double)k * rho, var = (double)k * rho * (1.0 - rho);
+  double sd = 0.0;
+  for (double lo = 0.0, hi = var + 1.0; hi - lo > 1e-9;) {  // sqrt without <cmath>: bisection on [0, var + 1]
+    sd = 0.5 * (lo + hi);
+    if (sd * sd < var) lo = sd; else hi = sd;
+  }
+  int64_t j = (int64_t)(mean + 5.0 * sd) + 2;
+  if (j < 1) j = 1;
+  return j < k ? j : k;
 }
 
 inline size_t bce_ws_bytes() { return (2 * BCE_SLOTS + 1) * sizeof(double) + 248; }

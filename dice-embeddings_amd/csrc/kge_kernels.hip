@@ -1,6 +1,7 @@
 // Entry points of the contraction path: materialised scores, fused filtered rank, fused top-k and
 // fused multi-hot BCE, plus the small helper kernels around the two MFMA main loops.
 #include "kge_contract.hip.h"
+#include "kge_topk_i8.hip.h"
 
 #include <string.h>
 
@@ -607,27 +608,33 @@ using host::TOPK_MAX_K;
 using host::TOPK_FIRST_ROWS;  // first round takes everything: must not exceed TOPK_CAP
 
 struct TopkWs {
-  float* tau;
+  float* tau;       // k-th best score so far (-inf while fewer than k are known)
+  float* tau_scan;  // what the next scan admits candidates with: tau, or the tighter guess of select_finish
   int32_t* cnt;
   int32_t* list_len;
   int32_t* dirty;
   int32_t* n_dirty;
   unsigned long long* list;  // [B, kpad]
-  unsigned long long* cand;  // [B, TOPK_CAP]
+  unsigned long long* cand;  // [B, TOPK_CAP] packed keys
+  uint32_t* cand_id;         // [B, TOPK_CAP] entity ids (int8 filter scan; scored into `cand` before they are ranked)
+  unsigned char* rowmeta;    // int8 filter scan: per 64 table rows one record
   int64_t kpad;
 };
 
-size_t topk_ws_layout(int64_t B, int64_t k, void* base, TopkWs* ws) {
-  const host::TopkWsOffsets o = host::topk_ws_offsets(B, k);
+size_t topk_ws_layout(int64_t B, int64_t N, int64_t k, void* base, TopkWs* ws) {
+  const host::TopkWsOffsets o = host::topk_ws_offsets(B, N, k);
   if (ws) {
     char* p = (char*)base;
     ws->tau = (float*)(p + o.tau);
+    ws->tau_scan = (float*)(p + o.tau_scan);
     ws->cnt = (int32_t*)(p + o.cnt);
     ws->list_len = (int32_t*)(p + o.list_len);
     ws->dirty = (int32_t*)(p + o.dirty);
     ws->n_dirty = (int32_t*)(p + o.n_dirty);
     ws->list = (unsigned long long*)(p + o.list);
     ws->cand = (unsigned long long*)(p + o.cand);
+    ws->cand_id = (uint32_t*)(p + o.cand_id);
+    ws->rowmeta = (unsigned char*)(p + o.rowmeta);
     ws->kpad = o.kpad;
   }
   return o.total;
@@ -637,6 +644,7 @@ __global__ void topk_init_kernel(TopkWs w, int64_t B) {
   const int64_t b = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (b < B) {
     w.tau[b] = __uint_as_float(0xff800000u);  // -inf
+    w.tau_scan[b] = __uint_as_float(0xff800000u);
     w.cnt[b] = 0;
     w.list_len[b] = 0;
     w.dirty[b] = 0;
@@ -692,13 +700,29 @@ __device__ __forceinline__ void wave_sort_desc(unsigned long long (&v)[KPL], int
 // by the first launch has its candidate count reset, so the second one skips it.
 constexpr int SELECT_SMALL = 1024;
 
+// `th_used`: the threshold this round's scan admitted candidates with.  When it was a guess above the k-th best
+// (th_used > tau_old), the round is complete only if the merged k-th best still beats it: every entity above the
+// merged k-th best was then admitted.  Otherwise the query is flagged and scanned again at the end with its k-th best.
+// `spec_key`: the key at rank j_spec - 1 of the merged list (0: none): the next scan's guess is just below its score.
 __device__ __forceinline__ void select_finish(const TopkWs& w, int64_t b, int k, int rescan, bool over, int new_len,
-                                              bool have_tau, float tau) {
+                                              bool have_tau, float tau, float tau_old, float th_used,
+                                              unsigned long long spec_key) {
+  const float NINF = __uint_as_float(0xff800000u);
   w.list_len[b] = new_len;
-  w.tau[b] = have_tau ? tau : __uint_as_float(0xff800000u);
+  const float tau_new = have_tau ? tau : NINF;
+  w.tau[b] = tau_new;
+  float guess = tau_new;
+  if (have_tau && spec_key != 0) {
+    // one step below the score at that rank, so that its ties are admitted too
+    const uint32_t o = (uint32_t)(spec_key >> 32);
+    const float below = (o > 0) ? ordered_to_f32(o - 1) : NINF;
+    if (below > guess) guess = below;  // never below the k-th best; NaN leaves it
+  }
+  w.tau_scan[b] = rescan ? tau_new : guess;
   w.cnt[b] = 0;
+  const bool short_of_guess = th_used > tau_old && !(have_tau && tau > th_used);
   if (!rescan) {
-    if (over && !w.dirty[b]) {
+    if ((over || short_of_guess) && !w.dirty[b]) {
       w.dirty[b] = 1;
       atomicAdd(w.n_dirty, 1);
     }
@@ -708,9 +732,44 @@ __device__ __forceinline__ void select_finish(const TopkWs& w, int64_t b, int k,
   }
 }
 
+// Int8 filter scan: this round's candidates of every query are entity ids that passed a bound.  Their exact scores,
+// by the chain every score of an int8 table goes through, as packed keys into `cand`; 0 where the score does not
+// beat the threshold the scan worked with (the bound lets more through than that).  A wave takes 32 candidates of
+// one query at a time; grid (B, y): the waves of the y blocks of a query share its candidates out.
+__global__ void __launch_bounds__(256) topk_rescore_kernel(TopkWs w, ContractArgs a, int rescan) {
+  const int lane = threadIdx.x & 63, c = lane & 31, hf = lane >> 5;
+  const int64_t b = blockIdx.x;
+  if (rescan && !w.dirty[b]) return;
+  const int raw = w.cnt[b];
+  const int nc = raw < TOPK_CAP ? raw : TOPK_CAP;
+  const float th = rescan ? w.tau[b] : w.tau_scan[b];
+  const uint32_t* ids = w.cand_id + b * TOPK_CAP;
+  unsigned long long* out = w.cand + b * TOPK_CAP;
+  const int wid = blockIdx.y * 4 + (threadIdx.x >> 6), nw = gridDim.y * 4;
+  for (int j0 = 32 * wid; j0 < nc; j0 += 32 * nw) {
+    const int j = j0 + c;
+    const int64_t e = (j < nc) ? (int64_t)ids[j] : -1;
+    const bool ok = e >= 0 && e < a.N;
+    f32x16 acc = chain_direct<KGE_I8>(a.E, a.d, ok ? e : -1, a.Q, b, hf);
+    const int isel = ((c >> 3) << 2) | (c & 3);  // diagonal element (entity row c, query column c)
+    float v = 0.f;
+#pragma unroll
+    for (int i = 0; i < 16; ++i)
+      if (i == isel) v = acc[i];
+    if (hf == ((c >> 2) & 1) && j < nc) {
+      unsigned long long key = 0;
+      if (ok) {
+        const float sc = v * a.scale[e];
+        if (sc > th) key = ((unsigned long long)f32_to_ordered(sc) << 32) | (unsigned long long)(0xffffffffu - (uint32_t)e);
+      }
+      out[j] = key;
+    }
+  }
+}
+
 template <int KPL>
 __device__ __forceinline__ void select_in_registers(const TopkWs& w, int64_t b, int k, int rescan, int len, int nc,
-                                                    float tau_old, int lane) {
+                                                    float tau_old, float th_used, int j_spec, int lane) {
   unsigned long long v[KPL];
 #pragma unroll
   for (int s = 0; s < KPL; ++s) {
@@ -731,23 +790,28 @@ __device__ __forceinline__ void select_in_registers(const TopkWs& w, int64_t b, 
 #pragma unroll
   for (int o = 32; o >= 1; o >>= 1) valid += __shfl_xor(valid, o, 64);
   const int new_len = valid < k ? valid : k;
-  unsigned long long kth = 0;  // the key at position k - 1, if this wave holds that position
+  unsigned long long kth = 0, spec = 0;  // the keys at positions k - 1 and j_spec - 1, if this lane holds them
 #pragma unroll
   for (int s = 0; s < KPL; ++s) {
     const int i = lane * KPL + s;
     if (i < new_len) w.list[b * w.kpad + i] = v[s];
     if (i == k - 1) kth = v[s];
+    if (i == j_spec - 1 && i < new_len) spec = v[s];
   }
 #pragma unroll
-  for (int o = 32; o >= 1; o >>= 1) kth |= __shfl_xor(kth, o, 64);  // one lane at most holds it
+  for (int o = 32; o >= 1; o >>= 1) {  // one lane at most holds each
+    kth |= __shfl_xor(kth, o, 64);
+    spec |= __shfl_xor(spec, o, 64);
+  }
   if (lane == 0)
-    select_finish(w, b, k, rescan, false, new_len, new_len == k, ordered_to_f32((uint32_t)(kth >> 32)));
+    select_finish(w, b, k, rescan, false, new_len, new_len == k, ordered_to_f32((uint32_t)(kth >> 32)), tau_old, th_used,
+                  spec);
 }
 
 // Merge a query's kept list with this round's candidates, keep the best k, publish the new
 // threshold.  In `rescan` mode (only queries flagged dirty) list entries above the old threshold
 // are dropped first: the rescan finds all of them again.
-__global__ void __launch_bounds__(64) topk_select_wave_kernel(TopkWs w, int k, int rescan) {
+__global__ void __launch_bounds__(64) topk_select_wave_kernel(TopkWs w, int k, int rescan, int j_spec) {
   const int lane = threadIdx.x;
   const int64_t b = blockIdx.x;
   if (rescan && !w.dirty[b]) return;
@@ -755,13 +819,14 @@ __global__ void __launch_bounds__(64) topk_select_wave_kernel(TopkWs w, int k, i
   const int raw = w.cnt[b];
   if (raw > TOPK_CAP || len + raw > SELECT_SMALL) return;  // left to topk_select_kernel
   const float tau_old = w.tau[b];
+  const float th_used = rescan ? tau_old : w.tau_scan[b];
   if (len + raw <= 512)
-    select_in_registers<8>(w, b, k, rescan, len, raw, tau_old, lane);
+    select_in_registers<8>(w, b, k, rescan, len, raw, tau_old, th_used, j_spec, lane);
   else
-    select_in_registers<16>(w, b, k, rescan, len, raw, tau_old, lane);
+    select_in_registers<16>(w, b, k, rescan, len, raw, tau_old, th_used, j_spec, lane);
 }
 
-__global__ void __launch_bounds__(256) topk_select_kernel(TopkWs w, int k, int rescan) {
+__global__ void __launch_bounds__(256) topk_select_kernel(TopkWs w, int k, int rescan, int j_spec) {
   extern __shared__ unsigned long long keys[];
   __shared__ int s_valid;
   const int tid = threadIdx.x;
@@ -772,6 +837,7 @@ __global__ void __launch_bounds__(256) topk_select_kernel(TopkWs w, int k, int r
   const int nc = raw < TOPK_CAP ? raw : TOPK_CAP;
   const bool over = raw > TOPK_CAP;
   const float tau_old = w.tau[b];
+  const float th_used = rescan ? tau_old : w.tau_scan[b];
   const int n = len + nc;
   if (n <= SELECT_SMALL) return;  // ranked by topk_select_wave_kernel (which reset the candidate count)
   int npad = 2;
@@ -811,7 +877,8 @@ __global__ void __launch_bounds__(256) topk_select_kernel(TopkWs w, int k, int r
   const int new_len = n_valid < k ? n_valid : k;
   for (int i = tid; i < new_len; i += 256) w.list[b * w.kpad + i] = keys[i];
   if (tid == 0)
-    select_finish(w, b, k, rescan, over, new_len, new_len == k, ordered_to_f32((uint32_t)(keys[k - 1] >> 32)));
+    select_finish(w, b, k, rescan, over, new_len, new_len == k, ordered_to_f32((uint32_t)(keys[k - 1] >> 32)), tau_old,
+                  th_used, (j_spec >= 1 && j_spec <= new_len) ? keys[j_spec - 1] : 0ull);
 }
 
 __global__ void topk_output_kernel(TopkWs w, int64_t B, int k, const float* bias, int apply_sigmoid,
@@ -1048,6 +1115,34 @@ static int64_t contract_grid_wgs(const ContractArgs& a) {
   return (a.n_chunks < 8) ? a.n_chunks * a.n_qgroups : (a.n_chunks + 7) / 8 * 8 * a.n_qgroups;
 }
 
+// HIP events around a main-loop launch while kge_profile_begin() is in effect (the bench's per-launch timing)
+struct LaunchTimer {
+  hipEvent_t ev0 = nullptr, ev1 = nullptr;
+  hipStream_t st = nullptr;
+  bool timed = false;
+  int begin(hipStream_t stream) {
+    st = stream;
+    {
+      std::lock_guard<std::mutex> lk(g_prof_mu);
+      timed = g_prof_on;
+    }
+    if (timed) {
+      KGE_HIP_CHECK(hipEventCreate(&ev0));
+      KGE_HIP_CHECK(hipEventCreate(&ev1));
+      KGE_HIP_CHECK(hipEventRecord(ev0, st));
+    }
+    return KGE_OK;
+  }
+  int end() {
+    if (timed) {
+      KGE_HIP_CHECK(hipEventRecord(ev1, st));
+      std::lock_guard<std::mutex> lk(g_prof_mu);
+      g_prof_events.emplace_back(ev0, ev1);
+    }
+    return KGE_OK;
+  }
+};
+
 template <template <int> class EpiT, class EArgs>
 int launch_contract(int dtype, const ContractArgs& a, const EArgs& ea, hipStream_t st, const char* name) {
   if (a.B == 0 || a.e_end <= a.e_begin) return KGE_OK;
@@ -1058,17 +1153,8 @@ int launch_contract(int dtype, const ContractArgs& a, const EArgs& ea, hipStream
   const bool f32_split = (dtype == KGE_F32);
   const bool wide_bf16 = (dtype == KGE_BF16 && a.d > 128);
   dim3 grid((unsigned)nwg), block(fast_i8 ? 64 * I8_WG_WAVES : persistent ? 64 * QA_WG_WAVES : (f32_split || wide_bf16) ? 512 : 256);
-  hipEvent_t ev0 = nullptr, ev1 = nullptr;
-  bool timed = false;
-  {
-    std::lock_guard<std::mutex> lk(g_prof_mu);
-    timed = g_prof_on;
-  }
-  if (timed) {
-    KGE_HIP_CHECK(hipEventCreate(&ev0));
-    KGE_HIP_CHECK(hipEventCreate(&ev1));
-    KGE_HIP_CHECK(hipEventRecord(ev0, st));
-  }
+  LaunchTimer timer;
+  if (int trc = timer.begin(st)) return trc;
   const bool rows_aligned = (a.d % 4 == 0) && (((uintptr_t)a.E | (uintptr_t)a.Q) % 16 == 0);
   if (f32_split && rows_aligned)
     hipLaunchKernelGGL((ksplit_kernel<EpiT, true>), grid, block, 0, st, a, ea);
@@ -1090,11 +1176,7 @@ int launch_contract(int dtype, const ContractArgs& a, const EArgs& ea, hipStream
   else
     hipLaunchKernelGGL((qreg_kernel<KGE_I8, EpiT>), grid, block, 0, st, a, ea);
   KGE_LAUNCH_CHECK(name);
-  if (timed) {
-    KGE_HIP_CHECK(hipEventRecord(ev1, st));
-    std::lock_guard<std::mutex> lk(g_prof_mu);
-    g_prof_events.emplace_back(ev0, ev1);
-  }
+  if (int trc = timer.end()) return trc;
   return KGE_OK;
 }
 
@@ -1109,27 +1191,14 @@ int launch_ksplit(const ContractArgs& a, const EArgs& ea, unsigned k_splits, hip
   const bool rows_aligned = (ldq % 4 == 0) && (lde % 4 == 0) && (((uintptr_t)a.E | (uintptr_t)a.Q) % 16 == 0) &&
                             (a.k_split_len % 4 == 0);
   dim3 grid((unsigned)nwg, k_splits), block(512);
-  hipEvent_t ev0 = nullptr, ev1 = nullptr;
-  bool timed = false;
-  {
-    std::lock_guard<std::mutex> lk(g_prof_mu);
-    timed = g_prof_on;
-  }
-  if (timed) {
-    KGE_HIP_CHECK(hipEventCreate(&ev0));
-    KGE_HIP_CHECK(hipEventCreate(&ev1));
-    KGE_HIP_CHECK(hipEventRecord(ev0, st));
-  }
+  LaunchTimer timer;
+  if (int trc = timer.begin(st)) return trc;
   if (rows_aligned)
     hipLaunchKernelGGL((ksplit_kernel<EpiT, true>), grid, block, 0, st, a, ea);
   else
     hipLaunchKernelGGL((ksplit_kernel<EpiT, false>), grid, block, 0, st, a, ea);
   KGE_LAUNCH_CHECK(name);
-  if (timed) {
-    KGE_HIP_CHECK(hipEventRecord(ev1, st));
-    std::lock_guard<std::mutex> lk(g_prof_mu);
-    g_prof_events.emplace_back(ev0, ev1);
-  }
+  if (int trc = timer.end()) return trc;
   return KGE_OK;
 }
 
@@ -1414,11 +1483,11 @@ extern "C" int kge_rank_filtered_static(const float* Q, const float* bias, const
 }
 
 extern "C" size_t kge_topk_workspace_bytes(int64_t B, int64_t N, int64_t k) {
-  (void)N;
   if (B < 1) B = 1;
+  if (N < 1) N = 1;
   if (k < 1) k = 1;
   if (k > TOPK_MAX_K) k = TOPK_MAX_K;
-  return topk_ws_layout(B, k, nullptr, nullptr);
+  return topk_ws_layout(B, N, k, nullptr, nullptr);
 }
 
 extern "C" int kge_topk(const float* Q, const float* bias, const void* E, int dtype, const float* scale, int64_t B,
@@ -1434,44 +1503,83 @@ extern "C" int kge_topk(const float* Q, const float* bias, const void* E, int dt
   KGE_REQUIRE(out_scores && out_idx, KGE_ERR_INVALID, "kge_topk: null output pointer");
   KGE_REQUIRE(workspace && workspace_bytes >= kge_topk_workspace_bytes(B, N, k), KGE_ERR_WORKSPACE,
               "kge_topk: workspace of %zu bytes, need %zu", workspace_bytes, kge_topk_workspace_bytes(B, N, k));
-  KGE_REQUIRE(((uintptr_t)workspace & 7) == 0, KGE_ERR_WORKSPACE, "kge_topk: workspace must be 8-byte aligned");
+  KGE_REQUIRE(((uintptr_t)workspace & 15) == 0, KGE_ERR_WORKSPACE, "kge_topk: workspace must be 16-byte aligned");
   hipStream_t st = (hipStream_t)stream;
   TopkWs ws;
-  topk_ws_layout(B, k, workspace, &ws);
+  topk_ws_layout(B, N, k, workspace, &ws);
   hipLaunchKernelGGL(topk_init_kernel, dim3((unsigned)((B + 255) / 256)), dim3(256), 0, st, ws, B);
   KGE_LAUNCH_CHECK("topk_init_kernel");
 
-  // ranks the list (<= k entries) and this round's candidates (<= min(TOPK_CAP, rows scanned) entries) of every query
-  auto launch_select = [&](int64_t rows, int rescan) {
-    hipLaunchKernelGGL(topk_select_wave_kernel, dim3((unsigned)B), dim3(64), 0, st, ws, (int)k, rescan);
+  // An int8 table with d == 128 is scanned by the integer filter (after the first round, which takes every row
+  // anyway): its candidates are entity ids that passed a bound, scored exactly before they are ranked.  Every other
+  // scan is the contraction's own top-k epilogue, whose candidates are exact keys.
+  const bool id_filter = (dtype == KGE_I8 && d == 128 && N > TOPK_FIRST_ROWS);
+  if (id_filter) {
+    const int64_t n_rec = (N + host::TOPK_ROWMETA_ROWS - 1) / host::TOPK_ROWMETA_ROWS;
+    hipLaunchKernelGGL(topk_i8_rowmeta_kernel, dim3((unsigned)((n_rec + 3) / 4)), dim3(256), 0, st, (const int8_t*)E,
+                       scale, N, ws.rowmeta);
+    KGE_LAUNCH_CHECK("topk_i8_rowmeta_kernel");
+  }
+  // One scan of entity rows [e0, e1) with the thresholds `tau`, for all queries or those flagged in `active`.
+  auto launch_scan = [&](int64_t e0, int64_t e1, const float* tau, const int32_t* active, int rescan,
+                         const char* name) -> int {
+    ContractArgs a = make_args(Q, E, dtype, scale, B, d, N, e0, e1);
+    if (!id_filter || e0 % host::TOPK_ROWMETA_ROWS != 0 || (e0 == 0 && e1 <= TOPK_FIRST_ROWS)) {
+      TopkArgs ea{tau, active, ws.cnt, ws.cand, TOPK_CAP};
+      return launch_contract<TopkEpi>(dtype, a, ea, st, name);
+    }
+    if (e1 <= e0) return KGE_OK;
+    // the filter's workgroups cover TF_WG_QUERIES queries, one workgroup per CU: the same walk, its own shape
+    a.n_qgroups = (int)((B + TF_WG_QUERIES - 1) / TF_WG_QUERIES);
+    a.n_lanes = 32 / a.n_qgroups;
+    if (a.n_lanes < 1) a.n_lanes = 1;
+    int64_t chunk = (e1 - e0) / (8 * (int64_t)a.n_lanes * 4);
+    chunk = (chunk + TF_STAGE_ROWS - 1) / TF_STAGE_ROWS * TF_STAGE_ROWS;
+    if (chunk < TF_STAGE_ROWS) chunk = TF_STAGE_ROWS;
+    if (chunk > 1024) chunk = 1024;
+    a.chunk_rows = (int)chunk;
+    a.n_chunks = (e1 - e0 + chunk - 1) / chunk;
+    const int64_t nwg = 8 * (int64_t)a.n_qgroups * a.n_lanes;
+    KGE_REQUIRE(nwg <= 0x7fffffffLL, KGE_ERR_INVALID, "%s: grid of %lld workgroups too large", name, (long long)nwg);
+    I8FilterArgs ea{tau, active, ws.cnt, ws.cand_id, TOPK_CAP, ws.rowmeta};
+    LaunchTimer timer;
+    if (int trc = timer.begin(st)) return trc;
+    hipLaunchKernelGGL(topk_i8_filter_kernel, dim3((unsigned)nwg), dim3(64 * TF_W), 0, st, a, ea);
+    KGE_LAUNCH_CHECK(name);
+    if (int trc = timer.end()) return trc;
+    hipLaunchKernelGGL(topk_rescore_kernel, dim3((unsigned)B, 4), dim3(256), 0, st, ws, a, rescan);
+    KGE_LAUNCH_CHECK("topk_rescore_kernel");
+    return KGE_OK;
+  };
+  // ranks the list (<= k entries) and this round's candidates (<= min(TOPK_CAP, rows scanned) entries) of every
+  // query; j_spec: the rank whose score the next scan may use as its threshold (k: the k-th best itself)
+  auto launch_select = [&](int64_t rows, int rescan, int64_t j_spec) {
+    hipLaunchKernelGGL(topk_select_wave_kernel, dim3((unsigned)B), dim3(64), 0, st, ws, (int)k, rescan, (int)j_spec);
     if (k + (rows < TOPK_CAP ? rows : TOPK_CAP) > SELECT_SMALL)  // kpad (<= 1024) + TOPK_CAP, padded to a power of two
       hipLaunchKernelGGL(topk_select_kernel, dim3((unsigned)B), dim3(256), 8192 * sizeof(unsigned long long), st, ws,
-                         (int)k, rescan);
+                         (int)k, rescan, (int)j_spec);
   };
   const int64_t growth = (k <= 256) ? 4 : 2;  // round r scans (growth - 1) x what is already ranked
   int64_t e0 = 0, e1 = (N < TOPK_FIRST_ROWS) ? N : TOPK_FIRST_ROWS;
   while (e0 < N) {
-    ContractArgs a = make_args(Q, E, dtype, scale, B, d, N, e0, e1);
-    TopkArgs ea{ws.tau, nullptr, ws.cnt, ws.cand, TOPK_CAP};
-    rc = launch_contract<TopkEpi>(dtype, a, ea, st, "kge_topk scan");
+    rc = launch_scan(e0, e1, ws.tau_scan, nullptr, 0, "kge_topk scan");
     if (rc) return rc;
-    launch_select(e1 - e0, 0);
+    int64_t next = e1 * growth;
+    next = (next < N) ? next : N;
+    launch_select(e1 - e0, 0, host::topk_speculative_rank(k, e1, next - e1));
     KGE_LAUNCH_CHECK("topk_select_kernel");
     e0 = e1;
-    int64_t next = e1 * growth;
-    e1 = (next < N) ? next : N;
+    e1 = next;
   }
-  // queries whose candidate buffer overflowed in some round lost entries: rescan with their final
-  // (tight) threshold until nothing overflows.
+  // queries whose candidate buffer overflowed in some round, or whose guessed threshold turned out too high, lost
+  // entries: scan again with their final k-th best (a valid, tight threshold) until nothing overflows.
   int32_t n_dirty = 0;
   KGE_HIP_CHECK(hipMemcpyAsync(&n_dirty, ws.n_dirty, sizeof(int32_t), hipMemcpyDeviceToHost, st));
   KGE_HIP_CHECK(hipStreamSynchronize(st));
   for (int iter = 0; n_dirty > 0 && iter < 16; ++iter) {
-    ContractArgs a = make_args(Q, E, dtype, scale, B, d, N, 0, N);
-    TopkArgs ea{ws.tau, ws.dirty, ws.cnt, ws.cand, TOPK_CAP};
-    rc = launch_contract<TopkEpi>(dtype, a, ea, st, "kge_topk rescan");
+    rc = launch_scan(0, N, ws.tau, ws.dirty, 1, "kge_topk rescan");
     if (rc) return rc;
-    launch_select(N, 1);
+    launch_select(N, 1, k);
     KGE_LAUNCH_CHECK("topk_select_kernel");
     KGE_HIP_CHECK(hipMemcpyAsync(&n_dirty, ws.n_dirty, sizeof(int32_t), hipMemcpyDeviceToHost, st));
     KGE_HIP_CHECK(hipStreamSynchronize(st));
@@ -1640,3 +1748,4 @@ extern "C" int kge_bce_multihot_backward(const float* Q, const float* bias, cons
   }
   return KGE_OK;
 }
+

@@ -1,0 +1,391 @@
+// Top-k over a per-row int8 table, d == 128: the scan as an integer filter.
+//
+// A round of kge_topk only has to find the entities whose score beats the query's threshold tau; nearly all of
+// the B x N scores do not.  The scan therefore works on a bound that is cheap to form:
+//   * the query row is rounded to bf16 (qb, the operand of the exact score) and then quantised once more to
+//     int8, qb = s_q * qh + delta with |delta| <= dq;  H = sum_k e_k qh_k is an exact int32 from the int8 MFMA
+//     (32x32x32, twice the bf16 rate, and the table rows go global -> LDS untouched);
+//   * the exact raw score A = fl(sum_k e_k qb_k) obeys |A - s_q H| <= mq L1(e), with L1(e) = sum_k |e_k| and mq = dq + 4e-3 s_q (the second term covers the fp32 rounding of the
+//     exact chain, at most 128 * 2^-23 * 127 s_q L1(e) = 1.9e-3 s_q L1(e), and of this bound's own arithmetic);
+//   * the row scale s_e is written unit * (m_e + r), unit = (largest scale of the 32-row tile) / 255, m_e an
+//     integer in [0, 255], |r| <= 0.51, so that  score = s_e A <= s_q unit (m_e H + 64.8 max L1) + mq max(s_e L1(e))
+//     (|H| <= 127 L1): per element one 24-bit integer multiply, per tile and lane one maximum and a few float
+//     operations.  A tile none of whose lanes can beat its query's tau is passed over; in the others the products
+//     are formed again and compared with the threshold turned into an integer.
+// An element that passes is only a candidate: its entity id goes to the query's candidate buffer, and the
+// selection kernel recomputes its score with the exact chain (the one kge_scores uses) and compares that with
+// tau.  So the filter decides nothing about the result, it only has to let every true candidate through.
+//
+// What the bound needs of the table (m_e per row; unit, max s_e L1(e), 64.8 max L1 and a "some scale is negative
+// or not finite" flag per 32-row tile) does not depend on the queries: topk_i8_rowmeta_kernel writes it once per
+// call, one 128-byte record per 64 rows, and the scan loads a stage's record with the stage.
+//
+// Pipeline: the persistent XCD-aware walk and the three-buffer global -> LDS ring of qstream_kernel, 64-row
+// stages of 8 KB, one barrier per stage; a tile's test runs under the next tile's MFMA chain.  Candidate ids are
+// parked in per-query LDS buckets and leave for global memory as one run per query when the workgroup ends.
+#pragma once
+#include "kge_contract.hip.h"
+
+namespace kge {
+
+typedef __attribute__((ext_vector_type(4))) int i32x4;
+typedef __attribute__((ext_vector_type(16))) int i32x16;
+
+struct I8FilterArgs {
+  const float* tau;       // per query: k-th best exact score so far (-inf while fewer than k known)
+  const int32_t* active;  // NULL = all queries; else only queries with active[b] != 0 collect
+  int32_t* cnt;           // per query: candidates appended this round
+  uint32_t* cand;         // [B, cap] candidate entity ids
+  int32_t cap;
+  const unsigned char* rowmeta;  // one record per 64 table rows (topk_i8_rowmeta_kernel)
+};
+
+constexpr int TF_NQT = 4;                              // 32-query tiles per wave
+constexpr int TF_W = 8;                                // waves per workgroup
+constexpr int TF_WG_QUERIES = TF_W * 32 * TF_NQT;      // 1024
+constexpr int TF_STAGE_ROWS = 64;
+constexpr int TF_STAGE_BYTES = TF_STAGE_ROWS * 128;    // 8 KB of int8 rows
+constexpr int TF_NBUF = 3;
+constexpr int TF_BUCKET = 16;                          // candidate ids a query can park in LDS
+constexpr int TF_VALU_PER_MFMA = 5;
+
+// One candidate id into its query's global buffer; slot is the query's running count.  A full buffer keeps a
+// uniform sample of what arrives (the query is repaired by a later rescan with its final threshold).
+__device__ __forceinline__ void tf_place(const I8FilterArgs& a, int64_t q, int32_t slot, uint32_t e) {
+  if (slot >= a.cap) {
+    uint32_t h = (e * 2654435761u) ^ ((uint32_t)slot * 0x9e3779b9u);
+    h ^= h >> 15; h *= 0x2c1b3c6du; h ^= h >> 12;
+    const uint32_t r = h % (uint32_t)(slot + 1);
+    slot = (r < (uint32_t)a.cap) ? (int32_t)r : -1;
+  }
+  if (slot >= 0) a.cand[q * a.cap + slot] = e;
+}
+
+// Per 64 table rows one record for the scan (layout: meta_lds in topk_i8_filter_kernel).  One wave per record, one
+// lane per row.  A row past the table's end counts for nothing; a negative or non-finite scale forces its tile.
+__global__ void __launch_bounds__(256) topk_i8_rowmeta_kernel(const int8_t* E, const float* scale, int64_t N,
+                                                              unsigned char* meta) {
+  const int lane = threadIdx.x & 63;
+  const int64_t rec = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (rec * 64 >= N) return;
+  const int64_t row = rec * 64 + lane;
+  const bool in = row < N;
+  uint32_t sad = 0;
+  float sc = 0.f;
+  if (in) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const u32x4 w = *(const u32x4*)(E + row * 128 + 16 * j);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) sad = __builtin_amdgcn_sad_u8(w[i] ^ 0x80808080u, 0x80808080u, sad);  // sum |int8|
+    }
+    sc = scale[row];
+  }
+  const float l1 = (float)sad;
+  const bool bad = in && !(sc >= 0.f && sc <= 3.4028234e38f);
+  const float scv = (in && !bad) ? sc : 0.f;
+  float l1M = l1, sM = scv, wM = scv * l1, fM = bad ? 1.f : 0.f;
+#pragma unroll
+  for (int o = 1; o <= 16; o <<= 1) {
+    l1M = __builtin_fmaxf(l1M, __shfl_xor(l1M, o, 64));
+    sM = __builtin_fmaxf(sM, __shfl_xor(sM, o, 64));
+    wM = __builtin_fmaxf(wM, __shfl_xor(wM, o, 64));
+    fM = __builtin_fmaxf(fM, __shfl_xor(fM, o, 64));
+  }
+  float m = (sM > 0.f) ? __builtin_rintf(255.f * scv / sM) : 0.f;
+  m = __builtin_fminf(__builtin_fmaxf(m, 0.f), 255.f);
+  const int et = lane >> 5, r = lane & 31;
+  unsigned char* out = meta + rec * host::TOPK_ROWMETA_BYTES;
+  out[(et * 2 + ((r >> 2) & 1)) * 16 + 4 * (r >> 3) + (r & 3)] = (unsigned char)(int)m;
+  if (r == 0) {
+    const f32x4 tc = {sM / 255.f, wM, 64.8f * l1M, fM};
+    *(f32x4*)(out + 64 + 16 * et) = tc;
+  }
+}
+
+__global__ void __launch_bounds__(64 * TF_W, 2) topk_i8_filter_kernel(ContractArgs a, I8FilterArgs ea) {
+  constexpr int NQT = TF_NQT, W = TF_W, WQ = TF_WG_QUERIES;
+  __shared__ __attribute__((aligned(1024))) unsigned char lds_e[TF_NBUF * TF_STAGE_BYTES];
+  // the stage's record: multipliers m_e as bytes in the order a lane's accumulators hold them ([tile][half][16]),
+  // then per tile {unit, max s L1, 64.8 max L1, forced}
+  __shared__ __attribute__((aligned(16))) unsigned char meta_lds[TF_NBUF][host::TOPK_ROWMETA_BYTES];
+  __shared__ uint32_t bucket[WQ * TF_BUCKET];
+  __shared__ int bcnt[WQ];
+
+  const int64_t wg = blockIdx.x;
+  const int xcd = (int)(wg & 7);
+  const int64_t slot = wg >> 3;
+  const int qg = (int)(slot % a.n_qgroups);
+  const int wlane = (int)(slot / a.n_qgroups);
+  const int tid = threadIdx.x, lane = tid & 63, c = lane & 31, hf = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  constexpr int d = 128;
+  const int64_t q_wg = (int64_t)qg * WQ;
+  const int ql0 = wave * (32 * NQT);
+  const float INF = __uint_as_float(0x7f800000u);
+
+  const int64_t c_first = xcd + 8 * (int64_t)wlane;
+  const int64_t c_stride = 8 * (int64_t)a.n_lanes;
+  if (c_first >= a.n_chunks) return;
+  const int my_chunks = (int)((a.n_chunks - 1 - c_first) / c_stride) + 1;
+  const int spc = a.chunk_rows / TF_STAGE_ROWS;
+  const int64_t r_end = a.e_end;
+  const int64_t row_first = a.e_begin + c_first * a.chunk_rows;
+  const int64_t row_last_chunk = row_first + c_stride * (int64_t)(my_chunks - 1) * a.chunk_rows;
+  int valid_last = (int)((r_end - row_last_chunk + TF_STAGE_ROWS - 1) / TF_STAGE_ROWS);
+  valid_last = valid_last < spc ? valid_last : spc;
+  const int n_st = (my_chunks - 1) * spc + valid_last;
+  const int64_t chunk_skip = (c_stride - 1) * (int64_t)a.chunk_rows;
+
+  for (int i = tid; i < WQ; i += 64 * W) bcnt[i] = 0;
+
+  // ---- the queries of this lane: int8 fragments and the constants of the bound ------------------
+  i32x4 qf[NQT][4];
+  float sq[NQT], mq[NQT], tau_lo[NQT];
+#pragma unroll
+  for (int t = 0; t < NQT; ++t) {
+    const int64_t q = q_wg + ql0 + 32 * t + c;
+    float xb[64];  // bf16-rounded components k = 32 s + 16 hf + j of the row
+    float amax = 0.f;
+    bool has_nan = false;
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+#pragma unroll
+      for (int j4 = 0; j4 < 4; ++j4) {
+        f32x4 v = {0.f, 0.f, 0.f, 0.f};
+        if (q < a.B) v = *(const f32x4*)(a.Q + q * d + 32 * s + 16 * hf + 4 * j4);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const float r = (float)(__bf16)v[j];
+          xb[16 * s + 4 * j4 + j] = r;
+          amax = __builtin_fmaxf(amax, __builtin_fabsf(r));
+          has_nan = has_nan || (r != r);  // fmax drops a NaN
+        }
+      }
+    }
+    amax = __builtin_fmaxf(amax, __shfl_xor(amax, 32, 64));
+    has_nan = has_nan || (__shfl_xor((int)has_nan, 32, 64) != 0);
+    const bool finite = !has_nan && amax <= 3.4028234e38f;
+    const float s_q = finite ? amax / 127.f : 0.f;
+    const float inv = (finite && amax > 0.f) ? 127.f / amax : 0.f;
+    float dq = 0.f;
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+      i32x4 w;
+#pragma unroll
+      for (int j4 = 0; j4 < 4; ++j4) {
+        uint32_t pk = 0;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const float r = finite ? xb[16 * s + 4 * j4 + j] : 0.f;
+          float h = __builtin_rintf(r * inv);
+          h = __builtin_fminf(__builtin_fmaxf(h, -127.f), 127.f);
+          dq = __builtin_fmaxf(dq, __builtin_fabsf(__builtin_fmaf(-s_q, h, r)));
+          pk |= ((uint32_t)(int)h & 0xffu) << (8 * j);
+        }
+        w[j4] = (int)pk;
+      }
+      qf[t][s] = w;
+    }
+    dq = __builtin_fmaxf(dq, __shfl_xor(dq, 32, 64));
+    sq[t] = s_q;
+    mq[t] = dq * 1.000001f + 4e-3f * s_q;
+    // a query with a non-finite component has no finite bound: it collects nothing (its scores are NaN or
+    // infinite anyway)
+    const bool on = q < a.B && finite && (ea.active == nullptr || ea.active[q] != 0);
+    float th = INF;
+    if (on) {
+      th = ea.tau[q];
+      if (th > -INF && th < INF) th = th - 1e-6f * __builtin_fabsf(th);  // the comparison's own rounding
+    }
+    tau_lo[t] = th;
+  }
+
+  // ---- staging: thread `tid` owns 16-byte slot `tid` of every stage -------------------------------
+  // slot = row * 8 + (piece ^ ((row >> 1) & 7)): the 16 rows a fragment read touches at a time fall on distinct
+  // bank groups.  Rows past the table's end repeat its last row (their entities are >= limit and are ignored).
+  const int lrow = tid >> 3;
+  const int lpiece = (tid & 7) ^ ((lrow >> 1) & 7);
+  const unsigned char* Eb = (const unsigned char*)a.E;
+  auto stage_issue = [&](int64_t row0, int buf) {
+    int64_t g = row0 + lrow;
+    g = (g < r_end) ? g : r_end - 1;
+    unsigned char* dst = lds_e + buf * TF_STAGE_BYTES + wave * 1024;
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(Eb + g * 128 + lpiece * 16),
+                                     (__attribute__((address_space(3))) void*)dst, 16, 0, 0);
+    if (wave == 0 && lane < host::TOPK_ROWMETA_BYTES / 4)  // row0 is a multiple of 64: the stage's record
+      __builtin_amdgcn_global_load_lds(
+          (const __attribute__((address_space(1))) void*)(ea.rowmeta + (row0 >> 6) * host::TOPK_ROWMETA_BYTES + lane * 4),
+          (__attribute__((address_space(3))) void*)&meta_lds[buf][0], 4, 0, 0);
+  };
+  int64_t issue_row = row_first;
+  int issue_so = 0;
+  auto issue_advance = [&]() {
+    issue_row += TF_STAGE_ROWS;
+    if (++issue_so == spc) {
+      issue_so = 0;
+      issue_row += chunk_skip;
+    }
+  };
+  int foff[4];
+#pragma unroll
+  for (int s = 0; s < 4; ++s) foff[s] = c * 128 + (((2 * s + hf) ^ ((c >> 1) & 7)) << 4);
+
+  // ---- the test of one finished tile ------------------------------------------------------------
+  // constants of the entity tile the finished accumulators belong to
+  u32x4 m_mul = {0u, 0u, 0u, 0u};
+  float m_unit = 0.f, m_W = 0.f, m_c2 = 0.f;
+  bool m_force = false;
+  int64_t e_prev = r_end;
+  auto tile_meta = [&](int buf, int et) {
+    m_mul = *(const u32x4*)&meta_lds[buf][(et * 2 + hf) * 16];
+    const f32x4 tc = *(const f32x4*)&meta_lds[buf][64 + 16 * et];
+    m_unit = tc[0];
+    m_W = tc[1];
+    m_c2 = tc[2];
+    m_force = tc[3] != 0.f;
+  };
+  auto product = [&](const i32x16& h, int i) -> int {
+    return __mul24(h[i], (int)((m_mul[i >> 2] >> (8 * (i & 3))) & 0xffu));
+  };
+  auto tile_test = [&](int t, const i32x16& h) {
+    int pm = product(h, 0);
+#pragma unroll
+    for (int i = 1; i < 16; ++i) {
+      const int p = product(h, i);
+      pm = pm > p ? pm : p;
+    }
+    const float su = sq[t] * m_unit, mw = mq[t] * m_W;
+    const float Bd = __builtin_fmaf(su, (float)pm + m_c2, mw);
+    const bool hit = (Bd > tau_lo[t]) || (m_force && tau_lo[t] < INF);
+    if (__builtin_expect(__builtin_amdgcn_ballot_w64(hit) != 0, 0)) {
+      // The same products against the threshold as an integer: su (P + c2) + mw > tau  <=>  P > (tau - mw) / su - c2,
+      // lowered by its own rounding and kept inside +-2^30 (|P| < 2^29) so that the difference below cannot wrap.
+      float x;
+      if (m_force && tau_lo[t] < INF)
+        x = -INF;
+      else if (su > 0.f) {
+        x = (tau_lo[t] - mw) / su - m_c2;
+        x = x - 1e-5f * __builtin_fabsf(x) - 1.f;
+      } else
+        x = (mw > tau_lo[t]) ? -INF : INF;
+      x = __builtin_fminf(__builtin_fmaxf(x, -1073741824.f), 1073741824.f);
+      const int thr = (x == x) ? (int)x : -1073741824;
+      uint32_t bits = 0;  // bit 15 - i: element i may beat the threshold
+#pragma unroll
+      for (int i = 0; i < 16; ++i) bits = __builtin_amdgcn_alignbit(bits, (uint32_t)(thr - product(h, i)), 31);
+      const int qlocal = ql0 + 32 * t + c;
+      while (__builtin_amdgcn_ballot_w64(bits != 0) != 0) {
+        if (bits != 0) {
+          const int b = 31 - __builtin_clz(bits);
+          bits &= ~(1u << b);
+          const int i = 15 - b;
+          const int64_t e = e_prev + ((i >> 2) << 3) + (hf << 2) + (i & 3);
+          if (e < r_end) {
+            const int idx = atomicAdd(&bcnt[qlocal], 1);
+            if (idx < TF_BUCKET)
+              bucket[qlocal * TF_BUCKET + idx] = (uint32_t)e;
+            else  // bucket full: straight to global memory
+              tf_place(ea, q_wg + qlocal, atomicAdd(&ea.cnt[q_wg + qlocal], 1), (uint32_t)e);
+          }
+        }
+      }
+    }
+  };
+
+  // A barrier that orders nothing but the waves: the loads it guards are waited for explicitly.
+  auto wg_barrier = [&]() {
+    __builtin_amdgcn_sched_barrier(0);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
+  };
+
+  stage_issue(issue_row, 0);
+  issue_advance();
+  stage_issue(issue_row, 1);
+  issue_advance();
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the cleared bucket counts
+  wg_barrier();
+  i32x4 ef[4];
+#pragma unroll
+  for (int s = 0; s < 4; ++s) ef[s] = *(const i32x4*)(lds_e + foff[s]);
+
+  // the first test has no tile to work on: e_prev past the limit keeps whatever it finds out of the buckets
+  i32x16 acc_prev;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) acc_prev[i] = 0;
+  int64_t row0 = row_first;
+  int so = 0;
+
+  auto run_stage = [&](auto bufc, int k) {
+    constexpr int BUF = decltype(bufc)::value;
+    constexpr int NEXT = (BUF + 1) % TF_NBUF, NEXT2 = (BUF + 2) % TF_NBUF;
+#pragma unroll
+    for (int et = 0; et < 2; ++et) {
+      if (et == 1) {
+        // stage k + 1 has landed for every wave, and everyone is done with the buffer of stage k - 1, which takes
+        // the loads of stage k + 2
+        wg_barrier();
+        stage_issue(issue_row, NEXT2);
+        if (k + 3 < n_st) issue_advance();
+      }
+      const int roff = (et == 0) ? BUF * TF_STAGE_BYTES + 4096 : NEXT * TF_STAGE_BYTES;
+#pragma unroll
+      for (int t = 0; t < NQT; ++t) {
+        const int t_prev = (t + NQT - 1) % NQT;
+        const bool refill = (t == NQT - 1);
+        i32x16 acc;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[i] = 0;
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+          acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(ef[s], qf[t][s], acc, 0, 0, 0);
+          if (refill) ef[s] = *(const i32x4*)(lds_e + roff + foff[s]);
+        }
+        tile_test(t_prev, acc_prev);
+        if (t == 0) {  // from here on the finished tiles belong to this entity tile
+          tile_meta(BUF, et);
+          e_prev = row0 + et * 32;
+        }
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x002, TF_VALU_PER_MFMA, 0);
+          if (refill) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        }
+        acc_prev = acc;
+      }
+    }
+    row0 += TF_STAGE_ROWS;
+    if (++so == spc) {
+      so = 0;
+      row0 += chunk_skip;
+    }
+  };
+  for (int k = 0;;) {
+    run_stage(std::integral_constant<int, 0>{}, k);
+    if (++k >= n_st) break;
+    run_stage(std::integral_constant<int, 1>{}, k);
+    if (++k >= n_st) break;
+    run_stage(std::integral_constant<int, 2>{}, k);
+    if (++k >= n_st) break;
+  }
+  tile_test(NQT - 1, acc_prev);
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // no load may land in LDS after the workgroup has gone
+
+  // ---- the parked candidates of every query leave as one run ---------------------------------------
+  __syncthreads();
+  for (int i = tid; i < WQ; i += 64 * W) {
+    const int64_t q = q_wg + i;
+    int n = bcnt[i];
+    n = n < TF_BUCKET ? n : TF_BUCKET;
+    if (n > 0 && q < a.B) {
+      const int32_t base = atomicAdd(&ea.cnt[q], n);
+      for (int j = 0; j < n; ++j) tf_place(ea, q, base + j, bucket[i * TF_BUCKET + j]);
+    }
+  }
+}
+
+}  // namespace kge

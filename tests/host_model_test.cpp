@@ -75,12 +75,31 @@ static void test_layouts() {
     }
     check_disjoint(parts, r.total);
     for (int64_t k : {1LL, 7LL, 8LL, 100LL, 1024LL}) {
-      const TopkWsOffsets t = topk_ws_offsets(B, k);
-      CHECK(t.kpad >= k && t.kpad % 8 == 0 && t.kpad < k + 8);
-      check_disjoint({{t.tau, (size_t)B * 4}, {t.cnt, (size_t)B * 4}, {t.list_len, (size_t)B * 4}, {t.dirty, (size_t)B * 4},
-                      {t.n_dirty, 4}, {t.list, (size_t)B * t.kpad * 8}, {t.cand, (size_t)B * TOPK_CAP * 8}}, t.total);
+      for (int64_t N : {1LL, 63LL, 64LL, 65LL, 10000000LL}) {
+        const TopkWsOffsets t = topk_ws_offsets(B, N, k);
+        CHECK(t.kpad >= k && t.kpad % 8 == 0 && t.kpad < k + 8);
+        const size_t n_rec = (size_t)((N + TOPK_ROWMETA_ROWS - 1) / TOPK_ROWMETA_ROWS);
+        CHECK((int64_t)n_rec * TOPK_ROWMETA_ROWS >= N);
+        check_disjoint({{t.tau, (size_t)B * 4}, {t.tau_scan, (size_t)B * 4}, {t.cnt, (size_t)B * 4},
+                        {t.list_len, (size_t)B * 4}, {t.dirty, (size_t)B * 4}, {t.n_dirty, 4},
+                        {t.list, (size_t)B * t.kpad * 8}, {t.cand, (size_t)B * TOPK_CAP * 8},
+                        {t.cand_id, (size_t)B * TOPK_CAP * 4}, {t.rowmeta, n_rec * TOPK_ROWMETA_BYTES}}, t.total);
+      }
     }
   }
+  // the rank whose score a scan may use as its threshold: between the expected number of survivors and k
+  for (int64_t k : {1LL, 10LL, 100LL, 1000LL}) {
+    CHECK(topk_speculative_rank(k, 0, 1000) == k && topk_speculative_rank(k, 1000, 0) == k);
+    int64_t prev = 0;
+    for (int64_t ranked : {1024LL, 4096LL, 1LL << 20}) {
+      const int64_t j = topk_speculative_rank(k, ranked, 3 * ranked);
+      CHECK(j >= 1 && j <= k && 4 * j >= k);             // never below the mean k / 4
+      CHECK(prev == 0 || j == prev);                     // depends on the ratio only
+      prev = j;
+    }
+    CHECK(topk_speculative_rank(k, 1 << 20, 1) == k || k > 20);   // almost nothing left to scan: nearly all survive
+  }
+  CHECK(topk_speculative_rank(100, 4096, 3 * 4096) == 48);        // 25 + 5 sqrt(18.75) = 46.65 -> 48
   // the static scratch array of kge_rank_filtered_static holds the layout of its largest batch
   CHECK(rank_ws_offsets(KGE_RANK_STATIC_MAX_B).total <= KGE_RANK_STATIC_SCRATCH_BYTES);
   CHECK(TOPK_FIRST_ROWS <= TOPK_CAP);
