@@ -117,7 +117,7 @@ inline RankWsOffsets rank_ws_offsets(int64_t B) {
 // keys; cand_id: this round's candidates as entity ids (int8 filter scan, scored exactly before they are ranked);
 // rowmeta: one TOPK_ROWMETA_BYTES record per TOPK_ROWMETA_ROWS table rows (int8 filter scan)
 constexpr int TOPK_ROWMETA_ROWS = 64;
-constexpr int TOPK_ROWMETA_BYTES = 128;
+constexpr int TOPK_ROWMETA_BYTES = 160;  // 64 int16 multipliers, then {unit, max |s| L1, c2, forced} per 32-row tile
 struct TopkWsOffsets {
   size_t tau, tau_scan, cnt, list_len, dirty, n_dirty, list, cand, cand_id, rowmeta, total;
   int64_t kpad;

@@ -736,13 +736,12 @@ __device__ __forceinline__ void select_finish(const TopkWs& w, int64_t b, int k,
 // by the chain every score of an int8 table goes through, as packed keys into `cand`; 0 where the score does not
 // beat the threshold the scan worked with (the bound lets more through than that).  A wave takes 32 candidates of
 // one query at a time; grid (B, y): the waves of the y blocks of a query share its candidates out.
-__global__ void __launch_bounds__(256) topk_rescore_kernel(TopkWs w, ContractArgs a, int rescan) {
+__global__ void __launch_bounds__(256) topk_rescore_kernel(TopkWs w, ContractArgs a) {
   const int lane = threadIdx.x & 63, c = lane & 31, hf = lane >> 5;
   const int64_t b = blockIdx.x;
-  if (rescan && !w.dirty[b]) return;
   const int raw = w.cnt[b];
   const int nc = raw < TOPK_CAP ? raw : TOPK_CAP;
-  const float th = rescan ? w.tau[b] : w.tau_scan[b];
+  const float th = w.tau_scan[b];
   const uint32_t* ids = w.cand_id + b * TOPK_CAP;
   unsigned long long* out = w.cand + b * TOPK_CAP;
   const int wid = blockIdx.y * 4 + (threadIdx.x >> 6), nw = gridDim.y * 4;
@@ -1524,7 +1523,9 @@ extern "C" int kge_topk(const float* Q, const float* bias, const void* E, int dt
   auto launch_scan = [&](int64_t e0, int64_t e1, const float* tau, const int32_t* active, int rescan,
                          const char* name) -> int {
     ContractArgs a = make_args(Q, E, dtype, scale, B, d, N, e0, e1);
-    if (!id_filter || e0 % host::TOPK_ROWMETA_ROWS != 0 || (e0 == 0 && e1 <= TOPK_FIRST_ROWS)) {
+    // (the repair scan is exact as well: a query the bound cannot separate from most of the table, its threshold
+    // tiny against the scales around it, would overflow its buffer again)
+    if (!id_filter || rescan || e0 % host::TOPK_ROWMETA_ROWS != 0 || (e0 == 0 && e1 <= TOPK_FIRST_ROWS)) {
       TopkArgs ea{tau, active, ws.cnt, ws.cand, TOPK_CAP};
       return launch_contract<TopkEpi>(dtype, a, ea, st, name);
     }
@@ -1547,7 +1548,7 @@ extern "C" int kge_topk(const float* Q, const float* bias, const void* E, int dt
     hipLaunchKernelGGL(topk_i8_filter_kernel, dim3((unsigned)nwg), dim3(64 * TF_W), 0, st, a, ea);
     KGE_LAUNCH_CHECK(name);
     if (int trc = timer.end()) return trc;
-    hipLaunchKernelGGL(topk_rescore_kernel, dim3((unsigned)B, 4), dim3(256), 0, st, ws, a, rescan);
+    hipLaunchKernelGGL(topk_rescore_kernel, dim3((unsigned)B, 4), dim3(256), 0, st, ws, a);
     KGE_LAUNCH_CHECK("topk_rescore_kernel");
     return KGE_OK;
   };

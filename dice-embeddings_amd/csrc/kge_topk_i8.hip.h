@@ -7,18 +7,20 @@
 //     (32x32x32, twice the bf16 rate, and the table rows go global -> LDS untouched);
 //   * the exact raw score A = fl(sum_k e_k qb_k) obeys |A - s_q H| <= mq L1(e), with L1(e) = sum_k |e_k| and mq = dq + 4e-3 s_q (the second term covers the fp32 rounding of the
 //     exact chain, at most 128 * 2^-23 * 127 s_q L1(e) = 1.9e-3 s_q L1(e), and of this bound's own arithmetic);
-//   * the row scale s_e is written unit * (m_e + r), unit = (largest scale of the 32-row tile) / 255, m_e an
-//     integer in [0, 255], |r| <= 0.51, so that  score = s_e A <= s_q unit (m_e H + 64.8 max L1) + mq max(s_e L1(e))
-//     (|H| <= 127 L1): per element one 24-bit integer multiply, per tile and lane one maximum and a few float
-//     operations.  A tile none of whose lanes can beat its query's tau is passed over; in the others the products
-//     are formed again and compared with the threshold turned into an integer.
+//   * the row scale s_e (of either sign) is written unit * (m_e + r), unit = (largest |scale| of the 32-row
+//     tile) / 511, m_e an integer in [-511, 511], |r| <= 0.51, so that
+//       score = s_e A <= s_q unit (m_e H + 64.8 max L1) + mq max(|s_e| L1(e))            (|H| <= 127 L1):
+//     per element one 24-bit integer multiply, per tile and lane one maximum and a few float operations.  A tile
+//     none of whose lanes can beat its query's tau is passed over; in the others the products are formed again and
+//     compared with the threshold turned into an integer.
 // An element that passes is only a candidate: its entity id goes to the query's candidate buffer, and the
 // selection kernel recomputes its score with the exact chain (the one kge_scores uses) and compares that with
 // tau.  So the filter decides nothing about the result, it only has to let every true candidate through.
 //
-// What the bound needs of the table (m_e per row; unit, max s_e L1(e), 64.8 max L1 and a "some scale is negative
-// or not finite" flag per 32-row tile) does not depend on the queries: topk_i8_rowmeta_kernel writes it once per
-// call, one 128-byte record per 64 rows, and the scan loads a stage's record with the stage.
+// What the bound needs of the table (m_e per row; unit, max |s_e| L1(e), 64.8 max L1 and a "some scale is not
+// finite" flag per 32-row tile, which then admits all its rows) does not depend on the queries:
+// topk_i8_rowmeta_kernel writes it once per call, one 160-byte record per 64 rows, and the scan loads a stage's
+// record with the stage.
 //
 // Pipeline: the persistent XCD-aware walk and the three-buffer global -> LDS ring of qstream_kernel, 64-row
 // stages of 8 KB, one barrier per stage; a tile's test runs under the next tile's MFMA chain.  Candidate ids are
@@ -62,7 +64,7 @@ __device__ __forceinline__ void tf_place(const I8FilterArgs& a, int64_t q, int32
 }
 
 // Per 64 table rows one record for the scan (layout: meta_lds in topk_i8_filter_kernel).  One wave per record, one
-// lane per row.  A row past the table's end counts for nothing; a negative or non-finite scale forces its tile.
+// lane per row.  A row past the table's end counts for nothing; a scale that is not finite forces its tile.
 __global__ void __launch_bounds__(256) topk_i8_rowmeta_kernel(const int8_t* E, const float* scale, int64_t N,
                                                               unsigned char* meta) {
   const int lane = threadIdx.x & 63;
@@ -82,9 +84,10 @@ __global__ void __launch_bounds__(256) topk_i8_rowmeta_kernel(const int8_t* E, c
     sc = scale[row];
   }
   const float l1 = (float)sad;
-  const bool bad = in && !(sc >= 0.f && sc <= 3.4028234e38f);
+  const bool bad = in && !(__builtin_fabsf(sc) <= 3.4028234e38f);
   const float scv = (in && !bad) ? sc : 0.f;
-  float l1M = l1, sM = scv, wM = scv * l1, fM = bad ? 1.f : 0.f;
+  const float sca = __builtin_fabsf(scv);
+  float l1M = l1, sM = sca, wM = sca * l1, fM = bad ? 1.f : 0.f;
 #pragma unroll
   for (int o = 1; o <= 16; o <<= 1) {
     l1M = __builtin_fmaxf(l1M, __shfl_xor(l1M, o, 64));
@@ -92,22 +95,22 @@ __global__ void __launch_bounds__(256) topk_i8_rowmeta_kernel(const int8_t* E, c
     wM = __builtin_fmaxf(wM, __shfl_xor(wM, o, 64));
     fM = __builtin_fmaxf(fM, __shfl_xor(fM, o, 64));
   }
-  float m = (sM > 0.f) ? __builtin_rintf(255.f * scv / sM) : 0.f;
-  m = __builtin_fminf(__builtin_fmaxf(m, 0.f), 255.f);
+  float m = (sM > 0.f) ? __builtin_rintf(511.f * scv / sM) : 0.f;
+  m = __builtin_fminf(__builtin_fmaxf(m, -511.f), 511.f);
   const int et = lane >> 5, r = lane & 31;
   unsigned char* out = meta + rec * host::TOPK_ROWMETA_BYTES;
-  out[(et * 2 + ((r >> 2) & 1)) * 16 + 4 * (r >> 3) + (r & 3)] = (unsigned char)(int)m;
+  ((int16_t*)out)[(et * 2 + ((r >> 2) & 1)) * 16 + 4 * (r >> 3) + (r & 3)] = (int16_t)(int)m;
   if (r == 0) {
-    const f32x4 tc = {sM / 255.f, wM, 64.8f * l1M, fM};
-    *(f32x4*)(out + 64 + 16 * et) = tc;
+    const f32x4 tc = {sM / 511.f, wM, 64.8f * l1M, fM};
+    *(f32x4*)(out + 128 + 16 * et) = tc;
   }
 }
 
 __global__ void __launch_bounds__(64 * TF_W, 2) topk_i8_filter_kernel(ContractArgs a, I8FilterArgs ea) {
   constexpr int NQT = TF_NQT, W = TF_W, WQ = TF_WG_QUERIES;
   __shared__ __attribute__((aligned(1024))) unsigned char lds_e[TF_NBUF * TF_STAGE_BYTES];
-  // the stage's record: multipliers m_e as bytes in the order a lane's accumulators hold them ([tile][half][16]),
-  // then per tile {unit, max s L1, 64.8 max L1, forced}
+  // the stage's record: multipliers m_e (int16) in the order a lane's accumulators hold them ([tile][half][16]),
+  // then per tile {unit, max |s| L1, 64.8 max L1, forced}
   __shared__ __attribute__((aligned(16))) unsigned char meta_lds[TF_NBUF][host::TOPK_ROWMETA_BYTES];
   __shared__ uint32_t bucket[WQ * TF_BUCKET];
   __shared__ int bcnt[WQ];
@@ -233,20 +236,22 @@ __global__ void __launch_bounds__(64 * TF_W, 2) topk_i8_filter_kernel(ContractAr
 
   // ---- the test of one finished tile ------------------------------------------------------------
   // constants of the entity tile the finished accumulators belong to
-  u32x4 m_mul = {0u, 0u, 0u, 0u};
+  u32x4 m_mul[2] = {{0u, 0u, 0u, 0u}, {0u, 0u, 0u, 0u}};
   float m_unit = 0.f, m_W = 0.f, m_c2 = 0.f;
   bool m_force = false;
   int64_t e_prev = r_end;
   auto tile_meta = [&](int buf, int et) {
-    m_mul = *(const u32x4*)&meta_lds[buf][(et * 2 + hf) * 16];
-    const f32x4 tc = *(const f32x4*)&meta_lds[buf][64 + 16 * et];
+    m_mul[0] = *(const u32x4*)&meta_lds[buf][(et * 2 + hf) * 32];
+    m_mul[1] = *(const u32x4*)&meta_lds[buf][(et * 2 + hf) * 32 + 16];
+    const f32x4 tc = *(const f32x4*)&meta_lds[buf][128 + 16 * et];
     m_unit = tc[0];
     m_W = tc[1];
     m_c2 = tc[2];
     m_force = tc[3] != 0.f;
   };
   auto product = [&](const i32x16& h, int i) -> int {
-    return __mul24(h[i], (int)((m_mul[i >> 2] >> (8 * (i & 3))) & 0xffu));
+    const uint32_t w = m_mul[i >> 3][(i >> 1) & 3];
+    return __mul24(h[i], (int)(int16_t)(uint16_t)(w >> (16 * (i & 1))));
   };
   auto tile_test = [&](int t, const i32x16& h) {
     int pm = product(h, 0);
@@ -260,7 +265,8 @@ __global__ void __launch_bounds__(64 * TF_W, 2) topk_i8_filter_kernel(ContractAr
     const bool hit = (Bd > tau_lo[t]) || (m_force && tau_lo[t] < INF);
     if (__builtin_expect(__builtin_amdgcn_ballot_w64(hit) != 0, 0)) {
       // The same products against the threshold as an integer: su (P + c2) + mw > tau  <=>  P > (tau - mw) / su - c2,
-      // lowered by its own rounding and kept inside +-2^30 (|P| < 2^29) so that the difference below cannot wrap.
+      // lowered by its own rounding and kept inside +-2^30 (|P| <= 127 * 128 * 127 * 511 < 2^30) so that the difference
+      // below cannot wrap.
       float x;
       if (m_force && tau_lo[t] < INF)
         x = -INF;

@@ -396,6 +396,84 @@ def test_topk_adversarial_order_overflows_and_recovers(ops):
     np.testing.assert_array_equal(vals.cpu().numpy(), wv)
 
 
+@pytest.mark.parametrize("storage", ["fp32", "int8"])
+def test_topk_best_rows_first_defeats_the_guessed_threshold(ops, storage):
+    """Scores that decrease with the entity id: the best k are all in the first round, so the threshold a later scan
+    guesses from the order statistics of a shuffled table (a rank above the k-th) is too high every time.  The
+    selection notices that fewer than k entries beat the guess, flags the query, and the final rescan with the k-th
+    best repairs it."""
+    N, d, B, k = 70000, 128, 70, 100
+    rng = np.random.default_rng(5)
+    v = rng.standard_normal(d).astype(np.float32)
+    E = ((N - np.arange(N, dtype=np.float32))[:, None] / N) * v[None, :]
+    E += (rng.standard_normal((N, d)) * 1e-4).astype(np.float32)
+    Q = (np.abs(rng.standard_normal((B, 1))).astype(np.float32) + 0.5) * v[None, :]
+    Et, sc, _, _, _ = stored_tables(E, E[:1], storage)
+    Eg, scg, Qg = dev(Et), dev(sc), dev(torch.from_numpy(Q))
+    vals, idx = ops.topk(Qg, None, Eg, scg, k)
+    S = ops.scores(Qg, None, Eg, scg).cpu().numpy()
+    wv, wi = ko.topk(S, k)
+    np.testing.assert_array_equal(idx.cpu().numpy(), wi)
+    np.testing.assert_array_equal(vals.cpu().numpy(), wv)
+
+
+@pytest.mark.parametrize("N,B,k", [(70001, 1100, 100), (200003, 33, 1), (150000, 40, 1024), (4100, 20, 10)])
+def test_topk_int8_filter_scan_edge_cases(ops, N, B, k):
+    """The int8 scan admits candidates by an integer bound and scores them exactly afterwards; whatever the bound
+    lets through or not, the result must be the top k of the library's own scores.  Rows: scales spread over four
+    orders of magnitude, zero and negative scales, all-zero rows, rows of +-127; queries: zero, one-hot, a huge
+    dynamic range, one whose scores are all negative; N not a multiple of the 64-row stage, a partial last query
+    group."""
+    rng = np.random.default_rng(N + k)
+    d = 128
+    q8 = rng.integers(-127, 128, (N, d)).astype(np.int8)
+    q8[rng.integers(0, N, 50)] = 0
+    q8[rng.integers(0, N, 50)] = 127
+    q8[rng.integers(0, N, 50)] = -127
+    sc = np.exp(rng.uniform(np.log(1e-5), np.log(1e-1), N)).astype(np.float32)
+    sc[rng.integers(0, N, 200)] = 0.0
+    neg = rng.integers(0, N, 200)
+    sc[neg] = -sc[neg]
+    Q = (rng.standard_normal((B, d)) * 0.1).astype(np.float32)
+    Q[0] = 0.0
+    Q[1] = 0.0
+    Q[1, 5] = 3.0
+    Q[2] *= np.exp(rng.uniform(-12, 2, d)).astype(np.float32)
+    base = np.abs(rng.standard_normal(d)).astype(np.float32)
+    Q[3] = -base                                       # against rows made non-negative below: every score <= 0
+    Eg, scg, Qg = dev(torch.from_numpy(q8)), dev(torch.from_numpy(sc)), dev(torch.from_numpy(Q))
+    vals, idx = ops.topk(Qg, None, Eg, scg, k)
+    S = ops.scores(Qg, None, Eg, scg).cpu().numpy()
+    wv, wi = ko.topk(S, k)
+    # (the zero query scores +0 or -0 everywhere: equal to numpy, ordered by sign in the library's keys)
+    np.testing.assert_array_equal(idx.cpu().numpy()[1:], wi[1:])
+    np.testing.assert_array_equal(vals.cpu().numpy(), wv)
+    # a table of non-negative rows and positive scales under the all-negative query
+    Ep = np.abs(q8.astype(np.int16)).clip(0, 127).astype(np.int8)
+    scp = np.abs(sc) + 1e-6
+    Eg, scg = dev(torch.from_numpy(Ep)), dev(torch.from_numpy(scp))
+    vals, idx = ops.topk(Qg[3:4], None, Eg, scg, k)
+    S = ops.scores(Qg[3:4], None, Eg, scg).cpu().numpy()
+    assert (S <= 0).all()
+    wv, wi = ko.topk(S, k)
+    np.testing.assert_array_equal(idx.cpu().numpy(), wi)
+    np.testing.assert_array_equal(vals.cpu().numpy(), wv)
+
+
+def test_topk_int8_query_with_a_nan_yields_nothing(ops):
+    N, d, B, k = 9000, 128, 3, 5
+    rng = np.random.default_rng(8)
+    q8 = rng.integers(-127, 128, (N, d)).astype(np.int8)
+    sc = np.full(N, 0.01, dtype=np.float32)
+    Q = rng.standard_normal((B, d)).astype(np.float32)
+    Q[1, 17] = np.nan
+    vals, idx = ops.topk(dev(torch.from_numpy(Q)), None, dev(torch.from_numpy(q8)), dev(torch.from_numpy(sc)), k)
+    assert torch.isnan(vals[1]).all() and (idx[1] == -1).all()
+    S = ops.scores(dev(torch.from_numpy(Q[[0, 2]])), None, dev(torch.from_numpy(q8)), dev(torch.from_numpy(sc))).cpu().numpy()
+    wv, wi = ko.topk(S, k)
+    np.testing.assert_array_equal(idx[[0, 2]].cpu().numpy(), wi)
+
+
 def test_topk_ties_prefer_lower_ids_and_k_equals_n(ops):
     N, d, B = 300, 16, 5
     E = torch.zeros((N, d), device="cuda")
