@@ -115,11 +115,13 @@ inline RankWsOffsets rank_ws_offsets(int64_t B) {
 // tau: k-th best score per query; tau_scan: the threshold the next scan admits candidates with (tau, or a tighter
 // guess that the selection verifies); list: the best k so far as packed keys; cand: this round's candidates as packed
 // keys; cand_id: this round's candidates as entity ids (int8 filter scan, scored exactly before they are ranked);
-// rowmeta: one TOPK_ROWMETA_BYTES record per TOPK_ROWMETA_ROWS table rows (int8 filter scan)
+// requant: the int8 table written again with one scale per 32-row tile, N x 128 bytes, and rowmeta: one
+// TOPK_ROWMETA_BYTES record per TOPK_ROWMETA_ROWS table rows (both for the int8 filter scan)
 constexpr int TOPK_ROWMETA_ROWS = 64;
-constexpr int TOPK_ROWMETA_BYTES = 160;  // 64 int16 multipliers, then {unit, max |s| L1, c2, forced} per 32-row tile
+constexpr int TOPK_ROWMETA_BYTES = 32;  // per 32-row tile {scale, max L1 + 64, forced, -}
+constexpr int TOPK_REQUANT_D = 128;
 struct TopkWsOffsets {
-  size_t tau, tau_scan, cnt, list_len, dirty, n_dirty, list, cand, cand_id, rowmeta, total;
+  size_t tau, tau_scan, cnt, list_len, dirty, n_dirty, list, cand, cand_id, rowmeta, requant, total;
   int64_t kpad;
 };
 inline TopkWsOffsets topk_ws_offsets(int64_t B, int64_t N, int64_t k) {
@@ -141,6 +143,7 @@ inline TopkWsOffsets topk_ws_offsets(int64_t B, int64_t N, int64_t k) {
   o.cand = take((size_t)B * TOPK_CAP * 8);
   o.cand_id = take((size_t)B * TOPK_CAP * 4);
   o.rowmeta = take((size_t)((N + TOPK_ROWMETA_ROWS - 1) / TOPK_ROWMETA_ROWS) * TOPK_ROWMETA_BYTES);
+  o.requant = take((size_t)N * TOPK_REQUANT_D);
   o.total = off;
   return o;
 }

@@ -618,6 +618,7 @@ struct TopkWs {
   unsigned long long* cand;  // [B, TOPK_CAP] packed keys
   uint32_t* cand_id;         // [B, TOPK_CAP] entity ids (int8 filter scan; scored into `cand` before they are ranked)
   unsigned char* rowmeta;    // int8 filter scan: per 64 table rows one record
+  int8_t* requant;           // int8 filter scan: the table with one scale per 32-row tile
   int64_t kpad;
 };
 
@@ -635,6 +636,7 @@ size_t topk_ws_layout(int64_t B, int64_t N, int64_t k, void* base, TopkWs* ws) {
     ws->cand = (unsigned long long*)(p + o.cand);
     ws->cand_id = (uint32_t*)(p + o.cand_id);
     ws->rowmeta = (unsigned char*)(p + o.rowmeta);
+    ws->requant = (int8_t*)(p + o.requant);
     ws->kpad = o.kpad;
   }
   return o.total;
@@ -1515,9 +1517,9 @@ extern "C" int kge_topk(const float* Q, const float* bias, const void* E, int dt
   const bool id_filter = (dtype == KGE_I8 && d == 128 && N > TOPK_FIRST_ROWS);
   if (id_filter) {
     const int64_t n_rec = (N + host::TOPK_ROWMETA_ROWS - 1) / host::TOPK_ROWMETA_ROWS;
-    hipLaunchKernelGGL(topk_i8_rowmeta_kernel, dim3((unsigned)((n_rec + 3) / 4)), dim3(256), 0, st, (const int8_t*)E,
-                       scale, N, ws.rowmeta);
-    KGE_LAUNCH_CHECK("topk_i8_rowmeta_kernel");
+    hipLaunchKernelGGL(topk_i8_requant_kernel, dim3((unsigned)n_rec), dim3(256), 0, st, (const int8_t*)E,
+                       scale, N, ws.requant, ws.rowmeta);
+    KGE_LAUNCH_CHECK("topk_i8_requant_kernel");
   }
   // One scan of entity rows [e0, e1) with the thresholds `tau`, for all queries or those flagged in `active`.
   auto launch_scan = [&](int64_t e0, int64_t e1, const float* tau, const int32_t* active, int rescan,
@@ -1542,7 +1544,7 @@ extern "C" int kge_topk(const float* Q, const float* bias, const void* E, int dt
     a.n_chunks = (e1 - e0 + chunk - 1) / chunk;
     const int64_t nwg = 8 * (int64_t)a.n_qgroups * a.n_lanes;
     KGE_REQUIRE(nwg <= 0x7fffffffLL, KGE_ERR_INVALID, "%s: grid of %lld workgroups too large", name, (long long)nwg);
-    I8FilterArgs ea{tau, active, ws.cnt, ws.cand_id, TOPK_CAP, ws.rowmeta};
+    I8FilterArgs ea{tau, active, ws.cnt, ws.cand_id, TOPK_CAP, ws.requant, ws.rowmeta};
     LaunchTimer timer;
     if (int trc = timer.begin(st)) return trc;
     hipLaunchKernelGGL(topk_i8_filter_kernel, dim3((unsigned)nwg), dim3(64 * TF_W), 0, st, a, ea);

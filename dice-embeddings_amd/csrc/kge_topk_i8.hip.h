@@ -2,25 +2,23 @@
 //
 // A round of kge_topk only has to find the entities whose score beats the query's threshold tau; nearly all of
 // the B x N scores do not.  The scan therefore works on a bound that is cheap to form:
-//   * the query row is rounded to bf16 (qb, the operand of the exact score) and then quantised once more to
-//     int8, qb = s_q * qh + delta with |delta| <= dq;  H = sum_k e_k qh_k is an exact int32 from the int8 MFMA
-//     (32x32x32, twice the bf16 rate, and the table rows go global -> LDS untouched);
-//   * the exact raw score A = fl(sum_k e_k qb_k) obeys |A - s_q H| <= mq L1(e), with L1(e) = sum_k |e_k| and mq = dq + 4e-3 s_q (the second term covers the fp32 rounding of the
-//     exact chain, at most 128 * 2^-23 * 127 s_q L1(e) = 1.9e-3 s_q L1(e), and of this bound's own arithmetic);
-//   * the row scale s_e (of either sign) is written unit * (m_e + r), unit = (largest |scale| of the 32-row
-//     tile) / 511, m_e an integer in [-511, 511], |r| <= 0.51, so that
-//       score = s_e A <= s_q unit (m_e H + 64.8 max L1) + mq max(|s_e| L1(e))            (|H| <= 127 L1):
-//     per element one 24-bit integer multiply, per tile and lane one maximum and a few float operations.  A tile
-//     none of whose lanes can beat its query's tau is passed over; in the others the products are formed again and
-//     compared with the threshold turned into an integer.
-// An element that passes is only a candidate: its entity id goes to the query's candidate buffer, and the
-// selection kernel recomputes its score with the exact chain (the one kge_scores uses) and compares that with
-// tau.  So the filter decides nothing about the result, it only has to let every true candidate through.
-//
-// What the bound needs of the table (m_e per row; unit, max |s_e| L1(e), 64.8 max L1 and a "some scale is not
-// finite" flag per 32-row tile, which then admits all its rows) does not depend on the queries:
-// topk_i8_rowmeta_kernel writes it once per call, one 160-byte record per 64 rows, and the scan loads a stage's
-// record with the stage.
+//   * once per call the table is written again with one scale per 32-row tile (topk_i8_requant_kernel):
+//     s_e e_k = S (e'_k + rho_k), S the tile's largest |scale|, e'_k an int8, |rho_k| <= 0.501.  The sign of a
+//     negative scale moves into e'; a row whose scale is tiny against its neighbours' becomes mostly zeros,
+//     which costs the bound tightness but not validity;
+//   * the query row is rounded to bf16 (qb, the operand of the exact score) and then quantised to int8,
+//     qb_k = s_q qh_k + delta_k with |delta_k| <= dq;  H' = sum_k e'_k qh_k is an exact int32 from the int8 MFMA
+//     (32x32x32, twice the bf16 rate, and the rows go global -> LDS untouched);
+//   * the exact score is fl(s_e A) with A = fl(sum_k e_k qb_k) (fp32 accumulation: |A - sum| is at most
+//     128 * 2^-23 * sum_k |e_k qb_k| <= 1.9e-3 s_q L1(e), L1(e) = sum_k |e_k|, since |qb_k| <= 127 s_q).  Hence
+//       s_e A <= S ( s_q H' + mq (L1(e') + 64) + 0.501 L1(qb) ),      mq = dq + 4e-3 s_q
+//     (the 64 covers sum_k |rho_k|, the 4e-3 the rounding of the chain and of this bound's own few operations).
+//     Per element nothing but the MFMA; per tile and lane the maximum of its 16 accumulators and five float
+//     operations.  A tile none of whose lanes can beat its query's tau is passed over; in the others the
+//     accumulators are compared with the threshold turned into an integer.
+// An element that passes is only a candidate: its entity id goes to the query's candidate buffer, and its score
+// is recomputed with the exact chain (the one kge_scores uses) before the selection compares it with tau.  So the
+// filter decides nothing about the result, it only has to let every true candidate through.
 //
 // Pipeline: the persistent XCD-aware walk and the three-buffer global -> LDS ring of qstream_kernel, 64-row
 // stages of 8 KB, one barrier per stage; a tile's test runs under the next tile's MFMA chain.  Candidate ids are
@@ -34,12 +32,13 @@ typedef __attribute__((ext_vector_type(4))) int i32x4;
 typedef __attribute__((ext_vector_type(16))) int i32x16;
 
 struct I8FilterArgs {
-  const float* tau;       // per query: k-th best exact score so far (-inf while fewer than k known)
+  const float* tau;       // per query: the threshold candidates must beat (-inf: everything is a candidate)
   const int32_t* active;  // NULL = all queries; else only queries with active[b] != 0 collect
   int32_t* cnt;           // per query: candidates appended this round
   uint32_t* cand;         // [B, cap] candidate entity ids
   int32_t cap;
-  const unsigned char* rowmeta;  // one record per 64 table rows (topk_i8_rowmeta_kernel)
+  const int8_t* Eq;              // the table with tile-common scales (topk_i8_requant_kernel)
+  const unsigned char* rowmeta;  // one record per 64 table rows: per 32-row tile {S, max L1(e') + 64, forced, -}
 };
 
 constexpr int TF_NQT = 4;                              // 32-query tiles per wave
@@ -49,7 +48,8 @@ constexpr int TF_STAGE_ROWS = 64;
 constexpr int TF_STAGE_BYTES = TF_STAGE_ROWS * 128;    // 8 KB of int8 rows
 constexpr int TF_NBUF = 3;
 constexpr int TF_BUCKET = 16;                          // candidate ids a query can park in LDS
-constexpr int TF_VALU_PER_MFMA = 5;
+constexpr int TF_VALU_PER_MFMA = 4;
+static_assert(host::TOPK_ROWMETA_ROWS == TF_STAGE_ROWS && host::TOPK_ROWMETA_BYTES == 32, "record per stage");
 
 // One candidate id into its query's global buffer; slot is the query's running count.  A full buffer keeps a
 // uniform sample of what arrives (the query is repaired by a later rescan with its final threshold).
@@ -63,54 +63,78 @@ __device__ __forceinline__ void tf_place(const I8FilterArgs& a, int64_t q, int32
   if (slot >= 0) a.cand[q * a.cap + slot] = e;
 }
 
-// Per 64 table rows one record for the scan (layout: meta_lds in topk_i8_filter_kernel).  One wave per record, one
-// lane per row.  A row past the table's end counts for nothing; a scale that is not finite forces its tile.
-__global__ void __launch_bounds__(256) topk_i8_rowmeta_kernel(const int8_t* E, const float* scale, int64_t N,
+// The table with one scale per 32-row tile, and per 64 rows one record for the scan.  One workgroup per 64 rows:
+// thread t takes 16 bytes of row (t >> 3) of each of the two tiles, so loads and stores are whole rows in order.
+// A row past the table's end counts for nothing; a scale that is not finite forces its tile (the scan then takes
+// all its rows as candidates).
+__global__ void __launch_bounds__(256) topk_i8_requant_kernel(const int8_t* E, const float* scale, int64_t N, int8_t* Eq,
                                                               unsigned char* meta) {
-  const int lane = threadIdx.x & 63;
-  const int64_t rec = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-  if (rec * 64 >= N) return;
-  const int64_t row = rec * 64 + lane;
-  const bool in = row < N;
-  uint32_t sad = 0;
-  float sc = 0.f;
-  if (in) {
+  __shared__ float s_max[2][4], s_bad[2][4], s_l1[2][4];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int64_t rec = blockIdx.x;
+  float scv[2];
+  u32x4 w[2];
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      const u32x4 w = *(const u32x4*)(E + row * 128 + 16 * j);
+  for (int it = 0; it < 2; ++it) {
+    const int64_t row = rec * 64 + it * 32 + (tid >> 3);
+    const bool in = row < N;
+    const float sc = in ? scale[row] : 0.f;
+    w[it] = in ? *(const u32x4*)(E + row * 128 + 16 * (tid & 7)) : u32x4{0u, 0u, 0u, 0u};
+    const bool bad = !(__builtin_fabsf(sc) <= 3.4028234e38f);
+    scv[it] = bad ? 0.f : sc;
+    float sM = __builtin_fabsf(scv[it]), fM = bad ? 1.f : 0.f;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) sad = __builtin_amdgcn_sad_u8(w[i] ^ 0x80808080u, 0x80808080u, sad);  // sum |int8|
+    for (int o = 8; o <= 32; o <<= 1) {
+      sM = __builtin_fmaxf(sM, __shfl_xor(sM, o, 64));
+      fM = __builtin_fmaxf(fM, __shfl_xor(fM, o, 64));
     }
-    sc = scale[row];
+    if (lane == 0) {
+      s_max[it][wave] = sM;
+      s_bad[it][wave] = fM;
+    }
   }
-  const float l1 = (float)sad;
-  const bool bad = in && !(__builtin_fabsf(sc) <= 3.4028234e38f);
-  const float scv = (in && !bad) ? sc : 0.f;
-  const float sca = __builtin_fabsf(scv);
-  float l1M = l1, sM = sca, wM = sca * l1, fM = bad ? 1.f : 0.f;
+  __syncthreads();
 #pragma unroll
-  for (int o = 1; o <= 16; o <<= 1) {
-    l1M = __builtin_fmaxf(l1M, __shfl_xor(l1M, o, 64));
-    sM = __builtin_fmaxf(sM, __shfl_xor(sM, o, 64));
-    wM = __builtin_fmaxf(wM, __shfl_xor(wM, o, 64));
-    fM = __builtin_fmaxf(fM, __shfl_xor(fM, o, 64));
+  for (int it = 0; it < 2; ++it) {
+    const int64_t row = rec * 64 + it * 32 + (tid >> 3);
+    const float S = __builtin_fmaxf(__builtin_fmaxf(s_max[it][0], s_max[it][1]), __builtin_fmaxf(s_max[it][2], s_max[it][3]));
+    const float ratio = (S > 0.f) ? scv[it] / S : 0.f;  // |ratio| <= 1: the products below stay within +-127
+    u32x4 o;
+    uint32_t l1 = 0;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      uint32_t pk = 0;
+#pragma unroll
+      for (int b = 0; b < 4; ++b) {
+        const float x = (float)(int)(int8_t)(w[it][i] >> (8 * b));
+        const int v = (int)__builtin_rintf(x * ratio);
+        pk |= ((uint32_t)v & 0xffu) << (8 * b);
+      }
+      o[i] = pk;
+      l1 = __builtin_amdgcn_sad_u8(pk ^ 0x80808080u, 0x80808080u, l1);  // sum |int8|
+    }
+    if (row < N) *(u32x4*)(Eq + row * 128 + 16 * (tid & 7)) = o;
+    l1 += __shfl_xor(l1, 1, 64);
+    l1 += __shfl_xor(l1, 2, 64);
+    l1 += __shfl_xor(l1, 4, 64);
+    float l1M = (float)l1;
+#pragma unroll
+    for (int s = 8; s <= 32; s <<= 1) l1M = __builtin_fmaxf(l1M, __shfl_xor(l1M, s, 64));
+    if (lane == 0) s_l1[it][wave] = l1M;
   }
-  float m = (sM > 0.f) ? __builtin_rintf(511.f * scv / sM) : 0.f;
-  m = __builtin_fminf(__builtin_fmaxf(m, -511.f), 511.f);
-  const int et = lane >> 5, r = lane & 31;
-  unsigned char* out = meta + rec * host::TOPK_ROWMETA_BYTES;
-  ((int16_t*)out)[(et * 2 + ((r >> 2) & 1)) * 16 + 4 * (r >> 3) + (r & 3)] = (int16_t)(int)m;
-  if (r == 0) {
-    const f32x4 tc = {sM / 511.f, wM, 64.8f * l1M, fM};
-    *(f32x4*)(out + 128 + 16 * et) = tc;
+  __syncthreads();
+  if (tid < 2) {
+    const float S = __builtin_fmaxf(__builtin_fmaxf(s_max[tid][0], s_max[tid][1]), __builtin_fmaxf(s_max[tid][2], s_max[tid][3]));
+    const float L = __builtin_fmaxf(__builtin_fmaxf(s_l1[tid][0], s_l1[tid][1]), __builtin_fmaxf(s_l1[tid][2], s_l1[tid][3]));
+    const float F = __builtin_fmaxf(__builtin_fmaxf(s_bad[tid][0], s_bad[tid][1]), __builtin_fmaxf(s_bad[tid][2], s_bad[tid][3]));
+    const f32x4 tc = {S, L + 64.f, F, 0.f};
+    *(f32x4*)(meta + rec * host::TOPK_ROWMETA_BYTES + 16 * tid) = tc;
   }
 }
 
 __global__ void __launch_bounds__(64 * TF_W, 2) topk_i8_filter_kernel(ContractArgs a, I8FilterArgs ea) {
   constexpr int NQT = TF_NQT, W = TF_W, WQ = TF_WG_QUERIES;
   __shared__ __attribute__((aligned(1024))) unsigned char lds_e[TF_NBUF * TF_STAGE_BYTES];
-  // the stage's record: multipliers m_e (int16) in the order a lane's accumulators hold them ([tile][half][16]),
-  // then per tile {unit, max |s| L1, 64.8 max L1, forced}
   __shared__ __attribute__((aligned(16))) unsigned char meta_lds[TF_NBUF][host::TOPK_ROWMETA_BYTES];
   __shared__ uint32_t bucket[WQ * TF_BUCKET];
   __shared__ int bcnt[WQ];
@@ -144,12 +168,12 @@ __global__ void __launch_bounds__(64 * TF_W, 2) topk_i8_filter_kernel(ContractAr
 
   // ---- the queries of this lane: int8 fragments and the constants of the bound ------------------
   i32x4 qf[NQT][4];
-  float sq[NQT], mq[NQT], tau_lo[NQT];
+  float sq[NQT], cq[NQT], mq[NQT], tau_lo[NQT];
 #pragma unroll
   for (int t = 0; t < NQT; ++t) {
     const int64_t q = q_wg + ql0 + 32 * t + c;
     float xb[64];  // bf16-rounded components k = 32 s + 16 hf + j of the row
-    float amax = 0.f;
+    float amax = 0.f, l1q = 0.f;
     bool has_nan = false;
 #pragma unroll
     for (int s = 0; s < 4; ++s) {
@@ -162,13 +186,15 @@ __global__ void __launch_bounds__(64 * TF_W, 2) topk_i8_filter_kernel(ContractAr
           const float r = (float)(__bf16)v[j];
           xb[16 * s + 4 * j4 + j] = r;
           amax = __builtin_fmaxf(amax, __builtin_fabsf(r));
+          l1q += __builtin_fabsf(r);
           has_nan = has_nan || (r != r);  // fmax drops a NaN
         }
       }
     }
     amax = __builtin_fmaxf(amax, __shfl_xor(amax, 32, 64));
+    l1q += __shfl_xor(l1q, 32, 64);
     has_nan = has_nan || (__shfl_xor((int)has_nan, 32, 64) != 0);
-    const bool finite = !has_nan && amax <= 3.4028234e38f;
+    const bool finite = !has_nan && amax <= 3.4028234e38f && l1q <= 3.4028234e38f;
     const float s_q = finite ? amax / 127.f : 0.f;
     const float inv = (finite && amax > 0.f) ? 127.f / amax : 0.f;
     float dq = 0.f;
@@ -193,6 +219,7 @@ __global__ void __launch_bounds__(64 * TF_W, 2) topk_i8_filter_kernel(ContractAr
     dq = __builtin_fmaxf(dq, __shfl_xor(dq, 32, 64));
     sq[t] = s_q;
     mq[t] = dq * 1.000001f + 4e-3f * s_q;
+    cq[t] = finite ? 0.501f * l1q * 1.00001f : 0.f;
     // a query with a non-finite component has no finite bound: it collects nothing (its scores are NaN or
     // infinite anyway)
     const bool on = q < a.B && finite && (ea.active == nullptr || ea.active[q] != 0);
@@ -209,7 +236,7 @@ __global__ void __launch_bounds__(64 * TF_W, 2) topk_i8_filter_kernel(ContractAr
   // bank groups.  Rows past the table's end repeat its last row (their entities are >= limit and are ignored).
   const int lrow = tid >> 3;
   const int lpiece = (tid & 7) ^ ((lrow >> 1) & 7);
-  const unsigned char* Eb = (const unsigned char*)a.E;
+  const unsigned char* Eb = (const unsigned char*)ea.Eq;
   auto stage_issue = [&](int64_t row0, int buf) {
     int64_t g = row0 + lrow;
     g = (g < r_end) ? g : r_end - 1;
@@ -236,50 +263,39 @@ __global__ void __launch_bounds__(64 * TF_W, 2) topk_i8_filter_kernel(ContractAr
 
   // ---- the test of one finished tile ------------------------------------------------------------
   // constants of the entity tile the finished accumulators belong to
-  u32x4 m_mul[2] = {{0u, 0u, 0u, 0u}, {0u, 0u, 0u, 0u}};
-  float m_unit = 0.f, m_W = 0.f, m_c2 = 0.f;
+  float m_S = 0.f, m_L1 = 0.f;
   bool m_force = false;
   int64_t e_prev = r_end;
   auto tile_meta = [&](int buf, int et) {
-    m_mul[0] = *(const u32x4*)&meta_lds[buf][(et * 2 + hf) * 32];
-    m_mul[1] = *(const u32x4*)&meta_lds[buf][(et * 2 + hf) * 32 + 16];
-    const f32x4 tc = *(const f32x4*)&meta_lds[buf][128 + 16 * et];
-    m_unit = tc[0];
-    m_W = tc[1];
-    m_c2 = tc[2];
-    m_force = tc[3] != 0.f;
-  };
-  auto product = [&](const i32x16& h, int i) -> int {
-    const uint32_t w = m_mul[i >> 3][(i >> 1) & 3];
-    return __mul24(h[i], (int)(int16_t)(uint16_t)(w >> (16 * (i & 1))));
+    const f32x4 tc = *(const f32x4*)&meta_lds[buf][16 * et];
+    m_S = tc[0];
+    m_L1 = tc[1];
+    m_force = tc[2] != 0.f;
   };
   auto tile_test = [&](int t, const i32x16& h) {
-    int pm = product(h, 0);
+    int hm = h[0];
 #pragma unroll
-    for (int i = 1; i < 16; ++i) {
-      const int p = product(h, i);
-      pm = pm > p ? pm : p;
-    }
-    const float su = sq[t] * m_unit, mw = mq[t] * m_W;
-    const float Bd = __builtin_fmaf(su, (float)pm + m_c2, mw);
+    for (int i = 1; i < 16; ++i) hm = hm > h[i] ? hm : h[i];
+    const float slack = __builtin_fmaf(mq[t], m_L1, cq[t]);
+    const float Bd = m_S * __builtin_fmaf(sq[t], (float)hm, slack);
     const bool hit = (Bd > tau_lo[t]) || (m_force && tau_lo[t] < INF);
     if (__builtin_expect(__builtin_amdgcn_ballot_w64(hit) != 0, 0)) {
-      // The same products against the threshold as an integer: su (P + c2) + mw > tau  <=>  P > (tau - mw) / su - c2,
-      // lowered by its own rounding and kept inside +-2^30 (|P| <= 127 * 128 * 127 * 511 < 2^30) so that the difference
+      // The accumulators against the threshold as an integer: S (s_q H + slack) > tau  <=>  H > (tau / S - slack) / s_q,
+      // lowered by its own rounding and kept inside +-2^30 (|H| <= 128 * 127 * 127 < 2^21) so that the difference
       // below cannot wrap.
       float x;
       if (m_force && tau_lo[t] < INF)
         x = -INF;
-      else if (su > 0.f) {
-        x = (tau_lo[t] - mw) / su - m_c2;
+      else if (m_S > 0.f && sq[t] > 0.f) {
+        x = (tau_lo[t] / m_S - slack) / sq[t];
         x = x - 1e-5f * __builtin_fabsf(x) - 1.f;
       } else
-        x = (mw > tau_lo[t]) ? -INF : INF;
+        x = (Bd > tau_lo[t]) ? -INF : INF;  // the bound does not depend on H
       x = __builtin_fminf(__builtin_fmaxf(x, -1073741824.f), 1073741824.f);
       const int thr = (x == x) ? (int)x : -1073741824;
       uint32_t bits = 0;  // bit 15 - i: element i may beat the threshold
 #pragma unroll
-      for (int i = 0; i < 16; ++i) bits = __builtin_amdgcn_alignbit(bits, (uint32_t)(thr - product(h, i)), 31);
+      for (int i = 0; i < 16; ++i) bits = __builtin_amdgcn_alignbit(bits, (uint32_t)(thr - h[i]), 31);
       const int qlocal = ql0 + 32 * t + c;
       while (__builtin_amdgcn_ballot_w64(bits != 0) != 0) {
         if (bits != 0) {

@@ -83,7 +83,8 @@ static void test_layouts() {
         check_disjoint({{t.tau, (size_t)B * 4}, {t.tau_scan, (size_t)B * 4}, {t.cnt, (size_t)B * 4},
                         {t.list_len, (size_t)B * 4}, {t.dirty, (size_t)B * 4}, {t.n_dirty, 4},
                         {t.list, (size_t)B * t.kpad * 8}, {t.cand, (size_t)B * TOPK_CAP * 8},
-                        {t.cand_id, (size_t)B * TOPK_CAP * 4}, {t.rowmeta, n_rec * TOPK_ROWMETA_BYTES}}, t.total);
+                        {t.cand_id, (size_t)B * TOPK_CAP * 4}, {t.rowmeta, n_rec * TOPK_ROWMETA_BYTES},
+                        {t.requant, (size_t)N * TOPK_REQUANT_D}}, t.total);
       }
     }
   }
