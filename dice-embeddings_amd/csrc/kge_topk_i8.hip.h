@@ -38,7 +38,7 @@ struct I8FilterArgs {
   uint32_t* cand;         // [B, cap] candidate entity ids
   int32_t cap;
   const int8_t* Eq;              // the table with tile-common scales (topk_i8_requant_kernel)
-  const unsigned char* rowmeta;  // one record per 64 table rows: per 32-row tile {S, max L1(e') + 64, forced, -}
+  const unsigned char* rowmeta;  // one record per 64 table rows: per 32-row tile {S, max L1(e') + 64, forced, 1 / S}
 };
 
 constexpr int TF_NQT = 4;                              // 32-query tiles per wave
@@ -127,7 +127,7 @@ __global__ void __launch_bounds__(256) topk_i8_requant_kernel(const int8_t* E, c
     const float S = __builtin_fmaxf(__builtin_fmaxf(s_max[tid][0], s_max[tid][1]), __builtin_fmaxf(s_max[tid][2], s_max[tid][3]));
     const float L = __builtin_fmaxf(__builtin_fmaxf(s_l1[tid][0], s_l1[tid][1]), __builtin_fmaxf(s_l1[tid][2], s_l1[tid][3]));
     const float F = __builtin_fmaxf(__builtin_fmaxf(s_bad[tid][0], s_bad[tid][1]), __builtin_fmaxf(s_bad[tid][2], s_bad[tid][3]));
-    const f32x4 tc = {S, L + 64.f, F, 0.f};
+    const f32x4 tc = {S, L + 64.f, F, S > 0.f ? 1.f / S : 0.f};
     *(f32x4*)(meta + rec * host::TOPK_ROWMETA_BYTES + 16 * tid) = tc;
   }
 }
@@ -168,7 +168,7 @@ __global__ void __launch_bounds__(64 * TF_W, 2) topk_i8_filter_kernel(ContractAr
 
   // ---- the queries of this lane: int8 fragments and the constants of the bound ------------------
   i32x4 qf[NQT][4];
-  float sq[NQT], cq[NQT], mq[NQT], tau_lo[NQT];
+  float sq[NQT], isq[NQT], cq[NQT], mq[NQT], tau_lo[NQT];
 #pragma unroll
   for (int t = 0; t < NQT; ++t) {
     const int64_t q = q_wg + ql0 + 32 * t + c;
@@ -218,6 +218,7 @@ __global__ void __launch_bounds__(64 * TF_W, 2) topk_i8_filter_kernel(ContractAr
     }
     dq = __builtin_fmaxf(dq, __shfl_xor(dq, 32, 64));
     sq[t] = s_q;
+    isq[t] = s_q > 0.f ? 1.f / s_q : 0.f;
     mq[t] = dq * 1.000001f + 4e-3f * s_q;
     cq[t] = finite ? 0.501f * l1q * 1.00001f : 0.f;
     // a query with a non-finite component has no finite bound: it collects nothing (its scores are NaN or
@@ -263,14 +264,15 @@ __global__ void __launch_bounds__(64 * TF_W, 2) topk_i8_filter_kernel(ContractAr
 
   // ---- the test of one finished tile ------------------------------------------------------------
   // constants of the entity tile the finished accumulators belong to
-  float m_S = 0.f, m_L1 = 0.f;
-  bool m_force = false;
+  float m_S = 0.f, m_L1 = 0.f, m_iS = 0.f;
+  bool m_force = false;  // the same for the whole wave
   int64_t e_prev = r_end;
   auto tile_meta = [&](int buf, int et) {
     const f32x4 tc = *(const f32x4*)&meta_lds[buf][16 * et];
     m_S = tc[0];
     m_L1 = tc[1];
-    m_force = tc[2] != 0.f;
+    m_force = __builtin_amdgcn_readfirstlane(__float_as_uint(tc[2])) != 0u;
+    m_iS = tc[3];
   };
   auto tile_test = [&](int t, const i32x16& h) {
     int hm = h[0];
@@ -278,16 +280,15 @@ __global__ void __launch_bounds__(64 * TF_W, 2) topk_i8_filter_kernel(ContractAr
     for (int i = 1; i < 16; ++i) hm = hm > h[i] ? hm : h[i];
     const float slack = __builtin_fmaf(mq[t], m_L1, cq[t]);
     const float Bd = m_S * __builtin_fmaf(sq[t], (float)hm, slack);
-    const bool hit = (Bd > tau_lo[t]) || (m_force && tau_lo[t] < INF);
-    if (__builtin_expect(__builtin_amdgcn_ballot_w64(hit) != 0, 0)) {
+    if (__builtin_expect(__builtin_amdgcn_ballot_w64(Bd > tau_lo[t]) != 0 || m_force, 0)) {
       // The accumulators against the threshold as an integer: S (s_q H + slack) > tau  <=>  H > (tau / S - slack) / s_q,
       // lowered by its own rounding and kept inside +-2^30 (|H| <= 128 * 127 * 127 < 2^21) so that the difference
       // below cannot wrap.
       float x;
-      if (m_force && tau_lo[t] < INF)
-        x = -INF;
+      if (m_force)
+        x = (tau_lo[t] < INF) ? -INF : INF;
       else if (m_S > 0.f && sq[t] > 0.f) {
-        x = (tau_lo[t] / m_S - slack) / sq[t];
+        x = (tau_lo[t] * m_iS - slack) * isq[t];
         x = x - 1e-5f * __builtin_fabsf(x) - 1.f;
       } else
         x = (Bd > tau_lo[t]) ? -INF : INF;  // the bound does not depend on H
