@@ -20,6 +20,11 @@
 // is recomputed with the exact chain (the one kge_scores uses) before the selection compares it with tau.  So the
 // filter decides nothing about the result, it only has to let every true candidate through.
 //
+// The tiles that do not pass as a whole are few, and in each of them one lane or two hold all the elements of
+// interest.  Such a lane parks its 16 accumulators, its integer threshold and its position in a small queue of its
+// wave; when 64 are waiting the wave works them off together, one lane per parked set.  (A tile most of whose lanes
+// are of interest, as in the first rounds of a call when thresholds are loose, is worked off on the spot.)
+//
 // Pipeline: the persistent XCD-aware walk and the three-buffer global -> LDS ring of qstream_kernel, 64-row
 // stages of 8 KB, one barrier per stage; a tile's test runs under the next tile's MFMA chain.  Candidate ids are
 // parked in per-query LDS buckets and leave for global memory as one run per query when the workgroup ends.
@@ -132,12 +137,70 @@ __global__ void __launch_bounds__(256) topk_i8_requant_kernel(const int8_t* E, c
   }
 }
 
+constexpr int TF_QUEUE = 64;         // parked accumulator sets per wave
+constexpr int TF_QUEUE_STRIDE = 21;  // dwords per set (19 used; odd: lanes reading their own set hit distinct banks)
+constexpr int TF_DENSE_LANES = 16;   // a tile with more lanes of interest than this is worked off on the spot
+
+struct TfShared {
+  uint32_t* bucket;  // [TF_WG_QUERIES][TF_BUCKET] candidate ids parked per query
+  int* bcnt;         // [TF_WG_QUERIES]
+};
+
+// The elements among h[0..16) above thr, as candidates of local query `qlocal`: entity e_base + row_of(i, hf).
+__device__ __forceinline__ void tf_collect(const int (&h)[16], int thr, bool on, int qlocal, int hf, int64_t e_base,
+                                           int64_t limit, int64_t q_wg, const TfShared& sh, const I8FilterArgs& ea) {
+  uint32_t bits = 0;  // bit 15 - i: element i may beat the threshold (|thr| <= 2^30, |h| < 2^21: no wrap)
+#pragma unroll
+  for (int i = 0; i < 16; ++i) bits = __builtin_amdgcn_alignbit(bits, (uint32_t)(thr - h[i]), 31);
+  if (!on) bits = 0;
+  while (__builtin_amdgcn_ballot_w64(bits != 0) != 0) {
+    if (bits != 0) {
+      const int b = 31 - __builtin_clz(bits);
+      bits &= ~(1u << b);
+      const int i = 15 - b;
+      const int64_t e = e_base + ((i >> 2) << 3) + (hf << 2) + (i & 3);
+      if (e < limit) {
+        const int idx = atomicAdd(&sh.bcnt[qlocal], 1);
+        if (idx < TF_BUCKET)
+          sh.bucket[qlocal * TF_BUCKET + idx] = (uint32_t)e;
+        else  // bucket full: straight to global memory
+          tf_place(ea, q_wg + qlocal, atomicAdd(&ea.cnt[q_wg + qlocal], 1), (uint32_t)e);
+      }
+    }
+  }
+}
+
+// A tile most of whose lanes are of interest: every lane tests its own 16 elements.  Out of line (one copy).
+__device__ __attribute__((noinline)) void tf_dense(i32x16 h, int thr, bool on, int qlocal, int hf, int64_t e_base,
+                                                   int64_t limit, int64_t q_wg, TfShared sh, I8FilterArgs ea) {
+  int hh[16];
+#pragma unroll
+  for (int i = 0; i < 16; ++i) hh[i] = h[i];
+  tf_collect(hh, thr, on, qlocal, hf, e_base, limit, q_wg, sh, ea);
+}
+
+// The parked sets of a wave, one lane per set.  Out of line (one copy).
+__device__ __attribute__((noinline)) void tf_drain(const uint32_t* queue, int n, int64_t limit, int64_t q_wg,
+                                                   TfShared sh, I8FilterArgs ea) {
+  const int lane = threadIdx.x & 63;
+  const bool on = lane < n;
+  const uint32_t* ent = queue + (on ? lane : 0) * TF_QUEUE_STRIDE;
+  int hh[16];
+#pragma unroll
+  for (int i = 0; i < 16; ++i) hh[i] = (int)ent[i];
+  const int thr = (int)ent[16];
+  const uint32_t where = ent[17];
+  const int64_t e_base = (int64_t)ent[18];
+  tf_collect(hh, thr, on, (int)(where & 0xffffu), (int)(where >> 16), e_base, limit, q_wg, sh, ea);
+}
+
 __global__ void __launch_bounds__(64 * TF_W, 2) topk_i8_filter_kernel(ContractArgs a, I8FilterArgs ea) {
   constexpr int NQT = TF_NQT, W = TF_W, WQ = TF_WG_QUERIES;
   __shared__ __attribute__((aligned(1024))) unsigned char lds_e[TF_NBUF * TF_STAGE_BYTES];
   __shared__ __attribute__((aligned(16))) unsigned char meta_lds[TF_NBUF][host::TOPK_ROWMETA_BYTES];
   __shared__ uint32_t bucket[WQ * TF_BUCKET];
   __shared__ int bcnt[WQ];
+  __shared__ uint32_t queue[W][TF_QUEUE * TF_QUEUE_STRIDE];
 
   const int64_t wg = blockIdx.x;
   const int xcd = (int)(wg & 7);
@@ -274,16 +337,19 @@ __global__ void __launch_bounds__(64 * TF_W, 2) topk_i8_filter_kernel(ContractAr
     m_force = __builtin_amdgcn_readfirstlane(__float_as_uint(tc[2])) != 0u;
     m_iS = tc[3];
   };
+  const TfShared shp{bucket, bcnt};
+  uint32_t* const wqueue = &queue[wave][0];
+  int qn = 0;  // sets parked in this wave's queue (the same in every lane)
   auto tile_test = [&](int t, const i32x16& h) {
     int hm = h[0];
 #pragma unroll
     for (int i = 1; i < 16; ++i) hm = hm > h[i] ? hm : h[i];
     const float slack = __builtin_fmaf(mq[t], m_L1, cq[t]);
     const float Bd = m_S * __builtin_fmaf(sq[t], (float)hm, slack);
-    if (__builtin_expect(__builtin_amdgcn_ballot_w64(Bd > tau_lo[t]) != 0 || m_force, 0)) {
+    const unsigned long long any = __builtin_amdgcn_ballot_w64(Bd > tau_lo[t]);
+    if (__builtin_expect(any != 0 || m_force, 0)) {
       // The accumulators against the threshold as an integer: S (s_q H + slack) > tau  <=>  H > (tau / S - slack) / s_q,
-      // lowered by its own rounding and kept inside +-2^30 (|H| <= 128 * 127 * 127 < 2^21) so that the difference
-      // below cannot wrap.
+      // lowered by its own rounding and kept inside +-2^30.
       float x;
       if (m_force)
         x = (tau_lo[t] < INF) ? -INF : INF;
@@ -294,24 +360,27 @@ __global__ void __launch_bounds__(64 * TF_W, 2) topk_i8_filter_kernel(ContractAr
         x = (Bd > tau_lo[t]) ? -INF : INF;  // the bound does not depend on H
       x = __builtin_fminf(__builtin_fmaxf(x, -1073741824.f), 1073741824.f);
       const int thr = (x == x) ? (int)x : -1073741824;
-      uint32_t bits = 0;  // bit 15 - i: element i may beat the threshold
-#pragma unroll
-      for (int i = 0; i < 16; ++i) bits = __builtin_amdgcn_alignbit(bits, (uint32_t)(thr - h[i]), 31);
+      const bool mine = (Bd > tau_lo[t]) || (m_force && tau_lo[t] < INF);
+      const unsigned long long who = __builtin_amdgcn_ballot_w64(mine);
+      const int n_new = __builtin_popcountll(who);
       const int qlocal = ql0 + 32 * t + c;
-      while (__builtin_amdgcn_ballot_w64(bits != 0) != 0) {
-        if (bits != 0) {
-          const int b = 31 - __builtin_clz(bits);
-          bits &= ~(1u << b);
-          const int i = 15 - b;
-          const int64_t e = e_prev + ((i >> 2) << 3) + (hf << 2) + (i & 3);
-          if (e < r_end) {
-            const int idx = atomicAdd(&bcnt[qlocal], 1);
-            if (idx < TF_BUCKET)
-              bucket[qlocal * TF_BUCKET + idx] = (uint32_t)e;
-            else  // bucket full: straight to global memory
-              tf_place(ea, q_wg + qlocal, atomicAdd(&ea.cnt[q_wg + qlocal], 1), (uint32_t)e);
-          }
+      if (n_new > TF_DENSE_LANES) {
+        tf_dense(h, thr, mine, qlocal, hf, e_prev, r_end, q_wg, shp, ea);
+      } else if (n_new > 0) {
+        if (qn + n_new > TF_QUEUE) {
+          tf_drain(wqueue, qn, r_end, q_wg, shp, ea);
+          qn = 0;
         }
+        if (mine) {
+          const int at = qn + (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(who >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)who, 0u));
+          uint32_t* ent = wqueue + at * TF_QUEUE_STRIDE;
+#pragma unroll
+          for (int i = 0; i < 16; ++i) ent[i] = (uint32_t)h[i];
+          ent[16] = (uint32_t)thr;
+          ent[17] = (uint32_t)qlocal | ((uint32_t)hf << 16);
+          ent[18] = (uint32_t)e_prev;
+        }
+        qn += n_new;
       }
     }
   };
@@ -396,6 +465,7 @@ __global__ void __launch_bounds__(64 * TF_W, 2) topk_i8_filter_kernel(ContractAr
     if (++k >= n_st) break;
   }
   tile_test(NQT - 1, acc_prev);
+  if (qn > 0) tf_drain(wqueue, qn, r_end, q_wg, shp, ea);
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // no load may land in LDS after the workgroup has gone
 
   // ---- the parked candidates of every query leave as one run ---------------------------------------
