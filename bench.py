@@ -28,7 +28,9 @@ for _p in (ROOT, os.path.join(ROOT, "dice-embeddings_amd")):
 # MI355X dense bf16 MFMA peak.  fp32 tables run on the same unit: each operand is split into three bf16
 # parts and a product is the sum of six bf16 products, so the ceiling for the 2*d flop of an fp32 score is a
 # sixth of the bf16 peak (above the 157.3 TFLOP/s of the fp32 MFMA itself).
-PEAK_TFLOPS = {"bf16": 2500.0, "fp32": 2500.0 / 6.0}
+# int8 tables with d = 128 are scanned for top-k by an int8 x int8 -> int32 MFMA filter (dense int8 peak 5.0 POP/s);
+# the candidates it lets through are scored again exactly (int8 row widened to bf16, bf16 x bf16 -> f32).
+PEAK_TFLOPS = {"bf16": 2500.0, "fp32": 2500.0 / 6.0, "int8": 5000.0}
 FP32_MFMA_PEAK_TFLOPS = 157.3
 # HBM bytes per launch of the main loop measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on the full-size
 # workload (each scaled by what the same counter reads for a plain 1 GiB copy kernel: x2.00 and x1.00).
@@ -220,6 +222,8 @@ def main():
     N, d = cfg.N, cfg.d
     scores = float(n_queries) * N
     compute = "fp32" if cfg.storage == "fp32" else "bf16"
+    if cfg.storage == "int8" and mode == "topk" and d == 128:
+        compute = "int8"
     flops = 2.0 * d * scores                                    # algorithmic: 2*d flop per entity score
     if mode in ("bcegrad", "train"):
         flops *= 3.0                                            # scores, dQ = g E, dE = g^T Q
@@ -236,7 +240,8 @@ def main():
         "n_gpus": 1, "steps": steps, "warmup": args.warmup,
         "ms_per_step": elapsed * 1e3 / steps,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": {"fp32": "f32 as 3 x bf16 parts, bf16 x bf16 -> f32", "bf16": "bf16 x bf16 -> f32", "int8": "int8 table as bf16 x bf16 -> f32"}[cfg.storage],
+        "dtype": {"fp32": "f32 as 3 x bf16 parts, bf16 x bf16 -> f32", "bf16": "bf16 x bf16 -> f32", "int8": "int8 table as bf16 x bf16 -> f32"}[cfg.storage]
+                 if compute != "int8" else "int8 x int8 -> i32 filter scan, candidates rescored as bf16 x bf16 -> f32",
         "data": "synthetic",
         "launch": "one HIP graph replay per step" if args.graph else "eager launches",
         "config": {"workload": f"{args.config}: {cfg.model} {mode}, N={N} entities, d={d}, {cfg.storage} tables, "
@@ -251,11 +256,14 @@ def main():
                      "frac": achieved / PEAK_TFLOPS[compute] if achieved is not None else None,
                      **({"peak_basis": "bf16 dense MFMA 2500 / 6 products per fp32 product",
                          "vs_fp32_mfma_peak": achieved / FP32_MFMA_PEAK_TFLOPS if achieved is not None else None}
-                        if compute == "fp32" else {}),
+                        if compute == "fp32" else
+                        {"peak_basis": "int8 dense MFMA, 5.0 POP/s (integer operations, not flop)",
+                         "vs_bf16_mfma_peak": achieved / PEAK_TFLOPS["bf16"] if achieved is not None else None}
+                        if compute == "int8" else {}),
                      "traffic": MEASURED_TRAFFIC_BYTES.get(args.config) if mode == MODE[args.config] else None
                      if args.scale == 1.0 and args.mode is None else None,
                      "traffic_source": "measured offline, not in this run: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on "
-                                       "this workload, scaled by a 1 GiB copy kernel (profiles/*_hbm_traffic.md)",
+                                       "this workload, scaled by a 1 GiB copy kernel (profiles/*_counters.md)",
                      "kernel": main_loop_kernel(cfg.storage, d, mode),
                      "kernel_ms_avg": kernel_ms / max(launches, 1), "launches": launches,
                      "kernel_time_share": kernel_ms * 1e-3 / elapsed},
