@@ -102,7 +102,7 @@ def main_loop_kernel(storage, d, mode):
     if d == 128:
         return "topk_i8_filter_kernel" if epi == "TopkEpi" else f"qreg_i8_kernel<{epi}>"
     if storage == "bf16" and d > 128:
-        return f"kchunk_bf16_kernel<{epi}>"
+        return f"kchunk_kernel<{epi}>"
     return f"qreg_kernel<{storage}, {epi}>"
 
 

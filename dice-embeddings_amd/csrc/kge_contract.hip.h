@@ -4,7 +4,7 @@
 //   qreg_async_kernel   bf16 table, d == 128: persistent, queries register-resident, entity rows global -> LDS
 //   qreg_i8_kernel      per-row int8 table, d == 128: the same walk, rows widened to bf16 on the way into LDS
 //   qreg_kernel         bf16 / int8 with d < 128
-//   kchunk_bf16_kernel  bf16 with d > 128: K in chunks of 64 through LDS
+//   kchunk_kernel       bf16 / int8 with d > 128: K in chunks of 64 through LDS
 //   ksplit_kernel       fp32 tables, any d: every operand as three bf16 parts, six part products per product
 // Reduction order of one score is fixed (k ascending in steps of the MFMA depth, nothing else), so
 // every kernel that forms dot(Q[b], E[e]) with these helpers produces the same fp32 bit pattern.
@@ -1678,8 +1678,9 @@ __global__ void __launch_bounds__(512, 2) ksplit_kernel(ContractArgs a, typename
 }
 
 // ============================================================================================
-// kchunk_bf16_kernel: bf16 table of any width (d % 8 == 0); used for d > 128, where the queries no longer
-// fit the register file of the persistent kernel.  The shape of ksplit_kernel with one part per operand:
+// kchunk_kernel: bf16 or per-row int8 table of any width (d % 8 == 0); used for d > 128, where the queries no
+// longer fit the register file of the persistent kernel.  int8 rows are widened to bf16 (exactly) on the way into
+// LDS and a finished tile's scores are multiplied by the row scales, as in the other int8 kernels.  The shape of ksplit_kernel with one part per operand:
 // 256 entities x 128 queries per workgroup of 8 waves (64 x 64 per wave), K in chunks of 64, both operands
 // staged through registers into double-buffered LDS (the fp32 queries are rounded to bf16 on the way, as in
 // the other bf16 kernels), one MFMA per 32 x 32 x 16 block.  Reduction order per score: K ascending in steps of
@@ -1692,8 +1693,10 @@ constexpr int KB_E_PLANE = KS_TILE_ROWS * 128;
 constexpr int KB_Q_PLANE = KS_WG_QUERIES * 128;
 constexpr int KB_STAGE_BYTES = KB_E_PLANE + KB_Q_PLANE;
 
-template <template <int> class EpiT>
-__global__ void __launch_bounds__(512, 2) kchunk_bf16_kernel(ContractArgs a, typename EpiT<KS_NQT>::Args ea) {
+template <int EDT, template <int> class EpiT>
+__global__ void __launch_bounds__(512, 2) kchunk_kernel(ContractArgs a, typename EpiT<KS_NQT>::Args ea) {
+  static_assert(EDT == KGE_BF16 || EDT == KGE_I8, "bf16 or int8 rows");
+  constexpr bool I8 = (EDT == KGE_I8);
   using Epi = EpiT<KS_NQT>;
   __shared__ __attribute__((aligned(1024))) unsigned char lds[2 * KB_STAGE_BYTES];
 
@@ -1716,9 +1719,11 @@ __global__ void __launch_bounds__(512, 2) kchunk_bf16_kernel(ContractArgs a, typ
   const int nkc = (d + KB_KC - 1) / KB_KC;
   const int n_et = (int)((r1 - r0 + KS_TILE_ROWS - 1) / KS_TILE_ROWS);
   const int n_it = n_et * nkc;
-  const uint16_t* Eb = (const uint16_t*)a.E;
+  const unsigned char* Eb = (const unsigned char*)a.E;
+  constexpr int ESZ = I8 ? 1 : 2;  // bytes per table element
 
-  // Staging (branch-free, clamped addresses, zeroing at store time): entity rows as 16-byte pieces of 8 bf16,
+  // Staging (branch-free, clamped addresses, zeroing at store time): entity rows as pieces of 8 elements (16 bytes
+  // of bf16, or 8 bytes of int8 that become 16 bytes of bf16 when stored),
   // 4 passes of 64 rows (8 lanes read one 128 B line); query rows as fp32, 4 passes of 32 rows (16 lanes read
   // 256 B of one row), rounded to bf16 when stored.
   const int e_row = tid >> 3, e_piece = tid & 7;
@@ -1744,7 +1749,13 @@ __global__ void __launch_bounds__(512, 2) kchunk_bf16_kernel(ContractArgs a, typ
     for (int g = 0; g < 4; ++g) {
       int64_t er = ld_row + 64 * g;
       er = er < e_last ? er : e_last;
-      se[g] = *(const u32x4*)(Eb + er * d + (ld_e_ok ? ke : 0));
+      const unsigned char* src = Eb + (er * d + (ld_e_ok ? ke : 0)) * ESZ;
+      if (I8) {
+        const u32x2 w = *(const u32x2*)src;
+        se[g] = u32x4{w[0], w[1], 0u, 0u};
+      } else {
+        se[g] = *(const u32x4*)src;
+      }
       sq[g] = *(const f32x4*)(q_ptr[g] + (ld_q_ok ? kq : 0));
     }
     const bool wrap = (ld_kc == nkc - 1);
@@ -1757,7 +1768,7 @@ __global__ void __launch_bounds__(512, 2) kchunk_bf16_kernel(ContractArgs a, typ
     unsigned char* base = lds + buf * KB_STAGE_BYTES;
 #pragma unroll
     for (int g = 0; g < 4; ++g) {
-      u32x4 v = se[g];
+      u32x4 v = I8 ? i8x8_to_bf16x8(se[g][0], se[g][1]) : se[g];
 #pragma unroll
       for (int j = 0; j < 4; ++j) v[j] = st_e_ok ? v[j] : 0u;
       *(u32x4*)(base + g * 8192 + e_off) = v;
@@ -1823,8 +1834,18 @@ __global__ void __launch_bounds__(512, 2) kchunk_bf16_kernel(ContractArgs a, typ
       for (int te = 0; te < 2; ++te) {
         const int64_t e_base = et0 + 64 * we + 32 * te;
         if (e_base < r1) {
+          float sc_col = 1.f;
+          if (I8) {  // the scales of the rows this lane holds (rows past the chunk's end: its last row's, ignored)
 #pragma unroll
-          for (int tq = 0; tq < 2; ++tq) epi.template tile<false>(tq, acc[te][tq], sc16, 1.f, e_base, r1);
+            for (int i = 0; i < 16; ++i) {
+              const int64_t er = e_base + row_of(i, hf);
+              sc16[i] = a.scale[er < e_last ? er : e_last];
+            }
+            const int64_t ec = e_base + c;
+            sc_col = a.scale[ec < e_last ? ec : e_last];
+          }
+#pragma unroll
+          for (int tq = 0; tq < 2; ++tq) epi.template tile<I8>(tq, acc[te][tq], sc16, sc_col, e_base, r1);
         }
 #pragma unroll
         for (int tq = 0; tq < 2; ++tq)

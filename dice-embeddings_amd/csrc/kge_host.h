@@ -72,7 +72,7 @@ inline Status contract_rules(const char* who, const void* Q, const void* E, int 
     case KGE_I8:
       if (!(d >= 16 && d % 16 == 0))
         KGE_HOST_FAIL(st, KGE_ERR_INVALID, "%s: int8 tables need d %% 16 == 0, got %lld", who, (long long)d);
-      if (d > 128) KGE_HOST_FAIL(st, KGE_ERR_UNSUPPORTED, "%s: int8 tables support d <= 128, got %lld", who, (long long)d);
+      if (d > 65536) KGE_HOST_FAIL(st, KGE_ERR_INVALID, "%s: d=%lld", who, (long long)d);
       if (!scale) KGE_HOST_FAIL(st, KGE_ERR_INVALID, "%s: int8 tables need per-row scales", who);
       break;
     default: KGE_HOST_FAIL(st, KGE_ERR_INVALID, "%s: unknown dtype %d", who, dtype);
@@ -120,11 +120,25 @@ inline RankWsOffsets rank_ws_offsets(int64_t B) {
 constexpr int TOPK_ROWMETA_ROWS = 64;
 constexpr int TOPK_ROWMETA_BYTES = 32;  // per 32-row tile {scale, max L1 + 64, forced, -}
 constexpr int TOPK_REQUANT_D = 128;
+// qh / qc: the queries as the int8 filter scan reads them (TOPK_REQUANT_D int8 per query, and per query the four
+// constants of its bound), written once per call.
 struct TopkWsOffsets {
-  size_t tau, tau_scan, cnt, list_len, dirty, n_dirty, list, cand, cand_id, rowmeta, requant, total;
+  size_t tau, tau_scan, cnt, list_len, dirty, n_dirty, list, cand, cand_id, qh, qc, rowmeta, requant, total;
   int64_t kpad;
 };
-inline TopkWsOffsets topk_ws_offsets(int64_t B, int64_t N, int64_t k) {
+// the prepared form of an int8 table (what kge_topk_prepare writes): rowmeta records, then the requantised rows
+struct TopkPreparedOffsets {
+  size_t rowmeta, requant, total;
+};
+inline TopkPreparedOffsets topk_prepared_offsets(int64_t N) {
+  TopkPreparedOffsets o{};
+  o.rowmeta = 0;
+  o.requant = align_up((size_t)((N + TOPK_ROWMETA_ROWS - 1) / TOPK_ROWMETA_ROWS) * TOPK_ROWMETA_BYTES, 256);
+  o.total = o.requant + align_up((size_t)N * TOPK_REQUANT_D, 256);
+  return o;
+}
+// with_table: the workspace also holds the prepared form of the table (a call that was not handed one)
+inline TopkWsOffsets topk_ws_offsets(int64_t B, int64_t N, int64_t k, bool with_table = true) {
   TopkWsOffsets o{};
   size_t off = 0;
   auto take = [&](size_t bytes) {
@@ -142,8 +156,16 @@ inline TopkWsOffsets topk_ws_offsets(int64_t B, int64_t N, int64_t k) {
   o.list = take((size_t)B * (size_t)o.kpad * 8);
   o.cand = take((size_t)B * TOPK_CAP * 8);
   o.cand_id = take((size_t)B * TOPK_CAP * 4);
-  o.rowmeta = take((size_t)((N + TOPK_ROWMETA_ROWS - 1) / TOPK_ROWMETA_ROWS) * TOPK_ROWMETA_BYTES);
-  o.requant = take((size_t)N * TOPK_REQUANT_D);
+  o.qh = take((size_t)B * TOPK_REQUANT_D);
+  o.qc = take((size_t)B * 16);
+  if (with_table) {
+    const TopkPreparedOffsets t = topk_prepared_offsets(N);
+    const size_t base = take(t.total);
+    o.rowmeta = base + t.rowmeta;
+    o.requant = base + t.requant;
+  } else {
+    o.rowmeta = o.requant = off;
+  }
   o.total = off;
   return o;
 }

@@ -619,11 +619,15 @@ struct TopkWs {
   uint32_t* cand_id;         // [B, TOPK_CAP] entity ids (int8 filter scan; scored into `cand` before they are ranked)
   unsigned char* rowmeta;    // int8 filter scan: per 64 table rows one record
   int8_t* requant;           // int8 filter scan: the table with one scale per 32-row tile
+  int8_t* qh;                // int8 filter scan: the queries as int8
+  f32x4* qc;                 // int8 filter scan: per query the constants of its bound
   int64_t kpad;
 };
 
-size_t topk_ws_layout(int64_t B, int64_t N, int64_t k, void* base, TopkWs* ws) {
-  const host::TopkWsOffsets o = host::topk_ws_offsets(B, N, k);
+// `prepared`: the table's prepared form is in the caller's hands (kge_topk_prepare); the workspace then holds none
+size_t topk_ws_layout(int64_t B, int64_t N, int64_t k, void* base, TopkWs* ws, const void* prepared = nullptr,
+                      bool with_table = true) {
+  const host::TopkWsOffsets o = host::topk_ws_offsets(B, N, k, with_table);
   if (ws) {
     char* p = (char*)base;
     ws->tau = (float*)(p + o.tau);
@@ -635,8 +639,16 @@ size_t topk_ws_layout(int64_t B, int64_t N, int64_t k, void* base, TopkWs* ws) {
     ws->list = (unsigned long long*)(p + o.list);
     ws->cand = (unsigned long long*)(p + o.cand);
     ws->cand_id = (uint32_t*)(p + o.cand_id);
-    ws->rowmeta = (unsigned char*)(p + o.rowmeta);
-    ws->requant = (int8_t*)(p + o.requant);
+    ws->qh = (int8_t*)(p + o.qh);
+    ws->qc = (f32x4*)(p + o.qc);
+    if (with_table) {
+      ws->rowmeta = (unsigned char*)(p + o.rowmeta);
+      ws->requant = (int8_t*)(p + o.requant);
+    } else {
+      const host::TopkPreparedOffsets t = host::topk_prepared_offsets(N);
+      ws->rowmeta = (unsigned char*)prepared + t.rowmeta;
+      ws->requant = (int8_t*)((unsigned char*)prepared + t.requant);
+    }
     ws->kpad = o.kpad;
   }
   return o.total;
@@ -1063,7 +1075,7 @@ ContractArgs make_args(const float* Q, const void* E, int dtype, const float* sc
   a.ldq = a.lde = 0;
   a.k_split_len = 0;
   const bool fast_bf16 = (dtype == KGE_BF16 && d == 128), fast_i8 = (dtype == KGE_I8 && d == 128);
-  const bool wide_bf16 = (dtype == KGE_BF16 && d > 128);  // kchunk_bf16_kernel: the workgroup shape of the split kernel
+  const bool wide_bf16 = ((dtype == KGE_BF16 || dtype == KGE_I8) && d > 128);  // kchunk_kernel: the workgroup shape of the split kernel
   const int wgq = (dtype == KGE_F32) ? KS_WG_QUERIES : fast_bf16 ? QA_WG_QUERIES : fast_i8 ? I8_WG_QUERIES
                   : wide_bf16 ? KS_WG_QUERIES : QREG_WG_QUERIES;
   a.n_qgroups = (int)((B + wgq - 1) / wgq);
@@ -1152,7 +1164,7 @@ int launch_contract(int dtype, const ContractArgs& a, const EArgs& ea, hipStream
   const int64_t nwg = persistent ? 8 * (int64_t)a.n_qgroups * a.n_lanes : contract_grid_wgs(a);
   KGE_REQUIRE(nwg <= 0x7fffffffLL, KGE_ERR_INVALID, "%s: grid of %lld workgroups too large", name, (long long)nwg);
   const bool f32_split = (dtype == KGE_F32);
-  const bool wide_bf16 = (dtype == KGE_BF16 && a.d > 128);
+  const bool wide_bf16 = ((dtype == KGE_BF16 || dtype == KGE_I8) && a.d > 128);
   dim3 grid((unsigned)nwg), block(fast_i8 ? 64 * I8_WG_WAVES : persistent ? 64 * QA_WG_WAVES : (f32_split || wide_bf16) ? 512 : 256);
   LaunchTimer timer;
   if (int trc = timer.begin(st)) return trc;
@@ -1168,8 +1180,10 @@ int launch_contract(int dtype, const ContractArgs& a, const EArgs& ea, hipStream
     else
       hipLaunchKernelGGL((qreg_async_kernel<EpiT>), grid, block, 0, st, a, ea);
   }
+  else if (wide_bf16 && dtype == KGE_BF16)
+    hipLaunchKernelGGL((kchunk_kernel<KGE_BF16, EpiT>), grid, block, 0, st, a, ea);
   else if (wide_bf16)
-    hipLaunchKernelGGL((kchunk_bf16_kernel<EpiT>), grid, block, 0, st, a, ea);
+    hipLaunchKernelGGL((kchunk_kernel<KGE_I8, EpiT>), grid, block, 0, st, a, ea);
   else if (dtype == KGE_BF16)
     hipLaunchKernelGGL((qreg_kernel<KGE_BF16, EpiT>), grid, block, 0, st, a, ea);
   else if (fast_i8)
@@ -1491,6 +1505,54 @@ extern "C" size_t kge_topk_workspace_bytes(int64_t B, int64_t N, int64_t k) {
   return topk_ws_layout(B, N, k, nullptr, nullptr);
 }
 
+namespace {
+// does a table of this storage and width have a prepared form for top-k?
+bool topk_has_prepared_form(int dtype, int64_t d) { return dtype == KGE_I8 && d == host::TOPK_REQUANT_D; }
+
+int topk_prepare_launch(const void* E, const float* scale, int64_t N, unsigned char* rowmeta, int8_t* requant,
+                        hipStream_t st) {
+  const int64_t n_rec = (N + host::TOPK_ROWMETA_ROWS - 1) / host::TOPK_ROWMETA_ROWS;
+  hipLaunchKernelGGL(topk_i8_requant_kernel, dim3((unsigned)n_rec), dim3(256), 0, st, (const int8_t*)E, scale, N, requant,
+                     rowmeta);
+  KGE_LAUNCH_CHECK("topk_i8_requant_kernel");
+  return KGE_OK;
+}
+
+int topk_impl(const char* who, const float* Q, const float* bias, const void* E, int dtype, const float* scale, int64_t B,
+              int64_t d, int64_t N, int64_t k, float* out_scores, int64_t* out_idx, int apply_sigmoid,
+              const void* prepared, void* workspace, hipStream_t st);
+}  // namespace
+
+extern "C" size_t kge_topk_prepared_bytes(int dtype, int64_t d, int64_t N) {
+  if (!topk_has_prepared_form(dtype, d) || N < 1) return 0;
+  return host::topk_prepared_offsets(N).total;
+}
+
+extern "C" int kge_topk_prepare(const void* E, int dtype, const float* scale, int64_t d, int64_t N, void* prepared,
+                                size_t prepared_bytes, void* stream) {
+  clear_error();
+  KGE_REQUIRE(topk_has_prepared_form(dtype, d), KGE_ERR_UNSUPPORTED,
+              "kge_topk_prepare: tables of dtype %d with d=%lld have no prepared form (int8 with d = %d does)", dtype,
+              (long long)d, host::TOPK_REQUANT_D);
+  KGE_REQUIRE(N >= 1 && N <= 0x7fffffffLL, KGE_ERR_INVALID, "kge_topk_prepare: N=%lld", (long long)N);
+  KGE_REQUIRE(E && scale && prepared, KGE_ERR_INVALID, "kge_topk_prepare: null pointer argument");
+  KGE_REQUIRE((((uintptr_t)E | (uintptr_t)prepared) & 15) == 0, KGE_ERR_INVALID,
+              "kge_topk_prepare: E and prepared must be 16-byte aligned");
+  KGE_REQUIRE(prepared_bytes >= kge_topk_prepared_bytes(dtype, d, N), KGE_ERR_WORKSPACE,
+              "kge_topk_prepare: buffer of %zu bytes, need %zu", prepared_bytes, kge_topk_prepared_bytes(dtype, d, N));
+  const host::TopkPreparedOffsets t = host::topk_prepared_offsets(N);
+  return topk_prepare_launch(E, scale, N, (unsigned char*)prepared + t.rowmeta,
+                             (int8_t*)((unsigned char*)prepared + t.requant), (hipStream_t)stream);
+}
+
+extern "C" size_t kge_topk_prepared_workspace_bytes(int64_t B, int64_t N, int64_t k) {
+  if (B < 1) B = 1;
+  if (N < 1) N = 1;
+  if (k < 1) k = 1;
+  if (k > TOPK_MAX_K) k = TOPK_MAX_K;
+  return topk_ws_layout(B, N, k, nullptr, nullptr, nullptr, false);
+}
+
 extern "C" int kge_topk(const float* Q, const float* bias, const void* E, int dtype, const float* scale, int64_t B,
                         int64_t d, int64_t N, int64_t k, float* out_scores, int64_t* out_idx, int apply_sigmoid,
                         void* workspace, size_t workspace_bytes, void* stream) {
@@ -1505,21 +1567,59 @@ extern "C" int kge_topk(const float* Q, const float* bias, const void* E, int dt
   KGE_REQUIRE(workspace && workspace_bytes >= kge_topk_workspace_bytes(B, N, k), KGE_ERR_WORKSPACE,
               "kge_topk: workspace of %zu bytes, need %zu", workspace_bytes, kge_topk_workspace_bytes(B, N, k));
   KGE_REQUIRE(((uintptr_t)workspace & 15) == 0, KGE_ERR_WORKSPACE, "kge_topk: workspace must be 16-byte aligned");
-  hipStream_t st = (hipStream_t)stream;
+  return topk_impl("kge_topk", Q, bias, E, dtype, scale, B, d, N, k, out_scores, out_idx, apply_sigmoid, nullptr,
+                   workspace, (hipStream_t)stream);
+}
+
+extern "C" int kge_topk_prepared(const float* Q, const float* bias, const void* E, int dtype, const float* scale, int64_t B,
+                                 int64_t d, int64_t N, int64_t k, float* out_scores, int64_t* out_idx, int apply_sigmoid,
+                                 const void* prepared, size_t prepared_bytes, void* workspace, size_t workspace_bytes,
+                                 void* stream) {
+  clear_error();
+  int rc = check_contract("kge_topk_prepared", Q, E, dtype, scale, B, d, N);
+  if (rc) return rc;
+  KGE_REQUIRE(k >= 1 && k <= N, KGE_ERR_INVALID, "kge_topk_prepared: k=%lld outside [1, N=%lld]", (long long)k,
+              (long long)N);
+  KGE_REQUIRE(k <= TOPK_MAX_K, KGE_ERR_UNSUPPORTED, "kge_topk_prepared: k=%lld above the supported maximum %d",
+              (long long)k, TOPK_MAX_K);
+  KGE_REQUIRE(topk_has_prepared_form(dtype, d), KGE_ERR_UNSUPPORTED,
+              "kge_topk_prepared: tables of dtype %d with d=%lld have no prepared form; call kge_topk", dtype, (long long)d);
+  KGE_REQUIRE(prepared && prepared_bytes >= kge_topk_prepared_bytes(dtype, d, N), KGE_ERR_WORKSPACE,
+              "kge_topk_prepared: prepared table of %zu bytes, need %zu", prepared_bytes,
+              kge_topk_prepared_bytes(dtype, d, N));
+  KGE_REQUIRE(((uintptr_t)prepared & 15) == 0, KGE_ERR_INVALID, "kge_topk_prepared: prepared must be 16-byte aligned");
+  if (B == 0) return KGE_OK;
+  KGE_REQUIRE(out_scores && out_idx, KGE_ERR_INVALID, "kge_topk_prepared: null output pointer");
+  KGE_REQUIRE(workspace && workspace_bytes >= kge_topk_prepared_workspace_bytes(B, N, k), KGE_ERR_WORKSPACE,
+              "kge_topk_prepared: workspace of %zu bytes, need %zu", workspace_bytes,
+              kge_topk_prepared_workspace_bytes(B, N, k));
+  KGE_REQUIRE(((uintptr_t)workspace & 15) == 0, KGE_ERR_WORKSPACE, "kge_topk_prepared: workspace must be 16-byte aligned");
+  return topk_impl("kge_topk_prepared", Q, bias, E, dtype, scale, B, d, N, k, out_scores, out_idx, apply_sigmoid, prepared,
+                   workspace, (hipStream_t)stream);
+}
+
+namespace {
+int topk_impl(const char* who, const float* Q, const float* bias, const void* E, int dtype, const float* scale, int64_t B,
+              int64_t d, int64_t N, int64_t k, float* out_scores, int64_t* out_idx, int apply_sigmoid,
+              const void* prepared, void* workspace, hipStream_t st) {
+  int rc = KGE_OK;
   TopkWs ws;
-  topk_ws_layout(B, N, k, workspace, &ws);
+  topk_ws_layout(B, N, k, workspace, &ws, prepared, prepared == nullptr);
   hipLaunchKernelGGL(topk_init_kernel, dim3((unsigned)((B + 255) / 256)), dim3(256), 0, st, ws, B);
   KGE_LAUNCH_CHECK("topk_init_kernel");
 
   // An int8 table with d == 128 is scanned by the integer filter (after the first round, which takes every row
   // anyway): its candidates are entity ids that passed a bound, scored exactly before they are ranked.  Every other
-  // scan is the contraction's own top-k epilogue, whose candidates are exact keys.
-  const bool id_filter = (dtype == KGE_I8 && d == 128 && N > TOPK_FIRST_ROWS);
+  // scan is the contraction's own top-k epilogue, whose candidates are exact keys.  The filter reads the table in
+  // its prepared form (the caller's, or made here in the workspace) and the queries as int8 (made here).
+  const bool id_filter = (topk_has_prepared_form(dtype, d) && N > TOPK_FIRST_ROWS);
   if (id_filter) {
-    const int64_t n_rec = (N + host::TOPK_ROWMETA_ROWS - 1) / host::TOPK_ROWMETA_ROWS;
-    hipLaunchKernelGGL(topk_i8_requant_kernel, dim3((unsigned)n_rec), dim3(256), 0, st, (const int8_t*)E,
-                       scale, N, ws.requant, ws.rowmeta);
-    KGE_LAUNCH_CHECK("topk_i8_requant_kernel");
+    if (prepared == nullptr) {
+      rc = topk_prepare_launch(E, scale, N, ws.rowmeta, ws.requant, st);
+      if (rc) return rc;
+    }
+    hipLaunchKernelGGL(topk_i8_qprep_kernel, dim3((unsigned)((B + 3) / 4)), dim3(256), 0, st, Q, B, ws.qh, ws.qc);
+    KGE_LAUNCH_CHECK("topk_i8_qprep_kernel");
   }
   // One scan of entity rows [e0, e1) with the thresholds `tau`, for all queries or those flagged in `active`.
   auto launch_scan = [&](int64_t e0, int64_t e1, const float* tau, const int32_t* active, int rescan,
@@ -1544,7 +1644,7 @@ extern "C" int kge_topk(const float* Q, const float* bias, const void* E, int dt
     a.n_chunks = (e1 - e0 + chunk - 1) / chunk;
     const int64_t nwg = 8 * (int64_t)a.n_qgroups * a.n_lanes;
     KGE_REQUIRE(nwg <= 0x7fffffffLL, KGE_ERR_INVALID, "%s: grid of %lld workgroups too large", name, (long long)nwg);
-    I8FilterArgs ea{tau, active, ws.cnt, ws.cand_id, TOPK_CAP, ws.requant, ws.rowmeta};
+    I8FilterArgs ea{tau, active, ws.cnt, ws.cand_id, TOPK_CAP, ws.requant, ws.rowmeta, ws.qh, ws.qc};
     LaunchTimer timer;
     if (int trc = timer.begin(st)) return trc;
     hipLaunchKernelGGL(topk_i8_filter_kernel, dim3((unsigned)nwg), dim3(64 * TF_W), 0, st, a, ea);
@@ -1587,13 +1687,14 @@ extern "C" int kge_topk(const float* Q, const float* bias, const void* E, int dt
     KGE_HIP_CHECK(hipMemcpyAsync(&n_dirty, ws.n_dirty, sizeof(int32_t), hipMemcpyDeviceToHost, st));
     KGE_HIP_CHECK(hipStreamSynchronize(st));
   }
-  KGE_REQUIRE(n_dirty == 0, KGE_ERR_OVERFLOW, "kge_topk: %d queries still overflow their candidate buffers", n_dirty);
+  KGE_REQUIRE(n_dirty == 0, KGE_ERR_OVERFLOW, "%s: %d queries still overflow their candidate buffers", who, n_dirty);
   const int64_t total = B * k;
   hipLaunchKernelGGL(topk_output_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, ws, B, (int)k, bias,
                      apply_sigmoid, out_scores, out_idx);
   KGE_LAUNCH_CHECK("topk_output_kernel");
   return KGE_OK;
 }
+}  // namespace
 
 extern "C" int kge_row_minmax(const float* Q, const float* bias, const void* E, int dtype, const float* scale,
                               int64_t B, int64_t d, int64_t N, float* out_min, float* out_max, void* stream) {

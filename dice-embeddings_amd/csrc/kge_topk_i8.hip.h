@@ -44,6 +44,8 @@ struct I8FilterArgs {
   int32_t cap;
   const int8_t* Eq;              // the table with tile-common scales (topk_i8_requant_kernel)
   const unsigned char* rowmeta;  // one record per 64 table rows: per 32-row tile {S, max L1(e') + 64, forced, 1 / S}
+  const int8_t* qh;              // [B, 128] the queries as int8 (topk_i8_qprep_kernel)
+  const f32x4* qc;               // [B] per query {s_q, mq, cq, finite ? 1 : 0}
 };
 
 constexpr int TF_NQT = 4;                              // 32-query tiles per wave
@@ -56,18 +58,8 @@ constexpr int TF_BUCKET = 16;                          // candidate ids a query 
 constexpr int TF_VALU_PER_MFMA = 4;
 static_assert(host::TOPK_ROWMETA_ROWS == TF_STAGE_ROWS && host::TOPK_ROWMETA_BYTES == 32, "record per stage");
 
-// One candidate id into its query's global buffer; slot is the query's running count.  A full buffer keeps a
-// uniform sample of what arrives (the query is repaired by a later rescan with its final threshold).
-__device__ __forceinline__ void tf_place(const I8FilterArgs& a, int64_t q, int32_t slot, uint32_t e) {
-  if (slot >= a.cap) {
-    uint32_t h = (e * 2654435761u) ^ ((uint32_t)slot * 0x9e3779b9u);
-    h ^= h >> 15; h *= 0x2c1b3c6du; h ^= h >> 12;
-    const uint32_t r = h % (uint32_t)(slot + 1);
-    slot = (r < (uint32_t)a.cap) ? (int32_t)r : -1;
-  }
-  if (slot >= 0) a.cand[q * a.cap + slot] = e;
-}
-
+// (a candidate id goes into its query's global buffer at the query's running count; a full buffer keeps a uniform
+// sample of what arrives, and the query is repaired by a later rescan with its final threshold: tf_place below)
 // The table with one scale per 32-row tile, and per 64 rows one record for the scan.  One workgroup per 64 rows:
 // thread t takes 16 bytes of row (t >> 3) of each of the two tiles, so loads and stores are whole rows in order.
 // A row past the table's end counts for nothing; a scale that is not finite forces its tile (the scan then takes
@@ -137,18 +129,77 @@ __global__ void __launch_bounds__(256) topk_i8_requant_kernel(const int8_t* E, c
   }
 }
 
+// The queries as the scan reads them, once per call.  One wave per query, two components per lane: the row rounded
+// to bf16 (qb, the operand of the exact score), its largest magnitude and L1 norm, then qb_k = s_q qh_k + delta_k with
+// qh_k an int8 and dq = max |delta_k|.  Per query {s_q, mq = dq + 4e-3 s_q, cq = 0.501 L1(qb), finite}: a row with a
+// component that is not finite has no finite bound (finite = 0: the scan collects nothing for it; its scores are NaN
+// or infinite anyway).
+__global__ void __launch_bounds__(256) topk_i8_qprep_kernel(const float* Q, int64_t B, int8_t* qh, f32x4* qc) {
+  const int lane = threadIdx.x & 63;
+  const int64_t q = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (q >= B) return;
+  const float* row = Q + q * 128;
+  const float r0 = (float)(__bf16)row[2 * lane], r1 = (float)(__bf16)row[2 * lane + 1];
+  float amax = __builtin_fmaxf(__builtin_fabsf(r0), __builtin_fabsf(r1));
+  float l1q = __builtin_fabsf(r0) + __builtin_fabsf(r1);
+  int bad = (r0 != r0 || r1 != r1) ? 1 : 0;  // fmax drops a NaN
+#pragma unroll
+  for (int o = 1; o < 64; o <<= 1) {
+    amax = __builtin_fmaxf(amax, __shfl_xor(amax, o, 64));
+    l1q += __shfl_xor(l1q, o, 64);
+    bad |= __shfl_xor(bad, o, 64);
+  }
+  const bool finite = !bad && amax <= 3.4028234e38f && l1q <= 3.4028234e38f;
+  const float s_q = finite ? amax / 127.f : 0.f;
+  const float inv = (finite && amax > 0.f) ? 127.f / amax : 0.f;
+  float dq = 0.f;
+  uint32_t pk = 0;
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    const float r = finite ? (j ? r1 : r0) : 0.f;
+    float h = __builtin_rintf(r * inv);
+    h = __builtin_fminf(__builtin_fmaxf(h, -127.f), 127.f);
+    dq = __builtin_fmaxf(dq, __builtin_fabsf(__builtin_fmaf(-s_q, h, r)));
+    pk |= ((uint32_t)(int)h & 0xffu) << (8 * j);
+  }
+#pragma unroll
+  for (int o = 1; o < 64; o <<= 1) dq = __builtin_fmaxf(dq, __shfl_xor(dq, o, 64));
+  ((uint16_t*)(qh + q * 128))[lane] = (uint16_t)pk;
+  if (lane == 0) {
+    const f32x4 c = {s_q, dq * 1.000001f + 4e-3f * s_q, finite ? 0.501f * l1q * 1.00001f : 0.f, finite ? 1.f : 0.f};
+    qc[q] = c;
+  }
+}
+
 constexpr int TF_QUEUE = 64;         // parked accumulator sets per wave
 constexpr int TF_QUEUE_STRIDE = 21;  // dwords per set (19 used; odd: lanes reading their own set hit distinct banks)
 constexpr int TF_DENSE_LANES = 16;   // a tile with more lanes of interest than this is worked off on the spot
 
-struct TfShared {
-  uint32_t* bucket;  // [TF_WG_QUERIES][TF_BUCKET] candidate ids parked per query
-  int* bcnt;         // [TF_WG_QUERIES]
+// What the out-of-line slow paths need, as few scalars as will do (every argument travels in a register: a struct
+// passed by value would go through the call frame in scratch memory, once per call and lane).
+struct TfSink {
+  uint32_t* bucket;  // LDS [TF_WG_QUERIES][TF_BUCKET] candidate ids parked per query
+  int* bcnt;         // LDS [TF_WG_QUERIES]
+  int32_t* cnt;      // global: per query, candidates appended this round
+  uint32_t* cand;    // global [B, cap]
+  int32_t cap;
+  int32_t q_wg;      // first query of the workgroup
+  uint32_t limit;    // entities >= limit are padding (ids stay below 2^31, a stage's padding rows below 2^31 + 64)
 };
 
+__device__ __forceinline__ void tf_place(const TfSink& k, int64_t q, int32_t slot, uint32_t e) {
+  if (slot >= k.cap) {
+    uint32_t h = (e * 2654435761u) ^ ((uint32_t)slot * 0x9e3779b9u);
+    h ^= h >> 15; h *= 0x2c1b3c6du; h ^= h >> 12;
+    const uint32_t r = h % (uint32_t)(slot + 1);
+    slot = (r < (uint32_t)k.cap) ? (int32_t)r : -1;
+  }
+  if (slot >= 0) k.cand[q * k.cap + slot] = e;
+}
+
 // The elements among h[0..16) above thr, as candidates of local query `qlocal`: entity e_base + row_of(i, hf).
-__device__ __forceinline__ void tf_collect(const int (&h)[16], int thr, bool on, int qlocal, int hf, int64_t e_base,
-                                           int64_t limit, int64_t q_wg, const TfShared& sh, const I8FilterArgs& ea) {
+__device__ __forceinline__ void tf_collect(const int (&h)[16], int thr, bool on, int qlocal, int hf, uint32_t e_base,
+                                           const TfSink& k) {
   uint32_t bits = 0;  // bit 15 - i: element i may beat the threshold (|thr| <= 2^30, |h| < 2^21: no wrap)
 #pragma unroll
   for (int i = 0; i < 16; ++i) bits = __builtin_amdgcn_alignbit(bits, (uint32_t)(thr - h[i]), 31);
@@ -158,30 +209,33 @@ __device__ __forceinline__ void tf_collect(const int (&h)[16], int thr, bool on,
       const int b = 31 - __builtin_clz(bits);
       bits &= ~(1u << b);
       const int i = 15 - b;
-      const int64_t e = e_base + ((i >> 2) << 3) + (hf << 2) + (i & 3);
-      if (e < limit) {
-        const int idx = atomicAdd(&sh.bcnt[qlocal], 1);
+      const uint32_t e = e_base + (uint32_t)(((i >> 2) << 3) + (hf << 2) + (i & 3));
+      if (e < k.limit) {
+        const int idx = atomicAdd(&k.bcnt[qlocal], 1);
         if (idx < TF_BUCKET)
-          sh.bucket[qlocal * TF_BUCKET + idx] = (uint32_t)e;
+          k.bucket[qlocal * TF_BUCKET + idx] = e;
         else  // bucket full: straight to global memory
-          tf_place(ea, q_wg + qlocal, atomicAdd(&ea.cnt[q_wg + qlocal], 1), (uint32_t)e);
+          tf_place(k, (int64_t)k.q_wg + qlocal, atomicAdd(&k.cnt[k.q_wg + qlocal], 1), e);
       }
     }
   }
 }
 
 // A tile most of whose lanes are of interest: every lane tests its own 16 elements.  Out of line (one copy).
-__device__ __attribute__((noinline)) void tf_dense(i32x16 h, int thr, bool on, int qlocal, int hf, int64_t e_base,
-                                                   int64_t limit, int64_t q_wg, TfShared sh, I8FilterArgs ea) {
+// where = qlocal | hf << 16 | on << 17.
+__device__ __attribute__((noinline)) void tf_dense(i32x16 h, int thr, uint32_t where, uint32_t e_base, uint32_t* bucket,
+                                                   int* bcnt, int32_t* cnt, uint32_t* cand, int32_t cap, int32_t q_wg,
+                                                   uint32_t limit) {
   int hh[16];
 #pragma unroll
   for (int i = 0; i < 16; ++i) hh[i] = h[i];
-  tf_collect(hh, thr, on, qlocal, hf, e_base, limit, q_wg, sh, ea);
+  const TfSink k{bucket, bcnt, cnt, cand, cap, q_wg, limit};
+  tf_collect(hh, thr, ((where >> 17) & 1u) != 0u, (int)(where & 0xffffu), (int)((where >> 16) & 1u), e_base, k);
 }
 
 // The parked sets of a wave, one lane per set.  Out of line (one copy).
-__device__ __attribute__((noinline)) void tf_drain(const uint32_t* queue, int n, int64_t limit, int64_t q_wg,
-                                                   TfShared sh, I8FilterArgs ea) {
+__device__ __attribute__((noinline)) void tf_drain(const uint32_t* queue, int n, uint32_t* bucket, int* bcnt, int32_t* cnt,
+                                                   uint32_t* cand, int32_t cap, int32_t q_wg, uint32_t limit) {
   const int lane = threadIdx.x & 63;
   const bool on = lane < n;
   const uint32_t* ent = queue + (on ? lane : 0) * TF_QUEUE_STRIDE;
@@ -190,8 +244,9 @@ __device__ __attribute__((noinline)) void tf_drain(const uint32_t* queue, int n,
   for (int i = 0; i < 16; ++i) hh[i] = (int)ent[i];
   const int thr = (int)ent[16];
   const uint32_t where = ent[17];
-  const int64_t e_base = (int64_t)ent[18];
-  tf_collect(hh, thr, on, (int)(where & 0xffffu), (int)(where >> 16), e_base, limit, q_wg, sh, ea);
+  const uint32_t e_base = ent[18];
+  const TfSink k{bucket, bcnt, cnt, cand, cap, q_wg, limit};
+  tf_collect(hh, thr, on, (int)(where & 0xffffu), (int)(where >> 16), e_base, k);
 }
 
 __global__ void __launch_bounds__(64 * TF_W, 2) topk_i8_filter_kernel(ContractArgs a, I8FilterArgs ea) {
@@ -235,55 +290,21 @@ __global__ void __launch_bounds__(64 * TF_W, 2) topk_i8_filter_kernel(ContractAr
 #pragma unroll
   for (int t = 0; t < NQT; ++t) {
     const int64_t q = q_wg + ql0 + 32 * t + c;
-    float xb[64];  // bf16-rounded components k = 32 s + 16 hf + j of the row
-    float amax = 0.f, l1q = 0.f;
-    bool has_nan = false;
+    // the query's int8 fragments (k = 32 s + 16 hf + 0..15: sixteen consecutive bytes of its row) and constants
+    f32x4 qcv = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int s = 0; s < 4; ++s) {
-#pragma unroll
-      for (int j4 = 0; j4 < 4; ++j4) {
-        f32x4 v = {0.f, 0.f, 0.f, 0.f};
-        if (q < a.B) v = *(const f32x4*)(a.Q + q * d + 32 * s + 16 * hf + 4 * j4);
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          const float r = (float)(__bf16)v[j];
-          xb[16 * s + 4 * j4 + j] = r;
-          amax = __builtin_fmaxf(amax, __builtin_fabsf(r));
-          l1q += __builtin_fabsf(r);
-          has_nan = has_nan || (r != r);  // fmax drops a NaN
-        }
-      }
-    }
-    amax = __builtin_fmaxf(amax, __shfl_xor(amax, 32, 64));
-    l1q += __shfl_xor(l1q, 32, 64);
-    has_nan = has_nan || (__shfl_xor((int)has_nan, 32, 64) != 0);
-    const bool finite = !has_nan && amax <= 3.4028234e38f && l1q <= 3.4028234e38f;
-    const float s_q = finite ? amax / 127.f : 0.f;
-    const float inv = (finite && amax > 0.f) ? 127.f / amax : 0.f;
-    float dq = 0.f;
-#pragma unroll
-    for (int s = 0; s < 4; ++s) {
-      i32x4 w;
-#pragma unroll
-      for (int j4 = 0; j4 < 4; ++j4) {
-        uint32_t pk = 0;
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          const float r = finite ? xb[16 * s + 4 * j4 + j] : 0.f;
-          float h = __builtin_rintf(r * inv);
-          h = __builtin_fminf(__builtin_fmaxf(h, -127.f), 127.f);
-          dq = __builtin_fmaxf(dq, __builtin_fabsf(__builtin_fmaf(-s_q, h, r)));
-          pk |= ((uint32_t)(int)h & 0xffu) << (8 * j);
-        }
-        w[j4] = (int)pk;
-      }
+      i32x4 w = {0, 0, 0, 0};
+      if (q < a.B) w = *(const i32x4*)(ea.qh + q * d + 32 * s + 16 * hf);
       qf[t][s] = w;
     }
-    dq = __builtin_fmaxf(dq, __shfl_xor(dq, 32, 64));
+    if (q < a.B) qcv = ea.qc[q];
+    const float s_q = qcv[0];
+    const bool finite = qcv[3] != 0.f;
     sq[t] = s_q;
     isq[t] = s_q > 0.f ? 1.f / s_q : 0.f;
-    mq[t] = dq * 1.000001f + 4e-3f * s_q;
-    cq[t] = finite ? 0.501f * l1q * 1.00001f : 0.f;
+    mq[t] = qcv[1];
+    cq[t] = qcv[2];
     // a query with a non-finite component has no finite bound: it collects nothing (its scores are NaN or
     // infinite anyway)
     const bool on = q < a.B && finite && (ea.active == nullptr || ea.active[q] != 0);
@@ -337,7 +358,7 @@ __global__ void __launch_bounds__(64 * TF_W, 2) topk_i8_filter_kernel(ContractAr
     m_force = __builtin_amdgcn_readfirstlane(__float_as_uint(tc[2])) != 0u;
     m_iS = tc[3];
   };
-  const TfShared shp{bucket, bcnt};
+  const TfSink sink{bucket, bcnt, ea.cnt, ea.cand, ea.cap, (int32_t)q_wg, (uint32_t)r_end};
   uint32_t* const wqueue = &queue[wave][0];
   int qn = 0;  // sets parked in this wave's queue (the same in every lane)
   auto tile_test = [&](int t, const i32x16& h) {
@@ -365,10 +386,11 @@ __global__ void __launch_bounds__(64 * TF_W, 2) topk_i8_filter_kernel(ContractAr
       const int n_new = __builtin_popcountll(who);
       const int qlocal = ql0 + 32 * t + c;
       if (n_new > TF_DENSE_LANES) {
-        tf_dense(h, thr, mine, qlocal, hf, e_prev, r_end, q_wg, shp, ea);
+        tf_dense(h, thr, (uint32_t)qlocal | ((uint32_t)hf << 16) | ((uint32_t)mine << 17), (uint32_t)e_prev, sink.bucket,
+                 sink.bcnt, sink.cnt, sink.cand, sink.cap, sink.q_wg, sink.limit);
       } else if (n_new > 0) {
         if (qn + n_new > TF_QUEUE) {
-          tf_drain(wqueue, qn, r_end, q_wg, shp, ea);
+          tf_drain(wqueue, qn, sink.bucket, sink.bcnt, sink.cnt, sink.cand, sink.cap, sink.q_wg, sink.limit);
           qn = 0;
         }
         if (mine) {
@@ -465,19 +487,22 @@ __global__ void __launch_bounds__(64 * TF_W, 2) topk_i8_filter_kernel(ContractAr
     if (++k >= n_st) break;
   }
   tile_test(NQT - 1, acc_prev);
-  if (qn > 0) tf_drain(wqueue, qn, r_end, q_wg, shp, ea);
+  if (qn > 0) tf_drain(wqueue, qn, sink.bucket, sink.bcnt, sink.cnt, sink.cand, sink.cap, sink.q_wg, sink.limit);
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // no load may land in LDS after the workgroup has gone
 
   // ---- the parked candidates of every query leave as one run ---------------------------------------
+  // (sixteen lanes per query, so that the ids of a run are written side by side: whole lines, not one per id)
   __syncthreads();
-  for (int i = tid; i < WQ; i += 64 * W) {
+  static_assert(TF_BUCKET == 16 && WQ % (4 * W) == 0, "one group of sixteen lanes per bucket");
+  for (int i = tid >> 4; i < WQ; i += 4 * W) {
     const int64_t q = q_wg + i;
+    const int j = tid & 15;
     int n = bcnt[i];
     n = n < TF_BUCKET ? n : TF_BUCKET;
-    if (n > 0 && q < a.B) {
-      const int32_t base = atomicAdd(&ea.cnt[q], n);
-      for (int j = 0; j < n; ++j) tf_place(ea, q, base + j, bucket[i * TF_BUCKET + j]);
-    }
+    int32_t base = 0;
+    if (j == 0 && n > 0 && q < a.B) base = atomicAdd(&ea.cnt[q], n);
+    base = __shfl(base, lane & ~15, 64);
+    if (j < n && q < a.B) tf_place(sink, q, base + j, bucket[i * TF_BUCKET + j]);
   }
 }
 

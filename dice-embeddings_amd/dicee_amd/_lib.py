@@ -48,6 +48,11 @@ SIGNATURES = {
     "kge_topk_workspace_bytes": (_sz, [_c_i64, _c_i64, _c_i64]),
     "kge_topk": (_c_int, [_vp, _vp, _vp, _c_int, _vp, _c_i64, _c_i64, _c_i64, _c_i64, _vp, _vp, _c_int, _vp, _sz,
                           _vp]),
+    "kge_topk_prepared_bytes": (_sz, [_c_int, _c_i64, _c_i64]),
+    "kge_topk_prepare": (_c_int, [_vp, _c_int, _vp, _c_i64, _c_i64, _vp, _sz, _vp]),
+    "kge_topk_prepared_workspace_bytes": (_sz, [_c_i64, _c_i64, _c_i64]),
+    "kge_topk_prepared": (_c_int, [_vp, _vp, _vp, _c_int, _vp, _c_i64, _c_i64, _c_i64, _c_i64, _vp, _vp, _c_int, _vp,
+                                   _sz, _vp, _sz, _vp]),
     "kge_profile_begin": (_c_int, []),
     "kge_profile_end": (_c_int, [ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_int64)]),
     "kge_row_minmax": (_c_int, [_vp, _vp, _vp, _c_int, _vp, _c_i64, _c_i64, _c_i64, _vp, _vp, _vp]),

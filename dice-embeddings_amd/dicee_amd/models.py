@@ -58,6 +58,7 @@ class BaseKGE(torch.nn.Module):
         self._scale = None
         self._rel_table = None
         self._snap_key = None    # identity and version of the parameters the bf16 / int8 copies were taken from
+        self._topk_prepared = None   # (table data_ptr, derived form of the table that top-k scans), made on first use
 
     # ------------------------------------------------------------------ storage
     def set_entity_storage(self, kind="fp32"):
@@ -83,6 +84,7 @@ class BaseKGE(torch.nn.Module):
             raise ValueError(kind)
         self._storage = kind
         self._snap_key = self._parameter_key()
+        self._topk_prepared = None
         return self
 
     def _parameter_key(self):
@@ -212,7 +214,13 @@ class BaseKGE(torch.nn.Module):
     def topk(self, x, k, sigmoid=False, heads=False):
         Q, bias = self.query(x, heads=heads)
         E, scale = self.table()
-        return ops.topk(Q, bias, E, scale, k, sigmoid=sigmoid)
+        # the quantised table's derived form for the scan lives and dies with the quantised table itself
+        prepared = None
+        if self._table is not None and scale is not None:
+            if self._topk_prepared is None or self._topk_prepared[0] != E.data_ptr():
+                self._topk_prepared = (E.data_ptr(), ops.topk_prepare(E, scale))
+            prepared = self._topk_prepared[1]
+        return ops.topk(Q, bias, E, scale, k, sigmoid=sigmoid, prepared=prepared)
 
     def kvsall_bce_loss(self, x, csr, label_smoothing=0.0):
         """Forward + loss of training_step (base_model.py:25-46) for a KvsAll batch whose multi-hot

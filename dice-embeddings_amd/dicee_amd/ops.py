@@ -242,8 +242,26 @@ def rank_filtered(Q, bias, E, scale, target, csr_row=None, row_ptr=None, col=Non
     return out
 
 
-def topk(Q, bias, E, scale, k, sigmoid=False):
-    """Fused top-k over all entities: ([B,k] fp32 descending, [B,k] int64)."""
+def topk_prepare(E, scale):
+    """The derived form of a table that ``topk`` scans (made once per table and handed to every call as
+    ``prepared=``), or None where the storage has none (every storage but per-row int8 with d = 128)."""
+    lib = _lib.load()
+    _require_gpu(E, scale)
+    N, d = E.shape
+    nbytes = lib.kge_topk_prepared_bytes(_table_dtype(E), d, N)
+    if nbytes == 0:
+        return None
+    if not E.is_contiguous() or scale is None or not scale.is_contiguous():
+        raise ValueError("E and scale must be contiguous")
+    buf = torch.empty((nbytes,), dtype=torch.uint8, device=E.device)
+    rc = lib.kge_topk_prepare(_ptr(E), _table_dtype(E), _ptr(scale), d, N, _ptr(buf), nbytes, _stream())
+    _lib.check(rc)
+    return buf
+
+
+def topk(Q, bias, E, scale, k, sigmoid=False, prepared=None):
+    """Fused top-k over all entities: ([B,k] fp32 descending, [B,k] int64).  ``prepared``: what ``topk_prepare``
+    returned for this very table (same results, without deriving it again in every call)."""
     lib = _lib.load()
     _require_gpu(Q, bias, E, scale)
     _check_qe(Q, E, scale, bias)
@@ -252,10 +270,18 @@ def topk(Q, bias, E, scale, k, sigmoid=False):
     dev = Q.device
     out_s = torch.empty((B, k), dtype=torch.float32, device=dev)
     out_i = torch.empty((B, k), dtype=torch.int64, device=dev)
-    ws_bytes = lib.kge_topk_workspace_bytes(B, N, k)
-    ws = torch.empty((ws_bytes,), dtype=torch.uint8, device=dev)
-    rc = lib.kge_topk(_ptr(Q), _ptr(bias), _ptr(E), _table_dtype(E), _ptr(scale), B, d, N, int(k), _ptr(out_s),
-                      _ptr(out_i), int(bool(sigmoid)), _ptr(ws), ws_bytes, _stream())
+    if prepared is not None:
+        _require_gpu(prepared)
+        ws_bytes = lib.kge_topk_prepared_workspace_bytes(B, N, k)
+        ws = torch.empty((ws_bytes,), dtype=torch.uint8, device=dev)
+        rc = lib.kge_topk_prepared(_ptr(Q), _ptr(bias), _ptr(E), _table_dtype(E), _ptr(scale), B, d, N, int(k),
+                                   _ptr(out_s), _ptr(out_i), int(bool(sigmoid)), _ptr(prepared), prepared.numel(),
+                                   _ptr(ws), ws_bytes, _stream())
+    else:
+        ws_bytes = lib.kge_topk_workspace_bytes(B, N, k)
+        ws = torch.empty((ws_bytes,), dtype=torch.uint8, device=dev)
+        rc = lib.kge_topk(_ptr(Q), _ptr(bias), _ptr(E), _table_dtype(E), _ptr(scale), B, d, N, int(k), _ptr(out_s),
+                          _ptr(out_i), int(bool(sigmoid)), _ptr(ws), ws_bytes, _stream())
     _lib.check(rc)
     return out_s, out_i
 

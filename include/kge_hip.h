@@ -16,7 +16,7 @@
  *   - Tables are row-major [rows, d].  All three storages compute on the bf16 MFMA with fp32 accumulation:
  *     KGE_F32 splits every operand into three bf16 parts and sums the six leading part products (fp32-level
  *     accuracy, any d); KGE_BF16 needs d % 8 == 0; KGE_I8 (per-row symmetric int8 with a float scale per
- *     row) needs d % 16 == 0 and d <= 128.
+ *     row) needs d % 16 == 0.
  *   - A score is `dot(Q[b], E[e]) (* scale[e]) (+ bias[b])`.  The fp32 value of the dot product
  *     is the same bit pattern in every entry point (fixed reduction order), so a rank computed
  *     by kge_rank_filtered equals the rank counted on kge_scores output exactly.
@@ -254,6 +254,25 @@ size_t kge_topk_workspace_bytes(int64_t B, int64_t N, int64_t k);
 int kge_topk(const float* Q, const float* bias, const void* E, int dtype, const float* scale,
              int64_t B, int64_t d, int64_t N, int64_t k, float* out_scores, int64_t* out_idx,
              int apply_sigmoid, void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * The same top-k over a table whose derived form for the scan is made once and kept by the caller, the way the
+ * int8 table itself is made once from the model's parameters (dicee keeps its tables as nn.Embedding weights and has
+ * no quantised storage: there is no reference line for this; the results are those of kge_topk, bit for bit).
+ * Per-row int8 tables with d = 128 have such a form (the rows written again with one scale per 32-row tile plus a
+ * 32-byte record per 64 rows: kge_topk derives it in its workspace on every call, 2.6 GB of traffic at N = 10M);
+ * kge_topk_prepared_bytes returns 0 for every other storage and kge_topk_prepare / kge_topk_prepared then return
+ * KGE_ERR_UNSUPPORTED.  The prepared buffer must be rebuilt whenever E or scale change; it is only read by
+ * kge_topk_prepared, so calls on several streams may share it.
+ */
+size_t kge_topk_prepared_bytes(int dtype, int64_t d, int64_t N);
+int kge_topk_prepare(const void* E, int dtype, const float* scale, int64_t d, int64_t N, void* prepared,
+                     size_t prepared_bytes, void* stream);
+size_t kge_topk_prepared_workspace_bytes(int64_t B, int64_t N, int64_t k);
+int kge_topk_prepared(const float* Q, const float* bias, const void* E, int dtype, const float* scale,
+                      int64_t B, int64_t d, int64_t N, int64_t k, float* out_scores, int64_t* out_idx,
+                      int apply_sigmoid, const void* prepared, size_t prepared_bytes, void* workspace,
+                      size_t workspace_bytes, void* stream);
 
 /*
  * Smallest and largest score of every query over all N entities: out_min[b] = min_e S[b, e],

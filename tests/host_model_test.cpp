@@ -43,7 +43,8 @@ static void test_contract_rules() {
   CHECK(contract_rules("t", buf, buf, KGE_BF16, nullptr, 1, 136, 5).ok());
   CHECK(contract_rules("t", buf, buf, KGE_I8, buf, 1, 128, 5).ok());
   CHECK(contract_rules("t", buf, buf, KGE_I8, nullptr, 1, 128, 5).code == KGE_ERR_INVALID);
-  CHECK(contract_rules("t", buf, buf, KGE_I8, buf, 1, 144, 5).code == KGE_ERR_UNSUPPORTED);
+  CHECK(contract_rules("t", buf, buf, KGE_I8, buf, 1, 144, 5).ok());
+  CHECK(contract_rules("t", buf, buf, KGE_I8, buf, 1, 65552, 5).code == KGE_ERR_INVALID);
   CHECK(contract_rules("t", buf, buf, KGE_I8, buf, 1, 24, 5).code == KGE_ERR_INVALID);
   CHECK(contract_rules("t", buf, buf, 7, nullptr, 1, 8, 5).code == KGE_ERR_INVALID);
   const Status st = contract_rules("kge_scores", buf, buf, KGE_BF16, nullptr, 1, 12, 5);
@@ -83,8 +84,15 @@ static void test_layouts() {
         check_disjoint({{t.tau, (size_t)B * 4}, {t.tau_scan, (size_t)B * 4}, {t.cnt, (size_t)B * 4},
                         {t.list_len, (size_t)B * 4}, {t.dirty, (size_t)B * 4}, {t.n_dirty, 4},
                         {t.list, (size_t)B * t.kpad * 8}, {t.cand, (size_t)B * TOPK_CAP * 8},
-                        {t.cand_id, (size_t)B * TOPK_CAP * 4}, {t.rowmeta, n_rec * TOPK_ROWMETA_BYTES},
+                        {t.cand_id, (size_t)B * TOPK_CAP * 4}, {t.qh, (size_t)B * TOPK_REQUANT_D},
+                        {t.qc, (size_t)B * 16}, {t.rowmeta, n_rec * TOPK_ROWMETA_BYTES},
                         {t.requant, (size_t)N * TOPK_REQUANT_D}}, t.total);
+        // a call that is handed the prepared table keeps none in its workspace
+        const TopkWsOffsets u = topk_ws_offsets(B, N, k, false);
+        CHECK(u.total <= t.total && u.qc + (size_t)B * 16 <= u.total && u.qh == t.qh && u.cand_id == t.cand_id);
+        const TopkPreparedOffsets pr = topk_prepared_offsets(N);
+        check_disjoint({{pr.rowmeta, n_rec * TOPK_ROWMETA_BYTES}, {pr.requant, (size_t)N * TOPK_REQUANT_D}}, pr.total);
+        CHECK(t.total - u.total >= pr.total);
       }
     }
   }

@@ -4,6 +4,8 @@ Bars: fp32 scores within 1e-5 relative, bf16 / int8 within 2e-2 relative (relati
 max(|s|, row RMS)); ranks, tie counters and top-k indices bit-exact with respect to the scores the
 library itself materialises, and inside the oracle's tolerance interval.
 """
+import ctypes
+
 import numpy as np
 import pytest
 import torch
@@ -130,11 +132,13 @@ SCORE_CASES = [
     ("QMult", 999, 5, 128, 130, "bf16", {}),
     ("DistMult", 5000, 7, 128, 600, "bf16", {}),
     ("ComplEx", 321, 7, 64, 40, "bf16", {}),
-    ("Keci", 1500, 6, 256, 300, "bf16", {"p": 0, "q": 1, "coeff_q": [1.0]}),      # d > 128: kchunk_bf16_kernel
+    ("Keci", 1500, 6, 256, 300, "bf16", {"p": 0, "q": 1, "coeff_q": [1.0]}),      # d > 128: kchunk_kernel
     ("ComplEx", 700, 7, 200, 150, "bf16", {}),
     ("DistMult", 300, 5, 136, 70, "bf16", {}),
     ("DistMult", 777, 9, 128, 70, "int8", {}),
     ("ComplEx", 2100, 9, 96, 520, "int8", {}),
+    ("ComplEx", 1300, 7, 256, 300, "int8", {}),      # int8 wider than 128: kchunk_kernel, scales applied per tile
+    ("DistMult", 777, 5, 144, 131, "int8", {}),      # K tail (144 = 2 chunks of 64 + 16), partial query group
 ]
 
 
@@ -350,6 +354,7 @@ TOPK_CASES = [
     ("ComplEx", 20011, 11, 200, 130, "fp32", 100),
     ("QMult", 20011, 5, 128, 600, "bf16", 10),
     ("DistMult", 30000, 9, 128, 70, "int8", 100),
+    ("DistMult", 9000, 9, 192, 70, "int8", 50),      # int8 wider than 128
     ("DistMult", 5000, 9, 64, 33, "bf16", 1),
     ("DistMult", 6000, 9, 64, 20, "fp32", 1024),
     ("DistMult", 700, 9, 64, 20, "fp32", 600),       # k above half of the one-wave select's capacity
@@ -448,6 +453,12 @@ def test_topk_int8_filter_scan_edge_cases(ops, N, B, k):
     # (the zero query scores +0 or -0 everywhere: equal to numpy, ordered by sign in the library's keys)
     np.testing.assert_array_equal(idx.cpu().numpy()[1:], wi[1:])
     np.testing.assert_array_equal(vals.cpu().numpy(), wv)
+    # the table's derived form made once and handed in: the same bits, on two calls that share it
+    prep = ops.topk_prepare(Eg, scg)
+    assert prep is not None and prep.numel() >= N * d
+    for _ in range(2):
+        v2, i2 = ops.topk(Qg, None, Eg, scg, k, prepared=prep)
+        assert torch.equal(v2, vals) and torch.equal(i2, idx)
     # a table of non-negative rows and positive scales under the all-negative query
     Ep = np.abs(q8.astype(np.int16)).clip(0, 127).astype(np.int8)
     scp = np.abs(sc) + 1e-6
@@ -458,6 +469,34 @@ def test_topk_int8_filter_scan_edge_cases(ops, N, B, k):
     wv, wi = ko.topk(S, k)
     np.testing.assert_array_equal(idx.cpu().numpy(), wi)
     np.testing.assert_array_equal(vals.cpu().numpy(), wv)
+
+
+def test_topk_prepared_form_exists_for_int8_d128_only(ops):
+    from dicee_amd import _lib
+    lib = _lib.load()
+    assert lib.kge_topk_prepared_bytes(2, 128, 1000) >= 1000 * 128 + 16 * 32
+    assert lib.kge_topk_prepared_bytes(2, 64, 1000) == 0 and lib.kge_topk_prepared_bytes(1, 128, 1000) == 0
+    assert lib.kge_topk_prepared_bytes(0, 128, 1000) == 0
+    E = torch.zeros((1000, 64), dtype=torch.int8, device="cuda")
+    sc = torch.ones(1000, device="cuda")
+    assert ops.topk_prepare(E, sc) is None
+    assert ops.topk_prepare(torch.zeros((1000, 128), dtype=torch.bfloat16, device="cuda"), None) is None
+    p256 = ctypes.c_void_p(256)
+    assert lib.kge_topk_prepare(p256, 1, p256, 128, 1000, p256, 1 << 30, None) == 2        # bf16: no prepared form
+    assert lib.kge_topk_prepare(p256, 2, p256, 128, 1000, p256, 100, None) == 3            # buffer too small
+    assert b"need" in lib.kge_last_error()
+    assert lib.kge_topk_prepared(p256, None, p256, 2, p256, 4, 128, 1000, 5, p256, p256, 0, p256, 100, p256, 1 << 30,
+                                 None) == 3                                                  # prepared too small
+    assert lib.kge_topk_prepared(p256, None, p256, 2, p256, 4, 64, 1000, 5, p256, p256, 0, p256, 1 << 30, p256, 1 << 30,
+                                 None) == 2                                                  # d = 64: call kge_topk
+    # a small table (one round, no filter scan) accepts a prepared buffer and ignores it
+    E8 = torch.randint(-127, 128, (500, 128), dtype=torch.int8, device="cuda")
+    s8 = torch.full((500,), 0.02, device="cuda")
+    Q = torch.randn((7, 128), device="cuda")
+    prep = ops.topk_prepare(E8, s8)
+    v1, i1 = ops.topk(Q, None, E8, s8, 9)
+    v2, i2 = ops.topk(Q, None, E8, s8, 9, prepared=prep)
+    assert torch.equal(v1, v2) and torch.equal(i1, i2)
 
 
 def test_topk_int8_query_with_a_nan_yields_nothing(ops):
@@ -489,6 +528,7 @@ def test_topk_ties_prefer_lower_ids_and_k_equals_n(ops):
     ("Keci", 1000, 6, 35, 70, "fp32", {"p": 3, "q": 3, "coeff_p": [0.7, 1.1, -0.3], "coeff_q": [1.3, -0.4, 0.9]}),
     ("QMult", 3000, 5, 128, 530, "bf16", {}),
     ("DistMult", 2000, 5, 64, 100, "int8", {}),
+    ("DistMult", 1100, 5, 160, 100, "int8", {}),
 ])
 @pytest.mark.parametrize("eps", [0.0, 0.1])
 def test_bce_multihot_vs_oracle(ops, FilterCSR, model, N, R, d, B, storage, kw, eps):
@@ -567,8 +607,8 @@ def test_argument_validation(ops):
                         torch.zeros((1, 2), dtype=torch.int64, device="cuda"), p=1, q=1,
                         coeff_p=torch.ones(1, device="cuda"), coeff_q=torch.ones(1, device="cuda"))
     with pytest.raises(KgeError):
-        ops.scores(torch.zeros((4, 256), device="cuda"), None, torch.zeros((10, 256), device="cuda", dtype=torch.int8),
-                   torch.ones(10, device="cuda"))                               # int8 d > 128
+        ops.scores(torch.zeros((4, 136), device="cuda"), None, torch.zeros((10, 136), device="cuda", dtype=torch.int8),
+                   torch.ones(10, device="cuda"))                               # int8 with d % 16 != 0
     with pytest.raises(RuntimeError):
         ops.scores(torch.zeros((4, 24)), None, torch.zeros((10, 24)))            # CPU tensors
     # empty batch is a no-op

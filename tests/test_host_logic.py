@@ -49,9 +49,9 @@ def test_host_side_argument_validation_without_gpu(lib_path):
     rc = lib.kge_topk(ctypes.c_void_p(256), None, ctypes.c_void_p(256), 0, None, 4, 16, 100, 200, None, None, 0,
                       None, 0, None)
     assert rc == 1 and b"k=200" in lib.kge_last_error()
-    rc = lib.kge_scores(ctypes.c_void_p(256), None, ctypes.c_void_p(256), 2, ctypes.c_void_p(256), 4, 256, 100,
+    rc = lib.kge_scores(ctypes.c_void_p(256), None, ctypes.c_void_p(256), 2, ctypes.c_void_p(256), 4, 136, 100,
                         ctypes.c_void_p(256), 100, None)
-    assert rc == 2                                              # int8 with d > 128: unsupported
+    assert rc == 1 and b"16" in lib.kge_last_error()            # int8 rows need d % 16 == 0
     rc = lib.kge_build_query(3, 1, 1, ctypes.c_void_p(256), 0, None, ctypes.c_void_p(256), 0, None, None, 1, None,
                              ctypes.c_void_p(256), 1, 7, 10, 2, ctypes.c_void_p(256), ctypes.c_void_p(256), None)
     assert rc == 1 and b"Keci" in lib.kge_last_error()
