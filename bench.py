@@ -34,8 +34,8 @@ PEAK_TFLOPS = {"bf16": 2500.0, "fp32": 2500.0 / 6.0, "int8": 5000.0}
 FP32_MFMA_PEAK_TFLOPS = 157.3
 # HBM bytes per launch of the main loop measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on the full-size
 # workload (each scaled by what the same counter reads for a plain 1 GiB copy kernel: x2.00 and x1.00).
-MEASURED_TRAFFIC_BYTES = {"c4": 658.0e6,     # per rank launch
-                          "c5": 323.0e6,     # average over the 8 launches of a top-k call (2.59 GB per call)
+MEASURED_TRAFFIC_BYTES = {"c4": 688.0e6,     # per rank launch (678 MB read, 9 MB written)
+                          "c5": 218.0e6,     # average over the 7 filter launches of a top-k call (6.5 GB per call over all kernels)
                           "c3": 59.4e6, "c2": 19.4e6}
 MODE = {"c1": "rank", "c2": "rank", "c3": "bce", "c4": "rank", "c5": "topk"}
 
@@ -294,7 +294,7 @@ def main():
     # side figures, outside the timed region: what the vendor's bf16 GEMM (torch.matmul -> hipBLASLt) sustains on this
     # box, on random and on all-zero operands (the gap is the power limit: random data toggles more), and at the
     # workload's own shape, where it has to write the B x N score matrix that the fused kernels never form
-    if not args.no_ceiling and compute == "bf16" and args.scale == 1.0:
+    if not args.no_ceiling and compute in ("bf16", "int8") and args.scale == 1.0:
         def gemm_rate(a_, b_, out_, seconds=0.7):
             for _ in range(3):
                 torch.matmul(a_, b_, out=out_)
@@ -327,6 +327,27 @@ def main():
         r, ms = gemm_rate(A, Bm, C)
         ceil["torch_matmul_bf16_8192_cubed_zeros"] = {"achieved": r, "frac": r / PEAK_TFLOPS["bf16"], "ms": ms}
         del A, Bm, C
+        if compute == "int8":
+            # the vendor's int8 GEMM on random int8 operands (int8 x int8 -> int32), against the int8 MFMA peak
+            try:
+                Ai = torch.randint(-127, 128, (n_sq, n_sq), device=dev, dtype=torch.int8, generator=g)
+                Bi = torch.randint(-127, 128, (n_sq, n_sq), device=dev, dtype=torch.int8, generator=g)
+                for _ in range(3):
+                    torch._int_mm(Ai, Bi)
+                torch.cuda.synchronize()
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+                for _ in range(20):
+                    torch._int_mm(Ai, Bi)
+                e1.record()
+                torch.cuda.synchronize()
+                ms = e0.elapsed_time(e1) / 20
+                r = 2.0 * n_sq ** 3 / (ms * 1e-3) / 1e12
+                ceil["torch_int_mm_int8_8192_cubed_randint"] = {"achieved": r, "frac": r / PEAK_TFLOPS["int8"], "ms": ms,
+                                                                "peak": PEAK_TFLOPS["int8"]}
+                del Ai, Bi
+            except Exception as exc:                                    # noqa: BLE001 (a side figure: report, go on)
+                ceil["torch_int_mm_int8_8192_cubed_randint"] = {"error": f"{type(exc).__name__}: {exc}"[:200]}
         if d == 128:
             E_t, _ = model.table()
             if E_t.dtype == torch.bfloat16:

@@ -14,9 +14,13 @@
  *   - Entity/relation ids are int64 (what torch.LongTensor holds).  Kernels never dereference an
  *     id outside [0,N) / [0,R): such a row yields NaN scores instead of a memory fault.
  *   - Tables are row-major [rows, d].  All three storages compute on the bf16 MFMA with fp32 accumulation:
- *     KGE_F32 splits every operand into three bf16 parts and sums the six leading part products (fp32-level
- *     accuracy, any d); KGE_BF16 needs d % 8 == 0; KGE_I8 (per-row symmetric int8 with a float scale per
- *     row) needs d % 16 == 0.
+ *     KGE_F32 splits every operand into three bf16 parts and sums the six leading part products (any d);
+ *     KGE_BF16 needs d % 8 == 0; KGE_I8 (per-row symmetric int8 with a float scale per row) needs d % 16 == 0.
+ *     Range of the KGE_F32 split: scores are within 1e-5 of an fp64 product (relative to max(|s|, row RMS)) while
+ *     the products q*e that make up a score are at least 2^-100 in magnitude and every value rounds to a finite
+ *     bf16 (|x| < 3.39e38).  Below that the low-order parts underflow one after the other and the result
+ *     degrades towards a bf16-grade score (2e-2); products that underflow fp32 altogether give exact zeros.  A
+ *     value whose bf16 rounding is infinite gives an infinite or NaN score.
  *   - A score is `dot(Q[b], E[e]) (* scale[e]) (+ bias[b])`.  The fp32 value of the dot product
  *     is the same bit pattern in every entry point (fixed reduction order), so a rank computed
  *     by kge_rank_filtered equals the rank counted on kge_scores output exactly.
