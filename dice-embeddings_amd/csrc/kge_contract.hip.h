@@ -385,13 +385,19 @@ struct TopkArgs {
   unsigned long long* cand;  // [B, cap] packed (ordered score << 32 | 0xffffffff - entity)
   int32_t cap;
 };
+// Repair scans: a candidate is what ranks above the packed key of the query's k-th best (0: none yet), i.e. a higher
+// score or an equal score at a lower entity id.  (Its own epilogue type, so that the scans of the ordinary rounds
+// carry nothing of it.)
+struct TopkKeyArgs : TopkArgs {
+  const unsigned long long* kth;
+};
 constexpr int TOPK_LQ = 512;   // candidates a workgroup parks in LDS between flushes
-template <int NQT>
-struct TopkEpi {
+template <int NQT, bool BYKEY>
+struct TopkEpiT {
   static constexpr bool SWAP = false;
   static constexpr bool STAGE_HOOK = true;
   static constexpr bool DEFER = false;
-  using Args = TopkArgs;
+  using Args = typename std::conditional<BYKEY, TopkKeyArgs, TopkArgs>::type;
   // Candidates are parked in LDS (cheap atomics) and moved to the per-query global buffers in bulk
   // at stage boundaries, so the hot loop never waits for a global atomic's round trip.
   struct Shared {
@@ -412,7 +418,15 @@ struct TopkEpi {
     for (int t = 0; t < NQT; ++t) {
       const int64_t q = q0 + 32 * t + c;
       const bool on = q < B && (a.active == nullptr || a.active[q] != 0);
-      tau[t] = on ? a.tau[q] : __uint_as_float(0x7f800000u);  // +inf: nothing qualifies
+      float th = on ? a.tau[q] : __uint_as_float(0x7f800000u);  // +inf: nothing qualifies
+      if constexpr (BYKEY) {
+        if (on && th > __uint_as_float(0xff800000u)) {
+          // ties with the k-th best must reach collect(): the hot path tests against one step below its score
+          const uint32_t o = f32_to_ordered(th);
+          th = ordered_to_f32(o - 1);
+        }
+      }
+      tau[t] = th;
     }
   }
   __device__ void bind(Shared* s) {
@@ -443,13 +457,21 @@ struct TopkEpi {
   // the hot loop's register budget.
   static __device__ __attribute__((noinline)) void collect(f32x16 s, float th, int64_t q, int64_t e_base, int64_t limit,
                                                            int hf, Shared* sh, int32_t* cnt, unsigned long long* cand,
-                                                           int32_t cap) {
+                                                           int32_t cap, const unsigned long long* kth) {
+    unsigned long long kk = 0ull;
+    if constexpr (BYKEY) {
+      bool any = false;  // (a lane past the batch's end has th = +inf: it must not read kth[q])
+#pragma unroll
+      for (int i = 0; i < 16; ++i) any = any || s[i] > th;
+      if (any) kk = kth[q];
+    }
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
       const int64_t e = e_base + row_of(i, hf);
-      if (s[i] > th && e < limit) {
-        const unsigned long long key =
-            ((unsigned long long)f32_to_ordered(s[i]) << 32) | (unsigned long long)(0xffffffffu - (uint32_t)e);
+      const unsigned long long key =
+          ((unsigned long long)f32_to_ordered(s[i]) << 32) | (unsigned long long)(0xffffffffu - (uint32_t)e);
+      const bool admit = BYKEY ? (s[i] > th && key > kk) : (s[i] > th);
+      if (admit && e < limit) {
         const int idx = atomicAdd(&sh->n, 1);
         if (idx < TOPK_LQ) {
           sh->q[idx] = (int)q;
@@ -474,7 +496,11 @@ struct TopkEpi {
     }
     const unsigned long long hit = __builtin_amdgcn_ballot_w64(mx > th);
     if (__builtin_expect(hit != 0, 0))
-      collect(s, th, q0 + 32 * qt + c, e_base, limit, hf, sh, a.cnt, a.cand, a.cap);
+      collect(s, th, q0 + 32 * qt + c, e_base, limit, hf, sh, a.cnt, a.cand, a.cap, key_ptr());
+  }
+  __device__ __forceinline__ const unsigned long long* key_ptr() const {
+    if constexpr (BYKEY) return a.kth;
+    else return nullptr;
   }
   // Empties the LDS queue.  Every wave of the workgroup is inside (nobody appends meanwhile).
   __device__ void flush() {
@@ -502,6 +528,11 @@ struct TopkEpi {
     flush();
   }
 };
+
+template <int NQT>
+using TopkEpi = TopkEpiT<NQT, false>;
+template <int NQT>
+using TopkKeyEpi = TopkEpiT<NQT, true>;
 
 using host::BCE_SLOTS;  // the accumulator is spread: same-address double atomics serialise
 struct BceArgs {

@@ -112,7 +112,7 @@ inline RankWsOffsets rank_ws_offsets(int64_t B) {
   return o;
 }
 
-// tau: k-th best score per query; tau_scan: the threshold the next scan admits candidates with (tau, or a tighter
+// tau: k-th best score per query (kth: the k-th best as a packed key, 0 while fewer than k are known); tau_scan: the threshold the next scan admits candidates with (tau, or a tighter
 // guess that the selection verifies); list: the best k so far as packed keys; cand: this round's candidates as packed
 // keys; cand_id: this round's candidates as entity ids (int8 filter scan, scored exactly before they are ranked);
 // requant: the int8 table written again with one scale per 32-row tile, N x 128 bytes, and rowmeta: one
@@ -123,7 +123,7 @@ constexpr int TOPK_REQUANT_D = 128;
 // qh / qc: the queries as the int8 filter scan reads them (TOPK_REQUANT_D int8 per query, and per query the four
 // constants of its bound), written once per call.
 struct TopkWsOffsets {
-  size_t tau, tau_scan, cnt, list_len, dirty, n_dirty, list, cand, cand_id, qh, qc, rowmeta, requant, total;
+  size_t tau, tau_scan, cnt, list_len, dirty, n_dirty, kth, list, cand, cand_id, qh, qc, rowmeta, requant, total;
   int64_t kpad;
 };
 // the prepared form of an int8 table (what kge_topk_prepare writes): rowmeta records, then the requantised rows
@@ -153,6 +153,7 @@ inline TopkWsOffsets topk_ws_offsets(int64_t B, int64_t N, int64_t k, bool with_
   o.list_len = take((size_t)B * 4);
   o.dirty = take((size_t)B * 4);
   o.n_dirty = take(4);
+  o.kth = take((size_t)B * 8);
   o.list = take((size_t)B * (size_t)o.kpad * 8);
   o.cand = take((size_t)B * TOPK_CAP * 8);
   o.cand_id = take((size_t)B * TOPK_CAP * 4);
@@ -189,6 +190,13 @@ inline int64_t topk_speculative_rank(int64_t k, int64_t ranked, int64_t n_next) 
   if (j < 1) j = 1;
   return j < k ? j : k;
 }
+
+// how many times the ranked prefix grows per round of kge_topk.  Larger factors were measured and are no faster,
+// with or without the guessed thresholds: every round costs a launch of the persistent scan, a selection and the gaps
+// between them, but a scan with a looser threshold spends more time in its slow paths and hands more candidates to
+// the selection (k = 100, N = 10M through the int8 filter: x4 11.9 ms, x8 12.1, x16 12.7 per call; k = 10, N = 2.5M,
+// bf16: x4 3.00 ms, x8 3.04, x16 3.03).
+inline int64_t topk_growth(int64_t k) { return k <= 256 ? 4 : 2; }
 
 inline size_t bce_ws_bytes() { return (2 * BCE_SLOTS + 1) * sizeof(double) + 248; }
 

@@ -614,6 +614,7 @@ struct TopkWs {
   int32_t* list_len;
   int32_t* dirty;
   int32_t* n_dirty;
+  unsigned long long* kth;   // per query: its k-th best as a packed key (0 while fewer than k are known)
   unsigned long long* list;  // [B, kpad]
   unsigned long long* cand;  // [B, TOPK_CAP] packed keys
   uint32_t* cand_id;         // [B, TOPK_CAP] entity ids (int8 filter scan; scored into `cand` before they are ranked)
@@ -636,6 +637,7 @@ size_t topk_ws_layout(int64_t B, int64_t N, int64_t k, void* base, TopkWs* ws, c
     ws->list_len = (int32_t*)(p + o.list_len);
     ws->dirty = (int32_t*)(p + o.dirty);
     ws->n_dirty = (int32_t*)(p + o.n_dirty);
+    ws->kth = (unsigned long long*)(p + o.kth);
     ws->list = (unsigned long long*)(p + o.list);
     ws->cand = (unsigned long long*)(p + o.cand);
     ws->cand_id = (uint32_t*)(p + o.cand_id);
@@ -662,13 +664,14 @@ __global__ void topk_init_kernel(TopkWs w, int64_t B) {
     w.cnt[b] = 0;
     w.list_len[b] = 0;
     w.dirty[b] = 0;
+    w.kth[b] = 0;
   }
   if (b == 0) *w.n_dirty = 0;
 }
 
 // Merge a query's kept list with this round's candidates, keep the best k, publish the new
-// threshold.  In `rescan` mode (only queries flagged dirty) list entries above the old threshold
-// are dropped first: the rescan finds all of them again.
+// threshold.  In `rescan` mode (only queries flagged dirty) the list entries that rank above the old k-th best (by
+// key: a higher score, or the same score and a lower entity id) are dropped first: the rescan finds all of them again.
 // Bitonic sort, descending, of 64 * KPL keys held by one wave: element i = lane * KPL + s sits in
 // v[s] of `lane`.  Exchanges at distance < KPL stay inside a lane's registers; larger distances are
 // a lane shuffle.  No LDS, no barriers.
@@ -719,12 +722,14 @@ constexpr int SELECT_SMALL = 1024;
 // merged k-th best was then admitted.  Otherwise the query is flagged and scanned again at the end with its k-th best.
 // `spec_key`: the key at rank j_spec - 1 of the merged list (0: none): the next scan's guess is just below its score.
 __device__ __forceinline__ void select_finish(const TopkWs& w, int64_t b, int k, int rescan, bool over, int new_len,
-                                              bool have_tau, float tau, float tau_old, float th_used,
+                                              bool have_tau, unsigned long long kth_key, float tau_old, float th_used,
                                               unsigned long long spec_key) {
   const float NINF = __uint_as_float(0xff800000u);
   w.list_len[b] = new_len;
+  const float tau = ordered_to_f32((uint32_t)(kth_key >> 32));
   const float tau_new = have_tau ? tau : NINF;
   w.tau[b] = tau_new;
+  w.kth[b] = have_tau ? kth_key : 0ull;
   float guess = tau_new;
   if (have_tau && spec_key != 0) {
     // one step below the score at that rank, so that its ties are admitted too
@@ -783,6 +788,7 @@ __global__ void __launch_bounds__(256) topk_rescore_kernel(TopkWs w, ContractArg
 template <int KPL>
 __device__ __forceinline__ void select_in_registers(const TopkWs& w, int64_t b, int k, int rescan, int len, int nc,
                                                     float tau_old, float th_used, int j_spec, int lane) {
+  const unsigned long long kth_old = w.kth[b];  // (every lane reads it before lane 0 publishes the new one below)
   unsigned long long v[KPL];
 #pragma unroll
   for (int s = 0; s < KPL; ++s) {
@@ -790,7 +796,7 @@ __device__ __forceinline__ void select_in_registers(const TopkWs& w, int64_t b, 
     unsigned long long key = 0;
     if (i < len) {
       key = w.list[b * w.kpad + i];
-      if (rescan && ordered_to_f32((uint32_t)(key >> 32)) > tau_old) key = 0;
+      if (rescan && key > kth_old) key = 0;
     } else if (i < len + nc) {
       key = w.cand[b * TOPK_CAP + (i - len)];
     }
@@ -817,8 +823,7 @@ __device__ __forceinline__ void select_in_registers(const TopkWs& w, int64_t b, 
     spec |= __shfl_xor(spec, o, 64);
   }
   if (lane == 0)
-    select_finish(w, b, k, rescan, false, new_len, new_len == k, ordered_to_f32((uint32_t)(kth >> 32)), tau_old, th_used,
-                  spec);
+    select_finish(w, b, k, rescan, false, new_len, new_len == k, kth, tau_old, th_used, spec);
 }
 
 // Merge a query's kept list with this round's candidates, keep the best k, publish the new
@@ -850,6 +855,7 @@ __global__ void __launch_bounds__(256) topk_select_kernel(TopkWs w, int k, int r
   const int nc = raw < TOPK_CAP ? raw : TOPK_CAP;
   const bool over = raw > TOPK_CAP;
   const float tau_old = w.tau[b];
+  const unsigned long long kth_old = w.kth[b];
   const float th_used = rescan ? tau_old : w.tau_scan[b];
   const int n = len + nc;
   if (n <= SELECT_SMALL) return;  // ranked by topk_select_wave_kernel (which reset the candidate count)
@@ -860,7 +866,7 @@ __global__ void __launch_bounds__(256) topk_select_kernel(TopkWs w, int k, int r
     unsigned long long key = 0;
     if (i < len) {
       key = w.list[b * w.kpad + i];
-      if (rescan && ordered_to_f32((uint32_t)(key >> 32)) > tau_old) key = 0;
+      if (rescan && key > kth_old) key = 0;
     } else if (i < n) {
       key = w.cand[b * TOPK_CAP + (i - len)];
     }
@@ -890,8 +896,8 @@ __global__ void __launch_bounds__(256) topk_select_kernel(TopkWs w, int k, int r
   const int new_len = n_valid < k ? n_valid : k;
   for (int i = tid; i < new_len; i += 256) w.list[b * w.kpad + i] = keys[i];
   if (tid == 0)
-    select_finish(w, b, k, rescan, over, new_len, new_len == k, ordered_to_f32((uint32_t)(keys[k - 1] >> 32)), tau_old,
-                  th_used, (j_spec >= 1 && j_spec <= new_len) ? keys[j_spec - 1] : 0ull);
+    select_finish(w, b, k, rescan, over, new_len, new_len == k, keys[k - 1], tau_old, th_used,
+                  (j_spec >= 1 && j_spec <= new_len) ? keys[j_spec - 1] : 0ull);
 }
 
 __global__ void topk_output_kernel(TopkWs w, int64_t B, int k, const float* bias, int apply_sigmoid,
@@ -1628,6 +1634,13 @@ int topk_impl(const char* who, const float* Q, const float* bias, const void* E,
     // (the repair scan is exact as well: a query the bound cannot separate from most of the table, its threshold
     // tiny against the scales around it, would overflow its buffer again)
     if (!id_filter || rescan || e0 % host::TOPK_ROWMETA_ROWS != 0 || (e0 == 0 && e1 <= TOPK_FIRST_ROWS)) {
+      if (rescan) {
+        // a repair scan admits what ranks above the query's k-th best by KEY, so that ties with it at lower entity
+        // ids, which an overflowing buffer may have dropped, are found again
+        TopkKeyArgs ek;
+        ek.tau = tau; ek.active = active; ek.cnt = ws.cnt; ek.cand = ws.cand; ek.cap = TOPK_CAP; ek.kth = ws.kth;
+        return launch_contract<TopkKeyEpi>(dtype, a, ek, st, name);
+      }
       TopkArgs ea{tau, active, ws.cnt, ws.cand, TOPK_CAP};
       return launch_contract<TopkEpi>(dtype, a, ea, st, name);
     }
@@ -1662,7 +1675,8 @@ int topk_impl(const char* who, const float* Q, const float* bias, const void* E,
       hipLaunchKernelGGL(topk_select_kernel, dim3((unsigned)B), dim3(256), 8192 * sizeof(unsigned long long), st, ws,
                          (int)k, rescan, (int)j_spec);
   };
-  const int64_t growth = (k <= 256) ? 4 : 2;  // round r scans (growth - 1) x what is already ranked
+  // round r scans (growth - 1) x what is already ranked
+  const int64_t growth = host::topk_growth(k);
   int64_t e0 = 0, e1 = (N < TOPK_FIRST_ROWS) ? N : TOPK_FIRST_ROWS;
   while (e0 < N) {
     rc = launch_scan(e0, e1, ws.tau_scan, nullptr, 0, "kge_topk scan");

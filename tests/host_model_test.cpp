@@ -82,7 +82,7 @@ static void test_layouts() {
         const size_t n_rec = (size_t)((N + TOPK_ROWMETA_ROWS - 1) / TOPK_ROWMETA_ROWS);
         CHECK((int64_t)n_rec * TOPK_ROWMETA_ROWS >= N);
         check_disjoint({{t.tau, (size_t)B * 4}, {t.tau_scan, (size_t)B * 4}, {t.cnt, (size_t)B * 4},
-                        {t.list_len, (size_t)B * 4}, {t.dirty, (size_t)B * 4}, {t.n_dirty, 4},
+                        {t.list_len, (size_t)B * 4}, {t.dirty, (size_t)B * 4}, {t.n_dirty, 4}, {t.kth, (size_t)B * 8},
                         {t.list, (size_t)B * t.kpad * 8}, {t.cand, (size_t)B * TOPK_CAP * 8},
                         {t.cand_id, (size_t)B * TOPK_CAP * 4}, {t.qh, (size_t)B * TOPK_REQUANT_D},
                         {t.qc, (size_t)B * 16}, {t.rowmeta, n_rec * TOPK_ROWMETA_BYTES},

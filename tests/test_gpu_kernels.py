@@ -523,6 +523,39 @@ def test_topk_ties_prefer_lower_ids_and_k_equals_n(ops):
     np.testing.assert_array_equal(idx.cpu().numpy(), np.tile(np.arange(N), (B, 1)))
 
 
+@pytest.mark.parametrize("storage", ["fp32", "bf16", "int8"])
+@pytest.mark.parametrize("k", [1, 3, 100])
+def test_topk_many_ties_at_the_top_survive_an_overflowing_round(ops, storage, k):
+    """Thousands of entities share the best score, and all of them fall into one round, whose candidate buffer
+    (4096 slots) overflows and keeps a random sample.  The repair scan must bring back the ties with the LOWEST ids,
+    which no score threshold can tell from the others: it admits by key (score, then entity id)."""
+    rng = np.random.default_rng(77 + k)
+    N, d, B = 60000, 128, 6
+    q = np.zeros((B, d), dtype=np.float32)
+    q[:, :8] = 1.0
+    lo = rng.integers(-40, 0, (N, d)).astype(np.int8)              # every ordinary row scores below zero
+    tied = np.sort(rng.choice(np.arange(1100, 16000), 9000, replace=False))
+    best = np.zeros(d, dtype=np.int8)
+    best[:8] = 90
+    lo[tied] = best                                                  # 9000 identical rows: one exact score
+    if storage == "int8":
+        E = dev(torch.from_numpy(lo))
+        sc = dev(torch.full((N,), 0.01))
+    else:
+        E = dev(torch.from_numpy(lo.astype(np.float32) * 0.01))
+        sc = None
+        if storage == "bf16":
+            E = E.to(torch.bfloat16)
+    Qg = dev(torch.from_numpy(q))
+    vals, idx = ops.topk(Qg, None, E, sc, k)
+    S = ops.scores(Qg, None, E, sc).cpu().numpy()
+    assert (S[:, tied] == S[0, tied[0]]).all() and S[0, tied[0]] == S.max()
+    wv, wi = ko.topk(S, k)
+    np.testing.assert_array_equal(idx.cpu().numpy(), wi)
+    np.testing.assert_array_equal(vals.cpu().numpy(), wv)
+    np.testing.assert_array_equal(idx.cpu().numpy()[0], tied[:k])
+
+
 @pytest.mark.parametrize("model,N,R,d,B,storage,kw", [
     ("Keci", 4099, 18, 256, 300, "fp32", {"p": 0, "q": 1, "coeff_q": [1.0]}),
     ("Keci", 1000, 6, 35, 70, "fp32", {"p": 3, "q": 3, "coeff_p": [0.7, 1.1, -0.3], "coeff_q": [1.3, -0.4, 0.9]}),
