@@ -39,6 +39,12 @@ def evaluate_lp(model, triple_idx, num_entities=None, er_vocab=None, re_vocab=No
     assert er_vocab is not None, "er_vocab must be provided"
     assert re_vocab is not None, "re_vocab must be provided"
     model.eval()
+    from .models import IdentityClass
+    if not isinstance(getattr(model, "normalize_tail_entity_embeddings", IdentityClass()), IdentityClass):
+        # the reference scores every candidate through forward_triples here, i.e. against NORMALISED tail rows
+        # (base_model.py:374); ranking against the table as it is would silently give other ranks
+        raise NotImplementedError("evaluate_lp: models that normalise the tail row (normalization with NegSample / "
+                                  "KvsSample) are not part of this path; forward_triples scores them")
     N, R = model.num_entities, model.num_relations
     assert num_entities is None or num_entities == N, "num_entities does not match the model"
     triple_idx = np.asarray(triple_idx)

@@ -41,14 +41,22 @@ class BaseKGE(torch.nn.Module):
         self.loss = torch.nn.BCEWithLogitsLoss()
         self.normalize_head_entity_embeddings = IdentityClass()
         self.normalize_relation_embeddings = IdentityClass()
+        self.normalize_tail_entity_embeddings = IdentityClass()
         self.hidden_normalizer = IdentityClass()
         norm = args.get("normalization")
+        # a model trained on single triples also normalises the tail row (base_model.py:287-294); KvsAll scoring
+        # never does (the table is used as it is), only forward_triples
+        tail_too = args.get("scoring_technique") in ("NegSample", "KvsSample")
         if norm == "LayerNorm":
             self.normalize_head_entity_embeddings = torch.nn.LayerNorm(self.embedding_dim)
             self.normalize_relation_embeddings = torch.nn.LayerNorm(self.embedding_dim)
+            if tail_too:
+                self.normalize_tail_entity_embeddings = torch.nn.LayerNorm(self.embedding_dim)
         elif norm == "BatchNorm1d":
             self.normalize_head_entity_embeddings = torch.nn.BatchNorm1d(self.embedding_dim, affine=False)
             self.normalize_relation_embeddings = torch.nn.BatchNorm1d(self.embedding_dim, affine=False)
+            if tail_too:
+                self.normalize_tail_entity_embeddings = torch.nn.BatchNorm1d(self.embedding_dim, affine=False)
         elif norm is not None:
             raise NotImplementedError(norm)
         self.entity_embeddings = torch.nn.Embedding(self.num_entities, self.embedding_dim)
@@ -175,7 +183,20 @@ class BaseKGE(torch.nn.Module):
         E, scale = self.table()
         x = x.to(device=E.device, dtype=torch.int64)
         Q, bias = self.query(x[:, :2].contiguous())
-        return ops.triple_scores(Q, bias, E, scale, x[:, 2].contiguous())
+        nt = self.normalize_tail_entity_embeddings
+        if isinstance(nt, IdentityClass):
+            return ops.triple_scores(Q, bias, E, scale, x[:, 2].contiguous())
+        # normalised tails (base_model.py:374) are not rows of the table: the reference's own normaliser module, with
+        # eval semantics, makes the n rows, and triple i is scored against row i of that small table
+        if self.training:
+            raise NotImplementedError("tail normalisation in training mode (batch statistics) is not part of this path")
+        w = self.entity_embeddings.weight.detach()
+        idx = x[:, 2].contiguous()
+        if (idx < 0).any() or (idx >= self.num_entities).any():
+            raise IndexError("index out of range in self")
+        with torch.no_grad():
+            tails = nt(w[idx]).contiguous().float()
+        return ops.triple_scores(Q, bias, tails, None, torch.arange(idx.numel(), device=E.device, dtype=torch.int64))
 
     def forward_all_heads(self, rt):
         """[B,N] fp32: score(x, r, t) of every entity x as head, for ``rt`` [B,2] = (relation, tail) pairs."""

@@ -457,6 +457,49 @@ def test_forward_triples_and_triple_score(name, d, extra):
         kge.triple_score("nobody", "r0", "e1")
 
 
+@pytest.mark.parametrize("kind", ["LayerNorm", "BatchNorm1d"])
+def test_forward_triples_normalises_the_tail_of_a_model_trained_on_single_triples(kind):
+    """normalization + NegSample / KvsSample: the reference also normalises the tail row (base_model.py:287-294,
+    :374); the module exists (so a stored state_dict loads strictly) and forward_triples applies it."""
+    from dicee_amd import evaluate_lp
+    d = 32
+    m, triples = _toy("DistMult", d, n=300, seed=41, normalization=kind, scoring_technique="NegSample")
+    assert any(k.startswith("normalize_tail_entity_embeddings.") for k in m.state_dict())
+    rng = np.random.default_rng(3)
+    with torch.no_grad():
+        for mod in (m.normalize_head_entity_embeddings, m.normalize_relation_embeddings, m.normalize_tail_entity_embeddings):
+            if kind == "LayerNorm":
+                mod.weight.copy_(torch.from_numpy(rng.normal(1.0, 0.2, d).astype(np.float32)))
+                mod.bias.copy_(torch.from_numpy(rng.normal(0.0, 0.1, d).astype(np.float32)))
+            else:
+                mod.running_mean.copy_(torch.from_numpy(rng.normal(0.0, 0.05, d).astype(np.float32)))
+                mod.running_var.copy_(torch.from_numpy(rng.uniform(0.5, 1.5, d).astype(np.float32)))
+    E = m.entity_embeddings.weight.detach().numpy().astype(np.float64)
+    Rel = m.relation_embeddings.weight.detach().numpy().astype(np.float64)
+
+    def normed(mod, x):
+        if kind == "LayerNorm":
+            return ko.layer_norm(x, mod.weight.detach().numpy(), mod.bias.detach().numpy(), mod.eps)
+        return ko.batch_norm_eval(x, mod.running_mean.numpy(), mod.running_var.numpy(), mod.eps)
+    h = normed(m.normalize_head_entity_embeddings, E[triples[:, 0]])
+    r = normed(m.normalize_relation_embeddings, Rel[triples[:, 1]])
+    t = normed(m.normalize_tail_entity_embeddings, E[triples[:, 2]])
+    ref = (h * r * t).sum(axis=1)
+    m = m.to("cuda").eval()
+    with torch.no_grad():
+        s = m(torch.from_numpy(triples).cuda())
+    assert s.shape == (300,)
+    assert np.abs(s.cpu().numpy() - ref).max() <= 1e-5 * np.sqrt((ref ** 2).mean()) + 1e-6
+    # a model without the tail normaliser (KvsAll-trained) keeps scoring against the table as it is
+    m2, _ = _toy("DistMult", d, n=10, seed=41, normalization=kind, scoring_technique="KvsAll")
+    assert not any(k.startswith("normalize_tail_entity_embeddings.") for k in m2.state_dict())
+    # ranking against the un-normalised table would be silently wrong for such a model: refused
+    with pytest.raises(NotImplementedError):
+        evaluate_lp(m, triples, er_vocab={}, re_vocab={}, info=None)
+    with pytest.raises(IndexError):
+        m(torch.tensor([[0, 0, 135]]).cuda())
+
+
 def test_string_triple_evaluators():
     from dicee_amd import (KGE, evaluate_lp, evaluate_link_prediction_performance,
                            evaluate_link_prediction_performance_with_reciprocals)
