@@ -420,11 +420,8 @@ struct TopkEpiT {
       const bool on = q < B && (a.active == nullptr || a.active[q] != 0);
       float th = on ? a.tau[q] : __uint_as_float(0x7f800000u);  // +inf: nothing qualifies
       if constexpr (BYKEY) {
-        if (on && th > __uint_as_float(0xff800000u)) {
-          // ties with the k-th best must reach collect(): the hot path tests against one step below its score
-          const uint32_t o = f32_to_ordered(th);
-          th = ordered_to_f32(o - 1);
-        }
+        // ties with the k-th best must reach collect(): the hot path tests against a threshold they beat
+        if (on) th = just_below(th);
       }
       tau[t] = th;
     }

@@ -55,4 +55,14 @@ __device__ __forceinline__ float ordered_to_f32(uint32_t k) {
   return __uint_as_float(u);
 }
 
+// A threshold that every score equal to x beats in a float comparison (`s > just_below(x)` holds for s == x), as
+// close below x as that allows.  One step down in the ordered encoding does it except around zero: the neighbour of
+// +0 there is -0, which compares EQUAL to it, and the denormals next to them depend on the comparison honouring
+// denormals; so for |x| below the smallest normal the answer is minus the smallest normal.  (-inf stays -inf.)
+__device__ __forceinline__ float just_below(float x) {
+  if (!(x > __uint_as_float(0xff800000u))) return x;                        // -inf, NaN
+  if (__builtin_fabsf(x) < 1.17549435e-38f) return -1.17549435e-38f;
+  return ordered_to_f32(f32_to_ordered(x) - 1u);
+}
+
 }  // namespace kge

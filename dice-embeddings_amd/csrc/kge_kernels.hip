@@ -732,9 +732,8 @@ __device__ __forceinline__ void select_finish(const TopkWs& w, int64_t b, int k,
   w.kth[b] = have_tau ? kth_key : 0ull;
   float guess = tau_new;
   if (have_tau && spec_key != 0) {
-    // one step below the score at that rank, so that its ties are admitted too
-    const uint32_t o = (uint32_t)(spec_key >> 32);
-    const float below = (o > 0) ? ordered_to_f32(o - 1) : NINF;
+    // just below the score at that rank, so that its ties are admitted too
+    const float below = just_below(ordered_to_f32((uint32_t)(spec_key >> 32)));
     if (below > guess) guess = below;  // never below the k-th best; NaN leaves it
   }
   w.tau_scan[b] = rescan ? tau_new : guess;

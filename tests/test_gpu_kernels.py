@@ -525,10 +525,12 @@ def test_topk_ties_prefer_lower_ids_and_k_equals_n(ops):
 
 @pytest.mark.parametrize("storage", ["fp32", "bf16", "int8"])
 @pytest.mark.parametrize("k", [1, 3, 100])
-def test_topk_many_ties_at_the_top_survive_an_overflowing_round(ops, storage, k):
+@pytest.mark.parametrize("best_value", [90, 0])
+def test_topk_many_ties_at_the_top_survive_an_overflowing_round(ops, storage, k, best_value):
     """Thousands of entities share the best score, and all of them fall into one round, whose candidate buffer
     (4096 slots) overflows and keeps a random sample.  The repair scan must bring back the ties with the LOWEST ids,
-    which no score threshold can tell from the others: it admits by key (score, then entity id)."""
+    which no score threshold can tell from the others: it admits by key (score, then entity id).  With best_value 0
+    the shared score is +0.0, whose neighbour in the ordered encoding (-0.0) compares equal to it."""
     rng = np.random.default_rng(77 + k)
     N, d, B = 60000, 128, 6
     q = np.zeros((B, d), dtype=np.float32)
@@ -536,7 +538,7 @@ def test_topk_many_ties_at_the_top_survive_an_overflowing_round(ops, storage, k)
     lo = rng.integers(-40, 0, (N, d)).astype(np.int8)              # every ordinary row scores below zero
     tied = np.sort(rng.choice(np.arange(1100, 16000), 9000, replace=False))
     best = np.zeros(d, dtype=np.int8)
-    best[:8] = 90
+    best[:8] = best_value
     lo[tied] = best                                                  # 9000 identical rows: one exact score
     if storage == "int8":
         E = dev(torch.from_numpy(lo))
