@@ -909,6 +909,58 @@ def test_build_query_backward_fp32(ops, model, d, kw):
 
 
 # ---------------------------------------------------------------------------------------------
+# top-k over tables built to defeat its shortcuts: several rounds, guessed thresholds, overflowing buffers, repairs
+# ---------------------------------------------------------------------------------------------
+def _topk_stress_cases():
+    cases = []
+    i = 0
+    for storage, d in (("fp32", 32), ("bf16", 128), ("bf16", 64), ("int8", 128), ("int8", 64)):
+        for pattern in ("pool1", "pool3", "pool50", "ascending", "descending", "two_values", "zero_rows"):
+            k = (1, 7, 100, 1000)[i % 4]
+            N = (5000, 20011, 70001)[i % 3]
+            B = (1, 5, 70)[(i // 2) % 3]
+            cases.append((i, storage, d, pattern, N, B, k))
+            i += 1
+    return cases
+
+
+@pytest.mark.parametrize("seed,storage,d,pattern,N,B,k", _topk_stress_cases())
+def test_topk_stress_patterns_match_the_materialised_scores(ops, seed, storage, d, pattern, N, B, k):
+    """Tables whose scores tie massively (rows drawn from a pool of 1, 3 or 50 distinct rows; only two distinct
+    scores; thousands of all-zero rows) or arrive in the worst order (best rows last: every guessed threshold fails;
+    best rows first), for every storage and across the rounds of a call: the result must be the top k of the
+    library's own scores, ties towards the lower entity id."""
+    rng = np.random.default_rng(1000 + seed)
+    k = min(k, N)
+    Q = (rng.standard_normal((B, d)) * 0.3).astype(np.float32)
+    ints = rng.integers(-90, 91, (N, d)).astype(np.int8)                  # every storage holds these exactly
+    if pattern.startswith("pool"):
+        pool = rng.integers(-90, 91, (int(pattern[4:]), d)).astype(np.int8)
+        ints = pool[rng.integers(0, len(pool), N)]
+    elif pattern == "two_values":
+        v = rng.integers(-90, 91, d).astype(np.int8)
+        ints = np.where(rng.random(N)[:, None] < 0.5, v[None, :], -v[None, :]).astype(np.int8)
+    elif pattern == "zero_rows":
+        ints[rng.random(N) < 0.4] = 0
+    if pattern in ("ascending", "descending"):
+        s0 = ints.astype(np.float64) @ Q[0].astype(np.float64)           # order by the first query's scores
+        order = np.argsort(s0 if pattern == "ascending" else -s0, kind="stable")
+        ints = ints[order]
+    if storage == "int8":
+        E, sc = dev(torch.from_numpy(ints)), dev(torch.full((N,), 0.01))
+    else:
+        E, sc = dev(torch.from_numpy(ints.astype(np.float32) * 0.01)), None
+        if storage == "bf16":
+            E = E.to(torch.bfloat16)
+    Qg = dev(torch.from_numpy(Q))
+    vals, idx = ops.topk(Qg, None, E, sc, k)
+    S = ops.scores(Qg, None, E, sc).cpu().numpy()
+    wv, wi = ko.topk(S, k)
+    np.testing.assert_array_equal(vals.cpu().numpy(), wv)
+    np.testing.assert_array_equal(idx.cpu().numpy(), wi)
+
+
+# ---------------------------------------------------------------------------------------------
 # seeded sweep over awkward shapes: every fused epilogue against the library's own materialised scores
 # ---------------------------------------------------------------------------------------------
 def _sweep_cases():
