@@ -960,6 +960,50 @@ def test_topk_stress_patterns_match_the_materialised_scores(ops, seed, storage, 
     np.testing.assert_array_equal(idx.cpu().numpy(), wi)
 
 
+@pytest.mark.parametrize("storage,d", [("fp32", 32), ("bf16", 128), ("bf16", 64), ("int8", 128), ("int8", 64), ("bf16", 256)])
+@pytest.mark.parametrize("pattern", ["pool1", "pool3", "pool50", "two_values", "zero_rows"])
+def test_rank_stress_patterns_match_the_materialised_scores(ops, FilterCSR, storage, d, pattern):
+    """The same massively tied tables under the filtered rank: the target ties with thousands of entities (every
+    stage of the bf16 d = 128 main loop takes its exact second pass), filter rows hold tied entities and the target
+    itself; counters must equal those counted on the library's own scores."""
+    rng = np.random.default_rng(sum(ord(ch) for ch in storage + pattern) * 1000 + d)
+    N, R, B = 9001, 5, 700
+    Q = (rng.standard_normal((B, d)) * 0.3).astype(np.float32)
+    ints = rng.integers(-90, 91, (N, d)).astype(np.int8)
+    if pattern.startswith("pool"):
+        pool = rng.integers(-90, 91, (int(pattern[4:]), d)).astype(np.int8)
+        ints = pool[rng.integers(0, len(pool), N)]
+    elif pattern == "two_values":
+        v = rng.integers(-90, 91, d).astype(np.int8)
+        ints = np.where(rng.random(N)[:, None] < 0.5, v[None, :], -v[None, :]).astype(np.int8)
+    elif pattern == "zero_rows":
+        ints[rng.random(N) < 0.4] = 0
+    if storage == "int8":
+        E, sc = dev(torch.from_numpy(ints)), dev(torch.full((N,), 0.01))
+    else:
+        E, sc = dev(torch.from_numpy(ints.astype(np.float32) * 0.01)), None
+        if storage == "bf16":
+            E = E.to(torch.bfloat16)
+    Qg = dev(torch.from_numpy(Q))
+    bias = dev(torch.from_numpy(rng.standard_normal(B).astype(np.float32)))
+    hr = random_hr(rng, N, R, B)
+    hr[B // 2:] = hr[:B - B // 2]                                    # every filter row shared by two queries ...
+    Q[B // 2:] = Q[:B - B // 2]                                      # ... that hold the same vector, as (h, r) pairs do
+    Qg = dev(torch.from_numpy(Q))
+    targets = rng.integers(0, N, B).astype(np.int64)
+    er = random_csr(rng, hr, targets, N, R, max_len=40)
+    csr = FilterCSR.from_er_vocab(er, R, device="cuda")
+    hr_g = dev(torch.from_numpy(hr))
+    out = ops.rank_filtered(Qg, bias, E, sc, dev(torch.from_numpy(targets)), csr.rows_for(hr_g), csr.row_ptr, csr.col)
+    S_raw = ops.scores(Qg, None, E, sc).cpu().numpy()
+    g, t, tl = _expected_counts(S_raw, targets, [er[(int(h), int(r))] for h, r in hr])
+    np.testing.assert_array_equal(out["n_greater"].cpu().numpy(), g)
+    np.testing.assert_array_equal(out["n_equal"].cpu().numpy(), t)
+    np.testing.assert_array_equal(out["n_equal_lower"].cpu().numpy(), tl)
+    if pattern == "pool1":
+        assert t.max() > N // 2                                       # the ties are really there
+
+
 # ---------------------------------------------------------------------------------------------
 # seeded sweep over awkward shapes: every fused epilogue against the library's own materialised scores
 # ---------------------------------------------------------------------------------------------
