@@ -25,7 +25,7 @@ namespace host {
 // ---- sizes shared by host and kernels -------------------------------------------------------------------
 constexpr int SORT_MAX = 8192;           // queries per sub-batch of the filter correction
 constexpr int WORK_MAX = 16 * SORT_MAX;  // upper bound on work items per sub-batch (bounds the slice count only)
-constexpr int SLICE_MIN = 128;           // shortest slice of a filter row
+constexpr int SLICE_MIN = 256;           // shortest slice of a filter row
 constexpr int PLAN_SLOTS = 2 * SORT_MAX; // hash table of the plan kernel: load factor <= 0.5
 constexpr int PLAN_HASH_SHIFT = 18;      // 32 - log2(PLAN_SLOTS)
 static_assert(PLAN_SLOTS == (1 << (32 - PLAN_HASH_SHIFT)), "hash width");

@@ -399,7 +399,21 @@ __global__ void __launch_bounds__(256) filter_fix_kernel(ContractArgs a, FixPlan
     if (tid < FIX_ITEMS) {
       const int64_t w = blockIdx.x + (int64_t)(k0 + tid) * gridDim.x;
       if (w < n_work) {
-        int lo = 0, hi = n_groups;  // last group whose first work item is <= w
+        int lo = 0, hi = n_groups;  // last group whose first work item is <= w: in [lo, hi)
+        // fifteen pivots per step, their loads in flight together: a sixteenth of the range is left (a search
+        // that halves the range is a chain of log2(n_groups) dependent loads at the head of every workgroup)
+        while (hi - lo > 16) {
+          const int step = (hi - lo) >> 4;
+          int first[15];
+#pragma unroll
+          for (int j = 0; j < 15; ++j) first[j] = plan.work[2 * (lo + step * (j + 1)) + 1];
+          int le = 0;  // pivots whose first work item is <= w: a prefix
+#pragma unroll
+          for (int j = 0; j < 15; ++j) le += (first[j] <= (int64_t)w) ? 1 : 0;
+          const int nlo = lo + step * le, nhi = (le < 15) ? lo + step * (le + 1) : hi;
+          lo = nlo;
+          hi = nhi;
+        }
         while (hi - lo > 1) {
           const int mid = (lo + hi) >> 1;
           if (plan.work[2 * mid + 1] <= w) lo = mid; else hi = mid;
@@ -468,6 +482,15 @@ __global__ void __launch_bounds__(256) filter_fix_kernel(ContractArgs a, FixPlan
           }
         }
         __syncthreads();
+      }
+      // the threshold and target of this thread's member of the first compare batch (nearly always the only batch):
+      // two dependent loads, issued here so that they travel while the slice's rows are gathered
+      int64_t pre_b = 0, pre_t = 0;
+      float pre_th = 0.f;
+      if (lead + mslot < m) {
+        pre_b = b0 + (int64_t)host::plan_key_pos(plan.skey[i0 + lead + mslot]);
+        pre_th = thr[pre_b];
+        pre_t = target[pre_b];
       }
       for (int64_t pass = z0; pass < z1; pass += CAP) {
         const int n_here = (int)((z1 - pass < CAP) ? z1 - pass : CAP);
@@ -555,9 +578,10 @@ __global__ void __launch_bounds__(256) filter_fix_kernel(ContractArgs a, FixPlan
           __syncthreads();
           int64_t b = 0;
           if (mine) {
-            b = b0 + (int64_t)host::plan_key_pos(plan.skey[i0 + mi]);
-            const float th = thr[b];
-            const int64_t t = target[b];
+            const bool pre = mbase == lead;
+            b = pre ? pre_b : b0 + (int64_t)host::plan_key_pos(plan.skey[i0 + mi]);
+            const float th = pre ? pre_th : thr[b];
+            const int64_t t = pre ? pre_t : target[b];
             int32_t g = 0, eq = 0, eql = 0;
             for (int j = sub; j < n_here; j += tpm) {
               const int32_t e = s_e[j];
