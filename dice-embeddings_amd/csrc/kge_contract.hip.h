@@ -183,6 +183,56 @@ struct StoreEpi {
   __device__ void finish() {}
 };
 
+// First round of kge_topk: every row scanned is a candidate (no threshold yet), so the scores go out as packed
+// keys in row order, cand[q, e - e_begin], lanes along the entity index (whole lines per store), instead of
+// through the candidate queues, which that many candidates would flush sixty times per workgroup.  A score that
+// no threshold admits (NaN, -inf: the rounds admit what beats the k-th best, -inf at the start) leaves key 0 (empty).
+struct TopkFirstArgs {
+  unsigned long long* cand;  // [B, cap]
+  int64_t cap;
+  int64_t e_begin;
+};
+template <int NQT>
+struct TopkFirstEpi {
+  static constexpr bool SWAP = true;
+  static constexpr bool STAGE_HOOK = false;
+  static constexpr bool DEFER = false;
+  using Args = TopkFirstArgs;
+  struct Shared {
+    int unused;
+  };
+  Args a;
+  int64_t q0, B;
+  int c, hf;
+  __device__ void init(const Args& args, int64_t q0_, int c_, int hf_, int64_t B_) {
+    a = args; q0 = q0_; c = c_; hf = hf_; B = B_;
+  }
+  __device__ void bind(Shared*) {}
+  __device__ void stage_mark() {}
+  __device__ void stage_end() {}
+  template <bool HAS_SCALE>
+  __device__ __forceinline__ void tile(int qt, const f32x16& acc, const float* sc16, float sc_col, int64_t e_base,
+                                       int64_t limit) {
+    const int64_t e = e_base + c;
+    if (e >= limit) return;
+    const int64_t qrow = q0 + 32 * qt + 4 * hf;  // query row of acc[0]; acc[4g + r] is row qrow + 8g + r
+    unsigned long long* p = a.cand + qrow * a.cap + (e - a.e_begin);
+    const unsigned long long id_part = (unsigned long long)(0xffffffffu - (uint32_t)e);
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        float v = acc[4 * g + r];
+        if (HAS_SCALE) v *= sc_col;
+        const unsigned long long key =
+            (v > __uint_as_float(0xff800000u)) ? (((unsigned long long)f32_to_ordered(v) << 32) | id_part) : 0ull;
+        if (qrow + 8 * g + r < B) p[(int64_t)(8 * g + r) * a.cap] = key;
+      }
+    }
+  }
+  __device__ void finish() {}
+};
+
 struct RankArgs {
   const float* thr;  // raw target score per query
   const int64_t* target;

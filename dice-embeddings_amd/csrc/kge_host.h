@@ -122,6 +122,7 @@ inline RankWsOffsets rank_ws_offsets(int64_t B) {
 constexpr int TOPK_ROWMETA_ROWS = 64;
 constexpr int TOPK_ROWMETA_BYTES = 32;  // per 32-row tile {scale, max L1 + 64, forced, -}
 constexpr int TOPK_REQUANT_D = 128;
+constexpr int64_t TOPK_FILTER_MIN_ROWS = 65536;  // rounds of at most this many rows skip the int8 filter scan
 // qh / qc: the queries as the int8 filter scan reads them (TOPK_REQUANT_D int8 per query, and per query the four
 // constants of its bound), written once per call.
 struct TopkWsOffsets {

@@ -680,12 +680,13 @@ size_t topk_ws_layout(int64_t B, int64_t N, int64_t k, void* base, TopkWs* ws, c
   return o.total;
 }
 
-__global__ void topk_init_kernel(TopkWs w, int64_t B) {
+// `first_rows`: the rows of the first round, whose scan writes one key per row into every query's candidate buffer
+__global__ void topk_init_kernel(TopkWs w, int64_t B, int32_t first_rows) {
   const int64_t b = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (b < B) {
     w.tau[b] = __uint_as_float(0xff800000u);  // -inf
     w.tau_scan[b] = __uint_as_float(0xff800000u);
-    w.cnt[b] = 0;
+    w.cnt[b] = first_rows;
     w.list_len[b] = 0;
     w.dirty[b] = 0;
     w.kth[b] = 0;
@@ -1634,7 +1635,8 @@ int topk_impl(const char* who, const float* Q, const float* bias, const void* E,
   int rc = KGE_OK;
   TopkWs ws;
   topk_ws_layout(B, N, k, workspace, &ws, prepared, prepared == nullptr);
-  hipLaunchKernelGGL(topk_init_kernel, dim3((unsigned)((B + 255) / 256)), dim3(256), 0, st, ws, B);
+  const int64_t first_rows = (N < TOPK_FIRST_ROWS) ? N : TOPK_FIRST_ROWS;
+  hipLaunchKernelGGL(topk_init_kernel, dim3((unsigned)((B + 255) / 256)), dim3(256), 0, st, ws, B, (int32_t)first_rows);
   KGE_LAUNCH_CHECK("topk_init_kernel");
 
   // An int8 table with d == 128 is scanned by the integer filter (after the first round, which takes every row
@@ -1654,9 +1656,16 @@ int topk_impl(const char* who, const float* Q, const float* bias, const void* E,
   auto launch_scan = [&](int64_t e0, int64_t e1, const float* tau, const int32_t* active, int rescan,
                          const char* name) -> int {
     ContractArgs a = make_args(Q, E, dtype, scale, B, d, N, e0, e1);
+    if (e0 == 0 && !rescan) {
+      // the first round: every row a candidate, written as dense keys (the candidate counts were set to match)
+      TopkFirstArgs ef{ws.cand, (int64_t)TOPK_CAP, e0};
+      return launch_contract<TopkFirstEpi>(dtype, a, ef, st, name);
+    }
     // (the repair scan is exact as well: a query the bound cannot separate from most of the table, its threshold
     // tiny against the scales around it, would overflow its buffer again)
-    if (!id_filter || rescan || e0 % host::TOPK_ROWMETA_ROWS != 0 || (e0 == 0 && e1 <= TOPK_FIRST_ROWS)) {
+    // (short rounds are exact as well: the filter's extra launch to score its candidates, and the candidates its
+    // bound lets through needlessly, cost more there than the exact epilogue does)
+    if (!id_filter || rescan || e0 % host::TOPK_ROWMETA_ROWS != 0 || e1 - e0 <= host::TOPK_FILTER_MIN_ROWS) {
       if (rescan) {
         // a repair scan admits what ranks above the query's k-th best by KEY, so that ties with it at lower entity
         // ids, which an overflowing buffer may have dropped, are found again
@@ -1700,7 +1709,7 @@ int topk_impl(const char* who, const float* Q, const float* bias, const void* E,
   };
   // round r scans (growth - 1) x what is already ranked
   const int64_t growth = host::topk_growth(k);
-  int64_t e0 = 0, e1 = (N < TOPK_FIRST_ROWS) ? N : TOPK_FIRST_ROWS;
+  int64_t e0 = 0, e1 = first_rows;
   while (e0 < N) {
     rc = launch_scan(e0, e1, ws.tau_scan, nullptr, 0, "kge_topk scan");
     if (rc) return rc;
