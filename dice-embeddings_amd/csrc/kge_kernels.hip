@@ -862,7 +862,12 @@ __global__ void __launch_bounds__(64) topk_select_wave_kernel(TopkWs w, int k, i
   if (raw > TOPK_CAP || len + raw > SELECT_SMALL) return;  // left to topk_select_kernel
   const float tau_old = w.tau[b];
   const float th_used = rescan ? tau_old : w.tau_scan[b];
-  if (len + raw <= 512)
+  // (the network's cost grows faster than the number of keys: short lists, the usual case for small k, take a small one)
+  if (len + raw <= 128)
+    select_in_registers<2>(w, b, k, rescan, len, raw, tau_old, th_used, j_spec, lane);
+  else if (len + raw <= 256)
+    select_in_registers<4>(w, b, k, rescan, len, raw, tau_old, th_used, j_spec, lane);
+  else if (len + raw <= 512)
     select_in_registers<8>(w, b, k, rescan, len, raw, tau_old, th_used, j_spec, lane);
   else
     select_in_registers<16>(w, b, k, rescan, len, raw, tau_old, th_used, j_spec, lane);
