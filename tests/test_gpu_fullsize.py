@@ -14,7 +14,7 @@ pytestmark = pytest.mark.gpu
 
 
 def test_c2_complex_filtered_mrr_eval_at_full_size():
-    """C2 as BASELINE.json states it: ComplEx, 14,541 entities, d = 200 fp32, 272k Zipf triples, 20k eval queries in
+    """The second benchmark configuration as it is specified: ComplEx, 14,541 entities, d = 200 fp32, 272k Zipf triples, 20k eval queries in
     batches of 1024 (the last holds 544) through the Evaluator (dicee/evaluation/evaluator.py:473-510).  Every rank
     lies inside the fp64 oracle's tolerance interval and equals the oracle's rank wherever that interval is one
     point; the counters of sampled batches are bit-exact against the library's own materialised scores."""
