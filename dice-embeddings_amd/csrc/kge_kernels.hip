@@ -129,6 +129,28 @@ __device__ __forceinline__ f32x16 chain_direct(const void* E, int d, int64_t e_r
   return acc;
 }
 
+// A member that is not its group's leader compares its vector with the leader's: the two halves of the wave
+// take alternate 16-byte pieces of the row (alternate words when the rows are not 16-byte aligned).
+__device__ __forceinline__ void group_vector_check(const ContractArgs& a, int64_t q, int hf, const int32_t* lead,
+                                                   int32_t* mixed) {
+  const int32_t l = lead[q];
+  if (l >= 0 && (int64_t)l != q) {
+    const uint32_t* x = (const uint32_t*)a.Q + q * a.d;
+    const uint32_t* y = (const uint32_t*)a.Q + (int64_t)l * a.d;
+    bool differs = false;
+    if ((a.d & 3) == 0 && ((uintptr_t)a.Q & 15) == 0) {
+#pragma unroll 4
+      for (int64_t k = hf * 4; k < a.d; k += 8) {
+        const uint4 u = *(const uint4*)(x + k), w = *(const uint4*)(y + k);
+        differs = differs || u.x != w.x || u.y != w.y || u.z != w.z || u.w != w.w;
+      }
+    } else {
+      for (int64_t k = hf; k < a.d; k += 2) differs = differs || x[k] != y[k];
+    }
+    if (differs) mixed[l] = 1;
+  }
+}
+
 // ---- raw score of each query's target (the rank threshold) + counter initialisation ---------
 // and, when the batch is filtered, the check the filter correction relies on: the correction scores a slice of a
 // filter row once per group of queries that share the row, with the query vector of the group's leader.  A member
@@ -140,7 +162,16 @@ __global__ void __launch_bounds__(256) target_score_kernel(ContractArgs a, const
                                                           int32_t* n_eq, int32_t* n_eql, const int32_t* lead,
                                                           int32_t* mixed) {
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, c = lane & 31, hf = lane >> 5;
-  const int64_t q = ((int64_t)blockIdx.x * 4 + wave) * 32 + c;
+  // With a filter the launch holds two sets of workgroups: the first forms the thresholds, the second makes the
+  // group check for the same queries at the same time on other CUs (both are short chains of dependent loads; one
+  // after the other in the same wave they would simply add up).
+  const int64_t n_score_wgs = (a.B + 127) / 128;
+  const bool check_role = (int64_t)blockIdx.x >= n_score_wgs;
+  const int64_t q = (((int64_t)blockIdx.x - (check_role ? n_score_wgs : 0)) * 4 + wave) * 32 + c;
+  if (check_role) {
+    if (lead != nullptr && q < a.B) group_vector_check(a, q, hf, lead, mixed);
+    return;
+  }
   const int64_t t = (q < a.B) ? target[q] : -1;
   const bool ok = t >= 0 && t < a.N;
   f32x16 acc = chain_direct<EDT>(a.E, a.d, ok ? t : -1, a.Q, (q < a.B) ? q : -1, hf);
@@ -158,26 +189,6 @@ __global__ void __launch_bounds__(256) target_score_kernel(ContractArgs a, const
     n_gt[q] = 0;
     n_eq[q] = ok ? -1 : 0;  // the main pass counts the target as tying with itself
     n_eql[q] = 0;
-  }
-  if (lead != nullptr && q < a.B) {
-    // a member that is not its group's leader compares its vector with the leader's: the two halves of the wave
-    // take alternate 16-byte pieces of the row (alternate words when the rows are not 16-byte aligned)
-    const int32_t l = lead[q];
-    if (l >= 0 && (int64_t)l != q) {
-      const uint32_t* x = (const uint32_t*)a.Q + q * a.d;
-      const uint32_t* y = (const uint32_t*)a.Q + (int64_t)l * a.d;
-      bool differs = false;
-      if ((a.d & 3) == 0 && ((uintptr_t)a.Q & 15) == 0) {
-#pragma unroll 4
-        for (int64_t k = hf * 4; k < a.d; k += 8) {
-          const uint4 u = *(const uint4*)(x + k), w = *(const uint4*)(y + k);
-          differs = differs || u.x != w.x || u.y != w.y || u.z != w.z || u.w != w.w;
-        }
-      } else {
-        for (int64_t k = hf; k < a.d; k += 2) differs = differs || x[k] != y[k];
-      }
-      if (differs) mixed[l] = 1;
-    }
   }
 }
 
@@ -1427,7 +1438,7 @@ int rank_filtered_launch(const char* who, const float* Q, const float* bias, con
     }
   }
   {
-    dim3 grid((unsigned)((B + 127) / 128)), block(256);
+    dim3 grid((unsigned)((B + 127) / 128 * (filtered ? 2 : 1))), block(256);  // (second half: the group check)
     KGE_DISPATCH_DTYPE(dtype, target_score_kernel, grid, block, 0, st, a, target, bias, ws.thr, target_score,
                        n_greater, n_equal, n_equal_lower, filtered ? (const int32_t*)ws.plan.lead : (const int32_t*)nullptr,
                        ws.plan.mixed);
