@@ -120,7 +120,7 @@ inline RankWsOffsets rank_ws_offsets(int64_t B) {
 // requant: the int8 table written again with one scale per 32-row tile, N x 128 bytes, and rowmeta: one
 // TOPK_ROWMETA_BYTES record per TOPK_ROWMETA_ROWS table rows (both for the int8 filter scan)
 constexpr int TOPK_ROWMETA_ROWS = 64;
-constexpr int TOPK_ROWMETA_BYTES = 32;  // per 32-row tile {scale, max L1 + 64, forced, -}
+constexpr int TOPK_ROWMETA_BYTES = 32;  // per 32-row tile {scale (negative: forced), max |e'|_2, max |rho|_2, 1 / scale}
 constexpr int TOPK_REQUANT_D = 128;
 constexpr int64_t TOPK_FILTER_MIN_ROWS = 65536;  // rounds of at most this many rows skip the int8 filter scan
 // qh / qc: the queries as the int8 filter scan reads them (TOPK_REQUANT_D int8 per query, and per query the four

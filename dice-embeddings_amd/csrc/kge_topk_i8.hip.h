@@ -7,13 +7,16 @@
 //     negative scale moves into e'; a row whose scale is tiny against its neighbours' becomes mostly zeros,
 //     which costs the bound tightness but not validity;
 //   * the query row is rounded to bf16 (qb, the operand of the exact score) and then quantised to int8,
-//     qb_k = s_q qh_k + delta_k with |delta_k| <= dq;  H' = sum_k e'_k qh_k is an exact int32 from the int8 MFMA
-//     (32x32x32, twice the bf16 rate, and the rows go global -> LDS untouched);
-//   * the exact score is fl(s_e A) with A = fl(sum_k e_k qb_k) (fp32 accumulation: |A - sum| is at most
-//     128 * 2^-23 * sum_k |e_k qb_k| <= 1.9e-3 s_q L1(e), L1(e) = sum_k |e_k|, since |qb_k| <= 127 s_q).  Hence
-//       s_e A <= S ( s_q H' + mq (L1(e') + 64) + 0.501 L1(qb) ),      mq = dq + 4e-3 s_q
-//     (the 64 covers sum_k |rho_k|, the 4e-3 the rounding of the chain and of this bound's own few operations).
-//     Per element nothing but the MFMA; per tile and lane the maximum of its 16 accumulators and five float
+//     qb_k = s_q qh_k + delta_k;  H' = sum_k e'_k qh_k is an exact int32 from the int8 MFMA (32x32x32, twice the
+//     bf16 rate, and the rows go global -> LDS untouched);
+//   * in exact arithmetic s_e sum_k e_k qb_k = S ( s_q H' + sum_k e'_k delta_k + sum_k rho_k qb_k ), and each of
+//     the two residual sums is at most the product of the two vectors' Euclidean norms.  The exact score is
+//     fl(s_e A) with A = fl(sum_k e_k qb_k) (fp32 accumulation: |A - sum| is at most 128 * 2^-23 * sum_k |e_k qb_k|
+//     <= 1.9e-3 s_q L1(e), since |qb_k| <= 127 s_q; S L1(e) <= S (L1(e') + 64) <= S (11.32 |e'|_2 + 64)).  Hence
+//       s_e A <= S ( s_q H' + m_q |e'|_2 + |rho|_2 |qb|_2 + 0.256 s_q ),      m_q = |delta|_2 + 0.0453 s_q
+//     (0.0453 = 4e-3 * 11.32 and 0.256 = 4e-3 * 64: the rounding of the chain, and of this bound's own few
+//     operations, with a factor two to spare).  |e'|_2 and |rho|_2 are the largest of the tile's rows, rounded up.
+//     Per element nothing but the MFMA; per tile and lane the maximum of its 16 accumulators and six float
 //     operations.  A tile none of whose lanes can beat its query's tau is passed over; in the others the
 //     accumulators are compared with the threshold turned into an integer.
 // An element that passes is only a candidate: its entity id goes to the query's candidate buffer, and its score
@@ -43,9 +46,9 @@ struct I8FilterArgs {
   uint32_t* cand;         // [B, cap] candidate entity ids
   int32_t cap;
   const int8_t* Eq;              // the table with tile-common scales (topk_i8_requant_kernel)
-  const unsigned char* rowmeta;  // one record per 64 table rows: per 32-row tile {S, max L1(e') + 64, forced, 1 / S}
+  const unsigned char* rowmeta;  // one record per 64 table rows: per 32-row tile {S (negative: forced), max |e'|_2, max |rho|_2, 1 / S}
   const int8_t* qh;              // [B, 128] the queries as int8 (topk_i8_qprep_kernel)
-  const f32x4* qc;               // [B] per query {s_q, mq, cq, finite ? 1 : 0}
+  const f32x4* qc;               // [B] per query {s_q, m_q, |qb|_2, finite ? 1 : 0}
 };
 
 constexpr int TF_NQT = 4;                              // 32-query tiles per wave
@@ -66,7 +69,7 @@ static_assert(host::TOPK_ROWMETA_ROWS == TF_STAGE_ROWS && host::TOPK_ROWMETA_BYT
 // all its rows as candidates).
 __global__ void __launch_bounds__(256) topk_i8_requant_kernel(const int8_t* E, const float* scale, int64_t N, int8_t* Eq,
                                                               unsigned char* meta) {
-  __shared__ float s_max[2][4], s_bad[2][4], s_l1[2][4];
+  __shared__ float s_max[2][4], s_bad[2][4], s_e2[2][4], s_r2[2][4];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int64_t rec = blockIdx.x;
   float scv[2];
@@ -97,43 +100,65 @@ __global__ void __launch_bounds__(256) topk_i8_requant_kernel(const int8_t* E, c
     const float S = __builtin_fmaxf(__builtin_fmaxf(s_max[it][0], s_max[it][1]), __builtin_fmaxf(s_max[it][2], s_max[it][3]));
     const float ratio = (S > 0.f) ? scv[it] / S : 0.f;  // |ratio| <= 1: the products below stay within +-127
     u32x4 o;
-    uint32_t l1 = 0;
+    int e2 = 0;       // sum of e'^2 over this thread's sixteen components (exact)
+    float r2 = 0.f;   // sum of rho^2 as computed (the true rho differs by at most 2e-5 per component)
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       uint32_t pk = 0;
 #pragma unroll
       for (int b = 0; b < 4; ++b) {
         const float x = (float)(int)(int8_t)(w[it][i] >> (8 * b));
-        const int v = (int)__builtin_rintf(x * ratio);
+        const float y = x * ratio;
+        const float yr = __builtin_rintf(y);
+        const int v = (int)yr;
         pk |= ((uint32_t)v & 0xffu) << (8 * b);
+        e2 += v * v;
+        r2 = __builtin_fmaf(y - yr, y - yr, r2);
       }
       o[i] = pk;
-      l1 = __builtin_amdgcn_sad_u8(pk ^ 0x80808080u, 0x80808080u, l1);  // sum |int8|
     }
     if (row < N) *(u32x4*)(Eq + row * 128 + 16 * (tid & 7)) = o;
-    l1 += __shfl_xor(l1, 1, 64);
-    l1 += __shfl_xor(l1, 2, 64);
-    l1 += __shfl_xor(l1, 4, 64);
-    float l1M = (float)l1;
 #pragma unroll
-    for (int s = 8; s <= 32; s <<= 1) l1M = __builtin_fmaxf(l1M, __shfl_xor(l1M, s, 64));
-    if (lane == 0) s_l1[it][wave] = l1M;
+    for (int s = 1; s <= 4; s <<= 1) {  // the eight threads of a row
+      e2 += __shfl_xor(e2, s, 64);
+      r2 += __shfl_xor(r2, s, 64);
+    }
+    float e2M = (float)e2;  // at most 128 * 127^2: exact
+    float r2M = r2;
+#pragma unroll
+    for (int s = 8; s <= 32; s <<= 1) {  // the eight rows of a wave
+      e2M = __builtin_fmaxf(e2M, __shfl_xor(e2M, s, 64));
+      r2M = __builtin_fmaxf(r2M, __shfl_xor(r2M, s, 64));
+    }
+    if (lane == 0) {
+      s_e2[it][wave] = e2M;
+      s_r2[it][wave] = r2M;
+    }
   }
   __syncthreads();
   if (tid < 2) {
     const float S = __builtin_fmaxf(__builtin_fmaxf(s_max[tid][0], s_max[tid][1]), __builtin_fmaxf(s_max[tid][2], s_max[tid][3]));
-    const float L = __builtin_fmaxf(__builtin_fmaxf(s_l1[tid][0], s_l1[tid][1]), __builtin_fmaxf(s_l1[tid][2], s_l1[tid][3]));
+    const float E2 = __builtin_fmaxf(__builtin_fmaxf(s_e2[tid][0], s_e2[tid][1]), __builtin_fmaxf(s_e2[tid][2], s_e2[tid][3]));
+    const float R2 = __builtin_fmaxf(__builtin_fmaxf(s_r2[tid][0], s_r2[tid][1]), __builtin_fmaxf(s_r2[tid][2], s_r2[tid][3]));
     const float F = __builtin_fmaxf(__builtin_fmaxf(s_bad[tid][0], s_bad[tid][1]), __builtin_fmaxf(s_bad[tid][2], s_bad[tid][3]));
-    const f32x4 tc = {S, L + 64.f, F, S > 0.f ? 1.f / S : 0.f};
+    // (a scale so small that 1 / S overflows: the tile is forced, like one with a scale that is not finite)
+    const float iS = S > 0.f ? 1.f / S : 0.f;
+    const bool forced = F != 0.f || !(iS <= 3.4028234e38f);
+    // norms rounded up: the square roots and the sums' own rounding (1e-5 relative), and for rho the difference
+    // between the computed and the true residuals (128 components of at most 2e-5: 2.3e-4 on the norm)
+    const f32x4 tc = {forced ? -S : S, __builtin_sqrtf(E2) * 1.00001f, __builtin_sqrtf(R2) * 1.00001f + 1e-3f,
+                      forced ? 0.f : iS};
     *(f32x4*)(meta + rec * host::TOPK_ROWMETA_BYTES + 16 * tid) = tc;
   }
 }
 
 // The queries as the scan reads them, once per call.  One wave per query, two components per lane: the row rounded
-// to bf16 (qb, the operand of the exact score), its largest magnitude and L1 norm, then qb_k = s_q qh_k + delta_k with
-// qh_k an int8 and dq = max |delta_k|.  Per query {s_q, mq = dq + 4e-3 s_q, cq = 0.501 L1(qb), finite}: a row with a
-// component that is not finite has no finite bound (finite = 0: the scan collects nothing for it; its scores are NaN
-// or infinite anyway).
+// to bf16 (qb, the operand of the exact score), its largest magnitude and Euclidean norm, then qb_k = s_q qh_k + delta_k
+// with qh_k an int8.  Per query {s_q, m_q = |delta|_2 + 0.0453 s_q, |qb|_2, kind} (norms rounded up).  kind 0: a row
+// with a component that is not finite has no finite bound; the scan collects nothing for it (its scores are NaN or
+// infinite anyway).  kind 2: components so large (about 1e34) that the bound's own arithmetic could overflow; the
+// scan takes every row as a candidate for it.  kind 1: everything else.
+constexpr float TF_NORM_MAX = 1e35f;  // m_q |e'|_2 + |rho|_2 |qb|_2 + s_q |H'| stays finite below this
 __global__ void __launch_bounds__(256) topk_i8_qprep_kernel(const float* Q, int64_t B, int8_t* qh, f32x4* qc) {
   const int lane = threadIdx.x & 63;
   const int64_t q = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
@@ -141,38 +166,56 @@ __global__ void __launch_bounds__(256) topk_i8_qprep_kernel(const float* Q, int6
   const float* row = Q + q * 128;
   const float r0 = (float)(__bf16)row[2 * lane], r1 = (float)(__bf16)row[2 * lane + 1];
   float amax = __builtin_fmaxf(__builtin_fabsf(r0), __builtin_fabsf(r1));
-  float l1q = __builtin_fabsf(r0) + __builtin_fabsf(r1);
   int bad = (r0 != r0 || r1 != r1) ? 1 : 0;  // fmax drops a NaN
 #pragma unroll
   for (int o = 1; o < 64; o <<= 1) {
     amax = __builtin_fmaxf(amax, __shfl_xor(amax, o, 64));
-    l1q += __shfl_xor(l1q, o, 64);
     bad |= __shfl_xor(bad, o, 64);
   }
-  const bool finite = !bad && amax <= 3.4028234e38f && l1q <= 3.4028234e38f;
+  const bool finite = !bad && amax <= 3.4028234e38f;
   const float s_q = finite ? amax / 127.f : 0.f;
   const float inv = (finite && amax > 0.f) ? 127.f / amax : 0.f;
-  float dq = 0.f;
+  // the squares are taken of the components times 2^-ex (below 1 in magnitude: neither overflow nor underflow of
+  // what matters), the norms scaled back after
+  int ex = 0;
+  if (finite) (void)__builtin_frexpf(amax, &ex);
+  float d2 = 0.f, n2 = 0.f;
   uint32_t pk = 0;
 #pragma unroll
   for (int j = 0; j < 2; ++j) {
     const float r = finite ? (j ? r1 : r0) : 0.f;
     float h = __builtin_rintf(r * inv);
     h = __builtin_fminf(__builtin_fmaxf(h, -127.f), 127.f);
-    dq = __builtin_fmaxf(dq, __builtin_fabsf(__builtin_fmaf(-s_q, h, r)));
+    const float dl = __builtin_ldexpf(__builtin_fmaf(-s_q, h, r), -ex);
+    const float rl = __builtin_ldexpf(r, -ex);
+    d2 = __builtin_fmaf(dl, dl, d2);
+    n2 = __builtin_fmaf(rl, rl, n2);
     pk |= ((uint32_t)(int)h & 0xffu) << (8 * j);
   }
 #pragma unroll
-  for (int o = 1; o < 64; o <<= 1) dq = __builtin_fmaxf(dq, __shfl_xor(dq, o, 64));
+  for (int o = 1; o < 64; o <<= 1) {
+    d2 += __shfl_xor(d2, o, 64);
+    n2 += __shfl_xor(n2, o, 64);
+  }
   ((uint16_t*)(qh + q * 128))[lane] = (uint16_t)pk;
   if (lane == 0) {
-    const f32x4 c = {s_q, dq * 1.000001f + 4e-3f * s_q, finite ? 0.501f * l1q * 1.00001f : 0.f, finite ? 1.f : 0.f};
+    // 1.0001: the roundings of the two sums of 128 squares and of the square roots
+    const float dn = __builtin_ldexpf(__builtin_sqrtf(d2) * 1.0001f, ex);
+    const float qn = __builtin_ldexpf(__builtin_sqrtf(n2) * 1.0001f, ex);
+    const float mq = dn + 0.0453f * s_q;
+    f32x4 c = {0.f, 0.f, 0.f, 0.f};
+    if (finite) {
+      if (mq <= TF_NORM_MAX && qn <= TF_NORM_MAX)
+        c = f32x4{s_q, mq, qn, 1.f};
+      else
+        c[3] = 2.f;
+    }
     qc[q] = c;
   }
 }
 
 constexpr int TF_QUEUE = 64;         // parked accumulator sets per wave
-constexpr int TF_QUEUE_STRIDE = 21;  // dwords per set (19 used; odd: lanes reading their own set hit distinct banks)
+constexpr int TF_QUEUE_STRIDE = 20;  // dwords per set (19 used): five 16-byte pieces, written and read as such
 constexpr int TF_DENSE_LANES = 16;   // a tile with more lanes of interest than this is worked off on the spot
 
 // What the out-of-line slow paths need, as few scalars as will do (every argument travels in a register: a struct
@@ -238,13 +281,18 @@ __device__ __attribute__((noinline)) void tf_drain(const uint32_t* queue, int n,
                                                    uint32_t* cand, int32_t cap, int32_t q_wg, uint32_t limit) {
   const int lane = threadIdx.x & 63;
   const bool on = lane < n;
-  const uint32_t* ent = queue + (on ? lane : 0) * TF_QUEUE_STRIDE;
+  const u32x4* ent = (const u32x4*)(queue + (on ? lane : 0) * TF_QUEUE_STRIDE);
   int hh[16];
 #pragma unroll
-  for (int i = 0; i < 16; ++i) hh[i] = (int)ent[i];
-  const int thr = (int)ent[16];
-  const uint32_t where = ent[17];
-  const uint32_t e_base = ent[18];
+  for (int p = 0; p < 4; ++p) {
+    const u32x4 v = ent[p];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) hh[4 * p + j] = (int)v[j];
+  }
+  const u32x4 tail = ent[4];
+  const int thr = (int)tail[0];
+  const uint32_t where = tail[1];
+  const uint32_t e_base = tail[2];
   const TfSink k{bucket, bcnt, cnt, cand, cap, q_wg, limit};
   tf_collect(hh, thr, on, (int)(where & 0xffffu), (int)(where >> 16), e_base, k);
 }
@@ -255,7 +303,7 @@ __global__ void __launch_bounds__(64 * TF_W, 2) topk_i8_filter_kernel(ContractAr
   __shared__ __attribute__((aligned(16))) unsigned char meta_lds[TF_NBUF][host::TOPK_ROWMETA_BYTES];
   __shared__ uint32_t bucket[WQ * TF_BUCKET];
   __shared__ int bcnt[WQ];
-  __shared__ uint32_t queue[W][TF_QUEUE * TF_QUEUE_STRIDE];
+  __shared__ __attribute__((aligned(16))) uint32_t queue[W][TF_QUEUE * TF_QUEUE_STRIDE];
 
   const int64_t wg = blockIdx.x;
   const int xcd = (int)(wg & 7);
@@ -286,7 +334,7 @@ __global__ void __launch_bounds__(64 * TF_W, 2) topk_i8_filter_kernel(ContractAr
 
   // ---- the queries of this lane: int8 fragments and the constants of the bound ------------------
   i32x4 qf[NQT][4];
-  float sq[NQT], isq[NQT], cq[NQT], mq[NQT], tau_lo[NQT];
+  float sq[NQT], isq[NQT], cq[NQT], mq[NQT], nq[NQT], tau_lo[NQT];
 #pragma unroll
   for (int t = 0; t < NQT; ++t) {
     const int64_t q = q_wg + ql0 + 32 * t + c;
@@ -301,10 +349,12 @@ __global__ void __launch_bounds__(64 * TF_W, 2) topk_i8_filter_kernel(ContractAr
     if (q < a.B) qcv = ea.qc[q];
     const float s_q = qcv[0];
     const bool finite = qcv[3] != 0.f;
+    const bool everything = qcv[3] == 2.f;  // no usable bound: s_q, m_q and the norm are 0 and the threshold -inf
     sq[t] = s_q;
     isq[t] = s_q > 0.f ? 1.f / s_q : 0.f;
     mq[t] = qcv[1];
-    cq[t] = qcv[2];
+    nq[t] = qcv[2];
+    cq[t] = 0.256f * s_q;
     // a query with a non-finite component has no finite bound: it collects nothing (its scores are NaN or
     // infinite anyway)
     const bool on = q < a.B && finite && (ea.active == nullptr || ea.active[q] != 0);
@@ -312,6 +362,7 @@ __global__ void __launch_bounds__(64 * TF_W, 2) topk_i8_filter_kernel(ContractAr
     if (on) {
       th = ea.tau[q];
       if (th > -INF && th < INF) th = th - 1e-6f * __builtin_fabsf(th);  // the comparison's own rounding
+      if (everything && th < INF) th = -INF;  // every bound (0 or more) passes, and so does every accumulator
     }
     tau_lo[t] = th;
   }
@@ -348,14 +399,15 @@ __global__ void __launch_bounds__(64 * TF_W, 2) topk_i8_filter_kernel(ContractAr
 
   // ---- the test of one finished tile ------------------------------------------------------------
   // constants of the entity tile the finished accumulators belong to
-  float m_S = 0.f, m_L1 = 0.f, m_iS = 0.f;
+  float m_S = 0.f, m_E2 = 0.f, m_R2 = 0.f, m_iS = 0.f;
   bool m_force = false;  // the same for the whole wave
   int64_t e_prev = r_end;
   auto tile_meta = [&](int buf, int et) {
     const f32x4 tc = *(const f32x4*)&meta_lds[buf][16 * et];
-    m_S = tc[0];
-    m_L1 = tc[1];
-    m_force = __builtin_amdgcn_readfirstlane(__float_as_uint(tc[2])) != 0u;
+    m_S = __builtin_fabsf(tc[0]);
+    m_E2 = tc[1];
+    m_R2 = tc[2];
+    m_force = (int)__builtin_amdgcn_readfirstlane(__float_as_uint(tc[0])) < 0;  // the sign of S: a forced tile
     m_iS = tc[3];
   };
   const TfSink sink{bucket, bcnt, ea.cnt, ea.cand, ea.cap, (int32_t)q_wg, (uint32_t)r_end};
@@ -365,23 +417,23 @@ __global__ void __launch_bounds__(64 * TF_W, 2) topk_i8_filter_kernel(ContractAr
     int hm = h[0];
 #pragma unroll
     for (int i = 1; i < 16; ++i) hm = hm > h[i] ? hm : h[i];
-    const float slack = __builtin_fmaf(mq[t], m_L1, cq[t]);
+    const float slack = __builtin_fmaf(mq[t], m_E2, __builtin_fmaf(m_R2, nq[t], cq[t]));
     const float Bd = m_S * __builtin_fmaf(sq[t], (float)hm, slack);
     const unsigned long long any = __builtin_amdgcn_ballot_w64(Bd > tau_lo[t]);
     if (__builtin_expect(any != 0 || m_force, 0)) {
       // The accumulators against the threshold as an integer: S (s_q H + slack) > tau  <=>  H > (tau / S - slack) / s_q,
       // lowered by its own rounding and kept inside +-2^30.
-      float x;
-      if (m_force)
+      // Where the bound does not depend on H (a tile of zero scales: 1 / S is stored as 0; a zero query: 1 / s_q is
+      // held as 0) every H of such a tile or query is 0 and the formula gives x <= -1 or NaN: everything passes, as
+      // it must when the bound has passed.  A NaN (0 times an infinite tau) falls to the lower clamp.
+      float x = (tau_lo[t] * m_iS - slack) * isq[t];
+      x = x - 1e-5f * __builtin_fabsf(x) - 1.f;
+      bool mine = Bd > tau_lo[t];
+      if (m_force) {  // the same for the whole wave
         x = (tau_lo[t] < INF) ? -INF : INF;
-      else if (m_S > 0.f && sq[t] > 0.f) {
-        x = (tau_lo[t] * m_iS - slack) * isq[t];
-        x = x - 1e-5f * __builtin_fabsf(x) - 1.f;
-      } else
-        x = (Bd > tau_lo[t]) ? -INF : INF;  // the bound does not depend on H
-      x = __builtin_fminf(__builtin_fmaxf(x, -1073741824.f), 1073741824.f);
-      const int thr = (x == x) ? (int)x : -1073741824;
-      const bool mine = (Bd > tau_lo[t]) || (m_force && tau_lo[t] < INF);
+        mine = tau_lo[t] < INF;
+      }
+      const int thr = (int)__builtin_fminf(__builtin_fmaxf(x, -1073741824.f), 1073741824.f);
       const unsigned long long who = __builtin_amdgcn_ballot_w64(mine);
       const int n_new = __builtin_popcountll(who);
       const int qlocal = ql0 + 32 * t + c;
@@ -395,12 +447,12 @@ __global__ void __launch_bounds__(64 * TF_W, 2) topk_i8_filter_kernel(ContractAr
         }
         if (mine) {
           const int at = qn + (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(who >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)who, 0u));
-          uint32_t* ent = wqueue + at * TF_QUEUE_STRIDE;
-#pragma unroll
-          for (int i = 0; i < 16; ++i) ent[i] = (uint32_t)h[i];
-          ent[16] = (uint32_t)thr;
-          ent[17] = (uint32_t)qlocal | ((uint32_t)hf << 16);
-          ent[18] = (uint32_t)e_prev;
+          i32x4* ent = (i32x4*)(wqueue + at * TF_QUEUE_STRIDE);
+          ent[0] = __builtin_shufflevector(h, h, 0, 1, 2, 3);
+          ent[1] = __builtin_shufflevector(h, h, 4, 5, 6, 7);
+          ent[2] = __builtin_shufflevector(h, h, 8, 9, 10, 11);
+          ent[3] = __builtin_shufflevector(h, h, 12, 13, 14, 15);
+          ent[4] = i32x4{thr, (int)((uint32_t)qlocal | ((uint32_t)hf << 16)), (int)(uint32_t)e_prev, 0};
         }
         qn += n_new;
       }

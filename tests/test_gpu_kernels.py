@@ -426,9 +426,10 @@ def test_topk_best_rows_first_defeats_the_guessed_threshold(ops, storage):
 def test_topk_int8_filter_scan_edge_cases(ops, N, B, k):
     """The int8 scan admits candidates by an integer bound and scores them exactly afterwards; whatever the bound
     lets through or not, the result must be the top k of the library's own scores.  Rows: scales spread over four
-    orders of magnitude, zero and negative scales, all-zero rows, rows of +-127; queries: zero, one-hot, a huge
-    dynamic range, one whose scores are all negative; N not a multiple of the 64-row stage, a partial last query
-    group."""
+    orders of magnitude, zero and negative scales, scales so small that their reciprocal overflows, all-zero rows,
+    rows of +-127; queries: zero, one-hot, a huge dynamic range, one whose scores are all negative, one of components
+    around 1e34 (beyond the range in which the bound's arithmetic stays finite: every row becomes a candidate), one
+    of components around 1e-36; N not a multiple of the 64-row stage, a partial last query group."""
     rng = np.random.default_rng(N + k)
     d = 128
     q8 = rng.integers(-127, 128, (N, d)).astype(np.int8)
@@ -439,6 +440,8 @@ def test_topk_int8_filter_scan_edge_cases(ops, N, B, k):
     sc[rng.integers(0, N, 200)] = 0.0
     neg = rng.integers(0, N, 200)
     sc[neg] = -sc[neg]
+    sc[rng.integers(0, N, 100)] = 1e-40                # 1 / scale is infinite in fp32
+    sc[N // 2 - 100:N // 2 + 100] = 2e-39              # whole tiles of them
     Q = (rng.standard_normal((B, d)) * 0.1).astype(np.float32)
     Q[0] = 0.0
     Q[1] = 0.0
@@ -446,6 +449,8 @@ def test_topk_int8_filter_scan_edge_cases(ops, N, B, k):
     Q[2] *= np.exp(rng.uniform(-12, 2, d)).astype(np.float32)
     base = np.abs(rng.standard_normal(d)).astype(np.float32)
     Q[3] = -base                                       # against rows made non-negative below: every score <= 0
+    Q[4] *= 2e35
+    Q[5] *= 1e-35
     Eg, scg, Qg = dev(torch.from_numpy(q8)), dev(torch.from_numpy(sc)), dev(torch.from_numpy(Q))
     vals, idx = ops.topk(Qg, None, Eg, scg, k)
     S = ops.scores(Qg, None, Eg, scg).cpu().numpy()
