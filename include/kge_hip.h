@@ -252,6 +252,9 @@ int kge_rank_filtered_static(const float* Q, const float* bias, const void* E, i
  * apply_sigmoid, the torch.sigmoid of KGE.predict_topk (:568), without writing B x N scores.
  *   out_scores [B,k] fp32 descending, out_idx [B,k] int64; equal scores are ordered by
  *   ascending entity id.  Requires 1 <= k <= min(N, 1024).
+ *   The order is that of the scores before the per-query bias is added (and before the sigmoid): two
+ *   entities whose scores become equal only through the rounding of score + bias, or of the sigmoid, keep
+ *   the order of their unbiased scores.
  * This call synchronises `stream` once before returning (it reads back one overflow counter).
  */
 size_t kge_topk_workspace_bytes(int64_t B, int64_t N, int64_t k);
