@@ -1075,3 +1075,117 @@ def test_shape_sweep_all_epilogues_agree_with_materialised_scores(ops, FilterCSR
     loss = ops.bce_multihot(Q, bias, Eg, scg, csr.rows_for(hr_g), csr.row_ptr, csr.col, 0.0)[0].item()
     want = ko.bce_multihot(S.cpu().numpy().astype(np.float64), pos)
     assert loss == pytest.approx(want, rel=1e-4, abs=1e-6)
+
+
+# ---------------------------------------------------------------------------------------------
+# random differential sweep: shapes, storages, table patterns, bias on and off, filter rows shared by queries
+# ---------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("seed", list(range(8)))
+def test_random_differential_sweep(ops, FilterCSR, seed):
+    """Thirty random cases per seed.  Filtered-rank counters, top-k (also through a prepared int8 table), row extrema
+    and single-entity scores must equal what follows from the library's own materialised scores, bit for bit: the
+    counters and the top-k order from the scores before the bias, ties towards the lower entity id.  Tables of
+    random rows, of small-integer rows (exact arithmetic: masses of ties), of rows drawn from a pool of one to 17,
+    and half-zero tables; queries that share a filter row and a vector; with and without a per-query bias."""
+    rng = np.random.default_rng(7000 + seed)
+    gen = torch.Generator(device="cuda").manual_seed(7000 + seed)
+    for case in range(30):
+        storage = ("fp32", "bf16", "int8")[case % 3]
+        B = int(rng.choice([1, 2, 31, 33, 64, 100, 257, 1000, 2500, 4097, 8193]))
+        if storage == "fp32":
+            d = int(rng.choice([1, 2, 5, 8, 16, 31, 32, 48, 64, 100, 128, 200, 256, 260]))
+        elif storage == "bf16":
+            d = int(rng.choice([8, 16, 40, 64, 72, 128, 136, 256, 384]))
+        else:
+            d = int(rng.choice([16, 32, 64, 128, 128, 128, 144, 256]))
+        N = int(rng.choice([1, 7, 64, 65, 1000, 4097, 20000, 70001] + ([150001] if case % 10 == 9 else [])))
+        if B * N > 1e8:
+            B = max(1, int(1e8 // N))
+        pattern = str(rng.choice(["randn", "randn", "ints", "pool", "half_zero"]))
+        with_bias = bool(rng.random() < 0.5)
+        label = f"seed {seed} case {case}: {storage} B={B} N={N} d={d} {pattern} bias={with_bias}"
+        print(label, flush=True)
+        if pattern == "ints":
+            E = torch.randint(-5, 6, (N, d), device="cuda", generator=gen).float() * 0.125
+            Q = torch.randint(-4, 5, (B, d), device="cuda", generator=gen).float() * 0.25
+        else:
+            Q = torch.randn(B, d, device="cuda", generator=gen) * 0.3
+            if pattern == "pool":
+                pool = torch.randn(int(rng.choice([1, 2, 17])), d, device="cuda", generator=gen)
+                E = pool[torch.randint(0, pool.shape[0], (N,), device="cuda", generator=gen)]
+            else:
+                E = torch.randn(N, d, device="cuda", generator=gen) * 0.3
+                if pattern == "half_zero":
+                    E[torch.rand(N, device="cuda", generator=gen) < 0.5] = 0
+        bias = torch.randn(B, device="cuda", generator=gen) if with_bias else None
+        sc = None
+        if storage == "bf16":
+            Et = E.to(torch.bfloat16).contiguous()
+        elif storage == "int8":
+            sc = (E.abs().amax(1) / 127).clamp_min(1e-12)
+            Et = torch.round(E / sc[:, None]).clamp(-127, 127).to(torch.int8).contiguous()
+            if rng.random() < 0.3:
+                sc = sc * torch.exp(torch.randn(N, device="cuda", generator=gen) * 2)
+        else:
+            Et = E.contiguous()
+        del E
+        R = 3
+        hr = torch.stack([torch.randint(0, N, (B,), device="cuda", generator=gen),
+                          torch.randint(0, R, (B,), device="cuda", generator=gen)], 1)
+        if rng.random() < 0.5 and B > 4:                                  # pairs of queries with one row and one vector
+            hr[B // 2:] = hr[:B - B // 2].clone()
+            Q[B // 2:] = Q[:B - B // 2].clone()
+        S_raw = ops.scores(Q, None, Et, sc)
+        S = ops.scores(Q, bias, Et, sc) if with_bias else S_raw
+        rows_all = torch.arange(B, device="cuda")
+        tgt = torch.randint(0, N, (B,), device="cuda", generator=gen)
+        # ---- filtered rank ----
+        per_query = int(rng.choice([0, 1, 5, 40]))
+        mask = torch.zeros((B, N), dtype=torch.bool, device="cuda")
+        if per_query == 0:
+            out = ops.rank_filtered(Q, bias, Et, sc, tgt)
+        else:
+            T = min(200000, B * per_query)
+            qi = torch.randint(0, B, (T,), device="cuda", generator=gen)
+            tails = torch.randint(0, N, (T,), device="cuda", generator=gen)
+            triples = torch.stack([hr[qi, 0], hr[qi, 1], tails], 1)
+            csr = FilterCSR.from_triples(triples.cpu().numpy(), R, device="cuda")
+            out = ops.rank_filtered(Q, bias, Et, sc, tgt, csr.rows_for(hr), csr.row_ptr, csr.col)
+            # every query whose (head, relation) pair equals the triple's is filtered by it
+            key_q = hr[:, 0] * R + hr[:, 1]
+            key_t = triples[:, 0] * R + triples[:, 1]
+            order = torch.argsort(key_q)
+            ks = key_q[order]
+            lo = torch.searchsorted(ks, key_t, right=False)
+            hi = torch.searchsorted(ks, key_t, right=True)
+            reps = hi - lo
+            t_idx = torch.repeat_interleave(torch.arange(T, device="cuda"), reps)
+            offs = torch.arange(int(reps.sum()), device="cuda") - torch.repeat_interleave(torch.cumsum(reps, 0) - reps, reps)
+            mask[order[lo[t_idx] + offs], tails[t_idx]] = True
+        mask[rows_all, tgt] = False                                      # the target itself always counts
+        thr = S_raw[rows_all, tgt][:, None]
+        keep = ~mask
+        eq = (S_raw == thr) & keep
+        assert torch.equal(out["n_greater"], ((S_raw > thr) & keep).sum(1).int()), label
+        assert torch.equal(out["n_equal"], eq.sum(1).int() - 1), label
+        assert torch.equal(out["n_equal_lower"], (eq & (torch.arange(N, device="cuda")[None, :] < tgt[:, None])).sum(1).int()), label
+        del mask, keep, eq
+        # ---- top-k ----
+        k = min(N, int(rng.choice([1, 3, 10, 100, 500, 1024])))
+        vals, idx = ops.topk(Q, bias, Et, sc, k)
+        key = S_raw.clone()
+        tv, ti = torch.sort(key, dim=1, descending=True, stable=True)
+        tv, ti = tv[:, :k], ti[:, :k]
+        if with_bias:
+            tv = tv + bias[:, None]
+        assert torch.equal(vals, tv), label
+        differ = idx != ti
+        assert bool((tv[differ] == (bias[:, None].expand_as(tv)[differ] if with_bias else 0)).all()), label  # -0 / +0 only
+        if storage == "int8" and d == 128:
+            v2, i2 = ops.topk(Q, bias, Et, sc, k, prepared=ops.topk_prepare(Et, sc))
+            assert torch.equal(v2, vals) and torch.equal(i2, idx), label
+        # ---- extrema, one entity per query ----
+        lo_, hi_ = ops.row_minmax(Q, bias, Et, sc)
+        assert torch.equal(lo_, S.min(1).values) and torch.equal(hi_, S.max(1).values), label
+        assert torch.equal(ops.triple_scores(Q, bias, Et, sc, tgt), S[rows_all, tgt]), label
+        del S, S_raw, key, tv, ti
