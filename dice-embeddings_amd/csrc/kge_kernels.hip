@@ -820,9 +820,12 @@ __global__ void __launch_bounds__(256) topk_rescore_kernel(TopkWs w, ContractArg
   }
 }
 
+// `packed` (LDS, or null): this round's candidates with the empty slots taken out, `nc` of them; otherwise the
+// candidates are read from the query's buffer as they lie.
 template <int KPL>
 __device__ __forceinline__ void select_in_registers(const TopkWs& w, int64_t b, int k, int rescan, int len, int nc,
-                                                    float tau_old, float th_used, int j_spec, int lane) {
+                                                    float tau_old, float th_used, int j_spec, int lane,
+                                                    const unsigned long long* packed = nullptr) {
   const unsigned long long kth_old = w.kth[b];  // (every lane reads it before lane 0 publishes the new one below)
   unsigned long long v[KPL];
 #pragma unroll
@@ -833,7 +836,7 @@ __device__ __forceinline__ void select_in_registers(const TopkWs& w, int64_t b, 
       key = w.list[b * w.kpad + i];
       if (rescan && key > kth_old) key = 0;
     } else if (i < len + nc) {
-      key = w.cand[b * TOPK_CAP + (i - len)];
+      key = packed ? packed[i - len] : w.cand[b * TOPK_CAP + (i - len)];
     }
     v[s] = key;
   }
@@ -864,7 +867,12 @@ __device__ __forceinline__ void select_in_registers(const TopkWs& w, int64_t b, 
 // Merge a query's kept list with this round's candidates, keep the best k, publish the new
 // threshold.  In `rescan` mode (only queries flagged dirty) list entries above the old threshold
 // are dropped first: the rescan finds all of them again.
-__global__ void __launch_bounds__(64) topk_select_wave_kernel(TopkWs w, int k, int rescan, int j_spec) {
+// `sparse`: the candidates come from the int8 filter scan, whose exact rescoring leaves a zero where a candidate did
+// not beat the threshold (most of them).  The keys that remain are packed in LDS first, so that the sorting network
+// is chosen by what there is to sort.
+constexpr int SELECT_PACKED = 512;  // packed candidates the one-wave selection keeps in LDS
+__global__ void __launch_bounds__(64) topk_select_wave_kernel(TopkWs w, int k, int rescan, int j_spec, int sparse) {
+  __shared__ unsigned long long packed[SELECT_PACKED];
   const int lane = threadIdx.x;
   const int64_t b = blockIdx.x;
   if (rescan && !w.dirty[b]) return;
@@ -873,15 +881,33 @@ __global__ void __launch_bounds__(64) topk_select_wave_kernel(TopkWs w, int k, i
   if (raw > TOPK_CAP || len + raw > SELECT_SMALL) return;  // left to topk_select_kernel
   const float tau_old = w.tau[b];
   const float th_used = rescan ? tau_old : w.tau_scan[b];
+  int nc = raw;
+  const unsigned long long* from = nullptr;
+  if (sparse && len + raw > 128) {
+    int n = 0;  // packed so far (the same in every lane)
+    for (int j0 = 0; j0 < raw; j0 += 64) {
+      const int j = j0 + lane;
+      const unsigned long long key = (j < raw) ? w.cand[b * TOPK_CAP + j] : 0ull;
+      const unsigned long long has = __builtin_amdgcn_ballot_w64(key != 0);
+      const int at = n + (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(has >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)has, 0u));
+      if (key != 0 && at < SELECT_PACKED) packed[at] = key;
+      n += __builtin_popcountll(has);
+    }
+    if (n <= SELECT_PACKED) {  // (more than that: sorted as they lie, zeros included)
+      nc = n;
+      from = packed;
+      __syncthreads();  // (one wave; the branch is the same for all of it)
+    }
+  }
   // (the network's cost grows faster than the number of keys: short lists, the usual case for small k, take a small one)
-  if (len + raw <= 128)
-    select_in_registers<2>(w, b, k, rescan, len, raw, tau_old, th_used, j_spec, lane);
-  else if (len + raw <= 256)
-    select_in_registers<4>(w, b, k, rescan, len, raw, tau_old, th_used, j_spec, lane);
-  else if (len + raw <= 512)
-    select_in_registers<8>(w, b, k, rescan, len, raw, tau_old, th_used, j_spec, lane);
+  if (len + nc <= 128)
+    select_in_registers<2>(w, b, k, rescan, len, nc, tau_old, th_used, j_spec, lane, from);
+  else if (len + nc <= 256)
+    select_in_registers<4>(w, b, k, rescan, len, nc, tau_old, th_used, j_spec, lane, from);
+  else if (len + nc <= 512)
+    select_in_registers<8>(w, b, k, rescan, len, nc, tau_old, th_used, j_spec, lane, from);
   else
-    select_in_registers<16>(w, b, k, rescan, len, raw, tau_old, th_used, j_spec, lane);
+    select_in_registers<16>(w, b, k, rescan, len, nc, tau_old, th_used, j_spec, lane, from);
 }
 
 __global__ void __launch_bounds__(256) topk_select_kernel(TopkWs w, int k, int rescan, int j_spec) {
@@ -1669,8 +1695,10 @@ int topk_impl(const char* who, const float* Q, const float* bias, const void* E,
     KGE_LAUNCH_CHECK("topk_i8_qprep_kernel");
   }
   // One scan of entity rows [e0, e1) with the thresholds `tau`, for all queries or those flagged in `active`.
+  bool scan_was_filter = false;  // the last scan went through the int8 filter: its candidate buffers hold zeros
   auto launch_scan = [&](int64_t e0, int64_t e1, const float* tau, const int32_t* active, int rescan,
                          const char* name) -> int {
+    scan_was_filter = false;
     ContractArgs a = make_args(Q, E, dtype, scale, B, d, N, e0, e1);
     if (e0 == 0 && !rescan) {
       // the first round: every row a candidate, written as dense keys (the candidate counts were set to match)
@@ -1693,6 +1721,7 @@ int topk_impl(const char* who, const float* Q, const float* bias, const void* E,
       return launch_contract<TopkEpi>(dtype, a, ea, st, name);
     }
     if (e1 <= e0) return KGE_OK;
+    scan_was_filter = true;
     // the filter's workgroups cover TF_WG_QUERIES queries, one workgroup per CU: the same walk, its own shape
     a.n_qgroups = (int)((B + TF_WG_QUERIES - 1) / TF_WG_QUERIES);
     a.n_lanes = 32 / a.n_qgroups;
@@ -1718,7 +1747,8 @@ int topk_impl(const char* who, const float* Q, const float* bias, const void* E,
   // ranks the list (<= k entries) and this round's candidates (<= min(TOPK_CAP, rows scanned) entries) of every
   // query; j_spec: the rank whose score the next scan may use as its threshold (k: the k-th best itself)
   auto launch_select = [&](int64_t rows, int rescan, int64_t j_spec) {
-    hipLaunchKernelGGL(topk_select_wave_kernel, dim3((unsigned)B), dim3(64), 0, st, ws, (int)k, rescan, (int)j_spec);
+    hipLaunchKernelGGL(topk_select_wave_kernel, dim3((unsigned)B), dim3(64), 0, st, ws, (int)k, rescan, (int)j_spec,
+                       scan_was_filter ? 1 : 0);
     if (k + (rows < TOPK_CAP ? rows : TOPK_CAP) > SELECT_SMALL)  // kpad (<= 1024) + TOPK_CAP, padded to a power of two
       hipLaunchKernelGGL(topk_select_kernel, dim3((unsigned)B), dim3(256), 8192 * sizeof(unsigned long long), st, ws,
                          (int)k, rescan, (int)j_spec);
