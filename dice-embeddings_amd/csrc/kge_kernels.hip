@@ -799,11 +799,30 @@ __global__ void __launch_bounds__(256) topk_rescore_kernel(TopkWs w, ContractArg
   const uint32_t* ids = w.cand_id + b * TOPK_CAP;
   unsigned long long* out = w.cand + b * TOPK_CAP;
   const int wid = blockIdx.y * 4 + (threadIdx.x >> 6), nw = gridDim.y * 4;
+  if (32 * wid >= nc) return;
+  // The query row as MFMA fragments, once per wave (d == 128 here: the filter scan exists for that width only):
+  // every tile multiplies the same row, and re-reading it per tile costs eight times the bytes of the gathered rows.
+  bf16x8 qfrag[8];
+#pragma unroll
+  for (int s = 0; s < 8; ++s) {
+    const f32x4* src = (const f32x4*)(a.Q + b * 128 + 16 * s + 8 * hf);
+    qfrag[s] = cvt_bf16x8(src[0], src[1]);
+  }
   for (int j0 = 32 * wid; j0 < nc; j0 += 32 * nw) {
     const int j = j0 + c;
     const int64_t e = (j < nc) ? (int64_t)ids[j] : -1;
     const bool ok = e >= 0 && e < a.N;
-    f32x16 acc = chain_direct<KGE_I8>(a.E, a.d, ok ? e : -1, a.Q, b, hf);
+    // the chain of chain_direct<KGE_I8> (K steps of 16 ascending, the row widened to bf16 exactly)
+    u32x2 wv[8];
+#pragma unroll
+    for (int s = 0; s < 8; ++s)
+      wv[s] = ok ? *(const u32x2*)((const int8_t*)a.E + e * 128 + 16 * s + 8 * hf) : u32x2{0u, 0u};
+    f32x16 acc;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[i] = 0.f;
+#pragma unroll
+    for (int s = 0; s < 8; ++s)
+      acc = mfma_bf16(__builtin_bit_cast(bf16x8, i8x8_to_bf16x8(wv[s][0], wv[s][1])), qfrag[s], acc);
     const int isel = ((c >> 3) << 2) | (c & 3);  // diagonal element (entity row c, query column c)
     float v = 0.f;
 #pragma unroll
