@@ -35,7 +35,7 @@ FP32_MFMA_PEAK_TFLOPS = 157.3
 # HBM bytes per launch of the main loop measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on the full-size
 # workload (each scaled by what the same counter reads for a plain 1 GiB copy kernel: x2.00 and x1.00).
 MEASURED_TRAFFIC_BYTES = {"c4": 688.0e6,     # per rank launch (678 MB read, 9 MB written)
-                          "c5": 350.0e6,     # average over the 4 filter scans of a top-k call (5.7 GB per call over all kernels)
+                          "c5": 350.0e6,     # average over the 4 filter scans of a top-k call (4.2 GB per call over all kernels)
                           "c3": 59.4e6, "c2": 19.4e6}
 MODE = {"c1": "rank", "c2": "rank", "c3": "bce", "c4": "rank", "c5": "topk"}
 
