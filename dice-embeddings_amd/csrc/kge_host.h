@@ -201,7 +201,8 @@ inline int64_t topk_speculative_rank(int64_t k, int64_t ranked, int64_t n_next) 
 // bf16: x4 3.00 ms, x8 3.04, x16 3.03).
 inline int64_t topk_growth(int64_t k) { return k <= 256 ? 4 : 2; }
 
-inline size_t bce_ws_bytes() { return (2 * BCE_SLOTS + 1) * sizeof(double) + 248; }
+constexpr int BCE_POS_SLOTS = 128;  // partial sums over the positives (one atomic per workgroup, spread)
+inline size_t bce_ws_bytes() { return (2 * BCE_SLOTS + BCE_POS_SLOTS) * sizeof(double) + 128; }
 
 struct BwdPlan {
   int64_t ldG, ldT;  // row strides of G [B, ldG] and GT [N, ldT] (multiples of 4)

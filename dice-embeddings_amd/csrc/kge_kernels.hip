@@ -1022,66 +1022,84 @@ __global__ void minmax_final_kernel(uint32_t* kmin, uint32_t* kmax, const float*
 }
 
 // ---- BCE helpers --------------------------------------------------------------------------------
-// accumulators: BCE_SLOTS partial sums of softplus(s), BCE_SLOTS of s, then the sum over the positives
+// accumulators: BCE_SLOTS partial sums of softplus(s), BCE_SLOTS of s, then BCE_POS_SLOTS of the sum over the positives
+using host::BCE_POS_SLOTS;
 __global__ void bce_init_kernel(double* sums) {
-  for (int i = threadIdx.x; i < 2 * BCE_SLOTS + 1; i += blockDim.x) sums[i] = 0.0;
+  for (int i = threadIdx.x; i < 2 * BCE_SLOTS + BCE_POS_SLOTS; i += blockDim.x) sums[i] = 0.0;
 }
 
-// sum of the logits of the positive (query, tail) pairs.  A workgroup strides over the queries; its four
-// waves take a row's positives in turn, the lanes of a wave split the embedding dimension.  One atomic per
-// workgroup at the end: thousands of double-precision atomics on one address would serialise.
+// sum of the logits of the positive (query, tail) pairs.  Grid (queries, BCE_POS_SPLIT): a workgroup is sixteen
+// groups of sixteen lanes, and positive j of a query's row goes to group j mod (16 * BCE_POS_SPLIT) of that query's
+// workgroups.  The usual row of one or two positives is a single chain of dependent loads (row -> extent -> tail ->
+// embedding row) that runs beside every other query's; a row of hundreds is shared out over 64 groups.  One atomic per
+// workgroup that found work, spread over a few addresses: thousands of double-precision atomics on one address
+// would serialise.
+constexpr int BCE_POS_SPLIT = 4;
 template <int EDT>
 __global__ void __launch_bounds__(256) bce_pos_kernel(ContractArgs a, const float* bias, const int64_t* csr_row,
                                                      const int64_t* row_ptr, const int32_t* col, int64_t n_rows,
                                                      double* sums) {
-  __shared__ double s_part[4];
-  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
-  double local = 0.0;  // every lane of a wave holds the same sum
-  for (int64_t q = blockIdx.x; q < a.B; q += gridDim.x) {
-    const int64_t row = csr_row[q];
-    if (row < 0 || row >= n_rows) continue;
-    const float bq = bias ? bias[q] : 0.f;
-    const float* qv = a.Q + q * a.d;
-    for (int64_t j = row_ptr[row] + wave; j < row_ptr[row + 1]; j += 4) {
-      const int64_t e = col[j];
-      if (e < 0 || e >= a.N) continue;  // uniform across the wave
-      float dot = 0.f;
-      for (int k = lane; k < a.d; k += 64) {
-        float x;
-        float qk = qv[k];
-        if (EDT == KGE_F32) {
-          x = ((const float*)a.E)[e * a.d + k];
-        } else {
-          qk = (float)(__bf16)qk;
-          if (EDT == KGE_BF16)
-            x = __uint_as_float((uint32_t)((const uint16_t*)a.E)[e * a.d + k] << 16);
-          else
-            x = (float)((const int8_t*)a.E)[e * a.d + k];
-        }
-        dot = fmaf(qk, x, dot);
+  __shared__ double s_part[16];
+  const int tid = threadIdx.x, grp = tid >> 4, sub = tid & 15;
+  const int64_t q = blockIdx.x;
+  const int64_t row = csr_row[q];
+  if (row < 0 || row >= n_rows) return;
+  const int64_t j0 = row_ptr[row], j1 = row_ptr[row + 1];
+  const int slot = (int)blockIdx.y * 16 + grp;
+  if (j0 + (int64_t)blockIdx.y * 16 >= j1) return;  // nothing for this workgroup (the same for all of it)
+  const float bq = bias ? bias[q] : 0.f;
+  const float* qv = a.Q + q * a.d;
+  double local = 0.0;  // every lane of a group holds the same sum
+  for (int64_t j = j0 + slot; j < j1; j += 16 * BCE_POS_SPLIT) {
+    const int64_t e = col[j];
+    if (e < 0 || e >= a.N) continue;  // uniform across the group
+    float dot = 0.f;
+    for (int k = sub; k < a.d; k += 16) {
+      float x;
+      float qk = qv[k];
+      if (EDT == KGE_F32) {
+        x = ((const float*)a.E)[e * a.d + k];
+      } else {
+        qk = (float)(__bf16)qk;
+        if (EDT == KGE_BF16)
+          x = __uint_as_float((uint32_t)((const uint16_t*)a.E)[e * a.d + k] << 16);
+        else
+          x = (float)((const int8_t*)a.E)[e * a.d + k];
       }
-#pragma unroll
-      for (int o = 32; o >= 1; o >>= 1) dot += __shfl_xor(dot, o, 64);
-      if (EDT == KGE_I8) dot *= a.scale[e];
-      local += (double)(dot + bq);
+      dot = fmaf(qk, x, dot);
     }
+#pragma unroll
+    for (int o = 8; o >= 1; o >>= 1) dot += __shfl_xor(dot, o, 64);
+    if (EDT == KGE_I8) dot *= a.scale[e];
+    local += (double)(dot + bq);
   }
-  if (lane == 0) s_part[wave] = local;
+  if (sub == 0) s_part[grp] = local;
   __syncthreads();
   if (tid == 0) {
-    const double t = s_part[0] + s_part[1] + s_part[2] + s_part[3];
-    if (t != 0.0) atomicAdd(&sums[2 * BCE_SLOTS], t);
+    double t = 0.0;
+#pragma unroll
+    for (int g = 0; g < 16; ++g) t += s_part[g];
+    if (t != 0.0) atomicAdd(&sums[2 * BCE_SLOTS + ((blockIdx.x + blockIdx.y) & (BCE_POS_SLOTS - 1))], t);
   }
 }
 
+// one wave: the partial sums are read side by side (one thread reading 384 doubles in turn is a chain of its own)
 __global__ void bce_final_kernel(const double* sums, double B, double N, float eps, float* loss) {
-  if (threadIdx.x == 0 && blockIdx.x == 0) {
-    double t = 0.0, s = 0.0;
-    for (int i = 0; i < BCE_SLOTS; ++i) {
-      t += sums[i];
-      s += sums[BCE_SLOTS + i];
-    }
-    const double pos = sums[2 * BCE_SLOTS];
+  const int lane = threadIdx.x;
+  if (blockIdx.x != 0 || lane >= 64) return;
+  double t = 0.0, s = 0.0, pos = 0.0;
+  for (int i = lane; i < BCE_SLOTS; i += 64) {
+    t += sums[i];
+    s += sums[BCE_SLOTS + i];
+  }
+  for (int i = lane; i < BCE_POS_SLOTS; i += 64) pos += sums[2 * BCE_SLOTS + i];
+#pragma unroll
+  for (int o = 32; o >= 1; o >>= 1) {
+    t += __shfl_xor(t, o, 64);
+    s += __shfl_xor(s, o, 64);
+    pos += __shfl_xor(pos, o, 64);
+  }
+  if (lane == 0) {
     if (eps != 0.f)
       t -= (1.0 - (double)eps) * pos + s / N;
     else
@@ -1853,7 +1871,7 @@ extern "C" int kge_bce_multihot(const float* Q, const float* bias, const void* E
   rc = launch_contract<BceEpi>(dtype, a, ea, st, "kge_bce_multihot");
   if (rc) return rc;
   if (csr_row && n_rows > 0) {
-    dim3 grid((unsigned)(B < 512 ? B : 512)), block(256);
+    dim3 grid((unsigned)B, BCE_POS_SPLIT), block(256);
     KGE_DISPATCH_DTYPE(dtype, bce_pos_kernel, grid, block, 0, st, a, bias, csr_row, row_ptr, col, n_rows, sums);
     KGE_LAUNCH_CHECK("bce_pos_kernel");
   }
@@ -1917,7 +1935,8 @@ extern "C" int kge_bce_multihot_backward(const float* Q, const float* bias, cons
   if (csr_row && n_rows > 0) {
     dim3 grid((unsigned)(B < 512 ? B : 512)), block(256);
     if (loss) {
-      hipLaunchKernelGGL((bce_pos_kernel<KGE_F32>), grid, block, 0, st, a, bias, csr_row, row_ptr, col, n_rows, sums);
+      hipLaunchKernelGGL((bce_pos_kernel<KGE_F32>), dim3((unsigned)B, BCE_POS_SPLIT), block, 0, st, a, bias, csr_row,
+                         row_ptr, col, n_rows, sums);
       KGE_LAUNCH_CHECK("bce_pos_kernel");
     }
     const float pos = (label_smoothing != 0.f ? 1.0f - label_smoothing : 1.0f) * inv_bn;
