@@ -1172,10 +1172,15 @@ constexpr int QS_NBUF = 3;
 // issue slots of its 32 cycles; about 42 epilogue instructions per 8 MFMAs: five per MFMA measured best of 4..8)
 constexpr int QS_VALU_PER_MFMA = 5;
 
-template <template <int> class EpiT, int NQT, int W, int OCC>
+// KSTEPS: K steps of 16 per score (8: d == 128; 16: d == 256, rows of 512 bytes, one query tile per wave).
+template <template <int> class EpiT, int NQT, int W, int OCC, int KSTEPS = 8>
 __global__ void __launch_bounds__(64 * W, OCC) qstream_kernel(ContractArgs a, typename EpiT<NQT>::Args ea) {
   using Epi = EpiT<NQT>;
-  __shared__ __attribute__((aligned(1024))) unsigned char lds_e[QS_NBUF * QS_STAGE_BYTES];
+  constexpr int d = 16 * KSTEPS;
+  constexpr int ROW_BYTES = 2 * d;                      // a bf16 row
+  constexpr int STAGE_BYTES = QS_STAGE_ROWS * ROW_BYTES;
+  constexpr int TILE_BYTES = 32 * ROW_BYTES;            // one 32-row entity tile of a stage
+  __shared__ __attribute__((aligned(1024))) unsigned char lds_e[QS_NBUF * STAGE_BYTES];
 
   const int64_t wg = blockIdx.x;
   const int xcd = (int)(wg & 7);
@@ -1184,7 +1189,6 @@ __global__ void __launch_bounds__(64 * W, OCC) qstream_kernel(ContractArgs a, ty
   const int wlane = (int)(slot / a.n_qgroups);
   const int tid = threadIdx.x, lane = tid & 63, c = lane & 31, hf = lane >> 5;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  constexpr int d = 128;
   const int64_t q0 = (int64_t)qg * (W * 32 * NQT) + wave * (32 * NQT);
 
   // chunks of this workgroup: first, stride, count; stages that hold at least one valid row
@@ -1201,12 +1205,12 @@ __global__ void __launch_bounds__(64 * W, OCC) qstream_kernel(ContractArgs a, ty
   const int n_st = (my_chunks - 1) * spc + valid_last;
   const int64_t chunk_skip = (c_stride - 1) * (int64_t)a.chunk_rows;
 
-  bf16x8 qf[NQT][8];
+  bf16x8 qf[NQT][KSTEPS];
 #pragma unroll
   for (int t = 0; t < NQT; ++t) {
     const int64_t q = q0 + 32 * t + c;
 #pragma unroll
-    for (int s = 0; s < 8; ++s) {
+    for (int s = 0; s < KSTEPS; ++s) {
       const int k = 16 * s + 8 * hf;
       f32x4 lo = {0.f, 0.f, 0.f, 0.f}, hi = {0.f, 0.f, 0.f, 0.f};
       if (q < a.B) {
@@ -1225,30 +1229,32 @@ __global__ void __launch_bounds__(64 * W, OCC) qstream_kernel(ContractArgs a, ty
   // this lane's share of a stage: rows lrow + RPI * j, always the same swizzled piece (RPI is a multiple of 16).
   // A full stage is a scalar base plus per-lane offsets that never change; in the table's last, partial stage the
   // rows past the end repeat its last row (the epilogues ignore them).
-  constexpr int RPI = 4 * W;
+  constexpr int LPR = ROW_BYTES / 16;   // lanes (16-byte pieces) per row
+  constexpr int RPW = 64 / LPR;         // rows one wave-wide load instruction covers (1 KB)
+  constexpr int RPI = RPW * W;
   constexpr int NLD = QS_STAGE_ROWS / RPI;
   static_assert(RPI % 16 == 0 && QS_STAGE_ROWS % RPI == 0, "stage / workgroup shape");
-  const int lrow = wave * 4 + (lane >> 4);
-  const int lpiece = (lane & 15) ^ (lrow & 15);
+  const int lrow = wave * RPW + lane / LPR;
+  const int lpiece = (lane % LPR) ^ (lrow & 15);  // (the swizzle permutes the low four bits of the piece index)
   const unsigned char* Eb = (const unsigned char*)a.E;
   uint32_t voff[NLD];
 #pragma unroll
-  for (int j = 0; j < NLD; ++j) voff[j] = (uint32_t)((lrow + RPI * j) * 256 + lpiece * 16);
+  for (int j = 0; j < NLD; ++j) voff[j] = (uint32_t)((lrow + RPI * j) * ROW_BYTES + lpiece * 16);
   auto stage_issue = [&](int64_t row0, int buf) {
-    unsigned char* dst = lds_e + buf * QS_STAGE_BYTES + wave * 1024;
+    unsigned char* dst = lds_e + buf * STAGE_BYTES + wave * 1024;
     if (__builtin_expect(row0 + QS_STAGE_ROWS <= r_end, 1)) {
-      const unsigned char* src = Eb + row0 * 256;  // wave-uniform
+      const unsigned char* src = Eb + row0 * ROW_BYTES;  // wave-uniform
 #pragma unroll
       for (int j = 0; j < NLD; ++j)
         __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src + voff[j]),
-                                         (__attribute__((address_space(3))) void*)(dst + j * (RPI * 256)), 16, 0, 0);
+                                         (__attribute__((address_space(3))) void*)(dst + j * (RPI * ROW_BYTES)), 16, 0, 0);
     } else {
 #pragma unroll
       for (int j = 0; j < NLD; ++j) {
         int64_t g = row0 + lrow + RPI * j;
         g = (g < r_end) ? g : r_end - 1;
-        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(Eb + g * 256 + lpiece * 16),
-                                         (__attribute__((address_space(3))) void*)(dst + j * (RPI * 256)), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(Eb + g * ROW_BYTES + lpiece * 16),
+                                         (__attribute__((address_space(3))) void*)(dst + j * (RPI * ROW_BYTES)), 16, 0, 0);
       }
     }
   };
@@ -1264,9 +1270,9 @@ __global__ void __launch_bounds__(64 * W, OCC) qstream_kernel(ContractArgs a, ty
   };
 
   // fragment addresses of this lane inside buffer 0 (row c of entity tile 0)
-  int foff[8];
+  int foff[KSTEPS];
 #pragma unroll
-  for (int s = 0; s < 8; ++s) foff[s] = c * 256 + (((2 * s + hf) ^ (c & 15)) << 4);
+  for (int s = 0; s < KSTEPS; ++s) foff[s] = c * ROW_BYTES + (((2 * s + hf) ^ (c & 15)) << 4);
 
   // the first epilogue has no tile to work on: e_prev past the limit says so to the branching epilogues, scores of
   // -inf (never greater than, never equal to a threshold) to the deferring one
@@ -1293,9 +1299,9 @@ __global__ void __launch_bounds__(64 * W, OCC) qstream_kernel(ContractArgs a, ty
   stage_issue(issue_row, 1);
   issue_advance();
   wg_barrier();
-  bf16x8 ef[8];
+  bf16x8 ef[KSTEPS];
 #pragma unroll
-  for (int s = 0; s < 8; ++s) ef[s] = *(const bf16x8*)(lds_e + foff[s]);
+  for (int s = 0; s < KSTEPS; ++s) ef[s] = *(const bf16x8*)(lds_e + foff[s]);
 
   int64_t row0 = row_first, prev_row0 = row_first;
   int so = 0;
@@ -1310,8 +1316,8 @@ __global__ void __launch_bounds__(64 * W, OCC) qstream_kernel(ContractArgs a, ty
 #pragma unroll
           for (int i = 0; i < 16; ++i) acc[i] = 0.f;
 #pragma unroll
-          for (int s = 0; s < 8; ++s) {
-            const bf16x8 f = *(const bf16x8*)(lds_e + BUF * QS_STAGE_BYTES + et * 8192 + foff[s]);
+          for (int s = 0; s < KSTEPS; ++s) {
+            const bf16x8 f = *(const bf16x8*)(lds_e + BUF * STAGE_BYTES + et * TILE_BYTES + foff[s]);
             acc = mfma_bf16(f, qf[t][s], acc);
           }
           epi.tile_slow(t, acc, rows0 + et * 32, r_end);
@@ -1344,7 +1350,7 @@ __global__ void __launch_bounds__(64 * W, OCC) qstream_kernel(ContractArgs a, ty
         if (k + 3 < n_st) issue_advance();
       }
       // where the next entity tile's fragments come from: the second tile of this stage, or the first of the next
-      const int roff = (et == 0) ? BUF * QS_STAGE_BYTES + 8192 : NEXT * QS_STAGE_BYTES;
+      const int roff = (et == 0) ? BUF * STAGE_BYTES + TILE_BYTES : NEXT * STAGE_BYTES;
 #pragma unroll
       for (int t = 0; t < NQT; ++t) {
         const int t_prev = (t + NQT - 1) % NQT;
@@ -1353,7 +1359,7 @@ __global__ void __launch_bounds__(64 * W, OCC) qstream_kernel(ContractArgs a, ty
 #pragma unroll
         for (int i = 0; i < 16; ++i) acc[i] = 0.f;
 #pragma unroll
-        for (int s = 0; s < 8; ++s) {
+        for (int s = 0; s < KSTEPS; ++s) {
           acc = Epi::SWAP ? mfma_bf16(qf[t][s], ef[s], acc) : mfma_bf16(ef[s], qf[t][s], acc);
           if (refill) ef[s] = *(const bf16x8*)(lds_e + roff + foff[s]);  // last use of fragment s: fetch its successor
         }
@@ -1365,7 +1371,7 @@ __global__ void __launch_bounds__(64 * W, OCC) qstream_kernel(ContractArgs a, ty
         // the order the scheduler is asked for: each MFMA of this chain, then a share of the previous tile's
         // epilogue, then (in a refilling chain) the read that replaces the fragment the MFMA consumed
 #pragma unroll
-        for (int s = 0; s < 8; ++s) {
+        for (int s = 0; s < KSTEPS; ++s) {
           __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
           __builtin_amdgcn_sched_group_barrier(0x002, QS_VALU_PER_MFMA, 0);
           if (refill) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);

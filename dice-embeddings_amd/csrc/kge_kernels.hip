@@ -1170,8 +1170,19 @@ int check_contract(const char* who, const float* Q, const void* E, int dtype, co
   return st.ok() ? KGE_OK : set_error(st.code, "%s", st.msg);
 }
 
+// `stream256` (asked for by the filtered rank and by kge_scores): bf16 rows of d == 256 go through the persistent
+// streaming kernel with one query tile per wave (256-query workgroups); the 16 query fragments of a 512-byte row still
+// fit the register file beside the 16 entity fragments.  The other epilogues of that width keep kchunk_kernel: the
+// streaming kernel runs the previous tile's epilogue inside the MFMA chain, which suits a short branch-free one (the
+// deferred rank count, a plain store: 2.0x and 1.5x faster) and not the branching or long ones (top-k and row
+// extrema 10 % slower, BCE twice as slow).
+constexpr int QS256_WG_QUERIES = QA_WG_WAVES * 32;
+template <template <int> class EpiT>
+constexpr bool stream256_epilogue() {
+  return std::is_same<EpiT<2>, RankEpi<2>>::value || std::is_same<EpiT<2>, StoreEpi<2>>::value;
+}
 ContractArgs make_args(const float* Q, const void* E, int dtype, const float* scale, int64_t B, int64_t d,
-                       int64_t N, int64_t e_begin, int64_t e_end) {
+                       int64_t N, int64_t e_begin, int64_t e_end, bool stream256 = false) {
   ContractArgs a;
   a.Q = Q;
   a.E = E;
@@ -1183,10 +1194,11 @@ ContractArgs make_args(const float* Q, const void* E, int dtype, const float* sc
   a.d = (int)d;
   a.ldq = a.lde = 0;
   a.k_split_len = 0;
-  const bool fast_bf16 = (dtype == KGE_BF16 && d == 128), fast_i8 = (dtype == KGE_I8 && d == 128);
-  const bool wide_bf16 = ((dtype == KGE_BF16 || dtype == KGE_I8) && d > 128);  // kchunk_kernel: the workgroup shape of the split kernel
-  const int wgq = (dtype == KGE_F32) ? KS_WG_QUERIES : fast_bf16 ? QA_WG_QUERIES : fast_i8 ? I8_WG_QUERIES
-                  : wide_bf16 ? KS_WG_QUERIES : QREG_WG_QUERIES;
+  stream256 = stream256 && dtype == KGE_BF16 && d == 256;
+  const bool fast_bf16 = (dtype == KGE_BF16 && d == 128) || stream256, fast_i8 = (dtype == KGE_I8 && d == 128);
+  const bool wide_bf16 = ((dtype == KGE_BF16 || dtype == KGE_I8) && d > 128) && !stream256;  // kchunk_kernel: the workgroup shape of the split kernel
+  const int wgq = (dtype == KGE_F32) ? KS_WG_QUERIES : stream256 ? QS256_WG_QUERIES : fast_bf16 ? QA_WG_QUERIES
+                  : fast_i8 ? I8_WG_QUERIES : wide_bf16 ? KS_WG_QUERIES : QREG_WG_QUERIES;
   a.n_qgroups = (int)((B + wgq - 1) / wgq);
   if (a.n_qgroups < 1) a.n_qgroups = 1;
   const int64_t rows = e_end - e_begin;
@@ -1269,11 +1281,12 @@ template <template <int> class EpiT, class EArgs>
 int launch_contract(int dtype, const ContractArgs& a, const EArgs& ea, hipStream_t st, const char* name) {
   if (a.B == 0 || a.e_end <= a.e_begin) return KGE_OK;
   const bool fast_i8 = (dtype == KGE_I8 && a.d == 128);
-  const bool persistent = (dtype == KGE_BF16 && a.d == 128) || fast_i8;
+  const bool stream256 = stream256_epilogue<EpiT>() && dtype == KGE_BF16 && a.d == 256;  // (planned so by make_args)
+  const bool persistent = (dtype == KGE_BF16 && a.d == 128) || fast_i8 || stream256;
   const int64_t nwg = persistent ? 8 * (int64_t)a.n_qgroups * a.n_lanes : contract_grid_wgs(a);
   KGE_REQUIRE(nwg <= 0x7fffffffLL, KGE_ERR_INVALID, "%s: grid of %lld workgroups too large", name, (long long)nwg);
   const bool f32_split = (dtype == KGE_F32);
-  const bool wide_bf16 = ((dtype == KGE_BF16 || dtype == KGE_I8) && a.d > 128);
+  const bool wide_bf16 = ((dtype == KGE_BF16 || dtype == KGE_I8) && a.d > 128) && !stream256;
   dim3 grid((unsigned)nwg), block(fast_i8 ? 64 * I8_WG_WAVES : persistent ? 64 * QA_WG_WAVES : (f32_split || wide_bf16) ? 512 : 256);
   LaunchTimer timer;
   if (int trc = timer.begin(st)) return trc;
@@ -1288,6 +1301,12 @@ int launch_contract(int dtype, const ContractArgs& a, const EArgs& ea, hipStream
       hipLaunchKernelGGL((qstream_kernel<RankFastEpi, QA_NQT, QA_WG_WAVES, QA_WAVES_PER_SIMD>), grid, block, 0, st, a, ea);
     else
       hipLaunchKernelGGL((qreg_async_kernel<EpiT>), grid, block, 0, st, a, ea);
+  }
+  else if (stream256) {
+    if constexpr (std::is_same<EpiT<2>, RankEpi<2>>::value)
+      hipLaunchKernelGGL((qstream_kernel<RankFastEpi, 1, QA_WG_WAVES, QA_WAVES_PER_SIMD, 16>), grid, block, 0, st, a, ea);
+    else if constexpr (stream256_epilogue<EpiT>())
+      hipLaunchKernelGGL((qstream_kernel<EpiT, 1, QA_WG_WAVES, QA_WAVES_PER_SIMD, 16>), grid, block, 0, st, a, ea);
   }
   else if (wide_bf16 && dtype == KGE_BF16)
     hipLaunchKernelGGL((kchunk_kernel<KGE_BF16, EpiT>), grid, block, 0, st, a, ea);
@@ -1409,7 +1428,7 @@ extern "C" int kge_scores(const float* Q, const float* bias, const void* E, int 
   if (B == 0) return KGE_OK;
   KGE_REQUIRE(S && ldS >= N, KGE_ERR_INVALID, "kge_scores: S is null or ldS=%lld < N=%lld", (long long)ldS,
               (long long)N);
-  ContractArgs a = make_args(Q, E, dtype, scale, B, d, N, 0, N);
+  ContractArgs a = make_args(Q, E, dtype, scale, B, d, N, 0, N, true);
   StoreArgs ea{S, bias, ldS, 0};
   return launch_contract<StoreEpi>(dtype, a, ea, (hipStream_t)stream, "kge_scores");
 }
@@ -1487,7 +1506,7 @@ int rank_filtered_launch(const char* who, const float* Q, const float* bias, con
                          int64_t B, int64_t d, int64_t N, const int64_t* target, const int64_t* csr_row,
                          const int64_t* row_ptr, const int32_t* col, int64_t n_rows, int32_t* n_greater, int32_t* n_equal,
                          int32_t* n_equal_lower, float* target_score, void* ws_base, hipStream_t st) {
-  ContractArgs a = make_args(Q, E, dtype, scale, B, d, N, 0, N);
+  ContractArgs a = make_args(Q, E, dtype, scale, B, d, N, 0, N, true);
   const bool filtered = csr_row != nullptr && n_rows > 0;
   RankWs ws;
   rank_ws_layout(B, ws_base, &ws);

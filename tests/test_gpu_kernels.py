@@ -132,7 +132,9 @@ SCORE_CASES = [
     ("QMult", 999, 5, 128, 130, "bf16", {}),
     ("DistMult", 5000, 7, 128, 600, "bf16", {}),
     ("ComplEx", 321, 7, 64, 40, "bf16", {}),
-    ("Keci", 1500, 6, 256, 300, "bf16", {"p": 0, "q": 1, "coeff_q": [1.0]}),      # d > 128: kchunk_kernel
+    ("Keci", 1500, 6, 256, 300, "bf16", {"p": 0, "q": 1, "coeff_q": [1.0]}),      # d = 256: the streaming kernel, 512-byte rows
+    ("DistMult", 9001, 5, 256, 700, "bf16", {}),     # the same over several stages per workgroup, partial last groups
+    ("DistMult", 500, 5, 384, 90, "bf16", {}),       # wider still: kchunk_kernel
     ("ComplEx", 700, 7, 200, 150, "bf16", {}),
     ("DistMult", 300, 5, 136, 70, "bf16", {}),
     ("DistMult", 777, 9, 128, 70, "int8", {}),
@@ -288,7 +290,7 @@ def test_rank_one_filter_row_shared_by_different_query_vectors(ops, FilterCSR, s
 
 
 @pytest.mark.parametrize("storage,d,N", [("bf16", 64, 4097), ("fp32", 1, 1000), ("fp32", 32, 3001), ("bf16", 128, 5000),
-                                         ("int8", 128, 2500), ("bf16", 256, 1300)])
+                                         ("int8", 128, 2500), ("bf16", 256, 1300), ("bf16", 256, 40000)])
 def test_rank_partial_last_query_group_with_a_bias(ops, FilterCSR, storage, d, N):
     """B = 2500 leaves the last query group of every main loop partly filled (256-, 512- and 128-query groups), and
     the per-query bias is non-zero: ranks compare un-biased scores, target_score carries the bias."""
