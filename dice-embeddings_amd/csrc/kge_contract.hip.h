@@ -33,6 +33,7 @@ struct ContractArgs {
   // workgroup sums (0: all of d; otherwise a multiple of 32, and blockIdx.y selects the range)
   int ldq, lde;
   int k_split_len;
+  int persistent;  // host side: the decomposition above is that of a persistent kernel (checked at launch)
 };
 
 __device__ __forceinline__ f32x16 mfma_bf16(bf16x8 a, bf16x8 b, f32x16 c) {
@@ -1172,7 +1173,7 @@ constexpr int QS_NBUF = 3;
 // issue slots of its 32 cycles; about 42 epilogue instructions per 8 MFMAs: five per MFMA measured best of 4..8)
 constexpr int QS_VALU_PER_MFMA = 5;
 
-// KSTEPS: K steps of 16 per score (8: d == 128; 16: d == 256, rows of 512 bytes, one query tile per wave).
+// KSTEPS: K steps of 16 per score (8: d == 128; 16: d == 256, rows of 512 bytes, one query tile per wave; 4: d == 64).
 template <template <int> class EpiT, int NQT, int W, int OCC, int KSTEPS = 8>
 __global__ void __launch_bounds__(64 * W, OCC) qstream_kernel(ContractArgs a, typename EpiT<NQT>::Args ea) {
   using Epi = EpiT<NQT>;
@@ -1234,8 +1235,10 @@ __global__ void __launch_bounds__(64 * W, OCC) qstream_kernel(ContractArgs a, ty
   constexpr int RPI = RPW * W;
   constexpr int NLD = QS_STAGE_ROWS / RPI;
   static_assert(RPI % 16 == 0 && QS_STAGE_ROWS % RPI == 0, "stage / workgroup shape");
+  constexpr int SWZ = LPR < 16 ? LPR - 1 : 15;  // the swizzle permutes the low four bits of the piece index (all of
+                                                // them in a row of fewer than sixteen pieces)
   const int lrow = wave * RPW + lane / LPR;
-  const int lpiece = (lane % LPR) ^ (lrow & 15);  // (the swizzle permutes the low four bits of the piece index)
+  const int lpiece = (lane % LPR) ^ (lrow & SWZ);
   const unsigned char* Eb = (const unsigned char*)a.E;
   uint32_t voff[NLD];
 #pragma unroll
@@ -1272,7 +1275,7 @@ __global__ void __launch_bounds__(64 * W, OCC) qstream_kernel(ContractArgs a, ty
   // fragment addresses of this lane inside buffer 0 (row c of entity tile 0)
   int foff[KSTEPS];
 #pragma unroll
-  for (int s = 0; s < KSTEPS; ++s) foff[s] = c * ROW_BYTES + (((2 * s + hf) ^ (c & 15)) << 4);
+  for (int s = 0; s < KSTEPS; ++s) foff[s] = c * ROW_BYTES + (((2 * s + hf) ^ (c & SWZ)) << 4);
 
   // the first epilogue has no tile to work on: e_prev past the limit says so to the branching epilogues, scores of
   // -inf (never greater than, never equal to a threshold) to the deferring one

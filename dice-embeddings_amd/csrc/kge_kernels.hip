@@ -1182,7 +1182,7 @@ constexpr bool stream256_epilogue() {
   return std::is_same<EpiT<2>, RankEpi<2>>::value || std::is_same<EpiT<2>, StoreEpi<2>>::value;
 }
 ContractArgs make_args(const float* Q, const void* E, int dtype, const float* scale, int64_t B, int64_t d,
-                       int64_t N, int64_t e_begin, int64_t e_end, bool stream256 = false) {
+                       int64_t N, int64_t e_begin, int64_t e_end, bool stream256 = false, bool stream64 = false) {
   ContractArgs a;
   a.Q = Q;
   a.E = E;
@@ -1194,8 +1194,10 @@ ContractArgs make_args(const float* Q, const void* E, int dtype, const float* sc
   a.d = (int)d;
   a.ldq = a.lde = 0;
   a.k_split_len = 0;
+  a.persistent = 0;
+  stream64 = stream64 && dtype == KGE_BF16 && d == 64;  // (the rank only; the d == 128 workgroup shape)
   stream256 = stream256 && dtype == KGE_BF16 && d == 256;
-  const bool fast_bf16 = (dtype == KGE_BF16 && d == 128) || stream256, fast_i8 = (dtype == KGE_I8 && d == 128);
+  const bool fast_bf16 = (dtype == KGE_BF16 && d == 128) || stream256 || stream64, fast_i8 = (dtype == KGE_I8 && d == 128);
   const bool wide_bf16 = ((dtype == KGE_BF16 || dtype == KGE_I8) && d > 128) && !stream256;  // kchunk_kernel: the workgroup shape of the split kernel
   const int wgq = (dtype == KGE_F32) ? KS_WG_QUERIES : stream256 ? QS256_WG_QUERIES : fast_bf16 ? QA_WG_QUERIES
                   : fast_i8 ? I8_WG_QUERIES : wide_bf16 ? KS_WG_QUERIES : QREG_WG_QUERIES;
@@ -1214,6 +1216,7 @@ ContractArgs make_args(const float* Q, const void* E, int dtype, const float* sc
     if (chunk > 1024) chunk = 1024;
     a.chunk_rows = (int)chunk;
     a.n_chunks = (rows + chunk - 1) / chunk;
+    a.persistent = 1;
     return a;
   }
   // non-persistent paths: one workgroup per (query group, chunk).  `resident` workgroups run at a time
@@ -1282,7 +1285,11 @@ int launch_contract(int dtype, const ContractArgs& a, const EArgs& ea, hipStream
   if (a.B == 0 || a.e_end <= a.e_begin) return KGE_OK;
   const bool fast_i8 = (dtype == KGE_I8 && a.d == 128);
   const bool stream256 = stream256_epilogue<EpiT>() && dtype == KGE_BF16 && a.d == 256;  // (planned so by make_args)
-  const bool persistent = (dtype == KGE_BF16 && a.d == 128) || fast_i8 || stream256;
+  const bool stream64 = std::is_same<EpiT<2>, RankEpi<2>>::value && dtype == KGE_BF16 && a.d == 64;  // (the rank asks make_args for it)
+  const bool persistent = (dtype == KGE_BF16 && a.d == 128) || fast_i8 || stream256 || stream64;
+  // (which kernel a launch goes to depends on the epilogue as well as on the table; a plan made for the other kind
+  // of kernel would be read as garbage)
+  KGE_REQUIRE((a.persistent != 0) == persistent, KGE_ERR_INVALID, "%s: work decomposition planned for another kernel", name);
   const int64_t nwg = persistent ? 8 * (int64_t)a.n_qgroups * a.n_lanes : contract_grid_wgs(a);
   KGE_REQUIRE(nwg <= 0x7fffffffLL, KGE_ERR_INVALID, "%s: grid of %lld workgroups too large", name, (long long)nwg);
   const bool f32_split = (dtype == KGE_F32);
@@ -1301,6 +1308,10 @@ int launch_contract(int dtype, const ContractArgs& a, const EArgs& ea, hipStream
       hipLaunchKernelGGL((qstream_kernel<RankFastEpi, QA_NQT, QA_WG_WAVES, QA_WAVES_PER_SIMD>), grid, block, 0, st, a, ea);
     else
       hipLaunchKernelGGL((qreg_async_kernel<EpiT>), grid, block, 0, st, a, ea);
+  }
+  else if (stream64) {
+    if constexpr (std::is_same<EpiT<2>, RankEpi<2>>::value)
+      hipLaunchKernelGGL((qstream_kernel<RankFastEpi, QA_NQT, QA_WG_WAVES, QA_WAVES_PER_SIMD, 4>), grid, block, 0, st, a, ea);
   }
   else if (stream256) {
     if constexpr (std::is_same<EpiT<2>, RankEpi<2>>::value)
@@ -1506,7 +1517,7 @@ int rank_filtered_launch(const char* who, const float* Q, const float* bias, con
                          int64_t B, int64_t d, int64_t N, const int64_t* target, const int64_t* csr_row,
                          const int64_t* row_ptr, const int32_t* col, int64_t n_rows, int32_t* n_greater, int32_t* n_equal,
                          int32_t* n_equal_lower, float* target_score, void* ws_base, hipStream_t st) {
-  ContractArgs a = make_args(Q, E, dtype, scale, B, d, N, 0, N, true);
+  ContractArgs a = make_args(Q, E, dtype, scale, B, d, N, 0, N, true, true);
   const bool filtered = csr_row != nullptr && n_rows > 0;
   RankWs ws;
   rank_ws_layout(B, ws_base, &ws);
