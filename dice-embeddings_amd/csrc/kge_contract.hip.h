@@ -1426,13 +1426,19 @@ constexpr int I8_WG_WAVES = KGE_I8_WG_WAVES;
 constexpr int I8_WG_QUERIES = I8_WG_WAVES * 32 * QREG_NQT;
 constexpr int I8_WGS_PER_CU = 8 / I8_WG_WAVES;  // 2 waves per SIMD
 
-template <template <int> class EpiT>
-__global__ void __launch_bounds__(64 * I8_WG_WAVES, 2) qreg_i8_kernel(ContractArgs a, typename EpiT<QREG_NQT>::Args ea) {
-  using Epi = EpiT<QREG_NQT>;
-  __shared__ __attribute__((aligned(1024))) unsigned char lds_e[2 * QA_BUF_BYTES];
+// NQT query tiles per wave and KSTEPS K steps of 16 per score: (2, 8) for d == 128; (1, 16) for d == 256, whose rows are
+// 512 bytes of bf16 in LDS (64 KB per stage buffer) and whose queries still fit the register file one tile per wave.
+template <template <int> class EpiT, int NQT = QREG_NQT, int KSTEPS = 8>
+__global__ void __launch_bounds__(64 * I8_WG_WAVES, 2) qreg_i8_kernel(ContractArgs a, typename EpiT<NQT>::Args ea) {
+  using Epi = EpiT<NQT>;
+  constexpr int d = 16 * KSTEPS;
+  constexpr int ROW_BYTES = 2 * d;                      // a row widened to bf16
+  constexpr int BUF_BYTES = QA_STAGE_ROWS * ROW_BYTES;
+  constexpr int PPR = d / 16;                           // 16-byte pieces of int8 per row
+  __shared__ __attribute__((aligned(1024))) unsigned char lds_e[2 * BUF_BYTES];
   __shared__ __attribute__((aligned(16))) float lds_sc[2][QA_STAGE_ROWS];
   constexpr int NT = 64 * I8_WG_WAVES;
-  constexpr int NPIECE = QA_STAGE_ROWS * 8 / NT;  // 16-byte pieces of int8 a thread stages per stage
+  constexpr int NPIECE = QA_STAGE_ROWS * PPR / NT;  // 16-byte pieces of int8 a thread stages per stage
 
   const int64_t wg = blockIdx.x;
   const int xcd = (int)(wg & 7);
@@ -1441,8 +1447,7 @@ __global__ void __launch_bounds__(64 * I8_WG_WAVES, 2) qreg_i8_kernel(ContractAr
   const int wlane = (int)(slot / a.n_qgroups);
   const int tid = threadIdx.x, lane = tid & 63, c = lane & 31, hf = lane >> 5;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  constexpr int d = 128;
-  const int64_t q0 = (int64_t)qg * I8_WG_QUERIES + wave * (32 * QREG_NQT);
+  const int64_t q0 = (int64_t)qg * (I8_WG_WAVES * 32 * NQT) + wave * (32 * NQT);
 
   const int64_t c_first = xcd + 8 * (int64_t)wlane;
   const int64_t c_stride = 8 * (int64_t)a.n_lanes;
@@ -1456,12 +1461,12 @@ __global__ void __launch_bounds__(64 * I8_WG_WAVES, 2) qreg_i8_kernel(ContractAr
     return a.e_begin + (c_first + c_stride * ci) * a.chunk_rows + (int64_t)so * QA_STAGE_ROWS;
   };
 
-  bf16x8 qf[QREG_NQT][8];
+  bf16x8 qf[NQT][KSTEPS];
 #pragma unroll
-  for (int t = 0; t < QREG_NQT; ++t) {
+  for (int t = 0; t < NQT; ++t) {
     const int64_t q = q0 + 32 * t + c;
 #pragma unroll
-    for (int s = 0; s < 8; ++s) {
+    for (int s = 0; s < KSTEPS; ++s) {
       const int k = 16 * s + 8 * hf;
       f32x4 lo = {0.f, 0.f, 0.f, 0.f}, hi = {0.f, 0.f, 0.f, 0.f};
       if (q < a.B) {
@@ -1477,14 +1482,14 @@ __global__ void __launch_bounds__(64 * I8_WG_WAVES, 2) qreg_i8_kernel(ContractAr
   __shared__ typename Epi::Shared epi_sh;
   epi.bind(&epi_sh);
 
-  // staging: 128 rows x 128 B = 1024 pieces of 16 int8; thread handles pieces tid + NT j
+  // staging: 128 rows x d bytes in pieces of 16 int8; thread handles pieces tid + NT j
   u32x4 stage[NPIECE];
   float stage_sc = 0.f;
   const int8_t* Eb = (const int8_t*)a.E;
   auto stage_load = [&](int64_t row0) {
 #pragma unroll
     for (int j = 0; j < NPIECE; ++j) {
-      const int idx = tid + NT * j, row = idx >> 3, piece = idx & 7;
+      const int idx = tid + NT * j, row = idx / PPR, piece = idx % PPR;
       int64_t g = row0 + row;
       g = (g < r_end) ? g : r_end - 1;  // padding rows repeat the last valid row; epilogues ignore them
       stage[j] = *(const u32x4*)(Eb + g * d + piece * 16);
@@ -1496,20 +1501,20 @@ __global__ void __launch_bounds__(64 * I8_WG_WAVES, 2) qreg_i8_kernel(ContractAr
     }
   };
   auto stage_store = [&](int buf) {
-    unsigned char* base = lds_e + buf * QA_BUF_BYTES;
+    unsigned char* base = lds_e + buf * BUF_BYTES;
 #pragma unroll
     for (int j = 0; j < NPIECE; ++j) {
-      const int idx = tid + NT * j, row = idx >> 3, piece = idx & 7;
-      const int p0 = 2 * piece, sw = row & 15;
-      *(u32x4*)(base + row * 256 + ((p0 ^ sw) << 4)) = i8x8_to_bf16x8(stage[j][0], stage[j][1]);
-      *(u32x4*)(base + row * 256 + (((p0 + 1) ^ sw) << 4)) = i8x8_to_bf16x8(stage[j][2], stage[j][3]);
+      const int idx = tid + NT * j, row = idx / PPR, piece = idx % PPR;
+      const int p0 = 2 * piece, sw = row & 15;  // (the swizzle permutes the low four bits of the piece index)
+      *(u32x4*)(base + row * ROW_BYTES + ((p0 ^ sw) << 4)) = i8x8_to_bf16x8(stage[j][0], stage[j][1]);
+      *(u32x4*)(base + row * ROW_BYTES + (((p0 + 1) ^ sw) << 4)) = i8x8_to_bf16x8(stage[j][2], stage[j][3]);
     }
     if (tid < QA_STAGE_ROWS) lds_sc[buf][tid] = stage_sc;
   };
 
-  int foff[8];
+  int foff[KSTEPS];
 #pragma unroll
-  for (int s = 0; s < 8; ++s) foff[s] = c * 256 + (((2 * s + hf) ^ (c & 15)) << 4);
+  for (int s = 0; s < KSTEPS; ++s) foff[s] = c * ROW_BYTES + (((2 * s + hf) ^ (c & 15)) << 4);
 
   constexpr int ET = QA_STAGE_ROWS / 32;
   // A tile's epilogue runs right after its MFMA chain (deferring it under the next chain, as the bf16
@@ -1533,19 +1538,19 @@ __global__ void __launch_bounds__(64 * I8_WG_WAVES, 2) qreg_i8_kernel(ContractAr
     } else {
       row_next = r_end;
     }
-    const unsigned char* base = lds_e + buf * QA_BUF_BYTES;
+    const unsigned char* base = lds_e + buf * BUF_BYTES;
 #pragma unroll
     for (int et = 0; et < ET; ++et) {
-      bf16x8 ef[8];
+      bf16x8 ef[KSTEPS];
 #pragma unroll
-      for (int s = 0; s < 8; ++s) ef[s] = *(const bf16x8*)(base + et * 8192 + foff[s]);
+      for (int s = 0; s < KSTEPS; ++s) ef[s] = *(const bf16x8*)(base + et * (32 * ROW_BYTES) + foff[s]);
 #pragma unroll
-      for (int t = 0; t < QREG_NQT; ++t) {
+      for (int t = 0; t < NQT; ++t) {
         f32x16 acc;
 #pragma unroll
         for (int i = 0; i < 16; ++i) acc[i] = 0.f;
 #pragma unroll
-        for (int s = 0; s < 8; ++s)
+        for (int s = 0; s < KSTEPS; ++s)
           acc = Epi::SWAP ? mfma_bf16(qf[t][s], ef[s], acc) : mfma_bf16(ef[s], qf[t][s], acc);
         if (t == 0) {  // row scales of this entity tile: fetched under the first chain
           if (Epi::SWAP) {

@@ -1197,9 +1197,11 @@ ContractArgs make_args(const float* Q, const void* E, int dtype, const float* sc
   a.persistent = 0;
   stream64 = stream64 && dtype == KGE_BF16 && d == 64;  // (the rank only; the d == 128 workgroup shape)
   stream256 = stream256 && dtype == KGE_BF16 && d == 256;
-  const bool fast_bf16 = (dtype == KGE_BF16 && d == 128) || stream256 || stream64, fast_i8 = (dtype == KGE_I8 && d == 128);
-  const bool wide_bf16 = ((dtype == KGE_BF16 || dtype == KGE_I8) && d > 128) && !stream256;  // kchunk_kernel: the workgroup shape of the split kernel
-  const int wgq = (dtype == KGE_F32) ? KS_WG_QUERIES : stream256 ? QS256_WG_QUERIES : fast_bf16 ? QA_WG_QUERIES
+  const bool i8_256 = (dtype == KGE_I8 && d == 256);  // qreg_i8_kernel with one query tile per wave, every epilogue
+  const bool fast_bf16 = (dtype == KGE_BF16 && d == 128) || stream256 || stream64;
+  const bool fast_i8 = (dtype == KGE_I8 && d == 128) || i8_256;
+  const bool wide_bf16 = ((dtype == KGE_BF16 || dtype == KGE_I8) && d > 128) && !stream256 && !i8_256;  // kchunk_kernel: the workgroup shape of the split kernel
+  const int wgq = (dtype == KGE_F32) ? KS_WG_QUERIES : (stream256 || i8_256) ? QS256_WG_QUERIES : fast_bf16 ? QA_WG_QUERIES
                   : fast_i8 ? I8_WG_QUERIES : wide_bf16 ? KS_WG_QUERIES : QREG_WG_QUERIES;
   a.n_qgroups = (int)((B + wgq - 1) / wgq);
   if (a.n_qgroups < 1) a.n_qgroups = 1;
@@ -1283,7 +1285,8 @@ struct LaunchTimer {
 template <template <int> class EpiT, class EArgs>
 int launch_contract(int dtype, const ContractArgs& a, const EArgs& ea, hipStream_t st, const char* name) {
   if (a.B == 0 || a.e_end <= a.e_begin) return KGE_OK;
-  const bool fast_i8 = (dtype == KGE_I8 && a.d == 128);
+  const bool i8_256 = (dtype == KGE_I8 && a.d == 256);
+  const bool fast_i8 = (dtype == KGE_I8 && a.d == 128) || i8_256;
   const bool stream256 = stream256_epilogue<EpiT>() && dtype == KGE_BF16 && a.d == 256;  // (planned so by make_args)
   const bool stream64 = std::is_same<EpiT<2>, RankEpi<2>>::value && dtype == KGE_BF16 && a.d == 64;  // (the rank asks make_args for it)
   const bool persistent = (dtype == KGE_BF16 && a.d == 128) || fast_i8 || stream256 || stream64;
@@ -1293,7 +1296,7 @@ int launch_contract(int dtype, const ContractArgs& a, const EArgs& ea, hipStream
   const int64_t nwg = persistent ? 8 * (int64_t)a.n_qgroups * a.n_lanes : contract_grid_wgs(a);
   KGE_REQUIRE(nwg <= 0x7fffffffLL, KGE_ERR_INVALID, "%s: grid of %lld workgroups too large", name, (long long)nwg);
   const bool f32_split = (dtype == KGE_F32);
-  const bool wide_bf16 = ((dtype == KGE_BF16 || dtype == KGE_I8) && a.d > 128) && !stream256;
+  const bool wide_bf16 = ((dtype == KGE_BF16 || dtype == KGE_I8) && a.d > 128) && !stream256 && !i8_256;
   dim3 grid((unsigned)nwg), block(fast_i8 ? 64 * I8_WG_WAVES : persistent ? 64 * QA_WG_WAVES : (f32_split || wide_bf16) ? 512 : 256);
   LaunchTimer timer;
   if (int trc = timer.begin(st)) return trc;
@@ -1325,6 +1328,8 @@ int launch_contract(int dtype, const ContractArgs& a, const EArgs& ea, hipStream
     hipLaunchKernelGGL((kchunk_kernel<KGE_I8, EpiT>), grid, block, 0, st, a, ea);
   else if (dtype == KGE_BF16)
     hipLaunchKernelGGL((qreg_kernel<KGE_BF16, EpiT>), grid, block, 0, st, a, ea);
+  else if (i8_256)
+    hipLaunchKernelGGL((qreg_i8_kernel<EpiT, 1, 16>), grid, block, 0, st, a, ea);
   else if (fast_i8)
     hipLaunchKernelGGL((qreg_i8_kernel<EpiT>), grid, block, 0, st, a, ea);
   else
