@@ -1016,10 +1016,17 @@ constexpr int QA_BUF_BYTES = QA_STAGE_ROWS * 256;
 // xcd + 8 * (lane + n_lanes * i), i = 0, 1, ...  All query groups of a (xcd, lane) pair walk the same
 // chunks in the same order, so a chunk is pulled from HBM once and shared through that XCD's L2.
 // Stages run back to back across chunk boundaries (the prefetch never drains).
-template <template <int> class EpiT>
-__global__ void __launch_bounds__(64 * QA_WG_WAVES, QA_WAVES_PER_SIMD) qreg_async_kernel(ContractArgs a, typename EpiT<QA_NQT>::Args ea) {
-  using Epi = EpiT<QA_NQT>;
-  __shared__ __attribute__((aligned(1024))) unsigned char lds_e[2 * QA_BUF_BYTES];
+// NQT query tiles per wave and KSTEPS K steps of 16 per score: (QA_NQT, 8) for d == 128; (1, 16) for d == 256 (512-byte
+// rows, two 64 KB stage buffers, the next tile's fragments read straight into the registers of the current ones).
+template <template <int> class EpiT, int NQT = QA_NQT, int KSTEPS = 8>
+__global__ void __launch_bounds__(64 * QA_WG_WAVES, QA_WAVES_PER_SIMD) qreg_async_kernel(ContractArgs a, typename EpiT<NQT>::Args ea) {
+  using Epi = EpiT<NQT>;
+  constexpr int d = 16 * KSTEPS;
+  constexpr int ROW_BYTES = 2 * d;
+  constexpr int BUF_BYTES = QA_STAGE_ROWS * ROW_BYTES;
+  constexpr int TILE_BYTES = 32 * ROW_BYTES;
+  constexpr bool INPLACE = (KSTEPS > 8);  // no second set of fragment registers
+  __shared__ __attribute__((aligned(1024))) unsigned char lds_e[2 * BUF_BYTES];
 
   const int64_t wg = blockIdx.x;
   const int xcd = (int)(wg & 7);
@@ -1028,8 +1035,7 @@ __global__ void __launch_bounds__(64 * QA_WG_WAVES, QA_WAVES_PER_SIMD) qreg_asyn
   const int wlane = (int)(slot / a.n_qgroups);
   const int tid = threadIdx.x, lane = tid & 63, c = lane & 31, hf = lane >> 5;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  constexpr int d = 128;
-  const int64_t q0 = (int64_t)qg * QA_WG_QUERIES + wave * (32 * QA_NQT);
+  const int64_t q0 = (int64_t)qg * (QA_WG_WAVES * 32 * NQT) + wave * (32 * NQT);
 
   // chunks of this workgroup: first, stride, count
   const int64_t c_first = xcd + 8 * (int64_t)wlane;
@@ -1044,12 +1050,12 @@ __global__ void __launch_bounds__(64 * QA_WG_WAVES, QA_WAVES_PER_SIMD) qreg_asyn
     return a.e_begin + (c_first + c_stride * ci) * a.chunk_rows + (int64_t)so * QA_STAGE_ROWS;
   };
 
-  bf16x8 qf[QA_NQT][8];
+  bf16x8 qf[NQT][KSTEPS];
 #pragma unroll
-  for (int t = 0; t < QA_NQT; ++t) {
+  for (int t = 0; t < NQT; ++t) {
     const int64_t q = q0 + 32 * t + c;
 #pragma unroll
-    for (int s = 0; s < 8; ++s) {
+    for (int s = 0; s < KSTEPS; ++s) {
       const int k = 16 * s + 8 * hf;
       f32x4 lo = {0.f, 0.f, 0.f, 0.f}, hi = {0.f, 0.f, 0.f, 0.f};
       if (q < a.B) {
@@ -1066,34 +1072,37 @@ __global__ void __launch_bounds__(64 * QA_WG_WAVES, QA_WAVES_PER_SIMD) qreg_asyn
   epi.bind(&epi_sh);
 
   // this lane's share of a stage: rows lrow + RPI * j, always the same swizzled piece (RPI is a multiple of 16)
-  constexpr int RPI = 4 * QA_WG_WAVES;            // rows one workgroup-wide load instruction covers
+  constexpr int LPR = ROW_BYTES / 16;             // lanes (16-byte pieces) per row
+  constexpr int RPW = 64 / LPR;                   // rows one wave-wide load instruction covers (1 KB)
+  constexpr int RPI = RPW * QA_WG_WAVES;          // rows one workgroup-wide load instruction covers
   constexpr int NLD = QA_STAGE_ROWS / RPI;        // load instructions per lane per stage
-  const int lrow = wave * 4 + (lane >> 4);
-  const int lpiece = (lane & 15) ^ (lrow & 15);
+  static_assert(RPI % 16 == 0 && QA_STAGE_ROWS % RPI == 0 && LPR >= 16, "stage / workgroup shape");
+  const int lrow = wave * RPW + lane / LPR;
+  const int lpiece = (lane % LPR) ^ (lrow & 15);  // (the swizzle permutes the low four bits of the piece index)
   const unsigned char* Eb = (const unsigned char*)a.E;
   auto stage_issue = [&](int64_t row0, int buf) {
-    unsigned char* dst = lds_e + buf * QA_BUF_BYTES + wave * 1024;
+    unsigned char* dst = lds_e + buf * BUF_BYTES + wave * 1024;
     if (row0 + QA_STAGE_ROWS <= r_end) {
-      const unsigned char* src = Eb + (row0 + lrow) * 256 + lpiece * 16;
+      const unsigned char* src = Eb + (row0 + lrow) * ROW_BYTES + lpiece * 16;
 #pragma unroll
       for (int j = 0; j < NLD; ++j)
-        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src + j * (RPI * 256)),
-                                         (__attribute__((address_space(3))) void*)(dst + j * (RPI * 256)), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src + j * (RPI * ROW_BYTES)),
+                                         (__attribute__((address_space(3))) void*)(dst + j * (RPI * ROW_BYTES)), 16, 0, 0);
     } else {
 #pragma unroll
       for (int j = 0; j < NLD; ++j) {
         int64_t g = row0 + lrow + RPI * j;
         g = (g < r_end) ? g : r_end - 1;  // padding rows repeat the last valid row; the epilogue ignores them
-        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(Eb + g * 256 + lpiece * 16),
-                                         (__attribute__((address_space(3))) void*)(dst + j * (RPI * 256)), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(Eb + g * ROW_BYTES + lpiece * 16),
+                                         (__attribute__((address_space(3))) void*)(dst + j * (RPI * ROW_BYTES)), 16, 0, 0);
       }
     }
   };
 
   // fragment addresses of this lane inside a stage buffer (row c of e-tile 0)
-  int foff[8];
+  int foff[KSTEPS];
 #pragma unroll
-  for (int s = 0; s < 8; ++s) foff[s] = c * 256 + (((2 * s + hf) ^ (c & 15)) << 4);
+  for (int s = 0; s < KSTEPS; ++s) foff[s] = c * ROW_BYTES + (((2 * s + hf) ^ (c & 15)) << 4);
 
   constexpr int ET = QA_STAGE_ROWS / 32;
   f32x16 acc_prev;
@@ -1118,37 +1127,42 @@ __global__ void __launch_bounds__(64 * QA_WG_WAVES, QA_WAVES_PER_SIMD) qreg_asyn
       row_next = stage_row(st + 1);
       if (row_next < r_end) stage_issue(row_next, buf ^ 1);
     }
-    const unsigned char* base = lds_e + buf * QA_BUF_BYTES;
-    bf16x8 ef[8];
+    const unsigned char* base = lds_e + buf * BUF_BYTES;
+    bf16x8 ef[KSTEPS];
 #pragma unroll
-    for (int s = 0; s < 8; ++s) ef[s] = *(const bf16x8*)(base + foff[s]);
+    for (int s = 0; s < KSTEPS; ++s) ef[s] = *(const bf16x8*)(base + foff[s]);
 #pragma unroll
     for (int et = 0; et < ET; ++et) {
 #pragma unroll
-      for (int t = 0; t < QA_NQT; ++t) {
-        const int t_prev = (t + QA_NQT - 1) % QA_NQT;
-        const bool refill = (t == QA_NQT - 1) && (et + 1 < ET);
-        bf16x8 efn[8];
+      for (int t = 0; t < NQT; ++t) {
+        const int t_prev = (t + NQT - 1) % NQT;
+        const bool refill = (t == NQT - 1) && (et + 1 < ET);
+        bf16x8 efn[INPLACE ? 1 : KSTEPS];
         f32x16 acc;
 #pragma unroll
         for (int i = 0; i < 16; ++i) acc[i] = 0.f;
 #pragma unroll
-        for (int s = 0; s < 8; ++s) {
+        for (int s = 0; s < KSTEPS; ++s) {
           acc = Epi::SWAP ? mfma_bf16(qf[t][s], ef[s], acc) : mfma_bf16(ef[s], qf[t][s], acc);
           // last use of fragment s for this e-tile: fetch the next e-tile's fragment into its place
-          if (refill) efn[s] = *(const bf16x8*)(base + (et + 1) * 8192 + foff[s]);
+          if (refill) {
+            if constexpr (INPLACE) ef[s] = *(const bf16x8*)(base + (et + 1) * TILE_BYTES + foff[s]);
+            else efn[s] = *(const bf16x8*)(base + (et + 1) * TILE_BYTES + foff[s]);
+          }
         }
         epi.template tile<false>(t_prev, acc_prev, sc_dummy, 1.f, e_prev, r_end);
         if (refill) {
+          if constexpr (!INPLACE) {
 #pragma unroll
-          for (int s = 0; s < 8; ++s) ef[s] = efn[s];
+            for (int s = 0; s < KSTEPS; ++s) ef[s] = efn[s];
+          }
         }
         acc_prev = acc;
         e_prev = row0 + et * 32;
       }
     }
   }
-  epi.template tile<false>(QA_NQT - 1, acc_prev, sc_dummy, 1.f, e_prev, r_end);
+  epi.template tile<false>(NQT - 1, acc_prev, sc_dummy, 1.f, e_prev, r_end);
   epi.finish();
 }
 

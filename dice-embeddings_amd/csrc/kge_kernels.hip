@@ -1170,19 +1170,21 @@ int check_contract(const char* who, const float* Q, const void* E, int dtype, co
   return st.ok() ? KGE_OK : set_error(st.code, "%s", st.msg);
 }
 
-// `stream256` (asked for by the filtered rank and by kge_scores): bf16 rows of d == 256 go through the persistent
-// streaming kernel with one query tile per wave (256-query workgroups); the 16 query fragments of a 512-byte row still
-// fit the register file beside the 16 entity fragments.  The other epilogues of that width keep kchunk_kernel: the
-// streaming kernel runs the previous tile's epilogue inside the MFMA chain, which suits a short branch-free one (the
-// deferred rank count, a plain store: 2.0x and 1.5x faster) and not the branching or long ones (top-k and row
-// extrema 10 % slower, BCE twice as slow).
+// bf16 rows of d == 256 go through the persistent kernels with ONE query tile per wave (256-query workgroups): the 16
+// query fragments of a 512-byte row still fit the register file beside the 16 entity fragments.  The filtered rank
+// and kge_scores take the streaming kernel, which runs the previous tile's epilogue inside the MFMA chain and suits a
+// short branch-free one (the deferred rank count, a plain store: 2.0x and 1.5x faster than kchunk_kernel) and not
+// the branching or long ones (there top-k and row extrema are 10 % slower, BCE twice as slow); those take
+// qreg_async_kernel, epilogue after the chain.
+// `stream64` (asked for by the filtered rank only): bf16 rows of d == 64 through the streaming kernel as well, in
+// the d == 128 workgroup shape.
 constexpr int QS256_WG_QUERIES = QA_WG_WAVES * 32;
 template <template <int> class EpiT>
 constexpr bool stream256_epilogue() {
   return std::is_same<EpiT<2>, RankEpi<2>>::value || std::is_same<EpiT<2>, StoreEpi<2>>::value;
 }
 ContractArgs make_args(const float* Q, const void* E, int dtype, const float* scale, int64_t B, int64_t d,
-                       int64_t N, int64_t e_begin, int64_t e_end, bool stream256 = false, bool stream64 = false) {
+                       int64_t N, int64_t e_begin, int64_t e_end, bool stream64 = false) {
   ContractArgs a;
   a.Q = Q;
   a.E = E;
@@ -1195,8 +1197,8 @@ ContractArgs make_args(const float* Q, const void* E, int dtype, const float* sc
   a.ldq = a.lde = 0;
   a.k_split_len = 0;
   a.persistent = 0;
-  stream64 = stream64 && dtype == KGE_BF16 && d == 64;  // (the rank only; the d == 128 workgroup shape)
-  stream256 = stream256 && dtype == KGE_BF16 && d == 256;
+  stream64 = stream64 && dtype == KGE_BF16 && d == 64;
+  const bool stream256 = dtype == KGE_BF16 && d == 256;  // (persistent whatever the epilogue)
   const bool i8_256 = (dtype == KGE_I8 && d == 256);  // qreg_i8_kernel with one query tile per wave, every epilogue
   const bool fast_bf16 = (dtype == KGE_BF16 && d == 128) || stream256 || stream64;
   const bool fast_i8 = (dtype == KGE_I8 && d == 128) || i8_256;
@@ -1287,7 +1289,7 @@ int launch_contract(int dtype, const ContractArgs& a, const EArgs& ea, hipStream
   if (a.B == 0 || a.e_end <= a.e_begin) return KGE_OK;
   const bool i8_256 = (dtype == KGE_I8 && a.d == 256);
   const bool fast_i8 = (dtype == KGE_I8 && a.d == 128) || i8_256;
-  const bool stream256 = stream256_epilogue<EpiT>() && dtype == KGE_BF16 && a.d == 256;  // (planned so by make_args)
+  const bool stream256 = dtype == KGE_BF16 && a.d == 256;
   const bool stream64 = std::is_same<EpiT<2>, RankEpi<2>>::value && dtype == KGE_BF16 && a.d == 64;  // (the rank asks make_args for it)
   const bool persistent = (dtype == KGE_BF16 && a.d == 128) || fast_i8 || stream256 || stream64;
   // (which kernel a launch goes to depends on the epilogue as well as on the table; a plan made for the other kind
@@ -1321,6 +1323,8 @@ int launch_contract(int dtype, const ContractArgs& a, const EArgs& ea, hipStream
       hipLaunchKernelGGL((qstream_kernel<RankFastEpi, 1, QA_WG_WAVES, QA_WAVES_PER_SIMD, 16>), grid, block, 0, st, a, ea);
     else if constexpr (stream256_epilogue<EpiT>())
       hipLaunchKernelGGL((qstream_kernel<EpiT, 1, QA_WG_WAVES, QA_WAVES_PER_SIMD, 16>), grid, block, 0, st, a, ea);
+    else
+      hipLaunchKernelGGL((qreg_async_kernel<EpiT, 1, 16>), grid, block, 0, st, a, ea);
   }
   else if (wide_bf16 && dtype == KGE_BF16)
     hipLaunchKernelGGL((kchunk_kernel<KGE_BF16, EpiT>), grid, block, 0, st, a, ea);
@@ -1444,7 +1448,7 @@ extern "C" int kge_scores(const float* Q, const float* bias, const void* E, int 
   if (B == 0) return KGE_OK;
   KGE_REQUIRE(S && ldS >= N, KGE_ERR_INVALID, "kge_scores: S is null or ldS=%lld < N=%lld", (long long)ldS,
               (long long)N);
-  ContractArgs a = make_args(Q, E, dtype, scale, B, d, N, 0, N, true);
+  ContractArgs a = make_args(Q, E, dtype, scale, B, d, N, 0, N);
   StoreArgs ea{S, bias, ldS, 0};
   return launch_contract<StoreEpi>(dtype, a, ea, (hipStream_t)stream, "kge_scores");
 }
@@ -1522,7 +1526,7 @@ int rank_filtered_launch(const char* who, const float* Q, const float* bias, con
                          int64_t B, int64_t d, int64_t N, const int64_t* target, const int64_t* csr_row,
                          const int64_t* row_ptr, const int32_t* col, int64_t n_rows, int32_t* n_greater, int32_t* n_equal,
                          int32_t* n_equal_lower, float* target_score, void* ws_base, hipStream_t st) {
-  ContractArgs a = make_args(Q, E, dtype, scale, B, d, N, 0, N, true, true);
+  ContractArgs a = make_args(Q, E, dtype, scale, B, d, N, 0, N, true);
   const bool filtered = csr_row != nullptr && n_rows > 0;
   RankWs ws;
   rank_ws_layout(B, ws_base, &ws);
