@@ -1017,7 +1017,8 @@ constexpr int QA_BUF_BYTES = QA_STAGE_ROWS * 256;
 // chunks in the same order, so a chunk is pulled from HBM once and shared through that XCD's L2.
 // Stages run back to back across chunk boundaries (the prefetch never drains).
 // NQT query tiles per wave and KSTEPS K steps of 16 per score: (QA_NQT, 8) for d == 128; (1, 16) for d == 256 (512-byte
-// rows, two 64 KB stage buffers, the next tile's fragments read straight into the registers of the current ones).
+// rows, two 64 KB stage buffers, the next tile's fragments read straight into the registers of the current ones);
+// (QA_NQT, 4) for d == 64.
 template <template <int> class EpiT, int NQT = QA_NQT, int KSTEPS = 8>
 __global__ void __launch_bounds__(64 * QA_WG_WAVES, QA_WAVES_PER_SIMD) qreg_async_kernel(ContractArgs a, typename EpiT<NQT>::Args ea) {
   using Epi = EpiT<NQT>;
@@ -1076,9 +1077,11 @@ __global__ void __launch_bounds__(64 * QA_WG_WAVES, QA_WAVES_PER_SIMD) qreg_asyn
   constexpr int RPW = 64 / LPR;                   // rows one wave-wide load instruction covers (1 KB)
   constexpr int RPI = RPW * QA_WG_WAVES;          // rows one workgroup-wide load instruction covers
   constexpr int NLD = QA_STAGE_ROWS / RPI;        // load instructions per lane per stage
-  static_assert(RPI % 16 == 0 && QA_STAGE_ROWS % RPI == 0 && LPR >= 16, "stage / workgroup shape");
+  static_assert(RPI % 16 == 0 && QA_STAGE_ROWS % RPI == 0, "stage / workgroup shape");
+  constexpr int SWZ = LPR < 16 ? LPR - 1 : 15;  // the swizzle permutes the low four bits of the piece index (all of
+                                                // them in a row of fewer than sixteen pieces)
   const int lrow = wave * RPW + lane / LPR;
-  const int lpiece = (lane % LPR) ^ (lrow & 15);  // (the swizzle permutes the low four bits of the piece index)
+  const int lpiece = (lane % LPR) ^ (lrow & SWZ);
   const unsigned char* Eb = (const unsigned char*)a.E;
   auto stage_issue = [&](int64_t row0, int buf) {
     unsigned char* dst = lds_e + buf * BUF_BYTES + wave * 1024;
@@ -1102,7 +1105,7 @@ __global__ void __launch_bounds__(64 * QA_WG_WAVES, QA_WAVES_PER_SIMD) qreg_asyn
   // fragment addresses of this lane inside a stage buffer (row c of e-tile 0)
   int foff[KSTEPS];
 #pragma unroll
-  for (int s = 0; s < KSTEPS; ++s) foff[s] = c * ROW_BYTES + (((2 * s + hf) ^ (c & 15)) << 4);
+  for (int s = 0; s < KSTEPS; ++s) foff[s] = c * ROW_BYTES + (((2 * s + hf) ^ (c & SWZ)) << 4);
 
   constexpr int ET = QA_STAGE_ROWS / 32;
   f32x16 acc_prev;

@@ -1176,15 +1176,14 @@ int check_contract(const char* who, const float* Q, const void* E, int dtype, co
 // short branch-free one (the deferred rank count, a plain store: 2.0x and 1.5x faster than kchunk_kernel) and not
 // the branching or long ones (there top-k and row extrema are 10 % slower, BCE twice as slow); those take
 // qreg_async_kernel, epilogue after the chain.
-// `stream64` (asked for by the filtered rank only): bf16 rows of d == 64 through the streaming kernel as well, in
-// the d == 128 workgroup shape.
+// bf16 rows of d == 64 take the same two kernels in the d == 128 workgroup shape, with four K steps.
 constexpr int QS256_WG_QUERIES = QA_WG_WAVES * 32;
 template <template <int> class EpiT>
 constexpr bool stream256_epilogue() {
   return std::is_same<EpiT<2>, RankEpi<2>>::value || std::is_same<EpiT<2>, StoreEpi<2>>::value;
 }
 ContractArgs make_args(const float* Q, const void* E, int dtype, const float* scale, int64_t B, int64_t d,
-                       int64_t N, int64_t e_begin, int64_t e_end, bool stream64 = false) {
+                       int64_t N, int64_t e_begin, int64_t e_end) {
   ContractArgs a;
   a.Q = Q;
   a.E = E;
@@ -1197,7 +1196,7 @@ ContractArgs make_args(const float* Q, const void* E, int dtype, const float* sc
   a.ldq = a.lde = 0;
   a.k_split_len = 0;
   a.persistent = 0;
-  stream64 = stream64 && dtype == KGE_BF16 && d == 64;
+  const bool stream64 = dtype == KGE_BF16 && d == 64;  // (persistent whatever the epilogue)
   const bool stream256 = dtype == KGE_BF16 && d == 256;  // (persistent whatever the epilogue)
   const bool i8_256 = (dtype == KGE_I8 && d == 256);  // qreg_i8_kernel with one query tile per wave, every epilogue
   const bool fast_bf16 = (dtype == KGE_BF16 && d == 128) || stream256 || stream64;
@@ -1290,7 +1289,7 @@ int launch_contract(int dtype, const ContractArgs& a, const EArgs& ea, hipStream
   const bool i8_256 = (dtype == KGE_I8 && a.d == 256);
   const bool fast_i8 = (dtype == KGE_I8 && a.d == 128) || i8_256;
   const bool stream256 = dtype == KGE_BF16 && a.d == 256;
-  const bool stream64 = std::is_same<EpiT<2>, RankEpi<2>>::value && dtype == KGE_BF16 && a.d == 64;  // (the rank asks make_args for it)
+  const bool stream64 = dtype == KGE_BF16 && a.d == 64;
   const bool persistent = (dtype == KGE_BF16 && a.d == 128) || fast_i8 || stream256 || stream64;
   // (which kernel a launch goes to depends on the epilogue as well as on the table; a plan made for the other kind
   // of kernel would be read as garbage)
@@ -1317,6 +1316,8 @@ int launch_contract(int dtype, const ContractArgs& a, const EArgs& ea, hipStream
   else if (stream64) {
     if constexpr (std::is_same<EpiT<2>, RankEpi<2>>::value)
       hipLaunchKernelGGL((qstream_kernel<RankFastEpi, QA_NQT, QA_WG_WAVES, QA_WAVES_PER_SIMD, 4>), grid, block, 0, st, a, ea);
+    else
+      hipLaunchKernelGGL((qreg_async_kernel<EpiT, QA_NQT, 4>), grid, block, 0, st, a, ea);
   }
   else if (stream256) {
     if constexpr (std::is_same<EpiT<2>, RankEpi<2>>::value)
@@ -1526,7 +1527,7 @@ int rank_filtered_launch(const char* who, const float* Q, const float* bias, con
                          int64_t B, int64_t d, int64_t N, const int64_t* target, const int64_t* csr_row,
                          const int64_t* row_ptr, const int32_t* col, int64_t n_rows, int32_t* n_greater, int32_t* n_equal,
                          int32_t* n_equal_lower, float* target_score, void* ws_base, hipStream_t st) {
-  ContractArgs a = make_args(Q, E, dtype, scale, B, d, N, 0, N, true);
+  ContractArgs a = make_args(Q, E, dtype, scale, B, d, N, 0, N);
   const bool filtered = csr_row != nullptr && n_rows > 0;
   RankWs ws;
   rank_ws_layout(B, ws_base, &ws);
