@@ -1444,7 +1444,8 @@ constexpr int I8_WG_QUERIES = I8_WG_WAVES * 32 * QREG_NQT;
 constexpr int I8_WGS_PER_CU = 8 / I8_WG_WAVES;  // 2 waves per SIMD
 
 // NQT query tiles per wave and KSTEPS K steps of 16 per score: (2, 8) for d == 128; (1, 16) for d == 256, whose rows are
-// 512 bytes of bf16 in LDS (64 KB per stage buffer) and whose queries still fit the register file one tile per wave.
+// 512 bytes of bf16 in LDS (64 KB per stage buffer) and whose queries still fit the register file one tile per wave;
+// (2, 4) for d == 64.
 template <template <int> class EpiT, int NQT = QREG_NQT, int KSTEPS = 8>
 __global__ void __launch_bounds__(64 * I8_WG_WAVES, 2) qreg_i8_kernel(ContractArgs a, typename EpiT<NQT>::Args ea) {
   using Epi = EpiT<NQT>;
@@ -1452,6 +1453,7 @@ __global__ void __launch_bounds__(64 * I8_WG_WAVES, 2) qreg_i8_kernel(ContractAr
   constexpr int ROW_BYTES = 2 * d;                      // a row widened to bf16
   constexpr int BUF_BYTES = QA_STAGE_ROWS * ROW_BYTES;
   constexpr int PPR = d / 16;                           // 16-byte pieces of int8 per row
+  constexpr int SWZ = 2 * PPR < 16 ? 2 * PPR - 1 : 15;  // swizzled bits of the index of a row's 16-byte bf16 pieces
   __shared__ __attribute__((aligned(1024))) unsigned char lds_e[2 * BUF_BYTES];
   __shared__ __attribute__((aligned(16))) float lds_sc[2][QA_STAGE_ROWS];
   constexpr int NT = 64 * I8_WG_WAVES;
@@ -1522,7 +1524,7 @@ __global__ void __launch_bounds__(64 * I8_WG_WAVES, 2) qreg_i8_kernel(ContractAr
 #pragma unroll
     for (int j = 0; j < NPIECE; ++j) {
       const int idx = tid + NT * j, row = idx / PPR, piece = idx % PPR;
-      const int p0 = 2 * piece, sw = row & 15;  // (the swizzle permutes the low four bits of the piece index)
+      const int p0 = 2 * piece, sw = row & SWZ;  // (the swizzle permutes the low four bits of the piece index)
       *(u32x4*)(base + row * ROW_BYTES + ((p0 ^ sw) << 4)) = i8x8_to_bf16x8(stage[j][0], stage[j][1]);
       *(u32x4*)(base + row * ROW_BYTES + (((p0 + 1) ^ sw) << 4)) = i8x8_to_bf16x8(stage[j][2], stage[j][3]);
     }
@@ -1531,7 +1533,7 @@ __global__ void __launch_bounds__(64 * I8_WG_WAVES, 2) qreg_i8_kernel(ContractAr
 
   int foff[KSTEPS];
 #pragma unroll
-  for (int s = 0; s < KSTEPS; ++s) foff[s] = c * ROW_BYTES + (((2 * s + hf) ^ (c & 15)) << 4);
+  for (int s = 0; s < KSTEPS; ++s) foff[s] = c * ROW_BYTES + (((2 * s + hf) ^ (c & SWZ)) << 4);
 
   constexpr int ET = QA_STAGE_ROWS / 32;
   // A tile's epilogue runs right after its MFMA chain (deferring it under the next chain, as the bf16

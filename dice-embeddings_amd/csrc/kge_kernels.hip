@@ -1200,7 +1200,8 @@ ContractArgs make_args(const float* Q, const void* E, int dtype, const float* sc
   const bool stream256 = dtype == KGE_BF16 && d == 256;  // (persistent whatever the epilogue)
   const bool i8_256 = (dtype == KGE_I8 && d == 256);  // qreg_i8_kernel with one query tile per wave, every epilogue
   const bool fast_bf16 = (dtype == KGE_BF16 && d == 128) || stream256 || stream64;
-  const bool fast_i8 = (dtype == KGE_I8 && d == 128) || i8_256;
+  const bool i8_64 = (dtype == KGE_I8 && d == 64);    // the same kernel in the d == 128 shape with four K steps
+  const bool fast_i8 = (dtype == KGE_I8 && d == 128) || i8_256 || i8_64;
   const bool wide_bf16 = ((dtype == KGE_BF16 || dtype == KGE_I8) && d > 128) && !stream256 && !i8_256;  // kchunk_kernel: the workgroup shape of the split kernel
   const int wgq = (dtype == KGE_F32) ? KS_WG_QUERIES : (stream256 || i8_256) ? QS256_WG_QUERIES : fast_bf16 ? QA_WG_QUERIES
                   : fast_i8 ? I8_WG_QUERIES : wide_bf16 ? KS_WG_QUERIES : QREG_WG_QUERIES;
@@ -1287,7 +1288,8 @@ template <template <int> class EpiT, class EArgs>
 int launch_contract(int dtype, const ContractArgs& a, const EArgs& ea, hipStream_t st, const char* name) {
   if (a.B == 0 || a.e_end <= a.e_begin) return KGE_OK;
   const bool i8_256 = (dtype == KGE_I8 && a.d == 256);
-  const bool fast_i8 = (dtype == KGE_I8 && a.d == 128) || i8_256;
+  const bool i8_64 = (dtype == KGE_I8 && a.d == 64);
+  const bool fast_i8 = (dtype == KGE_I8 && a.d == 128) || i8_256 || i8_64;
   const bool stream256 = dtype == KGE_BF16 && a.d == 256;
   const bool stream64 = dtype == KGE_BF16 && a.d == 64;
   const bool persistent = (dtype == KGE_BF16 && a.d == 128) || fast_i8 || stream256 || stream64;
@@ -1335,6 +1337,8 @@ int launch_contract(int dtype, const ContractArgs& a, const EArgs& ea, hipStream
     hipLaunchKernelGGL((qreg_kernel<KGE_BF16, EpiT>), grid, block, 0, st, a, ea);
   else if (i8_256)
     hipLaunchKernelGGL((qreg_i8_kernel<EpiT, 1, 16>), grid, block, 0, st, a, ea);
+  else if (i8_64)
+    hipLaunchKernelGGL((qreg_i8_kernel<EpiT, QREG_NQT, 4>), grid, block, 0, st, a, ea);
   else if (fast_i8)
     hipLaunchKernelGGL((qreg_i8_kernel<EpiT>), grid, block, 0, st, a, ea);
   else
