@@ -168,16 +168,28 @@ struct StoreEpi {
     if (e >= limit) return;
     const int64_t qrow = q0 + 32 * qt + 4 * hf;  // query row of acc[0]; acc[4g + r] is row qrow + 8g + r
     float* p = a.S + qrow * a.ldS + e;
-    const bool full = q0 + 32 * qt + 32 <= B;
+    if (q0 + 32 * qt + 32 <= B) {  // the same for the wave: every query row of the tile exists (no test per element)
 #pragma unroll
-    for (int g = 0; g < 4; ++g) {
-      const f32x4 b4 = *(const f32x4*)(lb + 32 * qt + 8 * g + 4 * hf);
+      for (int g = 0; g < 4; ++g) {
+        const f32x4 b4 = *(const f32x4*)(lb + 32 * qt + 8 * g + 4 * hf);
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        float v = acc[4 * g + r];
-        if (HAS_SCALE) v *= sc_col;
-        v += b4[r];
-        if (full || qrow + 8 * g + r < B) p[(int64_t)(8 * g + r) * a.ldS] = v;
+        for (int r = 0; r < 4; ++r) {
+          float v = acc[4 * g + r];
+          if (HAS_SCALE) v *= sc_col;
+          p[(int64_t)(8 * g + r) * a.ldS] = v + b4[r];
+        }
+      }
+    } else {
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const f32x4 b4 = *(const f32x4*)(lb + 32 * qt + 8 * g + 4 * hf);
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          float v = acc[4 * g + r];
+          if (HAS_SCALE) v *= sc_col;
+          v += b4[r];
+          if (qrow + 8 * g + r < B) p[(int64_t)(8 * g + r) * a.ldS] = v;
+        }
       }
     }
   }
@@ -623,17 +635,29 @@ struct BceEpi {
     // the factors 1 + exp(-|s|) lie in (1, 2], their product stays below 2^16 and carries a relative error of at
     // most sixteen roundings, which after the logarithm is an absolute 1e-6 on a sum of order 10.
     float tpos = 0.f, tss = 0.f, prod = 1.f;
-    const bool whole = e_base + 32 <= limit;  // the same for the wave: no row of the tile is padding
+    if (e_base + 32 <= limit) {  // the same for the wave: no row of the tile is padding (one branch, no masks)
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      float s = acc[i];
-      if (HAS_SCALE) s *= sc16[i];
-      s += bias[qt];
-      const bool ok = whole || e_base + row_of(i, hf) < limit;
-      const float e = __expf(-fabsf(s));
-      prod = __builtin_fmaf(prod, ok ? e : 0.f, prod);  // prod * (1 + e) in one rounding
-      tpos += ok ? fmaxf(s, 0.f) : 0.f;
-      tss += ok ? s : 0.f;
+      for (int i = 0; i < 16; ++i) {
+        float s = acc[i];
+        if (HAS_SCALE) s *= sc16[i];
+        s += bias[qt];
+        const float e = __expf(-fabsf(s));
+        prod = __builtin_fmaf(prod, e, prod);  // prod * (1 + e) in one rounding
+        tpos += fmaxf(s, 0.f);
+        tss += s;
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        float s = acc[i];
+        if (HAS_SCALE) s *= sc16[i];
+        s += bias[qt];
+        const bool ok = e_base + row_of(i, hf) < limit;
+        const float e = __expf(-fabsf(s));
+        prod = __builtin_fmaf(prod, ok ? e : 0.f, prod);
+        tpos += ok ? fmaxf(s, 0.f) : 0.f;
+        tss += ok ? s : 0.f;
+      }
     }
     sp += (double)(tpos + __logf(prod));
     ss += (double)tss;
@@ -803,14 +827,24 @@ struct MinMaxEpi {
   template <bool HAS_SCALE>
   __device__ __forceinline__ void tile(int qt, const f32x16& acc, const float* sc16, float sc_col, int64_t e_base,
                                        int64_t limit) {
-    const bool full = e_base + 32 <= limit;  // uniform
+    const bool full = e_base + 32 <= limit;  // uniform: one branch per tile, not a 64-bit compare per element
     float l = lo[qt], h = hi[qt];
+    if (full) {
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      const float s = HAS_SCALE ? acc[i] * sc16[i] : acc[i];
-      if (full || e_base + row_of(i, hf) < limit) {
-        l = __builtin_fminf(l, s);
-        h = __builtin_fmaxf(h, s);
+      for (int i = 0; i < 16; i += 2) {
+        const float s0 = HAS_SCALE ? acc[i] * sc16[i] : acc[i];
+        const float s1 = HAS_SCALE ? acc[i + 1] * sc16[i + 1] : acc[i + 1];
+        l = __builtin_fminf(__builtin_fminf(l, s0), s1);
+        h = __builtin_fmaxf(__builtin_fmaxf(h, s0), s1);
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const float s = HAS_SCALE ? acc[i] * sc16[i] : acc[i];
+        if (e_base + row_of(i, hf) < limit) {
+          l = __builtin_fminf(l, s);
+          h = __builtin_fmaxf(h, s);
+        }
       }
     }
     lo[qt] = l;
