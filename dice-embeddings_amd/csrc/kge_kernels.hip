@@ -1293,8 +1293,8 @@ int launch_contract(int dtype, const ContractArgs& a, const EArgs& ea, hipStream
   const bool stream256 = dtype == KGE_BF16 && a.d == 256;
   const bool stream64 = dtype == KGE_BF16 && a.d == 64;
   const bool persistent = (dtype == KGE_BF16 && a.d == 128) || fast_i8 || stream256 || stream64;
-  // (which kernel a launch goes to depends on the epilogue as well as on the table; a plan made for the other kind
-  // of kernel would be read as garbage)
+  // (make_args and this function both decide, from the table, between the persistent and the tiled kernels; a plan
+  // made for the other kind would be read as garbage, so the two must not drift apart)
   KGE_REQUIRE((a.persistent != 0) == persistent, KGE_ERR_INVALID, "%s: work decomposition planned for another kernel", name);
   const int64_t nwg = persistent ? 8 * (int64_t)a.n_qgroups * a.n_lanes : contract_grid_wgs(a);
   KGE_REQUIRE(nwg <= 0x7fffffffLL, KGE_ERR_INVALID, "%s: grid of %lld workgroups too large", name, (long long)nwg);
