@@ -734,34 +734,52 @@ struct GradEpi {
     const int64_t qrow = q0 + 32 * qt + 4 * hf;  // query row of acc[0]; acc[4g + r] is row qrow + 8g + r
     float* pg = a.G + qrow * a.ldG + e;
     float* pt = a.GT + e * a.ldT + qrow;
-    const bool full = q0 + 32 * qt + 32 <= B;
+    const bool full = q0 + 32 * qt + 32 <= B;  // the same for the wave: one branch, no test per element
     float tpos = 0.f, tss = 0.f, prod = 1.f;  // one logarithm for the sixteen elements, as in BceEpi
+    if (full) {
 #pragma unroll
-    for (int g = 0; g < 4; ++g) {
-      const f32x4 b4 = *(const f32x4*)(lb + 32 * qt + 8 * g + 4 * hf);
-      f32x4 out;
+      for (int g = 0; g < 4; ++g) {
+        const f32x4 b4 = *(const f32x4*)(lb + 32 * qt + 8 * g + 4 * hf);
+        f32x4 out;
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        float v = acc[4 * g + r];
-        if (HAS_SCALE) v *= sc_col;
-        v += b4[r];
-        const bool ok = full || qrow + 8 * g + r < B;
-        const float ex = __expf(-fabsf(v));                       // in (0, 1]
-        const float sig = (v >= 0.f ? 1.0f : ex) / (1.0f + ex);    // sigmoid without overflow
-        const float gr = ok ? sig * a.inv_bn - a.uniform : 0.f;
-        prod = __builtin_fmaf(prod, ok ? ex : 0.f, prod);
-        tpos += ok ? fmaxf(v, 0.f) : 0.f;
-        tss += ok ? v : 0.f;
-        out[r] = gr;
-        rowsum[qt][4 * g + r] += gr;
-        if (ok) pg[(int64_t)(8 * g + r) * a.ldG] = gr;
-      }
-      if (full) {
+        for (int r = 0; r < 4; ++r) {
+          float v = acc[4 * g + r];
+          if (HAS_SCALE) v *= sc_col;
+          v += b4[r];
+          const float ex = __expf(-fabsf(v));                       // in (0, 1]
+          const float sig = (v >= 0.f ? 1.0f : ex) / (1.0f + ex);    // sigmoid without overflow
+          const float gr = sig * a.inv_bn - a.uniform;
+          prod = __builtin_fmaf(prod, ex, prod);
+          tpos += fmaxf(v, 0.f);
+          tss += v;
+          out[r] = gr;
+          rowsum[qt][4 * g + r] += gr;
+          pg[(int64_t)(8 * g + r) * a.ldG] = gr;
+        }
         *(f32x4*)(pt + 8 * g) = out;
-      } else {
+      }
+    } else {
 #pragma unroll
-        for (int r = 0; r < 4; ++r)
-          if (qrow + 8 * g + r < B) pt[8 * g + r] = out[r];
+      for (int g = 0; g < 4; ++g) {
+        const f32x4 b4 = *(const f32x4*)(lb + 32 * qt + 8 * g + 4 * hf);
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          float v = acc[4 * g + r];
+          if (HAS_SCALE) v *= sc_col;
+          v += b4[r];
+          const bool ok = qrow + 8 * g + r < B;
+          const float ex = __expf(-fabsf(v));
+          const float sig = (v >= 0.f ? 1.0f : ex) / (1.0f + ex);
+          const float gr = ok ? sig * a.inv_bn - a.uniform : 0.f;
+          prod = __builtin_fmaf(prod, ok ? ex : 0.f, prod);
+          tpos += ok ? fmaxf(v, 0.f) : 0.f;
+          tss += ok ? v : 0.f;
+          rowsum[qt][4 * g + r] += gr;
+          if (ok) {
+            pg[(int64_t)(8 * g + r) * a.ldG] = gr;
+            pt[8 * g + r] = gr;
+          }
+        }
       }
     }
     sp += (double)(tpos + __logf(prod));
