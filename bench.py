@@ -118,6 +118,11 @@ def main():
                          "train: loss and the gradient of every parameter, i.e. bcegrad plus the query builder's backward)")
     ap.add_argument("--scale", type=float, default=1.0, help="shrink the workload (testing only)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--streams", type=int, default=1,
+                    help="consecutive steps on this many alternating streams, as dicee_amd.Evaluator runs the batches "
+                         "of an evaluation (2 there); a step short enough to be a chain of dependent launches gains "
+                         "(c2: 0.117 -> 0.075 ms), and the main-loop kernel's own duration then includes what it "
+                         "shares the GPU with")
     ap.add_argument("--graph", action="store_true",
                     help="capture one HIP graph per batch before the timed region and replay the graphs (rank, bce and "
                          "bcegrad steps only: the top-k call reads a counter back on the host and cannot be captured)")
@@ -206,6 +211,18 @@ def main():
 
         def step(i):                                             # noqa: F811 (replaces the eager step on purpose)
             graphs[i % len(graphs)].replay()
+    if args.streams > 1:
+        if args.graph:
+            print("bench.py: --streams does not apply to --graph", file=sys.stderr)
+            sys.exit(2)
+        pool = [torch.cuda.Stream() for _ in range(args.streams)]
+        for s_ in pool:
+            s_.wait_stream(torch.cuda.current_stream())
+        one_stream_step = step
+
+        def step(i):                                             # noqa: F811 (the same step on alternating streams)
+            with torch.cuda.stream(pool[i % len(pool)]):
+                return one_stream_step(i)
     for i in range(args.warmup):
         step(i)
     torch.cuda.synchronize()
@@ -243,7 +260,8 @@ def main():
         "dtype": {"fp32": "f32 as 3 x bf16 parts, bf16 x bf16 -> f32", "bf16": "bf16 x bf16 -> f32", "int8": "int8 table as bf16 x bf16 -> f32"}[cfg.storage]
                  if compute != "int8" else "int8 x int8 -> i32 filter scan, candidates rescored as bf16 x bf16 -> f32",
         "data": "synthetic",
-        "launch": "one HIP graph replay per step" if args.graph else "eager launches",
+        "launch": "one HIP graph replay per step" if args.graph else "eager launches" if args.streams <= 1
+                  else f"eager launches, consecutive steps alternating over {args.streams} streams",
         "config": {"workload": f"{args.config}: {cfg.model} {mode}, N={N} entities, d={d}, {cfg.storage} tables, "
                                f"batch {cfg.B}, {len(q_all)} queries"
                                + (f", filter CSR nnz={cfg.csr.nnz} max row {int(np.diff(cfg.csr.row_ptr_np).max())}"

@@ -57,8 +57,38 @@ def ranks_from_counts(n_greater, n_equal, n_equal_lower, tie="stable"):
     raise ValueError(tie)
 
 
+class _BatchStreams:
+    """Consecutive batches of an evaluation on alternating streams.  A batch is a short chain of dependent launches
+    (query vectors, filter rows, plan, thresholds, main loop, correction); two chains side by side fill the gaps each
+    leaves (ComplEx, 14,541 entities, batches of 1024: 0.117 -> 0.075 ms per batch).  The first batch runs on the
+    caller's stream, so that whatever the model derives lazily (its quantised table) exists before the streams
+    fork; ``join()`` makes the caller's stream wait for all of them."""
+
+    def __init__(self, device, n):
+        self.cur = torch.cuda.current_stream(device)
+        self.n = max(1, int(n))
+        self.device = device
+        self.pool = None
+        self.i = 0
+
+    def next(self):
+        """Context manager for the next batch."""
+        self.i += 1
+        if self.n == 1 or self.i == 1:
+            return torch.cuda.stream(self.cur)
+        if self.pool is None:
+            self.pool = [torch.cuda.Stream(device=self.device) for _ in range(self.n)]
+            for s in self.pool:
+                s.wait_stream(self.cur)
+        return torch.cuda.stream(self.pool[self.i % self.n])
+
+    def join(self):
+        for s in self.pool or ():
+            self.cur.wait_stream(s)
+
+
 class Evaluator:
-    def __init__(self, args=None, is_continual_training=False, tie="stable"):
+    def __init__(self, args=None, is_continual_training=False, tie="stable", streams=2):
         if args is None:
             args = SimpleNamespace(batch_size=1024, eval_model="train_val_test", scoring_technique="KvsAll",
                                    full_storage_path=None)
@@ -78,6 +108,7 @@ class Evaluator:
         self.report = {}
         self.during_training = False
         self.tie = tie
+        self.streams = streams   # batches of an evaluation alternate over this many streams (1: the caller's only)
         self.last_ranks = None
 
     # ------------------------------------------------------------------ filter preparation
@@ -259,13 +290,16 @@ class Evaluator:
         all_trip = torch.from_numpy(np.ascontiguousarray(triple_idx.astype(np.int64))).to(dev)
         out = torch.empty((num_triples,), dtype=torch.int64, device=dev)
         bs = int(self.args.batch_size)
+        lanes = _BatchStreams(dev, self.streams)
         with torch.no_grad():
             for i in range(0, num_triples, bs):
-                batch = all_trip[i:i + bs]
-                x = batch[:, [0, 2]].contiguous()
-                r = batch[:, 1].contiguous()
-                c = model.rank_filtered(x, r, csr)
-                out[i:i + bs] = ranks_from_counts(c["n_greater"], c["n_equal"], c["n_equal_lower"], self.tie)
+                with lanes.next():
+                    batch = all_trip[i:i + bs]
+                    x = batch[:, [0, 2]].contiguous()
+                    r = batch[:, 1].contiguous()
+                    c = model.rank_filtered(x, r, csr)
+                    out[i:i + bs] = ranks_from_counts(c["n_greater"], c["n_equal"], c["n_equal_lower"], self.tie)
+        lanes.join()
         return out.cpu().numpy()
 
     def _evaluate_entity_prediction(self, model, triple_idx, num_triples):
@@ -286,11 +320,14 @@ class Evaluator:
         all_trip = torch.from_numpy(np.ascontiguousarray(triple_idx.astype(np.int64))).to(dev)
         out = torch.empty((num_triples,), dtype=torch.int64, device=dev)
         bs = int(self.args.batch_size)
+        lanes = _BatchStreams(dev, self.streams)
         with torch.no_grad():
             for i in range(0, num_triples, bs):
-                batch = all_trip[i:i + bs]
-                x = batch[:, :2].contiguous()
-                t = batch[:, 2].contiguous()
-                c = model.rank_filtered(x, t, csr)
-                out[i:i + bs] = ranks_from_counts(c["n_greater"], c["n_equal"], c["n_equal_lower"], self.tie)
+                with lanes.next():
+                    batch = all_trip[i:i + bs]
+                    x = batch[:, :2].contiguous()
+                    t = batch[:, 2].contiguous()
+                    c = model.rank_filtered(x, t, csr)
+                    out[i:i + bs] = ranks_from_counts(c["n_greater"], c["n_equal"], c["n_equal_lower"], self.tie)
+        lanes.join()
         return out.cpu().numpy()

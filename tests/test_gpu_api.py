@@ -122,6 +122,29 @@ def test_evaluator_matches_the_reference_loop(name, d, extra, batch_size):
         np.testing.assert_array_equal(own, got)
 
 
+@pytest.mark.parametrize("storage", ["fp32", "bf16", "int8"])
+def test_evaluator_batches_on_alternating_streams_give_the_same_ranks(storage):
+    """The batches of an evaluation alternate over two streams by default.  Whatever the number of streams, the ranks
+    are those of the one-stream evaluation; with quantised storage the table's snapshot is taken lazily by the first
+    batch, before the streams fork."""
+    from dicee_amd import Evaluator
+    m, triples = _toy("DistMult", 64, N=3000, R=11, n=6000, seed=11)
+    er = {}
+    for h, r, t in triples:
+        er.setdefault((int(h), int(r)), []).append(int(t))
+    ranks = {}
+    for streams in (1, 2, 3):
+        model = m.to("cuda").set_entity_storage(storage)           # (a fresh snapshot for every run)
+        ev = Evaluator(SimpleNamespace(batch_size=256, eval_model="test", scoring_technique="KvsAll",
+                                       full_storage_path=None), streams=streams)
+        ev.set_filter(er, num_relations=11)
+        ev.evaluate_lp_k_vs_all(model, triples, form_of_labelling="EntityPrediction")
+        ranks[streams] = ev.last_ranks.copy()
+    np.testing.assert_array_equal(ranks[1], ranks[2])
+    np.testing.assert_array_equal(ranks[1], ranks[3])
+    assert len(ranks[1]) == len(triples) and ranks[1].min() >= 1
+
+
 @pytest.mark.parametrize("name,d,extra", [("DistMult", 32, {}), ("QMult", 64, {})])
 def test_relation_prediction_follows_the_reference_loop_literally(name, d, extra):
     """form_of_labelling='RelationPrediction' (evaluator.py:440-471): (head, tail) pairs through forward_k_vs_all,
