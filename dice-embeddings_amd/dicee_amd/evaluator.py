@@ -242,7 +242,7 @@ class Evaluator:
         assert self.csr is not None, "self.er_vocab cannot be None"
         return evaluate_lp(model, triple_idx, num_entities=self.num_entities, er_vocab=self.csr,
                            re_vocab=self._other_vocab("re", model), info=None if self.during_training else info,
-                           tie=self.tie)
+                           tie=self.tie, streams=self.streams)
 
     def evaluate_lp_k_vs_all(self, model, triple_idx, info=None, form_of_labelling=None):
         """Filtered link prediction with KvsAll scoring -> ``{'H@1','H@3','H@10','MRR'}``."""

@@ -13,7 +13,7 @@ import numpy as np
 import torch
 
 from .csr import FilterCSR
-from .evaluator import ranks_from_counts
+from .evaluator import ranks_from_counts, _BatchStreams
 
 
 def _as_csr(vocab, key_mult, device):
@@ -28,12 +28,14 @@ def _as_csr(vocab, key_mult, device):
 
 @torch.no_grad()
 def evaluate_lp(model, triple_idx, num_entities=None, er_vocab=None, re_vocab=None, info="Eval Starts",
-                batch_size=128, chunk_size=1000, tie="stable", return_ranks=False):
+                batch_size=128, chunk_size=1000, tie="stable", return_ranks=False, streams=2):
     """``{'H@1', 'H@3', 'H@10', 'MRR'}`` over head and tail prediction.
 
     ``er_vocab`` / ``re_vocab``: the reference's dicts ``(h, r) -> [t]`` / ``(r, t) -> [h]``, or ``FilterCSR``
     objects (``FilterCSR.from_triples_gpu(..., kind="er" | "re")``).  ``chunk_size`` is accepted for
-    signature compatibility; nothing is chunked.  ``return_ranks``: also return (head_ranks, tail_ranks)."""
+    signature compatibility; nothing is chunked.  ``return_ranks``: also return (head_ranks, tail_ranks).
+    ``streams``: the rank calls (two per batch, independent of one another) alternate over this many streams,
+    joined before the ranks are read; 1 keeps all of them on the caller's stream."""
     assert model is not None, "Model must be provided"
     assert triple_idx is not None, "triple_idx must be provided"
     assert er_vocab is not None, "er_vocab must be provided"
@@ -64,12 +66,16 @@ def evaluate_lp(model, triple_idx, num_entities=None, er_vocab=None, re_vocab=No
     tail_ranks = torch.empty((n,), dtype=torch.int64, device=dev)
     head_ranks = torch.empty((n,), dtype=torch.int64, device=dev)
     bs = int(batch_size)
+    lanes = _BatchStreams(dev, streams)
     for i in range(0, n, bs):
         b = trip[i:i + bs]
-        c = model.rank_filtered(b[:, :2].contiguous(), b[:, 2].contiguous(), er)
-        tail_ranks[i:i + bs] = ranks_from_counts(c["n_greater"], c["n_equal"], c["n_equal_lower"], tie)
-        c = model.rank_filtered(b[:, 1:].contiguous(), b[:, 0].contiguous(), re, heads=True)
-        head_ranks[i:i + bs] = ranks_from_counts(c["n_greater"], c["n_equal"], c["n_equal_lower"], tie)
+        with lanes.next():
+            c = model.rank_filtered(b[:, :2].contiguous(), b[:, 2].contiguous(), er)
+            tail_ranks[i:i + bs] = ranks_from_counts(c["n_greater"], c["n_equal"], c["n_equal_lower"], tie)
+        with lanes.next():
+            c = model.rank_filtered(b[:, 1:].contiguous(), b[:, 0].contiguous(), re, heads=True)
+            head_ranks[i:i + bs] = ranks_from_counts(c["n_greater"], c["n_equal"], c["n_equal_lower"], tie)
+    lanes.join()
     hr_, tr_ = head_ranks.cpu().numpy(), tail_ranks.cpu().numpy()
     divisor = float(2 * n) if n else 1.0
     results = {f"H@{k}": float((np.count_nonzero(hr_ <= k) + np.count_nonzero(tr_ <= k)) / divisor) for k in (1, 3, 10)}
@@ -92,7 +98,7 @@ def _csr_of_string_vocab(vocab, first, second, values, key_mult, device):
 
 
 @torch.no_grad()
-def evaluate_link_prediction_performance_with_reciprocals(model, triples, er_vocab, tie="stable"):
+def evaluate_link_prediction_performance_with_reciprocals(model, triples, er_vocab, tie="stable", streams=2):
     """Tail-only filtered evaluation of string triples for models trained with reciprocal relations
     (dicee/evaluation/link_prediction.py:116-174).  ``model``: a ``KGE`` (``.model``, ``.entity_to_idx``,
     ``.relation_to_idx``); ``er_vocab``: (head str, relation str) -> list of tail strs.  Batches of
@@ -108,10 +114,13 @@ def evaluate_link_prediction_performance_with_reciprocals(model, triples, er_voc
     n = len(ids)
     bs = int(net.args.get("batch_size", 1024) or 1024)
     out = torch.empty((n,), dtype=torch.int64, device=dev)
+    lanes = _BatchStreams(dev, streams)
     for i in range(0, n, bs):
         b = trip[i:i + bs]
-        c = net.rank_filtered(b[:, :2].contiguous(), b[:, 2].contiguous(), csr)
-        out[i:i + bs] = ranks_from_counts(c["n_greater"], c["n_equal"], c["n_equal_lower"], tie)
+        with lanes.next():
+            c = net.rank_filtered(b[:, :2].contiguous(), b[:, 2].contiguous(), csr)
+            out[i:i + bs] = ranks_from_counts(c["n_greater"], c["n_equal"], c["n_equal_lower"], tie)
+    lanes.join()
     ranks = out.cpu().numpy()
     assert len(triples) == len(ranks) == n
     hits = create_hits_dict()
@@ -121,7 +130,7 @@ def evaluate_link_prediction_performance_with_reciprocals(model, triples, er_voc
 
 
 @torch.no_grad()
-def evaluate_link_prediction_performance(model, triples, er_vocab, re_vocab, tie="stable"):
+def evaluate_link_prediction_performance(model, triples, er_vocab, re_vocab, tie="stable", streams=2):
     """Head and tail filtered evaluation of string triples (dicee/evaluation/link_prediction.py:22-113):
     ``er_vocab`` (head str, relation str) -> tails, ``re_vocab`` (relation str, tail str) -> heads."""
     net = model.model
@@ -132,4 +141,4 @@ def evaluate_link_prediction_performance(model, triples, er_vocab, re_vocab, tie
     re = _csr_of_string_vocab(re_vocab, model.relation_to_idx, model.entity_to_idx, model.entity_to_idx,
                               net.num_entities, dev)
     return evaluate_lp(net, ids, net.num_entities, er, re, info=None, batch_size=int(net.args.get("batch_size", 1024) or 1024),
-                       tie=tie)
+                       tie=tie, streams=streams)

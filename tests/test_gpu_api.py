@@ -143,6 +143,19 @@ def test_evaluator_batches_on_alternating_streams_give_the_same_ranks(storage):
     np.testing.assert_array_equal(ranks[1], ranks[2])
     np.testing.assert_array_equal(ranks[1], ranks[3])
     assert len(ranks[1]) == len(triples) and ranks[1].min() >= 1
+    # the head-and-tail evaluation: two rank calls per batch, on alternating streams as well
+    from dicee_amd import FilterCSR
+    from dicee_amd.link_prediction import evaluate_lp
+    model = m.to("cuda").set_entity_storage(storage)
+    dev_trip = torch.from_numpy(triples.astype(np.int64)).cuda()
+    er_csr = FilterCSR.from_triples_gpu(dev_trip, 3000, 11, kind="er")
+    re_csr = FilterCSR.from_triples_gpu(dev_trip, 3000, 11, kind="re")
+    both = {s: evaluate_lp(model, triples, 3000, er_csr, re_csr, info=None, batch_size=256, return_ranks=True,
+                           streams=s) for s in (1, 2, 3)}
+    for s in (2, 3):
+        assert both[s][0] == both[1][0]
+        np.testing.assert_array_equal(both[s][1][0], both[1][1][0])
+        np.testing.assert_array_equal(both[s][1][1], both[1][1][1])
 
 
 @pytest.mark.parametrize("name,d,extra", [("DistMult", 32, {}), ("QMult", 64, {})])
