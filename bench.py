@@ -97,11 +97,16 @@ def main_loop_kernel(storage, d, mode):
            "bcegrad": "GradEpi | StoreEpi", "train": "GradEpi | StoreEpi"}[mode]
     if storage == "fp32":
         return f"ksplit_kernel<{epi}, {'true' if d % 4 == 0 else 'false'}>"
-    if d == 128 and storage == "bf16":
-        return "qstream_kernel<RankFastEpi, 2, 8, 2>" if epi == "RankEpi" else f"qreg_async_kernel<{epi}>"
-    if d == 128:
-        return "topk_i8_filter_kernel" if epi == "TopkEpi" else f"qreg_i8_kernel<{epi}>"
-    if storage == "bf16" and d > 128:
+    if storage == "bf16" and d in (64, 128, 256):
+        nqt = 1 if d == 256 else 2
+        if epi == "RankEpi":
+            return f"qstream_kernel<RankFastEpi, {nqt}, 8, 2, {d // 16}>"
+        return f"qreg_async_kernel<{epi}, {nqt}, {d // 16}>"
+    if storage == "int8" and d in (64, 128, 256):
+        if d == 128 and epi == "TopkEpi":
+            return "topk_i8_filter_kernel"
+        return f"qreg_i8_kernel<{epi}, {1 if d == 256 else 2}, {d // 16}>"
+    if d > 128:
         return f"kchunk_kernel<{epi}>"
     return f"qreg_kernel<{storage}, {epi}>"
 
