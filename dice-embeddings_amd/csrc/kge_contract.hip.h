@@ -1,10 +1,12 @@
 // Query x all-entity contraction on MFMA with fused epilogues (gfx950).
 //
 // All main loops run on the bf16 MFMA (32x32x16) and share one epilogue interface:
-//   qreg_async_kernel   bf16 table, d == 128: persistent, queries register-resident, entity rows global -> LDS
-//   qreg_i8_kernel      per-row int8 table, d == 128: the same walk, rows widened to bf16 on the way into LDS
-//   qreg_kernel         bf16 / int8 with d < 128
-//   kchunk_kernel       bf16 / int8 with d > 128: K in chunks of 64 through LDS
+//   qreg_async_kernel   bf16 table, d == 64, 128 or 129..256: persistent, queries register-resident, entity rows
+//                       global -> LDS
+//   qstream_kernel      the same with a deeper pipeline and the epilogue inside the MFMA chain (filtered rank, scores)
+//   qreg_i8_kernel      per-row int8 table, the same widths and walk, rows widened to bf16 on the way into LDS
+//   qreg_kernel         bf16 / int8 with d < 128 (other than 64)
+//   kchunk_kernel       bf16 / int8 with d > 256: K in chunks of 64 through LDS
 //   ksplit_kernel       fp32 tables, any d: every operand as three bf16 parts, six part products per product
 // Reduction order of one score is fixed (k ascending in steps of the MFMA depth, nothing else), so
 // every kernel that forms dot(Q[b], E[e]) with these helpers produces the same fp32 bit pattern.
@@ -1071,11 +1073,16 @@ constexpr int QA_BUF_BYTES = QA_STAGE_ROWS * 256;
 // NQT query tiles per wave and KSTEPS K steps of 16 per score: (QA_NQT, 8) for d == 128; (1, 16) for d == 256 (512-byte
 // rows, two 64 KB stage buffers, the next tile's fragments read straight into the registers of the current ones);
 // (QA_NQT, 4) for d == 64.
-template <template <int> class EpiT, int NQT = QA_NQT, int KSTEPS = 8>
+// PAD: the table's rows are narrower than the LDS rows (a.d < 16 * KSTEPS, a.d % 8 == 0): a row is fetched with its
+// own stride, the 16-byte pieces past a.d are never written and stay the zeros the buffers start with, and the
+// queries' fragments are zero there as well, so the chain adds exact zeros after the row's last K step.
+template <template <int> class EpiT, int NQT = QA_NQT, int KSTEPS = 8, bool PAD = false>
 __global__ void __launch_bounds__(64 * QA_WG_WAVES, QA_WAVES_PER_SIMD) qreg_async_kernel(ContractArgs a, typename EpiT<NQT>::Args ea) {
   using Epi = EpiT<NQT>;
   constexpr int d = 16 * KSTEPS;
   constexpr int ROW_BYTES = 2 * d;
+  const int dq = PAD ? a.d : d;              // elements of a query row and of a table row in memory
+  const int64_t row_stride = 2 * (int64_t)dq;  // bytes of a table row in memory
   constexpr int BUF_BYTES = QA_STAGE_ROWS * ROW_BYTES;
   constexpr int TILE_BYTES = 32 * ROW_BYTES;
   constexpr bool INPLACE = (KSTEPS > 8);  // no second set of fragment registers
@@ -1111,8 +1118,8 @@ __global__ void __launch_bounds__(64 * QA_WG_WAVES, QA_WAVES_PER_SIMD) qreg_asyn
     for (int s = 0; s < KSTEPS; ++s) {
       const int k = 16 * s + 8 * hf;
       f32x4 lo = {0.f, 0.f, 0.f, 0.f}, hi = {0.f, 0.f, 0.f, 0.f};
-      if (q < a.B) {
-        const f32x4* src = (const f32x4*)(a.Q + q * d + k);
+      if (q < a.B && (!PAD || k < dq)) {
+        const f32x4* src = (const f32x4*)(a.Q + q * dq + k);
         lo = src[0];
         hi = src[1];
       }
@@ -1134,21 +1141,27 @@ __global__ void __launch_bounds__(64 * QA_WG_WAVES, QA_WAVES_PER_SIMD) qreg_asyn
                                                 // them in a row of fewer than sixteen pieces)
   const int lrow = wave * RPW + lane / LPR;
   const int lpiece = (lane % LPR) ^ (lrow & SWZ);
+  const bool lane_on = !PAD || 8 * lpiece < dq;  // (a lane fetches the same piece of every row it handles)
   const unsigned char* Eb = (const unsigned char*)a.E;
+  if constexpr (PAD) {
+    for (int i = tid * 16; i < 2 * BUF_BYTES; i += 64 * QA_WG_WAVES * 16) *(u32x4*)(lds_e + i) = u32x4{0u, 0u, 0u, 0u};
+    __syncthreads();  // no load may land before the zeros do
+  }
   auto stage_issue = [&](int64_t row0, int buf) {
     unsigned char* dst = lds_e + buf * BUF_BYTES + wave * 1024;
+    if (!lane_on) return;
     if (row0 + QA_STAGE_ROWS <= r_end) {
-      const unsigned char* src = Eb + (row0 + lrow) * ROW_BYTES + lpiece * 16;
+      const unsigned char* src = Eb + (row0 + lrow) * row_stride + lpiece * 16;
 #pragma unroll
       for (int j = 0; j < NLD; ++j)
-        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src + j * (RPI * ROW_BYTES)),
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src + j * (RPI * row_stride)),
                                          (__attribute__((address_space(3))) void*)(dst + j * (RPI * ROW_BYTES)), 16, 0, 0);
     } else {
 #pragma unroll
       for (int j = 0; j < NLD; ++j) {
         int64_t g = row0 + lrow + RPI * j;
         g = (g < r_end) ? g : r_end - 1;  // padding rows repeat the last valid row; the epilogue ignores them
-        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(Eb + g * ROW_BYTES + lpiece * 16),
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(Eb + g * row_stride + lpiece * 16),
                                          (__attribute__((address_space(3))) void*)(dst + j * (RPI * ROW_BYTES)), 16, 0, 0);
       }
     }
@@ -1243,11 +1256,14 @@ constexpr int QS_NBUF = 3;
 constexpr int QS_VALU_PER_MFMA = 5;
 
 // KSTEPS: K steps of 16 per score (8: d == 128; 16: d == 256, rows of 512 bytes, one query tile per wave; 4: d == 64).
-template <template <int> class EpiT, int NQT, int W, int OCC, int KSTEPS = 8>
+// PAD: rows narrower than the LDS rows, as in qreg_async_kernel.
+template <template <int> class EpiT, int NQT, int W, int OCC, int KSTEPS = 8, bool PAD = false>
 __global__ void __launch_bounds__(64 * W, OCC) qstream_kernel(ContractArgs a, typename EpiT<NQT>::Args ea) {
   using Epi = EpiT<NQT>;
   constexpr int d = 16 * KSTEPS;
-  constexpr int ROW_BYTES = 2 * d;                      // a bf16 row
+  constexpr int ROW_BYTES = 2 * d;                      // a bf16 row in LDS
+  const int dq = PAD ? a.d : d;                         // elements of a query row and of a table row in memory
+  const int64_t row_stride = 2 * (int64_t)dq;           // bytes of a table row in memory
   constexpr int STAGE_BYTES = QS_STAGE_ROWS * ROW_BYTES;
   constexpr int TILE_BYTES = 32 * ROW_BYTES;            // one 32-row entity tile of a stage
   __shared__ __attribute__((aligned(1024))) unsigned char lds_e[QS_NBUF * STAGE_BYTES];
@@ -1283,8 +1299,8 @@ __global__ void __launch_bounds__(64 * W, OCC) qstream_kernel(ContractArgs a, ty
     for (int s = 0; s < KSTEPS; ++s) {
       const int k = 16 * s + 8 * hf;
       f32x4 lo = {0.f, 0.f, 0.f, 0.f}, hi = {0.f, 0.f, 0.f, 0.f};
-      if (q < a.B) {
-        const f32x4* src = (const f32x4*)(a.Q + q * d + k);
+      if (q < a.B && (!PAD || k < dq)) {
+        const f32x4* src = (const f32x4*)(a.Q + q * dq + k);
         lo = src[0];
         hi = src[1];
       }
@@ -1308,14 +1324,20 @@ __global__ void __launch_bounds__(64 * W, OCC) qstream_kernel(ContractArgs a, ty
                                                 // them in a row of fewer than sixteen pieces)
   const int lrow = wave * RPW + lane / LPR;
   const int lpiece = (lane % LPR) ^ (lrow & SWZ);
+  const bool lane_on = !PAD || 8 * lpiece < dq;  // (a lane fetches the same piece of every row it handles)
   const unsigned char* Eb = (const unsigned char*)a.E;
+  if constexpr (PAD) {
+    for (int i = tid * 16; i < QS_NBUF * STAGE_BYTES; i += 64 * W * 16) *(u32x4*)(lds_e + i) = u32x4{0u, 0u, 0u, 0u};
+    __syncthreads();  // no load may land before the zeros do
+  }
   uint32_t voff[NLD];
 #pragma unroll
-  for (int j = 0; j < NLD; ++j) voff[j] = (uint32_t)((lrow + RPI * j) * ROW_BYTES + lpiece * 16);
+  for (int j = 0; j < NLD; ++j) voff[j] = (uint32_t)((lrow + RPI * j) * (int)row_stride + lpiece * 16);
   auto stage_issue = [&](int64_t row0, int buf) {
     unsigned char* dst = lds_e + buf * STAGE_BYTES + wave * 1024;
+    if (!lane_on) return;
     if (__builtin_expect(row0 + QS_STAGE_ROWS <= r_end, 1)) {
-      const unsigned char* src = Eb + row0 * ROW_BYTES;  // wave-uniform
+      const unsigned char* src = Eb + row0 * row_stride;  // wave-uniform
 #pragma unroll
       for (int j = 0; j < NLD; ++j)
         __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src + voff[j]),
@@ -1325,7 +1347,7 @@ __global__ void __launch_bounds__(64 * W, OCC) qstream_kernel(ContractArgs a, ty
       for (int j = 0; j < NLD; ++j) {
         int64_t g = row0 + lrow + RPI * j;
         g = (g < r_end) ? g : r_end - 1;
-        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(Eb + g * ROW_BYTES + lpiece * 16),
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(Eb + g * row_stride + lpiece * 16),
                                          (__attribute__((address_space(3))) void*)(dst + j * (RPI * ROW_BYTES)), 16, 0, 0);
       }
     }
@@ -1498,11 +1520,13 @@ constexpr int I8_WGS_PER_CU = 8 / I8_WG_WAVES;  // 2 waves per SIMD
 // NQT query tiles per wave and KSTEPS K steps of 16 per score: (2, 8) for d == 128; (1, 16) for d == 256, whose rows are
 // 512 bytes of bf16 in LDS (64 KB per stage buffer) and whose queries still fit the register file one tile per wave;
 // (2, 4) for d == 64.
-template <template <int> class EpiT, int NQT = QREG_NQT, int KSTEPS = 8>
+// PAD: rows narrower than the LDS rows (a.d < 16 * KSTEPS, a.d % 16 == 0): the pieces past a.d are stored as zeros.
+template <template <int> class EpiT, int NQT = QREG_NQT, int KSTEPS = 8, bool PAD = false>
 __global__ void __launch_bounds__(64 * I8_WG_WAVES, 2) qreg_i8_kernel(ContractArgs a, typename EpiT<NQT>::Args ea) {
   using Epi = EpiT<NQT>;
   constexpr int d = 16 * KSTEPS;
-  constexpr int ROW_BYTES = 2 * d;                      // a row widened to bf16
+  constexpr int ROW_BYTES = 2 * d;                      // a row widened to bf16, in LDS
+  const int dq = PAD ? a.d : d;                         // elements (and bytes) of a table row in memory
   constexpr int BUF_BYTES = QA_STAGE_ROWS * ROW_BYTES;
   constexpr int PPR = d / 16;                           // 16-byte pieces of int8 per row
   constexpr int SWZ = 2 * PPR < 16 ? 2 * PPR - 1 : 15;  // swizzled bits of the index of a row's 16-byte bf16 pieces
@@ -1540,8 +1564,8 @@ __global__ void __launch_bounds__(64 * I8_WG_WAVES, 2) qreg_i8_kernel(ContractAr
     for (int s = 0; s < KSTEPS; ++s) {
       const int k = 16 * s + 8 * hf;
       f32x4 lo = {0.f, 0.f, 0.f, 0.f}, hi = {0.f, 0.f, 0.f, 0.f};
-      if (q < a.B) {
-        const f32x4* src = (const f32x4*)(a.Q + q * d + k);
+      if (q < a.B && (!PAD || k < dq)) {
+        const f32x4* src = (const f32x4*)(a.Q + q * dq + k);
         lo = src[0];
         hi = src[1];
       }
@@ -1563,7 +1587,8 @@ __global__ void __launch_bounds__(64 * I8_WG_WAVES, 2) qreg_i8_kernel(ContractAr
       const int idx = tid + NT * j, row = idx / PPR, piece = idx % PPR;
       int64_t g = row0 + row;
       g = (g < r_end) ? g : r_end - 1;  // padding rows repeat the last valid row; epilogues ignore them
-      stage[j] = *(const u32x4*)(Eb + g * d + piece * 16);
+      stage[j] = u32x4{0u, 0u, 0u, 0u};
+      if (!PAD || 16 * piece < dq) stage[j] = *(const u32x4*)(Eb + g * dq + piece * 16);
     }
     if (tid < QA_STAGE_ROWS) {
       int64_t g = row0 + tid;

@@ -1177,7 +1177,11 @@ int check_contract(const char* who, const float* Q, const void* E, int dtype, co
 // the branching or long ones (there top-k and row extrema are 10 % slower, BCE twice as slow); those take
 // qreg_async_kernel, epilogue after the chain.
 // bf16 rows of d == 64 take the same two kernels in the d == 128 workgroup shape, with four K steps.
+// Rows between 128 and 256 elements take the same kernels with 512-byte LDS rows whose tail stays zero (PAD): the
+// chain runs its sixteen K steps, the last ones on zeros (d = 200: 0.78 of the d = 256 rate per useful product,
+// against half of it in kchunk_kernel).
 constexpr int QS256_WG_QUERIES = QA_WG_WAVES * 32;
+static inline bool rows_up_to_256(int64_t d) { return d > 128 && d <= 256; }
 template <template <int> class EpiT>
 constexpr bool stream256_epilogue() {
   return std::is_same<EpiT<2>, RankEpi<2>>::value || std::is_same<EpiT<2>, StoreEpi<2>>::value;
@@ -1197,8 +1201,8 @@ ContractArgs make_args(const float* Q, const void* E, int dtype, const float* sc
   a.k_split_len = 0;
   a.persistent = 0;
   const bool stream64 = dtype == KGE_BF16 && d == 64;  // (persistent whatever the epilogue)
-  const bool stream256 = dtype == KGE_BF16 && d == 256;  // (persistent whatever the epilogue)
-  const bool i8_256 = (dtype == KGE_I8 && d == 256);  // qreg_i8_kernel with one query tile per wave, every epilogue
+  const bool stream256 = dtype == KGE_BF16 && rows_up_to_256(d);  // (persistent whatever the epilogue)
+  const bool i8_256 = (dtype == KGE_I8 && rows_up_to_256(d));  // qreg_i8_kernel with one query tile per wave, every epilogue
   const bool fast_bf16 = (dtype == KGE_BF16 && d == 128) || stream256 || stream64;
   const bool i8_64 = (dtype == KGE_I8 && d == 64);    // the same kernel in the d == 128 shape with four K steps
   const bool fast_i8 = (dtype == KGE_I8 && d == 128) || i8_256 || i8_64;
@@ -1287,10 +1291,11 @@ struct LaunchTimer {
 template <template <int> class EpiT, class EArgs>
 int launch_contract(int dtype, const ContractArgs& a, const EArgs& ea, hipStream_t st, const char* name) {
   if (a.B == 0 || a.e_end <= a.e_begin) return KGE_OK;
-  const bool i8_256 = (dtype == KGE_I8 && a.d == 256);
+  const bool i8_256 = (dtype == KGE_I8 && rows_up_to_256(a.d));
+  const bool pad = a.d != 256;  // (of the two cases above: rows narrower than the LDS rows)
   const bool i8_64 = (dtype == KGE_I8 && a.d == 64);
   const bool fast_i8 = (dtype == KGE_I8 && a.d == 128) || i8_256 || i8_64;
-  const bool stream256 = dtype == KGE_BF16 && a.d == 256;
+  const bool stream256 = dtype == KGE_BF16 && rows_up_to_256(a.d);
   const bool stream64 = dtype == KGE_BF16 && a.d == 64;
   const bool persistent = (dtype == KGE_BF16 && a.d == 128) || fast_i8 || stream256 || stream64;
   // (make_args and this function both decide, from the table, between the persistent and the tiled kernels; a plan
@@ -1321,7 +1326,7 @@ int launch_contract(int dtype, const ContractArgs& a, const EArgs& ea, hipStream
     else
       hipLaunchKernelGGL((qreg_async_kernel<EpiT, QA_NQT, 4>), grid, block, 0, st, a, ea);
   }
-  else if (stream256) {
+  else if (stream256 && !pad) {
     if constexpr (std::is_same<EpiT<2>, RankEpi<2>>::value)
       hipLaunchKernelGGL((qstream_kernel<RankFastEpi, 1, QA_WG_WAVES, QA_WAVES_PER_SIMD, 16>), grid, block, 0, st, a, ea);
     else if constexpr (stream256_epilogue<EpiT>())
@@ -1329,14 +1334,24 @@ int launch_contract(int dtype, const ContractArgs& a, const EArgs& ea, hipStream
     else
       hipLaunchKernelGGL((qreg_async_kernel<EpiT, 1, 16>), grid, block, 0, st, a, ea);
   }
+  else if (stream256) {
+    if constexpr (std::is_same<EpiT<2>, RankEpi<2>>::value)
+      hipLaunchKernelGGL((qstream_kernel<RankFastEpi, 1, QA_WG_WAVES, QA_WAVES_PER_SIMD, 16, true>), grid, block, 0, st, a, ea);
+    else if constexpr (stream256_epilogue<EpiT>())
+      hipLaunchKernelGGL((qstream_kernel<EpiT, 1, QA_WG_WAVES, QA_WAVES_PER_SIMD, 16, true>), grid, block, 0, st, a, ea);
+    else
+      hipLaunchKernelGGL((qreg_async_kernel<EpiT, 1, 16, true>), grid, block, 0, st, a, ea);
+  }
   else if (wide_bf16 && dtype == KGE_BF16)
     hipLaunchKernelGGL((kchunk_kernel<KGE_BF16, EpiT>), grid, block, 0, st, a, ea);
   else if (wide_bf16)
     hipLaunchKernelGGL((kchunk_kernel<KGE_I8, EpiT>), grid, block, 0, st, a, ea);
   else if (dtype == KGE_BF16)
     hipLaunchKernelGGL((qreg_kernel<KGE_BF16, EpiT>), grid, block, 0, st, a, ea);
-  else if (i8_256)
+  else if (i8_256 && !pad)
     hipLaunchKernelGGL((qreg_i8_kernel<EpiT, 1, 16>), grid, block, 0, st, a, ea);
+  else if (i8_256)
+    hipLaunchKernelGGL((qreg_i8_kernel<EpiT, 1, 16, true>), grid, block, 0, st, a, ea);
   else if (i8_64)
     hipLaunchKernelGGL((qreg_i8_kernel<EpiT, QREG_NQT, 4>), grid, block, 0, st, a, ea);
   else if (fast_i8)

@@ -135,12 +135,15 @@ SCORE_CASES = [
     ("Keci", 1500, 6, 256, 300, "bf16", {"p": 0, "q": 1, "coeff_q": [1.0]}),      # d = 256: the streaming kernel, 512-byte rows
     ("DistMult", 9001, 5, 256, 700, "bf16", {}),     # the same over several stages per workgroup, partial last groups
     ("DistMult", 500, 5, 384, 90, "bf16", {}),       # wider still: kchunk_kernel
-    ("ComplEx", 700, 7, 200, 150, "bf16", {}),
+    ("ComplEx", 700, 7, 200, 150, "bf16", {}),       # between 128 and 256: the d = 256 kernels on rows whose LDS tail stays zero
     ("DistMult", 300, 5, 136, 70, "bf16", {}),
+    ("ComplEx", 9001, 5, 200, 700, "bf16", {}),      # the same over several stages per workgroup, partial last groups
     ("DistMult", 777, 9, 128, 70, "int8", {}),
     ("ComplEx", 2100, 9, 96, 520, "int8", {}),
-    ("ComplEx", 1300, 7, 256, 300, "int8", {}),      # int8 wider than 128: kchunk_kernel, scales applied per tile
-    ("DistMult", 777, 5, 144, 131, "int8", {}),      # K tail (144 = 2 chunks of 64 + 16), partial query group
+    ("ComplEx", 1300, 7, 256, 300, "int8", {}),      # int8 d = 256: one query tile per wave
+    ("DistMult", 777, 5, 144, 131, "int8", {}),      # between 128 and 256: the same kernel, rows padded with zeros in LDS
+    ("DistMult", 9001, 5, 240, 700, "int8", {}),
+    ("DistMult", 400, 5, 272, 90, "int8", {}),       # wider than 256: kchunk_kernel, scales applied per tile
 ]
 
 
@@ -290,7 +293,8 @@ def test_rank_one_filter_row_shared_by_different_query_vectors(ops, FilterCSR, s
 
 
 @pytest.mark.parametrize("storage,d,N", [("bf16", 64, 4097), ("fp32", 1, 1000), ("fp32", 32, 3001), ("bf16", 128, 5000),
-                                         ("int8", 128, 2500), ("bf16", 256, 1300), ("bf16", 256, 40000)])
+                                         ("int8", 128, 2500), ("bf16", 256, 1300), ("bf16", 256, 40000),
+                                         ("bf16", 200, 40000), ("int8", 192, 2500)])
 def test_rank_partial_last_query_group_with_a_bias(ops, FilterCSR, storage, d, N):
     """B = 2500 leaves the last query group of every main loop partly filled (256-, 512- and 128-query groups), and
     the per-query bias is non-zero: ranks compare un-biased scores, target_score carries the bias."""
@@ -571,6 +575,7 @@ def test_topk_many_ties_at_the_top_survive_an_overflowing_round(ops, storage, k,
     ("QMult", 3000, 5, 128, 530, "bf16", {}),
     ("DistMult", 2000, 5, 64, 100, "int8", {}),
     ("DistMult", 1100, 5, 160, 100, "int8", {}),
+    ("ComplEx", 3000, 5, 200, 530, "bf16", {}),
 ])
 @pytest.mark.parametrize("eps", [0.0, 0.1])
 def test_bce_multihot_vs_oracle(ops, FilterCSR, model, N, R, d, B, storage, kw, eps):
@@ -967,7 +972,8 @@ def test_topk_stress_patterns_match_the_materialised_scores(ops, seed, storage, 
     np.testing.assert_array_equal(idx.cpu().numpy(), wi)
 
 
-@pytest.mark.parametrize("storage,d", [("fp32", 32), ("bf16", 128), ("bf16", 64), ("int8", 128), ("int8", 64), ("bf16", 256)])
+@pytest.mark.parametrize("storage,d", [("fp32", 32), ("bf16", 128), ("bf16", 64), ("int8", 128), ("int8", 64), ("bf16", 256),
+                                       ("bf16", 200), ("int8", 144)])
 @pytest.mark.parametrize("pattern", ["pool1", "pool3", "pool50", "two_values", "zero_rows"])
 def test_rank_stress_patterns_match_the_materialised_scores(ops, FilterCSR, storage, d, pattern):
     """The same massively tied tables under the filtered rank: the target ties with thousands of entities (every
@@ -1097,9 +1103,9 @@ def test_random_differential_sweep(ops, FilterCSR, seed):
         if storage == "fp32":
             d = int(rng.choice([1, 2, 5, 8, 16, 31, 32, 48, 64, 100, 128, 200, 256, 260]))
         elif storage == "bf16":
-            d = int(rng.choice([8, 16, 40, 64, 72, 128, 136, 256, 384]))
+            d = int(rng.choice([8, 16, 40, 64, 72, 128, 136, 200, 248, 256, 384]))
         else:
-            d = int(rng.choice([16, 32, 64, 128, 128, 128, 144, 256]))
+            d = int(rng.choice([16, 32, 64, 128, 128, 128, 144, 192, 240, 256, 272]))
         N = int(rng.choice([1, 7, 64, 65, 1000, 4097, 20000, 70001] + ([150001] if case % 10 == 9 else [])))
         if B * N > 1e8:
             B = max(1, int(1e8 // N))
