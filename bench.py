@@ -97,20 +97,18 @@ def main_loop_kernel(storage, d, mode):
            "bcegrad": "GradEpi | StoreEpi", "train": "GradEpi | StoreEpi"}[mode]
     if storage == "fp32":
         return f"ksplit_kernel<{epi}, {'true' if d % 4 == 0 else 'false'}>"
-    wide = 128 < d <= 256                    # the d = 256 kernels; narrower rows are padded with zeros in LDS
-    pad = ", true" if wide and d != 256 else ""
-    if storage == "bf16" and (d in (64, 128) or wide):
-        nqt, ks = (1, 16) if wide else (2, d // 16)
-        if epi == "RankEpi":
-            return f"qstream_kernel<RankFastEpi, {nqt}, 8, 2, {ks}{pad}>"
-        return f"qreg_async_kernel<{epi}, {nqt}, {ks}{pad}>"
-    if storage == "int8" and (d in (64, 128) or wide):
-        if d == 128 and epi == "TopkEpi":
-            return "topk_i8_filter_kernel"
-        return f"qreg_i8_kernel<{epi}, {1 if wide else 2}, {16 if wide else d // 16}{pad}>"
-    if d > 128:
+    if d > 256:
         return f"kchunk_kernel<{epi}>"
-    return f"qreg_kernel<{storage}, {epi}>"
+    lds_d = 64 if d <= 64 else 128 if d <= 128 else 256   # LDS row of the instantiation; narrower rows are zero-padded
+    pad = ", true" if d != lds_d else ", false"
+    nqt = 1 if lds_d == 256 else 2
+    if storage == "bf16":
+        if epi == "RankEpi":
+            return f"qstream_kernel<RankFastEpi, {nqt}, 8, 2, {lds_d // 16}{pad}>"
+        return f"qreg_async_kernel<{epi}, {nqt}, {lds_d // 16}{pad}>"
+    if d == 128 and epi == "TopkEpi":
+        return "topk_i8_filter_kernel"
+    return f"qreg_i8_kernel<{epi}, {nqt}, {lds_d // 16}{pad}>"
 
 
 def main():

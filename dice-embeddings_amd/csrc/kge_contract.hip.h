@@ -1,11 +1,10 @@
 // Query x all-entity contraction on MFMA with fused epilogues (gfx950).
 //
 // All main loops run on the bf16 MFMA (32x32x16) and share one epilogue interface:
-//   qreg_async_kernel   bf16 table, d == 64, 128 or 129..256: persistent, queries register-resident, entity rows
-//                       global -> LDS
+//   qreg_async_kernel   bf16 table, d <= 256 (LDS rows of 64, 128 or 256 elements, narrower table rows zero-padded
+//                       there): persistent, queries register-resident, entity rows global -> LDS
 //   qstream_kernel      the same with a deeper pipeline and the epilogue inside the MFMA chain (filtered rank, scores)
 //   qreg_i8_kernel      per-row int8 table, the same widths and walk, rows widened to bf16 on the way into LDS
-//   qreg_kernel         bf16 / int8 with d < 128 (other than 64)
 //   kchunk_kernel       bf16 / int8 with d > 256: K in chunks of 64 through LDS
 //   ksplit_kernel       fp32 tables, any d: every operand as three bf16 parts, six part products per product
 // Reduction order of one score is fixed (k ascending in steps of the MFMA depth, nothing else), so
@@ -885,163 +884,13 @@ struct MinMaxEpi {
   }
 };
 
-// ============================================================================================
-// qreg_kernel: bf16 MFMA, register-stationary queries, LDS-streamed entity rows.
-// ============================================================================================
-constexpr int QREG_NQT = 2;            // 32-query tiles per wave
-constexpr int QREG_WG_QUERIES = 256;   // 4 waves x 64 queries
-constexpr int QREG_STAGE_ROWS = 64;
-constexpr int QREG_ROW_BYTES = 272;    // 256 B of bf16 + 16 B pad: conflict-free ds_read_b128 across rows
-
-template <int EDT, template <int> class EpiT>
-__global__ void __launch_bounds__(256, 2) qreg_kernel(ContractArgs a, typename EpiT<QREG_NQT>::Args ea) {
-  using Epi = EpiT<QREG_NQT>;
-  constexpr bool HAS_SCALE = (EDT == KGE_I8);
-  __shared__ __attribute__((aligned(16))) unsigned char lds_e[2][QREG_STAGE_ROWS * QREG_ROW_BYTES];
-  __shared__ float lds_sc[2][QREG_STAGE_ROWS];
-
-  int qg;
-  int64_t chunk;
-  if (!decompose_wg(a, qg, chunk)) return;
-  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, c = lane & 31, hf = lane >> 5;
-  const int d = a.d;
-  const int64_t q0 = (int64_t)qg * QREG_WG_QUERIES + wave * (32 * QREG_NQT);
-
-  // ---- query fragments: lane (c, hf) holds k = 16 s + 8 hf .. +8 of query q0 + 32 t + c ----
-  bf16x8 qf[QREG_NQT][8];
-#pragma unroll
-  for (int t = 0; t < QREG_NQT; ++t) {
-    const int64_t q = q0 + 32 * t + c;
-#pragma unroll
-    for (int s = 0; s < 8; ++s) {
-      const int k = 16 * s + 8 * hf;
-      f32x4 lo = {0.f, 0.f, 0.f, 0.f}, hi = {0.f, 0.f, 0.f, 0.f};
-      if (q < a.B && k < d) {
-        const f32x4* src = (const f32x4*)(a.Q + q * d + k);
-        lo = src[0];
-        hi = src[1];
-      }
-      qf[t][s] = cvt_bf16x8(lo, hi);
-    }
-  }
-  Epi epi;
-  epi.init(ea, q0, c, hf, a.B);
-  __shared__ typename Epi::Shared epi_sh;
-  epi.bind(&epi_sh);
-
-  const int64_t r0 = a.e_begin + chunk * a.chunk_rows;
-  const int64_t r1 = (r0 + a.chunk_rows < a.e_end) ? r0 + a.chunk_rows : a.e_end;
-  const int nst = (int)((r1 - r0 + QREG_STAGE_ROWS - 1) / QREG_STAGE_ROWS);
-
-  constexpr int NLD = (EDT == KGE_BF16) ? 4 : 2;
-  u32x4 stage[NLD];
-  float stage_sc = 0.f;
-
-  auto stage_load = [&](int64_t row0) {
-    if (EDT == KGE_BF16) {
-#pragma unroll
-      for (int j = 0; j < NLD; ++j) {
-        const int idx = tid + 256 * j, row = idx >> 4, piece = idx & 15;
-        const int64_t g = row0 + row;
-        u32x4 v = {0u, 0u, 0u, 0u};
-        if (g < r1 && piece * 8 < d) v = *(const u32x4*)((const uint16_t*)a.E + g * d + piece * 8);
-        stage[j] = v;
-      }
-    } else {
-#pragma unroll
-      for (int j = 0; j < NLD; ++j) {
-        const int idx = tid + 256 * j, row = idx >> 3, piece = idx & 7;
-        const int64_t g = row0 + row;
-        u32x4 v = {0u, 0u, 0u, 0u};
-        if (g < r1 && piece * 16 < d) v = *(const u32x4*)((const int8_t*)a.E + g * d + piece * 16);
-        stage[j] = v;
-      }
-      if (tid < QREG_STAGE_ROWS) stage_sc = (row0 + tid < r1) ? a.scale[row0 + tid] : 0.f;
-    }
-  };
-  auto stage_store = [&](int buf) {
-    if (EDT == KGE_BF16) {
-#pragma unroll
-      for (int j = 0; j < NLD; ++j) {
-        const int idx = tid + 256 * j, row = idx >> 4, piece = idx & 15;
-        *(u32x4*)(&lds_e[buf][row * QREG_ROW_BYTES + piece * 16]) = stage[j];
-      }
-    } else {
-#pragma unroll
-      for (int j = 0; j < NLD; ++j) {
-        const int idx = tid + 256 * j, row = idx >> 3, piece = idx & 7;
-        unsigned char* dst = &lds_e[buf][row * QREG_ROW_BYTES + piece * 32];
-        *(u32x4*)(dst) = i8x8_to_bf16x8(stage[j][0], stage[j][1]);
-        *(u32x4*)(dst + 16) = i8x8_to_bf16x8(stage[j][2], stage[j][3]);
-      }
-      if (tid < QREG_STAGE_ROWS) lds_sc[buf][tid] = stage_sc;
-    }
-  };
-
-  // Software pipeline over the 32x32 tiles: the MFMA chain of tile j is issued together with the
-  // epilogue of tile j-1 (they are independent), and the scheduler is told to interleave them, so
-  // the VALU compare/count work of one tile hides under the matrix pipe time of the next.
-  constexpr int ET = QREG_STAGE_ROWS / 32;
-  constexpr int TILES = ET * QREG_NQT;
-  f32x16 acc_prev;
-#pragma unroll
-  for (int i = 0; i < 16; ++i) acc_prev[i] = 0.f;
-  float sc_prev[16];
-#pragma unroll
-  for (int i = 0; i < 16; ++i) sc_prev[i] = 0.f;
-  float sc_col_prev = 0.f;
-  int64_t e_prev = r1;  // "nothing to do" for the first epilogue: a tile entirely past the limit
-
-  stage_load(r0);
-  stage_store(0);
-  __syncthreads();
-  for (int st = 0; st < nst; ++st) {
-    const int buf = st & 1;
-    const int64_t row0 = r0 + (int64_t)st * QREG_STAGE_ROWS;
-    if (st + 1 < nst) stage_load(row0 + QREG_STAGE_ROWS);
-    bf16x8 ef[ET][8];
-#pragma unroll
-    for (int et = 0; et < ET; ++et) {
-      const unsigned char* src = &lds_e[buf][(et * 32 + c) * QREG_ROW_BYTES + hf * 16];
-#pragma unroll
-      for (int s = 0; s < 8; ++s) ef[et][s] = *(const bf16x8*)(src + s * 32);
-    }
-#pragma unroll
-    for (int j = 0; j < TILES; ++j) {
-      const int et = j / QREG_NQT, t = j % QREG_NQT;
-      const int t_prev = (j + QREG_NQT - 1) % QREG_NQT;
-      f32x16 acc;
-#pragma unroll
-      for (int i = 0; i < 16; ++i) acc[i] = 0.f;
-#pragma unroll
-      for (int s = 0; s < 8; ++s)
-        acc = Epi::SWAP ? mfma_bf16(qf[t][s], ef[et][s], acc) : mfma_bf16(ef[et][s], qf[t][s], acc);
-      epi.template tile<HAS_SCALE>(t_prev, acc_prev, sc_prev, sc_col_prev, e_prev, r1);
-      acc_prev = acc;
-      e_prev = row0 + et * 32;
-      if (HAS_SCALE) {
-        if (Epi::SWAP) {
-          sc_col_prev = lds_sc[buf][et * 32 + c];
-        } else if (t == 0) {
-#pragma unroll
-          for (int i = 0; i < 16; ++i) sc_prev[i] = lds_sc[buf][et * 32 + row_of(i, hf)];
-        }
-      }
-    }
-    if (st + 1 < nst) stage_store(buf ^ 1);
-    if (Epi::STAGE_HOOK) epi.stage_mark();
-    __syncthreads();
-    if (Epi::STAGE_HOOK) epi.stage_end();
-  }
-  epi.template tile<HAS_SCALE>(QREG_NQT - 1, acc_prev, sc_prev, sc_col_prev, e_prev, r1);
-  epi.finish();
-}
+constexpr int QREG_NQT = 2;            // 32-query tiles per wave in the d <= 128 forms of the persistent kernels
 
 // ============================================================================================
-// qreg_async_kernel: the bf16, d == 128 fast path.  Same tiles, same reduction order and same
-// epilogues as qreg_kernel, but entity rows go from global memory straight into LDS
-// (global_load_lds_dwordx4: no staging registers, no ds_write), in 128-row stages, and each wave
-// prefetches the next stage while it computes the current one.
+// qreg_async_kernel: bf16 tables up to 256 elements wide (written for d == 128).  Queries live in registers as MFMA
+// fragments; entity rows go from global memory straight into LDS (global_load_lds_dwordx4: no staging
+// registers, no ds_write), in 128-row stages, and each wave prefetches the next stage while it computes the
+// current one.
 //
 // LDS layout of a stage: row r is 256 B = 16 pieces of 16 B; piece p of row r sits in slot
 // r*16 + (p ^ (r & 15)).  A direct-to-LDS load writes 64 consecutive slots per wave, so the swizzle

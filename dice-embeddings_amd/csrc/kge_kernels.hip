@@ -1170,18 +1170,25 @@ int check_contract(const char* who, const float* Q, const void* E, int dtype, co
   return st.ok() ? KGE_OK : set_error(st.code, "%s", st.msg);
 }
 
-// bf16 rows of d == 256 go through the persistent kernels with ONE query tile per wave (256-query workgroups): the 16
-// query fragments of a 512-byte row still fit the register file beside the 16 entity fragments.  The filtered rank
-// and kge_scores take the streaming kernel, which runs the previous tile's epilogue inside the MFMA chain and suits a
-// short branch-free one (the deferred rank count, a plain store: 2.0x and 1.5x faster than kchunk_kernel) and not
-// the branching or long ones (there top-k and row extrema are 10 % slower, BCE twice as slow); those take
-// qreg_async_kernel, epilogue after the chain.
-// bf16 rows of d == 64 take the same two kernels in the d == 128 workgroup shape, with four K steps.
-// Rows between 128 and 256 elements take the same kernels with 512-byte LDS rows whose tail stays zero (PAD): the
-// chain runs its sixteen K steps, the last ones on zeros (d = 200: 0.78 of the d = 256 rate per useful product,
-// against half of it in kchunk_kernel).
+// bf16 and int8 tables up to 256 elements wide run the persistent kernels, instantiated for LDS rows of 64, 128 or 256
+// elements; a table whose rows are narrower than the LDS row of its class takes the PAD form of the same kernel
+// (the row's tail stays zero in LDS: d = 200 runs at 0.78 of the d = 256 rate per useful product, against half of
+// it in kchunk_kernel; below 64 a tile is bound by its epilogue, not by its K steps, and d = 32 runs at the
+// scores-per-second of d = 64).  The 256 class keeps ONE query tile per wave (256-query workgroups): the 16 query
+// fragments of a 512-byte row still fit the register file beside the 16 entity fragments.  In the 64 and 256
+// classes the filtered rank and kge_scores take the streaming kernel, which runs the previous tile's epilogue inside
+// the MFMA chain and suits a short branch-free one (the deferred rank count, a plain store) and not the branching or
+// long ones (top-k and row extrema 10 % slower there, BCE twice as slow); those take qreg_async_kernel, epilogue
+// after the chain.  Wider tables: kchunk_kernel.
+struct RowClass {
+  int lds_d;  // elements of an LDS row: 64, 128, 256; 0: wider than any persistent kernel's
+  bool pad;   // the table's rows are narrower than that
+};
+static inline RowClass row_class(int64_t d) {
+  const int w = d <= 64 ? 64 : d <= 128 ? 128 : d <= 256 ? 256 : 0;
+  return RowClass{w, w != 0 && d != w};
+}
 constexpr int QS256_WG_QUERIES = QA_WG_WAVES * 32;
-static inline bool rows_up_to_256(int64_t d) { return d > 128 && d <= 256; }
 template <template <int> class EpiT>
 constexpr bool stream256_epilogue() {
   return std::is_same<EpiT<2>, RankEpi<2>>::value || std::is_same<EpiT<2>, StoreEpi<2>>::value;
@@ -1200,15 +1207,12 @@ ContractArgs make_args(const float* Q, const void* E, int dtype, const float* sc
   a.ldq = a.lde = 0;
   a.k_split_len = 0;
   a.persistent = 0;
-  const bool stream64 = dtype == KGE_BF16 && d == 64;  // (persistent whatever the epilogue)
-  const bool stream256 = dtype == KGE_BF16 && rows_up_to_256(d);  // (persistent whatever the epilogue)
-  const bool i8_256 = (dtype == KGE_I8 && rows_up_to_256(d));  // qreg_i8_kernel with one query tile per wave, every epilogue
-  const bool fast_bf16 = (dtype == KGE_BF16 && d == 128) || stream256 || stream64;
-  const bool i8_64 = (dtype == KGE_I8 && d == 64);    // the same kernel in the d == 128 shape with four K steps
-  const bool fast_i8 = (dtype == KGE_I8 && d == 128) || i8_256 || i8_64;
-  const bool wide_bf16 = ((dtype == KGE_BF16 || dtype == KGE_I8) && d > 128) && !stream256 && !i8_256;  // kchunk_kernel: the workgroup shape of the split kernel
-  const int wgq = (dtype == KGE_F32) ? KS_WG_QUERIES : (stream256 || i8_256) ? QS256_WG_QUERIES : fast_bf16 ? QA_WG_QUERIES
-                  : fast_i8 ? I8_WG_QUERIES : wide_bf16 ? KS_WG_QUERIES : QREG_WG_QUERIES;
+  const RowClass rc = row_class(d);
+  const bool fast_bf16 = dtype == KGE_BF16 && rc.lds_d != 0;  // (persistent whatever the epilogue)
+  const bool fast_i8 = dtype == KGE_I8 && rc.lds_d != 0;
+  const bool wide_bf16 = (dtype == KGE_BF16 || dtype == KGE_I8) && rc.lds_d == 0;  // kchunk_kernel: the workgroup shape of the split kernel
+  const int wgq = (dtype == KGE_F32 || wide_bf16) ? KS_WG_QUERIES : rc.lds_d == 256 ? QS256_WG_QUERIES
+                  : fast_bf16 ? QA_WG_QUERIES : I8_WG_QUERIES;
   a.n_qgroups = (int)((B + wgq - 1) / wgq);
   if (a.n_qgroups < 1) a.n_qgroups = 1;
   const int64_t rows = e_end - e_begin;
@@ -1227,14 +1231,12 @@ ContractArgs make_args(const float* Q, const void* E, int dtype, const float* sc
     a.persistent = 1;
     return a;
   }
-  // non-persistent paths: one workgroup per (query group, chunk).  `resident` workgroups run at a time
-  // (2 per CU, or 1 per CU for the 8-wave split kernel); choose the chunk length whose last round of
+  // non-persistent paths (the split kernel and kchunk_kernel: 8-wave workgroups of 256 entity rows, one per CU): one
+  // workgroup per (query group, chunk), `resident` workgroups at a time; choose the chunk length whose last round of
   // workgroups is fullest, preferring longer chunks (less per-workgroup set-up) among near-equal candidates.
-  const bool f32_split = (dtype == KGE_F32);
-  const bool big_tile = f32_split || wide_bf16;  // 8-wave workgroups of 256 entity rows, one per CU
-  const int tile = big_tile ? KS_TILE_ROWS : QREG_STAGE_ROWS;
-  const int max_chunk = (dtype == KGE_F32 || wide_bf16) ? 1024 : 2048;
-  const int64_t resident = big_tile ? 256 : 512;
+  const int tile = KS_TILE_ROWS;
+  const int max_chunk = 1024;
+  const int64_t resident = 256;
   int64_t best_chunk = tile;
   double best_eff = -1.0;
   for (int64_t chunk = tile; chunk <= max_chunk; chunk += tile) {
@@ -1291,21 +1293,19 @@ struct LaunchTimer {
 template <template <int> class EpiT, class EArgs>
 int launch_contract(int dtype, const ContractArgs& a, const EArgs& ea, hipStream_t st, const char* name) {
   if (a.B == 0 || a.e_end <= a.e_begin) return KGE_OK;
-  const bool i8_256 = (dtype == KGE_I8 && rows_up_to_256(a.d));
-  const bool pad = a.d != 256;  // (of the two cases above: rows narrower than the LDS rows)
-  const bool i8_64 = (dtype == KGE_I8 && a.d == 64);
-  const bool fast_i8 = (dtype == KGE_I8 && a.d == 128) || i8_256 || i8_64;
-  const bool stream256 = dtype == KGE_BF16 && rows_up_to_256(a.d);
-  const bool stream64 = dtype == KGE_BF16 && a.d == 64;
-  const bool persistent = (dtype == KGE_BF16 && a.d == 128) || fast_i8 || stream256 || stream64;
+  const RowClass rc = row_class(a.d);
+  const bool fast_bf16 = dtype == KGE_BF16 && rc.lds_d != 0;
+  const bool fast_i8 = dtype == KGE_I8 && rc.lds_d != 0;
+  const bool persistent = fast_bf16 || fast_i8;
+  const bool pad = rc.pad;
   // (make_args and this function both decide, from the table, between the persistent and the tiled kernels; a plan
   // made for the other kind would be read as garbage, so the two must not drift apart)
   KGE_REQUIRE((a.persistent != 0) == persistent, KGE_ERR_INVALID, "%s: work decomposition planned for another kernel", name);
   const int64_t nwg = persistent ? 8 * (int64_t)a.n_qgroups * a.n_lanes : contract_grid_wgs(a);
   KGE_REQUIRE(nwg <= 0x7fffffffLL, KGE_ERR_INVALID, "%s: grid of %lld workgroups too large", name, (long long)nwg);
   const bool f32_split = (dtype == KGE_F32);
-  const bool wide_bf16 = ((dtype == KGE_BF16 || dtype == KGE_I8) && a.d > 128) && !stream256 && !i8_256;
-  dim3 grid((unsigned)nwg), block(fast_i8 ? 64 * I8_WG_WAVES : persistent ? 64 * QA_WG_WAVES : (f32_split || wide_bf16) ? 512 : 256);
+  const bool wide_bf16 = (dtype == KGE_BF16 || dtype == KGE_I8) && rc.lds_d == 0;
+  dim3 grid((unsigned)nwg), block(fast_i8 ? 64 * I8_WG_WAVES : persistent ? 64 * QA_WG_WAVES : 512);
   LaunchTimer timer;
   if (int trc = timer.begin(st)) return trc;
   const bool rows_aligned = (a.d % 4 == 0) && (((uintptr_t)a.E | (uintptr_t)a.Q) % 16 == 0);
@@ -1313,51 +1313,40 @@ int launch_contract(int dtype, const ContractArgs& a, const EArgs& ea, hipStream
     hipLaunchKernelGGL((ksplit_kernel<EpiT, true>), grid, block, 0, st, a, ea);
   else if (f32_split)
     hipLaunchKernelGGL((ksplit_kernel<EpiT, false>), grid, block, 0, st, a, ea);
-  else if (dtype == KGE_BF16 && a.d == 128) {
-    // the rank epilogue has a branch-free form for the deeper-pipelined kernel (same workgroup shape, same counts)
-    if constexpr (std::is_same<EpiT<2>, RankEpi<2>>::value)
-      hipLaunchKernelGGL((qstream_kernel<RankFastEpi, QA_NQT, QA_WG_WAVES, QA_WAVES_PER_SIMD>), grid, block, 0, st, a, ea);
-    else
-      hipLaunchKernelGGL((qreg_async_kernel<EpiT>), grid, block, 0, st, a, ea);
-  }
-  else if (stream64) {
-    if constexpr (std::is_same<EpiT<2>, RankEpi<2>>::value)
-      hipLaunchKernelGGL((qstream_kernel<RankFastEpi, QA_NQT, QA_WG_WAVES, QA_WAVES_PER_SIMD, 4>), grid, block, 0, st, a, ea);
-    else
-      hipLaunchKernelGGL((qreg_async_kernel<EpiT, QA_NQT, 4>), grid, block, 0, st, a, ea);
-  }
-  else if (stream256 && !pad) {
-    if constexpr (std::is_same<EpiT<2>, RankEpi<2>>::value)
-      hipLaunchKernelGGL((qstream_kernel<RankFastEpi, 1, QA_WG_WAVES, QA_WAVES_PER_SIMD, 16>), grid, block, 0, st, a, ea);
-    else if constexpr (stream256_epilogue<EpiT>())
-      hipLaunchKernelGGL((qstream_kernel<EpiT, 1, QA_WG_WAVES, QA_WAVES_PER_SIMD, 16>), grid, block, 0, st, a, ea);
-    else
-      hipLaunchKernelGGL((qreg_async_kernel<EpiT, 1, 16>), grid, block, 0, st, a, ea);
-  }
-  else if (stream256) {
-    if constexpr (std::is_same<EpiT<2>, RankEpi<2>>::value)
-      hipLaunchKernelGGL((qstream_kernel<RankFastEpi, 1, QA_WG_WAVES, QA_WAVES_PER_SIMD, 16, true>), grid, block, 0, st, a, ea);
-    else if constexpr (stream256_epilogue<EpiT>())
-      hipLaunchKernelGGL((qstream_kernel<EpiT, 1, QA_WG_WAVES, QA_WAVES_PER_SIMD, 16, true>), grid, block, 0, st, a, ea);
-    else
-      hipLaunchKernelGGL((qreg_async_kernel<EpiT, 1, 16, true>), grid, block, 0, st, a, ea);
-  }
   else if (wide_bf16 && dtype == KGE_BF16)
     hipLaunchKernelGGL((kchunk_kernel<KGE_BF16, EpiT>), grid, block, 0, st, a, ea);
   else if (wide_bf16)
     hipLaunchKernelGGL((kchunk_kernel<KGE_I8, EpiT>), grid, block, 0, st, a, ea);
-  else if (dtype == KGE_BF16)
-    hipLaunchKernelGGL((qreg_kernel<KGE_BF16, EpiT>), grid, block, 0, st, a, ea);
-  else if (i8_256 && !pad)
-    hipLaunchKernelGGL((qreg_i8_kernel<EpiT, 1, 16>), grid, block, 0, st, a, ea);
-  else if (i8_256)
-    hipLaunchKernelGGL((qreg_i8_kernel<EpiT, 1, 16, true>), grid, block, 0, st, a, ea);
-  else if (i8_64)
-    hipLaunchKernelGGL((qreg_i8_kernel<EpiT, QREG_NQT, 4>), grid, block, 0, st, a, ea);
-  else if (fast_i8)
-    hipLaunchKernelGGL((qreg_i8_kernel<EpiT>), grid, block, 0, st, a, ea);
-  else
-    hipLaunchKernelGGL((qreg_kernel<KGE_I8, EpiT>), grid, block, 0, st, a, ea);
+  else if (fast_bf16) {
+    // the rank epilogue has a branch-free form for the deeper-pipelined kernel (same workgroup shape, same counts)
+    constexpr bool is_rank = std::is_same<EpiT<2>, RankEpi<2>>::value;
+    auto go = [&](auto nqt, auto ksteps, auto padc, auto streamed) {
+      constexpr int NQT = decltype(nqt)::value, KS = decltype(ksteps)::value;
+      constexpr bool PAD = decltype(padc)::value, STREAMED = decltype(streamed)::value;
+      if constexpr (is_rank)
+        hipLaunchKernelGGL((qstream_kernel<RankFastEpi, NQT, QA_WG_WAVES, QA_WAVES_PER_SIMD, KS, PAD>), grid, block, 0, st, a, ea);
+      else if constexpr (STREAMED)
+        hipLaunchKernelGGL((qstream_kernel<EpiT, NQT, QA_WG_WAVES, QA_WAVES_PER_SIMD, KS, PAD>), grid, block, 0, st, a, ea);
+      else
+        hipLaunchKernelGGL((qreg_async_kernel<EpiT, NQT, KS, PAD>), grid, block, 0, st, a, ea);
+    };
+    using std::integral_constant;
+    constexpr bool s256 = stream256_epilogue<EpiT>();
+    if (rc.lds_d == 128 && !pad) go(integral_constant<int, QA_NQT>{}, integral_constant<int, 8>{}, std::false_type{}, std::false_type{});
+    else if (rc.lds_d == 128) go(integral_constant<int, QA_NQT>{}, integral_constant<int, 8>{}, std::true_type{}, std::false_type{});
+    else if (rc.lds_d == 64 && !pad) go(integral_constant<int, QA_NQT>{}, integral_constant<int, 4>{}, std::false_type{}, std::false_type{});
+    else if (rc.lds_d == 64) go(integral_constant<int, QA_NQT>{}, integral_constant<int, 4>{}, std::true_type{}, std::false_type{});
+    else if (!pad) go(integral_constant<int, 1>{}, integral_constant<int, 16>{}, std::false_type{}, integral_constant<bool, s256>{});
+    else go(integral_constant<int, 1>{}, integral_constant<int, 16>{}, std::true_type{}, integral_constant<bool, s256>{});
+  }
+  else {
+    if (rc.lds_d == 128 && !pad) hipLaunchKernelGGL((qreg_i8_kernel<EpiT, QREG_NQT, 8, false>), grid, block, 0, st, a, ea);
+    else if (rc.lds_d == 128) hipLaunchKernelGGL((qreg_i8_kernel<EpiT, QREG_NQT, 8, true>), grid, block, 0, st, a, ea);
+    else if (rc.lds_d == 64 && !pad) hipLaunchKernelGGL((qreg_i8_kernel<EpiT, QREG_NQT, 4, false>), grid, block, 0, st, a, ea);
+    else if (rc.lds_d == 64) hipLaunchKernelGGL((qreg_i8_kernel<EpiT, QREG_NQT, 4, true>), grid, block, 0, st, a, ea);
+    else if (!pad) hipLaunchKernelGGL((qreg_i8_kernel<EpiT, 1, 16, false>), grid, block, 0, st, a, ea);
+    else hipLaunchKernelGGL((qreg_i8_kernel<EpiT, 1, 16, true>), grid, block, 0, st, a, ea);
+  }
   KGE_LAUNCH_CHECK(name);
   if (int trc = timer.end()) return trc;
   return KGE_OK;
