@@ -273,7 +273,7 @@ def test_predict_topk_and_predict_invariants():
         kge.predict_topk(h=3, r=["r0"])
 
 
-@pytest.mark.parametrize("d", [64, 128, 256])          # the three widths with kernels of their own
+@pytest.mark.parametrize("d", [32, 64, 96, 128, 192, 256, 320])   # LDS rows of 64, 128, 256 (exact and zero-padded); wider
 @pytest.mark.parametrize("storage", ["bf16", "int8"])
 def test_quantised_storage_follows_dequantised_fp32_math(storage, d):
     m, triples = _toy("QMult" if storage == "bf16" else "DistMult", d, N=3000, R=11, n=600, seed=7)
