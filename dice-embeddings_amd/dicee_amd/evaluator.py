@@ -62,11 +62,17 @@ class _BatchStreams:
     (query vectors, filter rows, plan, thresholds, main loop, correction); two chains side by side fill the gaps each
     leaves (ComplEx, 14,541 entities, batches of 1024: 0.117 -> 0.075 ms per batch).  The first batch runs on the
     caller's stream, so that whatever the model derives lazily (its quantised table) exists before the streams
-    fork; ``join()`` makes the caller's stream wait for all of them."""
+    fork; ``join()`` makes the caller's stream wait for all of them.  ``scores_per_batch`` (batch size x entities),
+    when given and below a million, keeps everything on the caller's stream: a batch that small is shorter than
+    what crossing streams costs (135 entities, batches of 512: 0.056 -> 0.065 ms per batch on two streams)."""
 
-    def __init__(self, device, n):
+    SMALL_BATCH = 1_000_000
+
+    def __init__(self, device, n, scores_per_batch=None):
         self.cur = torch.cuda.current_stream(device)
         self.n = max(1, int(n))
+        if scores_per_batch is not None and scores_per_batch < self.SMALL_BATCH:
+            self.n = 1
         self.device = device
         self.pool = None
         self.i = 0
@@ -290,7 +296,7 @@ class Evaluator:
         all_trip = torch.from_numpy(np.ascontiguousarray(triple_idx.astype(np.int64))).to(dev)
         out = torch.empty((num_triples,), dtype=torch.int64, device=dev)
         bs = int(self.args.batch_size)
-        lanes = _BatchStreams(dev, self.streams)
+        lanes = _BatchStreams(dev, self.streams, bs * model.num_entities)
         with torch.no_grad():
             for i in range(0, num_triples, bs):
                 with lanes.next():
@@ -320,7 +326,7 @@ class Evaluator:
         all_trip = torch.from_numpy(np.ascontiguousarray(triple_idx.astype(np.int64))).to(dev)
         out = torch.empty((num_triples,), dtype=torch.int64, device=dev)
         bs = int(self.args.batch_size)
-        lanes = _BatchStreams(dev, self.streams)
+        lanes = _BatchStreams(dev, self.streams, bs * model.num_entities)
         with torch.no_grad():
             for i in range(0, num_triples, bs):
                 with lanes.next():

@@ -66,7 +66,7 @@ def evaluate_lp(model, triple_idx, num_entities=None, er_vocab=None, re_vocab=No
     tail_ranks = torch.empty((n,), dtype=torch.int64, device=dev)
     head_ranks = torch.empty((n,), dtype=torch.int64, device=dev)
     bs = int(batch_size)
-    lanes = _BatchStreams(dev, streams)
+    lanes = _BatchStreams(dev, streams, bs * N)
     for i in range(0, n, bs):
         b = trip[i:i + bs]
         with lanes.next():
@@ -114,7 +114,7 @@ def evaluate_link_prediction_performance_with_reciprocals(model, triples, er_voc
     n = len(ids)
     bs = int(net.args.get("batch_size", 1024) or 1024)
     out = torch.empty((n,), dtype=torch.int64, device=dev)
-    lanes = _BatchStreams(dev, streams)
+    lanes = _BatchStreams(dev, streams, bs * net.num_entities)
     for i in range(0, n, bs):
         b = trip[i:i + bs]
         with lanes.next():

@@ -126,7 +126,8 @@ def test_evaluator_matches_the_reference_loop(name, d, extra, batch_size):
 def test_evaluator_batches_on_alternating_streams_give_the_same_ranks(storage):
     """The batches of an evaluation alternate over two streams by default.  Whatever the number of streams, the ranks
     are those of the one-stream evaluation; with quantised storage the table's snapshot is taken lazily by the first
-    batch, before the streams fork."""
+    batch, before the streams fork.  (Batches of 512 against 3000 entities: above the size below which the evaluator
+    keeps to one stream.)"""
     from dicee_amd import Evaluator
     m, triples = _toy("DistMult", 64, N=3000, R=11, n=6000, seed=11)
     er = {}
@@ -135,7 +136,7 @@ def test_evaluator_batches_on_alternating_streams_give_the_same_ranks(storage):
     ranks = {}
     for streams in (1, 2, 3):
         model = m.to("cuda").set_entity_storage(storage)           # (a fresh snapshot for every run)
-        ev = Evaluator(SimpleNamespace(batch_size=256, eval_model="test", scoring_technique="KvsAll",
+        ev = Evaluator(SimpleNamespace(batch_size=512, eval_model="test", scoring_technique="KvsAll",
                                        full_storage_path=None), streams=streams)
         ev.set_filter(er, num_relations=11)
         ev.evaluate_lp_k_vs_all(model, triples, form_of_labelling="EntityPrediction")
@@ -150,7 +151,7 @@ def test_evaluator_batches_on_alternating_streams_give_the_same_ranks(storage):
     dev_trip = torch.from_numpy(triples.astype(np.int64)).cuda()
     er_csr = FilterCSR.from_triples_gpu(dev_trip, 3000, 11, kind="er")
     re_csr = FilterCSR.from_triples_gpu(dev_trip, 3000, 11, kind="re")
-    both = {s: evaluate_lp(model, triples, 3000, er_csr, re_csr, info=None, batch_size=256, return_ranks=True,
+    both = {s: evaluate_lp(model, triples, 3000, er_csr, re_csr, info=None, batch_size=512, return_ranks=True,
                            streams=s) for s in (1, 2, 3)}
     for s in (2, 3):
         assert both[s][0] == both[1][0]
