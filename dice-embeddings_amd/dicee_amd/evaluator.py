@@ -13,6 +13,7 @@ gives it; every such position lies in ``[1 + n_greater, 1 + n_greater + n_equal]
 the representative reported here: ``"stable"`` (default; what a stable descending sort gives:
 ties ordered by entity id), ``"optimistic"``, ``"pessimistic"`` or ``"mean"``.
 """
+import contextlib
 import json
 import os
 from types import SimpleNamespace
@@ -69,10 +70,11 @@ class _BatchStreams:
     SMALL_BATCH = 1_000_000
 
     def __init__(self, device, n, scores_per_batch=None):
-        self.cur = torch.cuda.current_stream(device)
         self.n = max(1, int(n))
         if scores_per_batch is not None and scores_per_batch < self.SMALL_BATCH:
             self.n = 1
+        # (a model on the CPU has no stream: the first rank call raises what the ops raise for CPU tensors)
+        self.cur = torch.cuda.current_stream(device) if torch.device(device).type == "cuda" else None
         self.device = device
         self.pool = None
         self.i = 0
@@ -80,6 +82,8 @@ class _BatchStreams:
     def next(self):
         """Context manager for the next batch."""
         self.i += 1
+        if self.cur is None:
+            return contextlib.nullcontext()
         if self.n == 1 or self.i == 1:
             return torch.cuda.stream(self.cur)
         if self.pool is None:

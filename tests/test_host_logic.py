@@ -186,6 +186,23 @@ def test_models_mirror_reference_parameters_and_have_no_cpu_fallback():
         hd(torch.zeros((2, 2), dtype=torch.int64))
 
 
+def test_evaluating_a_model_on_the_cpu_raises_what_the_ops_raise():
+    """There is no CPU path: an evaluation of a model that was never moved to the GPU fails with the ops' own error
+    (not with one about streams from the evaluator's batch pipelining)."""
+    from types import SimpleNamespace
+    from dicee_amd import Evaluator, models
+    from dicee_amd.link_prediction import evaluate_lp
+    m = models.DistMult({"model": "DistMult", "embedding_dim": 32, "num_entities": 50, "num_relations": 5})
+    tr = np.stack([np.arange(20) % 50, np.arange(20) % 5, (np.arange(20) * 7) % 50], 1)
+    ev = Evaluator(SimpleNamespace(batch_size=16, eval_model="test", scoring_technique="KvsAll", full_storage_path=None))
+    with pytest.raises(RuntimeError, match="GPU"):
+        ev.evaluate_lp_k_vs_all(m, tr, form_of_labelling="EntityPrediction")
+    er = {(int(h), int(r)): [int(t)] for h, r, t in tr}
+    re_ = {(int(r), int(t)): [int(h)] for h, r, t in tr}
+    with pytest.raises(RuntimeError, match="GPU"):
+        evaluate_lp(m, tr, 50, er, re_, info=None, batch_size=16)
+
+
 def test_synthetic_configs_small_scale():
     from dicee_amd import synthetic
     c1 = synthetic.make_config("c1")
