@@ -1781,17 +1781,29 @@ __global__ void __launch_bounds__(512, 2) kchunk_kernel(ContractArgs a, typename
   u32x4 se[4];
   f32x4 sq[4];
   bool st_e_ok = false, st_q_ok = false, ld_e_ok = false, ld_q_ok = false;
+  bool st_tail = false, ld_tail = false;  // (uniform) the chunk reaches past d: only then is anything masked
   int ld_kc = 0;
   int64_t ld_row = r0 + e_row;
-  auto chunk_load = [&]() {
-    const int ke = ld_kc * KB_KC + 8 * e_piece, kq = ld_kc * KB_KC + 4 * q_piece;
-    ld_e_ok = ke < d;  // d % 8 == 0: a piece is inside d or outside as a whole
-    ld_q_ok = kq < d;
+  // the rows of the entity tile being requested, as pointers: recomputed when the tile changes, not per chunk
+  const unsigned char* e_ptr[4];
+  auto tile_rows = [&]() {
 #pragma unroll
     for (int g = 0; g < 4; ++g) {
       int64_t er = ld_row + 64 * g;
       er = er < e_last ? er : e_last;
-      const unsigned char* src = Eb + (er * d + (ld_e_ok ? ke : 0)) * ESZ;
+      e_ptr[g] = Eb + er * d * ESZ;
+    }
+  };
+  tile_rows();
+  auto chunk_load = [&]() {
+    const int ke = ld_kc * KB_KC + 8 * e_piece, kq = ld_kc * KB_KC + 4 * q_piece;
+    ld_e_ok = ke < d;  // d % 8 == 0: a piece is inside d or outside as a whole
+    ld_q_ok = kq < d;
+    ld_tail = (ld_kc + 1) * KB_KC > d;
+    const int e_col = (ld_e_ok ? ke : 0) * ESZ;
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const unsigned char* src = e_ptr[g] + e_col;
       if (I8) {
         const u32x2 w = *(const u32x2*)src;
         se[g] = u32x4{w[0], w[1], 0u, 0u};
@@ -1800,9 +1812,13 @@ __global__ void __launch_bounds__(512, 2) kchunk_kernel(ContractArgs a, typename
       }
       sq[g] = *(const f32x4*)(q_ptr[g] + (ld_q_ok ? kq : 0));
     }
-    const bool wrap = (ld_kc == nkc - 1);
-    ld_kc = wrap ? 0 : ld_kc + 1;
-    ld_row += wrap ? KS_TILE_ROWS : 0;
+    if (ld_kc == nkc - 1) {  // (uniform)
+      ld_kc = 0;
+      ld_row += KS_TILE_ROWS;
+      tile_rows();
+    } else {
+      ++ld_kc;
+    }
   };
   const int e_off = e_row * 128 + ((e_piece ^ (e_row & 7)) << 4);
   const int q_off = q_row * 128 + ((((q_piece >> 1) ^ (q_row & 7)) << 4) | ((q_piece & 1) << 3));
@@ -1811,12 +1827,14 @@ __global__ void __launch_bounds__(512, 2) kchunk_kernel(ContractArgs a, typename
 #pragma unroll
     for (int g = 0; g < 4; ++g) {
       u32x4 v = I8 ? i8x8_to_bf16x8(se[g][0], se[g][1]) : se[g];
-#pragma unroll
-      for (int j = 0; j < 4; ++j) v[j] = st_e_ok ? v[j] : 0u;
-      *(u32x4*)(base + g * 8192 + e_off) = v;
       f32x4 w = sq[g];
+      if (__builtin_expect(st_tail, 0)) {
 #pragma unroll
-      for (int j = 0; j < 4; ++j) w[j] = st_q_ok ? w[j] : 0.f;
+        for (int j = 0; j < 4; ++j) v[j] = st_e_ok ? v[j] : 0u;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) w[j] = st_q_ok ? w[j] : 0.f;
+      }
+      *(u32x4*)(base + g * 8192 + e_off) = v;
       bf16x4 b;
       b[0] = (__bf16)w[0]; b[1] = (__bf16)w[1]; b[2] = (__bf16)w[2]; b[3] = (__bf16)w[3];
       *(bf16x4*)(base + KB_E_PLANE + g * 4096 + q_off) = b;
@@ -1839,6 +1857,7 @@ __global__ void __launch_bounds__(512, 2) kchunk_kernel(ContractArgs a, typename
     chunk_load();
     st_e_ok = ld_e_ok;
     st_q_ok = ld_q_ok;
+    st_tail = ld_tail;
     chunk_store(0);
     chunk_load();  // past the last chunk the clamped addresses still point into the tables
   }
@@ -1850,6 +1869,7 @@ __global__ void __launch_bounds__(512, 2) kchunk_kernel(ContractArgs a, typename
     // chunk it+1 (loaded during the previous iteration) goes to the other buffer, then chunk it+2 is requested
     st_e_ok = ld_e_ok;
     st_q_ok = ld_q_ok;
+    st_tail = ld_tail;
     chunk_store(buf ^ 1);
     chunk_load();
     const unsigned char* be = lds + buf * KB_STAGE_BYTES + (64 * we) * 128;
