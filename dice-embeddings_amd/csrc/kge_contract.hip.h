@@ -1720,8 +1720,8 @@ __global__ void __launch_bounds__(512, 2) ksplit_kernel(ContractArgs a, typename
 }
 
 // ============================================================================================
-// kchunk_kernel: bf16 or per-row int8 table of any width (d % 8 == 0); used for d > 128, where the queries no
-// longer fit the register file of the persistent kernel.  int8 rows are widened to bf16 (exactly) on the way into
+// kchunk_kernel: bf16 or per-row int8 table of any width (d % 8 == 0); used for d > 256, where the queries no
+// longer fit the register file of the persistent kernels.  int8 rows are widened to bf16 (exactly) on the way into
 // LDS and a finished tile's scores are multiplied by the row scales, as in the other int8 kernels.  The shape of ksplit_kernel with one part per operand:
 // 256 entities x 128 queries per workgroup of 8 waves (64 x 64 per wave), K in chunks of 64, both operands
 // staged through registers into double-buffered LDS (the fp32 queries are rounded to bf16 on the way, as in
