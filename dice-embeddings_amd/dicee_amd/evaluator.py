@@ -97,6 +97,28 @@ class _BatchStreams:
             self.cur.wait_stream(s)
 
 
+def rank_in_batches(model, x_all, target_all, csr, batch_size, tie="stable", streams=2, heads=False):
+    """Ranks (int64 tensor [n] on the model's device) of ``target_all`` [n] for the queries ``x_all`` [n,2]: one fused
+    rank call per batch of ``batch_size`` queries, each writing its counters straight into the evaluation's arrays
+    (no per-batch copies or conversions: the batch is then nothing but the library's own launches), consecutive
+    batches on alternating streams, the ranks formed once at the end."""
+    from .ops import _RANK_OUT
+    n = int(x_all.shape[0])
+    dev = x_all.device
+    x_all = x_all.contiguous()
+    target_all = target_all.contiguous()
+    counts = {k: torch.empty((n,), dtype=dt, device=dev) for k, dt in _RANK_OUT}
+    bs = int(batch_size)
+    lanes = _BatchStreams(dev, streams, bs * model.num_entities)
+    with torch.no_grad():
+        for i in range(0, n, bs):
+            with lanes.next():
+                model.rank_filtered(x_all[i:i + bs], target_all[i:i + bs], csr, heads=heads,
+                                    out={k: v[i:i + bs] for k, v in counts.items()})
+    lanes.join()
+    return ranks_from_counts(counts["n_greater"], counts["n_equal"], counts["n_equal_lower"], tie)
+
+
 class Evaluator:
     def __init__(self, args=None, is_continual_training=False, tie="stable", streams=2):
         if args is None:
@@ -298,18 +320,8 @@ class Evaluator:
         if csr.device is None or csr.device != dev:
             csr.to(dev)
         all_trip = torch.from_numpy(np.ascontiguousarray(triple_idx.astype(np.int64))).to(dev)
-        out = torch.empty((num_triples,), dtype=torch.int64, device=dev)
-        bs = int(self.args.batch_size)
-        lanes = _BatchStreams(dev, self.streams, bs * model.num_entities)
-        with torch.no_grad():
-            for i in range(0, num_triples, bs):
-                with lanes.next():
-                    batch = all_trip[i:i + bs]
-                    x = batch[:, [0, 2]].contiguous()
-                    r = batch[:, 1].contiguous()
-                    c = model.rank_filtered(x, r, csr)
-                    out[i:i + bs] = ranks_from_counts(c["n_greater"], c["n_equal"], c["n_equal_lower"], self.tie)
-        lanes.join()
+        out = rank_in_batches(model, all_trip[:, [0, 2]], all_trip[:, 1], csr, self.args.batch_size, self.tie,
+                              self.streams)
         return out.cpu().numpy()
 
     def _evaluate_entity_prediction(self, model, triple_idx, num_triples):
@@ -328,16 +340,6 @@ class Evaluator:
         if csr is not None and (csr.device is None or csr.device != dev):
             csr.to(dev)
         all_trip = torch.from_numpy(np.ascontiguousarray(triple_idx.astype(np.int64))).to(dev)
-        out = torch.empty((num_triples,), dtype=torch.int64, device=dev)
-        bs = int(self.args.batch_size)
-        lanes = _BatchStreams(dev, self.streams, bs * model.num_entities)
-        with torch.no_grad():
-            for i in range(0, num_triples, bs):
-                with lanes.next():
-                    batch = all_trip[i:i + bs]
-                    x = batch[:, :2].contiguous()
-                    t = batch[:, 2].contiguous()
-                    c = model.rank_filtered(x, t, csr)
-                    out[i:i + bs] = ranks_from_counts(c["n_greater"], c["n_equal"], c["n_equal_lower"], self.tie)
-        lanes.join()
+        out = rank_in_batches(model, all_trip[:, :2], all_trip[:, 2], csr, self.args.batch_size, self.tie,
+                              self.streams)
         return out.cpu().numpy()

@@ -13,7 +13,7 @@ import numpy as np
 import torch
 
 from .csr import FilterCSR
-from .evaluator import ranks_from_counts, _BatchStreams
+from .evaluator import rank_in_batches
 
 
 def _as_csr(vocab, key_mult, device):
@@ -63,19 +63,8 @@ def evaluate_lp(model, triple_idx, num_entities=None, er_vocab=None, re_vocab=No
     er = _as_csr(er_vocab, R, dev)
     re = _as_csr(re_vocab, N, dev)
     trip = torch.from_numpy(np.ascontiguousarray(triple_idx.astype(np.int64))).to(dev)
-    tail_ranks = torch.empty((n,), dtype=torch.int64, device=dev)
-    head_ranks = torch.empty((n,), dtype=torch.int64, device=dev)
-    bs = int(batch_size)
-    lanes = _BatchStreams(dev, streams, bs * N)
-    for i in range(0, n, bs):
-        b = trip[i:i + bs]
-        with lanes.next():
-            c = model.rank_filtered(b[:, :2].contiguous(), b[:, 2].contiguous(), er)
-            tail_ranks[i:i + bs] = ranks_from_counts(c["n_greater"], c["n_equal"], c["n_equal_lower"], tie)
-        with lanes.next():
-            c = model.rank_filtered(b[:, 1:].contiguous(), b[:, 0].contiguous(), re, heads=True)
-            head_ranks[i:i + bs] = ranks_from_counts(c["n_greater"], c["n_equal"], c["n_equal_lower"], tie)
-    lanes.join()
+    tail_ranks = rank_in_batches(model, trip[:, :2], trip[:, 2], er, batch_size, tie, streams)
+    head_ranks = rank_in_batches(model, trip[:, 1:], trip[:, 0], re, batch_size, tie, streams, heads=True)
     hr_, tr_ = head_ranks.cpu().numpy(), tail_ranks.cpu().numpy()
     divisor = float(2 * n) if n else 1.0
     results = {f"H@{k}": float((np.count_nonzero(hr_ <= k) + np.count_nonzero(tr_ <= k)) / divisor) for k in (1, 3, 10)}
@@ -113,14 +102,7 @@ def evaluate_link_prediction_performance_with_reciprocals(model, triples, er_voc
     trip = torch.from_numpy(ids).to(dev)
     n = len(ids)
     bs = int(net.args.get("batch_size", 1024) or 1024)
-    out = torch.empty((n,), dtype=torch.int64, device=dev)
-    lanes = _BatchStreams(dev, streams, bs * net.num_entities)
-    for i in range(0, n, bs):
-        b = trip[i:i + bs]
-        with lanes.next():
-            c = net.rank_filtered(b[:, :2].contiguous(), b[:, 2].contiguous(), csr)
-            out[i:i + bs] = ranks_from_counts(c["n_greater"], c["n_equal"], c["n_equal_lower"], tie)
-    lanes.join()
+    out = rank_in_batches(net, trip[:, :2], trip[:, 2], csr, bs, tie, streams)
     ranks = out.cpu().numpy()
     assert len(triples) == len(ranks) == n
     hits = create_hits_dict()

@@ -220,17 +220,17 @@ class BaseKGE(torch.nn.Module):
         return self.entity_embeddings.weight.detach(), self.relation_embeddings.weight.detach()
 
     # ------------------------------------------------------------------ fused consumers
-    def rank_filtered(self, x, target, csr=None, heads=False):
+    def rank_filtered(self, x, target, csr=None, heads=False, out=None):
         """Fused filtered-rank counters for queries ``x`` [B,2] and true tails ``target`` [B].
         ``heads=True``: ``x`` = (relation, tail) pairs, ``target`` the true heads, ``csr`` the (r, t) -> heads
-        vocabulary."""
+        vocabulary.  ``out``: the dict of [B] tensors to write into (``ops.rank_filtered``)."""
         Q, bias = self.query(x, heads=heads)
         E, scale = self.table()
         target = target.to(device=E.device, dtype=torch.int64).contiguous()
         if csr is None:
-            return ops.rank_filtered(Q, bias, E, scale, target)
+            return ops.rank_filtered(Q, bias, E, scale, target, out=out)
         rows = csr.rows_for(x.to(device=E.device, dtype=torch.int64))
-        return ops.rank_filtered(Q, bias, E, scale, target, rows, csr.row_ptr, csr.col)
+        return ops.rank_filtered(Q, bias, E, scale, target, rows, csr.row_ptr, csr.col, out=out)
 
     def topk(self, x, k, sigmoid=False, heads=False):
         Q, bias = self.query(x, heads=heads)

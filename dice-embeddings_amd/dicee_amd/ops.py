@@ -215,17 +215,27 @@ def csr_build(triples, columns, ranges):
     return keys[:n_rows], row_ptr[:n_rows + 1], col[:nnz], dropped
 
 
-def rank_filtered(Q, bias, E, scale, target, csr_row=None, row_ptr=None, col=None):
+_RANK_OUT = (("n_greater", torch.int32), ("n_equal", torch.int32), ("n_equal_lower", torch.int32),
+             ("target_score", torch.float32))
+
+
+def rank_filtered(Q, bias, E, scale, target, csr_row=None, row_ptr=None, col=None, out=None):
     """Fused filtered rank. Returns dict of int32 ``n_greater, n_equal, n_equal_lower`` and fp32
-    ``target_score`` (all [B])."""
+    ``target_score`` (all [B]).  ``out``: such a dict of contiguous [B] tensors to write into (slices of an
+    evaluation's arrays, say) instead of new ones."""
     lib = _lib.load()
     _require_gpu(Q, bias, E, scale, target, csr_row, row_ptr, col)
     _check_qe(Q, E, scale, bias)
     B, d = Q.shape
     N = E.shape[0]
     dev = Q.device
-    out = {k: torch.empty((B,), dtype=torch.int32, device=dev) for k in ("n_greater", "n_equal", "n_equal_lower")}
-    out["target_score"] = torch.empty((B,), dtype=torch.float32, device=dev)
+    if out is None:
+        out = {k: torch.empty((B,), dtype=dt, device=dev) for k, dt in _RANK_OUT}
+    else:
+        for k, dt in _RANK_OUT:
+            o = out[k]
+            if o.dtype != dt or o.shape != (B,) or o.device != dev or not o.is_contiguous():
+                raise ValueError(f"out[{k!r}] must be a contiguous {dt} tensor of shape [{B}] on {dev}")
     ws_bytes = lib.kge_rank_workspace_bytes(B)
     ws = torch.empty((ws_bytes,), dtype=torch.uint8, device=dev)
     n_rows = 0 if row_ptr is None else row_ptr.numel() - 1

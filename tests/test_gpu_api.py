@@ -159,6 +159,34 @@ def test_evaluator_batches_on_alternating_streams_give_the_same_ranks(storage):
         np.testing.assert_array_equal(both[s][1][1], both[1][1][1])
 
 
+def test_rank_counters_written_into_the_callers_arrays():
+    """``out=``: a batch writes its counters into slices of the evaluation's arrays (what the evaluator's loop does);
+    the same numbers as the call that allocates, and arrays of another type, length or layout are refused."""
+    from dicee_amd import FilterCSR
+    m, triples = _toy("ComplEx", 64, N=900, R=7, n=700, seed=5)
+    m = m.to("cuda").eval()
+    trip = torch.from_numpy(triples.astype(np.int64)).cuda()
+    csr = FilterCSR.from_triples_gpu(trip, 900, 7, kind="er")
+    x, t = trip[:, :2].contiguous(), trip[:, 2].contiguous()
+    want = m.rank_filtered(x, t, csr)
+    n = len(triples)
+    full = {k: torch.full((n,), -7, dtype=v.dtype, device="cuda") for k, v in want.items()}
+    for i in range(0, n, 256):
+        got = m.rank_filtered(x[i:i + 256], t[i:i + 256], csr, out={k: v[i:i + 256] for k, v in full.items()})
+        assert got["n_greater"].data_ptr() == full["n_greater"][i:].data_ptr()
+    for k in want:
+        assert torch.equal(full[k], want[k]), k
+    bad = dict(full)
+    bad["n_equal"] = full["n_equal"].to(torch.int64)
+    with pytest.raises(ValueError, match="n_equal"):
+        m.rank_filtered(x, t, csr, out=bad)
+    with pytest.raises(ValueError):
+        m.rank_filtered(x[:10], t[:10], csr, out=full)                       # wrong length
+    strided = {k: torch.empty((2 * n,), dtype=v.dtype, device="cuda")[::2] for k, v in want.items()}
+    with pytest.raises(ValueError):
+        m.rank_filtered(x, t, csr, out=strided)
+
+
 @pytest.mark.parametrize("name,d,extra", [("DistMult", 32, {}), ("QMult", 64, {})])
 def test_relation_prediction_follows_the_reference_loop_literally(name, d, extra):
     """form_of_labelling='RelationPrediction' (evaluator.py:440-471): (head, tail) pairs through forward_k_vs_all,
