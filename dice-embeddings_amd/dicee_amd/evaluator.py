@@ -13,7 +13,6 @@ gives it; every such position lies in ``[1 + n_greater, 1 + n_greater + n_equal]
 the representative reported here: ``"stable"`` (default; what a stable descending sort gives:
 ties ordered by entity id), ``"optimistic"``, ``"pessimistic"`` or ``"mean"``.
 """
-import contextlib
 import json
 import os
 from types import SimpleNamespace
@@ -79,21 +78,24 @@ class _BatchStreams:
         self.pool = None
         self.i = 0
 
-    def next(self):
-        """Context manager for the next batch."""
+    def switch(self):
+        """Make the next batch's stream the current one (``join()`` gives the caller's back)."""
         self.i += 1
-        if self.cur is None:
-            return contextlib.nullcontext()
-        if self.n == 1 or self.i == 1:
-            return torch.cuda.stream(self.cur)
+        if self.cur is None or self.n == 1:
+            return
+        if self.i == 1:
+            return                      # the first batch: the caller's stream, which is current
         if self.pool is None:
             self.pool = [torch.cuda.Stream(device=self.device) for _ in range(self.n)]
             for s in self.pool:
                 s.wait_stream(self.cur)
-        return torch.cuda.stream(self.pool[self.i % self.n])
+        torch.cuda.set_stream(self.pool[self.i % self.n])
 
     def join(self):
-        for s in self.pool or ():
+        if self.cur is None or self.pool is None:
+            return
+        torch.cuda.set_stream(self.cur)
+        for s in self.pool:
             self.cur.wait_stream(s)
 
 
@@ -110,12 +112,14 @@ def rank_in_batches(model, x_all, target_all, csr, batch_size, tie="stable", str
     counts = {k: torch.empty((n,), dtype=dt, device=dev) for k, dt in _RANK_OUT}
     bs = int(batch_size)
     lanes = _BatchStreams(dev, streams, bs * model.num_entities)
-    with torch.no_grad():
-        for i in range(0, n, bs):
-            with lanes.next():
+    try:
+        with torch.no_grad():
+            for i in range(0, n, bs):
+                lanes.switch()
                 model.rank_filtered(x_all[i:i + bs], target_all[i:i + bs], csr, heads=heads,
                                     out={k: v[i:i + bs] for k, v in counts.items()})
-    lanes.join()
+    finally:
+        lanes.join()
     return ranks_from_counts(counts["n_greater"], counts["n_equal"], counts["n_equal_lower"], tie)
 
 
