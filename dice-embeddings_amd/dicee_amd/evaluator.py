@@ -57,6 +57,9 @@ def ranks_from_counts(n_greater, n_equal, n_equal_lower, tie="stable"):
     raise ValueError(tie)
 
 
+_STREAM_POOLS = {}   # (device index, streams) -> the side streams of evaluations on that device
+
+
 class _BatchStreams:
     """Consecutive batches of an evaluation on alternating streams.  A batch is a short chain of dependent launches
     (query vectors, filter rows, plan, thresholds, main loop, correction); two chains side by side fill the gaps each
@@ -86,7 +89,12 @@ class _BatchStreams:
         if self.i == 1:
             return                      # the first batch: the caller's stream, which is current
         if self.pool is None:
-            self.pool = [torch.cuda.Stream(device=self.device) for _ in range(self.n)]
+            # the same few streams for every evaluation on a device: torch's allocator keeps a pool of freed blocks
+            # per stream, and a fresh set of streams per evaluation would leave one behind each time
+            key = (torch.device(self.device).index, self.n)
+            if key not in _STREAM_POOLS:
+                _STREAM_POOLS[key] = [torch.cuda.Stream(device=self.device) for _ in range(self.n)]
+            self.pool = _STREAM_POOLS[key]
             for s in self.pool:
                 s.wait_stream(self.cur)
         torch.cuda.set_stream(self.pool[self.i % self.n])
