@@ -144,6 +144,16 @@ def test_evaluator_batches_on_alternating_streams_give_the_same_ranks(storage):
     np.testing.assert_array_equal(ranks[1], ranks[2])
     np.testing.assert_array_equal(ranks[1], ranks[3])
     assert len(ranks[1]) == len(triples) and ranks[1].min() >= 1
+    # called on a stream of the caller's: the evaluation forks from it, joins it and leaves it current
+    mine = torch.cuda.Stream()
+    with torch.cuda.stream(mine):
+        ev = Evaluator(SimpleNamespace(batch_size=512, eval_model="test", scoring_technique="KvsAll",
+                                       full_storage_path=None), streams=2)
+        ev.set_filter(er, num_relations=11)
+        ev.evaluate_lp_k_vs_all(model, triples, form_of_labelling="EntityPrediction")
+        assert torch.cuda.current_stream() == mine
+    np.testing.assert_array_equal(ev.last_ranks, ranks[1])
+    assert torch.cuda.current_stream() == torch.cuda.default_stream()
     # the head-and-tail evaluation: two rank calls per batch, on alternating streams as well
     from dicee_amd import FilterCSR
     from dicee_amd.link_prediction import evaluate_lp
