@@ -81,13 +81,11 @@ class _BatchStreams:
         self.pool = None
         self.i = 0
 
-    def switch(self):
-        """Make the next batch's stream the current one (``join()`` gives the caller's back)."""
-        self.i += 1
+    def fork(self):
+        """What the caller's stream has been given so far (a group's query vectors) is visible to the side streams."""
+        self.i = 0
         if self.cur is None or self.n == 1:
             return
-        if self.i == 1:
-            return                      # the first batch: the caller's stream, which is current
         if self.pool is None:
             # the same few streams for every evaluation on a device: torch's allocator keeps a pool of freed blocks
             # per stream, and a fresh set of streams per evaluation would leave one behind each time
@@ -95,8 +93,16 @@ class _BatchStreams:
             if key not in _STREAM_POOLS:
                 _STREAM_POOLS[key] = [torch.cuda.Stream(device=self.device) for _ in range(self.n)]
             self.pool = _STREAM_POOLS[key]
-            for s in self.pool:
-                s.wait_stream(self.cur)
+        for s in self.pool:
+            s.wait_stream(self.cur)
+
+    def switch(self):
+        """Make the next batch's stream the current one (``join()`` gives the caller's back)."""
+        self.i += 1
+        if self.cur is None or self.n == 1 or self.pool is None:
+            return
+        if self.i == 1:
+            return                      # the first batch of a group: the caller's stream, which is current
         torch.cuda.set_stream(self.pool[self.i % self.n])
 
     def join(self):
@@ -109,23 +115,36 @@ class _BatchStreams:
 
 def rank_in_batches(model, x_all, target_all, csr, batch_size, tie="stable", streams=2, heads=False):
     """Ranks (int64 tensor [n] on the model's device) of ``target_all`` [n] for the queries ``x_all`` [n,2]: one fused
-    rank call per batch of ``batch_size`` queries, each writing its counters straight into the evaluation's arrays
-    (no per-batch copies or conversions: the batch is then nothing but the library's own launches), consecutive
-    batches on alternating streams, the ranks formed once at the end."""
-    from .ops import _RANK_OUT
+    rank call per batch of ``batch_size`` queries.  What does not depend on the batching is done for many batches at a
+    time: the query vectors and the filter rows of a group of batches (at most 64 batches or 256 MB of vectors; every
+    row is a function of its own (h, r) pair alone, so the numbers are those of batch-wise calls) come from one launch
+    each, and a batch is then nothing but the library's rank launches, writing its counters straight into the
+    evaluation's arrays.  Consecutive batches run on alternating streams; the ranks are formed once at the end."""
+    from . import ops
     n = int(x_all.shape[0])
     dev = x_all.device
     x_all = x_all.contiguous()
-    target_all = target_all.contiguous()
-    counts = {k: torch.empty((n,), dtype=dt, device=dev) for k, dt in _RANK_OUT}
-    bs = int(batch_size)
+    target_all = target_all.to(dtype=torch.int64).contiguous()
+    counts = {k: torch.empty((n,), dtype=dt, device=dev) for k, dt in ops._RANK_OUT}
+    bs = max(1, int(batch_size))
+    d = int(model.entity_embeddings.weight.shape[1])
+    group = bs * max(1, min(64, (1 << 28) // (bs * d * 4)))
     lanes = _BatchStreams(dev, streams, bs * model.num_entities)
     try:
         with torch.no_grad():
-            for i in range(0, n, bs):
-                lanes.switch()
-                model.rank_filtered(x_all[i:i + bs], target_all[i:i + bs], csr, heads=heads,
-                                    out={k: v[i:i + bs] for k, v in counts.items()})
+            for g0 in range(0, n, group):
+                xs = x_all[g0:g0 + group]
+                Q, bias = model.query(xs, heads=heads)
+                E, scale = model.table()
+                rows = csr.rows_for(xs.to(device=E.device)) if csr is not None else None
+                lanes.fork()
+                for i in range(0, int(xs.shape[0]), bs):
+                    lanes.switch()
+                    ops.rank_filtered(Q[i:i + bs], None if bias is None else bias[i:i + bs], E, scale,
+                                      target_all[g0 + i:g0 + i + bs], None if rows is None else rows[i:i + bs],
+                                      None if csr is None else csr.row_ptr, None if csr is None else csr.col,
+                                      out={k: v[g0 + i:g0 + i + bs] for k, v in counts.items()})
+                lanes.join()    # before the group's vectors are released to the allocator of the caller's stream
     finally:
         lanes.join()
     return ranks_from_counts(counts["n_greater"], counts["n_equal"], counts["n_equal_lower"], tie)
