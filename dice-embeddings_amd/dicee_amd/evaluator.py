@@ -62,10 +62,11 @@ _STREAM_POOLS = {}   # (device index, streams) -> the side streams of evaluation
 
 class _BatchStreams:
     """Consecutive batches of an evaluation on alternating streams.  A batch is a short chain of dependent launches
-    (query vectors, filter rows, plan, thresholds, main loop, correction); two chains side by side fill the gaps each
-    leaves (ComplEx, 14,541 entities, batches of 1024: 0.117 -> 0.075 ms per batch).  The first batch runs on the
-    caller's stream, so that whatever the model derives lazily (its quantised table) exists before the streams
-    fork; ``join()`` makes the caller's stream wait for all of them.  ``scores_per_batch`` (batch size x entities),
+    (plan, thresholds, main loop, correction); two chains side by side fill the gaps each leaves (ComplEx, 14,541
+    entities, batches of 1024: 0.117 -> 0.075 ms per batch).  What a group of batches shares (query vectors, filter
+    rows, whatever the model derives lazily, such as its quantised table) is made on the caller's stream before
+    ``fork()``; the first batch of a group runs on the caller's stream too; ``join()`` makes the caller's stream
+    wait for all of them and makes it current again.  ``scores_per_batch`` (batch size x entities),
     when given and below a million, keeps everything on the caller's stream: a batch that small is shorter than
     what crossing streams costs (135 entities, batches of 512: 0.056 -> 0.065 ms per batch on two streams)."""
 
