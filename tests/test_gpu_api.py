@@ -144,6 +144,19 @@ def test_evaluator_batches_on_alternating_streams_give_the_same_ranks(storage):
     np.testing.assert_array_equal(ranks[1], ranks[2])
     np.testing.assert_array_equal(ranks[1], ranks[3])
     assert len(ranks[1]) == len(triples) and ranks[1].min() >= 1
+    # more batches than one group holds (64): the groups' vectors and rows are made, used and released in turn; the
+    # ranks do not depend on how the triples are cut into batches and groups
+    rng = np.random.default_rng(3)
+    many = np.stack([rng.integers(0, 3000, 40000), rng.integers(0, 11, 40000), rng.integers(0, 3000, 40000)], axis=1)
+    by_cut = {}
+    for bs, streams in ((512, 2), (512, 1), (4096, 2)):
+        ev = Evaluator(SimpleNamespace(batch_size=bs, eval_model="test", scoring_technique="KvsAll",
+                                       full_storage_path=None), streams=streams)
+        ev.set_filter(er, num_relations=11)
+        ev.evaluate_lp_k_vs_all(model, many, form_of_labelling="EntityPrediction")
+        by_cut[(bs, streams)] = ev.last_ranks.copy()
+    np.testing.assert_array_equal(by_cut[(512, 2)], by_cut[(512, 1)])
+    np.testing.assert_array_equal(by_cut[(512, 2)], by_cut[(4096, 2)])
     # called on a stream of the caller's: the evaluation forks from it, joins it and leaves it current
     mine = torch.cuda.Stream()
     with torch.cuda.stream(mine):
