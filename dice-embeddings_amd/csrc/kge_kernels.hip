@@ -1,6 +1,7 @@
 // Entry points of the contraction path: materialised scores, fused filtered rank, fused top-k and
 // fused multi-hot BCE, plus the small helper kernels around the two MFMA main loops.
 #include "kge_contract.hip.h"
+#include "kge_rank128.hip.h"
 #include "kge_topk_i8.hip.h"
 
 #include <string.h>
@@ -1352,6 +1353,39 @@ int launch_contract(int dtype, const ContractArgs& a, const EArgs& ea, hipStream
   return KGE_OK;
 }
 
+// The filtered-rank main loop of bf16 tables with d == 128: four query tiles per wave (rank128_kernel), when the batch
+// fills its 1024-query workgroups about as well as it fills the 512-query ones of the two-tile kernel.
+constexpr int R128_WG_WAVES = 8;
+constexpr int R128_WG_QUERIES = R128_WG_WAVES * 32 * R128_NQT;
+bool rank128_applies(int dtype, int64_t d, int64_t B) {
+  if (dtype != KGE_BF16 || d != 128) return false;
+  const int64_t slots4 = (B + R128_WG_QUERIES - 1) / R128_WG_QUERIES * R128_WG_QUERIES;
+  const int64_t slots2 = (B + QA_WG_QUERIES - 1) / QA_WG_QUERIES * QA_WG_QUERIES;
+  return slots4 * 10 <= slots2 * 11;  // at most a tenth more query slots than the two-tile kernel would multiply
+}
+int launch_rank128(const ContractArgs& base, const RankArgs& ea, hipStream_t st, const char* name) {
+  if (base.B == 0 || base.e_end <= base.e_begin) return KGE_OK;
+  ContractArgs a = base;
+  a.n_qgroups = (int)((a.B + R128_WG_QUERIES - 1) / R128_WG_QUERIES);
+  a.n_lanes = 32 * (8 / R128_WG_WAVES) / a.n_qgroups;  // the workgroups resident on one XCD, shared out among the query groups
+  if (a.n_lanes < 1) a.n_lanes = 1;
+  const int64_t rows = a.e_end - a.e_begin;
+  int64_t chunk = rows / (8 * (int64_t)a.n_lanes * 4);  // aim for >= 4 chunks per workgroup
+  chunk = (chunk + QA_STAGE_ROWS - 1) / QA_STAGE_ROWS * QA_STAGE_ROWS;
+  if (chunk < QA_STAGE_ROWS) chunk = QA_STAGE_ROWS;
+  if (chunk > 1024) chunk = 1024;
+  a.chunk_rows = (int)chunk;
+  a.n_chunks = (rows + chunk - 1) / chunk;
+  const int64_t nwg = 8 * (int64_t)a.n_qgroups * a.n_lanes;
+  KGE_REQUIRE(nwg <= 0x7fffffffLL, KGE_ERR_INVALID, "%s: grid of %lld workgroups too large", name, (long long)nwg);
+  LaunchTimer timer;
+  if (int trc = timer.begin(st)) return trc;
+  hipLaunchKernelGGL((rank128_kernel<R128_WG_WAVES>), dim3((unsigned)nwg), dim3(64 * R128_WG_WAVES), 0, st, a, ea);
+  KGE_LAUNCH_CHECK(name);
+  if (int trc = timer.end()) return trc;
+  return KGE_OK;
+}
+
 // ksplit_kernel alone (fp32 operands), with row strides and an optional split of K over grid.y.
 template <template <int> class EpiT, class EArgs>
 int launch_ksplit(const ContractArgs& a, const EArgs& ea, unsigned k_splits, hipStream_t st, const char* name) {
@@ -1556,7 +1590,7 @@ int rank_filtered_launch(const char* who, const float* Q, const float* bias, con
     KGE_LAUNCH_CHECK("target_score_kernel");
   }
   RankArgs ea{ws.thr, target, n_greater, n_equal, n_equal_lower};
-  int rc = launch_contract<RankEpi>(dtype, a, ea, st, who);
+  int rc = rank128_applies(dtype, d, B) ? launch_rank128(a, ea, st, who) : launch_contract<RankEpi>(dtype, a, ea, st, who);
   if (rc) return rc;
   if (filtered) {
     for (int64_t b0 = 0, sub = 0; b0 < B; b0 += SORT_MAX, ++sub) {
