@@ -59,8 +59,11 @@ def cpu_baseline(cfg, model, mode, seconds_budget=25.0):
     # sample size: keep B*N*4 bytes of scores around 0.5 GB per batch
     bs = int(max(1, min(cfg.B, (1 << 27) // max(N, 1))))
     q = cfg.queries
-    done, t_total, nb = 0, 0.0, 0
-    while t_total < seconds_budget and done + bs <= len(q) and nb < 8:
+    # protocol: one warm-up batch, then timed batches (at least 5 if the budget allows) and the MEDIAN batch time
+    times = []
+    done = 0
+    t_spent = 0.0
+    while done + bs <= len(q) and len(times) < 9 and (len(times) < 5 or t_spent < seconds_budget):
         batch = q[done:done + bs]
         t0 = time.perf_counter()
         if mode == "rank":
@@ -79,36 +82,28 @@ def cpu_baseline(cfg, model, mode, seconds_budget=25.0):
             pos = [cfg.csr.tails(int(h), int(r)).astype(np.int64) for h, r, _ in batch]
             tcp.kvsall_bce_step(name, E, Rel, torch.from_numpy(batch[:, :2].copy()), pos, 0.0, **kw)
         dt = time.perf_counter() - t0
-        if nb > 0 or dt > 2.0:                                  # first small batch is a warm-up
-            t_total += dt
-            done += bs
-        nb += 1
-    n_q = max(done, 1)
-    t_total = max(t_total, 1e-9)
-    return {"value": n_q * N / t_total, "unit": "scores/s", "cores": threads, "kind": "port",
-            "queries_per_sec": n_q / t_total,
-            "sample": f"{n_q} queries of {cfg.name} in batches of {bs} against all {N} entities, "
-                      f"torch {torch.__version__} CPU, {threads} threads"}
-
-
-def main_loop_kernel(storage, d, mode):
-    """Name of the contraction kernel the library picks for this table type and width."""
-    epi = {"rank": "RankEpi", "headrank": "RankEpi", "topk": "TopkEpi", "bce": "BceEpi",
-           "bcegrad": "GradEpi | StoreEpi", "train": "GradEpi | StoreEpi"}[mode]
-    if storage == "fp32":
-        return f"ksplit_kernel<{epi}, {'true' if d % 4 == 0 else 'false'}>"
-    if d > 256:
-        return f"kchunk_kernel<{epi}>"
-    lds_d = 64 if d <= 64 else 128 if d <= 128 else 256   # LDS row of the instantiation; narrower rows are zero-padded
-    pad = ", true" if d != lds_d else ", false"
-    nqt = 1 if lds_d == 256 else 2
-    if storage == "bf16":
-        if epi == "RankEpi":
-            return f"qstream_kernel<RankFastEpi, {nqt}, 8, 2, {lds_d // 16}{pad}>"
-        return f"qreg_async_kernel<{epi}, {nqt}, {lds_d // 16}{pad}>"
-    if d == 128 and epi == "TopkEpi":
-        return "topk_i8_filter_kernel"
-    return f"qreg_i8_kernel<{epi}, {nqt}, {lds_d // 16}{pad}>"
+        t_spent += dt
+        if done > 0:                                            # the first batch is the warm-up
+            times.append(dt)
+        done += bs
+        if t_spent > 3.0 * seconds_budget:
+            break
+    if not times:                                               # a workload of a single batch: the warm-up is all there is
+        times = [t_spent]
+    med = float(np.median(times))
+    cpu_model = "unknown CPU"
+    try:
+        with open("/proc/cpuinfo") as fh:
+            for line in fh:
+                if line.startswith("model name"):
+                    cpu_model = line.split(":", 1)[1].strip()
+                    break
+    except OSError:
+        pass
+    return {"value": bs * N / med, "unit": "scores/s", "cores": threads, "kind": "port",
+            "queries_per_sec": bs / med,
+            "sample": f"median of {len(times)} timed batches of {bs} queries of {cfg.name} (after one warm-up batch) "
+                      f"against all {N} entities, torch {torch.__version__} CPU, {threads} threads, {cpu_model}"}
 
 
 def main():
@@ -240,6 +235,7 @@ def main():
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
     kernel_ms, launches = ops.profile_end()
+    kernel_name = ops.profile_kernel()                           # what the library dispatched, in its own words
 
     N, d = cfg.N, cfg.d
     scores = float(n_queries) * N
@@ -287,7 +283,7 @@ def main():
                      if args.scale == 1.0 and args.mode is None else None,
                      "traffic_source": "measured offline, not in this run: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on "
                                        "this workload, scaled by a 1 GiB copy kernel (profiles/*_counters.md)",
-                     "kernel": main_loop_kernel(cfg.storage, d, mode),
+                     "kernel": kernel_name,
                      "kernel_ms_avg": kernel_ms / max(launches, 1), "launches": launches,
                      "kernel_time_share": kernel_ms * 1e-3 / elapsed},
         "setup_s": t_setup,
@@ -371,6 +367,24 @@ def main():
                 del Ai, Bi
             except Exception as exc:                                    # noqa: BLE001 (a side figure: report, go on)
                 ceil["torch_int_mm_int8_8192_cubed_randint"] = {"error": f"{type(exc).__name__}: {exc}"[:200]}
+        if d == 128 and mode == "rank" and model.table()[0].dtype == torch.bfloat16:
+            # the ladder of the rank main loop, bottom up, each rung sustained for ~0.7 s in this process (library
+            # measurement aids kge_probe_mfma / kge_probe_walk): the tile statement's MFMAs on random bf16 operands
+            # held in registers; with the rank count between them; with the entity fragments re-read from LDS; the
+            # whole walk over this table (global -> LDS stages, barriers) without the count.  The top rung is the
+            # timed kernel itself (roofline.achieved).
+            E_t, _ = model.table()
+            Qw, _ = model.query(batches[0][0])
+            lad = {}
+            for key, (cnt, rd) in (("mfma_registers_only", (0, 0)), ("mfma_with_count", (1, 0)),
+                                   ("mfma_with_lds_reads", (0, 1)), ("mfma_with_count_and_lds_reads", (1, 1))):
+                r, ms = ops.probe_mfma(cnt, rd, 0.7)
+                lad[key] = {"achieved": r, "frac": r / PEAK_TFLOPS["bf16"], "ms": ms}
+            r, ms = ops.probe_walk(Qw, E_t, 0.7)
+            lad["walk_without_count"] = {"achieved": r, "frac": r / PEAK_TFLOPS["bf16"], "ms": ms,
+                                         "shape": [int(Qw.shape[0]), d, N]}
+            ceil["rank_main_loop_ladder"] = lad
+            del Qw
         if d == 128:
             E_t, _ = model.table()
             if E_t.dtype == torch.bfloat16:

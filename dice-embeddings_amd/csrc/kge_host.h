@@ -38,6 +38,28 @@ constexpr int BCE_SLOTS = 128;
 constexpr int KS_WG_QUERIES = 128;       // workgroup shape of the fp32 contraction (also sizes the backward's K split)
 constexpr int KS_TILE_ROWS = 256;
 
+// Work decomposition of the four-tile filtered-rank main loop (bf16 tables, d == 128): 8-wave workgroups of
+// 4 x 32 queries per wave, one per CU; the workgroups resident on one XCD (32) are shared out among the query
+// groups; chunks of at most 512 rows (2442 chunks of 1024 rows over 64 workgroup lanes leave 39 to some lanes and
+// 38 to others: 2 % of the launch idle at its end; at 512 it is under 1 %), at least 4 per workgroup.
+constexpr int R128_WG_WAVES = 8;
+constexpr int R128_WG_QUERIES = R128_WG_WAVES * 32 * 4;
+constexpr int R128_MAX_CHUNK = 512;
+inline void rank128_plan(int64_t B, int64_t rows, int* n_qgroups, int* n_lanes, int* chunk_rows, int64_t* n_chunks) {
+  int g = (int)((B + R128_WG_QUERIES - 1) / R128_WG_QUERIES);
+  if (g < 1) g = 1;
+  int lanes = 32 / g;
+  if (lanes < 1) lanes = 1;
+  int64_t chunk = rows / (8 * (int64_t)lanes * 4);
+  chunk = (chunk + 127) / 128 * 128;
+  if (chunk < 128) chunk = 128;
+  if (chunk > R128_MAX_CHUNK) chunk = R128_MAX_CHUNK;
+  *n_qgroups = g;
+  *n_lanes = lanes;
+  *chunk_rows = (int)chunk;
+  *n_chunks = (rows + chunk - 1) / chunk;
+}
+
 struct Status {
   int code = KGE_OK;
   char msg[256] = "";

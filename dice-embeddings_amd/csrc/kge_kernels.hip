@@ -27,6 +27,7 @@ void clear_error() { g_err[0] = 0; }
 static std::mutex g_prof_mu;
 static bool g_prof_on = false;
 static std::vector<std::pair<hipEvent_t, hipEvent_t>> g_prof_events;
+static char g_prof_kernel[160] = "";  // the main loop most recently bracketed, as dispatched
 
 namespace {
 
@@ -1281,15 +1282,25 @@ struct LaunchTimer {
     }
     return KGE_OK;
   }
-  int end() {
+  int end(const char* kernel) {
     if (timed) {
       KGE_HIP_CHECK(hipEventRecord(ev1, st));
       std::lock_guard<std::mutex> lk(g_prof_mu);
       g_prof_events.emplace_back(ev0, ev1);
+      snprintf(g_prof_kernel, sizeof(g_prof_kernel), "%s", kernel);
     }
     return KGE_OK;
   }
 };
+
+template <template <int> class EpiT>
+constexpr const char* epilogue_name() {
+  using E = EpiT<2>;
+  return std::is_same<E, StoreEpi<2>>::value ? "StoreEpi" : std::is_same<E, RankEpi<2>>::value ? "RankEpi"
+       : std::is_same<E, TopkEpi<2>>::value ? "TopkEpi" : std::is_same<E, TopkKeyEpi<2>>::value ? "TopkKeyEpi"
+       : std::is_same<E, TopkFirstEpi<2>>::value ? "TopkFirstEpi" : std::is_same<E, BceEpi<2>>::value ? "BceEpi"
+       : std::is_same<E, GradEpi<2>>::value ? "GradEpi" : std::is_same<E, MinMaxEpi<2>>::value ? "MinMaxEpi" : "?";
+}
 
 template <template <int> class EpiT, class EArgs>
 int launch_contract(int dtype, const ContractArgs& a, const EArgs& ea, hipStream_t st, const char* name) {
@@ -1309,7 +1320,11 @@ int launch_contract(int dtype, const ContractArgs& a, const EArgs& ea, hipStream
   dim3 grid((unsigned)nwg), block(fast_i8 ? 64 * I8_WG_WAVES : persistent ? 64 * QA_WG_WAVES : 512);
   LaunchTimer timer;
   if (int trc = timer.begin(st)) return trc;
+  char kname[160];  // the kernel as dispatched below, for kge_profile_kernel()
+  const char* epi = epilogue_name<EpiT>();
   const bool rows_aligned = (a.d % 4 == 0) && (((uintptr_t)a.E | (uintptr_t)a.Q) % 16 == 0);
+  if (f32_split) snprintf(kname, sizeof(kname), "ksplit_kernel<%s, %s>", epi, rows_aligned ? "true" : "false");
+  else if (wide_bf16) snprintf(kname, sizeof(kname), "kchunk_kernel<%s, %s>", dtype == KGE_BF16 ? "KGE_BF16" : "KGE_I8", epi);
   if (f32_split && rows_aligned)
     hipLaunchKernelGGL((ksplit_kernel<EpiT, true>), grid, block, 0, st, a, ea);
   else if (f32_split)
@@ -1324,6 +1339,11 @@ int launch_contract(int dtype, const ContractArgs& a, const EArgs& ea, hipStream
     auto go = [&](auto nqt, auto ksteps, auto padc, auto streamed) {
       constexpr int NQT = decltype(nqt)::value, KS = decltype(ksteps)::value;
       constexpr bool PAD = decltype(padc)::value, STREAMED = decltype(streamed)::value;
+      if constexpr (is_rank || STREAMED)
+        snprintf(kname, sizeof(kname), "qstream_kernel<%s, %d, %d, %d, %d, %s>", is_rank ? "RankFastEpi" : epi, NQT, QA_WG_WAVES,
+                 QA_WAVES_PER_SIMD, KS, PAD ? "true" : "false");
+      else
+        snprintf(kname, sizeof(kname), "qreg_async_kernel<%s, %d, %d, %s>", epi, NQT, KS, PAD ? "true" : "false");
       if constexpr (is_rank)
         hipLaunchKernelGGL((qstream_kernel<RankFastEpi, NQT, QA_WG_WAVES, QA_WAVES_PER_SIMD, KS, PAD>), grid, block, 0, st, a, ea);
       else if constexpr (STREAMED)
@@ -1341,6 +1361,8 @@ int launch_contract(int dtype, const ContractArgs& a, const EArgs& ea, hipStream
     else go(integral_constant<int, 1>{}, integral_constant<int, 16>{}, std::true_type{}, integral_constant<bool, s256>{});
   }
   else {
+    snprintf(kname, sizeof(kname), "qreg_i8_kernel<%s, %d, %d, %s>", epi, rc.lds_d == 256 ? 1 : QREG_NQT, rc.lds_d / 16,
+             pad ? "true" : "false");
     if (rc.lds_d == 128 && !pad) hipLaunchKernelGGL((qreg_i8_kernel<EpiT, QREG_NQT, 8, false>), grid, block, 0, st, a, ea);
     else if (rc.lds_d == 128) hipLaunchKernelGGL((qreg_i8_kernel<EpiT, QREG_NQT, 8, true>), grid, block, 0, st, a, ea);
     else if (rc.lds_d == 64 && !pad) hipLaunchKernelGGL((qreg_i8_kernel<EpiT, QREG_NQT, 4, false>), grid, block, 0, st, a, ea);
@@ -1349,40 +1371,29 @@ int launch_contract(int dtype, const ContractArgs& a, const EArgs& ea, hipStream
     else hipLaunchKernelGGL((qreg_i8_kernel<EpiT, 1, 16, true>), grid, block, 0, st, a, ea);
   }
   KGE_LAUNCH_CHECK(name);
-  if (int trc = timer.end()) return trc;
+  if (int trc = timer.end(kname)) return trc;
   return KGE_OK;
 }
 
 // The filtered-rank main loop of bf16 tables with d == 128: four query tiles per wave (rank128_kernel), when the batch
 // fills its 1024-query workgroups about as well as it fills the 512-query ones of the two-tile kernel.
-constexpr int R128_WG_WAVES = 8;
-constexpr int R128_WG_QUERIES = R128_WG_WAVES * 32 * R128_NQT;
 bool rank128_applies(int dtype, int64_t d, int64_t B) {
   if (dtype != KGE_BF16 || d != 128) return false;
-  const int64_t slots4 = (B + R128_WG_QUERIES - 1) / R128_WG_QUERIES * R128_WG_QUERIES;
+  const int64_t slots4 = (B + host::R128_WG_QUERIES - 1) / host::R128_WG_QUERIES * host::R128_WG_QUERIES;
   const int64_t slots2 = (B + QA_WG_QUERIES - 1) / QA_WG_QUERIES * QA_WG_QUERIES;
   return slots4 * 10 <= slots2 * 11;  // at most a tenth more query slots than the two-tile kernel would multiply
 }
 int launch_rank128(const ContractArgs& base, const RankArgs& ea, hipStream_t st, const char* name) {
   if (base.B == 0 || base.e_end <= base.e_begin) return KGE_OK;
   ContractArgs a = base;
-  a.n_qgroups = (int)((a.B + R128_WG_QUERIES - 1) / R128_WG_QUERIES);
-  a.n_lanes = 32 * (8 / R128_WG_WAVES) / a.n_qgroups;  // the workgroups resident on one XCD, shared out among the query groups
-  if (a.n_lanes < 1) a.n_lanes = 1;
-  const int64_t rows = a.e_end - a.e_begin;
-  int64_t chunk = rows / (8 * (int64_t)a.n_lanes * 4);  // aim for >= 4 chunks per workgroup
-  chunk = (chunk + QA_STAGE_ROWS - 1) / QA_STAGE_ROWS * QA_STAGE_ROWS;
-  if (chunk < QA_STAGE_ROWS) chunk = QA_STAGE_ROWS;
-  if (chunk > 1024) chunk = 1024;
-  a.chunk_rows = (int)chunk;
-  a.n_chunks = (rows + chunk - 1) / chunk;
+  host::rank128_plan(a.B, a.e_end - a.e_begin, &a.n_qgroups, &a.n_lanes, &a.chunk_rows, &a.n_chunks);
   const int64_t nwg = 8 * (int64_t)a.n_qgroups * a.n_lanes;
   KGE_REQUIRE(nwg <= 0x7fffffffLL, KGE_ERR_INVALID, "%s: grid of %lld workgroups too large", name, (long long)nwg);
   LaunchTimer timer;
   if (int trc = timer.begin(st)) return trc;
-  hipLaunchKernelGGL((rank128_kernel<R128_WG_WAVES>), dim3((unsigned)nwg), dim3(64 * R128_WG_WAVES), 0, st, a, ea);
+  hipLaunchKernelGGL((rank128_kernel<host::R128_WG_WAVES>), dim3((unsigned)nwg), dim3(64 * host::R128_WG_WAVES), 0, st, a, ea);
   KGE_LAUNCH_CHECK(name);
-  if (int trc = timer.end()) return trc;
+  if (int trc = timer.end("rank128_kernel<8>")) return trc;
   return KGE_OK;
 }
 
@@ -1404,7 +1415,9 @@ int launch_ksplit(const ContractArgs& a, const EArgs& ea, unsigned k_splits, hip
   else
     hipLaunchKernelGGL((ksplit_kernel<EpiT, false>), grid, block, 0, st, a, ea);
   KGE_LAUNCH_CHECK(name);
-  if (int trc = timer.end()) return trc;
+  char kname[160];
+  snprintf(kname, sizeof(kname), "ksplit_kernel<%s, %s>", epilogue_name<EpiT>(), rows_aligned ? "true" : "false");
+  if (int trc = timer.end(kname)) return trc;
   return KGE_OK;
 }
 
@@ -1481,6 +1494,13 @@ extern "C" int kge_profile_end(double* total_ms, int64_t* launches) {
   if (total_ms) *total_ms = total;
   if (launches) *launches = (int64_t)evs.size();
   return rc;
+}
+
+extern "C" const char* kge_profile_kernel(void) {
+  static thread_local char out[160];
+  std::lock_guard<std::mutex> lk(g_prof_mu);
+  snprintf(out, sizeof(out), "%s", g_prof_kernel);
+  return out;
 }
 
 extern "C" int kge_scores(const float* Q, const float* bias, const void* E, int dtype, const float* scale, int64_t B,
@@ -1858,7 +1878,7 @@ int topk_impl(const char* who, const float* Q, const float* bias, const void* E,
     if (int trc = timer.begin(st)) return trc;
     hipLaunchKernelGGL(topk_i8_filter_kernel, dim3((unsigned)nwg), dim3(64 * TF_W), 0, st, a, ea);
     KGE_LAUNCH_CHECK(name);
-    if (int trc = timer.end()) return trc;
+    if (int trc = timer.end("topk_i8_filter_kernel")) return trc;
     hipLaunchKernelGGL(topk_rescore_kernel, dim3((unsigned)B, 4), dim3(256), 0, st, ws, a);
     KGE_LAUNCH_CHECK("topk_rescore_kernel");
     return KGE_OK;

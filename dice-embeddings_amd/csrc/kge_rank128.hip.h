@@ -48,19 +48,23 @@ constexpr int R128_NQT = 4;  // query tiles per wave
 #define R128_NOREAD(E, F) ""
 // one chain: accumulator NEW <- sum over the 8 K steps of ef[s] x q[s]; between its MFMAs the count of OLD
 // (registers o0 .. o15) against TH into GT / M; READ: R128_READ in the chain that consumes the fragments last
+#define R128_BCNT(GT) "v_bcnt_u32_b32 " GT ", %[bits], " GT "\n"
+// (the measurement aids of kge_probe.hip build the same statement without the count or without the reads)
+#define R128_NOPAIR(a0, a1, TH, M) ""
+#define R128_NOBCNT(GT) ""
 #define R128_CHAIN(NEW, Q0, Q1, Q2, Q3, Q4, Q5, Q6, Q7, o0, o1, o2, o3, o4, o5, o6, o7, o8, o9, o10, o11, o12, o13, \
-                   o14, o15, TH, GT, M, READ)                                                                        \
+                   o14, o15, TH, GT, M, READ, PAIR0, PAIR, BCNT)                                                     \
   R128_MFMA(NEW, "%[e0]", Q0, "0")                                                                                  \
   "s_nop 5\n"                                                                                                      \
-  R128_PAIR_FIRST(o0, o1, TH, M) READ("%[e0]", "%[f0]")                                                             \
-  R128_MFMA(NEW, "%[e1]", Q1, NEW) R128_PAIR(o2, o3, TH, M) READ("%[e1]", "%[f1]")                                  \
-  R128_MFMA(NEW, "%[e2]", Q2, NEW) R128_PAIR(o4, o5, TH, M) READ("%[e2]", "%[f2]")                                  \
-  R128_MFMA(NEW, "%[e3]", Q3, NEW) R128_PAIR(o6, o7, TH, M) READ("%[e3]", "%[f3]")                                  \
-  R128_MFMA(NEW, "%[e4]", Q4, NEW) R128_PAIR(o8, o9, TH, M) READ("%[e4]", "%[f4]")                                  \
-  R128_MFMA(NEW, "%[e5]", Q5, NEW) R128_PAIR(o10, o11, TH, M) READ("%[e5]", "%[f5]")                                \
-  R128_MFMA(NEW, "%[e6]", Q6, NEW) R128_PAIR(o12, o13, TH, M) READ("%[e6]", "%[f6]")                                \
-  R128_MFMA(NEW, "%[e7]", Q7, NEW) R128_PAIR(o14, o15, TH, M)                                                       \
-  "v_bcnt_u32_b32 " GT ", %[bits], " GT "\n" READ("%[e7]", "%[f7]")
+  PAIR0(o0, o1, TH, M) READ("%[e0]", "%[f0]")                                                                       \
+  R128_MFMA(NEW, "%[e1]", Q1, NEW) PAIR(o2, o3, TH, M) READ("%[e1]", "%[f1]")                                       \
+  R128_MFMA(NEW, "%[e2]", Q2, NEW) PAIR(o4, o5, TH, M) READ("%[e2]", "%[f2]")                                       \
+  R128_MFMA(NEW, "%[e3]", Q3, NEW) PAIR(o6, o7, TH, M) READ("%[e3]", "%[f3]")                                       \
+  R128_MFMA(NEW, "%[e4]", Q4, NEW) PAIR(o8, o9, TH, M) READ("%[e4]", "%[f4]")                                       \
+  R128_MFMA(NEW, "%[e5]", Q5, NEW) PAIR(o10, o11, TH, M) READ("%[e5]", "%[f5]")                                     \
+  R128_MFMA(NEW, "%[e6]", Q6, NEW) PAIR(o12, o13, TH, M) READ("%[e6]", "%[f6]")                                     \
+  R128_MFMA(NEW, "%[e7]", Q7, NEW) PAIR(o14, o15, TH, M)                                                            \
+  BCNT(GT) READ("%[e7]", "%[f7]")
 #define R128_X "v224", "v225", "v226", "v227", "v228", "v229", "v230", "v231", "v232", "v233", "v234", "v235", "v236", \
                "v237", "v238", "v239"
 #define R128_Y "v240", "v241", "v242", "v243", "v244", "v245", "v246", "v247", "v248", "v249", "v250", "v251", "v252", \
@@ -69,41 +73,49 @@ constexpr int R128_NQT = 4;  // query tiles per wave
 // one entity tile: on entry X holds the last result tile of the previous entity tile (query tile 3), not yet
 // counted; every query tile has a running minimum of its own
 #define R128_CHAIN_(...) R128_CHAIN(__VA_ARGS__)  // (expands the register lists before the chain counts its arguments)
-#define R128_TILE                                                                                 \
+#define R128_TILE_TEXT(READ, PAIR0, PAIR, BCNT)                                                   \
   "s_waitcnt lgkmcnt(0)\n"                                                                        \
-  R128_CHAIN_("%[Y]", R128_Q(0), R128_X, "%[t3]", "%[g3]", "%[m3]", R128_NOREAD)                   \
-  R128_CHAIN_("%[X]", R128_Q(1), R128_Y, "%[t0]", "%[g0]", "%[m0]", R128_NOREAD)                   \
-  R128_CHAIN_("%[Y]", R128_Q(2), R128_X, "%[t1]", "%[g1]", "%[m1]", R128_NOREAD)                   \
-  R128_CHAIN_("%[X]", R128_Q(3), R128_Y, "%[t2]", "%[g2]", "%[m2]", R128_READ)
+  R128_CHAIN_("%[Y]", R128_Q(0), R128_X, "%[t3]", "%[g3]", "%[m3]", R128_NOREAD, PAIR0, PAIR, BCNT) \
+  R128_CHAIN_("%[X]", R128_Q(1), R128_Y, "%[t0]", "%[g0]", "%[m0]", R128_NOREAD, PAIR0, PAIR, BCNT) \
+  R128_CHAIN_("%[Y]", R128_Q(2), R128_X, "%[t1]", "%[g1]", "%[m1]", R128_NOREAD, PAIR0, PAIR, BCNT) \
+  R128_CHAIN_("%[X]", R128_Q(3), R128_Y, "%[t2]", "%[g2]", "%[m2]", READ, PAIR0, PAIR, BCNT)
+#define R128_TILE R128_TILE_TEXT(R128_READ, R128_PAIR_FIRST, R128_PAIR, R128_BCNT)
 
 typedef __attribute__((ext_vector_type(16))) float r128_acc;
 
-// ROFF: where the fragments of the next entity tile are, relative to the addresses in fb[]
-template <int ROFF>
+// ROFF: where the fragments of the next entity tile are, relative to the addresses in fb[].
+// COUNT / READS: false only in the measurement aids (the statement without its count, without its fragment reads).
+template <int ROFF, bool COUNT = true, bool READS = true>
 __device__ __forceinline__ void r128_tile(const bf16x8 (&qf)[R128_NQT][8], bf16x8 (&ef)[8], const int (&foff)[8],
                                           r128_acc& X, const float (&thr)[R128_NQT], int32_t (&gt)[R128_NQT],
                                           float (&mn)[R128_NQT]) {
   float d0, d1;
   uint32_t bits;
   r128_acc Y;
-  asm volatile(R128_TILE
-  : [X] "+{v[224:239]}"(X), [Y] "=&{v[240:255]}"(Y), [e0] "+v"(ef[0]), [e1] "+v"(ef[1]), [e2] "+v"(ef[2]),
-    [e3] "+v"(ef[3]), [e4] "+v"(ef[4]), [e5] "+v"(ef[5]), [e6] "+v"(ef[6]), [e7] "+v"(ef[7]), [g0] "+v"(gt[0]),
-    [g1] "+v"(gt[1]), [g2] "+v"(gt[2]), [g3] "+v"(gt[3]), [m0] "+v"(mn[0]), [m1] "+v"(mn[1]), [m2] "+v"(mn[2]),
-    [m3] "+v"(mn[3]), [d0] "=&v"(d0), [d1] "=&v"(d1), [bits] "=&v"(bits)
-  : [q00] "v"(qf[0][0]), [q01] "v"(qf[0][1]), [q02] "v"(qf[0][2]), [q03] "v"(qf[0][3]), [q04] "v"(qf[0][4]),
-    [q05] "v"(qf[0][5]), [q06] "v"(qf[0][6]), [q07] "v"(qf[0][7]), [q10] "v"(qf[1][0]), [q11] "v"(qf[1][1]),
-    [q12] "v"(qf[1][2]), [q13] "v"(qf[1][3]), [q14] "v"(qf[1][4]), [q15] "v"(qf[1][5]), [q16] "v"(qf[1][6]),
-    [q17] "v"(qf[1][7]), [q20] "v"(qf[2][0]), [q21] "v"(qf[2][1]), [q22] "v"(qf[2][2]), [q23] "v"(qf[2][3]),
-    [q24] "v"(qf[2][4]), [q25] "v"(qf[2][5]), [q26] "v"(qf[2][6]), [q27] "v"(qf[2][7]), [q30] "v"(qf[3][0]),
-    [q31] "v"(qf[3][1]), [q32] "v"(qf[3][2]), [q33] "v"(qf[3][3]), [q34] "v"(qf[3][4]), [q35] "v"(qf[3][5]),
-    [q36] "v"(qf[3][6]), [q37] "v"(qf[3][7]), [f0] "v"(foff[0]), [f1] "v"(foff[1]), [f2] "v"(foff[2]),
-    [f3] "v"(foff[3]), [f4] "v"(foff[4]), [f5] "v"(foff[5]), [f6] "v"(foff[6]), [f7] "v"(foff[7]),
-    [t0] "v"(thr[0]), [t1] "v"(thr[1]), [t2] "v"(thr[2]), [t3] "v"(thr[3]), [roff] "n"(ROFF));
+#define R128_OPERANDS \
+  : [X] "+{v[224:239]}"(X), [Y] "=&{v[240:255]}"(Y), [e0] "+v"(ef[0]), [e1] "+v"(ef[1]), [e2] "+v"(ef[2]), \
+    [e3] "+v"(ef[3]), [e4] "+v"(ef[4]), [e5] "+v"(ef[5]), [e6] "+v"(ef[6]), [e7] "+v"(ef[7]), [g0] "+v"(gt[0]), \
+    [g1] "+v"(gt[1]), [g2] "+v"(gt[2]), [g3] "+v"(gt[3]), [m0] "+v"(mn[0]), [m1] "+v"(mn[1]), [m2] "+v"(mn[2]), \
+    [m3] "+v"(mn[3]), [d0] "=&v"(d0), [d1] "=&v"(d1), [bits] "=&v"(bits) \
+  : [q00] "v"(qf[0][0]), [q01] "v"(qf[0][1]), [q02] "v"(qf[0][2]), [q03] "v"(qf[0][3]), [q04] "v"(qf[0][4]), \
+    [q05] "v"(qf[0][5]), [q06] "v"(qf[0][6]), [q07] "v"(qf[0][7]), [q10] "v"(qf[1][0]), [q11] "v"(qf[1][1]), \
+    [q12] "v"(qf[1][2]), [q13] "v"(qf[1][3]), [q14] "v"(qf[1][4]), [q15] "v"(qf[1][5]), [q16] "v"(qf[1][6]), \
+    [q17] "v"(qf[1][7]), [q20] "v"(qf[2][0]), [q21] "v"(qf[2][1]), [q22] "v"(qf[2][2]), [q23] "v"(qf[2][3]), \
+    [q24] "v"(qf[2][4]), [q25] "v"(qf[2][5]), [q26] "v"(qf[2][6]), [q27] "v"(qf[2][7]), [q30] "v"(qf[3][0]), \
+    [q31] "v"(qf[3][1]), [q32] "v"(qf[3][2]), [q33] "v"(qf[3][3]), [q34] "v"(qf[3][4]), [q35] "v"(qf[3][5]), \
+    [q36] "v"(qf[3][6]), [q37] "v"(qf[3][7]), [f0] "v"(foff[0]), [f1] "v"(foff[1]), [f2] "v"(foff[2]), \
+    [f3] "v"(foff[3]), [f4] "v"(foff[4]), [f5] "v"(foff[5]), [f6] "v"(foff[6]), [f7] "v"(foff[7]), \
+    [t0] "v"(thr[0]), [t1] "v"(thr[1]), [t2] "v"(thr[2]), [t3] "v"(thr[3]), [roff] "n"(ROFF)
+  if constexpr (COUNT && READS) asm volatile(R128_TILE R128_OPERANDS);
+  else if constexpr (READS) asm volatile(R128_TILE_TEXT(R128_READ, R128_NOPAIR, R128_NOPAIR, R128_NOBCNT) R128_OPERANDS);
+  else if constexpr (COUNT) asm volatile(R128_TILE_TEXT(R128_NOREAD, R128_PAIR_FIRST, R128_PAIR, R128_BCNT) R128_OPERANDS);
+  else asm volatile(R128_TILE_TEXT(R128_NOREAD, R128_NOPAIR, R128_NOPAIR, R128_NOBCNT) R128_OPERANDS);
+#undef R128_OPERANDS
 }
 
 // W waves per workgroup (8: one workgroup per CU, 1024 queries; 4: two per CU, 512 queries each), two waves per SIMD.
-template <int W>
+// COUNT: false only in the measurement aid that times the walk without its count (kge_probe.hip).
+template <int W, bool COUNT = true>
 __global__ void __launch_bounds__(64 * W, 2) rank128_kernel(ContractArgs a, RankArgs ea) {
   constexpr int NQT = R128_NQT, KSTEPS = 8;
   constexpr int ROW_BYTES = 256;
@@ -301,7 +313,7 @@ __global__ void __launch_bounds__(64 * W, 2) rank128_kernel(ContractArgs a, Rank
   uint32_t dirty = 0;                       // query tiles 0..2 of the previous stage that need the exact pass
   for (int k = 0; k < n_st; ++k) {
     // first entity tile; the fragments of the second are fetched under its last chain
-    r128_tile<TILE_BYTES>(qf, ef, fb, X, thr, gt, mn);
+    r128_tile<TILE_BYTES, COUNT>(qf, ef, fb, X, thr, gt, mn);
     // every tile of the previous stage has been counted by now (query tile 3 of its second entity tile by the
     // statement above), and its buffer is intact until this wave passes the barrier below: the place for that
     // stage's exact pass, if it needs one
@@ -320,7 +332,7 @@ __global__ void __launch_bounds__(64 * W, 2) rank128_kernel(ContractArgs a, Rank
 #pragma unroll
     for (int s = 0; s < KSTEPS; ++s) fb[s] += step;
     // second entity tile; the fragments of the next stage's first tile are fetched under its last chain
-    r128_tile<0>(qf, ef, fb, X, thr, gt, mn);
+    r128_tile<0, COUNT>(qf, ef, fb, X, thr, gt, mn);
     dirty = tie_bit(mn[0], 0) | tie_bit(mn[1], 1) | tie_bit(mn[2], 2);
     prev_o = cur_o;
     cur_o = next_o;

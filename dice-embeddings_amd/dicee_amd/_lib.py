@@ -55,6 +55,11 @@ SIGNATURES = {
                                    _sz, _vp, _sz, _vp]),
     "kge_profile_begin": (_c_int, []),
     "kge_profile_end": (_c_int, [ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_int64)]),
+    "kge_profile_kernel": (ctypes.c_char_p, []),
+    "kge_probe_mfma": (_c_int, [_c_int, _c_int, ctypes.c_double, ctypes.POINTER(ctypes.c_double),
+                                ctypes.POINTER(ctypes.c_double), _vp]),
+    "kge_probe_walk": (_c_int, [_vp, _vp, _c_i64, _c_i64, ctypes.c_double, ctypes.POINTER(ctypes.c_double),
+                                ctypes.POINTER(ctypes.c_double), _vp]),
     "kge_row_minmax": (_c_int, [_vp, _vp, _vp, _c_int, _vp, _c_i64, _c_i64, _c_i64, _vp, _vp, _vp]),
     "kge_bce_workspace_bytes": (_sz, []),
     "kge_bce_multihot": (_c_int, [_vp, _vp, _vp, _c_int, _vp, _c_i64, _c_i64, _c_i64, _vp, _vp, _vp, _c_i64, _c_f,

@@ -6,7 +6,7 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(os.path.dirname(HERE), "csrc")
 OUT = os.path.join(HERE, "libkge_hip.so")
-SOURCES = ["kge_query.hip", "kge_kernels.hip", "kge_csr.hip"]
+SOURCES = ["kge_query.hip", "kge_kernels.hip", "kge_csr.hip", "kge_probe.hip"]
 # -ffp-contract=off: a score is compared bit for bit across kernels, so `acc * scale` must be rounded
 # before it is compared or subtracted; a fused multiply-add would skip that rounding.
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-shared", "-fPIC", "-ffp-contract=off",

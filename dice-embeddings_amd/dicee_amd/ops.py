@@ -356,3 +356,30 @@ def profile_end():
     n = ctypes.c_int64(0)
     _lib.check(_lib.load().kge_profile_end(ctypes.byref(ms), ctypes.byref(n)))
     return ms.value, n.value
+
+
+def profile_kernel():
+    """Name (with template arguments) of the main loop most recently timed while profiling was on, as the
+    library dispatched it."""
+    return _lib.load().kge_profile_kernel().decode("utf-8", "replace")
+
+
+def probe_mfma(count, reads, seconds=1.0):
+    """Measurement aid (``kge_probe_mfma``): the rank main loop's tile statement on random bf16 operands held in
+    registers, optionally with its count and with its fragment reads from LDS, for ``seconds``.
+    Returns (TFLOP/s of MFMAs issued, milliseconds per launch)."""
+    tf, ms = ctypes.c_double(0.0), ctypes.c_double(0.0)
+    _lib.check(_lib.load().kge_probe_mfma(int(bool(count)), int(bool(reads)), float(seconds), ctypes.byref(tf),
+                                          ctypes.byref(ms), _stream()))
+    return tf.value, ms.value
+
+
+def probe_walk(Q, E, seconds=1.0):
+    """Measurement aid (``kge_probe_walk``): the bf16 d = 128 rank main loop over ``E`` without its count.
+    Returns (TFLOP/s, milliseconds per launch)."""
+    assert Q.is_cuda and E.is_cuda and Q.dtype == torch.float32 and E.dtype == torch.bfloat16
+    assert Q.is_contiguous() and E.is_contiguous() and Q.shape[1] == 128 and E.shape[1] == 128
+    tf, ms = ctypes.c_double(0.0), ctypes.c_double(0.0)
+    _lib.check(_lib.load().kge_probe_walk(Q.data_ptr(), E.data_ptr(), Q.shape[0], E.shape[0], float(seconds),
+                                          ctypes.byref(tf), ctypes.byref(ms), _stream()))
+    return tf.value, ms.value

@@ -335,6 +335,27 @@ int kge_bce_multihot_backward(const float* Q, const float* bias, const void* E, 
  */
 int kge_profile_begin(void);
 int kge_profile_end(double* total_ms, int64_t* launches);
+/* Name (kernel and template arguments) of the main loop most recently bracketed while profiling was on, as the
+ * library itself dispatched it; "" before the first.  The pointer stays valid until the next call. */
+const char* kge_profile_kernel(void);
+
+/*
+ * Measurement aids; no counterpart in the reference and no part of any product path.  They time stripped-down
+ * forms of the filtered-rank main loop of bf16 tables with d == 128 for about `seconds` (at most 30) on `stream`
+ * and return the rate of the second half of the launches in TFLOP/s (2 * 32 * 32 * 16 flop per MFMA issued) and
+ * the average launch duration, so that a benchmark run can show from one box and one process what the MFMA unit
+ * sustains alone and what each part of the main loop costs:
+ *   kge_probe_mfma   256 workgroups of 8 waves (two waves per SIMD) issue the main loop's tile statement on random
+ *                    bf16 operands held in registers: count = 1 adds the rank count between the MFMAs (5 VALU
+ *                    instructions per MFMA), reads = 1 re-reads the entity fragments from LDS under every tile as
+ *                    the main loop does; no global memory traffic, no barriers.
+ *   kge_probe_walk   the main loop itself over the caller's bf16 table E [N,128] and queries Q [B,128] (fp32):
+ *                    global -> LDS stages, barriers, fragment reads and MFMAs, without the count.
+ * Both allocate (and free) a few bytes of device memory and synchronise the stream.
+ */
+int kge_probe_mfma(int count, int reads, double seconds, double* tflops, double* ms_per_launch, void* stream);
+int kge_probe_walk(const float* Q, const void* E, int64_t B, int64_t N, double seconds, double* tflops,
+                   double* ms_per_launch, void* stream);
 
 #ifdef __cplusplus
 }
