@@ -1683,6 +1683,12 @@ int scratch_on_current_device(unsigned char** out) {
 }
 }  // namespace
 
+extern "C" int kge_rank_static_init(void) {
+  clear_error();
+  unsigned char* base = nullptr;
+  return scratch_on_current_device(&base);
+}
+
 extern "C" int kge_rank_filtered_static(const float* Q, const float* bias, const void* E, int dtype, const float* scale,
                                         int64_t B, int64_t d, int64_t N, const int64_t* target, const int64_t* csr_row,
                                         const int64_t* row_ptr, const int32_t* col, int64_t n_rows, int32_t* n_greater,
@@ -1701,6 +1707,19 @@ extern "C" int kge_rank_filtered_static(const float* Q, const float* bias, const
   unsigned char* base = nullptr;
   rc = scratch_on_current_device(&base);
   if (rc) return rc;
+  // the scratch array used is the current device's: the operands must live there too (where the runtime cannot say,
+  // e.g. under a capture mode that refuses the query, the rule stays the caller's to keep)
+  {
+    int cur = -1;
+    KGE_HIP_CHECK(hipGetDevice(&cur));
+    hipPointerAttribute_t attr;
+    if (hipPointerGetAttributes(&attr, Q) == hipSuccess) {
+      KGE_REQUIRE(attr.device == cur, KGE_ERR_INVALID,
+                  "kge_rank_filtered_static: Q lives on device %d, the current device is %d", attr.device, cur);
+    } else {
+      (void)hipGetLastError();
+    }
+  }
   // nothing in the scratch needs clearing: thresholds, leaders and the mixed-group flags are written for every
   // query and every sub-batch's plan is rebuilt before anything reads it, so what an earlier call left behind is
   // never read

@@ -141,7 +141,10 @@ def rank_in_batches(model, x_all, target_all, csr, batch_size, tie="stable", str
                 lanes.fork()
                 for i in range(0, int(xs.shape[0]), bs):
                     lanes.switch()
-                    ops.rank_filtered(Q[i:i + bs], None if bias is None else bias[i:i + bs], E, scale,
+                    Qi = Q[i:i + bs]
+                    if Qi.data_ptr() % 16:      # (bs * d not a multiple of 4: the library wants 16-byte aligned rows)
+                        Qi = Qi.clone()
+                    ops.rank_filtered(Qi, None if bias is None else bias[i:i + bs], E, scale,
                                       target_all[g0 + i:g0 + i + bs], None if rows is None else rows[i:i + bs],
                                       None if csr is None else csr.row_ptr, None if csr is None else csr.col,
                                       out={k: v[g0 + i:g0 + i + bs] for k, v in counts.items()})

@@ -101,9 +101,20 @@ class BaseKGE(torch.nn.Module):
 
     def _refresh_storage(self):
         """The bf16 / int8 tables are copies: take them again when the parameters have changed since (an
-        optimizer step, ``load_state_dict``, a move to another device), so that scoring never reads stale weights."""
+        optimizer step, ``load_state_dict``, a move to another device).  The change is seen through the parameters'
+        storage address and autograd version counter, which in-place writes THROUGH ``weight.data`` do not advance
+        (``param_init(self.entity_embeddings.weight.data)`` in the reference, ``weight.data.copy_(...)`` in user
+        code): after such a write call ``refresh_storage()``."""
         if self._storage != "fp32" and self._snap_key != self._parameter_key():
             self.set_entity_storage(self._storage)
+
+    def refresh_storage(self):
+        """Take the bf16 / int8 copies of the tables (and the int8 table's prepared form for top-k) again from the
+        parameters as they are now.  Needed only after in-place writes through ``weight.data``, which leave no
+        trace the model could see; every other change of the parameters is picked up by itself."""
+        if self._storage != "fp32":
+            self.set_entity_storage(self._storage)
+        return self
 
     def table(self):
         """(entity table the kernels read, per-row scale or None)."""

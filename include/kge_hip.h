@@ -235,11 +235,17 @@ int kge_rank_filtered(const float* Q, const float* bias, const void* E, int dtyp
  * static device array inside the library (2.1 MB per GPU, held until the process ends), so
  *   - B <= KGE_RANK_STATIC_MAX_B, KGE_ERR_WORKSPACE otherwise (split the batch, or use kge_rank_filtered);
  *   - all calls on one GPU share that array: calls that overlap on one GPU (two streams, two threads) race;
- *   - the current device must be the one the pointers and the stream belong to.
+ *   - the current device must be the one the pointers and the stream belong to (checked for Q where the runtime
+ *     answers the question: KGE_ERR_INVALID on a mismatch);
+ *   - the first call on a device looks the array's address up (hipGetSymbolAddress, once per device): call
+ *     kge_rank_static_init() on that device, or make one ordinary call, BEFORE a stream capture begins, so
+ *     that nothing but kernel launches happens inside the capture.
  * Arguments, outputs and results are those of kge_rank_filtered, bit for bit.
+ * kge_rank_static_init: resolves and keeps the scratch address for the current device; allocates nothing.
  */
 #define KGE_RANK_STATIC_MAX_B 65536
 #define KGE_RANK_STATIC_SCRATCH_BYTES (12 * KGE_RANK_STATIC_MAX_B + 8 * (20 * 8192 + 1024) + 1024) /* 2.1 MB */
+int kge_rank_static_init(void);
 int kge_rank_filtered_static(const float* Q, const float* bias, const void* E, int dtype, const float* scale,
                              int64_t B, int64_t d, int64_t N, const int64_t* target, const int64_t* csr_row,
                              const int64_t* row_ptr, const int32_t* col, int64_t n_rows,
@@ -255,7 +261,9 @@ int kge_rank_filtered_static(const float* Q, const float* bias, const void* E, i
  *   The order is that of the scores before the per-query bias is added (and before the sigmoid): two
  *   entities whose scores become equal only through the rounding of score + bias, or of the sigmoid, keep
  *   the order of their unbiased scores.
- * This call synchronises `stream` once before returning (it reads back one overflow counter).
+ * This call (and kge_topk_prepared) synchronises `stream`: once before returning to read back one overflow
+ * counter, and once more per repair scan when a candidate buffer overflowed (at most 16 scans; still overflowing
+ * after those: KGE_ERR_OVERFLOW).  Neither can be captured into a HIP graph.
  */
 size_t kge_topk_workspace_bytes(int64_t B, int64_t N, int64_t k);
 int kge_topk(const float* Q, const float* bias, const void* E, int dtype, const float* scale,

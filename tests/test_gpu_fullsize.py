@@ -9,8 +9,52 @@ import pytest
 import torch
 
 from oracle import kge_oracle as ko
+from helpers import score_close
 
 pytestmark = pytest.mark.gpu
+
+
+def test_c1_toy_configuration_against_the_oracle():
+    """The first benchmark configuration itself (DistMult, 135 entities, 46 Zipf relations, 5,216 triples, d = 32
+    fp32, 512 queries, the filter CSR of all triples): every filtered rank against ``ko.filtered_ranks`` on the fp64
+    scores (equal wherever the tolerance interval is one point, inside it otherwise), scores at 1e-5, top-10 indices
+    wherever the oracle's order is decided beyond tolerance (dicee/evaluation/evaluator.py:473-510)."""
+    from dicee_amd import synthetic
+    from dicee_amd.evaluator import ranks_from_counts
+    cfg = synthetic.make_config("c1")
+    assert (cfg.N, cfg.R, cfg.d, cfg.B, len(cfg.queries), len(cfg.triples)) == (135, 46, 32, 512, 512, 5216)
+    model = synthetic.make_model(cfg, torch.device("cuda:0"))
+    cfg.csr.to("cuda")
+    q = cfg.queries
+    x = torch.from_numpy(q[:, :2].copy()).cuda()
+    t = torch.from_numpy(q[:, 2].copy()).cuda()
+    c = model.rank_filtered(x, t, cfg.csr)
+    ranks = ranks_from_counts(c["n_greater"], c["n_equal"], c["n_equal_lower"]).cpu().numpy()
+    S = ko.k_vs_all_scores("DistMult", cfg.E, cfg.Rel, q[:, :2])
+    ok, worst = score_close(model(x).cpu().numpy(), S, 1e-5)
+    assert ok, worst
+    filters = [cfg.csr.tails(int(h), int(r)) for h, r, _ in q]
+    want = ko.filtered_ranks(S, q[:, 2], filters)
+    rms = np.sqrt((S ** 2).mean(axis=1))
+    pinned = 0
+    for j in range(len(q)):
+        tol = 1e-5 * max(abs(S[j, q[j, 2]]), rms[j])
+        lo, hi = ko.rank_interval_with_tolerance(S[j], int(q[j, 2]), filters[j], tol)
+        assert lo <= ranks[j] <= hi, (j, lo, ranks[j], hi)
+        if lo == hi:
+            pinned += 1
+            assert ranks[j] == want[j]
+    assert pinned > 0.9 * len(q)
+    vals, idx = model.topk(x, 10)
+    order = np.argsort(-S, axis=1, kind="stable")
+    idx = idx.cpu().numpy()
+    decided = 0
+    for j in range(len(q)):
+        top = S[j, order[j, :11]]
+        if np.all(top[:-1] - top[1:] > 2e-5 * max(abs(top[0]), rms[j])):     # the first 11 are ordered beyond tolerance
+            decided += 1
+            np.testing.assert_array_equal(idx[j], order[j, :10])
+    assert decided > 0.5 * len(q)
 
 
 def test_c2_complex_filtered_mrr_eval_at_full_size():
@@ -101,6 +145,68 @@ def test_c4_fused_rank_matches_materialised_scores_and_is_batch_invariant(c4):
     assert np.all(plain["n_equal"].cpu().numpy() >= full["n_equal"].cpu().numpy())
 
 
+def test_c4_scores_ranks_and_topk_against_the_fp64_oracle(c4):
+    """The fourth configuration at its full size against the CPU oracle, for a sample of queries (the longest filter
+    rows among them) over all 2.5M entities: the bf16 tables are pulled to the host once and
+    ``ko.k_vs_all_scores("QMult", ...)`` scores them in fp64 (the reference's dequantised fp32 path up to fp32
+    rounding).  Scores within 2e-2; every fused rank inside the oracle's interval at that tolerance; and, against
+    fp64 products of the query vectors as the kernel reads them (rounded to bf16), scores within 1e-5, ranks inside
+    the interval at 1e-5 and top-10 indices equal wherever the 10th / 11th gap exceeds it
+    (dicee/evaluation/evaluator.py:473-510, knowledge_graph_embeddings.py:397-401)."""
+    from dicee_amd.evaluator import ranks_from_counts
+    cfg, model = c4
+    E_t, _ = model.table()
+    assert E_t.dtype == torch.bfloat16 and E_t.shape == (2_500_000, 128)
+    E = E_t.float().cpu().numpy()                                       # the bf16 values, exactly
+    Rel = model._rel().float().cpu().numpy()
+    q = cfg.queries[:4096]
+    x = torch.from_numpy(q[:, :2].copy()).cuda()
+    t = torch.from_numpy(q[:, 2].copy()).cuda()
+    full = model.rank_filtered(x, t, cfg.csr)
+    ranks = ranks_from_counts(full["n_greater"], full["n_equal"], full["n_equal_lower"]).cpu().numpy()
+    rows = cfg.csr.rows_for_numpy(q[:, :2])
+    lens = np.diff(cfg.csr.row_ptr_np)[rows]
+    pick = np.unique(np.concatenate([np.argsort(-lens)[:3], [1, 1500, 2047, 3071, 4095]]))
+    S64 = ko.k_vs_all_scores("QMult", E, Rel, q[pick, :2])              # [8, 2.5M] fp64
+    xs = x[pick].contiguous()
+    S_gpu = model(xs).cpu().numpy()
+    ok, worst = score_close(S_gpu, S64, 2e-2)
+    assert ok, worst
+    # the query vectors themselves follow the oracle's builder at fp32 grade
+    Qg, _ = model.query(xs)
+    Qo, _ = ko.build_query("QMult", E, Rel, q[pick, :2])
+    ok, worst = score_close(Qg.cpu().numpy(), Qo, 1e-5)
+    assert ok, worst
+    # ... and with them rounded to bf16 (what the MFMA multiplies) the fp64 product pins the scores at fp32 grade
+    Qb = ko.bf16_round(Qg.cpu().numpy()).astype(np.float64)
+    E64 = E.astype(np.float64)
+    S_tight = Qb @ E64.T
+    del E64
+    ok, worst = score_close(S_gpu, S_tight, 1e-5)
+    assert ok, worst
+    rms = np.sqrt((S64 ** 2).mean(axis=1))
+    vals, idx = model.topk(xs, 10)
+    idx = idx.cpu().numpy()
+    for j, b in enumerate(pick):
+        h, r, tt = (int(v) for v in q[b])
+        filt = cfg.csr.tails(h, r)
+        lo, hi = ko.rank_interval_with_tolerance(S64[j], tt, filt, 2e-2 * max(abs(S64[j, tt]), rms[j]))
+        assert lo <= ranks[b] <= hi, (b, lo, ranks[b], hi)
+        tol = 1e-5 * max(abs(S_tight[j, tt]), rms[j])
+        lo, hi = ko.rank_interval_with_tolerance(S_tight[j], tt, filt, tol)
+        assert lo <= ranks[b] <= hi, (b, lo, ranks[b], hi)
+        assert hi - lo <= 64                                            # (a handful of near-ties at most: the rank is pinned)
+        order = np.argsort(-S_tight[j], kind="stable")[:11]
+        top = S_tight[j, order]
+        tol_top = 1e-5 * max(abs(top[0]), rms[j])
+        if np.all(top[:-1] - top[1:] > 2 * tol_top):
+            np.testing.assert_array_equal(idx[j], order[:10])
+        else:                                                           # undecided order somewhere: same set beyond tolerance
+            assert set(np.nonzero(S_tight[j] > top[9] + 2 * tol_top)[0]) <= set(idx[j])
+            assert np.all(S_tight[j, idx[j]] >= top[9] - 2 * tol_top)
+    assert lens[pick].max() >= 10000
+
+
 def test_c4_topk_matches_materialised_scores(c4):
     cfg, model = c4
     q = torch.from_numpy(cfg.queries[4096:4096 + 600, :2].copy()).cuda()
@@ -158,15 +264,72 @@ def test_c5_int8_topk_matches_materialised_scores():
     wv, wi = ko.topk(S, cfg.k)
     np.testing.assert_array_equal(idx[::128].cpu().numpy(), wi)
     np.testing.assert_array_equal(vals[::128].cpu().numpy(), wv)
-    # scores follow fp32 math on the dequantised table within the int8 bar
+    # every sampled query against fp64 math on the dequantised table, over all 10M rows (the reference's path:
+    # full scores, then torch.topk, knowledge_graph_embeddings.py:397-401): values within the int8 bar, and the
+    # indices those of the oracle wherever its order is decided beyond tolerance
     E, scale = model.table()
-    rows = wi[0]
-    deq = (E[torch.from_numpy(rows).cuda()].float() * scale[torch.from_numpy(rows).cuda()][:, None]).cpu().numpy()
-    Q, _ = model.query(sub[:1])
-    ref = deq.astype(np.float64) @ Q[0].cpu().numpy().astype(np.float64)
-    np.testing.assert_allclose(wv[0], ref, rtol=2e-2)
+    Q, _ = model.query(sub)
+    Qn = Q.cpu().numpy()
+    Qo, _ = ko.build_query("DistMult", ko.dequantize_int8_rows(E[sub[:, 0]].cpu().numpy(), scale[sub[:, 0]].cpu().numpy()),
+                           model._rel().float().cpu().numpy(), np.stack([np.arange(len(sub)), sub[:, 1].cpu().numpy()], 1))
+    ok, worst = score_close(Qn, Qo, 1e-5)
+    assert ok, worst
+    Q64 = Qn.astype(np.float64)
+    Qb64 = ko.bf16_round(Qn).astype(np.float64)                          # the query as the kernels multiply it
+    S64 = np.empty((len(sub), cfg.N))
+    Sb64 = np.empty((len(sub), cfg.N))
+    step = 1_000_000
+    for r0 in range(0, cfg.N, step):
+        deq = E[r0:r0 + step].cpu().numpy().astype(np.float64) * scale[r0:r0 + step].cpu().numpy().astype(np.float64)[:, None]
+        S64[:, r0:r0 + step] = Q64 @ deq.T
+        Sb64[:, r0:r0 + step] = Qb64 @ deq.T
+    gi = idx[::128].cpu().numpy()
+    gv = vals[::128].cpu().numpy()
+    for j in range(len(sub)):
+        rms = np.sqrt((S64[j] ** 2).mean())
+        order = np.argsort(-S64[j], kind="stable")[:cfg.k + 1]
+        top = S64[j, order]
+        assert np.all(np.abs(gv[j] - S64[j, gi[j]]) <= 2e-2 * np.maximum(np.abs(S64[j, gi[j]]), rms))
+        tol = 2e-2 * max(abs(top[0]), rms)
+        assert set(np.nonzero(S64[j] > top[cfg.k - 1] + tol)[0]) <= set(gi[j])        # nothing clearly better is missing
+        assert np.all(S64[j, gi[j]] >= top[cfg.k - 1] - tol)                          # nothing clearly worse is in
+        # against the bf16-rounded query the scores are fp32-grade, which pins most positions exactly
+        tb = Sb64[j, np.argsort(-Sb64[j], kind="stable")[:cfg.k + 1]]
+        ob = np.argsort(-Sb64[j], kind="stable")[:cfg.k]
+        tol_b = 1e-5 * max(abs(tb[0]), rms)
+        assert np.all(np.abs(gv[j] - Sb64[j, gi[j]]) <= tol_b)
+        decided = np.concatenate([tb[:-2] - tb[1:-1] > 2 * tol_b, [tb[-2] - tb[-1] > 2 * tol_b]])
+        both = decided & np.concatenate([[True], decided[:-1]])           # both neighbours decided: the position is pinned
+        assert both.sum() > 0.8 * cfg.k
+        np.testing.assert_array_equal(gi[j][both], ob[both])
     del model
     torch.cuda.empty_cache()
+
+
+def test_c3_scores_and_loss_against_the_fp64_oracle():
+    """C3 at its full size against the CPU oracle: 16 rows of scores against ``ko.k_vs_all_scores("Keci", p=0, q=1)``
+    at 1e-5, and the fused loss of the whole 2048-row batch against ``ko.bce_multihot`` on the oracle's own fp64
+    scores (clifford.py:258-305, base_model.py:138, dataset_classes.py:354-361), with and without label smoothing."""
+    from dicee_amd import synthetic, ops
+    cfg = synthetic.make_config("c3")
+    assert (cfg.N, cfg.d, cfg.B, cfg.p, cfg.q) == (40943, 256, 2048, 0, 1)
+    model = synthetic.make_model(cfg, torch.device("cuda:0"))
+    cfg.csr.to("cuda")
+    hr = cfg.queries[:cfg.B, :2]
+    x = torch.from_numpy(hr.copy()).cuda()
+    kw = {"p": cfg.p, "q": cfg.q, "coeff_p": np.ones(cfg.p), "coeff_q": np.ones(cfg.q)}
+    S64 = ko.k_vs_all_scores("Keci", cfg.E, cfg.Rel, hr, **kw)          # [2048, 40943] fp64
+    rows = np.r_[0:8, 1020:1024, 2044:2048]
+    Q, bias = model.query(x[torch.from_numpy(rows).cuda()].contiguous())
+    E, _ = model.table()
+    ok, worst = score_close(ops.scores(Q, bias, E).cpu().numpy(), S64[rows], 1e-5)
+    assert ok, worst
+    positives = [cfg.csr.tails(int(h), int(r)) for h, r in hr]
+    assert max(len(p) for p in positives) >= 20                       # (multi-hot rows of tens of known tails among them)
+    for eps in (0.0, 0.1):
+        want = ko.bce_multihot(S64, positives, label_smoothing=eps)
+        got = model.kvsall_bce_loss(x, cfg.csr, label_smoothing=eps).item()
+        assert got == pytest.approx(want, rel=2e-6), (eps, got, want)
 
 
 def test_c3_bce_step_and_its_backward_at_full_size():

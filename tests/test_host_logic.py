@@ -81,6 +81,15 @@ def test_host_side_argument_validation_without_gpu(lib_path):
     assert rc != 0 and b"workspace" in lib.kge_last_error()
     rc = lib.kge_sample_scores(p256, None, p256, 0, None, 4, 16, 100, None, 3, None, None)
     assert rc == 1 and b"null" in lib.kge_last_error()
+    # operands must be 16-byte aligned: the second batch of d = 50 rows sliced out of one array of query vectors is not
+    off = ctypes.c_void_p(4096 + 3 * 50 * 4)
+    rc = lib.kge_rank_filtered(off, None, p256, 0, None, 3, 50, 100, p256, None, None, None, 0, p256, p256, p256, p256,
+                               p256, 1 << 20, None)
+    assert rc == 1 and b"16-byte aligned" in lib.kge_last_error()
+    # the measurement aids validate as well
+    rc = lib.kge_probe_mfma(0, 0, ctypes.c_double(100.0), None, None, None)
+    assert rc == 1 and b"kge_probe_mfma" in lib.kge_last_error()
+    assert lib.kge_profile_kernel() == b""
 
 
 def test_filter_csr_builders():
@@ -184,6 +193,27 @@ def test_models_mirror_reference_parameters_and_have_no_cpu_fallback():
                          "hidden_dropout_rate": 0.1})
     with pytest.raises(NotImplementedError, match="dropout"):
         hd(torch.zeros((2, 2), dtype=torch.int64))
+
+
+def test_quantised_copies_follow_the_parameters_except_through_weight_data():
+    """The bf16 / int8 copies are retaken when the parameters' version or storage changes; an in-place write through
+    ``weight.data`` leaves no trace (torch does not advance the version counter), which ``refresh_storage()`` covers."""
+    import torch
+    from dicee_amd import models
+    m = models.DistMult({"embedding_dim": 8, "num_entities": 12, "num_relations": 3})
+    m.set_entity_storage("bf16")
+    t0 = m.table()[0].clone()
+    with torch.no_grad():
+        m.entity_embeddings.weight.mul_(2.0)                 # an ordinary in-place update: seen
+    assert torch.equal(m.table()[0].float(), t0.float() * 2.0)
+    m.entity_embeddings.weight.data.mul_(0.5)                # through .data: not seen ...
+    assert torch.equal(m.table()[0].float(), t0.float() * 2.0)
+    m.refresh_storage()                                      # ... until asked
+    assert torch.equal(m.table()[0].float(), t0.float())
+    m.set_entity_storage("int8")
+    q0 = m.table()[1].clone()
+    m.entity_embeddings.weight.data.mul_(4.0)
+    assert torch.equal(m.refresh_storage().table()[1], q0 * 4.0)
 
 
 def test_evaluating_a_model_on_the_cpu_raises_what_the_ops_raise():

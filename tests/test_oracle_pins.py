@@ -393,6 +393,33 @@ def test_rank_counts_vs_bruteforce_and_invariants():
     assert ko.filtered_rank_counts(np.array([-np.inf, 0.0, -np.inf]), 1, []) == (0, 0, 0)
 
 
+def test_rank_interval_with_tolerance_against_brute_force():
+    """The checker every GPU rank test leans on.  At tol = 0 it is [1 + G, 1 + G + T] of ``filtered_rank_counts``;
+    at tol > 0 it is the set of ranks the target can take when every other kept score is moved anywhere within
+    +-tol of its value (brute force over the two extreme placements: all down, all up)."""
+    rng = np.random.default_rng(81)
+    N = 30
+    for trial in range(300):
+        s = rng.integers(-4, 5, N).astype(np.float64) / 4.0   # multiples of 0.25: ties and near-ties
+        t = int(rng.integers(0, N))
+        filt = list(rng.integers(0, N, rng.integers(0, 10)))
+        if trial % 3 == 0:
+            filt.append(t)
+        G, T, _ = ko.filtered_rank_counts(s, t, filt)
+        assert ko.rank_interval_with_tolerance(s, t, filt, 0.0) == (1 + G, 1 + G + T)
+        tol = float(rng.choice([0.1, 0.25, 0.3, 0.6]))
+        lo, hi = ko.rank_interval_with_tolerance(s, t, filt, tol)
+        keep = np.ones(N, bool)
+        keep[np.asarray(filt, dtype=int)] = False
+        keep[t] = False
+        # best case for the target: everybody else as low as allowed, and the target wins every tie
+        best = 1 + sum(1 for e in range(N) if keep[e] and s[e] - tol > s[t])
+        # worst case: everybody else as high as allowed, and the target loses every tie
+        worst = 1 + sum(1 for e in range(N) if keep[e] and s[e] + tol >= s[t])
+        assert (lo, hi) == (best, worst)
+        assert lo <= 1 + G and 1 + G + T <= hi                # the exact interval lies inside
+
+
 def test_evaluator_port_matches_closed_form_without_ties():
     rng = np.random.default_rng(9)
     N, Rn, d = 50, 5, 8

@@ -37,10 +37,15 @@ def _both(lib, Q, bias, E, dtype, scale, target, rows, row_ptr, col):
                                _p(col), n_rows, _p(want[0]), _p(want[1]), _p(want[2]), _p(want[3]), _p(ws), ws_bytes, st)
     assert rc == 0, lib.kge_last_error()
     got = outputs()
+    assert lib.kge_rank_static_init() == 0, lib.kge_last_error()
+    torch.cuda.synchronize()
+    held, free = torch.cuda.memory_allocated(), torch.cuda.mem_get_info()[0]
     rc = lib.kge_rank_filtered_static(_p(Q), _p(bias), _p(E), dtype, _p(scale), B, d, N, _p(target), _p(rows),
                                       _p(row_ptr), _p(col), n_rows, _p(got[0]), _p(got[1]), _p(got[2]), _p(got[3]), st)
     assert rc == 0, lib.kge_last_error()
     torch.cuda.synchronize()
+    # the call allocated nothing: neither through torch's allocator nor behind its back
+    assert torch.cuda.memory_allocated() == held and torch.cuda.mem_get_info()[0] == free
     return want, got
 
 
