@@ -414,6 +414,42 @@ def main():
                      "GB/s": gbytes / tg / 1e9, "frac_of_hbm_peak": gbytes / tg / 8e12,
                      "note": "head and relation rows read, query rows written; wall time of back-to-back calls from Python, "
                              "so launch and binding overhead are inside (the kernel alone: see profiles/)"}
+    # the same kernel at the size the evaluation loop runs it: the pairs of up to 64 batches in ONE launch
+    # (dicee_amd.evaluator.rank_in_batches), timed with events on the launch stream; bytes = the entity row and the
+    # query row of every pair (the relation rows, a few dozen distinct ones, stay in cache) + ids + bias
+    n_group = min(len(q_all), 64 * cfg.B)
+    xg_all = (q_all[:n_group, 1:] if mode == "headrank" else q_all[:n_group, :2]).contiguous()
+    for _ in range(3):
+        model.query(xg_all, heads=(mode == "headrank"))
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    reps = 30
+    e0.record()
+    for _ in range(reps):
+        model.query(xg_all, heads=(mode == "headrank"))
+    e1.record()
+    torch.cuda.synchronize()
+    tgg = e0.elapsed_time(e1) * 1e-3 / reps
+    gb_all = n_group * (d * esz + 4 * d + 16 + 4)
+    out["gather_grouped"] = {"kernel": "build_query_kernel", "pairs": n_group, "us_per_call": tgg * 1e6, "bytes": gb_all,
+                             "GB/s": gb_all / tgg / 1e9, "frac_of_hbm_peak": gb_all / tgg / 8e12,
+                             "note": "all pairs of an evaluation group in one launch, HIP events around 30 back-to-back "
+                                     "launches (allocation of the outputs by torch's caching allocator inside; at this "
+                                     "size the host's issue time per call is of the order of the kernel's)"}
+    # ... and over about a million pairs (the same pairs repeated), where the kernel's own duration dominates
+    rep_n = max(1, (1 << 20) // max(n_group, 1))
+    xg_big = xg_all.repeat(rep_n, 1).contiguous()
+    for _ in range(2):
+        model.query(xg_big, heads=(mode == "headrank"))
+    e0.record()
+    for _ in range(10):
+        model.query(xg_big, heads=(mode == "headrank"))
+    e1.record()
+    torch.cuda.synchronize()
+    tgb = e0.elapsed_time(e1) * 1e-3 / 10
+    gb_big = xg_big.shape[0] * (d * esz + 4 * d + 16 + 4)
+    out["gather_streaming"] = {"kernel": "build_query_kernel", "pairs": int(xg_big.shape[0]), "us_per_call": tgb * 1e6,
+                               "bytes": gb_big, "GB/s": gb_big / tgb / 1e9, "frac_of_hbm_peak": gb_big / tgb / 8e12}
+    del xg_big
     if len(cfg.triples):
         # side figure, outside the timed region: the known-answer vocabulary of all triples as a CSR, built on
         # the GPU (kge_csr_build) from ids already resident in HBM

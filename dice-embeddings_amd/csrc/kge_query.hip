@@ -526,8 +526,171 @@ __global__ void __launch_bounds__(64) build_query_backward_kernel(QueryBwdArgs a
   }
 }
 
+// ---- the same for the models whose query vector is elementwise in part-strided positions ------------------------
+// DistMult (1 part), ComplEx (2) and QMult (4), no normalisation layer: output element g of part j reads the head and
+// relation rows at g + i * d / parts only, so one THREAD owns one g of one pair, loads its 2 x parts elements straight
+// from the tables (lanes along g: whole lines per request), and stores its `parts` outputs; no LDS, no barrier, a
+// handful of registers.  QMult's relation normaliser divides every 4 CONSECUTIVE elements by their norm
+// (quaternion.py:28-43 on the flat row): the four lanes of a quad hold exactly such a group in every part (d / 4 is
+// a multiple of 4 whenever it matters: otherwise the general kernel runs), so the norm is a quad reduction.
+// A wave holds 64 x parts x 2 elements of reads in flight and nothing else, at full occupancy: the gather runs at
+// the memory system's rate for small requests instead of one 512-byte pair per wave lifetime.
+// VEC consecutive elements of a table row starting at element `off` (VEC = 4: one 16-, 8- or 4-byte load)
+template <int DT, int VEC>
+__device__ __forceinline__ void table_elems(const void* base, int64_t off, float (&v)[VEC]) {
+  if (VEC == 4) {
+    if (DT == KGE_F32) {
+      const f32x4 x = *(const f32x4*)((const float*)base + off);
+      v[0] = x[0]; v[1] = x[1]; v[2] = x[2]; v[3] = x[3];
+    } else if (DT == KGE_BF16) {
+      const u32x2 x = *(const u32x2*)((const uint16_t*)base + off);
+      v[0] = __uint_as_float(x[0] << 16); v[1] = __uint_as_float(x[0] & 0xffff0000u);
+      v[2] = __uint_as_float(x[1] << 16); v[3] = __uint_as_float(x[1] & 0xffff0000u);
+    } else {
+      const uint32_t x = *(const uint32_t*)((const int8_t*)base + off);
+      v[0] = (float)(int8_t)x; v[1] = (float)(int8_t)(x >> 8); v[2] = (float)(int8_t)(x >> 16); v[3] = (float)(int8_t)(x >> 24);
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) {
+      if (DT == KGE_F32) v[i] = ((const float*)base)[off + i];
+      else if (DT == KGE_BF16) v[i] = __uint_as_float((uint32_t)((const uint16_t*)base)[off + i] << 16);
+      else v[i] = (float)((const int8_t*)base)[off + i];
+    }
+  }
+}
+// x0 + x1 + x2 + x3 over the four lanes of a quad, added in that order in every lane (the order of the general kernel)
+__device__ __forceinline__ float quad_sum(float v, int lane) {
+  const int q0 = lane & ~3;
+  const float s0 = __shfl(v, q0, 64), s1 = __shfl(v, q0 + 1, 64), s2 = __shfl(v, q0 + 2, 64), s3 = __shfl(v, q0 + 3, 64);
+  return s0 + s1 + s2 + s3;
+}
+// A thread owns VEC consecutive elements g .. g + VEC - 1 of every part (VEC = 4 when a part's length and the rows'
+// addresses allow 16-byte accesses: one load per row and part, one 16-byte store per part, and the relation
+// normaliser's group of four inside the thread; VEC = 1 otherwise).  A workgroup of 256 threads takes floor(256 / u)
+// whole pairs when a part has at most 256 units (u = d / parts / VEC; `magic` = ceil(65536 / u) turns the thread number
+// into (pair, unit) without a division), otherwise one 256-unit block of one pair (`blocks` blocks per pair).
+template <int EDT, int RDT, int PARTS, int VEC>
+__global__ void __launch_bounds__(256) build_query_flat_kernel(QueryArgs a, int units, int ppw, int magic, int blocks) {
+  const int tid = threadIdx.x;
+  const int dp = units * VEC;
+  int64_t b;
+  int u;
+  bool live;
+  if (blocks == 1) {
+    const int pl = (tid * magic) >> 16;  // tid / units for tid < 256
+    u = tid - pl * units;
+    b = (int64_t)blockIdx.x * ppw + pl;
+    live = pl < ppw && b < a.B;  // (lanes past the end stay in the quad reductions with zeros)
+  } else {
+    b = blockIdx.x / blocks;
+    u = (int)(blockIdx.x - b * blocks) * 256 + tid;
+    live = u < units;
+    u = live ? u : 0;
+  }
+  const int g = u * VEC;
+  int64_t e_id = 0, r_id = 0;
+  if (live) {
+    e_id = a.hr[2 * b + (a.head_mode ? 1 : 0)];
+    r_id = a.hr[2 * b + (a.head_mode ? 0 : 1)];
+  }
+  const bool ok = live && e_id >= 0 && e_id < a.N && r_id >= 0 && r_id < a.R;
+  float h[PARTS][VEC], r[PARTS][VEC];
+#pragma unroll
+  for (int j = 0; j < PARTS; ++j) {
+    if (ok) {
+      table_elems<EDT, VEC>(a.ent, e_id * a.d + g + j * dp, h[j]);
+      table_elems<RDT, VEC>(a.rel, r_id * a.d + g + j * dp, r[j]);
+    } else {
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) h[j][i] = r[j][i] = 0.f;
+    }
+  }
+  if (EDT == KGE_I8) {
+    const float sc = ok ? a.ent_scale[e_id] : 0.f;
+#pragma unroll
+    for (int j = 0; j < PARTS; ++j)
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) h[j][i] *= sc;
+  }
+  if (PARTS == 4 && a.normalize_relation) {
+    // every 4 consecutive elements of the flat relation row by their norm, x / max(||x||, 1e-12)
+#pragma unroll
+    for (int j = 0; j < PARTS; ++j) {
+      float n;
+      if (VEC == 4) n = sqrtf(r[j][0] * r[j][0] + r[j][1] * r[j][1] + r[j][2] * r[j][2] + r[j][3] * r[j][3]);
+      else n = sqrtf(quad_sum(r[j][0] * r[j][0], tid & 63));
+      const float den = fmaxf(n, 1e-12f);
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) r[j][i] = r[j][i] / den;
+    }
+  }
+  float o[PARTS][VEC];
+#pragma unroll
+  for (int i = 0; i < VEC; ++i) {
+    if (PARTS == 1) {
+      o[0][i] = h[0][i] * r[0][i];
+    } else if (PARTS == 2) {
+      const float ri = a.head_mode ? -r[1][i] : r[1][i];
+      o[0][i] = h[0][i] * r[0][i] - h[1][i] * ri;
+      o[1][i] = h[0][i] * ri + h[1][i] * r[0][i];
+    } else {
+      const float conj = a.head_mode ? -1.f : 1.f;
+      const float ah = h[0][i], bh = h[1 % PARTS][i], ch = h[2 % PARTS][i], dh = h[3 % PARTS][i];
+      const float ar = r[0][i], br = conj * r[1 % PARTS][i], cr = conj * r[2 % PARTS][i], dr = conj * r[3 % PARTS][i];
+      o[0][i] = ah * ar - bh * br - ch * cr - dh * dr;
+      o[1 % PARTS][i] = ah * br + bh * ar + ch * dr - dh * cr;
+      o[2 % PARTS][i] = ah * cr - bh * dr + ch * ar + dh * br;
+      o[3 % PARTS][i] = ah * dr + bh * cr - ch * br + dh * ar;
+    }
+  }
+  if (!live) return;
+  const float nan = __uint_as_float(0x7fc00000u);
+  float* q = a.Q + b * a.d + g;
+#pragma unroll
+  for (int j = 0; j < PARTS; ++j) {
+    if (VEC == 4) {
+      f32x4 w = {ok ? o[j][0] : nan, ok ? o[j][1] : nan, ok ? o[j][2] : nan, ok ? o[j][3] : nan};
+      *(f32x4*)(q + j * dp) = w;
+    } else {
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) q[j * dp + i] = ok ? o[j][i] : nan;
+    }
+  }
+  if (u == 0) a.bias[b] = ok ? 0.f : nan;
+}
+
+template <int EDT, int PARTS>
+int launch_build_query_flat(const QueryArgs& a, int rel_dtype, hipStream_t st) {
+  const int dp = a.d / PARTS;
+  // 16-byte accesses: whole groups of four per part, rows that start on 16-byte (fp32), 8-byte (bf16), 4-byte (int8) bounds
+  const int eb = EDT == KGE_F32 ? 4 : EDT == KGE_BF16 ? 2 : 1, rb = rel_dtype == KGE_F32 ? 4 : 2;
+  const bool vec = dp % 4 == 0 && ((uintptr_t)a.ent % (4 * eb)) == 0 && ((uintptr_t)a.rel % (4 * rb)) == 0 &&
+                   ((uintptr_t)a.Q % 16) == 0;
+  const int units = vec ? dp / 4 : dp;
+  const int ppw = units <= 256 ? 256 / units : 1, blocks = units <= 256 ? 1 : (units + 255) / 256;
+  const int magic = (65536 + units - 1) / units;
+  const int64_t nwg = blocks == 1 ? (a.B + ppw - 1) / ppw : a.B * blocks;
+  KGE_REQUIRE(nwg <= 0x7fffffffLL, KGE_ERR_INVALID, "kge_build_query: B=%lld too large", (long long)a.B);
+  const dim3 grid((unsigned)nwg), block(256);
+  if (rel_dtype == KGE_F32) {
+    if (vec) hipLaunchKernelGGL((build_query_flat_kernel<EDT, KGE_F32, PARTS, 4>), grid, block, 0, st, a, units, ppw, magic, blocks);
+    else hipLaunchKernelGGL((build_query_flat_kernel<EDT, KGE_F32, PARTS, 1>), grid, block, 0, st, a, units, ppw, magic, blocks);
+  } else {
+    if (vec) hipLaunchKernelGGL((build_query_flat_kernel<EDT, KGE_BF16, PARTS, 4>), grid, block, 0, st, a, units, ppw, magic, blocks);
+    else hipLaunchKernelGGL((build_query_flat_kernel<EDT, KGE_BF16, PARTS, 1>), grid, block, 0, st, a, units, ppw, magic, blocks);
+  }
+  KGE_LAUNCH_CHECK("build_query_flat_kernel");
+  return KGE_OK;
+}
+
 template <int EDT>
 int launch_build_query(const QueryArgs& a, int model, int rel_dtype, hipStream_t st) {
+  if (a.norm.kind == KGE_NORM_NONE && a.B > 0) {
+    if (model == KGE_DISTMULT) return launch_build_query_flat<EDT, 1>(a, rel_dtype, st);
+    if (model == KGE_COMPLEX) return launch_build_query_flat<EDT, 2>(a, rel_dtype, st);
+    if (model == KGE_QMULT && (!a.normalize_relation || (a.d / 4) % 4 == 0)) return launch_build_query_flat<EDT, 4>(a, rel_dtype, st);
+  }
   dim3 grid((unsigned)a.B), block(64);
   size_t shmem = 2 * (size_t)a.d * sizeof(float);
   if (rel_dtype == KGE_F32)
