@@ -194,6 +194,13 @@ __global__ void __launch_bounds__(256) target_score_kernel(ContractArgs a, const
   }
 }
 
+// the one-vector-per-group check alone (a call whose thresholds were formed earlier, for many batches at once)
+__global__ void __launch_bounds__(256) group_check_kernel(ContractArgs a, const int32_t* lead, int32_t* mixed) {
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, c = lane & 31, hf = lane >> 5;
+  const int64_t q = ((int64_t)blockIdx.x * 4 + wave) * 32 + c;
+  if (q < a.B) group_vector_check(a, q, hf, lead, mixed);
+}
+
 // ---- scores of given entities per query: the same chain, nothing else ------------------------------
 // entity [B * group]: query b is scored against entity[b * group .. b * group + group - 1]
 // (group = 1: forward_triples; group = k: forward_k_vs_sample)
@@ -1588,11 +1595,13 @@ int check_rank_args(const char* who, const float* Q, const void* E, int dtype, c
 int rank_filtered_launch(const char* who, const float* Q, const float* bias, const void* E, int dtype, const float* scale,
                          int64_t B, int64_t d, int64_t N, const int64_t* target, const int64_t* csr_row,
                          const int64_t* row_ptr, const int32_t* col, int64_t n_rows, int32_t* n_greater, int32_t* n_equal,
-                         int32_t* n_equal_lower, float* target_score, void* ws_base, hipStream_t st) {
+                         int32_t* n_equal_lower, float* target_score, void* ws_base, hipStream_t st,
+                         const float* thr_in = nullptr, bool one_vector_per_row = false) {
   ContractArgs a = make_args(Q, E, dtype, scale, B, d, N, 0, N);
   const bool filtered = csr_row != nullptr && n_rows > 0;
   RankWs ws;
   rank_ws_layout(B, ws_base, &ws);
+  if (thr_in) ws.thr = const_cast<float*>(thr_in);  // formed (and the counters initialised) by kge_rank_thresholds
   if (filtered) {
     for (int64_t b0 = 0, sub = 0; b0 < B; b0 += SORT_MAX, ++sub) {
       const int nb = (int)((B - b0 < SORT_MAX) ? B - b0 : SORT_MAX);
@@ -1602,12 +1611,16 @@ int rank_filtered_launch(const char* who, const float* Q, const float* bias, con
       KGE_LAUNCH_CHECK("plan_fix_kernel");
     }
   }
-  {
+  if (!thr_in) {
     dim3 grid((unsigned)((B + 127) / 128 * (filtered ? 2 : 1))), block(256);  // (second half: the group check)
     KGE_DISPATCH_DTYPE(dtype, target_score_kernel, grid, block, 0, st, a, target, bias, ws.thr, target_score,
                        n_greater, n_equal, n_equal_lower, filtered ? (const int32_t*)ws.plan.lead : (const int32_t*)nullptr,
                        ws.plan.mixed);
     KGE_LAUNCH_CHECK("target_score_kernel");
+  } else if (filtered && !one_vector_per_row) {
+    hipLaunchKernelGGL(group_check_kernel, dim3((unsigned)((B + 127) / 128)), dim3(256), 0, st, a,
+                       (const int32_t*)ws.plan.lead, ws.plan.mixed);
+    KGE_LAUNCH_CHECK("group_check_kernel");
   }
   RankArgs ea{ws.thr, target, n_greater, n_equal, n_equal_lower};
   int rc = rank128_applies(dtype, d, B) ? launch_rank128(a, ea, st, who) : launch_contract<RankEpi>(dtype, a, ea, st, who);
@@ -1651,6 +1664,50 @@ extern "C" int kge_rank_filtered(const float* Q, const float* bias, const void* 
   KGE_REQUIRE(((uintptr_t)workspace & 7) == 0, KGE_ERR_WORKSPACE, "kge_rank_filtered: workspace must be 8-byte aligned");
   return rank_filtered_launch("kge_rank_filtered", Q, bias, E, dtype, scale, B, d, N, target, csr_row, row_ptr, col,
                               n_rows, n_greater, n_equal, n_equal_lower, target_score, workspace, (hipStream_t)stream);
+}
+
+// ---- thresholds of many batches at once, and the rank call that takes them ------------------------------
+extern "C" int kge_rank_thresholds(const float* Q, const float* bias, const void* E, int dtype, const float* scale,
+                                   int64_t B, int64_t d, int64_t N, const int64_t* target, float* thr,
+                                   int32_t* n_greater, int32_t* n_equal, int32_t* n_equal_lower, float* target_score,
+                                   void* stream) {
+  clear_error();
+  int rc = check_rank_args("kge_rank_thresholds", Q, E, dtype, scale, B, d, N, target, nullptr, nullptr, nullptr, 0,
+                           n_greater, n_equal, n_equal_lower, target_score);
+  if (rc) return rc;
+  if (B == 0) return KGE_OK;
+  KGE_REQUIRE(thr != nullptr, KGE_ERR_INVALID, "kge_rank_thresholds: null threshold array");
+  KGE_REQUIRE((B + 127) / 128 <= 0x7fffffffLL, KGE_ERR_INVALID, "kge_rank_thresholds: B=%lld too large", (long long)B);
+  ContractArgs a = make_args(Q, E, dtype, scale, B, d, N, 0, N);
+  hipStream_t st = (hipStream_t)stream;
+  dim3 grid((unsigned)((B + 127) / 128)), block(256);
+  KGE_DISPATCH_DTYPE(dtype, target_score_kernel, grid, block, 0, st, a, target, bias, thr, target_score, n_greater,
+                     n_equal, n_equal_lower, (const int32_t*)nullptr, (int32_t*)nullptr);
+  KGE_LAUNCH_CHECK("target_score_kernel");
+  return KGE_OK;
+}
+
+extern "C" int kge_rank_filtered_with_thresholds(const float* Q, const void* E, int dtype, const float* scale, int64_t B,
+                                                 int64_t d, int64_t N, const int64_t* target, const float* thr,
+                                                 const int64_t* csr_row, const int64_t* row_ptr, const int32_t* col,
+                                                 int64_t n_rows, int one_vector_per_row, int32_t* n_greater,
+                                                 int32_t* n_equal, int32_t* n_equal_lower, void* workspace,
+                                                 size_t workspace_bytes, void* stream) {
+  clear_error();
+  float dummy = 0.f;  // (target_score was written by kge_rank_thresholds; the argument check only wants a non-null pointer)
+  int rc = check_rank_args("kge_rank_filtered_with_thresholds", Q, E, dtype, scale, B, d, N, target, csr_row, row_ptr,
+                           col, n_rows, n_greater, n_equal, n_equal_lower, &dummy);
+  if (rc) return rc;
+  if (B == 0) return KGE_OK;
+  KGE_REQUIRE(thr != nullptr, KGE_ERR_INVALID, "kge_rank_filtered_with_thresholds: null threshold array");
+  KGE_REQUIRE(workspace && workspace_bytes >= kge_rank_workspace_bytes(B), KGE_ERR_WORKSPACE,
+              "kge_rank_filtered_with_thresholds: workspace of %zu bytes, need %zu", workspace_bytes,
+              kge_rank_workspace_bytes(B));
+  KGE_REQUIRE(((uintptr_t)workspace & 7) == 0, KGE_ERR_WORKSPACE,
+              "kge_rank_filtered_with_thresholds: workspace must be 8-byte aligned");
+  return rank_filtered_launch("kge_rank_filtered_with_thresholds", Q, nullptr, E, dtype, scale, B, d, N, target, csr_row,
+                              row_ptr, col, n_rows, n_greater, n_equal, n_equal_lower, nullptr, workspace,
+                              (hipStream_t)stream, thr, one_vector_per_row != 0);
 }
 
 // ---- the same call for callers that cannot allocate ---------------------------------------------------

@@ -43,6 +43,9 @@ SIGNATURES = {
     "kge_rank_workspace_bytes": (_sz, [_c_i64]),
     "kge_rank_filtered": (_c_int, [_vp, _vp, _vp, _c_int, _vp, _c_i64, _c_i64, _c_i64, _vp, _vp, _vp, _vp, _c_i64,
                                    _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
+    "kge_rank_thresholds": (_c_int, [_vp, _vp, _vp, _c_int, _vp, _c_i64, _c_i64, _c_i64, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
+    "kge_rank_filtered_with_thresholds": (_c_int, [_vp, _vp, _c_int, _vp, _c_i64, _c_i64, _c_i64, _vp, _vp, _vp, _vp, _vp,
+                                                   _c_i64, _c_int, _vp, _vp, _vp, _vp, _sz, _vp]),
     "kge_rank_static_init": (_c_int, []),
     "kge_rank_filtered_static": (_c_int, [_vp, _vp, _vp, _c_int, _vp, _c_i64, _c_i64, _c_i64, _vp, _vp, _vp, _vp, _c_i64,
                                           _vp, _vp, _vp, _vp, _vp]),

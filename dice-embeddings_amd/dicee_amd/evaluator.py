@@ -118,9 +118,9 @@ def rank_in_batches(model, x_all, target_all, csr, batch_size, tie="stable", str
     """Ranks (int64 tensor [n] on the model's device) of ``target_all`` [n] for the queries ``x_all`` [n,2]: one fused
     rank call per batch of ``batch_size`` queries.  What does not depend on the batching is done for many batches at a
     time: the query vectors and the filter rows of a group of batches (at most 64 batches or 256 MB of vectors; every
-    row is a function of its own (h, r) pair alone, so the numbers are those of batch-wise calls) come from one launch
-    each, and a batch is then nothing but the library's rank launches, writing its counters straight into the
-    evaluation's arrays.  Consecutive batches run on alternating streams; the ranks are formed once at the end."""
+    row is a function of its own (h, r) pair alone, so the numbers are those of batch-wise calls) and the thresholds
+    (the raw scores of the targets) come from one launch each, and a batch is then nothing but the plan of its filter
+    correction, the main loop and the correction, writing its counters straight into the evaluation's arrays.  Consecutive batches run on alternating streams; the ranks are formed once at the end."""
     from . import ops
     n = int(x_all.shape[0])
     dev = x_all.device
@@ -138,16 +138,22 @@ def rank_in_batches(model, x_all, target_all, csr, batch_size, tie="stable", str
                 Q, bias = model.query(xs, heads=heads)
                 E, scale = model.table()
                 rows = csr.rows_for(xs.to(device=E.device)) if csr is not None else None
+                g1 = g0 + int(xs.shape[0])
+                # the thresholds of the whole group (and its counters' initial values) come from one launch as well;
+                # a batch is then the plan of its filter correction, the main loop and the correction.  Query vectors
+                # and filter rows come from the same (h, r) pairs, so queries that share a row share a vector.
+                thr = ops.rank_thresholds(Q, bias, E, scale, target_all[g0:g1], {k: v[g0:g1] for k, v in counts.items()})
                 lanes.fork()
                 for i in range(0, int(xs.shape[0]), bs):
                     lanes.switch()
                     Qi = Q[i:i + bs]
                     if Qi.data_ptr() % 16:      # (bs * d not a multiple of 4: the library wants 16-byte aligned rows)
                         Qi = Qi.clone()
-                    ops.rank_filtered(Qi, None if bias is None else bias[i:i + bs], E, scale,
+                    ops.rank_filtered(Qi, None, E, scale,
                                       target_all[g0 + i:g0 + i + bs], None if rows is None else rows[i:i + bs],
                                       None if csr is None else csr.row_ptr, None if csr is None else csr.col,
-                                      out={k: v[g0 + i:g0 + i + bs] for k, v in counts.items()})
+                                      out={k: v[g0 + i:g0 + i + bs] for k, v in counts.items()},
+                                      thr=thr[i:i + bs], one_vector_per_row=True)
                 lanes.join()    # before the group's vectors are released to the allocator of the caller's stream
     finally:
         lanes.join()

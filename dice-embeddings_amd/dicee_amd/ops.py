@@ -226,10 +226,35 @@ _RANK_OUT = (("n_greater", torch.int32), ("n_equal", torch.int32), ("n_equal_low
              ("target_score", torch.float32))
 
 
-def rank_filtered(Q, bias, E, scale, target, csr_row=None, row_ptr=None, col=None, out=None):
+def rank_thresholds(Q, bias, E, scale, target, out):
+    """Thresholds (raw target scores) of ANY number of queries in one launch, for ``rank_filtered(..., thr=)``:
+    fills ``out`` (dict of [B] tensors as ``rank_filtered`` takes them: the counters initialised, ``target_score``
+    written) and returns the fp32 threshold tensor [B]."""
+    lib = _lib.load()
+    _require_gpu(Q, bias, E, scale, target)
+    _check_qe(Q, E, scale, bias)
+    B, d = Q.shape
+    if target.dtype != torch.int64:
+        raise TypeError("target must be int64")
+    for k, dt in _RANK_OUT:
+        o = out[k]
+        if o.dtype != dt or o.shape != (B,) or o.device != Q.device or not o.is_contiguous():
+            raise ValueError(f"out[{k!r}] must be a contiguous {dt} tensor of shape [{B}] on {Q.device}")
+    thr = torch.empty((B,), dtype=torch.float32, device=Q.device)
+    rc = lib.kge_rank_thresholds(_ptr(Q), _ptr(bias), _ptr(E), _table_dtype(E), _ptr(scale), B, d, E.shape[0],
+                                 _ptr(target), _ptr(thr), _ptr(out["n_greater"]), _ptr(out["n_equal"]),
+                                 _ptr(out["n_equal_lower"]), _ptr(out["target_score"]), _stream())
+    _lib.check(rc)
+    return thr
+
+
+def rank_filtered(Q, bias, E, scale, target, csr_row=None, row_ptr=None, col=None, out=None, thr=None,
+                  one_vector_per_row=False):
     """Fused filtered rank. Returns dict of int32 ``n_greater, n_equal, n_equal_lower`` and fp32
     ``target_score`` (all [B]).  ``out``: such a dict of contiguous [B] tensors to write into (slices of an
-    evaluation's arrays, say) instead of new ones."""
+    evaluation's arrays, say) instead of new ones.  ``thr``: this batch's slice of what ``rank_thresholds`` returned
+    for a larger set of queries (``out`` must then be the matching slices of the arrays that call initialised);
+    ``one_vector_per_row``: queries that share a filter row are known to hold the same query vector."""
     lib = _lib.load()
     _require_gpu(Q, bias, E, scale, target, csr_row, row_ptr, col)
     _check_qe(Q, E, scale, bias)
@@ -237,6 +262,8 @@ def rank_filtered(Q, bias, E, scale, target, csr_row=None, row_ptr=None, col=Non
     N = E.shape[0]
     dev = Q.device
     if out is None:
+        if thr is not None:
+            raise ValueError("thr= needs out=: the slices of the arrays that rank_thresholds initialised")
         out = {k: torch.empty((B,), dtype=dt, device=dev) for k, dt in _RANK_OUT}
     else:
         for k, dt in _RANK_OUT:
@@ -251,6 +278,15 @@ def rank_filtered(Q, bias, E, scale, target, csr_row=None, row_ptr=None, col=Non
             raise TypeError("csr_row/row_ptr must be int64 and col int32")
     if target.dtype != torch.int64:
         raise TypeError("target must be int64")
+    if thr is not None:
+        if thr.dtype != torch.float32 or thr.shape != (B,) or thr.device != dev or not thr.is_contiguous():
+            raise ValueError(f"thr must be a contiguous float32 tensor of shape [{B}] on {dev}")
+        rc = lib.kge_rank_filtered_with_thresholds(
+            _ptr(Q), _ptr(E), _table_dtype(E), _ptr(scale), B, d, N, _ptr(target), _ptr(thr), _ptr(csr_row),
+            _ptr(row_ptr), _ptr(col), n_rows, int(bool(one_vector_per_row)), _ptr(out["n_greater"]),
+            _ptr(out["n_equal"]), _ptr(out["n_equal_lower"]), _ptr(ws), ws_bytes, _stream())
+        _lib.check(rc)
+        return out
     rc = lib.kge_rank_filtered(_ptr(Q), _ptr(bias), _ptr(E), _table_dtype(E), _ptr(scale), B, d, N, _ptr(target),
                                _ptr(csr_row), _ptr(row_ptr), _ptr(col), n_rows, _ptr(out["n_greater"]),
                                _ptr(out["n_equal"]), _ptr(out["n_equal_lower"]), _ptr(out["target_score"]), _ptr(ws),

@@ -229,6 +229,27 @@ int kge_rank_filtered(const float* Q, const float* bias, const void* E, int dtyp
                       float* target_score, void* workspace, size_t workspace_bytes, void* stream);
 
 /*
+ * The same evaluation with the thresholds of MANY batches formed by one launch (evaluator.py:484-508 runs batch
+ * after batch; the threshold of a query, the raw score of its target, depends on nothing but its own row of Q):
+ *   kge_rank_thresholds   thr[b] = raw score of target[b] for b < B (any B: a whole evaluation), target_score[b]
+ *                         (+ bias), and the three counters initialised as kge_rank_filtered initialises them.
+ *   kge_rank_filtered_with_thresholds   kge_rank_filtered for a batch whose slices of thr and of the counters were
+ *                         prepared by that call: plan of the filter correction, main loop, correction.
+ *                         one_vector_per_row != 0: the caller guarantees that queries sharing a filter row hold the
+ *                         same query vector bit for bit (queries built from (head, relation) pairs and filter rows
+ *                         looked up from the same pairs do), which spares the launch that checks it.
+ * Results are those of kge_rank_filtered on the same batch, bit for bit.
+ */
+int kge_rank_thresholds(const float* Q, const float* bias, const void* E, int dtype, const float* scale, int64_t B,
+                        int64_t d, int64_t N, const int64_t* target, float* thr, int32_t* n_greater, int32_t* n_equal,
+                        int32_t* n_equal_lower, float* target_score, void* stream);
+int kge_rank_filtered_with_thresholds(const float* Q, const void* E, int dtype, const float* scale, int64_t B, int64_t d,
+                                      int64_t N, const int64_t* target, const float* thr, const int64_t* csr_row,
+                                      const int64_t* row_ptr, const int32_t* col, int64_t n_rows, int one_vector_per_row,
+                                      int32_t* n_greater, int32_t* n_equal, int32_t* n_equal_lower, void* workspace,
+                                      size_t workspace_bytes, void* stream);
+
+/*
  * kge_rank_filtered without a workspace argument and without any allocation.  No counterpart in the reference:
  * it exists for callers that cannot allocate device memory (code under HIP graph capture, tight serving
  * loops, harnesses that forbid hipMalloc).  The thresholds and the plan of the filter correction live in a

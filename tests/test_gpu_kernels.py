@@ -292,6 +292,47 @@ def test_rank_one_filter_row_shared_by_different_query_vectors(ops, FilterCSR, s
     np.testing.assert_array_equal(out["n_equal_lower"].cpu().numpy(), tl)
 
 
+@pytest.mark.parametrize("storage,d", [("fp32", 50), ("bf16", 128), ("bf16", 256), ("int8", 128)])
+def test_rank_with_hoisted_thresholds_equals_the_plain_call(ops, FilterCSR, storage, d):
+    """One threshold launch over all queries, then the rank in batches against slices of its result
+    (the evaluator's grouping, reference evaluator.py:484-508 processes the same batches one by one): counters and
+    target scores identical to ``rank_filtered`` over all queries at once.  With ``one_vector_per_row`` (rows and
+    vectors from the same (h, r) pairs) and without it (vectors that share a row but differ)."""
+    rng = np.random.default_rng(901 + d)
+    N, R, B, bs = 7000, 4, 1100, 256
+    E, Rel = random_tables(rng, N, R, d)
+    E[11] = E[12]                                   # an exact tie
+    hr = random_hr(rng, 60, R, B)
+    targets = rng.integers(0, N, B).astype(np.int64)
+    targets[:40] = 11
+    er = random_csr(rng, hr, targets, N, R, max_len=5, hub_rows=[(0, 3000)])
+    Et, sc, Rt, Ev, Rv = stored_tables(E, Rel, storage)
+    Eg, scg = dev(Et), dev(sc)
+    hr_g = dev(torch.from_numpy(hr))
+    tg = dev(torch.from_numpy(targets))
+    Q, _ = ops.build_query("DistMult", Eg, dev(Rt), hr_g, ent_scale=scg)
+    bias = dev(torch.from_numpy(rng.standard_normal(B).astype(np.float32)))
+    csr = FilterCSR.from_er_vocab(er, R, device="cuda")
+    rows = csr.rows_for(hr_g)
+    for same_vectors in (True, False):
+        if not same_vectors:
+            Q = Q.clone()
+            Q[::3] += dev(torch.from_numpy((rng.standard_normal((len(range(0, B, 3)), d)) * 0.01).astype(np.float32)))
+        want = ops.rank_filtered(Q, bias, Eg, scg, tg, rows, csr.row_ptr, csr.col)
+        got = {k: torch.full((B,), -7, dtype=v.dtype, device="cuda") for k, v in want.items()}
+        thr = ops.rank_thresholds(Q, bias, Eg, scg, tg, got)
+        np.testing.assert_array_equal(got["target_score"].cpu().numpy(), want["target_score"].cpu().numpy())
+        for i in range(0, B, bs):
+            sl = slice(i, min(i + bs, B))
+            Qi = Q[sl] if Q[sl].data_ptr() % 16 == 0 else Q[sl].clone()
+            ops.rank_filtered(Qi, None, Eg, scg, tg[sl], rows[sl], csr.row_ptr, csr.col,
+                              out={k: v[sl] for k, v in got.items()}, thr=thr[sl], one_vector_per_row=same_vectors)
+        for k in want:
+            np.testing.assert_array_equal(got[k].cpu().numpy(), want[k].cpu().numpy(), err_msg=f"{k} {same_vectors}")
+    with pytest.raises(ValueError):
+        ops.rank_filtered(Q, None, Eg, scg, tg, rows, csr.row_ptr, csr.col, thr=thr)      # thr= without out=
+
+
 @pytest.mark.parametrize("storage,d,N", [("bf16", 64, 4097), ("fp32", 1, 1000), ("fp32", 32, 3001), ("bf16", 128, 5000),
                                          ("int8", 128, 2500), ("bf16", 256, 1300), ("bf16", 256, 40000),
                                          ("bf16", 200, 40000), ("int8", 192, 2500)])
