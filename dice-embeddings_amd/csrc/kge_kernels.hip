@@ -2,6 +2,7 @@
 // fused multi-hot BCE, plus the small helper kernels around the two MFMA main loops.
 #include "kge_contract.hip.h"
 #include "kge_rank128.hip.h"
+#include "kge_wide.hip.h"
 #include "kge_topk_i8.hip.h"
 
 #include <string.h>
@@ -1198,6 +1199,9 @@ static inline RowClass row_class(int64_t d) {
   return RowClass{w, w != 0 && d != w};
 }
 constexpr int QS256_WG_QUERIES = QA_WG_WAVES * 32;
+// bf16 tables of 257..512 elements: the query row of one tile per wave in registers, entity rows through LDS in
+// segments of 128 columns (qwide_kernel)
+static inline bool wide_query_rows(int dtype, int64_t d) { return dtype == KGE_BF16 && d > 256 && d <= 512; }
 template <template <int> class EpiT>
 constexpr bool stream256_epilogue() {
   return std::is_same<EpiT<2>, RankEpi<2>>::value || std::is_same<EpiT<2>, StoreEpi<2>>::value;
@@ -1219,17 +1223,18 @@ ContractArgs make_args(const float* Q, const void* E, int dtype, const float* sc
   const RowClass rc = row_class(d);
   const bool fast_bf16 = dtype == KGE_BF16 && rc.lds_d != 0;  // (persistent whatever the epilogue)
   const bool fast_i8 = dtype == KGE_I8 && rc.lds_d != 0;
-  const bool wide_bf16 = (dtype == KGE_BF16 || dtype == KGE_I8) && rc.lds_d == 0;  // kchunk_kernel: the workgroup shape of the split kernel
-  const int wgq = (dtype == KGE_F32 || wide_bf16) ? KS_WG_QUERIES : rc.lds_d == 256 ? QS256_WG_QUERIES
+  const bool wide_q = wide_query_rows(dtype, d);  // qwide_kernel: persistent, one 32-query tile per wave
+  const bool wide_bf16 = (dtype == KGE_BF16 || dtype == KGE_I8) && rc.lds_d == 0 && !wide_q;  // kchunk_kernel: the workgroup shape of the split kernel
+  const int wgq = (dtype == KGE_F32 || wide_bf16) ? KS_WG_QUERIES : wide_q ? QW_WG_QUERIES : rc.lds_d == 256 ? QS256_WG_QUERIES
                   : fast_bf16 ? QA_WG_QUERIES : I8_WG_QUERIES;
   a.n_qgroups = (int)((B + wgq - 1) / wgq);
   if (a.n_qgroups < 1) a.n_qgroups = 1;
   const int64_t rows = e_end - e_begin;
   a.n_lanes = 1;
-  if (fast_bf16 || fast_i8) {
+  if (fast_bf16 || fast_i8 || wide_q) {
     // persistent paths: the workgroups resident on one XCD (32 CUs x workgroups per CU) are shared out
     // among the query groups
-    a.n_lanes = 32 * (fast_bf16 ? QA_WGS_PER_CU : I8_WGS_PER_CU) / a.n_qgroups;
+    a.n_lanes = 32 * (wide_q ? 1 : fast_bf16 ? QA_WGS_PER_CU : I8_WGS_PER_CU) / a.n_qgroups;
     if (a.n_lanes < 1) a.n_lanes = 1;
     int64_t chunk = rows / (8 * (int64_t)a.n_lanes * 4);  // aim for >= 4 chunks per workgroup
     chunk = (chunk + QA_STAGE_ROWS - 1) / QA_STAGE_ROWS * QA_STAGE_ROWS;
@@ -1315,7 +1320,8 @@ int launch_contract(int dtype, const ContractArgs& a, const EArgs& ea, hipStream
   const RowClass rc = row_class(a.d);
   const bool fast_bf16 = dtype == KGE_BF16 && rc.lds_d != 0;
   const bool fast_i8 = dtype == KGE_I8 && rc.lds_d != 0;
-  const bool persistent = fast_bf16 || fast_i8;
+  const bool wide_q = wide_query_rows(dtype, a.d);
+  const bool persistent = fast_bf16 || fast_i8 || wide_q;
   const bool pad = rc.pad;
   // (make_args and this function both decide, from the table, between the persistent and the tiled kernels; a plan
   // made for the other kind would be read as garbage, so the two must not drift apart)
@@ -1323,8 +1329,8 @@ int launch_contract(int dtype, const ContractArgs& a, const EArgs& ea, hipStream
   const int64_t nwg = persistent ? 8 * (int64_t)a.n_qgroups * a.n_lanes : contract_grid_wgs(a);
   KGE_REQUIRE(nwg <= 0x7fffffffLL, KGE_ERR_INVALID, "%s: grid of %lld workgroups too large", name, (long long)nwg);
   const bool f32_split = (dtype == KGE_F32);
-  const bool wide_bf16 = (dtype == KGE_BF16 || dtype == KGE_I8) && rc.lds_d == 0;
-  dim3 grid((unsigned)nwg), block(fast_i8 ? 64 * I8_WG_WAVES : persistent ? 64 * QA_WG_WAVES : 512);
+  const bool wide_bf16 = (dtype == KGE_BF16 || dtype == KGE_I8) && rc.lds_d == 0 && !wide_q;
+  dim3 grid((unsigned)nwg), block(fast_i8 ? 64 * I8_WG_WAVES : wide_q ? 64 * QW_WG_WAVES : persistent ? 64 * QA_WG_WAVES : 512);
   LaunchTimer timer;
   if (int trc = timer.begin(st)) return trc;
   char kname[160];  // the kernel as dispatched below, for kge_profile_kernel()
@@ -1340,6 +1346,15 @@ int launch_contract(int dtype, const ContractArgs& a, const EArgs& ea, hipStream
     hipLaunchKernelGGL((kchunk_kernel<KGE_BF16, EpiT>), grid, block, 0, st, a, ea);
   else if (wide_bf16)
     hipLaunchKernelGGL((kchunk_kernel<KGE_I8, EpiT>), grid, block, 0, st, a, ea);
+  else if (wide_q) {
+    const int ks = a.d <= 384 ? 24 : 32;
+    const bool wpad = a.d != 16 * ks;
+    snprintf(kname, sizeof(kname), "qwide_kernel<%s, %d, %s>", epi, ks, wpad ? "true" : "false");
+    if (ks == 24 && !wpad) hipLaunchKernelGGL((qwide_kernel<EpiT, 24, false>), grid, block, 0, st, a, ea);
+    else if (ks == 24) hipLaunchKernelGGL((qwide_kernel<EpiT, 24, true>), grid, block, 0, st, a, ea);
+    else if (!wpad) hipLaunchKernelGGL((qwide_kernel<EpiT, 32, false>), grid, block, 0, st, a, ea);
+    else hipLaunchKernelGGL((qwide_kernel<EpiT, 32, true>), grid, block, 0, st, a, ea);
+  }
   else if (fast_bf16) {
     // the rank epilogue has a branch-free form for the deeper-pipelined kernel (same workgroup shape, same counts)
     constexpr bool is_rank = std::is_same<EpiT<2>, RankEpi<2>>::value;

@@ -134,7 +134,11 @@ SCORE_CASES = [
     ("ComplEx", 321, 7, 64, 40, "bf16", {}),
     ("Keci", 1500, 6, 256, 300, "bf16", {"p": 0, "q": 1, "coeff_q": [1.0]}),      # d = 256: the streaming kernel, 512-byte rows
     ("DistMult", 9001, 5, 256, 700, "bf16", {}),     # the same over several stages per workgroup, partial last groups
-    ("DistMult", 500, 5, 384, 90, "bf16", {}),       # wider still: kchunk_kernel
+    ("DistMult", 500, 5, 384, 90, "bf16", {}),       # wider still: the query row in registers, rows through LDS by segments
+    ("DistMult", 9001, 5, 512, 700, "bf16", {}),     # the widest of that kernel, several stages and chunks, partial last groups
+    ("ComplEx", 4100, 5, 400, 300, "bf16", {}),      # its four-segment form on rows whose LDS tail stays zero
+    ("DistMult", 4100, 5, 264, 300, "bf16", {}),     # its three-segment form likewise
+    ("DistMult", 600, 5, 520, 90, "bf16", {}),       # wider than any register-resident form: kchunk_kernel
     ("ComplEx", 700, 7, 200, 150, "bf16", {}),       # between 128 and 256: the d = 256 kernels on rows whose LDS tail stays zero
     ("DistMult", 300, 5, 136, 70, "bf16", {}),
     ("ComplEx", 9001, 5, 200, 700, "bf16", {}),      # the same over several stages per workgroup, partial last groups
@@ -335,7 +339,8 @@ def test_rank_with_hoisted_thresholds_equals_the_plain_call(ops, FilterCSR, stor
 
 @pytest.mark.parametrize("storage,d,N", [("bf16", 64, 4097), ("fp32", 1, 1000), ("fp32", 32, 3001), ("bf16", 128, 5000),
                                          ("int8", 128, 2500), ("bf16", 256, 1300), ("bf16", 256, 40000),
-                                         ("bf16", 200, 40000), ("int8", 192, 2500)])
+                                         ("bf16", 200, 40000), ("int8", 192, 2500), ("bf16", 512, 40000),
+                                         ("bf16", 328, 2500)])
 def test_rank_partial_last_query_group_with_a_bias(ops, FilterCSR, storage, d, N):
     """B = 2500 leaves the last query group of every main loop partly filled (256-, 512- and 128-query groups), and
     the per-query bias is non-zero: ranks compare un-biased scores, target_score carries the bias."""
@@ -402,6 +407,8 @@ TOPK_CASES = [
     ("QMult", 20011, 5, 128, 600, "bf16", 10),
     ("DistMult", 30000, 9, 128, 70, "int8", 100),
     ("DistMult", 9000, 9, 192, 70, "int8", 50),      # int8 wider than 128
+    ("DistMult", 9000, 9, 512, 70, "bf16", 50),      # bf16 wider than 256: four segments of 128 columns
+    ("DistMult", 5000, 9, 320, 300, "bf16", 10),     # ... three, the last one partly zero
     ("DistMult", 5000, 9, 64, 33, "bf16", 1),
     ("DistMult", 6000, 9, 64, 20, "fp32", 1024),
     ("DistMult", 700, 9, 64, 20, "fp32", 600),       # k above half of the one-wave select's capacity
@@ -617,6 +624,7 @@ def test_topk_many_ties_at_the_top_survive_an_overflowing_round(ops, storage, k,
     ("DistMult", 2000, 5, 64, 100, "int8", {}),
     ("DistMult", 1100, 5, 160, 100, "int8", {}),
     ("ComplEx", 3000, 5, 200, 530, "bf16", {}),
+    ("DistMult", 3000, 5, 448, 300, "bf16", {}),
 ])
 @pytest.mark.parametrize("eps", [0.0, 0.1])
 def test_bce_multihot_vs_oracle(ops, FilterCSR, model, N, R, d, B, storage, kw, eps):
@@ -1014,7 +1022,7 @@ def test_topk_stress_patterns_match_the_materialised_scores(ops, seed, storage, 
 
 
 @pytest.mark.parametrize("storage,d", [("fp32", 32), ("bf16", 128), ("bf16", 64), ("int8", 128), ("int8", 64), ("bf16", 256),
-                                       ("bf16", 200), ("int8", 144)])
+                                       ("bf16", 200), ("int8", 144), ("bf16", 512), ("bf16", 360)])
 @pytest.mark.parametrize("pattern", ["pool1", "pool3", "pool50", "two_values", "zero_rows"])
 def test_rank_stress_patterns_match_the_materialised_scores(ops, FilterCSR, storage, d, pattern):
     """The same massively tied tables under the filtered rank: the target ties with thousands of entities (every
@@ -1075,6 +1083,10 @@ def _sweep_cases():
         N = int(rng.choice([1, 2, 31, 32, 33, 127, 128, 129, 257, 1000, 1025, 4097]))
         B = int(rng.choice([1, 2, 63, 64, 65, 255, 257, 513]))
         cases.append((i, storage, d, N, B))
+    # bf16 rows wider than 256 elements (the query row in registers, entity rows through LDS by segments)
+    for j, (d, N, B) in enumerate([(264, 33, 1), (384, 1, 257), (392, 129, 65), (512, 4097, 513), (512, 31, 2),
+                                   (456, 1025, 255), (272, 257, 64)]):
+        cases.append((36 + j, "bf16", d, N, B))
     return cases
 
 
