@@ -1199,9 +1199,9 @@ static inline RowClass row_class(int64_t d) {
   return RowClass{w, w != 0 && d != w};
 }
 constexpr int QS256_WG_QUERIES = QA_WG_WAVES * 32;
-// bf16 tables of 257..512 elements: the query row of one tile per wave in registers, entity rows through LDS in
-// segments of 128 columns (qwide_kernel)
-static inline bool wide_query_rows(int dtype, int64_t d) { return dtype == KGE_BF16 && d > 256 && d <= 512; }
+// bf16 and int8 tables of 257..512 elements: the query row of one tile per wave in registers, entity rows through LDS
+// in segments of 128 columns (qwide_kernel)
+static inline bool wide_query_rows(int dtype, int64_t d) { return (dtype == KGE_BF16 || dtype == KGE_I8) && d > 256 && d <= 512; }
 template <template <int> class EpiT>
 constexpr bool stream256_epilogue() {
   return std::is_same<EpiT<2>, RankEpi<2>>::value || std::is_same<EpiT<2>, StoreEpi<2>>::value;
@@ -1349,11 +1349,17 @@ int launch_contract(int dtype, const ContractArgs& a, const EArgs& ea, hipStream
   else if (wide_q) {
     const int ks = a.d <= 384 ? 24 : 32;
     const bool wpad = a.d != 16 * ks;
-    snprintf(kname, sizeof(kname), "qwide_kernel<%s, %d, %s>", epi, ks, wpad ? "true" : "false");
-    if (ks == 24 && !wpad) hipLaunchKernelGGL((qwide_kernel<EpiT, 24, false>), grid, block, 0, st, a, ea);
-    else if (ks == 24) hipLaunchKernelGGL((qwide_kernel<EpiT, 24, true>), grid, block, 0, st, a, ea);
-    else if (!wpad) hipLaunchKernelGGL((qwide_kernel<EpiT, 32, false>), grid, block, 0, st, a, ea);
-    else hipLaunchKernelGGL((qwide_kernel<EpiT, 32, true>), grid, block, 0, st, a, ea);
+    snprintf(kname, sizeof(kname), "qwide_kernel<%s, %s, %d, %s>", dtype == KGE_BF16 ? "KGE_BF16" : "KGE_I8", epi, ks,
+             wpad ? "true" : "false");
+    auto go = [&](auto edt) {
+      constexpr int EDT = decltype(edt)::value;
+      if (ks == 24 && !wpad) hipLaunchKernelGGL((qwide_kernel<EDT, EpiT, 24, false>), grid, block, 0, st, a, ea);
+      else if (ks == 24) hipLaunchKernelGGL((qwide_kernel<EDT, EpiT, 24, true>), grid, block, 0, st, a, ea);
+      else if (!wpad) hipLaunchKernelGGL((qwide_kernel<EDT, EpiT, 32, false>), grid, block, 0, st, a, ea);
+      else hipLaunchKernelGGL((qwide_kernel<EDT, EpiT, 32, true>), grid, block, 0, st, a, ea);
+    };
+    if (dtype == KGE_BF16) go(std::integral_constant<int, KGE_BF16>{});
+    else go(std::integral_constant<int, KGE_I8>{});
   }
   else if (fast_bf16) {
     // the rank epilogue has a branch-free form for the deeper-pipelined kernel (same workgroup shape, same counts)

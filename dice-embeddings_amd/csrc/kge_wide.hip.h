@@ -1,6 +1,6 @@
-// qwide_kernel: bf16 table, 256 < d <= 512 (gfx950).  The persistent walk of qstream_kernel with the whole query row
-// of ONE 32-query tile per wave in registers (32 fragments at d = 512: the 128 registers that hold four tiles at
-// d = 128) and the entity rows streamed through LDS in stages of one 32-row tile (rows of 1024 bytes, three buffers):
+// qwide_kernel: bf16 or per-row int8 table, 256 < d <= 512 (gfx950).  The persistent walk of qstream_kernel with the
+// whole query row of ONE 32-query tile per wave in registers (32 fragments at d = 512: the 128 registers that hold
+// four tiles at d = 128) and the entity rows streamed through LDS in stages of one 32-row tile (three buffers):
 // a score is ONE chain of d / 16 MFMAs on one accumulator, k ascending, as everywhere else, so the bits are those of
 // the other kernels.  The eight entity fragments a wave holds cover 128 columns (a segment); each is replaced, right
 // after the MFMA that consumed it, by the fragment of the same rows 128 columns on, and under the last segment by
@@ -8,6 +8,9 @@
 // of a kilobyte from L2 per MFMA (kchunk_kernel, which served these widths before: half a kilobyte, and the fp32
 // queries again for every entity tile).  Table rows narrower than the LDS row class (PAD) leave the row's tail zero
 // in LDS; a class is 24 or 32 K steps (d <= 384, d <= 512).
+// bf16 rows go global -> LDS directly, two stages ahead.  int8 rows are widened to bf16 (exactly) on the way: each
+// thread keeps its 32 bytes of the stage after next in registers for one stage, then converts and stores them; the
+// fp32 row scales ride along in LDS and a finished tile's scores are multiplied by them, as in the other int8 kernels.
 #pragma once
 #include "kge_contract.hip.h"
 
@@ -22,16 +25,19 @@ constexpr int QW_STAGE_ROWS = 32;
 constexpr int QW_STAGE_BYTES = QW_STAGE_ROWS * QW_ROW_BYTES;
 constexpr int QW_NBUF = 3;
 
-template <template <int> class EpiT, int KSTEPS, bool PAD>
+template <int EDT, template <int> class EpiT, int KSTEPS, bool PAD>
 __global__ void __launch_bounds__(64 * QW_WG_WAVES, 2) qwide_kernel(ContractArgs a, typename EpiT<1>::Args ea) {
   using Epi = EpiT<1>;
+  static_assert(EDT == KGE_BF16 || EDT == KGE_I8, "bf16 or int8 rows");
+  constexpr bool I8 = (EDT == KGE_I8);
   static_assert(KSTEPS == 24 || KSTEPS == 32, "three or four segments of eight K steps");
   static_assert(!Epi::DEFER, "the epilogue runs after its tile's chain");
   constexpr int NSEG = KSTEPS / 8;
   constexpr int d = 16 * KSTEPS;
   const int dq = PAD ? a.d : d;                         // elements of a query row and of a table row in memory
-  const int64_t row_stride = 2 * (int64_t)dq;           // bytes of a table row in memory
+  const int64_t row_stride = (I8 ? 1 : 2) * (int64_t)dq;  // bytes of a table row in memory
   __shared__ __attribute__((aligned(1024))) unsigned char lds_e[QW_NBUF * QW_STAGE_BYTES];
+  __shared__ __attribute__((aligned(16))) float lds_sc[I8 ? QW_NBUF : 1][QW_STAGE_ROWS];
 
   const int64_t wg = blockIdx.x;
   const int xcd = (int)(wg & 7);
@@ -77,34 +83,66 @@ __global__ void __launch_bounds__(64 * QW_WG_WAVES, 2) qwide_kernel(ContractArgs
   __shared__ typename Epi::Shared epi_sh;
   epi.bind(&epi_sh);
 
-  // This lane's share of a stage: piece `lane` (16 bytes) of the rows wave + 8 j, j = 0..3: one wave-wide load
-  // is one row, 1 KB in a piece.  In the table's last, partial stage the rows past the end repeat its last row
-  // (the epilogues ignore them).
+  // bf16: this lane's share of a stage is piece `lane` (16 bytes) of the rows wave + 8 j, j = 0..3: one wave-wide
+  // load is one row, 1 KB in a piece.  int8: this thread's share is piece tid % 32 (16 bytes, 16 elements) of the rows
+  // tid / 32 + 16 j, j = 0, 1.  In the table's last, partial stage the rows past the end repeat its last row (the
+  // epilogues ignore them).
   constexpr int NLD = QW_STAGE_ROWS / QW_WG_WAVES;
   const unsigned char* Eb = (const unsigned char*)a.E;
   if constexpr (PAD) {
     for (int i = tid * 16; i < QW_NBUF * QW_STAGE_BYTES; i += 64 * QW_WG_WAVES * 16) *(u32x4*)(lds_e + i) = u32x4{0u, 0u, 0u, 0u};
     __syncthreads();  // no load may land before the zeros do
   }
-  const bool lane_on = !PAD || 8 * lane < dq;  // (a lane past the row's end fetches nothing: its piece stays zero)
-  const uint32_t voff = (uint32_t)(wave * (int)row_stride + lane * 16);
+  const bool lane_on = !PAD || (I8 ? 16 * (tid & 31) : 8 * lane) < dq;  // (a lane past the row's end fetches nothing: its piece stays zero)
+  const uint32_t voff = I8 ? (uint32_t)((tid >> 5) * (int)row_stride + (tid & 31) * 16) : (uint32_t)(wave * (int)row_stride + lane * 16);
+  u32x4 held[I8 ? 2 : 1];  // int8: the rows on their way into LDS
+  float held_sc = 0.f;
   auto stage_issue = [&](int64_t row0, int buf_o) {
-    unsigned char* dst = lds_e + buf_o + wave * QW_ROW_BYTES;
-    if (!lane_on) return;
-    if (__builtin_expect(row0 + QW_STAGE_ROWS <= r_end, 1)) {
-      const unsigned char* src = Eb + row0 * row_stride;  // wave-uniform
+    if constexpr (I8) {
+      const bool full = row0 + QW_STAGE_ROWS <= r_end;  // (uniform)
 #pragma unroll
-      for (int j = 0; j < NLD; ++j)
-        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src + j * QW_WG_WAVES * row_stride + voff),
-                                         (__attribute__((address_space(3))) void*)(dst + j * (QW_WG_WAVES * QW_ROW_BYTES)), 16, 0, 0);
-    } else {
-#pragma unroll
-      for (int j = 0; j < NLD; ++j) {
-        int64_t g = row0 + wave + QW_WG_WAVES * j;
-        g = (g < r_end) ? g : r_end - 1;
-        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(Eb + g * row_stride + lane * 16),
-                                         (__attribute__((address_space(3))) void*)(dst + j * (QW_WG_WAVES * QW_ROW_BYTES)), 16, 0, 0);
+      for (int j = 0; j < 2; ++j) {
+        int64_t g = row0 + (tid >> 5) + 16 * j;
+        g = (full || g < r_end) ? g : r_end - 1;
+        if (lane_on) held[j] = *(const u32x4*)(Eb + g * row_stride + (tid & 31) * 16);
       }
+      if (tid < QW_STAGE_ROWS) {
+        int64_t g = row0 + tid;
+        g = (g < r_end) ? g : r_end - 1;
+        held_sc = a.scale[g];
+      }
+    } else {
+      unsigned char* dst = lds_e + buf_o + wave * QW_ROW_BYTES;
+      if (!lane_on) return;
+      if (__builtin_expect(row0 + QW_STAGE_ROWS <= r_end, 1)) {
+        const unsigned char* src = Eb + row0 * row_stride;  // wave-uniform
+#pragma unroll
+        for (int j = 0; j < NLD; ++j)
+          __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src + j * QW_WG_WAVES * row_stride + voff),
+                                           (__attribute__((address_space(3))) void*)(dst + j * (QW_WG_WAVES * QW_ROW_BYTES)), 16, 0, 0);
+      } else {
+#pragma unroll
+        for (int j = 0; j < NLD; ++j) {
+          int64_t g = row0 + wave + QW_WG_WAVES * j;
+          g = (g < r_end) ? g : r_end - 1;
+          __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(Eb + g * row_stride + lane * 16),
+                                           (__attribute__((address_space(3))) void*)(dst + j * (QW_WG_WAVES * QW_ROW_BYTES)), 16, 0, 0);
+        }
+      }
+    }
+  };
+  // int8: what stage_issue fetched goes into the buffer at byte offset buf_o (number buf_n)
+  auto stage_store = [&](int buf_o, int buf_n) {
+    if constexpr (I8) {
+      if (lane_on) {
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          unsigned char* dst = lds_e + buf_o + ((tid >> 5) + 16 * j) * QW_ROW_BYTES + (tid & 31) * 32;
+          *(u32x4*)dst = i8x8_to_bf16x8(held[j][0], held[j][1]);
+          *(u32x4*)(dst + 16) = i8x8_to_bf16x8(held[j][2], held[j][3]);
+        }
+      }
+      if (tid < QW_STAGE_ROWS) lds_sc[buf_n][tid] = held_sc;
     }
   };
   // the stage the next issue fetches (two ahead of the one being multiplied) and its position in its chunk
@@ -125,21 +163,31 @@ __global__ void __launch_bounds__(64 * QW_WG_WAVES, 2) qwide_kernel(ContractArgs
 #pragma unroll
   for (int i = 0; i < 16; ++i) sc_dummy[i] = 1.f;
 
-  // A barrier that orders nothing but the waves: the loads it guards are waited for explicitly, and the
-  // compiler is kept from moving LDS accesses across it.
+  // bf16: a barrier that orders nothing but the waves: the loads it guards are waited for explicitly, and the
+  // compiler is kept from moving LDS accesses across it.  int8: the stage went into LDS with ordinary stores.
   auto wg_barrier = [&]() {
-    __builtin_amdgcn_sched_barrier(0);
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __builtin_amdgcn_s_barrier();
-    asm volatile("" ::: "memory");
-    __builtin_amdgcn_sched_barrier(0);
+    if constexpr (I8) {
+      __syncthreads();
+    } else {
+      __builtin_amdgcn_sched_barrier(0);
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      __builtin_amdgcn_s_barrier();
+      asm volatile("" ::: "memory");
+      __builtin_amdgcn_sched_barrier(0);
+    }
   };
 
   stage_issue(issue_row, 0);
+  stage_store(0, 0);
   issue_advance();
   stage_issue(issue_row, QW_STAGE_BYTES);
+  stage_store(QW_STAGE_BYTES, 1);
   issue_advance();
   wg_barrier();
+  if constexpr (I8) {  // the stage after next waits in registers
+    stage_issue(issue_row, 0);
+    if (3 < n_st) issue_advance();
+  }
   bf16x8 ef[8];
 #pragma unroll
   for (int s = 0; s < 8; ++s) ef[s] = *(const bf16x8*)(lds_e + fbase + 32 * s);
@@ -147,6 +195,7 @@ __global__ void __launch_bounds__(64 * QW_WG_WAVES, 2) qwide_kernel(ContractArgs
   int64_t row0 = row_first;
   int so = 0;
   int cur_o = 0, next_o = QW_STAGE_BYTES, next2_o = 2 * QW_STAGE_BYTES;
+  int cur_n = 0, next_n = 1, next2_n = 2;  // (int8: the buffers' numbers, for the row scales)
 #pragma unroll 1
   for (int k = 0; k < n_st; ++k) {
     f32x16 acc;
@@ -174,9 +223,27 @@ __global__ void __launch_bounds__(64 * QW_WG_WAVES, 2) qwide_kernel(ContractArgs
     // stage k + 1 has landed for every wave, and everyone is done with the buffer of stage k - 1
     wg_barrier();
     if (Epi::STAGE_HOOK) epi.stage_end();
-    // stage k + 2 (past the last stage: the last stage's rows once more, into a buffer nobody reads)
+    // bf16: stage k + 2 is requested (past the last stage: the last stage's rows once more, into a buffer nobody
+    // reads).  int8: stage k + 2, requested a stage ago, is stored and stage k + 3 requested.
+    stage_store(next2_o, next2_n);
     stage_issue(issue_row, next2_o);
-    if (k + 3 < n_st) issue_advance();
+    if (k + (I8 ? 4 : 3) < n_st) issue_advance();
+    float sc16[16];
+    float sc_col = 1.f;
+    if constexpr (I8) {  // the row scales of this stage's tile: fetched under the last segment
+      if (Epi::SWAP) {
+        sc_col = lds_sc[cur_n][c];
+      } else {
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const f32x4 v = *(const f32x4*)&lds_sc[cur_n][8 * g + 4 * hf];
+          sc16[4 * g] = v[0];
+          sc16[4 * g + 1] = v[1];
+          sc16[4 * g + 2] = v[2];
+          sc16[4 * g + 3] = v[3];
+        }
+      }
+    }
     const unsigned char* nxt = lds_e + next_o + fbase;
 #pragma unroll
     for (int s = 0; s < 8; ++s) {
@@ -188,16 +255,20 @@ __global__ void __launch_bounds__(64 * QW_WG_WAVES, 2) qwide_kernel(ContractArgs
       __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
       __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
     }
-    epi.template tile<false>(0, acc, sc_dummy, 1.f, row0, r_end);
+    if constexpr (I8) epi.template tile<true>(0, acc, sc16, sc_col, row0, r_end);
+    else epi.template tile<false>(0, acc, sc_dummy, 1.f, row0, r_end);
     row0 += QW_STAGE_ROWS;
     if (++so == spc) {
       so = 0;
       row0 += chunk_skip;
     }
-    const int t = cur_o;
+    const int t = cur_o, tn = cur_n;
     cur_o = next_o;
     next_o = next2_o;
     next2_o = t;
+    cur_n = next_n;
+    next_n = next2_n;
+    next2_n = tn;
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // no load may land in LDS after the workgroup has gone
   epi.finish();

@@ -147,7 +147,10 @@ SCORE_CASES = [
     ("ComplEx", 1300, 7, 256, 300, "int8", {}),      # int8 d = 256: one query tile per wave
     ("DistMult", 777, 5, 144, 131, "int8", {}),      # between 128 and 256: the same kernel, rows padded with zeros in LDS
     ("DistMult", 9001, 5, 240, 700, "int8", {}),
-    ("DistMult", 400, 5, 272, 90, "int8", {}),       # wider than 256: kchunk_kernel, scales applied per tile
+    ("DistMult", 400, 5, 272, 90, "int8", {}),       # wider than 256: widened to bf16 on the way into the segmented LDS rows
+    ("DistMult", 9001, 5, 512, 700, "int8", {}),
+    ("ComplEx", 4100, 5, 400, 300, "int8", {}),
+    ("DistMult", 600, 5, 528, 90, "int8", {}),       # wider than any register-resident form: kchunk_kernel, scales applied per tile
 ]
 
 
@@ -340,7 +343,7 @@ def test_rank_with_hoisted_thresholds_equals_the_plain_call(ops, FilterCSR, stor
 @pytest.mark.parametrize("storage,d,N", [("bf16", 64, 4097), ("fp32", 1, 1000), ("fp32", 32, 3001), ("bf16", 128, 5000),
                                          ("int8", 128, 2500), ("bf16", 256, 1300), ("bf16", 256, 40000),
                                          ("bf16", 200, 40000), ("int8", 192, 2500), ("bf16", 512, 40000),
-                                         ("bf16", 328, 2500)])
+                                         ("bf16", 328, 2500), ("int8", 448, 2500)])
 def test_rank_partial_last_query_group_with_a_bias(ops, FilterCSR, storage, d, N):
     """B = 2500 leaves the last query group of every main loop partly filled (256-, 512- and 128-query groups), and
     the per-query bias is non-zero: ranks compare un-biased scores, target_score carries the bias."""
@@ -408,6 +411,7 @@ TOPK_CASES = [
     ("DistMult", 30000, 9, 128, 70, "int8", 100),
     ("DistMult", 9000, 9, 192, 70, "int8", 50),      # int8 wider than 128
     ("DistMult", 9000, 9, 512, 70, "bf16", 50),      # bf16 wider than 256: four segments of 128 columns
+    ("DistMult", 9000, 9, 512, 70, "int8", 50),      # int8 likewise
     ("DistMult", 5000, 9, 320, 300, "bf16", 10),     # ... three, the last one partly zero
     ("DistMult", 5000, 9, 64, 33, "bf16", 1),
     ("DistMult", 6000, 9, 64, 20, "fp32", 1024),
@@ -1022,7 +1026,7 @@ def test_topk_stress_patterns_match_the_materialised_scores(ops, seed, storage, 
 
 
 @pytest.mark.parametrize("storage,d", [("fp32", 32), ("bf16", 128), ("bf16", 64), ("int8", 128), ("int8", 64), ("bf16", 256),
-                                       ("bf16", 200), ("int8", 144), ("bf16", 512), ("bf16", 360)])
+                                       ("bf16", 200), ("int8", 144), ("bf16", 512), ("bf16", 360), ("int8", 512), ("int8", 368)])
 @pytest.mark.parametrize("pattern", ["pool1", "pool3", "pool50", "two_values", "zero_rows"])
 def test_rank_stress_patterns_match_the_materialised_scores(ops, FilterCSR, storage, d, pattern):
     """The same massively tied tables under the filtered rank: the target ties with thousands of entities (every
@@ -1087,6 +1091,9 @@ def _sweep_cases():
     for j, (d, N, B) in enumerate([(264, 33, 1), (384, 1, 257), (392, 129, 65), (512, 4097, 513), (512, 31, 2),
                                    (456, 1025, 255), (272, 257, 64)]):
         cases.append((36 + j, "bf16", d, N, B))
+    for j, (d, N, B) in enumerate([(272, 33, 1), (384, 1, 257), (400, 129, 65), (512, 4097, 513), (512, 31, 2),
+                                   (464, 1025, 255)]):
+        cases.append((43 + j, "int8", d, N, B))
     return cases
 
 
