@@ -34,7 +34,7 @@ PEAK_TFLOPS = {"bf16": 2500.0, "fp32": 2500.0 / 6.0, "int8": 5000.0}
 FP32_MFMA_PEAK_TFLOPS = 157.3
 # HBM bytes per launch of the main loop measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on the full-size
 # workload (each scaled by what the same counter reads for a plain 1 GiB copy kernel: x2.00 and x1.00).
-MEASURED_TRAFFIC_BYTES = {"c4": 688.0e6,     # per rank launch (678 MB read, 9 MB written)
+MEASURED_TRAFFIC_BYTES = {"c4": 660.0e6,     # per rank launch (659 MB read, 1.2 MB written)
                           "c5": 350.0e6,     # average over the 4 filter scans of a top-k call (4.2 GB per call over all kernels)
                           "c3": 59.4e6, "c2": 19.4e6}
 MODE = {"c1": "rank", "c2": "rank", "c3": "bce", "c4": "rank", "c5": "topk"}
@@ -131,6 +131,9 @@ def main():
                          "region; 0 switches it off)")
     ap.add_argument("--no-ceiling", action="store_true",
                     help="skip the `ceiling` side figures (vendor bf16 GEMM on random and on zero operands)")
+    ap.add_argument("--no-evaluation-pass", action="store_true",
+                    help="skip the `evaluation_pass` side figure (a profile of the step's own launches: the pass runs "
+                         "its batches on two streams, where a traced kernel's duration includes its wait for the other's CUs)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one plain 1 GiB-in / 1 GiB-out elementwise kernel (reference point for "
                          "FETCH_SIZE / WRITE_SIZE counters under rocprofv3 --pmc)")
@@ -313,7 +316,7 @@ def main():
     # side figure, outside the timed region: one whole evaluation pass over every query of the configuration as
     # dicee_amd.Evaluator runs it (vectors, filter rows and thresholds of a group of batches from one launch each,
     # batches alternating over two streams, the ranks formed at the end), wall clock of the best of three passes
-    if mode in ("rank", "headrank") and not args.graph:
+    if mode in ("rank", "headrank") and not args.graph and not args.no_evaluation_pass:
         from dicee_amd.evaluator import rank_in_batches
         xq = (q_all[:, 1:] if mode == "headrank" else q_all[:, :2]).contiguous()
         tq = (q_all[:, 0] if mode == "headrank" else q_all[:, 2]).contiguous()
