@@ -32,7 +32,9 @@ __global__ void __launch_bounds__(64 * QW_WG_WAVES, 2) qwide_kernel(ContractArgs
   constexpr bool I8 = (EDT == KGE_I8);
   static_assert(KSTEPS == 24 || KSTEPS == 32, "three or four segments of eight K steps");
   static_assert(!Epi::DEFER, "the epilogue runs after its tile's chain");
-  constexpr int NSEG = KSTEPS / 8;
+  constexpr int FR = 8;  // entity fragments a wave holds: a segment of 16 FR columns (4: no register left over is
+                         // needed any more, and the rank at d = 512 runs 2 - 3 % slower: a read has four MFMAs to land)
+  constexpr int NSEG = KSTEPS / FR;
   constexpr int d = 16 * KSTEPS;
   const int dq = PAD ? a.d : d;                         // elements of a query row and of a table row in memory
   const int64_t row_stride = (I8 ? 1 : 2) * (int64_t)dq;  // bytes of a table row in memory
@@ -76,6 +78,9 @@ __global__ void __launch_bounds__(64 * QW_WG_WAVES, 2) qwide_kernel(ContractArgs
         hi = src[1];
       }
       qf[s] = cvt_bf16x8(lo, hi);
+      // (one fragment at a time: with every fp32 load of the row in flight at once, the 128 registers of the
+      // finished fragments and the 256 of the loads do not fit, and fragments would live in scratch memory)
+      if (s % 4 == 3) asm volatile("" : "+v"(qf[s - 3]), "+v"(qf[s - 2]), "+v"(qf[s - 1]), "+v"(qf[s]));
     }
   }
   Epi epi;
@@ -188,9 +193,9 @@ __global__ void __launch_bounds__(64 * QW_WG_WAVES, 2) qwide_kernel(ContractArgs
     stage_issue(issue_row, 0);
     if (3 < n_st) issue_advance();
   }
-  bf16x8 ef[8];
+  bf16x8 ef[FR];
 #pragma unroll
-  for (int s = 0; s < 8; ++s) ef[s] = *(const bf16x8*)(lds_e + fbase + 32 * s);
+  for (int s = 0; s < FR; ++s) ef[s] = *(const bf16x8*)(lds_e + fbase + 32 * s);
 
   int64_t row0 = row_first;
   int so = 0;
@@ -205,13 +210,13 @@ __global__ void __launch_bounds__(64 * QW_WG_WAVES, 2) qwide_kernel(ContractArgs
 #pragma unroll
     for (int g = 0; g < NSEG - 1; ++g) {
 #pragma unroll
-      for (int s = 0; s < 8; ++s) {
-        acc = Epi::SWAP ? mfma_bf16(qf[8 * g + s], ef[s], acc) : mfma_bf16(ef[s], qf[8 * g + s], acc);
-        ef[s] = *(const bf16x8*)(cur + 32 * s + 256 * (g + 1));
+      for (int s = 0; s < FR; ++s) {
+        acc = Epi::SWAP ? mfma_bf16(qf[FR * g + s], ef[s], acc) : mfma_bf16(ef[s], qf[FR * g + s], acc);
+        ef[s] = *(const bf16x8*)(cur + 32 * s + 32 * FR * (g + 1));
       }
       // the order the scheduler is asked for: every MFMA followed by the read that replaces the fragment it consumed
 #pragma unroll
-      for (int s = 0; s < 8; ++s) {
+      for (int s = 0; s < FR; ++s) {
         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
         __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
       }
@@ -246,12 +251,12 @@ __global__ void __launch_bounds__(64 * QW_WG_WAVES, 2) qwide_kernel(ContractArgs
     }
     const unsigned char* nxt = lds_e + next_o + fbase;
 #pragma unroll
-    for (int s = 0; s < 8; ++s) {
-      acc = Epi::SWAP ? mfma_bf16(qf[8 * (NSEG - 1) + s], ef[s], acc) : mfma_bf16(ef[s], qf[8 * (NSEG - 1) + s], acc);
+    for (int s = 0; s < FR; ++s) {
+      acc = Epi::SWAP ? mfma_bf16(qf[FR * (NSEG - 1) + s], ef[s], acc) : mfma_bf16(ef[s], qf[FR * (NSEG - 1) + s], acc);
       ef[s] = *(const bf16x8*)(nxt + 32 * s);
     }
 #pragma unroll
-    for (int s = 0; s < 8; ++s) {
+    for (int s = 0; s < FR; ++s) {
       __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
       __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
     }
