@@ -422,6 +422,37 @@ TOPK_CASES = [
 ]
 
 
+@pytest.mark.parametrize("N,B,k,pattern", [(150001, 1100, 10, "random"), (70001, 2500, 100, "random"),
+                                           (140000, 1024, 10, "ties"), (131072, 900, 1, "best_last"),
+                                           (98304 + 17, 1030, 300, "random")])
+def test_topk_bf16_d128_long_rounds_equal_the_materialised_scores(ops, N, B, k, pattern):
+    """bf16 tables with d = 128, batches of a thousand queries and more, tables long enough for rounds of tens of
+    thousands of rows (the persistent scan with several chunks per workgroup).  Values and indices against the
+    library's own scores, ties towards the lower id; tables with thousands of exact ties, with the best rows at the
+    very end (every round collects), a partial last stage and a partial last query group."""
+    rng = np.random.default_rng(N + B + k)
+    d = 128
+    E = (rng.standard_normal((N, d)) * 0.1).astype(np.float32)
+    if pattern == "ties":
+        pool = (rng.standard_normal((7, d)) * 0.1).astype(np.float32)
+        E[rng.integers(0, N, N // 3)] = pool[rng.integers(0, 7, N // 3)]
+        E[N - 5000:] = pool[0]
+    if pattern == "best_last":
+        E *= np.linspace(0.2, 3.0, N, dtype=np.float32)[:, None]
+    Q = (rng.standard_normal((B, d)) * 0.1).astype(np.float32)
+    Q[3] = 0.0
+    Eg = dev(torch.from_numpy(E)).to(torch.bfloat16).contiguous()
+    Qg = dev(torch.from_numpy(Q))
+    bias = dev(torch.from_numpy(rng.standard_normal(B).astype(np.float32)))
+    vals, idx = ops.topk(Qg, bias, Eg, None, k)
+    # (the order is that of the scores before the bias, which is the same for every entity of a query: two raw scores
+    # that differ can round to one value once it is added)
+    S_raw = ops.scores(Qg, None, Eg, None).cpu().numpy()
+    wv, wi = ko.topk(S_raw, k)
+    np.testing.assert_array_equal(idx.cpu().numpy(), wi)
+    np.testing.assert_array_equal(vals.cpu().numpy(), (wv + bias.cpu().numpy()[:, None]).astype(np.float32))
+
+
 @pytest.mark.parametrize("model,N,R,d,B,storage,k", TOPK_CASES)
 def test_topk_exact_against_own_scores(ops, model, N, R, d, B, storage, k):
     rng, hr, Eg, scg, Q, bias, Ev, Rv = _setup(ops, model, N, R, d, B, storage, {}, seed=2)
