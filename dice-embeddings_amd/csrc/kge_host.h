@@ -24,13 +24,12 @@ namespace host {
 
 // ---- sizes shared by host and kernels -------------------------------------------------------------------
 constexpr int SORT_MAX = 8192;           // queries per sub-batch of the filter correction
-constexpr int WORK_MAX = 4 * SORT_MAX;   // upper bound on work items per sub-batch: sizes the work list, bounds the slice count
+constexpr int WORK_MAX = 16 * SORT_MAX;  // upper bound on work items per sub-batch (bounds the slice count only)
 constexpr int SLICE_MIN = 128;           // shortest slice of a filter row
 constexpr int SLICE_PREF = 256;          // slices of a large sub-batch are at least this long (fewer, longer work items)
 constexpr int SLICE_PREF_ITEMS = 4096;   // ... as long as that still leaves about this many work items
 constexpr int PLAN_SLOTS = 2 * SORT_MAX; // hash table of the plan kernel: load factor <= 0.5
 constexpr int PLAN_HASH_SHIFT = 18;      // 32 - log2(PLAN_SLOTS)
-constexpr int PLAN_ITEM_BYTES = 16;      // one record of the work list (PlanItem)
 static_assert(PLAN_SLOTS == (1 << (32 - PLAN_HASH_SHIFT)), "hash width");
 constexpr int TOPK_CAP = 4096;           // candidates a query can collect in one round
 constexpr int TOPK_MAX_K = 1024;
@@ -111,7 +110,7 @@ inline Status contract_rules(const char* who, const void* Q, const void* E, int 
 // sub-batch of SORT_MAX queries
 struct RankWsOffsets {
   size_t thr, lead, mixed, plans, total;
-  size_t plan_stride, skey, gend, work, meta, items;  // of one plan: stride between plans, offsets inside a plan
+  size_t plan_stride, skey, gend, work, meta;  // of one plan: stride between plans, offsets inside a plan
   int64_t n_plans;
 };
 inline RankWsOffsets rank_ws_offsets(int64_t B) {
@@ -132,8 +131,7 @@ inline RankWsOffsets rank_ws_offsets(int64_t B) {
   o.gend = align_up((size_t)SORT_MAX * 8, 256);
   o.work = o.gend + align_up((size_t)SORT_MAX * 4, 256);
   o.meta = o.work + align_up((size_t)SORT_MAX * 8, 256);
-  o.items = o.meta + 256;
-  o.plan_stride = o.items + (size_t)WORK_MAX * PLAN_ITEM_BYTES;
+  o.plan_stride = o.meta + 256;
   o.total = o.plans + (size_t)o.n_plans * o.plan_stride;
   return o;
 }
@@ -304,16 +302,6 @@ KGE_HD inline uint32_t plan_hash(int64_t row) { return ((uint32_t)row * 26544357
 KGE_HD inline unsigned long long plan_pack(unsigned long long members, unsigned long long slices) {
   return (1ull << 48) | (members << 32) | slices;
 }
-// a work item as the plan writes it and the correction reads it (16 bytes): the group's first member position and
-// member count, the entries of its slice, the slice's first entry in `col`
-struct PlanItem {
-  uint32_t first_members;  // first position | members << 16   (positions < SORT_MAX <= 2^13, members <= SORT_MAX)
-  int32_t entries;
-  int64_t col_begin;
-};
-KGE_HD inline uint32_t plan_item_pack(int first, int members) { return (uint32_t)first | ((uint32_t)members << 16); }
-KGE_HD inline int plan_item_first(uint32_t v) { return (int)(v & 0xffffu); }
-KGE_HD inline int plan_item_members(uint32_t v) { return (int)(v >> 16); }
 KGE_HD inline int plan_groups(unsigned long long v) { return (int)(v >> 48); }
 KGE_HD inline int plan_members(unsigned long long v) { return (int)((v >> 32) & 0xffffull); }
 KGE_HD inline unsigned int plan_slices(unsigned long long v) { return (unsigned int)(v & 0xffffffffull); }
@@ -345,7 +333,6 @@ KGE_HD inline int plan_key_pos(unsigned long long key) { return (int)(key & 0xff
 struct PlanModel {
   std::vector<unsigned long long> skey;
   std::vector<int32_t> gend, work;
-  std::vector<PlanItem> items;  // the work list: meta[0] records
   int32_t meta[3] = {0, 0, 0};
   const char* error = nullptr;
 };
@@ -423,20 +410,6 @@ inline PlanModel plan_fix_model(const int64_t* csr_row, int nb, int64_t n_rows, 
       m.work[2 * g + 1] = (int32_t)plan_slices(base);
       m.gend[first] = first + (int)members;
       tab_cnt[my_slot[i]] = first;
-      if ((unsigned long long)plan_slices(base) + n > (unsigned long long)WORK_MAX) {
-        fail("more work items than WORK_MAX");
-        return m;
-      }
-      for (unsigned long long z = 0; z < n; ++z) {  // the group's slices, one work item each
-        PlanItem it;
-        it.first_members = plan_item_pack(first, (int)members);
-        it.col_begin = row_ptr[my_row[i]] + (int64_t)z * slice;
-        const int64_t left = row_ptr[my_row[i] + 1] - it.col_begin;
-        it.entries = (int32_t)(left < slice ? left : slice);
-        if (plan_item_first(it.first_members) != first || plan_item_members(it.first_members) != (int)members || it.entries <= 0)
-          fail("a work item does not round-trip");
-        m.items.push_back(it);
-      }
       const unsigned long long next = base + val;
       if (plan_groups(next) != g + 1 || plan_members(next) != first + (int)members ||
           (unsigned long long)plan_slices(next) != (unsigned long long)plan_slices(base) + n)

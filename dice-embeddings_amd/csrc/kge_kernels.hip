@@ -259,7 +259,6 @@ struct FixPlan {
   int32_t* gend;             // [SORT_MAX] for a group's first position: one past its last position
   int32_t* work;             // [SORT_MAX][2] per group: (first position, index of its first work item)
   int32_t* meta;             // [0] work items, [1] slice length, [2] groups
-  host::PlanItem* items;     // [WORK_MAX] the work list: one record per (group, slice), in group order
   int32_t* lead;             // [B] per query: index of the first member of its group (itself for a leader), -1: no group
   int32_t* mixed;            // [B] per leader: set when some member of its group holds another query vector
 };
@@ -306,15 +305,14 @@ __global__ void __launch_bounds__(1024) plan_fix_kernel(const int64_t* csr_row, 
       my_pos[j] = atomicAdd(&tab_cnt[h], 1);
     }
   }
-  // leaders fetch their row's extent (unconditional loads of a valid row keep them in flight together)
-  int64_t len[QPT], row_begin[QPT];
+  // leaders fetch their row's length (unconditional loads of a valid row keep them in flight together)
+  int64_t len[QPT];
   unsigned long long my_total = 0;
 #pragma unroll
   for (int j = 0; j < QPT; ++j) {
     const bool lead = my_pos[j] == 0;
     const int64_t rr = lead ? my_row[j] : 0;
-    row_begin[j] = row_ptr[rr];
-    const int64_t l = row_ptr[rr + 1] - row_begin[j];
+    const int64_t l = row_ptr[rr + 1] - row_ptr[rr];
     len[j] = lead ? l : 0;
     my_total += (unsigned long long)len[j];
   }
@@ -346,20 +344,10 @@ __global__ void __launch_bounds__(1024) plan_fix_kernel(const int64_t* csr_row, 
   for (int j = 0; j < QPT; ++j) {
     if (val[j]) {
       const int g = host::plan_groups(base), first = host::plan_members(base);
-      const int members = tab_cnt[my_slot[j]];
       plan.work[2 * g] = first;
       plan.work[2 * g + 1] = (int)host::plan_slices(base);
-      plan.gend[first] = first + members;
+      plan.gend[first] = first + tab_cnt[my_slot[j]];
       tab_cnt[my_slot[j]] = first;  // only this leader reads or writes its group's slot in this phase
-      // the group's slices as work items (a hub row's few hundred stores leave one after the other: no wait)
-      host::PlanItem it;
-      it.first_members = host::plan_item_pack(first, members);
-      host::PlanItem* dst = plan.items + host::plan_slices(base);
-      for (int64_t z0 = 0; z0 < len[j]; z0 += slice, ++dst) {
-        it.col_begin = row_begin[j] + z0;
-        it.entries = (int32_t)((len[j] - z0 < slice) ? len[j] - z0 : slice);
-        *dst = it;
-      }
       tab_row[my_slot[j]] = tid + 1024 * j;  // the slot's row number has done its work: now the leader's index
     } else if (my_pos[j] == 0) {
       tab_cnt[my_slot[j]] = -1;     // empty filter row: nothing to take out for this group
@@ -420,9 +408,11 @@ __global__ void __launch_bounds__(256) filter_fix_kernel(ContractArgs a, FixPlan
   __shared__ int s_next;                       // first member still waiting after this round
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, c = lane & 31, hf = lane >> 5;
   const int n_work = plan.meta[0];
-  // This workgroup's work items are w = blockIdx.x + k * gridDim.x, read from the work list the plan wrote (before:
-  // a sixteen-way search in the group records, the member key and the row's extent, seven dependent loads at the
-  // head of every workgroup).  Up to FIX_ITEMS of them at a time are read by one thread each, side by side.
+  const int64_t slice = plan.meta[1];
+  const int n_groups = plan.meta[2];
+  // This workgroup's work items are w = blockIdx.x + k * gridDim.x.  Up to FIX_ITEMS of them at a time are
+  // resolved by one thread each, side by side (group by binary search, then the group's row and extent),
+  // so that their chains of dependent loads overlap instead of running once per item.
   __shared__ int32_t it_i0[FIX_ITEMS], it_m[FIX_ITEMS], it_mixed[FIX_ITEMS];
   __shared__ int64_t it_z0[FIX_ITEMS], it_z1[FIX_ITEMS];
   for (int k0 = 0; blockIdx.x + (int64_t)k0 * gridDim.x < n_work; k0 += FIX_ITEMS) {
@@ -430,15 +420,36 @@ __global__ void __launch_bounds__(256) filter_fix_kernel(ContractArgs a, FixPlan
     if (tid < FIX_ITEMS) {
       const int64_t w = blockIdx.x + (int64_t)(k0 + tid) * gridDim.x;
       if (w < n_work) {
-        const host::PlanItem it = plan.items[w];  // one 16-byte load: group, members, the slice's extent in `col`
-        const int i0 = host::plan_item_first(it.first_members);
-        const int m = host::plan_item_members(it.first_members);
+        int lo = 0, hi = n_groups;  // last group whose first work item is <= w: in [lo, hi)
+        // fifteen pivots per step, their loads in flight together: a sixteenth of the range is left (a search
+        // that halves the range is a chain of log2(n_groups) dependent loads at the head of every workgroup)
+        while (hi - lo > 16) {
+          const int step = (hi - lo) >> 4;
+          int first[15];
+#pragma unroll
+          for (int j = 0; j < 15; ++j) first[j] = plan.work[2 * (lo + step * (j + 1)) + 1];
+          int le = 0;  // pivots whose first work item is <= w: a prefix
+#pragma unroll
+          for (int j = 0; j < 15; ++j) le += (first[j] <= (int64_t)w) ? 1 : 0;
+          const int nlo = lo + step * le, nhi = (le < 15) ? lo + step * (le + 1) : hi;
+          lo = nlo;
+          hi = nhi;
+        }
+        while (hi - lo > 1) {
+          const int mid = (lo + hi) >> 1;
+          if (plan.work[2 * mid + 1] <= w) lo = mid; else hi = mid;
+        }
+        const int i0 = plan.work[2 * lo];
+        const int64_t z = w - plan.work[2 * lo + 1];
+        const unsigned long long key = plan.skey[i0];
+        const int64_t row = host::plan_key_row(key);
+        const int64_t L0 = row_ptr[row], L1 = row_ptr[row + 1];
+        const int64_t z0 = L0 + z * slice;
         it_i0[tid] = i0;
-        it_m[tid] = m;
-        // (only a group of several members can hold different vectors: two dependent loads, off the path of the rest)
-        it_mixed[tid] = (m > 1) ? plan.mixed[b0 + host::plan_key_pos(plan.skey[i0])] : 0;
-        it_z0[tid] = it.col_begin;
-        it_z1[tid] = it.col_begin + it.entries;
+        it_m[tid] = plan.gend[i0] - i0;
+        it_mixed[tid] = plan.mixed[b0 + host::plan_key_pos(key)];
+        it_z0[tid] = z0;
+        it_z1[tid] = (z0 + slice < L1) ? z0 + slice : L1;
       }
     }
     __syncthreads();
@@ -1463,7 +1474,6 @@ size_t rank_ws_layout(int64_t B, void* base, RankWs* ws, int64_t sub = 0) {
     ws->plan.gend = (int32_t*)(pl + o.gend);
     ws->plan.work = (int32_t*)(pl + o.work);
     ws->plan.meta = (int32_t*)(pl + o.meta);
-    ws->plan.items = (host::PlanItem*)(pl + o.items);
     ws->plan.lead = (int32_t*)(p + o.lead);
     ws->plan.mixed = (int32_t*)(p + o.mixed);
   }

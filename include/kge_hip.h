@@ -253,7 +253,7 @@ int kge_rank_filtered_with_thresholds(const float* Q, const void* E, int dtype, 
  * kge_rank_filtered without a workspace argument and without any allocation.  No counterpart in the reference:
  * it exists for callers that cannot allocate device memory (code under HIP graph capture, tight serving
  * loops, harnesses that forbid hipMalloc).  The thresholds and the plan of the filter correction live in a
- * static device array inside the library (6.3 MB per GPU, held until the process ends), so
+ * static device array inside the library (2.1 MB per GPU, held until the process ends), so
  *   - B <= KGE_RANK_STATIC_MAX_B, KGE_ERR_WORKSPACE otherwise (split the batch, or use kge_rank_filtered);
  *   - all calls on one GPU share that array: calls that overlap on one GPU (two streams, two threads) race;
  *   - the current device must be the one the pointers and the stream belong to (checked for Q where the runtime
@@ -265,7 +265,7 @@ int kge_rank_filtered_with_thresholds(const float* Q, const void* E, int dtype, 
  * kge_rank_static_init: resolves and keeps the scratch address for the current device; allocates nothing.
  */
 #define KGE_RANK_STATIC_MAX_B 65536
-#define KGE_RANK_STATIC_SCRATCH_BYTES (12 * KGE_RANK_STATIC_MAX_B + 8 * (20 * 8192 + 1024 + 16 * 4 * 8192) + 1024) /* 6.3 MB */
+#define KGE_RANK_STATIC_SCRATCH_BYTES (12 * KGE_RANK_STATIC_MAX_B + 8 * (20 * 8192 + 1024) + 1024) /* 2.1 MB */
 int kge_rank_static_init(void);
 int kge_rank_filtered_static(const float* Q, const float* bias, const void* E, int dtype, const float* scale,
                              int64_t B, int64_t d, int64_t N, const int64_t* target, const int64_t* csr_row,

@@ -807,11 +807,8 @@ def test_plan_written_by_the_gpu_satisfies_the_host_model_invariants(ops, Filter
     o_gend = o_skey + up(8 * SORT_MAX)
     o_work = o_gend + up(4 * SORT_MAX)
     o_meta = o_work + up(8 * SORT_MAX)
-    o_items = o_meta + 256
-    WORK_MAX = 4 * SORT_MAX
-    assert o_items + 16 * WORK_MAX == ws_bytes
+    assert o_meta + 256 == ws_bytes
     raw = ws.cpu().numpy()
-    items = raw[o_items:o_items + 16 * WORK_MAX].view(np.dtype([("fm", "<u4"), ("n", "<i4"), ("col", "<i8")]))
     skey = raw[o_skey:o_skey + 8 * SORT_MAX].view(np.uint64)
     gend = raw[o_gend:o_gend + 4 * SORT_MAX].view(np.int32)
     work = raw[o_work:o_work + 8 * SORT_MAX].view(np.int32).reshape(-1, 2)
@@ -838,15 +835,8 @@ def test_plan_written_by_the_gpu_satisfies_the_host_model_invariants(ops, Filter
         assert members == want[row]
         # every member knows the group's leader (the query at the group's first sorted position); no group mixes vectors
         assert all(int(lead[i]) == int(skey[first] & np.uint64(0xffffff)) for i in members)
-        # the group's records in the work list: its slices in order, together the whole row
-        at = int(rp[row])
-        for w in range(seen_work, seen_work + -(-(int(rp[row + 1] - rp[row])) // slice_len)):
-            assert int(items["fm"][w]) & 0xffff == first and int(items["fm"][w]) >> 16 == end - first
-            assert int(items["col"][w]) == at and 1 <= int(items["n"][w]) <= slice_len
-            at += int(items["n"][w])
-        assert at == int(rp[row + 1])
         seen_work += -(-(int(rp[row + 1] - rp[row])) // slice_len)
-    assert seen_work == n_work and n_work <= WORK_MAX
+    assert seen_work == n_work
     no_row = [i for i, r in enumerate(rows_h) if not (r >= 0 and rp[r + 1] > rp[r])]
     assert all(int(lead[i]) == -1 for i in no_row)
 
