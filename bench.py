@@ -393,6 +393,22 @@ def main():
                 del Ai, Bi
             except Exception as exc:                                    # noqa: BLE001 (a side figure: report, go on)
                 ceil["torch_int_mm_int8_8192_cubed_randint"] = {"error": f"{type(exc).__name__}: {exc}"[:200]}
+        if compute == "int8" and mode == "topk" and model._topk_prepared is not None and model._topk_prepared[1] is not None:
+            # the scan's hot loop alone (library measurement aid kge_probe_i8_scan): the same kernel over the whole
+            # prepared table with every threshold at +inf, so that no tile passes the bound and nothing is parked or
+            # collected; the rounds of a call run the same loop plus the slow path of the tiles that pass
+            try:
+                xq = batches[0][0]
+                Qp, _ = model.query(xq)
+                r, ms = ops.probe_i8_scan(Qp, model._topk_prepared[1], N, 1.0)
+                ceil["int8_scan_hot_loop_only"] = {
+                    "achieved": r, "frac": r / PEAK_TFLOPS["int8"], "ms": ms, "rows": N, "queries": int(Qp.shape[0]),
+                    "note": "one launch over all rows; a call's four filter rounds cover the rows past the first 65,536 "
+                            "once, so a call's hot-loop time is about this many ms and the rest of its filter time "
+                            "is the slow path of the tiles that pass the bound"}
+                del Qp
+            except Exception as exc:                                    # noqa: BLE001 (a side figure: report, go on)
+                ceil["int8_scan_hot_loop_only"] = {"error": f"{type(exc).__name__}: {exc}"[:200]}
         if d == 128 and mode == "rank" and model.table()[0].dtype == torch.bfloat16:
             # the ladder of the rank main loop, bottom up, each rung sustained for ~0.7 s in this process (library
             # measurement aids kge_probe_mfma / kge_probe_walk): the tile statement's MFMAs on random bf16 operands

@@ -7,9 +7,16 @@
 //   kge_probe_mfma(count = 0 / 1, reads = 1)  the same with the entity fragments re-read from LDS every tile
 //   kge_probe_walk                        the main loop itself over a caller's table (global -> LDS stages, barriers,
 //                                         fragment reads, MFMAs) without the count
+// and, for the top-k scan of int8 tables (topk_i8_filter_kernel):
+//   kge_probe_i8_scan                     the scan over a caller's prepared table with thresholds of +inf: no tile
+//                                         passes the bound, so what is timed is the hot loop alone (MFMAs, the test
+//                                         of every tile, the walk), none of the parking and collecting of candidates
 #include "kge_rank128.hip.h"
+#include "kge_topk_i8.hip.h"
 
 #include <string.h>
+
+#include <vector>
 
 namespace kge {
 namespace {
@@ -199,3 +206,66 @@ extern "C" int kge_probe_walk(const float* Q, const void* E, int64_t B, int64_t 
   if (ms_per_launch) *ms_per_launch = ms;
   return KGE_OK;
 }
+
+extern "C" int kge_probe_i8_scan(const float* Q, const void* prepared, int64_t B, int64_t N, double seconds, double* pops,
+                                 double* ms_per_launch, void* stream) {
+  clear_error();
+  KGE_REQUIRE(Q && prepared && B >= 1 && N >= 1 && N <= 0x7fffffffLL && pops && seconds > 0.0 && seconds <= 30.0,
+              KGE_ERR_INVALID, "kge_probe_i8_scan: bad arguments");
+  KGE_REQUIRE((((uintptr_t)Q | (uintptr_t)prepared) & 255) == 0, KGE_ERR_INVALID,
+              "kge_probe_i8_scan: Q and the prepared table must be 256-byte aligned");
+  hipStream_t st = (hipStream_t)stream;
+  const host::TopkPreparedOffsets t = host::topk_prepared_offsets(N);
+  // the queries as the scan reads them (int8 rows, four constants each), thresholds of +inf, candidate counters and
+  // a token candidate buffer (nothing is ever written to it)
+  auto up = [](size_t x) { return (x + 255) / 256 * 256; };
+  const size_t o_qh = 0, o_qc = up((size_t)B * 128), o_tau = o_qc + up((size_t)B * 16), o_cnt = o_tau + up((size_t)B * 4),
+               o_cand = o_cnt + up((size_t)B * 4), bytes = o_cand + up((size_t)B * 16 * 4);
+  char* buf = nullptr;
+  KGE_HIP_CHECK(hipMalloc(&buf, bytes));
+  struct Free {
+    char* p;
+    ~Free() { (void)hipFree(p); }
+  } guard{buf};
+  KGE_HIP_CHECK(hipMemsetAsync(buf, 0, bytes, st));
+  KGE_HIP_CHECK(hipMemsetAsync(buf + o_tau, 0x7f, (size_t)B * 4, st));  // 0x7f7f7f7f = 3.39e38: no bound reaches it ...
+  {
+    std::vector<float> inf((size_t)B, __builtin_inff());                    // ... and then +inf itself
+    KGE_HIP_CHECK(hipMemcpyAsync(buf + o_tau, inf.data(), (size_t)B * 4, hipMemcpyHostToDevice, st));
+    KGE_HIP_CHECK(hipStreamSynchronize(st));
+  }
+  hipLaunchKernelGGL(topk_i8_qprep_kernel, dim3((unsigned)((B + 3) / 4)), dim3(256), 0, st, Q, B, (int8_t*)(buf + o_qh),
+                     (f32x4*)(buf + o_qc));
+  KGE_LAUNCH_CHECK("topk_i8_qprep_kernel");
+  ContractArgs a;
+  memset(&a, 0, sizeof(a));
+  a.Q = Q;
+  a.B = B;
+  a.N = N;
+  a.e_begin = 0;
+  a.e_end = N;
+  a.d = 128;
+  a.n_qgroups = (int)((B + TF_WG_QUERIES - 1) / TF_WG_QUERIES);
+  a.n_lanes = 32 / a.n_qgroups;
+  if (a.n_lanes < 1) a.n_lanes = 1;
+  int64_t chunk = N / (8 * (int64_t)a.n_lanes * 4);
+  chunk = (chunk + TF_STAGE_ROWS - 1) / TF_STAGE_ROWS * TF_STAGE_ROWS;
+  if (chunk < TF_STAGE_ROWS) chunk = TF_STAGE_ROWS;
+  if (chunk > 1024) chunk = 1024;
+  a.chunk_rows = (int)chunk;
+  a.n_chunks = (N + chunk - 1) / chunk;
+  const int64_t nwg = 8 * (int64_t)a.n_qgroups * a.n_lanes;
+  KGE_REQUIRE(nwg <= 0x7fffffffLL, KGE_ERR_INVALID, "kge_probe_i8_scan: grid too large");
+  I8FilterArgs ea{(const float*)(buf + o_tau), nullptr, (int32_t*)(buf + o_cnt), (uint32_t*)(buf + o_cand), 16,
+                  (const int8_t*)((const unsigned char*)prepared + t.requant), (const unsigned char*)prepared + t.rowmeta,
+                  (const int8_t*)(buf + o_qh), (const f32x4*)(buf + o_qc)};
+  auto launch = [&]() { hipLaunchKernelGGL(topk_i8_filter_kernel, dim3((unsigned)nwg), dim3(64 * TF_W), 0, st, a, ea); };
+  double ms = 0.0;
+  int64_t n = 0;
+  const int rc = probe_run(launch, seconds, st, &ms, &n);
+  if (rc) return rc;
+  *pops = 2.0 * 128.0 * (double)B * (double)N / (ms * 1e-3) / 1e12;  // tera-operations per second
+  if (ms_per_launch) *ms_per_launch = ms;
+  return KGE_OK;
+}
+

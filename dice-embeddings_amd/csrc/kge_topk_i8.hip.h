@@ -35,6 +35,7 @@
 #include "kge_contract.hip.h"
 
 namespace kge {
+// (the kernels below have internal linkage: the library's main source and its measurement aids both include this file)
 
 typedef __attribute__((ext_vector_type(4))) int i32x4;
 typedef __attribute__((ext_vector_type(16))) int i32x16;
@@ -67,7 +68,7 @@ static_assert(host::TOPK_ROWMETA_ROWS == TF_STAGE_ROWS && host::TOPK_ROWMETA_BYT
 // thread t takes 16 bytes of row (t >> 3) of each of the two tiles, so loads and stores are whole rows in order.
 // A row past the table's end counts for nothing; a scale that is not finite forces its tile (the scan then takes
 // all its rows as candidates).
-__global__ void __launch_bounds__(256) topk_i8_requant_kernel(const int8_t* E, const float* scale, int64_t N, int8_t* Eq,
+static __global__ void __launch_bounds__(256) topk_i8_requant_kernel(const int8_t* E, const float* scale, int64_t N, int8_t* Eq,
                                                               unsigned char* meta) {
   __shared__ float s_max[2][4], s_bad[2][4], s_e2[2][4], s_r2[2][4];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -159,7 +160,7 @@ __global__ void __launch_bounds__(256) topk_i8_requant_kernel(const int8_t* E, c
 // infinite anyway).  kind 2: components so large (about 1e34) that the bound's own arithmetic could overflow; the
 // scan takes every row as a candidate for it.  kind 1: everything else.
 constexpr float TF_NORM_MAX = 1e35f;  // m_q |e'|_2 + |rho|_2 |qb|_2 + s_q |H'| stays finite below this
-__global__ void __launch_bounds__(256) topk_i8_qprep_kernel(const float* Q, int64_t B, int8_t* qh, f32x4* qc) {
+static __global__ void __launch_bounds__(256) topk_i8_qprep_kernel(const float* Q, int64_t B, int8_t* qh, f32x4* qc) {
   const int lane = threadIdx.x & 63;
   const int64_t q = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
   if (q >= B) return;
@@ -297,7 +298,7 @@ __device__ __attribute__((noinline)) void tf_drain(const uint32_t* queue, int n,
   tf_collect(hh, thr, on, (int)(where & 0xffffu), (int)(where >> 16), e_base, k);
 }
 
-__global__ void __launch_bounds__(64 * TF_W, 2) topk_i8_filter_kernel(ContractArgs a, I8FilterArgs ea) {
+static __global__ void __launch_bounds__(64 * TF_W, 2) topk_i8_filter_kernel(ContractArgs a, I8FilterArgs ea) {
   constexpr int NQT = TF_NQT, W = TF_W, WQ = TF_WG_QUERIES;
   __shared__ __attribute__((aligned(1024))) unsigned char lds_e[TF_NBUF * TF_STAGE_BYTES];
   __shared__ __attribute__((aligned(16))) unsigned char meta_lds[TF_NBUF][host::TOPK_ROWMETA_BYTES];

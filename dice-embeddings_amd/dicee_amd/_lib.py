@@ -64,6 +64,8 @@ SIGNATURES = {
                                 ctypes.POINTER(ctypes.c_double), _vp]),
     "kge_probe_walk": (_c_int, [_vp, _vp, _c_i64, _c_i64, ctypes.c_double, ctypes.POINTER(ctypes.c_double),
                                 ctypes.POINTER(ctypes.c_double), _vp]),
+    "kge_probe_i8_scan": (_c_int, [_vp, _vp, _c_i64, _c_i64, ctypes.c_double, ctypes.POINTER(ctypes.c_double),
+                                   ctypes.POINTER(ctypes.c_double), _vp]),
     "kge_row_minmax": (_c_int, [_vp, _vp, _vp, _c_int, _vp, _c_i64, _c_i64, _c_i64, _vp, _vp, _vp]),
     "kge_bce_workspace_bytes": (_sz, []),
     "kge_bce_multihot": (_c_int, [_vp, _vp, _vp, _c_int, _vp, _c_i64, _c_i64, _c_i64, _vp, _vp, _vp, _c_i64, _c_f,

@@ -410,6 +410,16 @@ def probe_mfma(count, reads, seconds=1.0):
     return tf.value, ms.value
 
 
+def probe_i8_scan(Q, prepared, N, seconds=1.0):
+    """Measurement aid (``kge_probe_i8_scan``): the int8 top-k scan over a prepared table with thresholds of +inf,
+    i.e. its hot loop alone.  Returns (tera-operations per second, milliseconds per launch)."""
+    assert Q.is_cuda and prepared.is_cuda and Q.dtype == torch.float32 and Q.is_contiguous() and Q.shape[1] == 128
+    tf, ms = ctypes.c_double(0.0), ctypes.c_double(0.0)
+    _lib.check(_lib.load().kge_probe_i8_scan(Q.data_ptr(), prepared.data_ptr(), Q.shape[0], int(N), float(seconds),
+                                             ctypes.byref(tf), ctypes.byref(ms), _stream()))
+    return tf.value, ms.value
+
+
 def probe_walk(Q, E, seconds=1.0):
     """Measurement aid (``kge_probe_walk``): the bf16 d = 128 rank main loop over ``E`` without its count.
     Returns (TFLOP/s, milliseconds per launch)."""

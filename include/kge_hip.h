@@ -380,11 +380,19 @@ const char* kge_profile_kernel(void);
  *                    the main loop does; no global memory traffic, no barriers.
  *   kge_probe_walk   the main loop itself over the caller's bf16 table E [N,128] and queries Q [B,128] (fp32):
  *                    global -> LDS stages, barriers, fragment reads and MFMAs, without the count.
- * Both allocate (and free) a few bytes of device memory and synchronise the stream.
+ *   kge_probe_i8_scan  the top-k scan of per-row int8 tables with d == 128 (the integer filter) over a table's prepared
+ *                    form (kge_topk_prepare; 256-byte aligned, as Q [B,128]) with every threshold at +inf: no tile
+ *                    passes the bound, so the launch is the scan's hot loop alone (int8 MFMAs, the test of every tile,
+ *                    the walk) without the parking and collecting of candidates; rate in tera-operations per second
+ *                    (2 * 128 per entity score).
+ * All three allocate (and free) a little device memory (kge_probe_i8_scan: 212 bytes per query) and synchronise the
+ * stream.
  */
 int kge_probe_mfma(int count, int reads, double seconds, double* tflops, double* ms_per_launch, void* stream);
 int kge_probe_walk(const float* Q, const void* E, int64_t B, int64_t N, double seconds, double* tflops,
                    double* ms_per_launch, void* stream);
+int kge_probe_i8_scan(const float* Q, const void* prepared, int64_t B, int64_t N, double seconds, double* tops,
+                      double* ms_per_launch, void* stream);
 
 #ifdef __cplusplus
 }

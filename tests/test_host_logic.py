@@ -87,6 +87,8 @@ def test_host_side_argument_validation_without_gpu(lib_path):
                                p256, 1 << 20, None)
     assert rc == 1 and b"16-byte aligned" in lib.kge_last_error()
     # the measurement aids validate as well
+    rc = lib.kge_probe_i8_scan(None, None, 8, 64, ctypes.c_double(1.0), None, None, None)
+    assert rc == 1 and b"kge_probe_i8_scan" in lib.kge_last_error()
     rc = lib.kge_probe_mfma(0, 0, ctypes.c_double(100.0), None, None, None)
     assert rc == 1 and b"kge_probe_mfma" in lib.kge_last_error()
     assert lib.kge_profile_kernel() == b""
