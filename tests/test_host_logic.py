@@ -86,6 +86,16 @@ def test_host_side_argument_validation_without_gpu(lib_path):
     rc = lib.kge_rank_filtered(off, None, p256, 0, None, 3, 50, 100, p256, None, None, None, 0, p256, p256, p256, p256,
                                p256, 1 << 20, None)
     assert rc == 1 and b"16-byte aligned" in lib.kge_last_error()
+    # the thresholds of many batches, and the rank call that takes a slice of them: null arrays, a short workspace
+    rc = lib.kge_rank_thresholds(p256, None, p256, 0, None, 4, 16, 100, p256, None, p256, p256, p256, p256, None)
+    assert rc == 1 and b"threshold" in lib.kge_last_error()
+    rc = lib.kge_rank_filtered_with_thresholds(p256, p256, 0, None, 4, 16, 100, p256, None, None, None, None, 0, 1, p256,
+                                               p256, p256, p256, 1 << 20, None)
+    assert rc == 1 and b"threshold" in lib.kge_last_error()
+    rc = lib.kge_rank_filtered_with_thresholds(p256, p256, 0, None, 4, 16, 100, p256, p256, None, None, None, 0, 1, p256,
+                                               p256, p256, p256, 8, None)
+    assert rc != 0 and b"workspace" in lib.kge_last_error()
+    assert lib.kge_rank_thresholds(p256, None, p256, 0, None, 0, 16, 100, None, None, None, None, None, None, None) == 0
     # the measurement aids validate as well
     rc = lib.kge_probe_i8_scan(None, None, 8, 64, ctypes.c_double(1.0), None, None, None)
     assert rc == 1 and b"kge_probe_i8_scan" in lib.kge_last_error()
