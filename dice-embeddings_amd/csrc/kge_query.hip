@@ -295,7 +295,11 @@ __global__ void __launch_bounds__(64) build_query_kernel(QueryArgs a, int model)
 // ---- backward of the query builder ---------------------------------------------------------------
 // Given dL/dQ[b, :] and dL/dbias[b], add dL/d(head row) to d_ent[h], dL/d(relation row) to d_rel[r] and, for
 // the Clifford models, dL/d(coefficients) to d_coeff_*.  One wavefront per pair; rows that several pairs share
-// are combined with floating-point atomics.  fp32 tables, no normalisation layer.
+// are combined with floating-point atomics.  fp32 tables.
+// NORM: the rows pass through LayerNorm / BatchNorm1d (running statistics) before the interaction, as in the forward:
+// the interaction's gradients at the normalised rows are collected in LDS (every element is produced exactly once per
+// pair) and sent through the normaliser's own backward before they are added to the tables; LayerNorm's weight and
+// bias receive their gradients too.
 struct QueryBwdArgs {
   const float* ent;
   const float* rel;
@@ -312,14 +316,58 @@ struct QueryBwdArgs {
   float* d_coeff_r;
   int64_t B, N, R;
   int d, p, q, r, normalize_relation;
+  kge_norm_params norm;
+  float* dn_h_a;  // LayerNorm: gradient of the head normaliser's weight / bias, of the relation normaliser's (may be null)
+  float* dn_h_b;
+  float* dn_r_a;
+  float* dn_r_b;
 };
 
+// One row through the backward of its normaliser: x the raw row, dy the gradient at the normalised row (both in LDS);
+// adds the gradient at the raw row to out[] and LayerNorm's parameter gradients to dw[] / db[].
+__device__ void normalise_row_backward(const float* x, const float* dy, int d, int lane, int kind, float eps,
+                                       const float* a, const float* b, float* out, float* dw, float* db) {
+  if (kind == KGE_NORM_LAYERNORM) {
+    // the statistics exactly as normalise_row forms them
+    float s = 0.f;
+    for (int k = lane; k < d; k += 64) s += x[k];
+    const float mu = wave_sum(s) / (float)d;
+    float v = 0.f;
+    for (int k = lane; k < d; k += 64) {
+      const float t = x[k] - mu;
+      v += t * t;
+    }
+    const float var = wave_sum(v) / (float)d;
+    const float inv = 1.0f / sqrtf(var + eps);
+    // y = xh * w + b with xh = (x - mu) * inv:  dx = inv * (g - mean(g) - xh * mean(g * xh)),  g = dy * w
+    float s1 = 0.f, s2 = 0.f;
+    for (int k = lane; k < d; k += 64) {
+      const float g = dy[k] * a[k];
+      s1 += g;
+      s2 += g * ((x[k] - mu) * inv);
+    }
+    const float m1 = wave_sum(s1) / (float)d, m2 = wave_sum(s2) / (float)d;
+    for (int k = lane; k < d; k += 64) {
+      const float xh = (x[k] - mu) * inv, g = dy[k] * a[k];
+      atomicAdd(&out[k], inv * (g - m1 - xh * m2));
+      if (dw) atomicAdd(&dw[k], dy[k] * xh);
+      if (db) atomicAdd(&db[k], dy[k]);
+    }
+  } else {  // BatchNorm1d with running statistics: an elementwise affine map
+    for (int k = lane; k < d; k += 64) atomicAdd(&out[k], dy[k] / sqrtf(b[k] + eps));
+  }
+}
+
+template <bool NORM>
 __global__ void __launch_bounds__(64) build_query_backward_kernel(QueryBwdArgs a, int model) {
   extern __shared__ float lds[];
   const int d = a.d;
   float* sh = lds;          // head row
   float* sr = lds + d;      // relation row
   float* sg = lds + 2 * d;  // dL/dQ row
+  float* sdh = lds + 3 * d;  // NORM: gradient at the normalised head row, at the normalised relation row, and the
+  float* sdr = lds + 4 * d;  // norms of the relation's quaternions before QMult's own normaliser
+  float* sn = lds + 5 * d;
   const int lane = threadIdx.x;
   const int64_t b = blockIdx.x;
   const int64_t h_id = a.hr[2 * b], r_id = a.hr[2 * b + 1];
@@ -330,21 +378,34 @@ __global__ void __launch_bounds__(64) build_query_backward_kernel(QueryBwdArgs a
     sg[k] = a.dQ[b * d + k];
   }
   __syncthreads();
+  if constexpr (NORM) {
+    normalise_row(sh, d, lane, a.norm.kind, a.norm.eps, a.norm.h_a, a.norm.h_b);
+    normalise_row(sr, d, lane, a.norm.kind, a.norm.eps, a.norm.r_a, a.norm.r_b);
+    __syncthreads();
+  }
   float* gh = a.d_ent + h_id * d;
   float* gr = a.d_rel + r_id * d;
+  auto emit_h = [&](int k, float v) {
+    if constexpr (NORM) sdh[k] = v;
+    else atomicAdd(&gh[k], v);
+  };
+  auto emit_r = [&](int k, float v) {
+    if constexpr (NORM) sdr[k] = v;
+    else atomicAdd(&gr[k], v);
+  };
   if (model == KGE_DISTMULT) {
     for (int k = lane; k < d; k += 64) {
-      atomicAdd(&gh[k], sg[k] * sr[k]);
-      atomicAdd(&gr[k], sg[k] * sh[k]);
+      emit_h(k, sg[k] * sr[k]);
+      emit_r(k, sg[k] * sh[k]);
     }
   } else if (model == KGE_COMPLEX) {
     const int d2 = d >> 1;
     for (int k = lane; k < d2; k += 64) {
       const float hr_ = sh[k], hi_ = sh[k + d2], rr_ = sr[k], ri_ = sr[k + d2], g0 = sg[k], g1 = sg[k + d2];
-      atomicAdd(&gh[k], g0 * rr_ + g1 * ri_);
-      atomicAdd(&gh[k + d2], -g0 * ri_ + g1 * rr_);
-      atomicAdd(&gr[k], g0 * hr_ + g1 * hi_);
-      atomicAdd(&gr[k + d2], -g0 * hi_ + g1 * hr_);
+      emit_h(k, g0 * rr_ + g1 * ri_);
+      emit_h(k + d2, -g0 * ri_ + g1 * rr_);
+      emit_r(k, g0 * hr_ + g1 * hi_);
+      emit_r(k + d2, -g0 * hi_ + g1 * hr_);
     }
   } else if (model == KGE_QMULT) {
     const int d4 = d >> 2;
@@ -352,7 +413,9 @@ __global__ void __launch_bounds__(64) build_query_backward_kernel(QueryBwdArgs a
     if (a.normalize_relation) {
       for (int g = lane; g < d4; g += 64) {
         const float x0 = sr[4 * g], x1 = sr[4 * g + 1], x2 = sr[4 * g + 2], x3 = sr[4 * g + 3];
-        const float den = fmaxf(sqrtf(x0 * x0 + x1 * x1 + x2 * x2 + x3 * x3), 1e-12f);
+        const float nrm = sqrtf(x0 * x0 + x1 * x1 + x2 * x2 + x3 * x3);
+        if constexpr (NORM) sn[g] = nrm;
+        const float den = fmaxf(nrm, 1e-12f);
         sr[4 * g] = x0 / den;
         sr[4 * g + 1] = x1 / den;
         sr[4 * g + 2] = x2 / den;
@@ -365,10 +428,10 @@ __global__ void __launch_bounds__(64) build_query_backward_kernel(QueryBwdArgs a
       const float ah = sh[g], bh = sh[g + d4], ch = sh[g + 2 * d4], dh = sh[g + 3 * d4];
       const float pr = sr[g], qr = sr[g + d4], ur = sr[g + 2 * d4], vr = sr[g + 3 * d4];
       const float G0 = sg[g], G1 = sg[g + d4], G2 = sg[g + 2 * d4], G3 = sg[g + 3 * d4];
-      atomicAdd(&gh[g], G0 * pr + G1 * qr + G2 * ur + G3 * vr);
-      atomicAdd(&gh[g + d4], -G0 * qr + G1 * pr - G2 * vr + G3 * ur);
-      atomicAdd(&gh[g + 2 * d4], -G0 * ur + G1 * vr + G2 * pr - G3 * qr);
-      atomicAdd(&gh[g + 3 * d4], -G0 * vr - G1 * ur + G2 * qr + G3 * pr);
+      emit_h(g, G0 * pr + G1 * qr + G2 * ur + G3 * vr);
+      emit_h(g + d4, -G0 * qr + G1 * pr - G2 * vr + G3 * ur);
+      emit_h(g + 2 * d4, -G0 * ur + G1 * vr + G2 * pr - G3 * qr);
+      emit_h(g + 3 * d4, -G0 * vr - G1 * ur + G2 * qr + G3 * pr);
       sh[g] = G0 * ah + G1 * bh + G2 * ch + G3 * dh;
       sh[g + d4] = -G0 * bh + G1 * ah + G2 * dh - G3 * ch;
       sh[g + 2 * d4] = -G0 * ch - G1 * dh + G2 * ah + G3 * bh;
@@ -376,27 +439,32 @@ __global__ void __launch_bounds__(64) build_query_backward_kernel(QueryBwdArgs a
     }
     __syncthreads();
     if (!a.normalize_relation) {
-      for (int k = lane; k < d; k += 64) atomicAdd(&gr[k], sh[k]);
+      for (int k = lane; k < d; k += 64) emit_r(k, sh[k]);
     } else {
       // y = x / max(|x|, eps) per group of 4 consecutive elements: dx = (dy - y (y . dy)) / |x|, or dy / eps
       // where the norm was clamped
       for (int g = lane; g < d4; g += 64) {
-        const float* raw = a.rel + r_id * d + 4 * g;
-        const float x0 = raw[0], x1 = raw[1], x2 = raw[2], x3 = raw[3];
-        const float n = sqrtf(x0 * x0 + x1 * x1 + x2 * x2 + x3 * x3);
+        float n;
+        if constexpr (NORM) {
+          n = sn[g];
+        } else {
+          const float* raw = a.rel + r_id * d + 4 * g;
+          const float x0 = raw[0], x1 = raw[1], x2 = raw[2], x3 = raw[3];
+          n = sqrtf(x0 * x0 + x1 * x1 + x2 * x2 + x3 * x3);
+        }
         const float y0 = sr[4 * g], y1 = sr[4 * g + 1], y2 = sr[4 * g + 2], y3 = sr[4 * g + 3];
         const float e0 = sh[4 * g], e1 = sh[4 * g + 1], e2 = sh[4 * g + 2], e3 = sh[4 * g + 3];
         if (n < 1e-12f) {
-          atomicAdd(&gr[4 * g], e0 / 1e-12f);
-          atomicAdd(&gr[4 * g + 1], e1 / 1e-12f);
-          atomicAdd(&gr[4 * g + 2], e2 / 1e-12f);
-          atomicAdd(&gr[4 * g + 3], e3 / 1e-12f);
+          emit_r(4 * g, e0 / 1e-12f);
+          emit_r(4 * g + 1, e1 / 1e-12f);
+          emit_r(4 * g + 2, e2 / 1e-12f);
+          emit_r(4 * g + 3, e3 / 1e-12f);
         } else {
           const float dot = y0 * e0 + y1 * e1 + y2 * e2 + y3 * e3;
-          atomicAdd(&gr[4 * g], (e0 - y0 * dot) / n);
-          atomicAdd(&gr[4 * g + 1], (e1 - y1 * dot) / n);
-          atomicAdd(&gr[4 * g + 2], (e2 - y2 * dot) / n);
-          atomicAdd(&gr[4 * g + 3], (e3 - y3 * dot) / n);
+          emit_r(4 * g, (e0 - y0 * dot) / n);
+          emit_r(4 * g + 1, (e1 - y1 * dot) / n);
+          emit_r(4 * g + 2, (e2 - y2 * dot) / n);
+          emit_r(4 * g + 3, (e3 - y3 * dot) / n);
         }
       }
     }
@@ -443,8 +511,8 @@ __global__ void __launch_bounds__(64) build_query_backward_kernel(QueryBwdArgs a
       }
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
-        atomicAdd(&gh[g + i * d8], dx[i]);
-        atomicAdd(&gr[g + i * d8], dy[i]);
+        emit_h(g + i * d8, dx[i]);
+        emit_r(g + i * d8, dy[i]);
       }
     }
   } else {  // KGE_KECI (r = 0) / KGE_DECAL
@@ -477,8 +545,8 @@ __global__ void __launch_bounds__(64) build_query_backward_kernel(QueryBwdArgs a
           dr0 += Gi * hs;
         }
         if (i0 == 0) {
-          atomicAdd(&gh[rho], dh0);
-          atomicAdd(&gr[rho], dr0);
+          emit_h(rho, dh0);
+          emit_r(rho, dr0);
         }
         const bool fam_on[3] = {pp, qq, kk};
         float before_h[3] = {0.f, 0.f, 0.f}, before_r[3] = {0.f, 0.f, 0.f};
@@ -507,8 +575,8 @@ __global__ void __launch_bounds__(64) build_query_backward_kernel(QueryBwdArgs a
           before_h[f] += hs;
           before_r[f] += rs;
           if (i0 == 0) {
-            atomicAdd(&gh[col(rho, i)], c * dhs);
-            atomicAdd(&gr[col(rho, i)], c * drs);
+            emit_h(col(rho, i), c * dhs);
+            emit_r(col(rho, i), c * drs);
           }
           if (i >= i0 && i < i0 + 16) dc[i - i0] += hraw * dhs + rraw * drs;
         }
@@ -523,6 +591,17 @@ __global__ void __launch_bounds__(64) build_query_backward_kernel(QueryBwdArgs a
         if (lane == 0 && dst) atomicAdd(&dst[idx], v);
       }
     }
+  }
+  if constexpr (NORM) {
+    // the raw rows once more, and each gradient through its normaliser
+    __syncthreads();
+    for (int k = lane; k < d; k += 64) {
+      sh[k] = a.ent[h_id * d + k];
+      sr[k] = a.rel[r_id * d + k];
+    }
+    __syncthreads();
+    normalise_row_backward(sh, sdh, d, lane, a.norm.kind, a.norm.eps, a.norm.h_a, a.norm.h_b, gh, a.dn_h_a, a.dn_h_b);
+    normalise_row_backward(sr, sdr, d, lane, a.norm.kind, a.norm.eps, a.norm.r_a, a.norm.r_b, gr, a.dn_r_a, a.dn_r_b);
   }
 }
 
@@ -815,12 +894,13 @@ extern "C" int kge_build_query_decal(int head, int p, int q, int r, const void* 
                           coeff_r, 0, norm, pairs, B, d, N, R, Q, bias, stream);
 }
 
-extern "C" int kge_build_query_backward(int model, int p, int q, int r, const float* ent, const float* rel,
-                                        const float* coeff_p, const float* coeff_q, const float* coeff_r,
-                                        int normalize_relation, const int64_t* hr, int64_t B, int64_t d, int64_t N,
-                                        int64_t R, const float* dQ, const float* dbias, float* d_ent, float* d_rel,
-                                        float* d_coeff_p, float* d_coeff_q, float* d_coeff_r, void* stream) {
-  using namespace kge;
+namespace kge {
+namespace {
+int build_query_backward_impl(int model, int p, int q, int r, const float* ent, const float* rel, const float* coeff_p,
+                              const float* coeff_q, const float* coeff_r, int normalize_relation,
+                              const kge_norm_params* norm, const kge_norm_grads* dnorm, const int64_t* hr, int64_t B,
+                              int64_t d, int64_t N, int64_t R, const float* dQ, const float* dbias, float* d_ent,
+                              float* d_rel, float* d_coeff_p, float* d_coeff_q, float* d_coeff_r, void* stream) {
   clear_error();
   KGE_REQUIRE(B >= 0 && N > 0 && R > 0, KGE_ERR_INVALID, "kge_build_query_backward: B=%lld N=%lld R=%lld", (long long)B,
               (long long)N, (long long)R);
@@ -872,8 +952,59 @@ extern "C" int kge_build_query_backward(int model, int p, int q, int r, const fl
   a.q = q;
   a.r = r;
   a.normalize_relation = normalize_relation;
+  a.norm.kind = KGE_NORM_NONE;
+  a.norm.eps = 0.f;
+  a.norm.h_a = a.norm.h_b = a.norm.r_a = a.norm.r_b = nullptr;
+  a.dn_h_a = a.dn_h_b = a.dn_r_a = a.dn_r_b = nullptr;
   hipStream_t st = (hipStream_t)stream;
-  hipLaunchKernelGGL(build_query_backward_kernel, dim3((unsigned)B), dim3(64), 3 * (size_t)d * sizeof(float), st, a, model);
+  if (norm && norm->kind != KGE_NORM_NONE) {
+    KGE_REQUIRE(norm->kind == KGE_NORM_LAYERNORM || norm->kind == KGE_NORM_BATCHNORM1D, KGE_ERR_INVALID,
+                "kge_build_query_backward_norm: unknown normalisation %d", norm->kind);
+    KGE_REQUIRE(norm->h_a && norm->h_b && norm->r_a && norm->r_b, KGE_ERR_INVALID,
+                "kge_build_query_backward_norm: normalisation parameters missing");
+    KGE_REQUIRE(d <= 4096, KGE_ERR_UNSUPPORTED,
+                "kge_build_query_backward_norm: d=%lld exceeds 4096 (five rows and a quarter per pair are kept in LDS)",
+                (long long)d);
+    a.norm = *norm;
+    if (dnorm) {
+      KGE_REQUIRE(norm->kind == KGE_NORM_LAYERNORM || !(dnorm->h_a || dnorm->h_b || dnorm->r_a || dnorm->r_b),
+                  KGE_ERR_INVALID,
+                  "kge_build_query_backward_norm: BatchNorm1d(affine=False) has no parameters to take a gradient");
+      a.dn_h_a = dnorm->h_a;
+      a.dn_h_b = dnorm->h_b;
+      a.dn_r_a = dnorm->r_a;
+      a.dn_r_b = dnorm->r_b;
+    }
+    const size_t lds_bytes = (5 * (size_t)d + (size_t)(d + 3) / 4) * sizeof(float);
+    hipLaunchKernelGGL(build_query_backward_kernel<true>, dim3((unsigned)B), dim3(64), lds_bytes, st, a, model);
+  } else {
+    hipLaunchKernelGGL(build_query_backward_kernel<false>, dim3((unsigned)B), dim3(64), 3 * (size_t)d * sizeof(float), st,
+                       a, model);
+  }
   KGE_LAUNCH_CHECK("build_query_backward_kernel");
   return KGE_OK;
+}
+}  // namespace
+}  // namespace kge
+
+extern "C" int kge_build_query_backward(int model, int p, int q, int r, const float* ent, const float* rel,
+                                        const float* coeff_p, const float* coeff_q, const float* coeff_r,
+                                        int normalize_relation, const int64_t* hr, int64_t B, int64_t d, int64_t N,
+                                        int64_t R, const float* dQ, const float* dbias, float* d_ent, float* d_rel,
+                                        float* d_coeff_p, float* d_coeff_q, float* d_coeff_r, void* stream) {
+  return kge::build_query_backward_impl(model, p, q, r, ent, rel, coeff_p, coeff_q, coeff_r, normalize_relation, nullptr,
+                                        nullptr, hr, B, d, N, R, dQ, dbias, d_ent, d_rel, d_coeff_p, d_coeff_q,
+                                        d_coeff_r, stream);
+}
+
+extern "C" int kge_build_query_backward_norm(int model, int p, int q, int r, const float* ent, const float* rel,
+                                             const float* coeff_p, const float* coeff_q, const float* coeff_r,
+                                             int normalize_relation, const kge_norm_params* norm,
+                                             const kge_norm_grads* dnorm, const int64_t* hr, int64_t B, int64_t d,
+                                             int64_t N, int64_t R, const float* dQ, const float* dbias, float* d_ent,
+                                             float* d_rel, float* d_coeff_p, float* d_coeff_q, float* d_coeff_r,
+                                             void* stream) {
+  return kge::build_query_backward_impl(model, p, q, r, ent, rel, coeff_p, coeff_q, coeff_r, normalize_relation, norm,
+                                        dnorm, hr, B, d, N, R, dQ, dbias, d_ent, d_rel, d_coeff_p, d_coeff_q, d_coeff_r,
+                                        stream);
 }

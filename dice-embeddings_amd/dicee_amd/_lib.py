@@ -22,6 +22,10 @@ class NormParams(ctypes.Structure):
                 ("h_a", _vp), ("h_b", _vp), ("r_a", _vp), ("r_b", _vp)]
 
 
+class NormGrads(ctypes.Structure):
+    _fields_ = [("h_a", _vp), ("h_b", _vp), ("r_a", _vp), ("r_b", _vp)]
+
+
 SIGNATURES = {
     "kge_last_error": (ctypes.c_char_p, []),
     "kge_abi_version": (_c_int, []),
@@ -33,6 +37,9 @@ SIGNATURES = {
                                        ctypes.POINTER(NormParams), _vp, _c_i64, _c_i64, _c_i64, _c_i64, _vp, _vp, _vp]),
     "kge_build_query_backward": (_c_int, [_c_int, _c_int, _c_int, _c_int, _vp, _vp, _vp, _vp, _vp, _c_int, _vp, _c_i64,
                                           _c_i64, _c_i64, _c_i64, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
+    "kge_build_query_backward_norm": (_c_int, [_c_int, _c_int, _c_int, _c_int, _vp, _vp, _vp, _vp, _vp, _c_int,
+                                               ctypes.POINTER(NormParams), ctypes.POINTER(NormGrads), _vp, _c_i64,
+                                               _c_i64, _c_i64, _c_i64, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     "kge_scores": (_c_int, [_vp, _vp, _vp, _c_int, _vp, _c_i64, _c_i64, _c_i64, _vp, _c_i64, _vp]),
     "kge_triple_scores": (_c_int, [_vp, _vp, _vp, _c_int, _vp, _c_i64, _c_i64, _c_i64, _vp, _vp, _vp]),
     "kge_sample_scores": (_c_int, [_vp, _vp, _vp, _c_int, _vp, _c_i64, _c_i64, _c_i64, _vp, _c_i64, _vp, _vp]),

@@ -280,9 +280,14 @@ class BaseKGE(torch.nn.Module):
         ``(loss, {parameter name: gradient})`` with ``entity_embeddings.weight`` [N,d] (the contraction's gradient
         plus the rows of the heads), ``relation_embeddings.weight`` [R,d] and, for Keci / DeCaL, the coefficient
         embeddings.  What ``loss_batch.backward()`` leaves in ``.grad`` after ``training_step`` (base_model.py:25-46)
-        for fp32 tables without a normalisation layer."""
-        if self._norm_params() is not None:
-            raise NotImplementedError("the backward does not pass through LayerNorm / BatchNorm1d")
+        for fp32 tables.  With ``normalization='LayerNorm'`` the gradient passes through both normalisers and their
+        weights and biases receive theirs (``normalize_head_entity_embeddings.weight`` ...); with ``'BatchNorm1d'``
+        it passes through the running statistics, which is what the module does in eval mode: in training mode the
+        reference normalises with the statistics of the batch, which this path does not form."""
+        norm = self._norm_params()
+        if norm is not None and norm["kind"] == "BatchNorm1d" and self.training:
+            raise NotImplementedError("BatchNorm1d in training mode (batch statistics) is not part of this path; "
+                                      "call model.eval() for the gradient through the running statistics")
         E, scale = self.table()
         if scale is not None or E.dtype != torch.float32:
             raise TypeError("the backward needs an fp32 entity table")
@@ -291,8 +296,17 @@ class BaseKGE(torch.nn.Module):
         rel = self._rel()
         dR = torch.zeros_like(rel)
         name = self.name if self.name != "CKeci" else "Keci"
-        dcoeff = ops.build_query_backward(name, E, rel, x, dQ, dbias, dE, dR, **self._query_kwargs())
+        dnorm = None
+        if norm is not None and norm["kind"] == "LayerNorm":
+            dnorm = {k: torch.zeros_like(norm[k], dtype=torch.float32) for k in ("h_a", "h_b", "r_a", "r_b")}
+        dcoeff = ops.build_query_backward(name, E, rel, x, dQ, dbias, dE, dR, norm=norm, dnorm=dnorm,
+                                          **self._query_kwargs())
         grads = {"entity_embeddings.weight": dE, "relation_embeddings.weight": dR}
+        if dnorm is not None:
+            grads["normalize_head_entity_embeddings.weight"] = dnorm["h_a"]
+            grads["normalize_head_entity_embeddings.bias"] = dnorm["h_b"]
+            grads["normalize_relation_embeddings.weight"] = dnorm["r_a"]
+            grads["normalize_relation_embeddings.bias"] = dnorm["r_b"]
         for key, g in zip(("p_coefficients.weight", "q_coefficients.weight", "r_coefficients.weight"), dcoeff):
             if g is not None:
                 grads[key] = g.reshape(1, -1)

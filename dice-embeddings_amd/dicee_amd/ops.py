@@ -98,10 +98,12 @@ def build_query(model, ent, rel, hr, *, ent_scale=None, p=0, q=0, r=0, coeff_p=N
 
 
 def build_query_backward(model, ent, rel, hr, dQ, dbias, d_ent, d_rel, *, p=0, q=0, r=0, coeff_p=None, coeff_q=None,
-                         coeff_r=None, normalize_relation=True):
+                         coeff_r=None, normalize_relation=True, norm=None, dnorm=None):
     """Adds the gradients that ``dQ`` [B,d] / ``dbias`` [B] send back through ``build_query`` into ``d_ent`` [N,d]
     and ``d_rel`` [R,d] (fp32, caller-initialised); returns the gradients of the Clifford coefficients
-    ``(d_coeff_p, d_coeff_q, d_coeff_r)`` (None where the model has none)."""
+    ``(d_coeff_p, d_coeff_q, d_coeff_r)`` (None where the model has none).  ``norm``: the normalisation layer of
+    ``build_query``; ``dnorm``: for LayerNorm, a dict with any of ``h_a, h_b, r_a, r_b`` ([d] fp32,
+    caller-initialised) that receive the gradients of the normalisers' weights and biases."""
     lib = _lib.load()
     _require_gpu(ent, rel, hr, dQ, dbias, d_ent, d_rel, coeff_p, coeff_q, coeff_r)
     for t in (ent, rel, dQ, d_ent, d_rel):
@@ -109,6 +111,23 @@ def build_query_backward(model, ent, rel, hr, dQ, dbias, d_ent, d_rel, *, p=0, q
             raise TypeError("build_query_backward needs contiguous fp32 tensors")
     B, (N, d), R = hr.shape[0], ent.shape, rel.shape[0]
     outs = [torch.zeros_like(c) if c is not None else None for c in (coeff_p, coeff_q, coeff_r)]
+    if norm is not None:
+        ns, keep = _norm_struct(norm)
+        gs = None
+        if dnorm:
+            for t in dnorm.values():
+                if t.dtype != torch.float32 or not t.is_contiguous() or t.numel() != d:
+                    raise TypeError("dnorm entries must be contiguous fp32 tensors of d elements")
+            _require_gpu(*dnorm.values())
+            gs = _lib.NormGrads(*[dnorm[k].data_ptr() if dnorm.get(k) is not None else None
+                                  for k in ("h_a", "h_b", "r_a", "r_b")])
+        rc = lib.kge_build_query_backward_norm(
+            MODEL_IDS[model], int(p), int(q), int(r), _ptr(ent), _ptr(rel), _ptr(coeff_p), _ptr(coeff_q), _ptr(coeff_r),
+            int(bool(normalize_relation)), ctypes.byref(ns), ctypes.byref(gs) if gs is not None else None, _ptr(hr), B, d,
+            N, R, _ptr(dQ), _ptr(dbias), _ptr(d_ent), _ptr(d_rel), _ptr(outs[0]), _ptr(outs[1]), _ptr(outs[2]), _stream())
+        _lib.check(rc)
+        del keep
+        return tuple(outs)
     rc = lib.kge_build_query_backward(MODEL_IDS[model], int(p), int(q), int(r), _ptr(ent), _ptr(rel), _ptr(coeff_p),
                                       _ptr(coeff_q), _ptr(coeff_r), int(bool(normalize_relation)), _ptr(hr), B, d, N, R,
                                       _ptr(dQ), _ptr(dbias), _ptr(d_ent), _ptr(d_rel), _ptr(outs[0]), _ptr(outs[1]),

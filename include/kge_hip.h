@@ -63,6 +63,16 @@ typedef struct kge_norm_params {
   const float* r_b;
 } kge_norm_params;
 
+/* Where kge_build_query_backward_norm ADDS the gradients of LayerNorm's parameters (each [d] fp32, caller
+ * initialised, may be NULL): h_a / h_b = weight / bias of the head normaliser, r_a / r_b of the relation
+ * normaliser.  BatchNorm1d(affine=False) has no parameters: all four NULL (or the struct itself NULL). */
+typedef struct kge_norm_grads {
+  float* h_a;
+  float* h_b;
+  float* r_a;
+  float* r_b;
+} kge_norm_grads;
+
 /* Text of the last error raised on the calling thread ("" if none). */
 const char* kge_last_error(void);
 
@@ -125,7 +135,8 @@ int kge_build_query_decal(int head, int p, int q, int r, const void* ent, int en
                           int64_t d, int64_t N, int64_t R, float* Q, float* bias, void* stream);
 
 /*
- * Backward of kge_build_query (tail direction, fp32 tables, no normalisation layer): given dL/dQ [B,d] and
+ * Backward of kge_build_query (tail direction, fp32 tables, no normalisation layer; with one:
+ * kge_build_query_backward_norm below): given dL/dQ [B,d] and
  * dL/dbias [B] (may be NULL), ADDS dL/d(head row) into d_ent[hr[b,0], :], dL/d(relation row) into
  * d_rel[hr[b,1], :] and, for Keci / DeCaL, dL/d(coefficients) into d_coeff_p/q/r (each may be NULL).  The
  * caller zeroes the outputs or passes gradients to accumulate onto (d_ent may be the dE of
@@ -141,6 +152,22 @@ int kge_build_query_backward(int model, int p, int q, int r, const float* ent, c
                              int normalize_relation, const int64_t* hr, int64_t B, int64_t d, int64_t N, int64_t R,
                              const float* dQ, const float* dbias, float* d_ent, float* d_rel, float* d_coeff_p,
                              float* d_coeff_q, float* d_coeff_r, void* stream);
+
+/*
+ * The same with the normalisation layer of kge_build_query between the lookups and the interaction
+ * (dicee/models/base_model.py:283-294 applied at :381-383; norm as there, NULL or KGE_NORM_NONE: exactly
+ * kge_build_query_backward).  LayerNorm: the gradient passes through
+ * y = (x - mean(x)) / sqrt(var(x) + eps) * weight + bias per row, and dL/dweight, dL/dbias of both normalisers are
+ * ADDED into dnorm's arrays (what autograd leaves in normalize_head_entity_embeddings.weight.grad etc.).
+ * BatchNorm1d(affine=False) with its running statistics (eval mode): the elementwise map
+ * dx = dy / sqrt(running_var + eps); batch statistics (training mode) are not part of this call.  d <= 4096.
+ */
+int kge_build_query_backward_norm(int model, int p, int q, int r, const float* ent, const float* rel,
+                                  const float* coeff_p, const float* coeff_q, const float* coeff_r,
+                                  int normalize_relation, const kge_norm_params* norm, const kge_norm_grads* dnorm,
+                                  const int64_t* hr, int64_t B, int64_t d, int64_t N, int64_t R, const float* dQ,
+                                  const float* dbias, float* d_ent, float* d_rel, float* d_coeff_p, float* d_coeff_q,
+                                  float* d_coeff_r, void* stream);
 
 /*
  * Materialised scores S[b, e] = dot(Q[b], E[e]) (* scale[e]) (+ bias[b]); S has row stride ldS.

@@ -559,7 +559,10 @@ def build_query_backward(model, E, R, hr, dQ, dbias=None, step=1e-6, **kw):
     embedding lookups and the model's interaction (dicee/models/base_model.py:377-384 and the elementwise part of
     each ``forward_k_vs_all``).  Formed by central differences in float64, one coordinate of the gathered rows at
     a time: independent of any hand-derived Jacobian (exact up to rounding for the bilinear models, ~1e-9
-    relative through the normalisers).  Returns (dE [N,d], dR [R,d], {"coeff_p": ..., ...})."""
+    relative through the normalisers).  Returns (dE [N,d], dR [R,d], {"coeff_p": ..., ...}).  With a
+    ``norm=`` layer (``gather_hr``) the differences pass through it as well, row by row (LayerNorm, or BatchNorm1d
+    with its running statistics: base_model.py:283-294), and the dict also holds the gradients of LayerNorm's
+    parameters under ``"h_weight", "h_bias", "r_weight", "r_bias"``."""
     E = np.asarray(E, dtype=np.float64)
     R = np.asarray(R, dtype=np.float64)
     hr = np.asarray(hr)
@@ -598,6 +601,20 @@ def build_query_backward(model, E, R, hr, dQ, dbias=None, step=1e-6, **kw):
             km[key][i] -= step
             grad[i] = ((per_pair(rows_h, rows_r, kp) - per_pair(rows_h, rows_r, km)) / (2 * step)).sum()
         dcoeff[key] = grad
+    norm = kw.get("norm")
+    if norm is not None and norm["kind"] == "LayerNorm":
+        for key in ("h_weight", "h_bias", "r_weight", "r_bias"):
+            w = np.asarray(norm[key], dtype=np.float64)
+            grad = np.zeros(len(w))
+            for i in range(len(w)):
+                np_, nm = dict(norm), dict(norm)
+                np_[key], nm[key] = w.copy(), w.copy()
+                np_[key][i] += step
+                nm[key][i] -= step
+                kp, km = dict(kw), dict(kw)
+                kp["norm"], km["norm"] = np_, nm
+                grad[i] = ((per_pair(rows_h, rows_r, kp) - per_pair(rows_h, rows_r, km)) / (2 * step)).sum()
+            dcoeff[key] = grad
     return dE, dR, dcoeff
 
 

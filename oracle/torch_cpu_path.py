@@ -93,10 +93,16 @@ def k_vs_all_score(model, emb_h, emb_r, emb_E, p=0, q=0, coeff_p=None, coeff_q=N
     raise ValueError(model)
 
 
-def forward_k_vs_all(model, E, R, x, **kw):
-    """``BaseKGE.forward`` for ``x`` of shape [B,2] (base_model.py:328-336, :377-384)."""
+def forward_k_vs_all(model, E, R, x, norm_h=None, norm_r=None, **kw):
+    """``BaseKGE.forward`` for ``x`` of shape [B,2] (base_model.py:328-336, :377-384).  ``norm_h`` / ``norm_r``:
+    the modules ``normalize_head_entity_embeddings`` / ``normalize_relation_embeddings`` (base_model.py:283-294),
+    applied to the looked-up rows as at :381-383."""
     emb_h = torch.nn.functional.embedding(x[:, 0], E)
     emb_r = torch.nn.functional.embedding(x[:, 1], R)
+    if norm_h is not None:
+        emb_h = norm_h(emb_h)
+    if norm_r is not None:
+        emb_r = norm_r(emb_r)
     return k_vs_all_score(model, emb_h, emb_r, E, **kw)
 
 

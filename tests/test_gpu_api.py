@@ -831,6 +831,69 @@ def test_full_step_gradients_match_autograd_through_the_reference_op_sequence(na
         assert np.abs(g - w).max() <= 3e-5 * rms + 1e-9, (key, np.abs(g - w).max() / rms)
 
 
+@pytest.mark.parametrize("name,d,extra,kind", [("DistMult", 32, {}, "LayerNorm"), ("QMult", 32, {}, "LayerNorm"),
+                                               ("Keci", 30, {"p": 2, "q": 2}, "LayerNorm"),
+                                               ("ComplEx", 32, {}, "BatchNorm1d")])
+def test_full_step_gradients_through_the_normalisation_layer_match_autograd(name, d, extra, kind):
+    """The same with ``normalization='LayerNorm'`` (in training mode: the layer has no other mode; its weights and
+    biases receive gradients too) and ``'BatchNorm1d'`` in eval mode (running statistics), against autograd through
+    torch's own modules placed where base_model.py:381-383 places them."""
+    from dicee_amd import FilterCSR
+    m, triples = _toy(name, d, n=900, seed=75, normalization=kind, **extra)
+    rng = np.random.default_rng(5)
+    with torch.no_grad():
+        for mod in (m.normalize_head_entity_embeddings, m.normalize_relation_embeddings):
+            if kind == "LayerNorm":
+                mod.weight.copy_(torch.from_numpy(rng.uniform(0.5, 1.5, d).astype(np.float32)))
+                mod.bias.copy_(torch.from_numpy(rng.normal(0, 0.2, d).astype(np.float32)))
+            else:
+                mod.running_mean.copy_(torch.from_numpy(rng.normal(0, 0.05, d).astype(np.float32)))
+                mod.running_var.copy_(torch.from_numpy(rng.uniform(0.005, 0.02, d).astype(np.float32)))
+    er = ko.vocab(triples, "er")
+    kw = _oracle_kw(m)
+    if name == "QMult":
+        kw["normalize_relation"] = False          # quaternion.py:138: only without another relation normaliser
+    E = m.entity_embeddings.weight.detach().double().clone().requires_grad_()
+    Rel = m.relation_embeddings.weight.detach().double().clone().requires_grad_()
+    tkw = {k: (torch.tensor(v, dtype=torch.float64, requires_grad=True) if k.startswith("coeff") else v)
+           for k, v in kw.items()}
+    import copy
+    ref_h = copy.deepcopy(m.normalize_head_entity_embeddings).double()
+    ref_r = copy.deepcopy(m.normalize_relation_embeddings).double()
+    if kind == "BatchNorm1d":
+        ref_h.eval(), ref_r.eval()
+    x_np = triples[:256, :2]
+    positives = [er[(int(h), int(r))] for h, r in x_np]
+    ref = tcp.kvsall_bce_step(name, E, Rel, torch.from_numpy(x_np.copy()), positives, 0.1, norm_h=ref_h, norm_r=ref_r,
+                              **tkw)
+    ref.backward()
+    m = m.to("cuda")
+    m = m.train() if kind == "LayerNorm" else m.eval()
+    csr = FilterCSR.from_er_vocab(er, 46, device="cuda")
+    loss, grads = m.kvsall_bce_gradients(torch.from_numpy(x_np.copy()).cuda(), csr, label_smoothing=0.1)
+    assert loss.item() == pytest.approx(ref.item(), rel=1e-5)
+    want = {"entity_embeddings.weight": E.grad, "relation_embeddings.weight": Rel.grad}
+    if "coeff_p" in tkw:
+        want["p_coefficients.weight"] = tkw["coeff_p"].grad.reshape(1, -1)
+    if "coeff_q" in tkw:
+        want["q_coefficients.weight"] = tkw["coeff_q"].grad.reshape(1, -1)
+    if kind == "LayerNorm":
+        want["normalize_head_entity_embeddings.weight"] = ref_h.weight.grad
+        want["normalize_head_entity_embeddings.bias"] = ref_h.bias.grad
+        want["normalize_relation_embeddings.weight"] = ref_r.weight.grad
+        want["normalize_relation_embeddings.bias"] = ref_r.bias.grad
+    assert set(grads) == set(want)
+    for key, w in want.items():
+        w = w.numpy()
+        g = grads[key].cpu().numpy()
+        assert g.shape == w.shape, key
+        rms = np.sqrt((w ** 2).mean())
+        assert np.abs(g - w).max() <= 5e-5 * rms + 1e-9, (key, np.abs(g - w).max() / rms)
+    if kind == "BatchNorm1d":
+        with pytest.raises(NotImplementedError):
+            m.train().kvsall_bce_gradients(torch.from_numpy(x_np.copy()).cuda(), csr)
+
+
 def test_full_step_gradients_of_omult_and_decal_against_the_composed_oracle():
     from dicee_amd import FilterCSR
     for name, d, extra in (("OMult", 32, {}), ("DeCaL", 32, {"p": 2, "q": 2, "r": 3})):

@@ -1004,6 +1004,78 @@ def test_build_query_backward_fp32(ops, model, d, kw):
             assert got is None or kw.get(key) is not None
 
 
+_NORM_BWD_CASES = [
+    ("DistMult", 32, {}),
+    ("ComplEx", 24, {}),
+    ("QMult", 32, {}),                                # LayerNorm, then the quaternion normaliser on top of it
+    ("QMult", 72, {"normalize_relation": False}),     # what the model classes run (quaternion.py:138)
+    ("OMult", 24, {}),
+    ("Keci", 28, {"p": 1, "q": 2, "coeff_p": [0.7], "coeff_q": [1.3, -0.4]}),
+    ("DeCaL", 28, {"p": 2, "q": 2, "r": 2, "coeff_p": [0.7, 1.1], "coeff_q": [1.3, -0.4], "coeff_r": [0.6, 1.2]}),
+]
+
+
+@pytest.mark.parametrize("kind", ["LayerNorm", "BatchNorm1d"])
+@pytest.mark.parametrize("model,d,kw", _NORM_BWD_CASES)
+def test_build_query_backward_through_the_normalisation_layer(ops, model, d, kw, kind):
+    """d_ent / d_rel / d_coeff and LayerNorm's own parameter gradients against central differences of the oracle's
+    query builder with the same layer (fp64); BatchNorm1d with its running statistics."""
+    rng = np.random.default_rng(700 + d)
+    N, R, B = 40, 9, 53
+    E, Rel = random_tables(rng, N, R, d, std=0.8)
+    hr = random_hr(rng, N, R, B)
+    dQ = rng.standard_normal((B, d)).astype(np.float32)
+    dbias = rng.standard_normal(B).astype(np.float32)
+    if kind == "LayerNorm":
+        a_h, a_r = rng.uniform(0.5, 1.5, d).astype(np.float32), rng.uniform(-1.5, 1.5, d).astype(np.float32)
+        b_h, b_r = rng.normal(0, 0.3, d).astype(np.float32), rng.normal(0, 0.3, d).astype(np.float32)
+        onorm = {"kind": kind, "h_weight": a_h, "h_bias": b_h, "r_weight": a_r, "r_bias": b_r}
+    else:
+        a_h, a_r = rng.normal(0, 0.3, d).astype(np.float32), rng.normal(0, 0.3, d).astype(np.float32)
+        b_h, b_r = rng.uniform(0.5, 2, d).astype(np.float32), rng.uniform(0.5, 2, d).astype(np.float32)
+        onorm = {"kind": kind, "h_mean": a_h, "h_var": b_h, "r_mean": a_r, "r_var": b_r}
+    gnorm = {"kind": kind, "eps": 1e-5, "h_a": dev(torch.from_numpy(a_h)), "h_b": dev(torch.from_numpy(b_h)),
+             "r_a": dev(torch.from_numpy(a_r)), "r_b": dev(torch.from_numpy(b_r))}
+    Eg, Rg = dev(torch.from_numpy(E)), dev(torch.from_numpy(Rel))
+    d_ent, d_rel = torch.zeros_like(Eg), torch.zeros_like(Rg)
+    dnorm = {k: torch.zeros(d, device="cuda") for k in ("h_a", "h_b", "r_a", "r_b")} if kind == "LayerNorm" else None
+    dcoeff = ops.build_query_backward(model, Eg, Rg, dev(torch.from_numpy(hr)), dev(torch.from_numpy(dQ)),
+                                      dev(torch.from_numpy(dbias)), d_ent, d_rel, norm=gnorm, dnorm=dnorm,
+                                      **_gpu_kwargs(kw))
+    wE, wR, wc = ko.build_query_backward(model, E, Rel, hr, dQ, dbias, norm=onorm, **kw)
+    for got, want, name in ((d_ent, wE, "d_ent"), (d_rel, wR, "d_rel")):
+        got = got.cpu().numpy()
+        rms = np.sqrt((want ** 2).mean())
+        assert np.abs(got - want).max() <= 5e-5 * rms + 2e-6, (name, np.abs(got - want).max() / rms)
+    for got, key in zip(dcoeff, ("coeff_p", "coeff_q", "coeff_r")):
+        if key in wc:
+            assert np.abs(got.cpu().numpy() - wc[key]).max() <= 5e-5 * np.abs(wc[key]).max() + 1e-4, key
+    if kind == "LayerNorm":
+        for gk, ok_ in (("h_a", "h_weight"), ("h_b", "h_bias"), ("r_a", "r_weight"), ("r_b", "r_bias")):
+            want = wc[ok_]
+            got = dnorm[gk].cpu().numpy()
+            assert np.abs(got - want).max() <= 5e-5 * np.sqrt((want ** 2).mean()) + 1e-5, (gk, got[:4], want[:4])
+
+
+def test_build_query_backward_norm_argument_checks(ops):
+    from dicee_amd._lib import KgeError
+    rng = np.random.default_rng(5)
+    E, Rel = random_tables(rng, 20, 3, 16)
+    hr = random_hr(rng, 20, 3, 6)
+    Eg, Rg = dev(torch.from_numpy(E)), dev(torch.from_numpy(Rel))
+    dQ = torch.ones(6, 16, device="cuda")
+    ones = torch.ones(16, device="cuda")
+    bn = {"kind": "BatchNorm1d", "eps": 1e-5, "h_a": ones, "h_b": ones, "r_a": ones, "r_b": ones}
+    with pytest.raises(KgeError) as err:      # BatchNorm1d(affine=False) has no parameters
+        ops.build_query_backward("DistMult", Eg, Rg, dev(torch.from_numpy(hr)), dQ, None, torch.zeros_like(Eg),
+                                 torch.zeros_like(Rg), norm=bn, dnorm={"h_a": torch.zeros(16, device="cuda")})
+    assert err.value.code == 1
+    # norm of kind none: the plain backward, bit for bit
+    a, b = torch.zeros_like(Eg), torch.zeros_like(Rg)
+    ops.build_query_backward("DistMult", Eg, Rg, dev(torch.from_numpy(hr)), dQ, None, a, b)
+    assert float(a.abs().sum()) > 0
+
+
 # ---------------------------------------------------------------------------------------------
 # top-k over tables built to defeat its shortcuts: several rounds, guessed thresholds, overflowing buffers, repairs
 # ---------------------------------------------------------------------------------------------

@@ -545,6 +545,53 @@ def test_query_builder_backward_vs_torch_autograd():
         np.testing.assert_allclose(dR, Rt.grad.numpy(), rtol=1e-7, atol=1e-8)
 
 
+def test_query_builder_backward_through_the_normalisation_layers_vs_torch_autograd():
+    """The same check with torch.nn.LayerNorm (its weight and bias included) and with BatchNorm1d(affine=False)
+    in eval mode between the lookups and the interaction, as base_model.py:381-383 places them."""
+    rng = np.random.default_rng(23)
+    N, R, B, d = 9, 3, 7, 8
+    E, Rel = rng.standard_normal((N, d)), rng.standard_normal((R, d))
+    hr = np.stack([rng.integers(0, N, B), rng.integers(0, R, B)], axis=1)
+    dQ = rng.standard_normal((B, d))
+    m = d // 2
+
+    def complex_(h, r):
+        return torch.cat([h[:, :m] * r[:, :m] - h[:, m:] * r[:, m:], h[:, :m] * r[:, m:] + h[:, m:] * r[:, :m]], dim=1)
+
+    ln_h, ln_r = torch.nn.LayerNorm(d).double(), torch.nn.LayerNorm(d).double()
+    with torch.no_grad():
+        for ln in (ln_h, ln_r):
+            ln.weight.copy_(torch.from_numpy(rng.uniform(0.5, 1.5, d)))
+            ln.bias.copy_(torch.from_numpy(rng.normal(0, 0.3, d)))
+    bn_h, bn_r = torch.nn.BatchNorm1d(d, affine=False).double().eval(), torch.nn.BatchNorm1d(d, affine=False).double().eval()
+    with torch.no_grad():
+        for bn in (bn_h, bn_r):
+            bn.running_mean.copy_(torch.from_numpy(rng.normal(0, 0.2, d)))
+            bn.running_var.copy_(torch.from_numpy(rng.uniform(0.5, 2.0, d)))
+    cases = (
+        ({"kind": "LayerNorm", "eps": ln_h.eps, "h_weight": ln_h.weight.detach().numpy(),
+          "h_bias": ln_h.bias.detach().numpy(), "r_weight": ln_r.weight.detach().numpy(),
+          "r_bias": ln_r.bias.detach().numpy()}, ln_h, ln_r),
+        ({"kind": "BatchNorm1d", "eps": bn_h.eps, "h_mean": bn_h.running_mean.numpy(), "h_var": bn_h.running_var.numpy(),
+          "r_mean": bn_r.running_mean.numpy(), "r_var": bn_r.running_var.numpy()}, bn_h, bn_r))
+    for norm, mod_h, mod_r in cases:
+        Et, Rt = torch.tensor(E, requires_grad=True), torch.tensor(Rel, requires_grad=True)
+        Q = complex_(mod_h(Et[torch.from_numpy(hr[:, 0])]), mod_r(Rt[torch.from_numpy(hr[:, 1])]))
+        np.testing.assert_allclose(Q.detach().numpy(), ko.build_query("ComplEx", E, Rel, hr, norm=norm)[0],
+                                   rtol=1e-12, atol=1e-12)
+        (Q * torch.from_numpy(dQ)).sum().backward()
+        dE, dR, extra = ko.build_query_backward("ComplEx", E, Rel, hr, dQ, norm=norm)
+        np.testing.assert_allclose(dE, Et.grad.numpy(), rtol=1e-6, atol=1e-7)
+        np.testing.assert_allclose(dR, Rt.grad.numpy(), rtol=1e-6, atol=1e-7)
+        if norm["kind"] == "LayerNorm":
+            for key, prm in (("h_weight", mod_h.weight), ("h_bias", mod_h.bias), ("r_weight", mod_r.weight),
+                             ("r_bias", mod_r.bias)):
+                np.testing.assert_allclose(extra[key], prm.grad.numpy(), rtol=1e-6, atol=1e-7)
+                prm.grad = None
+        else:
+            assert not any(k in extra for k in ("h_weight", "h_bias", "r_weight", "r_bias"))
+
+
 def test_bf16_round_vs_torch():
     rng = np.random.default_rng(13)
     x = np.concatenate([rng.normal(0, 1, 5000), rng.normal(0, 1e-20, 100), [0.0, -0.0, 1.0, 3.3895314e38]])
