@@ -321,6 +321,10 @@ struct QueryBwdArgs {
   float* dn_h_b;
   float* dn_r_a;
   float* dn_r_b;
+  // BatchNorm1d with the statistics of the batch (training mode): the gradients at the normalised rows are written
+  // here, [B, d] each, for the passes that need sums over the batch (null: every other mode)
+  float* dy_h;
+  float* dy_r;
 };
 
 // One row through the backward of its normaliser: x the raw row, dy the gradient at the normalised row (both in LDS);
@@ -371,7 +375,14 @@ __global__ void __launch_bounds__(64) build_query_backward_kernel(QueryBwdArgs a
   const int lane = threadIdx.x;
   const int64_t b = blockIdx.x;
   const int64_t h_id = a.hr[2 * b], r_id = a.hr[2 * b + 1];
-  if (h_id < 0 || h_id >= a.N || r_id < 0 || r_id >= a.R) return;  // the forward gave NaN for this pair
+  if (h_id < 0 || h_id >= a.N || r_id < 0 || r_id >= a.R) {  // the forward gave NaN for this pair
+    if constexpr (NORM) {
+      if (a.dy_h) {
+        for (int k = lane; k < d; k += 64) a.dy_h[b * d + k] = a.dy_r[b * d + k] = 0.f;
+      }
+    }
+    return;
+  }
   for (int k = lane; k < d; k += 64) {
     sh[k] = a.ent[h_id * d + k];
     sr[k] = a.rel[r_id * d + k];
@@ -600,8 +611,128 @@ __global__ void __launch_bounds__(64) build_query_backward_kernel(QueryBwdArgs a
       sr[k] = a.rel[r_id * d + k];
     }
     __syncthreads();
+    if (a.dy_h) {
+      for (int k = lane; k < d; k += 64) {
+        a.dy_h[b * d + k] = sdh[k];
+        a.dy_r[b * d + k] = sdr[k];
+      }
+      return;
+    }
     normalise_row_backward(sh, sdh, d, lane, a.norm.kind, a.norm.eps, a.norm.h_a, a.norm.h_b, gh, a.dn_h_a, a.dn_h_b);
     normalise_row_backward(sr, sdr, d, lane, a.norm.kind, a.norm.eps, a.norm.r_a, a.norm.r_b, gr, a.dn_r_a, a.dn_r_b);
+  }
+}
+
+// ---- BatchNorm1d(affine=False) with the statistics of the batch (training mode) -------------------------------
+// Sums over the batch per feature, for the head rows and the relation rows of the pairs: lanes along the features
+// (whole lines per request), the four waves of a workgroup and the workgroups of grid.y along the batch, fp64
+// partial sums met with atomics in sums[4][d].
+//   GRAD == false: sum x, sum x^2 of the looked-up rows (-> mean and biased variance)
+//   GRAD == true:  sum dy, sum dy * xh with xh = (x - mean) / sqrt(var + eps), dy read from dy_h / dy_r [B, d]
+// A pair with an id outside its table poisons the sums with NaN (the forward gives NaN for it as well).
+struct BnSumArgs {
+  const float* ent;
+  const float* rel;
+  const int64_t* hr;
+  const float* dy_h;
+  const float* dy_r;
+  kge_norm_params norm;
+  double* sums;
+  int64_t B, N, R;
+  int d;
+};
+
+template <bool GRAD>
+__global__ void __launch_bounds__(256) bn_sums_kernel(BnSumArgs a) {
+  __shared__ double part[4][4][64];
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  const int f = blockIdx.x * 64 + lane;
+  const int d = a.d;
+  const int64_t per = (a.B + gridDim.y - 1) / gridDim.y;
+  const int64_t b0 = (int64_t)blockIdx.y * per, b1 = (b0 + per < a.B) ? b0 + per : a.B;
+  double s0 = 0.0, s1 = 0.0, s2 = 0.0, s3 = 0.0;
+  float mh = 0.f, ih = 0.f, mr = 0.f, ir = 0.f;
+  if (GRAD && f < d) {
+    mh = a.norm.h_a[f];
+    ih = 1.0f / sqrtf(a.norm.h_b[f] + a.norm.eps);
+    mr = a.norm.r_a[f];
+    ir = 1.0f / sqrtf(a.norm.r_b[f] + a.norm.eps);
+  }
+  for (int64_t b = b0 + w; b < b1; b += 4) {
+    const int64_t h_id = a.hr[2 * b], r_id = a.hr[2 * b + 1];
+    if (h_id < 0 || h_id >= a.N || r_id < 0 || r_id >= a.R) {
+      s0 = s1 = s2 = s3 = __longlong_as_double(0x7ff8000000000000LL);
+      continue;
+    }
+    if (f < d) {
+      const float x = a.ent[h_id * d + f], y = a.rel[r_id * d + f];
+      if (GRAD) {
+        const float gh = a.dy_h[b * d + f], gr = a.dy_r[b * d + f];
+        s0 += (double)gh;
+        s1 += (double)gh * (double)((x - mh) * ih);
+        s2 += (double)gr;
+        s3 += (double)gr * (double)((y - mr) * ir);
+      } else {
+        s0 += (double)x;
+        s1 += (double)x * (double)x;
+        s2 += (double)y;
+        s3 += (double)y * (double)y;
+      }
+    }
+  }
+  part[w][0][lane] = s0;
+  part[w][1][lane] = s1;
+  part[w][2][lane] = s2;
+  part[w][3][lane] = s3;
+  __syncthreads();
+  if (f < d) {
+    const double v = part[0][w][lane] + part[1][w][lane] + part[2][w][lane] + part[3][w][lane];  // wave w: sum w
+    atomicAdd(&a.sums[(int64_t)w * d + f], v);
+  }
+}
+
+__global__ void bn_zero_kernel(double* p, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) p[i] = 0.0;
+}
+
+// mean and biased variance of the batch, and the update of the running statistics torch.nn.BatchNorm1d makes in
+// training mode: running = (1 - momentum) * running + momentum * (mean | variance * B / (B - 1))
+__global__ void bn_finish_stats_kernel(const double* sums, int d, int64_t B, float momentum, float* h_mean, float* h_var,
+                                       float* r_mean, float* r_var, float* run_h_mean, float* run_h_var,
+                                       float* run_r_mean, float* run_r_var) {
+  const int f = blockIdx.x * blockDim.x + threadIdx.x;
+  if (f >= d) return;
+  const double n = (double)B, unb = n / (n - 1.0);
+  for (int side = 0; side < 2; ++side) {
+    const double mean = sums[(2 * side) * (int64_t)d + f] / n;
+    double var = sums[(2 * side + 1) * (int64_t)d + f] / n - mean * mean;
+    var = var < 0.0 ? 0.0 : var;  // (NaN stays NaN)
+    (side ? r_mean : h_mean)[f] = (float)mean;
+    (side ? r_var : h_var)[f] = (float)var;
+    float* rm = side ? run_r_mean : run_h_mean;
+    float* rv = side ? run_r_var : run_h_var;
+    if (rm) rm[f] = (float)((1.0 - (double)momentum) * (double)rm[f] + (double)momentum * mean);
+    if (rv) rv[f] = (float)((1.0 - (double)momentum) * (double)rv[f] + (double)momentum * var * unb);
+  }
+}
+
+// dx = (dy - mean_B(dy) - xh * mean_B(dy * xh)) / sqrt(var + eps) per pair and feature, added to the tables' gradients
+__global__ void __launch_bounds__(256) bn_backward_apply_kernel(BnSumArgs a, float* d_ent, float* d_rel) {
+  const int d = a.d;
+  const int f = blockIdx.x * 64 + (threadIdx.x & 63);
+  if (f >= d) return;
+  const double n = (double)a.B;
+  const float mh = a.norm.h_a[f], ih = 1.0f / sqrtf(a.norm.h_b[f] + a.norm.eps);
+  const float mr = a.norm.r_a[f], ir = 1.0f / sqrtf(a.norm.r_b[f] + a.norm.eps);
+  const float h1 = (float)(a.sums[f] / n), h2 = (float)(a.sums[(int64_t)d + f] / n);
+  const float r1 = (float)(a.sums[2 * (int64_t)d + f] / n), r2 = (float)(a.sums[3 * (int64_t)d + f] / n);
+  for (int64_t b = (int64_t)blockIdx.y * 4 + (threadIdx.x >> 6); b < a.B; b += 4 * (int64_t)gridDim.y) {
+    const int64_t h_id = a.hr[2 * b], r_id = a.hr[2 * b + 1];
+    if (h_id < 0 || h_id >= a.N || r_id < 0 || r_id >= a.R) continue;
+    const float xh = (a.ent[h_id * d + f] - mh) * ih, yh = (a.rel[r_id * d + f] - mr) * ir;
+    atomicAdd(&d_ent[h_id * d + f], (a.dy_h[b * d + f] - h1 - xh * h2) * ih);
+    atomicAdd(&d_rel[r_id * d + f], (a.dy_r[b * d + f] - r1 - yh * r2) * ir);
   }
 }
 
@@ -894,13 +1025,16 @@ extern "C" int kge_build_query_decal(int head, int p, int q, int r, const void* 
                           coeff_r, 0, norm, pairs, B, d, N, R, Q, bias, stream);
 }
 
+extern "C" size_t kge_batchnorm_workspace_bytes(int64_t B, int64_t d);
+
 namespace kge {
 namespace {
 int build_query_backward_impl(int model, int p, int q, int r, const float* ent, const float* rel, const float* coeff_p,
                               const float* coeff_q, const float* coeff_r, int normalize_relation,
                               const kge_norm_params* norm, const kge_norm_grads* dnorm, const int64_t* hr, int64_t B,
                               int64_t d, int64_t N, int64_t R, const float* dQ, const float* dbias, float* d_ent,
-                              float* d_rel, float* d_coeff_p, float* d_coeff_q, float* d_coeff_r, void* stream) {
+                              float* d_rel, float* d_coeff_p, float* d_coeff_q, float* d_coeff_r, void* stream,
+                              bool batch_stats = false, void* workspace = nullptr, size_t workspace_bytes = 0) {
   clear_error();
   KGE_REQUIRE(B >= 0 && N > 0 && R > 0, KGE_ERR_INVALID, "kge_build_query_backward: B=%lld N=%lld R=%lld", (long long)B,
               (long long)N, (long long)R);
@@ -956,7 +1090,38 @@ int build_query_backward_impl(int model, int p, int q, int r, const float* ent, 
   a.norm.eps = 0.f;
   a.norm.h_a = a.norm.h_b = a.norm.r_a = a.norm.r_b = nullptr;
   a.dn_h_a = a.dn_h_b = a.dn_r_a = a.dn_r_b = nullptr;
+  a.dy_h = a.dy_r = nullptr;
   hipStream_t st = (hipStream_t)stream;
+  if (batch_stats) {
+    KGE_REQUIRE(norm && norm->kind == KGE_NORM_BATCHNORM1D && norm->h_a && norm->h_b && norm->r_a && norm->r_b,
+                KGE_ERR_INVALID,
+                "kge_build_query_backward_batchnorm: norm must be BatchNorm1d with the batch's statistics");
+    KGE_REQUIRE(d <= 4096, KGE_ERR_UNSUPPORTED, "kge_build_query_backward_batchnorm: d=%lld exceeds 4096", (long long)d);
+    KGE_REQUIRE(B >= 2, KGE_ERR_INVALID, "kge_build_query_backward_batchnorm: batch statistics need B >= 2");
+    const size_t need = kge_batchnorm_workspace_bytes(B, d);
+    KGE_REQUIRE(workspace && workspace_bytes >= need, KGE_ERR_WORKSPACE,
+                "kge_build_query_backward_batchnorm: workspace of %zu bytes, need %zu", workspace_bytes, need);
+    KGE_REQUIRE(((uintptr_t)workspace & 15) == 0, KGE_ERR_WORKSPACE,
+                "kge_build_query_backward_batchnorm: workspace must be 16-byte aligned");
+    double* sums = (double*)workspace;
+    a.norm = *norm;
+    a.dy_h = (float*)(sums + 4 * d);
+    a.dy_r = a.dy_h + B * d;
+    hipLaunchKernelGGL(bn_zero_kernel, dim3((unsigned)((4 * d + 255) / 256)), dim3(256), 0, st, sums, (int)(4 * d));
+    KGE_LAUNCH_CHECK("bn_zero_kernel");
+    // (1) the gradients at the normalised rows, (2) their sums over the batch, (3) the gradients at the raw rows
+    const size_t lds_bytes = (5 * (size_t)d + (size_t)(d + 3) / 4) * sizeof(float);
+    hipLaunchKernelGGL(build_query_backward_kernel<true>, dim3((unsigned)B), dim3(64), lds_bytes, st, a, model);
+    KGE_LAUNCH_CHECK("build_query_backward_kernel");
+    BnSumArgs sa{ent, rel, hr, a.dy_h, a.dy_r, *norm, sums, B, N, R, (int)d};
+    const unsigned slices = (unsigned)((B + 63) / 64 < 64 ? (B + 63) / 64 : 64);
+    dim3 grid((unsigned)((d + 63) / 64), slices);
+    hipLaunchKernelGGL(bn_sums_kernel<true>, grid, dim3(256), 0, st, sa);
+    KGE_LAUNCH_CHECK("bn_sums_kernel");
+    hipLaunchKernelGGL(bn_backward_apply_kernel, grid, dim3(256), 0, st, sa, d_ent, d_rel);
+    KGE_LAUNCH_CHECK("bn_backward_apply_kernel");
+    return KGE_OK;
+  }
   if (norm && norm->kind != KGE_NORM_NONE) {
     KGE_REQUIRE(norm->kind == KGE_NORM_LAYERNORM || norm->kind == KGE_NORM_BATCHNORM1D, KGE_ERR_INVALID,
                 "kge_build_query_backward_norm: unknown normalisation %d", norm->kind);
@@ -986,6 +1151,54 @@ int build_query_backward_impl(int model, int p, int q, int r, const float* ent, 
 }
 }  // namespace
 }  // namespace kge
+
+extern "C" size_t kge_batchnorm_workspace_bytes(int64_t B, int64_t d) {
+  if (B < 1 || d < 1) return 0;
+  return 4 * (size_t)d * sizeof(double) + 2 * (size_t)B * (size_t)d * sizeof(float);
+}
+
+extern "C" int kge_batchnorm_stats(const float* ent, const float* rel, const int64_t* hr, int64_t B, int64_t d, int64_t N,
+                                   int64_t R, float momentum, float* h_mean, float* h_var, float* r_mean, float* r_var,
+                                   float* run_h_mean, float* run_h_var, float* run_r_mean, float* run_r_var,
+                                   void* workspace, size_t workspace_bytes, void* stream) {
+  using namespace kge;
+  clear_error();
+  KGE_REQUIRE(N > 0 && R > 0 && d >= 1 && d <= 8192, KGE_ERR_INVALID, "kge_batchnorm_stats: N=%lld R=%lld d=%lld",
+              (long long)N, (long long)R, (long long)d);
+  KGE_REQUIRE(B >= 2 && B <= 0x7fffffff, KGE_ERR_INVALID,
+              "kge_batchnorm_stats: B=%lld (the statistics of a batch need at least two rows)", (long long)B);
+  KGE_REQUIRE(ent && rel && hr && h_mean && h_var && r_mean && r_var, KGE_ERR_INVALID,
+              "kge_batchnorm_stats: null pointer argument");
+  KGE_REQUIRE(momentum >= 0.f && momentum <= 1.f, KGE_ERR_INVALID, "kge_batchnorm_stats: momentum %g", (double)momentum);
+  KGE_REQUIRE(workspace && workspace_bytes >= 4 * (size_t)d * sizeof(double), KGE_ERR_WORKSPACE,
+              "kge_batchnorm_stats: workspace of %zu bytes, need %zu", workspace_bytes, 4 * (size_t)d * sizeof(double));
+  KGE_REQUIRE(((uintptr_t)workspace & 7) == 0, KGE_ERR_WORKSPACE, "kge_batchnorm_stats: workspace must be 8-byte aligned");
+  hipStream_t st = (hipStream_t)stream;
+  double* sums = (double*)workspace;
+  hipLaunchKernelGGL(bn_zero_kernel, dim3((unsigned)((4 * d + 255) / 256)), dim3(256), 0, st, sums, (int)(4 * d));
+  KGE_LAUNCH_CHECK("bn_zero_kernel");
+  kge_norm_params none{};
+  BnSumArgs sa{ent, rel, hr, nullptr, nullptr, none, sums, B, N, R, (int)d};
+  const unsigned slices = (unsigned)((B + 63) / 64 < 64 ? (B + 63) / 64 : 64);
+  hipLaunchKernelGGL(bn_sums_kernel<false>, dim3((unsigned)((d + 63) / 64), slices), dim3(256), 0, st, sa);
+  KGE_LAUNCH_CHECK("bn_sums_kernel");
+  hipLaunchKernelGGL(bn_finish_stats_kernel, dim3((unsigned)((d + 255) / 256)), dim3(256), 0, st, sums, (int)d, B, momentum,
+                     h_mean, h_var, r_mean, r_var, run_h_mean, run_h_var, run_r_mean, run_r_var);
+  KGE_LAUNCH_CHECK("bn_finish_stats_kernel");
+  return KGE_OK;
+}
+
+extern "C" int kge_build_query_backward_batchnorm(int model, int p, int q, int r, const float* ent, const float* rel,
+                                                  const float* coeff_p, const float* coeff_q, const float* coeff_r,
+                                                  int normalize_relation, const kge_norm_params* norm,
+                                                  const int64_t* hr, int64_t B, int64_t d, int64_t N, int64_t R,
+                                                  const float* dQ, const float* dbias, float* d_ent, float* d_rel,
+                                                  float* d_coeff_p, float* d_coeff_q, float* d_coeff_r,
+                                                  void* workspace, size_t workspace_bytes, void* stream) {
+  return kge::build_query_backward_impl(model, p, q, r, ent, rel, coeff_p, coeff_q, coeff_r, normalize_relation, norm,
+                                        nullptr, hr, B, d, N, R, dQ, dbias, d_ent, d_rel, d_coeff_p, d_coeff_q,
+                                        d_coeff_r, stream, true, workspace, workspace_bytes);
+}
 
 extern "C" int kge_build_query_backward(int model, int p, int q, int r, const float* ent, const float* rel,
                                         const float* coeff_p, const float* coeff_q, const float* coeff_r,

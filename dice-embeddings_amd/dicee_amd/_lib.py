@@ -40,6 +40,12 @@ SIGNATURES = {
     "kge_build_query_backward_norm": (_c_int, [_c_int, _c_int, _c_int, _c_int, _vp, _vp, _vp, _vp, _vp, _c_int,
                                                ctypes.POINTER(NormParams), ctypes.POINTER(NormGrads), _vp, _c_i64,
                                                _c_i64, _c_i64, _c_i64, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
+    "kge_batchnorm_workspace_bytes": (_sz, [_c_i64, _c_i64]),
+    "kge_batchnorm_stats": (_c_int, [_vp, _vp, _vp, _c_i64, _c_i64, _c_i64, _c_i64, _c_f, _vp, _vp, _vp, _vp, _vp, _vp,
+                                     _vp, _vp, _vp, _sz, _vp]),
+    "kge_build_query_backward_batchnorm": (_c_int, [_c_int, _c_int, _c_int, _c_int, _vp, _vp, _vp, _vp, _vp, _c_int,
+                                                    ctypes.POINTER(NormParams), _vp, _c_i64, _c_i64, _c_i64, _c_i64,
+                                                    _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
     "kge_scores": (_c_int, [_vp, _vp, _vp, _c_int, _vp, _c_i64, _c_i64, _c_i64, _vp, _c_i64, _vp]),
     "kge_triple_scores": (_c_int, [_vp, _vp, _vp, _c_int, _vp, _c_i64, _c_i64, _c_i64, _vp, _vp, _vp]),
     "kge_sample_scores": (_c_int, [_vp, _vp, _vp, _c_int, _vp, _c_i64, _c_i64, _c_i64, _vp, _c_i64, _vp, _vp]),

@@ -5,9 +5,10 @@ Parameter names follow dicee so that a dicee ``model.pt`` state_dict loads uncha
 ``q_coefficients.weight``, ``normalize_*_embeddings.*``): dicee/models/base_model.py:121-176,
 dicee/models/clifford.py:4-28.
 
-Only the inference-time semantics of the path are implemented: dropout is the identity
-(base_model.py:149-151 in eval mode) and BatchNorm1d uses its running statistics.  A model in training mode
-whose dropout rates are not zero refuses to score (the reference would drop elements there) instead of
+Normalisation layers follow the module's mode: LayerNorm is the same in both; BatchNorm1d normalises with its
+running statistics in eval mode and with the statistics of the batch in training mode (moving the running
+statistics, as torch does).  Dropout is the identity (base_model.py:149-151 in eval mode): a model in training
+mode whose dropout rates are not zero refuses to score (the reference would drop elements there) instead of
 silently scoring without dropout.
 """
 import torch
@@ -25,6 +26,9 @@ class IdentityClass(torch.nn.Module):
     @staticmethod
     def forward(x):
         return x
+
+
+_FROM_MODEL = object()   # "take the normalisation layer from the model" (None means: no layer)
 
 
 class BaseKGE(torch.nn.Module):
@@ -137,12 +141,32 @@ class BaseKGE(torch.nn.Module):
                 "call model.eval() or set the rates to zero")
 
     # ------------------------------------------------------------------ query construction
-    def _norm_params(self):
+    def _norm_params(self, x=None):
+        """The normalisation layer between the lookups and the interaction, as the kernels take it.  BatchNorm1d in
+        training mode normalises with the statistics of the batch ``x`` [B,2] itself and moves its running
+        statistics towards them (torch.nn.BatchNorm1d; base_model.py:289-294 applied at :381-383): every call with
+        a batch is one such forward."""
         nh, nr = self.normalize_head_entity_embeddings, self.normalize_relation_embeddings
         if isinstance(nh, torch.nn.LayerNorm):
             return {"kind": "LayerNorm", "eps": nh.eps, "h_a": nh.weight.detach(), "h_b": nh.bias.detach(),
                     "r_a": nr.weight.detach(), "r_b": nr.bias.detach()}
         if isinstance(nh, torch.nn.BatchNorm1d):
+            if self.training and x is not None:
+                if self._storage != "fp32":
+                    raise NotImplementedError("BatchNorm1d in training mode needs the fp32 tables")
+                if nh.momentum is None or nr.momentum is None or nh.momentum != nr.momentum:
+                    raise NotImplementedError("BatchNorm1d with a cumulative average (momentum=None) or two momenta")
+                E, _ = self.table()
+                pairs = x.to(device=E.device, dtype=torch.int64).contiguous()
+                running = None
+                if nh.track_running_stats and nh.running_mean is not None:
+                    running = {"h_mean": nh.running_mean, "h_var": nh.running_var, "r_mean": nr.running_mean,
+                               "r_var": nr.running_var}
+                norm = ops.batchnorm_stats(E, self._rel(), pairs, eps=nh.eps, momentum=nh.momentum, running=running)
+                if running is not None:
+                    nh.num_batches_tracked += 1
+                    nr.num_batches_tracked += 1
+                return norm
             return {"kind": "BatchNorm1d", "eps": nh.eps, "h_a": nh.running_mean, "h_b": nh.running_var,
                     "r_a": nr.running_mean, "r_b": nr.running_var}
         return None
@@ -150,7 +174,7 @@ class BaseKGE(torch.nn.Module):
     def _query_kwargs(self):
         return {}
 
-    def query(self, x, heads=False):
+    def query(self, x, heads=False, norm=_FROM_MODEL):
         """(Q [B,d], bias [B]) for ``x`` [B,2]: gather + interaction
         (get_head_relation_representation, base_model.py:377-384, then the model's elementwise part).
         ``heads=True``: ``x`` holds (relation, tail) pairs and ``Q @ E^T`` scores every entity as the head of
@@ -158,8 +182,10 @@ class BaseKGE(torch.nn.Module):
         self._refuse_dropout_in_training()
         E, scale = self.table()
         x = x.to(device=E.device, dtype=torch.int64).contiguous()
+        if norm is _FROM_MODEL:
+            norm = self._norm_params(None if heads else x)
         return ops.build_query(self.name if self.name != "CKeci" else "Keci", E, self._rel(), x, ent_scale=scale,
-                               norm=self._norm_params(), head=heads, **self._query_kwargs())
+                               norm=norm, head=heads, **self._query_kwargs())
 
     # ------------------------------------------------------------------ reference call surface
     def forward(self, x, y_idx=None):
@@ -262,12 +288,12 @@ class BaseKGE(torch.nn.Module):
         rows = csr.rows_for(x.to(device=E.device, dtype=torch.int64))
         return ops.bce_multihot(Q, bias, E, scale, rows, csr.row_ptr, csr.col, label_smoothing)[0]
 
-    def kvsall_bce_backward(self, x, csr, label_smoothing=0.0, grad_out=1.0):
+    def kvsall_bce_backward(self, x, csr, label_smoothing=0.0, grad_out=1.0, norm=_FROM_MODEL):
         """The same step with its backward through the scores: ``(loss, dQ [B,d], dbias [B], dE [N,d])`` where
         ``dQ`` / ``dbias`` are the gradients at the query vectors and per-query biases of ``self.query(x)`` and ``dE``
         the gradient the contraction sends to the entity table (fp32 tables only).  What
         ``loss_batch.backward()`` computes for the ``torch.mm`` / ``einsum`` and the loss of the reference's step."""
-        Q, bias = self.query(x)
+        Q, bias = self.query(x, norm=norm)
         E, scale = self.table()
         if scale is not None:
             raise TypeError("the backward needs an fp32 entity table")
@@ -282,17 +308,14 @@ class BaseKGE(torch.nn.Module):
         embeddings.  What ``loss_batch.backward()`` leaves in ``.grad`` after ``training_step`` (base_model.py:25-46)
         for fp32 tables.  With ``normalization='LayerNorm'`` the gradient passes through both normalisers and their
         weights and biases receive theirs (``normalize_head_entity_embeddings.weight`` ...); with ``'BatchNorm1d'``
-        it passes through the running statistics, which is what the module does in eval mode: in training mode the
-        reference normalises with the statistics of the batch, which this path does not form."""
-        norm = self._norm_params()
-        if norm is not None and norm["kind"] == "BatchNorm1d" and self.training:
-            raise NotImplementedError("BatchNorm1d in training mode (batch statistics) is not part of this path; "
-                                      "call model.eval() for the gradient through the running statistics")
+        it passes through the statistics of the batch in training mode (which also moves the running statistics, once)
+        and through the running statistics in eval mode."""
         E, scale = self.table()
         if scale is not None or E.dtype != torch.float32:
             raise TypeError("the backward needs an fp32 entity table")
         x = x.to(device=E.device, dtype=torch.int64).contiguous()
-        loss, dQ, dbias, dE = self.kvsall_bce_backward(x, csr, label_smoothing)
+        norm = self._norm_params(x)
+        loss, dQ, dbias, dE = self.kvsall_bce_backward(x, csr, label_smoothing, norm=norm)
         rel = self._rel()
         dR = torch.zeros_like(rel)
         name = self.name if self.name != "CKeci" else "Keci"

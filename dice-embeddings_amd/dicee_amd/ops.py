@@ -97,13 +97,45 @@ def build_query(model, ent, rel, hr, *, ent_scale=None, p=0, q=0, r=0, coeff_p=N
     return Q, bias
 
 
+def batchnorm_stats(ent, rel, hr, *, eps=1e-5, momentum=0.1, running=None):
+    """The normalisation layer ``BatchNorm1d(affine=False)`` applies to THIS batch in training mode: a ``norm`` dict
+    for ``build_query`` holding the mean and biased variance, per feature, of the looked-up head rows and relation
+    rows.  ``running``: dict with ``h_mean, h_var, r_mean, r_var`` ([d] fp32 GPU tensors, the modules' buffers),
+    updated in place as torch does in training mode."""
+    lib = _lib.load()
+    _require_gpu(ent, rel, hr)
+    if ent.dtype != torch.float32 or rel.dtype != torch.float32 or not ent.is_contiguous() or not rel.is_contiguous():
+        raise TypeError("batchnorm_stats needs contiguous fp32 tables")
+    if hr.dtype != torch.int64 or hr.dim() != 2 or hr.shape[1] != 2 or not hr.is_contiguous():
+        raise ValueError("hr must be a contiguous int64 tensor of shape [B, 2]")
+    B, (N, d), R = hr.shape[0], ent.shape, rel.shape[0]
+    if B < 2:
+        raise ValueError(f"Expected more than 1 value per channel when training, got input size [{B}, {d}]")
+    out = torch.empty((4, d), dtype=torch.float32, device=ent.device)
+    run = [None] * 4
+    if running is not None:
+        run = [running[k] for k in ("h_mean", "h_var", "r_mean", "r_var")]
+        for t in run:
+            if t.dtype != torch.float32 or not t.is_contiguous() or t.numel() != d:
+                raise TypeError("running statistics must be contiguous fp32 tensors of d elements")
+        _require_gpu(*run)
+    ws = torch.empty((4 * d,), dtype=torch.float64, device=ent.device)
+    rc = lib.kge_batchnorm_stats(_ptr(ent), _ptr(rel), _ptr(hr), B, d, N, R, float(momentum), _ptr(out[0]), _ptr(out[1]),
+                                 _ptr(out[2]), _ptr(out[3]), _ptr(run[0]), _ptr(run[1]), _ptr(run[2]), _ptr(run[3]),
+                                 _ptr(ws), ws.numel() * 8, _stream())
+    _lib.check(rc)
+    return {"kind": "BatchNorm1d", "eps": float(eps), "h_a": out[0], "h_b": out[1], "r_a": out[2], "r_b": out[3],
+            "batch": True}
+
+
 def build_query_backward(model, ent, rel, hr, dQ, dbias, d_ent, d_rel, *, p=0, q=0, r=0, coeff_p=None, coeff_q=None,
                          coeff_r=None, normalize_relation=True, norm=None, dnorm=None):
     """Adds the gradients that ``dQ`` [B,d] / ``dbias`` [B] send back through ``build_query`` into ``d_ent`` [N,d]
     and ``d_rel`` [R,d] (fp32, caller-initialised); returns the gradients of the Clifford coefficients
     ``(d_coeff_p, d_coeff_q, d_coeff_r)`` (None where the model has none).  ``norm``: the normalisation layer of
     ``build_query``; ``dnorm``: for LayerNorm, a dict with any of ``h_a, h_b, r_a, r_b`` ([d] fp32,
-    caller-initialised) that receive the gradients of the normalisers' weights and biases."""
+    caller-initialised) that receive the gradients of the normalisers' weights and biases.  A ``norm`` that
+    ``batchnorm_stats`` made for this batch (``norm["batch"]``) is differentiated as a function of the batch."""
     lib = _lib.load()
     _require_gpu(ent, rel, hr, dQ, dbias, d_ent, d_rel, coeff_p, coeff_q, coeff_r)
     for t in (ent, rel, dQ, d_ent, d_rel):
@@ -111,6 +143,17 @@ def build_query_backward(model, ent, rel, hr, dQ, dbias, d_ent, d_rel, *, p=0, q
             raise TypeError("build_query_backward needs contiguous fp32 tensors")
     B, (N, d), R = hr.shape[0], ent.shape, rel.shape[0]
     outs = [torch.zeros_like(c) if c is not None else None for c in (coeff_p, coeff_q, coeff_r)]
+    if norm is not None and norm.get("batch"):
+        ns, keep = _norm_struct(norm)
+        nbytes = lib.kge_batchnorm_workspace_bytes(B, d)
+        ws = torch.empty(((nbytes + 7) // 8,), dtype=torch.float64, device=ent.device)
+        rc = lib.kge_build_query_backward_batchnorm(
+            MODEL_IDS[model], int(p), int(q), int(r), _ptr(ent), _ptr(rel), _ptr(coeff_p), _ptr(coeff_q), _ptr(coeff_r),
+            int(bool(normalize_relation)), ctypes.byref(ns), _ptr(hr), B, d, N, R, _ptr(dQ), _ptr(dbias), _ptr(d_ent),
+            _ptr(d_rel), _ptr(outs[0]), _ptr(outs[1]), _ptr(outs[2]), _ptr(ws), ws.numel() * 8, _stream())
+        _lib.check(rc)
+        del keep
+        return tuple(outs)
     if norm is not None:
         ns, keep = _norm_struct(norm)
         gs = None

@@ -170,6 +170,35 @@ int kge_build_query_backward_norm(int model, int p, int q, int r, const float* e
                                   float* d_coeff_r, void* stream);
 
 /*
+ * BatchNorm1d(affine=False) in TRAINING mode (dicee/models/base_model.py:289-294 applied at :381-383 while
+ * `self.training`): the layer normalises with the statistics of the batch it is given.
+ *
+ * kge_batchnorm_stats: per feature, mean and biased variance over the B looked-up head rows -> h_mean / h_var [d]
+ * and over the B relation rows -> r_mean / r_var [d]; pass them to kge_build_query as a KGE_NORM_BATCHNORM1D
+ * layer (a = mean, b = variance) for this batch's forward.  run_* (each may be NULL): the module's running
+ * statistics, updated in place as torch does in training mode, running <- (1 - momentum) * running + momentum *
+ * (mean | variance * B / (B - 1)).  A pair with an id outside its table makes every statistic NaN.  B >= 2 (torch
+ * raises for one value per channel).  workspace: 32 * d bytes, 8-byte aligned.
+ *
+ * kge_build_query_backward_batchnorm: kge_build_query_backward through that layer, the statistics being functions
+ * of the batch: dx = (dy - mean_B(dy) - xh * mean_B(dy * xh)) / sqrt(var + eps) with xh the normalised row.  norm
+ * holds the SAME statistics the forward used.  workspace: kge_batchnorm_workspace_bytes(B, d) = 32 * d +
+ * 8 * B * d bytes (the gradients at the normalised rows make a round trip: their sums over the batch are needed
+ * before any gradient at a raw row can be formed), 16-byte aligned.  d <= 4096.
+ */
+size_t kge_batchnorm_workspace_bytes(int64_t B, int64_t d);
+int kge_batchnorm_stats(const float* ent, const float* rel, const int64_t* hr, int64_t B, int64_t d, int64_t N,
+                        int64_t R, float momentum, float* h_mean, float* h_var, float* r_mean, float* r_var,
+                        float* run_h_mean, float* run_h_var, float* run_r_mean, float* run_r_var, void* workspace,
+                        size_t workspace_bytes, void* stream);
+int kge_build_query_backward_batchnorm(int model, int p, int q, int r, const float* ent, const float* rel,
+                                       const float* coeff_p, const float* coeff_q, const float* coeff_r,
+                                       int normalize_relation, const kge_norm_params* norm, const int64_t* hr,
+                                       int64_t B, int64_t d, int64_t N, int64_t R, const float* dQ, const float* dbias,
+                                       float* d_ent, float* d_rel, float* d_coeff_p, float* d_coeff_q,
+                                       float* d_coeff_r, void* workspace, size_t workspace_bytes, void* stream);
+
+/*
  * Materialised scores S[b, e] = dot(Q[b], E[e]) (* scale[e]) (+ bias[b]); S has row stride ldS.
  * Replaces the torch.mm / einsum calls and B x N adds of real.py:32, complex.py:260-264,
  * quaternion.py:152-156, clifford.py:269-305.  For callers that need the whole matrix

@@ -163,13 +163,33 @@ def batch_norm_eval(x, running_mean, running_var, eps=1e-5):
     return (x - np.asarray(running_mean, np.float64)) / np.sqrt(np.asarray(running_var, np.float64) + eps)
 
 
+def batch_norm_train(x, eps=1e-5):
+    """torch.nn.BatchNorm1d(affine=False) in training mode (base_model.py:289-294 while ``self.training``): every
+    feature by the mean and the BIASED variance of the batch it is given."""
+    x = np.asarray(x, dtype=np.float64)
+    mu = x.mean(axis=0, keepdims=True)
+    var = ((x - mu) ** 2).mean(axis=0, keepdims=True)
+    return (x - mu) / np.sqrt(var + eps)
+
+
+def batch_norm_running_update(x, running_mean, running_var, momentum=0.1):
+    """What the same call leaves in the module's buffers: ``(1 - momentum) * running + momentum * statistic`` with the
+    batch mean and the UNBIASED batch variance (torch.nn.BatchNorm1d, training mode)."""
+    x = np.asarray(x, dtype=np.float64)
+    n = x.shape[0]
+    mu = x.mean(axis=0)
+    var_unbiased = ((x - mu) ** 2).sum(axis=0) / (n - 1)
+    return ((1 - momentum) * np.asarray(running_mean, np.float64) + momentum * mu,
+            (1 - momentum) * np.asarray(running_var, np.float64) + momentum * var_unbiased)
+
+
 def gather_hr(E, R, hr, norm=None, dtype=np.float64):
     """Head / relation rows for a batch of (head_id, relation_id) pairs.
 
     Dropout is the identity in eval mode (base_model.py:149-151).  ``norm`` is
     None (IdentityClass) or a dict: ``{"kind": "LayerNorm", "h_weight", "h_bias",
     "r_weight", "r_bias", "eps"}`` / ``{"kind": "BatchNorm1d", "h_mean", "h_var",
-    "r_mean", "r_var", "eps"}``.
+    "r_mean", "r_var", "eps"}`` / ``{"kind": "BatchNorm1dTrain", "eps"}`` (the statistics of this very batch).
     """
     hr = np.asarray(hr)
     h = np.take(np.asarray(E), hr[:, 0], axis=0).astype(dtype)
@@ -182,6 +202,9 @@ def gather_hr(E, R, hr, norm=None, dtype=np.float64):
         elif norm["kind"] == "BatchNorm1d":
             h = batch_norm_eval(h, norm["h_mean"], norm["h_var"], eps).astype(dtype)
             r = batch_norm_eval(r, norm["r_mean"], norm["r_var"], eps).astype(dtype)
+        elif norm["kind"] == "BatchNorm1dTrain":
+            h = batch_norm_train(h, eps).astype(dtype)
+            r = batch_norm_train(r, eps).astype(dtype)
         else:
             raise NotImplementedError(norm["kind"])
     return h, r
@@ -616,6 +639,38 @@ def build_query_backward(model, E, R, hr, dQ, dbias=None, step=1e-6, **kw):
                 grad[i] = ((per_pair(rows_h, rows_r, kp) - per_pair(rows_h, rows_r, km)) / (2 * step)).sum()
             dcoeff[key] = grad
     return dE, dR, dcoeff
+
+
+def build_query_backward_batch(model, E, R, hr, dQ, dbias=None, step=1e-6, **kw):
+    """``build_query_backward`` for a layer that couples the rows of the batch (``norm`` of kind
+    ``"BatchNorm1dTrain"``): central differences of the WHOLE batch's ``sum_b dQ[b] . Q[b] + dbias[b] * bias[b]``, one
+    coordinate of one looked-up row at a time, scattered to the tables.  O(B^2 d) work: small cases only.
+    Returns (dE [N,d], dR [R,d])."""
+    E = np.asarray(E, dtype=np.float64)
+    R = np.asarray(R, dtype=np.float64)
+    hr = np.asarray(hr)
+    dQ = np.asarray(dQ, dtype=np.float64)
+    B, d = dQ.shape
+    db = np.zeros(B) if dbias is None else np.asarray(dbias, dtype=np.float64)
+    rows_h, rows_r = E[hr[:, 0]].copy(), R[hr[:, 1]].copy()
+    pairs = np.stack([np.arange(B), np.arange(B)], axis=1)
+
+    def total(h_rows, r_rows):
+        Q, bias = build_query(model, h_rows, r_rows, pairs, dtype=np.float64, **kw)
+        return float((dQ * Q).sum() + (db * bias).sum())
+
+    dE, dR = np.zeros_like(E), np.zeros_like(R)
+    for b in range(B):
+        for k in range(d):
+            for rows, out, idx, which in ((rows_h, dE, hr[b, 0], 0), (rows_r, dR, hr[b, 1], 1)):
+                keep = rows[b, k]
+                rows[b, k] = keep + step
+                up = total(rows_h, rows_r)
+                rows[b, k] = keep - step
+                down = total(rows_h, rows_r)
+                rows[b, k] = keep
+                out[idx, k] += (up - down) / (2 * step)
+    return dE, dR
 
 
 def k_vs_all_scores(model, E, R, hr, **kw):

@@ -889,9 +889,47 @@ def test_full_step_gradients_through_the_normalisation_layer_match_autograd(name
         assert g.shape == w.shape, key
         rms = np.sqrt((w ** 2).mean())
         assert np.abs(g - w).max() <= 5e-5 * rms + 1e-9, (key, np.abs(g - w).max() / rms)
-    if kind == "BatchNorm1d":
-        with pytest.raises(NotImplementedError):
-            m.train().kvsall_bce_gradients(torch.from_numpy(x_np.copy()).cuda(), csr)
+
+
+def test_full_step_in_training_mode_with_batchnorm_matches_torch_modules_in_training_mode():
+    """normalization='BatchNorm1d', model.train(): loss, gradients and the running statistics the step leaves against
+    torch.nn.BatchNorm1d(affine=False).train() modules inside the reference's op sequence (float64, CPU)."""
+    from dicee_amd import FilterCSR
+    import copy
+    d = 32
+    m, triples = _toy("ComplEx", d, n=900, seed=77, normalization="BatchNorm1d")
+    er = ko.vocab(triples, "er")
+    E = m.entity_embeddings.weight.detach().double().clone().requires_grad_()
+    Rel = m.relation_embeddings.weight.detach().double().clone().requires_grad_()
+    ref_h = copy.deepcopy(m.normalize_head_entity_embeddings).double().train()
+    ref_r = copy.deepcopy(m.normalize_relation_embeddings).double().train()
+    x_np = triples[:256, :2]
+    positives = [er[(int(h), int(r))] for h, r in x_np]
+    ref = tcp.kvsall_bce_step("ComplEx", E, Rel, torch.from_numpy(x_np.copy()), positives, 0.1, norm_h=ref_h, norm_r=ref_r)
+    ref.backward()
+    m = m.to("cuda").train()
+    csr = FilterCSR.from_er_vocab(er, 46, device="cuda")
+    loss, grads = m.kvsall_bce_gradients(torch.from_numpy(x_np.copy()).cuda(), csr, label_smoothing=0.1)
+    assert loss.item() == pytest.approx(ref.item(), rel=1e-5)
+    want = {"entity_embeddings.weight": E.grad, "relation_embeddings.weight": Rel.grad}
+    assert set(grads) == set(want)
+    for key, w in want.items():
+        w = w.numpy()
+        g = grads[key].cpu().numpy()
+        rms = np.sqrt((w ** 2).mean())
+        assert np.abs(g - w).max() <= 1e-4 * rms + 1e-9, (key, np.abs(g - w).max() / rms)
+    for ours, theirs in ((m.normalize_head_entity_embeddings, ref_h), (m.normalize_relation_embeddings, ref_r)):
+        assert int(ours.num_batches_tracked) == int(theirs.num_batches_tracked) == 1
+        np.testing.assert_allclose(ours.running_mean.cpu().numpy(), theirs.running_mean.numpy(), rtol=1e-5, atol=1e-7)
+        np.testing.assert_allclose(ours.running_var.cpu().numpy(), theirs.running_var.numpy(), rtol=1e-5, atol=1e-7)
+    # eval mode afterwards scores with the running statistics, as the module does
+    m.eval()
+    s = m(torch.from_numpy(x_np[:8].copy()).cuda()).cpu().numpy()
+    with torch.no_grad():
+        want_s = tcp.forward_k_vs_all("ComplEx", E.detach(), Rel.detach(), torch.from_numpy(x_np[:8].copy()),
+                                      norm_h=ref_h.eval(), norm_r=ref_r.eval()).numpy()
+    ok, worst = score_close(s, want_s, 1e-4)
+    assert ok, worst
 
 
 def test_full_step_gradients_of_omult_and_decal_against_the_composed_oracle():

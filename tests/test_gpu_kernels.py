@@ -1057,6 +1057,72 @@ def test_build_query_backward_through_the_normalisation_layer(ops, model, d, kw,
             assert np.abs(got - want).max() <= 5e-5 * np.sqrt((want ** 2).mean()) + 1e-5, (gk, got[:4], want[:4])
 
 
+@pytest.mark.parametrize("model,d,kw,B", [("DistMult", 16, {}, 12), ("ComplEx", 70, {}, 9), ("QMult", 16, {}, 11),
+                                          ("Keci", 15, {"p": 2, "q": 2, "coeff_p": [0.7, 1.1], "coeff_q": [1.3, -0.4]}, 10),
+                                          ("OMult", 16, {"normalize_relation": False}, 2)])
+def test_batchnorm_training_mode_statistics_forward_and_backward(ops, model, d, kw, B):
+    """BatchNorm1d(affine=False) with the statistics of the batch: the statistics and the running-statistics update
+    against the oracle, the query vectors built with them, and the gradient through them against central
+    differences of the whole batch (fp64).  Pairs repeat heads and relations."""
+    rng = np.random.default_rng(900 + d)
+    N, R = 7, 3
+    E, Rel = random_tables(rng, N, R, d, std=0.8)
+    hr = random_hr(rng, N, R, B)
+    dQ = rng.standard_normal((B, d)).astype(np.float32)
+    dbias = rng.standard_normal(B).astype(np.float32)
+    run0 = {"h_mean": rng.normal(0, 0.2, d), "h_var": rng.uniform(0.5, 2, d), "r_mean": rng.normal(0, 0.2, d),
+            "r_var": rng.uniform(0.5, 2, d)}
+    running = {k: dev(torch.from_numpy(v.astype(np.float32))) for k, v in run0.items()}
+    Eg, Rg, hrg = dev(torch.from_numpy(E)), dev(torch.from_numpy(Rel)), dev(torch.from_numpy(hr))
+    norm = ops.batchnorm_stats(Eg, Rg, hrg, eps=1e-5, momentum=0.1, running=running)
+    rows = {"h": E[hr[:, 0]].astype(np.float64), "r": Rel[hr[:, 1]].astype(np.float64)}
+    for side in "hr":
+        x = rows[side]
+        np.testing.assert_allclose(norm[side + "_a"].cpu().numpy(), x.mean(axis=0), rtol=1e-6, atol=1e-7)
+        np.testing.assert_allclose(norm[side + "_b"].cpu().numpy(), x.var(axis=0), rtol=1e-5, atol=1e-7)
+        rm, rv = ko.batch_norm_running_update(x, run0[side + "_mean"].astype(np.float32), run0[side + "_var"].astype(np.float32), 0.1)
+        np.testing.assert_allclose(running[side + "_mean"].cpu().numpy(), rm, rtol=1e-6, atol=1e-7)
+        np.testing.assert_allclose(running[side + "_var"].cpu().numpy(), rv, rtol=1e-5, atol=1e-7)
+    onorm = {"kind": "BatchNorm1dTrain", "eps": 1e-5}
+    gkw = _gpu_kwargs(kw)
+    Q, bias = ops.build_query(model, Eg, Rg, hrg, norm=norm, **gkw)
+    Qr, br = ko.build_query(model, E, Rel, hr, norm=onorm, **kw)
+    ok, worst = score_close(Q.cpu().numpy(), Qr, 5e-5)
+    assert ok, worst
+    d_ent, d_rel = torch.zeros_like(Eg), torch.zeros_like(Rg)
+    ops.build_query_backward(model, Eg, Rg, hrg, dev(torch.from_numpy(dQ)), dev(torch.from_numpy(dbias)), d_ent, d_rel,
+                             norm=norm, **gkw)
+    wE, wR = ko.build_query_backward_batch(model, E, Rel, hr, dQ, dbias, norm=onorm, **kw)
+    for got, want, name in ((d_ent, wE, "d_ent"), (d_rel, wR, "d_rel")):
+        got = got.cpu().numpy()
+        rms = np.sqrt((want ** 2).mean())
+        assert np.abs(got - want).max() <= 2e-4 * rms + 2e-5, (name, np.abs(got - want).max() / rms)
+
+
+def test_batchnorm_statistics_over_a_large_batch_and_bad_arguments(ops):
+    from dicee_amd._lib import KgeError
+    rng = np.random.default_rng(77)
+    N, R, d, B = 500, 11, 200, 5000          # several batch slices per feature block, a ragged last feature block
+    E, Rel = random_tables(rng, N, R, d, std=1.0)
+    E += 3.0                                 # a mean far from zero: the variance must not cancel
+    hr = random_hr(rng, N, R, B)
+    Eg, Rg, hrg = dev(torch.from_numpy(E)), dev(torch.from_numpy(Rel)), dev(torch.from_numpy(hr))
+    norm = ops.batchnorm_stats(Eg, Rg, hrg)
+    x, y = E[hr[:, 0]].astype(np.float64), Rel[hr[:, 1]].astype(np.float64)
+    np.testing.assert_allclose(norm["h_a"].cpu().numpy(), x.mean(axis=0), rtol=1e-6)
+    np.testing.assert_allclose(norm["h_b"].cpu().numpy(), x.var(axis=0), rtol=1e-5)
+    np.testing.assert_allclose(norm["r_b"].cpu().numpy(), y.var(axis=0), rtol=1e-5)
+    with pytest.raises(ValueError):          # torch: "Expected more than 1 value per channel when training"
+        ops.batchnorm_stats(Eg, Rg, hrg[:1].contiguous())
+    bad = hr.copy()
+    bad[17, 0] = N
+    nb = ops.batchnorm_stats(Eg, Rg, dev(torch.from_numpy(bad)))
+    assert torch.isnan(nb["h_a"]).all() and torch.isnan(nb["r_b"]).all()
+    with pytest.raises(KgeError):            # the backward needs the statistics of at least two rows as well
+        ops.build_query_backward("DistMult", Eg, Rg, hrg[:1].contiguous(), torch.ones(1, d, device="cuda"), None,
+                                 torch.zeros_like(Eg), torch.zeros_like(Rg), norm=norm)
+
+
 def test_build_query_backward_norm_argument_checks(ops):
     from dicee_amd._lib import KgeError
     rng = np.random.default_rng(5)

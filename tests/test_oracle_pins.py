@@ -592,6 +592,36 @@ def test_query_builder_backward_through_the_normalisation_layers_vs_torch_autogr
             assert not any(k in extra for k in ("h_weight", "h_bias", "r_weight", "r_bias"))
 
 
+def test_batchnorm_training_mode_forward_running_statistics_and_backward_vs_torch():
+    """BatchNorm1d(affine=False).train(): the oracle's batch normalisation, the buffers the call leaves, and the
+    gradient through the batch statistics, against torch's module and autograd in float64."""
+    rng = np.random.default_rng(29)
+    N, R, B, d = 7, 3, 6, 8
+    E, Rel = rng.standard_normal((N, d)), rng.standard_normal((R, d))
+    hr = np.stack([rng.integers(0, N, B), rng.integers(0, R, B)], axis=1)
+    dQ = rng.standard_normal((B, d))
+    bn_h = torch.nn.BatchNorm1d(d, affine=False).double().train()
+    bn_r = torch.nn.BatchNorm1d(d, affine=False).double().train()
+    with torch.no_grad():
+        bn_h.running_mean.copy_(torch.from_numpy(rng.normal(0, 0.2, d)))
+        bn_h.running_var.copy_(torch.from_numpy(rng.uniform(0.5, 2.0, d)))
+    before = bn_h.running_mean.numpy().copy(), bn_h.running_var.numpy().copy()
+    Et, Rt = torch.tensor(E, requires_grad=True), torch.tensor(Rel, requires_grad=True)
+    h = bn_h(Et[torch.from_numpy(hr[:, 0])])
+    r = bn_r(Rt[torch.from_numpy(hr[:, 1])])
+    Q = h * r
+    norm = {"kind": "BatchNorm1dTrain", "eps": bn_h.eps}
+    np.testing.assert_allclose(Q.detach().numpy(), ko.build_query("DistMult", E, Rel, hr, norm=norm)[0],
+                               rtol=1e-12, atol=1e-12)
+    rm, rv = ko.batch_norm_running_update(E[hr[:, 0]], before[0], before[1], momentum=bn_h.momentum)
+    np.testing.assert_allclose(rm, bn_h.running_mean.numpy(), rtol=1e-12, atol=1e-14)
+    np.testing.assert_allclose(rv, bn_h.running_var.numpy(), rtol=1e-12, atol=1e-14)
+    (Q * torch.from_numpy(dQ)).sum().backward()
+    dE, dR = ko.build_query_backward_batch("DistMult", E, Rel, hr, dQ, norm=norm)
+    np.testing.assert_allclose(dE, Et.grad.numpy(), rtol=1e-6, atol=1e-7)
+    np.testing.assert_allclose(dR, Rt.grad.numpy(), rtol=1e-6, atol=1e-7)
+
+
 def test_bf16_round_vs_torch():
     rng = np.random.default_rng(13)
     x = np.concatenate([rng.normal(0, 1, 5000), rng.normal(0, 1e-20, 100), [0.0, -0.0, 1.0, 3.3895314e38]])
