@@ -23,10 +23,16 @@ struct QueryArgs {
   float* Q;
   float* bias;
   kge_norm_params norm;
+  kge_dropout_params drop;  // all masks null: no dropout
   int64_t B, N, R;
   int d, p, q, r, normalize_relation;
   int head_mode;  // pairs are (relation, tail) and Q is the head-direction query
 };
+
+// torch.nn.Dropout in training mode as a factor: 1 / (1 - rate) for a kept element, 0 for a dropped one (1 without a mask)
+__device__ __forceinline__ float drop_factor(const uint8_t* keep, int64_t idx, float scale) {
+  return keep ? (keep[idx] ? scale : 0.f) : 1.f;
+}
 
 template <int DT>
 __device__ __forceinline__ float load_elem(const void* base, int64_t row, int d, int k, const float* scale) {
@@ -80,8 +86,8 @@ __global__ void __launch_bounds__(64) build_query_kernel(QueryArgs a, int model)
     return;
   }
   for (int k = lane; k < d; k += 64) {
-    sh[k] = load_elem<EDT>(a.ent, h_id, d, k, a.ent_scale);
-    sr[k] = load_elem<RDT>(a.rel, r_id, d, k, nullptr);
+    sh[k] = load_elem<EDT>(a.ent, h_id, d, k, a.ent_scale) * drop_factor(a.drop.keep_h, b * d + k, a.drop.scale_in);
+    sr[k] = load_elem<RDT>(a.rel, r_id, d, k, nullptr) * drop_factor(a.drop.keep_r, b * d + k, a.drop.scale_in);
   }
   __syncthreads();
   if (a.norm.kind != KGE_NORM_NONE) {
@@ -91,7 +97,8 @@ __global__ void __launch_bounds__(64) build_query_kernel(QueryArgs a, int model)
   }
   float bias = 0.f;
   if (model == KGE_DISTMULT) {
-    for (int k = lane; k < d; k += 64) q[k] = sh[k] * sr[k];
+    for (int k = lane; k < d; k += 64)
+      q[k] = (sh[k] * sr[k]) * drop_factor(a.drop.keep_q, b * d + k, a.drop.scale_hidden);
   } else if (model == KGE_COMPLEX) {
     const int d2 = d >> 1;
     const float conj = a.head_mode ? -1.f : 1.f;
@@ -325,12 +332,15 @@ struct QueryBwdArgs {
   // here, [B, d] each, for the passes that need sums over the batch (null: every other mode)
   float* dy_h;
   float* dy_r;
+  kge_dropout_params drop;  // the masks of the forward (all null: none)
 };
 
-// One row through the backward of its normaliser: x the raw row, dy the gradient at the normalised row (both in LDS);
-// adds the gradient at the raw row to out[] and LayerNorm's parameter gradients to dw[] / db[].
+// One row through the backward of its normaliser: x the row the normaliser saw (after dropout, if any), dy the gradient
+// at the normalised row (both in LDS); adds the gradient at the raw row to out[] (through the row's dropout mask
+// `keep`, null: none) and LayerNorm's parameter gradients to dw[] / db[].
 __device__ void normalise_row_backward(const float* x, const float* dy, int d, int lane, int kind, float eps,
-                                       const float* a, const float* b, float* out, float* dw, float* db) {
+                                       const float* a, const float* b, float* out, float* dw, float* db,
+                                       const uint8_t* keep, float keep_scale) {
   if (kind == KGE_NORM_LAYERNORM) {
     // the statistics exactly as normalise_row forms them
     float s = 0.f;
@@ -353,12 +363,12 @@ __device__ void normalise_row_backward(const float* x, const float* dy, int d, i
     const float m1 = wave_sum(s1) / (float)d, m2 = wave_sum(s2) / (float)d;
     for (int k = lane; k < d; k += 64) {
       const float xh = (x[k] - mu) * inv, g = dy[k] * a[k];
-      atomicAdd(&out[k], inv * (g - m1 - xh * m2));
+      atomicAdd(&out[k], inv * (g - m1 - xh * m2) * drop_factor(keep, k, keep_scale));
       if (dw) atomicAdd(&dw[k], dy[k] * xh);
       if (db) atomicAdd(&db[k], dy[k]);
     }
   } else {  // BatchNorm1d with running statistics: an elementwise affine map
-    for (int k = lane; k < d; k += 64) atomicAdd(&out[k], dy[k] / sqrtf(b[k] + eps));
+    for (int k = lane; k < d; k += 64) atomicAdd(&out[k], dy[k] / sqrtf(b[k] + eps) * drop_factor(keep, k, keep_scale));
   }
 }
 
@@ -384,9 +394,9 @@ __global__ void __launch_bounds__(64) build_query_backward_kernel(QueryBwdArgs a
     return;
   }
   for (int k = lane; k < d; k += 64) {
-    sh[k] = a.ent[h_id * d + k];
-    sr[k] = a.rel[r_id * d + k];
-    sg[k] = a.dQ[b * d + k];
+    sh[k] = a.ent[h_id * d + k] * drop_factor(a.drop.keep_h, b * d + k, a.drop.scale_in);
+    sr[k] = a.rel[r_id * d + k] * drop_factor(a.drop.keep_r, b * d + k, a.drop.scale_in);
+    sg[k] = a.dQ[b * d + k] * drop_factor(a.drop.keep_q, b * d + k, a.drop.scale_hidden);
   }
   __syncthreads();
   if constexpr (NORM) {
@@ -398,11 +408,11 @@ __global__ void __launch_bounds__(64) build_query_backward_kernel(QueryBwdArgs a
   float* gr = a.d_rel + r_id * d;
   auto emit_h = [&](int k, float v) {
     if constexpr (NORM) sdh[k] = v;
-    else atomicAdd(&gh[k], v);
+    else atomicAdd(&gh[k], v * drop_factor(a.drop.keep_h, b * d + k, a.drop.scale_in));
   };
   auto emit_r = [&](int k, float v) {
     if constexpr (NORM) sdr[k] = v;
-    else atomicAdd(&gr[k], v);
+    else atomicAdd(&gr[k], v * drop_factor(a.drop.keep_r, b * d + k, a.drop.scale_in));
   };
   if (model == KGE_DISTMULT) {
     for (int k = lane; k < d; k += 64) {
@@ -460,7 +470,11 @@ __global__ void __launch_bounds__(64) build_query_backward_kernel(QueryBwdArgs a
           n = sn[g];
         } else {
           const float* raw = a.rel + r_id * d + 4 * g;
-          const float x0 = raw[0], x1 = raw[1], x2 = raw[2], x3 = raw[3];
+          const int64_t at = b * d + 4 * g;
+          const float x0 = raw[0] * drop_factor(a.drop.keep_r, at, a.drop.scale_in);
+          const float x1 = raw[1] * drop_factor(a.drop.keep_r, at + 1, a.drop.scale_in);
+          const float x2 = raw[2] * drop_factor(a.drop.keep_r, at + 2, a.drop.scale_in);
+          const float x3 = raw[3] * drop_factor(a.drop.keep_r, at + 3, a.drop.scale_in);
           n = sqrtf(x0 * x0 + x1 * x1 + x2 * x2 + x3 * x3);
         }
         const float y0 = sr[4 * g], y1 = sr[4 * g + 1], y2 = sr[4 * g + 2], y3 = sr[4 * g + 3];
@@ -607,8 +621,8 @@ __global__ void __launch_bounds__(64) build_query_backward_kernel(QueryBwdArgs a
     // the raw rows once more, and each gradient through its normaliser
     __syncthreads();
     for (int k = lane; k < d; k += 64) {
-      sh[k] = a.ent[h_id * d + k];
-      sr[k] = a.rel[r_id * d + k];
+      sh[k] = a.ent[h_id * d + k] * drop_factor(a.drop.keep_h, b * d + k, a.drop.scale_in);
+      sr[k] = a.rel[r_id * d + k] * drop_factor(a.drop.keep_r, b * d + k, a.drop.scale_in);
     }
     __syncthreads();
     if (a.dy_h) {
@@ -618,8 +632,10 @@ __global__ void __launch_bounds__(64) build_query_backward_kernel(QueryBwdArgs a
       }
       return;
     }
-    normalise_row_backward(sh, sdh, d, lane, a.norm.kind, a.norm.eps, a.norm.h_a, a.norm.h_b, gh, a.dn_h_a, a.dn_h_b);
-    normalise_row_backward(sr, sdr, d, lane, a.norm.kind, a.norm.eps, a.norm.r_a, a.norm.r_b, gr, a.dn_r_a, a.dn_r_b);
+    normalise_row_backward(sh, sdh, d, lane, a.norm.kind, a.norm.eps, a.norm.h_a, a.norm.h_b, gh, a.dn_h_a, a.dn_h_b,
+                           a.drop.keep_h ? a.drop.keep_h + b * d : nullptr, a.drop.scale_in);
+    normalise_row_backward(sr, sdr, d, lane, a.norm.kind, a.norm.eps, a.norm.r_a, a.norm.r_b, gr, a.dn_r_a, a.dn_r_b,
+                           a.drop.keep_r ? a.drop.keep_r + b * d : nullptr, a.drop.scale_in);
   }
 }
 
@@ -637,6 +653,7 @@ struct BnSumArgs {
   const float* dy_h;
   const float* dy_r;
   kge_norm_params norm;
+  kge_dropout_params drop;
   double* sums;
   int64_t B, N, R;
   int d;
@@ -665,7 +682,8 @@ __global__ void __launch_bounds__(256) bn_sums_kernel(BnSumArgs a) {
       continue;
     }
     if (f < d) {
-      const float x = a.ent[h_id * d + f], y = a.rel[r_id * d + f];
+      const float x = a.ent[h_id * d + f] * drop_factor(a.drop.keep_h, b * d + f, a.drop.scale_in);
+      const float y = a.rel[r_id * d + f] * drop_factor(a.drop.keep_r, b * d + f, a.drop.scale_in);
       if (GRAD) {
         const float gh = a.dy_h[b * d + f], gr = a.dy_r[b * d + f];
         s0 += (double)gh;
@@ -730,9 +748,11 @@ __global__ void __launch_bounds__(256) bn_backward_apply_kernel(BnSumArgs a, flo
   for (int64_t b = (int64_t)blockIdx.y * 4 + (threadIdx.x >> 6); b < a.B; b += 4 * (int64_t)gridDim.y) {
     const int64_t h_id = a.hr[2 * b], r_id = a.hr[2 * b + 1];
     if (h_id < 0 || h_id >= a.N || r_id < 0 || r_id >= a.R) continue;
-    const float xh = (a.ent[h_id * d + f] - mh) * ih, yh = (a.rel[r_id * d + f] - mr) * ir;
-    atomicAdd(&d_ent[h_id * d + f], (a.dy_h[b * d + f] - h1 - xh * h2) * ih);
-    atomicAdd(&d_rel[r_id * d + f], (a.dy_r[b * d + f] - r1 - yh * r2) * ir);
+    const float kh = drop_factor(a.drop.keep_h, b * d + f, a.drop.scale_in);
+    const float kr = drop_factor(a.drop.keep_r, b * d + f, a.drop.scale_in);
+    const float xh = (a.ent[h_id * d + f] * kh - mh) * ih, yh = (a.rel[r_id * d + f] * kr - mr) * ir;
+    atomicAdd(&d_ent[h_id * d + f], (a.dy_h[b * d + f] - h1 - xh * h2) * ih * kh);
+    atomicAdd(&d_rel[r_id * d + f], (a.dy_r[b * d + f] - r1 - yh * r2) * ir * kr);
   }
 }
 
@@ -896,7 +916,8 @@ int launch_build_query_flat(const QueryArgs& a, int rel_dtype, hipStream_t st) {
 
 template <int EDT>
 int launch_build_query(const QueryArgs& a, int model, int rel_dtype, hipStream_t st) {
-  if (a.norm.kind == KGE_NORM_NONE && a.B > 0) {
+  const bool dropout = a.drop.keep_h || a.drop.keep_r || a.drop.keep_q;
+  if (a.norm.kind == KGE_NORM_NONE && a.B > 0 && !dropout) {
     if (model == KGE_DISTMULT) return launch_build_query_flat<EDT, 1>(a, rel_dtype, st);
     if (model == KGE_COMPLEX) return launch_build_query_flat<EDT, 2>(a, rel_dtype, st);
     if (model == KGE_QMULT && (!a.normalize_relation || (a.d / 4) % 4 == 0)) return launch_build_query_flat<EDT, 4>(a, rel_dtype, st);
@@ -914,13 +935,27 @@ int launch_build_query(const QueryArgs& a, int model, int rel_dtype, hipStream_t
 }  // namespace
 }  // namespace kge
 
+namespace kge {
+namespace {
+// keep_q is DistMult's dropout on h * r (dicee/models/real.py:32); no other model of this path has one
+int check_dropout(const char* who, const kge_dropout_params* dp, int model) {
+  KGE_REQUIRE(!dp->keep_q || model == KGE_DISTMULT, KGE_ERR_INVALID, "%s: keep_q is DistMult's hidden dropout only", who);
+  KGE_REQUIRE(dp->scale_in >= 1.f && dp->scale_hidden >= 1.f && dp->scale_in < 1e30f && dp->scale_hidden < 1e30f,
+              KGE_ERR_INVALID, "%s: scales must be 1 / (1 - rate) with a rate in [0, 1), got %g and %g", who,
+              (double)dp->scale_in, (double)dp->scale_hidden);
+  return KGE_OK;
+}
+}  // namespace
+}  // namespace kge
+
 static int build_query_impl(int head_mode, int model, int p, int q, int r, const void* ent, int ent_dtype,
                             const float* ent_scale, const void* rel, int rel_dtype, const float* coeff_p,
                             const float* coeff_q, const float* coeff_r, int normalize_relation, const kge_norm_params* norm,
                             const int64_t* hr, int64_t B, int64_t d, int64_t N, int64_t R, float* Q, float* bias,
-                            void* stream) {
+                            void* stream, const kge_dropout_params* dropout = nullptr) {
   using namespace kge;
   clear_error();
+  KGE_REQUIRE(!head_mode || !dropout, KGE_ERR_UNSUPPORTED, "kge_build_query_head: no dropout in the head direction");
   KGE_REQUIRE(!head_mode || !norm || norm->kind == KGE_NORM_NONE, KGE_ERR_UNSUPPORTED,
               "kge_build_query_head: a normalised head row is not a row of the table; only normalisation 'none'");
   KGE_REQUIRE(B >= 0 && N > 0 && R > 0, KGE_ERR_INVALID, "kge_build_query: B=%lld N=%lld R=%lld", (long long)B,
@@ -981,6 +1016,11 @@ static int build_query_impl(int head_mode, int model, int p, int q, int r, const
                 "kge_build_query: normalisation parameters missing");
     a.norm = *norm;
   }
+  a.drop = kge_dropout_params{nullptr, nullptr, nullptr, 1.f, 1.f};
+  if (dropout) {
+    if (int rc = check_dropout("kge_build_query_dropout", dropout, model)) return rc;
+    a.drop = *dropout;
+  }
   a.B = B;
   a.N = N;
   a.R = R;
@@ -1025,6 +1065,16 @@ extern "C" int kge_build_query_decal(int head, int p, int q, int r, const void* 
                           coeff_r, 0, norm, pairs, B, d, N, R, Q, bias, stream);
 }
 
+extern "C" int kge_build_query_dropout(int model, int p, int q, int r, const void* ent, int ent_dtype,
+                                       const float* ent_scale, const void* rel, int rel_dtype, const float* coeff_p,
+                                       const float* coeff_q, const float* coeff_r, int normalize_relation,
+                                       const kge_norm_params* norm, const kge_dropout_params* dropout,
+                                       const int64_t* hr, int64_t B, int64_t d, int64_t N, int64_t R, float* Q,
+                                       float* bias, void* stream) {
+  return build_query_impl(0, model, p, q, model == KGE_DECAL ? r : 0, ent, ent_dtype, ent_scale, rel, rel_dtype, coeff_p,
+                          coeff_q, coeff_r, normalize_relation, norm, hr, B, d, N, R, Q, bias, stream, dropout);
+}
+
 extern "C" size_t kge_batchnorm_workspace_bytes(int64_t B, int64_t d);
 
 namespace kge {
@@ -1034,7 +1084,8 @@ int build_query_backward_impl(int model, int p, int q, int r, const float* ent, 
                               const kge_norm_params* norm, const kge_norm_grads* dnorm, const int64_t* hr, int64_t B,
                               int64_t d, int64_t N, int64_t R, const float* dQ, const float* dbias, float* d_ent,
                               float* d_rel, float* d_coeff_p, float* d_coeff_q, float* d_coeff_r, void* stream,
-                              bool batch_stats = false, void* workspace = nullptr, size_t workspace_bytes = 0) {
+                              const kge_dropout_params* dropout = nullptr, bool batch_stats = false,
+                              void* workspace = nullptr, size_t workspace_bytes = 0) {
   clear_error();
   KGE_REQUIRE(B >= 0 && N > 0 && R > 0, KGE_ERR_INVALID, "kge_build_query_backward: B=%lld N=%lld R=%lld", (long long)B,
               (long long)N, (long long)R);
@@ -1091,6 +1142,11 @@ int build_query_backward_impl(int model, int p, int q, int r, const float* ent, 
   a.norm.h_a = a.norm.h_b = a.norm.r_a = a.norm.r_b = nullptr;
   a.dn_h_a = a.dn_h_b = a.dn_r_a = a.dn_r_b = nullptr;
   a.dy_h = a.dy_r = nullptr;
+  a.drop = kge_dropout_params{nullptr, nullptr, nullptr, 1.f, 1.f};
+  if (dropout) {
+    if (int rc = check_dropout("kge_build_query_backward", dropout, model)) return rc;
+    a.drop = *dropout;
+  }
   hipStream_t st = (hipStream_t)stream;
   if (batch_stats) {
     KGE_REQUIRE(norm && norm->kind == KGE_NORM_BATCHNORM1D && norm->h_a && norm->h_b && norm->r_a && norm->r_b,
@@ -1113,7 +1169,7 @@ int build_query_backward_impl(int model, int p, int q, int r, const float* ent, 
     const size_t lds_bytes = (5 * (size_t)d + (size_t)(d + 3) / 4) * sizeof(float);
     hipLaunchKernelGGL(build_query_backward_kernel<true>, dim3((unsigned)B), dim3(64), lds_bytes, st, a, model);
     KGE_LAUNCH_CHECK("build_query_backward_kernel");
-    BnSumArgs sa{ent, rel, hr, a.dy_h, a.dy_r, *norm, sums, B, N, R, (int)d};
+    BnSumArgs sa{ent, rel, hr, a.dy_h, a.dy_r, *norm, a.drop, sums, B, N, R, (int)d};
     const unsigned slices = (unsigned)((B + 63) / 64 < 64 ? (B + 63) / 64 : 64);
     dim3 grid((unsigned)((d + 63) / 64), slices);
     hipLaunchKernelGGL(bn_sums_kernel<true>, grid, dim3(256), 0, st, sa);
@@ -1158,11 +1214,17 @@ extern "C" size_t kge_batchnorm_workspace_bytes(int64_t B, int64_t d) {
 }
 
 extern "C" int kge_batchnorm_stats(const float* ent, const float* rel, const int64_t* hr, int64_t B, int64_t d, int64_t N,
-                                   int64_t R, float momentum, float* h_mean, float* h_var, float* r_mean, float* r_var,
-                                   float* run_h_mean, float* run_h_var, float* run_r_mean, float* run_r_var,
-                                   void* workspace, size_t workspace_bytes, void* stream) {
+                                   int64_t R, const kge_dropout_params* dropout, float momentum, float* h_mean,
+                                   float* h_var, float* r_mean, float* r_var, float* run_h_mean, float* run_h_var,
+                                   float* run_r_mean, float* run_r_var, void* workspace, size_t workspace_bytes,
+                                   void* stream) {
   using namespace kge;
   clear_error();
+  kge_dropout_params drop{nullptr, nullptr, nullptr, 1.f, 1.f};
+  if (dropout) {
+    if (int rc = check_dropout("kge_batchnorm_stats", dropout, KGE_DISTMULT)) return rc;
+    drop = *dropout;
+  }
   KGE_REQUIRE(N > 0 && R > 0 && d >= 1 && d <= 8192, KGE_ERR_INVALID, "kge_batchnorm_stats: N=%lld R=%lld d=%lld",
               (long long)N, (long long)R, (long long)d);
   KGE_REQUIRE(B >= 2 && B <= 0x7fffffff, KGE_ERR_INVALID,
@@ -1178,7 +1240,7 @@ extern "C" int kge_batchnorm_stats(const float* ent, const float* rel, const int
   hipLaunchKernelGGL(bn_zero_kernel, dim3((unsigned)((4 * d + 255) / 256)), dim3(256), 0, st, sums, (int)(4 * d));
   KGE_LAUNCH_CHECK("bn_zero_kernel");
   kge_norm_params none{};
-  BnSumArgs sa{ent, rel, hr, nullptr, nullptr, none, sums, B, N, R, (int)d};
+  BnSumArgs sa{ent, rel, hr, nullptr, nullptr, none, drop, sums, B, N, R, (int)d};
   const unsigned slices = (unsigned)((B + 63) / 64 < 64 ? (B + 63) / 64 : 64);
   hipLaunchKernelGGL(bn_sums_kernel<false>, dim3((unsigned)((d + 63) / 64), slices), dim3(256), 0, st, sa);
   KGE_LAUNCH_CHECK("bn_sums_kernel");
@@ -1191,13 +1253,14 @@ extern "C" int kge_batchnorm_stats(const float* ent, const float* rel, const int
 extern "C" int kge_build_query_backward_batchnorm(int model, int p, int q, int r, const float* ent, const float* rel,
                                                   const float* coeff_p, const float* coeff_q, const float* coeff_r,
                                                   int normalize_relation, const kge_norm_params* norm,
-                                                  const int64_t* hr, int64_t B, int64_t d, int64_t N, int64_t R,
+                                                  const kge_dropout_params* dropout, const int64_t* hr, int64_t B,
+                                                  int64_t d, int64_t N, int64_t R,
                                                   const float* dQ, const float* dbias, float* d_ent, float* d_rel,
                                                   float* d_coeff_p, float* d_coeff_q, float* d_coeff_r,
                                                   void* workspace, size_t workspace_bytes, void* stream) {
   return kge::build_query_backward_impl(model, p, q, r, ent, rel, coeff_p, coeff_q, coeff_r, normalize_relation, norm,
                                         nullptr, hr, B, d, N, R, dQ, dbias, d_ent, d_rel, d_coeff_p, d_coeff_q,
-                                        d_coeff_r, stream, true, workspace, workspace_bytes);
+                                        d_coeff_r, stream, dropout, true, workspace, workspace_bytes);
 }
 
 extern "C" int kge_build_query_backward(int model, int p, int q, int r, const float* ent, const float* rel,
@@ -1213,11 +1276,12 @@ extern "C" int kge_build_query_backward(int model, int p, int q, int r, const fl
 extern "C" int kge_build_query_backward_norm(int model, int p, int q, int r, const float* ent, const float* rel,
                                              const float* coeff_p, const float* coeff_q, const float* coeff_r,
                                              int normalize_relation, const kge_norm_params* norm,
-                                             const kge_norm_grads* dnorm, const int64_t* hr, int64_t B, int64_t d,
+                                             const kge_norm_grads* dnorm, const kge_dropout_params* dropout,
+                                             const int64_t* hr, int64_t B, int64_t d,
                                              int64_t N, int64_t R, const float* dQ, const float* dbias, float* d_ent,
                                              float* d_rel, float* d_coeff_p, float* d_coeff_q, float* d_coeff_r,
                                              void* stream) {
   return kge::build_query_backward_impl(model, p, q, r, ent, rel, coeff_p, coeff_q, coeff_r, normalize_relation, norm,
                                         dnorm, hr, B, d, N, R, dQ, dbias, d_ent, d_rel, d_coeff_p, d_coeff_q, d_coeff_r,
-                                        stream);
+                                        stream, dropout);
 }

@@ -22,6 +22,11 @@ class NormParams(ctypes.Structure):
                 ("h_a", _vp), ("h_b", _vp), ("r_a", _vp), ("r_b", _vp)]
 
 
+class DropoutParams(ctypes.Structure):
+    _fields_ = [("keep_h", _vp), ("keep_r", _vp), ("keep_q", _vp), ("scale_in", ctypes.c_float),
+                ("scale_hidden", ctypes.c_float)]
+
+
 class NormGrads(ctypes.Structure):
     _fields_ = [("h_a", _vp), ("h_b", _vp), ("r_a", _vp), ("r_b", _vp)]
 
@@ -37,15 +42,20 @@ SIGNATURES = {
                                        ctypes.POINTER(NormParams), _vp, _c_i64, _c_i64, _c_i64, _c_i64, _vp, _vp, _vp]),
     "kge_build_query_backward": (_c_int, [_c_int, _c_int, _c_int, _c_int, _vp, _vp, _vp, _vp, _vp, _c_int, _vp, _c_i64,
                                           _c_i64, _c_i64, _c_i64, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
+    "kge_build_query_dropout": (_c_int, [_c_int, _c_int, _c_int, _c_int, _vp, _c_int, _vp, _vp, _c_int, _vp, _vp, _vp,
+                                         _c_int, ctypes.POINTER(NormParams), ctypes.POINTER(DropoutParams), _vp, _c_i64,
+                                         _c_i64, _c_i64, _c_i64, _vp, _vp, _vp]),
     "kge_build_query_backward_norm": (_c_int, [_c_int, _c_int, _c_int, _c_int, _vp, _vp, _vp, _vp, _vp, _c_int,
-                                               ctypes.POINTER(NormParams), ctypes.POINTER(NormGrads), _vp, _c_i64,
-                                               _c_i64, _c_i64, _c_i64, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
+                                               ctypes.POINTER(NormParams), ctypes.POINTER(NormGrads),
+                                               ctypes.POINTER(DropoutParams), _vp, _c_i64, _c_i64, _c_i64, _c_i64, _vp,
+                                               _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     "kge_batchnorm_workspace_bytes": (_sz, [_c_i64, _c_i64]),
-    "kge_batchnorm_stats": (_c_int, [_vp, _vp, _vp, _c_i64, _c_i64, _c_i64, _c_i64, _c_f, _vp, _vp, _vp, _vp, _vp, _vp,
-                                     _vp, _vp, _vp, _sz, _vp]),
+    "kge_batchnorm_stats": (_c_int, [_vp, _vp, _vp, _c_i64, _c_i64, _c_i64, _c_i64, ctypes.POINTER(DropoutParams), _c_f,
+                                     _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
     "kge_build_query_backward_batchnorm": (_c_int, [_c_int, _c_int, _c_int, _c_int, _vp, _vp, _vp, _vp, _vp, _c_int,
-                                                    ctypes.POINTER(NormParams), _vp, _c_i64, _c_i64, _c_i64, _c_i64,
-                                                    _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
+                                                    ctypes.POINTER(NormParams), ctypes.POINTER(DropoutParams), _vp,
+                                                    _c_i64, _c_i64, _c_i64, _c_i64, _vp, _vp, _vp, _vp, _vp, _vp, _vp,
+                                                    _vp, _sz, _vp]),
     "kge_scores": (_c_int, [_vp, _vp, _vp, _c_int, _vp, _c_i64, _c_i64, _c_i64, _vp, _c_i64, _vp]),
     "kge_triple_scores": (_c_int, [_vp, _vp, _vp, _c_int, _vp, _c_i64, _c_i64, _c_i64, _vp, _vp, _vp]),
     "kge_sample_scores": (_c_int, [_vp, _vp, _vp, _c_int, _vp, _c_i64, _c_i64, _c_i64, _vp, _c_i64, _vp, _vp]),

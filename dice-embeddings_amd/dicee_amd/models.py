@@ -5,11 +5,12 @@ Parameter names follow dicee so that a dicee ``model.pt`` state_dict loads uncha
 ``q_coefficients.weight``, ``normalize_*_embeddings.*``): dicee/models/base_model.py:121-176,
 dicee/models/clifford.py:4-28.
 
-Normalisation layers follow the module's mode: LayerNorm is the same in both; BatchNorm1d normalises with its
-running statistics in eval mode and with the statistics of the batch in training mode (moving the running
-statistics, as torch does).  Dropout is the identity (base_model.py:149-151 in eval mode): a model in training
-mode whose dropout rates are not zero refuses to score (the reference would drop elements there) instead of
-silently scoring without dropout.
+Layers follow the module's mode.  LayerNorm is the same in both; BatchNorm1d normalises with its running
+statistics in eval mode and with the statistics of the batch in training mode (moving the running statistics, as
+torch does).  Dropout (base_model.py:149-151) is the identity in eval mode; in training mode with
+``input_dropout_rate`` > 0 the looked-up head and relation rows, and DistMult's ``h * r``, are dropped element by
+element with masks drawn from torch's generator on the device (the distribution of torch.nn.Dropout, not its
+stream: no two implementations share that).
 """
 import torch
 
@@ -131,21 +132,31 @@ class BaseKGE(torch.nn.Module):
         self._refresh_storage()
         return self._rel_table if self._rel_table is not None else self.relation_embeddings.weight.detach()
 
-    def _refuse_dropout_in_training(self):
-        """The reference applies Dropout to the gathered rows (base_model.py:381-383) and to the interaction
-        (e.g. real.py:32) whenever the module is in training mode; this path has no dropout."""
-        if self.training and (self.input_dropout_rate > 0.0 or self.hidden_dropout_rate > 0.0):
-            raise NotImplementedError(
-                f"{self.name} is in training mode with input_dropout_rate={self.input_dropout_rate}, "
-                f"hidden_dropout_rate={self.hidden_dropout_rate}: the accelerated path has no dropout; "
-                "call model.eval() or set the rates to zero")
+    def _draw_dropout(self, B, device, rows=True):
+        """The masks one training-mode forward over B pairs applies: ``input_dp_ent_real`` on the head rows and
+        ``input_dp_rel_real`` on the relation rows (base_model.py:381-383), and for DistMult ``hidden_dropout`` on
+        ``h * r`` (real.py:32), all three built with ``input_dropout_rate`` (base_model.py:149-151; the models of this
+        path never read ``hidden_dropout_rate``).  None in eval mode or with a rate of zero."""
+        rate = self.input_dropout_rate
+        if not self.training or rate <= 0.0:
+            return None
+        if rate >= 1.0:
+            raise ValueError("a dropout rate of 1 leaves nothing")
+        d = self.embedding_dim
+        drop = {"scale_in": 1.0 / (1.0 - rate), "scale_hidden": 1.0 / (1.0 - rate)}
+        if rows:
+            drop["keep_h"] = (torch.rand((B, d), device=device) >= rate).to(torch.uint8)
+            drop["keep_r"] = (torch.rand((B, d), device=device) >= rate).to(torch.uint8)
+        if self.name == "DistMult":
+            drop["keep_q"] = (torch.rand((B, d), device=device) >= rate).to(torch.uint8)
+        return drop if len(drop) > 2 else None
 
     # ------------------------------------------------------------------ query construction
-    def _norm_params(self, x=None):
+    def _norm_params(self, x=None, dropout=None):
         """The normalisation layer between the lookups and the interaction, as the kernels take it.  BatchNorm1d in
         training mode normalises with the statistics of the batch ``x`` [B,2] itself and moves its running
         statistics towards them (torch.nn.BatchNorm1d; base_model.py:289-294 applied at :381-383): every call with
-        a batch is one such forward."""
+        a batch is one such forward.  ``dropout``: the masks of this forward (the layer sees the rows after dropout)."""
         nh, nr = self.normalize_head_entity_embeddings, self.normalize_relation_embeddings
         if isinstance(nh, torch.nn.LayerNorm):
             return {"kind": "LayerNorm", "eps": nh.eps, "h_a": nh.weight.detach(), "h_b": nh.bias.detach(),
@@ -162,7 +173,8 @@ class BaseKGE(torch.nn.Module):
                 if nh.track_running_stats and nh.running_mean is not None:
                     running = {"h_mean": nh.running_mean, "h_var": nh.running_var, "r_mean": nr.running_mean,
                                "r_var": nr.running_var}
-                norm = ops.batchnorm_stats(E, self._rel(), pairs, eps=nh.eps, momentum=nh.momentum, running=running)
+                norm = ops.batchnorm_stats(E, self._rel(), pairs, eps=nh.eps, momentum=nh.momentum, running=running,
+                                           dropout=dropout)
                 if running is not None:
                     nh.num_batches_tracked += 1
                     nr.num_batches_tracked += 1
@@ -174,18 +186,21 @@ class BaseKGE(torch.nn.Module):
     def _query_kwargs(self):
         return {}
 
-    def query(self, x, heads=False, norm=_FROM_MODEL):
+    def query(self, x, heads=False, norm=_FROM_MODEL, dropout=_FROM_MODEL):
         """(Q [B,d], bias [B]) for ``x`` [B,2]: gather + interaction
         (get_head_relation_representation, base_model.py:377-384, then the model's elementwise part).
         ``heads=True``: ``x`` holds (relation, tail) pairs and ``Q @ E^T`` scores every entity as the head of
         (x, r, t): what ``forward_triples`` gives triple by triple (base_model.py:346-362)."""
-        self._refuse_dropout_in_training()
         E, scale = self.table()
         x = x.to(device=E.device, dtype=torch.int64).contiguous()
+        if dropout is _FROM_MODEL:
+            dropout = self._draw_dropout(x.shape[0], E.device)
+        if heads and dropout is not None:
+            raise NotImplementedError("head-direction queries in training mode with dropout are not part of this path")
         if norm is _FROM_MODEL:
-            norm = self._norm_params(None if heads else x)
+            norm = self._norm_params(None if heads else x, dropout)
         return ops.build_query(self.name if self.name != "CKeci" else "Keci", E, self._rel(), x, ent_scale=scale,
-                               norm=norm, head=heads, **self._query_kwargs())
+                               norm=norm, head=heads, dropout=dropout, **self._query_kwargs())
 
     # ------------------------------------------------------------------ reference call surface
     def forward(self, x, y_idx=None):
@@ -242,13 +257,14 @@ class BaseKGE(torch.nn.Module):
         return ops.scores(Q, bias, E, scale)
 
     def k_vs_all_score(self, emb_h, emb_r, emb_E):
-        """Scores from already gathered rows: [B,d],[B,d],[N,d] -> [B,N]."""
-        self._refuse_dropout_in_training()
+        """Scores from already gathered rows: [B,d],[B,d],[N,d] -> [B,N] (in training mode DistMult drops elements of
+        ``h * r`` here, real.py:32; the rows themselves are the caller's)."""
         B = emb_h.shape[0]
         idx = torch.arange(B, device=emb_h.device, dtype=torch.int64)
         hr = torch.stack([idx, idx], dim=1).contiguous()
         Q, bias = ops.build_query(self.name if self.name != "CKeci" else "Keci", emb_h.contiguous().float(),
-                                  emb_r.contiguous().float(), hr, **self._query_kwargs())
+                                  emb_r.contiguous().float(), hr, dropout=self._draw_dropout(B, emb_h.device, rows=False),
+                                  **self._query_kwargs())
         return ops.scores(Q, bias, emb_E.contiguous().float())
 
     def get_embeddings(self):
@@ -288,12 +304,12 @@ class BaseKGE(torch.nn.Module):
         rows = csr.rows_for(x.to(device=E.device, dtype=torch.int64))
         return ops.bce_multihot(Q, bias, E, scale, rows, csr.row_ptr, csr.col, label_smoothing)[0]
 
-    def kvsall_bce_backward(self, x, csr, label_smoothing=0.0, grad_out=1.0, norm=_FROM_MODEL):
+    def kvsall_bce_backward(self, x, csr, label_smoothing=0.0, grad_out=1.0, norm=_FROM_MODEL, dropout=_FROM_MODEL):
         """The same step with its backward through the scores: ``(loss, dQ [B,d], dbias [B], dE [N,d])`` where
         ``dQ`` / ``dbias`` are the gradients at the query vectors and per-query biases of ``self.query(x)`` and ``dE``
         the gradient the contraction sends to the entity table (fp32 tables only).  What
         ``loss_batch.backward()`` computes for the ``torch.mm`` / ``einsum`` and the loss of the reference's step."""
-        Q, bias = self.query(x, norm=norm)
+        Q, bias = self.query(x, norm=norm, dropout=dropout)
         E, scale = self.table()
         if scale is not None:
             raise TypeError("the backward needs an fp32 entity table")
@@ -309,20 +325,22 @@ class BaseKGE(torch.nn.Module):
         for fp32 tables.  With ``normalization='LayerNorm'`` the gradient passes through both normalisers and their
         weights and biases receive theirs (``normalize_head_entity_embeddings.weight`` ...); with ``'BatchNorm1d'``
         it passes through the statistics of the batch in training mode (which also moves the running statistics, once)
-        and through the running statistics in eval mode."""
+        and through the running statistics in eval mode.  In training mode with ``input_dropout_rate`` > 0 one set of
+        masks is drawn for the step and used by its forward and its backward."""
         E, scale = self.table()
         if scale is not None or E.dtype != torch.float32:
             raise TypeError("the backward needs an fp32 entity table")
         x = x.to(device=E.device, dtype=torch.int64).contiguous()
-        norm = self._norm_params(x)
-        loss, dQ, dbias, dE = self.kvsall_bce_backward(x, csr, label_smoothing, norm=norm)
+        dropout = self._draw_dropout(x.shape[0], E.device)
+        norm = self._norm_params(x, dropout)
+        loss, dQ, dbias, dE = self.kvsall_bce_backward(x, csr, label_smoothing, norm=norm, dropout=dropout)
         rel = self._rel()
         dR = torch.zeros_like(rel)
         name = self.name if self.name != "CKeci" else "Keci"
         dnorm = None
         if norm is not None and norm["kind"] == "LayerNorm":
             dnorm = {k: torch.zeros_like(norm[k], dtype=torch.float32) for k in ("h_a", "h_b", "r_a", "r_b")}
-        dcoeff = ops.build_query_backward(name, E, rel, x, dQ, dbias, dE, dR, norm=norm, dnorm=dnorm,
+        dcoeff = ops.build_query_backward(name, E, rel, x, dQ, dbias, dE, dR, norm=norm, dnorm=dnorm, dropout=dropout,
                                           **self._query_kwargs())
         grads = {"entity_embeddings.weight": dE, "relation_embeddings.weight": dR}
         if dnorm is not None:

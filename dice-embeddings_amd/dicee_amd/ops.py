@@ -66,10 +66,32 @@ def _norm_struct(norm):
     return s, keep
 
 
+def _dropout_struct(dropout, B, d):
+    """dropout: None or dict with any of ``keep_h, keep_r, keep_q`` ([B,d] uint8 / bool GPU tensors, nonzero = keep)
+    and ``scale_in`` / ``scale_hidden`` (1 / (1 - rate))."""
+    if dropout is None:
+        return None, ()
+    keep = []
+    for k in ("keep_h", "keep_r", "keep_q"):
+        t = dropout.get(k)
+        if t is not None:
+            if t.dtype == torch.bool:
+                t = t.to(torch.uint8)
+            if t.dtype != torch.uint8 or tuple(t.shape) != (B, d):
+                raise TypeError(f"dropout mask {k} must be a [B, d] uint8 or bool tensor")
+            t = t.contiguous()
+            _require_gpu(t)
+        keep.append(t)
+    s = _lib.DropoutParams(*[t.data_ptr() if t is not None else None for t in keep],
+                           float(dropout.get("scale_in", 1.0)), float(dropout.get("scale_hidden", 1.0)))
+    return s, tuple(keep)
+
+
 def build_query(model, ent, rel, hr, *, ent_scale=None, p=0, q=0, r=0, coeff_p=None, coeff_q=None, coeff_r=None,
-                normalize_relation=True, norm=None, head=False):
+                normalize_relation=True, norm=None, head=False, dropout=None):
     """(Q [B,d] fp32, bias [B] fp32) with ``forward_k_vs_all(x) == Q @ E^T + bias[:, None]``.
-    ``head=True``: ``hr`` holds (relation, tail) pairs and ``Q @ E^T`` scores every entity as the head."""
+    ``head=True``: ``hr`` holds (relation, tail) pairs and ``Q @ E^T`` scores every entity as the head.
+    ``dropout``: the masks of a training-mode forward (``_dropout_struct``)."""
     lib = _lib.load()
     _require_gpu(ent, rel, hr, ent_scale, coeff_p, coeff_q, coeff_r)
     if hr.dtype != torch.int64 or hr.dim() != 2 or hr.shape[1] != 2:
@@ -80,6 +102,18 @@ def build_query(model, ent, rel, hr, *, ent_scale=None, p=0, q=0, r=0, coeff_p=N
     Q = torch.empty((B, d), dtype=torch.float32, device=ent.device)
     bias = torch.empty((B,), dtype=torch.float32, device=ent.device)
     ns, keep = _norm_struct(norm)
+    if dropout is not None:
+        if head:
+            raise ValueError("no dropout in the head direction")
+        ds, dkeep = _dropout_struct(dropout, B, d)
+        rc = lib.kge_build_query_dropout(MODEL_IDS[model], int(p), int(q), int(r), _ptr(ent), _table_dtype(ent),
+                                         _ptr(ent_scale), _ptr(rel), _table_dtype(rel), _ptr(coeff_p), _ptr(coeff_q),
+                                         _ptr(coeff_r), int(bool(normalize_relation)),
+                                         ctypes.byref(ns) if ns is not None else None, ctypes.byref(ds), _ptr(hr), B, d,
+                                         N, R, _ptr(Q), _ptr(bias), _stream())
+        _lib.check(rc)
+        del keep, dkeep
+        return Q, bias
     if model == "DeCaL":
         rc = lib.kge_build_query_decal(int(bool(head)), int(p), int(q), int(r), _ptr(ent), _table_dtype(ent),
                                        _ptr(ent_scale), _ptr(rel), _table_dtype(rel), _ptr(coeff_p), _ptr(coeff_q),
@@ -97,7 +131,7 @@ def build_query(model, ent, rel, hr, *, ent_scale=None, p=0, q=0, r=0, coeff_p=N
     return Q, bias
 
 
-def batchnorm_stats(ent, rel, hr, *, eps=1e-5, momentum=0.1, running=None):
+def batchnorm_stats(ent, rel, hr, *, eps=1e-5, momentum=0.1, running=None, dropout=None):
     """The normalisation layer ``BatchNorm1d(affine=False)`` applies to THIS batch in training mode: a ``norm`` dict
     for ``build_query`` holding the mean and biased variance, per feature, of the looked-up head rows and relation
     rows.  ``running``: dict with ``h_mean, h_var, r_mean, r_var`` ([d] fp32 GPU tensors, the modules' buffers),
@@ -120,16 +154,19 @@ def batchnorm_stats(ent, rel, hr, *, eps=1e-5, momentum=0.1, running=None):
                 raise TypeError("running statistics must be contiguous fp32 tensors of d elements")
         _require_gpu(*run)
     ws = torch.empty((4 * d,), dtype=torch.float64, device=ent.device)
-    rc = lib.kge_batchnorm_stats(_ptr(ent), _ptr(rel), _ptr(hr), B, d, N, R, float(momentum), _ptr(out[0]), _ptr(out[1]),
+    ds, dkeep = _dropout_struct(dropout, B, d)
+    rc = lib.kge_batchnorm_stats(_ptr(ent), _ptr(rel), _ptr(hr), B, d, N, R,
+                                 ctypes.byref(ds) if ds is not None else None, float(momentum), _ptr(out[0]), _ptr(out[1]),
                                  _ptr(out[2]), _ptr(out[3]), _ptr(run[0]), _ptr(run[1]), _ptr(run[2]), _ptr(run[3]),
                                  _ptr(ws), ws.numel() * 8, _stream())
     _lib.check(rc)
+    del dkeep
     return {"kind": "BatchNorm1d", "eps": float(eps), "h_a": out[0], "h_b": out[1], "r_a": out[2], "r_b": out[3],
             "batch": True}
 
 
 def build_query_backward(model, ent, rel, hr, dQ, dbias, d_ent, d_rel, *, p=0, q=0, r=0, coeff_p=None, coeff_q=None,
-                         coeff_r=None, normalize_relation=True, norm=None, dnorm=None):
+                         coeff_r=None, normalize_relation=True, norm=None, dnorm=None, dropout=None):
     """Adds the gradients that ``dQ`` [B,d] / ``dbias`` [B] send back through ``build_query`` into ``d_ent`` [N,d]
     and ``d_rel`` [R,d] (fp32, caller-initialised); returns the gradients of the Clifford coefficients
     ``(d_coeff_p, d_coeff_q, d_coeff_r)`` (None where the model has none).  ``norm``: the normalisation layer of
@@ -143,18 +180,20 @@ def build_query_backward(model, ent, rel, hr, dQ, dbias, d_ent, d_rel, *, p=0, q
             raise TypeError("build_query_backward needs contiguous fp32 tensors")
     B, (N, d), R = hr.shape[0], ent.shape, rel.shape[0]
     outs = [torch.zeros_like(c) if c is not None else None for c in (coeff_p, coeff_q, coeff_r)]
+    ds, dkeep = _dropout_struct(dropout, B, d)
+    dsp = ctypes.byref(ds) if ds is not None else None
     if norm is not None and norm.get("batch"):
         ns, keep = _norm_struct(norm)
         nbytes = lib.kge_batchnorm_workspace_bytes(B, d)
         ws = torch.empty(((nbytes + 7) // 8,), dtype=torch.float64, device=ent.device)
         rc = lib.kge_build_query_backward_batchnorm(
             MODEL_IDS[model], int(p), int(q), int(r), _ptr(ent), _ptr(rel), _ptr(coeff_p), _ptr(coeff_q), _ptr(coeff_r),
-            int(bool(normalize_relation)), ctypes.byref(ns), _ptr(hr), B, d, N, R, _ptr(dQ), _ptr(dbias), _ptr(d_ent),
+            int(bool(normalize_relation)), ctypes.byref(ns), dsp, _ptr(hr), B, d, N, R, _ptr(dQ), _ptr(dbias), _ptr(d_ent),
             _ptr(d_rel), _ptr(outs[0]), _ptr(outs[1]), _ptr(outs[2]), _ptr(ws), ws.numel() * 8, _stream())
         _lib.check(rc)
         del keep
         return tuple(outs)
-    if norm is not None:
+    if norm is not None or ds is not None:
         ns, keep = _norm_struct(norm)
         gs = None
         if dnorm:
@@ -166,8 +205,9 @@ def build_query_backward(model, ent, rel, hr, dQ, dbias, d_ent, d_rel, *, p=0, q
                                   for k in ("h_a", "h_b", "r_a", "r_b")])
         rc = lib.kge_build_query_backward_norm(
             MODEL_IDS[model], int(p), int(q), int(r), _ptr(ent), _ptr(rel), _ptr(coeff_p), _ptr(coeff_q), _ptr(coeff_r),
-            int(bool(normalize_relation)), ctypes.byref(ns), ctypes.byref(gs) if gs is not None else None, _ptr(hr), B, d,
-            N, R, _ptr(dQ), _ptr(dbias), _ptr(d_ent), _ptr(d_rel), _ptr(outs[0]), _ptr(outs[1]), _ptr(outs[2]), _stream())
+            int(bool(normalize_relation)), ctypes.byref(ns) if ns is not None else None,
+            ctypes.byref(gs) if gs is not None else None, dsp, _ptr(hr), B, d, N, R, _ptr(dQ), _ptr(dbias), _ptr(d_ent),
+            _ptr(d_rel), _ptr(outs[0]), _ptr(outs[1]), _ptr(outs[2]), _stream())
         _lib.check(rc)
         del keep
         return tuple(outs)

@@ -73,6 +73,20 @@ typedef struct kge_norm_grads {
   float* r_b;
 } kge_norm_grads;
 
+/* torch.nn.Dropout in training mode on the looked-up rows (dicee/models/base_model.py:149-151 applied at :381-383,
+ * before the normalisation layer) and, for DistMult, on h * r (dicee/models/real.py:32), with the masks given by
+ * the caller: keep_* [B,d] bytes, 1 = the element is kept (and multiplied by the scale), 0 = it is zeroed; a NULL
+ * mask means no dropout at that place.  scale_in = 1 / (1 - input_dropout_rate); scale_hidden the same for the rate
+ * of the module behind real.py:32 (base_model.py:151 builds it with input_dropout_rate as well).  The backward
+ * calls take the masks of their forward. */
+typedef struct kge_dropout_params {
+  const uint8_t* keep_h;
+  const uint8_t* keep_r;
+  const uint8_t* keep_q; /* DistMult only */
+  float scale_in;
+  float scale_hidden;
+} kge_dropout_params;
+
 /* Text of the last error raised on the calling thread ("" if none). */
 const char* kge_last_error(void);
 
@@ -135,6 +149,16 @@ int kge_build_query_decal(int head, int p, int q, int r, const void* ent, int en
                           int64_t d, int64_t N, int64_t R, float* Q, float* bias, void* stream);
 
 /*
+ * kge_build_query (any of the six models: r is DeCaL's third base count, ignored otherwise) with dropout in
+ * training mode; dropout NULL: the plain call.  Tail direction only.
+ */
+int kge_build_query_dropout(int model, int p, int q, int r, const void* ent, int ent_dtype, const float* ent_scale,
+                            const void* rel, int rel_dtype, const float* coeff_p, const float* coeff_q,
+                            const float* coeff_r, int normalize_relation, const kge_norm_params* norm,
+                            const kge_dropout_params* dropout, const int64_t* hr, int64_t B, int64_t d, int64_t N,
+                            int64_t R, float* Q, float* bias, void* stream);
+
+/*
  * Backward of kge_build_query (tail direction, fp32 tables, no normalisation layer; with one:
  * kge_build_query_backward_norm below): given dL/dQ [B,d] and
  * dL/dbias [B] (may be NULL), ADDS dL/d(head row) into d_ent[hr[b,0], :], dL/d(relation row) into
@@ -161,13 +185,15 @@ int kge_build_query_backward(int model, int p, int q, int r, const float* ent, c
  * ADDED into dnorm's arrays (what autograd leaves in normalize_head_entity_embeddings.weight.grad etc.).
  * BatchNorm1d(affine=False) with its running statistics (eval mode): the elementwise map
  * dx = dy / sqrt(running_var + eps); batch statistics (training mode) are not part of this call.  d <= 4096.
+ * dropout: NULL, or the masks of the forward (kge_build_query_dropout); with norm NULL this is the plain backward
+ * through dropout alone.
  */
 int kge_build_query_backward_norm(int model, int p, int q, int r, const float* ent, const float* rel,
                                   const float* coeff_p, const float* coeff_q, const float* coeff_r,
                                   int normalize_relation, const kge_norm_params* norm, const kge_norm_grads* dnorm,
-                                  const int64_t* hr, int64_t B, int64_t d, int64_t N, int64_t R, const float* dQ,
-                                  const float* dbias, float* d_ent, float* d_rel, float* d_coeff_p, float* d_coeff_q,
-                                  float* d_coeff_r, void* stream);
+                                  const kge_dropout_params* dropout, const int64_t* hr, int64_t B, int64_t d,
+                                  int64_t N, int64_t R, const float* dQ, const float* dbias, float* d_ent,
+                                  float* d_rel, float* d_coeff_p, float* d_coeff_q, float* d_coeff_r, void* stream);
 
 /*
  * BatchNorm1d(affine=False) in TRAINING mode (dicee/models/base_model.py:289-294 applied at :381-383 while
@@ -185,16 +211,19 @@ int kge_build_query_backward_norm(int model, int p, int q, int r, const float* e
  * holds the SAME statistics the forward used.  workspace: kge_batchnorm_workspace_bytes(B, d) = 32 * d +
  * 8 * B * d bytes (the gradients at the normalised rows make a round trip: their sums over the batch are needed
  * before any gradient at a raw row can be formed), 16-byte aligned.  d <= 4096.
+ * dropout (both calls): NULL, or the masks of this batch's forward; the statistics are those of the rows after
+ * dropout, which is what the layer is given (base_model.py:381-383).
  */
 size_t kge_batchnorm_workspace_bytes(int64_t B, int64_t d);
 int kge_batchnorm_stats(const float* ent, const float* rel, const int64_t* hr, int64_t B, int64_t d, int64_t N,
-                        int64_t R, float momentum, float* h_mean, float* h_var, float* r_mean, float* r_var,
-                        float* run_h_mean, float* run_h_var, float* run_r_mean, float* run_r_var, void* workspace,
-                        size_t workspace_bytes, void* stream);
+                        int64_t R, const kge_dropout_params* dropout, float momentum, float* h_mean, float* h_var,
+                        float* r_mean, float* r_var, float* run_h_mean, float* run_h_var, float* run_r_mean,
+                        float* run_r_var, void* workspace, size_t workspace_bytes, void* stream);
 int kge_build_query_backward_batchnorm(int model, int p, int q, int r, const float* ent, const float* rel,
                                        const float* coeff_p, const float* coeff_q, const float* coeff_r,
-                                       int normalize_relation, const kge_norm_params* norm, const int64_t* hr,
-                                       int64_t B, int64_t d, int64_t N, int64_t R, const float* dQ, const float* dbias,
+                                       int normalize_relation, const kge_norm_params* norm,
+                                       const kge_dropout_params* dropout, const int64_t* hr, int64_t B, int64_t d,
+                                       int64_t N, int64_t R, const float* dQ, const float* dbias,
                                        float* d_ent, float* d_rel, float* d_coeff_p, float* d_coeff_q,
                                        float* d_coeff_r, void* workspace, size_t workspace_bytes, void* stream);
 

@@ -183,17 +183,26 @@ def batch_norm_running_update(x, running_mean, running_var, momentum=0.1):
             (1 - momentum) * np.asarray(running_var, np.float64) + momentum * var_unbiased)
 
 
-def gather_hr(E, R, hr, norm=None, dtype=np.float64):
+def gather_hr(E, R, hr, norm=None, dtype=np.float64, dropout=None):
     """Head / relation rows for a batch of (head_id, relation_id) pairs.
 
     Dropout is the identity in eval mode (base_model.py:149-151).  ``norm`` is
     None (IdentityClass) or a dict: ``{"kind": "LayerNorm", "h_weight", "h_bias",
     "r_weight", "r_bias", "eps"}`` / ``{"kind": "BatchNorm1d", "h_mean", "h_var",
     "r_mean", "r_var", "eps"}`` / ``{"kind": "BatchNorm1dTrain", "eps"}`` (the statistics of this very batch).
+    ``dropout`` (training mode, base_model.py:381-383: on the looked-up rows, BEFORE the normaliser): dict with
+    ``keep_h`` / ``keep_r`` ([B,d] 0/1 masks, either may be missing) and ``scale_in`` = 1 / (1 - rate); torch.nn.Dropout
+    multiplies the kept elements by that scale and zeroes the others.
     """
     hr = np.asarray(hr)
     h = np.take(np.asarray(E), hr[:, 0], axis=0).astype(dtype)
     r = np.take(np.asarray(R), hr[:, 1], axis=0).astype(dtype)
+    if dropout is not None:
+        scale = dropout.get("scale_in", 1.0)
+        if dropout.get("keep_h") is not None:
+            h = (h * (np.asarray(dropout["keep_h"]) != 0) * scale).astype(dtype)
+        if dropout.get("keep_r") is not None:
+            r = (r * (np.asarray(dropout["keep_r"]) != 0) * scale).astype(dtype)
     if norm is not None:
         eps = norm.get("eps", 1e-5)
         if norm["kind"] == "LayerNorm":
@@ -558,11 +567,15 @@ def decal_head_query(r_emb, t, p, q, r, coeff_p=None, coeff_q=None, coeff_r=None
 
 
 def build_query(model, E, R, hr, p=0, q=0, coeff_p=None, coeff_q=None,
-                normalize_relation=True, norm=None, dtype=np.float64, r=0, coeff_r=None):
-    """(Q [B,d], bias [B]) such that ``scores = Q @ E.T + bias[:, None]``."""
-    h, r_ = gather_hr(E, R, hr, norm=norm, dtype=dtype)
+                normalize_relation=True, norm=None, dtype=np.float64, r=0, coeff_r=None, dropout=None):
+    """(Q [B,d], bias [B]) such that ``scores = Q @ E.T + bias[:, None]``.  ``dropout``: see ``gather_hr``; its
+    ``keep_q`` / ``scale_hidden`` are DistMult's dropout on ``h * r`` (real.py:32)."""
+    h, r_ = gather_hr(E, R, hr, norm=norm, dtype=dtype, dropout=dropout)
     if model == "DistMult":
-        return distmult_query(h, r_), np.zeros(len(h), dtype)
+        Q = distmult_query(h, r_)
+        if dropout is not None and dropout.get("keep_q") is not None:
+            Q = (Q * (np.asarray(dropout["keep_q"]) != 0) * dropout.get("scale_hidden", 1.0)).astype(dtype)
+        return Q, np.zeros(len(h), dtype)
     if model == "ComplEx":
         return complex_query(h, r_), np.zeros(len(h), dtype)
     if model == "QMult":

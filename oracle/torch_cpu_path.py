@@ -27,10 +27,12 @@ def _quaternion_normalizer(x):
 
 
 def k_vs_all_score(model, emb_h, emb_r, emb_E, p=0, q=0, coeff_p=None, coeff_q=None,
-                   normalize_relation=True):
-    """[B,N] scores with the reference's per-model sequence of torch ops."""
+                   normalize_relation=True, hidden=None):
+    """[B,N] scores with the reference's per-model sequence of torch ops.  ``hidden``: what stands for
+    ``hidden_dropout(hidden_normalizer(.))`` around DistMult's ``h * r`` (real.py:32); identity when None."""
     if model == "DistMult":                      # dicee/models/real.py:32
-        return torch.mm(emb_h * emb_r, emb_E.transpose(1, 0))
+        hr_ = emb_h * emb_r
+        return torch.mm(hr_ if hidden is None else hidden(hr_), emb_E.transpose(1, 0))
     if model == "ComplEx":                       # dicee/models/complex.py:254-264
         hr_, hi_ = torch.hsplit(emb_h, 2)
         rr_, ri_ = torch.hsplit(emb_r, 2)

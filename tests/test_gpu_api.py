@@ -891,6 +891,75 @@ def test_full_step_gradients_through_the_normalisation_layer_match_autograd(name
         assert np.abs(g - w).max() <= 5e-5 * rms + 1e-9, (key, np.abs(g - w).max() / rms)
 
 
+@pytest.mark.parametrize("name,d,extra", [("DistMult", 32, {}), ("Keci", 30, {"p": 2, "q": 2}),
+                                          ("ComplEx", 32, {"normalization": "LayerNorm"}),
+                                          ("QMult", 32, {"normalization": "BatchNorm1d"})])
+def test_full_step_in_training_mode_with_dropout_matches_autograd_given_the_masks_it_drew(name, d, extra):
+    """input_dropout_rate = 0.3, model.train(): the step draws its masks from torch's generator; with those masks
+    placed where the reference places its Dropout modules (base_model.py:381-383, real.py:32) autograd gives the same
+    loss and gradients.  Eval mode draws nothing and is unaffected."""
+    from dicee_amd import FilterCSR
+    import copy
+    m, triples = _toy(name, d, n=900, seed=79, input_dropout_rate=0.3, **extra)
+    er = ko.vocab(triples, "er")
+    kw = _oracle_kw(m)
+    if name == "QMult":
+        kw["normalize_relation"] = False
+    E = m.entity_embeddings.weight.detach().double().clone().requires_grad_()
+    Rel = m.relation_embeddings.weight.detach().double().clone().requires_grad_()
+    tkw = {k: (torch.tensor(v, dtype=torch.float64, requires_grad=True) if k.startswith("coeff") else v)
+           for k, v in kw.items()}
+    ref_h = copy.deepcopy(m.normalize_head_entity_embeddings).double().train()
+    ref_r = copy.deepcopy(m.normalize_relation_embeddings).double().train()
+    x_np = triples[:256, :2]
+    positives = [er[(int(h), int(r))] for h, r in x_np]
+    m = m.to("cuda").train()
+    csr = FilterCSR.from_er_vocab(er, 46, device="cuda")
+    drawn = []
+    draw = m._draw_dropout
+    m._draw_dropout = lambda *a, **k: drawn.append(draw(*a, **k)) or drawn[-1]
+    torch.manual_seed(123)
+    loss, grads = m.kvsall_bce_gradients(torch.from_numpy(x_np.copy()).cuda(), csr, label_smoothing=0.1)
+    assert len(drawn) == 1                     # one set of masks for the forward and the backward of the step
+    drop = drawn[0]
+    scale = 1 / 0.7
+    kh, kr = drop["keep_h"].cpu().double(), drop["keep_r"].cpu().double()
+    assert 0.6 < float(kh.mean()) < 0.8 and not torch.equal(kh, kr)
+    hidden = None
+    if name == "DistMult":
+        kq = drop["keep_q"].cpu().double()
+        hidden = lambda v: v * kq * scale      # noqa: E731
+    else:
+        assert "keep_q" not in drop
+    ref = tcp.kvsall_bce_step(name, E, Rel, torch.from_numpy(x_np.copy()), positives, 0.1,
+                              norm_h=lambda rows: ref_h(rows * kh * scale), norm_r=lambda rows: ref_r(rows * kr * scale),
+                              **({"hidden": hidden} if hidden else {}), **tkw)
+    ref.backward()
+    assert loss.item() == pytest.approx(ref.item(), rel=1e-5)
+    want = {"entity_embeddings.weight": E.grad, "relation_embeddings.weight": Rel.grad}
+    if "coeff_p" in tkw:
+        want["p_coefficients.weight"] = tkw["coeff_p"].grad.reshape(1, -1)
+        want["q_coefficients.weight"] = tkw["coeff_q"].grad.reshape(1, -1)
+    if extra.get("normalization") == "LayerNorm":
+        want["normalize_head_entity_embeddings.weight"] = ref_h.weight.grad
+        want["normalize_head_entity_embeddings.bias"] = ref_h.bias.grad
+        want["normalize_relation_embeddings.weight"] = ref_r.weight.grad
+        want["normalize_relation_embeddings.bias"] = ref_r.bias.grad
+    assert set(grads) == set(want)
+    for key, w in want.items():
+        w = w.numpy()
+        g = grads[key].cpu().numpy()
+        rms = np.sqrt((w ** 2).mean())
+        assert np.abs(g - w).max() <= 1e-4 * rms + 1e-9, (key, np.abs(g - w).max() / rms)
+    # a second step draws other masks; eval mode draws none and scores as a model without dropout
+    m.kvsall_bce_gradients(torch.from_numpy(x_np.copy()).cuda(), csr)
+    assert len(drawn) == 2 and not torch.equal(drawn[0]["keep_h"], drawn[1]["keep_h"])
+    m.eval()
+    s1 = m(torch.from_numpy(x_np[:4].copy()).cuda())
+    s2 = m(torch.from_numpy(x_np[:4].copy()).cuda())
+    assert torch.equal(s1, s2) and drawn[-1] is None
+
+
 def test_full_step_in_training_mode_with_batchnorm_matches_torch_modules_in_training_mode():
     """normalization='BatchNorm1d', model.train(): loss, gradients and the running statistics the step leaves against
     torch.nn.BatchNorm1d(affine=False).train() modules inside the reference's op sequence (float64, CPU)."""

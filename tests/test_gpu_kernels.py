@@ -1123,6 +1123,88 @@ def test_batchnorm_statistics_over_a_large_batch_and_bad_arguments(ops):
                                  torch.zeros_like(Eg), torch.zeros_like(Rg), norm=norm)
 
 
+@pytest.mark.parametrize("layer", ["none", "LayerNorm", "BatchNorm1d", "BatchNorm1dTrain"])
+@pytest.mark.parametrize("model,d,kw", [("DistMult", 24, {}), ("QMult", 16, {}), ("ComplEx", 70, {}),
+                                        ("Keci", 15, {"p": 2, "q": 2, "coeff_p": [0.7, 1.1], "coeff_q": [1.3, -0.4]})])
+def test_dropout_masks_forward_and_backward(ops, model, d, kw, layer):
+    """Training-mode dropout with the caller's masks on the looked-up rows (and on DistMult's h * r), alone and in
+    front of each normalisation layer: query vectors and gradients against the oracle with the same masks."""
+    rng = np.random.default_rng(1100 + d)
+    N, R, B = 9, 4, 13
+    E, Rel = random_tables(rng, N, R, d, std=0.8)
+    hr = random_hr(rng, N, R, B)
+    dQ = rng.standard_normal((B, d)).astype(np.float32)
+    dbias = rng.standard_normal(B).astype(np.float32)
+    keep = {k: (rng.random((B, d)) >= 0.3).astype(np.uint8) for k in ("keep_h", "keep_r")}
+    if model == "DistMult":
+        keep["keep_q"] = (rng.random((B, d)) >= 0.4).astype(np.uint8)
+    odrop = dict(keep, scale_in=1 / 0.7, scale_hidden=1 / 0.6)
+    gdrop = {k: (dev(torch.from_numpy(v)) if k.startswith("keep") else v) for k, v in odrop.items()}
+    Eg, Rg, hrg = dev(torch.from_numpy(E)), dev(torch.from_numpy(Rel)), dev(torch.from_numpy(hr))
+    onorm = gnorm = dnorm = None
+    if layer == "LayerNorm":
+        a_h, a_r = rng.uniform(0.5, 1.5, d).astype(np.float32), rng.uniform(0.5, 1.5, d).astype(np.float32)
+        b_h, b_r = rng.normal(0, 0.3, d).astype(np.float32), rng.normal(0, 0.3, d).astype(np.float32)
+        onorm = {"kind": layer, "h_weight": a_h, "h_bias": b_h, "r_weight": a_r, "r_bias": b_r}
+        dnorm = {k: torch.zeros(d, device="cuda") for k in ("h_a", "h_b", "r_a", "r_b")}
+    elif layer == "BatchNorm1d":
+        a_h, a_r = rng.normal(0, 0.3, d).astype(np.float32), rng.normal(0, 0.3, d).astype(np.float32)
+        b_h, b_r = rng.uniform(0.5, 2, d).astype(np.float32), rng.uniform(0.5, 2, d).astype(np.float32)
+        onorm = {"kind": layer, "h_mean": a_h, "h_var": b_h, "r_mean": a_r, "r_var": b_r}
+    if layer in ("LayerNorm", "BatchNorm1d"):
+        gnorm = {"kind": layer, "eps": 1e-5, "h_a": dev(torch.from_numpy(a_h)), "h_b": dev(torch.from_numpy(b_h)),
+                 "r_a": dev(torch.from_numpy(a_r)), "r_b": dev(torch.from_numpy(b_r))}
+    elif layer == "BatchNorm1dTrain":
+        onorm = {"kind": layer, "eps": 1e-5}
+        gnorm = ops.batchnorm_stats(Eg, Rg, hrg, dropout=gdrop)
+        x = E[hr[:, 0]].astype(np.float64) * keep["keep_h"] * (1 / 0.7)
+        np.testing.assert_allclose(gnorm["h_a"].cpu().numpy(), x.mean(axis=0), rtol=1e-5, atol=1e-6)
+        np.testing.assert_allclose(gnorm["h_b"].cpu().numpy(), x.var(axis=0), rtol=1e-5, atol=1e-6)
+    gkw = _gpu_kwargs(kw)
+    Q, bias = ops.build_query(model, Eg, Rg, hrg, norm=gnorm, dropout=gdrop, **gkw)
+    Qr, br = ko.build_query(model, E, Rel, hr, norm=onorm, dropout=odrop, **kw)
+    ok, worst = score_close(Q.cpu().numpy(), Qr, 5e-5)
+    assert ok, worst
+    assert np.abs(bias.cpu().numpy() - br).max() <= 5e-5 * (np.abs(br).max() + 1)
+    d_ent, d_rel = torch.zeros_like(Eg), torch.zeros_like(Rg)
+    ops.build_query_backward(model, Eg, Rg, hrg, dev(torch.from_numpy(dQ)), dev(torch.from_numpy(dbias)), d_ent, d_rel,
+                             norm=gnorm, dnorm=dnorm, dropout=gdrop, **gkw)
+    if layer == "BatchNorm1dTrain":
+        wE, wR = ko.build_query_backward_batch(model, E, Rel, hr, dQ, dbias, norm=onorm, dropout=odrop, **kw)
+        wc = {}
+    else:
+        wE, wR, wc = ko.build_query_backward(model, E, Rel, hr, dQ, dbias, norm=onorm, dropout=odrop, **kw)
+    for got, want, name in ((d_ent, wE, "d_ent"), (d_rel, wR, "d_rel")):
+        got = got.cpu().numpy()
+        rms = np.sqrt((want ** 2).mean())
+        assert np.abs(got - want).max() <= 2e-4 * rms + 2e-5, (name, np.abs(got - want).max() / rms)
+    if layer == "LayerNorm":
+        for gk, ok_ in (("h_a", "h_weight"), ("h_b", "h_bias"), ("r_a", "r_weight"), ("r_b", "r_bias")):
+            want = wc[ok_]
+            assert np.abs(dnorm[gk].cpu().numpy() - want).max() <= 1e-4 * np.sqrt((want ** 2).mean()) + 1e-5, gk
+
+
+def test_dropout_argument_checks(ops):
+    from dicee_amd._lib import KgeError
+    rng = np.random.default_rng(6)
+    E, Rel = random_tables(rng, 20, 3, 16)
+    hr = random_hr(rng, 20, 3, 6)
+    Eg, Rg, hrg = dev(torch.from_numpy(E)), dev(torch.from_numpy(Rel)), dev(torch.from_numpy(hr))
+    ones = torch.ones(6, 16, dtype=torch.uint8, device="cuda")
+    with pytest.raises(KgeError):      # a hidden mask for a model without hidden dropout
+        ops.build_query("ComplEx", Eg, Rg, hrg, dropout={"keep_q": ones})
+    with pytest.raises(KgeError):      # a scale below one is no 1 / (1 - rate)
+        ops.build_query("DistMult", Eg, Rg, hrg, dropout={"keep_h": ones, "scale_in": 0.5})
+    with pytest.raises(ValueError):
+        ops.build_query("DistMult", Eg, Rg, hrg, dropout={"keep_h": ones}, head=True)
+    with pytest.raises(TypeError):
+        ops.build_query("DistMult", Eg, Rg, hrg, dropout={"keep_h": ones[:3]})
+    # all-ones masks with scale one: the plain query vectors, bit for bit
+    Q0, _ = ops.build_query("DistMult", Eg, Rg, hrg)
+    Q1, _ = ops.build_query("DistMult", Eg, Rg, hrg, dropout={"keep_h": ones, "keep_r": ones, "keep_q": ones})
+    assert torch.equal(Q0, Q1)
+
+
 def test_build_query_backward_norm_argument_checks(ops):
     from dicee_amd._lib import KgeError
     rng = np.random.default_rng(5)

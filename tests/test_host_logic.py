@@ -188,23 +188,30 @@ def test_models_mirror_reference_parameters_and_have_no_cpu_fallback():
         d((torch.zeros((2, 2), dtype=torch.int64), torch.zeros((2, 3), dtype=torch.int64)))   # forward_k_vs_sample too
     with pytest.raises(NotImplementedError):
         d(torch.zeros((2, 3, 4), dtype=torch.int64))               # byte-pair-encoded input
-    # dropout: the reference drops elements in training mode (base_model.py:381-383); this path refuses instead
+    # dropout: in training mode the masks of one forward are drawn from input_dropout_rate (base_model.py:149-151 builds
+    # all three modules of this path with it); eval mode and a rate of zero draw none
     dp = models.DistMult({"model": "DistMult", "embedding_dim": 8, "num_entities": 5, "num_relations": 2,
                           "input_dropout_rate": 0.3})
     assert dp.training
-    for call in (lambda: dp(torch.zeros((2, 2), dtype=torch.int64)),
-                 lambda: dp.kvsall_training_step(torch.zeros((2, 2), dtype=torch.int64), None),
-                 lambda: dp.kvsall_bce_gradients(torch.zeros((2, 2), dtype=torch.int64), None),
-                 lambda: dp.rank_filtered(torch.zeros((2, 2), dtype=torch.int64), torch.zeros(2, dtype=torch.int64))):
-        with pytest.raises(NotImplementedError, match="dropout"):
-            call()
-    dp.eval()
-    with pytest.raises(RuntimeError):                              # eval mode: past the dropout check, then no CPU path
+    torch.manual_seed(0)
+    drop = dp._draw_dropout(1000, "cpu")
+    assert set(drop) == {"keep_h", "keep_r", "keep_q", "scale_in", "scale_hidden"}
+    assert drop["scale_in"] == pytest.approx(1 / 0.7) and drop["scale_hidden"] == pytest.approx(1 / 0.7)
+    for k in ("keep_h", "keep_r", "keep_q"):
+        assert drop[k].dtype == torch.uint8 and tuple(drop[k].shape) == (1000, 8)
+        assert abs(float(drop[k].float().mean()) - 0.7) < 0.03
+    assert set(dp._draw_dropout(4, "cpu", rows=False)) == {"keep_q", "scale_in", "scale_hidden"}
+    with pytest.raises(RuntimeError):                              # CPU tensors: refuses, never falls back
         dp(torch.zeros((2, 2), dtype=torch.int64))
+    dp.eval()
+    assert dp._draw_dropout(4, "cpu") is None
+    cx = models.ComplEx({"model": "ComplEx", "embedding_dim": 8, "num_entities": 5, "num_relations": 2,
+                         "input_dropout_rate": 0.5})
+    assert set(cx._draw_dropout(4, "cpu")) == {"keep_h", "keep_r", "scale_in", "scale_hidden"}
+    assert cx._draw_dropout(4, "cpu", rows=False) is None          # only DistMult drops elements of h * r (real.py:32)
     hd = models.ComplEx({"model": "ComplEx", "embedding_dim": 8, "num_entities": 5, "num_relations": 2,
                          "hidden_dropout_rate": 0.1})
-    with pytest.raises(NotImplementedError, match="dropout"):
-        hd(torch.zeros((2, 2), dtype=torch.int64))
+    assert hd._draw_dropout(4, "cpu") is None                      # no module of this path is built with that rate
 
 
 def test_quantised_copies_follow_the_parameters_except_through_weight_data():

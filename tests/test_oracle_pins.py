@@ -622,6 +622,32 @@ def test_batchnorm_training_mode_forward_running_statistics_and_backward_vs_torc
     np.testing.assert_allclose(dR, Rt.grad.numpy(), rtol=1e-6, atol=1e-7)
 
 
+def test_dropout_masks_in_the_query_builder_vs_torch_ops():
+    """Dropout with given masks on the looked-up rows (before LayerNorm) and on DistMult's h * r: forward and the
+    central-difference backward against autograd through x * mask * scale written out in torch."""
+    rng = np.random.default_rng(31)
+    N, R, B, d = 9, 3, 7, 8
+    E, Rel = rng.standard_normal((N, d)), rng.standard_normal((R, d))
+    hr = np.stack([rng.integers(0, N, B), rng.integers(0, R, B)], axis=1)
+    dQ = rng.standard_normal((B, d))
+    keep = {k: (rng.random((B, d)) >= 0.3).astype(np.uint8) for k in ("keep_h", "keep_r", "keep_q")}
+    drop = dict(keep, scale_in=1 / 0.7, scale_hidden=1 / 0.6)
+    ln_h, ln_r = torch.nn.LayerNorm(d).double(), torch.nn.LayerNorm(d).double()
+    norm = {"kind": "LayerNorm", "eps": ln_h.eps, "h_weight": ln_h.weight.detach().numpy(),
+            "h_bias": ln_h.bias.detach().numpy(), "r_weight": ln_r.weight.detach().numpy(),
+            "r_bias": ln_r.bias.detach().numpy()}
+    Et, Rt = torch.tensor(E, requires_grad=True), torch.tensor(Rel, requires_grad=True)
+    h = ln_h(Et[torch.from_numpy(hr[:, 0])] * torch.from_numpy(keep["keep_h"]) * (1 / 0.7))
+    r = ln_r(Rt[torch.from_numpy(hr[:, 1])] * torch.from_numpy(keep["keep_r"]) * (1 / 0.7))
+    Q = (h * r) * torch.from_numpy(keep["keep_q"]) * (1 / 0.6)
+    np.testing.assert_allclose(Q.detach().numpy(), ko.build_query("DistMult", E, Rel, hr, norm=norm, dropout=drop)[0],
+                               rtol=1e-12, atol=1e-12)
+    (Q * torch.from_numpy(dQ)).sum().backward()
+    dE, dR, _ = ko.build_query_backward("DistMult", E, Rel, hr, dQ, norm=norm, dropout=drop)
+    np.testing.assert_allclose(dE, Et.grad.numpy(), rtol=1e-6, atol=1e-7)
+    np.testing.assert_allclose(dR, Rt.grad.numpy(), rtol=1e-6, atol=1e-7)
+
+
 def test_bf16_round_vs_torch():
     rng = np.random.default_rng(13)
     x = np.concatenate([rng.normal(0, 1, 5000), rng.normal(0, 1e-20, 100), [0.0, -0.0, 1.0, 3.3895314e38]])
