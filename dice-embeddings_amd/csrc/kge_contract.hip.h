@@ -679,14 +679,14 @@ struct BceEpi {
 };
 
 // Backward of the multi-hot BCE step: g = (sigmoid(s) - y') * inv_bn for the dense part of y' (the
-// known tails are subtracted afterwards from the CSR), written both as G [B, ldG] and as its
-// transpose GT [N, ldT] (the operands of the two gradient contractions), plus the loss sums of
-// BceEpi and the row sums of g (the gradient of the per-query bias).
+// known tails are subtracted afterwards from the CSR), written as G [B, ldG] and, when GT is given, also as its
+// transpose GT [N, ldT] (the operands of the two gradient contractions when they take row-major operands only), plus
+// the loss sums of BceEpi and the row sums of g (the gradient of the per-query bias).
 struct GradArgs {
   const float* bias;
   double* sums;      // as BceArgs::sums
   float* G;
-  float* GT;
+  float* GT;         // may be null
   float* dbias;      // [B], zero-initialised; may be null
   int64_t ldG, ldT;
   float inv_bn;      // upstream gradient / (B * N)
@@ -757,7 +757,7 @@ struct GradEpi {
           rowsum[qt][4 * g + r] += gr;
           pg[(int64_t)(8 * g + r) * a.ldG] = gr;
         }
-        *(f32x4*)(pt + 8 * g) = out;
+        if (a.GT) *(f32x4*)(pt + 8 * g) = out;
       }
     } else {
 #pragma unroll
@@ -778,7 +778,7 @@ struct GradEpi {
           rowsum[qt][4 * g + r] += gr;
           if (ok) {
             pg[(int64_t)(8 * g + r) * a.ldG] = gr;
-            pt[8 * g + r] = gr;
+            if (a.GT) pt[8 * g + r] = gr;
           }
         }
       }
@@ -1540,9 +1540,19 @@ constexpr int KS_E_PLANE = KS_TILE_ROWS * 64;
 constexpr int KS_Q_PLANE = KS_WG_QUERIES * 64;
 constexpr int KS_STAGE_BYTES = 3 * KS_E_PLANE + 3 * KS_Q_PLANE;
 
-template <template <int> class EpiT, bool VEC>
-__global__ void __launch_bounds__(512, 2) ksplit_kernel(ContractArgs a, typename EpiT<KS_NQT>::Args ea) {
+// KMAJ (bit 0: the entity operand, bit 1: the query operand; VEC only): that operand is given K-MAJOR, X[k][row] with
+// the rows contiguous (row pitch lde / ldq), as the backward of a contraction meets its operands (dQ = G E sums over
+// the rows of E, dE = G^T Q over the rows of both).  Its plane in LDS is then K-major too, [32 k][rows] bf16, filled
+// with 8-byte stores of four neighbouring rows at one k (32-byte segment s of the row of k kept at s ^ 2 (k & 3), which
+// spreads a fragment read's four k rows over all banks), and a fragment is two transposing reads
+// (ds_read_b64_tr_b16: within 16 lanes, lane j receives element j % 4 of the 8 bytes that lanes j / 4 + 4 i
+// addressed, i = 0..3), each giving a lane its row at four consecutive k.  Same products in the same order as the
+// row-major form.  The K-major operand's row count and pitch must be multiples of 4 and its base 16-byte aligned.
+template <template <int> class EpiT, bool VEC, int KMAJ>
+__device__ __forceinline__ void ksplit_body(const ContractArgs& a, const typename EpiT<KS_NQT>::Args& ea) {
   using Epi = EpiT<KS_NQT>;
+  static_assert(KMAJ == 0 || VEC, "K-major operands are loaded 16 bytes at a time");
+  constexpr bool KE = (KMAJ & 1) != 0, KQ = (KMAJ & 2) != 0;
   __shared__ __attribute__((aligned(1024))) unsigned char lds[2 * KS_STAGE_BYTES];
 
   int qg;
@@ -1566,7 +1576,7 @@ __global__ void __launch_bounds__(512, 2) ksplit_kernel(ContractArgs a, typename
   const int nkc = (d + KS_KC - 1) / KS_KC;
   const int n_et = (int)((r1 - r0 + KS_TILE_ROWS - 1) / KS_TILE_ROWS);
   const int n_it = n_et * nkc;
-  const float* Ef = (const float*)a.E + k_off;
+  const float* Ef = (const float*)a.E + (KE ? (int64_t)k_off * lde : (int64_t)k_off);
 
   // Staging: a chunk is 384 rows (256 entity rows, then 128 query rows) of 128 B, taken in six passes of
   // 64 rows; in pass g thread tid takes 16 B piece (tid & 7) of row 64 g + tid / 8, so eight neighbouring
@@ -1583,17 +1593,38 @@ __global__ void __launch_bounds__(512, 2) ksplit_kernel(ContractArgs a, typename
     qr = qr < q_last ? qr : q_last;
     q_ptr[g] = a.Q + k_off + qr * ldq;
   }
+  // K-major operands: pass g of the entity operand is k rows 8 g + wave of the chunk, lane l the four rows 4 l ..;
+  // pass g of the query operand k rows 16 (g - 4) + tid / 32, four rows 4 (tid % 32) ..  A quad of rows past the
+  // operand's end is read from the last quad inside the pitch instead (its scores are never stored).
+  const int ke_kk = wave, ke_mq = lane, kq_kk = tid >> 5, kq_mq = tid & 31;
+  int64_t kq_col = q_base + 4 * kq_mq;
+  if (KQ) kq_col = (kq_col + 4 <= ldq) ? kq_col : ldq - 4;
+  const float* Qk = a.Q + (int64_t)k_off * ldq;
+  int st_k0 = 0, ld_k0 = 0;  // first k of the staged chunk, of the chunk being loaded
   f32x4 staged[6];             // passes 0..3: entity rows, 4..5: query rows
   int st_valid = 0;            // how many of this thread's four columns of the staged chunk are inside d
   int ld_valid = 0, ld_k = 0;  // the same, and the first column, for the chunk being loaded
   int ld_kc = 0;               // K chunk and first row of the tile the next loads fetch
-  int64_t ld_row = r0 + s_row;
+  int64_t ld_row = KE ? r0 : r0 + s_row;
   auto load_begin = [&]() {
     ld_k = ld_kc * KS_KC + 4 * s_piece;
     ld_valid = d - ld_k;
+    ld_k0 = ld_kc * KS_KC;
   };
   auto load_pass = [&](int g) {
     const float* row_ptr;
+    if (KE && g < 4) {
+      const int k = ld_k0 + 8 * g + ke_kk;
+      int64_t col = ld_row + 4 * ke_mq;
+      col = (col + 4 <= r1) ? col : r1 - 4;
+      staged[g] = *(const f32x4*)(Ef + (int64_t)(k < d ? k : 0) * lde + col);
+      return;
+    }
+    if (KQ && g >= 4) {
+      const int k = ld_k0 + 16 * (g - 4) + kq_kk;
+      staged[g] = *(const f32x4*)(Qk + (int64_t)(k < d ? k : 0) * ldq + kq_col);
+      return;
+    }
     if (g < 4) {
       int64_t er = ld_row + 64 * g;
       er = er < e_last ? er : e_last;
@@ -1613,10 +1644,27 @@ __global__ void __launch_bounds__(512, 2) ksplit_kernel(ContractArgs a, typename
     ld_kc = wrap ? 0 : ld_kc + 1;
     ld_row += wrap ? KS_TILE_ROWS : 0;
     st_valid = ld_valid;
+    st_k0 = ld_k0;
   };
   // 8-byte half (s_piece & 1) of 16-byte piece (s_piece >> 1); rows 64 g + s_row share the swizzle of s_row
   const int st_off = s_row * 64 + ((((s_piece >> 1) ^ ((s_row >> 2) & 3)) << 4) | ((s_piece & 1) << 3));
   auto store_pass = [&](int buf, int g) {
+    if ((KE && g < 4) || (KQ && g >= 4)) {
+      const bool e_side = g < 4;
+      const int kk = e_side ? 8 * g + ke_kk : 16 * (g - 4) + kq_kk, mq = e_side ? ke_mq : kq_mq;
+      const int pitch = e_side ? 2 * KS_TILE_ROWS : 2 * KS_WG_QUERIES, plane = e_side ? KS_E_PLANE : KS_Q_PLANE;
+      unsigned char* base = lds + buf * KS_STAGE_BYTES + (e_side ? 0 : 3 * KS_E_PLANE) + kk * pitch +
+                            ((((mq >> 2) ^ (2 * (kk & 3))) << 5) | ((mq & 3) << 3));
+      f32x4 v = staged[g];
+      const bool live = st_k0 + kk < d;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) v[j] = live ? v[j] : 0.f;
+      bf16x4 s[3];
+      split3_bf16x4(v, s);
+#pragma unroll
+      for (int part = 0; part < 3; ++part) *(bf16x4*)(base + part * plane) = s[part];
+      return;
+    }
     unsigned char* base = lds + buf * KS_STAGE_BYTES + st_off +
                           (g < 4 ? g * 4096 : 3 * KS_E_PLANE + (g - 4) * 4096);
     const int plane = g < 4 ? KS_E_PLANE : KS_Q_PLANE;
@@ -1633,6 +1681,20 @@ __global__ void __launch_bounds__(512, 2) ksplit_kernel(ContractArgs a, typename
   int foff[KS_KC / 16];
 #pragma unroll
   for (int ks = 0; ks < KS_KC / 16; ++ks) foff[ks] = c * 64 + (((2 * ks + hf) ^ ((c >> 2) & 3)) << 4);
+  // K-major planes: this lane's address inside a 32-row tile for the transposing reads of K step 0, first half (k rows
+  // 8 hf + (lane % 16) / 4, rows 16 ((lane / 16) % 2) + 4 (lane % 4) ..); per row pitch: the tile's first segment is
+  // added before the swizzle, so the two parts are kept apart
+  const int tr_k = 8 * hf + ((lane & 15) >> 2);
+  const int tr_seg = (lane >> 4) & 1, tr_in = (lane & 3) << 3;
+  auto tr_fragment = [&](const unsigned char* plane_base, int pitch, int row0, int ks) -> bf16x8 {
+    typedef __attribute__((ext_vector_type(4))) short s16x4;
+    const int seg = ((row0 >> 4) + tr_seg) ^ (2 * (tr_k & 3));
+    const unsigned char* p0 = plane_base + (16 * ks + tr_k) * pitch + (seg << 5) + tr_in;
+    const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(p0));
+    const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(p0 + 4 * pitch));
+    typedef __attribute__((ext_vector_type(8))) short s16x8;
+    return __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+  };
 
   f32x16 acc[2][2];
 #pragma unroll
@@ -1668,8 +1730,15 @@ __global__ void __launch_bounds__(512, 2) ksplit_kernel(ContractArgs a, typename
       for (int part = 0; part < 3; ++part)
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
-          fe[ks][part][t] = *(const bf16x8*)(be + part * KS_E_PLANE + t * 2048 + foff[ks]);
-          fq[ks][part][t] = *(const bf16x8*)(bq + part * KS_Q_PLANE + t * 2048 + foff[ks]);
+          if constexpr (KE)
+            fe[ks][part][t] = tr_fragment(lds + buf * KS_STAGE_BYTES + part * KS_E_PLANE, 2 * KS_TILE_ROWS, 64 * we + 32 * t, ks);
+          else
+            fe[ks][part][t] = *(const bf16x8*)(be + part * KS_E_PLANE + t * 2048 + foff[ks]);
+          if constexpr (KQ)
+            fq[ks][part][t] = tr_fragment(lds + buf * KS_STAGE_BYTES + 3 * KS_E_PLANE + part * KS_Q_PLANE,
+                                          2 * KS_WG_QUERIES, 64 * wq + 32 * t, ks);
+          else
+            fq[ks][part][t] = *(const bf16x8*)(bq + part * KS_Q_PLANE + t * 2048 + foff[ks]);
         }
     };
     // The iteration in six slices, fenced so that each keeps its share of the work: eight of the chunk's
@@ -1717,6 +1786,16 @@ __global__ void __launch_bounds__(512, 2) ksplit_kernel(ContractArgs a, typename
     }
   }
   epi.finish();
+}
+
+template <template <int> class EpiT, bool VEC>
+__global__ void __launch_bounds__(512, 2) ksplit_kernel(ContractArgs a, typename EpiT<KS_NQT>::Args ea) {
+  ksplit_body<EpiT, VEC, 0>(a, ea);
+}
+// the same with K-major operands (KMAJ = 1: the entity operand, 3: both)
+template <template <int> class EpiT, int KMAJ>
+__global__ void __launch_bounds__(512, 2) ksplit_kmajor_kernel(ContractArgs a, typename EpiT<KS_NQT>::Args ea) {
+  ksplit_body<EpiT, true, KMAJ>(a, ea);
 }
 
 // ============================================================================================

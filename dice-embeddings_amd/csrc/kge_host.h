@@ -229,6 +229,7 @@ inline size_t bce_ws_bytes() { return (2 * BCE_SLOTS + BCE_POS_SLOTS) * sizeof(d
 struct BwdPlan {
   int64_t ldG, ldT;  // row strides of G [B, ldG] and GT [N, ldT] (multiples of 4)
   int k_splits, k_split_len;
+  bool kmajor;  // d a multiple of 4: the gradient contractions read G, E and Q where they lie (no GT, ET, QT)
   size_t off_G, off_GT, off_ET, off_QT, off_part, total;
 };
 inline BwdPlan bwd_plan(int64_t B, int64_t d, int64_t N) {
@@ -246,9 +247,10 @@ inline BwdPlan bwd_plan(int64_t B, int64_t d, int64_t N) {
   auto up = [](size_t x) { return (x + 255) / 256 * 256; };
   size_t off = up(bce_ws_bytes());
   p.off_G = off;     off += up((size_t)B * p.ldG * sizeof(float));
-  p.off_GT = off;    off += up((size_t)N * p.ldT * sizeof(float));
-  p.off_ET = off;    off += up((size_t)d * p.ldG * sizeof(float));
-  p.off_QT = off;    off += up((size_t)d * p.ldT * sizeof(float));
+  p.kmajor = d % 4 == 0;
+  p.off_GT = off;    off += p.kmajor ? 0 : up((size_t)N * p.ldT * sizeof(float));
+  p.off_ET = off;    off += p.kmajor ? 0 : up((size_t)d * p.ldG * sizeof(float));
+  p.off_QT = off;    off += p.kmajor ? 0 : up((size_t)d * p.ldT * sizeof(float));
   p.off_part = off;  off += up((size_t)p.k_splits * B * d * sizeof(float));
   p.total = off;
   return p;

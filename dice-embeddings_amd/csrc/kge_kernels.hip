@@ -1155,7 +1155,7 @@ __global__ void __launch_bounds__(256) grad_pos_kernel(const int64_t* csr_row, c
       const int64_t e = col[j];
       if (e < 0 || e >= N) continue;
       G[q * ldG + e] -= pos;  // a row's tails are distinct: no two threads touch one element
-      GT[e * ldT + q] -= pos;
+      if (GT) GT[e * ldT + q] -= pos;
       ++n_valid;
     }
     if (dbias && n_valid) atomicAdd(&dbias[q], -pos * (float)n_valid);
@@ -1426,8 +1426,10 @@ int launch_rank128(const ContractArgs& base, const RankArgs& ea, hipStream_t st,
 }
 
 // ksplit_kernel alone (fp32 operands), with row strides and an optional split of K over grid.y.
+// kmaj (StoreEpi only): bit 0 / bit 1: the entity / query operand is K-major (ksplit_kmajor_kernel).
 template <template <int> class EpiT, class EArgs>
-int launch_ksplit(const ContractArgs& a, const EArgs& ea, unsigned k_splits, hipStream_t st, const char* name) {
+int launch_ksplit(const ContractArgs& a, const EArgs& ea, unsigned k_splits, hipStream_t st, const char* name,
+                  int kmaj = 0) {
   if (a.B == 0 || a.e_end <= a.e_begin) return KGE_OK;
   const int64_t nwg = contract_grid_wgs(a);
   KGE_REQUIRE(nwg <= 0x7fffffffLL && k_splits >= 1 && k_splits <= 65535, KGE_ERR_INVALID,
@@ -1438,6 +1440,20 @@ int launch_ksplit(const ContractArgs& a, const EArgs& ea, unsigned k_splits, hip
   dim3 grid((unsigned)nwg, k_splits), block(512);
   LaunchTimer timer;
   if (int trc = timer.begin(st)) return trc;
+  if constexpr (std::is_same<EpiT<KS_NQT>, StoreEpi<KS_NQT>>::value) {
+    if (kmaj) {
+      // a K-major operand: whole quads of rows, 16-byte aligned (the caller chooses this form only then)
+      KGE_REQUIRE(rows_aligned && (a.e_end - a.e_begin) % 4 == 0 && a.e_begin % 4 == 0 && (kmaj == 1 || kmaj == 3),
+                  KGE_ERR_INVALID, "%s: K-major operands need aligned quads of rows", name);
+      if (kmaj == 1) hipLaunchKernelGGL((ksplit_kmajor_kernel<EpiT, 1>), grid, block, 0, st, a, ea);
+      else hipLaunchKernelGGL((ksplit_kmajor_kernel<EpiT, 3>), grid, block, 0, st, a, ea);
+      KGE_LAUNCH_CHECK(name);
+      char kname[160];
+      snprintf(kname, sizeof(kname), "ksplit_kmajor_kernel<%s, %d>", epilogue_name<EpiT>(), kmaj);
+      if (int trc = timer.end(kname)) return trc;
+      return KGE_OK;
+    }
+  }
   if (rows_aligned)
     hipLaunchKernelGGL((ksplit_kernel<EpiT, true>), grid, block, 0, st, a, ea);
   else
@@ -2113,7 +2129,10 @@ extern "C" int kge_bce_multihot_backward(const float* Q, const float* bias, cons
   char* ws = (char*)workspace;
   double* sums = (double*)ws;
   float* G = (float*)(ws + p.off_G);
-  float* GT = (float*)(ws + p.off_GT);
+  // K-major form (d a multiple of 4): both gradient contractions read G, E and Q where they lie; otherwise G is
+  // also written transposed and E, Q are transposed into the workspace
+  const bool kmajor = p.kmajor;  // (Q and E are 16-byte aligned: check_contract)
+  float* GT = kmajor ? nullptr : (float*)(ws + p.off_GT);
   float* ET = (float*)(ws + p.off_ET);
   float* QT = (float*)(ws + p.off_QT);
   float* part = (float*)(ws + p.off_part);
@@ -2148,20 +2167,23 @@ extern "C" int kge_bce_multihot_backward(const float* Q, const float* bias, cons
     KGE_LAUNCH_CHECK("bce_final_kernel");
   }
   // (2) the other operands with the summed index contiguous: ET [d, ldG], QT [d, ldT]
-  hipLaunchKernelGGL(transpose_kernel, dim3((unsigned)((d + 31) / 32), (unsigned)((N + 31) / 32)), dim3(256), 0, st,
-                     (const float*)E, N, d, d, ET, p.ldG);
-  KGE_LAUNCH_CHECK("transpose_kernel");
-  hipLaunchKernelGGL(transpose_kernel, dim3((unsigned)((d + 31) / 32), (unsigned)((B + 31) / 32)), dim3(256), 0, st, Q, B,
-                     d, d, QT, p.ldT);
-  KGE_LAUNCH_CHECK("transpose_kernel");
-  // (3) dQ [B, d] = G . E: rows of G against rows of ET, K = N split over grid.y, partial sums reduced in order
+  if (!kmajor) {
+    hipLaunchKernelGGL(transpose_kernel, dim3((unsigned)((d + 31) / 32), (unsigned)((N + 31) / 32)), dim3(256), 0, st,
+                       (const float*)E, N, d, d, ET, p.ldG);
+    KGE_LAUNCH_CHECK("transpose_kernel");
+    hipLaunchKernelGGL(transpose_kernel, dim3((unsigned)((d + 31) / 32), (unsigned)((B + 31) / 32)), dim3(256), 0, st, Q,
+                       B, d, d, QT, p.ldT);
+    KGE_LAUNCH_CHECK("transpose_kernel");
+  }
+  // (3) dQ [B, d] = G . E: rows of G against rows of ET (or E itself, K-major), K = N split over grid.y, partial sums
+  // reduced in order
   {
-    ContractArgs b = make_args(G, ET, KGE_F32, nullptr, B, N, d, 0, d);
+    ContractArgs b = make_args(G, kmajor ? (const float*)E : ET, KGE_F32, nullptr, B, N, d, 0, d);
     b.ldq = (int)p.ldG;
-    b.lde = (int)p.ldG;
+    b.lde = kmajor ? (int)d : (int)p.ldG;
     b.k_split_len = p.k_split_len;
     StoreArgs sa{p.k_splits > 1 ? part : dQ, nullptr, d, (int64_t)B * d};
-    rc = launch_ksplit<StoreEpi>(b, sa, (unsigned)p.k_splits, st, "kge_bce_multihot_backward: dQ");
+    rc = launch_ksplit<StoreEpi>(b, sa, (unsigned)p.k_splits, st, "kge_bce_multihot_backward: dQ", kmajor ? 1 : 0);
     if (rc) return rc;
     if (p.k_splits > 1) {
       const int64_t n = B * d;
@@ -2170,13 +2192,13 @@ extern "C" int kge_bce_multihot_backward(const float* Q, const float* bias, cons
       KGE_LAUNCH_CHECK("reduce_splits_kernel");
     }
   }
-  // (4) dE [N, d] = G^T . Q: rows of GT against rows of QT, K = B
+  // (4) dE [N, d] = G^T . Q: rows of GT against rows of QT, K = B (or G and Q themselves, both K-major)
   {
-    ContractArgs b = make_args(GT, QT, KGE_F32, nullptr, N, B, d, 0, d);
-    b.ldq = (int)p.ldT;
-    b.lde = (int)p.ldT;
+    ContractArgs b = make_args(kmajor ? G : GT, kmajor ? Q : QT, KGE_F32, nullptr, N, B, d, 0, d);
+    b.ldq = kmajor ? (int)p.ldG : (int)p.ldT;
+    b.lde = kmajor ? (int)d : (int)p.ldT;
     StoreArgs sa{dE, nullptr, d, 0};
-    rc = launch_ksplit<StoreEpi>(b, sa, 1, st, "kge_bce_multihot_backward: dE");
+    rc = launch_ksplit<StoreEpi>(b, sa, 1, st, "kge_bce_multihot_backward: dE", kmajor ? 3 : 0);
     if (rc) return rc;
   }
   return KGE_OK;

@@ -430,8 +430,10 @@ int kge_bce_multihot(const float* Q, const float* bias, const void* E, int dtype
  * the backward of the torch.mm / einsum of the model's k_vs_all_score).  `loss` may be NULL; otherwise
  * it receives L as kge_bce_multihot gives it.  dQ, dbias and dE are overwritten.  fp32 tables only
  * (KGE_ERR_UNSUPPORTED otherwise), N <= 2^24.  g is formed once by the fused contraction and kept in
- * the workspace in both layouts ([B,N] and [N,B]) for the two gradient contractions, which run on the
- * same three-part bf16 MFMA kernel as the scores; the workspace is about 8 * B * N bytes.  dQ and dE are
+ * the workspace as [B,N] for the two gradient contractions, which run on the same three-part bf16 MFMA
+ * kernel as the scores and read g, E and Q where they lie (K-major operands); the workspace is about
+ * 4 * B * N bytes.  When d is not a multiple of 4, g is kept in both layouts and E and Q are transposed
+ * into the workspace as well (about 8 * B * N bytes).  dQ and dE are
  * reproducible bit for bit from call to call; dbias is summed with floating-point atomics (order varies).
  */
 size_t kge_bce_backward_workspace_bytes(int64_t B, int64_t d, int64_t N);

@@ -118,9 +118,13 @@ static void test_layouts() {
     CHECK(p.k_splits >= 1 && p.k_splits <= 64 && p.k_split_len % 32 == 0);
     CHECK((int64_t)p.k_splits * p.k_split_len >= bdn[2]);                       // the splits cover the summed index
     CHECK((int64_t)(p.k_splits - 1) * p.k_split_len < bdn[2]);                  // and none of them is empty
-    check_disjoint({{0, bce_ws_bytes()}, {p.off_G, (size_t)bdn[0] * p.ldG * 4}, {p.off_GT, (size_t)bdn[2] * p.ldT * 4},
-                    {p.off_ET, (size_t)bdn[1] * p.ldG * 4}, {p.off_QT, (size_t)bdn[1] * p.ldT * 4},
-                    {p.off_part, (size_t)p.k_splits * bdn[0] * bdn[1] * 4}}, p.total);
+    // the transposed copies exist only where the contractions cannot read G, E and Q in place (d not a multiple of 4)
+    CHECK(p.kmajor == (bdn[1] % 4 == 0));
+    const size_t copies = p.kmajor ? 0 : 1;
+    check_disjoint({{0, bce_ws_bytes()}, {p.off_G, (size_t)bdn[0] * p.ldG * 4},
+                    {p.off_GT, copies * bdn[2] * p.ldT * 4}, {p.off_ET, copies * bdn[1] * p.ldG * 4},
+                    {p.off_QT, copies * bdn[1] * p.ldT * 4}, {p.off_part, (size_t)p.k_splits * bdn[0] * bdn[1] * 4}},
+                   p.total);
   }
 }
 

@@ -681,6 +681,11 @@ def test_bce_multihot_vs_oracle(ops, FilterCSR, model, N, R, d, B, storage, kw, 
     ("DistMult", 777, 5, 64, 1, {}),
     ("ComplEx", 130, 5, 200, 513, {}),
     ("DistMult", 40, 3, 7, 33, {}),
+    # widths that are multiples of 4 take the gradient contractions with K-major operands: a second entity tile of
+    # four rows, a single quad, several K splits with a ragged last one on both products
+    ("DistMult", 1000, 5, 260, 130, {}),
+    ("DistMult", 37, 3, 4, 2, {}),
+    ("ComplEx", 5003, 5, 512, 2100, {}),
 ])
 @pytest.mark.parametrize("eps", [0.0, 0.1])
 def test_bce_backward_vs_oracle(ops, FilterCSR, model, N, R, d, B, kw, eps):
