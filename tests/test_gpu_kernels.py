@@ -1210,6 +1210,40 @@ def test_dropout_argument_checks(ops):
     assert torch.equal(Q0, Q1)
 
 
+@pytest.mark.parametrize("d,layer", [(4096, "LayerNorm"), (8192, None), (4100, "LayerNorm")])
+def test_build_query_backward_at_the_widest_rows(ops, d, layer):
+    """The widest rows the backward keeps in LDS (5.25 rows per pair with a normalisation layer: d <= 4096; 3 rows
+    without: d <= 8192), against torch autograd in float64; one element past the limit is refused."""
+    from dicee_amd._lib import KgeError
+    g = torch.Generator().manual_seed(d)
+    N, R, B = 20, 3, 9
+    E = dev(torch.randn(N, d, generator=g) * 0.5)
+    Rel = dev(torch.randn(R, d, generator=g) * 0.5)
+    hr = torch.stack([torch.randint(0, N, (B,), generator=g), torch.randint(0, R, (B,), generator=g)], 1)
+    dQ = torch.randn(B, d, generator=g)
+    norm = dn = None
+    if layer:
+        w = [torch.rand(d, generator=g) + 0.5 for _ in range(2)]
+        b = [torch.randn(d, generator=g) * 0.1 for _ in range(2)]
+        norm = {"kind": layer, "eps": 1e-5, "h_a": dev(w[0]), "h_b": dev(b[0]), "r_a": dev(w[1]), "r_b": dev(b[1])}
+        dn = {k: torch.zeros(d, device="cuda") for k in ("h_a", "h_b", "r_a", "r_b")}
+    dE, dR = torch.zeros_like(E), torch.zeros_like(Rel)
+    if d > 4096 and layer:
+        with pytest.raises(KgeError) as err:
+            ops.build_query_backward("DistMult", E, Rel, dev(hr), dev(dQ), None, dE, dR, norm=norm, dnorm=dn)
+        assert err.value.code == 2
+        return
+    ops.build_query_backward("DistMult", E, Rel, dev(hr), dev(dQ), None, dE, dR, norm=norm, dnorm=dn)
+    Et, Rt = E.double().cpu().requires_grad_(), Rel.double().cpu().requires_grad_()
+    h, r = Et[hr[:, 0]], Rt[hr[:, 1]]
+    if layer:
+        h = torch.nn.functional.layer_norm(h, (d,), w[0].double(), b[0].double(), 1e-5)
+        r = torch.nn.functional.layer_norm(r, (d,), w[1].double(), b[1].double(), 1e-5)
+    ((h * r) * dQ.double()).sum().backward()
+    for got, want in ((dE, Et.grad), (dR, Rt.grad)):
+        assert (got.double().cpu() - want).abs().max().item() <= 2e-5 * want.abs().max().item()
+
+
 def test_build_query_backward_norm_argument_checks(ops):
     from dicee_amd._lib import KgeError
     rng = np.random.default_rng(5)
