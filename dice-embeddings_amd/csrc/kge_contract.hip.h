@@ -133,6 +133,44 @@ struct StoreArgs {
   const float* bias;
   int64_t ldS;
   int64_t split_stride;  // K-split launches: partial result of range y goes to S + y * split_stride
+  int64_t row_limit;     // StoreTEpi: entity rows from this one on are not stored (0: no such limit)
+};
+// The transposed result, S[e * ldS + q]: lanes along the queries, so a wave writes runs of 128 bytes of one entity's
+// row (fp32 tables, no bias).  For products whose "entity" side is the larger matrix (dE = G^T Q as the rows of G
+// against the rows of Q: the result row is an entity's).
+template <int NQT>
+struct StoreTEpi {
+  static constexpr bool SWAP = false;
+  static constexpr bool STAGE_HOOK = false;
+  static constexpr bool DEFER = false;
+  using Args = StoreArgs;
+  struct Shared {
+    int unused;
+  };
+  Args a;
+  int64_t q0, B;
+  int c, hf;
+  __device__ void init(const Args& args, int64_t q0_, int c_, int hf_, int64_t B_) {
+    a = args; q0 = q0_; c = c_; hf = hf_; B = B_;
+  }
+  __device__ void bind(Shared*) {}
+  __device__ void stage_mark() {}
+  __device__ void stage_end() {}
+  template <bool HAS_SCALE>
+  __device__ __forceinline__ void tile(int qt, const f32x16& acc, const float* sc16, float sc_col, int64_t e_base,
+                                       int64_t limit) {
+    static_assert(!HAS_SCALE, "fp32 tables only");
+    const int64_t q = q0 + 32 * qt + c;
+    if (q >= B) return;
+    const int64_t lim = (a.row_limit && a.row_limit < limit) ? a.row_limit : limit;
+    float* p = a.S + q;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int64_t e = e_base + row_of(i, hf);
+      if (e < lim) p[e * a.ldS] = acc[i];
+    }
+  }
+  __device__ void finish() {}
 };
 template <int NQT>
 struct StoreEpi {

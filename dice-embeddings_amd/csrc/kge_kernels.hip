@@ -1308,7 +1308,8 @@ struct LaunchTimer {
 template <template <int> class EpiT>
 constexpr const char* epilogue_name() {
   using E = EpiT<2>;
-  return std::is_same<E, StoreEpi<2>>::value ? "StoreEpi" : std::is_same<E, RankEpi<2>>::value ? "RankEpi"
+  return std::is_same<E, StoreEpi<2>>::value ? "StoreEpi" : std::is_same<E, StoreTEpi<2>>::value ? "StoreTEpi"
+       : std::is_same<E, RankEpi<2>>::value ? "RankEpi"
        : std::is_same<E, TopkEpi<2>>::value ? "TopkEpi" : std::is_same<E, TopkKeyEpi<2>>::value ? "TopkKeyEpi"
        : std::is_same<E, TopkFirstEpi<2>>::value ? "TopkFirstEpi" : std::is_same<E, BceEpi<2>>::value ? "BceEpi"
        : std::is_same<E, GradEpi<2>>::value ? "GradEpi" : std::is_same<E, MinMaxEpi<2>>::value ? "MinMaxEpi" : "?";
@@ -1440,7 +1441,7 @@ int launch_ksplit(const ContractArgs& a, const EArgs& ea, unsigned k_splits, hip
   dim3 grid((unsigned)nwg, k_splits), block(512);
   LaunchTimer timer;
   if (int trc = timer.begin(st)) return trc;
-  if constexpr (std::is_same<EpiT<KS_NQT>, StoreEpi<KS_NQT>>::value) {
+  if constexpr (std::is_same<EpiT<KS_NQT>, StoreEpi<KS_NQT>>::value || std::is_same<EpiT<KS_NQT>, StoreTEpi<KS_NQT>>::value) {
     if (kmaj) {
       // a K-major operand: whole quads of rows, 16-byte aligned (the caller chooses this form only then)
       KGE_REQUIRE(rows_aligned && (a.e_end - a.e_begin) % 4 == 0 && a.e_begin % 4 == 0 && (kmaj == 1 || kmaj == 3),
@@ -2194,11 +2195,21 @@ extern "C" int kge_bce_multihot_backward(const float* Q, const float* bias, cons
   }
   // (4) dE [N, d] = G^T . Q: rows of GT against rows of QT, K = B (or G and Q themselves, both K-major)
   {
-    ContractArgs b = make_args(kmajor ? G : GT, kmajor ? Q : QT, KGE_F32, nullptr, N, B, d, 0, d);
-    b.ldq = kmajor ? (int)p.ldG : (int)p.ldT;
-    b.lde = kmajor ? (int)d : (int)p.ldT;
-    StoreArgs sa{dE, nullptr, d, 0};
-    rc = launch_ksplit<StoreEpi>(b, sa, 1, st, "kge_bce_multihot_backward: dE", kmajor ? 3 : 0);
+    if (kmajor) {
+      // the rows of Q as the "queries", the rows of G (N of them, read up to the padded pitch) as the "entities": a
+      // workgroup's share of G is 256 neighbouring columns (1 KB of every row), and the result is stored transposed
+      ContractArgs b = make_args(Q, G, KGE_F32, nullptr, d, B, p.ldG, 0, p.ldG);
+      b.ldq = (int)d;
+      b.lde = (int)p.ldG;
+      StoreArgs sa{dE, nullptr, d, 0, N};
+      rc = launch_ksplit<StoreTEpi>(b, sa, 1, st, "kge_bce_multihot_backward: dE", 3);
+    } else {
+      ContractArgs b = make_args(GT, QT, KGE_F32, nullptr, N, B, d, 0, d);
+      b.ldq = (int)p.ldT;
+      b.lde = (int)p.ldT;
+      StoreArgs sa{dE, nullptr, d, 0};
+      rc = launch_ksplit<StoreEpi>(b, sa, 1, st, "kge_bce_multihot_backward: dE");
+    }
     if (rc) return rc;
   }
   return KGE_OK;
