@@ -204,7 +204,9 @@ int kge_build_query_backward_norm(int model, int p, int q, int r, const float* e
  * layer (a = mean, b = variance) for this batch's forward.  run_* (each may be NULL): the module's running
  * statistics, updated in place as torch does in training mode, running <- (1 - momentum) * running + momentum *
  * (mean | variance * B / (B - 1)).  A pair with an id outside its table makes every statistic NaN.  B >= 2 (torch
- * raises for one value per channel).  workspace: 32 * d bytes, 8-byte aligned.
+ * raises for one value per channel).  workspace: 32 * d bytes, 8-byte aligned.  The sums over the batch are taken
+ * in double precision and met with floating-point atomics: the statistics can differ in their last bit from call
+ * to call (and so can everything formed with them).
  *
  * kge_build_query_backward_batchnorm: kge_build_query_backward through that layer, the statistics being functions
  * of the batch: dx = (dy - mean_B(dy) - xh * mean_B(dy * xh)) / sqrt(var + eps) with xh the normalised row.  norm
