@@ -34,6 +34,9 @@ struct ContractArgs {
   // workgroup sums (0: all of d; otherwise a multiple of 32, and blockIdx.y selects the range)
   int ldq, lde;
   int k_split_len;
+  // ksplit_kernel only: 0, or the number of K ranges (a multiple of 8) of a launch whose grid is flat: range y is
+  // dealt to XCD y % 8, so that the workgroups that read one range of a K-major operand share an L2
+  int k_split_xcd;
   int persistent;  // host side: the decomposition above is that of a persistent kernel (checked at launch)
 };
 
@@ -107,8 +110,7 @@ __device__ __forceinline__ u32x4 i8x8_to_bf16x8(uint32_t w0, uint32_t w1) {
 // the 8 XCDs, so ids with the same (id % 8) share an L2.  Consecutive slots on one XCD walk the
 // query groups of ONE entity chunk, which keeps that chunk's rows hot in that XCD's L2.
 // contract_grid_wgs() (host) gives the matching grid size.
-__device__ __forceinline__ bool decompose_wg(const ContractArgs& a, int& qg, int64_t& chunk) {
-  const int64_t wg = blockIdx.x;
+__device__ __forceinline__ bool decompose_wg(const ContractArgs& a, int& qg, int64_t& chunk, int64_t wg = blockIdx.x) {
   if (a.n_chunks < 8) {  // too few chunks to give every XCD one: plain order, so that all XCDs get work
     qg = (int)(wg % a.n_qgroups);
     chunk = wg / a.n_qgroups;
@@ -1595,17 +1597,27 @@ __device__ __forceinline__ void ksplit_body(const ContractArgs& a, const typenam
 
   int qg;
   int64_t chunk;
-  if (!decompose_wg(a, qg, chunk)) return;
+  int64_t wg_flat = blockIdx.x;
+  int k_range = (int)blockIdx.y;
+  if (a.k_split_xcd) {  // flat grid: consecutive ids go round the XCDs, and an XCD keeps to its K ranges
+    const int64_t per_range = a.n_chunks * a.n_qgroups, slot = wg_flat >> 3;
+    k_range = (int)(wg_flat & 7) + 8 * (int)(slot / per_range);
+    wg_flat = slot % per_range;
+  }
+  if (!decompose_wg(a, qg, chunk, wg_flat)) return;
   const int tid = threadIdx.x, lane = tid & 63, c = lane & 31, hf = lane >> 5;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int we = wave >> 1, wq = wave & 1;
   const int ldq = a.ldq ? a.ldq : a.d, lde = a.lde ? a.lde : a.d;
-  const int k_off = a.k_split_len ? (int)blockIdx.y * a.k_split_len : 0;
+  const int k_off = a.k_split_len ? k_range * a.k_split_len : 0;
   const int d = (a.k_split_len && a.d - k_off > a.k_split_len) ? a.k_split_len : a.d - k_off;  // K range of this workgroup
   const int64_t q_base = (int64_t)qg * KS_WG_QUERIES;
   const int64_t q0 = q_base + 64 * wq;
   Epi epi;
   epi.init(ea, q0, c, hf, a.B);
+  if constexpr (std::is_same<Epi, StoreEpi<KS_NQT>>::value) {
+    if (a.k_split_xcd) epi.a.S += (int64_t)k_range * epi.a.split_stride;  // (blockIdx.y is 0 in a flat grid)
+  }
   __shared__ typename Epi::Shared epi_sh;
   epi.bind(&epi_sh);
 

@@ -1219,6 +1219,7 @@ ContractArgs make_args(const float* Q, const void* E, int dtype, const float* sc
   a.d = (int)d;
   a.ldq = a.lde = 0;
   a.k_split_len = 0;
+  a.k_split_xcd = 0;
   a.persistent = 0;
   const RowClass rc = row_class(d);
   const bool fast_bf16 = dtype == KGE_BF16 && rc.lds_d != 0;  // (persistent whatever the epilogue)
@@ -1446,8 +1447,15 @@ int launch_ksplit(const ContractArgs& a, const EArgs& ea, unsigned k_splits, hip
       // a K-major operand: whole quads of rows, 16-byte aligned (the caller chooses this form only then)
       KGE_REQUIRE(rows_aligned && (a.e_end - a.e_begin) % 4 == 0 && a.e_begin % 4 == 0 && (kmaj == 1 || kmaj == 3),
                   KGE_ERR_INVALID, "%s: K-major operands need aligned quads of rows", name);
-      if (kmaj == 1) hipLaunchKernelGGL((ksplit_kmajor_kernel<EpiT, 1>), grid, block, 0, st, a, ea);
-      else hipLaunchKernelGGL((ksplit_kmajor_kernel<EpiT, 3>), grid, block, 0, st, a, ea);
+      // K ranges in eights with few entity chunks: a flat grid that keeps every range on one XCD (the workgroups of
+      // a range read the same rows of the K-major entity operand)
+      ContractArgs ax = a;
+      if (k_splits % 8 == 0 && a.n_chunks < 8 && nwg * k_splits <= 0x7fffffffLL) {
+        ax.k_split_xcd = (int)k_splits;
+        grid = dim3((unsigned)(nwg * k_splits), 1);
+      }
+      if (kmaj == 1) hipLaunchKernelGGL((ksplit_kmajor_kernel<EpiT, 1>), grid, block, 0, st, ax, ea);
+      else hipLaunchKernelGGL((ksplit_kmajor_kernel<EpiT, 3>), grid, block, 0, st, ax, ea);
       KGE_LAUNCH_CHECK(name);
       char kname[160];
       snprintf(kname, sizeof(kname), "ksplit_kmajor_kernel<%s, %d>", epilogue_name<EpiT>(), kmaj);
