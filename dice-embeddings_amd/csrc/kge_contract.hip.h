@@ -795,7 +795,7 @@ struct GradEpi {
           tss += v;
           out[r] = gr;
           rowsum[qt][4 * g + r] += gr;
-          pg[(int64_t)(8 * g + r) * a.ldG] = gr;
+          __builtin_nontemporal_store(gr, &pg[(int64_t)(8 * g + r) * a.ldG]);  // (streamed: the table stays in L2)
         }
         if (a.GT) *(f32x4*)(pt + 8 * g) = out;
       }
@@ -817,7 +817,7 @@ struct GradEpi {
           tss += ok ? v : 0.f;
           rowsum[qt][4 * g + r] += gr;
           if (ok) {
-            pg[(int64_t)(8 * g + r) * a.ldG] = gr;
+            __builtin_nontemporal_store(gr, &pg[(int64_t)(8 * g + r) * a.ldG]);  // (streamed: the table stays in L2)
             if (a.GT) pt[8 * g + r] = gr;
           }
         }

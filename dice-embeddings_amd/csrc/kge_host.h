@@ -227,14 +227,14 @@ constexpr int BCE_POS_SLOTS = 128;  // partial sums over the positives (one atom
 inline size_t bce_ws_bytes() { return (2 * BCE_SLOTS + BCE_POS_SLOTS) * sizeof(double) + 128; }
 
 struct BwdPlan {
-  int64_t ldG, ldT;  // row strides of G [B, ldG] and GT [N, ldT] (multiples of 4)
+  int64_t ldG, ldT;  // row strides of G [B, ldG] (a multiple of 32) and GT [N, ldT] (a multiple of 4)
   int k_splits, k_split_len;
   bool kmajor;  // d a multiple of 4: the gradient contractions read G, E and Q where they lie (no GT, ET, QT)
   size_t off_G, off_GT, off_ET, off_QT, off_part, total;
 };
 inline BwdPlan bwd_plan(int64_t B, int64_t d, int64_t N) {
   BwdPlan p{};
-  p.ldG = (N + 3) / 4 * 4;
+  p.ldG = (N + 31) / 32 * 32;  // rows start on 128-byte lines: a wave's run of 32 gradients is one whole line
   p.ldT = (B + 3) / 4 * 4;
   // dQ = G . E sums over N: split so that about 256 workgroups run
   const int64_t tiles = ((B + KS_WG_QUERIES - 1) / KS_WG_QUERIES) * ((d + KS_TILE_ROWS - 1) / KS_TILE_ROWS);
