@@ -326,20 +326,27 @@ def main():
         tq = (q_all[:, 0] if mode == "headrank" else q_all[:, 2]).contiguous()
         f_csr = re_csr if mode == "headrank" else cfg.csr
         best = {}
-        for n_streams in (2, 1):
+        # (streams, call_queries): the evaluator's default merges whole batches into calls of at least 8192 queries
+        # (a query's counters do not depend on what else is in its call); 0 keeps one call per batch
+        for key in ((2, 8192), (2, 0), (1, 0)):
             for _ in range(4):
                 torch.cuda.synchronize()
                 tp = time.perf_counter()
-                ranks_all = rank_in_batches(model, xq, tq, f_csr, cfg.B, streams=n_streams, heads=(mode == "headrank"))
+                ranks_all = rank_in_batches(model, xq, tq, f_csr, cfg.B, streams=key[0], heads=(mode == "headrank"),
+                                            call_queries=key[1])
                 torch.cuda.synchronize()
                 tp = time.perf_counter() - tp
-                best[n_streams] = tp if n_streams not in best else min(best[n_streams], tp)
+                best[key] = tp if key not in best else min(best[key], tp)
         n_batches = (int(xq.shape[0]) + cfg.B - 1) // cfg.B
-        out["evaluation_pass"] = {"queries": int(xq.shape[0]), "batch": cfg.B, "streams": 2, "ms": best[2] * 1e3,
-                                  "queries_per_sec": xq.shape[0] / best[2], "value": float(xq.shape[0]) * N / best[2],
-                                  "unit": "scores/s", "mrr": float((1.0 / ranks_all.double()).mean().item()),
-                                  "batches": n_batches, "ms_per_batch": best[2] * 1e3 / n_batches,
-                                  "one_stream_ms": best[1] * 1e3, "one_stream_ms_per_batch": best[1] * 1e3 / n_batches}
+        t_def, t_pb, t_pb1 = best[(2, 8192)], best[(2, 0)], best[(1, 0)]
+        out["evaluation_pass"] = {"queries": int(xq.shape[0]), "batch": cfg.B, "streams": 2, "call_queries": 8192,
+                                  "ms": t_def * 1e3, "queries_per_sec": xq.shape[0] / t_def,
+                                  "value": float(xq.shape[0]) * N / t_def, "unit": "scores/s",
+                                  "mrr": float((1.0 / ranks_all.double()).mean().item()),
+                                  "one_call_per_batch": {"batches": n_batches, "ms": t_pb * 1e3,
+                                                         "ms_per_batch": t_pb * 1e3 / n_batches,
+                                                         "one_stream_ms": t_pb1 * 1e3,
+                                                         "one_stream_ms_per_batch": t_pb1 * 1e3 / n_batches}}
         del ranks_all
     # side figures, outside the timed region: what the vendor's bf16 GEMM (torch.matmul -> hipBLASLt) sustains on this
     # box, on random and on all-zero operands (the gap is the power limit: random data toggles more), and at the

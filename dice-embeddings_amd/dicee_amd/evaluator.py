@@ -114,9 +114,14 @@ class _BatchStreams:
             self.cur.wait_stream(s)
 
 
-def rank_in_batches(model, x_all, target_all, csr, batch_size, tie="stable", streams=2, heads=False):
+def rank_in_batches(model, x_all, target_all, csr, batch_size, tie="stable", streams=2, heads=False,
+                    call_queries=8192):
     """Ranks (int64 tensor [n] on the model's device) of ``target_all`` [n] for the queries ``x_all`` [n,2]: one fused
-    rank call per batch of ``batch_size`` queries.  What does not depend on the batching is done for many batches at a
+    rank call per batch of ``batch_size`` queries, or per run of whole batches that together hold at least
+    ``call_queries`` queries (the reference's batch size bounds the B x N score matrix it materialises,
+    evaluator.py:484-508; the fused call forms no such matrix, a query's counters do not depend on what else is in
+    its call, and a call's fixed cost (the plan of its correction, launches, the last round of workgroups) is paid
+    once per call: ``call_queries=0`` keeps one call per batch).  What does not depend on the batching is done for many batches at a
     time: the query vectors and the filter rows of a group of batches (at most 64 batches or 256 MB of vectors; every
     row is a function of its own (h, r) pair alone, so the numbers are those of batch-wise calls) and the thresholds
     (the raw scores of the targets) come from one launch each, and a batch is then nothing but the plan of its filter
@@ -128,9 +133,11 @@ def rank_in_batches(model, x_all, target_all, csr, batch_size, tie="stable", str
     target_all = target_all.to(dtype=torch.int64).contiguous()
     counts = {k: torch.empty((n,), dtype=dt, device=dev) for k, dt in ops._RANK_OUT}
     bs = max(1, int(batch_size))
+    if call_queries and bs < int(call_queries):
+        bs *= -(-int(call_queries) // bs)
     d = int(model.entity_embeddings.weight.shape[1])
     group = bs * max(1, min(64, (1 << 28) // (bs * d * 4)))
-    lanes = _BatchStreams(dev, streams, bs * model.num_entities)
+    lanes = _BatchStreams(dev, streams, min(bs, n) * model.num_entities)
     try:
         with torch.no_grad():
             for g0 in range(0, n, group):

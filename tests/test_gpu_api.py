@@ -89,10 +89,14 @@ def test_evaluation_in_batches_whose_query_rows_are_not_16_byte_aligned(d, batch
     csr.to("cuda")
     x = torch.from_numpy(triples[:100, :2].copy()).cuda()
     t = torch.from_numpy(triples[:100, 2].copy()).cuda()
-    got = rank_in_batches(m, x, t, csr, batch_size)
+    got = rank_in_batches(m, x, t, csr, batch_size, call_queries=0)      # one call per batch
     c = m.rank_filtered(x, t, csr)
     want = ranks_from_counts(c["n_greater"], c["n_equal"], c["n_equal_lower"])
     assert torch.equal(got, want)
+    # whole batches merged into calls of at least ten queries (still off alignment), and into one call (the default
+    # merges up to 8192 queries): the same ranks
+    assert torch.equal(rank_in_batches(m, x, t, csr, batch_size, call_queries=10), want)
+    assert torch.equal(rank_in_batches(m, x, t, csr, batch_size), want)
     S = ko.k_vs_all_scores("DistMult", m.entity_embeddings.weight.detach().cpu().numpy(),
                            m.relation_embeddings.weight.detach().cpu().numpy(), triples[:100, :2])
     for j, (h, r, tt) in enumerate(triples[:100]):
