@@ -1415,14 +1415,28 @@ bool rank128_applies(int dtype, int64_t d, int64_t B) {
 }
 int launch_rank128(const ContractArgs& base, const RankArgs& ea, hipStream_t st, const char* name) {
   if (base.B == 0 || base.e_end <= base.e_begin) return KGE_OK;
-  ContractArgs a = base;
-  host::rank128_plan(a.B, a.e_end - a.e_begin, &a.n_qgroups, &a.n_lanes, &a.chunk_rows, &a.n_chunks);
-  const int64_t nwg = 8 * (int64_t)a.n_qgroups * a.n_lanes;
-  KGE_REQUIRE(nwg <= 0x7fffffffLL, KGE_ERR_INVALID, "%s: grid of %lld workgroups too large", name, (long long)nwg);
+  // At most 16,384 queries per launch: the query groups of a launch share the workgroup slots of an XCD, and with
+  // more than sixteen of them a group is left with a single walk over its XCD's share of the table, 32 such walks
+  // drift apart and the rows stop being shared through the L2 (C4's table, 32,768 queries: 27.9 against 24.0 ms).
+  constexpr int64_t MAX_QUERIES = 16384;
   LaunchTimer timer;
   if (int trc = timer.begin(st)) return trc;
-  hipLaunchKernelGGL((rank128_kernel<host::R128_WG_WAVES>), dim3((unsigned)nwg), dim3(64 * host::R128_WG_WAVES), 0, st, a, ea);
-  KGE_LAUNCH_CHECK(name);
+  for (int64_t s = 0; s < base.B; s += MAX_QUERIES) {
+    ContractArgs a = base;
+    RankArgs eb = ea;
+    a.B = base.B - s < MAX_QUERIES ? base.B - s : MAX_QUERIES;
+    a.Q = base.Q + s * 128;
+    eb.thr += s;
+    eb.target += s;
+    eb.n_gt += s;
+    eb.n_eq += s;
+    eb.n_eql += s;
+    host::rank128_plan(a.B, a.e_end - a.e_begin, &a.n_qgroups, &a.n_lanes, &a.chunk_rows, &a.n_chunks);
+    const int64_t nwg = 8 * (int64_t)a.n_qgroups * a.n_lanes;
+    KGE_REQUIRE(nwg <= 0x7fffffffLL, KGE_ERR_INVALID, "%s: grid of %lld workgroups too large", name, (long long)nwg);
+    hipLaunchKernelGGL((rank128_kernel<host::R128_WG_WAVES>), dim3((unsigned)nwg), dim3(64 * host::R128_WG_WAVES), 0, st, a, eb);
+    KGE_LAUNCH_CHECK(name);
+  }
   if (int trc = timer.end("rank128_kernel<8>")) return trc;
   return KGE_OK;
 }

@@ -373,6 +373,28 @@ def test_rank_partial_last_query_group_with_a_bias(ops, FilterCSR, storage, d, N
     np.testing.assert_array_equal(S_b, (S_raw + bias.cpu().numpy()[:, None]).astype(np.float32))
 
 
+def test_rank_of_more_queries_than_one_launch_of_the_four_tile_kernel_takes(ops):
+    """bf16, d = 128, B = 40,000: the four-tile rank kernel is launched per 16,384 queries (two full launches and a
+    ragged third); counters, without a filter, against torch reductions of the library's own score matrix, on the GPU."""
+    g = torch.Generator(device="cuda").manual_seed(77)
+    N, d, B = 1500, 128, 40000
+    E = (torch.randn((N, d), device="cuda", generator=g) * 0.3).to(torch.bfloat16).contiguous()
+    E[7] = E[3]                                    # ties
+    Q = torch.randn((B, d), device="cuda", generator=g) * 0.3
+    tgt = torch.randint(0, N, (B,), device="cuda", generator=g)
+    tgt[::5] = 3
+    out = ops.rank_filtered(Q, None, E, None, tgt)
+    S = ops.scores(Q, None, E, None)
+    thr = S[torch.arange(B, device="cuda"), tgt]
+    assert torch.equal(out["target_score"], thr)
+    assert torch.equal(out["n_greater"], (S > thr[:, None]).sum(1).int())
+    eq = S == thr[:, None]
+    assert torch.equal(out["n_equal"], eq.sum(1).int() - 1)
+    lower = torch.arange(N, device="cuda")[None, :] < tgt[:, None]
+    assert torch.equal(out["n_equal_lower"], (eq & lower).sum(1).int())
+    assert int(out["n_equal"].max()) >= 1
+
+
 @pytest.mark.parametrize("sq,se", [(1e-6, 1e-6), (1e6, 1e6), (1e-12, 1e-3), (1e-15, 1e-15), (3e17, 3e17), (1e-30, 1.0)])
 def test_fp32_scores_hold_their_accuracy_across_magnitudes(ops, sq, se):
     """fp32 tables run as three bf16 parts per operand.  Inside the documented range (every product q*e of a score
