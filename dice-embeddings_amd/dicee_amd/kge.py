@@ -12,6 +12,17 @@ from typing import List, Union
 import torch
 
 
+def _call_size(batch_size, fused_topk):
+    """Queries per library call.  The reference's batch size bounds the B x N score matrix of a batch
+    (knowledge_graph_embeddings.py:397-401); the fused top-k forms none and a query's top-k does not depend on what else
+    is in its call, so whole batches are merged into calls of at least 4096 queries (one launch chain and one copy to
+    the host per call instead of per batch; the reference's default batch is 2 pairs)."""
+    batch_size = max(1, int(batch_size))
+    if fused_topk and batch_size < 4096:
+        batch_size *= -(-4096 // batch_size)
+    return batch_size
+
+
 class KGE:
     def __init__(self, path=None, model=None, entity_to_idx=None, relation_to_idx=None, model_name=None,
                  device="cuda"):
@@ -66,6 +77,7 @@ class KGE:
             indices = torch.zeros(P, topk, dtype=torch.long)
         else:
             scores = torch.zeros(P * T)
+        batch_size = _call_size(batch_size, return_indices)
         for i in range(0, P, batch_size):
             batch_hr = hr_pairs[i:i + batch_size].to(dev)
             B = batch_hr.size(0)
@@ -101,6 +113,7 @@ class KGE:
             indices = torch.zeros(P, topk, dtype=torch.long)
         else:
             scores = torch.zeros(P * H)
+        batch_size = _call_size(batch_size, return_indices)
         for i in range(0, P, batch_size):
             batch = tr_pairs[i:i + batch_size]
             rt = torch.stack([batch[:, 1], batch[:, 0]], dim=1).to(dev)      # the kernels take (relation, tail)
